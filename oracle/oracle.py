@@ -1,0 +1,178 @@
+"""ctypes binding of the C oracle (oracle/qmm_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: the product package never imports this module.  Each
+function forwards to the C restatement of candle-core 0.10.2's scalar CPU path;
+see the header of qmm_oracle.c for what pins each of them.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle_qmm.so")
+
+GGML_Q8_0 = 8
+GGML_Q4_K = 12
+BLOCK_SIZE = {GGML_Q8_0: 32, GGML_Q4_K: 256}
+TYPE_SIZE = {GGML_Q8_0: 34, GGML_Q4_K: 144}
+# activation-side ("vec dot") block of each weight type
+ACT_BLOCK_SIZE = {GGML_Q8_0: 32, GGML_Q4_K: 256}
+ACT_TYPE_SIZE = {GGML_Q8_0: 34, GGML_Q4_K: 292}
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with the Makefile beside it (gcc, -ffp-contract=off)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle_qmm.so"],
+                              stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(_LIB_PATH)
+        i64, f32p, vp = C.c_int64, C.POINTER(C.c_float), C.c_void_p
+        L.oracle_f16_to_f32.restype = C.c_float
+        L.oracle_f16_to_f32.argtypes = [C.c_uint16]
+        L.oracle_f32_to_f16.restype = C.c_uint16
+        L.oracle_f32_to_f16.argtypes = [C.c_float]
+        L.oracle_storage_bytes.restype = i64
+        L.oracle_storage_bytes.argtypes = [C.c_int, i64, i64]
+        L.oracle_qmatmul.restype = C.c_int
+        L.oracle_qmatmul.argtypes = [C.c_int, i64, i64, i64, vp, vp, vp]
+        L.oracle_quantize.restype = C.c_int
+        L.oracle_quantize.argtypes = [C.c_int, i64, i64, vp, vp]
+        L.oracle_dequantize.restype = C.c_int
+        L.oracle_dequantize.argtypes = [C.c_int, i64, i64, vp, vp]
+        L.oracle_quantize_activations.restype = C.c_int
+        L.oracle_quantize_activations.argtypes = [C.c_int, i64, i64, vp, vp]
+        L.oracle_moe_route.restype = None
+        L.oracle_moe_route.argtypes = [vp, i64, C.c_int, C.c_int, vp, vp]
+        L.oracle_moe_sort.restype = None
+        L.oracle_moe_sort.argtypes = [vp, i64, C.c_int, C.c_int, vp, vp]
+        L.oracle_moe_forward.restype = C.c_int
+        L.oracle_moe_forward.argtypes = [C.c_int, i64, C.c_int, C.c_int, i64, i64,
+                                         vp, vp, vp, vp, vp, vp, vp]
+        L.oracle_fill_normal.restype = None
+        L.oracle_fill_normal.argtypes = [C.c_uint64, i64, i64, C.c_float, C.c_float, vp]
+        L.oracle_get_scale_min_k4.restype = None
+        L.oracle_get_scale_min_k4.argtypes = [C.c_int, vp, vp, vp]
+        _lib = L
+    return _lib
+
+
+def _ptr(a: np.ndarray) -> int:
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data
+
+
+def storage_bytes(dtype: int, rows: int, cols: int) -> int:
+    """`quantized_storage_bytes` (qwen3/core.rs:891-909); -1 when not divisible."""
+    return int(lib().oracle_storage_bytes(dtype, rows, cols))
+
+
+def f16_to_f32(bits: int) -> float:
+    return float(lib().oracle_f16_to_f32(bits))
+
+
+def f32_to_f16(v: float) -> int:
+    return int(lib().oracle_f32_to_f16(v))
+
+
+def randn(seed: int, shape, mean: float = 0.0, std: float = 1.0, offset: int = 0) -> np.ndarray:
+    """Seeded N(mean, std) f32 array from the oracle's counter-based generator."""
+    out = np.empty(shape, dtype=np.float32)
+    lib().oracle_fill_normal(seed, offset, out.size, mean, std, _ptr(out))
+    return out
+
+
+def quantize(dtype: int, w: np.ndarray) -> np.ndarray:
+    """`QTensor::quantize(w, dtype)` -> raw GGUF block bytes, uint8 [rows * bytes_per_row]."""
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    rows, cols = w.shape
+    nbytes = storage_bytes(dtype, rows, cols)
+    if nbytes < 0 or cols % BLOCK_SIZE[dtype]:
+        raise ValueError("last dim is not a multiple of the block size")
+    out = np.empty(nbytes, dtype=np.uint8)
+    rc = lib().oracle_quantize(dtype, rows, cols, _ptr(w), _ptr(out))
+    if rc:
+        raise ValueError("oracle_quantize rejected the shape")
+    return out
+
+
+def dequantize(dtype: int, blocks: np.ndarray, rows: int, cols: int) -> np.ndarray:
+    """`QTensor::dequantize` -> f32 [rows, cols]."""
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    assert blocks.size == storage_bytes(dtype, rows, cols)
+    out = np.empty((rows, cols), dtype=np.float32)
+    rc = lib().oracle_dequantize(dtype, rows, cols, _ptr(blocks), _ptr(out))
+    if rc:
+        raise ValueError("oracle_dequantize rejected the shape")
+    return out
+
+
+def quantize_activations(weight_dtype: int, x: np.ndarray) -> np.ndarray:
+    """Rows of x quantized to the weight type's dot type (Q8_0 -> Q8_0, Q4_K -> Q8_K)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    m, k = x.shape
+    nb = k // ACT_BLOCK_SIZE[weight_dtype]
+    out = np.zeros(m * nb * ACT_TYPE_SIZE[weight_dtype], dtype=np.uint8)
+    rc = lib().oracle_quantize_activations(weight_dtype, m, k, _ptr(x), _ptr(out))
+    if rc:
+        raise ValueError("oracle_quantize_activations rejected the shape")
+    return out
+
+
+def qmatmul(dtype: int, x: np.ndarray, blocks: np.ndarray, n: int) -> np.ndarray:
+    """`QMatMul::forward` on CPU: x [m, k] f32, weight [n, k] blocks -> y [m, n] f32."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    m, k = x.shape
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    assert blocks.size == storage_bytes(dtype, n, k), "weight byte count does not match [n, k]"
+    y = np.empty((m, n), dtype=np.float32)
+    rc = lib().oracle_qmatmul(dtype, m, k, n, _ptr(x), _ptr(blocks), _ptr(y))
+    if rc:
+        raise ValueError("oracle_qmatmul rejected the shape")
+    return y
+
+
+def moe_route(logits: np.ndarray, top_k: int):
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    T, E = logits.shape
+    ids = np.empty((T, top_k), dtype=np.int32)
+    wts = np.empty((T, top_k), dtype=np.float32)
+    lib().oracle_moe_route(_ptr(logits), T, E, top_k, _ptr(ids), _ptr(wts))
+    return ids, wts
+
+
+def moe_sort(ids: np.ndarray, n_experts: int):
+    ids = np.ascontiguousarray(ids, dtype=np.int32)
+    T, top_k = ids.shape
+    perm = np.empty(T * top_k, dtype=np.int32)
+    offsets = np.empty(n_experts + 1, dtype=np.int32)
+    lib().oracle_moe_sort(_ptr(ids), T, top_k, n_experts, _ptr(perm), _ptr(offsets))
+    return perm, offsets
+
+
+def moe_forward(dtype: int, x: np.ndarray, ids: np.ndarray, wts: np.ndarray, gate: np.ndarray,
+                up: np.ndarray, down: np.ndarray, n_experts: int, inter: int) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    T, hidden = x.shape
+    ids = np.ascontiguousarray(ids, dtype=np.int32)
+    wts = np.ascontiguousarray(wts, dtype=np.float32)
+    top_k = ids.shape[1]
+    out = np.empty((T, hidden), dtype=np.float32)
+    rc = lib().oracle_moe_forward(dtype, T, n_experts, top_k, hidden, inter, _ptr(x), _ptr(ids),
+                                  _ptr(wts), _ptr(gate), _ptr(up), _ptr(down), _ptr(out))
+    if rc:
+        raise ValueError("oracle_moe_forward rejected the shape")
+    return out
