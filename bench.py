@@ -1,0 +1,263 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized linear-layer path on one MI355X.
+
+Default workload (`decode_q4k_8b_stack`): one decode token's worth of
+projections of a Qwen3-8B-shaped decoder with Q4_K weights at M = 1 — 36 layers
+x (q, k, v, o, gate, up, down) plus the LM head, 253 fused dequant+GEMV
+launches over 4.26 GB of distinct weight buffers (far beyond the 256 MB
+last-level cache, so the weights stream from HBM every step).  A step is one
+pass over all of them, replayed from a HIP graph.  `value` is algorithmic
+bytes (GGUF weight bytes + f32 activations in and out) per second.
+
+Prints ONE JSON line.  `--gpus N` with N > 1 is refused: this build is
+single-GPU (the path shards by output rows without communication; see
+DESIGN.md).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E peak
+BF16_PEAK_TFLOPS = 2500.0    # MI355X published dense bf16 MFMA peak
+
+Q8_0, Q4_K = 8, 12
+BPE = {Q8_0: 34 / 32, Q4_K: 144 / 256}
+
+# Qwen3-8B projections: (name, n, k)
+LAYER_8B = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
+            ("gate", 12288, 4096), ("up", 12288, 4096), ("down", 4096, 12288)]
+LM_HEAD_8B = ("lm_head", 151936, 4096)
+N_LAYERS_8B = 36
+
+
+def gemv_bytes(dtype, n, k, m):
+    return n * k * BPE[dtype] + 4 * m * k + 4 * m * n
+
+
+def make_blocks(oracle, dtype, n, k, seed, pool_rows=None):
+    """Seeded N(0, 0.02) weights quantized with the oracle's quantizer.  For very tall
+    matrices only `pool_rows` distinct rows are generated and repeated."""
+    import numpy as np
+    rows = n if pool_rows is None else min(n, pool_rows)
+    blocks = oracle.quantize(dtype, oracle.randn(seed, (rows, k), std=0.02))
+    if rows < n:
+        per_row = blocks.size // rows
+        reps = -(-n // rows)
+        blocks = np.tile(blocks.reshape(rows, per_row), (reps, 1))[:n].reshape(-1).copy()
+    return blocks
+
+
+def time_graph(torch, fn, steps, warmup):
+    """Captures fn() in a HIP graph and times `steps` replays with events on the
+    replay stream.  Returns (ms_per_step, graph)."""
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        fn()  # warm caches / lazy module loads outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        fn()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        for _ in range(warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        start.record(stream)
+        for _ in range(steps):
+            graph.replay()
+        end.record(stream)
+        torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps, graph
+
+
+def time_eager(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def build_decode_stack(torch, qa, oracle, dtype, m, n_layers, with_lm_head):
+    """Distinct device buffers for every projection of every layer (same seeded
+    byte content per projection kind).  Returns (calls, total_bytes, launches)."""
+    gg = qa.GgmlDType(dtype)
+    host = {name: make_blocks(oracle, dtype, n, k, 1000 + i) for i, (name, n, k) in enumerate(LAYER_8B)}
+    xs = {k: torch.from_numpy(oracle.randn(7 + k, (m, k))).cuda() for k in (4096, 12288)}
+    calls, total = [], 0.0
+    for _layer in range(n_layers):
+        for name, n, k in LAYER_8B:
+            mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, host[name], (n, k)))
+            y = torch.empty((m, n), dtype=torch.float32, device="cuda")
+            calls.append((mm, xs[k], y))
+            total += gemv_bytes(dtype, n, k, m)
+    if with_lm_head:
+        name, n, k = LM_HEAD_8B
+        blocks = make_blocks(oracle, dtype, n, k, 2000, pool_rows=16384)
+        mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, blocks, (n, k)))
+        calls.append((mm, xs[k], torch.empty((m, n), dtype=torch.float32, device="cuda")))
+        total += gemv_bytes(dtype, n, k, m)
+    del host
+    return calls, total
+
+
+def run_calls(qa, calls):
+    from izwi_amd import capi
+    from izwi_amd.qmatmul import _stream_ptr
+    L = capi.lib()
+    sp = _stream_ptr()
+    for mm, x, y in calls:
+        rc = L.izwi_qmm_forward_f32(mm.qtensor._h, x.data_ptr(), x.shape[0], y.data_ptr(), capi.DEVICE, sp)
+        if rc:
+            capi.check(rc)
+
+
+def cpu_baseline(oracle, dtype, m, budget_s=12.0):
+    """The oracle (C restatement of candle-core's scalar CPU matmul, OpenMP over
+    output columns) timed on one layer's seven projections of the same workload."""
+    import numpy as np
+    mats = []
+    for i, (name, n, k) in enumerate(LAYER_8B):
+        mats.append((n, k, make_blocks(oracle, dtype, n, k, 1000 + i), oracle.randn(7 + k, (m, k))))
+    layer_bytes = sum(gemv_bytes(dtype, n, k, m) for n, k, _, _ in mats)
+    for n, k, b, x in mats[:2]:
+        oracle.qmatmul(dtype, x, b, n)  # warm
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        for n, k, b, x in mats:
+            oracle.qmatmul(dtype, x, b, n)
+        passes += 1
+        dt = time.perf_counter() - t0
+        if dt > budget_s or passes >= 200:
+            break
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {
+        "value": round(layer_bytes * passes / dt / 1e9, 3),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{passes} passes over one Qwen3-8B layer's 7 projections (M={m}, "
+                  f"{layer_bytes / 1e6:.1f} MB algorithmic bytes per pass), {dt:.1f} s; "
+                  "C restatement of candle-core 0.10.2 scalar path, not the Candle binary",
+    }
+
+
+def prefill_extra(torch, qa, oracle, dtype, m, steps=10, warmup=3):
+    """TFLOP/s of the prefill kernel per projection (extra report, not `value`)."""
+    out = {}
+    gg = qa.GgmlDType(dtype)
+    for i, (name, n, k) in enumerate([LAYER_8B[0], LAYER_8B[1], LAYER_8B[4], LAYER_8B[6]]):
+        mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, make_blocks(oracle, dtype, n, k, 1000 + i, 4096), (n, k)))
+        x = torch.from_numpy(oracle.randn(3, (m, k))).cuda().to(torch.bfloat16)
+        ms = time_eager(torch, lambda: mm.forward(x), steps, warmup)
+        out[name] = round(2.0 * m * n * k / (ms * 1e-3) / 1e12, 2)
+        del mm
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="decode_q4k_8b_stack",
+                    choices=["decode_q4k_8b_stack", "decode_q8_0_8b_stack"])
+    ap.add_argument("--m", type=int, default=1, help="activation rows per call (decode batch)")
+    ap.add_argument("--layers", type=int, default=N_LAYERS_8B)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
+              "(no collectives are part of the path)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import izwi_amd as qa
+    from oracle import oracle  # cpu_baseline leg and seeded input generation only
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    qa.lib()
+    dtype = Q4_K if args.workload == "decode_q4k_8b_stack" else Q8_0
+
+    calls, total_bytes = build_decode_stack(torch, qa, oracle, dtype, args.m, args.layers, True)
+    launches = len(calls)
+    ms, _graph = time_graph(torch, lambda: run_calls(qa, calls), args.steps, args.warmup)
+    gbs = total_bytes / (ms * 1e-3) / 1e9
+    eager_ms = time_eager(torch, lambda: run_calls(qa, calls), max(3, args.steps // 5), 2)
+
+    result = {
+        "metric": "quant GEMV HBM GB/s (% peak) + prefill GEMM TFLOPS, Qwen3 shapes, 1 MI355X",
+        "value": round(gbs, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "i8 block dots, f32 scale/accumulate" if args.m <= 64 else "bf16",
+        "data": "synthetic: seeded N(0,0.02) weights quantized to "
+                f"{'Q4_K' if dtype == Q4_K else 'Q8_0'}, N(0,1) f32 activations; every layer has its own "
+                "device buffers (same seeded bytes per projection kind); lm_head repeats 16384 seeded rows",
+        "config": {
+            "workload": f"{args.workload}: Qwen3-8B shapes, {args.layers} layers x 7 projections + lm_head, "
+                        f"M={args.m}, {launches} launches/step, {total_bytes / 1e9:.3f} GB algorithmic bytes/step, "
+                        "HIP-graph replay",
+            "m": args.m,
+            "launches_per_step": launches,
+            "algorithmic_bytes_per_step": int(total_bytes),
+        },
+        "pct_of_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
+        "eager_ms_per_step": round(eager_ms, 4),
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "gemv_kernel (fused activation-quantize + block-dot decode kernel)",
+            "achieved": round(gbs, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "avg_launch_us": round(ms * 1e3 / launches, 3),
+            "avg_algorithmic_bytes_per_launch": int(total_bytes / launches),
+        },
+    }
+    del calls, _graph
+    torch.cuda.empty_cache()
+
+    if not args.no_extras:
+        extras = {}
+        try:
+            extras["prefill_tflops_m2048_q4k"] = prefill_extra(torch, qa, oracle, Q4_K, 2048)
+            extras["prefill_tflops_m2048_q8_0"] = prefill_extra(torch, qa, oracle, Q8_0, 2048)
+            best = max(extras["prefill_tflops_m2048_q4k"].values())
+            extras["prefill_best_frac_of_bf16_peak"] = round(best / BF16_PEAK_TFLOPS, 4)
+        except Exception as exc:  # extras never invalidate the headline number
+            extras["error"] = repr(exc)
+        result["extras"] = extras
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(oracle, dtype, args.m)
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,211 @@
+/*
+ * izwi_qmm — C ABI of the MI355X (gfx950) quantized linear-layer library.
+ *
+ * This is the drop-in boundary for the Candle `QMatMul` forward that
+ * izwi-core's Qwen3-family decoders call for every projection and the LM head
+ * (reference: crates/izwi-core/src/models/architectures/qwen3/core.rs:791-831).
+ * Every entry point is plain C: pointers, sizes and integer codes; no C++ or
+ * framework types cross it.  A Rust FFI crate (or cgo / ctypes) binds exactly
+ * these symbols.
+ *
+ * Conventions
+ *   - every function returns IZWI_QMM_OK (0) or a negative izwi_qmm_status;
+ *     the message of the last failure on the calling thread is returned by
+ *     izwi_qmm_last_error().  Shape and dtype mismatches are errors, never
+ *     aborts (the reference maps them to Error::InferenceError,
+ *     crates/izwi-core/src/error.rs:69-73).
+ *   - weights are `[n, k]` row-major in GGUF block layout (blocks along k),
+ *     ggml dtype ids as in GGUF: Q8_0 = 8, Q4_K = 12.
+ *   - `mem_space` says where the caller's buffers live: IZWI_QMM_DEVICE (HIP
+ *     device pointers, the fast path, asynchronous on `stream`) or
+ *     IZWI_QMM_HOST (ordinary host memory; the library stages it and the call
+ *     is synchronous).
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *   - all entry points are re-entrant; a weight handle is immutable after
+ *     creation and may be shared by concurrent callers (the reference calls
+ *     forward from several threads, engine/executor/dispatch.rs:150-204).
+ *   - there is no CPU fallback: without a usable HIP device every call fails
+ *     with IZWI_QMM_ERR_NO_DEVICE.
+ */
+#ifndef IZWI_QMM_H
+#define IZWI_QMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define IZWI_QMM_ABI_VERSION 1
+
+typedef enum izwi_qmm_status {
+    IZWI_QMM_OK = 0,
+    IZWI_QMM_ERR_INVALID = -1,     /* bad shape, size, dtype or NULL pointer */
+    IZWI_QMM_ERR_UNSUPPORTED = -2, /* valid request this build cannot run */
+    IZWI_QMM_ERR_HIP = -3,         /* a HIP runtime call failed */
+    IZWI_QMM_ERR_NO_DEVICE = -4    /* no gfx950 device available */
+} izwi_qmm_status;
+
+/* ggml / GGUF tensor type ids (candle-core GgmlDType) */
+#define IZWI_QMM_Q8_0 8
+#define IZWI_QMM_Q4_K 12
+
+typedef enum izwi_qmm_mem_space { IZWI_QMM_DEVICE = 0, IZWI_QMM_HOST = 1 } izwi_qmm_mem_space;
+
+/* element type of y in izwi_qmm_forward_bf16 */
+typedef enum izwi_qmm_out_dtype { IZWI_QMM_OUT_F32 = 0, IZWI_QMM_OUT_BF16 = 1 } izwi_qmm_out_dtype;
+
+typedef struct izwi_qmm_weight izwi_qmm_weight; /* opaque: QTensor + QMatMul */
+
+typedef struct izwi_qmm_weight_info {
+    int32_t ggml_dtype;
+    int32_t n_stacked; /* 1 for a plain matrix, E for an expert stack */
+    int64_t n;         /* output features (rows) */
+    int64_t k;         /* input features (cols) */
+    uint64_t nbytes;   /* GGUF block bytes of the whole handle */
+    int32_t device;    /* HIP device ordinal the weights live on */
+    int32_t reserved;
+} izwi_qmm_weight_info;
+
+/* Mirrors Qwen3RuntimeProfileSnapshot (qwen3/core.rs:571-582): the counters
+ * `izwi bench` reads (crates/izwi-cli/src/commands/bench.rs:266-289).  Times
+ * are host wall time around the call, synchronised on the stream when
+ * profiling is enabled. */
+typedef struct izwi_qmm_profile_snapshot {
+    uint64_t qmatmul_calls;
+    uint64_t qmatmul_ns;
+    uint64_t qmatmul_input_casts;
+    uint64_t qmatmul_input_cast_ns;
+    uint64_t qmatmul_output_casts;
+    uint64_t qmatmul_output_cast_ns;
+    uint64_t lm_head_calls;
+    uint64_t lm_head_ns;
+    uint64_t silu_mul_fused_calls;
+    uint64_t silu_mul_fallback_calls;
+} izwi_qmm_profile_snapshot;
+
+/* --- library ------------------------------------------------------------ */
+
+int izwi_qmm_abi_version(void);
+
+/* Selects and checks the HIP device (must be gfx950).  Optional: the first
+ * weight_create calls it with the current device. */
+int izwi_qmm_init(int device);
+
+/* Thread-local message of the last failing call ("" if none). */
+const char* izwi_qmm_last_error(void);
+
+/* --- weights: QTensor / QMatMul construction ---------------------------- */
+
+/* `quantized_storage_bytes(rows, cols, dtype)` (qwen3/core.rs:891-909):
+ * rows*cols must divide by the block size; bytes = blocks * type_size. */
+int izwi_qmm_storage_bytes(int ggml_dtype, int64_t rows, int64_t cols, uint64_t* out_bytes);
+
+/* `QMatMul::from_arc(Arc<QTensor>)` as used by `Qwen3Projection::quantized`
+ * (qwen3/core.rs:710-715): takes the tensor's raw GGUF block bytes
+ * (`QTensor::data()`), validates `nbytes` with the rule above, copies them to
+ * the device and re-tiles them for the kernels.  `k` must divide by the block
+ * size (`QTensor::quantize` requirement). */
+int izwi_qmm_weight_create(int ggml_dtype, int64_t n, int64_t k, const void* blocks,
+                           uint64_t nbytes, int mem_space, izwi_qmm_weight** out);
+
+/* `packed_qmatmul_from_qtensors` (qwen3/core.rs:846-889): row-concatenates
+ * `n_parts` tensors of equal `k` and dtype into one `[sum(rows), k]` weight
+ * (fused QKV / gate-up, qwen3/core.rs:992-1044,1179-1221).  Errors mirror the
+ * reference: empty group, input (k) mismatch, byte-count mismatch. */
+int izwi_qmm_weight_create_packed(int ggml_dtype, int32_t n_parts, const int64_t* part_rows,
+                                  int64_t k, const void* const* part_blocks,
+                                  const uint64_t* part_nbytes, int mem_space,
+                                  izwi_qmm_weight** out);
+
+/* Expert stack for the grouped MoE form: `n_experts` consecutive `[n, k]`
+ * matrices in one buffer.  No counterpart in the reference (it has no MoE
+ * code); the stacking matches how GGUF stores `ffn_*_exps` tensors. */
+int izwi_qmm_weight_create_stacked(int ggml_dtype, int32_t n_experts, int64_t n, int64_t k,
+                                   const void* blocks, uint64_t nbytes, int mem_space,
+                                   izwi_qmm_weight** out);
+
+/* Drop of the Arc<QTensor>. NULL is ignored. */
+void izwi_qmm_weight_destroy(izwi_qmm_weight* w);
+
+/* `QTensor::{dtype, shape}`. */
+int izwi_qmm_weight_get_info(const izwi_qmm_weight* w, izwi_qmm_weight_info* out);
+
+/* `QTensor::data()` (qwen3/core.rs:855,870): the original GGUF block bytes,
+ * byte-identical to what weight_create was given. */
+int izwi_qmm_weight_data(const izwi_qmm_weight* w, void* out_blocks, uint64_t nbytes,
+                         int mem_space, void* stream);
+
+/* `QTensor::dequantize` (shared/weights/gguf.rs:127-143): f32 `[n_stacked*n, k]`,
+ * bit-identical to candle-core's `to_float`. */
+int izwi_qmm_dequantize_f32(const izwi_qmm_weight* w, float* out, int mem_space, void* stream);
+
+/* --- forward: QMatMul::forward ------------------------------------------ */
+
+/* `QMatMul::forward(x)` for f32 activations (qwen3/core.rs:812; the reference
+ * always hands f32 to the op on accelerators, qwen3/core.rs:772-789).
+ * x is `[m, k]` row-major contiguous, y is `[m, n]`.  Any m >= 0; m <= 64 runs
+ * the fused decode kernel, larger m the tiled MFMA kernel.  Activations are
+ * quantized on chip to the weight type's dot type exactly as candle-core does
+ * (Q8_0 -> Q8_0 blocks, Q4_K -> Q8_K blocks), so results agree with the
+ * reference's CPU path up to f32 summation order. */
+int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, float* y,
+                         int mem_space, void* stream);
+
+/* Prefill form: bf16 activations `[m, k]`, weights dequantized to bf16 in LDS,
+ * MFMA with f32 accumulation; y is f32 or bf16 per `out_dtype`.  Replaces the
+ * to_dtype(F32) -> QMatMul -> to_dtype(activation dtype) sequence of
+ * qwen3/core.rs:798-828 with one kernel. */
+int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int64_t m, void* y,
+                          int out_dtype, int mem_space, void* stream);
+
+/* `T::VecDotType::from_float` per row (candle-core k_quants.rs `matmul`):
+ * the activation blocks the decode kernel builds on chip, written out in the
+ * reference's block layout (BlockQ8_0, 34 B per 32 values, for Q8_0 weights;
+ * BlockQ8K, 292 B per 256 values, for Q4_K weights).  Exported so that the
+ * on-chip quantizer can be checked bit for bit. */
+int izwi_qmm_quantize_activations(int ggml_weight_dtype, const float* x, int64_t m, int64_t k,
+                                  void* out_blocks, int mem_space, void* stream);
+
+/* --- expert-grouped MoE form (no counterpart in the reference) ----------- */
+
+/* Router: per token the top_k largest logits (ties: lower expert index), slots
+ * in descending-logit order; weights = softmax restricted to the selected
+ * slots (== renormalised softmax).  logits `[t, n_experts]`, ids/weights
+ * `[t, top_k]`.  ids are bit-exact by construction. */
+int izwi_moe_route(const float* logits, int64_t t, int32_t n_experts, int32_t top_k,
+                   int32_t* ids, float* weights, int mem_space, void* stream);
+
+/* Stable counting sort of the t*top_k (token, slot) pairs by expert id:
+ * perm `[t*top_k]` lists pair indices grouped by expert (ascending pair index
+ * inside a group), offsets `[n_experts+1]` is the exclusive prefix sum of the
+ * per-expert counts. */
+int izwi_moe_sort(const int32_t* ids, int64_t t, int32_t top_k, int32_t n_experts, int32_t* perm,
+                  int32_t* offsets, int mem_space, void* stream);
+
+/* Grouped expert MLP: for every pair p = (token, slot) with expert e:
+ *   h = silu(W_gate[e] x_token) * (W_up[e] x_token),  y_p = W_down[e] h
+ * (each matmul with QMatMul semantics), then out[token] = sum_slot w * y_p in
+ * slot order.  gate/up are stacks of `[inter, hidden]`, down of
+ * `[hidden, inter]`; x `[t, hidden]`, out `[t, hidden]`, all f32. */
+int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
+                         const izwi_qmm_weight* down, const float* x, int64_t t,
+                         const int32_t* ids, const float* weights, int32_t top_k,
+                         const int32_t* perm, const int32_t* offsets, float* out, int mem_space,
+                         void* stream);
+
+/* --- profiling counters (IZWI_QWEN3_PROFILE, qwen3/core.rs:624-657) ------ */
+
+/* Enabled by izwi_qmm_profile_enable(1) or the IZWI_QWEN3_PROFILE env toggle.
+ * `is_lm_head` calls are additionally counted in lm_head_* when the caller
+ * marks the handle with izwi_qmm_weight_set_lm_head. */
+int izwi_qmm_profile_enable(int enabled);
+int izwi_qmm_profile_snapshot_get(izwi_qmm_profile_snapshot* out);
+int izwi_qmm_profile_reset(void);
+int izwi_qmm_weight_set_lm_head(izwi_qmm_weight* w, int is_lm_head);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* IZWI_QMM_H */

@@ -1,0 +1,22 @@
+"""izwi_amd: MI355X-native quantized linear layer (Candle ``QMatMul`` forward).
+
+The package is a thin host-side mirror of the reference's operator interface
+(``QTensor`` / ``QMatMul`` / ``Qwen3Projection``) over the C ABI of
+``libizwi_qmm.so`` (include/izwi_qmm.h).  All arithmetic runs in hand-written
+HIP kernels for gfx950; there is no CPU or PyTorch fallback: if the library is
+missing or no GPU is present, calls raise.
+"""
+from .capi import QmmError, lib, library_path  # noqa: F401
+from .qmatmul import (  # noqa: F401
+    GgmlDType,
+    MoeExperts,
+    QMatMul,
+    QTensor,
+    Qwen3Projection,
+    moe_route,
+    moe_sort,
+    packed_qmatmul_from_qtensors,
+    profile_snapshot,
+    quantize_activations,
+    quantized_storage_bytes,
+)

@@ -1,0 +1,92 @@
+"""ctypes binding of include/izwi_qmm.h (one prototype per exported symbol)."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+OK = 0
+DEVICE, HOST = 0, 1
+OUT_F32, OUT_BF16 = 0, 1
+
+
+class QmmError(RuntimeError):
+    """A failing izwi_qmm call; mirrors the reference's Error::InferenceError."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"izwi_qmm error {code}: {message}")
+        self.code = code
+        self.message = message
+
+
+class WeightInfo(C.Structure):
+    _fields_ = [("ggml_dtype", C.c_int32), ("n_stacked", C.c_int32), ("n", C.c_int64),
+                ("k", C.c_int64), ("nbytes", C.c_uint64), ("device", C.c_int32),
+                ("reserved", C.c_int32)]
+
+
+class ProfileSnapshot(C.Structure):
+    _fields_ = [(name, C.c_uint64) for name in (
+        "qmatmul_calls", "qmatmul_ns", "qmatmul_input_casts", "qmatmul_input_cast_ns",
+        "qmatmul_output_casts", "qmatmul_output_cast_ns", "lm_head_calls", "lm_head_ns",
+        "silu_mul_fused_calls", "silu_mul_fallback_calls")]
+
+
+_i32, _i64, _u64, _vp = C.c_int32, C.c_int64, C.c_uint64, C.c_void_p
+_pp = C.POINTER(C.c_void_p)
+
+# name -> (restype, argtypes); must list every symbol include/izwi_qmm.h declares
+PROTOTYPES = {
+    "izwi_qmm_abi_version": (C.c_int, []),
+    "izwi_qmm_init": (C.c_int, [C.c_int]),
+    "izwi_qmm_last_error": (C.c_char_p, []),
+    "izwi_qmm_storage_bytes": (C.c_int, [C.c_int, _i64, _i64, C.POINTER(_u64)]),
+    "izwi_qmm_weight_create": (C.c_int, [C.c_int, _i64, _i64, _vp, _u64, C.c_int, _pp]),
+    "izwi_qmm_weight_create_packed": (C.c_int, [C.c_int, _i32, C.POINTER(_i64), _i64, _pp,
+                                                C.POINTER(_u64), C.c_int, _pp]),
+    "izwi_qmm_weight_create_stacked": (C.c_int, [C.c_int, _i32, _i64, _i64, _vp, _u64, C.c_int, _pp]),
+    "izwi_qmm_weight_destroy": (None, [_vp]),
+    "izwi_qmm_weight_get_info": (C.c_int, [_vp, C.POINTER(WeightInfo)]),
+    "izwi_qmm_weight_data": (C.c_int, [_vp, _vp, _u64, C.c_int, _vp]),
+    "izwi_qmm_dequantize_f32": (C.c_int, [_vp, _vp, C.c_int, _vp]),
+    "izwi_qmm_forward_f32": (C.c_int, [_vp, _vp, _i64, _vp, C.c_int, _vp]),
+    "izwi_qmm_forward_bf16": (C.c_int, [_vp, _vp, _i64, _vp, C.c_int, C.c_int, _vp]),
+    "izwi_qmm_quantize_activations": (C.c_int, [C.c_int, _vp, _i64, _i64, _vp, C.c_int, _vp]),
+    "izwi_moe_route": (C.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, C.c_int, _vp]),
+    "izwi_moe_sort": (C.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, C.c_int, _vp]),
+    "izwi_moe_forward_f32": (C.c_int, [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _vp, _vp,
+                                       C.c_int, _vp]),
+    "izwi_qmm_profile_enable": (C.c_int, [C.c_int]),
+    "izwi_qmm_profile_snapshot_get": (C.c_int, [C.POINTER(ProfileSnapshot)]),
+    "izwi_qmm_profile_reset": (C.c_int, []),
+    "izwi_qmm_weight_set_lm_head": (C.c_int, [_vp, C.c_int]),
+}
+
+_lib = None
+
+
+def library_path() -> str:
+    return os.path.join(_HERE, "libizwi_qmm.so")
+
+
+def lib() -> C.CDLL:
+    """Loads the in-tree HIP library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        path = library_path()
+        if not os.path.exists(path):
+            raise QmmError(-4, f"{path} is missing: build it with __graft_entry__.build() "
+                               "(make -C izwi_amd/csrc); there is no fallback path")
+        L = C.CDLL(path)
+        for name, (restype, argtypes) in PROTOTYPES.items():
+            fn = getattr(L, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = L
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != OK:
+        raise QmmError(rc, lib().izwi_qmm_last_error().decode("utf-8", "replace"))

@@ -1,0 +1,605 @@
+// C ABI of libizwi_qmm: argument checking, device memory staging and kernel
+// dispatch.  No arithmetic of the path lives here and there is no CPU fallback.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "izwi_qmm.h"
+#include "qmm_internal.h"
+
+struct izwi_qmm_weight {
+    QmmLayout layout;
+    uint64_t nbytes; // GGUF block bytes
+    void* tiled;     // device, layout.n_stacked * layout.matrix_bytes
+    int device;
+    int n_cus;
+    std::atomic<int> is_lm_head;
+};
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_error = buf;
+    return code;
+}
+
+int fail_hip(hipError_t e, const char* what) {
+    return fail(IZWI_QMM_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                                   \
+    do {                                                \
+        hipError_t _e = (expr);                         \
+        if (_e != hipSuccess) return fail_hip(_e, #expr); \
+    } while (0)
+
+struct DeviceInfo {
+    bool ok = false;
+    int n_cus = 0;
+};
+std::mutex g_dev_mutex;
+DeviceInfo g_devices[64];
+
+int ensure_device(int device, int* n_cus) {
+    if (device < 0 || device >= 64) return fail(IZWI_QMM_ERR_INVALID, "bad device ordinal %d", device);
+    std::lock_guard<std::mutex> lock(g_dev_mutex);
+    if (!g_devices[device].ok) {
+        int count = 0;
+        hipError_t e = hipGetDeviceCount(&count);
+        if (e != hipSuccess || count == 0) {
+            (void)hipGetLastError();
+            return fail(IZWI_QMM_ERR_NO_DEVICE,
+                        "no HIP device available (%s); libizwi_qmm has no CPU fallback",
+                        e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+        }
+        if (device >= count)
+            return fail(IZWI_QMM_ERR_NO_DEVICE, "device %d requested but only %d present", device, count);
+        hipDeviceProp_t prop;
+        HIP_TRY(hipGetDeviceProperties(&prop, device));
+        if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+            return fail(IZWI_QMM_ERR_NO_DEVICE, "device %d is %s; this library is built for gfx950 only",
+                        device, prop.gcnArchName);
+        g_devices[device].ok = true;
+        g_devices[device].n_cus = prop.multiProcessorCount;
+    }
+    if (n_cus) *n_cus = g_devices[device].n_cus;
+    return IZWI_QMM_OK;
+}
+
+int type_supported(int dtype) { return dtype == IZWI_QMM_Q8_0 || dtype == IZWI_QMM_Q4_K; }
+
+int storage_bytes(int dtype, int64_t rows, int64_t cols, uint64_t* out) {
+    if (!type_supported(dtype))
+        return fail(IZWI_QMM_ERR_UNSUPPORTED, "ggml dtype %d is not supported (Q8_0 = 8, Q4_K = 12)", dtype);
+    if (rows < 0 || cols < 0) return fail(IZWI_QMM_ERR_INVALID, "negative shape [%lld, %lld]", (long long)rows, (long long)cols);
+    unsigned __int128 elems = (unsigned __int128)rows * (unsigned __int128)cols;
+    if (elems > (unsigned __int128)1 << 62)
+        return fail(IZWI_QMM_ERR_INVALID, "quantized projection shape overflows");
+    uint64_t e = (uint64_t)elems;
+    uint64_t bs = (uint64_t)qmm_block_elems(dtype);
+    if (e % bs)
+        return fail(IZWI_QMM_ERR_INVALID,
+                    "quantized projection element count %llu is not divisible by block size %llu",
+                    (unsigned long long)e, (unsigned long long)bs);
+    *out = e / bs * (uint64_t)qmm_block_bytes(dtype);
+    return IZWI_QMM_OK;
+}
+
+struct Part {
+    const void* data;
+    uint64_t nbytes;
+};
+
+// Uploads the parts back to back, re-tiles them and returns the handle.
+int create_from_parts(int dtype, int64_t n_stacked, int64_t n, int64_t k, const Part* parts,
+                      int n_parts, int mem_space, izwi_qmm_weight** out) {
+    if (!out) return fail(IZWI_QMM_ERR_INVALID, "out is NULL");
+    *out = nullptr;
+    if (mem_space != IZWI_QMM_DEVICE && mem_space != IZWI_QMM_HOST)
+        return fail(IZWI_QMM_ERR_INVALID, "bad mem_space %d", mem_space);
+    if (k <= 0 || k % qmm_block_elems(dtype))
+        return fail(IZWI_QMM_ERR_INVALID, "k = %lld is not a positive multiple of the block size %d",
+                    (long long)k, qmm_block_elems(dtype));
+    int device = 0;
+    HIP_TRY(hipGetDevice(&device));
+    int n_cus = 0;
+    int rc = ensure_device(device, &n_cus);
+    if (rc) return rc;
+
+    uint64_t total = 0;
+    for (int i = 0; i < n_parts; i++) total += parts[i].nbytes;
+    QmmLayout L = qmm_make_layout(dtype, n_stacked, n, k);
+    izwi_qmm_weight* w = new izwi_qmm_weight();
+    w->layout = L;
+    w->nbytes = total;
+    w->tiled = nullptr;
+    w->device = device;
+    w->n_cus = n_cus;
+    w->is_lm_head = 0;
+    const uint64_t tiled_bytes = (uint64_t)L.n_stacked * (uint64_t)L.matrix_bytes;
+    if (tiled_bytes == 0) {
+        *out = w;
+        return IZWI_QMM_OK;
+    }
+    void* staging = nullptr;
+    hipError_t e = hipMalloc(&w->tiled, tiled_bytes);
+    if (e == hipSuccess) e = hipMalloc(&staging, total);
+    uint64_t off = 0;
+    for (int i = 0; i < n_parts && e == hipSuccess; i++) {
+        if (parts[i].nbytes)
+            e = hipMemcpy((uint8_t*)staging + off, parts[i].data, parts[i].nbytes,
+                          mem_space == IZWI_QMM_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice);
+        off += parts[i].nbytes;
+    }
+    if (e == hipSuccess) e = qmm_launch_repack(L, staging, w->tiled, nullptr);
+    if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+    if (staging) (void)hipFree(staging);
+    if (e != hipSuccess) {
+        if (w->tiled) (void)hipFree(w->tiled);
+        delete w;
+        return fail_hip(e, "weight upload");
+    }
+    *out = w;
+    return IZWI_QMM_OK;
+}
+
+// Device view of a caller buffer: the pointer itself, or a staged copy.
+struct Staged {
+    void* dev = nullptr;
+    void* host = nullptr;
+    size_t bytes = 0;
+    bool owned = false;
+    bool copy_back = false;
+    ~Staged() {
+        if (owned && dev) (void)hipFree(dev);
+    }
+    hipError_t in(const void* p, size_t n, int mem_space) {
+        bytes = n;
+        if (mem_space == IZWI_QMM_DEVICE || n == 0) {
+            dev = const_cast<void*>(p);
+            return hipSuccess;
+        }
+        owned = true;
+        hipError_t e = hipMalloc(&dev, n);
+        if (e != hipSuccess) return e;
+        return hipMemcpy(dev, p, n, hipMemcpyHostToDevice);
+    }
+    hipError_t out(void* p, size_t n, int mem_space) {
+        bytes = n;
+        if (mem_space == IZWI_QMM_DEVICE || n == 0) {
+            dev = p;
+            return hipSuccess;
+        }
+        owned = true;
+        copy_back = true;
+        host = p;
+        return hipMalloc(&dev, n);
+    }
+    hipError_t finish(hipStream_t stream) {
+        if (!copy_back) return hipSuccess;
+        hipError_t e = hipStreamSynchronize(stream);
+        if (e != hipSuccess) return e;
+        return hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost);
+    }
+};
+
+int check_space(int mem_space) {
+    if (mem_space != IZWI_QMM_DEVICE && mem_space != IZWI_QMM_HOST)
+        return fail(IZWI_QMM_ERR_INVALID, "bad mem_space %d", mem_space);
+    return IZWI_QMM_OK;
+}
+
+// ---- profiling -----------------------------------------------------------
+std::atomic<int> g_profile{-1}; // -1: read the environment on first use
+std::atomic<uint64_t> g_calls{0}, g_ns{0}, g_in_casts{0}, g_in_cast_ns{0}, g_out_casts{0},
+    g_out_cast_ns{0}, g_lm_calls{0}, g_lm_ns{0}, g_silu_fused{0}, g_silu_fallback{0};
+
+bool parse_env_bool(const char* raw) {
+    if (!raw) return false;
+    std::string s(raw);
+    for (auto& c : s) c = (char)tolower(c);
+    return s == "1" || s == "true" || s == "yes" || s == "on";
+}
+
+bool profiling() {
+    int v = g_profile.load(std::memory_order_relaxed);
+    if (v < 0) {
+        v = parse_env_bool(getenv("IZWI_QWEN3_PROFILE")) ? 1 : 0;
+        g_profile.store(v, std::memory_order_relaxed);
+    }
+    return v != 0;
+}
+
+struct ProfileScope {
+    bool on;
+    hipStream_t stream;
+    const izwi_qmm_weight* w;
+    std::chrono::steady_clock::time_point t0;
+    ProfileScope(const izwi_qmm_weight* w_, hipStream_t s) : on(profiling()), stream(s), w(w_) {
+        if (on) t0 = std::chrono::steady_clock::now();
+    }
+    ~ProfileScope() {
+        if (!on) return;
+        (void)hipStreamSynchronize(stream); // time the execution, not the launch
+        uint64_t ns = (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(
+                          std::chrono::steady_clock::now() - t0)
+                          .count();
+        g_calls.fetch_add(1, std::memory_order_relaxed);
+        g_ns.fetch_add(ns, std::memory_order_relaxed);
+        if (w && w->is_lm_head.load(std::memory_order_relaxed)) {
+            g_lm_calls.fetch_add(1, std::memory_order_relaxed);
+            g_lm_ns.fetch_add(ns, std::memory_order_relaxed);
+        }
+    }
+};
+
+} // namespace
+
+extern "C" {
+
+int izwi_qmm_abi_version(void) { return IZWI_QMM_ABI_VERSION; }
+
+const char* izwi_qmm_last_error(void) { return g_error.c_str(); }
+
+int izwi_qmm_init(int device) {
+    int rc = ensure_device(device, nullptr);
+    if (rc) return rc;
+    HIP_TRY(hipSetDevice(device));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_storage_bytes(int ggml_dtype, int64_t rows, int64_t cols, uint64_t* out_bytes) {
+    if (!out_bytes) return fail(IZWI_QMM_ERR_INVALID, "out_bytes is NULL");
+    return storage_bytes(ggml_dtype, rows, cols, out_bytes);
+}
+
+int izwi_qmm_weight_create(int ggml_dtype, int64_t n, int64_t k, const void* blocks,
+                           uint64_t nbytes, int mem_space, izwi_qmm_weight** out) {
+    return izwi_qmm_weight_create_stacked(ggml_dtype, 1, n, k, blocks, nbytes, mem_space, out);
+}
+
+int izwi_qmm_weight_create_stacked(int ggml_dtype, int32_t n_experts, int64_t n, int64_t k,
+                                   const void* blocks, uint64_t nbytes, int mem_space,
+                                   izwi_qmm_weight** out) {
+    if (n_experts < 1) return fail(IZWI_QMM_ERR_INVALID, "n_experts must be >= 1");
+    uint64_t expected = 0;
+    int rc = storage_bytes(ggml_dtype, (int64_t)n_experts * n, k, &expected);
+    if (rc) return rc;
+    if (nbytes != expected)
+        return fail(IZWI_QMM_ERR_INVALID, "quantized projection has %llu bytes, expected %llu",
+                    (unsigned long long)nbytes, (unsigned long long)expected);
+    if (expected && !blocks) return fail(IZWI_QMM_ERR_INVALID, "blocks is NULL");
+    Part part{blocks, nbytes};
+    return create_from_parts(ggml_dtype, n_experts, n, k, &part, 1, mem_space, out);
+}
+
+int izwi_qmm_weight_create_packed(int ggml_dtype, int32_t n_parts, const int64_t* part_rows,
+                                  int64_t k, const void* const* part_blocks,
+                                  const uint64_t* part_nbytes, int mem_space,
+                                  izwi_qmm_weight** out) {
+    if (n_parts <= 0 || !part_rows || !part_blocks || !part_nbytes)
+        return fail(IZWI_QMM_ERR_INVALID, "Cannot pack empty Qwen3 quantized projection group");
+    int64_t total_rows = 0;
+    uint64_t total_bytes = 0;
+    std::vector<Part> parts;
+    for (int i = 0; i < n_parts; i++) {
+        uint64_t expected = 0;
+        int rc = storage_bytes(ggml_dtype, part_rows[i], k, &expected);
+        if (rc) return rc;
+        if (part_nbytes[i] != expected)
+            return fail(IZWI_QMM_ERR_INVALID,
+                        "Qwen3 quantized projection group input mismatch: part %d has %llu bytes, "
+                        "expected %llu for [%lld, %lld]",
+                        i, (unsigned long long)part_nbytes[i], (unsigned long long)expected,
+                        (long long)part_rows[i], (long long)k);
+        if (expected && !part_blocks[i]) return fail(IZWI_QMM_ERR_INVALID, "part %d is NULL", i);
+        total_rows += part_rows[i];
+        total_bytes += part_nbytes[i];
+        parts.push_back(Part{part_blocks[i], part_nbytes[i]});
+    }
+    uint64_t expected_total = 0;
+    int rc = storage_bytes(ggml_dtype, total_rows, k, &expected_total);
+    if (rc) return rc;
+    if (expected_total != total_bytes)
+        return fail(IZWI_QMM_ERR_INVALID,
+                    "Qwen3 packed quantized projection has %llu bytes, expected %llu",
+                    (unsigned long long)total_bytes, (unsigned long long)expected_total);
+    return create_from_parts(ggml_dtype, 1, total_rows, k, parts.data(), n_parts, mem_space, out);
+}
+
+void izwi_qmm_weight_destroy(izwi_qmm_weight* w) {
+    if (!w) return;
+    if (w->tiled) (void)hipFree(w->tiled);
+    delete w;
+}
+
+int izwi_qmm_weight_get_info(const izwi_qmm_weight* w, izwi_qmm_weight_info* out) {
+    if (!w || !out) return fail(IZWI_QMM_ERR_INVALID, "NULL argument");
+    out->ggml_dtype = w->layout.dtype;
+    out->n_stacked = (int32_t)w->layout.n_stacked;
+    out->n = w->layout.n;
+    out->k = w->layout.k;
+    out->nbytes = w->nbytes;
+    out->device = w->device;
+    out->reserved = 0;
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_weight_set_lm_head(izwi_qmm_weight* w, int is_lm_head) {
+    if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    w->is_lm_head.store(is_lm_head ? 1 : 0, std::memory_order_relaxed);
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_weight_data(const izwi_qmm_weight* w, void* out_blocks, uint64_t nbytes,
+                         int mem_space, void* stream_) {
+    if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    if (int rc = check_space(mem_space)) return rc;
+    if (nbytes != w->nbytes)
+        return fail(IZWI_QMM_ERR_INVALID, "buffer has %llu bytes, tensor data has %llu",
+                    (unsigned long long)nbytes, (unsigned long long)w->nbytes);
+    if (nbytes == 0) return IZWI_QMM_OK;
+    if (!out_blocks) return fail(IZWI_QMM_ERR_INVALID, "out_blocks is NULL");
+    hipStream_t stream = (hipStream_t)stream_;
+    Staged o;
+    HIP_TRY(o.out(out_blocks, nbytes, mem_space));
+    HIP_TRY(qmm_launch_unpack(w->layout, w->tiled, o.dev, stream));
+    HIP_TRY(o.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_dequantize_f32(const izwi_qmm_weight* w, float* out, int mem_space, void* stream_) {
+    if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    if (int rc = check_space(mem_space)) return rc;
+    const QmmLayout& L = w->layout;
+    size_t bytes = (size_t)L.n_stacked * L.n * L.k * sizeof(float);
+    if (bytes == 0) return IZWI_QMM_OK;
+    if (!out) return fail(IZWI_QMM_ERR_INVALID, "out is NULL");
+    hipStream_t stream = (hipStream_t)stream_;
+    Staged o;
+    HIP_TRY(o.out(out, bytes, mem_space));
+    HIP_TRY(qmm_launch_dequant(L, w->tiled, (float*)o.dev, stream));
+    HIP_TRY(o.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_quantize_activations(int ggml_weight_dtype, const float* x, int64_t m, int64_t k,
+                                  void* out_blocks, int mem_space, void* stream_) {
+    if (!type_supported(ggml_weight_dtype))
+        return fail(IZWI_QMM_ERR_UNSUPPORTED, "ggml dtype %d is not supported", ggml_weight_dtype);
+    if (int rc = check_space(mem_space)) return rc;
+    if (m < 0 || k < 0) return fail(IZWI_QMM_ERR_INVALID, "negative shape");
+    const int bs = ggml_weight_dtype == IZWI_QMM_Q8_0 ? 32 : 256;
+    const int ts = ggml_weight_dtype == IZWI_QMM_Q8_0 ? 34 : 292;
+    if (k % bs) return fail(IZWI_QMM_ERR_INVALID, "k = %lld is not a multiple of %d", (long long)k, bs);
+    if (m == 0 || k == 0) return IZWI_QMM_OK;
+    if (!x || !out_blocks) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    int device = 0;
+    HIP_TRY(hipGetDevice(&device));
+    if (int rc = ensure_device(device, nullptr)) return rc;
+    hipStream_t stream = (hipStream_t)stream_;
+    Staged xi, o;
+    HIP_TRY(xi.in(x, (size_t)m * k * sizeof(float), mem_space));
+    HIP_TRY(o.out(out_blocks, (size_t)m * (k / bs) * ts, mem_space));
+    HIP_TRY(qmm_launch_quantize_activations(ggml_weight_dtype, (const float*)xi.dev, m, k, o.dev, stream));
+    HIP_TRY(o.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, float* y,
+                         int mem_space, void* stream_) {
+    if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    if (int rc = check_space(mem_space)) return rc;
+    const QmmLayout& L = w->layout;
+    if (L.n_stacked != 1)
+        return fail(IZWI_QMM_ERR_INVALID, "forward on an expert stack: use izwi_moe_forward_f32");
+    if (m < 0) return fail(IZWI_QMM_ERR_INVALID, "negative m");
+    if (m == 0 || L.n == 0) return IZWI_QMM_OK;
+    if (!x) return fail(IZWI_QMM_ERR_INVALID, "x is NULL");
+    if (!y) return fail(IZWI_QMM_ERR_INVALID, "y is NULL");
+    hipStream_t stream = (hipStream_t)stream_;
+    ProfileScope prof(w, stream);
+    Staged xi, yo;
+    HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
+    HIP_TRY(yo.out(y, (size_t)m * L.n * sizeof(float), mem_space));
+    if (m <= 64) {
+        HIP_TRY(qmm_launch_gemv(L, w->tiled, (const float*)xi.dev, m, (float*)yo.dev, w->n_cus, stream));
+    } else {
+        // prefill-sized m with f32 activations: convert once, then the MFMA kernel
+        void* xb = nullptr;
+        HIP_TRY(hipMallocAsync(&xb, (size_t)m * L.k * sizeof(uint16_t), stream));
+        hipError_t e = qmm_launch_f32_to_bf16((const float*)xi.dev, (uint16_t*)xb, m * L.k, stream);
+        if (e == hipSuccess)
+            e = qmm_launch_gemm_bf16(L, w->tiled, (const uint16_t*)xb, m, yo.dev, 0, w->n_cus, stream);
+        hipError_t e2 = hipFreeAsync(xb, stream);
+        if (e != hipSuccess) return fail_hip(e, "prefill kernel");
+        if (e2 != hipSuccess) return fail_hip(e2, "hipFreeAsync");
+    }
+    HIP_TRY(yo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int64_t m, void* y,
+                          int out_dtype, int mem_space, void* stream_) {
+    if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    if (int rc = check_space(mem_space)) return rc;
+    if (out_dtype != IZWI_QMM_OUT_F32 && out_dtype != IZWI_QMM_OUT_BF16)
+        return fail(IZWI_QMM_ERR_INVALID, "bad out_dtype %d", out_dtype);
+    const QmmLayout& L = w->layout;
+    if (L.n_stacked != 1) return fail(IZWI_QMM_ERR_INVALID, "forward on an expert stack");
+    if (m < 0) return fail(IZWI_QMM_ERR_INVALID, "negative m");
+    if (m == 0 || L.n == 0) return IZWI_QMM_OK;
+    if (!x_bf16) return fail(IZWI_QMM_ERR_INVALID, "x is NULL");
+    if (!y) return fail(IZWI_QMM_ERR_INVALID, "y is NULL");
+    hipStream_t stream = (hipStream_t)stream_;
+    ProfileScope prof(w, stream);
+    const size_t ybytes = (size_t)m * L.n * (out_dtype == IZWI_QMM_OUT_BF16 ? 2 : 4);
+    Staged xi, yo;
+    HIP_TRY(xi.in(x_bf16, (size_t)m * L.k * sizeof(uint16_t), mem_space));
+    HIP_TRY(yo.out(y, ybytes, mem_space));
+    HIP_TRY(qmm_launch_gemm_bf16(L, w->tiled, (const uint16_t*)xi.dev, m, yo.dev,
+                                 out_dtype == IZWI_QMM_OUT_BF16, w->n_cus, stream));
+    HIP_TRY(yo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_moe_route(const float* logits, int64_t t, int32_t n_experts, int32_t top_k, int32_t* ids,
+                   float* weights, int mem_space, void* stream_) {
+    if (int rc = check_space(mem_space)) return rc;
+    if (t < 0) return fail(IZWI_QMM_ERR_INVALID, "negative t");
+    if (n_experts < 1 || n_experts > 1024)
+        return fail(IZWI_QMM_ERR_UNSUPPORTED, "n_experts = %d outside 1..1024", n_experts);
+    if (top_k < 1 || top_k > n_experts || top_k > 64)
+        return fail(IZWI_QMM_ERR_INVALID, "top_k = %d outside 1..min(n_experts, 64)", top_k);
+    if (t == 0) return IZWI_QMM_OK;
+    if (!logits || !ids || !weights) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    int device = 0;
+    HIP_TRY(hipGetDevice(&device));
+    if (int rc = ensure_device(device, nullptr)) return rc;
+    hipStream_t stream = (hipStream_t)stream_;
+    Staged li, io, wo;
+    HIP_TRY(li.in(logits, (size_t)t * n_experts * sizeof(float), mem_space));
+    HIP_TRY(io.out(ids, (size_t)t * top_k * sizeof(int32_t), mem_space));
+    HIP_TRY(wo.out(weights, (size_t)t * top_k * sizeof(float), mem_space));
+    HIP_TRY(qmm_launch_moe_route((const float*)li.dev, t, n_experts, top_k, (int32_t*)io.dev,
+                                 (float*)wo.dev, stream));
+    HIP_TRY(io.finish(stream));
+    HIP_TRY(wo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_moe_sort(const int32_t* ids, int64_t t, int32_t top_k, int32_t n_experts, int32_t* perm,
+                  int32_t* offsets, int mem_space, void* stream_) {
+    if (int rc = check_space(mem_space)) return rc;
+    if (t < 0 || top_k < 1 || n_experts < 1 || n_experts > 8192)
+        return fail(IZWI_QMM_ERR_INVALID, "bad sort shape t=%lld top_k=%d n_experts=%d", (long long)t, top_k, n_experts);
+    const int64_t pairs = t * top_k;
+    if (pairs > 0x7fffffff) return fail(IZWI_QMM_ERR_UNSUPPORTED, "too many pairs");
+    if (!offsets || (pairs && (!ids || !perm))) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    int device = 0;
+    HIP_TRY(hipGetDevice(&device));
+    if (int rc = ensure_device(device, nullptr)) return rc;
+    hipStream_t stream = (hipStream_t)stream_;
+    Staged ii, po, oo;
+    HIP_TRY(ii.in(ids, (size_t)pairs * sizeof(int32_t), mem_space));
+    HIP_TRY(po.out(perm, (size_t)pairs * sizeof(int32_t), mem_space));
+    HIP_TRY(oo.out(offsets, (size_t)(n_experts + 1) * sizeof(int32_t), mem_space));
+    void* scratch = nullptr;
+    HIP_TRY(hipMallocAsync(&scratch, (size_t)qmm_moe_sort_scratch_ints(pairs, n_experts) * sizeof(int32_t), stream));
+    hipError_t e = qmm_launch_moe_sort((const int32_t*)ii.dev, pairs, n_experts, (int32_t*)po.dev,
+                                       (int32_t*)oo.dev, nullptr, (int32_t*)scratch, stream);
+    hipError_t e2 = hipFreeAsync(scratch, stream);
+    if (e != hipSuccess) return fail_hip(e, "sort kernels");
+    if (e2 != hipSuccess) return fail_hip(e2, "hipFreeAsync");
+    HIP_TRY(po.finish(stream));
+    HIP_TRY(oo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
+                         const izwi_qmm_weight* down, const float* x, int64_t t,
+                         const int32_t* ids, const float* weights, int32_t top_k,
+                         const int32_t* perm, const int32_t* offsets, float* out, int mem_space,
+                         void* stream_) {
+    if (!gate || !up || !down) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    if (int rc = check_space(mem_space)) return rc;
+    const QmmLayout& G = gate->layout;
+    const QmmLayout& U = up->layout;
+    const QmmLayout& D = down->layout;
+    if (G.dtype != U.dtype || G.n != U.n || G.k != U.k || G.n_stacked != U.n_stacked)
+        return fail(IZWI_QMM_ERR_INVALID, "gate and up stacks differ in shape or dtype");
+    if (D.n_stacked != G.n_stacked || D.k != G.n || D.n != G.k)
+        return fail(IZWI_QMM_ERR_INVALID, "down stack [%lld, %lld] does not match gate/up [%lld, %lld]",
+                    (long long)D.n, (long long)D.k, (long long)G.n, (long long)G.k);
+    if (t < 0 || top_k < 1) return fail(IZWI_QMM_ERR_INVALID, "bad t / top_k");
+    if (t == 0) return IZWI_QMM_OK;
+    if (!x || !ids || !weights || !perm || !offsets || !out)
+        return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    const int64_t pairs = t * top_k;
+    const int n_experts = (int)G.n_stacked;
+    const int64_t hidden = G.k, inter = G.n;
+    // every expert adds at most one partly filled segment
+    const int64_t max_segments = pairs / QMM_MOE_SEG_ROWS + (pairs < n_experts ? pairs : n_experts);
+    if (max_segments > 65535)
+        return fail(IZWI_QMM_ERR_UNSUPPORTED, "t * top_k = %lld is too large for one grouped launch", (long long)pairs);
+    hipStream_t stream = (hipStream_t)stream_;
+    ProfileScope prof(nullptr, stream);
+    Staged xi, ii, wi, pi, oi, oo;
+    HIP_TRY(xi.in(x, (size_t)t * hidden * sizeof(float), mem_space));
+    HIP_TRY(ii.in(ids, (size_t)pairs * sizeof(int32_t), mem_space));
+    HIP_TRY(wi.in(weights, (size_t)pairs * sizeof(float), mem_space));
+    HIP_TRY(pi.in(perm, (size_t)pairs * sizeof(int32_t), mem_space));
+    HIP_TRY(oi.in(offsets, (size_t)(n_experts + 1) * sizeof(int32_t), mem_space));
+    HIP_TRY(oo.out(out, (size_t)t * hidden * sizeof(float), mem_space));
+
+    // workspace: h [pairs, inter] | y [pairs, hidden] | seg_offsets [E + 1]
+    const size_t h_bytes = (size_t)pairs * inter * sizeof(float);
+    const size_t y_bytes = (size_t)pairs * hidden * sizeof(float);
+    const size_t s_bytes = (size_t)(n_experts + 1) * sizeof(int32_t);
+    uint8_t* ws = nullptr;
+    HIP_TRY(hipMallocAsync((void**)&ws, h_bytes + y_bytes + s_bytes, stream));
+    float* h = (float*)ws;
+    float* y = (float*)(ws + h_bytes);
+    int32_t* seg = (int32_t*)(ws + h_bytes + y_bytes);
+    hipError_t e = qmm_launch_moe_segments((const int32_t*)oi.dev, n_experts, seg, stream);
+    if (e == hipSuccess)
+        e = qmm_launch_gemv_grouped(G, gate->tiled, up->tiled, (const float*)xi.dev, top_k, h,
+                                    (const int32_t*)pi.dev, (const int32_t*)oi.dev, seg, n_experts,
+                                    max_segments, gate->n_cus, stream);
+    if (e == hipSuccess)
+        e = qmm_launch_gemv_grouped(D, down->tiled, nullptr, h, 1, y, (const int32_t*)pi.dev,
+                                    (const int32_t*)oi.dev, seg, n_experts, max_segments,
+                                    gate->n_cus, stream);
+    if (e == hipSuccess)
+        e = qmm_launch_moe_combine(y, (const float*)wi.dev, t, top_k, hidden, (float*)oo.dev, stream);
+    hipError_t e2 = hipFreeAsync(ws, stream);
+    if (e != hipSuccess) return fail_hip(e, "grouped expert kernels");
+    if (e2 != hipSuccess) return fail_hip(e2, "hipFreeAsync");
+    if (profiling()) g_silu_fused.fetch_add(1, std::memory_order_relaxed);
+    HIP_TRY(oo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_profile_enable(int enabled) {
+    g_profile.store(enabled ? 1 : 0, std::memory_order_relaxed);
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_profile_snapshot_get(izwi_qmm_profile_snapshot* out) {
+    if (!out) return fail(IZWI_QMM_ERR_INVALID, "out is NULL");
+    out->qmatmul_calls = g_calls.load(std::memory_order_relaxed);
+    out->qmatmul_ns = g_ns.load(std::memory_order_relaxed);
+    out->qmatmul_input_casts = g_in_casts.load(std::memory_order_relaxed);
+    out->qmatmul_input_cast_ns = g_in_cast_ns.load(std::memory_order_relaxed);
+    out->qmatmul_output_casts = g_out_casts.load(std::memory_order_relaxed);
+    out->qmatmul_output_cast_ns = g_out_cast_ns.load(std::memory_order_relaxed);
+    out->lm_head_calls = g_lm_calls.load(std::memory_order_relaxed);
+    out->lm_head_ns = g_lm_ns.load(std::memory_order_relaxed);
+    out->silu_mul_fused_calls = g_silu_fused.load(std::memory_order_relaxed);
+    out->silu_mul_fallback_calls = g_silu_fallback.load(std::memory_order_relaxed);
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_profile_reset(void) {
+    for (auto* c : {&g_calls, &g_ns, &g_in_casts, &g_in_cast_ns, &g_out_casts, &g_out_cast_ns,
+                    &g_lm_calls, &g_lm_ns, &g_silu_fused, &g_silu_fallback})
+        c->store(0, std::memory_order_relaxed);
+    return IZWI_QMM_OK;
+}
+
+} // extern "C"

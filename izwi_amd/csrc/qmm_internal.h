@@ -1,0 +1,112 @@
+// Internal interfaces between the C ABI (qmm_api.hip) and the kernel files.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "qmm_layout.h"
+
+// ---- device helpers --------------------------------------------------------
+#if defined(__HIPCC__)
+
+__device__ __forceinline__ float qmm_f16_bits_to_f32(uint16_t bits) {
+    union {
+        uint16_t u;
+        _Float16 h;
+    } c;
+    c.u = bits;
+    return (float)c.h; // exact
+}
+
+__device__ __forceinline__ uint16_t qmm_f32_to_f16_bits(float f) {
+    union {
+        uint16_t u;
+        _Float16 h;
+    } c;
+    c.h = (_Float16)f; // round to nearest even, as half::f16::from_f32
+    return c.u;
+}
+
+// The 12 scale bytes of a Q4_K block (three little-endian dwords) -> packed
+// 6-bit scales and mins: byte j of sc_lo/sc_hi is scale j / j+4, same for mins.
+__device__ __forceinline__ void qmm_unpack_q4k_scales(uint32_t u0, uint32_t u1, uint32_t u2,
+                                                      uint32_t& sc_lo, uint32_t& sc_hi,
+                                                      uint32_t& mn_lo, uint32_t& mn_hi) {
+    sc_lo = u0 & 0x3f3f3f3fu;
+    mn_lo = u1 & 0x3f3f3f3fu;
+    sc_hi = (u2 & 0x0f0f0f0fu) | (((u0 >> 6) & 0x03030303u) << 4);
+    mn_hi = ((u2 >> 4) & 0x0f0f0f0fu) | (((u1 >> 6) & 0x03030303u) << 4);
+}
+
+__device__ __forceinline__ uint32_t qmm_byte_of(uint32_t lo, uint32_t hi, int j) {
+    return ((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xffu;
+}
+
+__device__ __forceinline__ float qmm_bf16_bits_to_f32(uint16_t b) {
+    return __uint_as_float((uint32_t)b << 16);
+}
+
+// round to nearest even, NaN kept quiet
+__device__ __forceinline__ uint16_t qmm_f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+#endif // __HIPCC__
+
+// ---- launchers -------------------------------------------------------------
+hipError_t qmm_launch_repack(const QmmLayout& L, const void* native, void* tiled,
+                             hipStream_t stream);
+hipError_t qmm_launch_unpack(const QmmLayout& L, const void* tiled, void* native,
+                             hipStream_t stream);
+hipError_t qmm_launch_dequant(const QmmLayout& L, const void* tiled, float* out,
+                              hipStream_t stream);
+
+// Decode kernel: y[m, n] = QMatMul(x[m, k]) for one matrix of the handle.
+// `n_cus` sizes the grid.  Returns hipErrorInvalidValue for shapes it cannot run.
+hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
+                           float* y, int n_cus, hipStream_t stream);
+
+// Activation quantizer written out in the reference's block layout.
+hipError_t qmm_launch_quantize_activations(int weight_dtype, const float* x, int64_t m, int64_t k,
+                                           void* out_blocks, hipStream_t stream);
+
+// Prefill kernel: bf16 activations, bf16 MFMA, f32 accumulate.
+hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uint16_t* x_bf16,
+                                int64_t m, void* y, int out_bf16, int n_cus, hipStream_t stream);
+// f32 activations for m > 64: converted to bf16 into `x_bf16_ws` (m*k elements) first.
+hipError_t qmm_launch_f32_to_bf16(const float* x, uint16_t* out, int64_t count,
+                                  hipStream_t stream);
+
+// ---- MoE ---------------------------------------------------------------------
+// Sorted pairs are processed in segments of this many rows that share one expert.
+#define QMM_MOE_SEG_ROWS 4
+
+hipError_t qmm_launch_moe_route(const float* logits, int64_t t, int n_experts, int top_k,
+                                int32_t* ids, float* weights, hipStream_t stream);
+
+// Stable counting sort of `pairs` expert ids.  `seg_offsets` (n_experts + 1 ints,
+// may be NULL) receives the exclusive prefix sum of ceil(count / QMM_MOE_SEG_ROWS).
+// `scratch` must hold qmm_moe_sort_scratch_ints(pairs, n_experts) ints.
+hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts, int32_t* perm,
+                               int32_t* offsets, int32_t* seg_offsets, int32_t* scratch,
+                               hipStream_t stream);
+int64_t qmm_moe_sort_scratch_ints(int64_t pairs, int n_experts);
+
+// Expert-grouped decode kernel over sorted pairs.  Row i of the sorted list is
+// pair p = perm[i]; its activation row is x[p / x_div], its output row y[p].
+// With `tiled2` the result is silu(W x) * (W2 x).
+hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
+                                   const float* x, int x_div, float* y, const int32_t* perm,
+                                   const int32_t* offsets, const int32_t* seg_offsets,
+                                   int n_experts, int64_t max_segments, int n_cus,
+                                   hipStream_t stream);
+
+// seg_offsets from caller-provided offsets (same definition as in qmm_launch_moe_sort).
+hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int32_t* seg_offsets,
+                                   hipStream_t stream);
+
+// out[t, :] = sum over slots s (in order) of weights[t, s] * y[t * top_k + s, :]
+hipError_t qmm_launch_moe_combine(const float* y, const float* weights, int64_t t, int top_k,
+                                  int64_t hidden, float* out, hipStream_t stream);

@@ -1,0 +1,227 @@
+// Layout conversion (GGUF blocks <-> panel tiles) and bit-exact dequantization.
+// All three are load-time / diagnostic operations bounded by HBM bandwidth;
+// none is on the per-token path.
+#include <hip/hip_runtime.h>
+
+#include "qmm_internal.h"
+
+namespace {
+
+struct Piece {
+    int64_t e, row, unit;
+    int piece;  // 0 = header, 1 + c = quant chunk c
+    bool valid; // false: padding (row >= n or unit >= k_units)
+};
+
+// Decodes the index of a 16-byte piece of the tiled buffer.
+__device__ inline Piece decode_piece(const QmmLayout& L, int64_t idx) {
+    const int64_t pieces_per_panel = (int64_t)L.slots * (1 + L.qc);
+    int64_t panel = idx / pieces_per_panel;
+    int64_t in_panel = idx - panel * pieces_per_panel;
+    Piece p;
+    p.piece = (int)(in_panel / L.slots);
+    int slot = (int)(in_panel - (int64_t)p.piece * L.slots);
+    int64_t kg = panel % L.k_groups;
+    int64_t rt_all = panel / L.k_groups;
+    p.e = rt_all / L.row_tiles;
+    int64_t rt = rt_all - p.e * L.row_tiles;
+    p.row = rt * QMM_PANEL_ROWS + (slot & 15);
+    p.unit = kg * L.s + (slot >> 4);
+    p.valid = p.row < L.n && p.unit < L.k_units;
+    return p;
+}
+
+// Byte offset of a 16-byte piece of (e, row, unit) inside the tiled buffer.
+__device__ inline int64_t piece_offset(const QmmLayout& L, int64_t e, int64_t row, int64_t unit,
+                                       int piece) {
+    int64_t rt = row / QMM_PANEL_ROWS, r = row % QMM_PANEL_ROWS;
+    int64_t kg = unit / L.s, us = unit % L.s;
+    int64_t panel = (e * L.row_tiles + rt) * L.k_groups + kg;
+    return panel * L.panel_bytes + ((int64_t)piece * L.slots + us * 16 + r) * 16;
+}
+
+__global__ void repack_q4k_kernel(QmmLayout L, const uint8_t* __restrict__ src,
+                                  uint8_t* __restrict__ dst, int64_t n_pieces) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_pieces) return;
+    Piece p = decode_piece(L, idx);
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (p.valid) {
+        int64_t blk = (p.e * L.n + p.row) * L.k_units + p.unit;
+        v = *reinterpret_cast<const uint4*>(src + blk * 144 + 16 * p.piece);
+    }
+    *reinterpret_cast<uint4*>(dst + idx * 16) = v;
+}
+
+__global__ void repack_q80_kernel(QmmLayout L, const uint8_t* __restrict__ src,
+                                  uint8_t* __restrict__ dst, int64_t n_pieces) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_pieces) return;
+    Piece p = decode_piece(L, idx);
+    const int64_t blocks_per_row = L.k / 32;
+    union {
+        uint4 v;
+        uint16_t h[8];
+    } u;
+    u.v = make_uint4(0, 0, 0, 0);
+    if (p.valid) {
+        int64_t row_blk = (p.e * L.n + p.row) * blocks_per_row;
+        if (p.piece == 0) {
+            for (int b = 0; b < 8; b++) {
+                int64_t kb = p.unit * 8 + b;
+                if (kb < blocks_per_row)
+                    u.h[b] = *reinterpret_cast<const uint16_t*>(src + (row_blk + kb) * 34);
+            }
+        } else {
+            int c = p.piece - 1;
+            int64_t kb = p.unit * 8 + (c >> 1);
+            if (kb < blocks_per_row) {
+                const uint16_t* s =
+                    reinterpret_cast<const uint16_t*>(src + (row_blk + kb) * 34 + 2 + 16 * (c & 1));
+                for (int i = 0; i < 8; i++) u.h[i] = s[i];
+            }
+        }
+    }
+    *reinterpret_cast<uint4*>(dst + idx * 16) = u.v;
+}
+
+__global__ void unpack_q4k_kernel(QmmLayout L, const uint8_t* __restrict__ tiled,
+                                  uint8_t* __restrict__ dst, int64_t n_chunks) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; // 16-byte chunk of native bytes
+    if (idx >= n_chunks) return;
+    int64_t blk = idx / 9;
+    int piece = (int)(idx - blk * 9);
+    int64_t unit = blk % L.k_units;
+    int64_t row_all = blk / L.k_units;
+    int64_t e = row_all / L.n, row = row_all % L.n;
+    *reinterpret_cast<uint4*>(dst + idx * 16) =
+        *reinterpret_cast<const uint4*>(tiled + piece_offset(L, e, row, unit, piece));
+}
+
+__global__ void unpack_q80_kernel(QmmLayout L, const uint8_t* __restrict__ tiled,
+                                  uint8_t* __restrict__ dst, int64_t n_blocks) {
+    int64_t blk = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; // native 34-byte block
+    if (blk >= n_blocks) return;
+    const int64_t blocks_per_row = L.k / 32;
+    int64_t kb = blk % blocks_per_row;
+    int64_t row_all = blk / blocks_per_row;
+    int64_t e = row_all / L.n, row = row_all % L.n;
+    int64_t unit = kb / 8;
+    int b = (int)(kb % 8);
+    uint16_t* out = reinterpret_cast<uint16_t*>(dst + blk * 34);
+    out[0] = reinterpret_cast<const uint16_t*>(tiled + piece_offset(L, e, row, unit, 0))[b];
+    for (int h = 0; h < 2; h++) {
+        const uint16_t* s =
+            reinterpret_cast<const uint16_t*>(tiled + piece_offset(L, e, row, unit, 1 + 2 * b + h));
+        for (int i = 0; i < 8; i++) out[1 + 8 * h + i] = s[i];
+    }
+}
+
+// One thread per 16-byte quant chunk; f32 products are rounded after each
+// operation (__fmul_rn / __fsub_rn never contract into an FMA).
+__global__ void dequant_q4k_kernel(QmmLayout L, const uint8_t* __restrict__ tiled,
+                                   float* __restrict__ out, int64_t n_chunks) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_chunks) return;
+    int c = (int)(idx & 7);
+    int64_t blk = idx >> 3;
+    int64_t unit = blk % L.k_units;
+    int64_t row_all = blk / L.k_units;
+    int64_t e = row_all / L.n, row = row_all % L.n;
+    uint4 hdr = *reinterpret_cast<const uint4*>(tiled + piece_offset(L, e, row, unit, 0));
+    uint4 qv = *reinterpret_cast<const uint4*>(tiled + piece_offset(L, e, row, unit, 1 + c));
+    float d = qmm_f16_bits_to_f32((uint16_t)(hdr.x & 0xffffu));
+    float dmin = qmm_f16_bits_to_f32((uint16_t)(hdr.x >> 16));
+    uint32_t sc_lo, sc_hi, mn_lo, mn_hi;
+    qmm_unpack_q4k_scales(hdr.y, hdr.z, hdr.w, sc_lo, sc_hi, mn_lo, mn_hi);
+    int g = c >> 1, h = c & 1;
+    int s0 = 2 * g, s1 = 2 * g + 1;
+    float d1 = __fmul_rn(d, (float)qmm_byte_of(sc_lo, sc_hi, s0));
+    float m1 = __fmul_rn(dmin, (float)qmm_byte_of(mn_lo, mn_hi, s0));
+    float d2 = __fmul_rn(d, (float)qmm_byte_of(sc_lo, sc_hi, s1));
+    float m2 = __fmul_rn(dmin, (float)qmm_byte_of(mn_lo, mn_hi, s1));
+    float* o = out + row_all * L.k + unit * 256 + 64 * g + 16 * h;
+    uint32_t w[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            uint32_t byte = (w[j] >> (8 * b)) & 0xffu;
+            o[4 * j + b] = __fsub_rn(__fmul_rn(d1, (float)(byte & 0xF)), m1);
+            o[32 + 4 * j + b] = __fsub_rn(__fmul_rn(d2, (float)(byte >> 4)), m2);
+        }
+    }
+}
+
+__global__ void dequant_q80_kernel(QmmLayout L, const uint8_t* __restrict__ tiled,
+                                   float* __restrict__ out, int64_t n_chunks) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; // 16-byte half block
+    if (idx >= n_chunks) return;
+    const int64_t blocks_per_row = L.k / 32;
+    int h = (int)(idx & 1);
+    int64_t blk = idx >> 1;
+    int64_t kb = blk % blocks_per_row;
+    int64_t row_all = blk / blocks_per_row;
+    int64_t e = row_all / L.n, row = row_all % L.n;
+    int64_t unit = kb / 8;
+    int b = (int)(kb % 8);
+    uint16_t dbits = reinterpret_cast<const uint16_t*>(tiled + piece_offset(L, e, row, unit, 0))[b];
+    float d = qmm_f16_bits_to_f32(dbits);
+    uint4 qv = *reinterpret_cast<const uint4*>(tiled + piece_offset(L, e, row, unit, 1 + 2 * b + h));
+    float* o = out + row_all * L.k + kb * 32 + 16 * h;
+    uint32_t w[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            o[4 * j + i] = __fmul_rn((float)(int8_t)((w[j] >> (8 * i)) & 0xffu), d);
+}
+
+inline unsigned grid_for(int64_t n, int block) { return (unsigned)((n + block - 1) / block); }
+
+} // namespace
+
+hipError_t qmm_launch_repack(const QmmLayout& L, const void* native, void* tiled,
+                             hipStream_t stream) {
+    int64_t n_pieces = L.n_stacked * L.matrix_bytes / 16;
+    if (n_pieces == 0) return hipSuccess;
+    if (L.dtype == QMM_Q4_K)
+        repack_q4k_kernel<<<grid_for(n_pieces, 256), 256, 0, stream>>>(
+            L, (const uint8_t*)native, (uint8_t*)tiled, n_pieces);
+    else
+        repack_q80_kernel<<<grid_for(n_pieces, 256), 256, 0, stream>>>(
+            L, (const uint8_t*)native, (uint8_t*)tiled, n_pieces);
+    return hipGetLastError();
+}
+
+hipError_t qmm_launch_unpack(const QmmLayout& L, const void* tiled, void* native,
+                             hipStream_t stream) {
+    if (L.dtype == QMM_Q4_K) {
+        int64_t n_chunks = L.n_stacked * L.n * L.k_units * 9;
+        if (n_chunks == 0) return hipSuccess;
+        unpack_q4k_kernel<<<grid_for(n_chunks, 256), 256, 0, stream>>>(
+            L, (const uint8_t*)tiled, (uint8_t*)native, n_chunks);
+    } else {
+        int64_t n_blocks = L.n_stacked * L.n * (L.k / 32);
+        if (n_blocks == 0) return hipSuccess;
+        unpack_q80_kernel<<<grid_for(n_blocks, 256), 256, 0, stream>>>(
+            L, (const uint8_t*)tiled, (uint8_t*)native, n_blocks);
+    }
+    return hipGetLastError();
+}
+
+hipError_t qmm_launch_dequant(const QmmLayout& L, const void* tiled, float* out,
+                              hipStream_t stream) {
+    if (L.dtype == QMM_Q4_K) {
+        int64_t n_chunks = L.n_stacked * L.n * L.k_units * 8;
+        if (n_chunks == 0) return hipSuccess;
+        dequant_q4k_kernel<<<grid_for(n_chunks, 256), 256, 0, stream>>>(L, (const uint8_t*)tiled,
+                                                                        out, n_chunks);
+    } else {
+        int64_t n_chunks = L.n_stacked * L.n * (L.k / 32) * 2;
+        if (n_chunks == 0) return hipSuccess;
+        dequant_q80_kernel<<<grid_for(n_chunks, 256), 256, 0, stream>>>(L, (const uint8_t*)tiled,
+                                                                        out, n_chunks);
+    }
+    return hipGetLastError();
+}

@@ -1,0 +1,282 @@
+"""Host-side mirror of the reference's quantized projection interface.
+
+Names and error behaviour follow the reference (izwi-core, qwen3/core.rs, and
+the Candle types it calls): ``QTensor`` carries GGUF block bytes and a 2-D
+shape, ``QMatMul.forward`` multiplies activations by the transposed weight,
+``Qwen3Projection`` adds the activation-dtype policy and
+``packed_qmatmul_from_qtensors`` row-concatenates projections.  torch tensors
+only supply device memory and the current HIP stream; every operation is a
+call into libizwi_qmm.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import enum
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from . import capi
+from .capi import DEVICE, HOST, check, lib
+
+
+class GgmlDType(enum.IntEnum):
+    """candle_core::quantized::GgmlDType, the two block formats of the path."""
+    Q8_0 = 8
+    Q4K = 12
+
+    def block_size(self) -> int:
+        return 32 if self == GgmlDType.Q8_0 else 256
+
+    def type_size(self) -> int:
+        return 34 if self == GgmlDType.Q8_0 else 144
+
+
+def quantized_storage_bytes(rows: int, cols: int, dtype: GgmlDType) -> int:
+    """qwen3/core.rs:891-909: bytes of a [rows, cols] tensor, or an error."""
+    out = C.c_uint64()
+    check(lib().izwi_qmm_storage_bytes(int(dtype), rows, cols, C.byref(out)))
+    return out.value
+
+
+def _stream_ptr(t: torch.Tensor | None = None) -> int:
+    if t is not None and not t.is_cuda:
+        return 0
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _space(t: torch.Tensor) -> int:
+    return DEVICE if t.is_cuda else HOST
+
+
+def _blocks_arg(blocks):
+    """(pointer, nbytes, mem_space, keepalive) for numpy / bytes / torch uint8 input."""
+    if isinstance(blocks, torch.Tensor):
+        if blocks.dtype != torch.uint8 or not blocks.is_contiguous():
+            raise ValueError("block bytes must be a contiguous uint8 tensor")
+        return blocks.data_ptr(), blocks.numel(), _space(blocks), blocks
+    arr = np.ascontiguousarray(np.frombuffer(blocks, dtype=np.uint8) if isinstance(blocks, (bytes, bytearray)) else blocks)
+    if arr.dtype != np.uint8:
+        raise ValueError("block bytes must be uint8")
+    return arr.ctypes.data, arr.size, HOST, arr
+
+
+class QTensor:
+    """candle_core::quantized::QTensor for a [n, k] (or stacked [e, n, k]) weight on the GPU."""
+
+    def __init__(self, handle: int, keep=None):
+        self._h = C.c_void_p(handle)
+        info = capi.WeightInfo()
+        check(lib().izwi_qmm_weight_get_info(self._h, C.byref(info)))
+        self._dtype = GgmlDType(info.ggml_dtype)
+        self._n, self._k, self._e = info.n, info.k, info.n_stacked
+        self._nbytes = info.nbytes
+
+    # -- constructors --------------------------------------------------------
+    @classmethod
+    def from_blocks(cls, dtype: GgmlDType, blocks, shape: Sequence[int]) -> "QTensor":
+        """ggml_file::qtensor_from_ggml(dtype, raw, dims, device): raw GGUF bytes -> tensor."""
+        if len(shape) == 2:
+            e, (n, k) = 1, shape
+        elif len(shape) == 3:
+            e, n, k = shape
+        else:
+            raise capi.QmmError(-1, f"unexpected rank, expected: 2, got: {len(shape)} ({tuple(shape)})")
+        ptr, nbytes, space, keep = _blocks_arg(blocks)
+        h = C.c_void_p()
+        if e == 1 and len(shape) == 2:
+            check(lib().izwi_qmm_weight_create(int(dtype), n, k, ptr, nbytes, space, C.byref(h)))
+        else:
+            check(lib().izwi_qmm_weight_create_stacked(int(dtype), e, n, k, ptr, nbytes, space, C.byref(h)))
+        del keep
+        return cls(h.value)
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            try:
+                lib().izwi_qmm_weight_destroy(h)
+            except Exception:
+                pass
+
+    # -- QTensor accessors ---------------------------------------------------
+    def dtype(self) -> GgmlDType:
+        return self._dtype
+
+    def shape(self):
+        return (self._n, self._k) if self._e == 1 else (self._e, self._n, self._k)
+
+    def dims2(self):
+        if self._e != 1:
+            raise capi.QmmError(-1, f"unexpected rank, expected: 2, got: 3 ({self.shape()})")
+        return self._n, self._k
+
+    def storage_size_in_bytes(self) -> int:
+        return self._nbytes
+
+    def data(self) -> np.ndarray:
+        """QTensor::data(): the GGUF block bytes this tensor was built from."""
+        out = np.empty(self._nbytes, dtype=np.uint8)
+        check(lib().izwi_qmm_weight_data(self._h, out.ctypes.data, out.size, HOST, None))
+        return out
+
+    def dequantize(self, device: str | torch.device = "cuda") -> torch.Tensor:
+        """QTensor::dequantize: f32 tensor, bit-identical to candle-core's to_float."""
+        out = torch.empty((self._e * self._n, self._k), dtype=torch.float32, device=device)
+        check(lib().izwi_qmm_dequantize_f32(self._h, out.data_ptr(), _space(out), _stream_ptr(out)))
+        return out if self._e == 1 else out.view(self._e, self._n, self._k)
+
+
+class QMatMul:
+    """candle_core::quantized::QMatMul (the QTensor arm): ``forward(x) = x @ W^T``."""
+
+    def __init__(self, qtensor: QTensor):
+        self.qtensor = qtensor
+
+    @classmethod
+    def from_qtensor(cls, qtensor: QTensor) -> "QMatMul":
+        qtensor.dims2()
+        return cls(qtensor)
+
+    from_arc = from_qtensor
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        n, k = self.qtensor.dims2()
+        if x.dim() < 1 or x.shape[-1] != k:
+            raise capi.QmmError(-1, f"shape mismatch in qmatmul, lhs: {tuple(x.shape)}, rhs: ({n}, {k})")
+        if not x.is_contiguous():
+            raise capi.QmmError(-1, "qmatmul requires a contiguous input")
+        m = x.numel() // k if k else 0
+        out_shape = tuple(x.shape[:-1]) + (n,)
+        h = self.qtensor._h
+        if x.dtype == torch.float32:
+            y = torch.empty(out_shape, dtype=torch.float32, device=x.device)
+            check(lib().izwi_qmm_forward_f32(h, x.data_ptr(), m, y.data_ptr(), _space(x), _stream_ptr(x)))
+            return y
+        if x.dtype == torch.bfloat16:
+            y = torch.empty(out_shape, dtype=torch.bfloat16, device=x.device)
+            check(lib().izwi_qmm_forward_bf16(h, x.data_ptr(), m, y.data_ptr(), capi.OUT_BF16,
+                                              _space(x), _stream_ptr(x)))
+            return y
+        raise capi.QmmError(-1, f"unsupported dtype {x.dtype} for qmatmul, expected f32 or bf16")
+
+    def forward_bf16_to_f32(self, x: torch.Tensor) -> torch.Tensor:
+        """bf16 activations, f32 result (the MFMA kernel's accumulators, unrounded)."""
+        n, k = self.qtensor.dims2()
+        if x.dtype != torch.bfloat16 or x.shape[-1] != k or not x.is_contiguous():
+            raise capi.QmmError(-1, "expected a contiguous bf16 input with last dim k")
+        y = torch.empty(tuple(x.shape[:-1]) + (n,), dtype=torch.float32, device=x.device)
+        check(lib().izwi_qmm_forward_bf16(self.qtensor._h, x.data_ptr(), x.numel() // k, y.data_ptr(),
+                                          capi.OUT_F32, _space(x), _stream_ptr(x)))
+        return y
+
+
+def packed_qmatmul_from_qtensors(parts: Sequence[tuple]) -> QMatMul:
+    """qwen3/core.rs:846-889 over (dtype, blocks, (rows, cols)) triples: byte-concatenate
+    projections of equal input width and dtype into one QMatMul (fused QKV / gate-up)."""
+    if len(parts) == 0:
+        raise capi.QmmError(-1, "Cannot pack empty Qwen3 quantized projection group")
+    dtype, _, (_, common_cols) = parts[0]
+    rows, ptrs, sizes, keep, spaces = [], [], [], [], set()
+    for dt, blocks, (r, c) in parts:
+        if c != common_cols:
+            raise capi.QmmError(-1, f"Qwen3 quantized projection group input mismatch: expected {common_cols}, got {c}")
+        if dt != dtype:
+            raise capi.QmmError(-1, f"Qwen3 quantized projection group dtype mismatch: expected {dtype!r}, got {dt!r}")
+        ptr, nbytes, space, ka = _blocks_arg(blocks)
+        rows.append(r)
+        ptrs.append(ptr)
+        sizes.append(nbytes)
+        keep.append(ka)
+        spaces.add(space)
+    if len(spaces) != 1:
+        raise ValueError("all parts must live in the same memory space")
+    n = len(parts)
+    h = C.c_void_p()
+    check(lib().izwi_qmm_weight_create_packed(
+        int(dtype), n, (C.c_int64 * n)(*rows), common_cols, (C.c_void_p * n)(*ptrs),
+        (C.c_uint64 * n)(*sizes), spaces.pop(), C.byref(h)))
+    return QMatMul(QTensor(h.value))
+
+
+class Qwen3Projection:
+    """The Quantized arm of izwi-core's Qwen3Projection (qwen3/core.rs:671-832)."""
+
+    def __init__(self, qmatmul: QMatMul, is_lm_head: bool = False):
+        self.qmatmul = qmatmul
+        if is_lm_head:
+            check(lib().izwi_qmm_weight_set_lm_head(qmatmul.qtensor._h, 1))
+
+    @classmethod
+    def quantized(cls, dtype: GgmlDType, blocks, shape, is_lm_head: bool = False) -> "Qwen3Projection":
+        return cls(QMatMul.from_arc(QTensor.from_blocks(dtype, blocks, shape)), is_lm_head)
+
+    @classmethod
+    def packed_quantized(cls, parts) -> "Qwen3Projection":
+        return cls(packed_qmatmul_from_qtensors(parts))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """qwen3/core.rs:791-831.  f32 goes straight to the op.  bf16 prefill-sized
+        inputs use the bf16 kernel (input and output casts fused away); other
+        dtypes are cast to f32 and back as the reference does on accelerators."""
+        if x.dtype == torch.float32:
+            return self.qmatmul.forward(x)
+        k = x.shape[-1]
+        m = x.numel() // k if k else 0
+        if x.dtype == torch.bfloat16 and m > 64:
+            return self.qmatmul.forward(x)
+        return self.qmatmul.forward(x.to(torch.float32)).to(x.dtype)
+
+
+def quantize_activations(weight_dtype: GgmlDType, x: torch.Tensor) -> torch.Tensor:
+    """The activation blocks the decode kernel builds (reference block layout, uint8)."""
+    assert x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2
+    m, k = x.shape
+    per = 34 if weight_dtype == GgmlDType.Q8_0 else 292
+    out = torch.empty(m * (k // weight_dtype.block_size()) * per, dtype=torch.uint8, device=x.device)
+    check(lib().izwi_qmm_quantize_activations(int(weight_dtype), x.data_ptr(), m, k, out.data_ptr(),
+                                              _space(x), _stream_ptr(x)))
+    return out
+
+
+def moe_route(logits: torch.Tensor, top_k: int):
+    assert logits.dtype == torch.float32 and logits.is_contiguous() and logits.dim() == 2
+    t, e = logits.shape
+    ids = torch.empty((t, top_k), dtype=torch.int32, device=logits.device)
+    wts = torch.empty((t, top_k), dtype=torch.float32, device=logits.device)
+    check(lib().izwi_moe_route(logits.data_ptr(), t, e, top_k, ids.data_ptr(), wts.data_ptr(),
+                               _space(logits), _stream_ptr(logits)))
+    return ids, wts
+
+
+def moe_sort(ids: torch.Tensor, n_experts: int):
+    assert ids.dtype == torch.int32 and ids.is_contiguous() and ids.dim() == 2
+    t, top_k = ids.shape
+    perm = torch.empty(t * top_k, dtype=torch.int32, device=ids.device)
+    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=ids.device)
+    check(lib().izwi_moe_sort(ids.data_ptr(), t, top_k, n_experts, perm.data_ptr(), offsets.data_ptr(),
+                              _space(ids), _stream_ptr(ids)))
+    return perm, offsets
+
+
+class MoeExperts:
+    """Expert stacks of one MoE layer: gate/up [e, inter, hidden], down [e, hidden, inter]."""
+
+    def __init__(self, gate: QTensor, up: QTensor, down: QTensor):
+        self.gate, self.up, self.down = gate, up, down
+
+    def forward(self, x, ids, wts, perm, offsets) -> torch.Tensor:
+        assert x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2
+        t = x.shape[0]
+        out = torch.empty_like(x)
+        check(lib().izwi_moe_forward_f32(self.gate._h, self.up._h, self.down._h, x.data_ptr(), t,
+                                         ids.data_ptr(), wts.data_ptr(), ids.shape[1], perm.data_ptr(),
+                                         offsets.data_ptr(), out.data_ptr(), _space(x), _stream_ptr(x)))
+        return out
+
+
+def profile_snapshot() -> dict:
+    snap = capi.ProfileSnapshot()
+    check(lib().izwi_qmm_profile_snapshot_get(C.byref(snap)))
+    return {name: getattr(snap, name) for name, _ in snap._fields_}

@@ -1,0 +1,345 @@
+"""GPU parity tests (pytest -m gpu): the HIP path, called through the C ABI,
+against the CPU oracle on the same seeded inputs.
+
+Bars: weight dequantization, weight bytes, on-chip activation quantization and
+MoE indices are bit-exact; matmul outputs within max|y - y_ref| / max|y_ref|
+<= 1e-2 (the tolerance the path's target states; the decode kernel, which
+follows the reference's integer arithmetic, is held to 1e-4)."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import np_ref
+
+pytestmark = pytest.mark.gpu
+
+Q8_0, Q4_K = 8, 12
+DECODE_TOL = 1e-4
+PREFILL_TOL = 1e-2
+
+
+def _say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def qa():
+    if not torch.cuda.is_available():
+        pytest.fail("no GPU visible: the HIP path cannot run (there is no fallback)")
+    import izwi_amd
+    izwi_amd.lib()
+    torch.cuda.set_device(0)
+    return izwi_amd
+
+
+def rel_err(y, want):
+    return float(np.abs(y.astype(np.float64) - want).max() / max(np.abs(want).max(), 1e-30))
+
+
+def make_weight(oracle, dtype, n, k, seed):
+    w = oracle.randn(seed, (n, k), std=0.02)
+    return oracle.quantize(dtype, w)
+
+
+# ------------------------------------------------------------------ codecs --
+@pytest.mark.parametrize("dtype", [Q8_0, Q4_K])
+@pytest.mark.parametrize("n,k", [(16, 256), (5, 512), (33, 768), (64, 1024), (40, 1280), (128, 4096), (17, 12288)])
+def test_dequantize_and_data_bit_exact(qa, oracle, dtype, n, k):
+    _say(f"dequant dtype={dtype} n={n} k={k}")
+    blocks = make_weight(oracle, dtype, n, k, 1000 + n + k)
+    q = qa.QTensor.from_blocks(qa.GgmlDType(dtype), blocks, (n, k))
+    got = q.dequantize().cpu().numpy()
+    want = oracle.dequantize(dtype, blocks, n, k)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(q.data(), blocks)  # QTensor::data() returns the original bytes
+
+
+def test_dequantize_random_bytes_and_q8_0_ragged_k(qa, oracle):
+    rng = np.random.default_rng(9)
+    raw = rng.integers(0, 256, size=(48 * 5, 144), dtype=np.uint8)
+    raw[:, 1] &= 0x3F
+    raw[:, 3] &= 0x3F
+    q = qa.QTensor.from_blocks(qa.GgmlDType.Q4K, raw.reshape(-1), (48, 1280))
+    assert np.array_equal(q.dequantize().cpu().numpy().view(np.uint32),
+                          np_ref.dequant_q4_k(raw.reshape(-1), 48, 1280).view(np.uint32))
+    # Q8_0 only needs k % 32 == 0: 96 is not a multiple of the 256-element tile unit
+    raw8 = rng.integers(0, 256, size=(20 * 3, 34), dtype=np.uint8)
+    raw8[:, 1] &= 0x7B
+    q8 = qa.QTensor.from_blocks(qa.GgmlDType.Q8_0, raw8.reshape(-1), (20, 96))
+    assert np.array_equal(q8.dequantize().cpu().numpy().view(np.uint32),
+                          np_ref.dequant_q8_0(raw8.reshape(-1), 20, 96).view(np.uint32))
+    assert np.array_equal(q8.data(), raw8.reshape(-1))
+
+
+def test_q4_k_hand_block_on_device(qa):
+    scales = bytes([0x41, 0x82, 0xC3, 0xC4, 0x40, 0x85, 0xCA, 0xCF, 0x41, 0x82, 0xC3, 0xFF])
+    blk = bytes([0x00, 0x3C, 0x00, 0x38]) + scales + bytes(range(128))
+    q = qa.QTensor.from_blocks(qa.GgmlDType.Q4K, blk, (1, 256))
+    y = q.dequantize().cpu().numpy()[0]
+    for i, v in {0: 0, 31: 15, 32: -2.5, 64: -5, 79: 40, 127: 4.5, 160: 116, 224: 346.5, 255: 409.5}.items():
+        assert y[i] == np.float32(v)
+    assert float(y.astype(np.float64).sum()) == 32224.0
+
+
+@pytest.mark.parametrize("dtype", [Q8_0, Q4_K])
+def test_activation_quantizer_bit_exact(qa, oracle, dtype):
+    x = oracle.randn(77, (9, 2048))
+    x[2, 256:512] = 0.0
+    x[4, 5], x[4, 9] = -7.5, 7.5      # equal magnitudes: the first occurrence decides the sign
+    x[5, 700], x[5, 600] = 8.0, -8.0
+    x[6] *= 1e-3
+    x[7] *= 1e4
+    got = qa.quantize_activations(qa.GgmlDType(dtype), torch.from_numpy(x).cuda()).cpu().numpy()
+    want = oracle.quantize_activations(dtype, x)
+    assert np.array_equal(got, want)
+
+
+# ------------------------------------------------------------------ decode --
+def run_forward(qa, dtype, blocks, n, k, x):
+    q = qa.QTensor.from_blocks(qa.GgmlDType(dtype), blocks, (n, k))
+    mm = qa.QMatMul.from_qtensor(q)
+    y = mm.forward(torch.from_numpy(x).cuda())
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def test_config1_q8_0_matvec(qa, oracle):
+    # BASELINE config 1: x [1,1024] ~ N(0,1), W [3072,1024] ~ N(0,0.02) -> Q8_0
+    blocks = make_weight(oracle, Q8_0, 3072, 1024, 1)
+    x = oracle.randn(2, (1, 1024))
+    y = run_forward(qa, Q8_0, blocks, 3072, 1024, x)
+    want = oracle.qmatmul(Q8_0, x, blocks, 3072)
+    assert rel_err(y, want) < DECODE_TOL
+    dense = x.astype(np.float64) @ oracle.dequantize(Q8_0, blocks, 3072, 1024).astype(np.float64).T
+    assert rel_err(y, dense) < 1e-2
+
+
+LAYER_06B = [("q", 2048, 1024), ("k", 1024, 1024), ("o", 1024, 2048), ("gate", 3072, 1024), ("down", 1024, 3072)]
+
+
+@pytest.mark.parametrize("m", [1, 4, 16, 64])
+def test_config2_q8_0_layer(qa, oracle, m):
+    for i, (name, n, k) in enumerate(LAYER_06B):
+        _say(f"config2 {name} m={m}")
+        blocks = make_weight(oracle, Q8_0, n, k, 10 + i)
+        x = oracle.randn(20 + i + m, (m, k))
+        y = run_forward(qa, Q8_0, blocks, n, k, x)
+        assert rel_err(y, oracle.qmatmul(Q8_0, x, blocks, n)) < DECODE_TOL, name
+
+
+SHAPES_8B = [("q", 4096, 4096), ("k", 1024, 4096), ("gate", 12288, 4096), ("down", 4096, 12288)]
+
+
+@pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
+@pytest.mark.parametrize("m", [1, 8, 16])
+def test_config3_8b_shapes(qa, oracle, dtype, m):
+    for i, (name, n, k) in enumerate(SHAPES_8B):
+        _say(f"config3 dtype={dtype} {name} m={m}")
+        blocks = make_weight(oracle, dtype, n, k, 30 + i)
+        x = oracle.randn(40 + i + m, (m, k))
+        y = run_forward(qa, dtype, blocks, n, k, x)
+        assert rel_err(y, oracle.qmatmul(dtype, x, blocks, n)) < DECODE_TOL, name
+
+
+def test_config3_lm_head_full_size(qa, oracle):
+    n, k = 151936, 4096
+    blocks = make_weight(oracle, Q4_K, n, k, 50)
+    x = oracle.randn(51, (1, k))
+    y = run_forward(qa, Q4_K, blocks, n, k, x)
+    assert rel_err(y, oracle.qmatmul(Q4_K, x, blocks, n)) < DECODE_TOL
+
+
+@pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
+@pytest.mark.parametrize("n,k,m", [(1, 256, 1), (15, 256, 2), (17, 512, 3), (100, 768, 5), (250, 1280, 7),
+                                   (33, 2048, 64), (7, 16384, 2), (4100, 256, 1)])
+def test_ragged_shapes(qa, oracle, dtype, n, k, m):
+    _say(f"ragged dtype={dtype} n={n} k={k} m={m}")
+    blocks = make_weight(oracle, dtype, n, k, 60 + n)
+    x = oracle.randn(61 + k, (m, k))
+    y = run_forward(qa, dtype, blocks, n, k, x)
+    assert rel_err(y, oracle.qmatmul(dtype, x, blocks, n)) < DECODE_TOL
+
+
+def test_q8_0_k_not_multiple_of_256(qa, oracle):
+    for k in (32, 96, 352):
+        blocks = make_weight(oracle, Q8_0, 24, k, 70 + k)
+        x = oracle.randn(71, (3, k))
+        y = run_forward(qa, Q8_0, blocks, 24, k, x)
+        assert rel_err(y, oracle.qmatmul(Q8_0, x, blocks, 24)) < DECODE_TOL
+
+
+def test_empty_and_zero_inputs(qa, oracle):
+    blocks = make_weight(oracle, Q4_K, 32, 512, 80)
+    q = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q4K, blocks, (32, 512)))
+    y0 = q.forward(torch.empty((0, 512), device="cuda"))
+    assert tuple(y0.shape) == (0, 32)
+    yz = q.forward(torch.zeros((2, 512), device="cuda")).cpu().numpy()
+    assert not yz.any()
+    # leading dims are flattened: [b, s, k] -> [b, s, n]
+    x = oracle.randn(81, (2, 3, 512))
+    y = q.forward(torch.from_numpy(x).cuda()).cpu().numpy()
+    assert y.shape == (2, 3, 32)
+    assert rel_err(y.reshape(6, 32), oracle.qmatmul(Q4_K, x.reshape(6, 512), blocks, 32)) < DECODE_TOL
+
+
+def test_host_memory_space_matches_device(qa, oracle):
+    blocks = make_weight(oracle, Q8_0, 64, 512, 90)
+    q = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q8_0, blocks, (64, 512)))
+    x = torch.from_numpy(oracle.randn(91, (2, 512)))
+    assert torch.equal(q.forward(x), q.forward(x.cuda()).cpu())
+
+
+def test_shape_and_dtype_errors(qa, oracle):
+    blocks = make_weight(oracle, Q4_K, 32, 512, 92)
+    q = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q4K, blocks, (32, 512)))
+    with pytest.raises(qa.QmmError):
+        q.forward(torch.zeros((2, 256), device="cuda"))
+    with pytest.raises(qa.QmmError):
+        q.forward(torch.zeros((512, 4), device="cuda").t())
+    with pytest.raises(qa.QmmError):
+        q.forward(torch.zeros((2, 512), device="cuda", dtype=torch.float16))
+    with pytest.raises(qa.QmmError):
+        qa.QTensor.from_blocks(qa.GgmlDType.Q4K, blocks[:-1], (32, 512))
+
+
+# ------------------------------------------------------- packed projections --
+def test_packed_qmatmul_matches_separate_q8_0(qa, oracle):
+    # the reference's own test, qwen3/core.rs:3099-3142, plus its known answers
+    w1 = ((np.arange(64, dtype=np.float32) - 31.0) / 8.0).reshape(2, 32)
+    w2 = ((15.0 - np.arange(32, dtype=np.float32)) / 7.0).reshape(1, 32)
+    x = ((np.arange(32, dtype=np.float32) + 1.0) / 16.0).reshape(1, 32)
+    q1, q2 = oracle.quantize(Q8_0, w1), oracle.quantize(Q8_0, w2)
+    dt = qa.GgmlDType.Q8_0
+    packed = qa.packed_qmatmul_from_qtensors([(dt, q1, (2, 32)), (dt, q2, (1, 32))])
+    xg = torch.from_numpy(x).cuda()
+    got = packed.forward(xg).cpu().numpy()
+    sep = np.concatenate([run_forward(qa, Q8_0, q1, 2, 32, x), run_forward(qa, Q8_0, q2, 1, 32, x)], axis=1)
+    assert np.abs(got - sep).max() < 1e-5
+    assert np.allclose(got[0], [-42.692207, 89.229607, -26.613434], rtol=0, atol=1e-5)
+    assert np.array_equal(packed.qtensor.data(), np.concatenate([q1, q2]))
+    with pytest.raises(qa.QmmError, match="input mismatch"):
+        qa.packed_qmatmul_from_qtensors([(dt, q1, (2, 32)), (dt, oracle.quantize(Q8_0, np.zeros((1, 64), np.float32)), (1, 64))])
+    with pytest.raises(qa.QmmError, match="empty"):
+        qa.packed_qmatmul_from_qtensors([])
+
+
+def test_packed_qkv_q4_k_split_offsets(qa, oracle):
+    # fused QKV (qwen3/core.rs:1028-1035): one matmul, then narrow at 0, q, q+k
+    k, nq, nkv = 1024, 512, 128
+    parts = [make_weight(oracle, Q4_K, n, k, 95 + i) for i, n in enumerate((nq, nkv, nkv))]
+    dt = qa.GgmlDType.Q4K
+    proj = qa.Qwen3Projection.packed_quantized([(dt, p, (n, k)) for p, n in zip(parts, (nq, nkv, nkv))])
+    x = oracle.randn(99, (2, k))
+    y = proj.forward(torch.from_numpy(x).cuda()).cpu().numpy()
+    off = 0
+    for p, n in zip(parts, (nq, nkv, nkv)):
+        assert rel_err(y[:, off:off + n], oracle.qmatmul(Q4_K, x, p, n)) < DECODE_TOL
+        off += n
+
+
+def test_projection_dtype_policy(qa, oracle):
+    blocks = make_weight(oracle, Q4_K, 64, 512, 120)
+    proj = qa.Qwen3Projection.quantized(qa.GgmlDType.Q4K, blocks, (64, 512))
+    x = oracle.randn(121, (1, 512))
+    xb = torch.from_numpy(x).cuda().to(torch.bfloat16)
+    y = proj.forward(xb)
+    assert y.dtype == torch.bfloat16  # cast back to the activation dtype, qwen3/core.rs:817-828
+    want = oracle.qmatmul(Q4_K, xb.float().cpu().numpy(), blocks, 64)
+    assert rel_err(y.float().cpu().numpy(), want) < 1e-2
+
+
+# ----------------------------------------------------------------- prefill --
+@pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
+@pytest.mark.parametrize("m,n,k", [(512, 1024, 4096), (300, 200, 768), (64, 256, 256), (1, 16, 512)])
+def test_prefill_bf16_against_oracle(qa, oracle, dtype, m, n, k):
+    _say(f"prefill oracle dtype={dtype} m={m} n={n} k={k}")
+    blocks = make_weight(oracle, dtype, n, k, 130 + n)
+    xb = torch.from_numpy(oracle.randn(131 + m, (m, k))).cuda().to(torch.bfloat16)
+    q = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType(dtype), blocks, (n, k)))
+    y = q.forward_bf16_to_f32(xb).cpu().numpy()
+    want = oracle.qmatmul(dtype, xb.float().cpu().numpy(), blocks, n)
+    assert rel_err(y, want) < PREFILL_TOL
+    yb = q.forward(xb).float().cpu().numpy()
+    assert rel_err(yb, want) < PREFILL_TOL
+
+
+@pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
+@pytest.mark.parametrize("m", [512, 2048])
+def test_config4_prefill_full_shapes_against_fp32(qa, oracle, dtype, m):
+    # full 8B shapes: checked against a plain fp32 matmul of the (bit-exact) dequantized weight
+    for i, (name, n, k) in enumerate(SHAPES_8B):
+        _say(f"config4 dtype={dtype} {name} m={m}")
+        blocks = make_weight(oracle, dtype, n, k, 140 + i)
+        qt = qa.QTensor.from_blocks(qa.GgmlDType(dtype), blocks, (n, k))
+        xb = torch.from_numpy(oracle.randn(150 + i, (m, k))).cuda().to(torch.bfloat16)
+        y = qa.QMatMul.from_qtensor(qt).forward_bf16_to_f32(xb)
+        ref = xb.float() @ qt.dequantize().t()
+        err = float((y - ref).abs().max() / ref.abs().max())
+        assert err < 5e-3, (name, err)
+        del qt, y, ref
+
+
+def test_forward_f32_large_m_uses_prefill_kernel(qa, oracle):
+    blocks = make_weight(oracle, Q4_K, 256, 1024, 160)
+    x = oracle.randn(161, (200, 1024))
+    y = run_forward(qa, Q4_K, blocks, 256, 1024, x)
+    assert rel_err(y, oracle.qmatmul(Q4_K, x, blocks, 256)) < PREFILL_TOL
+
+
+# --------------------------------------------------------------------- MoE --
+@pytest.mark.parametrize("t", [1, 16, 512])
+def test_moe_route_and_sort_bit_exact(qa, oracle, t):
+    logits = oracle.randn(170 + t, (t, 128))
+    if t >= 16:
+        logits[3, 10] = logits[3, 90] = logits[3].max() + 1.0
+        logits[5, :] = 0.25
+    ids, wts = qa.moe_route(torch.from_numpy(logits).cuda(), 8)
+    want_ids, want_wts = oracle.moe_route(logits, 8)
+    assert np.array_equal(ids.cpu().numpy(), want_ids)
+    assert np.allclose(wts.cpu().numpy(), want_wts, rtol=1e-5, atol=1e-7)
+    perm, offsets = qa.moe_sort(ids, 128)
+    want_perm, want_off = oracle.moe_sort(want_ids, 128)
+    assert np.array_equal(perm.cpu().numpy(), want_perm)
+    assert np.array_equal(offsets.cpu().numpy(), want_off)
+
+
+def test_moe_sort_many_pairs(qa, oracle):
+    rng = np.random.default_rng(3)
+    ids = rng.integers(0, 128, size=(5000, 8)).astype(np.int32)
+    perm, offsets = qa.moe_sort(torch.from_numpy(ids).cuda(), 128)
+    want_perm, want_off = oracle.moe_sort(ids, 128)
+    assert np.array_equal(perm.cpu().numpy(), want_perm) and np.array_equal(offsets.cpu().numpy(), want_off)
+
+
+@pytest.fixture(scope="module")
+def moe_weights(oracle):
+    # BASELINE config 5 at full size: 128 experts, hidden 2048, intermediate 768, Q4_K
+    E, hidden, inter = 128, 2048, 768
+    gate = oracle.quantize(Q4_K, oracle.randn(180, (E * inter, hidden), std=0.02))
+    up = oracle.quantize(Q4_K, oracle.randn(181, (E * inter, hidden), std=0.02))
+    down = oracle.quantize(Q4_K, oracle.randn(182, (E * hidden, inter), std=0.02))
+    return E, hidden, inter, gate, up, down
+
+
+@pytest.mark.parametrize("t", [1, 16, 512])
+def test_config5_moe_forward(qa, oracle, moe_weights, t):
+    E, hidden, inter, gate, up, down = moe_weights
+    dt = qa.GgmlDType.Q4K
+    experts = qa.MoeExperts(qa.QTensor.from_blocks(dt, gate, (E, inter, hidden)),
+                            qa.QTensor.from_blocks(dt, up, (E, inter, hidden)),
+                            qa.QTensor.from_blocks(dt, down, (E, hidden, inter)))
+    x = oracle.randn(190 + t, (t, hidden))
+    logits = oracle.randn(191 + t, (t, E))
+    xg = torch.from_numpy(x).cuda()
+    ids, wts = qa.moe_route(torch.from_numpy(logits).cuda(), 8)
+    perm, offsets = qa.moe_sort(ids, E)
+    out = experts.forward(xg, ids, wts, perm, offsets).cpu().numpy()
+    # the oracle is scalar: check every token for small t, a spread of 12 tokens at t = 512
+    rows = np.arange(t) if t <= 16 else np.linspace(0, t - 1, 12).astype(np.int64)
+    want_ids, want_wts = oracle.moe_route(logits, 8)
+    want = oracle.moe_forward(Q4_K, x[rows], want_ids[rows], want_wts[rows], gate, up, down, E, inter)
+    assert rel_err(out[rows], want) < 1e-3
+    assert np.isfinite(out).all()
