@@ -10,6 +10,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "izwi_qmm.h"
@@ -197,6 +198,47 @@ struct Staged {
         return hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost);
     }
 };
+
+// Scratch for kernels that need device memory beyond inputs and outputs (the
+// quantized activations of the batched decode kernel).  One buffer per
+// (device, stream): work on a stream is ordered, so consecutive calls may reuse
+// it; different streams never share.  It only grows; growing frees the old
+// buffer with hipFree, which waits for the device first.  Growth is not
+// possible while the stream is being captured into a graph: run one call of
+// the same size before capturing.
+struct Scratch {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+std::mutex g_scratch_mutex;
+std::unordered_map<uint64_t, Scratch> g_scratch;
+
+hipError_t get_scratch(int device, hipStream_t stream, size_t bytes, void** out) {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    Scratch& s = g_scratch[((uint64_t)(uintptr_t)stream) ^ ((uint64_t)device << 56)];
+    if (s.bytes < bytes) {
+        size_t want = bytes < (1u << 20) ? (1u << 20) : bytes + bytes / 4;
+        void* p = nullptr;
+        hipError_t e = hipMalloc(&p, want);
+        if (e != hipSuccess) return e;
+        if (s.ptr) (void)hipFree(s.ptr);
+        s.ptr = p;
+        s.bytes = want;
+    }
+    *out = s.ptr;
+    return hipSuccess;
+}
+
+// Smallest m that takes the batched (MFMA) decode kernel; below it the fused
+// single-launch kernel runs.  IZWI_QMM_MFMA_MIN_M overrides (tuning knob).
+int mfma_min_m() {
+    static int v = [] {
+        const char* e = getenv("IZWI_QMM_MFMA_MIN_M");
+        int n = e ? atoi(e) : 0;
+        return n > 0 ? n : 3;
+    }();
+    return v;
+}
 
 int check_space(int mem_space) {
     if (mem_space != IZWI_QMM_DEVICE && mem_space != IZWI_QMM_HOST)
@@ -417,8 +459,13 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
     Staged xi, yo;
     HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
     HIP_TRY(yo.out(y, (size_t)m * L.n * sizeof(float), mem_space));
-    if (m <= 64) {
+    if (m < mfma_min_m()) {
         HIP_TRY(qmm_launch_gemv(L, w->tiled, (const float*)xi.dev, m, (float*)yo.dev, w->n_cus, stream));
+    } else if (m <= 64) {
+        void* scratch = nullptr;
+        HIP_TRY(get_scratch(w->device, stream, qmm_gemv_mfma_workspace_bytes(L, m), &scratch));
+        HIP_TRY(qmm_launch_gemv_mfma(L, w->tiled, (const float*)xi.dev, m, (float*)yo.dev, scratch,
+                                     w->n_cus, stream));
     } else {
         // prefill-sized m with f32 activations: convert once, then the MFMA kernel
         void* xb = nullptr;

@@ -68,6 +68,13 @@ hipError_t qmm_launch_dequant(const QmmLayout& L, const void* tiled, float* out,
 hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
                            float* y, int n_cus, hipStream_t stream);
 
+// Batched decode kernel (int8 MFMA) for 3 <= m <= 64.  `workspace` must hold
+// qmm_gemv_mfma_workspace_bytes(L, m) bytes and stay untouched until the work
+// queued on `stream` has run.
+size_t qmm_gemv_mfma_workspace_bytes(const QmmLayout& L, int64_t m);
+hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
+                                float* y, void* workspace, int n_cus, hipStream_t stream);
+
 // Activation quantizer written out in the reference's block layout.
 hipError_t qmm_launch_quantize_activations(int weight_dtype, const float* x, int64_t m, int64_t k,
                                            void* out_blocks, hipStream_t stream);
