@@ -278,7 +278,7 @@ __device__ __forceinline__ void multiply_panel(const Panel<QT>& p, const XLds<QT
                 dlo = dot16(lo1, xq[4 * g + 1], dlo);
                 int dhi = dot16(hi0, xq[4 * g + 2], 0);
                 dhi = dot16(hi1, xq[4 * g + 3], dhi);
-                isum[mi] += sc0 * dlo + sc1 * dhi;
+                isum[mi] += __mul24(sc0, dlo) + __mul24(sc1, dhi); // |dot| < 2^17, scale < 64
             }
         }
         const float d = qmm_f16_bits_to_f32((uint16_t)(p.hdr.x & 0xffffu));
@@ -288,10 +288,11 @@ __device__ __forceinline__ void multiply_panel(const Panel<QT>& p, const XLds<QT
             const int item = mi * k_units + unit;
             const int4* bs = reinterpret_cast<const int4*>(l.xbs + item * 8);
             const int4 b0 = bs[0], b1 = bs[1];
-            int msum = (int)qmm_byte_of(mn_lo, mn_hi, 0) * b0.x + (int)qmm_byte_of(mn_lo, mn_hi, 1) * b0.y +
-                       (int)qmm_byte_of(mn_lo, mn_hi, 2) * b0.z + (int)qmm_byte_of(mn_lo, mn_hi, 3) * b0.w +
-                       (int)qmm_byte_of(mn_lo, mn_hi, 4) * b1.x + (int)qmm_byte_of(mn_lo, mn_hi, 5) * b1.y +
-                       (int)qmm_byte_of(mn_lo, mn_hi, 6) * b1.z + (int)qmm_byte_of(mn_lo, mn_hi, 7) * b1.w;
+            // 24-bit multiplies: mins < 64, |sub-block sums| <= 32 * 128
+            int msum = __mul24((int)qmm_byte_of(mn_lo, mn_hi, 0), b0.x) + __mul24((int)qmm_byte_of(mn_lo, mn_hi, 1), b0.y) +
+                       __mul24((int)qmm_byte_of(mn_lo, mn_hi, 2), b0.z) + __mul24((int)qmm_byte_of(mn_lo, mn_hi, 3), b0.w) +
+                       __mul24((int)qmm_byte_of(mn_lo, mn_hi, 4), b1.x) + __mul24((int)qmm_byte_of(mn_lo, mn_hi, 5), b1.y) +
+                       __mul24((int)qmm_byte_of(mn_lo, mn_hi, 6), b1.z) + __mul24((int)qmm_byte_of(mn_lo, mn_hi, 7), b1.w);
             const float dx = l.xd[item];
             acc[mi] += (d * dx) * (float)isum[mi] - (dmin * dx) * (float)msum;
         }

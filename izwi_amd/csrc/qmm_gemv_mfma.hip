@@ -55,9 +55,12 @@ struct XWs {
     int k_units;
     int n_tiles; // ceil(m / 16)
     __host__ __device__ size_t xq_bytes() const { return (size_t)n_tiles * k_units * kUnitBytes; }
-    // Q4_K: one scale per (unit, row); Q8_0: one per (unit, block, row)
+    // side information per unit, in floats.  Q4_K: 16 row scales, then per row the
+    // eight sub-block sums of the quants split into two int8 planes (sum = 128 * hi + lo).
+    // Q8_0: one scale per (block, row).
+    __host__ __device__ static int xd_per_unit(int qt) { return qt == QMM_Q4_K ? 16 + 64 : 128; }
     __host__ __device__ size_t xd_floats(int qt) const {
-        return (size_t)n_tiles * k_units * 16 * (qt == QMM_Q4_K ? 1 : 8);
+        return (size_t)n_tiles * k_units * xd_per_unit(qt);
     }
 };
 
@@ -105,7 +108,7 @@ __global__ void quantize_ws_kernel(const float* __restrict__ x, int m, int k, XW
             scale_mul = __fdiv_rn(-128.0f, (key & 1) ? -amax : amax);
             d = __fdiv_rn(1.0f, scale_mul);
         }
-        if (j == 0) xd[tu * 16 + mr] = d;
+        if (j == 0) xd[tu * 80 + mr] = d;
     } else {
         // BlockQ8_0::from_float on the lane pair's 32 values
         amax = fmaxf(amax, __int_as_float(dpp<kDppXor1>(__float_as_int(amax))));
@@ -127,6 +130,18 @@ __global__ void quantize_ws_kernel(const float* __restrict__ x, int m, int k, XW
         q[w] = packed;
     }
     const int s = j >> 1, oct = 2 * (j & 1);
+    if (QT == QMM_Q4_K) {
+        int s16 = __builtin_amdgcn_sdot4((int)q[0], 0x01010101, 0, false);
+        s16 = __builtin_amdgcn_sdot4((int)q[1], 0x01010101, s16, false);
+        s16 = __builtin_amdgcn_sdot4((int)q[2], 0x01010101, s16, false);
+        s16 = __builtin_amdgcn_sdot4((int)q[3], 0x01010101, s16, false);
+        const int bsum = s16 + dpp<kDppXor1>(s16); // the sub-block's 32 quants
+        if ((j & 1) == 0) {
+            uint8_t* side = reinterpret_cast<uint8_t*>(xd + tu * 80 + 16) + mr * 16;
+            side[s] = (uint8_t)(bsum & 127);
+            side[8 + s] = (uint8_t)(bsum >> 7);
+        }
+    }
     uint8_t* dst = xq + ((tu * 8 + s) * 4 + oct) * 128 + mr * 8;
     *reinterpret_cast<uint2*>(dst) = make_uint2(q[0], q[1]);
     *reinterpret_cast<uint2*>(dst + 128) = make_uint2(q[2], q[3]);
@@ -163,7 +178,7 @@ __device__ __forceinline__ long pack64(uint32_t lo, uint32_t hi) {
 template <int QT>
 __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_kernel(MfmaParams P) {
     constexpr int QC = QT == QMM_Q4_K ? 8 : 16;
-    constexpr int XD_PER_UNIT = QT == QMM_Q4_K ? 16 : 128; // floats of x scales per unit
+    constexpr int XD_PER_UNIT = QT == QMM_Q4_K ? 80 : 128; // floats of side information per unit
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* lds_xq = smem;                                                        // chunk_units * 4096
     float* lds_xd = reinterpret_cast<float*>(smem + (size_t)P.chunk_units * kUnitBytes); // chunk_units * XD_PER_UNIT
@@ -178,38 +193,56 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_kernel(MfmaParams P)
     const bool rt_ok = rt < P.row_tiles;
     const bool lane_active = lane < P.slots;
 
+    auto load_panel = [&](int kg, u32x4 (&hdr)[4], u32x4 (&q)[QC]) {
+        const bool ok = rt_ok && lane_active;
+        const u32x4* base =
+            reinterpret_cast<const u32x4*>(P.w + (int64_t)(rt * P.k_groups + kg) * P.panel_bytes);
+#pragma unroll
+        for (int c = 0; c < QC; c++)
+            q[c] = ok ? __builtin_nontemporal_load(base + (size_t)(1 + c) * P.slots + lane)
+                      : u32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int u = 0; u < 4; u++) hdr[u] = (rt_ok && u < P.s) ? base[u * 16 + j] : u32x4{0, 0, 0, 0};
+    };
+
     for (int tile = 0; tile < P.n_tiles; tile++) {
         float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         for (int cu0 = 0; cu0 < P.k_units; cu0 += P.chunk_units) {
             const int cu_n = min(P.chunk_units, P.k_units - cu0);
-            // ---- this chunk's quantized activations -> LDS (verbatim copy)
-            __syncthreads();
+            const int kg0 = cu0 / P.s, kg1 = (cu0 + cu_n + P.s - 1) / P.s;
+            // A workgroup barrier also waits for the calling wave's outstanding loads, so
+            // everything this chunk needs is requested before the one barrier that follows:
+            // first the activations (global -> LDS without passing through registers, each
+            // wave moving 1 KiB pieces, 16 B per lane), then the wave's first weight panel
+            // (this lane's (row j, unit grp) header + quants, and the headers of all units
+            // of row j).
+            if (tile != 0 || cu0 != 0) __syncthreads(); // every wave is done reading the previous chunk
             {
                 const u32x4* src = reinterpret_cast<const u32x4*>(
                     P.xq + ((size_t)tile * P.k_units + cu0) * kUnitBytes);
-                u32x4* dst = reinterpret_cast<u32x4*>(lds_xq);
-                for (int i = threadIdx.x; i < cu_n * (kUnitBytes / 16); i += blockDim.x) dst[i] = src[i];
+                const int pieces = cu_n * (kUnitBytes / 1024);
+                const int waves = blockDim.x >> 6;
+                for (int c = wave; c < pieces; c += waves)
+                    __builtin_amdgcn_global_load_lds(
+                        (const __attribute__((address_space(1))) void*)(src + c * 64 + lane),
+                        (__attribute__((address_space(3))) void*)(lds_xq + c * 1024), 16, 0, 0);
+            }
+            u32x4 hdr[4];
+            u32x4 q[QC];
+            bool have_panel = false;
+            if (kg0 + wk < kg1) {
+                load_panel(kg0 + wk, hdr, q);
+                have_panel = true;
+            }
+            {
                 const float* sd = P.xd + ((size_t)tile * P.k_units + cu0) * XD_PER_UNIT;
                 for (int i = threadIdx.x; i < cu_n * XD_PER_UNIT; i += blockDim.x) lds_xd[i] = sd[i];
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the LDS-direct loads have landed
             }
             __syncthreads();
-            const int kg0 = cu0 / P.s, kg1 = (cu0 + cu_n + P.s - 1) / P.s;
             for (int kg = kg0 + wk; kg < kg1; kg += P.nwk) {
-                // ---- panel: this lane's (row j, unit grp) header + quants, headers of all units of row j
-                u32x4 hdr[4];
-                u32x4 q[QC];
-                {
-                    const bool ok = rt_ok && lane_active;
-                    const u32x4* base = reinterpret_cast<const u32x4*>(
-                        P.w + (int64_t)(rt * P.k_groups + kg) * P.panel_bytes);
-#pragma unroll
-                    for (int c = 0; c < QC; c++)
-                        q[c] = ok ? __builtin_nontemporal_load(base + (size_t)(1 + c) * P.slots + lane)
-                                  : u32x4{0, 0, 0, 0};
-#pragma unroll
-                    for (int u = 0; u < 4; u++)
-                        hdr[u] = (rt_ok && u < P.s) ? base[u * 16 + j] : u32x4{0, 0, 0, 0};
-                }
+                if (!have_panel) load_panel(kg, hdr, q);
+                have_panel = false;
                 // ---- (row, unit) per lane -> (row, octet) per lane, for each unit u in register slot u
 #pragma unroll
                 for (int b = 0; b < QC / 2; b++) {
@@ -231,33 +264,45 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_kernel(MfmaParams P)
                     if (QT == QMM_Q4_K) {
                         uint32_t sc_lo, sc_hi, mn_lo, mn_hi;
                         qmm_unpack_q4k_scales(hdr[u].y, hdr[u].z, hdr[u].w, sc_lo, sc_hi, mn_lo, mn_hi);
-                        int isum[4] = {0, 0, 0, 0};
-                        i32x4 macc = {0, 0, 0, 0};
+                        // all eight block-dot MFMAs (and the two of the min term) are issued
+                        // back to back; their results are consumed afterwards, so the matrix
+                        // pipe's latency is paid once per unit, not once per sub-block
+                        i32x4 dd[8];
 #pragma unroll
                         for (int g = 0; g < 4; g++) {
                             const u32x4 qq = q[2 * g + (u >> 1)];
                             const uint32_t w0 = (u & 1) ? qq.z : qq.x, w1 = (u & 1) ? qq.w : qq.y;
-#pragma unroll
-                            for (int half = 0; half < 2; half++) {
-                                const int s = 2 * g + half;
-                                const long bq = half ? pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib)
-                                                     : pack64(w0 & kNib, w1 & kNib);
-                                const long a = *reinterpret_cast<const long*>(xu + s * 512);
-                                i32x4 dd = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, bq, i32x4{0, 0, 0, 0}, 0, 0, 0);
-                                const int sc = (int)qmm_byte_of(sc_lo, sc_hi, s);
-#pragma unroll
-                                for (int r = 0; r < 4; r++) isum[r] += sc * dd[r];
-                                const uint32_t mn = qmm_byte_of(mn_lo, mn_hi, s) * 0x01010101u;
-                                macc = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, pack64(mn, mn), macc, 0, 0, 0);
-                            }
+                            const long a_lo = *reinterpret_cast<const long*>(xu + (2 * g) * 512);
+                            const long a_hi = *reinterpret_cast<const long*>(xu + (2 * g + 1) * 512);
+                            dd[2 * g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(
+                                a_lo, pack64(w0 & kNib, w1 & kNib), i32x4{0, 0, 0, 0}, 0, 0, 0);
+                            dd[2 * g + 1] = __builtin_amdgcn_mfma_i32_16x16x32_i8(
+                                a_hi, pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib), i32x4{0, 0, 0, 0}, 0, 0, 0);
                         }
                         const float d = qmm_f16_bits_to_f32((uint16_t)(hdr[u].x & 0xffffu));
                         const float dmin = qmm_f16_bits_to_f32((uint16_t)(hdr[u].x >> 16));
-                        const float4 dx = *reinterpret_cast<const float4*>(lds_xd + lu * 16 + grp * 4);
+                        // min term: sum_s min_s * bsum_s as two MFMAs over k = sub-block index; only
+                        // the first 16-lane row carries data (k slots 0..7), the rest multiply zeros
+                        const uint8_t* side = reinterpret_cast<const uint8_t*>(lds_xd + lu * 80 + 16) + j * 16;
+                        const long bs_lo = grp == 0 ? *reinterpret_cast<const long*>(side) : 0L;
+                        const long bs_hi = grp == 0 ? *reinterpret_cast<const long*>(side + 8) : 0L;
+                        const long bmn = pack64(mn_lo, mn_hi);
+                        const i32x4 m_lo = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_lo, bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
+                        const i32x4 m_hi = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_hi, bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
+                        const float4 dx = *reinterpret_cast<const float4*>(lds_xd + lu * 80 + grp * 4);
                         const float dxs[4] = {dx.x, dx.y, dx.z, dx.w};
+                        int isum[4] = {0, 0, 0, 0};
 #pragma unroll
-                        for (int r = 0; r < 4; r++)
-                            acc[r] += (d * dxs[r]) * (float)isum[r] - (dmin * dxs[r]) * (float)macc[r];
+                        for (int s8 = 0; s8 < 8; s8++) {
+                            const int sc = (int)qmm_byte_of(sc_lo, sc_hi, s8);
+#pragma unroll
+                            for (int r = 0; r < 4; r++) isum[r] += __mul24(sc, dd[s8][r]); // |dd| < 2^17, sc < 64
+                        }
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            const int msum = m_lo[r] + (m_hi[r] << 7);
+                            acc[r] += (d * dxs[r]) * (float)isum[r] - (dmin * dxs[r]) * (float)msum;
+                        }
                     } else {
                         const uint32_t hw[4] = {hdr[u].x, hdr[u].y, hdr[u].z, hdr[u].w};
 #pragma unroll
@@ -358,7 +403,7 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     P.nwr = nwr;
     P.wave_magic = (65536 + nwk - 1) / nwk;
     const int waves = nwk * nwr;
-    const int xd_per_unit = L.dtype == QMM_Q4_K ? 16 : 128;
+    const int xd_per_unit = XWs::xd_per_unit(L.dtype);
     size_t lds = (size_t)P.chunk_units * kUnitBytes + (size_t)P.chunk_units * xd_per_unit * 4 +
                  (size_t)waves * 256 * 4;
     const void* fn = L.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_kernel<QMM_Q4_K>)
