@@ -1,16 +1,19 @@
 // Prefill kernel: y[m, n] = x[m, k] * dequant(W)[n, k]^T with bf16 MFMA.
 //
-// A workgroup (4 waves, 2 x 2) owns a 256 x 256 output tile; each wave a
-// 128 x 128 sub-tile held as 4 x 4 v_mfma_f32_32x32x16_bf16 accumulators
-// (256 f32 registers).  Per 64-wide k step the workgroup
-//   * copies the 256 x 64 bf16 activation tile to LDS,
-//   * reads the matching 64 k-elements of 256 weight rows straight from the
-//     panel layout (header + two nibble chunks for Q4_K, header + four int8
-//     chunks for Q8_0), dequantizes them in registers and writes bf16 to LDS,
-//   * runs 4 k16 steps of 16 MFMAs per wave, operands read from LDS as one
+// A workgroup (4 waves, 2 x 2) owns a BM x BN output tile (256 x 256 when the
+// problem fills the chip with such tiles, smaller tiles otherwise); each wave
+// a (BM/2) x (BN/2) sub-tile held in v_mfma_f32_32x32x16_bf16 accumulators.
+// Per 64-wide k step the workgroup
+//   * copies the BM x 64 bf16 activation tile to LDS,
+//   * reads the matching 64 k-elements of BN weight rows straight from the
+//     panel layout (header + nibble / int8 chunks), dequantizes them in
+//     registers and writes bf16 to LDS,
+//   * runs 4 k16 steps of MFMAs per wave, operands read from LDS as one
 //     16-byte load per lane (row stride padded to 144 B: conflict free).
-// Global loads of the next k step are issued before the MFMAs of the current
-// one, so HBM/L2 latency hides behind the matrix work.
+// LDS holds two such stages: while the MFMAs of step i run out of one, the
+// tile of step i+1 (loaded to registers during step i-1) is dequantized into
+// the other and the global loads of step i+2 are issued, with one barrier per
+// step.
 #include <hip/hip_runtime.h>
 
 #include "qmm_internal.h"
@@ -21,7 +24,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int BK = 64;
 constexpr int kThreads = 256;
 constexpr int kRowStride = 144; // bytes per LDS tile row: 64 bf16 + 16 B pad
 
@@ -37,25 +40,30 @@ struct GemmParams {
 };
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-    return (uint32_t)qmm_f32_to_bf16_bits(a) | ((uint32_t)qmm_f32_to_bf16_bits(b) << 16);
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    bf16x2 v = {(__bf16)a, (__bf16)b}; // v_cvt_pk_bf16_f32: round to nearest even
+    return __builtin_bit_cast(uint32_t, v);
 }
 
-template <int QT>
+// Quant chunks a thread holds for its share of one weight row and k step.
+template <int QT, int TPR>
 struct WRegs {
-    static constexpr int NC = QT == QMM_Q4_K ? 2 : 4;
+    static constexpr int NC = (QT == QMM_Q4_K ? 2 : 4) / TPR;
     u32x4 hdr;
     u32x4 q[NC];
 };
 
-// Weight row `row` (global), k step kt (64 elements): header + its quant chunks.
-template <int QT>
-__device__ __forceinline__ void load_w(WRegs<QT>& r, const GemmParams& P, int64_t row, int kt) {
-    const int unit = kt >> 2, part = kt & 3;
+// Weight row `row`, k step kt (64 elements), part `part` of TPR: header + chunks.
+template <int QT, int TPR>
+__device__ __forceinline__ void load_w(WRegs<QT, TPR>& r, const GemmParams& P, int64_t row, int kt,
+                                       int part) {
+    constexpr int NC = WRegs<QT, TPR>::NC;
+    const int unit = kt >> 2, sub = kt & 3;
     const int64_t rt = row >> 4;
     if (rt >= P.row_tiles || unit >= P.k_units) {
         r.hdr = u32x4{0, 0, 0, 0};
 #pragma unroll
-        for (int c = 0; c < WRegs<QT>::NC; c++) r.q[c] = u32x4{0, 0, 0, 0};
+        for (int c = 0; c < NC; c++) r.q[c] = u32x4{0, 0, 0, 0};
         return;
     }
     const int kg = unit / P.s, us = unit - kg * P.s;
@@ -64,14 +72,14 @@ __device__ __forceinline__ void load_w(WRegs<QT>& r, const GemmParams& P, int64_
         reinterpret_cast<const u32x4*>(P.w + (rt * P.k_groups + kg) * P.panel_bytes) + slot;
     r.hdr = base[0];
 #pragma unroll
-    for (int c = 0; c < WRegs<QT>::NC; c++)
-        r.q[c] = base[(size_t)(1 + part * WRegs<QT>::NC + c) * P.slots];
+    for (int c = 0; c < NC; c++)
+        r.q[c] = base[(size_t)(1 + sub * NC * TPR + part * NC + c) * P.slots];
 }
 
-// Dequantizes the 64 k-elements held in r to bf16 and writes one LDS tile row.
-template <int QT>
-__device__ __forceinline__ void store_w(const WRegs<QT>& r, int kt, uint8_t* lds_row) {
-    uint32_t out[32];
+// Dequantizes the thread's share of the 64 k-elements to bf16 and writes it to the LDS row.
+template <int QT, int TPR>
+__device__ __forceinline__ void store_w(const WRegs<QT, TPR>& r, int kt, int part, uint8_t* lds_row) {
+    constexpr int NC = WRegs<QT, TPR>::NC;
     if (QT == QMM_Q4_K) {
         const int g = kt & 3;
         const float d = qmm_f16_bits_to_f32((uint16_t)(r.hdr.x & 0xffffu));
@@ -83,80 +91,92 @@ __device__ __forceinline__ void store_w(const WRegs<QT>& r, int kt, uint8_t* lds
         const float d2 = d * (float)qmm_byte_of(sc_lo, sc_hi, 2 * g + 1);
         const float m2 = dmin * (float)qmm_byte_of(mn_lo, mn_hi, 2 * g + 1);
 #pragma unroll
-        for (int c = 0; c < 2; c++) {
+        for (int c = 0; c < NC; c++) {
+            const int h = part * NC + c; // which 16-byte half of the 32 nibble bytes
+            uint32_t lo[8], hi[8];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                uint32_t v = r.q[c][j];
-                float lo[4], hi[4];
+                const uint32_t v = r.q[c][j];
+                float fl[4], fh[4];
 #pragma unroll
                 for (int b = 0; b < 4; b++) {
-                    uint32_t byte = (v >> (8 * b)) & 0xffu;
-                    lo[b] = d1 * (float)(byte & 0xF) - m1;
-                    hi[b] = d2 * (float)(byte >> 4) - m2;
+                    const uint32_t byte = (v >> (8 * b)) & 0xffu;
+                    fl[b] = d1 * (float)(byte & 0xF) - m1;
+                    fh[b] = d2 * (float)(byte >> 4) - m2;
                 }
-                // low nibbles: k 16c + 4j .., high nibbles: k 32 + 16c + 4j ..
-                out[8 * c + 2 * j] = pack_bf16(lo[0], lo[1]);
-                out[8 * c + 2 * j + 1] = pack_bf16(lo[2], lo[3]);
-                out[16 + 8 * c + 2 * j] = pack_bf16(hi[0], hi[1]);
-                out[16 + 8 * c + 2 * j + 1] = pack_bf16(hi[2], hi[3]);
+                lo[2 * j] = pack_bf16(fl[0], fl[1]);
+                lo[2 * j + 1] = pack_bf16(fl[2], fl[3]);
+                hi[2 * j] = pack_bf16(fh[0], fh[1]);
+                hi[2 * j + 1] = pack_bf16(fh[2], fh[3]);
             }
+            // low nibbles: k 16h .. 16h+15, high nibbles: k 32 + 16h ..
+            uint4* dl = reinterpret_cast<uint4*>(lds_row + 32 * h);
+            uint4* dh = reinterpret_cast<uint4*>(lds_row + 64 + 32 * h);
+            dl[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+            dl[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+            dh[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+            dh[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
         }
     } else {
-        const int b0 = (kt & 3) * 2; // first of the two 32-element blocks
+        const int b0 = (kt & 3) * 2; // first of the two 32-element blocks of this k step
         const uint32_t hw[4] = {r.hdr.x, r.hdr.y, r.hdr.z, r.hdr.w};
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const int b = b0 + (c >> 1);
+        for (int c = 0; c < NC; c++) {
+            const int cc = part * NC + c; // chunk 0..3 of the step: block cc / 2, half cc % 2
+            const int b = b0 + (cc >> 1);
             const float d = qmm_f16_bits_to_f32((uint16_t)((hw[b >> 1] >> (16 * (b & 1))) & 0xffffu));
+            uint32_t o[8];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                uint32_t v = r.q[c][j];
+                const uint32_t v = r.q[c][j];
                 float f[4];
 #pragma unroll
                 for (int i = 0; i < 4; i++) f[i] = (float)(int8_t)((v >> (8 * i)) & 0xffu) * d;
-                out[8 * c + 2 * j] = pack_bf16(f[0], f[1]);
-                out[8 * c + 2 * j + 1] = pack_bf16(f[2], f[3]);
+                o[2 * j] = pack_bf16(f[0], f[1]);
+                o[2 * j + 1] = pack_bf16(f[2], f[3]);
             }
+            uint4* dst = reinterpret_cast<uint4*>(lds_row + 32 * cc);
+            dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+            dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
         }
     }
-    uint4* dst = reinterpret_cast<uint4*>(lds_row);
-#pragma unroll
-    for (int i = 0; i < 8; i++)
-        dst[i] = make_uint4(out[4 * i], out[4 * i + 1], out[4 * i + 2], out[4 * i + 3]);
 }
 
-template <int QT>
+template <int QT, int BM, int BN>
 __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams P) {
+    constexpr int MT = BM / 64, NT = BN / 64; // 32x32 MFMA tiles per wave in m and n
+    constexpr int XC = BM / 32;               // 16-byte activation chunks per thread and k step
+    constexpr int TPR = kThreads / BN;        // threads sharing one weight row
+    constexpr int kStage = (BM + BN) * kRowStride;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    uint8_t* xs = smem;
-    uint8_t* ws = smem + BM * kRowStride;
 
     // consecutive workgroups walk down m inside one weight column block, so the
-    // 256 weight rows they share stay in L2 while all of m is swept
+    // weight rows they share stay in L2 while all of m is swept
     const int tm = blockIdx.x % P.tiles_m;
     const int tn = blockIdx.x / P.tiles_m;
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int k_steps = P.k_units * 4;
+    const int w_row = tid % BN, w_part = tid / BN;
 
-    f32x16 acc[4][4];
+    f32x16 acc[MT][NT];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < MT; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < NT; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    // activation tile: 256 rows x 8 chunks of 16 B; thread t copies chunks t + 256 i
-    u32x4 xr[8];
-    WRegs<QT> wr;
+    // activation tile: BM rows x 8 chunks of 16 B; thread t copies chunks t + 256 i
+    u32x4 xr[XC];
+    WRegs<QT, TPR> wr;
     auto load_x = [&](int kt) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            int c = tid + kThreads * i;
-            int row = c >> 3, kc = c & 7;
-            int64_t gm = m0 + row, gk = (int64_t)kt * BK + kc * 8;
+        for (int i = 0; i < XC; i++) {
+            const int c = tid + kThreads * i;
+            const int row = c >> 3, kc = c & 7;
+            const int64_t gm = m0 + row, gk = (int64_t)kt * BK + kc * 8;
             if (gm < P.m && gk + 8 <= P.k) {
                 xr[i] = *reinterpret_cast<const u32x4*>(P.x + gm * P.k + gk);
             } else {
@@ -172,56 +192,66 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams P) {
             }
         }
     };
-    auto store_x = [&]() {
+    auto store_tile = [&](int kt, uint8_t* stage) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            int c = tid + kThreads * i;
-            int row = c >> 3, kc = c & 7;
-            *reinterpret_cast<u32x4*>(xs + row * kRowStride + kc * 16) = xr[i];
+        for (int i = 0; i < XC; i++) {
+            const int c = tid + kThreads * i;
+            const int row = c >> 3, kc = c & 7;
+            *reinterpret_cast<u32x4*>(stage + row * kRowStride + kc * 16) = xr[i];
         }
+        store_w<QT, TPR>(wr, kt, w_part, stage + (BM + w_row) * kRowStride);
+    };
+    auto load_tile = [&](int kt) {
+        load_x(kt);
+        load_w<QT, TPR>(wr, P, n0 + w_row, kt, w_part);
     };
 
-    load_x(0);
-    load_w<QT>(wr, P, n0 + tid, 0);
+    load_tile(0);
+    store_tile(0, smem);
+    if (k_steps > 1) load_tile(1);
+    __syncthreads();
 
     for (int kt = 0; kt < k_steps; kt++) {
-        store_x();
-        store_w<QT>(wr, kt, ws + tid * kRowStride);
-        __syncthreads();
-        if (kt + 1 < k_steps) {
-            load_x(kt + 1);
-            load_w<QT>(wr, P, n0 + tid, kt + 1);
-        }
+        const uint8_t* xs = smem + (kt & 1) * kStage;
+        const uint8_t* ws = xs + BM * kRowStride;
+        uint8_t* next = smem + ((kt + 1) & 1) * kStage;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
             const int koff = kk * 32 + (lane >> 5) * 16; // bytes inside the tile row
-            bf16x8 a[4], b[4];
+            bf16x8 a[MT], b[NT];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
+            for (int i = 0; i < MT; i++)
                 a[i] = *reinterpret_cast<const bf16x8*>(
-                    xs + (wm * 128 + i * 32 + (lane & 31)) * kRowStride + koff);
-                b[i] = *reinterpret_cast<const bf16x8*>(
-                    ws + (wn * 128 + i * 32 + (lane & 31)) * kRowStride + koff);
-            }
+                    xs + (wm * (BM / 2) + i * 32 + (lane & 31)) * kRowStride + koff);
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+            for (int j = 0; j < NT; j++)
+                b[j] = *reinterpret_cast<const bf16x8*>(
+                    ws + (wn * (BN / 2) + j * 32 + (lane & 31)) * kRowStride + koff);
 #pragma unroll
-                for (int j = 0; j < 4; j++)
+            for (int i = 0; i < MT; i++)
+#pragma unroll
+                for (int j = 0; j < NT; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+            if (kk == 0 && kt + 1 < k_steps) {
+                // next step's tile (in registers since the previous step) goes to the other
+                // stage while this step's MFMAs run; then the loads of the step after are issued
+                store_tile(kt + 1, next);
+                if (kt + 2 < k_steps) load_tile(kt + 2);
+            }
         }
         __syncthreads();
     }
 
     // D[i][j]: lane holds column j = lane % 32 and rows 8*(r/4) + 4*(lane/32) + r%4
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < MT; i++) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int64_t gn = n0 + wn * 128 + j * 32 + (lane & 31);
+        for (int j = 0; j < NT; j++) {
+            const int64_t gn = n0 + wn * (BN / 2) + j * 32 + (lane & 31);
             if (gn >= P.n) continue;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int64_t gm = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                const int64_t gm = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 if (gm >= P.m) continue;
                 if (P.out_bf16)
                     reinterpret_cast<uint16_t*>(P.y)[gm * P.n + gn] = qmm_f32_to_bf16_bits(acc[i][j][r]);
@@ -246,11 +276,36 @@ __global__ void f32_to_bf16_kernel(const float* __restrict__ x, uint16_t* __rest
     }
 }
 
+template <int QT, int BM, int BN>
+hipError_t launch_tile(GemmParams P, hipStream_t stream) {
+    P.tiles_m = (int)((P.m + BM - 1) / BM);
+    P.tiles_n = (int)((P.n + BN - 1) / BN);
+    const int64_t grid = (int64_t)P.tiles_m * P.tiles_n;
+    if (grid > 0x7fffffff) return hipErrorInvalidValue;
+    const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
+    const void* fn = reinterpret_cast<const void*>(&gemm_kernel<QT, BM, BN>);
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    gemm_kernel<QT, BM, BN><<<dim3((unsigned)grid), dim3(kThreads), lds, stream>>>(P);
+    return hipGetLastError();
+}
+
+// Largest tile whose grid still covers every CU at least once (big tiles reuse
+// each LDS byte most, but a grid smaller than the chip leaves CUs idle).
+template <int QT>
+hipError_t launch_qt(const GemmParams& P, int n_cus, hipStream_t stream) {
+    auto tiles = [&](int bm, int bn) { return ((P.m + bm - 1) / bm) * ((P.n + bn - 1) / bn); };
+    if (tiles(256, 256) >= n_cus) return launch_tile<QT, 256, 256>(P, stream);
+    if (tiles(128, 256) >= n_cus) return launch_tile<QT, 128, 256>(P, stream);
+    return launch_tile<QT, 128, 128>(P, stream);
+}
+
 } // namespace
 
 hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uint16_t* x_bf16,
                                 int64_t m, void* y, int out_bf16, int n_cus, hipStream_t stream) {
-    (void)n_cus;
     if (m <= 0 || L.n == 0) return hipSuccess;
     GemmParams P;
     P.w = (const uint8_t*)tiled;
@@ -266,20 +321,9 @@ hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uin
     P.row_tiles = L.row_tiles;
     P.panel_bytes = L.panel_bytes;
     P.out_bf16 = out_bf16;
-    P.tiles_m = (int)((m + BM - 1) / BM);
-    P.tiles_n = (int)((L.n + BN - 1) / BN);
-    int64_t grid = (int64_t)P.tiles_m * P.tiles_n;
-    if (grid > 0x7fffffff) return hipErrorInvalidValue;
-    const size_t lds = (size_t)(BM + BN) * kRowStride;
-    const void* fn = L.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemm_kernel<QMM_Q4_K>)
-                                         : reinterpret_cast<const void*>(&gemm_kernel<QMM_Q8_0>);
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    if (L.dtype == QMM_Q4_K)
-        gemm_kernel<QMM_Q4_K><<<dim3((unsigned)grid), dim3(kThreads), lds, stream>>>(P);
-    else
-        gemm_kernel<QMM_Q8_0><<<dim3((unsigned)grid), dim3(kThreads), lds, stream>>>(P);
-    return hipGetLastError();
+    P.tiles_m = P.tiles_n = 0;
+    return L.dtype == QMM_Q4_K ? launch_qt<QMM_Q4_K>(P, n_cus, stream)
+                               : launch_qt<QMM_Q8_0>(P, n_cus, stream);
 }
 
 hipError_t qmm_launch_f32_to_bf16(const float* x, uint16_t* out, int64_t count,
