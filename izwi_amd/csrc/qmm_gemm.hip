@@ -16,6 +16,8 @@
 // step.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "qmm_internal.h"
 
 namespace {
@@ -45,6 +47,12 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
     return __builtin_bit_cast(uint32_t, v);
 }
 
+// byte N of v as float (v_cvt_f32_ubyteN)
+template <int N>
+__device__ __forceinline__ float ubyte_f32(uint32_t v) {
+    return (float)((v >> (8 * N)) & 0xffu);
+}
+
 // Quant chunks a thread holds for its share of one weight row and k step.
 template <int QT, int TPR>
 struct WRegs {
@@ -59,27 +67,45 @@ __device__ __forceinline__ void load_w(WRegs<QT, TPR>& r, const GemmParams& P, i
                                        int part) {
     constexpr int NC = WRegs<QT, TPR>::NC;
     const int unit = kt >> 2, sub = kt & 3;
-    const int64_t rt = row >> 4;
-    if (rt >= P.row_tiles || unit >= P.k_units) {
-        r.hdr = u32x4{0, 0, 0, 0};
-#pragma unroll
-        for (int c = 0; c < NC; c++) r.q[c] = u32x4{0, 0, 0, 0};
-        return;
-    }
-    const int kg = unit / P.s, us = unit - kg * P.s;
+    // branch-free: out-of-range rows / units read a valid address and are zeroed by a select
+    // when the tile is written to LDS, so the k loop stays one basic block and loads, LDS
+    // traffic and MFMAs can interleave
+    const bool ok = (row >> 4) < P.row_tiles && unit < P.k_units;
+    const int64_t rt = ok ? (row >> 4) : 0;
+    const int u = ok ? unit : 0;
+    const int kg = u / P.s, us = u - kg * P.s;
     const int slot = us * 16 + (int)(row & 15);
     const u32x4* base =
         reinterpret_cast<const u32x4*>(P.w + (rt * P.k_groups + kg) * P.panel_bytes) + slot;
+    // (the select itself happens in store_w: applying it here would make every load wait)
     r.hdr = base[0];
 #pragma unroll
-    for (int c = 0; c < NC; c++)
-        r.q[c] = base[(size_t)(1 + sub * NC * TPR + part * NC + c) * P.slots];
+    for (int c = 0; c < NC; c++) r.q[c] = base[(size_t)(1 + sub * NC * TPR + part * NC + c) * P.slots];
 }
 
 // Dequantizes the thread's share of the 64 k-elements to bf16 and writes it to the LDS row.
 template <int QT, int TPR>
-__device__ __forceinline__ void store_w(const WRegs<QT, TPR>& r, int kt, int part, uint8_t* lds_row) {
+__device__ __forceinline__ void store_w(const WRegs<QT, TPR>& r, int kt, int part, bool ok,
+                                        uint8_t* lds_row) {
     constexpr int NC = WRegs<QT, TPR>::NC;
+    if (!ok) { // row or unit outside the matrix: zeros (uniform per wave except at the ragged edge)
+        const uint4 z = make_uint4(0, 0, 0, 0);
+        uint4* dst = reinterpret_cast<uint4*>(lds_row);
+        if (QT == QMM_Q4_K) {
+#pragma unroll
+            for (int c = 0; c < NC; c++) {
+                const int h = part * NC + c;
+                dst[2 * h] = z, dst[2 * h + 1] = z, dst[4 + 2 * h] = z, dst[4 + 2 * h + 1] = z;
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < NC; c++) dst[2 * (part * NC + c)] = z, dst[2 * (part * NC + c) + 1] = z;
+        }
+        return;
+    }
+    // This kernel's results are compared within a tolerance (bf16 operands), so the
+    // dequantization may use fused multiply-adds and per-byte converts:
+    // 1 convert + 1 fma + half a pack per weight.
     if (QT == QMM_Q4_K) {
         const int g = kt & 3;
         const float d = qmm_f16_bits_to_f32((uint16_t)(r.hdr.x & 0xffffu));
@@ -87,27 +113,24 @@ __device__ __forceinline__ void store_w(const WRegs<QT, TPR>& r, int kt, int par
         uint32_t sc_lo, sc_hi, mn_lo, mn_hi;
         qmm_unpack_q4k_scales(r.hdr.y, r.hdr.z, r.hdr.w, sc_lo, sc_hi, mn_lo, mn_hi);
         const float d1 = d * (float)qmm_byte_of(sc_lo, sc_hi, 2 * g);
-        const float m1 = dmin * (float)qmm_byte_of(mn_lo, mn_hi, 2 * g);
+        const float m1 = -(dmin * (float)qmm_byte_of(mn_lo, mn_hi, 2 * g));
         const float d2 = d * (float)qmm_byte_of(sc_lo, sc_hi, 2 * g + 1);
-        const float m2 = dmin * (float)qmm_byte_of(mn_lo, mn_hi, 2 * g + 1);
+        const float m2 = -(dmin * (float)qmm_byte_of(mn_lo, mn_hi, 2 * g + 1));
 #pragma unroll
         for (int c = 0; c < NC; c++) {
             const int h = part * NC + c; // which 16-byte half of the 32 nibble bytes
             uint32_t lo[8], hi[8];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const uint32_t v = r.q[c][j];
-                float fl[4], fh[4];
-#pragma unroll
-                for (int b = 0; b < 4; b++) {
-                    const uint32_t byte = (v >> (8 * b)) & 0xffu;
-                    fl[b] = d1 * (float)(byte & 0xF) - m1;
-                    fh[b] = d2 * (float)(byte >> 4) - m2;
-                }
-                lo[2 * j] = pack_bf16(fl[0], fl[1]);
-                lo[2 * j + 1] = pack_bf16(fl[2], fl[3]);
-                hi[2 * j] = pack_bf16(fh[0], fh[1]);
-                hi[2 * j + 1] = pack_bf16(fh[2], fh[3]);
+                const uint32_t vl = r.q[c][j] & 0x0f0f0f0fu, vh = (r.q[c][j] >> 4) & 0x0f0f0f0fu;
+                lo[2 * j] = pack_bf16(__builtin_fmaf(d1, ubyte_f32<0>(vl), m1),
+                                      __builtin_fmaf(d1, ubyte_f32<1>(vl), m1));
+                lo[2 * j + 1] = pack_bf16(__builtin_fmaf(d1, ubyte_f32<2>(vl), m1),
+                                          __builtin_fmaf(d1, ubyte_f32<3>(vl), m1));
+                hi[2 * j] = pack_bf16(__builtin_fmaf(d2, ubyte_f32<0>(vh), m2),
+                                      __builtin_fmaf(d2, ubyte_f32<1>(vh), m2));
+                hi[2 * j + 1] = pack_bf16(__builtin_fmaf(d2, ubyte_f32<2>(vh), m2),
+                                          __builtin_fmaf(d2, ubyte_f32<3>(vh), m2));
             }
             // low nibbles: k 16h .. 16h+15, high nibbles: k 32 + 16h ..
             uint4* dl = reinterpret_cast<uint4*>(lds_row + 32 * h);
@@ -125,15 +148,15 @@ __device__ __forceinline__ void store_w(const WRegs<QT, TPR>& r, int kt, int par
             const int cc = part * NC + c; // chunk 0..3 of the step: block cc / 2, half cc % 2
             const int b = b0 + (cc >> 1);
             const float d = qmm_f16_bits_to_f32((uint16_t)((hw[b >> 1] >> (16 * (b & 1))) & 0xffffu));
+            const float bias = -128.0f * d; // int8 q as unsigned byte u = q + 128: q * d = u * d - 128 d
             uint32_t o[8];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const uint32_t v = r.q[c][j];
-                float f[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) f[i] = (float)(int8_t)((v >> (8 * i)) & 0xffu) * d;
-                o[2 * j] = pack_bf16(f[0], f[1]);
-                o[2 * j + 1] = pack_bf16(f[2], f[3]);
+                const uint32_t u = r.q[c][j] ^ 0x80808080u;
+                o[2 * j] = pack_bf16(__builtin_fmaf(d, ubyte_f32<0>(u), bias),
+                                     __builtin_fmaf(d, ubyte_f32<1>(u), bias));
+                o[2 * j + 1] = pack_bf16(__builtin_fmaf(d, ubyte_f32<2>(u), bias),
+                                         __builtin_fmaf(d, ubyte_f32<3>(u), bias));
             }
             uint4* dst = reinterpret_cast<uint4*>(lds_row + 32 * cc);
             dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
@@ -171,25 +194,16 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams P) {
     // activation tile: BM rows x 8 chunks of 16 B; thread t copies chunks t + 256 i
     u32x4 xr[XC];
     WRegs<QT, TPR> wr;
+    // rows past m read row m-1 (their results are never stored); k is a multiple of 32, so a
+    // 16-byte chunk is entirely inside or outside [0, k): outside chunks become zeros
     auto load_x = [&](int kt) {
 #pragma unroll
         for (int i = 0; i < XC; i++) {
             const int c = tid + kThreads * i;
             const int row = c >> 3, kc = c & 7;
-            const int64_t gm = m0 + row, gk = (int64_t)kt * BK + kc * 8;
-            if (gm < P.m && gk + 8 <= P.k) {
-                xr[i] = *reinterpret_cast<const u32x4*>(P.x + gm * P.k + gk);
-            } else {
-                union {
-                    u32x4 v;
-                    uint16_t h[8];
-                } u;
-                u.v = u32x4{0, 0, 0, 0};
-                if (gm < P.m)
-                    for (int e = 0; e < 8; e++)
-                        if (gk + e < P.k) u.h[e] = P.x[gm * P.k + gk + e];
-                xr[i] = u.v;
-            }
+            const int64_t gm = min(m0 + row, P.m - 1);
+            const int64_t gk = (int64_t)kt * BK + kc * 8;
+            xr[i] = *reinterpret_cast<const u32x4*>(P.x + gm * P.k + (gk < P.k ? gk : 0));
         }
     };
     auto store_tile = [&](int kt, uint8_t* stage) {
@@ -197,9 +211,11 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams P) {
         for (int i = 0; i < XC; i++) {
             const int c = tid + kThreads * i;
             const int row = c >> 3, kc = c & 7;
-            *reinterpret_cast<u32x4*>(stage + row * kRowStride + kc * 16) = xr[i];
+            const bool ok = (int64_t)kt * BK + kc * 8 < P.k;
+            *reinterpret_cast<u32x4*>(stage + row * kRowStride + kc * 16) = ok ? xr[i] : u32x4{0, 0, 0, 0};
         }
-        store_w<QT, TPR>(wr, kt, w_part, stage + (BM + w_row) * kRowStride);
+        const bool w_ok = ((n0 + w_row) >> 4) < P.row_tiles && (kt >> 2) < P.k_units;
+        store_w<QT, TPR>(wr, kt, w_part, w_ok, stage + (BM + w_row) * kRowStride);
     };
     auto load_tile = [&](int kt) {
         load_x(kt);
@@ -211,10 +227,14 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams P) {
     if (k_steps > 1) load_tile(1);
     __syncthreads();
 
-    for (int kt = 0; kt < k_steps; kt++) {
-        const uint8_t* xs = smem + (kt & 1) * kStage;
-        const uint8_t* ws = xs + BM * kRowStride;
-        uint8_t* next = smem + ((kt + 1) & 1) * kStage;
+    // One k step: MFMAs out of `cur`; with FEED, the next step's tile (in registers since the
+    // previous step) is dequantized into `next` and the loads of the step after are issued.
+    // No branch inside, so the whole step is one basic block and the scheduler is free to
+    // interleave LDS traffic, dequantization and global loads with the MFMAs.
+    auto k_step = [&](int kt, const uint8_t* cur, uint8_t* next, auto feed) {
+        constexpr bool FEED = decltype(feed)::value;
+        const uint8_t* xs = cur;
+        const uint8_t* ws = cur + BM * kRowStride;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
             const int koff = kk * 32 + (lane >> 5) * 16; // bytes inside the tile row
@@ -232,15 +252,16 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams P) {
 #pragma unroll
                 for (int j = 0; j < NT; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
-            if (kk == 0 && kt + 1 < k_steps) {
-                // next step's tile (in registers since the previous step) goes to the other
-                // stage while this step's MFMAs run; then the loads of the step after are issued
+            if (FEED && kk == 0) {
                 store_tile(kt + 1, next);
-                if (kt + 2 < k_steps) load_tile(kt + 2);
+                load_tile(kt + 2); // past the end this reads a valid address and yields zeros
             }
         }
         __syncthreads();
-    }
+    };
+    for (int kt = 0; kt + 1 < k_steps; kt++)
+        k_step(kt, smem + (kt & 1) * kStage, smem + ((kt + 1) & 1) * kStage, std::true_type{});
+    k_step(k_steps - 1, smem + ((k_steps - 1) & 1) * kStage, nullptr, std::false_type{});
 
     // D[i][j]: lane holds column j = lane % 32 and rows 8*(r/4) + 4*(lane/32) + r%4
 #pragma unroll
