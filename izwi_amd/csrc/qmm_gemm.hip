@@ -17,6 +17,7 @@
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
+#include <utility>
 
 #include "qmm_internal.h"
 
@@ -88,28 +89,14 @@ template <int QT, int TPR>
 __device__ __forceinline__ void store_w(const WRegs<QT, TPR>& r, int kt, int part, bool ok,
                                         uint8_t* lds_row) {
     constexpr int NC = WRegs<QT, TPR>::NC;
-    if (!ok) { // row or unit outside the matrix: zeros (uniform per wave except at the ragged edge)
-        const uint4 z = make_uint4(0, 0, 0, 0);
-        uint4* dst = reinterpret_cast<uint4*>(lds_row);
-        if (QT == QMM_Q4_K) {
-#pragma unroll
-            for (int c = 0; c < NC; c++) {
-                const int h = part * NC + c;
-                dst[2 * h] = z, dst[2 * h + 1] = z, dst[4 + 2 * h] = z, dst[4 + 2 * h + 1] = z;
-            }
-        } else {
-#pragma unroll
-            for (int c = 0; c < NC; c++) dst[2 * (part * NC + c)] = z, dst[2 * (part * NC + c) + 1] = z;
-        }
-        return;
-    }
     // This kernel's results are compared within a tolerance (bf16 operands), so the
     // dequantization may use fused multiply-adds and per-byte converts:
     // 1 convert + 1 fma + half a pack per weight.
     if (QT == QMM_Q4_K) {
         const int g = kt & 3;
-        const float d = qmm_f16_bits_to_f32((uint16_t)(r.hdr.x & 0xffffu));
-        const float dmin = qmm_f16_bits_to_f32((uint16_t)(r.hdr.x >> 16));
+        // a row or unit outside the matrix gets zero scales: every weight becomes 0, no branch
+        const float d = ok ? qmm_f16_bits_to_f32((uint16_t)(r.hdr.x & 0xffffu)) : 0.0f;
+        const float dmin = ok ? qmm_f16_bits_to_f32((uint16_t)(r.hdr.x >> 16)) : 0.0f;
         uint32_t sc_lo, sc_hi, mn_lo, mn_hi;
         qmm_unpack_q4k_scales(r.hdr.y, r.hdr.z, r.hdr.w, sc_lo, sc_hi, mn_lo, mn_hi);
         const float d1 = d * (float)qmm_byte_of(sc_lo, sc_hi, 2 * g);
@@ -147,7 +134,8 @@ __device__ __forceinline__ void store_w(const WRegs<QT, TPR>& r, int kt, int par
         for (int c = 0; c < NC; c++) {
             const int cc = part * NC + c; // chunk 0..3 of the step: block cc / 2, half cc % 2
             const int b = b0 + (cc >> 1);
-            const float d = qmm_f16_bits_to_f32((uint16_t)((hw[b >> 1] >> (16 * (b & 1))) & 0xffffu));
+            const float d =
+                ok ? qmm_f16_bits_to_f32((uint16_t)((hw[b >> 1] >> (16 * (b & 1))) & 0xffffu)) : 0.0f;
             const float bias = -128.0f * d; // int8 q as unsigned byte u = q + 128: q * d = u * d - 128 d
             uint32_t o[8];
 #pragma unroll
@@ -257,6 +245,18 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams P) {
                 load_tile(kt + 2); // past the end this reads a valid address and yields zeros
             }
         }
+#ifdef QMM_GEMM_SCHED
+        if (FEED) {
+#pragma unroll
+            for (int i = 0; i < MT * NT * 4; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x002, QMM_GEMM_SCHED, 0); // VALU
+                if (i % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
+                if (i % 4 == 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); // DS write
+                if (i % 5 == 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
+            }
+        }
+#endif
         __syncthreads();
     };
     for (int kt = 0; kt + 1 < k_steps; kt++)
@@ -264,6 +264,222 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams P) {
     k_step(k_steps - 1, smem + ((k_steps - 1) & 1) * kStage, nullptr, std::false_type{});
 
     // D[i][j]: lane holds column j = lane % 32 and rows 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+    for (int i = 0; i < MT; i++) {
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            const int64_t gn = n0 + wn * (BN / 2) + j * 32 + (lane & 31);
+            if (gn >= P.n) continue;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int64_t gm = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (gm >= P.m) continue;
+                if (P.out_bf16)
+                    reinterpret_cast<uint16_t*>(P.y)[gm * P.n + gn] = qmm_f32_to_bf16_bits(acc[i][j][r]);
+                else
+                    reinterpret_cast<float*>(P.y)[gm * P.n + gn] = acc[i][j][r];
+            }
+        }
+    }
+}
+
+// ---- software-pipelined variant (BN = 256: one weight row per thread) ----------------
+// With one wave per SIMD nothing hides a wave's own non-matrix work, so the next tile's
+// staging (dequantization, LDS writes, global loads) is cut into slices and one slice
+// is placed after every group of four MFMAs; scheduling fences keep the slices there.
+// The MFMA pipe then drains its queue while the VALU / LDS / memory slices issue.
+template <int N, class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl<N>(f, std::make_integer_sequence<int, N>{});
+}
+
+template <int QT, int BM>
+__global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
+    constexpr int BN = 256;
+    constexpr int MT = BM / 64, NT = BN / 64;
+    constexpr int XC = BM / 32;
+    constexpr int NC = QT == QMM_Q4_K ? 2 : 4;
+    constexpr int GPK = MT * NT / 4; // groups of four MFMAs per k16 step
+    constexpr int NG = 4 * GPK;      // groups per k step: 16 (BM = 256) or 8 (BM = 128)
+    constexpr int kStage = (BM + BN) * kRowStride;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    const int tm = blockIdx.x % P.tiles_m;
+    const int tn = blockIdx.x / P.tiles_m;
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int k_steps = P.k_units * 4;
+
+    f32x16 acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < NT; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    // ---- staging state: tile kt+1 sits in xr / wr while step kt runs
+    u32x4 xr[XC];
+    WRegs<QT, 1> wr;
+    const uint16_t* x_src[XC]; // row base + chunk offset of each activation chunk
+    int x_lds[XC];
+#pragma unroll
+    for (int i = 0; i < XC; i++) {
+        const int c = tid + kThreads * i;
+        const int row = c >> 3, kc = c & 7;
+        x_src[i] = P.x + min(m0 + row, P.m - 1) * P.k + kc * 8;
+        x_lds[i] = row * kRowStride + kc * 16;
+    }
+    const int64_t w_row = n0 + tid;
+    const bool w_row_ok = (w_row >> 4) < P.row_tiles;
+    const int w_lds = (BM + tid) * kRowStride;
+
+    auto x_load = [&](int kt, int i) {
+        const int64_t gk = (int64_t)kt * BK;
+        // chunks at or past k read chunk 0 of the row; x_write turns them into zeros
+        xr[i] = *reinterpret_cast<const u32x4*>(x_src[i] + (gk + (tid & 7) * 8 < P.k ? gk : -(int64_t)((tid & 7) * 8)));
+    };
+    auto x_write = [&](int kt, int i, uint8_t* stage) {
+        const bool ok = (int64_t)kt * BK + (tid & 7) * 8 < P.k;
+        *reinterpret_cast<u32x4*>(stage + x_lds[i]) = ok ? xr[i] : u32x4{0, 0, 0, 0};
+    };
+    auto w_base = [&](int kt) -> const u32x4* {
+        const int unit = kt >> 2;
+        const bool ok = w_row_ok && unit < P.k_units;
+        const int u = ok ? unit : 0;
+        const int kg = u / P.s, us = u - kg * P.s;
+        return reinterpret_cast<const u32x4*>(P.w + ((ok ? (w_row >> 4) : 0) * P.k_groups + kg) * P.panel_bytes) +
+               us * 16 + (int)(w_row & 15);
+    };
+    // scales of the tile being staged
+    float sa = 0, ba = 0, sb = 0, bb = 0; // Q4_K: (d1, -m1, d2, -m2); Q8_0: (dA, -128 dA, dB, -128 dB)
+    auto w_scales = [&](int kt) {
+        const bool ok = w_row_ok && (kt >> 2) < P.k_units;
+        if (QT == QMM_Q4_K) {
+            const int g = kt & 3;
+            const float d = ok ? qmm_f16_bits_to_f32((uint16_t)(wr.hdr.x & 0xffffu)) : 0.0f;
+            const float dmin = ok ? qmm_f16_bits_to_f32((uint16_t)(wr.hdr.x >> 16)) : 0.0f;
+            uint32_t sc_lo, sc_hi, mn_lo, mn_hi;
+            qmm_unpack_q4k_scales(wr.hdr.y, wr.hdr.z, wr.hdr.w, sc_lo, sc_hi, mn_lo, mn_hi);
+            sa = d * (float)qmm_byte_of(sc_lo, sc_hi, 2 * g);
+            ba = -(dmin * (float)qmm_byte_of(mn_lo, mn_hi, 2 * g));
+            sb = d * (float)qmm_byte_of(sc_lo, sc_hi, 2 * g + 1);
+            bb = -(dmin * (float)qmm_byte_of(mn_lo, mn_hi, 2 * g + 1));
+        } else {
+            const int b0 = (kt & 3) * 2;
+            const uint32_t hw[4] = {wr.hdr.x, wr.hdr.y, wr.hdr.z, wr.hdr.w};
+            const uint32_t pair = hw[b0 >> 1]; // blocks b0 (low half) and b0 + 1 (high half)
+            sa = ok ? qmm_f16_bits_to_f32((uint16_t)(pair & 0xffffu)) : 0.0f;
+            sb = ok ? qmm_f16_bits_to_f32((uint16_t)(pair >> 16)) : 0.0f;
+            ba = -128.0f * sa;
+            bb = -128.0f * sb;
+        }
+    };
+    uint32_t stash[8]; // finished bf16 pairs waiting for their 16-byte LDS write
+    // slice S of 8: one eighth of the thread's 64 weights, converted and (every other slice) written
+    auto w_slice = [&](auto S, uint8_t* stage) {
+        constexpr int sidx = decltype(S)::value;
+        uint8_t* row = stage + w_lds;
+        if (QT == QMM_Q4_K) {
+            constexpr int c = sidx / 4, j = sidx % 4; // chunk (16-byte half h = c), dword j
+            const uint32_t v = wr.q[c][j];
+            const uint32_t vl = v & 0x0f0f0f0fu, vh = (v >> 4) & 0x0f0f0f0fu;
+            constexpr int o = (j & 1) * 2;
+            stash[o] = pack_bf16(__builtin_fmaf(sa, ubyte_f32<0>(vl), ba), __builtin_fmaf(sa, ubyte_f32<1>(vl), ba));
+            stash[o + 1] = pack_bf16(__builtin_fmaf(sa, ubyte_f32<2>(vl), ba), __builtin_fmaf(sa, ubyte_f32<3>(vl), ba));
+            stash[4 + o] = pack_bf16(__builtin_fmaf(sb, ubyte_f32<0>(vh), bb), __builtin_fmaf(sb, ubyte_f32<1>(vh), bb));
+            stash[4 + o + 1] = pack_bf16(__builtin_fmaf(sb, ubyte_f32<2>(vh), bb), __builtin_fmaf(sb, ubyte_f32<3>(vh), bb));
+            if (j & 1) { // low nibbles: k 16c + 8 (j/2) .., high nibbles: k 32 + 16c + 8 (j/2) ..
+                *reinterpret_cast<uint4*>(row + 32 * c + 16 * (j >> 1)) = make_uint4(stash[0], stash[1], stash[2], stash[3]);
+                *reinterpret_cast<uint4*>(row + 64 + 32 * c + 16 * (j >> 1)) = make_uint4(stash[4], stash[5], stash[6], stash[7]);
+            }
+        } else {
+            constexpr int c = sidx / 2, jj = (sidx % 2) * 2; // chunk c: block c / 2, dwords jj, jj + 1
+            const float d = (c >> 1) ? sb : sa, bias = (c >> 1) ? bb : ba;
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const uint32_t u = wr.q[c][jj + t] ^ 0x80808080u;
+                stash[2 * t] = pack_bf16(__builtin_fmaf(d, ubyte_f32<0>(u), bias), __builtin_fmaf(d, ubyte_f32<1>(u), bias));
+                stash[2 * t + 1] = pack_bf16(__builtin_fmaf(d, ubyte_f32<2>(u), bias), __builtin_fmaf(d, ubyte_f32<3>(u), bias));
+            }
+            *reinterpret_cast<uint4*>(row + 32 * c + 16 * (sidx % 2)) = make_uint4(stash[0], stash[1], stash[2], stash[3]);
+        }
+    };
+    auto w_load_hdr = [&](int kt) { wr.hdr = w_base(kt)[0]; };
+    auto w_load_q = [&](int kt, int c) { wr.q[c] = w_base(kt)[(size_t)(1 + (kt & 3) * NC + c) * P.slots]; };
+
+    // ---- prologue: tile 0 -> stage 0, tile 1 -> registers
+#pragma unroll
+    for (int i = 0; i < XC; i++) x_load(0, i);
+    w_load_hdr(0);
+#pragma unroll
+    for (int c = 0; c < NC; c++) w_load_q(0, c);
+#pragma unroll
+    for (int i = 0; i < XC; i++) x_write(0, i, smem);
+    w_scales(0);
+    static_for<8>([&](auto S) { w_slice(S, smem); });
+#pragma unroll
+    for (int i = 0; i < XC; i++) x_load(1, i);
+    w_load_hdr(1);
+#pragma unroll
+    for (int c = 0; c < NC; c++) w_load_q(1, c);
+    __syncthreads();
+
+    auto k_step = [&](int kt, const uint8_t* cur, uint8_t* next, auto feed) {
+        constexpr bool FEED = decltype(feed)::value;
+        const uint8_t* xs = cur + (wm * (BM / 2) + (lane & 31)) * kRowStride + (lane >> 5) * 16;
+        const uint8_t* ws = cur + (BM + wn * (BN / 2) + (lane & 31)) * kRowStride + (lane >> 5) * 16;
+        bf16x8 fa[2][MT], fb[2][NT];
+        auto read_frags = [&](int kk, int set) {
+#pragma unroll
+            for (int i = 0; i < MT; i++)
+                fa[set][i] = *reinterpret_cast<const bf16x8*>(xs + i * 32 * kRowStride + kk * 32);
+#pragma unroll
+            for (int j = 0; j < NT; j++)
+                fb[set][j] = *reinterpret_cast<const bf16x8*>(ws + j * 32 * kRowStride + kk * 32);
+        };
+        read_frags(0, 0);
+        static_for<4>([&](auto KK) {
+            constexpr int kk = decltype(KK)::value;
+            if (kk < 3) read_frags(kk + 1, (kk + 1) & 1);
+            static_for<GPK>([&](auto GI) {
+                constexpr int gi = decltype(GI)::value;
+                constexpr int g = kk * GPK + gi;
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int t = gi * 4 + q, i = t / NT, j = t % NT;
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kk & 1][i], fb[kk & 1][j], acc[i][j], 0, 0, 0);
+                }
+                if (FEED) {
+                    // group g's share of staging tile kt+1 and fetching tile kt+2
+                    constexpr int s0 = NG == 16 ? 1 : 0; // first group that runs a weight slice
+                    if (g == 0) w_scales(kt + 1);
+                    if (g < XC) x_write(kt + 1, g, next);
+                    if (g >= s0 && g < s0 + 8) w_slice(std::integral_constant<int, (g >= s0 && g < s0 + 8) ? g - s0 : 0>{}, next);
+                    if (g >= 2 && g < 2 + XC) x_load(kt + 2, g - 2);
+                    if (NG == 16) {
+                        if (g == 10) w_load_hdr(kt + 2);
+                        if (g >= 11 && g < 11 + NC) w_load_q(kt + 2, g - 11);
+                    } else if (g == NG - 1) {
+                        w_load_hdr(kt + 2);
+#pragma unroll
+                        for (int c = 0; c < NC; c++) w_load_q(kt + 2, c);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        });
+        __syncthreads();
+    };
+    for (int kt = 0; kt + 1 < k_steps; kt++)
+        k_step(kt, smem + (kt & 1) * kStage, smem + ((kt + 1) & 1) * kStage, std::true_type{});
+    k_step(k_steps - 1, smem + ((k_steps - 1) & 1) * kStage, nullptr, std::false_type{});
+
 #pragma unroll
     for (int i = 0; i < MT; i++) {
 #pragma unroll
@@ -304,12 +520,17 @@ hipError_t launch_tile(GemmParams P, hipStream_t stream) {
     const int64_t grid = (int64_t)P.tiles_m * P.tiles_n;
     if (grid > 0x7fffffff) return hipErrorInvalidValue;
     const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
-    const void* fn = reinterpret_cast<const void*>(&gemm_kernel<QT, BM, BN>);
+    const void* fn;
+    if constexpr (BN == 256) fn = reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM>);
+    else fn = reinterpret_cast<const void*>(&gemm_kernel<QT, BM, BN>);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
     }
-    gemm_kernel<QT, BM, BN><<<dim3((unsigned)grid), dim3(kThreads), lds, stream>>>(P);
+    if constexpr (BN == 256)
+        gemm_pipe_kernel<QT, BM><<<dim3((unsigned)grid), dim3(kThreads), lds, stream>>>(P);
+    else
+        gemm_kernel<QT, BM, BN><<<dim3((unsigned)grid), dim3(kThreads), lds, stream>>>(P);
     return hipGetLastError();
 }
 
