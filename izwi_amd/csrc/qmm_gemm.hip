@@ -470,6 +470,18 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
 #pragma unroll
                         for (int c = 0; c < NC; c++) w_load_q(kt + 2, c);
                     }
+                    if (BM == 256) {
+                        // inside the group: one MFMA, then a few of the slice's VALU ops, so the
+                        // matrix pipe is fed while the slice issues
+#pragma unroll
+                        for (int q = 0; q < 4; q++) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+                            if (q == 1) __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
+                            if (q == 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                            if (q == 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                        }
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
@@ -534,13 +546,19 @@ hipError_t launch_tile(GemmParams P, hipStream_t stream) {
     return hipGetLastError();
 }
 
-// Largest tile whose grid still covers every CU at least once (big tiles reuse
-// each LDS byte most, but a grid smaller than the chip leaves CUs idle).
+// Tile choice: big tiles reuse each LDS byte most, but the grid runs in rounds of one
+// workgroup per CU and a partly filled last round idles CUs.  Score = fraction of CU
+// slots doing work x relative efficiency of the tile (measured on the 8B shapes).
 template <int QT>
 hipError_t launch_qt(const GemmParams& P, int n_cus, hipStream_t stream) {
-    auto tiles = [&](int bm, int bn) { return ((P.m + bm - 1) / bm) * ((P.n + bn - 1) / bn); };
-    if (tiles(256, 256) >= n_cus) return launch_tile<QT, 256, 256>(P, stream);
-    if (tiles(128, 256) >= n_cus) return launch_tile<QT, 128, 256>(P, stream);
+    auto score = [&](int bm, int bn, double quality) {
+        const int64_t tiles = ((P.m + bm - 1) / bm) * ((P.n + bn - 1) / bn);
+        const int64_t rounds = (tiles + n_cus - 1) / n_cus;
+        return quality * (double)tiles / (double)(rounds * n_cus);
+    };
+    const double s256 = score(256, 256, 1.0), s128 = score(128, 256, 0.72), s64 = score(128, 128, 0.4);
+    if (s256 >= s128 && s256 >= s64) return launch_tile<QT, 256, 256>(P, stream);
+    if (s128 >= s64) return launch_tile<QT, 128, 256>(P, stream);
     return launch_tile<QT, 128, 128>(P, stream);
 }
 
