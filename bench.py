@@ -143,7 +143,7 @@ def cpu_baseline(oracle, dtype, m, budget_s=12.0):
             oracle.qmatmul(dtype, x, b, n)
         passes += 1
         dt = time.perf_counter() - t0
-        if dt > budget_s or passes >= 200:
+        if dt > budget_s:
             break
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     return {
@@ -157,17 +157,47 @@ def cpu_baseline(oracle, dtype, m, budget_s=12.0):
     }
 
 
-def prefill_extra(torch, qa, oracle, dtype, m, steps=10, warmup=3):
-    """TFLOP/s of the prefill kernel per projection (extra report, not `value`)."""
+def prefill_extra(torch, qa, oracle, dtype, m, steps=20, warmup=5):
+    """TFLOP/s of the prefill kernel per projection (extra report, not `value`):
+    bf16 activations in HBM, bf16 output, called through the C ABI on preallocated buffers."""
+    from izwi_amd import capi
+    from izwi_amd.qmatmul import _stream_ptr
+    L = capi.lib()
     out = {}
     gg = qa.GgmlDType(dtype)
     for i, (name, n, k) in enumerate([LAYER_8B[0], LAYER_8B[1], LAYER_8B[4], LAYER_8B[6]]):
         mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, make_blocks(oracle, dtype, n, k, 1000 + i, 4096), (n, k)))
         x = torch.from_numpy(oracle.randn(3, (m, k))).cuda().to(torch.bfloat16)
-        ms = time_eager(torch, lambda: mm.forward(x), steps, warmup)
+        y = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+        sp = _stream_ptr()
+
+        def call():
+            rc = L.izwi_qmm_forward_bf16(mm.qtensor._h, x.data_ptr(), m, y.data_ptr(), capi.OUT_BF16, capi.DEVICE, sp)
+            if rc:
+                capi.check(rc)
+
+        ms = time_eager(torch, call, steps, warmup)
         out[name] = round(2.0 * m * n * k / (ms * 1e-3) / 1e12, 2)
-        del mm
+        del mm, x, y
     return out
+
+
+def measured_traffic(workload, m, avg_algorithmic):
+    """HBM bytes per launch of the decode kernel from the committed rocprofv3 --pmc
+    summary (profiles/decode_traffic.json: FETCH_SIZE and WRITE_SIZE per dispatch, each
+    scaled by the same counter's reading for a 1 GiB copy).  None when no summary
+    matches this workload."""
+    path = os.path.join(ROOT, "profiles", "decode_traffic.json")
+    try:
+        with open(path) as f:
+            rec = json.load(f).get(f"{workload}:m={m}")
+    except (OSError, ValueError):
+        return None
+    if not rec:
+        return None
+    return {"bytes_per_launch": rec["bytes_per_launch"],
+            "vs_algorithmic": round(rec["bytes_per_launch"] / avg_algorithmic, 3),
+            "source": "profiles/decode_traffic.json"}
 
 
 def main():
@@ -180,6 +210,9 @@ def main():
     ap.add_argument("--m", type=int, default=1, help="activation rows per call (decode batch)")
     ap.add_argument("--layers", type=int, default=N_LAYERS_8B)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy (a known-size kernel that scales "
+                         "the rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--no-extras", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -195,6 +228,13 @@ def main():
     torch.cuda.set_device(0)
     qa.lib()
     dtype = Q4_K if args.workload == "decode_q4k_8b_stack" else Q8_0
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # 1 GiB read + 1 GiB written by one elementwise copy kernel
+        torch.cuda.synchronize()
+        del src, dst
 
     calls, total_bytes = build_decode_stack(torch, qa, oracle, dtype, args.m, args.layers, True)
     launches = len(calls)
@@ -234,7 +274,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": measured_traffic(args.workload, args.m, total_bytes / launches),
             "avg_launch_us": round(ms * 1e3 / launches, 3),
             "avg_algorithmic_bytes_per_launch": int(total_bytes / launches),
         },

@@ -125,6 +125,13 @@ int create_from_parts(int dtype, int64_t n_stacked, int64_t n, int64_t k, const 
     uint64_t total = 0;
     for (int i = 0; i < n_parts; i++) total += parts[i].nbytes;
     QmmLayout L = qmm_make_layout(dtype, n_stacked, n, k);
+    // the kernels index panels, rows and k-units with 32-bit integers
+    if (n > ((int64_t)1 << 24) || k > ((int64_t)1 << 22) || n_stacked > 65536 ||
+        L.row_tiles * L.k_groups >= ((int64_t)1 << 31))
+        return fail(IZWI_QMM_ERR_UNSUPPORTED,
+                    "shape [%lld x %lld x %lld] exceeds the kernels' limits (n <= 2^24, k <= 2^22, "
+                    "n*k/4096 < 2^31 panels, <= 65536 stacked matrices)",
+                    (long long)n_stacked, (long long)n, (long long)k);
     izwi_qmm_weight* w = new izwi_qmm_weight();
     w->layout = L;
     w->nbytes = total;
