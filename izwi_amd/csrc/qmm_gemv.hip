@@ -126,22 +126,33 @@ __device__ __forceinline__ void quantize_q80_lane(const float (&v)[16], uint32_t
     }
 }
 
-__device__ __forceinline__ void load16(const float* __restrict__ row, int64_t k0, int64_t k,
-                                       bool row_ok, float (&v)[16]) {
-    if (row_ok && k0 + 16 <= k) {
-        const float4* p = reinterpret_cast<const float4*>(row + k0);
+// Sixteen consecutive activations of one row as four 16 B loads.  k is a
+// multiple of 32, so a 16-value run is either inside the row or entirely past
+// its end.  The loads are unconditional (out-of-range lanes read the start of
+// `safe` instead) so that the issuing code stays one basic block and the waits
+// on these loads can be counted separately from the weight loads behind them;
+// x16_finish applies the range check to the values.
+__device__ __forceinline__ void x16_issue(const float* __restrict__ src, const float* __restrict__ safe,
+                                          bool in_range, float4 (&f)[4]) {
+    const float4* p = reinterpret_cast<const float4*>(in_range ? src : safe);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            float4 f = p[i];
-            v[4 * i] = f.x;
-            v[4 * i + 1] = f.y;
-            v[4 * i + 2] = f.z;
-            v[4 * i + 3] = f.w;
-        }
-    } else {
+    for (int i = 0; i < 4; i++) f[i] = p[i];
+}
+__device__ __forceinline__ void x16_finish(const float4 (&f)[4], bool in_range, float (&v)[16]) {
 #pragma unroll
-        for (int i = 0; i < 16; i++) v[i] = (row_ok && k0 + i < k) ? row[k0 + i] : 0.0f;
+    for (int i = 0; i < 4; i++) {
+        v[4 * i] = in_range ? f[i].x : 0.0f;
+        v[4 * i + 1] = in_range ? f[i].y : 0.0f;
+        v[4 * i + 2] = in_range ? f[i].z : 0.0f;
+        v[4 * i + 3] = in_range ? f[i].w : 0.0f;
     }
+}
+
+// Workgroup barrier that orders LDS traffic only: the compiler's own barrier
+// also waits for every outstanding global load of the wave, which would
+// serialize the weight panel behind the activation quantizer.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
 // ---- LDS view ---------------------------------------------------------------
@@ -189,13 +200,16 @@ struct XSource {
 };
 
 template <int MT>
-__device__ __forceinline__ void x_item_load(const XSource& s, int item, float (&v)[16]) {
+__device__ __forceinline__ bool x_item_issue(const XSource& s, int item, bool item_ok, float4 (&f)[4]) {
     const int j = threadIdx.x & 15;
     const int mi = item % MT, unit = item / MT;
-    const bool row_ok = s.m0 + mi < s.m;
+    const bool row_ok = item_ok && s.m0 + mi < s.m;
     int64_t xr = s.m0 + mi;
     if (s.perm != nullptr) xr = row_ok ? s.perm[s.m0 + mi] / s.x_div : 0;
-    load16(s.x + xr * s.k, (int64_t)unit * 256 + 16 * j, s.k, row_ok, v);
+    const int64_t k0 = (int64_t)unit * 256 + 16 * j;
+    const bool in_range = row_ok && k0 + 16 <= s.k;
+    x16_issue(s.x + xr * s.k + k0, s.x, in_range, f);
+    return in_range;
 }
 
 template <int QT, int MT>
@@ -229,20 +243,24 @@ struct Panel {
     u32x4 q[QC];
 };
 
+// Unconditional loads (see x16_issue): a lane without a slot reads lane 0's
+// data and the caller clears its header, which zeroes every scale and with
+// them the lane's contribution.
 template <int QT>
 __device__ __forceinline__ void load_panel(Panel<QT>& p, const uint8_t* __restrict__ base,
                                            int slots, int lane, bool active) {
-    if (active) {
-        const u32x4* src = reinterpret_cast<const u32x4*>(base) + lane;
-        p.hdr = __builtin_nontemporal_load(src);
+    const u32x4* src = reinterpret_cast<const u32x4*>(base) + (active ? lane : 0);
+    p.hdr = __builtin_nontemporal_load(src);
 #pragma unroll
-        for (int c = 0; c < Panel<QT>::QC; c++)
-            p.q[c] = __builtin_nontemporal_load(src + (size_t)(1 + c) * slots);
-    } else {
-        p.hdr = u32x4{0, 0, 0, 0};
-#pragma unroll
-        for (int c = 0; c < Panel<QT>::QC; c++) p.q[c] = u32x4{0, 0, 0, 0};
-    }
+    for (int c = 0; c < Panel<QT>::QC; c++)
+        p.q[c] = __builtin_nontemporal_load(src + (size_t)(1 + c) * slots);
+}
+template <int QT>
+__device__ __forceinline__ void mask_panel(Panel<QT>& p, bool active) {
+    p.hdr.x = active ? p.hdr.x : 0u;
+    p.hdr.y = active ? p.hdr.y : 0u;
+    p.hdr.z = active ? p.hdr.z : 0u;
+    p.hdr.w = active ? p.hdr.w : 0u;
 }
 
 __device__ __forceinline__ int dot16(const u32x4& a, const uint4& b, int acc) {
@@ -386,30 +404,36 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
                 const bool ok = rt < P.row_tiles && kg < P.k_groups;
                 const int64_t off = ok ? (int64_t)(rt * P.k_groups + kg) * P.panel_bytes : 0;
                 Panel<QT> p;
+                const bool active = ok && lane_active;
                 if (!x_ready) {
                     // Loads return in issue order: the small activation load goes first so
                     // that it can be consumed (quantized) while the panel loads still fly.
                     const int group = threadIdx.x >> 4, n_groups = blockDim.x >> 4;
                     const int items = MT * P.k_units;
                     const XSource xs{P.x, GROUPED ? P.perm : nullptr, P.x_div, m0, m_end, P.k, P.k_units};
+                    float4 f[4];
                     float v[16];
-                    if (group < items) x_item_load<MT>(xs, group, v);
-                    load_panel<QT>(p, wbase + off, P.slots, lane, ok && lane_active);
-                    if (m0 != m_begin) __syncthreads();
+                    const bool in0 = x_item_issue<MT>(xs, group, group < items, f);
+                    load_panel<QT>(p, wbase + off, P.slots, lane, active);
+                    if (m0 != m_begin) lds_barrier(); // the previous rows' readers are done
+                    x16_finish(f, in0, v);
                     if (group < items) x_item_quantize<QT, MT>(l, P.k_units, group, v);
                     for (int item = group + n_groups; item < items; item += n_groups) {
-                        x_item_load<MT>(xs, item, v);
+                        const bool in1 = x_item_issue<MT>(xs, item, true, f);
+                        x16_finish(f, in1, v);
                         x_item_quantize<QT, MT>(l, P.k_units, item, v);
                     }
-                    __syncthreads();
+                    lds_barrier();
                     x_ready = true;
                 } else {
-                    load_panel<QT>(p, wbase + off, P.slots, lane, ok && lane_active);
+                    load_panel<QT>(p, wbase + off, P.slots, lane, active);
                 }
+                mask_panel<QT>(p, active);
                 const int unit = min(kg * P.s + us, P.k_units - 1);
                 multiply_panel<QT, MT>(p, l, unit, P.k_units, acc[0]);
                 if (GATED) { // the second stack reuses the panel registers
-                    load_panel<QT>(p, wbase2 + off, P.slots, lane, ok && lane_active);
+                    load_panel<QT>(p, wbase2 + off, P.slots, lane, active);
+                    mask_panel<QT>(p, active);
                     multiply_panel<QT, MT>(p, l, unit, P.k_units, acc[G - 1]);
                 }
             }
@@ -555,7 +579,13 @@ __global__ void quantize_export_kernel(const float* __restrict__ x, int64_t m, i
     if (group >= m * k_units) return; // whole 16-lane groups leave together
     int64_t mi = group / k_units, unit = group - mi * k_units;
     float v[16];
-    load16(x + mi * k, unit * 256 + 16 * j, k, true, v);
+    {
+        const int64_t k0 = unit * 256 + 16 * j;
+        const bool in_range = k0 + 16 <= k;
+        float4 f[4];
+        x16_issue(x + mi * k + k0, x, in_range, f);
+        x16_finish(f, in_range, v);
+    }
     uint32_t q[4];
     if (QT == QMM_Q4_K) {
         float d;
