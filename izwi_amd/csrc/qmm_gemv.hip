@@ -358,8 +358,11 @@ __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 
 // MT rows per pass.  GATED: two weight stacks share x and the result is
 // silu(w x) * (w2 x) (the expert MLP's gate/up pair).  GROUPED: rows are sorted
-// (token, slot) pairs of one expert.
-template <int QT, int MT, bool GATED, bool GROUPED>
+// (token, slot) pairs of one expert.  ONESHOT: the launch gives every wave exactly
+// one panel (one pass of rows, one row-tile group per workgroup, one k step), so
+// the three loops below run once and the kernel is straight-line code from its
+// entry to the first load.
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
     constexpr int G = GATED ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -389,17 +392,18 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
     }
     const XLds<QT> l = carve<QT, MT, G>(smem, P.k_units);
 
-    for (int m0 = m_begin; m0 < m_end; m0 += MT) {
+    for (int m0 = m_begin; ONESHOT ? m0 == m_begin : m0 < m_end; m0 += MT) {
         bool x_ready = false;
         int red_buf = 0;
-        for (int rtg = blockIdx.x; rtg < P.rt_groups; rtg += gridDim.x) {
+        for (int rtg = blockIdx.x; ONESHOT ? rtg == (int)blockIdx.x : rtg < P.rt_groups;
+             rtg += ONESHOT ? 1 : (int)gridDim.x) {
             const int rt = rtg * P.nwr + wr;
             float acc[G][MT];
 #pragma unroll
             for (int g = 0; g < G; g++)
 #pragma unroll
                 for (int mi = 0; mi < MT; mi++) acc[g][mi] = 0.0f;
-            for (int ks = 0; ks < P.kpw; ks++) {
+            for (int ks = 0; ONESHOT ? ks < 1 : ks < P.kpw; ks++) {
                 const int kg = ks * P.nwk + wk;
                 const bool ok = rt < P.row_tiles && kg < P.k_groups;
                 const int64_t off = ok ? (int64_t)(rt * P.k_groups + kg) * P.panel_bytes : 0;
@@ -516,18 +520,22 @@ template <int QT, int MT, bool GATED, bool GROUPED>
 hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipStream_t stream) {
     size_t lds = lds_bytes<QT, MT, GATED ? 2 : 1>(P.k_units, waves);
     if (lds > 160 * 1024) return hipErrorInvalidValue;
-    if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(
-            reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-    }
     int64_t cap = (int64_t)n_cus * 32;
     if (grid_y > 1) cap = cap / grid_y > 64 ? cap / grid_y : 64;
     int64_t grid = P.rt_groups < cap ? P.rt_groups : cap;
     if (grid < 1) grid = 1;
-    gemv_kernel<QT, MT, GATED, GROUPED>
-        <<<dim3((unsigned)grid, (unsigned)grid_y), dim3(64 * waves), lds, stream>>>(P);
+    const bool oneshot = !GROUPED && !GATED && P.m <= MT && P.kpw == 1 && grid == P.rt_groups;
+    const void* fn = oneshot ? reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, !GROUPED && !GATED>)
+                             : reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, false>);
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+    }
+    const dim3 g((unsigned)grid, (unsigned)grid_y), b(64 * waves);
+    if (oneshot)
+        gemv_kernel<QT, MT, GATED, GROUPED, !GROUPED && !GATED><<<g, b, lds, stream>>>(P);
+    else
+        gemv_kernel<QT, MT, GATED, GROUPED, false><<<g, b, lds, stream>>>(P);
     return hipGetLastError();
 }
 
