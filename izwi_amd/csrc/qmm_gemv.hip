@@ -22,6 +22,8 @@
 // small matrices then fit in one round of workgroups.
 #include <hip/hip_runtime.h>
 
+#include <cstddef>
+
 #include "qmm_internal.h"
 
 namespace {
@@ -331,20 +333,24 @@ __device__ __forceinline__ void multiply_panel(const Panel<QT>& p, const XLds<QT
     }
 }
 
+// The first 64 bytes hold everything a wave needs to issue its first loads, so
+// that one scalar load fetches them.
 struct GemvParams {
     const uint8_t* w;  // tiled matrix (expert 0 of a stack)
-    const uint8_t* w2; // gated form only: the second stack ("up"), same layout as w
     const float* x;    // [m, k]            (grouped: [tokens, k] or [pairs, k])
     float* y;          // [m, n]            (grouped: [pairs, n])
     int m, n, k;
-    int k_units, k_groups, s, slots;
+    int k_groups, slots; // the kernel derives k_units = ceil(k / 256) and s = slots / 16
     int row_tiles, panel_bytes;
-    int64_t matrix_bytes;
     // split of the workgroup's waves: nwk along k times nwr row-tiles side by side
     int nwk, nwr;
+    int wave_magic; // ceil(65536 / nwk): wave / nwk == (wave * wave_magic) >> 16
+    // ---- 64 bytes ----
+    int k_units, s;
+    const uint8_t* w2; // gated form only: the second stack ("up"), same layout as w
+    int64_t matrix_bytes;
     int kpw;        // ceil(k_groups / nwk): panels per row-tile for every wave
     int rt_groups;  // ceil(row_tiles / nwr)
-    int wave_magic; // ceil(65536 / nwk): wave / nwk == (wave * wave_magic) >> 16
     // grouped (expert) form: blockIdx.y is a segment of up to QMM_MOE_SEG_ROWS
     // sorted pairs that share one expert
     const int32_t* perm;
@@ -353,6 +359,7 @@ struct GemvParams {
     int n_experts;
     int x_div; // x row of pair p is p / x_div
 };
+static_assert(offsetof(GemvParams, k_units) == 64, "first-load fields must fill one 64-byte line");
 
 __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 
@@ -372,6 +379,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
     const int wk = wave - wr * P.nwk;
     const bool lane_active = lane < P.slots;
     const int us = lane >> 4;
+    const int k_units = (P.k + 255) >> 8, s_units = P.slots >> 4;
 
     int m_begin = 0, m_end = P.m;
     const uint8_t* wbase = P.w;
@@ -390,7 +398,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
         wbase += (int64_t)lo * P.matrix_bytes;
         if (GATED) wbase2 += (int64_t)lo * P.matrix_bytes;
     }
-    const XLds<QT> l = carve<QT, MT, G>(smem, P.k_units);
+    const XLds<QT> l = carve<QT, MT, G>(smem, k_units);
 
     for (int m0 = m_begin; ONESHOT ? m0 == m_begin : m0 < m_end; m0 += MT) {
         bool x_ready = false;
@@ -412,20 +420,20 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
                 if (!x_ready) {
                     // Loads return in issue order: the small activation load goes first so
                     // that it can be consumed (quantized) while the panel loads still fly.
-                    const int group = threadIdx.x >> 4, n_groups = blockDim.x >> 4;
-                    const int items = MT * P.k_units;
-                    const XSource xs{P.x, GROUPED ? P.perm : nullptr, P.x_div, m0, m_end, P.k, P.k_units};
+                    const int group = threadIdx.x >> 4, n_groups = 4 * P.nwk * P.nwr; // = blockDim.x / 16
+                    const int items = MT * k_units;
+                    const XSource xs{P.x, GROUPED ? P.perm : nullptr, P.x_div, m0, m_end, P.k, k_units};
                     float4 f[4];
                     float v[16];
                     const bool in0 = x_item_issue<MT>(xs, group, group < items, f);
                     load_panel<QT>(p, wbase + off, P.slots, lane, active);
                     if (m0 != m_begin) lds_barrier(); // the previous rows' readers are done
                     x16_finish(f, in0, v);
-                    if (group < items) x_item_quantize<QT, MT>(l, P.k_units, group, v);
+                    if (group < items) x_item_quantize<QT, MT>(l, k_units, group, v);
                     for (int item = group + n_groups; item < items; item += n_groups) {
                         const bool in1 = x_item_issue<MT>(xs, item, true, f);
                         x16_finish(f, in1, v);
-                        x_item_quantize<QT, MT>(l, P.k_units, item, v);
+                        x_item_quantize<QT, MT>(l, k_units, item, v);
                     }
                     lds_barrier();
                     x_ready = true;
@@ -433,12 +441,12 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
                     load_panel<QT>(p, wbase + off, P.slots, lane, active);
                 }
                 mask_panel<QT>(p, active);
-                const int unit = min(kg * P.s + us, P.k_units - 1);
-                multiply_panel<QT, MT>(p, l, unit, P.k_units, acc[0]);
+                const int unit = min(kg * s_units + us, k_units - 1);
+                multiply_panel<QT, MT>(p, l, unit, k_units, acc[0]);
                 if (GATED) { // the second stack reuses the panel registers
                     load_panel<QT>(p, wbase2 + off, P.slots, lane, active);
                     mask_panel<QT>(p, active);
-                    multiply_panel<QT, MT>(p, l, unit, P.k_units, acc[G - 1]);
+                    multiply_panel<QT, MT>(p, l, unit, k_units, acc[G - 1]);
                 }
             }
             // row-tile finished: combine the S units of a row, then the waves that split k
@@ -462,7 +470,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
                     }
                 }
             } else {
-                const int waves = blockDim.x >> 6;
+                const int waves = P.nwk * P.nwr; // = blockDim.x / 64, without the dispatch packet read
                 float* red = l.red + red_buf * (waves * G * MT * 16);
                 if (lane < 16) {
 #pragma unroll
