@@ -1,21 +1,32 @@
-// Batched decode kernel (M = 3..64): the same arithmetic as the M <= 2 kernel
+// Batched decode kernels (M = 3..64): the same arithmetic as the M <= 2 kernel
 // (candle-core's integer block dots on Q8-quantized activations), with the
 // int8 products on v_mfma_i32_16x16x32_i8 so that the cost per weight byte does
 // not grow with M.
 //
 // Two launches:
-//  1. the activations are quantized ONCE into a workspace laid out exactly as
-//     the MFMA A operand wants them (16 rows per tile: [unit][sub-block]
-//     [octet][row][8 B]), so the matmul workgroups copy it to LDS verbatim;
-//  2. each wave streams weight panels (16 rows x S units) as in the M <= 2
-//     kernel.  A panel lane holds one (row, unit); the MFMA B operand wants
-//     (row, 8-element octet) per lane, so the quants are transposed between
-//     the four 16-lane rows in registers (v_permlane32_swap + v_permlane16_swap,
-//     two swaps per dword).  One MFMA per 32-element sub-block: D[m][row] are
-//     the block dots of 16 activation rows at once; the 6-bit sub-block scales
-//     are applied on integers (v_mad_i32_i24), the Q4_K min term comes from a
-//     second chained MFMA whose B operand is the min replicated over the octet
-//     (min * sum of activation quants, accumulated over the 8 sub-blocks).
+//  1. the activations are quantized ONCE into a workspace of self-contained
+//     unit records (256 k-values of 16 rows): 4096 B of int8 laid out exactly as
+//     the MFMA A operand wants them ([sub-block][octet][row][8 B]) followed by
+//     the unit's side information (row scales; for Q4_K also the sub-block sums
+//     as two int8 planes), so the matmul workgroups move a run of units to LDS
+//     verbatim with LDS-direct loads;
+//  2. a wave streams weight panels (16 rows x S units) as in the M <= 2 kernel.
+//     A panel lane holds one (row, unit); the MFMA B operand wants (row, 8-element
+//     octet) per lane, so the quants are transposed between the four 16-lane rows
+//     in registers (v_permlane32_swap + v_permlane16_swap, two swaps per dword).
+//     One MFMA per 32-element sub-block: D[m][row] are the block dots of 16
+//     activation rows at once; the 6-bit sub-block scales are applied on integers
+//     (v_mad_i32_i24), the Q4_K min term is itself a matmul over the sub-block
+//     index (two MFMAs per unit).  The panel is consumed chunk pair by chunk pair
+//     in load order, so the arithmetic runs while the rest of the panel arrives.
+//
+// Two forms of launch 2:
+//  * one-shot: every wave owns exactly one panel, all panels of the matrix are
+//    requested at once (after the first activation window); a workgroup is nwk
+//    waves along k times nwr row-tiles.  Activation windows (up to 32 units) that
+//    do not fit LDS together follow one another, the panels stay in registers;
+//  * streaming (very tall matrices): a wave owns whole row-tiles and walks their
+//    panels, the activation window stays in LDS for all of them.
 #include <hip/hip_runtime.h>
 
 #include "qmm_internal.h"
@@ -23,8 +34,6 @@
 namespace {
 
 constexpr int kMaxWaves = 12;
-constexpr int kChunkUnits = 16;       // units of x held in LDS at a time (64 KiB of int8)
-constexpr int kUnitBytes = 4096;      // [8 sub-blocks][4 octets][16 rows][8 B]
 constexpr uint32_t kNib = 0x0f0f0f0fu;
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
@@ -50,50 +59,57 @@ __device__ __forceinline__ int row16_min(int v) {
     return v;
 }
 
-// workspace geometry for one call
-struct XWs {
-    int k_units;
-    int n_tiles; // ceil(m / 16)
-    __host__ __device__ size_t xq_bytes() const { return (size_t)n_tiles * k_units * kUnitBytes; }
-    // side information per unit, in floats.  Q4_K: 16 row scales, then per row the
-    // eight sub-block sums of the quants split into two int8 planes (sum = 128 * hi + lo).
-    // Q8_0: one scale per (block, row).
-    __host__ __device__ static int xd_per_unit(int qt) { return qt == QMM_Q4_K ? 16 + 64 : 128; }
-    __host__ __device__ size_t xd_floats(int qt) const {
-        return (size_t)n_tiles * k_units * xd_per_unit(qt);
-    }
-};
 
-// ---- launch 1: activation quantizer into the MFMA layout --------------------
+template <int QT>
+struct Unit {
+    static constexpr int kQuant = 4096; // [8 sub-blocks][4 octets][16 rows][8 B]
+    // Q4_K: 16 row scales (f32), then per row the eight sub-block sums of the quants split
+    // into two int8 planes (sum = 128 * hi + lo): 64 + 16 * 16 bytes.
+    // Q8_0: one f32 scale per (block, row): 8 * 16 * 4 bytes.
+    static constexpr int kSide = QT == QMM_Q4_K ? 320 : 512;
+    static constexpr int kBytes = kQuant + kSide;
+};
+constexpr int kWindowUnits = 32; // activation units resident in LDS at a time
+
+__host__ __device__ inline int unit_bytes(int qt) { return qt == QMM_Q4_K ? Unit<QMM_Q4_K>::kBytes : Unit<QMM_Q8_0>::kBytes; }
+
+// Workgroup barrier that orders LDS traffic only (the compiler's own barrier also
+// waits for every outstanding global load of the wave).
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// ---- launch 1: activation quantizer into the unit records -------------------
 // One 16-lane group per (row, unit); lane j holds elements 16j..16j+15, i.e.
 // sub-block j / 2, octets 2 (j % 2) and 2 (j % 2) + 1.
 template <int QT>
-__global__ void quantize_ws_kernel(const float* __restrict__ x, int m, int k, XWs ws,
-                                   uint8_t* __restrict__ xq, float* __restrict__ xd) {
+__global__ void quantize_ws_kernel(const float* __restrict__ x, int m, int k, int k_units, int n_tiles,
+                                   uint8_t* __restrict__ ws) {
     const int group = (blockIdx.x * blockDim.x + threadIdx.x) >> 4;
     const int j = threadIdx.x & 15;
-    const int rows = ws.n_tiles * 16;
-    if (group >= rows * ws.k_units) return; // whole 16-lane groups leave together
-    const int row = group / ws.k_units, unit = group - row * ws.k_units;
+    const int rows = n_tiles * 16;
+    if (group >= rows * k_units) return; // whole 16-lane groups leave together
+    const int row = group / k_units, unit = group - row * k_units;
     const int tile = row >> 4, mr = row & 15;
     float v[16];
     const int k0 = unit * 256 + 16 * j;
-    if (row < m && k0 + 16 <= k) {
-        const float4* p = reinterpret_cast<const float4*>(x + (int64_t)row * k + k0);
+    {
+        // k is a multiple of 32: a 16-value run is inside the row or past its end
+        const bool in_range = row < m && k0 + 16 <= k;
+        const float4* p = reinterpret_cast<const float4*>(in_range ? x + (int64_t)row * k + k0 : x);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             float4 f = p[i];
-            v[4 * i] = f.x, v[4 * i + 1] = f.y, v[4 * i + 2] = f.z, v[4 * i + 3] = f.w;
+            v[4 * i] = in_range ? f.x : 0.0f, v[4 * i + 1] = in_range ? f.y : 0.0f;
+            v[4 * i + 2] = in_range ? f.z : 0.0f, v[4 * i + 3] = in_range ? f.w : 0.0f;
         }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 16; i++) v[i] = (row < m && k0 + i < k) ? x[(int64_t)row * k + k0 + i] : 0.0f;
     }
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < 16; i++) amax = fmaxf(amax, fabsf(v[i]));
     float scale_mul; // quant = round(v * scale_mul)
-    const int64_t tu = (int64_t)tile * ws.k_units + unit;
+    uint8_t* rec = ws + ((int64_t)tile * k_units + unit) * Unit<QT>::kBytes;
+    float* side = reinterpret_cast<float*>(rec + Unit<QT>::kQuant);
     if (QT == QMM_Q4_K) {
         // BlockQ8K::from_float: iscale = -128 / (first value of largest magnitude)
         amax = row16_max(amax);
@@ -108,13 +124,13 @@ __global__ void quantize_ws_kernel(const float* __restrict__ x, int m, int k, XW
             scale_mul = __fdiv_rn(-128.0f, (key & 1) ? -amax : amax);
             d = __fdiv_rn(1.0f, scale_mul);
         }
-        if (j == 0) xd[tu * 80 + mr] = d;
+        if (j == 0) side[mr] = d;
     } else {
         // BlockQ8_0::from_float on the lane pair's 32 values
         amax = fmaxf(amax, __int_as_float(dpp<kDppXor1>(__float_as_int(amax))));
         const float d = __fdiv_rn(amax, 127.0f);
         scale_mul = d != 0.0f ? __fdiv_rn(1.0f, d) : 0.0f;
-        if ((j & 1) == 0) xd[(tu * 8 + (j >> 1)) * 16 + mr] = qmm_f16_bits_to_f32(qmm_f32_to_f16_bits(d));
+        if ((j & 1) == 0) side[(j >> 1) * 16 + mr] = qmm_f16_bits_to_f32(qmm_f32_to_f16_bits(d));
     }
     uint32_t q[4];
 #pragma unroll
@@ -137,12 +153,12 @@ __global__ void quantize_ws_kernel(const float* __restrict__ x, int m, int k, XW
         s16 = __builtin_amdgcn_sdot4((int)q[3], 0x01010101, s16, false);
         const int bsum = s16 + dpp<kDppXor1>(s16); // the sub-block's 32 quants
         if ((j & 1) == 0) {
-            uint8_t* side = reinterpret_cast<uint8_t*>(xd + tu * 80 + 16) + mr * 16;
-            side[s] = (uint8_t)(bsum & 127);
-            side[8 + s] = (uint8_t)(bsum >> 7);
+            uint8_t* planes = reinterpret_cast<uint8_t*>(side + 16) + mr * 16;
+            planes[s] = (uint8_t)(bsum & 127);
+            planes[8 + s] = (uint8_t)(bsum >> 7);
         }
     }
-    uint8_t* dst = xq + ((tu * 8 + s) * 4 + oct) * 128 + mr * 8;
+    uint8_t* dst = rec + (s * 4 + oct) * 128 + mr * 8;
     *reinterpret_cast<uint2*>(dst) = make_uint2(q[0], q[1]);
     *reinterpret_cast<uint2*>(dst + 128) = make_uint2(q[2], q[3]);
 }
@@ -150,15 +166,15 @@ __global__ void quantize_ws_kernel(const float* __restrict__ x, int m, int k, XW
 // ---- launch 2 ------------------------------------------------------------------
 struct MfmaParams {
     const uint8_t* w;
-    const uint8_t* xq;
-    const float* xd;
+    const uint8_t* ws; // unit records [n_tiles][k_units]
     float* y;
-    int m, n, k;
-    int k_units, k_groups, s, slots;
+    int m, n;
+    int k_units, k_groups, slots;
     int row_tiles, panel_bytes;
     int nwk, nwr, wave_magic;
-    int chunk_units; // multiple of s, <= kChunkUnits
     int n_tiles;
+    int window_units; // multiple of s, <= kWindowUnits
+    int rt_groups;
 };
 
 // 4x4 transpose of one dword between the four 16-lane rows: on entry row u
@@ -175,151 +191,201 @@ __device__ __forceinline__ long pack64(uint32_t lo, uint32_t hi) {
     return (long)(((unsigned long)hi << 32) | lo);
 }
 
+// (row, unit) per lane -> (row, octet) per lane for chunk pair b: afterwards unit u of
+// the pair sits in dwords (x,y) / (z,w) of q[2b] / q[2b+1]:
+//   u = 0: q[2b].xy   u = 1: q[2b].zw   u = 2: q[2b+1].xy   u = 3: q[2b+1].zw
+__device__ __forceinline__ void transpose_pair(u32x4& q0, u32x4& q1) {
+    uint32_t a0 = q0.x, a1 = q0.z, a2 = q1.x, a3 = q1.z;
+    uint32_t b0 = q0.y, b1 = q0.w, b2 = q1.y, b3 = q1.w;
+    transpose_rows(a0, a1, a2, a3);
+    transpose_rows(b0, b1, b2, b3);
+    q0 = u32x4{a0, b0, a1, b1};
+    q1 = u32x4{a2, b2, a3, b3};
+}
+
 template <int QT>
-__global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_kernel(MfmaParams P) {
-    constexpr int QC = QT == QMM_Q4_K ? 8 : 16;
-    constexpr int XD_PER_UNIT = QT == QMM_Q4_K ? 80 : 128; // floats of side information per unit
+struct WPanel {
+    static constexpr int QC = QT == QMM_Q4_K ? 8 : 16;
+    u32x4 hdr[4]; // headers of the four units of row j
+    u32x4 q[QC];
+};
+
+// Unconditional loads (one basic block, so the waits can be counted): a lane
+// without a slot reads slot 0, units past s re-read unit 0's header; neither is
+// used afterwards.
+template <int QT>
+__device__ __forceinline__ void load_wpanel(WPanel<QT>& p, const uint8_t* __restrict__ base, int slots,
+                                            int lane, int j) {
+    const u32x4* b = reinterpret_cast<const u32x4*>(base);
+    const int ln = lane < slots ? lane : 0;
+#pragma unroll
+    for (int u = 0; u < 4; u++) p.hdr[u] = b[(u * 16 < slots ? u * 16 : 0) + j];
+#pragma unroll
+    for (int c = 0; c < WPanel<QT>::QC; c++)
+        p.q[c] = __builtin_nontemporal_load(b + (size_t)(1 + c) * slots + ln);
+}
+
+// acc[r] += block dots of the panel's units against activation rows 4 grp + r of
+// the tile whose unit records start at `xu0` (LDS, record of the panel's unit 0).
+// FIRST: the quants are still in load layout and are transposed pair by pair, in
+// load order.  `n_units` (uniform) is the number of the panel's units that exist.
+template <int QT, bool FIRST>
+__device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int n_units, int j, int grp,
+                                          float (&acc)[4]) {
+    constexpr int UB = Unit<QT>::kBytes;
+    const int lane8 = (grp * 16 + j) * 8;
+    if (QT == QMM_Q4_K) {
+        uint32_t sc_lo[4], sc_hi[4], mn_lo[4], mn_hi[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            qmm_unpack_q4k_scales(p.hdr[u].y, p.hdr[u].z, p.hdr[u].w, sc_lo[u], sc_hi[u], mn_lo[u], mn_hi[u]);
+        int isum[4][4];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) isum[u][r] = 0;
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            if (FIRST) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
+            // the eight MFMAs of the pair are issued back to back, their results are
+            // consumed afterwards: the matrix pipe's latency is paid once per pair
+            i32x4 dlo[4], dhi[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (u >= n_units) continue; // uniform
+                const u32x4 qq = p.q[2 * b + (u >> 1)];
+                const uint32_t w0 = (u & 1) ? qq.z : qq.x, w1 = (u & 1) ? qq.w : qq.y;
+                const uint8_t* xu = xu0 + u * UB + lane8;
+                const long a_lo = *reinterpret_cast<const long*>(xu + (2 * b) * 512);
+                const long a_hi = *reinterpret_cast<const long*>(xu + (2 * b + 1) * 512);
+                dlo[u] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, pack64(w0 & kNib, w1 & kNib),
+                                                               i32x4{0, 0, 0, 0}, 0, 0, 0);
+                dhi[u] = __builtin_amdgcn_mfma_i32_16x16x32_i8(
+                    a_hi, pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib), i32x4{0, 0, 0, 0}, 0, 0, 0);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (u >= n_units) continue;
+                const int sc0 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b);
+                const int sc1 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b + 1);
+#pragma unroll
+                for (int r = 0; r < 4; r++) // |dot| < 2^17, scale < 64
+                    isum[u][r] += __mul24(sc0, dlo[u][r]) + __mul24(sc1, dhi[u][r]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            if (u >= n_units) continue;
+            const float d = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x & 0xffffu));
+            const float dmin = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x >> 16));
+            // min term: sum_s min_s * bsum_s as two MFMAs over k = sub-block index; only
+            // the first 16-lane row carries data (k slots 0..7), the rest multiply zeros
+            const uint8_t* side = xu0 + u * UB + Unit<QT>::kQuant;
+            const uint8_t* planes = side + 64 + j * 16;
+            const long bs_lo = grp == 0 ? *reinterpret_cast<const long*>(planes) : 0L;
+            const long bs_hi = grp == 0 ? *reinterpret_cast<const long*>(planes + 8) : 0L;
+            const long bmn = pack64(mn_lo[u], mn_hi[u]);
+            const i32x4 m_lo = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_lo, bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
+            const i32x4 m_hi = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_hi, bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
+            const float4 dx = *reinterpret_cast<const float4*>(side + grp * 16);
+            const float dxs[4] = {dx.x, dx.y, dx.z, dx.w};
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int msum = m_lo[r] + (m_hi[r] << 7);
+                acc[r] += (d * dxs[r]) * (float)isum[u][r] - (dmin * dxs[r]) * (float)msum;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            if (FIRST) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
+            i32x4 dd[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (u >= n_units) continue;
+                const u32x4 qq = p.q[2 * b + (u >> 1)];
+                const uint32_t w0 = (u & 1) ? qq.z : qq.x, w1 = (u & 1) ? qq.w : qq.y;
+                const long a = *reinterpret_cast<const long*>(xu0 + u * UB + lane8 + b * 512);
+                dd[u] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, pack64(w0, w1), i32x4{0, 0, 0, 0}, 0, 0, 0);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (u >= n_units) continue;
+                const uint32_t hw = b < 2 ? p.hdr[u].x : b < 4 ? p.hdr[u].y : b < 6 ? p.hdr[u].z : p.hdr[u].w;
+                const float dw = qmm_f16_bits_to_f32((uint16_t)((hw >> (16 * (b & 1))) & 0xffffu));
+                const float4 dx = *reinterpret_cast<const float4*>(xu0 + u * UB + Unit<QT>::kQuant +
+                                                                   (b * 16 + grp * 4) * 4);
+                acc[0] += ((float)dd[u][0] * dw) * dx.x;
+                acc[1] += ((float)dd[u][1] * dw) * dx.y;
+                acc[2] += ((float)dd[u][2] * dw) * dx.z;
+                acc[3] += ((float)dd[u][3] * dw) * dx.w;
+            }
+        }
+    }
+}
+
+// Moves `n_units` unit records of a tile from the workspace to LDS, 1 KiB pieces
+// spread over the workgroup's waves, 16 B per lane, without passing through
+// registers.  Completion is the caller's business (vmcnt).
+template <int QT>
+__device__ __forceinline__ void issue_window_copy(const uint8_t* __restrict__ src, uint8_t* lds, int n_units,
+                                                  int wave, int waves, int lane) {
+    const int bytes = n_units * Unit<QT>::kBytes; // a multiple of 64
+    for (int piece = wave; piece * 1024 < bytes; piece += waves) {
+        const int off = piece * 1024 + lane * 16;
+        if (off < bytes)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + off),
+                                             (__attribute__((address_space(3))) void*)(lds + piece * 1024),
+                                             16, 0, 0);
+    }
+}
+
+// One-shot form: wave (wr, wk) owns panel wk of row-tile blockIdx.x * nwr + wr.
+template <int QT>
+__global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaParams P) {
+    constexpr int UB = Unit<QT>::kBytes;
+    constexpr int NL = WPanel<QT>::QC + 4; // loads of one panel
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    uint8_t* lds_xq = smem;                                                        // chunk_units * 4096
-    float* lds_xd = reinterpret_cast<float*>(smem + (size_t)P.chunk_units * kUnitBytes); // chunk_units * XD_PER_UNIT
-    float* lds_red = lds_xd + P.chunk_units * XD_PER_UNIT;                         // waves * 256
+    uint8_t* lds_x = smem;                                                       // window_units * UB
+    float* lds_red = reinterpret_cast<float*>(smem + (size_t)P.window_units * UB); // waves * 256
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
+    const int waves = P.nwk * P.nwr;
     const int wr = (wave * P.wave_magic) >> 16;
     const int wk = wave - wr * P.nwk;
     const int j = lane & 15, grp = lane >> 4;
+    const int s_units = P.slots >> 4;
     const int rt = blockIdx.x * P.nwr + wr;
     const bool rt_ok = rt < P.row_tiles;
-    const bool lane_active = lane < P.slots;
+    const int unit0 = wk * s_units;                       // first unit of this wave's panel
+    const int n_units = min(s_units, P.k_units - unit0);  // its units that exist (>= 1)
 
-    auto load_panel = [&](int kg, u32x4 (&hdr)[4], u32x4 (&q)[QC]) {
-        const bool ok = rt_ok && lane_active;
-        const u32x4* base =
-            reinterpret_cast<const u32x4*>(P.w + (int64_t)(rt * P.k_groups + kg) * P.panel_bytes);
-#pragma unroll
-        for (int c = 0; c < QC; c++)
-            q[c] = ok ? __builtin_nontemporal_load(base + (size_t)(1 + c) * P.slots + lane)
-                      : u32x4{0, 0, 0, 0};
-#pragma unroll
-        for (int u = 0; u < 4; u++) hdr[u] = (rt_ok && u < P.s) ? base[u * 16 + j] : u32x4{0, 0, 0, 0};
-    };
+    // the first activation window goes first (loads return in order), then the panel
+    const int w0_units = min(P.window_units, P.k_units);
+    issue_window_copy<QT>(P.ws, lds_x, w0_units, wave, waves, lane);
+    asm volatile("" ::: "memory");
+    WPanel<QT> p;
+    load_wpanel<QT>(p, P.w + (int64_t)((rt_ok ? rt : 0) * P.k_groups + wk) * P.panel_bytes, P.slots, lane, j);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory"); // the window has landed, the panel may still fly
+    lds_barrier();
 
+    bool first = true;
     for (int tile = 0; tile < P.n_tiles; tile++) {
         float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (int cu0 = 0; cu0 < P.k_units; cu0 += P.chunk_units) {
-            const int cu_n = min(P.chunk_units, P.k_units - cu0);
-            const int kg0 = cu0 / P.s, kg1 = (cu0 + cu_n + P.s - 1) / P.s;
-            // A workgroup barrier also waits for the calling wave's outstanding loads, so
-            // everything this chunk needs is requested before the one barrier that follows:
-            // first the activations (global -> LDS without passing through registers, each
-            // wave moving 1 KiB pieces, 16 B per lane), then the wave's first weight panel
-            // (this lane's (row j, unit grp) header + quants, and the headers of all units
-            // of row j).
-            if (tile != 0 || cu0 != 0) __syncthreads(); // every wave is done reading the previous chunk
-            {
-                const u32x4* src = reinterpret_cast<const u32x4*>(
-                    P.xq + ((size_t)tile * P.k_units + cu0) * kUnitBytes);
-                const int pieces = cu_n * (kUnitBytes / 1024);
-                const int waves = blockDim.x >> 6;
-                for (int c = wave; c < pieces; c += waves)
-                    __builtin_amdgcn_global_load_lds(
-                        (const __attribute__((address_space(1))) void*)(src + c * 64 + lane),
-                        (__attribute__((address_space(3))) void*)(lds_xq + c * 1024), 16, 0, 0);
+        for (int wu0 = 0; wu0 < P.k_units; wu0 += P.window_units) {
+            const int wn = min(P.window_units, P.k_units - wu0);
+            if (tile != 0 || wu0 != 0) {
+                lds_barrier(); // every wave is done with the previous window
+                issue_window_copy<QT>(P.ws + ((size_t)tile * P.k_units + wu0) * UB, lds_x, wn, wave, waves, lane);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                lds_barrier();
             }
-            u32x4 hdr[4];
-            u32x4 q[QC];
-            bool have_panel = false;
-            if (kg0 + wk < kg1) {
-                load_panel(kg0 + wk, hdr, q);
-                have_panel = true;
-            }
-            {
-                const float* sd = P.xd + ((size_t)tile * P.k_units + cu0) * XD_PER_UNIT;
-                for (int i = threadIdx.x; i < cu_n * XD_PER_UNIT; i += blockDim.x) lds_xd[i] = sd[i];
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the LDS-direct loads have landed
-            }
-            __syncthreads();
-            for (int kg = kg0 + wk; kg < kg1; kg += P.nwk) {
-                if (!have_panel) load_panel(kg, hdr, q);
-                have_panel = false;
-                // ---- (row, unit) per lane -> (row, octet) per lane, for each unit u in register slot u
-#pragma unroll
-                for (int b = 0; b < QC / 2; b++) {
-                    uint32_t a0 = q[2 * b].x, a1 = q[2 * b].z, a2 = q[2 * b + 1].x, a3 = q[2 * b + 1].z;
-                    uint32_t b0 = q[2 * b].y, b1 = q[2 * b].w, b2 = q[2 * b + 1].y, b3 = q[2 * b + 1].w;
-                    transpose_rows(a0, a1, a2, a3);
-                    transpose_rows(b0, b1, b2, b3);
-                    q[2 * b] = u32x4{a0, b0, a1, b1};
-                    q[2 * b + 1] = u32x4{a2, b2, a3, b3};
-                }
-                // after the transpose, unit u of group b sits in dwords (x,y) / (z,w) of q[2b] / q[2b+1]:
-                //   u = 0: q[2b].xy   u = 1: q[2b].zw   u = 2: q[2b+1].xy   u = 3: q[2b+1].zw
-#pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    const int unit = kg * P.s + u;
-                    if (u >= P.s || unit >= P.k_units) continue; // uniform
-                    const int lu = unit - cu0;
-                    const uint8_t* xu = lds_xq + (size_t)lu * kUnitBytes + grp * 128 + j * 8;
-                    if (QT == QMM_Q4_K) {
-                        uint32_t sc_lo, sc_hi, mn_lo, mn_hi;
-                        qmm_unpack_q4k_scales(hdr[u].y, hdr[u].z, hdr[u].w, sc_lo, sc_hi, mn_lo, mn_hi);
-                        // all eight block-dot MFMAs (and the two of the min term) are issued
-                        // back to back; their results are consumed afterwards, so the matrix
-                        // pipe's latency is paid once per unit, not once per sub-block
-                        i32x4 dd[8];
-#pragma unroll
-                        for (int g = 0; g < 4; g++) {
-                            const u32x4 qq = q[2 * g + (u >> 1)];
-                            const uint32_t w0 = (u & 1) ? qq.z : qq.x, w1 = (u & 1) ? qq.w : qq.y;
-                            const long a_lo = *reinterpret_cast<const long*>(xu + (2 * g) * 512);
-                            const long a_hi = *reinterpret_cast<const long*>(xu + (2 * g + 1) * 512);
-                            dd[2 * g] = __builtin_amdgcn_mfma_i32_16x16x32_i8(
-                                a_lo, pack64(w0 & kNib, w1 & kNib), i32x4{0, 0, 0, 0}, 0, 0, 0);
-                            dd[2 * g + 1] = __builtin_amdgcn_mfma_i32_16x16x32_i8(
-                                a_hi, pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib), i32x4{0, 0, 0, 0}, 0, 0, 0);
-                        }
-                        const float d = qmm_f16_bits_to_f32((uint16_t)(hdr[u].x & 0xffffu));
-                        const float dmin = qmm_f16_bits_to_f32((uint16_t)(hdr[u].x >> 16));
-                        // min term: sum_s min_s * bsum_s as two MFMAs over k = sub-block index; only
-                        // the first 16-lane row carries data (k slots 0..7), the rest multiply zeros
-                        const uint8_t* side = reinterpret_cast<const uint8_t*>(lds_xd + lu * 80 + 16) + j * 16;
-                        const long bs_lo = grp == 0 ? *reinterpret_cast<const long*>(side) : 0L;
-                        const long bs_hi = grp == 0 ? *reinterpret_cast<const long*>(side + 8) : 0L;
-                        const long bmn = pack64(mn_lo, mn_hi);
-                        const i32x4 m_lo = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_lo, bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
-                        const i32x4 m_hi = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_hi, bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
-                        const float4 dx = *reinterpret_cast<const float4*>(lds_xd + lu * 80 + grp * 4);
-                        const float dxs[4] = {dx.x, dx.y, dx.z, dx.w};
-                        int isum[4] = {0, 0, 0, 0};
-#pragma unroll
-                        for (int s8 = 0; s8 < 8; s8++) {
-                            const int sc = (int)qmm_byte_of(sc_lo, sc_hi, s8);
-#pragma unroll
-                            for (int r = 0; r < 4; r++) isum[r] += __mul24(sc, dd[s8][r]); // |dd| < 2^17, sc < 64
-                        }
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            const int msum = m_lo[r] + (m_hi[r] << 7);
-                            acc[r] += (d * dxs[r]) * (float)isum[r] - (dmin * dxs[r]) * (float)msum;
-                        }
-                    } else {
-                        const uint32_t hw[4] = {hdr[u].x, hdr[u].y, hdr[u].z, hdr[u].w};
-#pragma unroll
-                        for (int b = 0; b < 8; b++) {
-                            const u32x4 qq = q[2 * b + (u >> 1)];
-                            const uint32_t w0 = (u & 1) ? qq.z : qq.x, w1 = (u & 1) ? qq.w : qq.y;
-                            const long a = *reinterpret_cast<const long*>(xu + b * 512);
-                            i32x4 dd = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, pack64(w0, w1), i32x4{0, 0, 0, 0}, 0, 0, 0);
-                            const float dw = qmm_f16_bits_to_f32((uint16_t)((hw[b >> 1] >> (16 * (b & 1))) & 0xffffu));
-                            const float4 dx = *reinterpret_cast<const float4*>(lds_xd + (lu * 8 + b) * 16 + grp * 4);
-                            acc[0] += ((float)dd[0] * dw) * dx.x;
-                            acc[1] += ((float)dd[1] * dw) * dx.y;
-                            acc[2] += ((float)dd[2] * dw) * dx.z;
-                            acc[3] += ((float)dd[3] * dw) * dx.w;
-                        }
-                    }
-                }
+            if (unit0 >= wu0 && unit0 < wu0 + wn) {
+                const uint8_t* xu0 = lds_x + (size_t)(unit0 - wu0) * UB;
+                if (first) panel_dot<QT, true>(p, xu0, n_units, j, grp, acc);
+                else panel_dot<QT, false>(p, xu0, n_units, j, grp, acc);
+                first = false;
             }
         }
         // ---- combine the waves that split k, write y[tile*16 + 4*grp + r][rt*16 + j]
@@ -333,10 +399,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_kernel(MfmaParams P)
                 }
             }
         } else {
-            __syncthreads();
+            if (tile != 0) lds_barrier(); // the previous tile's sums have been read
 #pragma unroll
             for (int r = 0; r < 4; r++) lds_red[(wave * 4 + r) * 64 + lane] = acc[r];
-            __syncthreads();
+            lds_barrier();
             if (wk == 0 && rt_ok && row < P.n) {
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
@@ -350,11 +416,60 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_kernel(MfmaParams P)
     }
 }
 
+// Streaming form: wave `wave` of workgroup b owns row-tiles (b * waves + wave),
+// + gridDim.x * waves, ... and walks all their panels; the activation window
+// stays in LDS meanwhile.  Windows that split k accumulate into y (the same
+// wave adds the same row-tile's windows in order, so the result is deterministic).
+template <int QT>
+__global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_stream_kernel(MfmaParams P) {
+    constexpr int UB = Unit<QT>::kBytes;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint8_t* lds_x = smem;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int waves = P.nwr;
+    const int j = lane & 15, grp = lane >> 4;
+    const int s_units = P.slots >> 4;
+    const int window_groups = P.window_units / s_units;
+
+    for (int tile = 0; tile < P.n_tiles; tile++) {
+        for (int wu0 = 0; wu0 < P.k_units; wu0 += P.window_units) {
+            const int wn = min(P.window_units, P.k_units - wu0);
+            if (tile != 0 || wu0 != 0) lds_barrier();
+            issue_window_copy<QT>(P.ws + ((size_t)tile * P.k_units + wu0) * UB, lds_x, wn, wave, waves, lane);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            lds_barrier();
+            const int kg0 = wu0 / s_units;
+            const int kg1 = min(P.k_groups, kg0 + window_groups);
+            for (int rt = blockIdx.x * waves + wave; rt < P.row_tiles; rt += gridDim.x * waves) {
+                float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                for (int kg = kg0; kg < kg1; kg++) {
+                    WPanel<QT> p;
+                    load_wpanel<QT>(p, P.w + (int64_t)(rt * P.k_groups + kg) * P.panel_bytes, P.slots, lane, j);
+                    const int unit0 = kg * s_units;
+                    panel_dot<QT, true>(p, lds_x + (size_t)(unit0 - wu0) * UB, min(s_units, P.k_units - unit0),
+                                        j, grp, acc);
+                }
+                const int row = rt * 16 + j;
+                if (row < P.n) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int mm = tile * 16 + grp * 4 + r;
+                        if (mm < P.m) {
+                            float* dst = P.y + (int64_t)mm * P.n + row;
+                            *dst = wu0 == 0 ? acc[r] : *dst + acc[r];
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
 } // namespace
 
 size_t qmm_gemv_mfma_workspace_bytes(const QmmLayout& L, int64_t m) {
-    XWs ws{(int)L.k_units, (int)((m + 15) / 16)};
-    return ws.xq_bytes() + ws.xd_floats(L.dtype) * sizeof(float);
+    return (size_t)((m + 15) / 16) * (size_t)L.k_units * (size_t)unit_bytes(L.dtype);
 }
 
 hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
@@ -363,59 +478,79 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     if (L.n > 0x3fffffff || L.k > 0x3fffffff || m > 0x3fffffff ||
         L.row_tiles * L.k_groups > 0x7fffffff)
         return hipErrorInvalidValue;
-    XWs ws{(int)L.k_units, (int)((m + 15) / 16)};
-    uint8_t* xq = (uint8_t*)workspace;
-    float* xd = (float*)(xq + ws.xq_bytes());
+    if (n_cus <= 0) n_cus = 1;
+    const int n_tiles = (int)((m + 15) / 16);
+    uint8_t* ws = (uint8_t*)workspace;
     {
-        int64_t threads = (int64_t)ws.n_tiles * 16 * ws.k_units * 16;
+        int64_t threads = (int64_t)n_tiles * 16 * L.k_units * 16;
         unsigned grid = (unsigned)((threads + 255) / 256);
         if (L.dtype == QMM_Q4_K)
-            quantize_ws_kernel<QMM_Q4_K><<<grid, 256, 0, stream>>>(x, (int)m, (int)L.k, ws, xq, xd);
+            quantize_ws_kernel<QMM_Q4_K><<<grid, 256, 0, stream>>>(x, (int)m, (int)L.k, (int)L.k_units, n_tiles, ws);
         else
-            quantize_ws_kernel<QMM_Q8_0><<<grid, 256, 0, stream>>>(x, (int)m, (int)L.k, ws, xq, xd);
+            quantize_ws_kernel<QMM_Q8_0><<<grid, 256, 0, stream>>>(x, (int)m, (int)L.k, (int)L.k_units, n_tiles, ws);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     MfmaParams P;
     P.w = (const uint8_t*)tiled;
-    P.xq = xq;
-    P.xd = xd;
+    P.ws = ws;
     P.y = y;
     P.m = (int)m;
     P.n = (int)L.n;
-    P.k = (int)L.k;
     P.k_units = (int)L.k_units;
     P.k_groups = (int)L.k_groups;
-    P.s = L.s;
     P.slots = L.slots;
     P.row_tiles = (int)L.row_tiles;
     P.panel_bytes = (int)L.panel_bytes;
-    P.n_tiles = ws.n_tiles;
-    P.chunk_units = (kChunkUnits / L.s) * L.s;
-    if (P.chunk_units > P.k_units) P.chunk_units = ((P.k_units + L.s - 1) / L.s) * L.s;
-    // waves along k inside a chunk, row-tiles side by side to amortize the LDS copy of x
-    int chunk_groups = P.chunk_units / L.s;
-    int nwk = chunk_groups < 4 ? chunk_groups : 4;
-    int nwr_max = kMaxWaves / nwk;
-    int64_t want = L.row_tiles / (n_cus > 0 ? n_cus : 1);
-    int nwr = (int)(want < 1 ? 1 : (want > nwr_max ? nwr_max : want));
-    P.nwk = nwk;
-    P.nwr = nwr;
-    P.wave_magic = (65536 + nwk - 1) / nwk;
-    const int waves = nwk * nwr;
-    const int xd_per_unit = XWs::xd_per_unit(L.dtype);
-    size_t lds = (size_t)P.chunk_units * kUnitBytes + (size_t)P.chunk_units * xd_per_unit * 4 +
-                 (size_t)waves * 256 * 4;
-    const void* fn = L.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_kernel<QMM_Q4_K>)
-                                         : reinterpret_cast<const void*>(&gemv_mfma_kernel<QMM_Q8_0>);
+    P.n_tiles = n_tiles;
+    P.window_units = (kWindowUnits / L.s) * L.s;
+    const int padded_units = (int)(L.k_groups * L.s);
+    if (P.window_units > padded_units) P.window_units = padded_units;
+    const size_t window_bytes = (size_t)P.window_units * unit_bytes(L.dtype);
+
+    // Every panel in flight at once needs one wave per panel of a row-tile; very tall
+    // matrices (many row-tiles per CU) amortize the activation window better when it
+    // stays resident while a wave walks whole row-tiles.
+    const bool oneshot = L.k_groups <= kMaxWaves && L.row_tiles < 8 * (int64_t)n_cus;
+    size_t lds;
+    unsigned grid;
+    int waves;
+    if (oneshot) {
+        P.nwk = (int)L.k_groups;
+        int nwr_max = kMaxWaves / P.nwk;
+        int64_t want = L.row_tiles / n_cus;
+        P.nwr = (int)(want < 1 ? 1 : (want > nwr_max ? nwr_max : want));
+        waves = P.nwk * P.nwr;
+        P.rt_groups = (int)((L.row_tiles + P.nwr - 1) / P.nwr);
+        grid = (unsigned)P.rt_groups;
+        lds = window_bytes + (size_t)waves * 256 * 4;
+    } else {
+        P.nwk = 1;
+        P.nwr = kMaxWaves;
+        waves = kMaxWaves;
+        P.rt_groups = (int)((L.row_tiles + waves - 1) / waves);
+        grid = (unsigned)(P.rt_groups < n_cus ? P.rt_groups : n_cus);
+        lds = window_bytes;
+    }
+    P.wave_magic = (65536 + P.nwk - 1) / P.nwk;
+    if (lds > 160 * 1024) return hipErrorInvalidValue;
+    const void* fn;
+    if (oneshot)
+        fn = L.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K>)
+                                 : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0>);
+    else
+        fn = L.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_stream_kernel<QMM_Q4_K>)
+                                 : reinterpret_cast<const void*>(&gemv_mfma_stream_kernel<QMM_Q8_0>);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
-    unsigned grid = (unsigned)((L.row_tiles + nwr - 1) / nwr);
-    if (L.dtype == QMM_Q4_K)
-        gemv_mfma_kernel<QMM_Q4_K><<<grid, 64 * waves, lds, stream>>>(P);
-    else
-        gemv_mfma_kernel<QMM_Q8_0><<<grid, 64 * waves, lds, stream>>>(P);
+    if (oneshot) {
+        if (L.dtype == QMM_Q4_K) gemv_mfma_oneshot_kernel<QMM_Q4_K><<<grid, 64 * waves, lds, stream>>>(P);
+        else gemv_mfma_oneshot_kernel<QMM_Q8_0><<<grid, 64 * waves, lds, stream>>>(P);
+    } else {
+        if (L.dtype == QMM_Q4_K) gemv_mfma_stream_kernel<QMM_Q4_K><<<grid, 64 * waves, lds, stream>>>(P);
+        else gemv_mfma_stream_kernel<QMM_Q8_0><<<grid, 64 * waves, lds, stream>>>(P);
+    }
     return hipGetLastError();
 }
