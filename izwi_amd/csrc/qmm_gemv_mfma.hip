@@ -234,11 +234,27 @@ __device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int
                                           float (&acc)[4]) {
     constexpr int UB = Unit<QT>::kBytes;
     const int lane8 = (grp * 16 + j) * 8;
-    if (QT == QMM_Q4_K) {
-        uint32_t sc_lo[4], sc_hi[4], mn_lo[4], mn_hi[4];
+    // Units of the panel that do not exist (ragged k, S < 4) are not skipped, which
+    // would split the arithmetic into many small blocks: they read unit 0's
+    // activations and their weight scale is multiplied by zero.  (Their header is
+    // zero padding or a copy of unit 0's, so every factor is finite.)
+    int xo[4];
+    float ef[4];
 #pragma unroll
-        for (int u = 0; u < 4; u++)
-            qmm_unpack_q4k_scales(p.hdr[u].y, p.hdr[u].z, p.hdr[u].w, sc_lo[u], sc_hi[u], mn_lo[u], mn_hi[u]);
+    for (int u = 0; u < 4; u++) {
+        const bool exists = u < n_units; // uniform
+        xo[u] = exists ? u * UB : 0;
+        ef[u] = exists ? 1.0f : 0.0f;
+    }
+    if (QT == QMM_Q4_K) {
+        // 6-bit scales of the four units (byte i of sc_lo / sc_hi = scale i / i + 4); the
+        // mins are only needed at the end and are unpacked there
+        uint32_t sc_lo[4], sc_hi[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            sc_lo[u] = p.hdr[u].y & 0x3f3f3f3fu;
+            sc_hi[u] = (p.hdr[u].w & 0x0f0f0f0fu) | (((p.hdr[u].y >> 6) & 0x03030303u) << 4);
+        }
         int isum[4][4];
 #pragma unroll
         for (int u = 0; u < 4; u++)
@@ -247,44 +263,51 @@ __device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int
 #pragma unroll
         for (int b = 0; b < 4; b++) {
             if (FIRST) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
-            // the eight MFMAs of the pair are issued back to back, their results are
-            // consumed afterwards: the matrix pipe's latency is paid once per pair
-            i32x4 dlo[4], dhi[4];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                if (u >= n_units) continue; // uniform
-                const u32x4 qq = p.q[2 * b + (u >> 1)];
-                const uint32_t w0 = (u & 1) ? qq.z : qq.x, w1 = (u & 1) ? qq.w : qq.y;
-                const uint8_t* xu = xu0 + u * UB + lane8;
-                const long a_lo = *reinterpret_cast<const long*>(xu + (2 * b) * 512);
-                const long a_hi = *reinterpret_cast<const long*>(xu + (2 * b + 1) * 512);
-                dlo[u] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, pack64(w0 & kNib, w1 & kNib),
-                                                               i32x4{0, 0, 0, 0}, 0, 0, 0);
-                dhi[u] = __builtin_amdgcn_mfma_i32_16x16x32_i8(
-                    a_hi, pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib), i32x4{0, 0, 0, 0}, 0, 0, 0);
-            }
+            for (int h = 0; h < 2; h++) {
+                // two units at a time: their four MFMAs are issued back to back and the
+                // results consumed afterwards (the matrix pipe's latency is paid once)
+                const u32x4 qq = p.q[2 * b + h];
+                i32x4 dlo[2], dhi[2];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                if (u >= n_units) continue;
-                const int sc0 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b);
-                const int sc1 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b + 1);
+                for (int e = 0; e < 2; e++) {
+                    const int u = 2 * h + e;
+                    if (u >= n_units) continue; // uniform
+                    const uint32_t w0 = e ? qq.z : qq.x, w1 = e ? qq.w : qq.y;
+                    const uint8_t* xu = xu0 + xo[u] + lane8;
+                    const long a_lo = *reinterpret_cast<const long*>(xu + (2 * b) * 512);
+                    const long a_hi = *reinterpret_cast<const long*>(xu + (2 * b + 1) * 512);
+                    dlo[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, pack64(w0 & kNib, w1 & kNib),
+                                                                   i32x4{0, 0, 0, 0}, 0, 0, 0);
+                    dhi[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(
+                        a_hi, pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib), i32x4{0, 0, 0, 0}, 0, 0, 0);
+                }
 #pragma unroll
-                for (int r = 0; r < 4; r++) // |dot| < 2^17, scale < 64
-                    isum[u][r] += __mul24(sc0, dlo[u][r]) + __mul24(sc1, dhi[u][r]);
+                for (int e = 0; e < 2; e++) {
+                    const int u = 2 * h + e;
+                    if (u >= n_units) continue;
+                    const int sc0 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b);
+                    const int sc1 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b + 1);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) // |dot| < 2^17, scale < 64
+                        isum[u][r] += __mul24(sc0, dlo[e][r]) + __mul24(sc1, dhi[e][r]);
+                }
             }
         }
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             if (u >= n_units) continue;
-            const float d = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x & 0xffffu));
-            const float dmin = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x >> 16));
+            const float d = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x & 0xffffu)) * ef[u];
+            const float dmin = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x >> 16)) * ef[u];
+            const uint32_t mn_lo = p.hdr[u].z & 0x3f3f3f3fu;
+            const uint32_t mn_hi = ((p.hdr[u].w >> 4) & 0x0f0f0f0fu) | (((p.hdr[u].z >> 6) & 0x03030303u) << 4);
             // min term: sum_s min_s * bsum_s as two MFMAs over k = sub-block index; only
             // the first 16-lane row carries data (k slots 0..7), the rest multiply zeros
-            const uint8_t* side = xu0 + u * UB + Unit<QT>::kQuant;
+            const uint8_t* side = xu0 + xo[u] + Unit<QT>::kQuant;
             const uint8_t* planes = side + 64 + j * 16;
             const long bs_lo = grp == 0 ? *reinterpret_cast<const long*>(planes) : 0L;
             const long bs_hi = grp == 0 ? *reinterpret_cast<const long*>(planes + 8) : 0L;
-            const long bmn = pack64(mn_lo[u], mn_hi[u]);
+            const long bmn = pack64(mn_lo, mn_hi);
             const i32x4 m_lo = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_lo, bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
             const i32x4 m_hi = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_hi, bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
             const float4 dx = *reinterpret_cast<const float4*>(side + grp * 16);
@@ -302,18 +325,18 @@ __device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int
             i32x4 dd[4];
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                if (u >= n_units) continue;
+                if (u >= n_units) continue; // uniform
                 const u32x4 qq = p.q[2 * b + (u >> 1)];
                 const uint32_t w0 = (u & 1) ? qq.z : qq.x, w1 = (u & 1) ? qq.w : qq.y;
-                const long a = *reinterpret_cast<const long*>(xu0 + u * UB + lane8 + b * 512);
+                const long a = *reinterpret_cast<const long*>(xu0 + xo[u] + lane8 + b * 512);
                 dd[u] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, pack64(w0, w1), i32x4{0, 0, 0, 0}, 0, 0, 0);
             }
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 if (u >= n_units) continue;
                 const uint32_t hw = b < 2 ? p.hdr[u].x : b < 4 ? p.hdr[u].y : b < 6 ? p.hdr[u].z : p.hdr[u].w;
-                const float dw = qmm_f16_bits_to_f32((uint16_t)((hw >> (16 * (b & 1))) & 0xffffu));
-                const float4 dx = *reinterpret_cast<const float4*>(xu0 + u * UB + Unit<QT>::kQuant +
+                const float dw = qmm_f16_bits_to_f32((uint16_t)((hw >> (16 * (b & 1))) & 0xffffu)) * ef[u];
+                const float4 dx = *reinterpret_cast<const float4*>(xu0 + xo[u] + Unit<QT>::kQuant +
                                                                    (b * 16 + grp * 4) * 4);
                 acc[0] += ((float)dd[u][0] * dw) * dx.x;
                 acc[1] += ((float)dd[u][1] * dw) * dx.y;
@@ -326,22 +349,28 @@ __device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int
 
 // Moves `n_units` unit records of a tile from the workspace to LDS, 1 KiB pieces
 // spread over the workgroup's waves, 16 B per lane, without passing through
-// registers.  Completion is the caller's business (vmcnt).
+// registers.  Completion is the caller's business (vmcnt, then a barrier).
+// The LDS-direct load is issued from inline assembly on purpose: for the
+// compiler's own form it conservatively waits for ALL outstanding vector loads
+// before the first LDS read that follows, which would put the whole weight panel
+// in front of the arithmetic; the callers order these copies explicitly.
 template <int QT>
 __device__ __forceinline__ void issue_window_copy(const uint8_t* __restrict__ src, uint8_t* lds, int n_units,
                                                   int wave, int waves, int lane) {
     const int bytes = n_units * Unit<QT>::kBytes; // a multiple of 64
+    const uint32_t lds_base = (uint32_t)(uintptr_t)lds; // LDS byte address (uniform)
     for (int piece = wave; piece * 1024 < bytes; piece += waves) {
         const int off = piece * 1024 + lane * 16;
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + piece * 1024);
         if (off < bytes)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + off),
-                                             (__attribute__((address_space(3))) void*)(lds + piece * 1024),
-                                             16, 0, 0);
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(src + off)
+                         : "memory", "m0");
     }
 }
 
 // One-shot form: wave (wr, wk) owns panel wk of row-tile blockIdx.x * nwr + wr.
-template <int QT>
+// SINGLE: one tile of rows and one activation window, i.e. straight-line code.
+template <int QT, bool SINGLE>
 __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaParams P) {
     constexpr int UB = Unit<QT>::kBytes;
     constexpr int NL = WPanel<QT>::QC + 4; // loads of one panel
@@ -350,7 +379,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
     float* lds_red = reinterpret_cast<float*>(smem + (size_t)P.window_units * UB); // waves * 256
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // wave-uniform by construction
     const int waves = P.nwk * P.nwr;
     const int wr = (wave * P.wave_magic) >> 16;
     const int wk = wave - wr * P.nwk;
@@ -360,6 +389,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
     const bool rt_ok = rt < P.row_tiles;
     const int unit0 = wk * s_units;                       // first unit of this wave's panel
     const int n_units = min(s_units, P.k_units - unit0);  // its units that exist (>= 1)
+    const int row = rt * 16 + j;
 
     // the first activation window goes first (loads return in order), then the panel
     const int w0_units = min(P.window_units, P.k_units);
@@ -370,26 +400,29 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory"); // the window has landed, the panel may still fly
     lds_barrier();
 
-    bool first = true;
-    for (int tile = 0; tile < P.n_tiles; tile++) {
-        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (int wu0 = 0; wu0 < P.k_units; wu0 += P.window_units) {
-            const int wn = min(P.window_units, P.k_units - wu0);
-            if (tile != 0 || wu0 != 0) {
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    bool transposed = false;
+    if (SINGLE || unit0 < w0_units) {
+        panel_dot<QT, true>(p, lds_x + (size_t)unit0 * UB, n_units, j, grp, acc);
+        transposed = true;
+    }
+    for (int tile = 0; SINGLE ? tile < 1 : tile < P.n_tiles; tile++) {
+        if (!SINGLE) {
+            for (int wu0 = tile == 0 ? P.window_units : 0; wu0 < P.k_units; wu0 += P.window_units) {
+                const int wn = min(P.window_units, P.k_units - wu0);
                 lds_barrier(); // every wave is done with the previous window
                 issue_window_copy<QT>(P.ws + ((size_t)tile * P.k_units + wu0) * UB, lds_x, wn, wave, waves, lane);
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 lds_barrier();
-            }
-            if (unit0 >= wu0 && unit0 < wu0 + wn) {
-                const uint8_t* xu0 = lds_x + (size_t)(unit0 - wu0) * UB;
-                if (first) panel_dot<QT, true>(p, xu0, n_units, j, grp, acc);
-                else panel_dot<QT, false>(p, xu0, n_units, j, grp, acc);
-                first = false;
+                if (unit0 >= wu0 && unit0 < wu0 + wn) {
+                    const uint8_t* xu0 = lds_x + (size_t)(unit0 - wu0) * UB;
+                    if (!transposed) panel_dot<QT, true>(p, xu0, n_units, j, grp, acc);
+                    else panel_dot<QT, false>(p, xu0, n_units, j, grp, acc);
+                    transposed = true;
+                }
             }
         }
         // ---- combine the waves that split k, write y[tile*16 + 4*grp + r][rt*16 + j]
-        const int row = rt * 16 + j;
         if (P.nwk == 1) {
             if (rt_ok && row < P.n) {
 #pragma unroll
@@ -413,6 +446,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
                 }
             }
         }
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[r] = 0.0f;
     }
 }
 
@@ -426,7 +461,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_stream_kernel(MfmaPa
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* lds_x = smem;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int waves = P.nwr;
     const int j = lane & 15, grp = lane >> 4;
     const int s_units = P.slots >> 4;
@@ -534,10 +569,14 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     }
     P.wave_magic = (65536 + P.nwk - 1) / P.nwk;
     if (lds > 160 * 1024) return hipErrorInvalidValue;
+    const bool single = n_tiles == 1 && L.k_units <= P.window_units;
     const void* fn;
-    if (oneshot)
-        fn = L.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K>)
-                                 : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0>);
+    if (oneshot && single)
+        fn = L.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true>)
+                                 : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, true>);
+    else if (oneshot)
+        fn = L.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false>)
+                                 : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, false>);
     else
         fn = L.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_stream_kernel<QMM_Q4_K>)
                                  : reinterpret_cast<const void*>(&gemv_mfma_stream_kernel<QMM_Q8_0>);
@@ -545,9 +584,12 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
-    if (oneshot) {
-        if (L.dtype == QMM_Q4_K) gemv_mfma_oneshot_kernel<QMM_Q4_K><<<grid, 64 * waves, lds, stream>>>(P);
-        else gemv_mfma_oneshot_kernel<QMM_Q8_0><<<grid, 64 * waves, lds, stream>>>(P);
+    if (oneshot && single) {
+        if (L.dtype == QMM_Q4_K) gemv_mfma_oneshot_kernel<QMM_Q4_K, true><<<grid, 64 * waves, lds, stream>>>(P);
+        else gemv_mfma_oneshot_kernel<QMM_Q8_0, true><<<grid, 64 * waves, lds, stream>>>(P);
+    } else if (oneshot) {
+        if (L.dtype == QMM_Q4_K) gemv_mfma_oneshot_kernel<QMM_Q4_K, false><<<grid, 64 * waves, lds, stream>>>(P);
+        else gemv_mfma_oneshot_kernel<QMM_Q8_0, false><<<grid, 64 * waves, lds, stream>>>(P);
     } else {
         if (L.dtype == QMM_Q4_K) gemv_mfma_stream_kernel<QMM_Q4_K><<<grid, 64 * waves, lds, stream>>>(P);
         else gemv_mfma_stream_kernel<QMM_Q8_0><<<grid, 64 * waves, lds, stream>>>(P);
