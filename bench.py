@@ -93,26 +93,30 @@ def time_eager(torch, fn, steps, warmup):
     return start.elapsed_time(end) / steps
 
 
-def build_decode_stack(torch, qa, oracle, dtype, m, n_layers, with_lm_head):
+def build_decode_weights(torch, qa, oracle, dtype, n_layers, with_lm_head):
     """Distinct device buffers for every projection of every layer (same seeded
-    byte content per projection kind).  Returns (calls, total_bytes, launches)."""
+    byte content per projection kind).  Returns [(QMatMul, n, k)]."""
     gg = qa.GgmlDType(dtype)
     host = {name: make_blocks(oracle, dtype, n, k, 1000 + i) for i, (name, n, k) in enumerate(LAYER_8B)}
-    xs = {k: torch.from_numpy(oracle.randn(7 + k, (m, k))).cuda() for k in (4096, 12288)}
-    calls, total = [], 0.0
+    weights = []
     for _layer in range(n_layers):
         for name, n, k in LAYER_8B:
-            mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, host[name], (n, k)))
-            y = torch.empty((m, n), dtype=torch.float32, device="cuda")
-            calls.append((mm, xs[k], y))
-            total += gemv_bytes(dtype, n, k, m)
+            weights.append((qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, host[name], (n, k))), n, k))
     if with_lm_head:
         name, n, k = LM_HEAD_8B
         blocks = make_blocks(oracle, dtype, n, k, 2000, pool_rows=16384)
-        mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, blocks, (n, k)))
+        weights.append((qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, blocks, (n, k))), n, k))
+    del host
+    return weights
+
+
+def decode_calls(torch, oracle, dtype, weights, m):
+    """(calls, algorithmic bytes) of one decode step with m activation rows."""
+    xs = {k: torch.from_numpy(oracle.randn(7 + k, (m, k))).cuda() for k in (4096, 12288)}
+    calls, total = [], 0.0
+    for mm, n, k in weights:
         calls.append((mm, xs[k], torch.empty((m, n), dtype=torch.float32, device="cuda")))
         total += gemv_bytes(dtype, n, k, m)
-    del host
     return calls, total
 
 
@@ -182,6 +186,32 @@ def prefill_extra(torch, qa, oracle, dtype, m, steps=20, warmup=5):
     return out
 
 
+def moe_extra(torch, qa, oracle, steps=20, warmup=3):
+    """Microseconds of one MoE layer (route + sort + grouped expert MLP + combine) at the
+    Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, expert intermediate 768, Q4_K."""
+    e, top_k, hidden, inter = 128, 8, 2048, 768
+    gg = qa.GgmlDType(Q4_K)
+
+    def stack(n, k, seed):
+        one = make_blocks(oracle, Q4_K, 8 * n, k, seed)  # 8 distinct experts, repeated
+        import numpy as np
+        return qa.QTensor.from_blocks(gg, np.tile(one, e // 8), (e, n, k))
+
+    experts = qa.MoeExperts(stack(inter, hidden, 31), stack(inter, hidden, 32), stack(hidden, inter, 33))
+    out = {}
+    for t in (1, 16, 512):
+        x = torch.from_numpy(oracle.randn(40 + t, (t, hidden))).cuda()
+        logits = torch.from_numpy(oracle.randn(50 + t, (t, e))).cuda()
+
+        def layer():
+            ids, wts = qa.moe_route(logits, top_k)
+            perm, offsets = qa.moe_sort(ids, e)
+            return experts.forward(x, ids, wts, perm, offsets)
+
+        out[f"t{t}"] = round(time_eager(torch, layer, steps, warmup) * 1e3, 1)
+    return out
+
+
 def measured_traffic(workload, m, avg_algorithmic):
     """HBM bytes per launch of the decode kernel from the committed rocprofv3 --pmc
     summary (profiles/decode_traffic.json: FETCH_SIZE and WRITE_SIZE per dispatch, each
@@ -236,7 +266,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    calls, total_bytes = build_decode_stack(torch, qa, oracle, dtype, args.m, args.layers, True)
+    weights = build_decode_weights(torch, qa, oracle, dtype, args.layers, True)
+    calls, total_bytes = decode_calls(torch, oracle, dtype, weights, args.m)
     launches = len(calls)
     ms, _graph = time_graph(torch, lambda: run_calls(qa, calls), args.steps, args.warmup)
     gbs = total_bytes / (ms * 1e-3) / 1e9
@@ -280,10 +311,29 @@ def main():
         },
     }
     del calls, _graph
+
+    extras = {}
+    if not args.no_extras:
+        # the same stack at the other decode batch sizes of the configuration
+        try:
+            for m in (8, 16):
+                if m == args.m:
+                    continue
+                c, tb = decode_calls(torch, oracle, dtype, weights, m)
+                t, g = time_graph(torch, lambda: run_calls(qa, c), max(5, args.steps // 5), 3)
+                extras[f"decode_gbs_m{m}"] = round(tb / (t * 1e-3) / 1e9, 1)
+                extras[f"decode_ms_per_step_m{m}"] = round(t, 4)
+                del c, g
+        except Exception as exc:  # extras never invalidate the headline number
+            extras["decode_error"] = repr(exc)
+    del weights
     torch.cuda.empty_cache()
 
     if not args.no_extras:
-        extras = {}
+        try:
+            extras["moe_30b_a3b_q4k_us"] = moe_extra(torch, qa, oracle)
+        except Exception as exc:
+            extras["moe_error"] = repr(exc)
         try:
             extras["prefill_tflops_m2048_q4k"] = prefill_extra(torch, qa, oracle, Q4_K, 2048)
             extras["prefill_tflops_m2048_q8_0"] = prefill_extra(torch, qa, oracle, Q8_0, 2048)
@@ -291,6 +341,7 @@ def main():
             extras["prefill_best_frac_of_bf16_peak"] = round(best / BF16_PEAK_TFLOPS, 4)
         except Exception as exc:  # extras never invalidate the headline number
             extras["error"] = repr(exc)
+    if extras:
         result["extras"] = extras
 
     if not args.no_cpu_baseline:

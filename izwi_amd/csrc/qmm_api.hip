@@ -82,6 +82,17 @@ int ensure_device(int device, int* n_cus) {
     return IZWI_QMM_OK;
 }
 
+// Average sorted pairs per expert from which the expert MLP runs on 16-row matrix-core
+// tiles instead of 4-row dot4 segments (IZWI_QMM_MOE_MFMA_MIN_ROWS, default 8).
+int moe_mfma_min_rows() {
+    static const int v = [] {
+        const char* s = getenv("IZWI_QMM_MOE_MFMA_MIN_ROWS");
+        int n = s ? atoi(s) : 8;
+        return n < 1 ? 1 : n;
+    }();
+    return v;
+}
+
 int type_supported(int dtype) { return dtype == IZWI_QMM_Q8_0 || dtype == IZWI_QMM_Q4_K; }
 
 int storage_bytes(int dtype, int64_t rows, int64_t cols, uint64_t* out) {
@@ -589,8 +600,6 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
     const int64_t hidden = G.k, inter = G.n;
     // every expert adds at most one partly filled segment
     const int64_t max_segments = pairs / QMM_MOE_SEG_ROWS + (pairs < n_experts ? pairs : n_experts);
-    if (max_segments > 65535)
-        return fail(IZWI_QMM_ERR_UNSUPPORTED, "t * top_k = %lld is too large for one grouped launch", (long long)pairs);
     hipStream_t stream = (hipStream_t)stream_;
     ProfileScope prof(nullptr, stream);
     Staged xi, ii, wi, pi, oi, oo;
@@ -601,24 +610,60 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
     HIP_TRY(oi.in(offsets, (size_t)(n_experts + 1) * sizeof(int32_t), mem_space));
     HIP_TRY(oo.out(out, (size_t)t * hidden * sizeof(float), mem_space));
 
+    // Many pairs per expert: 16-row tiles on the int8 matrix cores (the weights of an
+    // expert are read once for all its pairs).  Few: 4-row segments on the dot4 kernel.
+    const bool tiles = pairs >= (int64_t)moe_mfma_min_rows() * n_experts &&
+                       qmm_gemv_mfma_grouped_supported(G) && qmm_gemv_mfma_grouped_supported(D);
+    if (!tiles && max_segments > 65535)
+        return fail(IZWI_QMM_ERR_UNSUPPORTED, "t * top_k = %lld is too large for one grouped launch", (long long)pairs);
     // workspace: h [pairs, inter] | y [pairs, hidden] | seg_offsets [E + 1]
+    //            (tiles: + u [pairs, inter] | activation records)
     const size_t h_bytes = (size_t)pairs * inter * sizeof(float);
     const size_t y_bytes = (size_t)pairs * hidden * sizeof(float);
-    const size_t s_bytes = (size_t)(n_experts + 1) * sizeof(int32_t);
+    const size_t s_bytes = (((size_t)(n_experts + 1) * sizeof(int32_t)) + 255) & ~(size_t)255;
+    const int64_t max_tiles = pairs / QMM_MOE_TILE_ROWS + (pairs < n_experts ? pairs : n_experts);
+    size_t r_bytes = 0;
+    if (tiles) {
+        const size_t r1 = qmm_moe_records_bytes(G.dtype, max_tiles, hidden);
+        const size_t r2 = qmm_moe_records_bytes(D.dtype, max_tiles, inter);
+        r_bytes = r1 > r2 ? r1 : r2;
+    }
     uint8_t* ws = nullptr;
-    HIP_TRY(hipMallocAsync((void**)&ws, h_bytes + y_bytes + s_bytes, stream));
+    HIP_TRY(hipMallocAsync((void**)&ws, h_bytes + y_bytes + s_bytes + (tiles ? h_bytes + r_bytes : 0), stream));
     float* h = (float*)ws;
     float* y = (float*)(ws + h_bytes);
     int32_t* seg = (int32_t*)(ws + h_bytes + y_bytes);
-    hipError_t e = qmm_launch_moe_segments((const int32_t*)oi.dev, n_experts, seg, stream);
-    if (e == hipSuccess)
-        e = qmm_launch_gemv_grouped(G, gate->tiled, up->tiled, (const float*)xi.dev, top_k, h,
-                                    (const int32_t*)pi.dev, (const int32_t*)oi.dev, seg, n_experts,
-                                    max_segments, gate->n_cus, stream);
-    if (e == hipSuccess)
-        e = qmm_launch_gemv_grouped(D, down->tiled, nullptr, h, 1, y, (const int32_t*)pi.dev,
-                                    (const int32_t*)oi.dev, seg, n_experts, max_segments,
-                                    gate->n_cus, stream);
+    hipError_t e;
+    if (tiles) {
+        float* u = (float*)(ws + h_bytes + y_bytes + s_bytes);
+        void* records = ws + h_bytes + y_bytes + s_bytes + h_bytes;
+        const int32_t* pm = (const int32_t*)pi.dev;
+        const int32_t* of = (const int32_t*)oi.dev;
+        e = qmm_launch_moe_segments(of, n_experts, QMM_MOE_TILE_ROWS, seg, stream);
+        if (e == hipSuccess)
+            e = qmm_launch_quantize_grouped(G.dtype, (const float*)xi.dev, nullptr, top_k, hidden, pm, of, seg,
+                                            n_experts, max_tiles, records, stream);
+        if (e == hipSuccess)
+            e = qmm_launch_gemv_mfma_grouped(G, gate->tiled, records, h, pm, of, seg, n_experts, stream);
+        if (e == hipSuccess)
+            e = qmm_launch_gemv_mfma_grouped(U, up->tiled, records, u, pm, of, seg, n_experts, stream);
+        // silu(gate) * up is applied while the down projection's input is quantized
+        if (e == hipSuccess)
+            e = qmm_launch_quantize_grouped(D.dtype, h, u, 1, inter, pm, of, seg, n_experts, max_tiles,
+                                            records, stream);
+        if (e == hipSuccess)
+            e = qmm_launch_gemv_mfma_grouped(D, down->tiled, records, y, pm, of, seg, n_experts, stream);
+    } else {
+        e = qmm_launch_moe_segments((const int32_t*)oi.dev, n_experts, QMM_MOE_SEG_ROWS, seg, stream);
+        if (e == hipSuccess)
+            e = qmm_launch_gemv_grouped(G, gate->tiled, up->tiled, (const float*)xi.dev, top_k, h,
+                                        (const int32_t*)pi.dev, (const int32_t*)oi.dev, seg, n_experts,
+                                        max_segments, gate->n_cus, stream);
+        if (e == hipSuccess)
+            e = qmm_launch_gemv_grouped(D, down->tiled, nullptr, h, 1, y, (const int32_t*)pi.dev,
+                                        (const int32_t*)oi.dev, seg, n_experts, max_segments,
+                                        gate->n_cus, stream);
+    }
     if (e == hipSuccess)
         e = qmm_launch_moe_combine(y, (const float*)wi.dev, t, top_k, hidden, (float*)oo.dev, stream);
     hipError_t e2 = hipFreeAsync(ws, stream);

@@ -80,35 +80,15 @@ __device__ __forceinline__ void lds_barrier() {
 }
 
 // ---- launch 1: activation quantizer into the unit records -------------------
-// One 16-lane group per (row, unit); lane j holds elements 16j..16j+15, i.e.
-// sub-block j / 2, octets 2 (j % 2) and 2 (j % 2) + 1.
+// One 16-lane group per (row, unit); lane j holds elements 16j..16j+15 of the
+// unit in v, i.e. sub-block j / 2, octets 2 (j % 2) and 2 (j % 2) + 1.  `mr` is
+// the row inside the 16-row tile whose record starts at `rec`.
 template <int QT>
-__global__ void quantize_ws_kernel(const float* __restrict__ x, int m, int k, int k_units, int n_tiles,
-                                   uint8_t* __restrict__ ws) {
-    const int group = (blockIdx.x * blockDim.x + threadIdx.x) >> 4;
-    const int j = threadIdx.x & 15;
-    const int rows = n_tiles * 16;
-    if (group >= rows * k_units) return; // whole 16-lane groups leave together
-    const int row = group / k_units, unit = group - row * k_units;
-    const int tile = row >> 4, mr = row & 15;
-    float v[16];
-    const int k0 = unit * 256 + 16 * j;
-    {
-        // k is a multiple of 32: a 16-value run is inside the row or past its end
-        const bool in_range = row < m && k0 + 16 <= k;
-        const float4* p = reinterpret_cast<const float4*>(in_range ? x + (int64_t)row * k + k0 : x);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            float4 f = p[i];
-            v[4 * i] = in_range ? f.x : 0.0f, v[4 * i + 1] = in_range ? f.y : 0.0f;
-            v[4 * i + 2] = in_range ? f.z : 0.0f, v[4 * i + 3] = in_range ? f.w : 0.0f;
-        }
-    }
+__device__ __forceinline__ void quantize_into_record(const float (&v)[16], int j, int mr, uint8_t* rec) {
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < 16; i++) amax = fmaxf(amax, fabsf(v[i]));
     float scale_mul; // quant = round(v * scale_mul)
-    uint8_t* rec = ws + ((int64_t)tile * k_units + unit) * Unit<QT>::kBytes;
     float* side = reinterpret_cast<float*>(rec + Unit<QT>::kQuant);
     if (QT == QMM_Q4_K) {
         // BlockQ8K::from_float: iscale = -128 / (first value of largest magnitude)
@@ -163,6 +143,75 @@ __global__ void quantize_ws_kernel(const float* __restrict__ x, int m, int k, in
     *reinterpret_cast<uint2*>(dst + 128) = make_uint2(q[2], q[3]);
 }
 
+// Sixteen consecutive values of a row (k is a multiple of 32: the run is inside
+// the row or past its end), zeros when out of range.
+__device__ __forceinline__ void load_run16(const float* __restrict__ src, const float* __restrict__ safe,
+                                           bool in_range, float (&v)[16]) {
+    const float4* p = reinterpret_cast<const float4*>(in_range ? src : safe);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float4 f = p[i];
+        v[4 * i] = in_range ? f.x : 0.0f, v[4 * i + 1] = in_range ? f.y : 0.0f;
+        v[4 * i + 2] = in_range ? f.z : 0.0f, v[4 * i + 3] = in_range ? f.w : 0.0f;
+    }
+}
+
+template <int QT>
+__global__ void quantize_ws_kernel(const float* __restrict__ x, int m, int k, int k_units, int n_tiles,
+                                   uint8_t* __restrict__ ws) {
+    const int group = (blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+    const int j = threadIdx.x & 15;
+    const int rows = n_tiles * 16;
+    if (group >= rows * k_units) return; // whole 16-lane groups leave together
+    const int row = group / k_units, unit = group - row * k_units;
+    const int tile = row >> 4, mr = row & 15;
+    float v[16];
+    const int k0 = unit * 256 + 16 * j;
+    load_run16(x + (int64_t)row * k + k0, x, row < m && k0 + 16 <= k, v);
+    quantize_into_record<QT>(v, j, mr, ws + ((int64_t)tile * k_units + unit) * Unit<QT>::kBytes);
+}
+
+__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
+
+// Expert-grouped form: tile g of the list belongs to the expert e with
+// tile_offsets[e] <= g < tile_offsets[e + 1]; its row r is sorted pair
+// offsets[e] + 16 (g - tile_offsets[e]) + r (rows past the expert's end are zero),
+// pair p = perm[..] reads activation row p / x_div; with x2 the value is
+// silu(x) * x2 (the expert MLP's gate/up product feeding the down projection).
+template <int QT>
+__global__ void quantize_grouped_kernel(const float* __restrict__ x, const float* __restrict__ x2, int x_div,
+                                        int k, int k_units, const int32_t* __restrict__ perm,
+                                        const int32_t* __restrict__ offsets,
+                                        const int32_t* __restrict__ tile_offsets, int n_experts,
+                                        uint8_t* __restrict__ ws) {
+    const int64_t group = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+    const int j = threadIdx.x & 15;
+    const int64_t row = group / k_units;
+    const int unit = (int)(group - row * k_units);
+    const int tile = (int)(row >> 4), mr = (int)(row & 15);
+    if (tile >= tile_offsets[n_experts]) return; // whole 16-lane groups leave together
+    int lo = 0, hi = n_experts; // last e with tile_offsets[e] <= tile
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (tile_offsets[mid] <= tile) lo = mid;
+        else hi = mid;
+    }
+    const int pos = offsets[lo] + (tile - tile_offsets[lo]) * 16 + mr;
+    const bool row_ok = pos < offsets[lo + 1];
+    const int64_t src_row = row_ok ? perm[pos] / x_div : 0;
+    const int k0 = unit * 256 + 16 * j;
+    const bool in_range = row_ok && k0 + 16 <= k;
+    float v[16];
+    load_run16(x + src_row * k + k0, x, in_range, v);
+    if (x2 != nullptr) {
+        float u[16];
+        load_run16(x2 + src_row * k + k0, x2, in_range, u);
+#pragma unroll
+        for (int i = 0; i < 16; i++) v[i] = silu_f(v[i]) * u[i];
+    }
+    quantize_into_record<QT>(v, j, mr, ws + ((int64_t)tile * k_units + unit) * Unit<QT>::kBytes);
+}
+
 // ---- launch 2 ------------------------------------------------------------------
 struct MfmaParams {
     const uint8_t* w;
@@ -175,6 +224,11 @@ struct MfmaParams {
     int n_tiles;
     int window_units; // multiple of s, <= kWindowUnits
     int rt_groups;
+    // expert-grouped form: blockIdx.y is the expert
+    const int32_t* perm;
+    const int32_t* offsets;      // sorted pairs of expert e: [offsets[e], offsets[e + 1])
+    const int32_t* tile_offsets; // its 16-row tiles (records): [tile_offsets[e], tile_offsets[e + 1])
+    int64_t matrix_bytes;
 };
 
 // 4x4 transpose of one dword between the four 16-lane rows: on entry row u
@@ -370,7 +424,9 @@ __device__ __forceinline__ void issue_window_copy(const uint8_t* __restrict__ sr
 
 // One-shot form: wave (wr, wk) owns panel wk of row-tile blockIdx.x * nwr + wr.
 // SINGLE: one tile of rows and one activation window, i.e. straight-line code.
-template <int QT, bool SINGLE>
+// GROUPED: blockIdx.y is an expert; its weights are matrix blockIdx.y of the
+// stack, its rows the expert's tiles of sorted pairs, output row = pair index.
+template <int QT, bool SINGLE, bool GROUPED = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaParams P) {
     constexpr int UB = Unit<QT>::kBytes;
     constexpr int NL = WPanel<QT>::QC + 4; // loads of one panel
@@ -391,12 +447,26 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
     const int n_units = min(s_units, P.k_units - unit0);  // its units that exist (>= 1)
     const int row = rt * 16 + j;
 
+    const uint8_t* wbase = P.w;
+    const uint8_t* records = P.ws;
+    int n_tiles = P.n_tiles, pos_begin = 0, pos_end = 0;
+    if (GROUPED) {
+        const int e = blockIdx.y;
+        const int tile_begin = P.tile_offsets[e];
+        n_tiles = P.tile_offsets[e + 1] - tile_begin;
+        if (n_tiles == 0) return; // uniform for the workgroup: nobody reaches a barrier
+        pos_begin = P.offsets[e];
+        pos_end = P.offsets[e + 1];
+        wbase += (int64_t)e * P.matrix_bytes;
+        records += (size_t)tile_begin * P.k_units * UB;
+    }
+
     // the first activation window goes first (loads return in order), then the panel
     const int w0_units = min(P.window_units, P.k_units);
-    issue_window_copy<QT>(P.ws, lds_x, w0_units, wave, waves, lane);
+    issue_window_copy<QT>(records, lds_x, w0_units, wave, waves, lane);
     asm volatile("" ::: "memory");
     WPanel<QT> p;
-    load_wpanel<QT>(p, P.w + (int64_t)((rt_ok ? rt : 0) * P.k_groups + wk) * P.panel_bytes, P.slots, lane, j);
+    load_wpanel<QT>(p, wbase + (int64_t)((rt_ok ? rt : 0) * P.k_groups + wk) * P.panel_bytes, P.slots, lane, j);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory"); // the window has landed, the panel may still fly
     lds_barrier();
 
@@ -406,12 +476,12 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
         panel_dot<QT, true>(p, lds_x + (size_t)unit0 * UB, n_units, j, grp, acc);
         transposed = true;
     }
-    for (int tile = 0; SINGLE ? tile < 1 : tile < P.n_tiles; tile++) {
+    for (int tile = 0; SINGLE ? tile < 1 : tile < n_tiles; tile++) {
         if (!SINGLE) {
             for (int wu0 = tile == 0 ? P.window_units : 0; wu0 < P.k_units; wu0 += P.window_units) {
                 const int wn = min(P.window_units, P.k_units - wu0);
                 lds_barrier(); // every wave is done with the previous window
-                issue_window_copy<QT>(P.ws + ((size_t)tile * P.k_units + wu0) * UB, lds_x, wn, wave, waves, lane);
+                issue_window_copy<QT>(records + ((size_t)tile * P.k_units + wu0) * UB, lds_x, wn, wave, waves, lane);
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 lds_barrier();
                 if (unit0 >= wu0 && unit0 < wu0 + wn) {
@@ -423,13 +493,19 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
             }
         }
         // ---- combine the waves that split k, write y[tile*16 + 4*grp + r][rt*16 + j]
+        // (grouped: the row is a sorted position of the expert, y row its pair index)
+        auto store = [&](int r, float v) {
+            const int mm = tile * 16 + grp * 4 + r;
+            if (GROUPED) {
+                if (pos_begin + mm < pos_end) P.y[(int64_t)P.perm[pos_begin + mm] * P.n + row] = v;
+            } else if (mm < P.m) {
+                P.y[(int64_t)mm * P.n + row] = v;
+            }
+        };
         if (P.nwk == 1) {
             if (rt_ok && row < P.n) {
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const int mm = tile * 16 + grp * 4 + r;
-                    if (mm < P.m) P.y[(int64_t)mm * P.n + row] = acc[r];
-                }
+                for (int r = 0; r < 4; r++) store(r, acc[r]);
             }
         } else {
             if (tile != 0) lds_barrier(); // the previous tile's sums have been read
@@ -441,8 +517,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
                 for (int r = 0; r < 4; r++) {
                     float sum = 0.0f;
                     for (int w2 = 0; w2 < P.nwk; w2++) sum += lds_red[((wr * P.nwk + w2) * 4 + r) * 64 + lane];
-                    const int mm = tile * 16 + grp * 4 + r;
-                    if (mm < P.m) P.y[(int64_t)mm * P.n + row] = sum;
+                    store(r, sum);
                 }
             }
         }
@@ -538,6 +613,10 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     P.row_tiles = (int)L.row_tiles;
     P.panel_bytes = (int)L.panel_bytes;
     P.n_tiles = n_tiles;
+    P.perm = nullptr;
+    P.offsets = nullptr;
+    P.tile_offsets = nullptr;
+    P.matrix_bytes = 0;
     P.window_units = (kWindowUnits / L.s) * L.s;
     const int padded_units = (int)(L.k_groups * L.s);
     if (P.window_units > padded_units) P.window_units = padded_units;
@@ -594,5 +673,81 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
         if (L.dtype == QMM_Q4_K) gemv_mfma_stream_kernel<QMM_Q4_K><<<grid, 64 * waves, lds, stream>>>(P);
         else gemv_mfma_stream_kernel<QMM_Q8_0><<<grid, 64 * waves, lds, stream>>>(P);
     }
+    return hipGetLastError();
+}
+
+size_t qmm_moe_records_bytes(int dtype, int64_t max_tiles, int64_t k) {
+    return (size_t)max_tiles * (size_t)((k + 255) / 256) * (size_t)unit_bytes(dtype);
+}
+
+hipError_t qmm_launch_quantize_grouped(int dtype, const float* x, const float* x2, int x_div,
+                                       int64_t k, const int32_t* perm, const int32_t* offsets,
+                                       const int32_t* tile_offsets, int n_experts,
+                                       int64_t max_tiles, void* records, hipStream_t stream) {
+    const int64_t k_units = (k + 255) / 256;
+    const int64_t threads = max_tiles * 16 * k_units * 16;
+    if (threads <= 0) return hipSuccess;
+    if (threads > 0x7fffffff00ll || k > 0x3fffffff) return hipErrorInvalidValue;
+    const unsigned grid = (unsigned)((threads + 255) / 256);
+    if (dtype == QMM_Q4_K)
+        quantize_grouped_kernel<QMM_Q4_K><<<grid, 256, 0, stream>>>(x, x2, x_div, (int)k, (int)k_units, perm,
+                                                                    offsets, tile_offsets, n_experts,
+                                                                    (uint8_t*)records);
+    else
+        quantize_grouped_kernel<QMM_Q8_0><<<grid, 256, 0, stream>>>(x, x2, x_div, (int)k, (int)k_units, perm,
+                                                                    offsets, tile_offsets, n_experts,
+                                                                    (uint8_t*)records);
+    return hipGetLastError();
+}
+
+bool qmm_gemv_mfma_grouped_supported(const QmmLayout& L) { return L.k_groups <= kMaxWaves; }
+
+hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* records,
+                                        float* y, const int32_t* perm, const int32_t* offsets,
+                                        const int32_t* tile_offsets, int n_experts,
+                                        hipStream_t stream) {
+    if (L.n == 0 || n_experts <= 0) return hipSuccess;
+    if (!qmm_gemv_mfma_grouped_supported(L) || n_experts > 65535 || L.n > 0x3fffffff)
+        return hipErrorInvalidValue;
+    MfmaParams P;
+    P.w = (const uint8_t*)tiled;
+    P.ws = (const uint8_t*)records;
+    P.y = y;
+    P.m = 0;
+    P.n = (int)L.n;
+    P.k_units = (int)L.k_units;
+    P.k_groups = (int)L.k_groups;
+    P.slots = L.slots;
+    P.row_tiles = (int)L.row_tiles;
+    P.panel_bytes = (int)L.panel_bytes;
+    P.n_tiles = 0;
+    P.window_units = (kWindowUnits / L.s) * L.s;
+    const int padded_units = (int)(L.k_groups * L.s);
+    if (P.window_units > padded_units) P.window_units = padded_units;
+    P.nwk = (int)L.k_groups;
+    int nwr = kMaxWaves / P.nwk;
+    if (nwr > L.row_tiles) nwr = (int)L.row_tiles;
+    P.nwr = nwr;
+    P.wave_magic = (65536 + P.nwk - 1) / P.nwk;
+    P.rt_groups = (int)((L.row_tiles + nwr - 1) / nwr);
+    P.perm = perm;
+    P.offsets = offsets;
+    P.tile_offsets = tile_offsets;
+    P.matrix_bytes = L.matrix_bytes;
+    const int waves = P.nwk * P.nwr;
+    const size_t lds = (size_t)P.window_units * unit_bytes(L.dtype) + (size_t)waves * 256 * 4;
+    if (lds > 160 * 1024) return hipErrorInvalidValue;
+    const void* fn = L.dtype == QMM_Q4_K
+                         ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true>)
+                         : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, false, true>);
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+    }
+    const dim3 grid((unsigned)P.rt_groups, (unsigned)n_experts);
+    if (L.dtype == QMM_Q4_K)
+        gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true><<<grid, 64 * waves, lds, stream>>>(P);
+    else
+        gemv_mfma_oneshot_kernel<QMM_Q8_0, false, true><<<grid, 64 * waves, lds, stream>>>(P);
     return hipGetLastError();
 }

@@ -110,9 +110,29 @@ hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const 
                                    int n_experts, int64_t max_segments, int n_cus,
                                    hipStream_t stream);
 
-// seg_offsets from caller-provided offsets (same definition as in qmm_launch_moe_sort).
-hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int32_t* seg_offsets,
-                                   hipStream_t stream);
+// seg_offsets[e] = exclusive prefix sum of ceil(count(e) / seg_rows) from caller-provided offsets.
+hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int seg_rows,
+                                   int32_t* seg_offsets, hipStream_t stream);
+
+// Expert-grouped batched decode on the int8 matrix cores (many pairs per expert).
+// Sorted pairs are cut into tiles of QMM_MOE_TILE_ROWS rows that share one expert;
+// `tile_offsets` is qmm_launch_moe_segments(.., QMM_MOE_TILE_ROWS, ..).
+// Step 1 quantizes the activation rows of all tiles into `records`
+// (qmm_moe_records_bytes): row i of the sorted list is pair p = perm[i], its
+// activations are x[p / x_div] or, with x2, silu(x[p / x_div]) * x2[p / x_div].
+// Step 2 multiplies: output row y[p].
+#define QMM_MOE_TILE_ROWS 16
+size_t qmm_moe_records_bytes(int dtype, int64_t max_tiles, int64_t k);
+hipError_t qmm_launch_quantize_grouped(int dtype, const float* x, const float* x2, int x_div,
+                                       int64_t k, const int32_t* perm, const int32_t* offsets,
+                                       const int32_t* tile_offsets, int n_experts,
+                                       int64_t max_tiles, void* records, hipStream_t stream);
+// false if the matrix shape has no grouped matrix-core form (too many panels per row-tile)
+bool qmm_gemv_mfma_grouped_supported(const QmmLayout& L);
+hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* records,
+                                        float* y, const int32_t* perm, const int32_t* offsets,
+                                        const int32_t* tile_offsets, int n_experts,
+                                        hipStream_t stream);
 
 // out[t, :] = sum over slots s (in order) of weights[t, s] * y[t * top_k + s, :]
 hipError_t qmm_launch_moe_combine(const float* y, const float* weights, int64_t t, int top_k,

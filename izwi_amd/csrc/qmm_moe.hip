@@ -152,14 +152,14 @@ __global__ void sort_scatter_kernel(const int32_t* __restrict__ ids, int64_t pai
     }
 }
 
-// seg_offsets[e] = sum over e' < e of ceil(count(e') / QMM_MOE_SEG_ROWS)
-__global__ void segments_kernel(const int32_t* __restrict__ offsets, int n_experts,
+// seg_offsets[e] = sum over e' < e of ceil(count(e') / seg_rows)
+__global__ void segments_kernel(const int32_t* __restrict__ offsets, int n_experts, int seg_rows,
                                 int32_t* __restrict__ seg_offsets) {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
     int32_t seg = 0;
     for (int e = 0; e < n_experts; e++) {
         seg_offsets[e] = seg;
-        seg += (offsets[e + 1] - offsets[e] + QMM_MOE_SEG_ROWS - 1) / QMM_MOE_SEG_ROWS;
+        seg += (offsets[e + 1] - offsets[e] + seg_rows - 1) / seg_rows;
     }
     seg_offsets[n_experts] = seg;
 }
@@ -215,9 +215,9 @@ hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts,
     return hipGetLastError();
 }
 
-hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int32_t* seg_offsets,
-                                   hipStream_t stream) {
-    segments_kernel<<<1, 64, 0, stream>>>(offsets, n_experts, seg_offsets);
+hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int seg_rows,
+                                   int32_t* seg_offsets, hipStream_t stream) {
+    segments_kernel<<<1, 64, 0, stream>>>(offsets, n_experts, seg_rows, seg_offsets);
     return hipGetLastError();
 }
 

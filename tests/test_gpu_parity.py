@@ -354,3 +354,27 @@ def test_config5_moe_forward(qa, oracle, moe_weights, t):
     want = oracle.moe_forward(Q4_K, x[rows], want_ids[rows], want_wts[rows], gate, up, down, E, inter)
     assert rel_err(out[rows], want) < 1e-3
     assert np.isfinite(out).all()
+
+
+@pytest.mark.parametrize("dtype,E,hidden,inter,t,top_k", [
+    (Q8_0, 8, 512, 256, 64, 4),     # 32 pairs per expert: matrix-core tiles, Q8_0, one unit per panel
+    (Q4_K, 4, 1280, 768, 40, 2),    # ragged k (5 units), three-unit panels on the way down
+    (Q4_K, 16, 512, 512, 6, 8),     # 3 pairs per expert: 4-row segments
+])
+def test_moe_forward_small_shapes(qa, oracle, dtype, E, hidden, inter, t, top_k):
+    gate = oracle.quantize(dtype, oracle.randn(301, (E * inter, hidden), std=0.05))
+    up = oracle.quantize(dtype, oracle.randn(302, (E * inter, hidden), std=0.05))
+    down = oracle.quantize(dtype, oracle.randn(303, (E * hidden, inter), std=0.05))
+    dt = qa.GgmlDType(dtype)
+    experts = qa.MoeExperts(qa.QTensor.from_blocks(dt, gate, (E, inter, hidden)),
+                            qa.QTensor.from_blocks(dt, up, (E, inter, hidden)),
+                            qa.QTensor.from_blocks(dt, down, (E, hidden, inter)))
+    x = oracle.randn(304, (t, hidden))
+    logits = oracle.randn(305, (t, E))
+    ids, wts = qa.moe_route(torch.from_numpy(logits).cuda(), top_k)
+    perm, offsets = qa.moe_sort(ids, E)
+    out = experts.forward(torch.from_numpy(x).cuda(), ids, wts, perm, offsets).cpu().numpy()
+    want_ids, want_wts = oracle.moe_route(logits, top_k)
+    want = oracle.moe_forward(dtype, x, want_ids, want_wts, gate, up, down, E, inter)
+    assert np.array_equal(ids.cpu().numpy(), want_ids)
+    assert rel_err(out, want) < 1e-3
