@@ -187,7 +187,7 @@ def prefill_extra(torch, qa, oracle, dtype, m, steps=20, warmup=5):
 
 
 def moe_extra(torch, qa, oracle, steps=20, warmup=3):
-    """Microseconds of one MoE layer (route + sort + grouped expert MLP + combine) at the
+    """One MoE layer (route + sort + grouped expert MLP + combine, HIP-graph replay) at the
     Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, expert intermediate 768, Q4_K."""
     e, top_k, hidden, inter = 128, 8, 2048, 768
     gg = qa.GgmlDType(Q4_K)
@@ -199,16 +199,27 @@ def moe_extra(torch, qa, oracle, steps=20, warmup=3):
 
     experts = qa.MoeExperts(stack(inter, hidden, 31), stack(inter, hidden, 32), stack(hidden, inter, 33))
     out = {}
+    expert_bytes = 3 * inter * hidden * BPE[Q4_K]
     for t in (1, 16, 512):
         x = torch.from_numpy(oracle.randn(40 + t, (t, hidden))).cuda()
-        logits = torch.from_numpy(oracle.randn(50 + t, (t, e))).cuda()
+        logits_h = oracle.randn(50 + t, (t, e))
+        logits = torch.from_numpy(logits_h).cuda()
 
         def layer():
             ids, wts = qa.moe_route(logits, top_k)
             perm, offsets = qa.moe_sort(ids, e)
             return experts.forward(x, ids, wts, perm, offsets)
 
-        out[f"t{t}"] = round(time_eager(torch, layer, steps, warmup) * 1e3, 1)
+        us, g = time_graph(torch, layer, steps, warmup)
+        us *= 1e3
+        ids_h, _ = oracle.moe_route(logits_h, top_k)
+        distinct = len(set(ids_h.reshape(-1).tolist()))
+        rec = {"us": round(us, 1), "distinct_experts": distinct}
+        # algorithmic bytes: the distinct experts' weights + x in + out; flops: 3 matmuls per pair
+        rec["gbs"] = round((distinct * expert_bytes + 2 * t * hidden * 4) / us / 1e3, 1)
+        rec["tflops"] = round(2.0 * t * top_k * 3 * hidden * inter / us / 1e6, 2)
+        out[f"t{t}"] = rec
+        del g
     return out
 
 
@@ -331,7 +342,7 @@ def main():
 
     if not args.no_extras:
         try:
-            extras["moe_30b_a3b_q4k_us"] = moe_extra(torch, qa, oracle)
+            extras["moe_30b_a3b_q4k"] = moe_extra(torch, qa, oracle)
         except Exception as exc:
             extras["moe_error"] = repr(exc)
         try:

@@ -218,7 +218,8 @@ struct Staged {
 };
 
 // Scratch for kernels that need device memory beyond inputs and outputs (the
-// quantized activations of the batched decode kernel).  One buffer per
+// quantized activations of the batched decode kernels, the intermediates of the
+// expert MLP, the counting sort's histograms).  One buffer per
 // (device, stream): work on a stream is ordered, so consecutive calls may reuse
 // it; different streams never share.  It only grows; growing frees the old
 // buffer with hipFree, which waits for the device first.  Growth is not
@@ -487,13 +488,11 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
     } else {
         // prefill-sized m with f32 activations: convert once, then the MFMA kernel
         void* xb = nullptr;
-        HIP_TRY(hipMallocAsync(&xb, (size_t)m * L.k * sizeof(uint16_t), stream));
+        HIP_TRY(get_scratch(w->device, stream, (size_t)m * L.k * sizeof(uint16_t), &xb));
         hipError_t e = qmm_launch_f32_to_bf16((const float*)xi.dev, (uint16_t*)xb, m * L.k, stream);
         if (e == hipSuccess)
             e = qmm_launch_gemm_bf16(L, w->tiled, (const uint16_t*)xb, m, yo.dev, 0, w->n_cus, stream);
-        hipError_t e2 = hipFreeAsync(xb, stream);
         if (e != hipSuccess) return fail_hip(e, "prefill kernel");
-        if (e2 != hipSuccess) return fail_hip(e2, "hipFreeAsync");
     }
     HIP_TRY(yo.finish(stream));
     return IZWI_QMM_OK;
@@ -565,12 +564,10 @@ int izwi_moe_sort(const int32_t* ids, int64_t t, int32_t top_k, int32_t n_expert
     HIP_TRY(po.out(perm, (size_t)pairs * sizeof(int32_t), mem_space));
     HIP_TRY(oo.out(offsets, (size_t)(n_experts + 1) * sizeof(int32_t), mem_space));
     void* scratch = nullptr;
-    HIP_TRY(hipMallocAsync(&scratch, (size_t)qmm_moe_sort_scratch_ints(pairs, n_experts) * sizeof(int32_t), stream));
+    HIP_TRY(get_scratch(device, stream, (size_t)qmm_moe_sort_scratch_ints(pairs, n_experts) * sizeof(int32_t), &scratch));
     hipError_t e = qmm_launch_moe_sort((const int32_t*)ii.dev, pairs, n_experts, (int32_t*)po.dev,
                                        (int32_t*)oo.dev, nullptr, (int32_t*)scratch, stream);
-    hipError_t e2 = hipFreeAsync(scratch, stream);
     if (e != hipSuccess) return fail_hip(e, "sort kernels");
-    if (e2 != hipSuccess) return fail_hip(e2, "hipFreeAsync");
     HIP_TRY(po.finish(stream));
     HIP_TRY(oo.finish(stream));
     return IZWI_QMM_OK;
@@ -629,7 +626,8 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
         r_bytes = r1 > r2 ? r1 : r2;
     }
     uint8_t* ws = nullptr;
-    HIP_TRY(hipMallocAsync((void**)&ws, h_bytes + y_bytes + s_bytes + (tiles ? h_bytes + r_bytes : 0), stream));
+    HIP_TRY(get_scratch(gate->device, stream, h_bytes + y_bytes + s_bytes + (tiles ? h_bytes + r_bytes : 0),
+                        (void**)&ws));
     float* h = (float*)ws;
     float* y = (float*)(ws + h_bytes);
     int32_t* seg = (int32_t*)(ws + h_bytes + y_bytes);
@@ -666,9 +664,7 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
     }
     if (e == hipSuccess)
         e = qmm_launch_moe_combine(y, (const float*)wi.dev, t, top_k, hidden, (float*)oo.dev, stream);
-    hipError_t e2 = hipFreeAsync(ws, stream);
     if (e != hipSuccess) return fail_hip(e, "grouped expert kernels");
-    if (e2 != hipSuccess) return fail_hip(e2, "hipFreeAsync");
     if (profiling()) g_silu_fused.fetch_add(1, std::memory_order_relaxed);
     HIP_TRY(oo.finish(stream));
     return IZWI_QMM_OK;

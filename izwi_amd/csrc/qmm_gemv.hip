@@ -163,20 +163,20 @@ struct XLds {
     uint8_t* xq;  // [MT][k_units][kXUnitStride]
     float* xd;    // Q4_K: [MT][k_units]      Q8_0: [MT][k_units][8]
     int* xbs;     // Q4_K: [MT][k_units][8]   Q8_0: unused
-    float* red;   // [2][waves][G][MT][16]
+    float* red;   // [2][waves][MT][16]
 };
 
-template <int QT, int MT, int G>
+template <int QT, int MT>
 __host__ __device__ inline size_t lds_bytes(int64_t k_units, int waves) {
     size_t b = (size_t)MT * k_units * kXUnitStride;
     b += (size_t)MT * k_units * (QT == QMM_Q4_K ? 1 : 8) * sizeof(float);
     if (QT == QMM_Q4_K) b += (size_t)MT * k_units * 8 * sizeof(int);
     b = (b + 15) & ~(size_t)15;
-    b += (size_t)2 * waves * G * MT * 16 * sizeof(float);
+    b += (size_t)2 * waves * MT * 16 * sizeof(float);
     return b;
 }
 
-template <int QT, int MT, int G>
+template <int QT, int MT>
 __device__ inline XLds<QT> carve(uint8_t* base, int64_t k_units) {
     XLds<QT> l;
     l.xq = base;
@@ -364,26 +364,30 @@ static_assert(offsetof(GemvParams, k_units) == 64, "first-load fields must fill 
 __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 
 // MT rows per pass.  GATED: two weight stacks share x and the result is
-// silu(w x) * (w2 x) (the expert MLP's gate/up pair).  GROUPED: rows are sorted
+// silu(w x) * (w2 x) (the expert MLP's gate/up pair); the second half of the
+// workgroup's waves works on the second stack, so that the panels of both are
+// in flight together, and the two are combined where the k-split is summed.  GROUPED: rows are sorted
 // (token, slot) pairs of one expert.  ONESHOT: the launch gives every wave exactly
 // one panel (one pass of rows, one row-tile group per workgroup, one k step), so
 // the three loops below run once and the kernel is straight-line code from its
 // entry to the first load.
 template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
-    constexpr int G = GATED ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int wr = (wave * P.wave_magic) >> 16;
-    const int wk = wave - wr * P.nwk;
+    const int stack_waves = P.nwk * P.nwr;               // waves per weight stack
+    const int waves = GATED ? 2 * stack_waves : stack_waves; // = blockDim.x / 64, without the dispatch packet read
+    const int stack = GATED && wave >= stack_waves ? 1 : 0;
+    const int sw = wave - stack * stack_waves;
+    const int wr = (sw * P.wave_magic) >> 16;
+    const int wk = sw - wr * P.nwk;
     const bool lane_active = lane < P.slots;
     const int us = lane >> 4;
     const int k_units = (P.k + 255) >> 8, s_units = P.slots >> 4;
 
     int m_begin = 0, m_end = P.m;
-    const uint8_t* wbase = P.w;
-    const uint8_t* wbase2 = P.w2;
+    const uint8_t* wbase = stack ? P.w2 : P.w;
     if (GROUPED) {
         const int seg = blockIdx.y;
         if (seg >= P.seg_offsets[P.n_experts]) return; // uniform for the block
@@ -396,9 +400,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
         m_begin = P.offsets[lo] + (seg - P.seg_offsets[lo]) * QMM_MOE_SEG_ROWS;
         m_end = min(P.offsets[lo + 1], m_begin + QMM_MOE_SEG_ROWS);
         wbase += (int64_t)lo * P.matrix_bytes;
-        if (GATED) wbase2 += (int64_t)lo * P.matrix_bytes;
     }
-    const XLds<QT> l = carve<QT, MT, G>(smem, k_units);
+    const XLds<QT> l = carve<QT, MT>(smem, k_units);
 
     for (int m0 = m_begin; ONESHOT ? m0 == m_begin : m0 < m_end; m0 += MT) {
         bool x_ready = false;
@@ -406,11 +409,9 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
         for (int rtg = blockIdx.x; ONESHOT ? rtg == (int)blockIdx.x : rtg < P.rt_groups;
              rtg += ONESHOT ? 1 : (int)gridDim.x) {
             const int rt = rtg * P.nwr + wr;
-            float acc[G][MT];
+            float acc[MT];
 #pragma unroll
-            for (int g = 0; g < G; g++)
-#pragma unroll
-                for (int mi = 0; mi < MT; mi++) acc[g][mi] = 0.0f;
+            for (int mi = 0; mi < MT; mi++) acc[mi] = 0.0f;
             for (int ks = 0; ONESHOT ? ks < 1 : ks < P.kpw; ks++) {
                 const int kg = ks * P.nwk + wk;
                 const bool ok = rt < P.row_tiles && kg < P.k_groups;
@@ -420,7 +421,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
                 if (!x_ready) {
                     // Loads return in issue order: the small activation load goes first so
                     // that it can be consumed (quantized) while the panel loads still fly.
-                    const int group = threadIdx.x >> 4, n_groups = 4 * P.nwk * P.nwr; // = blockDim.x / 16
+                    const int group = threadIdx.x >> 4, n_groups = 4 * waves; // = blockDim.x / 16
                     const int items = MT * k_units;
                     const XSource xs{P.x, GROUPED ? P.perm : nullptr, P.x_div, m0, m_end, P.k, k_units};
                     float4 f[4];
@@ -442,57 +443,43 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
                 }
                 mask_panel<QT>(p, active);
                 const int unit = min(kg * s_units + us, k_units - 1);
-                multiply_panel<QT, MT>(p, l, unit, k_units, acc[0]);
-                if (GATED) { // the second stack reuses the panel registers
-                    load_panel<QT>(p, wbase2 + off, P.slots, lane, active);
-                    mask_panel<QT>(p, active);
-                    multiply_panel<QT, MT>(p, l, unit, k_units, acc[G - 1]);
-                }
+                multiply_panel<QT, MT>(p, l, unit, k_units, acc);
             }
             // row-tile finished: combine the S units of a row, then the waves that split k
 #pragma unroll
-            for (int g = 0; g < G; g++)
-#pragma unroll
-                for (int mi = 0; mi < MT; mi++) {
-                    acc[g][mi] += __shfl_xor(acc[g][mi], 16);
-                    acc[g][mi] += __shfl_xor(acc[g][mi], 32);
-                }
-            if (P.nwk == 1) {
+            for (int mi = 0; mi < MT; mi++) {
+                acc[mi] += __shfl_xor(acc[mi], 16);
+                acc[mi] += __shfl_xor(acc[mi], 32);
+            }
+            if (P.nwk == 1 && !GATED) {
                 const int row = rt * 16 + lane;
                 if (lane < 16 && rt < P.row_tiles && row < P.n) {
 #pragma unroll
                     for (int mi = 0; mi < MT; mi++) {
                         if (m0 + mi < m_end) {
                             int64_t yr = GROUPED ? P.perm[m0 + mi] : m0 + mi;
-                            float v = GATED ? silu(acc[0][mi]) * acc[G - 1][mi] : acc[0][mi];
-                            P.y[yr * P.n + row] = v;
+                            P.y[yr * P.n + row] = acc[mi];
                         }
                     }
                 }
             } else {
-                const int waves = P.nwk * P.nwr; // = blockDim.x / 64, without the dispatch packet read
-                float* red = l.red + red_buf * (waves * G * MT * 16);
+                float* red = l.red + red_buf * (waves * MT * 16);
                 if (lane < 16) {
 #pragma unroll
-                    for (int g = 0; g < G; g++)
-#pragma unroll
-                        for (int mi = 0; mi < MT; mi++)
-                            red[((wave * G + g) * MT + mi) * 16 + lane] = acc[g][mi];
+                    for (int mi = 0; mi < MT; mi++) red[(wave * MT + mi) * 16 + lane] = acc[mi];
                 }
                 __syncthreads();
-                if (wk == 0 && lane < 16 * MT) {
+                if (wk == 0 && stack == 0 && lane < 16 * MT) {
                     const int mi = lane >> 4, r = lane & 15;
-                    float sum[G];
-#pragma unroll
-                    for (int g = 0; g < G; g++) {
-                        sum[g] = 0.0f;
-                        for (int w2 = 0; w2 < P.nwk; w2++)
-                            sum[g] += red[(((wr * P.nwk + w2) * G + g) * MT + mi) * 16 + r];
+                    float sum = 0.0f, sum2 = 0.0f;
+                    for (int w2 = 0; w2 < P.nwk; w2++) {
+                        sum += red[((wr * P.nwk + w2) * MT + mi) * 16 + r];
+                        if (GATED) sum2 += red[((stack_waves + wr * P.nwk + w2) * MT + mi) * 16 + r];
                     }
                     const int row = rt * 16 + r;
                     if (rt < P.row_tiles && row < P.n && m0 + mi < m_end) {
                         int64_t yr = GROUPED ? P.perm[m0 + mi] : m0 + mi;
-                        P.y[yr * P.n + row] = GATED ? silu(sum[0]) * sum[G - 1] : sum[0];
+                        P.y[yr * P.n + row] = GATED ? silu(sum) * sum2 : sum;
                     }
                 }
                 red_buf ^= 1;
@@ -506,9 +493,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
 // flight at once, times as many row-tiles side by side as still leave one
 // workgroup per CU: the activations are quantized once per workgroup, so
 // taller workgroups amortize that work and its L2 traffic.
-void choose_split(const QmmLayout& L, int n_cus, int grid_y, GemvParams& P, int& waves) {
-    int nwk = (int)(L.k_groups < kMaxWaves ? L.k_groups : kMaxWaves);
-    int nwr_max = kMaxWaves / nwk;
+void choose_split(const QmmLayout& L, int n_cus, int grid_y, bool gated, GemvParams& P, int& waves) {
+    const int budget = gated ? kMaxWaves / 2 : kMaxWaves; // waves per weight stack
+    int nwk = (int)(L.k_groups < budget ? L.k_groups : budget);
+    int nwr_max = budget / nwk;
     int64_t want = L.row_tiles * grid_y / (n_cus > 0 ? n_cus : 1);
     int nwr = (int)(want < 1 ? 1 : (want > nwr_max ? nwr_max : want));
     if (grid_y == 1 && L.row_tiles >= 16 * (int64_t)n_cus) {
@@ -526,7 +514,8 @@ void choose_split(const QmmLayout& L, int n_cus, int grid_y, GemvParams& P, int&
 
 template <int QT, int MT, bool GATED, bool GROUPED>
 hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipStream_t stream) {
-    size_t lds = lds_bytes<QT, MT, GATED ? 2 : 1>(P.k_units, waves);
+    const int all_waves = GATED ? 2 * waves : waves;
+    size_t lds = lds_bytes<QT, MT>(P.k_units, all_waves);
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     int64_t cap = (int64_t)n_cus * 32;
     if (grid_y > 1) cap = cap / grid_y > 64 ? cap / grid_y : 64;
@@ -539,7 +528,7 @@ hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipS
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
-    const dim3 g((unsigned)grid, (unsigned)grid_y), b(64 * waves);
+    const dim3 g((unsigned)grid, (unsigned)grid_y), b(64 * all_waves);
     if (oneshot)
         gemv_kernel<QT, MT, GATED, GROUPED, !GROUPED && !GATED><<<g, b, lds, stream>>>(P);
     else
@@ -551,8 +540,8 @@ template <int QT>
 hipError_t launch_plain(const GemvParams& P, int waves, int n_cus, hipStream_t stream) {
     // the widest row tile whose quantized activations fit comfortably in LDS
     int mt = P.m >= 3 ? 4 : (P.m == 2 ? 2 : 1);
-    if (mt == 4 && lds_bytes<QT, 4, 1>(P.k_units, waves) > 64 * 1024) mt = 2;
-    if (mt == 2 && lds_bytes<QT, 2, 1>(P.k_units, waves) > 64 * 1024) mt = 1;
+    if (mt == 4 && lds_bytes<QT, 4>(P.k_units, waves) > 64 * 1024) mt = 2;
+    if (mt == 2 && lds_bytes<QT, 2>(P.k_units, waves) > 64 * 1024) mt = 1;
     if (mt == 4) return launch_mt<QT, 4, false, false>(P, waves, n_cus, 1, stream);
     if (mt == 2) return launch_mt<QT, 2, false, false>(P, waves, n_cus, 1, stream);
     return launch_mt<QT, 1, false, false>(P, waves, n_cus, 1, stream);
@@ -641,7 +630,7 @@ hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x
     GemvParams P;
     if (!make_params(L, tiled, x, m, y, P)) return hipErrorInvalidValue;
     int waves;
-    choose_split(L, n_cus, 1, P, waves);
+    choose_split(L, n_cus, 1, false, P, waves);
     return L.dtype == QMM_Q4_K ? launch_plain<QMM_Q4_K>(P, waves, n_cus, stream)
                                : launch_plain<QMM_Q8_0>(P, waves, n_cus, stream);
 }
@@ -661,9 +650,9 @@ hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const 
     P.seg_offsets = seg_offsets;
     P.n_experts = n_experts;
     P.x_div = x_div;
-    int waves;
-    choose_split(L, n_cus, (int)max_segments, P, waves);
     const bool gated = tiled2 != nullptr;
+    int waves;
+    choose_split(L, n_cus, (int)max_segments, gated, P, waves);
     if (L.dtype == QMM_Q4_K)
         return gated ? launch_mt<QMM_Q4_K, 2, true, true>(P, waves, n_cus, (int)max_segments, stream)
                      : launch_mt<QMM_Q4_K, 4, false, true>(P, waves, n_cus, (int)max_segments, stream);

@@ -152,16 +152,30 @@ __global__ void sort_scatter_kernel(const int32_t* __restrict__ ids, int64_t pai
     }
 }
 
-// seg_offsets[e] = sum over e' < e of ceil(count(e') / seg_rows)
+// seg_offsets[e] = sum over e' < e of ceil(count(e') / seg_rows).  One block:
+// every thread sums a contiguous run of experts, the runs are scanned in LDS.
 __global__ void segments_kernel(const int32_t* __restrict__ offsets, int n_experts, int seg_rows,
                                 int32_t* __restrict__ seg_offsets) {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    int32_t seg = 0;
-    for (int e = 0; e < n_experts; e++) {
-        seg_offsets[e] = seg;
-        seg += (offsets[e + 1] - offsets[e] + seg_rows - 1) / seg_rows;
+    __shared__ int32_t part[256];
+    const int per = (n_experts + 255) / 256;
+    const int e0 = min(n_experts, (int)threadIdx.x * per), e1 = min(n_experts, e0 + per);
+    int32_t sum = 0;
+    for (int e = e0; e < e1; e++) sum += (offsets[e + 1] - offsets[e] + seg_rows - 1) / seg_rows;
+    part[threadIdx.x] = sum;
+    __syncthreads();
+    // inclusive scan over the 256 partial sums (integers: any order gives the same result)
+    for (int d = 1; d < 256; d <<= 1) {
+        const int32_t add = threadIdx.x >= (unsigned)d ? part[threadIdx.x - d] : 0;
+        __syncthreads();
+        part[threadIdx.x] += add;
+        __syncthreads();
     }
-    seg_offsets[n_experts] = seg;
+    int32_t run = part[threadIdx.x] - sum;
+    for (int e = e0; e < e1; e++) {
+        seg_offsets[e] = run;
+        run += (offsets[e + 1] - offsets[e] + seg_rows - 1) / seg_rows;
+    }
+    if (threadIdx.x == 255) seg_offsets[n_experts] = part[255];
 }
 
 __global__ void combine_kernel(const float* __restrict__ y, const float* __restrict__ weights,
@@ -217,7 +231,7 @@ hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts,
 
 hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int seg_rows,
                                    int32_t* seg_offsets, hipStream_t stream) {
-    segments_kernel<<<1, 64, 0, stream>>>(offsets, n_experts, seg_rows, seg_offsets);
+    segments_kernel<<<1, 256, 0, stream>>>(offsets, n_experts, seg_rows, seg_offsets);
     return hipGetLastError();
 }
 
