@@ -626,7 +626,8 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
         r_bytes = r1 > r2 ? r1 : r2;
     }
     uint8_t* ws = nullptr;
-    HIP_TRY(get_scratch(gate->device, stream, h_bytes + y_bytes + s_bytes + (tiles ? h_bytes + r_bytes : 0),
+    HIP_TRY(get_scratch(gate->device, stream,
+                        h_bytes + y_bytes + s_bytes + (tiles ? h_bytes + r_bytes : (size_t)max_segments * 4),
                         (void**)&ws));
     float* h = (float*)ws;
     float* y = (float*)(ws + h_bytes);
@@ -637,7 +638,7 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
         void* records = ws + h_bytes + y_bytes + s_bytes + h_bytes;
         const int32_t* pm = (const int32_t*)pi.dev;
         const int32_t* of = (const int32_t*)oi.dev;
-        e = qmm_launch_moe_segments(of, n_experts, QMM_MOE_TILE_ROWS, seg, stream);
+        e = qmm_launch_moe_segments(of, n_experts, QMM_MOE_TILE_ROWS, seg, nullptr, 0, stream);
         if (e == hipSuccess)
             e = qmm_launch_quantize_grouped(G.dtype, (const float*)xi.dev, nullptr, top_k, hidden, pm, of, seg,
                                             n_experts, max_tiles, records, stream);
@@ -652,14 +653,16 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
         if (e == hipSuccess)
             e = qmm_launch_gemv_mfma_grouped(D, down->tiled, records, y, pm, of, seg, n_experts, stream);
     } else {
-        e = qmm_launch_moe_segments((const int32_t*)oi.dev, n_experts, QMM_MOE_SEG_ROWS, seg, stream);
+        int32_t* seg_expert = (int32_t*)(ws + h_bytes + y_bytes + s_bytes);
+        e = qmm_launch_moe_segments((const int32_t*)oi.dev, n_experts, QMM_MOE_SEG_ROWS, seg, seg_expert,
+                                    max_segments, stream);
         if (e == hipSuccess)
             e = qmm_launch_gemv_grouped(G, gate->tiled, up->tiled, (const float*)xi.dev, top_k, h,
-                                        (const int32_t*)pi.dev, (const int32_t*)oi.dev, seg, n_experts,
-                                        max_segments, gate->n_cus, stream);
+                                        (const int32_t*)pi.dev, (const int32_t*)oi.dev, seg, seg_expert,
+                                        n_experts, max_segments, gate->n_cus, stream);
         if (e == hipSuccess)
             e = qmm_launch_gemv_grouped(D, down->tiled, nullptr, h, 1, y, (const int32_t*)pi.dev,
-                                        (const int32_t*)oi.dev, seg, n_experts, max_segments,
+                                        (const int32_t*)oi.dev, seg, seg_expert, n_experts, max_segments,
                                         gate->n_cus, stream);
     }
     if (e == hipSuccess)

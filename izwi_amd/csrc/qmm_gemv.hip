@@ -356,6 +356,7 @@ struct GemvParams {
     const int32_t* perm;
     const int32_t* offsets;     // [n_experts + 1]
     const int32_t* seg_offsets; // [n_experts + 1]
+    const int32_t* seg_expert;  // [max segments]: expert of the segment, -1 past the last
     int n_experts;
     int x_div; // x row of pair p is p / x_div
 };
@@ -390,13 +391,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
     const uint8_t* wbase = stack ? P.w2 : P.w;
     if (GROUPED) {
         const int seg = blockIdx.y;
-        if (seg >= P.seg_offsets[P.n_experts]) return; // uniform for the block
-        int lo = 0, hi = P.n_experts; // last e with seg_offsets[e] <= seg
-        while (hi - lo > 1) {
-            int mid = (lo + hi) >> 1;
-            if (P.seg_offsets[mid] <= seg) lo = mid;
-            else hi = mid;
-        }
+        const int lo = P.seg_expert[seg]; // uniform for the block
+        if (lo < 0) return;               // past the last segment
         m_begin = P.offsets[lo] + (seg - P.seg_offsets[lo]) * QMM_MOE_SEG_ROWS;
         m_end = min(P.offsets[lo + 1], m_begin + QMM_MOE_SEG_ROWS);
         wbase += (int64_t)lo * P.matrix_bytes;
@@ -494,7 +490,11 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
 // workgroup per CU: the activations are quantized once per workgroup, so
 // taller workgroups amortize that work and its L2 traffic.
 void choose_split(const QmmLayout& L, int n_cus, int grid_y, bool gated, GemvParams& P, int& waves) {
-    const int budget = gated ? kMaxWaves / 2 : kMaxWaves; // waves per weight stack
+    // Waves per weight stack.  The grouped (expert) launches run many short workgroups
+    // one after the other on a CU: small workgroups fill the wave slots that the
+    // register count leaves (several side by side, one loads while another multiplies).
+    const int total = grid_y > 1 ? 4 : kMaxWaves;
+    const int budget = gated ? total / 2 : total;
     int nwk = (int)(L.k_groups < budget ? L.k_groups : budget);
     int nwr_max = budget / nwk;
     int64_t want = L.row_tiles * grid_y / (n_cus > 0 ? n_cus : 1);
@@ -521,8 +521,11 @@ hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipS
     if (grid_y > 1) cap = cap / grid_y > 64 ? cap / grid_y : 64;
     int64_t grid = P.rt_groups < cap ? P.rt_groups : cap;
     if (grid < 1) grid = 1;
-    const bool oneshot = !GROUPED && !GATED && P.m <= MT && P.kpw == 1 && grid == P.rt_groups;
-    const void* fn = oneshot ? reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, !GROUPED && !GATED>)
+    // straight-line form: one pass of rows (a segment never has more than MT rows in the
+    // grouped form), one row-tile group per workgroup, one k step
+    constexpr bool kCanOneshot = GROUPED ? MT == QMM_MOE_SEG_ROWS : !GATED;
+    const bool oneshot = kCanOneshot && (GROUPED || P.m <= MT) && P.kpw == 1 && grid == P.rt_groups;
+    const void* fn = oneshot ? reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot>)
                              : reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, false>);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -530,7 +533,7 @@ hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipS
     }
     const dim3 g((unsigned)grid, (unsigned)grid_y), b(64 * all_waves);
     if (oneshot)
-        gemv_kernel<QT, MT, GATED, GROUPED, !GROUPED && !GATED><<<g, b, lds, stream>>>(P);
+        gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot><<<g, b, lds, stream>>>(P);
     else
         gemv_kernel<QT, MT, GATED, GROUPED, false><<<g, b, lds, stream>>>(P);
     return hipGetLastError();
@@ -570,6 +573,7 @@ bool make_params(const QmmLayout& L, const void* tiled, const float* x, int64_t 
     P.perm = nullptr;
     P.offsets = nullptr;
     P.seg_offsets = nullptr;
+    P.seg_expert = nullptr;
     P.n_experts = 0;
     P.x_div = 1;
     return true;
@@ -638,8 +642,8 @@ hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x
 hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
                                    const float* x, int x_div, float* y, const int32_t* perm,
                                    const int32_t* offsets, const int32_t* seg_offsets,
-                                   int n_experts, int64_t max_segments, int n_cus,
-                                   hipStream_t stream) {
+                                   const int32_t* seg_expert, int n_experts, int64_t max_segments,
+                                   int n_cus, hipStream_t stream) {
     if (max_segments <= 0 || L.n == 0) return hipSuccess;
     if (max_segments > 65535) return hipErrorInvalidValue;
     GemvParams P;
@@ -648,15 +652,16 @@ hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const 
     P.perm = perm;
     P.offsets = offsets;
     P.seg_offsets = seg_offsets;
+    P.seg_expert = seg_expert;
     P.n_experts = n_experts;
     P.x_div = x_div;
     const bool gated = tiled2 != nullptr;
     int waves;
     choose_split(L, n_cus, (int)max_segments, gated, P, waves);
     if (L.dtype == QMM_Q4_K)
-        return gated ? launch_mt<QMM_Q4_K, 2, true, true>(P, waves, n_cus, (int)max_segments, stream)
+        return gated ? launch_mt<QMM_Q4_K, 4, true, true>(P, waves, n_cus, (int)max_segments, stream)
                      : launch_mt<QMM_Q4_K, 4, false, true>(P, waves, n_cus, (int)max_segments, stream);
-    return gated ? launch_mt<QMM_Q8_0, 2, true, true>(P, waves, n_cus, (int)max_segments, stream)
+    return gated ? launch_mt<QMM_Q8_0, 4, true, true>(P, waves, n_cus, (int)max_segments, stream)
                  : launch_mt<QMM_Q8_0, 4, false, true>(P, waves, n_cus, (int)max_segments, stream);
 }
 

@@ -107,12 +107,15 @@ int64_t qmm_moe_sort_scratch_ints(int64_t pairs, int n_experts);
 hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
                                    const float* x, int x_div, float* y, const int32_t* perm,
                                    const int32_t* offsets, const int32_t* seg_offsets,
-                                   int n_experts, int64_t max_segments, int n_cus,
-                                   hipStream_t stream);
+                                   const int32_t* seg_expert, int n_experts, int64_t max_segments,
+                                   int n_cus, hipStream_t stream);
 
-// seg_offsets[e] = exclusive prefix sum of ceil(count(e) / seg_rows) from caller-provided offsets.
+// seg_offsets[e] = exclusive prefix sum of ceil(count(e) / seg_rows) from caller-provided
+// offsets; seg_expert (may be NULL; max_segments ints) = the expert of every segment, -1
+// past the last one.
 hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int seg_rows,
-                                   int32_t* seg_offsets, hipStream_t stream);
+                                   int32_t* seg_offsets, int32_t* seg_expert, int64_t max_segments,
+                                   hipStream_t stream);
 
 // Expert-grouped batched decode on the int8 matrix cores (many pairs per expert).
 // Sorted pairs are cut into tiles of QMM_MOE_TILE_ROWS rows that share one expert;

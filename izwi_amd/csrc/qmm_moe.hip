@@ -154,8 +154,11 @@ __global__ void sort_scatter_kernel(const int32_t* __restrict__ ids, int64_t pai
 
 // seg_offsets[e] = sum over e' < e of ceil(count(e') / seg_rows).  One block:
 // every thread sums a contiguous run of experts, the runs are scanned in LDS.
+// With seg_expert: seg_expert[s] = expert of segment s, -1 for s past the last
+// segment (up to max_segments entries).
 __global__ void segments_kernel(const int32_t* __restrict__ offsets, int n_experts, int seg_rows,
-                                int32_t* __restrict__ seg_offsets) {
+                                int32_t* __restrict__ seg_offsets, int32_t* __restrict__ seg_expert,
+                                int max_segments) {
     __shared__ int32_t part[256];
     const int per = (n_experts + 255) / 256;
     const int e0 = min(n_experts, (int)threadIdx.x * per), e1 = min(n_experts, e0 + per);
@@ -173,9 +176,15 @@ __global__ void segments_kernel(const int32_t* __restrict__ offsets, int n_exper
     int32_t run = part[threadIdx.x] - sum;
     for (int e = e0; e < e1; e++) {
         seg_offsets[e] = run;
-        run += (offsets[e + 1] - offsets[e] + seg_rows - 1) / seg_rows;
+        const int32_t n = (offsets[e + 1] - offsets[e] + seg_rows - 1) / seg_rows;
+        if (seg_expert)
+            for (int32_t i = 0; i < n && run + i < max_segments; i++) seg_expert[run + i] = e;
+        run += n;
     }
-    if (threadIdx.x == 255) seg_offsets[n_experts] = part[255];
+    const int32_t total = part[255];
+    if (threadIdx.x == 255) seg_offsets[n_experts] = total;
+    if (seg_expert)
+        for (int s = total + threadIdx.x; s < max_segments; s += 256) seg_expert[s] = -1;
 }
 
 __global__ void combine_kernel(const float* __restrict__ y, const float* __restrict__ weights,
@@ -230,8 +239,10 @@ hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts,
 }
 
 hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int seg_rows,
-                                   int32_t* seg_offsets, hipStream_t stream) {
-    segments_kernel<<<1, 256, 0, stream>>>(offsets, n_experts, seg_rows, seg_offsets);
+                                   int32_t* seg_offsets, int32_t* seg_expert, int64_t max_segments,
+                                   hipStream_t stream) {
+    segments_kernel<<<1, 256, 0, stream>>>(offsets, n_experts, seg_rows, seg_offsets, seg_expert,
+                                           (int)max_segments);
     return hipGetLastError();
 }
 
