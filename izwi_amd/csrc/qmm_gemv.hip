@@ -372,9 +372,9 @@ __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 // one panel (one pass of rows, one row-tile group per workgroup, one k step), so
 // the three loops below run once and the kernel is straight-line code from its
 // entry to the first load.
-template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false>
-__global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT>
+__device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int m_end, int64_t w_offset,
+                                          uint8_t* smem) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int stack_waves = P.nwk * P.nwr;               // waves per weight stack
@@ -386,17 +386,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
     const bool lane_active = lane < P.slots;
     const int us = lane >> 4;
     const int k_units = (P.k + 255) >> 8, s_units = P.slots >> 4;
-
-    int m_begin = 0, m_end = P.m;
-    const uint8_t* wbase = stack ? P.w2 : P.w;
-    if (GROUPED) {
-        const int seg = blockIdx.y;
-        const int lo = P.seg_expert[seg]; // uniform for the block
-        if (lo < 0) return;               // past the last segment
-        m_begin = P.offsets[lo] + (seg - P.seg_offsets[lo]) * QMM_MOE_SEG_ROWS;
-        m_end = min(P.offsets[lo + 1], m_begin + QMM_MOE_SEG_ROWS);
-        wbase += (int64_t)lo * P.matrix_bytes;
-    }
+    const uint8_t* wbase = (stack ? P.w2 : P.w) + w_offset;
     const XLds<QT> l = carve<QT, MT>(smem, k_units);
 
     for (int m0 = m_begin; ONESHOT ? m0 == m_begin : m0 < m_end; m0 += MT) {
@@ -481,6 +471,33 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
                 red_buf ^= 1;
             }
         }
+    }
+}
+
+// The grouped straight-line form picks the row count of its segment (1, 2 or up to
+// QMM_MOE_SEG_ROWS rows; uniform for the workgroup) at run time: most segments of a
+// small batch hold one or two pairs, and a row costs its share of the arithmetic
+// whether it exists or not.
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false>
+__global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int m_begin = 0, m_end = P.m;
+    int64_t w_offset = 0;
+    if (GROUPED) {
+        const int seg = blockIdx.y;
+        const int lo = P.seg_expert[seg]; // uniform for the block
+        if (lo < 0) return;               // past the last segment
+        m_begin = P.offsets[lo] + (seg - P.seg_offsets[lo]) * QMM_MOE_SEG_ROWS;
+        m_end = min(P.offsets[lo + 1], m_begin + QMM_MOE_SEG_ROWS);
+        w_offset = (int64_t)lo * P.matrix_bytes;
+    }
+    if (GROUPED && ONESHOT && MT == 4) {
+        const int rows = m_end - m_begin;
+        if (rows == 1) gemv_body<QT, 1, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_offset, smem);
+        else if (rows == 2) gemv_body<QT, 2, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_offset, smem);
+        else gemv_body<QT, 4, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_offset, smem);
+    } else {
+        gemv_body<QT, MT, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_offset, smem);
     }
 }
 
