@@ -643,15 +643,15 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
             e = qmm_launch_quantize_grouped(G.dtype, (const float*)xi.dev, nullptr, top_k, hidden, pm, of, seg,
                                             n_experts, max_tiles, records, stream);
         if (e == hipSuccess)
-            e = qmm_launch_gemv_mfma_grouped(G, gate->tiled, records, h, pm, of, seg, n_experts, stream);
-        if (e == hipSuccess)
-            e = qmm_launch_gemv_mfma_grouped(U, up->tiled, records, u, pm, of, seg, n_experts, stream);
+            e = qmm_launch_gemv_mfma_grouped(G, gate->tiled, up->tiled, records, h, u, pm, of, seg, n_experts,
+                                             stream);
         // silu(gate) * up is applied while the down projection's input is quantized
         if (e == hipSuccess)
             e = qmm_launch_quantize_grouped(D.dtype, h, u, 1, inter, pm, of, seg, n_experts, max_tiles,
                                             records, stream);
         if (e == hipSuccess)
-            e = qmm_launch_gemv_mfma_grouped(D, down->tiled, records, y, pm, of, seg, n_experts, stream);
+            e = qmm_launch_gemv_mfma_grouped(D, down->tiled, nullptr, records, y, nullptr, pm, of, seg,
+                                             n_experts, stream);
     } else {
         int32_t* seg_expert = (int32_t*)(ws + h_bytes + y_bytes + s_bytes);
         e = qmm_launch_moe_segments((const int32_t*)oi.dev, n_experts, QMM_MOE_SEG_ROWS, seg, seg_expert,

@@ -217,6 +217,9 @@ struct MfmaParams {
     const uint8_t* w;
     const uint8_t* ws; // unit records [n_tiles][k_units]
     float* y;
+    const uint8_t* w2; // grouped form, blockIdx.z == 1: second stack and its output
+    float* y2;
+    int double_buf;    // two LDS windows
     int m, n;
     int k_units, k_groups, slots;
     int row_tiles, panel_bytes;
@@ -432,7 +435,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
     constexpr int NL = WPanel<QT>::QC + 4; // loads of one panel
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* lds_x = smem;                                                       // window_units * UB
-    float* lds_red = reinterpret_cast<float*>(smem + (size_t)P.window_units * UB); // waves * 256
+    float* lds_red = reinterpret_cast<float*>(smem + (size_t)(P.double_buf ? 2 : 1) * P.window_units * UB); // waves * 256
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // wave-uniform by construction
@@ -449,9 +452,11 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
 
     const uint8_t* wbase = P.w;
     const uint8_t* records = P.ws;
+    float* yout = P.y;
     int n_tiles = P.n_tiles, pos_begin = 0, pos_end = 0;
     if (GROUPED) {
         const int e = blockIdx.y;
+        if (blockIdx.z != 0) wbase = P.w2, yout = P.y2; // second weight stack on the same activations
         const int tile_begin = P.tile_offsets[e];
         n_tiles = P.tile_offsets[e + 1] - tile_begin;
         if (n_tiles == 0) return; // uniform for the workgroup: nobody reaches a barrier
@@ -471,58 +476,82 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
     lds_barrier();
 
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    // (row tile, window) stages in order; with two LDS buffers the next stage's window is
+    // copied while this one is multiplied
+    const int n_win = SINGLE ? 1 : (P.k_units + P.window_units - 1) / P.window_units;
+    const int n_stages = SINGLE ? 1 : n_tiles * n_win;
+    const size_t buf_bytes = (size_t)P.window_units * UB;
     bool transposed = false;
-    if (SINGLE || unit0 < w0_units) {
-        panel_dot<QT, true>(p, lds_x + (size_t)unit0 * UB, n_units, j, grp, acc);
-        transposed = true;
-    }
-    for (int tile = 0; SINGLE ? tile < 1 : tile < n_tiles; tile++) {
-        if (!SINGLE) {
-            for (int wu0 = tile == 0 ? P.window_units : 0; wu0 < P.k_units; wu0 += P.window_units) {
-                const int wn = min(P.window_units, P.k_units - wu0);
-                lds_barrier(); // every wave is done with the previous window
-                issue_window_copy<QT>(records + ((size_t)tile * P.k_units + wu0) * UB, lds_x, wn, wave, waves, lane);
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    int tile = 0, win = 0;
+    for (int s = 0; s < n_stages; s++) {
+        const int wu0 = win * P.window_units;
+        const int wn = min(P.window_units, P.k_units - wu0);
+        uint8_t* cur = lds_x + (P.double_buf ? (s & 1) * buf_bytes : 0);
+        int ntile = tile, nwin = win + 1;
+        if (nwin == n_win) nwin = 0, ntile = tile + 1;
+        const bool more = !SINGLE && s + 1 < n_stages;
+        const uint8_t* next_src = records + ((size_t)ntile * P.k_units + (size_t)nwin * P.window_units) * UB;
+        const int next_n = min(P.window_units, P.k_units - nwin * P.window_units);
+        if (more && P.double_buf)
+            issue_window_copy<QT>(next_src, lds_x + ((s + 1) & 1) * buf_bytes, next_n, wave, waves, lane);
+        if (SINGLE || (unit0 >= wu0 && unit0 < wu0 + wn)) {
+            const uint8_t* xu0 = cur + (size_t)(unit0 - wu0) * UB;
+            if (SINGLE) {
+                panel_dot<QT, true>(p, xu0, n_units, j, grp, acc);
+            } else {
+                // several stages reuse the panel: transpose it once, up front (one copy of
+                // the arithmetic in the code keeps the register count down)
+                if (!transposed) {
+#pragma unroll
+                    for (int b = 0; b < WPanel<QT>::QC / 2; b++) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
+                }
+                transposed = true;
+                panel_dot<QT, false>(p, xu0, n_units, j, grp, acc);
+            }
+        }
+        if (win == n_win - 1) {
+            // ---- row tile finished: combine the waves that split k, write
+            // y[tile*16 + 4*grp + r][rt*16 + j] (grouped: the row is a sorted position of the
+            // expert, the y row its pair index)
+            auto store = [&](int r, float v) {
+                const int mm = tile * 16 + grp * 4 + r;
+                if (GROUPED) {
+                    if (pos_begin + mm < pos_end) yout[(int64_t)P.perm[pos_begin + mm] * P.n + row] = v;
+                } else if (mm < P.m) {
+                    yout[(int64_t)mm * P.n + row] = v;
+                }
+            };
+            if (P.nwk == 1) {
+                if (rt_ok && row < P.n) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) store(r, acc[r]);
+                }
+            } else {
+                if (tile != 0) lds_barrier(); // the previous tile's sums have been read
+#pragma unroll
+                for (int r = 0; r < 4; r++) lds_red[(wave * 4 + r) * 64 + lane] = acc[r];
                 lds_barrier();
-                if (unit0 >= wu0 && unit0 < wu0 + wn) {
-                    const uint8_t* xu0 = lds_x + (size_t)(unit0 - wu0) * UB;
-                    if (!transposed) panel_dot<QT, true>(p, xu0, n_units, j, grp, acc);
-                    else panel_dot<QT, false>(p, xu0, n_units, j, grp, acc);
-                    transposed = true;
+                if (wk == 0 && rt_ok && row < P.n) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        float sum = 0.0f;
+                        for (int w2 = 0; w2 < P.nwk; w2++) sum += lds_red[((wr * P.nwk + w2) * 4 + r) * 64 + lane];
+                        store(r, sum);
+                    }
                 }
             }
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] = 0.0f;
         }
-        // ---- combine the waves that split k, write y[tile*16 + 4*grp + r][rt*16 + j]
-        // (grouped: the row is a sorted position of the expert, y row its pair index)
-        auto store = [&](int r, float v) {
-            const int mm = tile * 16 + grp * 4 + r;
-            if (GROUPED) {
-                if (pos_begin + mm < pos_end) P.y[(int64_t)P.perm[pos_begin + mm] * P.n + row] = v;
-            } else if (mm < P.m) {
-                P.y[(int64_t)mm * P.n + row] = v;
+        if (more) {
+            if (!P.double_buf) {
+                lds_barrier(); // every wave is done with this window
+                issue_window_copy<QT>(next_src, lds_x, next_n, wave, waves, lane);
             }
-        };
-        if (P.nwk == 1) {
-            if (rt_ok && row < P.n) {
-#pragma unroll
-                for (int r = 0; r < 4; r++) store(r, acc[r]);
-            }
-        } else {
-            if (tile != 0) lds_barrier(); // the previous tile's sums have been read
-#pragma unroll
-            for (int r = 0; r < 4; r++) lds_red[(wave * 4 + r) * 64 + lane] = acc[r];
-            lds_barrier();
-            if (wk == 0 && rt_ok && row < P.n) {
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    float sum = 0.0f;
-                    for (int w2 = 0; w2 < P.nwk; w2++) sum += lds_red[((wr * P.nwk + w2) * 4 + r) * 64 + lane];
-                    store(r, sum);
-                }
-            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            lds_barrier(); // the next window has landed; with two buffers: and this one is free
         }
-#pragma unroll
-        for (int r = 0; r < 4; r++) acc[r] = 0.0f;
+        tile = ntile, win = nwin;
     }
 }
 
@@ -617,6 +646,9 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     P.offsets = nullptr;
     P.tile_offsets = nullptr;
     P.matrix_bytes = 0;
+    P.w2 = nullptr;
+    P.y2 = nullptr;
+    P.double_buf = 0;
     P.window_units = (kWindowUnits / L.s) * L.s;
     const int padded_units = (int)(L.k_groups * L.s);
     if (P.window_units > padded_units) P.window_units = padded_units;
@@ -637,7 +669,9 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
         waves = P.nwk * P.nwr;
         P.rt_groups = (int)((L.row_tiles + P.nwr - 1) / P.nwr);
         grid = (unsigned)P.rt_groups;
-        lds = window_bytes + (size_t)waves * 256 * 4;
+        const bool single_stage = n_tiles == 1 && L.k_units <= P.window_units;
+        P.double_buf = !single_stage && 2 * window_bytes + (size_t)waves * 256 * 4 <= 160 * 1024;
+        lds = (P.double_buf ? 2 : 1) * window_bytes + (size_t)waves * 256 * 4;
     } else {
         P.nwk = 1;
         P.nwr = kMaxWaves;
@@ -702,10 +736,10 @@ hipError_t qmm_launch_quantize_grouped(int dtype, const float* x, const float* x
 
 bool qmm_gemv_mfma_grouped_supported(const QmmLayout& L) { return L.k_groups <= kMaxWaves; }
 
-hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* records,
-                                        float* y, const int32_t* perm, const int32_t* offsets,
-                                        const int32_t* tile_offsets, int n_experts,
-                                        hipStream_t stream) {
+hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
+                                        const void* records, float* y, float* y2, const int32_t* perm,
+                                        const int32_t* offsets, const int32_t* tile_offsets,
+                                        int n_experts, hipStream_t stream) {
     if (L.n == 0 || n_experts <= 0) return hipSuccess;
     if (!qmm_gemv_mfma_grouped_supported(L) || n_experts > 65535 || L.n > 0x3fffffff)
         return hipErrorInvalidValue;
@@ -734,8 +768,12 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     P.offsets = offsets;
     P.tile_offsets = tile_offsets;
     P.matrix_bytes = L.matrix_bytes;
+    P.w2 = (const uint8_t*)tiled2;
+    P.y2 = y2;
     const int waves = P.nwk * P.nwr;
-    const size_t lds = (size_t)P.window_units * unit_bytes(L.dtype) + (size_t)waves * 256 * 4;
+    const size_t window_bytes = (size_t)P.window_units * unit_bytes(L.dtype);
+    P.double_buf = 2 * window_bytes + (size_t)waves * 256 * 4 <= 160 * 1024;
+    const size_t lds = (P.double_buf ? 2 : 1) * window_bytes + (size_t)waves * 256 * 4;
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     const void* fn = L.dtype == QMM_Q4_K
                          ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true>)
@@ -744,7 +782,7 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
-    const dim3 grid((unsigned)P.rt_groups, (unsigned)n_experts);
+    const dim3 grid((unsigned)P.rt_groups, (unsigned)n_experts, tiled2 ? 2u : 1u);
     if (L.dtype == QMM_Q4_K)
         gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true><<<grid, 64 * waves, lds, stream>>>(P);
     else

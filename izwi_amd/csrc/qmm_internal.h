@@ -132,10 +132,12 @@ hipError_t qmm_launch_quantize_grouped(int dtype, const float* x, const float* x
                                        int64_t max_tiles, void* records, hipStream_t stream);
 // false if the matrix shape has no grouped matrix-core form (too many panels per row-tile)
 bool qmm_gemv_mfma_grouped_supported(const QmmLayout& L);
-hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* records,
-                                        float* y, const int32_t* perm, const int32_t* offsets,
-                                        const int32_t* tile_offsets, int n_experts,
-                                        hipStream_t stream);
+// With tiled2 / y2 a second stack of the same shape is multiplied by the same records
+// in the same launch (the expert MLP's gate and up projections).
+hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
+                                        const void* records, float* y, float* y2, const int32_t* perm,
+                                        const int32_t* offsets, const int32_t* tile_offsets,
+                                        int n_experts, hipStream_t stream);
 
 // out[t, :] = sum over slots s (in order) of weights[t, s] * y[t * top_k + s, :]
 hipError_t qmm_launch_moe_combine(const float* y, const float* weights, int64_t t, int top_k,
