@@ -154,7 +154,12 @@ def test_config3_lm_head_full_size(qa, oracle):
 
 @pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
 @pytest.mark.parametrize("n,k,m", [(1, 256, 1), (15, 256, 2), (17, 512, 3), (100, 768, 5), (250, 1280, 7),
-                                   (33, 2048, 64), (7, 16384, 2), (4100, 256, 1)])
+                                   (33, 2048, 64), (7, 16384, 2), (4100, 256, 1),
+                                   # batched (matrix-core) forms: more panels per row-tile than waves
+                                   # (streaming form, two activation windows, y accumulated per window),
+                                   # several row tiles with one LDS window buffer, ragged row tiles
+                                   (20, 16384, 5), (33, 12288, 40), (50, 3072, 17),
+                                   (40000, 1024, 9)])  # very tall: streaming form with a resident window
 def test_ragged_shapes(qa, oracle, dtype, n, k, m):
     _say(f"ragged dtype={dtype} n={n} k={k} m={m}")
     blocks = make_weight(oracle, dtype, n, k, 60 + n)
