@@ -10,8 +10,7 @@ pass over all of them, replayed from a HIP graph.  `value` is algorithmic
 bytes (GGUF weight bytes + f32 activations in and out) per second.
 
 Prints ONE JSON line.  `--gpus N` with N > 1 is refused: this build is
-single-GPU (the path shards by output rows without communication; see
-DESIGN.md).
+single-GPU (the path would shard by output rows without communication).
 """
 import argparse
 import json

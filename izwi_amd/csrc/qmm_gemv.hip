@@ -1,4 +1,5 @@
-// Decode kernel: fused activation-quantize + block dot products, M = 1..64.
+// Decode kernel: fused activation-quantize + block dot products, M = 1, 2 and
+// the expert-grouped segments of up to four rows.
 //
 // The arithmetic is candle-core's CPU `matmul` (quantize each activation row to
 // the weight type's dot type, integer block dots, f32 scaling); only the f32
@@ -9,17 +10,18 @@
 //     the quants; lane (u, r) owns unit u of row r, so no weight byte is
 //     shuffled between lanes and all nibble / int8 products run on
 //     v_dot4_i32_i8 (about 0.7 VALU lane-ops per weight element);
-//   * all of a wave's first panel loads are issued before anything else (the
-//     activations are quantized while they fly); afterwards the other resident
-//     waves of the CU keep loads in flight while one multiplies;
+//   * a wave issues its activation loads and then all loads of its panel before
+//     anything else, unconditionally and in one basic block, so that the waits
+//     can be counted: the activations are quantized while the panel flies, the
+//     panel is multiplied chunk by chunk while its rest arrives;
 //   * the workgroup quantizes the activations once into LDS (16 lanes per
 //     256-value block, reductions on DPP); lanes of one 16-row group read the
 //     same LDS words (broadcast), the unit stride is padded by 16 B so the S
 //     groups hit different banks;
 //   * the S partial sums of a row are combined with two cross-lane steps, the
 //     k-split between the waves of a workgroup through LDS.
-// Registers are capped at 128 per lane so that 16 waves stay resident per CU:
-// small matrices then fit in one round of workgroups.
+// The launch bound of 768 threads caps a wave at 168 registers (three waves per
+// SIMD): a 28 MB matrix then fits in one round of 12-wave workgroups.
 #include <hip/hip_runtime.h>
 
 #include <cstddef>

@@ -107,7 +107,7 @@ def run_forward(qa, dtype, blocks, n, k, x):
 
 
 def test_config1_q8_0_matvec(qa, oracle):
-    # BASELINE config 1: x [1,1024] ~ N(0,1), W [3072,1024] ~ N(0,0.02) -> Q8_0
+    # benchmark configuration 1: x [1,1024] ~ N(0,1), W [3072,1024] ~ N(0,0.02) -> Q8_0
     blocks = make_weight(oracle, Q8_0, 3072, 1024, 1)
     x = oracle.randn(2, (1, 1024))
     y = run_forward(qa, Q8_0, blocks, 3072, 1024, x)
@@ -332,7 +332,7 @@ def test_moe_sort_many_pairs(qa, oracle):
 
 @pytest.fixture(scope="module")
 def moe_weights(oracle):
-    # BASELINE config 5 at full size: 128 experts, hidden 2048, intermediate 768, Q4_K
+    # benchmark configuration 5 at full size: 128 experts, hidden 2048, intermediate 768, Q4_K
     E, hidden, inter = 128, 2048, 768
     gate = oracle.quantize(Q4_K, oracle.randn(180, (E * inter, hidden), std=0.02))
     up = oracle.quantize(Q4_K, oracle.randn(181, (E * inter, hidden), std=0.02))
