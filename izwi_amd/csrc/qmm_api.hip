@@ -93,6 +93,17 @@ int moe_mfma_min_rows() {
     return v;
 }
 
+// hipGetDevice with the missing-GPU case reported as such (not as a generic HIP error)
+int current_device(int* device) {
+    hipError_t e = hipGetDevice(device);
+    if (e == hipSuccess) return IZWI_QMM_OK;
+    (void)hipGetLastError();
+    if (e == hipErrorNoDevice || e == hipErrorInsufficientDriver || e == hipErrorInvalidDevice)
+        return fail(IZWI_QMM_ERR_NO_DEVICE, "no HIP device available (%s); libizwi_qmm has no CPU fallback",
+                    hipGetErrorString(e));
+    return fail_hip(e, "hipGetDevice");
+}
+
 int type_supported(int dtype) { return dtype == IZWI_QMM_Q8_0 || dtype == IZWI_QMM_Q4_K; }
 
 int storage_bytes(int dtype, int64_t rows, int64_t cols, uint64_t* out) {
@@ -128,7 +139,7 @@ int create_from_parts(int dtype, int64_t n_stacked, int64_t n, int64_t k, const 
         return fail(IZWI_QMM_ERR_INVALID, "k = %lld is not a positive multiple of the block size %d",
                     (long long)k, qmm_block_elems(dtype));
     int device = 0;
-    HIP_TRY(hipGetDevice(&device));
+    if (int rc = current_device(&device)) return rc;
     int n_cus = 0;
     int rc = ensure_device(device, &n_cus);
     if (rc) return rc;
@@ -451,7 +462,7 @@ int izwi_qmm_quantize_activations(int ggml_weight_dtype, const float* x, int64_t
     if (m == 0 || k == 0) return IZWI_QMM_OK;
     if (!x || !out_blocks) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
     int device = 0;
-    HIP_TRY(hipGetDevice(&device));
+    if (int rc = current_device(&device)) return rc;
     if (int rc = ensure_device(device, nullptr)) return rc;
     hipStream_t stream = (hipStream_t)stream_;
     Staged xi, o;
@@ -533,7 +544,7 @@ int izwi_moe_route(const float* logits, int64_t t, int32_t n_experts, int32_t to
     if (t == 0) return IZWI_QMM_OK;
     if (!logits || !ids || !weights) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
     int device = 0;
-    HIP_TRY(hipGetDevice(&device));
+    if (int rc = current_device(&device)) return rc;
     if (int rc = ensure_device(device, nullptr)) return rc;
     hipStream_t stream = (hipStream_t)stream_;
     Staged li, io, wo;
@@ -556,7 +567,7 @@ int izwi_moe_sort(const int32_t* ids, int64_t t, int32_t top_k, int32_t n_expert
     if (pairs > 0x7fffffff) return fail(IZWI_QMM_ERR_UNSUPPORTED, "too many pairs");
     if (!offsets || (pairs && (!ids || !perm))) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
     int device = 0;
-    HIP_TRY(hipGetDevice(&device));
+    if (int rc = current_device(&device)) return rc;
     if (int rc = ensure_device(device, nullptr)) return rc;
     hipStream_t stream = (hipStream_t)stream_;
     Staged ii, po, oo;

@@ -1,0 +1,209 @@
+// C++ host-side mirror of the reference's quantized projection interface over
+// the C ABI of libizwi_qmm (include/izwi_qmm.h).  Header-only; link with
+// -lizwi_qmm.
+//
+// Names and error behaviour follow the reference (izwi-core,
+// crates/izwi-core/src/models/architectures/qwen3/core.rs, and the Candle types
+// it calls):
+//   QTensor                       candle_core::quantized::QTensor (core.rs:710-715, 853-895)
+//   QMatMul                       candle_core::quantized::QMatMul::{from_arc, from_qtensor, forward}
+//   packed_qmatmul_from_qtensors  core.rs:846-889
+//   quantized_storage_bytes       core.rs:891-909
+//   Qwen3Projection               core.rs:671-674, 710-718, 791-831 (quantized arm)
+//   Error                         crates/izwi-core/src/error.rs:69-73 (InferenceError /
+//                                 ModelLoadError / InvalidInput)
+// There is no CPU fallback: without a gfx950 device every operation throws.
+#pragma once
+
+#include <cstdint>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "izwi_qmm.h"
+
+namespace izwi {
+
+enum class GgmlDType : int { Q8_0 = IZWI_QMM_Q8_0, Q4K = IZWI_QMM_Q4_K };
+inline int block_size(GgmlDType t) { return t == GgmlDType::Q8_0 ? 32 : 256; }
+inline int type_size(GgmlDType t) { return t == GgmlDType::Q8_0 ? 34 : 144; }
+
+enum class MemSpace : int { Device = IZWI_QMM_DEVICE, Host = IZWI_QMM_HOST };
+
+// The reference maps Candle errors to InferenceError, load-time ones to ModelLoadError.
+class Error : public std::runtime_error {
+public:
+    enum class Kind { InvalidInput, ModelLoadError, InferenceError };
+    Error(Kind kind, int status, const std::string& msg) : std::runtime_error(msg), kind_(kind), status_(status) {}
+    Kind kind() const { return kind_; }
+    int status() const { return status_; }
+
+private:
+    Kind kind_;
+    int status_;
+};
+
+inline void check(int rc) {
+    if (rc == IZWI_QMM_OK) return;
+    const std::string msg = izwi_qmm_last_error();
+    switch (rc) {
+        case IZWI_QMM_ERR_INVALID: throw Error(Error::Kind::InvalidInput, rc, msg);
+        case IZWI_QMM_ERR_UNSUPPORTED:
+        case IZWI_QMM_ERR_NO_DEVICE: throw Error(Error::Kind::ModelLoadError, rc, msg);
+        default: throw Error(Error::Kind::InferenceError, rc, msg);
+    }
+}
+
+// `quantized_storage_bytes(rows, cols, dtype)`, core.rs:891-909.
+inline uint64_t quantized_storage_bytes(int64_t rows, int64_t cols, GgmlDType dtype) {
+    uint64_t out = 0;
+    check(izwi_qmm_storage_bytes((int)dtype, rows, cols, &out));
+    return out;
+}
+
+// A quantized [n, k] weight (or a stack [e, n, k] of expert weights) on the GPU.
+class QTensor {
+public:
+    // `ggml_file::qtensor_from_ggml(dtype, raw, dims, device)`: raw GGUF block bytes -> tensor.
+    static std::shared_ptr<QTensor> from_blocks(GgmlDType dtype, const void* blocks, uint64_t nbytes,
+                                                int64_t n, int64_t k, MemSpace space = MemSpace::Host) {
+        izwi_qmm_weight* h = nullptr;
+        check(izwi_qmm_weight_create((int)dtype, n, k, blocks, nbytes, (int)space, &h));
+        return std::shared_ptr<QTensor>(new QTensor(h));
+    }
+    static std::shared_ptr<QTensor> from_expert_blocks(GgmlDType dtype, const void* blocks, uint64_t nbytes,
+                                                       int32_t n_experts, int64_t n, int64_t k,
+                                                       MemSpace space = MemSpace::Host) {
+        izwi_qmm_weight* h = nullptr;
+        check(izwi_qmm_weight_create_stacked((int)dtype, n_experts, n, k, blocks, nbytes, (int)space, &h));
+        return std::shared_ptr<QTensor>(new QTensor(h));
+    }
+    // takes ownership of a handle made by the C ABI
+    static std::shared_ptr<QTensor> adopt(izwi_qmm_weight* h) { return std::shared_ptr<QTensor>(new QTensor(h)); }
+    ~QTensor() { izwi_qmm_weight_destroy(h_); }
+    QTensor(const QTensor&) = delete;
+    QTensor& operator=(const QTensor&) = delete;
+
+    GgmlDType dtype() const { return (GgmlDType)info_.ggml_dtype; }
+    int64_t rows() const { return info_.n; }
+    int64_t cols() const { return info_.k; }
+    int32_t n_stacked() const { return info_.n_stacked; }
+    // `shape().dims2()`: an expert stack is rank 3
+    std::pair<int64_t, int64_t> dims2() const {
+        if (info_.n_stacked != 1)
+            throw Error(Error::Kind::InvalidInput, IZWI_QMM_ERR_INVALID, "unexpected rank, expected: 2, got: 3");
+        return {info_.n, info_.k};
+    }
+    uint64_t storage_size_in_bytes() const { return info_.nbytes; }
+    // `QTensor::data()`: the GGUF block bytes the tensor was built from.
+    std::vector<uint8_t> data() const {
+        std::vector<uint8_t> out(info_.nbytes);
+        check(izwi_qmm_weight_data(h_, out.data(), out.size(), IZWI_QMM_HOST, nullptr));
+        return out;
+    }
+    // `QTensor::dequantize(device)`: f32 [n_stacked * n, k].
+    std::vector<float> dequantize() const {
+        std::vector<float> out((size_t)info_.n_stacked * info_.n * info_.k);
+        check(izwi_qmm_dequantize_f32(h_, out.data(), IZWI_QMM_HOST, nullptr));
+        return out;
+    }
+    izwi_qmm_weight* handle() const { return h_; }
+
+private:
+    explicit QTensor(izwi_qmm_weight* h) : h_(h) {
+        const int rc = izwi_qmm_weight_get_info(h, &info_);
+        if (rc != IZWI_QMM_OK) {
+            izwi_qmm_weight_destroy(h);
+            check(rc);
+        }
+    }
+    izwi_qmm_weight* h_;
+    izwi_qmm_weight_info info_{};
+};
+
+// `QMatMul`: y[.., n] = x[.., k] * W^T.
+class QMatMul {
+public:
+    static QMatMul from_arc(std::shared_ptr<QTensor> q) {
+        q->dims2(); // a projection is rank 2
+        return QMatMul(std::move(q));
+    }
+    static QMatMul from_qtensor(std::shared_ptr<QTensor> q) { return from_arc(std::move(q)); }
+
+    // `Module::forward` for f32 activations: x is [m, k] contiguous, y [m, n]; both in `space`.
+    // Device pointers: asynchronous on `stream`.  Host pointers: returns when y is written.
+    void forward(const float* x, int64_t m, float* y, MemSpace space, void* stream = nullptr) const {
+        check(izwi_qmm_forward_f32(q_->handle(), x, m, y, (int)space, stream));
+    }
+    // host convenience form: x.size() must be a multiple of k
+    std::vector<float> forward(const std::vector<float>& x) const {
+        const int64_t k = q_->cols();
+        if (k == 0 || x.size() % (size_t)k)
+            throw Error(Error::Kind::InvalidInput, IZWI_QMM_ERR_INVALID,
+                        "input has " + std::to_string(x.size()) + " elements, not a multiple of k = " + std::to_string(k));
+        const int64_t m = (int64_t)(x.size() / (size_t)k);
+        std::vector<float> y((size_t)m * q_->rows());
+        forward(x.data(), m, y.data(), MemSpace::Host);
+        return y;
+    }
+    // prefill form: bf16 activations, y bf16 (out_bf16) or f32
+    void forward_bf16(const uint16_t* x, int64_t m, void* y, bool out_bf16, MemSpace space,
+                      void* stream = nullptr) const {
+        check(izwi_qmm_forward_bf16(q_->handle(), x, m, y, out_bf16 ? IZWI_QMM_OUT_BF16 : IZWI_QMM_OUT_F32,
+                                    (int)space, stream));
+    }
+    const std::shared_ptr<QTensor>& qtensor() const { return q_; }
+    int64_t out_features() const { return q_->rows(); }
+    int64_t in_features() const { return q_->cols(); }
+
+private:
+    explicit QMatMul(std::shared_ptr<QTensor> q) : q_(std::move(q)) {}
+    std::shared_ptr<QTensor> q_;
+};
+
+// `packed_qmatmul_from_qtensors` (core.rs:846-889): one [sum(rows), k] projection from
+// several tensors of equal k and dtype (fused QKV, fused gate/up).
+inline QMatMul packed_qmatmul_from_qtensors(const std::vector<std::shared_ptr<QTensor>>& parts) {
+    if (parts.empty())
+        throw Error(Error::Kind::ModelLoadError, IZWI_QMM_ERR_INVALID, "Packed quantized projection group was empty");
+    std::vector<std::vector<uint8_t>> datas;
+    std::vector<int64_t> rows;
+    std::vector<const void*> ptrs;
+    std::vector<uint64_t> lens;
+    for (const auto& p : parts) {
+        p->dims2();
+        datas.push_back(p->data());
+        rows.push_back(p->rows());
+    }
+    for (const auto& d : datas) {
+        ptrs.push_back(d.data());
+        lens.push_back(d.size());
+    }
+    izwi_qmm_weight* h = nullptr;
+    check(izwi_qmm_weight_create_packed((int)parts[0]->dtype(), (int32_t)parts.size(), rows.data(),
+                                        parts[0]->cols(), ptrs.data(), lens.data(), IZWI_QMM_HOST, &h));
+    return QMatMul::from_arc(QTensor::adopt(h)); // the new handle owns its own copy of the bytes
+}
+
+// `Qwen3Projection` (quantized arm): the op always receives f32 activations and
+// returns f32 (core.rs:772-831); callers with other activation dtypes cast around it.
+class Qwen3Projection {
+public:
+    static Qwen3Projection quantized(std::shared_ptr<QTensor> q) { return Qwen3Projection(QMatMul::from_arc(std::move(q))); }
+    static Qwen3Projection packed_quantized(const std::vector<std::shared_ptr<QTensor>>& parts) {
+        return Qwen3Projection(packed_qmatmul_from_qtensors(parts));
+    }
+    void forward(const float* x, int64_t m, float* y, MemSpace space, void* stream = nullptr) const {
+        mm_.forward(x, m, y, space, stream);
+    }
+    std::vector<float> forward(const std::vector<float>& x) const { return mm_.forward(x); }
+    const QMatMul& qmatmul() const { return mm_; }
+
+private:
+    explicit Qwen3Projection(QMatMul mm) : mm_(std::move(mm)) {}
+    QMatMul mm_;
+};
+
+} // namespace izwi

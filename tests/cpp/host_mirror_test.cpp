@@ -1,0 +1,135 @@
+// Exercises the C++ host-side mirror (izwi_amd/host/izwi_qmm.hpp) the way the
+// reference's own unit tests exercise its Rust types.
+//   host_mirror_test cpu   host logic only: byte-size rule and its errors, loud failure
+//                          without a gfx950 device
+//   host_mirror_test gpu   the reference's packed-projection test
+//                          (crates/izwi-core/src/models/architectures/qwen3/core.rs:3099-3142)
+//                          and a Q4_K projection, checked against the CPU oracle
+// Test infrastructure: links the oracle (liboracle_qmm.so) as the checker.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "izwi_qmm.hpp"
+
+extern "C" {
+int oracle_qmatmul(int dtype, int64_t m, int64_t k, int64_t n, const float* lhs, const void* rhs_t, float* dst);
+int oracle_quantize(int dtype, int64_t rows, int64_t cols, const float* src, void* dst);
+int64_t oracle_storage_bytes(int dtype, int64_t rows, int64_t cols);
+void oracle_fill_normal(uint64_t seed, int64_t offset, int64_t count, float mean, float std, float* out);
+}
+
+static int failures = 0;
+#define EXPECT(cond)                                                        \
+    do {                                                                    \
+        if (!(cond)) {                                                      \
+            std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);     \
+            failures++;                                                     \
+        }                                                                   \
+    } while (0)
+
+template <class F>
+static bool throws(izwi::Error::Kind kind, const char* needle, F&& f) {
+    try {
+        f();
+    } catch (const izwi::Error& e) {
+        if (e.kind() != kind) std::printf("  wrong kind, message: %s\n", e.what());
+        if (needle && !std::strstr(e.what(), needle)) std::printf("  message lacks '%s': %s\n", needle, e.what());
+        return e.kind() == kind && (!needle || std::strstr(e.what(), needle));
+    }
+    return false;
+}
+
+static std::vector<uint8_t> quantize(izwi::GgmlDType dt, const std::vector<float>& w, int64_t n, int64_t k) {
+    std::vector<uint8_t> blocks((size_t)oracle_storage_bytes((int)dt, n, k));
+    if (oracle_quantize((int)dt, n, k, w.data(), blocks.data())) std::printf("oracle_quantize rejected the shape\n");
+    return blocks;
+}
+
+static float max_rel(const std::vector<float>& a, const std::vector<float>& b) {
+    float mx = 0.0f, scale = 0.0f;
+    for (size_t i = 0; i < b.size(); i++) scale = std::fmax(scale, std::fabs(b[i]));
+    for (size_t i = 0; i < b.size(); i++) mx = std::fmax(mx, std::fabs(a[i] - b[i]));
+    return mx / (scale > 0 ? scale : 1.0f);
+}
+
+static void host_logic() {
+    using izwi::GgmlDType;
+    EXPECT(izwi::quantized_storage_bytes(3072, 1024, GgmlDType::Q8_0) == 3342336u);
+    EXPECT(izwi::quantized_storage_bytes(12288, 4096, GgmlDType::Q4K) == 28311552u);
+    EXPECT(izwi::quantized_storage_bytes(0, 4096, GgmlDType::Q4K) == 0u);
+    EXPECT(throws(izwi::Error::Kind::InvalidInput, "not divisible by block size",
+                  [] { izwi::quantized_storage_bytes(3, 100, GgmlDType::Q4K); }));
+    EXPECT(throws(izwi::Error::Kind::ModelLoadError, "not supported",
+                  [] { izwi::quantized_storage_bytes(4, 256, (GgmlDType)14); }));
+    EXPECT(izwi::block_size(GgmlDType::Q4K) == 256 && izwi::type_size(GgmlDType::Q4K) == 144);
+    EXPECT(izwi::block_size(GgmlDType::Q8_0) == 32 && izwi::type_size(GgmlDType::Q8_0) == 34);
+}
+
+static void no_device_is_loud() {
+    std::vector<uint8_t> blocks(34 * 2, 0);
+    EXPECT(throws(izwi::Error::Kind::ModelLoadError, "no CPU fallback", [&] {
+        izwi::QTensor::from_blocks(izwi::GgmlDType::Q8_0, blocks.data(), blocks.size(), 2, 32);
+    }));
+}
+
+static void packed_matches_separate_q8_0() {
+    using izwi::GgmlDType;
+    std::vector<float> w1(64), w2(32), x(32);
+    for (int i = 0; i < 64; i++) w1[i] = (float)(i - 31) / 8.0f;
+    for (int i = 0; i < 32; i++) w2[i] = (float)(15 - i) / 7.0f;
+    for (int i = 0; i < 32; i++) x[i] = (float)(i + 1) / 16.0f;
+    auto b1 = quantize(GgmlDType::Q8_0, w1, 2, 32), b2 = quantize(GgmlDType::Q8_0, w2, 1, 32);
+    auto q1 = izwi::QTensor::from_blocks(GgmlDType::Q8_0, b1.data(), b1.size(), 2, 32);
+    auto q2 = izwi::QTensor::from_blocks(GgmlDType::Q8_0, b2.data(), b2.size(), 1, 32);
+    EXPECT(q1->data() == b1 && q2->data() == b2);
+    auto y1 = izwi::QMatMul::from_arc(q1).forward(x);
+    auto y2 = izwi::QMatMul::from_qtensor(q2).forward(x);
+    auto packed = izwi::Qwen3Projection::packed_quantized({q1, q2});
+    EXPECT(packed.qmatmul().out_features() == 3 && packed.qmatmul().in_features() == 32);
+    auto yp = packed.forward(x);
+    EXPECT(yp.size() == 3);
+    // the reference asserts packed == cat(separate) within 1e-5
+    EXPECT(std::fabs(yp[0] - y1[0]) < 1e-5f && std::fabs(yp[1] - y1[1]) < 1e-5f && std::fabs(yp[2] - y2[0]) < 1e-5f);
+    // absolute values of candle-core's algorithm on this input
+    const float want[3] = {-42.692207f, 89.229607f, -26.613434f};
+    for (int i = 0; i < 3; i++) EXPECT(std::fabs(yp[i] - want[i]) < 1e-4f);
+    // error texts of the packing rule
+    EXPECT(throws(izwi::Error::Kind::ModelLoadError, "empty", [] { izwi::packed_qmatmul_from_qtensors({}); }));
+    std::vector<float> w3(64, 0.5f);
+    auto b3 = quantize(GgmlDType::Q8_0, w3, 1, 64);
+    auto q3 = izwi::QTensor::from_blocks(GgmlDType::Q8_0, b3.data(), b3.size(), 1, 64);
+    EXPECT(throws(izwi::Error::Kind::InvalidInput, nullptr, [&] { izwi::packed_qmatmul_from_qtensors({q1, q3}); }));
+    EXPECT(throws(izwi::Error::Kind::InvalidInput, "multiple of k", [&] { izwi::QMatMul::from_arc(q1).forward(std::vector<float>(33, 1.0f)); }));
+}
+
+static void q4k_projection_matches_oracle() {
+    using izwi::GgmlDType;
+    const int64_t n = 200, k = 1280, m = 5;
+    std::vector<float> w((size_t)n * k), x((size_t)m * k);
+    oracle_fill_normal(11, 0, (int64_t)w.size(), 0.0f, 0.02f, w.data());
+    oracle_fill_normal(12, 0, (int64_t)x.size(), 0.0f, 1.0f, x.data());
+    auto blocks = quantize(GgmlDType::Q4K, w, n, k);
+    auto q = izwi::QTensor::from_blocks(GgmlDType::Q4K, blocks.data(), blocks.size(), n, k);
+    EXPECT(q->dtype() == GgmlDType::Q4K && q->dims2().first == n && q->dims2().second == k);
+    EXPECT(q->data() == blocks);
+    auto y = izwi::Qwen3Projection::quantized(q).forward(x);
+    std::vector<float> want((size_t)m * n);
+    EXPECT(oracle_qmatmul((int)GgmlDType::Q4K, m, k, n, x.data(), blocks.data(), want.data()) == 0);
+    EXPECT(max_rel(y, want) < 1e-4f);
+}
+
+int main(int argc, char** argv) {
+    const std::string mode = argc > 1 ? argv[1] : "cpu";
+    host_logic();
+    if (mode == "gpu") {
+        packed_matches_separate_q8_0();
+        q4k_projection_matches_oracle();
+    } else if (mode == "nodevice") {
+        no_device_is_loud();
+    }
+    std::printf(failures ? "%d check(s) failed\n" : "all checks passed\n", failures);
+    return failures ? 1 : 0;
+}
