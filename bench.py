@@ -109,6 +109,28 @@ def build_decode_weights(torch, qa, oracle, dtype, n_layers, with_lm_head):
     return weights
 
 
+def build_packed_weights(torch, qa, oracle, dtype, n_layers):
+    """The same stack with q|k|v and gate|up row-concatenated into one weight each, as the
+    reference's packed_qmatmul_from_qtensors does where it enables projection grouping:
+    4 launches per layer instead of 7, identical weight bytes and outputs."""
+    gg = qa.GgmlDType(dtype)
+    host = {name: (make_blocks(oracle, dtype, n, k, 1000 + i), n, k) for i, (name, n, k) in enumerate(LAYER_8B)}
+
+    def packed(names):
+        return qa.packed_qmatmul_from_qtensors([(gg, host[nm][0], (host[nm][1], host[nm][2])) for nm in names])
+
+    weights = []
+    for _layer in range(n_layers):
+        weights.append((packed(("q", "k", "v")), 4096 + 2 * 1024, 4096))
+        weights.append((qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, host["o"][0], (4096, 4096))), 4096, 4096))
+        weights.append((packed(("gate", "up")), 2 * 12288, 4096))
+        weights.append((qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, host["down"][0], (4096, 12288))), 4096, 12288))
+    name, n, k = LM_HEAD_8B
+    blocks = make_blocks(oracle, dtype, n, k, 2000, pool_rows=16384)
+    weights.append((qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, blocks, (n, k))), n, k))
+    return weights
+
+
 def decode_calls(torch, oracle, dtype, weights, m):
     """(calls, algorithmic bytes) of one decode step with m activation rows."""
     xs = {k: torch.from_numpy(oracle.randn(7 + k, (m, k))).cuda() for k in (4096, 12288)}
@@ -340,6 +362,18 @@ def main():
     torch.cuda.empty_cache()
 
     if not args.no_extras:
+        try:
+            pw = build_packed_weights(torch, qa, oracle, dtype, args.layers)
+            c, tb = decode_calls(torch, oracle, dtype, pw, args.m)
+            t, g = time_graph(torch, lambda: run_calls(qa, c), max(5, args.steps // 2), 3)
+            extras["decode_packed_qkv_gateup"] = {
+                "gbs": round(tb / (t * 1e-3) / 1e9, 1), "ms_per_step": round(t, 4), "launches_per_step": len(c),
+                "note": "same projections, q|k|v and gate|up as one packed weight each (the reference's "
+                        "packed_qmatmul_from_qtensors); not the headline: the reference packs on Metal only"}
+            del pw, c, g
+            torch.cuda.empty_cache()
+        except Exception as exc:
+            extras["decode_packed_error"] = repr(exc)
         try:
             extras["moe_30b_a3b_q4k"] = moe_extra(torch, qa, oracle)
         except Exception as exc:
