@@ -1,0 +1,101 @@
+"""Writes the golden fixtures of this directory.
+
+Neither fixture comes from running the reference (it cannot be built here, and the crate
+that holds the arithmetic is not in its tree).  They restate, as data:
+
+* q4k_hand_block.json - one Q4_K block built from the public GGUF block format with the
+  answers of its closed form y = d * sc * q - dmin * m worked out independently of any
+  code under test (all 256 values; the scale bytes exercise both branches of the 6-bit
+  unpacking).
+* packed_q8_0_case.json - the inputs of the reference's own unit test
+  `packed_qmatmul_matches_separate_q8_0_on_cpu`
+  (crates/izwi-core/src/models/architectures/qwen3/core.rs:3099-3142), their Q8_0 block
+  bytes and the outputs of candle-core's algorithm on them, computed here with plain
+  numpy arithmetic (no code of the oracle or of the library is used).
+
+Run:  python tests/golden/make_fixtures.py
+"""
+import json
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def q4k_hand_block():
+    d, dmin = np.float16(1.0), np.float16(0.5)
+    scales = bytes([0x41, 0x82, 0xC3, 0xC4, 0x40, 0x85, 0xCA, 0xCF, 0x41, 0x82, 0xC3, 0xFF])
+    qs = bytes(range(128))
+    block = d.tobytes() + dmin.tobytes() + scales + qs
+    assert len(block) == 144
+    sc = [1, 2, 3, 4, 17, 34, 51, 63]   # what the twelve scale bytes encode
+    mn = [0, 5, 10, 15, 20, 40, 60, 63]
+    y = np.zeros(256, dtype=np.float64)
+    for g in range(4):                   # 64 elements: 32 low nibbles, then 32 high nibbles
+        for l in range(32):
+            b = qs[32 * g + l]
+            y[64 * g + l] = 1.0 * sc[2 * g] * (b & 15) - 0.5 * mn[2 * g]
+            y[64 * g + 32 + l] = 1.0 * sc[2 * g + 1] * (b >> 4) - 0.5 * mn[2 * g + 1]
+    assert y.sum() == 32224.0 and y[224] == 346.5 and y[255] == 409.5 and y[32] == -2.5
+    return {"ggml_dtype": 12, "rows": 1, "cols": 256, "block_hex": block.hex(),
+            "scales": sc, "mins": mn, "expected_f32": [float(v) for v in y], "expected_sum": 32224.0}
+
+
+def q8_0_quantize_rows(w):
+    """BlockQ8_0::from_float: d = amax / 127 (stored as f16), q = round(x / d) with d in f32."""
+    rows, cols = w.shape
+    out = bytearray()
+    scale_bits = []
+    for r in range(rows):
+        for b in range(cols // 32):
+            v = w[r, 32 * b:32 * b + 32].astype(np.float32)
+            amax = np.float32(np.abs(v).max())
+            d = np.float32(amax / np.float32(127.0))
+            inv = np.float32(1.0) / d if d != 0 else np.float32(0.0)
+            q = np.clip(np.sign(v * inv) * np.floor(np.abs(v * inv) + np.float32(0.5)), -128, 127).astype(np.int8)
+            h = np.float16(d)
+            scale_bits.append(int(h.view(np.uint16)))
+            out += h.tobytes() + q.tobytes()
+    return bytes(out), scale_bits
+
+
+def q8_0_vec_dot(wblocks, xblocks, k):
+    """sum over blocks of (sum q_w * q_x) * d_w * d_x, accumulated in f32 in block order."""
+    acc = np.float32(0.0)
+    for b in range(k // 32):
+        wb, xb = wblocks[34 * b:34 * b + 34], xblocks[34 * b:34 * b + 34]
+        dw = np.float32(np.frombuffer(wb[:2], np.float16)[0])
+        dx = np.float32(np.frombuffer(xb[:2], np.float16)[0])
+        s = int(np.dot(np.frombuffer(wb[2:], np.int8).astype(np.int32), np.frombuffer(xb[2:], np.int8).astype(np.int32)))
+        acc = np.float32(acc + np.float32(s) * np.float32(dw * dx))
+    return acc
+
+
+def packed_case():
+    idx = np.arange(64, dtype=np.float32)
+    w1 = ((idx - 31.0) / 8.0).reshape(2, 32)
+    w2 = ((15.0 - idx[:32]) / 7.0).reshape(1, 32)
+    x = ((idx[:32] + 1.0) / 16.0).reshape(1, 32)
+    b1, s1 = q8_0_quantize_rows(w1)
+    b2, s2 = q8_0_quantize_rows(w2)
+    bx, sx = q8_0_quantize_rows(x)      # the activation row is quantized the same way
+    packed = b1 + b2                     # packed_qmatmul_from_qtensors: byte concatenation
+    y = [float(q8_0_vec_dot(packed[34 * r:34 * r + 34], bx, 32)) for r in range(3)]
+    assert s1 + s2 == [10192, 10248, 9372] and sx == [9224]
+    assert np.allclose(y, [-42.692207, 89.229607, -26.613434], rtol=0, atol=2e-6)
+    return {"ggml_dtype": 8, "k": 32,
+            "w1_f32": [float(v) for v in w1.reshape(-1)], "w1_rows": 2,
+            "w2_f32": [float(v) for v in w2.reshape(-1)], "w2_rows": 1,
+            "x_f32": [float(v) for v in x.reshape(-1)],
+            "w1_blocks_hex": b1.hex(), "w2_blocks_hex": b2.hex(), "x_blocks_hex": bx.hex(),
+            "weight_scale_f16_bits": s1 + s2, "activation_scale_f16_bits": sx,
+            "expected_y": y, "exact_math_y": [-42.625, 89.375, -26.714286],
+            "reference_tolerance_packed_vs_separate": 1e-5}
+
+
+if __name__ == "__main__":
+    for name, rec in (("q4k_hand_block.json", q4k_hand_block()), ("packed_q8_0_case.json", packed_case())):
+        with open(os.path.join(HERE, name), "w") as f:
+            json.dump(rec, f, indent=1)
+        print("wrote", name)

@@ -1,0 +1,82 @@
+"""The committed golden fixtures (tests/golden/*.json, written by tests/golden/make_fixtures.py)
+against the CPU oracle and, on a GPU, against the library through its C ABI."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+Q8_0, Q4_K = 8, 12
+
+
+def load(name):
+    with open(os.path.join(GOLDEN, name)) as f:
+        return json.load(f)
+
+
+def blocks(hex_string):
+    return np.frombuffer(bytes.fromhex(hex_string), dtype=np.uint8).copy()
+
+
+# ---- CPU: the oracle ----------------------------------------------------------
+def test_oracle_q4k_hand_block_fixture(oracle):
+    fx = load("q4k_hand_block.json")
+    y = oracle.dequantize(Q4_K, blocks(fx["block_hex"]), fx["rows"], fx["cols"])[0]
+    assert np.array_equal(y, np.array(fx["expected_f32"], dtype=np.float32))
+    assert float(y.astype(np.float64).sum()) == fx["expected_sum"]
+
+
+def test_oracle_packed_q8_0_fixture(oracle):
+    fx = load("packed_q8_0_case.json")
+    k = fx["k"]
+    w1 = np.array(fx["w1_f32"], dtype=np.float32).reshape(fx["w1_rows"], k)
+    w2 = np.array(fx["w2_f32"], dtype=np.float32).reshape(fx["w2_rows"], k)
+    x = np.array(fx["x_f32"], dtype=np.float32).reshape(1, k)
+    # the oracle's quantizers reproduce the fixture's block bytes
+    assert np.array_equal(oracle.quantize(Q8_0, w1), blocks(fx["w1_blocks_hex"]))
+    assert np.array_equal(oracle.quantize(Q8_0, w2), blocks(fx["w2_blocks_hex"]))
+    assert np.array_equal(oracle.quantize_activations(Q8_0, x), blocks(fx["x_blocks_hex"]))
+    packed = np.concatenate([blocks(fx["w1_blocks_hex"]), blocks(fx["w2_blocks_hex"])])
+    y = oracle.qmatmul(Q8_0, x, packed, 3)[0]
+    assert np.allclose(y, np.array(fx["expected_y"], dtype=np.float32), rtol=0, atol=2e-6)
+
+
+# ---- GPU: the library ---------------------------------------------------------
+@pytest.fixture(scope="module")
+def qa():
+    import torch
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    import izwi_amd
+    izwi_amd.lib()
+    return izwi_amd
+
+
+@pytest.mark.gpu
+def test_device_q4k_hand_block_fixture(qa):
+    fx = load("q4k_hand_block.json")
+    q = qa.QTensor.from_blocks(qa.GgmlDType.Q4K, blocks(fx["block_hex"]), (fx["rows"], fx["cols"]))
+    y = q.dequantize().cpu().numpy()[0]
+    assert np.array_equal(y, np.array(fx["expected_f32"], dtype=np.float32))
+    assert np.array_equal(q.data(), blocks(fx["block_hex"]))
+
+
+@pytest.mark.gpu
+def test_device_packed_q8_0_fixture(qa):
+    import torch
+    fx = load("packed_q8_0_case.json")
+    k = fx["k"]
+    dt = qa.GgmlDType.Q8_0
+    x = torch.tensor(fx["x_f32"], dtype=torch.float32).reshape(1, k).cuda()
+    b1, b2 = blocks(fx["w1_blocks_hex"]), blocks(fx["w2_blocks_hex"])
+    packed = qa.packed_qmatmul_from_qtensors([(dt, b1, (fx["w1_rows"], k)), (dt, b2, (fx["w2_rows"], k))])
+    y = packed.forward(x).cpu().numpy()[0]
+    sep = np.concatenate([qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, b1, (fx["w1_rows"], k))).forward(x).cpu().numpy()[0],
+                          qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, b2, (fx["w2_rows"], k))).forward(x).cpu().numpy()[0]])
+    # the reference's own assertion, then the absolute values
+    assert np.abs(y - sep).max() <= fx["reference_tolerance_packed_vs_separate"]
+    assert np.allclose(y, np.array(fx["expected_y"], dtype=np.float32), rtol=0, atol=1e-5)
+    # the on-chip activation quantizer writes the fixture's activation block
+    xq = qa.quantize_activations(dt, x)
+    assert np.array_equal(np.asarray(xq.cpu()).reshape(-1), blocks(fx["x_blocks_hex"]))
