@@ -498,11 +498,15 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
                                      w->n_cus, stream));
     } else {
         // prefill-sized m with f32 activations: convert once, then the MFMA kernel
+        // scratch: [bf16 copy of x | split-k partial tiles]
+        const size_t xb_bytes = (((size_t)m * L.k * sizeof(uint16_t)) + 255) & ~(size_t)255;
+        const size_t ws_bytes = qmm_gemm_workspace_bytes(L, m, w->n_cus);
         void* xb = nullptr;
-        HIP_TRY(get_scratch(w->device, stream, (size_t)m * L.k * sizeof(uint16_t), &xb));
+        HIP_TRY(get_scratch(w->device, stream, xb_bytes + ws_bytes, &xb));
         hipError_t e = qmm_launch_f32_to_bf16((const float*)xi.dev, (uint16_t*)xb, m * L.k, stream);
         if (e == hipSuccess)
-            e = qmm_launch_gemm_bf16(L, w->tiled, (const uint16_t*)xb, m, yo.dev, 0, w->n_cus, stream);
+            e = qmm_launch_gemm_bf16(L, w->tiled, (const uint16_t*)xb, m, yo.dev, 0,
+                                     ws_bytes ? (uint8_t*)xb + xb_bytes : nullptr, w->n_cus, stream);
         if (e != hipSuccess) return fail_hip(e, "prefill kernel");
     }
     HIP_TRY(yo.finish(stream));
@@ -527,8 +531,11 @@ int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int6
     Staged xi, yo;
     HIP_TRY(xi.in(x_bf16, (size_t)m * L.k * sizeof(uint16_t), mem_space));
     HIP_TRY(yo.out(y, ybytes, mem_space));
+    void* workspace = nullptr; // split-k partial tiles, for products with few output tiles only
+    if (const size_t ws_bytes = qmm_gemm_workspace_bytes(L, m, w->n_cus))
+        HIP_TRY(get_scratch(w->device, stream, ws_bytes, &workspace));
     HIP_TRY(qmm_launch_gemm_bf16(L, w->tiled, (const uint16_t*)xi.dev, m, yo.dev,
-                                 out_dtype == IZWI_QMM_OUT_BF16, w->n_cus, stream));
+                                 out_dtype == IZWI_QMM_OUT_BF16, workspace, w->n_cus, stream));
     HIP_TRY(yo.finish(stream));
     return IZWI_QMM_OK;
 }

@@ -16,6 +16,8 @@
 // step.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include <type_traits>
 #include <utility>
 
@@ -36,10 +38,15 @@ struct GemmParams {
     const uint16_t* x; // bf16 [m, k]
     void* y;
     int64_t m, n, k;
+    int64_t n_begin, n_end; // output columns (weight rows) of this launch, n_begin a multiple of 256
     int k_units, k_groups, s, slots;
     int64_t row_tiles, panel_bytes;
     int out_bf16;
     int tiles_m, tiles_n;
+    // split-k form (blockIdx.y = slice): slice s covers k steps [s * slice_steps, ..) and
+    // writes its f32 tile to partial[s][m][n]; a second kernel adds the slices in order
+    int slice_steps;
+    float* partial;
 };
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
@@ -165,7 +172,7 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams P) {
     // weight rows they share stay in L2 while all of m is swept
     const int tm = blockIdx.x % P.tiles_m;
     const int tn = blockIdx.x / P.tiles_m;
-    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t m0 = (int64_t)tm * BM, n0 = P.n_begin + (int64_t)tn * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int k_steps = P.k_units * 4;
@@ -269,7 +276,7 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams P) {
 #pragma unroll
         for (int j = 0; j < NT; j++) {
             const int64_t gn = n0 + wn * (BN / 2) + j * 32 + (lane & 31);
-            if (gn >= P.n) continue;
+            if (gn >= P.n_end) continue;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int64_t gm = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
@@ -310,10 +317,12 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
 
     const int tm = blockIdx.x % P.tiles_m;
     const int tn = blockIdx.x / P.tiles_m;
-    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t m0 = (int64_t)tm * BM, n0 = P.n_begin + (int64_t)tn * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int k_steps = P.k_units * 4;
+    const int k_steps_all = P.k_units * 4;
+    const int kt0 = P.partial ? (int)blockIdx.y * P.slice_steps : 0;              // first k step of this workgroup
+    const int kt1 = P.partial ? min(k_steps_all, kt0 + P.slice_steps) : k_steps_all; // one past its last
 
     f32x16 acc[MT][NT];
 #pragma unroll
@@ -415,19 +424,19 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
 
     // ---- prologue: tile 0 -> stage 0, tile 1 -> registers
 #pragma unroll
-    for (int i = 0; i < XC; i++) x_load(0, i);
-    w_load_hdr(0);
+    for (int i = 0; i < XC; i++) x_load(kt0, i);
+    w_load_hdr(kt0);
 #pragma unroll
-    for (int c = 0; c < NC; c++) w_load_q(0, c);
+    for (int c = 0; c < NC; c++) w_load_q(kt0, c);
 #pragma unroll
-    for (int i = 0; i < XC; i++) x_write(0, i, smem);
-    w_scales(0);
+    for (int i = 0; i < XC; i++) x_write(kt0, i, smem);
+    w_scales(kt0);
     static_for<8>([&](auto S) { w_slice(S, smem); });
 #pragma unroll
-    for (int i = 0; i < XC; i++) x_load(1, i);
-    w_load_hdr(1);
+    for (int i = 0; i < XC; i++) x_load(kt0 + 1, i);
+    w_load_hdr(kt0 + 1);
 #pragma unroll
-    for (int c = 0; c < NC; c++) w_load_q(1, c);
+    for (int c = 0; c < NC; c++) w_load_q(kt0 + 1, c);
     __syncthreads();
 
     auto k_step = [&](int kt, const uint8_t* cur, uint8_t* next, auto feed) {
@@ -488,27 +497,44 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
         });
         __syncthreads();
     };
-    for (int kt = 0; kt + 1 < k_steps; kt++)
-        k_step(kt, smem + (kt & 1) * kStage, smem + ((kt + 1) & 1) * kStage, std::true_type{});
-    k_step(k_steps - 1, smem + ((k_steps - 1) & 1) * kStage, nullptr, std::false_type{});
+    for (int kt = kt0; kt + 1 < kt1; kt++)
+        k_step(kt, smem + ((kt - kt0) & 1) * kStage, smem + ((kt - kt0 + 1) & 1) * kStage, std::true_type{});
+    k_step(kt1 - 1, smem + ((kt1 - 1 - kt0) & 1) * kStage, nullptr, std::false_type{});
 
+    // a split-k slice stores f32 into its own [m, n] plane of the workspace
+    float* out_f32 = P.partial ? P.partial + (int64_t)blockIdx.y * P.m * P.n : reinterpret_cast<float*>(P.y);
+    const bool out_bf16 = P.partial == nullptr && P.out_bf16 != 0;
 #pragma unroll
     for (int i = 0; i < MT; i++) {
 #pragma unroll
         for (int j = 0; j < NT; j++) {
             const int64_t gn = n0 + wn * (BN / 2) + j * 32 + (lane & 31);
-            if (gn >= P.n) continue;
+            if (gn >= P.n_end) continue;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int64_t gm = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 if (gm >= P.m) continue;
-                if (P.out_bf16)
+                if (out_bf16)
                     reinterpret_cast<uint16_t*>(P.y)[gm * P.n + gn] = qmm_f32_to_bf16_bits(acc[i][j][r]);
                 else
-                    reinterpret_cast<float*>(P.y)[gm * P.n + gn] = acc[i][j][r];
+                    out_f32[gm * P.n + gn] = acc[i][j][r];
             }
         }
     }
+}
+
+// out[i] = sum over slices (in order) of partial[s][i], as f32 or bf16; i runs over the
+// columns [n_begin, n_end) of all rows
+__global__ void splitk_reduce_kernel(const float* __restrict__ partial, int slices, int64_t m, int64_t n,
+                                     int64_t n_begin, int64_t n_end, void* __restrict__ y, int out_bf16) {
+    const int64_t width = n_end - n_begin;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= m * width) return;
+    const int64_t row = idx / width, col = n_begin + (idx - row * width);
+    float sum = 0.0f;
+    for (int s = 0; s < slices; s++) sum += partial[((int64_t)s * m + row) * n + col];
+    if (out_bf16) reinterpret_cast<uint16_t*>(y)[row * n + col] = qmm_f32_to_bf16_bits(sum);
+    else reinterpret_cast<float*>(y)[row * n + col] = sum;
 }
 
 __global__ void f32_to_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ out,
@@ -526,9 +552,9 @@ __global__ void f32_to_bf16_kernel(const float* __restrict__ x, uint16_t* __rest
 }
 
 template <int QT, int BM, int BN>
-hipError_t launch_tile(GemmParams P, hipStream_t stream) {
+hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
     P.tiles_m = (int)((P.m + BM - 1) / BM);
-    P.tiles_n = (int)((P.n + BN - 1) / BN);
+    P.tiles_n = (int)((P.n_end - P.n_begin + BN - 1) / BN);
     const int64_t grid = (int64_t)P.tiles_m * P.tiles_n;
     if (grid > 0x7fffffff) return hipErrorInvalidValue;
     const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
@@ -539,40 +565,107 @@ hipError_t launch_tile(GemmParams P, hipStream_t stream) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
     }
-    if constexpr (BN == 256)
-        gemm_pipe_kernel<QT, BM><<<dim3((unsigned)grid), dim3(kThreads), lds, stream>>>(P);
-    else
+    if constexpr (BN == 256) {
+        float* partial = P.partial;
+        if (slices > 1) {
+            const int k_steps = P.k_units * 4;
+            P.slice_steps = (k_steps + slices - 1) / slices;
+        } else {
+            P.partial = nullptr;
+        }
+        gemm_pipe_kernel<QT, BM><<<dim3((unsigned)grid, (unsigned)slices), dim3(kThreads), lds, stream>>>(P);
+        if (slices > 1) {
+            const int64_t count = P.m * (P.n_end - P.n_begin);
+            splitk_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(
+                partial, slices, P.m, P.n, P.n_begin, P.n_end, P.y, P.out_bf16);
+        }
+    } else {
         gemm_kernel<QT, BM, BN><<<dim3((unsigned)grid), dim3(kThreads), lds, stream>>>(P);
+    }
     return hipGetLastError();
 }
 
-// Tile choice: big tiles reuse each LDS byte most, but the grid runs in rounds of one
-// workgroup per CU and a partly filled last round idles CUs.  Score = fraction of CU
-// slots doing work x relative efficiency of the tile (measured on the 8B shapes).
-template <int QT>
-hipError_t launch_qt(const GemmParams& P, int n_cus, hipStream_t stream) {
-    auto score = [&](int bm, int bn, double quality) {
-        const int64_t tiles = ((P.m + bm - 1) / bm) * ((P.n + bn - 1) / bn);
-        const int64_t rounds = (tiles + n_cus - 1) / n_cus;
-        return quality * (double)tiles / (double)(rounds * n_cus);
+// How a [m, n] x k product is cut into launches.  Big tiles reuse each LDS byte most, but
+// the grid runs in rounds of one workgroup per CU and a partly filled last round idles
+// CUs; a product with few tiles can be split along k (each slice writes an f32 tile, a
+// second kernel adds the slices in order).  Costs are in k steps of a 256 x 256 tile
+// (relative tile efficiencies measured on the 8B shapes).
+struct GemmPlan {
+    int bm, bn;          // tile of the only / the second launch
+    int slices;          // split along k (BN == 256 tiles only)
+    int64_t full_cols;   // > 0: first a launch of 256 x 256 tiles over this many 256-column strips
+};
+
+GemmPlan plan_gemm(int64_t m, int64_t n, int k_steps, int n_cus) {
+    constexpr double kQ128 = 0.72, kQ64 = 0.4;
+    auto tiles = [&](int bm, int bn, int64_t cols) { return ((m + bm - 1) / bm) * ((cols + bn - 1) / bn); };
+    auto rounds = [&](int64_t t) { return (double)((t + n_cus - 1) / n_cus); };
+    GemmPlan best{256, 256, 1, 0};
+    double best_cost = rounds(tiles(256, 256, n)) * k_steps;
+    auto consider = [&](GemmPlan p, double cost) {
+        if (cost < 0.97 * best_cost) best = p, best_cost = cost;
     };
-    const double s256 = score(256, 256, 1.0), s128 = score(128, 256, 0.72), s64 = score(128, 128, 0.4);
-    if (s256 >= s128 && s256 >= s64) return launch_tile<QT, 256, 256>(P, stream);
-    if (s128 >= s64) return launch_tile<QT, 128, 256>(P, stream);
-    return launch_tile<QT, 128, 128>(P, stream);
+    consider({128, 256, 1, 0}, rounds(tiles(128, 256, n)) * k_steps * 0.5 / kQ128);
+    consider({128, 128, 1, 0}, rounds(tiles(128, 128, n)) * k_steps * 0.25 / kQ64);
+    // whole rounds of 256 x 256 tiles first, the rest as 128 x 256 tiles
+    const int64_t tiles_m256 = (m + 255) / 256, cols256 = (n + 255) / 256;
+    const int64_t full_cols = (tiles_m256 * cols256 / n_cus) * n_cus / tiles_m256;
+    if (full_cols > 0 && full_cols < cols256)
+        consider({128, 256, 1, full_cols},
+                 (double)(tiles_m256 * full_cols / n_cus) * k_steps +
+                     rounds(tiles(128, 256, n - full_cols * 256)) * k_steps * 0.5 / kQ128);
+    // split along k: the slices' f32 tiles are written and read once more (about 4 TB/s,
+    // a 256 x 256 k step takes about 1.5 us)
+    for (int slices = 2; slices <= 8; slices *= 2) {
+        if (k_steps / slices < 8) break;
+        const double reduce_cost = 2.0 * slices * (double)m * (double)n * 4.0 / 4e12 * 1e6 / 1.5 + 2.0;
+        const double steps = (double)((k_steps + slices - 1) / slices);
+        consider({256, 256, slices, 0}, rounds(tiles(256, 256, n) * slices) * steps + reduce_cost);
+        consider({128, 256, slices, 0}, rounds(tiles(128, 256, n) * slices) * steps * 0.5 / kQ128 + reduce_cost);
+    }
+    return best;
+}
+
+template <int QT>
+hipError_t launch_qt(const GemmParams& P0, int n_cus, hipStream_t stream) {
+    const GemmPlan plan = plan_gemm(P0.m, P0.n, P0.k_units * 4, n_cus);
+    GemmParams P = P0;
+    P.n_begin = 0;
+    P.n_end = P0.n;
+    if (plan.slices > 1 && P0.partial == nullptr) return hipErrorInvalidValue;
+    if (plan.full_cols > 0) {
+        P.n_end = plan.full_cols * 256;
+        hipError_t e = launch_tile<QT, 256, 256>(P, 1, stream);
+        if (e != hipSuccess) return e;
+        P.n_begin = P.n_end;
+        P.n_end = P0.n;
+    }
+    if (plan.bm == 256) return launch_tile<QT, 256, 256>(P, plan.slices, stream);
+    if (plan.bn == 256) return launch_tile<QT, 128, 256>(P, plan.slices, stream);
+    return launch_tile<QT, 128, 128>(P, 1, stream);
 }
 
 } // namespace
 
+size_t qmm_gemm_workspace_bytes(const QmmLayout& L, int64_t m, int n_cus) {
+    if (m <= 0 || L.n == 0) return 0;
+    const GemmPlan plan = plan_gemm(m, L.n, (int)L.k_units * 4, n_cus > 0 ? n_cus : 1);
+    return plan.slices > 1 ? (size_t)plan.slices * (size_t)m * (size_t)L.n * sizeof(float) : 0;
+}
+
 hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uint16_t* x_bf16,
-                                int64_t m, void* y, int out_bf16, int n_cus, hipStream_t stream) {
+                                int64_t m, void* y, int out_bf16, void* workspace, int n_cus,
+                                hipStream_t stream) {
     if (m <= 0 || L.n == 0) return hipSuccess;
+    if (n_cus <= 0) n_cus = 1;
     GemmParams P;
     P.w = (const uint8_t*)tiled;
     P.x = x_bf16;
     P.y = y;
     P.m = m;
     P.n = L.n;
+    P.n_begin = 0;
+    P.n_end = L.n;
     P.k = L.k;
     P.k_units = (int)L.k_units;
     P.k_groups = (int)L.k_groups;
@@ -582,6 +675,8 @@ hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uin
     P.panel_bytes = L.panel_bytes;
     P.out_bf16 = out_bf16;
     P.tiles_m = P.tiles_n = 0;
+    P.slice_steps = 0;
+    P.partial = (float*)workspace;
     return L.dtype == QMM_Q4_K ? launch_qt<QMM_Q4_K>(P, n_cus, stream)
                                : launch_qt<QMM_Q8_0>(P, n_cus, stream);
 }

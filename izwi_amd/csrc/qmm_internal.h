@@ -79,9 +79,12 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
 hipError_t qmm_launch_quantize_activations(int weight_dtype, const float* x, int64_t m, int64_t k,
                                            void* out_blocks, hipStream_t stream);
 
-// Prefill kernel: bf16 activations, bf16 MFMA, f32 accumulate.
+// Prefill kernel: bf16 activations, bf16 MFMA, f32 accumulate.  Products with few output
+// tiles are split along k and need `workspace` (qmm_gemm_workspace_bytes, 0 if not split).
+size_t qmm_gemm_workspace_bytes(const QmmLayout& L, int64_t m, int n_cus);
 hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uint16_t* x_bf16,
-                                int64_t m, void* y, int out_bf16, int n_cus, hipStream_t stream);
+                                int64_t m, void* y, int out_bf16, void* workspace, int n_cus,
+                                hipStream_t stream);
 // f32 activations for m > 64: converted to bf16 into `x_bf16_ws` (m*k elements) first.
 hipError_t qmm_launch_f32_to_bf16(const float* x, uint16_t* out, int64_t count,
                                   hipStream_t stream);
