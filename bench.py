@@ -142,14 +142,44 @@ def decode_calls(torch, oracle, dtype, weights, m):
 
 
 def run_calls(qa, calls):
+    """calls: (QMatMul, x, y) single projections or ([QMatMul...], x, [y...]) projection groups."""
+    import ctypes as C
     from izwi_amd import capi
     from izwi_amd.qmatmul import _stream_ptr
     L = capi.lib()
     sp = _stream_ptr()
     for mm, x, y in calls:
-        rc = L.izwi_qmm_forward_f32(mm.qtensor._h, x.data_ptr(), x.shape[0], y.data_ptr(), capi.DEVICE, sp)
+        if isinstance(mm, (list, tuple)):
+            n = len(mm)
+            handles = (C.c_void_p * n)(*[p.qtensor._h for p in mm])
+            outs = (C.c_void_p * n)(*[t.data_ptr() for t in y])
+            rc = L.izwi_qmm_forward_group_f32(handles, n, x.data_ptr(), x.shape[0], outs, capi.DEVICE, sp)
+        else:
+            rc = L.izwi_qmm_forward_f32(mm.qtensor._h, x.data_ptr(), x.shape[0], y.data_ptr(), capi.DEVICE, sp)
         if rc:
             capi.check(rc)
+
+
+def grouped_decode_calls(torch, oracle, dtype, weights, m):
+    """The same projections called the way Qwen3Attention::forward / Qwen3Mlp::forward call
+    them (qwen3/core.rs:1599, 1787): qkv_proj.forward(x) and gate_up_proj.forward(x) are one
+    call each (three / two separate weights), o and down single calls: 4 calls per layer."""
+    xs = {k: torch.from_numpy(oracle.randn(7 + k, (m, k))).cuda() for k in (4096, 12288)}
+    out = lambda n: torch.empty((m, n), dtype=torch.float32, device="cuda")
+    calls, total = [], 0.0
+    per_layer = len(LAYER_8B)
+    n_layers = (len(weights) - 1) // per_layer
+    for layer in range(n_layers):
+        w = weights[layer * per_layer:(layer + 1) * per_layer]  # q k v o gate up down
+        calls.append(([w[0][0], w[1][0], w[2][0]], xs[4096], [out(w[0][1]), out(w[1][1]), out(w[2][1])]))
+        calls.append((w[3][0], xs[4096], out(w[3][1])))
+        calls.append(([w[4][0], w[5][0]], xs[4096], [out(w[4][1]), out(w[5][1])]))
+        calls.append((w[6][0], xs[12288], out(w[6][1])))
+        total += sum(gemv_bytes(dtype, n, k, m) for _, n, k in w)
+    mm, n, k = weights[-1]
+    calls.append((mm, xs[k], out(n)))
+    total += gemv_bytes(dtype, n, k, m)
+    return calls, total
 
 
 def cpu_baseline(oracle, dtype, m, budget_s=12.0):
@@ -356,6 +386,11 @@ def main():
                 extras[f"decode_gbs_m{m}"] = round(tb / (t * 1e-3) / 1e9, 1)
                 extras[f"decode_ms_per_step_m{m}"] = round(t, 4)
                 del c, g
+            c, tb = grouped_decode_calls(torch, oracle, dtype, weights, args.m)
+            t, g = time_graph(torch, lambda: run_calls(qa, c), max(5, args.steps // 2), 3)
+            extras["decode_grouped_calls"] = {"gbs": round(tb / (t * 1e-3) / 1e9, 1), "ms_per_step": round(t, 4),
+                                              "calls_per_step": len(c)}
+            del c, g
         except Exception as exc:  # extras never invalidate the headline number
             extras["decode_error"] = repr(exc)
     del weights

@@ -153,6 +153,16 @@ int izwi_qmm_dequantize_f32(const izwi_qmm_weight* w, float* out, int mem_space,
 int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, float* y,
                          int mem_space, void* stream);
 
+/* `Qwen3QkvProjection::forward` and `Qwen3GateUpProjection::forward`, `Separate` arms
+ * (qwen3/core.rs:1119-1127, 1274-1282): several projections applied to the same
+ * activations, y_i = QMatMul_i.forward(x), bit-identical to n_weights calls of
+ * izwi_qmm_forward_f32.  The weights must share k; with equal block types the decode
+ * sizes run as one kernel launch (m <= 2) or share one activation quantization
+ * (m <= 64).  n_weights <= 4. */
+int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_weights,
+                               const float* x, int64_t m, float* const* ys, int mem_space,
+                               void* stream);
+
 /* Prefill form: bf16 activations `[m, k]`, weights dequantized to bf16 in LDS,
  * MFMA with f32 accumulation; y is f32 or bf16 per `out_dtype`.  Replaces the
  * to_dtype(F32) -> QMatMul -> to_dtype(activation dtype) sequence of

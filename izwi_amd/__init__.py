@@ -12,7 +12,10 @@ from .qmatmul import (  # noqa: F401
     MoeExperts,
     QMatMul,
     QTensor,
+    Qwen3GateUpProjection,
     Qwen3Projection,
+    Qwen3QkvProjection,
+    forward_group,
     moe_route,
     moe_sort,
     packed_qmatmul_from_qtensors,

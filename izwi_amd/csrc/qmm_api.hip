@@ -513,6 +513,60 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
     return IZWI_QMM_OK;
 }
 
+int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_weights,
+                               const float* x, int64_t m, float* const* ys, int mem_space,
+                               void* stream_) {
+    if (!weights || !ys) return fail(IZWI_QMM_ERR_INVALID, "NULL argument");
+    if (n_weights < 1 || n_weights > QMM_MAX_GROUP)
+        return fail(IZWI_QMM_ERR_INVALID, "projection group of %d weights (1..%d supported)", n_weights, QMM_MAX_GROUP);
+    if (int rc = check_space(mem_space)) return rc;
+    bool uniform = true;
+    for (int i = 0; i < n_weights; i++) {
+        if (!weights[i]) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+        const QmmLayout& L = weights[i]->layout;
+        if (L.n_stacked != 1) return fail(IZWI_QMM_ERR_INVALID, "forward on an expert stack");
+        if (L.k != weights[0]->layout.k)
+            return fail(IZWI_QMM_ERR_INVALID, "projection group input mismatch: expected %lld, got %lld",
+                        (long long)weights[0]->layout.k, (long long)L.k);
+        if (L.dtype != weights[0]->layout.dtype || L.n == 0 || weights[i]->device != weights[0]->device)
+            uniform = false;
+        if (m > 0 && L.n > 0 && !ys[i]) return fail(IZWI_QMM_ERR_INVALID, "y is NULL");
+    }
+    if (m < 0) return fail(IZWI_QMM_ERR_INVALID, "negative m");
+    if (m == 0) return IZWI_QMM_OK;
+    if (!x) return fail(IZWI_QMM_ERR_INVALID, "x is NULL");
+    // host buffers, mixed types, prefill sizes: one call per projection (same results)
+    if (mem_space != IZWI_QMM_DEVICE || !uniform || n_weights == 1 || m > 64) {
+        for (int i = 0; i < n_weights; i++)
+            if (int rc = izwi_qmm_forward_f32(weights[i], x, m, ys[i], mem_space, stream_)) return rc;
+        return IZWI_QMM_OK;
+    }
+    hipStream_t stream = (hipStream_t)stream_;
+    const izwi_qmm_weight* w0 = weights[0];
+    if (m < mfma_min_m()) {
+        const QmmLayout* layouts[QMM_MAX_GROUP];
+        const void* tiled[QMM_MAX_GROUP];
+        for (int i = 0; i < n_weights; i++) layouts[i] = &weights[i]->layout, tiled[i] = weights[i]->tiled;
+        ProfileScope prof(w0, stream);
+        hipError_t e = qmm_launch_gemv_multi(layouts, tiled, n_weights, x, m, ys, w0->n_cus, stream);
+        if (e == hipSuccess) return IZWI_QMM_OK;
+        if (e != hipErrorNotSupported) return fail_hip(e, "grouped decode kernel");
+        (void)hipGetLastError();
+        for (int i = 0; i < n_weights; i++)
+            if (int rc = izwi_qmm_forward_f32(weights[i], x, m, ys[i], mem_space, stream_)) return rc;
+        return IZWI_QMM_OK;
+    }
+    // 3 <= m <= 64: the activations are quantized once, every projection reads the same records
+    void* scratch = nullptr;
+    HIP_TRY(get_scratch(w0->device, stream, qmm_gemv_mfma_workspace_bytes(w0->layout, m), &scratch));
+    for (int i = 0; i < n_weights; i++) {
+        ProfileScope prof(weights[i], stream);
+        HIP_TRY(qmm_launch_gemv_mfma(weights[i]->layout, weights[i]->tiled, x, m, ys[i], scratch,
+                                     weights[i]->n_cus, stream, i == 0));
+    }
+    return IZWI_QMM_OK;
+}
+
 int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int64_t m, void* y,
                           int out_dtype, int mem_space, void* stream_) {
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");

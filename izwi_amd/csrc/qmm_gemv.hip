@@ -361,6 +361,13 @@ struct GemvParams {
     const int32_t* seg_expert;  // [max segments]: expert of the segment, -1 past the last
     int n_experts;
     int x_div; // x row of pair p is p / x_div
+    // several weights of equal k and type on the same activations in one launch:
+    // workgroup b belongs to weight i with rtg_end[i - 1] <= b < rtg_end[i]
+    int n_weights; // 0 or 1: just w / y / n / row_tiles above
+    int rtg_end[QMM_MAX_GROUP];
+    int nv[QMM_MAX_GROUP], row_tiles_v[QMM_MAX_GROUP];
+    const uint8_t* wv[QMM_MAX_GROUP];
+    float* yv[QMM_MAX_GROUP];
 };
 static_assert(offsetof(GemvParams, k_units) == 64, "first-load fields must fill one 64-byte line");
 
@@ -375,8 +382,8 @@ __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 // the three loops below run once and the kernel is straight-line code from its
 // entry to the first load.
 template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT>
-__device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int m_end, int64_t w_offset,
-                                          uint8_t* smem) {
+__device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int m_end, const uint8_t* w_first,
+                                          float* y_out, int n_rows, int row_tiles, int rtg0, uint8_t* smem) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int stack_waves = P.nwk * P.nwr;               // waves per weight stack
@@ -388,13 +395,13 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
     const bool lane_active = lane < P.slots;
     const int us = lane >> 4;
     const int k_units = (P.k + 255) >> 8, s_units = P.slots >> 4;
-    const uint8_t* wbase = (stack ? P.w2 : P.w) + w_offset;
+    const uint8_t* wbase = stack ? P.w2 + (w_first - P.w) : w_first; // the second stack at the same offset
     const XLds<QT> l = carve<QT, MT>(smem, k_units);
 
     for (int m0 = m_begin; ONESHOT ? m0 == m_begin : m0 < m_end; m0 += MT) {
         bool x_ready = false;
         int red_buf = 0;
-        for (int rtg = blockIdx.x; ONESHOT ? rtg == (int)blockIdx.x : rtg < P.rt_groups;
+        for (int rtg = rtg0; ONESHOT ? rtg == rtg0 : rtg < P.rt_groups;
              rtg += ONESHOT ? 1 : (int)gridDim.x) {
             const int rt = rtg * P.nwr + wr;
             float acc[MT];
@@ -402,7 +409,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
             for (int mi = 0; mi < MT; mi++) acc[mi] = 0.0f;
             for (int ks = 0; ONESHOT ? ks < 1 : ks < P.kpw; ks++) {
                 const int kg = ks * P.nwk + wk;
-                const bool ok = rt < P.row_tiles && kg < P.k_groups;
+                const bool ok = rt < row_tiles && kg < P.k_groups;
                 const int64_t off = ok ? (int64_t)(rt * P.k_groups + kg) * P.panel_bytes : 0;
                 Panel<QT> p;
                 const bool active = ok && lane_active;
@@ -441,12 +448,12 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
             }
             if (P.nwk == 1 && !GATED) {
                 const int row = rt * 16 + lane;
-                if (lane < 16 && rt < P.row_tiles && row < P.n) {
+                if (lane < 16 && rt < row_tiles && row < n_rows) {
 #pragma unroll
                     for (int mi = 0; mi < MT; mi++) {
                         if (m0 + mi < m_end) {
                             int64_t yr = GROUPED ? P.perm[m0 + mi] : m0 + mi;
-                            P.y[yr * P.n + row] = acc[mi];
+                            y_out[yr * n_rows + row] = acc[mi];
                         }
                     }
                 }
@@ -465,9 +472,9 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                         if (GATED) sum2 += red[((stack_waves + wr * P.nwk + w2) * MT + mi) * 16 + r];
                     }
                     const int row = rt * 16 + r;
-                    if (rt < P.row_tiles && row < P.n && m0 + mi < m_end) {
+                    if (rt < row_tiles && row < n_rows && m0 + mi < m_end) {
                         int64_t yr = GROUPED ? P.perm[m0 + mi] : m0 + mi;
-                        P.y[yr * P.n + row] = GATED ? silu(sum) * sum2 : sum;
+                        y_out[yr * n_rows + row] = GATED ? silu(sum) * sum2 : sum;
                     }
                 }
                 red_buf ^= 1;
@@ -493,13 +500,28 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
         m_end = min(P.offsets[lo + 1], m_begin + QMM_MOE_SEG_ROWS);
         w_offset = (int64_t)lo * P.matrix_bytes;
     }
+    const uint8_t* w_first = P.w + w_offset;
+    float* y_out = P.y;
+    int n_rows = P.n, row_tiles = P.row_tiles, rtg0 = blockIdx.x;
+    if (!GROUPED && ONESHOT && P.n_weights > 1) {
+        int i = 0;
+        while (i + 1 < P.n_weights && (int)blockIdx.x >= P.rtg_end[i]) i++;
+        rtg0 = blockIdx.x - (i ? P.rtg_end[i - 1] : 0);
+        w_first = P.wv[i];
+        y_out = P.yv[i];
+        n_rows = P.nv[i];
+        row_tiles = P.row_tiles_v[i];
+    }
     if (GROUPED && ONESHOT && MT == 4) {
         const int rows = m_end - m_begin;
-        if (rows == 1) gemv_body<QT, 1, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_offset, smem);
-        else if (rows == 2) gemv_body<QT, 2, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_offset, smem);
-        else gemv_body<QT, 4, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_offset, smem);
+        if (rows == 1)
+            gemv_body<QT, 1, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
+        else if (rows == 2)
+            gemv_body<QT, 2, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
+        else
+            gemv_body<QT, 4, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     } else {
-        gemv_body<QT, MT, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_offset, smem);
+        gemv_body<QT, MT, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     }
 }
 
@@ -595,6 +617,7 @@ bool make_params(const QmmLayout& L, const void* tiled, const float* x, int64_t 
     P.seg_expert = nullptr;
     P.n_experts = 0;
     P.x_div = 1;
+    P.n_weights = 0;
     return true;
 }
 
@@ -656,6 +679,56 @@ hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x
     choose_split(L, n_cus, 1, false, P, waves);
     return L.dtype == QMM_Q4_K ? launch_plain<QMM_Q4_K>(P, waves, n_cus, stream)
                                : launch_plain<QMM_Q8_0>(P, waves, n_cus, stream);
+}
+
+hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
+                                 const float* x, int64_t m, float* const* ys, int n_cus,
+                                 hipStream_t stream) {
+    if (n_weights < 1 || n_weights > QMM_MAX_GROUP || m < 1 || m > 2) return hipErrorInvalidValue;
+    const QmmLayout& L0 = *layouts[0];
+    int64_t total_row_tiles = 0;
+    for (int i = 0; i < n_weights; i++) {
+        const QmmLayout& L = *layouts[i];
+        if (L.dtype != L0.dtype || L.k != L0.k || L.n_stacked != 1 || L.n == 0) return hipErrorInvalidValue;
+        total_row_tiles += L.row_tiles;
+    }
+    if (L0.k_groups > kMaxWaves) return hipErrorNotSupported; // no straight-line form: the caller launches one by one
+    GemvParams P;
+    if (!make_params(L0, tiled[0], x, m, ys[0], P)) return hipErrorInvalidValue;
+    // the split of a single matrix with all the row-tiles
+    QmmLayout all = L0;
+    all.row_tiles = total_row_tiles;
+    int waves;
+    choose_split(all, n_cus, 1, false, P, waves);
+    if (P.kpw != 1) return hipErrorNotSupported;
+    P.n_weights = n_weights;
+    int64_t groups = 0;
+    for (int i = 0; i < n_weights; i++) {
+        const QmmLayout& L = *layouts[i];
+        if (L.n > 0x3fffffff) return hipErrorInvalidValue;
+        groups += (L.row_tiles + P.nwr - 1) / P.nwr;
+        P.rtg_end[i] = (int)groups;
+        P.nv[i] = (int)L.n;
+        P.row_tiles_v[i] = (int)L.row_tiles;
+        P.wv[i] = (const uint8_t*)tiled[i];
+        P.yv[i] = ys[i];
+    }
+    if (groups > (int64_t)n_cus * 32) return hipErrorNotSupported;
+    P.rt_groups = (int)groups;
+    const int mt = m == 2 ? 2 : 1;
+    const size_t lds = mt == 2 ? lds_bytes<QMM_Q4_K, 2>(P.k_units, waves) : lds_bytes<QMM_Q4_K, 1>(P.k_units, waves);
+    const size_t lds8 = mt == 2 ? lds_bytes<QMM_Q8_0, 2>(P.k_units, waves) : lds_bytes<QMM_Q8_0, 1>(P.k_units, waves);
+    const size_t need = L0.dtype == QMM_Q4_K ? lds : lds8;
+    if (need > 48 * 1024) return hipErrorNotSupported;
+    const dim3 g((unsigned)groups), b(64 * waves);
+    if (L0.dtype == QMM_Q4_K) {
+        if (mt == 2) gemv_kernel<QMM_Q4_K, 2, false, false, true><<<g, b, need, stream>>>(P);
+        else gemv_kernel<QMM_Q4_K, 1, false, false, true><<<g, b, need, stream>>>(P);
+    } else {
+        if (mt == 2) gemv_kernel<QMM_Q8_0, 2, false, false, true><<<g, b, need, stream>>>(P);
+        else gemv_kernel<QMM_Q8_0, 1, false, false, true><<<g, b, need, stream>>>(P);
+    }
+    return hipGetLastError();
 }
 
 hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,

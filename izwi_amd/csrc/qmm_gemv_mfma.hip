@@ -612,7 +612,8 @@ size_t qmm_gemv_mfma_workspace_bytes(const QmmLayout& L, int64_t m) {
 }
 
 hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
-                                float* y, void* workspace, int n_cus, hipStream_t stream) {
+                                float* y, void* workspace, int n_cus, hipStream_t stream,
+                                bool quantize) {
     if (m <= 0 || L.n == 0) return hipSuccess;
     if (L.n > 0x3fffffff || L.k > 0x3fffffff || m > 0x3fffffff ||
         L.row_tiles * L.k_groups > 0x7fffffff)
@@ -620,7 +621,7 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     if (n_cus <= 0) n_cus = 1;
     const int n_tiles = (int)((m + 15) / 16);
     uint8_t* ws = (uint8_t*)workspace;
-    {
+    if (quantize) {
         int64_t threads = (int64_t)n_tiles * 16 * L.k_units * 16;
         unsigned grid = (unsigned)((threads + 255) / 256);
         if (L.dtype == QMM_Q4_K)

@@ -71,9 +71,12 @@ hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x
 // Batched decode kernel (int8 MFMA) for 3 <= m <= 64.  `workspace` must hold
 // qmm_gemv_mfma_workspace_bytes(L, m) bytes and stay untouched until the work
 // queued on `stream` has run.
+// `quantize` false: the workspace already holds the quantized activations of x for this k
+// and type (a previous call on the same x), only the matmul is launched.
 size_t qmm_gemv_mfma_workspace_bytes(const QmmLayout& L, int64_t m);
 hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
-                                float* y, void* workspace, int n_cus, hipStream_t stream);
+                                float* y, void* workspace, int n_cus, hipStream_t stream,
+                                bool quantize = true);
 
 // Activation quantizer written out in the reference's block layout.
 hipError_t qmm_launch_quantize_activations(int weight_dtype, const float* x, int64_t m, int64_t k,
@@ -88,6 +91,14 @@ hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uin
 // f32 activations for m > 64: converted to bf16 into `x_bf16_ws` (m*k elements) first.
 hipError_t qmm_launch_f32_to_bf16(const float* x, uint16_t* out, int64_t count,
                                   hipStream_t stream);
+
+// Several weights of equal k and type applied to the same activations (m <= 2) in one launch
+// of the decode kernel; y_i = x W_i^T exactly as separate launches would give.
+// hipErrorNotSupported: the shapes have no single-launch form, launch them one by one.
+#define QMM_MAX_GROUP 4
+hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
+                                 const float* x, int64_t m, float* const* ys, int n_cus,
+                                 hipStream_t stream);
 
 // ---- MoE ---------------------------------------------------------------------
 // Sorted pairs are processed in segments of this many rows that share one expert.

@@ -187,6 +187,16 @@ inline QMatMul packed_qmatmul_from_qtensors(const std::vector<std::shared_ptr<QT
     return QMatMul::from_arc(QTensor::adopt(h)); // the new handle owns its own copy of the bytes
 }
 
+// The `Separate` arms of `Qwen3QkvProjection::forward` / `Qwen3GateUpProjection::forward`
+// (core.rs:1119-1127, 1274-1282): several projections on the same activations in one call;
+// ys[i] is [m, projections[i].out_features()].
+inline void forward_group(const std::vector<const QMatMul*>& projections, const float* x, int64_t m,
+                          const std::vector<float*>& ys, MemSpace space, void* stream = nullptr) {
+    std::vector<const izwi_qmm_weight*> handles;
+    for (const QMatMul* p : projections) handles.push_back(p->qtensor()->handle());
+    check(izwi_qmm_forward_group_f32(handles.data(), (int32_t)handles.size(), x, m, ys.data(), (int)space, stream));
+}
+
 // `Qwen3Projection` (quantized arm): the op always receives f32 activations and
 // returns f32 (core.rs:772-831); callers with other activation dtypes cast around it.
 class Qwen3Projection {

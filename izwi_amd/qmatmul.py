@@ -229,6 +229,57 @@ class Qwen3Projection:
         return self.qmatmul.forward(x.to(torch.float32)).to(x.dtype)
 
 
+def forward_group(projections: Sequence["QMatMul"], x: torch.Tensor):
+    """Several projections on the same activations in one call (the `Separate` arms of
+    Qwen3QkvProjection::forward / Qwen3GateUpProjection::forward, qwen3/core.rs:1119-1127,
+    1274-1282).  Returns one output per projection, identical to separate forwards."""
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    k = x.shape[-1]
+    m = x.numel() // k if k else 0
+    n = len(projections)
+    ys = [torch.empty(tuple(x.shape[:-1]) + (p.qtensor.dims2()[0],), dtype=torch.float32, device=x.device)
+          for p in projections]
+    handles = (C.c_void_p * n)(*[p.qtensor._h for p in projections])
+    outs = (C.c_void_p * n)(*[y.data_ptr() for y in ys])
+    check(lib().izwi_qmm_forward_group_f32(handles, n, x.data_ptr(), m, outs, _space(x), _stream_ptr(x)))
+    return tuple(ys)
+
+
+class Qwen3QkvProjection:
+    """izwi-core's Qwen3QkvProjection with quantized weights: `new_separate` keeps q, k, v as
+    three weights (the reference's default off Metal), `new_quantized_grouped` packs them."""
+
+    def __init__(self, parts=None, fused=None, splits=None):
+        self._parts, self._fused, self._splits = parts, fused, splits
+
+    @classmethod
+    def new_separate(cls, q_proj: "QMatMul", k_proj: "QMatMul", v_proj: "QMatMul"):
+        return cls(parts=(q_proj, k_proj, v_proj))
+
+    @classmethod
+    def new_quantized_grouped(cls, parts: Sequence[tuple]):
+        fused = packed_qmatmul_from_qtensors(parts)
+        return cls(fused=fused, splits=[shape[0] for _, _, shape in parts])
+
+    def forward(self, x: torch.Tensor):
+        if self._fused is None:
+            return forward_group(self._parts, x)
+        y = self._fused.forward(x)  # one matmul, then `narrow` on the last dim
+        outs, off = [], 0
+        for rows in self._splits:
+            outs.append(y.narrow(-1, off, rows))
+            off += rows
+        return tuple(outs)
+
+
+class Qwen3GateUpProjection(Qwen3QkvProjection):
+    """izwi-core's Qwen3GateUpProjection (gate, up) with quantized weights."""
+
+    @classmethod
+    def new_separate(cls, gate_proj: "QMatMul", up_proj: "QMatMul"):  # noqa: D102
+        return cls(parts=(gate_proj, up_proj))
+
+
 def quantize_activations(weight_dtype: GgmlDType, x: torch.Tensor) -> torch.Tensor:
     """The activation blocks the decode kernel builds (reference block layout, uint8)."""
     assert x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2

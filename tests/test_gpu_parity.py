@@ -383,3 +383,38 @@ def test_moe_forward_small_shapes(qa, oracle, dtype, E, hidden, inter, t, top_k)
     want = oracle.moe_forward(dtype, x, want_ids, want_wts, gate, up, down, E, inter)
     assert np.array_equal(ids.cpu().numpy(), want_ids)
     assert rel_err(out, want) < 1e-3
+
+
+@pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
+@pytest.mark.parametrize("m", [1, 2, 5, 16, 40, 80])
+def test_projection_group_equals_separate_calls(qa, oracle, dtype, m):
+    """Qwen3QkvProjection / Qwen3GateUpProjection `Separate` arms as one call: bit-identical to
+    separate forwards (one launch for m <= 2, shared activation quantization up to 64)."""
+    k = 1024
+    dt = qa.GgmlDType(dtype)
+    parts = [qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, make_weight(oracle, dtype, n, k, 400 + n), (n, k)))
+             for n in (2048, 1024, 1000)]
+    x = torch.from_numpy(oracle.randn(401 + m, (m, k))).cuda()
+    q, kk, v = qa.Qwen3QkvProjection.new_separate(*parts).forward(x)
+    for got, p in zip((q, kk, v), parts):
+        assert torch.equal(got, p.forward(x))
+    # and against the oracle for one of them
+    want = oracle.qmatmul(dtype, x.cpu().numpy(), make_weight(oracle, dtype, 1000, k, 1400), 1000)
+    tol = DECODE_TOL if m <= 64 else PREFILL_TOL
+    assert rel_err(v.cpu().numpy(), want) < tol
+
+
+def test_projection_group_8b_gate_up_and_errors(qa, oracle):
+    dt = qa.GgmlDType.Q4K
+    gate = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, make_weight(oracle, Q4_K, 12288, 4096, 410), (12288, 4096)))
+    up = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, make_weight(oracle, Q4_K, 12288, 4096, 411), (12288, 4096)))
+    x = torch.from_numpy(oracle.randn(412, (1, 4096))).cuda()
+    g, u = qa.Qwen3GateUpProjection.new_separate(gate, up).forward(x)
+    assert torch.equal(g, gate.forward(x)) and torch.equal(u, up.forward(x))
+    other_k = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, make_weight(oracle, Q4_K, 64, 1024, 413), (64, 1024)))
+    with pytest.raises(qa.QmmError, match="input mismatch"):
+        qa.forward_group([gate, other_k], x)
+    # mixed block types still work (one call per projection inside)
+    q8 = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q8_0, make_weight(oracle, Q8_0, 96, 4096, 414), (96, 4096)))
+    a, b = qa.forward_group([up, q8], x)
+    assert torch.equal(a, up.forward(x)) and torch.equal(b, q8.forward(x))
