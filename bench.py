@@ -3,9 +3,12 @@
 
 Default workload (`decode_q4k_8b_stack`): one decode token's worth of
 projections of a Qwen3-8B-shaped decoder with Q4_K weights at M = 1 — 36 layers
-x (q, k, v, o, gate, up, down) plus the LM head, 253 fused dequant+GEMV
-launches over 4.26 GB of distinct weight buffers (far beyond the 256 MB
-last-level cache, so the weights stream from HBM every step).  A step is one
+x (q, k, v, o, gate, up, down) plus the LM head over 4.26 GB of distinct weight
+buffers (far beyond the 256 MB last-level cache, so the weights stream from HBM
+every step), called as the reference's attention and MLP blocks call them:
+qkv_proj.forward(x) and gate_up_proj.forward(x) are one projection-group call
+each (three / two separate weights), o, down and the LM head single calls =
+145 calls per step (`--calls per-projection`: 253 single calls).  A step is one
 pass over all of them, replayed from a HIP graph.  `value` is algorithmic
 bytes (GGUF weight bytes + f32 activations in and out) per second.
 
@@ -306,6 +309,10 @@ def main():
                     help="also run one plain 1 GiB device copy (a known-size kernel that scales "
                          "the rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--calls", default="grouped", choices=["grouped", "per-projection"],
+                    help="grouped: qkv_proj.forward(x) and gate_up_proj.forward(x) are one call each, as "
+                         "the reference's attention and MLP blocks make them (4 calls per layer); "
+                         "per-projection: seven izwi_qmm_forward_f32 calls per layer")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -329,7 +336,8 @@ def main():
         del src, dst
 
     weights = build_decode_weights(torch, qa, oracle, dtype, args.layers, True)
-    calls, total_bytes = decode_calls(torch, oracle, dtype, weights, args.m)
+    make_calls = grouped_decode_calls if args.calls == "grouped" else decode_calls
+    calls, total_bytes = make_calls(torch, oracle, dtype, weights, args.m)
     launches = len(calls)
     ms, _graph = time_graph(torch, lambda: run_calls(qa, calls), args.steps, args.warmup)
     gbs = total_bytes / (ms * 1e-3) / 1e9
@@ -352,9 +360,13 @@ def main():
                 "device buffers (same seeded bytes per projection kind); lm_head repeats 16384 seeded rows",
         "config": {
             "workload": f"{args.workload}: Qwen3-8B shapes, {args.layers} layers x 7 projections + lm_head, "
-                        f"M={args.m}, {launches} launches/step, {total_bytes / 1e9:.3f} GB algorithmic bytes/step, "
-                        "HIP-graph replay",
+                        f"M={args.m}, {launches} calls/step ("
+                        + ("qkv and gate/up as one projection-group call each, o / down / lm_head single calls: "
+                           "the calls of the reference's Qwen3Attention::forward and Qwen3Mlp::forward"
+                           if args.calls == "grouped" else "one call per projection")
+                        + f"), {total_bytes / 1e9:.3f} GB algorithmic bytes/step, HIP-graph replay",
             "m": args.m,
+            "calls": args.calls,
             "launches_per_step": launches,
             "algorithmic_bytes_per_step": int(total_bytes),
         },
@@ -367,7 +379,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": measured_traffic(args.workload, args.m, total_bytes / launches),
+            "traffic": measured_traffic(f"{args.workload}:{args.calls}", args.m, total_bytes / launches),
             "avg_launch_us": round(ms * 1e3 / launches, 3),
             "avg_algorithmic_bytes_per_launch": int(total_bytes / launches),
         },
@@ -381,15 +393,17 @@ def main():
             for m in (8, 16):
                 if m == args.m:
                     continue
-                c, tb = decode_calls(torch, oracle, dtype, weights, m)
+                c, tb = make_calls(torch, oracle, dtype, weights, m)
                 t, g = time_graph(torch, lambda: run_calls(qa, c), max(5, args.steps // 5), 3)
                 extras[f"decode_gbs_m{m}"] = round(tb / (t * 1e-3) / 1e9, 1)
                 extras[f"decode_ms_per_step_m{m}"] = round(t, 4)
                 del c, g
-            c, tb = grouped_decode_calls(torch, oracle, dtype, weights, args.m)
+            # the other call structure at the headline's m
+            other = decode_calls if args.calls == "grouped" else grouped_decode_calls
+            c, tb = other(torch, oracle, dtype, weights, args.m)
             t, g = time_graph(torch, lambda: run_calls(qa, c), max(5, args.steps // 2), 3)
-            extras["decode_grouped_calls"] = {"gbs": round(tb / (t * 1e-3) / 1e9, 1), "ms_per_step": round(t, 4),
-                                              "calls_per_step": len(c)}
+            extras["decode_per_projection_calls" if args.calls == "grouped" else "decode_grouped_calls"] = {
+                "gbs": round(tb / (t * 1e-3) / 1e9, 1), "ms_per_step": round(t, 4), "calls_per_step": len(c)}
             del c, g
         except Exception as exc:  # extras never invalidate the headline number
             extras["decode_error"] = repr(exc)
