@@ -557,12 +557,24 @@ int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_
         return IZWI_QMM_OK;
     }
     // 3 <= m <= 64: the activations are quantized once, every projection reads the same records
+    // (up to 16 rows in one launch for all of them)
     void* scratch = nullptr;
     HIP_TRY(get_scratch(w0->device, stream, qmm_gemv_mfma_workspace_bytes(w0->layout, m), &scratch));
+    HIP_TRY(qmm_launch_quantize_ws(w0->layout.dtype, x, m, w0->layout.k, scratch, stream));
+    {
+        const QmmLayout* layouts[QMM_MAX_GROUP];
+        const void* tiled[QMM_MAX_GROUP];
+        for (int i = 0; i < n_weights; i++) layouts[i] = &weights[i]->layout, tiled[i] = weights[i]->tiled;
+        ProfileScope prof(w0, stream);
+        hipError_t e = qmm_launch_gemv_mfma_multi(layouts, tiled, n_weights, m, ys, scratch, w0->n_cus, stream);
+        if (e == hipSuccess) return IZWI_QMM_OK;
+        if (e != hipErrorNotSupported) return fail_hip(e, "grouped batched decode kernel");
+        (void)hipGetLastError();
+    }
     for (int i = 0; i < n_weights; i++) {
         ProfileScope prof(weights[i], stream);
         HIP_TRY(qmm_launch_gemv_mfma(weights[i]->layout, weights[i]->tiled, x, m, ys[i], scratch,
-                                     weights[i]->n_cus, stream, i == 0));
+                                     weights[i]->n_cus, stream, false));
     }
     return IZWI_QMM_OK;
 }

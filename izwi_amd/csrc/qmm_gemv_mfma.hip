@@ -220,6 +220,13 @@ struct MfmaParams {
     const uint8_t* w2; // grouped form, blockIdx.z == 1: second stack and its output
     float* y2;
     int double_buf;    // two LDS windows
+    // several weights of equal k and type on the same records in one launch (SINGLE form):
+    // workgroup b belongs to weight i with rtg_end[i - 1] <= b < rtg_end[i]
+    int n_weights; // 0 or 1: just w / y / n / row_tiles above
+    int rtg_end[QMM_MAX_GROUP];
+    int nv[QMM_MAX_GROUP], row_tiles_v[QMM_MAX_GROUP];
+    const uint8_t* wv[QMM_MAX_GROUP];
+    float* yv[QMM_MAX_GROUP];
     int m, n;
     int k_units, k_groups, slots;
     int row_tiles, panel_bytes;
@@ -444,15 +451,25 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
     const int wk = wave - wr * P.nwk;
     const int j = lane & 15, grp = lane >> 4;
     const int s_units = P.slots >> 4;
-    const int rt = blockIdx.x * P.nwr + wr;
-    const bool rt_ok = rt < P.row_tiles;
+    const uint8_t* wbase = P.w;
+    float* yout = P.y;
+    int n_rows = P.n, row_tiles = P.row_tiles, rtg = blockIdx.x;
+    if (SINGLE && !GROUPED && P.n_weights > 1) {
+        int i = 0;
+        while (i + 1 < P.n_weights && (int)blockIdx.x >= P.rtg_end[i]) i++;
+        rtg = blockIdx.x - (i ? P.rtg_end[i - 1] : 0);
+        wbase = P.wv[i];
+        yout = P.yv[i];
+        n_rows = P.nv[i];
+        row_tiles = P.row_tiles_v[i];
+    }
+    const int rt = rtg * P.nwr + wr;
+    const bool rt_ok = rt < row_tiles;
     const int unit0 = wk * s_units;                       // first unit of this wave's panel
     const int n_units = min(s_units, P.k_units - unit0);  // its units that exist (>= 1)
     const int row = rt * 16 + j;
 
-    const uint8_t* wbase = P.w;
     const uint8_t* records = P.ws;
-    float* yout = P.y;
     int n_tiles = P.n_tiles, pos_begin = 0, pos_end = 0;
     if (GROUPED) {
         const int e = blockIdx.y;
@@ -516,13 +533,13 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
             auto store = [&](int r, float v) {
                 const int mm = tile * 16 + grp * 4 + r;
                 if (GROUPED) {
-                    if (pos_begin + mm < pos_end) yout[(int64_t)P.perm[pos_begin + mm] * P.n + row] = v;
+                    if (pos_begin + mm < pos_end) yout[(int64_t)P.perm[pos_begin + mm] * n_rows + row] = v;
                 } else if (mm < P.m) {
-                    yout[(int64_t)mm * P.n + row] = v;
+                    yout[(int64_t)mm * n_rows + row] = v;
                 }
             };
             if (P.nwk == 1) {
-                if (rt_ok && row < P.n) {
+                if (rt_ok && row < n_rows) {
 #pragma unroll
                     for (int r = 0; r < 4; r++) store(r, acc[r]);
                 }
@@ -531,7 +548,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
 #pragma unroll
                 for (int r = 0; r < 4; r++) lds_red[(wave * 4 + r) * 64 + lane] = acc[r];
                 lds_barrier();
-                if (wk == 0 && rt_ok && row < P.n) {
+                if (wk == 0 && rt_ok && row < n_rows) {
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
                         float sum = 0.0f;
@@ -607,6 +624,20 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_stream_kernel(MfmaPa
 
 } // namespace
 
+hipError_t qmm_launch_quantize_ws(int dtype, const float* x, int64_t m, int64_t k, void* workspace,
+                                  hipStream_t stream) {
+    if (m <= 0 || k <= 0 || m > 0x3fffffff || k > 0x3fffffff) return hipErrorInvalidValue;
+    const int n_tiles = (int)((m + 15) / 16);
+    const int64_t k_units = (k + 255) / 256;
+    const int64_t threads = (int64_t)n_tiles * 16 * k_units * 16;
+    const unsigned grid = (unsigned)((threads + 255) / 256);
+    if (dtype == QMM_Q4_K)
+        quantize_ws_kernel<QMM_Q4_K><<<grid, 256, 0, stream>>>(x, (int)m, (int)k, (int)k_units, n_tiles, (uint8_t*)workspace);
+    else
+        quantize_ws_kernel<QMM_Q8_0><<<grid, 256, 0, stream>>>(x, (int)m, (int)k, (int)k_units, n_tiles, (uint8_t*)workspace);
+    return hipGetLastError();
+}
+
 size_t qmm_gemv_mfma_workspace_bytes(const QmmLayout& L, int64_t m) {
     return (size_t)((m + 15) / 16) * (size_t)L.k_units * (size_t)unit_bytes(L.dtype);
 }
@@ -622,13 +653,7 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     const int n_tiles = (int)((m + 15) / 16);
     uint8_t* ws = (uint8_t*)workspace;
     if (quantize) {
-        int64_t threads = (int64_t)n_tiles * 16 * L.k_units * 16;
-        unsigned grid = (unsigned)((threads + 255) / 256);
-        if (L.dtype == QMM_Q4_K)
-            quantize_ws_kernel<QMM_Q4_K><<<grid, 256, 0, stream>>>(x, (int)m, (int)L.k, (int)L.k_units, n_tiles, ws);
-        else
-            quantize_ws_kernel<QMM_Q8_0><<<grid, 256, 0, stream>>>(x, (int)m, (int)L.k, (int)L.k_units, n_tiles, ws);
-        hipError_t e = hipGetLastError();
+        hipError_t e = qmm_launch_quantize_ws(L.dtype, x, m, L.k, ws, stream);
         if (e != hipSuccess) return e;
     }
     MfmaParams P;
@@ -650,6 +675,7 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     P.w2 = nullptr;
     P.y2 = nullptr;
     P.double_buf = 0;
+    P.n_weights = 0;
     P.window_units = (kWindowUnits / L.s) * L.s;
     const int padded_units = (int)(L.k_groups * L.s);
     if (P.window_units > padded_units) P.window_units = padded_units;
@@ -771,6 +797,7 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     P.matrix_bytes = L.matrix_bytes;
     P.w2 = (const uint8_t*)tiled2;
     P.y2 = y2;
+    P.n_weights = 0;
     const int waves = P.nwk * P.nwr;
     const size_t window_bytes = (size_t)P.window_units * unit_bytes(L.dtype);
     P.double_buf = 2 * window_bytes + (size_t)waves * 256 * 4 <= 160 * 1024;
@@ -788,5 +815,76 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
         gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true><<<grid, 64 * waves, lds, stream>>>(P);
     else
         gemv_mfma_oneshot_kernel<QMM_Q8_0, false, true><<<grid, 64 * waves, lds, stream>>>(P);
+    return hipGetLastError();
+}
+
+hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
+                                      int64_t m, float* const* ys, const void* workspace, int n_cus,
+                                      hipStream_t stream) {
+    if (n_weights < 1 || n_weights > QMM_MAX_GROUP || m < 1) return hipErrorInvalidValue;
+    if (n_cus <= 0) n_cus = 1;
+    const QmmLayout& L0 = *layouts[0];
+    int64_t total_row_tiles = 0;
+    for (int i = 0; i < n_weights; i++) {
+        const QmmLayout& L = *layouts[i];
+        if (L.dtype != L0.dtype || L.k != L0.k || L.n_stacked != 1 || L.n == 0 || L.n > 0x3fffffff)
+            return hipErrorInvalidValue;
+        total_row_tiles += L.row_tiles;
+    }
+    MfmaParams P;
+    P.w = (const uint8_t*)tiled[0];
+    P.ws = (const uint8_t*)workspace;
+    P.y = ys[0];
+    P.m = (int)m;
+    P.n = (int)L0.n;
+    P.k_units = (int)L0.k_units;
+    P.k_groups = (int)L0.k_groups;
+    P.slots = L0.slots;
+    P.row_tiles = (int)L0.row_tiles;
+    P.panel_bytes = (int)L0.panel_bytes;
+    P.n_tiles = 1;
+    P.perm = nullptr;
+    P.offsets = nullptr;
+    P.tile_offsets = nullptr;
+    P.matrix_bytes = 0;
+    P.w2 = nullptr;
+    P.y2 = nullptr;
+    P.double_buf = 0;
+    P.window_units = (kWindowUnits / L0.s) * L0.s;
+    const int padded_units = (int)(L0.k_groups * L0.s);
+    if (P.window_units > padded_units) P.window_units = padded_units;
+    // the straight-line form only: one row tile, one window, one wave per panel of a row-tile
+    if (m > 16 || L0.k_units > P.window_units || L0.k_groups > kMaxWaves || total_row_tiles >= 8 * (int64_t)n_cus)
+        return hipErrorNotSupported;
+    P.nwk = (int)L0.k_groups;
+    const int nwr_max = kMaxWaves / P.nwk;
+    const int64_t want = total_row_tiles / n_cus;
+    P.nwr = (int)(want < 1 ? 1 : (want > nwr_max ? nwr_max : want));
+    P.wave_magic = (65536 + P.nwk - 1) / P.nwk;
+    P.n_weights = n_weights;
+    int64_t groups = 0;
+    for (int i = 0; i < n_weights; i++) {
+        const QmmLayout& L = *layouts[i];
+        groups += (L.row_tiles + P.nwr - 1) / P.nwr;
+        P.rtg_end[i] = (int)groups;
+        P.nv[i] = (int)L.n;
+        P.row_tiles_v[i] = (int)L.row_tiles;
+        P.wv[i] = (const uint8_t*)tiled[i];
+        P.yv[i] = ys[i];
+    }
+    P.rt_groups = (int)groups;
+    const int waves = P.nwk * P.nwr;
+    const size_t lds = (size_t)P.window_units * unit_bytes(L0.dtype) + (size_t)waves * 256 * 4;
+    if (lds > 160 * 1024) return hipErrorNotSupported;
+    const void* fn = L0.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true>)
+                                          : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, true>);
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+    }
+    if (L0.dtype == QMM_Q4_K)
+        gemv_mfma_oneshot_kernel<QMM_Q4_K, true><<<(unsigned)groups, 64 * waves, lds, stream>>>(P);
+    else
+        gemv_mfma_oneshot_kernel<QMM_Q8_0, true><<<(unsigned)groups, 64 * waves, lds, stream>>>(P);
     return hipGetLastError();
 }

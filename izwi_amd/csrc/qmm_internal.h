@@ -100,6 +100,14 @@ hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* co
                                  const float* x, int64_t m, float* const* ys, int n_cus,
                                  hipStream_t stream);
 
+// The same for 3 <= m <= 16 on the matrix cores: `workspace` holds the activations already
+// quantized (qmm_launch_quantize_ws), all weights read the same records in one launch.
+hipError_t qmm_launch_quantize_ws(int dtype, const float* x, int64_t m, int64_t k, void* workspace,
+                                  hipStream_t stream);
+hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
+                                      int64_t m, float* const* ys, const void* workspace, int n_cus,
+                                      hipStream_t stream);
+
 // ---- MoE ---------------------------------------------------------------------
 // Sorted pairs are processed in segments of this many rows that share one expert.
 #define QMM_MOE_SEG_ROWS 4
