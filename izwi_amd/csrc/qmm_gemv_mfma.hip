@@ -29,6 +29,8 @@
 //    panels, the activation window stays in LDS for all of them.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include "qmm_internal.h"
 
 namespace {
@@ -442,7 +444,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
     constexpr int NL = WPanel<QT>::QC + 4; // loads of one panel
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* lds_x = smem;                                                       // window_units * UB
-    float* lds_red = reinterpret_cast<float*>(smem + (size_t)(P.double_buf ? 2 : 1) * P.window_units * UB); // waves * 256
+    // the sums of the k-split (waves * 256 floats): behind the window(s); in the single-stage form
+    // over the window itself, which nobody reads any more by then (two workgroups then fit a CU)
+    float* lds_red = SINGLE ? reinterpret_cast<float*>(smem)
+                            : reinterpret_cast<float*>(smem + (size_t)(P.double_buf ? 2 : 1) * P.window_units * UB);
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // wave-uniform by construction
@@ -544,7 +549,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
                     for (int r = 0; r < 4; r++) store(r, acc[r]);
                 }
             } else {
-                if (tile != 0) lds_barrier(); // the previous tile's sums have been read
+                if (SINGLE || tile != 0) lds_barrier(); // the window / the previous tile's sums have been read
 #pragma unroll
                 for (int r = 0; r < 4; r++) lds_red[(wave * 4 + r) * 64 + lane] = acc[r];
                 lds_barrier();
@@ -698,7 +703,8 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
         grid = (unsigned)P.rt_groups;
         const bool single_stage = n_tiles == 1 && L.k_units <= P.window_units;
         P.double_buf = !single_stage && 2 * window_bytes + (size_t)waves * 256 * 4 <= 160 * 1024;
-        lds = (P.double_buf ? 2 : 1) * window_bytes + (size_t)waves * 256 * 4;
+        lds = single_stage ? std::max(window_bytes, (size_t)waves * 256 * 4)
+                           : (P.double_buf ? 2 : 1) * window_bytes + (size_t)waves * 256 * 4;
     } else {
         P.nwk = 1;
         P.nwr = kMaxWaves;
@@ -874,7 +880,7 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
     }
     P.rt_groups = (int)groups;
     const int waves = P.nwk * P.nwr;
-    const size_t lds = (size_t)P.window_units * unit_bytes(L0.dtype) + (size_t)waves * 256 * 4;
+    const size_t lds = std::max((size_t)P.window_units * unit_bytes(L0.dtype), (size_t)waves * 256 * 4);
     if (lds > 160 * 1024) return hipErrorNotSupported;
     const void* fn = L0.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true>)
                                           : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, true>);
