@@ -32,6 +32,9 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 constexpr int BK = 64;
 constexpr int kThreads = 256;
 constexpr int kRowStride = 144; // bytes per LDS tile row: 64 bf16 + 16 B pad
+#ifndef QMM_GEMM_VALU_PER_MFMA
+#define QMM_GEMM_VALU_PER_MFMA 5
+#endif
 
 struct GemmParams {
     const uint8_t* w;
@@ -43,9 +46,10 @@ struct GemmParams {
     int64_t row_tiles, panel_bytes;
     int out_bf16;
     int tiles_m, tiles_n;
-    // split-k form (blockIdx.y = slice): slice s covers k steps [s * slice_steps, ..) and
-    // writes its f32 tile to partial[s][m][n]; a second kernel adds the slices in order
-    int slice_steps;
+    // split-k form (blockIdx.y = slice): slice s covers units [s * slice_units, ..) of 256
+    // k-elements and writes its f32 tile to partial[s][m][n]; a second kernel adds the slices
+    // in order
+    int slice_units;
     float* partial;
 };
 
@@ -304,7 +308,22 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl<N>(f, std::make_integer_sequence<int, N>{});
 }
 
-template <int QT, int BM>
+// Keeps the compiler from folding a later shift-and-mask of v into one bit-field extract
+// of the original word: the bytes of v are then converted with v_cvt_f32_ubyteN (one
+// instruction per weight instead of two).
+__device__ __forceinline__ uint32_t opaque(uint32_t v) {
+    asm("" : "+v"(v));
+    return v;
+}
+
+// Pipelined 256-column tile.  The k loop runs over units of 256 k-elements with the four
+// 64-wide steps of a unit unrolled, so that the sub-block index, the LDS stage and the
+// chunk offsets inside the panel are compile-time constants; whatever depends on the
+// step otherwise (unit offset inside the panel row, activation column) is uniform and
+// stays in scalar registers, the per-lane part of every address is a 32-bit offset
+// computed once.  XTAIL: k is not a multiple of 64 (Q8_0 only), activation chunks at or
+// past k are zeroed on their way to LDS.
+template <int QT, int BM, bool XTAIL>
 __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
     constexpr int BN = 256;
     constexpr int MT = BM / 64, NT = BN / 64;
@@ -320,9 +339,9 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
     const int64_t m0 = (int64_t)tm * BM, n0 = P.n_begin + (int64_t)tn * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int k_steps_all = P.k_units * 4;
-    const int kt0 = P.partial ? (int)blockIdx.y * P.slice_steps : 0;              // first k step of this workgroup
-    const int kt1 = P.partial ? min(k_steps_all, kt0 + P.slice_steps) : k_steps_all; // one past its last
+    const int u0 = P.partial ? (int)blockIdx.y * P.slice_units : 0;             // first unit of this workgroup
+    const int u1 = P.partial ? min(P.k_units, u0 + P.slice_units) : P.k_units;  // one past its last
+    const int last_step = P.k_units * 4 - 1;
 
     f32x16 acc[MT][NT];
 #pragma unroll
@@ -335,56 +354,88 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
     // ---- staging state: tile kt+1 sits in xr / wr while step kt runs
     u32x4 xr[XC];
     WRegs<QT, 1> wr;
-    const uint16_t* x_src[XC]; // row base + chunk offset of each activation chunk
+    // activations: uniform tile base + uniform column + per-lane (row, chunk) offset
+    const uint8_t* x_tile = reinterpret_cast<const uint8_t*>(P.x) + m0 * P.k * 2;
+    uint32_t x_off[XC];
     int x_lds[XC];
 #pragma unroll
     for (int i = 0; i < XC; i++) {
         const int c = tid + kThreads * i;
         const int row = c >> 3, kc = c & 7;
-        x_src[i] = P.x + min(m0 + row, P.m - 1) * P.k + kc * 8;
+        x_off[i] = (uint32_t)((min(m0 + row, P.m - 1) - m0) * P.k * 2 + kc * 16);
         x_lds[i] = row * kRowStride + kc * 16;
     }
-    const int64_t w_row = n0 + tid;
-    const bool w_row_ok = (w_row >> 4) < P.row_tiles;
+    // weights: thread t stages row n0 + t; rows past the matrix read the last row-tile
+    // (their output columns are never stored)
+    const int64_t rt0 = n0 >> 4;
+    const int64_t rowtile_bytes = (int64_t)P.k_groups * P.panel_bytes;
+    const uint8_t* w_tile = P.w + rt0 * rowtile_bytes;
+    const uint32_t w_off =
+        (uint32_t)((min(rt0 + (tid >> 4), P.row_tiles - 1) - rt0) * rowtile_bytes) + (uint32_t)(tid & 15) * 16u;
+    const uint32_t slot_bytes = (uint32_t)P.slots * 16u;
     const int w_lds = (BM + tid) * kRowStride;
+    // load cursor: the unit whose chunks are fetched next (clamped to the last unit)
+    int cur_us = u0 < P.k_units ? u0 % P.s : 0;
+    uint32_t cur_kg_off = (uint32_t)((u0 < P.k_units ? u0 / P.s : 0) * P.panel_bytes);
+    int cur_unit = min(u0, P.k_units - 1);
+    auto advance_cursor = [&]() {
+        if (cur_unit + 1 < P.k_units) {
+            cur_unit++;
+            cur_us++;
+            if (cur_us == P.s) cur_us = 0, cur_kg_off += (uint32_t)P.panel_bytes;
+        }
+    };
 
     auto x_load = [&](int kt, int i) {
-        const int64_t gk = (int64_t)kt * BK;
-        // chunks at or past k read chunk 0 of the row; x_write turns them into zeros
-        xr[i] = *reinterpret_cast<const u32x4*>(x_src[i] + (gk + (tid & 7) * 8 < P.k ? gk : -(int64_t)((tid & 7) * 8)));
+        if (XTAIL) {
+            // chunks at or past k read chunk 0 of the row; x_write turns them into zeros
+            const bool ok = (int64_t)kt * BK + (tid & 7) * 8 < P.k;
+            xr[i] = *reinterpret_cast<const u32x4*>(x_tile + (ok ? (int64_t)kt * (BK * 2) : -(int64_t)((tid & 7) * 16)) + x_off[i]);
+        } else {
+            xr[i] = *reinterpret_cast<const u32x4*>(x_tile + (size_t)min(kt, last_step) * (BK * 2) + x_off[i]);
+        }
     };
     auto x_write = [&](int kt, int i, uint8_t* stage) {
-        const bool ok = (int64_t)kt * BK + (tid & 7) * 8 < P.k;
-        *reinterpret_cast<u32x4*>(stage + x_lds[i]) = ok ? xr[i] : u32x4{0, 0, 0, 0};
+        if (XTAIL) {
+            const bool ok = (int64_t)kt * BK + (tid & 7) * 8 < P.k;
+            *reinterpret_cast<u32x4*>(stage + x_lds[i]) = ok ? xr[i] : u32x4{0, 0, 0, 0};
+        } else {
+            *reinterpret_cast<u32x4*>(stage + x_lds[i]) = xr[i];
+        }
     };
-    auto w_base = [&](int kt) -> const u32x4* {
-        const int unit = kt >> 2;
-        const bool ok = w_row_ok && unit < P.k_units;
-        const int u = ok ? unit : 0;
-        const int kg = u / P.s, us = u - kg * P.s;
-        return reinterpret_cast<const u32x4*>(P.w + ((ok ? (w_row >> 4) : 0) * P.k_groups + kg) * P.panel_bytes) +
-               us * 16 + (int)(w_row & 15);
+    auto w_load_hdr = [&]() {
+        wr.hdr = *reinterpret_cast<const u32x4*>(w_tile + (cur_kg_off + (uint32_t)cur_us * 256u) + w_off);
+    };
+    auto w_load_q = [&](int sub, int c) {
+        wr.q[c] = *reinterpret_cast<const u32x4*>(
+            w_tile + (cur_kg_off + (uint32_t)cur_us * 256u + (uint32_t)(1 + sub * NC + c) * slot_bytes) + w_off);
+    };
+    // header of the unit being staged, unpacked once per unit
+    float hd = 0, hdmin = 0;                            // Q4_K: d, dmin
+    uint32_t sc_lo = 0, sc_hi = 0, mn_lo = 0, mn_hi = 0; // Q4_K: 8 scale bytes, 8 min bytes; Q8_0: 8 f16 scales
+    auto w_unpack = [&]() {
+        if (QT == QMM_Q4_K) {
+            hd = qmm_f16_bits_to_f32((uint16_t)(wr.hdr.x & 0xffffu));
+            hdmin = -qmm_f16_bits_to_f32((uint16_t)(wr.hdr.x >> 16));
+            qmm_unpack_q4k_scales(wr.hdr.y, wr.hdr.z, wr.hdr.w, sc_lo, sc_hi, mn_lo, mn_hi);
+        } else {
+            sc_lo = wr.hdr.x, sc_hi = wr.hdr.y, mn_lo = wr.hdr.z, mn_hi = wr.hdr.w;
+        }
     };
     // scales of the tile being staged
     float sa = 0, ba = 0, sb = 0, bb = 0; // Q4_K: (d1, -m1, d2, -m2); Q8_0: (dA, -128 dA, dB, -128 dB)
-    auto w_scales = [&](int kt) {
-        const bool ok = w_row_ok && (kt >> 2) < P.k_units;
+    auto w_scales = [&](auto SUB) {
+        constexpr int g = decltype(SUB)::value;
         if (QT == QMM_Q4_K) {
-            const int g = kt & 3;
-            const float d = ok ? qmm_f16_bits_to_f32((uint16_t)(wr.hdr.x & 0xffffu)) : 0.0f;
-            const float dmin = ok ? qmm_f16_bits_to_f32((uint16_t)(wr.hdr.x >> 16)) : 0.0f;
-            uint32_t sc_lo, sc_hi, mn_lo, mn_hi;
-            qmm_unpack_q4k_scales(wr.hdr.y, wr.hdr.z, wr.hdr.w, sc_lo, sc_hi, mn_lo, mn_hi);
-            sa = d * (float)qmm_byte_of(sc_lo, sc_hi, 2 * g);
-            ba = -(dmin * (float)qmm_byte_of(mn_lo, mn_hi, 2 * g));
-            sb = d * (float)qmm_byte_of(sc_lo, sc_hi, 2 * g + 1);
-            bb = -(dmin * (float)qmm_byte_of(mn_lo, mn_hi, 2 * g + 1));
+            const uint32_t sc = g < 2 ? sc_lo : sc_hi, mn = g < 2 ? mn_lo : mn_hi;
+            sa = hd * ubyte_f32<(2 * g) & 3>(sc);
+            ba = hdmin * ubyte_f32<(2 * g) & 3>(mn);
+            sb = hd * ubyte_f32<(2 * g + 1) & 3>(sc);
+            bb = hdmin * ubyte_f32<(2 * g + 1) & 3>(mn);
         } else {
-            const int b0 = (kt & 3) * 2;
-            const uint32_t hw[4] = {wr.hdr.x, wr.hdr.y, wr.hdr.z, wr.hdr.w};
-            const uint32_t pair = hw[b0 >> 1]; // blocks b0 (low half) and b0 + 1 (high half)
-            sa = ok ? qmm_f16_bits_to_f32((uint16_t)(pair & 0xffffu)) : 0.0f;
-            sb = ok ? qmm_f16_bits_to_f32((uint16_t)(pair >> 16)) : 0.0f;
+            const uint32_t pair = g == 0 ? sc_lo : g == 1 ? sc_hi : g == 2 ? mn_lo : mn_hi; // blocks 2g, 2g + 1
+            sa = qmm_f16_bits_to_f32((uint16_t)(pair & 0xffffu));
+            sb = qmm_f16_bits_to_f32((uint16_t)(pair >> 16));
             ba = -128.0f * sa;
             bb = -128.0f * sb;
         }
@@ -397,7 +448,7 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
         if (QT == QMM_Q4_K) {
             constexpr int c = sidx / 4, j = sidx % 4; // chunk (16-byte half h = c), dword j
             const uint32_t v = wr.q[c][j];
-            const uint32_t vl = v & 0x0f0f0f0fu, vh = (v >> 4) & 0x0f0f0f0fu;
+            const uint32_t vl = opaque(v & 0x0f0f0f0fu), vh = opaque((v >> 4) & 0x0f0f0f0fu);
             constexpr int o = (j & 1) * 2;
             stash[o] = pack_bf16(__builtin_fmaf(sa, ubyte_f32<0>(vl), ba), __builtin_fmaf(sa, ubyte_f32<1>(vl), ba));
             stash[o + 1] = pack_bf16(__builtin_fmaf(sa, ubyte_f32<2>(vl), ba), __builtin_fmaf(sa, ubyte_f32<3>(vl), ba));
@@ -412,35 +463,23 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
             const float d = (c >> 1) ? sb : sa, bias = (c >> 1) ? bb : ba;
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-                const uint32_t u = wr.q[c][jj + t] ^ 0x80808080u;
+                const uint32_t u = opaque(wr.q[c][jj + t] ^ 0x80808080u);
                 stash[2 * t] = pack_bf16(__builtin_fmaf(d, ubyte_f32<0>(u), bias), __builtin_fmaf(d, ubyte_f32<1>(u), bias));
                 stash[2 * t + 1] = pack_bf16(__builtin_fmaf(d, ubyte_f32<2>(u), bias), __builtin_fmaf(d, ubyte_f32<3>(u), bias));
             }
             *reinterpret_cast<uint4*>(row + 32 * c + 16 * (sidx % 2)) = make_uint4(stash[0], stash[1], stash[2], stash[3]);
         }
     };
-    auto w_load_hdr = [&](int kt) { wr.hdr = w_base(kt)[0]; };
-    auto w_load_q = [&](int kt, int c) { wr.q[c] = w_base(kt)[(size_t)(1 + (kt & 3) * NC + c) * P.slots]; };
 
-    // ---- prologue: tile 0 -> stage 0, tile 1 -> registers
-#pragma unroll
-    for (int i = 0; i < XC; i++) x_load(kt0, i);
-    w_load_hdr(kt0);
-#pragma unroll
-    for (int c = 0; c < NC; c++) w_load_q(kt0, c);
-#pragma unroll
-    for (int i = 0; i < XC; i++) x_write(kt0, i, smem);
-    w_scales(kt0);
-    static_for<8>([&](auto S) { w_slice(S, smem); });
-#pragma unroll
-    for (int i = 0; i < XC; i++) x_load(kt0 + 1, i);
-    w_load_hdr(kt0 + 1);
-#pragma unroll
-    for (int c = 0; c < NC; c++) w_load_q(kt0 + 1, c);
-    __syncthreads();
-
-    auto k_step = [&](int kt, const uint8_t* cur, uint8_t* next, auto feed) {
-        constexpr bool FEED = decltype(feed)::value;
+    // One k step: MFMAs out of stage SUB & 1; between them tile kt+1 goes from registers to the
+    // other stage and tile kt+2 is fetched.  Steps past the workgroup's last one stage and fetch
+    // the (clamped) last tile again: nobody reads it.
+    auto k_step = [&](int unit, auto SUB) {
+        constexpr int sub = decltype(SUB)::value;
+        constexpr int nsub = (sub + 1) & 3, lsub = (sub + 2) & 3; // sub-block staged / fetched meanwhile
+        const int kt = unit * 4 + sub;
+        const uint8_t* cur = smem + (sub & 1) * kStage;
+        uint8_t* next = smem + ((sub + 1) & 1) * kStage;
         const uint8_t* xs = cur + (wm * (BM / 2) + (lane & 31)) * kRowStride + (lane >> 5) * 16;
         const uint8_t* ws = cur + (BM + wn * (BN / 2) + (lane & 31)) * kRowStride + (lane >> 5) * 16;
         bf16x8 fa[2][MT], fb[2][NT];
@@ -464,32 +503,39 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
                     const int t = gi * 4 + q, i = t / NT, j = t % NT;
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kk & 1][i], fb[kk & 1][j], acc[i][j], 0, 0, 0);
                 }
-                if (FEED) {
-                    // group g's share of staging tile kt+1 and fetching tile kt+2
-                    constexpr int s0 = NG == 16 ? 1 : 0; // first group that runs a weight slice
-                    if (g == 0) w_scales(kt + 1);
-                    if (g < XC) x_write(kt + 1, g, next);
-                    if (g >= s0 && g < s0 + 8) w_slice(std::integral_constant<int, (g >= s0 && g < s0 + 8) ? g - s0 : 0>{}, next);
-                    if (g >= 2 && g < 2 + XC) x_load(kt + 2, g - 2);
-                    if (NG == 16) {
-                        if (g == 10) w_load_hdr(kt + 2);
-                        if (g >= 11 && g < 11 + NC) w_load_q(kt + 2, g - 11);
-                    } else if (g == NG - 1) {
-                        w_load_hdr(kt + 2);
-#pragma unroll
-                        for (int c = 0; c < NC; c++) w_load_q(kt + 2, c);
+                // group g's share of staging tile kt+1 and fetching tile kt+2
+                constexpr int s0 = NG == 16 ? 1 : 0; // first group that runs a weight slice
+                if (g == 0) {
+                    if (sub == 3) w_unpack(); // tile kt+1 opens the next unit: its header arrived a step ago
+                    w_scales(std::integral_constant<int, nsub>{});
+                }
+                if (g < XC) x_write(kt + 1, g, next);
+                if (g >= s0 && g < s0 + 8) w_slice(std::integral_constant<int, (g >= s0 && g < s0 + 8) ? g - s0 : 0>{}, next);
+                if (g >= 2 && g < 2 + XC) x_load(kt + 2, g - 2);
+                if (NG == 16) {
+                    if (g == 10 && sub == 2) {
+                        advance_cursor();
+                        w_load_hdr();
                     }
-                    if (BM == 256) {
-                        // inside the group: one MFMA, then a few of the slice's VALU ops, so the
-                        // matrix pipe is fed while the slice issues
+                    if (g >= 11 && g < 11 + NC) w_load_q(lsub, g - 11);
+                } else if (g == NG - 1) {
+                    if (sub == 2) {
+                        advance_cursor();
+                        w_load_hdr();
+                    }
 #pragma unroll
-                        for (int q = 0; q < 4; q++) {
-                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                            __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
-                            if (q == 1) __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
-                            if (q == 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-                            if (q == 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                        }
+                    for (int c = 0; c < NC; c++) w_load_q(lsub, c);
+                }
+                if (BM == 256) {
+                    // inside the group: one MFMA, then a few of the slice's VALU ops, so the
+                    // matrix pipe is fed while the slice issues
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, QMM_GEMM_VALU_PER_MFMA, 0);
+                        if (q == 1) __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
+                        if (q == 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                        if (q == 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -497,9 +543,27 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
         });
         __syncthreads();
     };
-    for (int kt = kt0; kt + 1 < kt1; kt++)
-        k_step(kt, smem + ((kt - kt0) & 1) * kStage, smem + ((kt - kt0 + 1) & 1) * kStage, std::true_type{});
-    k_step(kt1 - 1, smem + ((kt1 - 1 - kt0) & 1) * kStage, nullptr, std::false_type{});
+
+    if (u0 < u1) {
+        // ---- prologue: tile (u0, 0) -> stage 0, tile (u0, 1) -> registers
+#pragma unroll
+        for (int i = 0; i < XC; i++) x_load(u0 * 4, i);
+        w_load_hdr();
+#pragma unroll
+        for (int c = 0; c < NC; c++) w_load_q(0, c);
+#pragma unroll
+        for (int i = 0; i < XC; i++) x_write(u0 * 4, i, smem);
+        w_unpack();
+        w_scales(std::integral_constant<int, 0>{});
+        static_for<8>([&](auto S) { w_slice(S, smem); });
+#pragma unroll
+        for (int i = 0; i < XC; i++) x_load(u0 * 4 + 1, i);
+#pragma unroll
+        for (int c = 0; c < NC; c++) w_load_q(1, c);
+        __syncthreads();
+
+        for (int unit = u0; unit < u1; unit++) static_for<4>([&](auto SUB) { k_step(unit, SUB); });
+    }
 
     // a split-k slice stores f32 into its own [m, n] plane of the workspace
     float* out_f32 = P.partial ? P.partial + (int64_t)blockIdx.y * P.m * P.n : reinterpret_cast<float*>(P.y);
@@ -558,8 +622,11 @@ hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
     const int64_t grid = (int64_t)P.tiles_m * P.tiles_n;
     if (grid > 0x7fffffff) return hipErrorInvalidValue;
     const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
+    const bool x_tail = (P.k & 63) != 0;
     const void* fn;
-    if constexpr (BN == 256) fn = reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM>);
+    if constexpr (BN == 256)
+        fn = x_tail ? reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, true>)
+                    : reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, false>);
     else fn = reinterpret_cast<const void*>(&gemm_kernel<QT, BM, BN>);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -567,13 +634,11 @@ hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
     }
     if constexpr (BN == 256) {
         float* partial = P.partial;
-        if (slices > 1) {
-            const int k_steps = P.k_units * 4;
-            P.slice_steps = (k_steps + slices - 1) / slices;
-        } else {
-            P.partial = nullptr;
-        }
-        gemm_pipe_kernel<QT, BM><<<dim3((unsigned)grid, (unsigned)slices), dim3(kThreads), lds, stream>>>(P);
+        if (slices > 1) P.slice_units = (P.k_units + slices - 1) / slices;
+        else P.partial = nullptr;
+        const dim3 grid2((unsigned)grid, (unsigned)slices);
+        if (x_tail) gemm_pipe_kernel<QT, BM, true><<<grid2, dim3(kThreads), lds, stream>>>(P);
+        else gemm_pipe_kernel<QT, BM, false><<<grid2, dim3(kThreads), lds, stream>>>(P);
         if (slices > 1) {
             const int64_t count = P.m * (P.n_end - P.n_begin);
             splitk_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(
@@ -619,7 +684,7 @@ GemmPlan plan_gemm(int64_t m, int64_t n, int k_steps, int n_cus) {
     for (int slices = 2; slices <= 8; slices *= 2) {
         if (k_steps / slices < 8) break;
         const double reduce_cost = 2.0 * slices * (double)m * (double)n * 4.0 / 4e12 * 1e6 / 1.5 + 2.0;
-        const double steps = (double)((k_steps + slices - 1) / slices);
+        const double steps = 4.0 * (double)((k_steps / 4 + slices - 1) / slices); // slices are whole units
         consider({256, 256, slices, 0}, rounds(tiles(256, 256, n) * slices) * steps + reduce_cost);
         consider({128, 256, slices, 0}, rounds(tiles(128, 256, n) * slices) * steps * 0.5 / kQ128 + reduce_cost);
     }
@@ -675,7 +740,7 @@ hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uin
     P.panel_bytes = L.panel_bytes;
     P.out_bf16 = out_bf16;
     P.tiles_m = P.tiles_n = 0;
-    P.slice_steps = 0;
+    P.slice_units = 0;
     P.partial = (float*)workspace;
     return L.dtype == QMM_Q4_K ? launch_qt<QMM_Q4_K>(P, n_cus, stream)
                                : launch_qt<QMM_Q8_0>(P, n_cus, stream);
