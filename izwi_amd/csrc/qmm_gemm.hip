@@ -17,6 +17,8 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 
 #include <type_traits>
 #include <utility>
@@ -33,7 +35,7 @@ constexpr int BK = 64;
 constexpr int kThreads = 256;
 constexpr int kRowStride = 144; // bytes per LDS tile row: 64 bf16 + 16 B pad
 #ifndef QMM_GEMM_VALU_PER_MFMA
-#define QMM_GEMM_VALU_PER_MFMA 5
+#define QMM_GEMM_VALU_PER_MFMA 4
 #endif
 
 struct GemmParams {
@@ -50,6 +52,10 @@ struct GemmParams {
     // k-elements and writes its f32 tile to partial[s][m][n]; a second kernel adds the slices
     // in order
     int slice_units;
+    // 0x0f0f0f0f, passed as data: with the constant in the code the compiler folds mask and
+    // byte select into one bit-field extract per weight, followed by a convert; with an unknown
+    // mask it emits one AND per four weights and v_cvt_f32_ubyteN for each
+    uint32_t nibble_mask;
     float* partial;
 };
 
@@ -308,14 +314,6 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_impl<N>(f, std::make_integer_sequence<int, N>{});
 }
 
-// Keeps the compiler from folding a later shift-and-mask of v into one bit-field extract
-// of the original word: the bytes of v are then converted with v_cvt_f32_ubyteN (one
-// instruction per weight instead of two).
-__device__ __forceinline__ uint32_t opaque(uint32_t v) {
-    asm("" : "+v"(v));
-    return v;
-}
-
 // Pipelined 256-column tile.  The k loop runs over units of 256 k-elements with the four
 // 64-wide steps of a unit unrolled, so that the sub-block index, the LDS stage and the
 // chunk offsets inside the panel are compile-time constants; whatever depends on the
@@ -323,12 +321,14 @@ __device__ __forceinline__ uint32_t opaque(uint32_t v) {
 // stays in scalar registers, the per-lane part of every address is a 32-bit offset
 // computed once.  XTAIL: k is not a multiple of 64 (Q8_0 only), activation chunks at or
 // past k are zeroed on their way to LDS.
-template <int QT, int BM, bool XTAIL>
+template <int QT, int BM, int BN, bool XTAIL>
 __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
-    constexpr int BN = 256;
     constexpr int MT = BM / 64, NT = BN / 64;
     constexpr int XC = BM / 32;
-    constexpr int NC = QT == QMM_Q4_K ? 2 : 4;
+    constexpr int TPR = kThreads / BN;                   // threads that share a weight row: 1 or 2
+    constexpr int NCR = QT == QMM_Q4_K ? 2 : 4;          // quant chunks per row and k step
+    constexpr int NC = NCR / TPR;                        // ... per thread
+    constexpr int NP = 16 / TPR;                         // pieces of four weights per thread and k step
     constexpr int GPK = MT * NT / 4; // groups of four MFMAs per k16 step
     constexpr int NG = 4 * GPK;      // groups per k step: 16 (BM = 256) or 8 (BM = 128)
     constexpr int kStage = (BM + BN) * kRowStride;
@@ -352,8 +352,13 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
     // ---- staging state: tile kt+1 sits in xr / wr while step kt runs
-    u32x4 xr[XC];
-    WRegs<QT, 1> wr;
+    // activation chunks in flight: tile kt+1 (written to LDS during step kt) and, where the
+    // register file allows, tile kt+2 behind it, so that a chunk is requested XD k steps
+    // before it is needed
+    constexpr int XD = BN == 128 ? 2 : 1;
+    u32x4 xr[XD][XC];
+    u32x4 w_hdr;      // header of the unit fetched last
+    u32x4 wq[2][NC];  // quant chunks of tile kt+1 (being dequantized) and tile kt+2 (in flight), by parity
     // activations: uniform tile base + uniform column + per-lane (row, chunk) offset
     const uint8_t* x_tile = reinterpret_cast<const uint8_t*>(P.x) + m0 * P.k * 2;
     uint32_t x_off[XC];
@@ -365,15 +370,18 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
         x_off[i] = (uint32_t)((min(m0 + row, P.m - 1) - m0) * P.k * 2 + kc * 16);
         x_lds[i] = row * kRowStride + kc * 16;
     }
-    // weights: thread t stages row n0 + t; rows past the matrix read the last row-tile
-    // (their output columns are never stored)
+    // weights: thread t stages part t % TPR of row n0 + t / TPR; rows past the matrix read the
+    // last row-tile (their output columns are never stored)
+    const int w_row = tid / TPR, w_part = tid % TPR;
     const int64_t rt0 = n0 >> 4;
     const int64_t rowtile_bytes = (int64_t)P.k_groups * P.panel_bytes;
     const uint8_t* w_tile = P.w + rt0 * rowtile_bytes;
-    const uint32_t w_off =
-        (uint32_t)((min(rt0 + (tid >> 4), P.row_tiles - 1) - rt0) * rowtile_bytes) + (uint32_t)(tid & 15) * 16u;
     const uint32_t slot_bytes = (uint32_t)P.slots * 16u;
-    const int w_lds = (BM + tid) * kRowStride;
+    const uint32_t w_off =
+        (uint32_t)((min(rt0 + (w_row >> 4), P.row_tiles - 1) - rt0) * rowtile_bytes) + (uint32_t)(w_row & 15) * 16u;
+    const uint32_t w_off_q = w_off + (uint32_t)(w_part * NC) * slot_bytes; // this thread's first chunk of a step
+    // Q4_K: part p holds nibble bytes 16p .. 16p+15 of the step; Q8_0: int8 32p .. 32p+31
+    const int w_lds = (BM + w_row) * kRowStride + w_part * (QT == QMM_Q4_K ? 32 : 64);
     // load cursor: the unit whose chunks are fetched next (clamped to the last unit)
     int cur_us = u0 < P.k_units ? u0 % P.s : 0;
     uint32_t cur_kg_off = (uint32_t)((u0 < P.k_units ? u0 / P.s : 0) * P.panel_bytes);
@@ -386,44 +394,45 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
         }
     };
 
-    auto x_load = [&](int kt, int i) {
+    auto x_load = [&](int kt, int buf, int i) {
         if (XTAIL) {
             // chunks at or past k read chunk 0 of the row; x_write turns them into zeros
             const bool ok = (int64_t)kt * BK + (tid & 7) * 8 < P.k;
-            xr[i] = *reinterpret_cast<const u32x4*>(x_tile + (ok ? (int64_t)kt * (BK * 2) : -(int64_t)((tid & 7) * 16)) + x_off[i]);
+            xr[buf][i] = *reinterpret_cast<const u32x4*>(x_tile + (ok ? (int64_t)kt * (BK * 2) : -(int64_t)((tid & 7) * 16)) + x_off[i]);
         } else {
-            xr[i] = *reinterpret_cast<const u32x4*>(x_tile + (size_t)min(kt, last_step) * (BK * 2) + x_off[i]);
+            xr[buf][i] = *reinterpret_cast<const u32x4*>(x_tile + (size_t)min(kt, last_step) * (BK * 2) + x_off[i]);
         }
     };
-    auto x_write = [&](int kt, int i, uint8_t* stage) {
+    auto x_write = [&](int kt, int buf, int i, uint8_t* stage) {
         if (XTAIL) {
             const bool ok = (int64_t)kt * BK + (tid & 7) * 8 < P.k;
-            *reinterpret_cast<u32x4*>(stage + x_lds[i]) = ok ? xr[i] : u32x4{0, 0, 0, 0};
+            *reinterpret_cast<u32x4*>(stage + x_lds[i]) = ok ? xr[buf][i] : u32x4{0, 0, 0, 0};
         } else {
-            *reinterpret_cast<u32x4*>(stage + x_lds[i]) = xr[i];
+            *reinterpret_cast<u32x4*>(stage + x_lds[i]) = xr[buf][i];
         }
     };
     auto w_load_hdr = [&]() {
-        wr.hdr = *reinterpret_cast<const u32x4*>(w_tile + (cur_kg_off + (uint32_t)cur_us * 256u) + w_off);
+        w_hdr = *reinterpret_cast<const u32x4*>(w_tile + (cur_kg_off + (uint32_t)cur_us * 256u) + w_off);
     };
     auto w_load_q = [&](int sub, int c) {
-        wr.q[c] = *reinterpret_cast<const u32x4*>(
-            w_tile + (cur_kg_off + (uint32_t)cur_us * 256u + (uint32_t)(1 + sub * NC + c) * slot_bytes) + w_off);
+        wq[sub & 1][c] = *reinterpret_cast<const u32x4*>(
+            w_tile + (cur_kg_off + (uint32_t)cur_us * 256u + (uint32_t)(1 + sub * NCR + c) * slot_bytes) + w_off_q);
     };
     // header of the unit being staged, unpacked once per unit
     float hd = 0, hdmin = 0;                            // Q4_K: d, dmin
     uint32_t sc_lo = 0, sc_hi = 0, mn_lo = 0, mn_hi = 0; // Q4_K: 8 scale bytes, 8 min bytes; Q8_0: 8 f16 scales
     auto w_unpack = [&]() {
         if (QT == QMM_Q4_K) {
-            hd = qmm_f16_bits_to_f32((uint16_t)(wr.hdr.x & 0xffffu));
-            hdmin = -qmm_f16_bits_to_f32((uint16_t)(wr.hdr.x >> 16));
-            qmm_unpack_q4k_scales(wr.hdr.y, wr.hdr.z, wr.hdr.w, sc_lo, sc_hi, mn_lo, mn_hi);
+            hd = qmm_f16_bits_to_f32((uint16_t)(w_hdr.x & 0xffffu));
+            hdmin = -qmm_f16_bits_to_f32((uint16_t)(w_hdr.x >> 16));
+            qmm_unpack_q4k_scales(w_hdr.y, w_hdr.z, w_hdr.w, sc_lo, sc_hi, mn_lo, mn_hi);
         } else {
-            sc_lo = wr.hdr.x, sc_hi = wr.hdr.y, mn_lo = wr.hdr.z, mn_hi = wr.hdr.w;
+            sc_lo = w_hdr.x, sc_hi = w_hdr.y, mn_lo = w_hdr.z, mn_hi = w_hdr.w;
         }
     };
     // scales of the tile being staged
     float sa = 0, ba = 0, sb = 0, bb = 0; // Q4_K: (d1, -m1, d2, -m2); Q8_0: (dA, -128 dA, dB, -128 dB)
+    float sw = 0, bw = 0;                 // Q8_0, two threads per row: the scale of this thread's block
     auto w_scales = [&](auto SUB) {
         constexpr int g = decltype(SUB)::value;
         if (QT == QMM_Q4_K) {
@@ -438,129 +447,154 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
             sb = qmm_f16_bits_to_f32((uint16_t)(pair >> 16));
             ba = -128.0f * sa;
             bb = -128.0f * sb;
+            sw = w_part ? sb : sa;
+            bw = -128.0f * sw;
         }
     };
-    uint32_t stash[8]; // finished bf16 pairs waiting for their 16-byte LDS write
-    // slice S of 8: one eighth of the thread's 64 weights, converted and (every other slice) written
-    auto w_slice = [&](auto S, uint8_t* stage) {
-        constexpr int sidx = decltype(S)::value;
+    const uint32_t nibble_mask = P.nibble_mask;
+    uint32_t stash[4]; // finished bf16 pairs waiting for their 16-byte LDS write
+    // piece H of NP of the tile with sub-block parity PAR: four of the thread's weights (Q4_K: the
+    // low or the high nibbles of one dword; Q8_0: one dword), converted and, every other piece,
+    // written as 16 bytes
+    auto w_piece = [&](auto PAR, auto HH, uint8_t* stage) {
+        constexpr int par = decltype(PAR)::value, h = decltype(HH)::value;
         uint8_t* row = stage + w_lds;
-        if (QT == QMM_Q4_K) {
-            constexpr int c = sidx / 4, j = sidx % 4; // chunk (16-byte half h = c), dword j
-            const uint32_t v = wr.q[c][j];
-            const uint32_t vl = opaque(v & 0x0f0f0f0fu), vh = opaque((v >> 4) & 0x0f0f0f0fu);
-            constexpr int o = (j & 1) * 2;
-            stash[o] = pack_bf16(__builtin_fmaf(sa, ubyte_f32<0>(vl), ba), __builtin_fmaf(sa, ubyte_f32<1>(vl), ba));
-            stash[o + 1] = pack_bf16(__builtin_fmaf(sa, ubyte_f32<2>(vl), ba), __builtin_fmaf(sa, ubyte_f32<3>(vl), ba));
-            stash[4 + o] = pack_bf16(__builtin_fmaf(sb, ubyte_f32<0>(vh), bb), __builtin_fmaf(sb, ubyte_f32<1>(vh), bb));
-            stash[4 + o + 1] = pack_bf16(__builtin_fmaf(sb, ubyte_f32<2>(vh), bb), __builtin_fmaf(sb, ubyte_f32<3>(vh), bb));
-            if (j & 1) { // low nibbles: k 16c + 8 (j/2) .., high nibbles: k 32 + 16c + 8 (j/2) ..
-                *reinterpret_cast<uint4*>(row + 32 * c + 16 * (j >> 1)) = make_uint4(stash[0], stash[1], stash[2], stash[3]);
-                *reinterpret_cast<uint4*>(row + 64 + 32 * c + 16 * (j >> 1)) = make_uint4(stash[4], stash[5], stash[6], stash[7]);
-            }
+        if constexpr (QT == QMM_Q4_K) {
+            // dwords (c, j) and (c, j + 1) of a chunk, low nibbles of both, then high nibbles of both
+            constexpr int c = h / 8, jp = (h % 8) / 4, hi = (h % 4) / 2, j = 2 * jp + (h % 2);
+            const uint32_t v = wq[par][c][j];
+            const uint32_t q4 = (hi ? v >> 4 : v) & nibble_mask;
+            const float sc = hi ? sb : sa, bi = hi ? bb : ba;
+            constexpr int o = (h % 2) * 2;
+            stash[o] = pack_bf16(__builtin_fmaf(sc, ubyte_f32<0>(q4), bi), __builtin_fmaf(sc, ubyte_f32<1>(q4), bi));
+            stash[o + 1] = pack_bf16(__builtin_fmaf(sc, ubyte_f32<2>(q4), bi), __builtin_fmaf(sc, ubyte_f32<3>(q4), bi));
+            if (h % 2) // low nibbles: k 16c + 8 jp .., high nibbles: k 32 + 16c + 8 jp ..
+                *reinterpret_cast<uint4*>(row + 64 * hi + 32 * c + 16 * jp) = make_uint4(stash[0], stash[1], stash[2], stash[3]);
         } else {
-            constexpr int c = sidx / 2, jj = (sidx % 2) * 2; // chunk c: block c / 2, dwords jj, jj + 1
-            const float d = (c >> 1) ? sb : sa, bias = (c >> 1) ? bb : ba;
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-                const uint32_t u = opaque(wr.q[c][jj + t] ^ 0x80808080u);
-                stash[2 * t] = pack_bf16(__builtin_fmaf(d, ubyte_f32<0>(u), bias), __builtin_fmaf(d, ubyte_f32<1>(u), bias));
-                stash[2 * t + 1] = pack_bf16(__builtin_fmaf(d, ubyte_f32<2>(u), bias), __builtin_fmaf(d, ubyte_f32<3>(u), bias));
-            }
-            *reinterpret_cast<uint4*>(row + 32 * c + 16 * (sidx % 2)) = make_uint4(stash[0], stash[1], stash[2], stash[3]);
+            constexpr int c = h / 4, j = h % 4; // the thread's chunk c: block (part * NC + c) / 2 of the step
+            float d, bias;
+            if (TPR == 1) d = (c >> 1) ? sb : sa, bias = (c >> 1) ? bb : ba;
+            else d = sw, bias = bw;
+            const uint32_t u = wq[par][c][j] ^ 0x80808080u;
+            constexpr int o = (j % 2) * 2;
+            stash[o] = pack_bf16(__builtin_fmaf(d, ubyte_f32<0>(u), bias), __builtin_fmaf(d, ubyte_f32<1>(u), bias));
+            stash[o + 1] = pack_bf16(__builtin_fmaf(d, ubyte_f32<2>(u), bias), __builtin_fmaf(d, ubyte_f32<3>(u), bias));
+            if (j % 2) *reinterpret_cast<uint4*>(row + 32 * c + 16 * (j / 2)) = make_uint4(stash[0], stash[1], stash[2], stash[3]);
         }
     };
 
+    // Operand fragments of one k16 step, two sets: the MFMAs of step kk read set kk & 1 while
+    // the other set is filled.  A group of four MFMAs uses one row fragment and all column
+    // fragments, so the column fragments are fetched first.
+    bf16x8 fa[2][MT], fb[2][NT];
+    const int frag_x = (wm * (BM / 2) + (lane & 31)) * kRowStride + (lane >> 5) * 16;
+    const int frag_w = (BM + wn * (BN / 2) + (lane & 31)) * kRowStride + (lane >> 5) * 16;
+    // part gi of GPK: read while group gi runs, used from group gi of the next k16 step on
+    auto read_frags = [&](const uint8_t* stage, int kk, int set, auto PART) {
+        constexpr int part = decltype(PART)::value;
+        constexpr int jb = NT == 4 ? (part < GPK / 2 ? part * 2 * NT / GPK : NT) : (part == 0 ? 0 : NT);
+        constexpr int je = NT == 4 ? (part < GPK / 2 ? (part + 1) * 2 * NT / GPK : NT) : NT;
+        constexpr int ib = NT == 4 ? (part < GPK / 2 ? 0 : (part - GPK / 2) * 2 * MT / GPK) : (part == 0 ? 0 : MT / 2);
+        constexpr int ie = NT == 4 ? (part < GPK / 2 ? 0 : (part - GPK / 2 + 1) * 2 * MT / GPK) : (part == 0 ? MT / 2 : MT);
+#pragma unroll
+        for (int j = jb; j < je; j++)
+            fb[set][j] = *reinterpret_cast<const bf16x8*>(stage + frag_w + j * 32 * kRowStride + kk * 32);
+#pragma unroll
+        for (int i = ib; i < ie; i++)
+            fa[set][i] = *reinterpret_cast<const bf16x8*>(stage + frag_x + i * 32 * kRowStride + kk * 32);
+    };
+
     // One k step: MFMAs out of stage SUB & 1; between them tile kt+1 goes from registers to the
-    // other stage and tile kt+2 is fetched.  Steps past the workgroup's last one stage and fetch
-    // the (clamped) last tile again: nobody reads it.
+    // other stage (first three quarters of the step), tile kt+2 is fetched, and after the
+    // step's only barrier, which follows the last fragment reads of this stage and the last
+    // writes to the other one, the first fragments of step kt+1 are read while the last quarter
+    // of the MFMAs runs.  Steps past the workgroup's last one stage and fetch the (clamped) last
+    // tile again: nobody uses it.
     auto k_step = [&](int unit, auto SUB) {
         constexpr int sub = decltype(SUB)::value;
         constexpr int nsub = (sub + 1) & 3, lsub = (sub + 2) & 3; // sub-block staged / fetched meanwhile
         const int kt = unit * 4 + sub;
         const uint8_t* cur = smem + (sub & 1) * kStage;
         uint8_t* next = smem + ((sub + 1) & 1) * kStage;
-        const uint8_t* xs = cur + (wm * (BM / 2) + (lane & 31)) * kRowStride + (lane >> 5) * 16;
-        const uint8_t* ws = cur + (BM + wn * (BN / 2) + (lane & 31)) * kRowStride + (lane >> 5) * 16;
-        bf16x8 fa[2][MT], fb[2][NT];
-        auto read_frags = [&](int kk, int set) {
-#pragma unroll
-            for (int i = 0; i < MT; i++)
-                fa[set][i] = *reinterpret_cast<const bf16x8*>(xs + i * 32 * kRowStride + kk * 32);
-#pragma unroll
-            for (int j = 0; j < NT; j++)
-                fb[set][j] = *reinterpret_cast<const bf16x8*>(ws + j * 32 * kRowStride + kk * 32);
-        };
-        read_frags(0, 0);
         static_for<4>([&](auto KK) {
             constexpr int kk = decltype(KK)::value;
-            if (kk < 3) read_frags(kk + 1, (kk + 1) & 1);
             static_for<GPK>([&](auto GI) {
                 constexpr int gi = decltype(GI)::value;
                 constexpr int g = kk * GPK + gi;
+                // the operands of the next k16 step (of the next k step in the last quarter)
+                read_frags(kk < 3 ? cur : next, (kk + 1) & 3, (kk + 1) & 1, GI);
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     const int t = gi * 4 + q, i = t / NT, j = t % NT;
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kk & 1][i], fb[kk & 1][j], acc[i][j], 0, 0, 0);
                 }
-                // group g's share of staging tile kt+1 and fetching tile kt+2
-                constexpr int s0 = NG == 16 ? 1 : 0; // first group that runs a weight slice
+                // group g's share of staging tile kt+1 (the thread's NP weight pieces and XC
+                // activation chunks over the first 3 NG / 4 groups) and of fetching tile kt+2
+                constexpr int NGS = 3 * NG / 4;
+                constexpr int p0 = (NP * g + NGS - 1) / NGS, p1 = g < NGS ? (NP * (g + 1) + NGS - 1) / NGS : p0;
+                constexpr int c0 = (XC * g + NGS - 1) / NGS, c1 = g < NGS ? (XC * (g + 1) + NGS - 1) / NGS : c0;
+                constexpr int l0 = g == 0 ? 0 : (XC * (g - 1) + NGS - 1) / NGS, l1 = g == 0 ? 0 : c0; // chunks written a group ago
                 if (g == 0) {
                     if (sub == 3) w_unpack(); // tile kt+1 opens the next unit: its header arrived a step ago
                     w_scales(std::integral_constant<int, nsub>{});
                 }
-                if (g < XC) x_write(kt + 1, g, next);
-                if (g >= s0 && g < s0 + 8) w_slice(std::integral_constant<int, (g >= s0 && g < s0 + 8) ? g - s0 : 0>{}, next);
-                if (g >= 2 && g < 2 + XC) x_load(kt + 2, g - 2);
-                if (NG == 16) {
-                    if (g == 10 && sub == 2) {
-                        advance_cursor();
-                        w_load_hdr();
-                    }
-                    if (g >= 11 && g < 11 + NC) w_load_q(lsub, g - 11);
-                } else if (g == NG - 1) {
-                    if (sub == 2) {
-                        advance_cursor();
-                        w_load_hdr();
-                    }
+                static_for<p1 - p0>([&](auto PI) {
+                    w_piece(std::integral_constant<int, nsub & 1>{},
+                            std::integral_constant<int, (p0 + decltype(PI)::value) % NP>{}, next);
+                });
+                constexpr int xbuf = (sub + 1) % XD; // registers of tile kt+1, refilled with tile kt+1+XD
 #pragma unroll
-                    for (int c = 0; c < NC; c++) w_load_q(lsub, c);
+                for (int i = c0; i < c1; i++) x_write(kt + 1, xbuf, i, next);
+#pragma unroll
+                for (int i = l0; i < (g <= NGS ? l1 : l0); i++) x_load(kt + 1 + XD, xbuf, i);
+                if (g == 1 && sub == 2) {
+                    advance_cursor();
+                    w_load_hdr();
                 }
-                if (BM == 256) {
-                    // inside the group: one MFMA, then a few of the slice's VALU ops, so the
-                    // matrix pipe is fed while the slice issues
+                if (g >= 2 && g < 2 + NC) w_load_q(lsub, g - 2);
+                // inside the group: one MFMA, then its share of the other instructions, so
+                // the matrix pipe is fed while they issue
+                constexpr int valu = 3 * (p1 - p0) + (g == 0 ? 4 : 1);
+                constexpr int reads = NT == 4 ? (gi < GPK / 2 ? 2 * NT / GPK : 2 * MT / GPK) : (gi == 0 ? NT + MT / 2 : MT / 2);
 #pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x002, QMM_GEMM_VALU_PER_MFMA, 0);
-                        if (q == 1) __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
-                        if (q == 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-                        if (q == 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                    }
+                for (int q = 0; q < 4; q++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, valu, 0);
+                    if (q == 0) __builtin_amdgcn_sched_group_barrier(0x100, (reads + 1) / 2, 0);
+                    if (q == 1) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+                    if (q == 2) __builtin_amdgcn_sched_group_barrier(0x100, reads / 2, 0);
+                    if (q == 3) __builtin_amdgcn_sched_group_barrier(0x200, 3, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
+            if (kk == 2) {
+                // this stage's fragments are all in registers, the other stage is complete
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+            }
         });
-        __syncthreads();
     };
 
     if (u0 < u1) {
         // ---- prologue: tile (u0, 0) -> stage 0, tile (u0, 1) -> registers
 #pragma unroll
-        for (int i = 0; i < XC; i++) x_load(u0 * 4, i);
+        for (int i = 0; i < XC; i++) x_load(u0 * 4, 0, i);
         w_load_hdr();
 #pragma unroll
         for (int c = 0; c < NC; c++) w_load_q(0, c);
 #pragma unroll
-        for (int i = 0; i < XC; i++) x_write(u0 * 4, i, smem);
+        for (int i = 0; i < XC; i++) x_write(u0 * 4, 0, i, smem);
         w_unpack();
         w_scales(std::integral_constant<int, 0>{});
-        static_for<8>([&](auto S) { w_slice(S, smem); });
+        static_for<NP>([&](auto HH) { w_piece(std::integral_constant<int, 0>{}, HH, smem); });
 #pragma unroll
-        for (int i = 0; i < XC; i++) x_load(u0 * 4 + 1, i);
+        for (int d = 1; d <= XD; d++)
+#pragma unroll
+            for (int i = 0; i < XC; i++) x_load(u0 * 4 + d, d % XD, i);
 #pragma unroll
         for (int c = 0; c < NC; c++) w_load_q(1, c);
         __syncthreads();
+        static_for<GPK>([&](auto PART) { read_frags(smem, 0, 0, PART); });
 
         for (int unit = u0; unit < u1; unit++) static_for<4>([&](auto SUB) { k_step(unit, SUB); });
     }
@@ -623,22 +657,23 @@ hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
     if (grid > 0x7fffffff) return hipErrorInvalidValue;
     const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
     const bool x_tail = (P.k & 63) != 0;
+    constexpr bool kPipe = BM == 256 || BN == 256;
     const void* fn;
-    if constexpr (BN == 256)
-        fn = x_tail ? reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, true>)
-                    : reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, false>);
+    if constexpr (kPipe)
+        fn = x_tail ? reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, BN, true>)
+                    : reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, BN, false>);
     else fn = reinterpret_cast<const void*>(&gemm_kernel<QT, BM, BN>);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
     }
-    if constexpr (BN == 256) {
+    if constexpr (kPipe) {
         float* partial = P.partial;
         if (slices > 1) P.slice_units = (P.k_units + slices - 1) / slices;
         else P.partial = nullptr;
         const dim3 grid2((unsigned)grid, (unsigned)slices);
-        if (x_tail) gemm_pipe_kernel<QT, BM, true><<<grid2, dim3(kThreads), lds, stream>>>(P);
-        else gemm_pipe_kernel<QT, BM, false><<<grid2, dim3(kThreads), lds, stream>>>(P);
+        if (x_tail) gemm_pipe_kernel<QT, BM, BN, true><<<grid2, dim3(kThreads), lds, stream>>>(P);
+        else gemm_pipe_kernel<QT, BM, BN, false><<<grid2, dim3(kThreads), lds, stream>>>(P);
         if (slices > 1) {
             const int64_t count = P.m * (P.n_end - P.n_begin);
             splitk_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(
@@ -661,8 +696,35 @@ struct GemmPlan {
     int64_t full_cols;   // > 0: first a launch of 256 x 256 tiles over this many 256-column strips
 };
 
+// IZWI_QMM_GEMM_TILE="bm,bn,slices" (tuning aid) replaces the plan: bm, bn in {128, 256}.
+bool forced_plan(GemmPlan& plan) {
+    static const GemmPlan forced = [] {
+        GemmPlan p{0, 0, 1, 0};
+        const char* e = getenv("IZWI_QMM_GEMM_TILE");
+        if (e && sscanf(e, "%d,%d,%d", &p.bm, &p.bn, &p.slices) >= 2) {
+            const bool ok = (p.bm == 128 || p.bm == 256) && (p.bn == 128 || p.bn == 256) && p.slices >= 1 && p.slices <= 8;
+            if (!ok || (p.bm == 128 && p.bn == 128)) p.slices = 1;
+            if (!ok) p.bm = p.bn = 0;
+        }
+        return p;
+    }();
+    if (forced.bm == 0) return false;
+    plan = forced;
+    return true;
+}
+
 GemmPlan plan_gemm(int64_t m, int64_t n, int k_steps, int n_cus) {
-    constexpr double kQ128 = 0.72, kQ64 = 0.4;
+    // relative rate of a half-size tile (256 x 128 dequantizes half as many weights per MFMA
+    // as 128 x 256 and is used whenever there are more than 128 rows) and of a quarter-size one
+    const double kQ128 = m > 128 ? 0.76 : 0.68, kQ64 = 0.4;
+    const int hm = m > 128 ? 256 : 128, hn = m > 128 ? 128 : 256; // the half-size tile
+    {
+        GemmPlan forced;
+        if (forced_plan(forced)) {
+            while (forced.slices > 1 && k_steps / 4 < forced.slices) forced.slices /= 2;
+            return forced;
+        }
+    }
     auto tiles = [&](int bm, int bn, int64_t cols) { return ((m + bm - 1) / bm) * ((cols + bn - 1) / bn); };
     auto rounds = [&](int64_t t) { return (double)((t + n_cus - 1) / n_cus); };
     GemmPlan best{256, 256, 1, 0};
@@ -670,15 +732,15 @@ GemmPlan plan_gemm(int64_t m, int64_t n, int k_steps, int n_cus) {
     auto consider = [&](GemmPlan p, double cost) {
         if (cost < 0.97 * best_cost) best = p, best_cost = cost;
     };
-    consider({128, 256, 1, 0}, rounds(tiles(128, 256, n)) * k_steps * 0.5 / kQ128);
+    consider({hm, hn, 1, 0}, rounds(tiles(hm, hn, n)) * k_steps * 0.5 / kQ128);
     consider({128, 128, 1, 0}, rounds(tiles(128, 128, n)) * k_steps * 0.25 / kQ64);
-    // whole rounds of 256 x 256 tiles first, the rest as 128 x 256 tiles
+    // whole rounds of 256 x 256 tiles first, the remaining columns as half-size tiles
     const int64_t tiles_m256 = (m + 255) / 256, cols256 = (n + 255) / 256;
     const int64_t full_cols = (tiles_m256 * cols256 / n_cus) * n_cus / tiles_m256;
     if (full_cols > 0 && full_cols < cols256)
-        consider({128, 256, 1, full_cols},
+        consider({hm, hn, 1, full_cols},
                  (double)(tiles_m256 * full_cols / n_cus) * k_steps +
-                     rounds(tiles(128, 256, n - full_cols * 256)) * k_steps * 0.5 / kQ128);
+                     rounds(tiles(hm, hn, n - full_cols * 256)) * k_steps * 0.5 / kQ128);
     // split along k: the slices' f32 tiles are written and read once more (about 4 TB/s,
     // a 256 x 256 k step takes about 1.5 us)
     for (int slices = 2; slices <= 8; slices *= 2) {
@@ -686,7 +748,7 @@ GemmPlan plan_gemm(int64_t m, int64_t n, int k_steps, int n_cus) {
         const double reduce_cost = 2.0 * slices * (double)m * (double)n * 4.0 / 4e12 * 1e6 / 1.5 + 2.0;
         const double steps = 4.0 * (double)((k_steps / 4 + slices - 1) / slices); // slices are whole units
         consider({256, 256, slices, 0}, rounds(tiles(256, 256, n) * slices) * steps + reduce_cost);
-        consider({128, 256, slices, 0}, rounds(tiles(128, 256, n) * slices) * steps * 0.5 / kQ128 + reduce_cost);
+        consider({hm, hn, slices, 0}, rounds(tiles(hm, hn, n) * slices) * steps * 0.5 / kQ128 + reduce_cost);
     }
     return best;
 }
@@ -705,7 +767,8 @@ hipError_t launch_qt(const GemmParams& P0, int n_cus, hipStream_t stream) {
         P.n_begin = P.n_end;
         P.n_end = P0.n;
     }
-    if (plan.bm == 256) return launch_tile<QT, 256, 256>(P, plan.slices, stream);
+    if (plan.bm == 256 && plan.bn == 256) return launch_tile<QT, 256, 256>(P, plan.slices, stream);
+    if (plan.bm == 256) return launch_tile<QT, 256, 128>(P, plan.slices, stream);
     if (plan.bn == 256) return launch_tile<QT, 128, 256>(P, plan.slices, stream);
     return launch_tile<QT, 128, 128>(P, 1, stream);
 }
@@ -741,6 +804,7 @@ hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uin
     P.out_bf16 = out_bf16;
     P.tiles_m = P.tiles_n = 0;
     P.slice_units = 0;
+    P.nibble_mask = 0x0f0f0f0fu;
     P.partial = (float*)workspace;
     return L.dtype == QMM_Q4_K ? launch_qt<QMM_Q4_K>(P, n_cus, stream)
                                : launch_qt<QMM_Q8_0>(P, n_cus, stream);
