@@ -547,11 +547,15 @@ int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_
         const QmmLayout* layouts[QMM_MAX_GROUP];
         const void* tiled[QMM_MAX_GROUP];
         for (int i = 0; i < n_weights; i++) layouts[i] = &weights[i]->layout, tiled[i] = weights[i]->tiled;
-        ProfileScope prof(w0, stream);
-        hipError_t e = qmm_launch_gemv_multi(layouts, tiled, n_weights, x, m, ys, w0->n_cus, stream);
-        if (e == hipSuccess) return IZWI_QMM_OK;
-        if (e != hipErrorNotSupported) return fail_hip(e, "grouped decode kernel");
-        (void)hipGetLastError();
+        // one launch for up to two rows; more rows on this kernel (threshold raised through the
+        // environment) go projection by projection
+        if (m <= 2) {
+            ProfileScope prof(w0, stream);
+            hipError_t e = qmm_launch_gemv_multi(layouts, tiled, n_weights, x, m, ys, w0->n_cus, stream);
+            if (e == hipSuccess) return IZWI_QMM_OK;
+            if (e != hipErrorNotSupported) return fail_hip(e, "grouped decode kernel");
+            (void)hipGetLastError();
+        }
         for (int i = 0; i < n_weights; i++)
             if (int rc = izwi_qmm_forward_f32(weights[i], x, m, ys[i], mem_space, stream_)) return rc;
         return IZWI_QMM_OK;

@@ -540,6 +540,10 @@ void choose_split(const QmmLayout& L, int n_cus, int grid_y, bool gated, GemvPar
     int nwr_max = budget / nwk;
     int64_t want = L.row_tiles * grid_y / (n_cus > 0 ? n_cus : 1);
     int nwr = (int)(want < 1 ? 1 : (want > nwr_max ? nwr_max : want));
+    // More than one full workgroup per CU (gate|up group): the register count lets 20 waves
+    // share a CU, so two 8-wave workgroups run side by side (one loads while the other
+    // multiplies) where a second 12-wave workgroup would wait for the first to end.
+    if (grid_y == 1 && nwk * nwr > 8 && nwk <= 4 && L.row_tiles > (int64_t)nwr * n_cus) nwr = 8 / nwk;
     if (grid_y == 1 && L.row_tiles >= 16 * (int64_t)n_cus) {
         // very tall (LM head): whole row-tiles per wave, no barrier per row-tile
         nwk = 1;
