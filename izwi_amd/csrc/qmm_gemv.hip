@@ -431,7 +431,11 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                         x16_finish(f, in1, v);
                         x_item_quantize<QT, MT>(l, k_units, item, v);
                     }
-                    lds_barrier();
+                    // One row, one row-tile per workgroup, four units per panel: wave wk has just
+                    // quantized exactly the units 4 wk .. 4 wk + 3 that its own panel multiplies
+                    // (LDS serves a wave's accesses in order), so no wave waits for another here.
+                    const bool own_units = ONESHOT && MT == 1 && !GATED && !GROUPED && P.nwr == 1 && P.slots == 64;
+                    if (!own_units) lds_barrier();
                     x_ready = true;
                 } else {
                     load_panel<QT>(p, wbase + off, P.slots, lane, active);
