@@ -384,16 +384,17 @@ __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT>
 __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int m_end, const uint8_t* w_first,
                                           float* y_out, int n_rows, int row_tiles, int rtg0, uint8_t* smem) {
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int lane0 = threadIdx.x & 63;
+    // wave-uniform by construction; said so, the row-tile, panel offset and output row that
+    // derive from it live in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int stack_waves = P.nwk * P.nwr;               // waves per weight stack
     const int waves = GATED ? 2 * stack_waves : stack_waves; // = blockDim.x / 64, without the dispatch packet read
     const int stack = GATED && wave >= stack_waves ? 1 : 0;
     const int sw = wave - stack * stack_waves;
     const int wr = (sw * P.wave_magic) >> 16;
     const int wk = sw - wr * P.nwk;
-    const bool lane_active = lane < P.slots;
-    const int us = lane >> 4;
+    const bool lane_active = lane0 < P.slots;
     const int k_units = (P.k + 255) >> 8, s_units = P.slots >> 4;
     const uint8_t* wbase = stack ? P.w2 + (w_first - P.w) : w_first; // the second stack at the same offset
     const XLds<QT> l = carve<QT, MT>(smem, k_units);
@@ -422,7 +423,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                     float4 f[4];
                     float v[16];
                     const bool in0 = x_item_issue<MT>(xs, group, group < items, f);
-                    load_panel<QT>(p, wbase + off, P.slots, lane, active);
+                    load_panel<QT>(p, wbase + off, P.slots, lane0, active);
                     if (m0 != m_begin) lds_barrier(); // the previous rows' readers are done
                     x16_finish(f, in0, v);
                     if (group < items) x_item_quantize<QT, MT>(l, k_units, group, v);
@@ -438,12 +439,16 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                     if (!own_units) lds_barrier();
                     x_ready = true;
                 } else {
-                    load_panel<QT>(p, wbase + off, P.slots, lane, active);
+                    load_panel<QT>(p, wbase + off, P.slots, lane0, active);
                 }
-                mask_panel<QT>(p, active);
-                const int unit = min(kg * s_units + us, k_units - 1);
+                // the lane index again, from the hardware: nothing lane-derived has to stay in a
+                // register across the quantizer
+                const int lane_m = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+                mask_panel<QT>(p, ok && lane_m < P.slots);
+                const int unit = min(kg * s_units + (lane_m >> 4), k_units - 1);
                 multiply_panel<QT, MT>(p, l, unit, k_units, acc);
             }
+            const int lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); // as above
             // row-tile finished: combine the S units of a row, then the waves that split k
 #pragma unroll
             for (int mi = 0; mi < MT; mi++) {
@@ -491,8 +496,11 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
 // QMM_MOE_SEG_ROWS rows; uniform for the workgroup) at run time: most segments of a
 // small batch hold one or two pairs, and a row costs its share of the arithmetic
 // whether it exists or not.
+// The dense straight-line single-row Q4_K form is held to 80 registers: six waves per SIMD,
+// i.e. two 12-wave workgroups per CU.
 template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false>
-__global__ __launch_bounds__(64 * kMaxWaves) void gemv_kernel(GemvParams P) {
+__global__ __launch_bounds__(64 * kMaxWaves)
+__attribute__((amdgpu_waves_per_eu((ONESHOT && !GROUPED && MT == 1 && QT == QMM_Q4_K) ? 6 : 3))) void gemv_kernel(GemvParams P) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int m_begin = 0, m_end = P.m;
     int64_t w_offset = 0;
