@@ -7,6 +7,7 @@ HIP kernels for gfx950; there is no CPU or PyTorch fallback: if the library is
 missing or no GPU is present, calls raise.
 """
 from .capi import QmmError, lib, library_path  # noqa: F401
+from .gguf import GgufLoader, GgufModelInfo, is_gguf_file  # noqa: F401
 from .qmatmul import (  # noqa: F401
     GgmlDType,
     MoeExperts,

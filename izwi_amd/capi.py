@@ -1,4 +1,4 @@
-"""ctypes binding of include/izwi_qmm.h (one prototype per exported symbol)."""
+"""ctypes binding of include/izwi_qmm.h and include/izwi_gguf.h (one prototype per exported symbol)."""
 from __future__ import annotations
 
 import ctypes as C
@@ -33,10 +33,17 @@ class ProfileSnapshot(C.Structure):
         "silu_mul_fused_calls", "silu_mul_fallback_calls")]
 
 
+class GgufTensorInfo(C.Structure):
+    """izwi_gguf_tensor_info (include/izwi_gguf.h)."""
+    _fields_ = [("ggml_dtype", C.c_int32), ("n_dims", C.c_int32), ("dims", C.c_int64 * 8),
+                ("offset", C.c_uint64), ("nbytes", C.c_uint64), ("data", C.c_void_p)]
+
+
 _i32, _i64, _u64, _vp = C.c_int32, C.c_int64, C.c_uint64, C.c_void_p
 _pp = C.POINTER(C.c_void_p)
+_cpp = C.POINTER(C.c_char_p)
 
-# name -> (restype, argtypes); must list every symbol include/izwi_qmm.h declares
+# name -> (restype, argtypes); must list every symbol include/izwi_qmm.h and include/izwi_gguf.h declare
 PROTOTYPES = {
     "izwi_qmm_abi_version": (C.c_int, []),
     "izwi_qmm_init": (C.c_int, [C.c_int]),
@@ -62,6 +69,25 @@ PROTOTYPES = {
     "izwi_qmm_profile_snapshot_get": (C.c_int, [C.POINTER(ProfileSnapshot)]),
     "izwi_qmm_profile_reset": (C.c_int, []),
     "izwi_qmm_weight_set_lm_head": (C.c_int, [_vp, C.c_int]),
+    # include/izwi_gguf.h
+    "izwi_gguf_is_gguf_file": (C.c_int, [C.c_char_p]),
+    "izwi_gguf_open": (C.c_int, [C.c_char_p, _pp]),
+    "izwi_gguf_close": (None, [_vp]),
+    "izwi_gguf_header": (C.c_int, [_vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(_u64)]),
+    "izwi_gguf_tensor_count": (_i64, [_vp]),
+    "izwi_gguf_tensor_name": (C.c_int, [_vp, _i64, _cpp]),
+    "izwi_gguf_tensor_info_get": (C.c_int, [_vp, C.c_char_p, C.POINTER(GgufTensorInfo)]),
+    "izwi_gguf_metadata_count": (_i64, [_vp]),
+    "izwi_gguf_metadata_key": (C.c_int, [_vp, _i64, _cpp]),
+    "izwi_gguf_metadata_type": (C.c_int, [_vp, C.c_char_p]),
+    "izwi_gguf_metadata_string": (C.c_int, [_vp, C.c_char_p, _pp, C.POINTER(_u64)]),
+    "izwi_gguf_metadata_u64": (C.c_int, [_vp, C.c_char_p, C.POINTER(_u64)]),
+    "izwi_gguf_metadata_f64": (C.c_int, [_vp, C.c_char_p, C.POINTER(C.c_double)]),
+    "izwi_gguf_metadata_array": (C.c_int, [_vp, C.c_char_p, C.POINTER(_i32), C.POINTER(_u64), _pp]),
+    "izwi_gguf_metadata_array_string": (C.c_int, [_vp, C.c_char_p, _u64, _pp, C.POINTER(_u64)]),
+    "izwi_gguf_load_weight": (C.c_int, [_vp, C.c_char_p, _pp]),
+    "izwi_gguf_load_packed": (C.c_int, [_vp, _cpp, _i32, _pp]),
+    "izwi_gguf_load_tensor_f32": (C.c_int, [_vp, C.c_char_p, _vp, _u64, C.c_int, _vp]),
 }
 
 _lib = None

@@ -39,6 +39,21 @@ int fail(int code, const char* fmt, ...) {
     return code;
 }
 
+} // namespace
+
+// the same thread-local message for the library's other translation units
+int qmm_fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_error = buf;
+    return code;
+}
+
+namespace {
+
 int fail_hip(hipError_t e, const char* what) {
     return fail(IZWI_QMM_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }

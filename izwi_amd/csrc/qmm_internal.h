@@ -55,6 +55,9 @@ __device__ __forceinline__ uint16_t qmm_f32_to_bf16_bits(float f) {
 
 #endif // __HIPCC__
 
+// Records the calling thread's error message (read with izwi_qmm_last_error) and returns `code`.
+int qmm_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
 // ---- launchers -------------------------------------------------------------
 hipError_t qmm_launch_repack(const QmmLayout& L, const void* native, void* tiled,
                              hipStream_t stream);

@@ -10,6 +10,7 @@
 //   packed_qmatmul_from_qtensors  core.rs:846-889
 //   quantized_storage_bytes       core.rs:891-909
 //   Qwen3Projection               core.rs:671-674, 710-718, 791-831 (quantized arm)
+//   GgufLoader, is_gguf_file      crates/izwi-core/src/models/shared/weights/gguf.rs:36-203, 366-377
 //   Error                         crates/izwi-core/src/error.rs:69-73 (InferenceError /
 //                                 ModelLoadError / InvalidInput)
 // There is no CPU fallback: without a gfx950 device every operation throws.
@@ -22,6 +23,7 @@
 #include <utility>
 #include <vector>
 
+#include "izwi_gguf.h"
 #include "izwi_qmm.h"
 
 namespace izwi {
@@ -214,6 +216,90 @@ public:
 private:
     explicit Qwen3Projection(QMatMul mm) : mm_(std::move(mm)) {}
     QMatMul mm_;
+};
+
+// `is_gguf_file` (gguf.rs:366-377).
+inline bool is_gguf_file(const std::string& path) { return izwi_gguf_is_gguf_file(path.c_str()) != 0; }
+
+// `GgufLoader` (gguf.rs:36-203): one mapped GGUF file; tensors go from the mapping straight
+// into weight handles on the current HIP device.  Parsing and lookups need no GPU.
+class GgufLoader {
+public:
+    static std::shared_ptr<GgufLoader> from_path(const std::string& path) {
+        izwi_gguf* g = nullptr;
+        const int rc = izwi_gguf_open(path.c_str(), &g);
+        if (rc != IZWI_QMM_OK) // `Error::ModelLoadError("Failed to open / parse GGUF file: ...")`
+            throw Error(Error::Kind::ModelLoadError, rc, izwi_qmm_last_error());
+        return std::shared_ptr<GgufLoader>(new GgufLoader(g));
+    }
+    ~GgufLoader() { izwi_gguf_close(g_); }
+    GgufLoader(const GgufLoader&) = delete;
+    GgufLoader& operator=(const GgufLoader&) = delete;
+
+    size_t tensor_count() const { return (size_t)izwi_gguf_tensor_count(g_); }
+    std::vector<std::string> tensor_names() const {
+        std::vector<std::string> out;
+        for (int64_t i = 0; i < izwi_gguf_tensor_count(g_); i++) {
+            const char* name = nullptr;
+            check(izwi_gguf_tensor_name(g_, i, &name));
+            out.emplace_back(name);
+        }
+        return out;
+    }
+    bool has_tensor(const std::string& name) const {
+        izwi_gguf_tensor_info info;
+        return izwi_gguf_tensor_info_get(g_, name.c_str(), &info) == IZWI_QMM_OK;
+    }
+    // `tensor_shape`: empty optional upstream, here an empty vector with `found` false
+    std::vector<int64_t> tensor_shape(const std::string& name, bool* found = nullptr) const {
+        izwi_gguf_tensor_info info;
+        const bool ok = izwi_gguf_tensor_info_get(g_, name.c_str(), &info) == IZWI_QMM_OK;
+        if (found) *found = ok;
+        return ok ? std::vector<int64_t>(info.dims, info.dims + info.n_dims) : std::vector<int64_t>();
+    }
+    // `get_metadata_string` / `get_metadata_u64`: false if the key is absent or of another type
+    bool get_metadata_string(const std::string& key, std::string* out) const {
+        const char* p = nullptr;
+        uint64_t n = 0;
+        if (izwi_gguf_metadata_string(g_, key.c_str(), &p, &n) != IZWI_QMM_OK) return false;
+        out->assign(p, n);
+        return true;
+    }
+    bool get_metadata_u64(const std::string& key, uint64_t* out) const {
+        return izwi_gguf_metadata_u64(g_, key.c_str(), out) == IZWI_QMM_OK;
+    }
+    // `load_qtensor(name, device)`
+    std::shared_ptr<QTensor> load_qtensor(const std::string& name) const {
+        izwi_qmm_weight* h = nullptr;
+        const int rc = izwi_gguf_load_weight(g_, name.c_str(), &h);
+        if (rc != IZWI_QMM_OK) throw Error(Error::Kind::ModelLoadError, rc, izwi_qmm_last_error());
+        return QTensor::adopt(h);
+    }
+    // `packed_quantized_qmatmul(loader, device, names)` (core.rs:834-845)
+    QMatMul load_packed_qmatmul(const std::vector<std::string>& names) const {
+        std::vector<const char*> ptrs;
+        for (const std::string& n : names) ptrs.push_back(n.c_str());
+        izwi_qmm_weight* h = nullptr;
+        check(izwi_gguf_load_packed(g_, ptrs.data(), (int32_t)ptrs.size(), &h));
+        return QMatMul::from_qtensor(QTensor::adopt(h));
+    }
+    // `load_tensor(name, DType::F32, device)` into host memory
+    std::vector<float> load_tensor(const std::string& name) const {
+        izwi_gguf_tensor_info info;
+        const int rc = izwi_gguf_tensor_info_get(g_, name.c_str(), &info);
+        if (rc != IZWI_QMM_OK) throw Error(Error::Kind::ModelLoadError, rc, izwi_qmm_last_error());
+        uint64_t count = 1;
+        for (int i = 0; i < info.n_dims; i++) count *= (uint64_t)info.dims[i];
+        std::vector<float> out(count);
+        const int rc2 = izwi_gguf_load_tensor_f32(g_, name.c_str(), out.data(), count, IZWI_QMM_HOST, nullptr);
+        if (rc2 != IZWI_QMM_OK) throw Error(Error::Kind::ModelLoadError, rc2, izwi_qmm_last_error());
+        return out;
+    }
+    const izwi_gguf* handle() const { return g_; }
+
+private:
+    explicit GgufLoader(izwi_gguf* g) : g_(g) {}
+    izwi_gguf* g_;
 };
 
 } // namespace izwi

@@ -1,7 +1,7 @@
 // Exercises the C++ host-side mirror (izwi_amd/host/izwi_qmm.hpp) the way the
 // reference's own unit tests exercise its Rust types.
-//   host_mirror_test cpu   host logic only: byte-size rule and its errors, loud failure
-//                          without a gfx950 device
+//   host_mirror_test cpu [fixture]   host logic only: byte-size rule and its errors, GGUF
+//                          container parse of tests/golden/tiny.gguf
 //   host_mirror_test gpu   the reference's packed-projection test
 //                          (crates/izwi-core/src/models/architectures/qwen3/core.rs:3099-3142)
 //                          and a Q4_K projection, checked against the CPU oracle
@@ -121,12 +121,59 @@ static void q4k_projection_matches_oracle() {
     EXPECT(max_rel(y, want) < 1e-4f);
 }
 
+// The committed GGUF fixture (tests/golden/tiny.gguf, laid out by hand from the container
+// format): three tensors, alignment 64.  Parsing needs no GPU.
+static void gguf_parse(const std::string& fixture) {
+    EXPECT(izwi::is_gguf_file(fixture));
+    EXPECT(!izwi::is_gguf_file(fixture + ".absent"));
+    auto g = izwi::GgufLoader::from_path(fixture);
+    EXPECT(g->tensor_count() == 3);
+    const std::vector<std::string> names = g->tensor_names();
+    EXPECT(names.size() == 3 && names[0] == "a" && names[1] == "blk.q" && names[2] == "hand.q4k");
+    EXPECT(g->has_tensor("blk.q") && !g->has_tensor("blk.k"));
+    EXPECT((g->tensor_shape("hand.q4k") == std::vector<int64_t>{1, 256}));
+    bool found = true;
+    EXPECT(g->tensor_shape("nope", &found).empty() && !found);
+    std::string arch;
+    uint64_t v = 0;
+    EXPECT(g->get_metadata_string("general.architecture", &arch) && arch == "qwen3");
+    EXPECT(g->get_metadata_u64("general.alignment", &v) && v == 64);
+    EXPECT(!g->get_metadata_string("general.alignment", &arch) && !g->get_metadata_u64("absent", &v));
+    EXPECT(throws(izwi::Error::Kind::ModelLoadError, "Failed to open GGUF file",
+                  [&] { izwi::GgufLoader::from_path(fixture + ".absent"); }));
+    EXPECT(throws(izwi::Error::Kind::ModelLoadError, "not supported", [&] { g->load_qtensor("a"); }));
+    EXPECT(throws(izwi::Error::Kind::ModelLoadError, "tensor not found", [&] { g->load_qtensor("nope"); }));
+}
+
+// ... and its tensors on the GPU: the Q4_K tensor is the hand-built block whose closed form
+// sums to 32224; the Q8_0 block is d = 1, q = -16 .. 15.
+static void gguf_load(const std::string& fixture) {
+    auto g = izwi::GgufLoader::from_path(fixture);
+    auto q4 = g->load_qtensor("hand.q4k");
+    EXPECT(q4->dtype() == izwi::GgmlDType::Q4K && q4->rows() == 1 && q4->cols() == 256);
+    const std::vector<float> deq = q4->dequantize();
+    double sum = 0;
+    for (float f : deq) sum += f;
+    EXPECT(sum == 32224.0 && deq[224] == 346.5f && deq[32] == -2.5f);
+    EXPECT(g->load_tensor("hand.q4k") == deq);
+    const std::vector<float> q8 = g->load_tensor("blk.q");
+    EXPECT(q8.size() == 32 && q8[0] == -16.0f && q8[31] == 15.0f);
+    EXPECT((g->load_tensor("a") == std::vector<float>{1.0f, 2.0f, 3.0f, 4.0f}));
+    // a projection loaded from the file: y = x . w with x = ones gives the row sum
+    std::vector<float> x(32, 1.0f);
+    const std::vector<float> y = izwi::QMatMul::from_qtensor(g->load_qtensor("blk.q")).forward(x);
+    EXPECT(y.size() == 1 && std::fabs(y[0] - (-16.0f)) < 1e-3f);
+}
+
 int main(int argc, char** argv) {
     const std::string mode = argc > 1 ? argv[1] : "cpu";
+    const std::string fixture = argc > 2 ? argv[2] : "tests/golden/tiny.gguf";
     host_logic();
+    gguf_parse(fixture);
     if (mode == "gpu") {
         packed_matches_separate_q8_0();
         q4k_projection_matches_oracle();
+        gguf_load(fixture);
     } else if (mode == "nodevice") {
         no_device_is_loud();
     }

@@ -13,6 +13,10 @@ that holds the arithmetic is not in its tree).  They restate, as data:
   bytes and the outputs of candle-core's algorithm on them, computed here with plain
   numpy arithmetic (no code of the oracle or of the library is used).
 
+* tiny.gguf + tiny_gguf.json - a small GGUF version 3 file assembled byte by byte from the
+  public container format (no writer or reader of this repository is used), and what a
+  reader must report for it; its Q4_K tensor is the hand block above.
+
 Run:  python tests/golden/make_fixtures.py
 """
 import json
@@ -94,7 +98,48 @@ def packed_case():
             "reference_tolerance_packed_vs_separate": 1e-5}
 
 
+def tiny_gguf():
+    """A GGUF version 3 file laid out by hand from the public container format: header, three
+    metadata entries (alignment 64), three tensor infos, padding, data.  Returns the file's
+    bytes and what a reader must report."""
+    import struct
+
+    def s(text):
+        b = text.encode("utf-8")
+        return struct.pack("<Q", len(b)) + b
+
+    f32 = np.array([[1.0, 2.0], [3.0, 4.0]], dtype=np.float32).tobytes()
+    q8 = np.float16(1.0).tobytes() + bytes(np.arange(-16, 16, dtype=np.int8).view(np.uint8))
+    q4 = bytes.fromhex(q4k_hand_block()["block_hex"])
+    head = b"GGUF" + struct.pack("<IQQ", 3, 3, 3)
+    head += s("general.architecture") + struct.pack("<I", 8) + s("qwen3")
+    head += s("general.alignment") + struct.pack("<I", 4) + struct.pack("<I", 64)
+    head += s("test.ids") + struct.pack("<I", 9) + struct.pack("<IQ", 2, 3) + struct.pack("<HHH", 1, 2, 3)
+    # dims are written innermost first; offsets are multiples of the alignment
+    head += s("a") + struct.pack("<I", 2) + struct.pack("<QQ", 2, 2) + struct.pack("<IQ", 0, 0)
+    head += s("blk.q") + struct.pack("<I", 2) + struct.pack("<QQ", 32, 1) + struct.pack("<IQ", 8, 64)
+    head += s("hand.q4k") + struct.pack("<I", 2) + struct.pack("<QQ", 256, 1) + struct.pack("<IQ", 12, 128)
+    data_offset = (len(head) + 63) // 64 * 64
+    blob = head + bytes(data_offset - len(head))
+    blob += f32 + bytes(64 - len(f32)) + q8 + bytes(64 - len(q8)) + q4
+    want = {"header": [3, 64, data_offset],
+            "metadata": {"general.architecture": "qwen3", "general.alignment": 64, "test.ids": [1, 2, 3]},
+            "tensors": [
+                {"name": "a", "shape": [2, 2], "ggml_dtype": 0, "offset": 0, "bytes_hex": f32.hex()},
+                {"name": "blk.q", "shape": [1, 32], "ggml_dtype": 8, "offset": 64, "bytes_hex": q8.hex()},
+                {"name": "hand.q4k", "shape": [1, 256], "ggml_dtype": 12, "offset": 128, "bytes_hex": q4.hex()}],
+            "dequantized": {"a": [1.0, 2.0, 3.0, 4.0], "blk.q": [float(v) for v in range(-16, 16)],
+                            "hand.q4k": q4k_hand_block()["expected_f32"]}}
+    return blob, want
+
+
 if __name__ == "__main__":
+    blob, want = tiny_gguf()
+    with open(os.path.join(HERE, "tiny.gguf"), "wb") as f:
+        f.write(blob)
+    with open(os.path.join(HERE, "tiny_gguf.json"), "w") as f:
+        json.dump(want, f, indent=1)
+    print("wrote tiny.gguf, tiny_gguf.json")
     for name, rec in (("q4k_hand_block.json", q4k_hand_block()), ("packed_q8_0_case.json", packed_case())):
         with open(os.path.join(HERE, name), "w") as f:
             json.dump(rec, f, indent=1)

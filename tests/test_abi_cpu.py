@@ -10,9 +10,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def header_symbols():
-    text = open(os.path.join(ROOT, "include", "izwi_qmm.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(izwi_(?:qmm|moe)_[a-z0-9_]+)\s*\(", text)))
+    names = set()
+    for header in ("izwi_qmm.h", "izwi_gguf.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(izwi_(?:qmm|moe|gguf)_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 @pytest.fixture(scope="module")
@@ -29,7 +32,7 @@ def test_library_exports_every_declared_symbol(capi):
     names = header_symbols()
     assert len(names) >= 20
     for name in names:
-        assert hasattr(L, name), f"{name} declared in izwi_qmm.h but not exported"
+        assert hasattr(L, name), f"{name} declared in include/*.h but not exported"
 
 
 def test_binding_covers_every_declared_symbol(capi):

@@ -21,7 +21,8 @@ def _binary(may_build: bool) -> str:
 
 
 def _run(mode: str, may_build: bool):
-    proc = subprocess.run([_binary(may_build), mode], capture_output=True, text=True, timeout=120)
+    fixture = os.path.join(HERE, "golden", "tiny.gguf")
+    proc = subprocess.run([_binary(may_build), mode, fixture], capture_output=True, text=True, timeout=120)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "all checks passed" in proc.stdout
 
