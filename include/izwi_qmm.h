@@ -163,6 +163,19 @@ int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_
                                const float* x, int64_t m, float* const* ys, int mem_space,
                                void* stream);
 
+/* The gate / up pair of `Qwen3Mlp::forward` (qwen3/core.rs:1786-1798) with its activation:
+ *     h[m, n] = silu(gate.forward(x)) * up.forward(x)
+ * i.e. `gate_up_proj.forward(x)` followed by `try_fused_silu_mul` (kernels/mod.rs:94-108) or
+ * `ops::silu(&gate)?.broadcast_mul(&up)` in one call.  `gate` and `up` are [n, k] weights of the
+ * same shape and type.  The two sums are those of izwi_qmm_forward_f32 bit for bit; silu(v) =
+ * v / (1 + exp(-v)) in f32.  For m <= 2 the product is applied inside the decode kernel (one
+ * launch, h is the only output written); for larger m the two projections run as a projection
+ * group into scratch and one elementwise kernel follows.  Counted in
+ * `silu_mul_fused_calls` of the profile snapshot. */
+int izwi_qmm_forward_gate_up_silu_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
+                                      const float* x, int64_t m, float* h, int mem_space,
+                                      void* stream);
+
 /* Prefill form: bf16 activations `[m, k]`, weights dequantized to bf16 in LDS,
  * MFMA with f32 accumulation; y is f32 or bf16 per `out_dtype`.  Replaces the
  * to_dtype(F32) -> QMatMul -> to_dtype(activation dtype) sequence of

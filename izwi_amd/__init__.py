@@ -14,6 +14,7 @@ from .qmatmul import (  # noqa: F401
     QMatMul,
     QTensor,
     Qwen3GateUpProjection,
+    Qwen3Mlp,
     Qwen3Projection,
     Qwen3QkvProjection,
     forward_group,

@@ -598,6 +598,56 @@ int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_
     return IZWI_QMM_OK;
 }
 
+int izwi_qmm_forward_gate_up_silu_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
+                                      const float* x, int64_t m, float* h, int mem_space,
+                                      void* stream_) {
+    if (!gate || !up) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    if (int rc = check_space(mem_space)) return rc;
+    const QmmLayout& L = gate->layout;
+    const QmmLayout& U = up->layout;
+    if (L.n_stacked != 1 || U.n_stacked != 1) return fail(IZWI_QMM_ERR_INVALID, "forward on an expert stack");
+    if (L.n != U.n || L.k != U.k)
+        return fail(IZWI_QMM_ERR_INVALID, "gate is [%lld, %lld], up is [%lld, %lld]", (long long)L.n, (long long)L.k,
+                    (long long)U.n, (long long)U.k);
+    if (L.dtype != U.dtype) return fail(IZWI_QMM_ERR_INVALID, "gate and up have different ggml dtypes (%d, %d)", L.dtype, U.dtype);
+    if (gate->device != up->device) return fail(IZWI_QMM_ERR_INVALID, "gate and up live on different devices");
+    if (m < 0) return fail(IZWI_QMM_ERR_INVALID, "negative m");
+    if (m == 0 || L.n == 0) return IZWI_QMM_OK;
+    if (!x) return fail(IZWI_QMM_ERR_INVALID, "x is NULL");
+    if (!h) return fail(IZWI_QMM_ERR_INVALID, "h is NULL");
+    hipStream_t stream = (hipStream_t)stream_;
+    Staged xi, ho;
+    HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
+    HIP_TRY(ho.out(h, (size_t)m * L.n * sizeof(float), mem_space));
+    if (profiling()) g_silu_fused.fetch_add(1, std::memory_order_relaxed);
+    if (m < mfma_min_m() && m <= 2) {
+        ProfileScope prof(gate, stream);
+        HIP_TRY(qmm_launch_gemv_gated(L, gate->tiled, up->tiled, (const float*)xi.dev, m, (float*)ho.dev,
+                                      gate->n_cus, stream));
+    } else {
+        // both projections into scratch (one projection-group call), then the elementwise product
+        const size_t part = (size_t)m * L.n * sizeof(float);
+        void* gu = nullptr;
+        {
+            // the group call below uses the start of the same per-stream scratch for the quantized
+            // activations: its own need comes first, the two outputs behind it
+            const size_t group_need =
+                m <= 64 ? qmm_gemv_mfma_workspace_bytes(L, m)
+                        : ((((size_t)m * L.k * sizeof(uint16_t)) + 255) & ~(size_t)255) + qmm_gemm_workspace_bytes(L, m, gate->n_cus);
+            const size_t base = (group_need + 255) & ~(size_t)255;
+            void* scratch = nullptr;
+            HIP_TRY(get_scratch(gate->device, stream, base + 2 * part, &scratch));
+            gu = static_cast<uint8_t*>(scratch) + base;
+        }
+        const izwi_qmm_weight* ws[2] = {gate, up};
+        float* ys[2] = {static_cast<float*>(gu), reinterpret_cast<float*>(static_cast<uint8_t*>(gu) + part)};
+        if (int rc = izwi_qmm_forward_group_f32(ws, 2, (const float*)xi.dev, m, ys, IZWI_QMM_DEVICE, stream_)) return rc;
+        HIP_TRY(qmm_launch_silu_mul(ys[0], ys[1], (float*)ho.dev, (int64_t)m * L.n, stream));
+    }
+    HIP_TRY(ho.finish(stream));
+    return IZWI_QMM_OK;
+}
+
 int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int64_t m, void* y,
                           int out_dtype, int mem_space, void* stream_) {
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");

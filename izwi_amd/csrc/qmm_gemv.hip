@@ -580,7 +580,7 @@ hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipS
     if (grid < 1) grid = 1;
     // straight-line form: one pass of rows (a segment never has more than MT rows in the
     // grouped form), one row-tile group per workgroup, one k step
-    constexpr bool kCanOneshot = GROUPED ? MT == QMM_MOE_SEG_ROWS : !GATED;
+    constexpr bool kCanOneshot = GROUPED ? MT == QMM_MOE_SEG_ROWS : true;
     const bool oneshot = kCanOneshot && (GROUPED || P.m <= MT) && P.kpw == 1 && grid == P.rt_groups;
     const void* fn = oneshot ? reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot>)
                              : reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, false>);
@@ -695,6 +695,41 @@ hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x
     choose_split(L, n_cus, 1, false, P, waves);
     return L.dtype == QMM_Q4_K ? launch_plain<QMM_Q4_K>(P, waves, n_cus, stream)
                                : launch_plain<QMM_Q8_0>(P, waves, n_cus, stream);
+}
+
+namespace {
+
+__global__ void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                float* __restrict__ out, int64_t count) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) out[i] = silu(gate[i]) * up[i];
+}
+
+} // namespace
+
+hipError_t qmm_launch_silu_mul(const float* gate, const float* up, float* out, int64_t count,
+                               hipStream_t stream) {
+    if (count <= 0) return hipSuccess;
+    const int64_t grid = (count + 255) / 256;
+    if (grid > 0x7fffffff) return hipErrorInvalidValue;
+    silu_mul_kernel<<<(unsigned)grid, 256, 0, stream>>>(gate, up, out, count);
+    return hipGetLastError();
+}
+
+hipError_t qmm_launch_gemv_gated(const QmmLayout& L, const void* tiled_gate, const void* tiled_up,
+                                 const float* x, int64_t m, float* y, int n_cus, hipStream_t stream) {
+    if (m <= 0 || L.n == 0) return hipSuccess;
+    if (m > 2) return hipErrorNotSupported;
+    GemvParams P;
+    if (!make_params(L, tiled_gate, x, m, y, P)) return hipErrorInvalidValue;
+    P.w2 = (const uint8_t*)tiled_up;
+    int waves;
+    choose_split(L, n_cus, 1, true, P, waves);
+    if (L.dtype == QMM_Q4_K)
+        return m == 2 ? launch_mt<QMM_Q4_K, 2, true, false>(P, waves, n_cus, 1, stream)
+                      : launch_mt<QMM_Q4_K, 1, true, false>(P, waves, n_cus, 1, stream);
+    return m == 2 ? launch_mt<QMM_Q8_0, 2, true, false>(P, waves, n_cus, 1, stream)
+                  : launch_mt<QMM_Q8_0, 1, true, false>(P, waves, n_cus, 1, stream);
 }
 
 hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,

@@ -71,6 +71,15 @@ hipError_t qmm_launch_dequant(const QmmLayout& L, const void* tiled, float* out,
 hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
                            float* y, int n_cus, hipStream_t stream);
 
+// Decode kernel for the gate / up pair of an MLP: y[m, n] = silu(W_gate x) * (W_up x), both
+// matrices of layout L, m <= 2 (hipErrorNotSupported beyond).  The sums are those of
+// qmm_launch_gemv; the product is applied where the waves that split k are combined.
+hipError_t qmm_launch_gemv_gated(const QmmLayout& L, const void* tiled_gate, const void* tiled_up,
+                                 const float* x, int64_t m, float* y, int n_cus, hipStream_t stream);
+// out[i] = silu(gate[i]) * up[i]
+hipError_t qmm_launch_silu_mul(const float* gate, const float* up, float* out, int64_t count,
+                               hipStream_t stream);
+
 // Batched decode kernel (int8 MFMA) for 3 <= m <= 64.  `workspace` must hold
 // qmm_gemv_mfma_workspace_bytes(L, m) bytes and stay untouched until the work
 // queued on `stream` has run.

@@ -279,6 +279,34 @@ class Qwen3GateUpProjection(Qwen3QkvProjection):
     def new_separate(cls, gate_proj: "QMatMul", up_proj: "QMatMul"):  # noqa: D102
         return cls(parts=(gate_proj, up_proj))
 
+    def forward_silu_mul(self, x: torch.Tensor) -> torch.Tensor:
+        """`forward(x)` followed by `try_fused_silu_mul(gate, up)` (qwen3/core.rs:1786-1796,
+        kernels/mod.rs:94-108) in one call: silu(gate x) * (up x)."""
+        if self._fused is not None:
+            gate, up = self.forward(x)
+            return torch.nn.functional.silu(gate) * up
+        gate_proj, up_proj = self._parts
+        assert x.dtype == torch.float32 and x.is_contiguous()
+        n, k = gate_proj.qtensor.dims2()
+        if x.dim() < 1 or x.shape[-1] != k:
+            raise capi.QmmError(-1, f"shape mismatch in qmatmul, lhs: {tuple(x.shape)}, rhs: ({n}, {k})")
+        m = x.numel() // k if k else 0
+        h = torch.empty(tuple(x.shape[:-1]) + (n,), dtype=torch.float32, device=x.device)
+        check(lib().izwi_qmm_forward_gate_up_silu_f32(gate_proj.qtensor._h, up_proj.qtensor._h, x.data_ptr(), m,
+                                                      h.data_ptr(), _space(x), _stream_ptr(x)))
+        return h
+
+
+class Qwen3Mlp:
+    """izwi-core's Qwen3Mlp (qwen3/core.rs:1740-1798) with quantized weights:
+    down(silu(gate x) * (up x))."""
+
+    def __init__(self, gate_up_proj: Qwen3GateUpProjection, down_proj: "QMatMul"):
+        self.gate_up_proj, self.down_proj = gate_up_proj, down_proj
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.down_proj.forward(self.gate_up_proj.forward_silu_mul(x))
+
 
 def quantize_activations(weight_dtype: GgmlDType, x: torch.Tensor) -> torch.Tensor:
     """The activation blocks the decode kernel builds (reference block layout, uint8)."""

@@ -418,3 +418,57 @@ def test_projection_group_8b_gate_up_and_errors(qa, oracle):
     q8 = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q8_0, make_weight(oracle, Q8_0, 96, 4096, 414), (96, 4096)))
     a, b = qa.forward_group([up, q8], x)
     assert torch.equal(a, up.forward(x)) and torch.equal(b, q8.forward(x))
+
+
+# ------------------------------------------------- gate / up with its activation --
+@pytest.mark.parametrize("dtype,n,k", [(Q4_K, 12288, 4096), (Q8_0, 3072, 1024), (Q4_K, 80, 768), (Q8_0, 40, 96)])
+@pytest.mark.parametrize("m", [1, 2, 5, 16, 80])
+def test_gate_up_silu_matches_separate_projections(qa, oracle, dtype, n, k, m):
+    """Qwen3Mlp::forward's gate_up_proj + silu * up (qwen3/core.rs:1786-1796) in one call: the two
+    sums are the separate projections' bit for bit, so the result equals silu(g) * u computed
+    from them up to the rounding of silu itself; against the oracle within the decode tolerance."""
+    _say(f"gate_up_silu dtype={dtype} n={n} k={k} m={m}")
+    dt = qa.GgmlDType(dtype)
+    wg, wu = make_weight(oracle, dtype, n, k, 500), make_weight(oracle, dtype, n, k, 501)
+    gate = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, wg, (n, k)))
+    up = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, wu, (n, k)))
+    x = torch.from_numpy(oracle.randn(502 + m, (m, k))).cuda()
+    proj = qa.Qwen3GateUpProjection.new_separate(gate, up)
+    h = proj.forward_silu_mul(x)
+    g, u = gate.forward(x), up.forward(x)
+    want = (g.double() / (1.0 + torch.exp(-g.double())) * u.double()).float()
+    assert h.shape == (m, n)
+    assert (h - want).abs().max().item() <= 2e-6 * max(want.abs().max().item(), 1e-30)
+    if m <= 16 and n <= 3072:
+        xo = x.cpu().numpy()
+        go, uo = oracle.qmatmul(dtype, xo, wg, n), oracle.qmatmul(dtype, xo, wu, n)
+        ref = go / (1.0 + np.exp(-go.astype(np.float64))) * uo
+        assert rel_err(h.cpu().numpy(), ref.astype(np.float32)) < (1e-4 if m <= 64 else 1e-2)
+
+
+def test_gate_up_silu_mlp_mirror_host_pointers_and_errors(qa, oracle):
+    dt = qa.GgmlDType.Q4K
+    n, k = 64, 512
+    wg, wu, wd = make_weight(oracle, Q4_K, n, k, 510), make_weight(oracle, Q4_K, n, k, 511), make_weight(oracle, Q4_K, k, 256, 512)
+    gate = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, wg, (n, k)))
+    up = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, wu, (n, k)))
+    proj = qa.Qwen3GateUpProjection.new_separate(gate, up)
+    x = torch.from_numpy(oracle.randn(513, (3, k)))
+    assert torch.equal(proj.forward_silu_mul(x), proj.forward_silu_mul(x.cuda()).cpu())       # host pointers
+    # Qwen3Mlp: down(silu(gate x) * up x); inner width 256 here needs its own gate / up
+    g2 = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, make_weight(oracle, Q4_K, 256, k, 514), (256, k)))
+    u2 = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, make_weight(oracle, Q4_K, 256, k, 515), (256, k)))
+    down = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, wd, (k, 256)))
+    mlp = qa.Qwen3Mlp(qa.Qwen3GateUpProjection.new_separate(g2, u2), down)
+    xc = x.cuda()
+    y = mlp.forward(xc)
+    assert torch.equal(y, down.forward(qa.Qwen3GateUpProjection.new_separate(g2, u2).forward_silu_mul(xc)))
+    assert y.shape == (3, k)
+    # shape and type mismatches are errors
+    with pytest.raises(qa.QmmError, match="gate is"):
+        qa.Qwen3GateUpProjection.new_separate(gate, g2).forward_silu_mul(xc)
+    q8 = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q8_0, make_weight(oracle, Q8_0, n, k, 516), (n, k)))
+    with pytest.raises(qa.QmmError, match="different ggml dtypes"):
+        qa.Qwen3GateUpProjection.new_separate(gate, q8).forward_silu_mul(xc)
+    with pytest.raises(qa.QmmError, match="shape mismatch"):
+        proj.forward_silu_mul(torch.zeros((1, 256), device="cuda"))
