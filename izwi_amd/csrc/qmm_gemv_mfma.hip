@@ -30,6 +30,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdlib>
 
 #include "qmm_internal.h"
 
@@ -577,6 +578,161 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
     }
 }
 
+// Register-direct form (Q4_K, one row tile of activations, one row-tile of weights per
+// workgroup): wave wk multiplies panel wk, which needs only units 4 wk .. 4 wk + 3 of the
+// activations, and no other wave of the workgroup needs them.  Staging them in LDS would buy no
+// reuse and cost a barrier, so every lane loads its share of the MFMA A operands (and the
+// units' side information) straight into registers, ahead of the panel: no LDS, no barrier
+// before the arithmetic, and k of any length (the LDS forms need several windows from 32
+// units on).  Returns acc[r] for activation rows 4 grp + r.
+__device__ __forceinline__ void panel_dot_direct_q4k(WPanel<QMM_Q4_K>& p, const long (&a)[4][8],
+                                                     const long (&bs_lo)[4], const long (&bs_hi)[4],
+                                                     const float4 (&dx)[4], int n_units, float (&acc)[4]) {
+    uint32_t sc_lo[4], sc_hi[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        sc_lo[u] = p.hdr[u].y & 0x3f3f3f3fu;
+        sc_hi[u] = (p.hdr[u].w & 0x0f0f0f0fu) | (((p.hdr[u].y >> 6) & 0x03030303u) << 4);
+    }
+    int isum[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) isum[u][r] = 0;
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const u32x4 qq = p.q[2 * b + h];
+            i32x4 dlo[2], dhi[2];
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int u = 2 * h + e;
+                if (u >= n_units) continue; // uniform
+                const uint32_t w0 = e ? qq.z : qq.x, w1 = e ? qq.w : qq.y;
+                dlo[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[u][2 * b], pack64(w0 & kNib, w1 & kNib),
+                                                               i32x4{0, 0, 0, 0}, 0, 0, 0);
+                dhi[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[u][2 * b + 1], pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib),
+                                                               i32x4{0, 0, 0, 0}, 0, 0, 0);
+            }
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int u = 2 * h + e;
+                if (u >= n_units) continue;
+                const int sc0 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b);
+                const int sc1 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b + 1);
+#pragma unroll
+                for (int r = 0; r < 4; r++) isum[u][r] += __mul24(sc0, dlo[e][r]) + __mul24(sc1, dhi[e][r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        if (u >= n_units) continue;
+        const float d = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x & 0xffffu));
+        const float dmin = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x >> 16));
+        const uint32_t mn_lo = p.hdr[u].z & 0x3f3f3f3fu;
+        const uint32_t mn_hi = ((p.hdr[u].w >> 4) & 0x0f0f0f0fu) | (((p.hdr[u].z >> 6) & 0x03030303u) << 4);
+        const long bmn = pack64(mn_lo, mn_hi);
+        const i32x4 m_lo = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_lo[u], bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
+        const i32x4 m_hi = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_hi[u], bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
+        const float dxs[4] = {dx[u].x, dx[u].y, dx[u].z, dx[u].w};
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int msum = m_lo[r] + (m_hi[r] << 7);
+            acc[r] += (d * dxs[r]) * (float)isum[u][r] - (dmin * dxs[r]) * (float)msum;
+        }
+    }
+}
+
+__global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(MfmaParams P) {
+    constexpr int QT = QMM_Q4_K;
+    constexpr int UB = Unit<QT>::kBytes;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    float* lds_red = reinterpret_cast<float*>(smem); // the sums of the k-split: waves * 256 floats
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wr = (wave * P.wave_magic) >> 16;
+    const int wk = wave - wr * P.nwk;
+    const int j = lane & 15, grp = lane >> 4;
+    const int s_units = P.slots >> 4;
+    const uint8_t* wbase = P.w;
+    float* yout = P.y;
+    int n_rows = P.n, row_tiles = P.row_tiles, rtg = blockIdx.x;
+    if (P.n_weights > 1) {
+        int i = 0;
+        while (i + 1 < P.n_weights && (int)blockIdx.x >= P.rtg_end[i]) i++;
+        rtg = blockIdx.x - (i ? P.rtg_end[i - 1] : 0);
+        wbase = P.wv[i];
+        yout = P.yv[i];
+        n_rows = P.nv[i];
+        row_tiles = P.row_tiles_v[i];
+    }
+    const int rt = rtg * P.nwr + wr;
+    const bool rt_ok = rt < row_tiles;
+    const int unit0 = wk * s_units;
+    const int n_units = min(s_units, P.k_units - unit0); // uniform, >= 1
+    const int row = rt * 16 + j;
+
+    // the activations first (they come from the L2 and return first), then the panel
+    long a[4][8], bs_lo[4], bs_hi[4];
+    float4 dx[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const uint8_t* rec = P.ws + (size_t)(unit0 + (u < n_units ? u : 0)) * UB; // missing units re-read unit 0
+#pragma unroll
+        for (int sb = 0; sb < 8; sb++) a[u][sb] = *reinterpret_cast<const long*>(rec + sb * 512 + lane * 8);
+        const uint8_t* side = rec + Unit<QT>::kQuant;
+        // the sub-block sums occupy k slots 0..7 of the min-term MFMA: the first 16-lane row only
+        const long lo = *reinterpret_cast<const long*>(side + 64 + j * 16);
+        const long hi = *reinterpret_cast<const long*>(side + 64 + j * 16 + 8);
+        bs_lo[u] = grp == 0 ? lo : 0L;
+        bs_hi[u] = grp == 0 ? hi : 0L;
+        dx[u] = *reinterpret_cast<const float4*>(side + grp * 16);
+    }
+    WPanel<QT> p;
+    load_wpanel<QT>(p, wbase + (int64_t)((rt_ok ? rt : 0) * P.k_groups + wk) * P.panel_bytes, P.slots, lane, j);
+
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    panel_dot_direct_q4k(p, a, bs_lo, bs_hi, dx, n_units, acc);
+
+    // combine the waves that split k, write y[4 grp + r][rt * 16 + j]
+    if (P.nwk == 1) {
+        if (rt_ok && row < n_rows) {
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                if (grp * 4 + r < P.m) yout[(int64_t)(grp * 4 + r) * n_rows + row] = acc[r];
+        }
+        return;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; r++) lds_red[(wave * 4 + r) * 64 + lane] = acc[r];
+    lds_barrier();
+    if (wk == 0 && rt_ok && row < n_rows) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            float sum = 0.0f;
+            for (int w2 = 0; w2 < P.nwk; w2++) sum += lds_red[((wr * P.nwk + w2) * 4 + r) * 64 + lane];
+            if (grp * 4 + r < P.m) yout[(int64_t)(grp * 4 + r) * n_rows + row] = sum;
+        }
+    }
+}
+
+// One row tile of activations (m <= 16), one row-tile of weights per workgroup, Q4_K, and k
+// longer than one LDS window (measured on the 8B shapes at m = 16: 4096 x 12288 17.0 -> 15.4 us
+// per call; with k = 4096 the single-window LDS form is the faster one, 10.2 against 10.4 us
+// and 11.9 against 12.7 us for the q|k|v group).  IZWI_QMM_MFMA_DIRECT=0 keeps the LDS forms
+// (tuning aid).
+bool direct_form_applies(int dtype, int n_tiles, int nwr, bool one_window) {
+    static const bool enabled = [] {
+        const char* e = getenv("IZWI_QMM_MFMA_DIRECT");
+        return !(e && e[0] == '0');
+    }();
+    return enabled && dtype == QMM_Q4_K && n_tiles == 1 && nwr == 1 && !one_window;
+}
+
 // Streaming form: wave `wave` of workgroup b owns row-tiles (b * waves + wave),
 // + gridDim.x * waves, ... and walks all their panels; the activation window
 // stays in LDS meanwhile.  Windows that split k accumulate into y (the same
@@ -714,6 +870,10 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
         lds = window_bytes;
     }
     P.wave_magic = (65536 + P.nwk - 1) / P.nwk;
+    if (oneshot && direct_form_applies(L.dtype, n_tiles, P.nwr, L.k_units <= P.window_units)) {
+        gemv_mfma_direct_q4k_kernel<<<grid, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
+        return hipGetLastError();
+    }
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     const bool single = n_tiles == 1 && L.k_units <= P.window_units;
     const void* fn;
@@ -880,6 +1040,10 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
     }
     P.rt_groups = (int)groups;
     const int waves = P.nwk * P.nwr;
+    if (direct_form_applies(L0.dtype, 1, P.nwr, true)) {
+        gemv_mfma_direct_q4k_kernel<<<(unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
+        return hipGetLastError();
+    }
     const size_t lds = std::max((size_t)P.window_units * unit_bytes(L0.dtype), (size_t)waves * 256 * 4);
     if (lds > 160 * 1024) return hipErrorNotSupported;
     const void* fn = L0.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true>)

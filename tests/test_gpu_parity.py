@@ -159,7 +159,10 @@ def test_config3_lm_head_full_size(qa, oracle):
                                    # (streaming form, two activation windows, y accumulated per window),
                                    # several row tiles with one LDS window buffer, ragged row tiles
                                    (20, 16384, 5), (33, 12288, 40), (50, 3072, 17),
-                                   (40000, 1024, 9)])  # very tall: streaming form with a resident window
+                                   (40000, 1024, 9),  # very tall: streaming form with a resident window
+                                   # k longer than one window, one row tile of activations: the
+                                   # register-direct form (Q4_K), also with 3 units per panel
+                                   (100, 12288, 7), (4096, 12288, 16), (33, 9216, 3), (48, 8448, 5)])
 def test_ragged_shapes(qa, oracle, dtype, n, k, m):
     _say(f"ragged dtype={dtype} n={n} k={k} m={m}")
     blocks = make_weight(oracle, dtype, n, k, 60 + n)
