@@ -215,7 +215,7 @@ def cpu_baseline(oracle, dtype, m, budget_s=12.0):
     }
 
 
-def prefill_extra(torch, qa, oracle, dtype, m, steps=20, warmup=5):
+def prefill_extra(torch, qa, oracle, dtype, m, steps=20, warmup=5, only=None):
     """TFLOP/s of the prefill kernel per projection (extra report, not `value`):
     bf16 activations in HBM, bf16 output, called through the C ABI on preallocated buffers."""
     from izwi_amd import capi
@@ -224,6 +224,8 @@ def prefill_extra(torch, qa, oracle, dtype, m, steps=20, warmup=5):
     out = {}
     gg = qa.GgmlDType(dtype)
     for i, (name, n, k) in enumerate([LAYER_8B[0], LAYER_8B[1], LAYER_8B[4], LAYER_8B[6]]):
+        if only is not None and name != only:
+            continue
         mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, make_blocks(oracle, dtype, n, k, 1000 + i, 4096), (n, k)))
         x = torch.from_numpy(oracle.randn(3, (m, k))).cuda().to(torch.bfloat16)
         y = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
@@ -313,6 +315,9 @@ def main():
                     help="grouped: qkv_proj.forward(x) and gate_up_proj.forward(x) are one call each, as "
                          "the reference's attention and MLP blocks make them (4 calls per layer); "
                          "per-projection: seven izwi_qmm_forward_f32 calls per layer")
+    ap.add_argument("--prefill-only", default=None, choices=["q", "k", "gate", "down"],
+                    help="profiling aid: run only the prefill call of one 8B projection (--m rows, default "
+                         "2048 here; --steps calls) and print its TFLOP/s, nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -327,6 +332,13 @@ def main():
     torch.cuda.set_device(0)
     qa.lib()
     dtype = Q4_K if args.workload == "decode_q4k_8b_stack" else Q8_0
+
+    if args.prefill_only:
+        m = args.m if args.m > 1 else 2048
+        tf = prefill_extra(torch, qa, oracle, dtype, m, args.steps, args.warmup, only=args.prefill_only)
+        print(json.dumps({"prefill_only": args.prefill_only, "m": m, "dtype": "Q4_K" if dtype == Q4_K else "Q8_0",
+                          "tflops": tf[args.prefill_only]}))
+        return
 
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()

@@ -370,9 +370,10 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
         x_off[i] = (uint32_t)((min(m0 + row, P.m - 1) - m0) * P.k * 2 + kc * 16);
         x_lds[i] = row * kRowStride + kc * 16;
     }
-    // weights: thread t stages part t % TPR of row n0 + t / TPR; rows past the matrix read the
-    // last row-tile (their output columns are never stored)
-    const int w_row = tid / TPR, w_part = tid % TPR;
+    // weights: thread t stages part t / BN of row n0 + t % BN (the lanes of a wave write 64
+    // different rows of the padded LDS tile: no bank conflicts, and the part is wave-uniform);
+    // rows past the matrix read the last row-tile (their output columns are never stored)
+    const int w_row = tid % BN, w_part = tid / BN;
     const int64_t rt0 = n0 >> 4;
     const int64_t rowtile_bytes = (int64_t)P.k_groups * P.panel_bytes;
     const uint8_t* w_tile = P.w + rt0 * rowtile_bytes;
