@@ -244,7 +244,8 @@ def prefill_extra(torch, qa, oracle, dtype, m, steps=20, warmup=5, only=None):
 
 def moe_extra(torch, qa, oracle, steps=20, warmup=3):
     """One MoE layer (route + sort + grouped expert MLP + combine, HIP-graph replay) at the
-    Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, expert intermediate 768, Q4_K."""
+    Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, expert intermediate 768, Q4_K; as one
+    call and as the three calls it is composed of."""
     e, top_k, hidden, inter = 128, 8, 2048, 768
     gg = qa.GgmlDType(Q4_K)
 
@@ -261,16 +262,20 @@ def moe_extra(torch, qa, oracle, steps=20, warmup=3):
         logits_h = oracle.randn(50 + t, (t, e))
         logits = torch.from_numpy(logits_h).cuda()
 
-        def layer():
+        def three_calls():
             ids, wts = qa.moe_route(logits, top_k)
             perm, offsets = qa.moe_sort(ids, e)
             return experts.forward(x, ids, wts, perm, offsets)
 
-        us, g = time_graph(torch, layer, steps, warmup)
+        us3, g3 = time_graph(torch, three_calls, steps, warmup)
+        del g3
+        # the same layer as one call (izwi_moe_layer_f32): identical results
+        us, g = time_graph(torch, lambda: experts.layer(logits, x, top_k), steps, warmup)
         us *= 1e3
         ids_h, _ = oracle.moe_route(logits_h, top_k)
         distinct = len(set(ids_h.reshape(-1).tolist()))
-        rec = {"us": round(us, 1), "distinct_experts": distinct}
+        rec = {"us": round(us, 1), "us_route_sort_forward_as_three_calls": round(us3 * 1e3, 1),
+               "distinct_experts": distinct}
         # algorithmic bytes: the distinct experts' weights + x in + out; flops: 3 matmuls per pair
         rec["gbs"] = round((distinct * expert_bytes + 2 * t * hidden * 4) / us / 1e3, 1)
         rec["tflops"] = round(2.0 * t * top_k * 3 * hidden * inter / us / 1e6, 2)

@@ -218,6 +218,16 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
                          const int32_t* perm, const int32_t* offsets, float* out, int mem_space,
                          void* stream);
 
+/* One MoE layer in one call: izwi_moe_route, izwi_moe_sort and izwi_moe_forward_f32 composed
+ * (same results bit for bit).  logits `[t, n_experts]`, x and out `[t, hidden]`; ids_out /
+ * weights_out `[t, top_k]` receive the routing if not NULL.  Up to 1024 (token, slot) pairs and
+ * 256 experts, routing, sort and the kernel's segment tables are one launch (the layer is then 4
+ * launches instead of 8). */
+int izwi_moe_layer_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
+                       const izwi_qmm_weight* down, const float* logits, const float* x, int64_t t,
+                       int32_t top_k, float* out, int32_t* ids_out, float* weights_out,
+                       int mem_space, void* stream);
+
 /* --- profiling counters (IZWI_QWEN3_PROFILE, qwen3/core.rs:624-657) ------ */
 
 /* Enabled by izwi_qmm_profile_enable(1) or the IZWI_QWEN3_PROFILE env toggle.

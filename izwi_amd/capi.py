@@ -64,6 +64,7 @@ PROTOTYPES = {
     "izwi_qmm_quantize_activations": (C.c_int, [C.c_int, _vp, _i64, _i64, _vp, C.c_int, _vp]),
     "izwi_moe_route": (C.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, C.c_int, _vp]),
     "izwi_moe_sort": (C.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, C.c_int, _vp]),
+    "izwi_moe_layer_f32": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _vp, _vp, _vp, C.c_int, _vp]),
     "izwi_moe_forward_f32": (C.c_int, [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _vp, _vp,
                                        C.c_int, _vp]),
     "izwi_qmm_profile_enable": (C.c_int, [C.c_int]),

@@ -726,13 +726,10 @@ int izwi_moe_sort(const int32_t* ids, int64_t t, int32_t top_k, int32_t n_expert
     return IZWI_QMM_OK;
 }
 
-int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
-                         const izwi_qmm_weight* down, const float* x, int64_t t,
-                         const int32_t* ids, const float* weights, int32_t top_k,
-                         const int32_t* perm, const int32_t* offsets, float* out, int mem_space,
-                         void* stream_) {
+namespace {
+
+int moe_check_stacks(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_qmm_weight* down) {
     if (!gate || !up || !down) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
-    if (int rc = check_space(mem_space)) return rc;
     const QmmLayout& G = gate->layout;
     const QmmLayout& U = up->layout;
     const QmmLayout& D = down->layout;
@@ -741,24 +738,24 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
     if (D.n_stacked != G.n_stacked || D.k != G.n || D.n != G.k)
         return fail(IZWI_QMM_ERR_INVALID, "down stack [%lld, %lld] does not match gate/up [%lld, %lld]",
                     (long long)D.n, (long long)D.k, (long long)G.n, (long long)G.k);
-    if (t < 0 || top_k < 1) return fail(IZWI_QMM_ERR_INVALID, "bad t / top_k");
-    if (t == 0) return IZWI_QMM_OK;
-    if (!x || !ids || !weights || !perm || !offsets || !out)
-        return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    return IZWI_QMM_OK;
+}
+
+// The expert MLP on device buffers.  With `logits` the routing is computed here too (ids,
+// weights, perm, offsets are then ignored; ids_out / weights_out, if not NULL, receive it): for
+// small batches routing, sort and segment tables are ONE launch.
+int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_qmm_weight* down,
+             const float* x, int64_t t, int32_t top_k, const float* logits, const int32_t* ids,
+             const float* weights, const int32_t* perm, const int32_t* offsets, int32_t* ids_out,
+             float* weights_out, float* out, hipStream_t stream) {
+    const QmmLayout& G = gate->layout;
+    const QmmLayout& D = down->layout;
     const int64_t pairs = t * top_k;
     const int n_experts = (int)G.n_stacked;
     const int64_t hidden = G.k, inter = G.n;
     // every expert adds at most one partly filled segment
     const int64_t max_segments = pairs / QMM_MOE_SEG_ROWS + (pairs < n_experts ? pairs : n_experts);
-    hipStream_t stream = (hipStream_t)stream_;
     ProfileScope prof(nullptr, stream);
-    Staged xi, ii, wi, pi, oi, oo;
-    HIP_TRY(xi.in(x, (size_t)t * hidden * sizeof(float), mem_space));
-    HIP_TRY(ii.in(ids, (size_t)pairs * sizeof(int32_t), mem_space));
-    HIP_TRY(wi.in(weights, (size_t)pairs * sizeof(float), mem_space));
-    HIP_TRY(pi.in(perm, (size_t)pairs * sizeof(int32_t), mem_space));
-    HIP_TRY(oi.in(offsets, (size_t)(n_experts + 1) * sizeof(int32_t), mem_space));
-    HIP_TRY(oo.out(out, (size_t)t * hidden * sizeof(float), mem_space));
 
     // Many pairs per expert: 16-row tiles on the int8 matrix cores (the weights of an
     // expert are read once for all its pairs).  Few: 4-row segments on the dot4 kernel.
@@ -767,62 +764,144 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
     if (!tiles && max_segments > 65535)
         return fail(IZWI_QMM_ERR_UNSUPPORTED, "t * top_k = %lld is too large for one grouped launch", (long long)pairs);
     // workspace: h [pairs, inter] | y [pairs, hidden] | seg_offsets [E + 1]
-    //            (tiles: + u [pairs, inter] | activation records)
-    const size_t h_bytes = (size_t)pairs * inter * sizeof(float);
-    const size_t y_bytes = (size_t)pairs * hidden * sizeof(float);
-    const size_t s_bytes = (((size_t)(n_experts + 1) * sizeof(int32_t)) + 255) & ~(size_t)255;
+    //            | tiles: u [pairs, inter], activation records; else: seg_expert [max_segments]
+    //            | routing computed here: ids, weights, perm [pairs], offsets [E + 1], sort scratch
+    auto align256 = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t h_bytes = align256((size_t)pairs * inter * sizeof(float));
+    const size_t y_bytes = align256((size_t)pairs * hidden * sizeof(float));
+    const size_t s_bytes = align256((size_t)(n_experts + 1) * sizeof(int32_t));
     const int64_t max_tiles = pairs / QMM_MOE_TILE_ROWS + (pairs < n_experts ? pairs : n_experts);
     size_t r_bytes = 0;
     if (tiles) {
         const size_t r1 = qmm_moe_records_bytes(G.dtype, max_tiles, hidden);
         const size_t r2 = qmm_moe_records_bytes(D.dtype, max_tiles, inter);
-        r_bytes = r1 > r2 ? r1 : r2;
+        r_bytes = align256(r1 > r2 ? r1 : r2);
     }
+    const size_t mid_bytes = tiles ? h_bytes + r_bytes : align256((size_t)max_segments * 4);
+    const size_t p_bytes = align256((size_t)pairs * 4);
+    const size_t sort_bytes = align256((size_t)qmm_moe_sort_scratch_ints(pairs, n_experts) * sizeof(int32_t));
+    const size_t route_bytes = logits ? 3 * p_bytes + s_bytes + sort_bytes : 0;
     uint8_t* ws = nullptr;
-    HIP_TRY(get_scratch(gate->device, stream,
-                        h_bytes + y_bytes + s_bytes + (tiles ? h_bytes + r_bytes : (size_t)max_segments * 4),
-                        (void**)&ws));
+    HIP_TRY(get_scratch(gate->device, stream, h_bytes + y_bytes + s_bytes + mid_bytes + route_bytes, (void**)&ws));
     float* h = (float*)ws;
     float* y = (float*)(ws + h_bytes);
     int32_t* seg = (int32_t*)(ws + h_bytes + y_bytes);
-    hipError_t e;
+    uint8_t* mid = ws + h_bytes + y_bytes + s_bytes;
+    int32_t* seg_expert = (int32_t*)mid; // 4-row segment path only
+    bool segments_ready = false;
+    hipError_t e = hipSuccess;
+    if (logits) {
+        uint8_t* r = mid + mid_bytes;
+        int32_t* r_ids = (int32_t*)r;
+        float* r_w = (float*)(r + p_bytes);
+        int32_t* r_perm = (int32_t*)(r + 2 * p_bytes);
+        int32_t* r_off = (int32_t*)(r + 3 * p_bytes);
+        int32_t* r_sort = (int32_t*)(r + 3 * p_bytes + s_bytes);
+        if (!tiles && qmm_moe_plan_small_supported(t, n_experts, top_k)) {
+            e = qmm_launch_moe_plan_small(logits, t, n_experts, top_k, QMM_MOE_SEG_ROWS, max_segments, r_ids, r_w,
+                                          r_perm, r_off, seg, seg_expert, stream);
+            segments_ready = true;
+        } else {
+            e = qmm_launch_moe_route(logits, t, n_experts, top_k, r_ids, r_w, stream);
+            if (e == hipSuccess) e = qmm_launch_moe_sort(r_ids, pairs, n_experts, r_perm, r_off, nullptr, r_sort, stream);
+        }
+        if (e != hipSuccess) return fail_hip(e, "routing kernels");
+        if (ids_out) HIP_TRY(hipMemcpyAsync(ids_out, r_ids, (size_t)pairs * 4, hipMemcpyDeviceToDevice, stream));
+        if (weights_out) HIP_TRY(hipMemcpyAsync(weights_out, r_w, (size_t)pairs * 4, hipMemcpyDeviceToDevice, stream));
+        ids = r_ids, weights = r_w, perm = r_perm, offsets = r_off;
+    }
     if (tiles) {
-        float* u = (float*)(ws + h_bytes + y_bytes + s_bytes);
-        void* records = ws + h_bytes + y_bytes + s_bytes + h_bytes;
-        const int32_t* pm = (const int32_t*)pi.dev;
-        const int32_t* of = (const int32_t*)oi.dev;
-        e = qmm_launch_moe_segments(of, n_experts, QMM_MOE_TILE_ROWS, seg, nullptr, 0, stream);
+        float* u = (float*)mid;
+        void* records = mid + h_bytes;
+        e = qmm_launch_moe_segments(offsets, n_experts, QMM_MOE_TILE_ROWS, seg, nullptr, 0, stream);
         if (e == hipSuccess)
-            e = qmm_launch_quantize_grouped(G.dtype, (const float*)xi.dev, nullptr, top_k, hidden, pm, of, seg,
-                                            n_experts, max_tiles, records, stream);
+            e = qmm_launch_quantize_grouped(G.dtype, x, nullptr, top_k, hidden, perm, offsets, seg, n_experts,
+                                            max_tiles, records, stream);
         if (e == hipSuccess)
-            e = qmm_launch_gemv_mfma_grouped(G, gate->tiled, up->tiled, records, h, u, pm, of, seg, n_experts,
+            e = qmm_launch_gemv_mfma_grouped(G, gate->tiled, up->tiled, records, h, u, perm, offsets, seg, n_experts,
                                              stream);
         // silu(gate) * up is applied while the down projection's input is quantized
         if (e == hipSuccess)
-            e = qmm_launch_quantize_grouped(D.dtype, h, u, 1, inter, pm, of, seg, n_experts, max_tiles,
+            e = qmm_launch_quantize_grouped(D.dtype, h, u, 1, inter, perm, offsets, seg, n_experts, max_tiles,
                                             records, stream);
         if (e == hipSuccess)
-            e = qmm_launch_gemv_mfma_grouped(D, down->tiled, nullptr, records, y, nullptr, pm, of, seg,
+            e = qmm_launch_gemv_mfma_grouped(D, down->tiled, nullptr, records, y, nullptr, perm, offsets, seg,
                                              n_experts, stream);
     } else {
-        int32_t* seg_expert = (int32_t*)(ws + h_bytes + y_bytes + s_bytes);
-        e = qmm_launch_moe_segments((const int32_t*)oi.dev, n_experts, QMM_MOE_SEG_ROWS, seg, seg_expert,
-                                    max_segments, stream);
+        if (!segments_ready)
+            e = qmm_launch_moe_segments(offsets, n_experts, QMM_MOE_SEG_ROWS, seg, seg_expert, max_segments, stream);
         if (e == hipSuccess)
-            e = qmm_launch_gemv_grouped(G, gate->tiled, up->tiled, (const float*)xi.dev, top_k, h,
-                                        (const int32_t*)pi.dev, (const int32_t*)oi.dev, seg, seg_expert,
+            e = qmm_launch_gemv_grouped(G, gate->tiled, up->tiled, x, top_k, h, perm, offsets, seg, seg_expert,
                                         n_experts, max_segments, gate->n_cus, stream);
         if (e == hipSuccess)
-            e = qmm_launch_gemv_grouped(D, down->tiled, nullptr, h, 1, y, (const int32_t*)pi.dev,
-                                        (const int32_t*)oi.dev, seg, seg_expert, n_experts, max_segments,
-                                        gate->n_cus, stream);
+            e = qmm_launch_gemv_grouped(D, down->tiled, nullptr, h, 1, y, perm, offsets, seg, seg_expert, n_experts,
+                                        max_segments, gate->n_cus, stream);
     }
-    if (e == hipSuccess)
-        e = qmm_launch_moe_combine(y, (const float*)wi.dev, t, top_k, hidden, (float*)oo.dev, stream);
+    if (e == hipSuccess) e = qmm_launch_moe_combine(y, weights, t, top_k, hidden, out, stream);
     if (e != hipSuccess) return fail_hip(e, "grouped expert kernels");
     if (profiling()) g_silu_fused.fetch_add(1, std::memory_order_relaxed);
+    return IZWI_QMM_OK;
+}
+
+} // namespace
+
+int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
+                         const izwi_qmm_weight* down, const float* x, int64_t t,
+                         const int32_t* ids, const float* weights, int32_t top_k,
+                         const int32_t* perm, const int32_t* offsets, float* out, int mem_space,
+                         void* stream_) {
+    if (int rc = moe_check_stacks(gate, up, down)) return rc;
+    if (int rc = check_space(mem_space)) return rc;
+    if (t < 0 || top_k < 1) return fail(IZWI_QMM_ERR_INVALID, "bad t / top_k");
+    if (t == 0) return IZWI_QMM_OK;
+    if (!x || !ids || !weights || !perm || !offsets || !out)
+        return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    const int64_t pairs = t * top_k;
+    const int n_experts = (int)gate->layout.n_stacked;
+    const int64_t hidden = gate->layout.k;
+    hipStream_t stream = (hipStream_t)stream_;
+    Staged xi, ii, wi, pi, oi, oo;
+    HIP_TRY(xi.in(x, (size_t)t * hidden * sizeof(float), mem_space));
+    HIP_TRY(ii.in(ids, (size_t)pairs * sizeof(int32_t), mem_space));
+    HIP_TRY(wi.in(weights, (size_t)pairs * sizeof(float), mem_space));
+    HIP_TRY(pi.in(perm, (size_t)pairs * sizeof(int32_t), mem_space));
+    HIP_TRY(oi.in(offsets, (size_t)(n_experts + 1) * sizeof(int32_t), mem_space));
+    HIP_TRY(oo.out(out, (size_t)t * hidden * sizeof(float), mem_space));
+    if (int rc = moe_core(gate, up, down, (const float*)xi.dev, t, top_k, nullptr, (const int32_t*)ii.dev,
+                          (const float*)wi.dev, (const int32_t*)pi.dev, (const int32_t*)oi.dev, nullptr, nullptr,
+                          (float*)oo.dev, stream))
+        return rc;
     HIP_TRY(oo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_moe_layer_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_qmm_weight* down,
+                       const float* logits, const float* x, int64_t t, int32_t top_k, float* out,
+                       int32_t* ids_out, float* weights_out, int mem_space, void* stream_) {
+    if (int rc = moe_check_stacks(gate, up, down)) return rc;
+    if (int rc = check_space(mem_space)) return rc;
+    const int n_experts = (int)gate->layout.n_stacked;
+    if (t < 0) return fail(IZWI_QMM_ERR_INVALID, "negative t");
+    if (n_experts > 1024) return fail(IZWI_QMM_ERR_UNSUPPORTED, "n_experts = %d outside 1..1024", n_experts);
+    if (top_k < 1 || top_k > n_experts || top_k > 64)
+        return fail(IZWI_QMM_ERR_INVALID, "top_k = %d outside 1..min(n_experts, 64)", top_k);
+    if (t == 0) return IZWI_QMM_OK;
+    if (t * (int64_t)top_k > 0x7fffffff) return fail(IZWI_QMM_ERR_UNSUPPORTED, "too many pairs");
+    if (!logits || !x || !out) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    const int64_t pairs = t * top_k, hidden = gate->layout.k;
+    hipStream_t stream = (hipStream_t)stream_;
+    Staged li, xi, oo, io, wo;
+    HIP_TRY(li.in(logits, (size_t)t * n_experts * sizeof(float), mem_space));
+    HIP_TRY(xi.in(x, (size_t)t * hidden * sizeof(float), mem_space));
+    HIP_TRY(oo.out(out, (size_t)t * hidden * sizeof(float), mem_space));
+    if (ids_out) HIP_TRY(io.out(ids_out, (size_t)pairs * sizeof(int32_t), mem_space));
+    if (weights_out) HIP_TRY(wo.out(weights_out, (size_t)pairs * sizeof(float), mem_space));
+    if (int rc = moe_core(gate, up, down, (const float*)xi.dev, t, top_k, (const float*)li.dev, nullptr, nullptr,
+                          nullptr, nullptr, (int32_t*)io.dev, (float*)wo.dev, (float*)oo.dev, stream))
+        return rc;
+    HIP_TRY(oo.finish(stream));
+    if (ids_out) HIP_TRY(io.finish(stream));
+    if (weights_out) HIP_TRY(wo.finish(stream));
     return IZWI_QMM_OK;
 }
 

@@ -173,6 +173,14 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
                                         const int32_t* offsets, const int32_t* tile_offsets,
                                         int n_experts, hipStream_t stream);
 
+// Small batches: routing, sort and the segment tables (seg_rows rows per segment) of the grouped
+// decode kernel in one launch; same results as route + sort + segments.
+bool qmm_moe_plan_small_supported(int64_t t, int n_experts, int top_k);
+hipError_t qmm_launch_moe_plan_small(const float* logits, int64_t t, int n_experts, int top_k, int seg_rows,
+                                     int64_t max_segments, int32_t* ids, float* weights, int32_t* perm,
+                                     int32_t* offsets, int32_t* seg_offsets, int32_t* seg_expert,
+                                     hipStream_t stream);
+
 // out[t, :] = sum over slots s (in order) of weights[t, s] * y[t * top_k + s, :]
 hipError_t qmm_launch_moe_combine(const float* y, const float* weights, int64_t t, int top_k,
                                   int64_t hidden, float* out, hipStream_t stream);

@@ -223,6 +223,65 @@ __global__ void segments_kernel(const int32_t* __restrict__ offsets, int n_exper
         for (int s = total + threadIdx.x; s < max_segments; s += 256) seg_expert[s] = -1;
 }
 
+// Small batches (t * top_k <= kPlanMaxPairs): routing, stable counting sort and the segment tables
+// of the grouped decode kernel in ONE workgroup and launch.  Results equal route_kernel +
+// sort_* + segments_kernel bit for bit (same routing function, integer-only sort).
+constexpr int kPlanMaxPairs = 1024, kPlanMaxExperts = 256, kPlanThreads = 256;
+template <int PER_LANE>
+__global__ __launch_bounds__(kPlanThreads) void moe_plan_small_kernel(
+    const float* __restrict__ logits, int t, int n_experts, int top_k, int max_segments,
+    int32_t* __restrict__ ids, float* __restrict__ weights, int32_t* __restrict__ perm,
+    int32_t* __restrict__ offsets, int32_t* __restrict__ seg_offsets, int32_t* __restrict__ seg_expert) {
+    __shared__ int32_t s_ids[kPlanMaxPairs];
+    __shared__ int32_t s_count[kPlanMaxExperts], s_start[kPlanMaxExperts];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = kPlanThreads / 64;
+    const int pairs = t * top_k;
+    constexpr int seg_rows = QMM_MOE_SEG_ROWS; // a constant: the divisions below are shifts
+    for (int e = threadIdx.x; e < n_experts; e += kPlanThreads) s_count[e] = 0;
+    // 1. routing: one wave per token
+    for (int tok = wave; tok < t; tok += waves) {
+        int id;
+        float w;
+        route_token<PER_LANE>(logits + (int64_t)tok * n_experts, n_experts, top_k, lane, id, w);
+        if (lane < top_k) {
+            ids[tok * top_k + lane] = id;
+            weights[tok * top_k + lane] = w;
+            s_ids[tok * top_k + lane] = id;
+        }
+    }
+    __syncthreads();
+    // 2. per-expert counts (integer adds: order-free)
+    for (int p = threadIdx.x; p < pairs; p += kPlanThreads) atomicAdd(&s_count[s_ids[p]], 1);
+    __syncthreads();
+    // 3. exclusive prefix sums of the counts and of the segment counts: thread e sums what lies
+    //    before expert e (LDS broadcast reads)
+    for (int e = threadIdx.x; e <= n_experts; e += kPlanThreads) {
+        int32_t run = 0, seg = 0;
+        for (int i = 0; i < e; i++) {
+            const int32_t c = s_count[i];
+            run += c;
+            seg += (c + seg_rows - 1) / seg_rows;
+        }
+        offsets[e] = run;
+        seg_offsets[e] = seg;
+        if (e < n_experts) {
+            s_start[e] = run;
+            const int32_t n = (s_count[e] + seg_rows - 1) / seg_rows;
+            for (int32_t i = 0; i < n && seg + i < max_segments; i++) seg_expert[seg + i] = e;
+        } else {
+            for (int sidx = seg; sidx < max_segments; sidx++) seg_expert[sidx] = -1; // past the last segment
+        }
+    }
+    __syncthreads();
+    // 4. stable scatter: pair p goes behind the earlier pairs of its expert
+    for (int p = threadIdx.x; p < pairs; p += kPlanThreads) {
+        const int32_t e = s_ids[p];
+        int32_t rank = 0;
+        for (int q = 0; q < p; q++) rank += s_ids[q] == e;
+        perm[s_start[e] + rank] = p;
+    }
+}
+
 __global__ void combine_kernel(const float* __restrict__ y, const float* __restrict__ weights,
                                int64_t t, int top_k, int64_t hidden, float* __restrict__ out) {
     int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -279,6 +338,25 @@ hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int se
                                    hipStream_t stream) {
     segments_kernel<<<1, 256, 0, stream>>>(offsets, n_experts, seg_rows, seg_offsets, seg_expert,
                                            (int)max_segments);
+    return hipGetLastError();
+}
+
+bool qmm_moe_plan_small_supported(int64_t t, int n_experts, int top_k) {
+    return t > 0 && t * top_k <= kPlanMaxPairs && n_experts <= kPlanMaxExperts && top_k <= 64 && top_k <= n_experts;
+}
+
+hipError_t qmm_launch_moe_plan_small(const float* logits, int64_t t, int n_experts, int top_k, int seg_rows,
+                                     int64_t max_segments, int32_t* ids, float* weights, int32_t* perm,
+                                     int32_t* offsets, int32_t* seg_offsets, int32_t* seg_expert,
+                                     hipStream_t stream) {
+    if (!qmm_moe_plan_small_supported(t, n_experts, top_k) || max_segments > 0x7fffffff || seg_rows != QMM_MOE_SEG_ROWS)
+        return hipErrorInvalidValue;
+    if (n_experts <= 128)
+        moe_plan_small_kernel<2><<<1, kPlanThreads, 0, stream>>>(logits, (int)t, n_experts, top_k, (int)max_segments,
+                                                                 ids, weights, perm, offsets, seg_offsets, seg_expert);
+    else
+        moe_plan_small_kernel<4><<<1, kPlanThreads, 0, stream>>>(logits, (int)t, n_experts, top_k, (int)max_segments,
+                                                                 ids, weights, perm, offsets, seg_offsets, seg_expert);
     return hipGetLastError();
 }
 

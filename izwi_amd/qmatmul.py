@@ -354,6 +354,22 @@ class MoeExperts:
                                          offsets.data_ptr(), out.data_ptr(), _space(x), _stream_ptr(x)))
         return out
 
+    def layer(self, logits: torch.Tensor, x: torch.Tensor, top_k: int, return_routing: bool = False):
+        """Route, sort, expert MLP and combine in one call (izwi_moe_layer_f32): the same results
+        as moe_route + moe_sort + forward."""
+        assert x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2
+        assert logits.dtype == torch.float32 and logits.is_contiguous() and logits.shape[0] == x.shape[0]
+        t = x.shape[0]
+        out = torch.empty_like(x)
+        ids = wts = None
+        if return_routing:
+            ids = torch.empty((t, top_k), dtype=torch.int32, device=x.device)
+            wts = torch.empty((t, top_k), dtype=torch.float32, device=x.device)
+        check(lib().izwi_moe_layer_f32(self.gate._h, self.up._h, self.down._h, logits.data_ptr(), x.data_ptr(), t,
+                                       top_k, out.data_ptr(), ids.data_ptr() if return_routing else None,
+                                       wts.data_ptr() if return_routing else None, _space(x), _stream_ptr(x)))
+        return (out, ids, wts) if return_routing else out
+
 
 def profile_snapshot() -> dict:
     snap = capi.ProfileSnapshot()

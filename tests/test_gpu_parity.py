@@ -364,6 +364,40 @@ def test_config5_moe_forward(qa, oracle, moe_weights, t):
     assert np.isfinite(out).all()
 
 
+@pytest.mark.parametrize("t", [1, 3, 16, 100, 128, 129, 512])
+def test_config5_moe_layer_one_call_equals_the_three_calls(qa, oracle, moe_weights, t):
+    """izwi_moe_layer_f32 = route + sort + forward, bit for bit (ids, weights, outputs): up to
+    1024 pairs routing, sort and segment tables come from one launch, beyond from the
+    separate kernels."""
+    _say(f"moe layer t={t}")
+    E, hidden, inter, gate, up, down = moe_weights
+    dt = qa.GgmlDType.Q4K
+    experts = qa.MoeExperts(qa.QTensor.from_blocks(dt, gate, (E, inter, hidden)),
+                            qa.QTensor.from_blocks(dt, up, (E, inter, hidden)),
+                            qa.QTensor.from_blocks(dt, down, (E, hidden, inter)))
+    x = torch.from_numpy(oracle.randn(290 + t, (t, hidden))).cuda()
+    logits_h = oracle.randn(291 + t, (t, E))
+    if t >= 3:  # ties, an infinity and a NaN in the logits of some tokens
+        logits_h[1, 5] = logits_h[1, 77] = logits_h[1].max() + 1.0
+        logits_h[2, 9] = np.inf
+        logits_h[2, 100] = np.nan
+        logits_h[0, :] = 0.25
+    logits = torch.from_numpy(logits_h).cuda()
+    ids, wts = qa.moe_route(logits, 8)
+    perm, offsets = qa.moe_sort(ids, E)
+    want = experts.forward(x, ids, wts, perm, offsets)
+    out, ids2, wts2 = experts.layer(logits, x, 8, return_routing=True)
+    assert torch.equal(ids2, ids)
+    assert torch.equal(wts2.view(torch.int32), wts.view(torch.int32))
+    assert torch.equal(out.view(torch.int32), want.view(torch.int32))
+    assert torch.equal(experts.layer(logits, x, 8).view(torch.int32), want.view(torch.int32))
+    want_ids, _ = oracle.moe_route(logits_h, 8)
+    assert np.array_equal(ids2.cpu().numpy(), want_ids)
+    if t <= 16:  # host pointers
+        out_h = experts.layer(logits.cpu(), x.cpu(), 8)
+        assert torch.equal(out_h.view(torch.int32), want.cpu().view(torch.int32))
+
+
 @pytest.mark.parametrize("dtype,E,hidden,inter,t,top_k", [
     (Q8_0, 8, 512, 256, 64, 4),     # 32 pairs per expert: matrix-core tiles, Q8_0, one unit per panel
     (Q4_K, 4, 1280, 768, 40, 2),    # ragged k (5 units), three-unit panels on the way down
