@@ -118,8 +118,9 @@ int izwi_gguf_load_packed(const izwi_gguf* g, const char* const* names, int32_t 
 
 /* `load_tensor(name, DType::F32, device)` (gguf.rs:127-144): the tensor as dense f32 in row-major
  * order, `count` = number of elements `out` holds (must equal the tensor's element count).  F32 is
- * copied, F16 / BF16 converted, Q8_0 / Q4_K dequantized bit-exactly as candle-core's `to_float`;
- * conversion runs on the device (`mem_space` says where `out` lives). */
+ * copied, F16 / BF16 converted, Q8_0 / Q4_K / Q6_K dequantized bit-exactly as candle-core's
+ * `to_float` (Q6_K, which Q4_K_M files use for some tensors, is a load-time codec only: it has no
+ * weight handle); conversion runs on the device (`mem_space` says where `out` lives). */
 int izwi_gguf_load_tensor_f32(const izwi_gguf* g, const char* name, float* out, uint64_t count,
                               int mem_space, void* stream);
 

@@ -214,6 +214,31 @@ __global__ void half_to_f32_kernel(const uint16_t* __restrict__ in, float* __res
     out[i] = is_bf16 ? qmm_bf16_bits_to_f32(in[i]) : qmm_f16_bits_to_f32(in[i]);
 }
 
+// Q6_K blocks in their file layout (ql[128], qh[64], int8 scales[16], f16 d: 210 B per 256
+// elements) -> f32, as candle-core's `BlockQ6K::to_float`: y = d * scale * (q - 32), evaluated
+// left to right (the library is built without floating-point contraction).  One thread per
+// (block, half, l): the four elements l, l + 32, l + 64, l + 96 of a half of 128.
+__global__ void dequant_q6k_kernel(const uint8_t* __restrict__ blocks, float* __restrict__ out, uint64_t n_blocks) {
+    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t blk = idx >> 6;
+    if (blk >= n_blocks) return;
+    const int half = (int)(idx >> 5) & 1, l = (int)idx & 31, is = l >> 4;
+    const uint8_t* b = blocks + blk * 210;
+    const uint8_t* ql = b + 64 * half;
+    const uint8_t qh = b[128 + 32 * half + l];
+    const int8_t* sc = reinterpret_cast<const int8_t*>(b + 192) + 8 * half;
+    const float d = qmm_f16_bits_to_f32((uint16_t)(b[208] | (b[209] << 8)));
+    const int q1 = (int)((ql[l] & 0xF) | ((qh & 3) << 4)) - 32;
+    const int q2 = (int)((ql[l + 32] & 0xF) | (((qh >> 2) & 3) << 4)) - 32;
+    const int q3 = (int)((ql[l] >> 4) | (((qh >> 4) & 3) << 4)) - 32;
+    const int q4 = (int)((ql[l + 32] >> 4) | (((qh >> 6) & 3) << 4)) - 32;
+    float* y = out + blk * 256 + 128 * half;
+    y[l] = d * (float)sc[is] * (float)q1;
+    y[l + 32] = d * (float)sc[is + 2] * (float)q2;
+    y[l + 64] = d * (float)sc[is + 4] * (float)q3;
+    y[l + 96] = d * (float)sc[is + 6] * (float)q4;
+}
+
 struct DeviceBuffer {
     void* p = nullptr;
     ~DeviceBuffer() {
@@ -522,6 +547,7 @@ int izwi_gguf_load_tensor_f32(const izwi_gguf* g, const char* name, float* out, 
         return e == hipSuccess ? IZWI_QMM_OK : hip_fail(e, "copy to the device");
     }
     case 1:    // F16
+    case 14:   // Q6_K (dense load only: not a matmul type of this library)
     case 30: { // BF16
         DeviceBuffer raw, tmp;
         hipError_t e = hipMalloc(&raw.p, (size_t)ti.nbytes);
@@ -536,8 +562,12 @@ int izwi_gguf_load_tensor_f32(const izwi_gguf* g, const char* name, float* out, 
         }
         const uint64_t grid = ((uint64_t)elems + 255) / 256;
         if (grid > 0x7fffffffu) return qmm_fail(IZWI_QMM_ERR_UNSUPPORTED, "tensor '%s' is too large to convert", name);
-        half_to_f32_kernel<<<(unsigned)grid, 256, 0, stream>>>(static_cast<const uint16_t*>(raw.p), dst,
-                                                              (uint64_t)elems, ti.ggml_dtype == 30);
+        if (ti.ggml_dtype == 14) // 64 threads per block of 256 elements
+            dequant_q6k_kernel<<<(unsigned)(((uint64_t)elems / 4 + 255) / 256), 256, 0, stream>>>(
+                static_cast<const uint8_t*>(raw.p), dst, (uint64_t)elems / 256);
+        else
+            half_to_f32_kernel<<<(unsigned)grid, 256, 0, stream>>>(static_cast<const uint16_t*>(raw.p), dst,
+                                                                  (uint64_t)elems, ti.ggml_dtype == 30);
         e = hipGetLastError();
         if (e == hipSuccess) e = hipStreamSynchronize(stream); // `raw` is freed on return
         if (e != hipSuccess) return hip_fail(e, "conversion kernel");
@@ -564,7 +594,7 @@ int izwi_gguf_load_tensor_f32(const izwi_gguf* g, const char* name, float* out, 
     }
     default:
         return qmm_fail(IZWI_QMM_ERR_UNSUPPORTED,
-                        "Failed to dequantize tensor '%s': ggml dtype %d is not supported (F32, F16, BF16, Q8_0, Q4_K)",
+                        "Failed to dequantize tensor '%s': ggml dtype %d is not supported (F32, F16, BF16, Q8_0, Q4_K, Q6_K)",
                         name, ti.ggml_dtype);
     }
 }

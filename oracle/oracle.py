@@ -17,8 +17,9 @@ _LIB_PATH = os.path.join(_HERE, "liboracle_qmm.so")
 
 GGML_Q8_0 = 8
 GGML_Q4_K = 12
-BLOCK_SIZE = {GGML_Q8_0: 32, GGML_Q4_K: 256}
-TYPE_SIZE = {GGML_Q8_0: 34, GGML_Q4_K: 144}
+GGML_Q6_K = 14  # dequantize only (GGUF ingress to dense f32)
+BLOCK_SIZE = {GGML_Q8_0: 32, GGML_Q4_K: 256, GGML_Q6_K: 256}
+TYPE_SIZE = {GGML_Q8_0: 34, GGML_Q4_K: 144, GGML_Q6_K: 210}
 # activation-side ("vec dot") block of each weight type
 ACT_BLOCK_SIZE = {GGML_Q8_0: 32, GGML_Q4_K: 256}
 ACT_TYPE_SIZE = {GGML_Q8_0: 34, GGML_Q4_K: 292}

@@ -59,6 +59,14 @@ typedef struct {
     int16_t bsums[QK_K / 16];
 } __attribute__((packed)) block_q8_k; /* 292 bytes */
 
+typedef struct {
+    uint8_t ql[QK_K / 2];     /* low 4 bits of the 6-bit quants */
+    uint8_t qh[QK_K / 4];     /* high 2 bits */
+    int8_t scales[QK_K / 16]; /* one 8-bit scale per 16 elements */
+    uint16_t d;               /* f16 bits, super-block scale */
+} __attribute__((packed)) block_q6_k; /* 210 bytes */
+
+_Static_assert(sizeof(block_q6_k) == 210, "Q6_K block is 210 bytes");
 _Static_assert(sizeof(block_q8_0) == 34, "Q8_0 block is 34 bytes");
 _Static_assert(sizeof(block_q4_k) == 144, "Q4_K block is 144 bytes");
 _Static_assert(sizeof(block_q8_k) == 292, "Q8_K block is 292 bytes");
@@ -207,6 +215,35 @@ void oracle_dequantize_row_q4_k(const block_q4_k* x, float* y, int64_t k) {
             for (int l = 0; l < 32; l++) *yo++ = d2 * (float)(q[l] >> 4) - m2;
             q += 32;
             is += 2;
+        }
+    }
+}
+
+/* candle-core k_quants.rs, `BlockQ6K::to_float` (ggml `dequantize_row_q6_K`): per half of 128
+ * elements, byte l of ql / qh carries elements l, l+32 (low nibbles of ql[l], ql[l+32]) and l+64,
+ * l+96 (high nibbles); y = d * scale * (q - 32), evaluated left to right.  Load-time codec only
+ * (GGUF ingress to dense f32): Q6_K is not a matmul type of this library. */
+void oracle_dequantize_row_q6_k(const block_q6_k* x, float* y, int64_t k) {
+    int64_t nb = k / QK_K;
+    for (int64_t i = 0; i < nb; i++) {
+        const float d = oracle_f16_to_f32(x[i].d);
+        for (int n = 0; n < QK_K; n += 128) {
+            const int idx = n / 128;
+            float* yo = y + i * QK_K + n;
+            const int8_t* sc = x[i].scales + 8 * idx;
+            const uint8_t* ql = x[i].ql + 64 * idx;
+            const uint8_t* qh = x[i].qh + 32 * idx;
+            for (int l = 0; l < 32; l++) {
+                const int is = l / 16;
+                const int8_t q1 = (int8_t)((ql[l] & 0xF) | ((qh[l] & 3) << 4)) - 32;
+                const int8_t q2 = (int8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+                const int8_t q3 = (int8_t)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+                const int8_t q4 = (int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+                yo[l] = d * (float)sc[is] * (float)q1;
+                yo[l + 32] = d * (float)sc[is + 2] * (float)q2;
+                yo[l + 64] = d * (float)sc[is + 4] * (float)q3;
+                yo[l + 96] = d * (float)sc[is + 6] * (float)q4;
+            }
         }
     }
 }
@@ -406,11 +443,13 @@ float oracle_vec_dot_q4_k_q8_k(int64_t k, const block_q4_k* w, const block_q8_k*
 /* GGML dtype ids as the reference sees them (GgmlDType in candle-core mod.rs). */
 #define GGML_Q8_0 8
 #define GGML_Q4_K 12
+#define GGML_Q6_K 14 /* dequantize only */
 
 int64_t oracle_storage_bytes(int dtype, int64_t rows, int64_t cols) {
     int64_t elems = rows * cols;
     if (dtype == GGML_Q8_0) return elems % QK8_0 ? -1 : elems / QK8_0 * 34;
     if (dtype == GGML_Q4_K) return elems % QK_K ? -1 : elems / QK_K * 144;
+    if (dtype == GGML_Q6_K) return elems % QK_K ? -1 : elems / QK_K * 210;
     return -1;
 }
 
@@ -484,6 +523,14 @@ int oracle_dequantize(int dtype, int64_t rows, int64_t cols, const void* src, fl
 #pragma omp parallel for schedule(static)
         for (int64_t r = 0; r < rows; r++)
             oracle_dequantize_row_q4_k((const block_q4_k*)src + r * (cols / QK_K), dst + r * cols,
+                                       cols);
+        return 0;
+    }
+    if (dtype == GGML_Q6_K) {
+        if (cols % QK_K) return -1;
+#pragma omp parallel for schedule(static)
+        for (int64_t r = 0; r < rows; r++)
+            oracle_dequantize_row_q6_k((const block_q6_k*)src + r * (cols / QK_K), dst + r * cols,
                                        cols);
         return 0;
     }

@@ -13,6 +13,8 @@ that holds the arithmetic is not in its tree).  They restate, as data:
   bytes and the outputs of candle-core's algorithm on them, computed here with plain
   numpy arithmetic (no code of the oracle or of the library is used).
 
+* q6k_hand_block.json - one Q6_K block (a load-time codec: GGUF ingress to dense f32) built
+  the same way, all 256 values of y = d * scale * (q - 32) from per-element index arithmetic.
 * tiny.gguf + tiny_gguf.json - a small GGUF version 3 file assembled byte by byte from the
   public container format (no writer or reader of this repository is used), and what a
   reader must report for it; its Q4_K tensor is the hand block above.
@@ -98,6 +100,28 @@ def packed_case():
             "reference_tolerance_packed_vs_separate": 1e-5}
 
 
+def q6k_hand_block():
+    """One Q6_K block from the public block format (ql[128], qh[64], int8 scales[16], f16 d) with
+    every value of y = d * scale * (q - 32) worked out element by element."""
+    ql = bytes((7 * i + 3) % 256 for i in range(128))
+    qh = bytes((13 * i + 5) % 256 for i in range(64))
+    scales = [1, -2, 3, -4, 5, -6, 7, -8, 9, 10, -11, 12, 127, -128, 64, -1]
+    d = np.float16(0.25)
+    block = ql + qh + bytes(v & 0xFF for v in scales) + d.tobytes()
+    assert len(block) == 210
+    y = np.zeros(256, dtype=np.float64)
+    for e in range(256):
+        half, r = divmod(e, 128)      # which 128-element half
+        g, l = divmod(r, 32)          # group 0..3 inside the half, position 0..31
+        byte = ql[64 * half + 32 * (g % 2) + l]
+        low = (byte & 0xF) if g < 2 else (byte >> 4)
+        high = (qh[32 * half + l] >> (2 * g)) & 3
+        q = (low | (high << 4)) - 32
+        y[e] = 0.25 * scales[8 * half + 2 * g + l // 16] * q   # exact in f32: small integers times 2^-2
+    return {"ggml_dtype": 14, "rows": 1, "cols": 256, "block_hex": block.hex(), "scales": scales,
+            "expected_f32": [float(v) for v in y], "expected_sum": float(y.sum())}
+
+
 def tiny_gguf():
     """A GGUF version 3 file laid out by hand from the public container format: header, three
     metadata entries (alignment 64), three tensor infos, padding, data.  Returns the file's
@@ -140,7 +164,8 @@ if __name__ == "__main__":
     with open(os.path.join(HERE, "tiny_gguf.json"), "w") as f:
         json.dump(want, f, indent=1)
     print("wrote tiny.gguf, tiny_gguf.json")
-    for name, rec in (("q4k_hand_block.json", q4k_hand_block()), ("packed_q8_0_case.json", packed_case())):
+    for name, rec in (("q4k_hand_block.json", q4k_hand_block()), ("packed_q8_0_case.json", packed_case()),
+                      ("q6k_hand_block.json", q6k_hand_block())):
         with open(os.path.join(HERE, name), "w") as f:
             json.dump(rec, f, indent=1)
         print("wrote", name)

@@ -46,6 +46,26 @@ def dequant_q4_k(blocks: np.ndarray, rows: int, cols: int) -> np.ndarray:
     return y.astype(np.float32).reshape(rows, cols)
 
 
+def dequant_q6_k(blocks: np.ndarray, rows: int, cols: int) -> np.ndarray:
+    """Q6_K blocks (ql[128], qh[64], int8 scales[16], f16 d = 210 B) -> f32, vectorized from the
+    public block format: element 128 h + 32 g + l of a block has the quant
+    (nibble g % 2 of ql[64 h + 32 (g // 2)... see below) and scale index 8 h + 2 g + l // 16."""
+    b = np.ascontiguousarray(blocks, dtype=np.uint8).reshape(-1, 210)
+    ql = b[:, :128].reshape(-1, 2, 2, 32)           # [blk, half, which 32 bytes, l]
+    qh = b[:, 128:192].reshape(-1, 2, 32)           # [blk, half, l]
+    sc = b[:, 192:208].view(np.int8).reshape(-1, 2, 8).astype(np.float32)
+    d = b[:, 208:210].copy().view(np.float16).astype(np.float32).reshape(-1)
+    # groups g = 0..3 of a half: (ql bytes 0..31 low nibble, bytes 32..63 low, 0..31 high, 32..63 high)
+    lo = np.stack([ql[:, :, 0] & 0xF, ql[:, :, 1] & 0xF, ql[:, :, 0] >> 4, ql[:, :, 1] >> 4], axis=2)
+    hi = np.stack([(qh >> (2 * g)) & 3 for g in range(4)], axis=2)
+    q = (lo | (hi << 4)).astype(np.int32) - 32       # [blk, half, g, l]
+    l16 = (np.arange(32) // 16)
+    scale = np.stack([sc[:, :, 2 * g + l16] for g in range(4)], axis=2)  # [blk, half, g, l]
+    ds = (d[:, None, None, None] * scale).astype(np.float32)             # one rounding
+    y = (ds * q.astype(np.float32)).astype(np.float32)                   # one rounding
+    return y.reshape(rows, cols)
+
+
 def quant_act_q8_0(x: np.ndarray):
     """Q8_0 activation quantization -> (d as f32 of the f16-rounded scale, int8 q)."""
     xb = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, 32)

@@ -285,6 +285,34 @@ def test_committed_fixture_dequantizes_to_its_closed_form(qa):
 
 
 @pytest.mark.gpu
+def test_q6_k_tensors_load_as_dense_f32(qa, oracle, tmp_path):
+    """Q4_K_M files keep some tensors in Q6_K: they are listed with shape, type and size, load as
+    dense f32 bit-exactly (device kernel against the oracle's BlockQ6K::to_float) and are refused
+    as projections."""
+    from izwi_amd.capi import QmmError
+    rng = np.random.default_rng(16)
+    n, k = 24, 1024
+    nb = n * k // 256
+    b = rng.integers(0, 256, nb * 210, dtype=np.uint8).reshape(nb, 210)
+    b[:, 208:210] = (rng.standard_normal(nb) * 0.02).astype(np.float16).view(np.uint8).reshape(nb, 2)
+    hand = bytes.fromhex(json.load(open(os.path.join(HERE, "golden", "q6k_hand_block.json")))["block_hex"])
+    path = str(tmp_path / "q6.gguf")
+    gw.write_gguf(path, [], [("blk.0.ffn_down.weight", (n, k), 14, b.tobytes()), ("hand", (1, 256), 14, hand)])
+    g = qa.GgufLoader.from_path(path)
+    assert g.tensor_dtype("blk.0.ffn_down.weight") == 14 and g._info("blk.0.ffn_down.weight").nbytes == nb * 210
+    assert g.get_model_info().quantization == "Q6K"
+    want = oracle.dequantize(14, b.reshape(-1), n, k)
+    for device in ("cuda", "cpu"):
+        got = g.load_tensor("blk.0.ffn_down.weight", device=device).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    fx = json.load(open(os.path.join(HERE, "golden", "q6k_hand_block.json")))
+    assert np.array_equal(g.load_tensor("hand").cpu().numpy().reshape(-1), np.array(fx["expected_f32"], dtype=np.float32))
+    with pytest.raises(QmmError) as e:
+        g.load_qtensor("blk.0.ffn_down.weight")
+    assert e.value.code == -2
+
+
+@pytest.mark.gpu
 def test_load_packed_matches_packing_separately_loaded_tensors(qa, oracle, tmp_path):
     import torch
     path, blocks, _, _ = _model_file(tmp_path, oracle)

@@ -27,6 +27,26 @@ def test_oracle_q4k_hand_block_fixture(oracle):
     assert float(y.astype(np.float64).sum()) == fx["expected_sum"]
 
 
+def test_oracle_q6k_hand_block_fixture(oracle):
+    """Q6_K is a load-time codec (GGUF ingress to dense f32); the oracle's restatement of
+    BlockQ6K::to_float against the hand-built block and against an independent numpy version."""
+    import np_ref
+    fx = load("q6k_hand_block.json")
+    want = np.array(fx["expected_f32"], dtype=np.float32)
+    y = oracle.dequantize(14, blocks(fx["block_hex"]), 1, 256)[0]
+    assert np.array_equal(y, want) and float(y.astype(np.float64).sum()) == fx["expected_sum"]
+    assert np.array_equal(np_ref.dequant_q6_k(blocks(fx["block_hex"]), 1, 256)[0], want)
+    # random block bytes with finite scales: the two restatements agree bit for bit
+    rng = np.random.default_rng(6)
+    nb = 64
+    b = rng.integers(0, 256, nb * 210, dtype=np.uint8).reshape(nb, 210)
+    b[:, 208:210] = (rng.standard_normal(nb) * 0.01).astype(np.float16).view(np.uint8).reshape(nb, 2)
+    a = oracle.dequantize(14, b.reshape(-1), 8, 2048)
+    c = np_ref.dequant_q6_k(b.reshape(-1), 8, 2048)
+    assert np.array_equal(a.view(np.uint32), c.view(np.uint32))
+    assert oracle.storage_bytes(14, 8, 2048) == nb * 210
+
+
 def test_oracle_packed_q8_0_fixture(oracle):
     fx = load("packed_q8_0_case.json")
     k = fx["k"]
