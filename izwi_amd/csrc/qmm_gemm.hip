@@ -321,11 +321,14 @@ __device__ __forceinline__ void static_for(F&& f) {
 // stays in scalar registers, the per-lane part of every address is a 32-bit offset
 // computed once.  XTAIL: k is not a multiple of 64 (Q8_0 only), activation chunks at or
 // past k are zeroed on their way to LDS.
-template <int QT, int BM, int BN, bool XTAIL>
-__global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
-    constexpr int MT = BM / 64, NT = BN / 64;
-    constexpr int XC = BM / 32;
-    constexpr int TPR = kThreads / BN;                   // threads that share a weight row: 1 or 2
+template <int QT, int BM, int BN, bool XTAIL, int NW = 4>
+__global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
+    // NW waves as a (NW / 2) x 2 grid of wave tiles; with eight waves two share a SIMD, each with
+    // half the accumulators, and one issues while the other waits
+    constexpr int THREADS = 64 * NW, WM = NW / 2;
+    constexpr int MT = BM / WM / 32, NT = BN / 64;       // 32 x 32 accumulator tiles per wave
+    constexpr int XC = BM * 8 / THREADS;                 // 16-byte activation chunks per thread and k step
+    constexpr int TPR = THREADS / BN;                    // threads that share a weight row: 1 or 2
     constexpr int NCR = QT == QMM_Q4_K ? 2 : 4;          // quant chunks per row and k step
     constexpr int NC = NCR / TPR;                        // ... per thread
     constexpr int NP = 16 / TPR;                         // pieces of four weights per thread and k step
@@ -355,7 +358,7 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
     // activation chunks in flight: tile kt+1 (written to LDS during step kt) and, where the
     // register file allows, tile kt+2 behind it, so that a chunk is requested XD k steps
     // before it is needed
-    constexpr int XD = BN == 128 ? 2 : 1;
+    constexpr int XD = BN == 128 && NW == 4 ? 2 : 1;
     u32x4 xr[XD][XC];
     u32x4 w_hdr;      // header of the unit fetched last
     u32x4 wq[2][NC];  // quant chunks of tile kt+1 (being dequantized) and tile kt+2 (in flight), by parity
@@ -365,7 +368,7 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
     int x_lds[XC];
 #pragma unroll
     for (int i = 0; i < XC; i++) {
-        const int c = tid + kThreads * i;
+        const int c = tid + THREADS * i;
         const int row = c >> 3, kc = c & 7;
         x_off[i] = (uint32_t)((min(m0 + row, P.m - 1) - m0) * P.k * 2 + kc * 16);
         x_lds[i] = row * kRowStride + kc * 16;
@@ -488,7 +491,7 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
     // the other set is filled.  A group of four MFMAs uses one row fragment and all column
     // fragments, so the column fragments are fetched first.
     bf16x8 fa[2][MT], fb[2][NT];
-    const int frag_x = (wm * (BM / 2) + (lane & 31)) * kRowStride + (lane >> 5) * 16;
+    const int frag_x = (wm * (BM / WM) + (lane & 31)) * kRowStride + (lane >> 5) * 16;
     const int frag_w = (BM + wn * (BN / 2) + (lane & 31)) * kRowStride + (lane >> 5) * 16;
     // part gi of GPK: read while group gi runs, used from group gi of the next k16 step on
     auto read_frags = [&](const uint8_t* stage, int kk, int set, auto PART) {
@@ -611,7 +614,7 @@ __global__ __launch_bounds__(kThreads) void gemm_pipe_kernel(GemmParams P) {
             if (gn >= P.n_end) continue;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int64_t gm = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                const int64_t gm = m0 + wm * (BM / WM) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 if (gm >= P.m) continue;
                 if (out_bf16)
                     reinterpret_cast<uint16_t*>(P.y)[gm * P.n + gn] = qmm_f32_to_bf16_bits(acc[i][j][r]);
@@ -650,7 +653,7 @@ __global__ void f32_to_bf16_kernel(const float* __restrict__ x, uint16_t* __rest
     }
 }
 
-template <int QT, int BM, int BN>
+template <int QT, int BM, int BN, int NW = 4>
 hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
     P.tiles_m = (int)((P.m + BM - 1) / BM);
     P.tiles_n = (int)((P.n_end - P.n_begin + BN - 1) / BN);
@@ -661,8 +664,8 @@ hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
     constexpr bool kPipe = BM == 256 || BN == 256;
     const void* fn;
     if constexpr (kPipe)
-        fn = x_tail ? reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, BN, true>)
-                    : reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, BN, false>);
+        fn = x_tail ? reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, BN, true, NW>)
+                    : reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, BN, false, NW>);
     else fn = reinterpret_cast<const void*>(&gemm_kernel<QT, BM, BN>);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -673,8 +676,8 @@ hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
         if (slices > 1) P.slice_units = (P.k_units + slices - 1) / slices;
         else P.partial = nullptr;
         const dim3 grid2((unsigned)grid, (unsigned)slices);
-        if (x_tail) gemm_pipe_kernel<QT, BM, BN, true><<<grid2, dim3(kThreads), lds, stream>>>(P);
-        else gemm_pipe_kernel<QT, BM, BN, false><<<grid2, dim3(kThreads), lds, stream>>>(P);
+        if (x_tail) gemm_pipe_kernel<QT, BM, BN, true, NW><<<grid2, dim3(64 * NW), lds, stream>>>(P);
+        else gemm_pipe_kernel<QT, BM, BN, false, NW><<<grid2, dim3(64 * NW), lds, stream>>>(P);
         if (slices > 1) {
             const int64_t count = P.m * (P.n_end - P.n_begin);
             splitk_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(
@@ -763,12 +766,12 @@ hipError_t launch_qt(const GemmParams& P0, int n_cus, hipStream_t stream) {
     if (plan.slices > 1 && P0.partial == nullptr) return hipErrorInvalidValue;
     if (plan.full_cols > 0) {
         P.n_end = plan.full_cols * 256;
-        hipError_t e = launch_tile<QT, 256, 256>(P, 1, stream);
+        hipError_t e = launch_tile<QT, 256, 256, 8>(P, 1, stream);
         if (e != hipSuccess) return e;
         P.n_begin = P.n_end;
         P.n_end = P0.n;
     }
-    if (plan.bm == 256 && plan.bn == 256) return launch_tile<QT, 256, 256>(P, plan.slices, stream);
+    if (plan.bm == 256 && plan.bn == 256) return launch_tile<QT, 256, 256, 8>(P, plan.slices, stream);
     if (plan.bm == 256) return launch_tile<QT, 256, 128>(P, plan.slices, stream);
     if (plan.bn == 256) return launch_tile<QT, 128, 256>(P, plan.slices, stream);
     return launch_tile<QT, 128, 128>(P, 1, stream);
