@@ -328,9 +328,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
     constexpr int THREADS = 64 * NW, WM = NW / 2;
     constexpr int MT = BM / WM / 32, NT = BN / 64;       // 32 x 32 accumulator tiles per wave
     constexpr int XC = BM * 8 / THREADS;                 // 16-byte activation chunks per thread and k step
-    constexpr int TPR = THREADS / BN;                    // threads that share a weight row: 1 or 2
-    constexpr int NCR = QT == QMM_Q4_K ? 2 : 4;          // quant chunks per row and k step
-    constexpr int NC = NCR / TPR;                        // ... per thread
+    constexpr int TPR = THREADS / BN;                    // threads that share a weight row: 1, 2 or 4
+    constexpr int NCR = QT == QMM_Q4_K ? 2 : 4;          // 16-byte quant chunks per row and k step
+    constexpr int ND = 4 * NCR / TPR;                    // the thread's run of quant dwords: 2 .. 16
+    constexpr int NC = ND >= 4 ? ND / 4 : 1;             // loads per thread and k step (16 bytes; 8 if ND = 2)
     constexpr int NP = 16 / TPR;                         // pieces of four weights per thread and k step
     constexpr int GPK = MT * NT / 4; // groups of four MFMAs per k16 step
     constexpr int NG = 4 * GPK;      // groups per k step: 16 (BM = 256) or 8 (BM = 128)
@@ -358,10 +359,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
     // activation chunks in flight: tile kt+1 (written to LDS during step kt) and, where the
     // register file allows, tile kt+2 behind it, so that a chunk is requested XD k steps
     // before it is needed
-    constexpr int XD = BN == 128 && NW == 4 ? 2 : 1;
+    constexpr int XD = BN == 128 ? 2 : 1;
     u32x4 xr[XD][XC];
     u32x4 w_hdr;      // header of the unit fetched last
-    u32x4 wq[2][NC];  // quant chunks of tile kt+1 (being dequantized) and tile kt+2 (in flight), by parity
+    uint32_t wq[2][ND]; // quant dwords of tile kt+1 (being dequantized) and tile kt+2 (in flight), by parity
     // activations: uniform tile base + uniform column + per-lane (row, chunk) offset
     const uint8_t* x_tile = reinterpret_cast<const uint8_t*>(P.x) + m0 * P.k * 2;
     uint32_t x_off[XC];
@@ -383,9 +384,12 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
     const uint32_t slot_bytes = (uint32_t)P.slots * 16u;
     const uint32_t w_off =
         (uint32_t)((min(rt0 + (w_row >> 4), P.row_tiles - 1) - rt0) * rowtile_bytes) + (uint32_t)(w_row & 15) * 16u;
-    const uint32_t w_off_q = w_off + (uint32_t)(w_part * NC) * slot_bytes; // this thread's first chunk of a step
-    // Q4_K: part p holds nibble bytes 16p .. 16p+15 of the step; Q8_0: int8 32p .. 32p+31
-    const int w_lds = (BM + w_row) * kRowStride + w_part * (QT == QMM_Q4_K ? 32 : 64);
+    // part p holds dwords p ND .. p ND + ND - 1 of the row's quant dwords of a step (Q4_K: 8
+    // dwords of nibbles, dword D = elements 4 D .. (low) and 32 + 4 D .. (high); Q8_0: 16 dwords of
+    // int8): its first chunk (and, for half a chunk, the offset inside it) and its LDS position
+    const int w_d0 = w_part * ND;
+    const uint32_t w_off_q = w_off + (uint32_t)(w_d0 / 4) * slot_bytes + (uint32_t)(w_d0 % 4) * 4u;
+    const int w_lds = (BM + w_row) * kRowStride + w_d0 * 8;
     // load cursor: the unit whose chunks are fetched next (clamped to the last unit)
     int cur_us = u0 < P.k_units ? u0 % P.s : 0;
     uint32_t cur_kg_off = (uint32_t)((u0 < P.k_units ? u0 / P.s : 0) * P.panel_bytes);
@@ -419,8 +423,15 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
         w_hdr = *reinterpret_cast<const u32x4*>(w_tile + (cur_kg_off + (uint32_t)cur_us * 256u) + w_off);
     };
     auto w_load_q = [&](int sub, int c) {
-        wq[sub & 1][c] = *reinterpret_cast<const u32x4*>(
-            w_tile + (cur_kg_off + (uint32_t)cur_us * 256u + (uint32_t)(1 + sub * NCR + c) * slot_bytes) + w_off_q);
+        const uint8_t* src =
+            w_tile + (cur_kg_off + (uint32_t)cur_us * 256u + (uint32_t)(1 + sub * NCR + c) * slot_bytes) + w_off_q;
+        if constexpr (ND >= 4) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(src);
+            wq[sub & 1][4 * c] = v.x, wq[sub & 1][4 * c + 1] = v.y, wq[sub & 1][4 * c + 2] = v.z, wq[sub & 1][4 * c + 3] = v.w;
+        } else {
+            const uint2 v = *reinterpret_cast<const uint2*>(src);
+            wq[sub & 1][0] = v.x, wq[sub & 1][1] = v.y;
+        }
     };
     // header of the unit being staged, unpacked once per unit
     float hd = 0, hdmin = 0;                            // Q4_K: d, dmin
@@ -451,7 +462,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
             sb = qmm_f16_bits_to_f32((uint16_t)(pair >> 16));
             ba = -128.0f * sa;
             bb = -128.0f * sb;
-            sw = w_part ? sb : sa;
+            sw = (w_d0 / 8) ? sb : sa; // the thread's dwords lie in one block of 8 dwords
             bw = -128.0f * sw;
         }
     };
@@ -464,26 +475,26 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
         constexpr int par = decltype(PAR)::value, h = decltype(HH)::value;
         uint8_t* row = stage + w_lds;
         if constexpr (QT == QMM_Q4_K) {
-            // dwords (c, j) and (c, j + 1) of a chunk, low nibbles of both, then high nibbles of both
-            constexpr int c = h / 8, jp = (h % 8) / 4, hi = (h % 4) / 2, j = 2 * jp + (h % 2);
-            const uint32_t v = wq[par][c][j];
+            // the thread's dword pair pp: low nibbles of both dwords, then high nibbles of both
+            constexpr int pp = h / 4, hi = (h % 4) / 2;
+            const uint32_t v = wq[par][2 * pp + (h % 2)];
             const uint32_t q4 = (hi ? v >> 4 : v) & nibble_mask;
             const float sc = hi ? sb : sa, bi = hi ? bb : ba;
             constexpr int o = (h % 2) * 2;
             stash[o] = pack_bf16(__builtin_fmaf(sc, ubyte_f32<0>(q4), bi), __builtin_fmaf(sc, ubyte_f32<1>(q4), bi));
             stash[o + 1] = pack_bf16(__builtin_fmaf(sc, ubyte_f32<2>(q4), bi), __builtin_fmaf(sc, ubyte_f32<3>(q4), bi));
-            if (h % 2) // low nibbles: k 16c + 8 jp .., high nibbles: k 32 + 16c + 8 jp ..
-                *reinterpret_cast<uint4*>(row + 64 * hi + 32 * c + 16 * jp) = make_uint4(stash[0], stash[1], stash[2], stash[3]);
+            if (h % 2) // low nibbles: k 8 (d0 / 2 + pp) .., high nibbles: 32 elements further
+                *reinterpret_cast<uint4*>(row + 64 * hi + 16 * pp) = make_uint4(stash[0], stash[1], stash[2], stash[3]);
         } else {
-            constexpr int c = h / 4, j = h % 4; // the thread's chunk c: block (part * NC + c) / 2 of the step
+            // the thread's dword h: block (d0 + h) / 8 of the step
             float d, bias;
-            if (TPR == 1) d = (c >> 1) ? sb : sa, bias = (c >> 1) ? bb : ba;
+            if (TPR == 1) d = (h >> 3) ? sb : sa, bias = (h >> 3) ? bb : ba;
             else d = sw, bias = bw;
-            const uint32_t u = wq[par][c][j] ^ 0x80808080u;
-            constexpr int o = (j % 2) * 2;
+            const uint32_t u = wq[par][h] ^ 0x80808080u;
+            constexpr int o = (h % 2) * 2;
             stash[o] = pack_bf16(__builtin_fmaf(d, ubyte_f32<0>(u), bias), __builtin_fmaf(d, ubyte_f32<1>(u), bias));
             stash[o + 1] = pack_bf16(__builtin_fmaf(d, ubyte_f32<2>(u), bias), __builtin_fmaf(d, ubyte_f32<3>(u), bias));
-            if (j % 2) *reinterpret_cast<uint4*>(row + 32 * c + 16 * (j / 2)) = make_uint4(stash[0], stash[1], stash[2], stash[3]);
+            if (h % 2) *reinterpret_cast<uint4*>(row + 16 * (h / 2)) = make_uint4(stash[0], stash[1], stash[2], stash[3]);
         }
     };
 
@@ -496,10 +507,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
     // part gi of GPK: read while group gi runs, used from group gi of the next k16 step on
     auto read_frags = [&](const uint8_t* stage, int kk, int set, auto PART) {
         constexpr int part = decltype(PART)::value;
-        constexpr int jb = NT == 4 ? (part < GPK / 2 ? part * 2 * NT / GPK : NT) : (part == 0 ? 0 : NT);
-        constexpr int je = NT == 4 ? (part < GPK / 2 ? (part + 1) * 2 * NT / GPK : NT) : NT;
-        constexpr int ib = NT == 4 ? (part < GPK / 2 ? 0 : (part - GPK / 2) * 2 * MT / GPK) : (part == 0 ? 0 : MT / 2);
-        constexpr int ie = NT == 4 ? (part < GPK / 2 ? 0 : (part - GPK / 2 + 1) * 2 * MT / GPK) : (part == 0 ? MT / 2 : MT);
+        constexpr int jb = GPK == 1 ? 0 : NT == 4 ? (part < GPK / 2 ? part * 2 * NT / GPK : NT) : (part == 0 ? 0 : NT);
+        constexpr int je = GPK == 1 ? NT : NT == 4 ? (part < GPK / 2 ? (part + 1) * 2 * NT / GPK : NT) : NT;
+        constexpr int ib = GPK == 1 ? 0 : NT == 4 ? (part < GPK / 2 ? 0 : (part - GPK / 2) * 2 * MT / GPK) : (part == 0 ? 0 : MT / 2);
+        constexpr int ie = GPK == 1 ? MT : NT == 4 ? (part < GPK / 2 ? 0 : (part - GPK / 2 + 1) * 2 * MT / GPK) : (part == 0 ? MT / 2 : MT);
 #pragma unroll
         for (int j = jb; j < je; j++)
             fb[set][j] = *reinterpret_cast<const bf16x8*>(stage + frag_w + j * 32 * kRowStride + kk * 32);
@@ -559,7 +570,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
                 // inside the group: one MFMA, then its share of the other instructions, so
                 // the matrix pipe is fed while they issue
                 constexpr int valu = 3 * (p1 - p0) + (g == 0 ? 4 : 1);
-                constexpr int reads = NT == 4 ? (gi < GPK / 2 ? 2 * NT / GPK : 2 * MT / GPK) : (gi == 0 ? NT + MT / 2 : MT / 2);
+                constexpr int reads = GPK == 1 ? NT + MT : NT == 4 ? (gi < GPK / 2 ? 2 * NT / GPK : 2 * MT / GPK) : (gi == 0 ? NT + MT / 2 : MT / 2);
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -772,7 +783,7 @@ hipError_t launch_qt(const GemmParams& P0, int n_cus, hipStream_t stream) {
         P.n_end = P0.n;
     }
     if (plan.bm == 256 && plan.bn == 256) return launch_tile<QT, 256, 256, 8>(P, plan.slices, stream);
-    if (plan.bm == 256) return launch_tile<QT, 256, 128>(P, plan.slices, stream);
+    if (plan.bm == 256) return launch_tile<QT, 256, 128, 8>(P, plan.slices, stream);
     if (plan.bn == 256) return launch_tile<QT, 128, 256>(P, plan.slices, stream);
     return launch_tile<QT, 128, 128>(P, 1, stream);
 }
