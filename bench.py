@@ -242,7 +242,7 @@ def prefill_extra(torch, qa, oracle, dtype, m, steps=20, warmup=5, only=None):
     return out
 
 
-def moe_extra(torch, qa, oracle, steps=20, warmup=3):
+def moe_extra(torch, qa, oracle, steps=50, warmup=5):
     """One MoE layer (route + sort + grouped expert MLP + combine, HIP-graph replay) at the
     Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, expert intermediate 768, Q4_K; as one
     call and as the three calls it is composed of."""
