@@ -441,12 +441,27 @@ def main():
         except Exception as exc:
             extras["decode_packed_error"] = repr(exc)
         try:
+            # the other block format of the configuration on the same stack and call structure
+            other_dtype = Q8_0 if dtype == Q4_K else Q4_K
+            ow = build_decode_weights(torch, qa, oracle, other_dtype, args.layers, True)
+            c, tb = make_calls(torch, oracle, other_dtype, ow, args.m)
+            t, g = time_graph(torch, lambda: run_calls(qa, c), max(5, args.steps // 2), 3)
+            extras["decode_q8_0_8b_stack" if other_dtype == Q8_0 else "decode_q4k_8b_stack"] = {
+                "gbs": round(tb / (t * 1e-3) / 1e9, 1), "ms_per_step": round(t, 4),
+                "pct_of_hbm_peak": round(100.0 * tb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2), "m": args.m,
+                "calls_per_step": len(c)}
+            del ow, c, g
+            torch.cuda.empty_cache()
+        except Exception as exc:
+            extras["decode_other_dtype_error"] = repr(exc)
+        try:
             extras["moe_30b_a3b_q4k"] = moe_extra(torch, qa, oracle)
         except Exception as exc:
             extras["moe_error"] = repr(exc)
         try:
             extras["prefill_tflops_m2048_q4k"] = prefill_extra(torch, qa, oracle, Q4_K, 2048)
             extras["prefill_tflops_m2048_q8_0"] = prefill_extra(torch, qa, oracle, Q8_0, 2048)
+            extras["prefill_tflops_m512_q4k"] = prefill_extra(torch, qa, oracle, Q4_K, 512)
             best = max(extras["prefill_tflops_m2048_q4k"].values())
             extras["prefill_best_frac_of_bf16_peak"] = round(best / BF16_PEAK_TFLOPS, 4)
         except Exception as exc:  # extras never invalidate the headline number
