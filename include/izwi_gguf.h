@@ -1,6 +1,6 @@
 /*
  * izwi_gguf — GGUF ingress for the quantized linear-layer library: container
- * parse, tensor lookup and upload of Q8_0 / Q4_K tensors straight into
+ * parse, tensor lookup and upload of Q8_0 / Q4_K / Q6_K tensors straight into
  * izwi_qmm weight handles.
  *
  * It replaces, for this library's device, the reference's
@@ -107,7 +107,7 @@ int izwi_gguf_metadata_array_string(const izwi_gguf* g, const char* key, uint64_
 
 /* `load_qtensor` (gguf.rs:117-124) followed by `QMatMul::from_arc` (core.rs:710-715): the
  * tensor's block bytes go from the mapping into a weight handle on the current HIP device.  The
- * tensor must have two dimensions [n, k] and type Q8_0 or Q4_K; other quantized types are
+ * tensor must have two dimensions [n, k] and type Q8_0, Q4_K or Q6_K; other quantized types are
  * IZWI_QMM_ERR_UNSUPPORTED. */
 int izwi_gguf_load_weight(const izwi_gguf* g, const char* name, izwi_qmm_weight** out);
 
@@ -119,8 +119,7 @@ int izwi_gguf_load_packed(const izwi_gguf* g, const char* const* names, int32_t 
 /* `load_tensor(name, DType::F32, device)` (gguf.rs:127-144): the tensor as dense f32 in row-major
  * order, `count` = number of elements `out` holds (must equal the tensor's element count).  F32 is
  * copied, F16 / BF16 converted, Q8_0 / Q4_K / Q6_K dequantized bit-exactly as candle-core's
- * `to_float` (Q6_K, which Q4_K_M files use for some tensors, is a load-time codec only: it has no
- * weight handle); conversion runs on the device (`mem_space` says where `out` lives). */
+ * `to_float`; conversion runs on the device (`mem_space` says where `out` lives). */
 int izwi_gguf_load_tensor_f32(const izwi_gguf* g, const char* name, float* out, uint64_t count,
                               int mem_space, void* stream);
 

@@ -15,7 +15,7 @@
  *     aborts (the reference maps them to Error::InferenceError,
  *     crates/izwi-core/src/error.rs:69-73).
  *   - weights are `[n, k]` row-major in GGUF block layout (blocks along k),
- *     ggml dtype ids as in GGUF: Q8_0 = 8, Q4_K = 12.
+ *     ggml dtype ids as in GGUF: Q8_0 = 8, Q4_K = 12, Q6_K = 14.
  *   - `mem_space` says where the caller's buffers live: IZWI_QMM_DEVICE (HIP
  *     device pointers, the fast path, asynchronous on `stream`) or
  *     IZWI_QMM_HOST (ordinary host memory; the library stages it and the call
@@ -50,6 +50,7 @@ typedef enum izwi_qmm_status {
 /* ggml / GGUF tensor type ids (candle-core GgmlDType) */
 #define IZWI_QMM_Q8_0 8
 #define IZWI_QMM_Q4_K 12
+#define IZWI_QMM_Q6_K 14 /* single projections only: no projection-group launch, no expert stacks */
 
 typedef enum izwi_qmm_mem_space { IZWI_QMM_DEVICE = 0, IZWI_QMM_HOST = 1 } izwi_qmm_mem_space;
 
@@ -148,7 +149,7 @@ int izwi_qmm_dequantize_f32(const izwi_qmm_weight* w, float* out, int mem_space,
  * x is `[m, k]` row-major contiguous, y is `[m, n]`.  Any m >= 0; m <= 64 runs
  * the fused decode kernel, larger m the tiled MFMA kernel.  Activations are
  * quantized on chip to the weight type's dot type exactly as candle-core does
- * (Q8_0 -> Q8_0 blocks, Q4_K -> Q8_K blocks), so results agree with the
+ * (Q8_0 -> Q8_0 blocks, Q4_K and Q6_K -> Q8_K blocks), so results agree with the
  * reference's CPU path up to f32 summation order. */
 int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, float* y,
                          int mem_space, void* stream);

@@ -475,9 +475,9 @@ int izwi_gguf_load_weight(const izwi_gguf* g, const char* name, izwi_qmm_weight*
     const Tensor* t = find_tensor(g, name);
     if (!t) return qmm_fail(IZWI_QMM_ERR_INVALID, "Failed to load tensor '%s' from GGUF: tensor not found", name);
     const izwi_gguf_tensor_info& ti = t->info;
-    if (ti.ggml_dtype != IZWI_QMM_Q8_0 && ti.ggml_dtype != IZWI_QMM_Q4_K)
+    if (ti.ggml_dtype != IZWI_QMM_Q8_0 && ti.ggml_dtype != IZWI_QMM_Q4_K && ti.ggml_dtype != IZWI_QMM_Q6_K)
         return qmm_fail(IZWI_QMM_ERR_UNSUPPORTED,
-                        "Failed to load tensor '%s' from GGUF: ggml dtype %d is not supported (Q8_0 = 8, Q4_K = 12)",
+                        "Failed to load tensor '%s' from GGUF: ggml dtype %d is not supported (Q8_0 = 8, Q4_K = 12, Q6_K = 14)",
                         name, ti.ggml_dtype);
     if (ti.n_dims != 2)
         return qmm_fail(IZWI_QMM_ERR_INVALID, "Failed to load tensor '%s' from GGUF: %d dimensions, a projection has 2",
@@ -547,7 +547,7 @@ int izwi_gguf_load_tensor_f32(const izwi_gguf* g, const char* name, float* out, 
         return e == hipSuccess ? IZWI_QMM_OK : hip_fail(e, "copy to the device");
     }
     case 1:    // F16
-    case 14:   // Q6_K (dense load only: not a matmul type of this library)
+    case 14:   // Q6_K straight from its file layout
     case 30: { // BF16
         DeviceBuffer raw, tmp;
         hipError_t e = hipMalloc(&raw.p, (size_t)ti.nbytes);

@@ -119,11 +119,11 @@ int current_device(int* device) {
     return fail_hip(e, "hipGetDevice");
 }
 
-int type_supported(int dtype) { return dtype == IZWI_QMM_Q8_0 || dtype == IZWI_QMM_Q4_K; }
+int type_supported(int dtype) { return dtype == IZWI_QMM_Q8_0 || dtype == IZWI_QMM_Q4_K || dtype == IZWI_QMM_Q6_K; }
 
 int storage_bytes(int dtype, int64_t rows, int64_t cols, uint64_t* out) {
     if (!type_supported(dtype))
-        return fail(IZWI_QMM_ERR_UNSUPPORTED, "ggml dtype %d is not supported (Q8_0 = 8, Q4_K = 12)", dtype);
+        return fail(IZWI_QMM_ERR_UNSUPPORTED, "ggml dtype %d is not supported (Q8_0 = 8, Q4_K = 12, Q6_K = 14)", dtype);
     if (rows < 0 || cols < 0) return fail(IZWI_QMM_ERR_INVALID, "negative shape [%lld, %lld]", (long long)rows, (long long)cols);
     unsigned __int128 elems = (unsigned __int128)rows * (unsigned __int128)cols;
     if (elems > (unsigned __int128)1 << 62)
@@ -504,7 +504,8 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
     Staged xi, yo;
     HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
     HIP_TRY(yo.out(y, (size_t)m * L.n * sizeof(float), mem_space));
-    if (m < mfma_min_m()) {
+    if (m < mfma_min_m() || (L.dtype == IZWI_QMM_Q6_K && m <= 64)) {
+        // (Q6_K has no matrix-core decode form: the dot4 kernel takes its rows four at a time)
         HIP_TRY(qmm_launch_gemv(L, w->tiled, (const float*)xi.dev, m, (float*)yo.dev, w->n_cus, stream));
     } else if (m <= 64) {
         void* scratch = nullptr;
@@ -543,7 +544,8 @@ int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_
         if (L.k != weights[0]->layout.k)
             return fail(IZWI_QMM_ERR_INVALID, "projection group input mismatch: expected %lld, got %lld",
                         (long long)weights[0]->layout.k, (long long)L.k);
-        if (L.dtype != weights[0]->layout.dtype || L.n == 0 || weights[i]->device != weights[0]->device)
+        if (L.dtype != weights[0]->layout.dtype || L.n == 0 || weights[i]->device != weights[0]->device ||
+            L.dtype == IZWI_QMM_Q6_K) // Q6_K has no multi-weight launch
             uniform = false;
         if (m > 0 && L.n > 0 && !ys[i]) return fail(IZWI_QMM_ERR_INVALID, "y is NULL");
     }
@@ -620,7 +622,7 @@ int izwi_qmm_forward_gate_up_silu_f32(const izwi_qmm_weight* gate, const izwi_qm
     HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
     HIP_TRY(ho.out(h, (size_t)m * L.n * sizeof(float), mem_space));
     if (profiling()) g_silu_fused.fetch_add(1, std::memory_order_relaxed);
-    if (m < mfma_min_m() && m <= 2) {
+    if (m < mfma_min_m() && m <= 2 && L.dtype != IZWI_QMM_Q6_K) {
         ProfileScope prof(gate, stream);
         HIP_TRY(qmm_launch_gemv_gated(L, gate->tiled, up->tiled, (const float*)xi.dev, m, (float*)ho.dev,
                                       gate->n_cus, stream));
@@ -735,6 +737,8 @@ int moe_check_stacks(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, con
     const QmmLayout& D = down->layout;
     if (G.dtype != U.dtype || G.n != U.n || G.k != U.k || G.n_stacked != U.n_stacked)
         return fail(IZWI_QMM_ERR_INVALID, "gate and up stacks differ in shape or dtype");
+    if (G.dtype == IZWI_QMM_Q6_K || D.dtype == IZWI_QMM_Q6_K)
+        return fail(IZWI_QMM_ERR_UNSUPPORTED, "expert stacks of Q6_K weights are not supported (Q8_0, Q4_K)");
     if (D.n_stacked != G.n_stacked || D.k != G.n || D.n != G.k)
         return fail(IZWI_QMM_ERR_INVALID, "down stack [%lld, %lld] does not match gate/up [%lld, %lld]",
                     (long long)D.n, (long long)D.k, (long long)G.n, (long long)G.k);

@@ -77,6 +77,9 @@ struct WRegs {
     static constexpr int NC = (QT == QMM_Q4_K ? 2 : 4) / TPR;
     u32x4 hdr;
     u32x4 q[NC];
+    // Q6_K only (two threads per row): the 32 bytes of high bit pairs and the chunk with d
+    u32x4 qh[2];
+    u32x4 dch;
 };
 
 // Weight row `row`, k step kt (64 elements), part `part` of TPR: header + chunks.
@@ -97,6 +100,18 @@ __device__ __forceinline__ void load_w(WRegs<QT, TPR>& r, const GemmParams& P, i
         reinterpret_cast<const u32x4*>(P.w + (rt * P.k_groups + kg) * P.panel_bytes) + slot;
     // (the select itself happens in store_w: applying it here would make every load wait)
     r.hdr = base[0];
+    if (QT == QMM_Q6_K) {
+        // the 64 elements of step `sub` are one nibble (sub & 1) of the 64 ql bytes of half
+        // sub >> 1 and one bit pair of its 32 qh bytes; byte e of the 64 pairs with qh byte e % 32
+        static_assert(QT != QMM_Q6_K || TPR == 2, "Q6_K tiles use two threads per weight row");
+        const int h = sub >> 1;
+#pragma unroll
+        for (int c = 0; c < NC; c++) r.q[c] = base[(size_t)(1 + 4 * h + part * NC + c) * P.slots];
+        r.qh[0] = base[(size_t)(9 + 2 * h) * P.slots];
+        r.qh[1] = base[(size_t)(10 + 2 * h) * P.slots];
+        r.dch = base[(size_t)13 * P.slots];
+        return;
+    }
 #pragma unroll
     for (int c = 0; c < NC; c++) r.q[c] = base[(size_t)(1 + sub * NC * TPR + part * NC + c) * P.slots];
 }
@@ -143,6 +158,33 @@ __device__ __forceinline__ void store_w(const WRegs<QT, TPR>& r, int kt, int par
             dl[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
             dh[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
             dh[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+        }
+    } else if (QT == QMM_Q6_K) {
+        // part p holds the elements 32 p .. 32 p + 31 of the step: nibble s1 of its two ql chunks,
+        // bit pair 4 s1 + 2 p of the 32 qh bytes; the 16-element groups 4 sub + 2 p, + 1 carry
+        // the scales.  w = d * scale * (q - 32) as one fma per weight.
+        const int sub = kt & 3, s1 = sub & 1;
+        const float d = ok ? qmm_f16_bits_to_f32((uint16_t)(r.dch.x & 0xffffu)) : 0.0f;
+        const uint32_t hw[4] = {r.hdr.x, r.hdr.y, r.hdr.z, r.hdr.w};
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+            const int j = 4 * sub + 2 * part + c;
+            const float ds = d * (float)(int8_t)((hw[j >> 2] >> (8 * (j & 3))) & 0xffu);
+            const float bias = -32.0f * ds;
+            uint32_t o[8];
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const uint32_t nib = (r.q[c][w] >> (4 * s1)) & 0x0f0f0f0fu;
+                const uint32_t two = (r.qh[c][w] >> (4 * s1 + 2 * part)) & 0x03030303u;
+                const uint32_t q6 = nib | (two << 4);
+                o[2 * w] = pack_bf16(__builtin_fmaf(ds, ubyte_f32<0>(q6), bias),
+                                     __builtin_fmaf(ds, ubyte_f32<1>(q6), bias));
+                o[2 * w + 1] = pack_bf16(__builtin_fmaf(ds, ubyte_f32<2>(q6), bias),
+                                         __builtin_fmaf(ds, ubyte_f32<3>(q6), bias));
+            }
+            uint4* dst = reinterpret_cast<uint4*>(lds_row + 64 * part + 32 * c);
+            dst[0] = make_uint4(o[0], o[1], o[2], o[3]);
+            dst[1] = make_uint4(o[4], o[5], o[6], o[7]);
         }
     } else {
         const int b0 = (kt & 3) * 2; // first of the two 32-element blocks of this k step
@@ -791,7 +833,7 @@ hipError_t launch_qt(const GemmParams& P0, int n_cus, hipStream_t stream) {
 } // namespace
 
 size_t qmm_gemm_workspace_bytes(const QmmLayout& L, int64_t m, int n_cus) {
-    if (m <= 0 || L.n == 0) return 0;
+    if (m <= 0 || L.n == 0 || L.dtype == QMM_Q6_K) return 0;
     const GemmPlan plan = plan_gemm(m, L.n, (int)L.k_units * 4, n_cus > 0 ? n_cus : 1);
     return plan.slices > 1 ? (size_t)plan.slices * (size_t)m * (size_t)L.n * sizeof(float) : 0;
 }
@@ -821,6 +863,7 @@ hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uin
     P.slice_units = 0;
     P.nibble_mask = 0x0f0f0f0fu;
     P.partial = (float*)workspace;
+    if (L.dtype == QMM_Q6_K) return launch_tile<QMM_Q6_K, 128, 128>(P, 1, stream); // the plain tile kernel only
     return L.dtype == QMM_Q4_K ? launch_qt<QMM_Q4_K>(P, n_cus, stream)
                                : launch_qt<QMM_Q8_0>(P, n_cus, stream);
 }

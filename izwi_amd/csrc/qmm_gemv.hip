@@ -6,8 +6,8 @@
 // summation order differs.  The work is bounded by streaming the weight bytes
 // from HBM once:
 //   * a wavefront reads a panel (16 rows x S units of 256 k-elements) as one
-//     16 B/lane coalesced load for the headers plus 8 (Q4_K) or 16 (Q8_0) for
-//     the quants; lane (u, r) owns unit u of row r, so no weight byte is
+//     16 B/lane coalesced load for the headers plus 8 (Q4_K), 13 (Q6_K) or
+//     16 (Q8_0) for the quants; lane (u, r) owns unit u of row r, so no weight byte is
 //     shuffled between lanes and all nibble / int8 products run on
 //     v_dot4_i32_i8 (about 0.7 VALU lane-ops per weight element);
 //   * a wave issues its activation loads and then all loads of its panel before
@@ -163,16 +163,21 @@ __device__ __forceinline__ void lds_barrier() {
 template <int QT>
 struct XLds {
     uint8_t* xq;  // [MT][k_units][kXUnitStride]
-    float* xd;    // Q4_K: [MT][k_units]      Q8_0: [MT][k_units][8]
-    int* xbs;     // Q4_K: [MT][k_units][8]   Q8_0: unused
+    float* xd;    // Q4_K, Q6_K: [MT][k_units]   Q8_0: [MT][k_units][8]
+    int* xbs;     // Q4_K: [MT][k_units][8] sums of 32   Q6_K: [MT][k_units][16] sums of 16   Q8_0: unused
     float* red;   // [2][waves][MT][16]
 };
+// block scales and partial sums kept per quantized unit of x
+template <int QT>
+constexpr int kXdPerItem = QT == QMM_Q8_0 ? 8 : 1;
+template <int QT>
+constexpr int kXbsPerItem = QT == QMM_Q4_K ? 8 : (QT == QMM_Q6_K ? 16 : 0);
 
 template <int QT, int MT>
 __host__ __device__ inline size_t lds_bytes(int64_t k_units, int waves) {
     size_t b = (size_t)MT * k_units * kXUnitStride;
-    b += (size_t)MT * k_units * (QT == QMM_Q4_K ? 1 : 8) * sizeof(float);
-    if (QT == QMM_Q4_K) b += (size_t)MT * k_units * 8 * sizeof(int);
+    b += (size_t)MT * k_units * kXdPerItem<QT> * sizeof(float);
+    b += (size_t)MT * k_units * kXbsPerItem<QT> * sizeof(int);
     b = (b + 15) & ~(size_t)15;
     b += (size_t)2 * waves * MT * 16 * sizeof(float);
     return b;
@@ -184,9 +189,9 @@ __device__ inline XLds<QT> carve(uint8_t* base, int64_t k_units) {
     l.xq = base;
     size_t b = (size_t)MT * k_units * kXUnitStride;
     l.xd = reinterpret_cast<float*>(base + b);
-    b += (size_t)MT * k_units * (QT == QMM_Q4_K ? 1 : 8) * sizeof(float);
+    b += (size_t)MT * k_units * kXdPerItem<QT> * sizeof(float);
     l.xbs = reinterpret_cast<int*>(base + b);
-    if (QT == QMM_Q4_K) b += (size_t)MT * k_units * 8 * sizeof(int);
+    b += (size_t)MT * k_units * kXbsPerItem<QT> * sizeof(int);
     b = (b + 15) & ~(size_t)15;
     l.red = reinterpret_cast<float*>(base + b);
     return l;
@@ -229,6 +234,12 @@ __device__ __forceinline__ void x_item_quantize(const XLds<QT>& l, int k_units, 
         int s32 = s16 + dpp<kDppXor1>(s16);
         if ((j & 1) == 0) l.xbs[slot * 8 + (j >> 1)] = s32;
         if (j == 0) l.xd[slot] = d;
+    } else if (QT == QMM_Q6_K) {
+        float d;
+        int s16;
+        quantize_q8k_lane(v, j, q, d, s16);
+        l.xbs[slot * 16 + j] = s16;
+        if (j == 0) l.xd[slot] = d;
     } else {
         float d;
         uint16_t bits;
@@ -242,7 +253,7 @@ __device__ __forceinline__ void x_item_quantize(const XLds<QT>& l, int k_units, 
 // ---- panel registers ----------------------------------------------------------
 template <int QT>
 struct Panel {
-    static constexpr int QC = QT == QMM_Q4_K ? 8 : 16;
+    static constexpr int QC = QT == QMM_Q4_K ? 8 : (QT == QMM_Q6_K ? 13 : 16);
     u32x4 hdr;
     u32x4 q[QC];
 };
@@ -318,6 +329,43 @@ __device__ __forceinline__ void multiply_panel(const Panel<QT>& p, const XLds<QT
             const float dx = l.xd[item];
             acc[mi] += (d * dx) * (float)isum[mi] - (dmin * dx) * (float)msum;
         }
+    } else if (QT == QMM_Q6_K) {
+        // q[0..7] = ql, q[8..11] = qh, q[12].x = d; hdr = 16 signed scales, scale j for the
+        // elements 16 j .. 16 j + 15.  Element 128 h + 32 g + e (e < 32) is
+        // nibble(g >> 1) of ql[64 h + 32 (g & 1) + e] | bits 2g, 2g+1 of qh[32 h + e], minus 32:
+        // the 32 is taken off through the sums of x (dot - 32 * sum of the 16 quants of x).
+        const uint32_t hw[4] = {p.hdr.x, p.hdr.y, p.hdr.z, p.hdr.w};
+        constexpr uint32_t kTwo = 0x03030303u;
+        int isum[MT];
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) isum[mi] = 0;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+#pragma unroll
+            for (int lb = 0; lb < 2; lb++) {
+                const u32x4 a = p.q[4 * h + lb], b = p.q[4 * h + 2 + lb], hh = p.q[8 + 2 * h + lb];
+                u32x4 v[4];
+                v[0] = (a & kNib) | ((hh & kTwo) << 4);
+                v[1] = (b & kNib) | (((hh >> 2) & kTwo) << 4);
+                v[2] = ((a >> 4) & kNib) | (((hh >> 4) & kTwo) << 4);
+                v[3] = ((b >> 4) & kNib) | (((hh >> 6) & kTwo) << 4);
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int j = 8 * h + 2 * g + lb; // scale index = 16-element group of the unit
+                    const int sc = (int)(int8_t)((hw[j >> 2] >> (8 * (j & 3))) & 0xffu);
+#pragma unroll
+                    for (int mi = 0; mi < MT; mi++) {
+                        const int item = mi * k_units + unit;
+                        const uint4* xq = reinterpret_cast<const uint4*>(l.xq + (size_t)item * kXUnitStride);
+                        const int dot = dot16(v[g], xq[j], 0) - 32 * l.xbs[item * 16 + j];
+                        isum[mi] += __mul24(sc, dot); // |dot| < 2^18, |scale| <= 128
+                    }
+                }
+            }
+        }
+        const float d = qmm_f16_bits_to_f32((uint16_t)(p.q[12].x & 0xffffu));
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) acc[mi] += (d * l.xd[mi * k_units + unit]) * (float)isum[mi];
     } else {
         const uint32_t hw[4] = {p.hdr.x, p.hdr.y, p.hdr.z, p.hdr.w};
 #pragma unroll
@@ -693,6 +741,7 @@ hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x
     if (!make_params(L, tiled, x, m, y, P)) return hipErrorInvalidValue;
     int waves;
     choose_split(L, n_cus, 1, false, P, waves);
+    if (L.dtype == QMM_Q6_K) return launch_plain<QMM_Q6_K>(P, waves, n_cus, stream);
     return L.dtype == QMM_Q4_K ? launch_plain<QMM_Q4_K>(P, waves, n_cus, stream)
                                : launch_plain<QMM_Q8_0>(P, waves, n_cus, stream);
 }
@@ -719,7 +768,7 @@ hipError_t qmm_launch_silu_mul(const float* gate, const float* up, float* out, i
 hipError_t qmm_launch_gemv_gated(const QmmLayout& L, const void* tiled_gate, const void* tiled_up,
                                  const float* x, int64_t m, float* y, int n_cus, hipStream_t stream) {
     if (m <= 0 || L.n == 0) return hipSuccess;
-    if (m > 2) return hipErrorNotSupported;
+    if (m > 2 || L.dtype == QMM_Q6_K) return hipErrorNotSupported;
     GemvParams P;
     if (!make_params(L, tiled_gate, x, m, y, P)) return hipErrorInvalidValue;
     P.w2 = (const uint8_t*)tiled_up;
@@ -743,7 +792,7 @@ hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* co
         if (L.dtype != L0.dtype || L.k != L0.k || L.n_stacked != 1 || L.n == 0) return hipErrorInvalidValue;
         total_row_tiles += L.row_tiles;
     }
-    if (L0.k_groups > kMaxWaves) return hipErrorNotSupported; // no straight-line form: the caller launches one by one
+    if (L0.k_groups > kMaxWaves || L0.dtype == QMM_Q6_K) return hipErrorNotSupported; // no single-launch form: the caller launches one by one
     GemvParams P;
     if (!make_params(L0, tiled[0], x, m, ys[0], P)) return hipErrorInvalidValue;
     // the split of a single matrix with all the row-tiles
@@ -789,6 +838,7 @@ hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const 
                                    int n_cus, hipStream_t stream) {
     if (max_segments <= 0 || L.n == 0) return hipSuccess;
     if (max_segments > 65535) return hipErrorInvalidValue;
+    if (L.dtype == QMM_Q6_K) return hipErrorNotSupported;
     GemvParams P;
     if (!make_params(L, tiled, x, 0, y, P)) return hipErrorInvalidValue;
     P.w2 = (const uint8_t*)tiled2;
@@ -814,7 +864,7 @@ hipError_t qmm_launch_quantize_activations(int weight_dtype, const float* x, int
     int64_t threads = m * k_units * 16;
     if (threads == 0) return hipSuccess;
     unsigned grid = (unsigned)((threads + 255) / 256);
-    if (weight_dtype == QMM_Q4_K)
+    if (weight_dtype == QMM_Q4_K || weight_dtype == QMM_Q6_K) // both dot types are Q8_K
         quantize_export_kernel<QMM_Q4_K>
             <<<grid, 256, 0, stream>>>(x, m, k, k_units, (uint8_t*)out_blocks);
     else

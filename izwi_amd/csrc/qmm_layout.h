@@ -9,6 +9,9 @@
 //   unit   = 256 consecutive k-elements of one row
 //            Q4_K: one block   = 16 B header (d, dmin, 12 scale bytes) + 8 x 16 B of nibbles
 //            Q8_0: eight blocks = 16 B header (8 f16 scales)           + 16 x 16 B of int8
+//            Q6_K: one block   = 16 B header (16 int8 scales) + 8 x 16 B of low nibbles (ql)
+//                                + 4 x 16 B of high bit pairs (qh) + 16 B holding d (f16) and
+//                                14 zero bytes: 224 B for the block's 210
 //   panel  = 16 rows x S units (S = 1..4), slot = unit_in_panel * 16 + row_in_panel
 //            bytes: [slots x 16 B headers][QC x (slots x 16 B quant chunks)]
 //            so that lane `slot` of a wavefront reads its header and its c-th
@@ -20,14 +23,15 @@
 
 #define QMM_Q8_0 8
 #define QMM_Q4_K 12
+#define QMM_Q6_K 14
 
 #define QMM_UNIT_ELEMS 256
 #define QMM_PANEL_ROWS 16
 
 struct QmmLayout {
-    int dtype;           // QMM_Q8_0 / QMM_Q4_K
+    int dtype;           // QMM_Q8_0 / QMM_Q4_K / QMM_Q6_K
     int s;               // units per panel along k (1..4)
-    int qc;              // 16-byte quant chunks per unit: 8 (Q4_K) or 16 (Q8_0)
+    int qc;              // 16-byte chunks per unit after the header: 8 (Q4_K), 16 (Q8_0), 13 (Q6_K)
     int slots;           // 16 * s
     int64_t n, k;        // logical shape of one matrix
     int64_t n_stacked;   // matrices in the handle
@@ -39,7 +43,7 @@ struct QmmLayout {
 };
 
 static inline int qmm_block_elems(int dtype) { return dtype == QMM_Q8_0 ? 32 : 256; }
-static inline int qmm_block_bytes(int dtype) { return dtype == QMM_Q8_0 ? 34 : 144; }
+static inline int qmm_block_bytes(int dtype) { return dtype == QMM_Q8_0 ? 34 : (dtype == QMM_Q6_K ? 210 : 144); }
 
 static inline QmmLayout qmm_make_layout(int dtype, int64_t n_stacked, int64_t n, int64_t k) {
     QmmLayout L;
@@ -55,7 +59,7 @@ static inline QmmLayout qmm_make_layout(int dtype, int64_t n_stacked, int64_t n,
     else if (L.k_units % 2 == 0) s = 2;
     else if (L.k_units == 1) s = 1;
     L.s = s;
-    L.qc = dtype == QMM_Q8_0 ? 16 : 8;
+    L.qc = dtype == QMM_Q8_0 ? 16 : (dtype == QMM_Q6_K ? 13 : 8);
     L.slots = 16 * s;
     L.k_groups = (L.k_units + s - 1) / s;
     L.panel_bytes = (int64_t)L.slots * 16 * (1 + L.qc);

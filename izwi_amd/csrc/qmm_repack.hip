@@ -177,6 +177,76 @@ __global__ void dequant_q80_kernel(QmmLayout L, const uint8_t* __restrict__ tile
             o[4 * j + i] = __fmul_rn((float)(int8_t)((w[j] >> (8 * i)) & 0xffu), d);
 }
 
+// Q6_K block: ql[128] | qh[64] | scales[16] | d (f16) at bytes 0, 128, 192, 208.  The 210-byte
+// block is only 2-byte aligned, so the pieces are gathered as 16-bit words.
+// Tiled pieces: 0 = scales, 1..8 = ql, 9..12 = qh, 13 = d followed by zeros.
+__device__ inline int q6k_piece_src(int piece) {
+    return piece == 0 ? 192 : (piece <= 8 ? 16 * (piece - 1) : (piece <= 12 ? 128 + 16 * (piece - 9) : 208));
+}
+
+__global__ void repack_q6k_kernel(QmmLayout L, const uint8_t* __restrict__ src,
+                                  uint8_t* __restrict__ dst, int64_t n_pieces) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_pieces) return;
+    Piece p = decode_piece(L, idx);
+    union {
+        uint4 v;
+        uint16_t h[8];
+    } u;
+    u.v = make_uint4(0, 0, 0, 0);
+    if (p.valid) {
+        int64_t blk = (p.e * L.n + p.row) * L.k_units + p.unit;
+        const uint16_t* s = reinterpret_cast<const uint16_t*>(src + blk * 210 + q6k_piece_src(p.piece));
+        if (p.piece == 13) u.h[0] = s[0];
+        else
+            for (int i = 0; i < 8; i++) u.h[i] = s[i];
+    }
+    *reinterpret_cast<uint4*>(dst + idx * 16) = u.v;
+}
+
+__global__ void unpack_q6k_kernel(QmmLayout L, const uint8_t* __restrict__ tiled,
+                                  uint8_t* __restrict__ dst, int64_t n_items) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; // (block, piece)
+    if (idx >= n_items) return;
+    int64_t blk = idx / 14;
+    int piece = (int)(idx - blk * 14);
+    int64_t unit = blk % L.k_units;
+    int64_t row_all = blk / L.k_units;
+    int64_t e = row_all / L.n, row = row_all % L.n;
+    const uint16_t* s = reinterpret_cast<const uint16_t*>(tiled + piece_offset(L, e, row, unit, piece));
+    uint16_t* out = reinterpret_cast<uint16_t*>(dst + blk * 210 + q6k_piece_src(piece));
+    if (piece == 13) out[0] = s[0];
+    else
+        for (int i = 0; i < 8; i++) out[i] = s[i];
+}
+
+// One thread per (block, half of 128, l < 32): the elements l, l + 32, l + 64, l + 96 of the
+// half, d * scale * (q - 32) evaluated left to right with a rounding after each product.
+__global__ void dequant_q6k_tiled_kernel(QmmLayout L, const uint8_t* __restrict__ tiled,
+                                         float* __restrict__ out, int64_t n_items) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_items) return;
+    const int l = (int)(idx & 31), half = (int)(idx >> 5) & 1, is = l >> 4;
+    int64_t blk = idx >> 6;
+    int64_t unit = blk % L.k_units;
+    int64_t row_all = blk / L.k_units;
+    int64_t e = row_all / L.n, row = row_all % L.n;
+    const int8_t* sc = reinterpret_cast<const int8_t*>(tiled + piece_offset(L, e, row, unit, 0)) + 8 * half;
+    const uint8_t qa = tiled[piece_offset(L, e, row, unit, 1 + 4 * half + (l >> 4)) + (l & 15)];      // ql[64 half + l]
+    const uint8_t qb = tiled[piece_offset(L, e, row, unit, 1 + 4 * half + 2 + (l >> 4)) + (l & 15)];  // ql[64 half + 32 + l]
+    const uint8_t qh = tiled[piece_offset(L, e, row, unit, 9 + 2 * half + (l >> 4)) + (l & 15)];
+    const float d = qmm_f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(tiled + piece_offset(L, e, row, unit, 13)));
+    const int q1 = (int)((qa & 0xF) | ((qh & 3) << 4)) - 32;
+    const int q2 = (int)((qb & 0xF) | (((qh >> 2) & 3) << 4)) - 32;
+    const int q3 = (int)((qa >> 4) | (((qh >> 4) & 3) << 4)) - 32;
+    const int q4 = (int)((qb >> 4) | (((qh >> 6) & 3) << 4)) - 32;
+    float* y = out + row_all * L.k + unit * 256 + 128 * half;
+    y[l] = __fmul_rn(__fmul_rn(d, (float)sc[is]), (float)q1);
+    y[l + 32] = __fmul_rn(__fmul_rn(d, (float)sc[is + 2]), (float)q2);
+    y[l + 64] = __fmul_rn(__fmul_rn(d, (float)sc[is + 4]), (float)q3);
+    y[l + 96] = __fmul_rn(__fmul_rn(d, (float)sc[is + 6]), (float)q4);
+}
+
 inline unsigned grid_for(int64_t n, int block) { return (unsigned)((n + block - 1) / block); }
 
 } // namespace
@@ -187,6 +257,9 @@ hipError_t qmm_launch_repack(const QmmLayout& L, const void* native, void* tiled
     if (n_pieces == 0) return hipSuccess;
     if (L.dtype == QMM_Q4_K)
         repack_q4k_kernel<<<grid_for(n_pieces, 256), 256, 0, stream>>>(
+            L, (const uint8_t*)native, (uint8_t*)tiled, n_pieces);
+    else if (L.dtype == QMM_Q6_K)
+        repack_q6k_kernel<<<grid_for(n_pieces, 256), 256, 0, stream>>>(
             L, (const uint8_t*)native, (uint8_t*)tiled, n_pieces);
     else
         repack_q80_kernel<<<grid_for(n_pieces, 256), 256, 0, stream>>>(
@@ -201,6 +274,11 @@ hipError_t qmm_launch_unpack(const QmmLayout& L, const void* tiled, void* native
         if (n_chunks == 0) return hipSuccess;
         unpack_q4k_kernel<<<grid_for(n_chunks, 256), 256, 0, stream>>>(
             L, (const uint8_t*)tiled, (uint8_t*)native, n_chunks);
+    } else if (L.dtype == QMM_Q6_K) {
+        int64_t n_items = L.n_stacked * L.n * L.k_units * 14;
+        if (n_items == 0) return hipSuccess;
+        unpack_q6k_kernel<<<grid_for(n_items, 256), 256, 0, stream>>>(
+            L, (const uint8_t*)tiled, (uint8_t*)native, n_items);
     } else {
         int64_t n_blocks = L.n_stacked * L.n * (L.k / 32);
         if (n_blocks == 0) return hipSuccess;
@@ -217,6 +295,11 @@ hipError_t qmm_launch_dequant(const QmmLayout& L, const void* tiled, float* out,
         if (n_chunks == 0) return hipSuccess;
         dequant_q4k_kernel<<<grid_for(n_chunks, 256), 256, 0, stream>>>(L, (const uint8_t*)tiled,
                                                                         out, n_chunks);
+    } else if (L.dtype == QMM_Q6_K) {
+        int64_t n_items = L.n_stacked * L.n * L.k_units * 64;
+        if (n_items == 0) return hipSuccess;
+        dequant_q6k_tiled_kernel<<<grid_for(n_items, 256), 256, 0, stream>>>(L, (const uint8_t*)tiled,
+                                                                              out, n_items);
     } else {
         int64_t n_chunks = L.n_stacked * L.n * (L.k / 32) * 2;
         if (n_chunks == 0) return hipSuccess;

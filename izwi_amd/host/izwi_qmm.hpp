@@ -28,9 +28,9 @@
 
 namespace izwi {
 
-enum class GgmlDType : int { Q8_0 = IZWI_QMM_Q8_0, Q4K = IZWI_QMM_Q4_K };
+enum class GgmlDType : int { Q8_0 = IZWI_QMM_Q8_0, Q4K = IZWI_QMM_Q4_K, Q6K = IZWI_QMM_Q6_K };
 inline int block_size(GgmlDType t) { return t == GgmlDType::Q8_0 ? 32 : 256; }
-inline int type_size(GgmlDType t) { return t == GgmlDType::Q8_0 ? 34 : 144; }
+inline int type_size(GgmlDType t) { return t == GgmlDType::Q8_0 ? 34 : (t == GgmlDType::Q6K ? 210 : 144); }
 
 enum class MemSpace : int { Device = IZWI_QMM_DEVICE, Host = IZWI_QMM_HOST };
 

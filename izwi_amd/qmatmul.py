@@ -22,15 +22,17 @@ from .capi import DEVICE, HOST, check, lib
 
 
 class GgmlDType(enum.IntEnum):
-    """candle_core::quantized::GgmlDType, the two block formats of the path."""
+    """candle_core::quantized::GgmlDType, the block formats of the path (Q6K: single projections
+    only, no projection-group launch and no expert stacks)."""
     Q8_0 = 8
     Q4K = 12
+    Q6K = 14
 
     def block_size(self) -> int:
         return 32 if self == GgmlDType.Q8_0 else 256
 
     def type_size(self) -> int:
-        return 34 if self == GgmlDType.Q8_0 else 144
+        return {GgmlDType.Q8_0: 34, GgmlDType.Q4K: 144, GgmlDType.Q6K: 210}[self]
 
 
 def quantized_storage_bytes(rows: int, cols: int, dtype: GgmlDType) -> int:

@@ -17,12 +17,12 @@ _LIB_PATH = os.path.join(_HERE, "liboracle_qmm.so")
 
 GGML_Q8_0 = 8
 GGML_Q4_K = 12
-GGML_Q6_K = 14  # dequantize only (GGUF ingress to dense f32)
+GGML_Q6_K = 14  # dequantize and matmul; no quantizer (tests build Q6_K blocks directly)
 BLOCK_SIZE = {GGML_Q8_0: 32, GGML_Q4_K: 256, GGML_Q6_K: 256}
 TYPE_SIZE = {GGML_Q8_0: 34, GGML_Q4_K: 144, GGML_Q6_K: 210}
 # activation-side ("vec dot") block of each weight type
-ACT_BLOCK_SIZE = {GGML_Q8_0: 32, GGML_Q4_K: 256}
-ACT_TYPE_SIZE = {GGML_Q8_0: 34, GGML_Q4_K: 292}
+ACT_BLOCK_SIZE = {GGML_Q8_0: 32, GGML_Q4_K: 256, GGML_Q6_K: 256}
+ACT_TYPE_SIZE = {GGML_Q8_0: 34, GGML_Q4_K: 292, GGML_Q6_K: 292}
 
 
 def build(force: bool = False) -> str:

@@ -26,6 +26,12 @@
  *                                    block BYTES are the input of the path.
  *   vec_dot_q8_0_q8_0 / q4_k_q8_k .. integer brute force + f64 bound + the
  *                                    reference test's known answers
+ *   dequantize_row_q6_k ............ hand-built block with all 256 closed-form values +
+ *                                    numpy restatement of the public block format
+ *   vec_dot_q6_k_q8_k .............. integer brute force from the numpy restatement of the
+ *                                    block format + f64 bound; the reference's tests hold no
+ *                                    Q6_K vector, so both Q6_K functions stay "parity
+ *                                    unpinned" against the crate's own bytes
  *   moe_* .......................... no counterpart in the reference (it has no
  *                                    MoE code); defined by the build's config and
  *                                    pinned by brute force (numpy stable argsort).
@@ -221,8 +227,7 @@ void oracle_dequantize_row_q4_k(const block_q4_k* x, float* y, int64_t k) {
 
 /* candle-core k_quants.rs, `BlockQ6K::to_float` (ggml `dequantize_row_q6_K`): per half of 128
  * elements, byte l of ql / qh carries elements l, l+32 (low nibbles of ql[l], ql[l+32]) and l+64,
- * l+96 (high nibbles); y = d * scale * (q - 32), evaluated left to right.  Load-time codec only
- * (GGUF ingress to dense f32): Q6_K is not a matmul type of this library. */
+ * l+96 (high nibbles); y = d * scale * (q - 32), evaluated left to right. */
 void oracle_dequantize_row_q6_k(const block_q6_k* x, float* y, int64_t k) {
     int64_t nb = k / QK_K;
     for (int64_t i = 0; i < nb; i++) {
@@ -439,11 +444,58 @@ float oracle_vec_dot_q4_k_q8_k(int64_t k, const block_q4_k* w, const block_q8_k*
     return sumf + tail;
 }
 
+/* candle-core k_quants.rs, `BlockQ6K::vec_dot_unopt` (ggml `ggml_vec_dot_q6_K_q8_K`, scalar
+ * path): the 256 six-bit quants are expanded to int8 (q - 32), each group of 16 is multiplied
+ * with the Q8_K quants into eight running lanes weighted by the group's int8 scale, the lanes are
+ * scaled by d_w * d_x per block and summed at the end.  The lane sums are integers below 2^24,
+ * so holding them in int32 or in f32 gives the same values. */
+float oracle_vec_dot_q6_k_q8_k(int64_t k, const block_q6_k* w, const block_q8_k* a) {
+    int64_t nb = k / QK_K;
+    int8_t aux8[QK_K];
+    int16_t aux16[8];
+    float sums[8];
+    int32_t aux32[8];
+    memset(sums, 0, sizeof sums);
+    for (int64_t i = 0; i < nb; i++) {
+        const uint8_t* q4 = w[i].ql;
+        const uint8_t* qh = w[i].qh;
+        const int8_t* q8 = a[i].qs;
+        memset(aux32, 0, sizeof aux32);
+        int8_t* ap = aux8;
+        for (int j = 0; j < QK_K; j += 128) {
+            for (int l = 0; l < 32; l++) {
+                ap[l] = (int8_t)((int)((q4[l] & 0xF) | ((qh[l] & 3) << 4)) - 32);
+                ap[l + 32] = (int8_t)((int)((q4[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32);
+                ap[l + 64] = (int8_t)((int)((q4[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32);
+                ap[l + 96] = (int8_t)((int)((q4[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32);
+            }
+            ap += 128;
+            q4 += 64;
+            qh += 32;
+        }
+        const int8_t* av = aux8;
+        for (int j = 0; j < QK_K / 16; j++) {
+            const int32_t scale = w[i].scales[j];
+            for (int r = 0; r < 2; r++) {
+                for (int l = 0; l < 8; l++) aux16[l] = (int16_t)((int16_t)q8[l] * (int16_t)av[l]);
+                for (int l = 0; l < 8; l++) aux32[l] += scale * (int32_t)aux16[l];
+                q8 += 8;
+                av += 8;
+            }
+        }
+        float d = oracle_f16_to_f32(w[i].d) * a[i].d;
+        for (int l = 0; l < 8; l++) sums[l] += d * (float)aux32[l];
+    }
+    float total = 0.0f;
+    for (int l = 0; l < 8; l++) total += sums[l];
+    return total;
+}
+
 /* ------------------------------------------------------------ matmul ----- */
 /* GGML dtype ids as the reference sees them (GgmlDType in candle-core mod.rs). */
 #define GGML_Q8_0 8
 #define GGML_Q4_K 12
-#define GGML_Q6_K 14 /* dequantize only */
+#define GGML_Q6_K 14 /* no quantizer here: tests build Q6_K blocks directly */
 
 int64_t oracle_storage_bytes(int dtype, int64_t rows, int64_t cols) {
     int64_t elems = rows * cols;
@@ -483,6 +535,20 @@ int oracle_qmatmul(int dtype, int64_t m, int64_t k, int64_t n, const float* lhs,
 #pragma omp parallel for schedule(static)
             for (int64_t c = 0; c < n; c++)
                 dst[r * n + c] = oracle_vec_dot_q4_k_q8_k(k, w + c * kb, lb + r * kb);
+        }
+        free(lb);
+        return 0;
+    }
+    if (dtype == GGML_Q6_K) {
+        if (k % QK_K) return -1;
+        int64_t kb = k / QK_K;
+        block_q8_k* lb = (block_q8_k*)calloc((size_t)(m * kb), sizeof(block_q8_k));
+        for (int64_t r = 0; r < m; r++) oracle_quantize_row_q8_k(lhs + r * k, lb + r * kb, k);
+        const block_q6_k* w = (const block_q6_k*)rhs_t;
+        for (int64_t r = 0; r < m; r++) {
+#pragma omp parallel for schedule(static)
+            for (int64_t c = 0; c < n; c++)
+                dst[r * n + c] = oracle_vec_dot_q6_k_q8_k(k, w + c * kb, lb + r * kb);
         }
         free(lb);
         return 0;
@@ -546,7 +612,7 @@ int oracle_quantize_activations(int weight_dtype, int64_t m, int64_t k, const fl
             oracle_quantize_row_q8_0(x + r * k, (block_q8_0*)out + r * (k / QK8_0), k);
         return 0;
     }
-    if (weight_dtype == GGML_Q4_K) {
+    if (weight_dtype == GGML_Q4_K || weight_dtype == GGML_Q6_K) { /* both dot types are Q8_K */
         if (k % QK_K) return -1;
         memset(out, 0, (size_t)(m * (k / QK_K)) * sizeof(block_q8_k));
         for (int64_t r = 0; r < m; r++)

@@ -63,9 +63,11 @@ static void host_logic() {
     EXPECT(throws(izwi::Error::Kind::InvalidInput, "not divisible by block size",
                   [] { izwi::quantized_storage_bytes(3, 100, GgmlDType::Q4K); }));
     EXPECT(throws(izwi::Error::Kind::ModelLoadError, "not supported",
-                  [] { izwi::quantized_storage_bytes(4, 256, (GgmlDType)14); }));
+                  [] { izwi::quantized_storage_bytes(4, 256, (GgmlDType)13); }));
     EXPECT(izwi::block_size(GgmlDType::Q4K) == 256 && izwi::type_size(GgmlDType::Q4K) == 144);
     EXPECT(izwi::block_size(GgmlDType::Q8_0) == 32 && izwi::type_size(GgmlDType::Q8_0) == 34);
+    EXPECT(izwi::block_size(GgmlDType::Q6K) == 256 && izwi::type_size(GgmlDType::Q6K) == 210);
+    EXPECT(izwi::quantized_storage_bytes(4096, 12288, GgmlDType::Q6K) == 4096u * 48u * 210u);
 }
 
 static void no_device_is_loud() {

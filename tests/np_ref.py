@@ -46,24 +46,39 @@ def dequant_q4_k(blocks: np.ndarray, rows: int, cols: int) -> np.ndarray:
     return y.astype(np.float32).reshape(rows, cols)
 
 
-def dequant_q6_k(blocks: np.ndarray, rows: int, cols: int) -> np.ndarray:
-    """Q6_K blocks (ql[128], qh[64], int8 scales[16], f16 d = 210 B) -> f32, vectorized from the
-    public block format: element 128 h + 32 g + l of a block has the quant
-    (nibble g % 2 of ql[64 h + 32 (g // 2)... see below) and scale index 8 h + 2 g + l // 16."""
+def q6_k_fields(blocks: np.ndarray):
+    """Q6_K blocks (ql[128], qh[64], int8 scales[16], f16 d = 210 B) -> (d f32 [blk], scales int8
+    [blk, 16], q int32 [blk, 256] in element order, already minus 32), from the public block format:
+    element 128 h + 32 g + l of a block (g < 4, l < 32) takes nibble g // 2 of ql[64 h + 32 (g % 2) + l]
+    and bits 2 g, 2 g + 1 of qh[32 h + l]; scale j belongs to the elements 16 j .. 16 j + 15."""
     b = np.ascontiguousarray(blocks, dtype=np.uint8).reshape(-1, 210)
     ql = b[:, :128].reshape(-1, 2, 2, 32)           # [blk, half, which 32 bytes, l]
     qh = b[:, 128:192].reshape(-1, 2, 32)           # [blk, half, l]
-    sc = b[:, 192:208].view(np.int8).reshape(-1, 2, 8).astype(np.float32)
+    sc = b[:, 192:208].view(np.int8)
     d = b[:, 208:210].copy().view(np.float16).astype(np.float32).reshape(-1)
-    # groups g = 0..3 of a half: (ql bytes 0..31 low nibble, bytes 32..63 low, 0..31 high, 32..63 high)
     lo = np.stack([ql[:, :, 0] & 0xF, ql[:, :, 1] & 0xF, ql[:, :, 0] >> 4, ql[:, :, 1] >> 4], axis=2)
     hi = np.stack([(qh >> (2 * g)) & 3 for g in range(4)], axis=2)
     q = (lo | (hi << 4)).astype(np.int32) - 32       # [blk, half, g, l]
-    l16 = (np.arange(32) // 16)
-    scale = np.stack([sc[:, :, 2 * g + l16] for g in range(4)], axis=2)  # [blk, half, g, l]
-    ds = (d[:, None, None, None] * scale).astype(np.float32)             # one rounding
+    return d, sc, q.reshape(-1, 256)
+
+
+def dequant_q6_k(blocks: np.ndarray, rows: int, cols: int) -> np.ndarray:
+    d, sc, q = q6_k_fields(blocks)
+    scale = np.repeat(sc.astype(np.float32), 16, axis=1)                 # [blk, 256]
+    ds = (d[:, None] * scale).astype(np.float32)                         # one rounding
     y = (ds * q.astype(np.float32)).astype(np.float32)                   # one rounding
     return y.reshape(rows, cols)
+
+
+def random_q6_k_blocks(seed: int, rows: int, cols: int, d_scale: float = 1e-3) -> np.ndarray:
+    """Random but well-formed Q6_K bytes for a [rows, cols] tensor: every quant and scale value
+    occurs, d is a finite positive f16 around d_scale (weights of order 0.02 .. 0.1)."""
+    rng = np.random.default_rng(seed)
+    nb = rows * cols // 256
+    b = rng.integers(0, 256, size=(nb, 210), dtype=np.uint8)
+    d = (d_scale * rng.uniform(0.5, 2.0, size=nb)).astype(np.float16)
+    b[:, 208:210] = d.view(np.uint8).reshape(nb, 2)
+    return b.reshape(-1)
 
 
 def quant_act_q8_0(x: np.ndarray):
@@ -107,6 +122,18 @@ def qmatmul_int(dtype: int, x: np.ndarray, blocks: np.ndarray, n: int) -> np.nda
             qx = qx.reshape(k // 32, 32).astype(np.int64)
             sumi = np.einsum("nbj,bj->nb", qw, qx)
             y[r] = (sumi * dw * dx.astype(np.float64)[None, :]).sum(axis=1)
+        return y
+    if dtype == 14:
+        nb = k // 256
+        d, sc, q = q6_k_fields(blocks)
+        d = d.reshape(n, nb).astype(np.float64)
+        sc = sc.reshape(n, nb, 16).astype(np.int64)
+        q = q.reshape(n, nb, 16, 16).astype(np.int64)
+        for r in range(m):
+            dx, qx = quant_act_q8_k(x[r])
+            qx = qx.reshape(nb, 16, 16).astype(np.int64)
+            dots = np.einsum("nbsj,bsj->nbs", q, qx)
+            y[r] = ((dots * sc).sum(axis=2) * d * dx.astype(np.float64)[None, :]).sum(axis=1)
         return y
     d, dmin, sc, mn, q = q4_k_fields(blocks)
     nb = k // 256

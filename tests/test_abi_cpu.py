@@ -48,7 +48,8 @@ def test_abi_version_and_storage_bytes_rule(capi):
     assert L.izwi_qmm_storage_bytes(12, 151936, 4096, C.byref(out)) == 0 and out.value == 350_060_544
     assert L.izwi_qmm_storage_bytes(12, 3, 100, C.byref(out)) == -1
     assert b"not divisible by block size 256" in L.izwi_qmm_last_error()
-    assert L.izwi_qmm_storage_bytes(14, 4, 256, C.byref(out)) == -2  # Q6_K: not built yet
+    assert L.izwi_qmm_storage_bytes(14, 4, 256, C.byref(out)) == 0 and out.value == 4 * 210  # Q6_K
+    assert L.izwi_qmm_storage_bytes(13, 4, 256, C.byref(out)) == -2  # Q5_K: no kernel for it
     assert L.izwi_qmm_storage_bytes(8, -1, 32, C.byref(out)) == -1
 
 

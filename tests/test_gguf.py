@@ -8,6 +8,8 @@ import os
 import struct
 
 import numpy as np
+
+import np_ref
 import pytest
 
 import gguf_writer as gw
@@ -285,30 +287,37 @@ def test_committed_fixture_dequantizes_to_its_closed_form(qa):
 
 
 @pytest.mark.gpu
-def test_q6_k_tensors_load_as_dense_f32(qa, oracle, tmp_path):
+def test_q6_k_tensors_load_dense_and_as_projections(qa, oracle, tmp_path):
     """Q4_K_M files keep some tensors in Q6_K: they are listed with shape, type and size, load as
-    dense f32 bit-exactly (device kernel against the oracle's BlockQ6K::to_float) and are refused
-    as projections."""
+    dense f32 bit-exactly (device kernel against the oracle's BlockQ6K::to_float) and as projections;
+    a type the library has no kernel for (Q5_K) is refused."""
+    import torch
     from izwi_amd.capi import QmmError
-    rng = np.random.default_rng(16)
     n, k = 24, 1024
     nb = n * k // 256
-    b = rng.integers(0, 256, nb * 210, dtype=np.uint8).reshape(nb, 210)
-    b[:, 208:210] = (rng.standard_normal(nb) * 0.02).astype(np.float16).view(np.uint8).reshape(nb, 2)
+    b = np_ref.random_q6_k_blocks(16, n, k).reshape(nb, 210)
     hand = bytes.fromhex(json.load(open(os.path.join(HERE, "golden", "q6k_hand_block.json")))["block_hex"])
     path = str(tmp_path / "q6.gguf")
-    gw.write_gguf(path, [], [("blk.0.ffn_down.weight", (n, k), 14, b.tobytes()), ("hand", (1, 256), 14, hand)])
+    gw.write_gguf(path, [], [("blk.0.ffn_down.weight", (n, k), 14, b.tobytes()), ("hand", (1, 256), 14, hand),
+                             ("q5", (2, 256), 13, bytes(2 * 176))])
     g = qa.GgufLoader.from_path(path)
     assert g.tensor_dtype("blk.0.ffn_down.weight") == 14 and g._info("blk.0.ffn_down.weight").nbytes == nb * 210
-    assert g.get_model_info().quantization == "Q6K"
+    assert g.get_model_info().quantization == "mixed:Q5K,Q6K"
     want = oracle.dequantize(14, b.reshape(-1), n, k)
     for device in ("cuda", "cpu"):
         got = g.load_tensor("blk.0.ffn_down.weight", device=device).cpu().numpy()
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     fx = json.load(open(os.path.join(HERE, "golden", "q6k_hand_block.json")))
     assert np.array_equal(g.load_tensor("hand").cpu().numpy().reshape(-1), np.array(fx["expected_f32"], dtype=np.float32))
+    q = g.load_qtensor("blk.0.ffn_down.weight")
+    assert q.dtype() == qa.GgmlDType.Q6K and q.shape() == (n, k) and np.array_equal(q.data(), b.reshape(-1))
+    assert np.array_equal(q.dequantize().cpu().numpy().view(np.uint32), want.view(np.uint32))
+    x = oracle.randn(17, (2, k))
+    y = qa.QMatMul.from_qtensor(q).forward(torch.from_numpy(x).cuda()).cpu().numpy()
+    ref = oracle.qmatmul(14, x, b.reshape(-1), n)
+    assert np.abs(y - ref).max() <= 1e-4 * np.abs(ref).max()
     with pytest.raises(QmmError) as e:
-        g.load_qtensor("blk.0.ffn_down.weight")
+        g.load_qtensor("q5")
     assert e.value.code == -2
 
 

@@ -1,0 +1,157 @@
+"""GPU parity of the Q6_K block format (pytest -m gpu): weight bytes and dequantization bit-exact,
+decode within 1e-4 and prefill within 1e-2 of the CPU oracle, through the C ABI.
+
+Q6_K weights are built from random block bytes (the oracle has no Q6_K quantizer): every six-bit
+quant, bit pair and signed scale occurs, d is a finite f16 around 1e-3."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import np_ref
+
+pytestmark = pytest.mark.gpu
+
+Q4_K, Q6_K = 12, 14
+DECODE_TOL = 1e-4
+PREFILL_TOL = 1e-2
+
+
+def _say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def qa():
+    if not torch.cuda.is_available():
+        pytest.fail("no GPU visible: the HIP path cannot run (there is no fallback)")
+    import izwi_amd
+    izwi_amd.lib()
+    torch.cuda.set_device(0)
+    return izwi_amd
+
+
+def rel_err(y, want):
+    return float(np.abs(y.astype(np.float64) - want).max() / max(np.abs(want).max(), 1e-30))
+
+
+@pytest.mark.parametrize("n,k", [(16, 256), (5, 512), (33, 768), (64, 1024), (40, 1280), (128, 4096), (17, 12288)])
+def test_q6_k_dequantize_and_data_bit_exact(qa, oracle, n, k):
+    _say(f"q6k dequant n={n} k={k}")
+    blocks = np_ref.random_q6_k_blocks(n + k, n, k)
+    q = qa.QTensor.from_blocks(qa.GgmlDType.Q6K, blocks, (n, k))
+    got = q.dequantize().cpu().numpy()
+    want = oracle.dequantize(Q6_K, blocks, n, k)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(got.view(np.uint32), np_ref.dequant_q6_k(blocks, n, k).view(np.uint32))
+    assert np.array_equal(q.data(), blocks)
+    assert qa.quantized_storage_bytes(n, k, qa.GgmlDType.Q6K) == blocks.size
+
+
+def test_q6_k_hand_block_on_device(qa):
+    import json
+    import os
+    fx = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "q6k_hand_block.json")))
+    blk = np.frombuffer(bytes.fromhex(fx["block_hex"]), np.uint8)
+    q = qa.QTensor.from_blocks(qa.GgmlDType.Q6K, blk, (1, 256))
+    assert np.array_equal(q.dequantize().cpu().numpy().reshape(-1), np.array(fx["expected_f32"], dtype=np.float32))
+
+
+def test_q6_k_activation_blocks_are_q8_k(qa, oracle):
+    x = oracle.randn(5, (3, 1024))
+    got = qa.quantize_activations(qa.GgmlDType.Q6K, torch.from_numpy(x).cuda()).cpu().numpy()
+    assert np.array_equal(got, oracle.quantize_activations(Q6_K, x))
+
+
+@pytest.mark.parametrize("n,k,m", [(1, 256, 1), (15, 256, 2), (17, 512, 3), (100, 768, 5), (250, 1280, 7),
+                                   (64, 1024, 16), (130, 2048, 33), (48, 4096, 64), (31, 12288, 4)])
+def test_q6_k_decode_ragged_shapes(qa, oracle, n, k, m):
+    _say(f"q6k decode n={n} k={k} m={m}")
+    blocks = np_ref.random_q6_k_blocks(7 * n + k + m, n, k)
+    x = oracle.randn(n + k + m, (m, k))
+    mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q6K, blocks, (n, k)))
+    y = mm.forward(torch.from_numpy(x).cuda()).cpu().numpy()
+    want = oracle.qmatmul(Q6_K, x, blocks, n)
+    assert y.shape == (m, n)
+    assert rel_err(y, want) <= DECODE_TOL
+    # and against the integer dot products of the independent numpy reading of the format
+    assert rel_err(y, np_ref.qmatmul_int(Q6_K, x, blocks, n)) <= DECODE_TOL
+
+
+@pytest.mark.parametrize("n,k", [(4096, 12288), (1024, 4096), (151936 // 8, 4096)])
+@pytest.mark.parametrize("m", [1, 2])
+def test_q6_k_decode_8b_shapes(qa, oracle, n, k, m):
+    """The tensors a Q4_K_M file of the 8B model keeps in Q6_K: ffn_down, attn_v and (an eighth
+    of) the output matrix."""
+    _say(f"q6k 8B n={n} k={k} m={m}")
+    blocks = np_ref.random_q6_k_blocks(n + m, n, k)
+    x = oracle.randn(n + k, (m, k))
+    mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q6K, blocks, (n, k)))
+    xd = torch.from_numpy(x).cuda()
+    y = mm.forward(xd)
+    assert torch.equal(y, mm.forward(xd))  # repeatable bit for bit
+    want = oracle.qmatmul(Q6_K, x, blocks, n)
+    assert rel_err(y.cpu().numpy(), want) <= DECODE_TOL
+    # scaling the activations by a power of two scales the result exactly
+    assert torch.equal(mm.forward(xd * 4.0), y * 4.0)
+
+
+def test_q6_k_rows_are_independent(qa, oracle):
+    n, k = 96, 2048
+    blocks = np_ref.random_q6_k_blocks(3, n, k)
+    mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q6K, blocks, (n, k)))
+    x = torch.from_numpy(oracle.randn(4, (7, k))).cuda()
+    y = mm.forward(x)
+    for r in range(7):
+        assert rel_err(mm.forward(x[r:r + 1].contiguous()).cpu().numpy(), y[r:r + 1].cpu().numpy().astype(np.float64)) <= 2e-6
+
+
+@pytest.mark.parametrize("m,n,k", [(512, 1024, 4096), (300, 200, 768), (65, 256, 1024), (129, 144, 1280), (70, 16, 256)])
+def test_q6_k_prefill_against_oracle(qa, oracle, m, n, k):
+    _say(f"q6k prefill m={m} n={n} k={k}")
+    blocks = np_ref.random_q6_k_blocks(m + n, n, k)
+    xb = torch.from_numpy(oracle.randn(m + k, (m, k))).cuda().to(torch.bfloat16)
+    xf = xb.float().cpu().numpy()
+    mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q6K, blocks, (n, k)))
+    y = mm.forward_bf16_to_f32(xb).cpu().numpy()
+    yb = mm.forward(xb)
+    assert yb.dtype == torch.bfloat16
+    # (a) the kernel's own arithmetic: exact bf16 activations x bf16-rounded dequantized weights
+    dense = xf.astype(np.float64) @ oracle.dequantize(Q6_K, blocks, n, k).astype(np.float64).T
+    assert rel_err(y, dense) < 4e-3
+    assert rel_err(yb.float().cpu().numpy(), dense) < 1e-2
+    # f32 activations with m > 64 take the same kernel after one conversion
+    assert torch.equal(mm.forward(xb.float()), torch.from_numpy(y).cuda())
+    # (b) the reference's CPU result, which also carries its int8 activation rounding (about 0.5 %
+    # of the output scale): the 1e-2 bar where the output row is long enough for max|y_ref| to
+    # stand above that noise's tail
+    if n >= 128:
+        assert rel_err(y, oracle.qmatmul(Q6_K, xf, blocks, n)) < PREFILL_TOL
+
+
+def test_q6_k_in_groups_and_mlp(qa, oracle):
+    """A projection group or a gate/up pair with a Q6_K member runs projection by projection and
+    gives the results of separate calls; expert stacks of Q6_K are refused."""
+    from izwi_amd.capi import QmmError
+    k, n = 1024, 512
+    b6 = np_ref.random_q6_k_blocks(1, n, k)
+    b4 = oracle.quantize(Q4_K, oracle.randn(2, (n, k), std=0.02))
+    w6 = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q6K, b6, (n, k)))
+    w4 = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q4K, b4, (n, k)))
+    gu = qa.Qwen3GateUpProjection.new_separate(w6, w6)
+    for m in (1, 5, 80):
+        x = torch.from_numpy(oracle.randn(10 + m, (m, k))).cuda()
+        ys = qa.forward_group([w4, w6, w6], x)
+        assert torch.equal(ys[0], w4.forward(x)) and torch.equal(ys[1], w6.forward(x)) and torch.equal(ys[2], ys[1])
+        g = w6.forward(x)
+        assert torch.allclose(gu.forward_silu_mul(x), torch.nn.functional.silu(g) * g, rtol=1e-5, atol=1e-6)
+    stack = lambda seed, rows, cols: qa.QTensor.from_blocks(  # noqa: E731
+        qa.GgmlDType.Q6K, np_ref.random_q6_k_blocks(seed, 2 * rows, cols), (2, rows, cols))
+    experts = qa.MoeExperts(stack(5, n, k), stack(6, n, k), stack(7, k, n))
+    ids = torch.zeros(1, 1, dtype=torch.int32, device="cuda")
+    perm, offsets = qa.moe_sort(ids, 2)
+    with pytest.raises(QmmError) as e:
+        experts.forward(torch.zeros(1, k, device="cuda"), ids, torch.ones(1, 1, device="cuda"), perm, offsets)
+    assert e.value.code == -2

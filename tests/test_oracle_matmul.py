@@ -6,7 +6,7 @@ import pytest
 
 import np_ref
 
-Q8_0, Q4_K = 8, 12
+Q8_0, Q4_K, Q6_K = 8, 12, 14
 
 
 def reference_packed_case():
@@ -72,6 +72,61 @@ def test_q4_k_min_term_sign_and_scale(oracle):
     blk2 = bytes([0x00, 0x3C, 0x00, 0x38]) + scales + bytes(qs)
     y2 = oracle.qmatmul(Q4_K, x, np.frombuffer(blk2, np.uint8), 1)
     assert y2[0, 0] == y[0, 0] + 4 * 9
+
+
+@pytest.mark.parametrize("k", [256, 768, 1024])
+def test_q6_k_matmul_equals_integer_brute_force(oracle, k):
+    """The reference's tests hold no Q6_K vector: the oracle's vec_dot is held to the integer dot
+    products of an independent numpy reading of the public block format (random block bytes, so
+    every quant, bit pair and signed scale occurs) and to the dense product of the dequantized
+    weights."""
+    n, m = 40, 3
+    blocks = np_ref.random_q6_k_blocks(500 + k, n, k)
+    x = oracle.randn(600 + k, (m, k))
+    y = oracle.qmatmul(Q6_K, x, blocks, n)
+    want = np_ref.qmatmul_int(Q6_K, x, blocks, n)
+    assert np.abs(y - want).max() <= 2e-6 * np.abs(want).max()
+    dense = x.astype(np.float64) @ oracle.dequantize(Q6_K, blocks, n, k).astype(np.float64).T
+    assert np.abs(y - dense).max() <= 1e-2 * np.abs(dense).max()
+    # activations of a Q6_K weight are Q8_K blocks, the same bytes as for Q4_K
+    assert np.array_equal(oracle.quantize_activations(Q6_K, x), oracle.quantize_activations(Q4_K, x))
+
+
+def test_q6_k_closed_form_single_elements(oracle):
+    """One block, d = 1, x = 1 everywhere (quantizes to -128 with d_x = -1/128, exact): y is the sum of
+    scale_j * (q - 32) over the block, worked out by hand for a few byte patterns."""
+    x = np.ones((1, 256), np.float32)
+
+    def block(ql=None, qh=None, scales=None):
+        b = bytearray(210)
+        b[0:128] = ql if ql is not None else bytes(128)
+        b[128:192] = qh if qh is not None else bytes(64)
+        b[192:208] = bytes((s & 0xFF) for s in (scales if scales is not None else [1] * 16))
+        b[208:210] = bytes([0x00, 0x3C])  # f16 1.0
+        return np.frombuffer(bytes(b), np.uint8)
+
+    # all quants zero: every element is -32, scales all 1 -> -32 * 256
+    assert oracle.qmatmul(Q6_K, x, block(), 1)[0, 0] == -32.0 * 256
+    # scales j = j - 8 (signed): sum_j (j - 8) * 16 * (-32)
+    sc = [j - 8 for j in range(16)]
+    assert oracle.qmatmul(Q6_K, x, block(scales=sc), 1)[0, 0] == -32.0 * 16 * sum(sc)
+    # high nibble of ql[32 + 5] = 0xA: element 96 + 5 of the first half (group 6), scale 3 there
+    ql = bytearray(128)
+    ql[37] = 0xA0
+    sc = [1] * 16
+    sc[6] = 3
+    base = -32.0 * 16 * sum(sc)
+    assert oracle.qmatmul(Q6_K, x, block(ql=bytes(ql), scales=sc), 1)[0, 0] == base + 3 * 10
+    # bits 4, 5 of qh[32 + 20] = 0b10: element 128 + 64 + 20 (group 8 + 5), adds 2 << 4 = 32
+    qh = bytearray(64)
+    qh[52] = 0x20
+    sc = [1] * 16
+    sc[13] = -7
+    base = -32.0 * 16 * sum(sc)
+    assert oracle.qmatmul(Q6_K, x, block(qh=bytes(qh), scales=sc), 1)[0, 0] == base + (-7) * 32
+    # and the dequantized block says the same about that element
+    w = oracle.dequantize(Q6_K, block(qh=bytes(qh), scales=sc), 1, 256)[0]
+    assert w[128 + 64 + 20] == 0.0 and w[128 + 64 + 21] == -7 * -32.0
 
 
 def test_rows_are_independent_and_m_loops(oracle):
