@@ -54,7 +54,7 @@ typedef enum izwi_qmm_status {
 
 typedef enum izwi_qmm_mem_space { IZWI_QMM_DEVICE = 0, IZWI_QMM_HOST = 1 } izwi_qmm_mem_space;
 
-/* element type of y in izwi_qmm_forward_bf16 */
+/* element type of y in izwi_qmm_forward_bf16, of x and y in izwi_qmm_forward_fused */
 typedef enum izwi_qmm_out_dtype { IZWI_QMM_OUT_F32 = 0, IZWI_QMM_OUT_BF16 = 1 } izwi_qmm_out_dtype;
 
 typedef struct izwi_qmm_weight izwi_qmm_weight; /* opaque: QTensor + QMatMul */
@@ -183,6 +183,21 @@ int izwi_qmm_forward_gate_up_silu_f32(const izwi_qmm_weight* gate, const izwi_qm
  * qwen3/core.rs:798-828 with one kernel. */
 int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int64_t m, void* y,
                           int out_dtype, int mem_space, void* stream);
+
+/* `Qwen3Projection::forward`, `Quantized` arm (qwen3/core.rs:795-829), with the residual add of
+ * `Qwen3Layer::forward` (qwen3/core.rs:1875, 1879) folded in: the cast of the activations to f32,
+ * the product, the cast of the result back to the activation type and `x.broadcast_add(&out)` as
+ * ONE call whose kernels read x in its own type and store y once.
+ *   x: `[m, k]` of x_dtype; y: `[m, n]` of y_dtype (izwi_qmm_out_dtype values: f32 = 0, bf16 = 1);
+ *   residual: `[m, n]` of y_dtype or NULL; it may be y itself (each element is read before it is
+ *   written by the same thread).
+ * The sums are those of izwi_qmm_forward_f32 on the widened activations, bit for bit, for m <= 64
+ * (bf16 -> f32 is exact), those of izwi_qmm_forward_bf16 beyond; y = sum + residual is rounded
+ * once (the reference rounds the product to the activation type first and the sum again).  The
+ * profile snapshot counts the folded casts (`qmatmul_input_casts` for bf16 x, `qmatmul_output_casts`
+ * for bf16 y); their time is inside `qmatmul_ns`, the `_cast_ns` fields stay 0. */
+int izwi_qmm_forward_fused(const izwi_qmm_weight* w, const void* x, int x_dtype, int64_t m,
+                           const void* residual, void* y, int y_dtype, int mem_space, void* stream);
 
 /* `T::VecDotType::from_float` per row (candle-core k_quants.rs `matmul`):
  * the activation blocks the decode kernel builds on chip, written out in the

@@ -61,6 +61,7 @@ PROTOTYPES = {
     "izwi_qmm_forward_group_f32": (C.c_int, [_vp, _i32, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_gate_up_silu_f32": (C.c_int, [_vp, _vp, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_bf16": (C.c_int, [_vp, _vp, _i64, _vp, C.c_int, C.c_int, _vp]),
+    "izwi_qmm_forward_fused": (C.c_int, [_vp, _vp, C.c_int, _i64, _vp, _vp, C.c_int, C.c_int, _vp]),
     "izwi_qmm_quantize_activations": (C.c_int, [C.c_int, _vp, _i64, _i64, _vp, C.c_int, _vp]),
     "izwi_moe_route": (C.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, C.c_int, _vp]),
     "izwi_moe_sort": (C.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, C.c_int, _vp]),

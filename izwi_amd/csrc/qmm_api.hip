@@ -677,6 +677,77 @@ int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int6
     return IZWI_QMM_OK;
 }
 
+int izwi_qmm_forward_fused(const izwi_qmm_weight* w, const void* x, int x_dtype, int64_t m,
+                           const void* residual, void* y, int y_dtype, int mem_space, void* stream_) {
+    if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    if (int rc = check_space(mem_space)) return rc;
+    if ((x_dtype != IZWI_QMM_OUT_F32 && x_dtype != IZWI_QMM_OUT_BF16) ||
+        (y_dtype != IZWI_QMM_OUT_F32 && y_dtype != IZWI_QMM_OUT_BF16))
+        return fail(IZWI_QMM_ERR_INVALID, "bad x_dtype %d / y_dtype %d (f32 = 0, bf16 = 1)", x_dtype, y_dtype);
+    const QmmLayout& L = w->layout;
+    if (L.n_stacked != 1) return fail(IZWI_QMM_ERR_INVALID, "forward on an expert stack");
+    if (m < 0) return fail(IZWI_QMM_ERR_INVALID, "negative m");
+    if (m == 0 || L.n == 0) return IZWI_QMM_OK;
+    if (!x) return fail(IZWI_QMM_ERR_INVALID, "x is NULL");
+    if (!y) return fail(IZWI_QMM_ERR_INVALID, "y is NULL");
+    hipStream_t stream = (hipStream_t)stream_;
+    const bool x_bf16 = x_dtype == IZWI_QMM_OUT_BF16, y_bf16 = y_dtype == IZWI_QMM_OUT_BF16;
+    if (profiling()) {
+        // the casts of Qwen3Projection::forward happen inside the kernels: counted, their time is
+        // part of qmatmul_ns
+        if (x_bf16) g_in_casts.fetch_add(1, std::memory_order_relaxed);
+        if (y_bf16) g_out_casts.fetch_add(1, std::memory_order_relaxed);
+    }
+    ProfileScope prof(w, stream);
+    const size_t xbytes = (size_t)m * L.k * (x_bf16 ? 2 : 4), ybytes = (size_t)m * L.n * (y_bf16 ? 2 : 4);
+    Staged xi, ri, yo;
+    HIP_TRY(xi.in(x, xbytes, mem_space));
+    if (residual) HIP_TRY(ri.in(residual, ybytes, mem_space));
+    HIP_TRY(yo.out(y, ybytes, mem_space));
+    QmmIo io{x_bf16 ? 1 : 0, residual ? ri.dev : nullptr, y_bf16 ? 1 : 0};
+    if (m < mfma_min_m() || (L.dtype == IZWI_QMM_Q6_K && m <= 64)) {
+        const float* xf = (const float*)xi.dev;
+        if (x_bf16 && m > 2) { // this kernel reads bf16 rows only in its one- and two-row forms
+            void* wide = nullptr;
+            HIP_TRY(get_scratch(w->device, stream, (size_t)m * L.k * sizeof(float), &wide));
+            HIP_TRY(qmm_launch_bf16_to_f32((const uint16_t*)xi.dev, (float*)wide, m * L.k, stream));
+            xf = (const float*)wide;
+            io.x_bf16 = 0;
+        }
+        HIP_TRY(qmm_launch_gemv(L, w->tiled, xf, m, (float*)yo.dev, w->n_cus, stream, &io));
+    } else if (m <= 64) {
+        const size_t ws_bytes = (qmm_gemv_mfma_workspace_bytes(L, m) + 255) & ~(size_t)255;
+        void* scratch = nullptr;
+        HIP_TRY(get_scratch(w->device, stream, ws_bytes + (size_t)m * L.n * sizeof(float), &scratch));
+        hipError_t e = qmm_launch_gemv_mfma(L, w->tiled, (const float*)xi.dev, m, (float*)yo.dev, scratch, w->n_cus,
+                                            stream, true, &io);
+        if (e == hipErrorNotSupported) {
+            // (very tall matrix with k beyond one activation window) sums into scratch, then the epilogue
+            (void)hipGetLastError();
+            float* sums = reinterpret_cast<float*>(static_cast<uint8_t*>(scratch) + ws_bytes);
+            const QmmIo plain{io.x_bf16, nullptr, 0};
+            e = qmm_launch_gemv_mfma(L, w->tiled, (const float*)xi.dev, m, sums, scratch, w->n_cus, stream, true, &plain);
+            if (e == hipSuccess) e = qmm_launch_epilogue(sums, io.residual, yo.dev, io.y_bf16, m * L.n, stream);
+        }
+        if (e != hipSuccess) return fail_hip(e, "batched decode kernel");
+    } else {
+        const size_t xb_bytes = x_bf16 ? 0 : ((((size_t)m * L.k * sizeof(uint16_t)) + 255) & ~(size_t)255);
+        const size_t ws_bytes = qmm_gemm_workspace_bytes(L, m, w->n_cus);
+        void* scratch = nullptr;
+        if (xb_bytes + ws_bytes) HIP_TRY(get_scratch(w->device, stream, xb_bytes + ws_bytes, &scratch));
+        const uint16_t* xb = (const uint16_t*)xi.dev;
+        if (!x_bf16) {
+            HIP_TRY(qmm_launch_f32_to_bf16((const float*)xi.dev, (uint16_t*)scratch, m * L.k, stream));
+            xb = (const uint16_t*)scratch;
+        }
+        HIP_TRY(qmm_launch_gemm_bf16(L, w->tiled, xb, m, yo.dev, io.y_bf16,
+                                     ws_bytes ? static_cast<uint8_t*>(scratch) + xb_bytes : nullptr, w->n_cus, stream,
+                                     io.residual));
+    }
+    HIP_TRY(yo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
 int izwi_moe_route(const float* logits, int64_t t, int32_t n_experts, int32_t top_k, int32_t* ids,
                    float* weights, int mem_space, void* stream_) {
     if (int rc = check_space(mem_space)) return rc;

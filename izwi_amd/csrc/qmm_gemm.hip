@@ -57,6 +57,7 @@ struct GemmParams {
     // mask it emits one AND per four weights and v_cvt_f32_ubyteN for each
     uint32_t nibble_mask;
     float* partial;
+    const void* residual; // of y's type, added to the sums before they are stored (may alias y)
 };
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
@@ -333,10 +334,7 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams P) {
             for (int r = 0; r < 16; r++) {
                 const int64_t gm = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 if (gm >= P.m) continue;
-                if (P.out_bf16)
-                    reinterpret_cast<uint16_t*>(P.y)[gm * P.n + gn] = qmm_f32_to_bf16_bits(acc[i][j][r]);
-                else
-                    reinterpret_cast<float*>(P.y)[gm * P.n + gn] = acc[i][j][r];
+                qmm_store(P.y, QmmEpilogue{P.residual, P.out_bf16}, gm * P.n + gn, acc[i][j][r]);
             }
         }
     }
@@ -658,7 +656,6 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
 
     // a split-k slice stores f32 into its own [m, n] plane of the workspace
     float* out_f32 = P.partial ? P.partial + (int64_t)blockIdx.y * P.m * P.n : reinterpret_cast<float*>(P.y);
-    const bool out_bf16 = P.partial == nullptr && P.out_bf16 != 0;
 #pragma unroll
     for (int i = 0; i < MT; i++) {
 #pragma unroll
@@ -669,10 +666,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
             for (int r = 0; r < 16; r++) {
                 const int64_t gm = m0 + wm * (BM / WM) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 if (gm >= P.m) continue;
-                if (out_bf16)
-                    reinterpret_cast<uint16_t*>(P.y)[gm * P.n + gn] = qmm_f32_to_bf16_bits(acc[i][j][r]);
-                else
-                    out_f32[gm * P.n + gn] = acc[i][j][r];
+                if (P.partial) out_f32[gm * P.n + gn] = acc[i][j][r]; // a slice: the second kernel finishes
+                else qmm_store(P.y, QmmEpilogue{P.residual, P.out_bf16}, gm * P.n + gn, acc[i][j][r]);
             }
         }
     }
@@ -681,15 +676,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
 // out[i] = sum over slices (in order) of partial[s][i], as f32 or bf16; i runs over the
 // columns [n_begin, n_end) of all rows
 __global__ void splitk_reduce_kernel(const float* __restrict__ partial, int slices, int64_t m, int64_t n,
-                                     int64_t n_begin, int64_t n_end, void* __restrict__ y, int out_bf16) {
+                                     int64_t n_begin, int64_t n_end, void* y, int out_bf16, const void* residual) {
     const int64_t width = n_end - n_begin;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= m * width) return;
     const int64_t row = idx / width, col = n_begin + (idx - row * width);
     float sum = 0.0f;
     for (int s = 0; s < slices; s++) sum += partial[((int64_t)s * m + row) * n + col];
-    if (out_bf16) reinterpret_cast<uint16_t*>(y)[row * n + col] = qmm_f32_to_bf16_bits(sum);
-    else reinterpret_cast<float*>(y)[row * n + col] = sum;
+    qmm_store(y, QmmEpilogue{residual, out_bf16}, row * n + col, sum);
 }
 
 __global__ void f32_to_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ out,
@@ -704,6 +698,17 @@ __global__ void f32_to_bf16_kernel(const float* __restrict__ x, uint16_t* __rest
     } else {
         for (; i < count; i++) out[i] = qmm_f32_to_bf16_bits(x[i]);
     }
+}
+
+__global__ void epilogue_kernel(const float* __restrict__ t, const void* residual, void* y, int y_bf16,
+                                int64_t count) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) qmm_store(y, QmmEpilogue{residual, y_bf16}, i, t[i]);
+}
+
+__global__ void bf16_to_f32_kernel(const uint16_t* __restrict__ x, float* __restrict__ out, int64_t count) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) out[i] = qmm_bf16_bits_to_f32(x[i]);
 }
 
 template <int QT, int BM, int BN, int NW = 4>
@@ -734,7 +739,7 @@ hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
         if (slices > 1) {
             const int64_t count = P.m * (P.n_end - P.n_begin);
             splitk_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(
-                partial, slices, P.m, P.n, P.n_begin, P.n_end, P.y, P.out_bf16);
+                partial, slices, P.m, P.n, P.n_begin, P.n_end, P.y, P.out_bf16, P.residual);
         }
     } else {
         gemm_kernel<QT, BM, BN><<<dim3((unsigned)grid), dim3(kThreads), lds, stream>>>(P);
@@ -840,7 +845,7 @@ size_t qmm_gemm_workspace_bytes(const QmmLayout& L, int64_t m, int n_cus) {
 
 hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uint16_t* x_bf16,
                                 int64_t m, void* y, int out_bf16, void* workspace, int n_cus,
-                                hipStream_t stream) {
+                                hipStream_t stream, const void* residual) {
     if (m <= 0 || L.n == 0) return hipSuccess;
     if (n_cus <= 0) n_cus = 1;
     GemmParams P;
@@ -863,6 +868,7 @@ hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uin
     P.slice_units = 0;
     P.nibble_mask = 0x0f0f0f0fu;
     P.partial = (float*)workspace;
+    P.residual = residual;
     if (L.dtype == QMM_Q6_K) return launch_tile<QMM_Q6_K, 128, 128>(P, 1, stream); // the plain tile kernel only
     return L.dtype == QMM_Q4_K ? launch_qt<QMM_Q4_K>(P, n_cus, stream)
                                : launch_qt<QMM_Q8_0>(P, n_cus, stream);
@@ -873,5 +879,20 @@ hipError_t qmm_launch_f32_to_bf16(const float* x, uint16_t* out, int64_t count,
     if (count <= 0) return hipSuccess;
     int64_t threads = (count + 3) / 4;
     f32_to_bf16_kernel<<<(unsigned)((threads + 255) / 256), 256, 0, stream>>>(x, out, count);
+    return hipGetLastError();
+}
+
+hipError_t qmm_launch_epilogue(const float* t, const void* residual, void* y, int y_bf16, int64_t count,
+                               hipStream_t stream) {
+    if (count <= 0) return hipSuccess;
+    if ((count + 255) / 256 > 0x7fffffff) return hipErrorInvalidValue;
+    epilogue_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(t, residual, y, y_bf16, count);
+    return hipGetLastError();
+}
+
+hipError_t qmm_launch_bf16_to_f32(const uint16_t* x, float* out, int64_t count, hipStream_t stream) {
+    if (count <= 0) return hipSuccess;
+    if ((count + 255) / 256 > 0x7fffffff) return hipErrorInvalidValue;
+    bf16_to_f32_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(x, out, count);
     return hipGetLastError();
 }

@@ -136,13 +136,29 @@ __device__ __forceinline__ void quantize_q80_lane(const float (&v)[16], uint32_t
 // `safe` instead) so that the issuing code stays one basic block and the waits
 // on these loads can be counted separately from the weight loads behind them;
 // x16_finish applies the range check to the values.
-__device__ __forceinline__ void x16_issue(const float* __restrict__ src, const float* __restrict__ safe,
+// XB: the activations are bf16 (two 16 B loads per run, widened to f32 exactly) instead of f32.
+template <bool XB = false>
+__device__ __forceinline__ void x16_issue(const void* __restrict__ src, const void* __restrict__ safe,
                                           bool in_range, float4 (&f)[4]) {
     const float4* p = reinterpret_cast<const float4*>(in_range ? src : safe);
 #pragma unroll
-    for (int i = 0; i < 4; i++) f[i] = p[i];
+    for (int i = 0; i < (XB ? 2 : 4); i++) f[i] = p[i];
 }
+template <bool XB = false>
 __device__ __forceinline__ void x16_finish(const float4 (&f)[4], bool in_range, float (&v)[16]) {
+    if (XB) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint32_t w[4] = {__float_as_uint(f[i].x), __float_as_uint(f[i].y), __float_as_uint(f[i].z),
+                                   __float_as_uint(f[i].w)};
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                v[8 * i + 2 * c] = in_range ? __uint_as_float(w[c] << 16) : 0.0f;
+                v[8 * i + 2 * c + 1] = in_range ? __uint_as_float(w[c] & 0xffff0000u) : 0.0f;
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         v[4 * i] = in_range ? f[i].x : 0.0f;
@@ -201,14 +217,14 @@ __device__ inline XLds<QT> carve(uint8_t* base, int64_t k_units) {
 // Item i of a pass is unit i / MT of row m0 + i % MT; rows >= m are zero.
 // With `perm` the row is x[perm[row] / x_div] (expert-grouped pairs).
 struct XSource {
-    const float* x;
+    const void* x; // f32 or bf16 rows
     const int32_t* perm;
     int x_div;
     int m0, m, k;
     int k_units;
 };
 
-template <int MT>
+template <int MT, bool XB = false>
 __device__ __forceinline__ bool x_item_issue(const XSource& s, int item, bool item_ok, float4 (&f)[4]) {
     const int j = threadIdx.x & 15;
     const int mi = item % MT, unit = item / MT;
@@ -217,7 +233,8 @@ __device__ __forceinline__ bool x_item_issue(const XSource& s, int item, bool it
     if (s.perm != nullptr) xr = row_ok ? s.perm[s.m0 + mi] / s.x_div : 0;
     const int64_t k0 = (int64_t)unit * 256 + 16 * j;
     const bool in_range = row_ok && k0 + 16 <= s.k;
-    x16_issue(s.x + xr * s.k + k0, s.x, in_range, f);
+    if (XB) x16_issue<true>(static_cast<const uint16_t*>(s.x) + xr * s.k + k0, s.x, in_range, f);
+    else x16_issue<false>(static_cast<const float*>(s.x) + xr * s.k + k0, s.x, in_range, f);
     return in_range;
 }
 
@@ -416,6 +433,8 @@ struct GemvParams {
     int nv[QMM_MAX_GROUP], row_tiles_v[QMM_MAX_GROUP];
     const uint8_t* wv[QMM_MAX_GROUP];
     float* yv[QMM_MAX_GROUP];
+    // plain form only: y = sums (+ residual), stored as f32 or bf16 (P.y then points to bf16)
+    QmmEpilogue ep;
 };
 static_assert(offsetof(GemvParams, k_units) == 64, "first-load fields must fill one 64-byte line");
 
@@ -429,9 +448,12 @@ __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 // one panel (one pass of rows, one row-tile group per workgroup, one k step), so
 // the three loops below run once and the kernel is straight-line code from its
 // entry to the first load.
-template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT>
+// IO: 0 = f32 activations and a plain f32 store; 1 = f32 activations, 2 = bf16 activations, both
+// with the epilogue of P.ep (residual add, f32 or bf16 store).
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT, int IO = 0>
 __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int m_end, const uint8_t* w_first,
                                           float* y_out, int n_rows, int row_tiles, int rtg0, uint8_t* smem) {
+    constexpr bool XB = IO == 2, EP = IO != 0;
     const int lane0 = threadIdx.x & 63;
     // wave-uniform by construction; said so, the row-tile, panel offset and output row that
     // derive from it live in scalar registers
@@ -470,14 +492,14 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                     const XSource xs{P.x, GROUPED ? P.perm : nullptr, P.x_div, m0, m_end, P.k, k_units};
                     float4 f[4];
                     float v[16];
-                    const bool in0 = x_item_issue<MT>(xs, group, group < items, f);
+                    const bool in0 = x_item_issue<MT, XB>(xs, group, group < items, f);
                     load_panel<QT>(p, wbase + off, P.slots, lane0, active);
                     if (m0 != m_begin) lds_barrier(); // the previous rows' readers are done
-                    x16_finish(f, in0, v);
+                    x16_finish<XB>(f, in0, v);
                     if (group < items) x_item_quantize<QT, MT>(l, k_units, group, v);
                     for (int item = group + n_groups; item < items; item += n_groups) {
-                        const bool in1 = x_item_issue<MT>(xs, item, true, f);
-                        x16_finish(f, in1, v);
+                        const bool in1 = x_item_issue<MT, XB>(xs, item, true, f);
+                        x16_finish<XB>(f, in1, v);
                         x_item_quantize<QT, MT>(l, k_units, item, v);
                     }
                     // One row, one row-tile per workgroup, four units per panel: wave wk has just
@@ -510,7 +532,8 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                     for (int mi = 0; mi < MT; mi++) {
                         if (m0 + mi < m_end) {
                             int64_t yr = GROUPED ? P.perm[m0 + mi] : m0 + mi;
-                            y_out[yr * n_rows + row] = acc[mi];
+                            if (EP) qmm_store(y_out, P.ep, yr * n_rows + row, acc[mi]);
+                            else y_out[yr * n_rows + row] = acc[mi];
                         }
                     }
                 }
@@ -531,7 +554,8 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                     const int row = rt * 16 + r;
                     if (rt < row_tiles && row < n_rows && m0 + mi < m_end) {
                         int64_t yr = GROUPED ? P.perm[m0 + mi] : m0 + mi;
-                        y_out[yr * n_rows + row] = GATED ? silu(sum) * sum2 : sum;
+                        if (EP) qmm_store(y_out, P.ep, yr * n_rows + row, sum);
+                        else y_out[yr * n_rows + row] = GATED ? silu(sum) * sum2 : sum;
                     }
                 }
                 red_buf ^= 1;
@@ -546,7 +570,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
 // whether it exists or not.
 // The dense straight-line single-row Q4_K form is held to 80 registers: six waves per SIMD,
 // i.e. two 12-wave workgroups per CU.
-template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false>
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false, int IO = 0>
 __global__ __launch_bounds__(64 * kMaxWaves)
 __attribute__((amdgpu_waves_per_eu((ONESHOT && !GROUPED && MT == 1 && QT == QMM_Q4_K) ? 6 : 3))) void gemv_kernel(GemvParams P) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -581,7 +605,7 @@ __attribute__((amdgpu_waves_per_eu((ONESHOT && !GROUPED && MT == 1 && QT == QMM_
         else
             gemv_body<QT, 4, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     } else {
-        gemv_body<QT, MT, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
+        gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     }
 }
 
@@ -617,7 +641,7 @@ void choose_split(const QmmLayout& L, int n_cus, int grid_y, bool gated, GemvPar
     P.wave_magic = (65536 + nwk - 1) / nwk;
 }
 
-template <int QT, int MT, bool GATED, bool GROUPED>
+template <int QT, int MT, bool GATED, bool GROUPED, int IO = 0>
 hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipStream_t stream) {
     const int all_waves = GATED ? 2 * waves : waves;
     size_t lds = lds_bytes<QT, MT>(P.k_units, all_waves);
@@ -630,26 +654,36 @@ hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipS
     // grouped form), one row-tile group per workgroup, one k step
     constexpr bool kCanOneshot = GROUPED ? MT == QMM_MOE_SEG_ROWS : true;
     const bool oneshot = kCanOneshot && (GROUPED || P.m <= MT) && P.kpw == 1 && grid == P.rt_groups;
-    const void* fn = oneshot ? reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot>)
-                             : reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, false>);
+    const void* fn = oneshot ? reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot, IO>)
+                             : reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, false, IO>);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
     const dim3 g((unsigned)grid, (unsigned)grid_y), b(64 * all_waves);
     if (oneshot)
-        gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot><<<g, b, lds, stream>>>(P);
+        gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot, IO><<<g, b, lds, stream>>>(P);
     else
-        gemv_kernel<QT, MT, GATED, GROUPED, false><<<g, b, lds, stream>>>(P);
+        gemv_kernel<QT, MT, GATED, GROUPED, false, IO><<<g, b, lds, stream>>>(P);
     return hipGetLastError();
 }
 
 template <int QT>
-hipError_t launch_plain(const GemvParams& P, int waves, int n_cus, hipStream_t stream) {
+hipError_t launch_plain(const GemvParams& P, int waves, int n_cus, int io, hipStream_t stream) {
     // the widest row tile whose quantized activations fit comfortably in LDS
     int mt = P.m >= 3 ? 4 : (P.m == 2 ? 2 : 1);
     if (mt == 4 && lds_bytes<QT, 4>(P.k_units, waves) > 64 * 1024) mt = 2;
     if (mt == 2 && lds_bytes<QT, 2>(P.k_units, waves) > 64 * 1024) mt = 1;
+    if (io == 2) { // bf16 activations: the one- and two-row forms only
+        if (P.m > 2) return hipErrorNotSupported;
+        if (mt == 2) return launch_mt<QT, 2, false, false, 2>(P, waves, n_cus, 1, stream);
+        return launch_mt<QT, 1, false, false, 2>(P, waves, n_cus, 1, stream);
+    }
+    if (io == 1) {
+        if (mt == 4) return launch_mt<QT, 4, false, false, 1>(P, waves, n_cus, 1, stream);
+        if (mt == 2) return launch_mt<QT, 2, false, false, 1>(P, waves, n_cus, 1, stream);
+        return launch_mt<QT, 1, false, false, 1>(P, waves, n_cus, 1, stream);
+    }
     if (mt == 4) return launch_mt<QT, 4, false, false>(P, waves, n_cus, 1, stream);
     if (mt == 2) return launch_mt<QT, 2, false, false>(P, waves, n_cus, 1, stream);
     return launch_mt<QT, 1, false, false>(P, waves, n_cus, 1, stream);
@@ -682,6 +716,8 @@ bool make_params(const QmmLayout& L, const void* tiled, const float* x, int64_t 
     P.n_experts = 0;
     P.x_div = 1;
     P.n_weights = 0;
+    P.ep.residual = nullptr;
+    P.ep.y_bf16 = 0;
     return true;
 }
 
@@ -735,15 +771,18 @@ __global__ void quantize_export_kernel(const float* __restrict__ x, int64_t m, i
 } // namespace
 
 hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
-                           float* y, int n_cus, hipStream_t stream) {
+                           float* y, int n_cus, hipStream_t stream, const QmmIo* io) {
     if (m <= 0 || L.n == 0) return hipSuccess;
     GemvParams P;
     if (!make_params(L, tiled, x, m, y, P)) return hipErrorInvalidValue;
+    // kernel variant: plain, or with the epilogue (and f32 / bf16 activations)
+    const int iom = !io ? 0 : (io->x_bf16 ? 2 : (io->residual || io->y_bf16 ? 1 : 0));
+    if (io) P.ep = QmmEpilogue{io->residual, io->y_bf16};
     int waves;
     choose_split(L, n_cus, 1, false, P, waves);
-    if (L.dtype == QMM_Q6_K) return launch_plain<QMM_Q6_K>(P, waves, n_cus, stream);
-    return L.dtype == QMM_Q4_K ? launch_plain<QMM_Q4_K>(P, waves, n_cus, stream)
-                               : launch_plain<QMM_Q8_0>(P, waves, n_cus, stream);
+    if (L.dtype == QMM_Q6_K) return launch_plain<QMM_Q6_K>(P, waves, n_cus, iom, stream);
+    return L.dtype == QMM_Q4_K ? launch_plain<QMM_Q4_K>(P, waves, n_cus, iom, stream)
+                               : launch_plain<QMM_Q8_0>(P, waves, n_cus, iom, stream);
 }
 
 namespace {

@@ -148,8 +148,24 @@ __device__ __forceinline__ void quantize_into_record(const float (&v)[16], int j
 
 // Sixteen consecutive values of a row (k is a multiple of 32: the run is inside
 // the row or past its end), zeros when out of range.
-__device__ __forceinline__ void load_run16(const float* __restrict__ src, const float* __restrict__ safe,
+// XB: the values are bf16 (widened exactly).
+template <bool XB = false>
+__device__ __forceinline__ void load_run16(const void* __restrict__ src, const void* __restrict__ safe,
                                            bool in_range, float (&v)[16]) {
+    if (XB) {
+        const uint4* p = reinterpret_cast<const uint4*>(in_range ? src : safe);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint4 f = p[i];
+            const uint32_t w[4] = {f.x, f.y, f.z, f.w};
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                v[8 * i + 2 * c] = in_range ? __uint_as_float(w[c] << 16) : 0.0f;
+                v[8 * i + 2 * c + 1] = in_range ? __uint_as_float(w[c] & 0xffff0000u) : 0.0f;
+            }
+        }
+        return;
+    }
     const float4* p = reinterpret_cast<const float4*>(in_range ? src : safe);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -159,8 +175,8 @@ __device__ __forceinline__ void load_run16(const float* __restrict__ src, const 
     }
 }
 
-template <int QT>
-__global__ void quantize_ws_kernel(const float* __restrict__ x, int m, int k, int k_units, int n_tiles,
+template <int QT, bool XB = false>
+__global__ void quantize_ws_kernel(const void* __restrict__ x, int m, int k, int k_units, int n_tiles,
                                    uint8_t* __restrict__ ws) {
     const int group = (blockIdx.x * blockDim.x + threadIdx.x) >> 4;
     const int j = threadIdx.x & 15;
@@ -170,7 +186,8 @@ __global__ void quantize_ws_kernel(const float* __restrict__ x, int m, int k, in
     const int tile = row >> 4, mr = row & 15;
     float v[16];
     const int k0 = unit * 256 + 16 * j;
-    load_run16(x + (int64_t)row * k + k0, x, row < m && k0 + 16 <= k, v);
+    if (XB) load_run16<true>(static_cast<const uint16_t*>(x) + (int64_t)row * k + k0, x, row < m && k0 + 16 <= k, v);
+    else load_run16<false>(static_cast<const float*>(x) + (int64_t)row * k + k0, x, row < m && k0 + 16 <= k, v);
     quantize_into_record<QT>(v, j, mr, ws + ((int64_t)tile * k_units + unit) * Unit<QT>::kBytes);
 }
 
@@ -242,6 +259,8 @@ struct MfmaParams {
     const int32_t* offsets;      // sorted pairs of expert e: [offsets[e], offsets[e + 1])
     const int32_t* tile_offsets; // its 16-row tiles (records): [tile_offsets[e], tile_offsets[e + 1])
     int64_t matrix_bytes;
+    // dense forms only: y = sums (+ residual), stored as f32 or bf16 (y then points to bf16)
+    QmmEpilogue ep;
 };
 
 // 4x4 transpose of one dword between the four 16-lane rows: on entry row u
@@ -439,7 +458,8 @@ __device__ __forceinline__ void issue_window_copy(const uint8_t* __restrict__ sr
 // SINGLE: one tile of rows and one activation window, i.e. straight-line code.
 // GROUPED: blockIdx.y is an expert; its weights are matrix blockIdx.y of the
 // stack, its rows the expert's tiles of sorted pairs, output row = pair index.
-template <int QT, bool SINGLE, bool GROUPED = false>
+// EP: the sums go through the epilogue of P.ep (residual add, f32 or bf16 store).
+template <int QT, bool SINGLE, bool GROUPED = false, bool EP = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaParams P) {
     constexpr int UB = Unit<QT>::kBytes;
     constexpr int NL = WPanel<QT>::QC + 4; // loads of one panel
@@ -541,7 +561,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
                 if (GROUPED) {
                     if (pos_begin + mm < pos_end) yout[(int64_t)P.perm[pos_begin + mm] * n_rows + row] = v;
                 } else if (mm < P.m) {
-                    yout[(int64_t)mm * n_rows + row] = v;
+                    if (EP) qmm_store(yout, P.ep, (int64_t)mm * n_rows + row, v);
+                    else yout[(int64_t)mm * n_rows + row] = v;
                 }
             };
             if (P.nwk == 1) {
@@ -646,6 +667,7 @@ __device__ __forceinline__ void panel_dot_direct_q4k(WPanel<QMM_Q4_K>& p, const 
     }
 }
 
+template <bool EP = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(MfmaParams P) {
     constexpr int QT = QMM_Q4_K;
     constexpr int UB = Unit<QT>::kBytes;
@@ -703,7 +725,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(Mf
         if (rt_ok && row < n_rows) {
 #pragma unroll
             for (int r = 0; r < 4; r++)
-                if (grp * 4 + r < P.m) yout[(int64_t)(grp * 4 + r) * n_rows + row] = acc[r];
+                if (grp * 4 + r < P.m) {
+                    if (EP) qmm_store(yout, P.ep, (int64_t)(grp * 4 + r) * n_rows + row, acc[r]);
+                    else yout[(int64_t)(grp * 4 + r) * n_rows + row] = acc[r];
+                }
         }
         return;
     }
@@ -715,7 +740,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(Mf
         for (int r = 0; r < 4; r++) {
             float sum = 0.0f;
             for (int w2 = 0; w2 < P.nwk; w2++) sum += lds_red[((wr * P.nwk + w2) * 4 + r) * 64 + lane];
-            if (grp * 4 + r < P.m) yout[(int64_t)(grp * 4 + r) * n_rows + row] = sum;
+            if (grp * 4 + r < P.m) {
+                if (EP) qmm_store(yout, P.ep, (int64_t)(grp * 4 + r) * n_rows + row, sum);
+                else yout[(int64_t)(grp * 4 + r) * n_rows + row] = sum;
+            }
         }
     }
 }
@@ -737,7 +765,7 @@ bool direct_form_applies(int dtype, int n_tiles, int nwr, bool one_window) {
 // + gridDim.x * waves, ... and walks all their panels; the activation window
 // stays in LDS meanwhile.  Windows that split k accumulate into y (the same
 // wave adds the same row-tile's windows in order, so the result is deterministic).
-template <int QT>
+template <int QT, bool EP = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_stream_kernel(MfmaParams P) {
     constexpr int UB = Unit<QT>::kBytes;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -773,8 +801,11 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_stream_kernel(MfmaPa
                     for (int r = 0; r < 4; r++) {
                         const int mm = tile * 16 + grp * 4 + r;
                         if (mm < P.m) {
+                            // one window covers k: the sums are final (the launcher folds the
+                            // epilogue only then); otherwise y accumulates the windows in f32
                             float* dst = P.y + (int64_t)mm * P.n + row;
-                            *dst = wu0 == 0 ? acc[r] : *dst + acc[r];
+                            if (EP && P.k_units <= P.window_units) qmm_store(P.y, P.ep, (int64_t)mm * P.n + row, acc[r]);
+                            else *dst = wu0 == 0 ? acc[r] : *dst + acc[r];
                         }
                     }
                 }
@@ -785,17 +816,38 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_stream_kernel(MfmaPa
 
 } // namespace
 
+namespace {
+// form 0: one tile of rows, one activation window; 1: the general one-shot form; 2: streaming
+template <int QT, bool EP>
+hipError_t launch_dense_form(int form, const MfmaParams& P, unsigned grid, int waves, size_t lds, hipStream_t stream) {
+    const void* fn = form == 0   ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QT, true, false, EP>)
+                     : form == 1 ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QT, false, false, EP>)
+                                 : reinterpret_cast<const void*>(&gemv_mfma_stream_kernel<QT, EP>);
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+    }
+    if (form == 0) gemv_mfma_oneshot_kernel<QT, true, false, EP><<<grid, 64 * waves, lds, stream>>>(P);
+    else if (form == 1) gemv_mfma_oneshot_kernel<QT, false, false, EP><<<grid, 64 * waves, lds, stream>>>(P);
+    else gemv_mfma_stream_kernel<QT, EP><<<grid, 64 * waves, lds, stream>>>(P);
+    return hipGetLastError();
+}
+} // namespace
+
 hipError_t qmm_launch_quantize_ws(int dtype, const float* x, int64_t m, int64_t k, void* workspace,
-                                  hipStream_t stream) {
+                                  hipStream_t stream, bool x_bf16) {
     if (m <= 0 || k <= 0 || m > 0x3fffffff || k > 0x3fffffff) return hipErrorInvalidValue;
     const int n_tiles = (int)((m + 15) / 16);
     const int64_t k_units = (k + 255) / 256;
     const int64_t threads = (int64_t)n_tiles * 16 * k_units * 16;
     const unsigned grid = (unsigned)((threads + 255) / 256);
-    if (dtype == QMM_Q4_K)
-        quantize_ws_kernel<QMM_Q4_K><<<grid, 256, 0, stream>>>(x, (int)m, (int)k, (int)k_units, n_tiles, (uint8_t*)workspace);
-    else
-        quantize_ws_kernel<QMM_Q8_0><<<grid, 256, 0, stream>>>(x, (int)m, (int)k, (int)k_units, n_tiles, (uint8_t*)workspace);
+    if (dtype == QMM_Q4_K) {
+        if (x_bf16) quantize_ws_kernel<QMM_Q4_K, true><<<grid, 256, 0, stream>>>(x, (int)m, (int)k, (int)k_units, n_tiles, (uint8_t*)workspace);
+        else quantize_ws_kernel<QMM_Q4_K><<<grid, 256, 0, stream>>>(x, (int)m, (int)k, (int)k_units, n_tiles, (uint8_t*)workspace);
+    } else {
+        if (x_bf16) quantize_ws_kernel<QMM_Q8_0, true><<<grid, 256, 0, stream>>>(x, (int)m, (int)k, (int)k_units, n_tiles, (uint8_t*)workspace);
+        else quantize_ws_kernel<QMM_Q8_0><<<grid, 256, 0, stream>>>(x, (int)m, (int)k, (int)k_units, n_tiles, (uint8_t*)workspace);
+    }
     return hipGetLastError();
 }
 
@@ -805,7 +857,7 @@ size_t qmm_gemv_mfma_workspace_bytes(const QmmLayout& L, int64_t m) {
 
 hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
                                 float* y, void* workspace, int n_cus, hipStream_t stream,
-                                bool quantize) {
+                                bool quantize, const QmmIo* io) {
     if (m <= 0 || L.n == 0) return hipSuccess;
     if (L.n > 0x3fffffff || L.k > 0x3fffffff || m > 0x3fffffff ||
         L.row_tiles * L.k_groups > 0x7fffffff)
@@ -813,11 +865,18 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     if (n_cus <= 0) n_cus = 1;
     const int n_tiles = (int)((m + 15) / 16);
     uint8_t* ws = (uint8_t*)workspace;
+    const bool epilogue = io && (io->residual || io->y_bf16);
+    MfmaParams P;
+    P.ep = QmmEpilogue{nullptr, 0};
+    if (io) P.ep = QmmEpilogue{io->residual, io->y_bf16};
+    P.window_units = (kWindowUnits / L.s) * L.s;
+    // the streaming form adds up activation windows in y itself: no folded epilogue there
+    if (epilogue && !(L.k_groups <= kMaxWaves && L.row_tiles < 8 * (int64_t)n_cus) && L.k_units > P.window_units)
+        return hipErrorNotSupported;
     if (quantize) {
-        hipError_t e = qmm_launch_quantize_ws(L.dtype, x, m, L.k, ws, stream);
+        hipError_t e = qmm_launch_quantize_ws(L.dtype, x, m, L.k, ws, stream, io && io->x_bf16);
         if (e != hipSuccess) return e;
     }
-    MfmaParams P;
     P.w = (const uint8_t*)tiled;
     P.ws = ws;
     P.y = y;
@@ -871,36 +930,18 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     }
     P.wave_magic = (65536 + P.nwk - 1) / P.nwk;
     if (oneshot && direct_form_applies(L.dtype, n_tiles, P.nwr, L.k_units <= P.window_units)) {
-        gemv_mfma_direct_q4k_kernel<<<grid, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
+        if (epilogue) gemv_mfma_direct_q4k_kernel<true><<<grid, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
+        else gemv_mfma_direct_q4k_kernel<false><<<grid, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
         return hipGetLastError();
     }
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     const bool single = n_tiles == 1 && L.k_units <= P.window_units;
-    const void* fn;
-    if (oneshot && single)
-        fn = L.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true>)
-                                 : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, true>);
-    else if (oneshot)
-        fn = L.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false>)
-                                 : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, false>);
-    else
-        fn = L.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_stream_kernel<QMM_Q4_K>)
-                                 : reinterpret_cast<const void*>(&gemv_mfma_stream_kernel<QMM_Q8_0>);
-    if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-    }
-    if (oneshot && single) {
-        if (L.dtype == QMM_Q4_K) gemv_mfma_oneshot_kernel<QMM_Q4_K, true><<<grid, 64 * waves, lds, stream>>>(P);
-        else gemv_mfma_oneshot_kernel<QMM_Q8_0, true><<<grid, 64 * waves, lds, stream>>>(P);
-    } else if (oneshot) {
-        if (L.dtype == QMM_Q4_K) gemv_mfma_oneshot_kernel<QMM_Q4_K, false><<<grid, 64 * waves, lds, stream>>>(P);
-        else gemv_mfma_oneshot_kernel<QMM_Q8_0, false><<<grid, 64 * waves, lds, stream>>>(P);
-    } else {
-        if (L.dtype == QMM_Q4_K) gemv_mfma_stream_kernel<QMM_Q4_K><<<grid, 64 * waves, lds, stream>>>(P);
-        else gemv_mfma_stream_kernel<QMM_Q8_0><<<grid, 64 * waves, lds, stream>>>(P);
-    }
-    return hipGetLastError();
+    const int form = oneshot ? (single ? 0 : 1) : 2;
+    if (L.dtype == QMM_Q4_K)
+        return epilogue ? launch_dense_form<QMM_Q4_K, true>(form, P, grid, waves, lds, stream)
+                        : launch_dense_form<QMM_Q4_K, false>(form, P, grid, waves, lds, stream);
+    return epilogue ? launch_dense_form<QMM_Q8_0, true>(form, P, grid, waves, lds, stream)
+                    : launch_dense_form<QMM_Q8_0, false>(form, P, grid, waves, lds, stream);
 }
 
 size_t qmm_moe_records_bytes(int dtype, int64_t max_tiles, int64_t k) {
@@ -937,6 +978,7 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     if (!qmm_gemv_mfma_grouped_supported(L) || n_experts > 65535 || L.n > 0x3fffffff)
         return hipErrorInvalidValue;
     MfmaParams P;
+    P.ep = QmmEpilogue{nullptr, 0};
     P.w = (const uint8_t*)tiled;
     P.ws = (const uint8_t*)records;
     P.y = y;
@@ -998,6 +1040,7 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
         total_row_tiles += L.row_tiles;
     }
     MfmaParams P;
+    P.ep = QmmEpilogue{nullptr, 0};
     P.w = (const uint8_t*)tiled[0];
     P.ws = (const uint8_t*)workspace;
     P.y = ys[0];
@@ -1041,7 +1084,7 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
     P.rt_groups = (int)groups;
     const int waves = P.nwk * P.nwr;
     if (direct_form_applies(L0.dtype, 1, P.nwr, true)) {
-        gemv_mfma_direct_q4k_kernel<<<(unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
+        gemv_mfma_direct_q4k_kernel<false><<<(unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
         return hipGetLastError();
     }
     const size_t lds = std::max((size_t)P.window_units * unit_bytes(L0.dtype), (size_t)waves * 256 * 4);

@@ -55,6 +55,31 @@ __device__ __forceinline__ uint16_t qmm_f32_to_bf16_bits(float f) {
 
 #endif // __HIPCC__
 
+// What a projection call folds into its kernels besides the product: the activations may be
+// bf16 (widened to f32 exactly on load), the result may get a residual of the output's type
+// added and may be stored as bf16 (one rounding, of sum + residual).  residual may alias y.
+struct QmmIo {
+    int x_bf16;
+    const void* residual;
+    int y_bf16;
+};
+struct QmmEpilogue {
+    const void* residual;
+    int y_bf16;
+};
+
+#if defined(__HIPCC__)
+__device__ __forceinline__ void qmm_store(void* y, const QmmEpilogue& ep, int64_t idx, float v) {
+    if (ep.y_bf16) {
+        if (ep.residual) v += qmm_bf16_bits_to_f32(static_cast<const uint16_t*>(ep.residual)[idx]);
+        static_cast<uint16_t*>(y)[idx] = qmm_f32_to_bf16_bits(v);
+    } else {
+        if (ep.residual) v += static_cast<const float*>(ep.residual)[idx];
+        static_cast<float*>(y)[idx] = v;
+    }
+}
+#endif
+
 // Records the calling thread's error message (read with izwi_qmm_last_error) and returns `code`.
 int qmm_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 
@@ -68,8 +93,10 @@ hipError_t qmm_launch_dequant(const QmmLayout& L, const void* tiled, float* out,
 
 // Decode kernel: y[m, n] = QMatMul(x[m, k]) for one matrix of the handle.
 // `n_cus` sizes the grid.  Returns hipErrorInvalidValue for shapes it cannot run.
+// With `io`: x and y are of the types it names (bf16 activations: m <= 2 only,
+// hipErrorNotSupported beyond).
 hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
-                           float* y, int n_cus, hipStream_t stream);
+                           float* y, int n_cus, hipStream_t stream, const QmmIo* io = nullptr);
 
 // Decode kernel for the gate / up pair of an MLP: y[m, n] = silu(W_gate x) * (W_up x), both
 // matrices of layout L, m <= 2 (hipErrorNotSupported beyond).  The sums are those of
@@ -86,9 +113,11 @@ hipError_t qmm_launch_silu_mul(const float* gate, const float* up, float* out, i
 // `quantize` false: the workspace already holds the quantized activations of x for this k
 // and type (a previous call on the same x), only the matmul is launched.
 size_t qmm_gemv_mfma_workspace_bytes(const QmmLayout& L, int64_t m);
+// With `io`: x and y are of the types it names; hipErrorNotSupported (nothing launched) if the
+// epilogue cannot be folded into the form this shape takes.
 hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
                                 float* y, void* workspace, int n_cus, hipStream_t stream,
-                                bool quantize = true);
+                                bool quantize = true, const QmmIo* io = nullptr);
 
 // Activation quantizer written out in the reference's block layout.
 hipError_t qmm_launch_quantize_activations(int weight_dtype, const float* x, int64_t m, int64_t k,
@@ -97,9 +126,16 @@ hipError_t qmm_launch_quantize_activations(int weight_dtype, const float* x, int
 // Prefill kernel: bf16 activations, bf16 MFMA, f32 accumulate.  Products with few output
 // tiles are split along k and need `workspace` (qmm_gemm_workspace_bytes, 0 if not split).
 size_t qmm_gemm_workspace_bytes(const QmmLayout& L, int64_t m, int n_cus);
+// `residual` (of y's type, may alias y, may be NULL) is added to the sums before the store.
 hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uint16_t* x_bf16,
                                 int64_t m, void* y, int out_bf16, void* workspace, int n_cus,
-                                hipStream_t stream);
+                                hipStream_t stream, const void* residual = nullptr);
+// y[i] = t[i] (+ residual[i]) as f32 or bf16: the epilogue as a kernel of its own, for the forms
+// that cannot fold it
+hipError_t qmm_launch_epilogue(const float* t, const void* residual, void* y, int y_bf16, int64_t count,
+                               hipStream_t stream);
+// bf16 -> f32, exact
+hipError_t qmm_launch_bf16_to_f32(const uint16_t* x, float* out, int64_t count, hipStream_t stream);
 // f32 activations for m > 64: converted to bf16 into `x_bf16_ws` (m*k elements) first.
 hipError_t qmm_launch_f32_to_bf16(const float* x, uint16_t* out, int64_t count,
                                   hipStream_t stream);
@@ -115,7 +151,7 @@ hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* co
 // The same for 3 <= m <= 16 on the matrix cores: `workspace` holds the activations already
 // quantized (qmm_launch_quantize_ws), all weights read the same records in one launch.
 hipError_t qmm_launch_quantize_ws(int dtype, const float* x, int64_t m, int64_t k, void* workspace,
-                                  hipStream_t stream);
+                                  hipStream_t stream, bool x_bf16 = false);
 hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
                                       int64_t m, float* const* ys, const void* workspace, int n_cus,
                                       hipStream_t stream);

@@ -163,6 +163,31 @@ class QMatMul:
             return y
         raise capi.QmmError(-1, f"unsupported dtype {x.dtype} for qmatmul, expected f32 or bf16")
 
+    def forward_fused(self, x: torch.Tensor, residual: torch.Tensor | None = None,
+                      out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+        """Qwen3Projection::forward (qwen3/core.rs:795-829) plus the layer's residual add
+        (core.rs:1875, 1879) in one call: x is f32 or bf16 and is read in its own type, the result is
+        ``x @ W^T (+ residual)`` in ``out_dtype`` (default: x's type, as the reference casts back).
+        ``out`` may be ``residual`` itself (in-place add)."""
+        n, k = self.qtensor.dims2()
+        code = {torch.float32: capi.OUT_F32, torch.bfloat16: capi.OUT_BF16}
+        if x.dtype not in code or x.dim() < 1 or x.shape[-1] != k or not x.is_contiguous():
+            raise capi.QmmError(-1, f"expected a contiguous f32 or bf16 input with last dim {k}, got {x.dtype} {tuple(x.shape)}")
+        out_dtype = out_dtype or x.dtype
+        if out_dtype not in code:
+            raise capi.QmmError(-1, f"unsupported output dtype {out_dtype}")
+        out_shape = tuple(x.shape[:-1]) + (n,)
+        if residual is not None and (residual.dtype != out_dtype or tuple(residual.shape) != out_shape
+                                     or not residual.is_contiguous() or residual.device != x.device):
+            raise capi.QmmError(-1, f"residual must be a contiguous {out_dtype} tensor of shape {out_shape} on {x.device}")
+        y = out if out is not None else torch.empty(out_shape, dtype=out_dtype, device=x.device)
+        if y.dtype != out_dtype or tuple(y.shape) != out_shape or not y.is_contiguous() or y.device != x.device:
+            raise capi.QmmError(-1, f"out must be a contiguous {out_dtype} tensor of shape {out_shape} on {x.device}")
+        check(lib().izwi_qmm_forward_fused(self.qtensor._h, x.data_ptr(), code[x.dtype], x.numel() // k if k else 0,
+                                           residual.data_ptr() if residual is not None else None, y.data_ptr(),
+                                           code[out_dtype], _space(x), _stream_ptr(x)))
+        return y
+
     def forward_bf16_to_f32(self, x: torch.Tensor) -> torch.Tensor:
         """bf16 activations, f32 result (the MFMA kernel's accumulators, unrounded)."""
         n, k = self.qtensor.dims2()

@@ -1,0 +1,138 @@
+"""GPU tests of izwi_qmm_forward_fused (pytest -m gpu): casts and residual add folded into the
+projection kernels.  The sums must be those of the plain entry points bit for bit, so every case
+is compared exactly with the unfused composition (plain call, then torch's add / cast)."""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import np_ref
+
+pytestmark = pytest.mark.gpu
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+
+
+def _say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def qa():
+    if not torch.cuda.is_available():
+        pytest.fail("no GPU visible: the HIP path cannot run (there is no fallback)")
+    import izwi_amd
+    izwi_amd.lib()
+    torch.cuda.set_device(0)
+    return izwi_amd
+
+
+def make_qmatmul(qa, oracle, dtype, n, k, seed):
+    if dtype == Q6_K:
+        blocks = np_ref.random_q6_k_blocks(seed, n, k)
+    else:
+        rows = min(n, 1024)
+        b = oracle.quantize(dtype, oracle.randn(seed, (rows, k), std=0.02)).reshape(rows, -1)
+        blocks = np.tile(b, ((n + rows - 1) // rows, 1))[:n].reshape(-1)
+    return qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType(dtype), blocks, (n, k)))
+
+
+def unfused_sums(mm, x):
+    """f32 sums of the plain entry points for the same activations."""
+    m = x.numel() // x.shape[-1]
+    if x.dtype == torch.float32:
+        return mm.forward(x)
+    return mm.forward(x.float()) if m <= 64 else mm.forward_bf16_to_f32(x)
+
+
+def check_all_forms(qa, mm, x32, label):
+    n = mm.qtensor.dims2()[0]
+    m = x32.shape[0]
+    res32 = torch.randn(m, n, device="cuda")
+    for xdt in (torch.float32, torch.bfloat16):
+        x = x32.to(xdt)
+        sums = unfused_sums(mm, x)
+        for ydt in (torch.float32, torch.bfloat16):
+            _say(f"{label} m={m} x={xdt} y={ydt}")
+            res = res32.to(ydt)
+            # no residual: the plain result, cast once
+            assert torch.equal(mm.forward_fused(x, out_dtype=ydt), sums.to(ydt))
+            # residual: one rounding of sum + residual
+            want = (sums + res.float()).to(ydt)
+            assert torch.equal(mm.forward_fused(x, residual=res, out_dtype=ydt), want)
+            # in place: y is the residual buffer
+            buf = res.clone()
+            out = mm.forward_fused(x, residual=buf, out_dtype=ydt, out=buf)
+            assert out.data_ptr() == buf.data_ptr() and torch.equal(buf, want)
+
+
+@pytest.mark.parametrize("dtype", [Q4_K, Q8_0, Q6_K])
+@pytest.mark.parametrize("m", [1, 2, 3, 16, 33, 64, 65, 300])
+def test_fused_equals_unfused_composition(qa, oracle, dtype, m):
+    n, k = 528, 1024
+    mm = make_qmatmul(qa, oracle, dtype, n, k, 3 + dtype)
+    x = torch.from_numpy(oracle.randn(40 + m, (m, k))).cuda()
+    check_all_forms(qa, mm, x, f"fused dtype={dtype}")
+
+
+@pytest.mark.parametrize("n,k,m", [(4096, 4096, 1), (4096, 12288, 2), (12288, 4096, 8), (4096, 12288, 16),
+                                   (40000, 4096, 1), (40000, 4096, 5), (33000, 8448, 4), (1024, 4096, 512)])
+def test_fused_8b_and_tall_shapes_q4_k(qa, oracle, n, k, m):
+    """The 8B projection shapes, a matrix tall enough for the streaming form of the batched kernel
+    (k inside one activation window: folded; k beyond: sums in scratch, then the epilogue kernel)
+    and a prefill shape with split k."""
+    mm = make_qmatmul(qa, oracle, Q4_K, n, k, n % 97)
+    x = torch.from_numpy(oracle.randn(n % 89 + m, (m, k))).cuda()
+    check_all_forms(qa, mm, x, f"fused n={n} k={k}")
+
+
+def test_fused_against_the_oracle_and_reference_rounding(qa, oracle):
+    """bf16 in, bf16 out with a residual, as the reference's layer does it (cast in, matmul, cast out,
+    add): the fused call is within one bf16 rounding of that sequence and closer to the exact sum."""
+    n, k, m = 1024, 4096, 2
+    blocks = oracle.quantize(Q4_K, oracle.randn(1, (n, k), std=0.02))
+    mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q4K, blocks, (n, k)))
+    xb = torch.from_numpy(oracle.randn(2, (m, k))).cuda().to(torch.bfloat16)
+    res = torch.randn(m, n, device="cuda").to(torch.bfloat16)
+    sums = oracle.qmatmul(Q4_K, xb.float().cpu().numpy(), blocks, n)  # the reference's f32 product
+    exact = sums.astype(np.float64) + res.float().cpu().numpy()
+    reference = (torch.from_numpy(sums).cuda().to(torch.bfloat16) + res).float().cpu().numpy()  # two roundings
+    got = mm.forward_fused(xb, residual=res).float().cpu().numpy()
+    scale = np.abs(exact).max()
+    assert np.abs(got - exact).max() <= 2.0 ** -8 * scale           # one bf16 rounding (+ 1e-4 of the sums)
+    assert np.abs(got - reference).max() <= 2.0 ** -7 * scale
+    assert np.abs(got - exact).mean() <= np.abs(reference - exact).mean()
+
+
+def test_fused_host_memory_profile_counters_and_errors(qa, oracle):
+    from izwi_amd import capi
+    n, k, m = 96, 512, 3
+    mm = make_qmatmul(qa, oracle, Q8_0, n, k, 9)
+    x = torch.from_numpy(oracle.randn(5, (m, k)))
+    res = torch.randn(m, n)
+    want = mm.forward(x.cuda()) + res.cuda()
+    assert torch.equal(mm.forward_fused(x, residual=res).cuda(), want)  # host pointers in, host pointer out
+    L = capi.lib()
+    L.izwi_qmm_profile_enable(1)
+    L.izwi_qmm_profile_reset()
+    xb = x.cuda().to(torch.bfloat16)
+    mm.forward_fused(xb)
+    mm.forward_fused(xb, out_dtype=torch.float32)
+    snap = qa.profile_snapshot()
+    L.izwi_qmm_profile_enable(0)
+    assert snap["qmatmul_calls"] == 2 and snap["qmatmul_input_casts"] == 2 and snap["qmatmul_output_casts"] == 1
+    assert snap["qmatmul_input_cast_ns"] == 0 and snap["qmatmul_output_cast_ns"] == 0
+    y = torch.empty(m, n, device="cuda")
+    xd = x.cuda()
+    h = mm.qtensor._h
+    assert L.izwi_qmm_forward_fused(h, xd.data_ptr(), 2, m, None, y.data_ptr(), 0, capi.DEVICE, None) == -1
+    assert L.izwi_qmm_forward_fused(h, xd.data_ptr(), 0, m, None, y.data_ptr(), 7, capi.DEVICE, None) == -1
+    assert L.izwi_qmm_forward_fused(h, None, 0, m, None, y.data_ptr(), 0, capi.DEVICE, None) == -1
+    assert L.izwi_qmm_forward_fused(h, xd.data_ptr(), 0, 0, None, None, 0, capi.DEVICE, None) == 0  # m = 0
+    with pytest.raises(capi.QmmError):
+        mm.forward_fused(xd, residual=torch.zeros(m, n + 1, device="cuda"))
+    with pytest.raises(capi.QmmError):
+        mm.forward_fused(xd, residual=torch.zeros(m, n, device="cuda", dtype=torch.bfloat16))
