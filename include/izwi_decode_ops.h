@@ -1,0 +1,72 @@
+/*
+ * izwi_decode_ops — the decode-step neighbours of the quantized projections: RMSNorm, the
+ * q/k head norm, rotary embedding and single-token grouped-query attention, f32.
+ *
+ * Each entry point is the device side of one of the reference's fused-kernel hooks
+ * (crates/izwi-core/src/kernels/mod.rs:109-225), which today dispatch to Metal only
+ * (crates/izwi-core/src/kernels/metal.rs) and return None elsewhere, so that the caller falls
+ * back to Candle's eager operators.  Arithmetic follows the reference's shaders
+ * (metal.rs:59-381) in f32; only the order of the sums differs (the reference's tests allow
+ * 1e-5 against the eager operators, metal.rs:2956).
+ *
+ * Conventions are those of izwi_qmm.h: return IZWI_QMM_OK or a negative izwi_qmm_status, message
+ * through izwi_qmm_last_error(); `mem_space` says whether the pointers are device or host
+ * memory (host buffers are staged, synchronous); `stream` is a hipStream_t or NULL.  All tensors
+ * are contiguous row-major f32.  Outputs may alias the corresponding inputs (in-place).
+ */
+#ifndef IZWI_DECODE_OPS_H
+#define IZWI_DECODE_OPS_H
+
+#include <stdint.h>
+
+#include "izwi_qmm.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* `try_fused_rms_norm(input, weight, eps)` (kernels/mod.rs:141-155, metal.rs:1979-2024, shader
+ * metal.rs:147-186): y[r, i] = x[r, i] * rsqrt(mean_i(x[r, :]^2) + eps) * weight[i] for `rows` rows
+ * of `hidden` values.  The reference refuses rows == 0 and hidden == 0 (returns None): here rows ==
+ * 0 is a no-op and hidden == 0 is IZWI_QMM_ERR_INVALID. */
+int izwi_rms_norm_f32(const float* x, const float* weight, int64_t rows, int64_t hidden, float eps,
+                      float* y, int mem_space, void* stream);
+
+/* `try_fused_qk_rms_norm(q, k, qk_weight, eps)` (kernels/mod.rs:109-123, metal.rs:1906-1975,
+ * shader metal.rs:59-101): the per-head norms of Qwen3 attention (qwen3/core.rs:1470) in one
+ * launch.  q is `[q_rows, head_dim]` (q_rows = batch * heads for one token), k is
+ * `[k_rows, head_dim]`, qk_weight is `[2 * head_dim]`: q's weights, then k's.  The reference's
+ * shader is limited to head_dim <= 256 and one token; this kernel takes any row counts and
+ * head_dim <= 8192. */
+int izwi_qk_rms_norm_f32(const float* q, const float* k, const float* qk_weight, int64_t q_rows,
+                         int64_t k_rows, int64_t head_dim, float eps, float* q_out, float* k_out,
+                         int mem_space, void* stream);
+
+/* `try_fused_rope_pair_bshd(q, k, cos_sin)` (kernels/mod.rs:157-171, metal.rs:2026-2094, shader
+ * metal.rs:227-265): q is `[batch, seq, q_heads, head_dim]`, k is `[batch, seq, k_heads,
+ * head_dim]`, cos_sin is `[seq, head_dim]` with the cosines in the first half of a row and the
+ * sines in the second; head_dim even.  The two halves of a head rotate against each other:
+ * out[d] = x[d] cos[d] - x[half + d] sin[d], out[half + d] = x[d] sin[d] + x[half + d] cos[d]. */
+int izwi_rope_pair_bshd_f32(const float* q, const float* k, const float* cos_sin, int64_t batch,
+                            int64_t seq, int64_t q_heads, int64_t k_heads, int64_t head_dim,
+                            float* q_out, float* k_out, int mem_space, void* stream);
+
+/* `try_fused_decode_gqa_attention_with_kv_len(q, k, v, num_heads, num_kv_heads, head_dim, kv_len,
+ * scale)` (kernels/mod.rs:199-225, metal.rs:2121-2193, shader metal.rs:307-381): attention of one
+ * query token.  q is `[1, num_heads, 1, head_dim]`, k and v are `[1, num_kv_heads, kv_capacity,
+ * head_dim]` (head-major cache) of which the first kv_len positions count; head h reads kv head
+ * h / (num_heads / num_kv_heads); out is `[1, num_heads, 1, head_dim]`,
+ * softmax_p((q . k_p) * scale) . v.  The reference's shader refuses kv_len > 2048; here the
+ * positions are split over workgroups and merged (any kv_len).  head_dim must be 64, 128 or 256
+ * (IZWI_QMM_ERR_UNSUPPORTED otherwise).  Uses the library's per-stream scratch when the positions
+ * are split. */
+int izwi_decode_gqa_attention_f32(const float* q, const float* k, const float* v, int64_t num_heads,
+                                  int64_t num_kv_heads, int64_t head_dim, int64_t kv_len,
+                                  int64_t kv_capacity, float scale, float* out, int mem_space,
+                                  void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* IZWI_DECODE_OPS_H */

@@ -7,6 +7,13 @@ HIP kernels for gfx950; there is no CPU or PyTorch fallback: if the library is
 missing or no GPU is present, calls raise.
 """
 from .capi import QmmError, lib, library_path  # noqa: F401
+from .decode_ops import (  # noqa: F401
+    try_fused_decode_gqa_attention,
+    try_fused_decode_gqa_attention_with_kv_len,
+    try_fused_qk_rms_norm,
+    try_fused_rms_norm,
+    try_fused_rope_pair_bshd,
+)
 from .gguf import GgufLoader, GgufModelInfo, is_gguf_file  # noqa: F401
 from .qmatmul import (  # noqa: F401
     GgmlDType,

@@ -63,6 +63,11 @@ PROTOTYPES = {
     "izwi_qmm_forward_bf16": (C.c_int, [_vp, _vp, _i64, _vp, C.c_int, C.c_int, _vp]),
     "izwi_qmm_forward_fused": (C.c_int, [_vp, _vp, C.c_int, _i64, _vp, _vp, C.c_int, C.c_int, _vp]),
     "izwi_qmm_quantize_activations": (C.c_int, [C.c_int, _vp, _i64, _i64, _vp, C.c_int, _vp]),
+    "izwi_rms_norm_f32": (C.c_int, [_vp, _vp, _i64, _i64, C.c_float, _vp, C.c_int, _vp]),
+    "izwi_qk_rms_norm_f32": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, C.c_float, _vp, _vp, C.c_int, _vp]),
+    "izwi_rope_pair_bshd_f32": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, C.c_int, _vp]),
+    "izwi_decode_gqa_attention_f32": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, C.c_float, _vp,
+                                                C.c_int, _vp]),
     "izwi_moe_route": (C.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, C.c_int, _vp]),
     "izwi_moe_sort": (C.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, C.c_int, _vp]),
     "izwi_moe_layer_f32": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _vp, _vp, _vp, C.c_int, _vp]),

@@ -1,0 +1,516 @@
+// Decode-step neighbours of the quantized projections: RMSNorm, q/k head norm, rotary
+// embedding, single-token grouped-query attention (f32).  All four are bounded by HBM traffic or,
+// at one token, by launch latency; none is GEMM-shaped.
+//
+//  * norms: one workgroup per row, 16-byte loads when the row allows it, the row stays in
+//    registers between the reduction and the scaling (read once, written once);
+//  * rotary: one thread per (row, pair);
+//  * attention: the KV cache of a kv head is read ONCE for all query heads that share it.
+//    Positions are split over workgroups (enough of them to fill the chip at any cache length),
+//    each keeps running (max, sum, weighted value sum) per head and the splits are merged by a
+//    second small kernel.  Inside a workgroup 8 lanes share a cache row as 8 x 16 B pieces of
+//    every 128-byte segment (coalesced), 32 rows are in flight per workgroup.
+#include <hip/hip_runtime.h>
+
+#include <math.h>
+
+#include "../../include/izwi_decode_ops.h"
+#include "qmm_internal.h"
+
+namespace {
+
+#define OPS_TRY(expr)                                                                     \
+    do {                                                                                  \
+        hipError_t e_ = (expr);                                                           \
+        if (e_ != hipSuccess) {                                                           \
+            (void)hipGetLastError();                                                      \
+            return qmm_fail(IZWI_QMM_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e_));    \
+        }                                                                                 \
+    } while (0)
+
+// Device view of a caller buffer: the pointer itself, or a staged copy of host memory.
+struct Buf {
+    void* dev = nullptr;
+    void* host = nullptr;
+    size_t bytes = 0;
+    bool owned = false, copy_back = false;
+    ~Buf() {
+        if (owned && dev) (void)hipFree(dev);
+    }
+    hipError_t in(const void* p, size_t n, int mem_space) {
+        bytes = n;
+        if (mem_space == IZWI_QMM_DEVICE || n == 0) {
+            dev = const_cast<void*>(p);
+            return hipSuccess;
+        }
+        owned = true;
+        hipError_t e = hipMalloc(&dev, n);
+        return e != hipSuccess ? e : hipMemcpy(dev, p, n, hipMemcpyHostToDevice);
+    }
+    hipError_t out(void* p, size_t n, int mem_space) {
+        bytes = n;
+        if (mem_space == IZWI_QMM_DEVICE || n == 0) {
+            dev = p;
+            return hipSuccess;
+        }
+        owned = copy_back = true;
+        host = p;
+        return hipMalloc(&dev, n);
+    }
+    hipError_t finish(hipStream_t stream) {
+        if (!copy_back) return hipSuccess;
+        hipError_t e = hipStreamSynchronize(stream);
+        return e != hipSuccess ? e : hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost);
+    }
+};
+
+int check_space(int mem_space) {
+    if (mem_space != IZWI_QMM_DEVICE && mem_space != IZWI_QMM_HOST)
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "bad mem_space %d", mem_space);
+    return IZWI_QMM_OK;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+// ---- norms ---------------------------------------------------------------------------
+// Row r < rows_a comes from a / goes to out_a with weight_a, the others from b (the q/k pair);
+// a plain RMSNorm has rows_b == 0.  VEC: hidden is a multiple of 4 and all rows are 16-byte
+// aligned.  A thread keeps up to PER values of its row in registers; longer rows are re-read.
+struct NormParams {
+    const float* a;
+    const float* b;
+    const float* weight_a;
+    const float* weight_b;
+    float* out_a;
+    float* out_b;
+    int64_t rows_a, rows_b;
+    int hidden;
+    float eps;
+};
+
+template <bool VEC>
+__global__ void rms_norm_kernel(NormParams P) {
+    constexpr int PER = 4; // float4s (VEC) or floats kept per thread
+    __shared__ float partial[16];
+    const int64_t row = blockIdx.x;
+    const bool first = row < P.rows_a;
+    const float* x = first ? P.a + row * P.hidden : P.b + (row - P.rows_a) * P.hidden;
+    const float* w = first ? P.weight_a : P.weight_b;
+    float* y = first ? P.out_a + row * P.hidden : P.out_b + (row - P.rows_a) * P.hidden;
+    const int tid = threadIdx.x, nt = blockDim.x;
+    float sum = 0.0f;
+    float4 keep4[PER];
+    float keep1[PER];
+    if (VEC) {
+        const int n4 = P.hidden >> 2;
+        const float4* x4 = reinterpret_cast<const float4*>(x);
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int idx = tid + i * nt;
+            keep4[i] = idx < n4 ? x4[idx] : make_float4(0, 0, 0, 0);
+            sum += keep4[i].x * keep4[i].x + keep4[i].y * keep4[i].y + keep4[i].z * keep4[i].z + keep4[i].w * keep4[i].w;
+        }
+        for (int idx = tid + PER * nt; idx < n4; idx += nt) {
+            const float4 v = x4[idx];
+            sum += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int idx = tid + i * nt;
+            keep1[i] = idx < P.hidden ? x[idx] : 0.0f;
+            sum += keep1[i] * keep1[i];
+        }
+        for (int idx = tid + PER * nt; idx < P.hidden; idx += nt) sum += x[idx] * x[idx];
+    }
+    sum = wave_sum(sum);
+    if ((tid & 63) == 0) partial[tid >> 6] = sum;
+    __syncthreads();
+    float total = 0.0f;
+    for (int i = 0; i < (nt + 63) / 64; i++) total += partial[i];
+    const float scale = 1.0f / sqrtf(total / (float)P.hidden + P.eps);
+    if (VEC) {
+        const int n4 = P.hidden >> 2;
+        const float4* w4 = reinterpret_cast<const float4*>(w);
+        float4* y4 = reinterpret_cast<float4*>(y);
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int idx = tid + i * nt;
+            if (idx < n4) {
+                const float4 ww = w4[idx], v = keep4[i];
+                y4[idx] = make_float4(v.x * scale * ww.x, v.y * scale * ww.y, v.z * scale * ww.z, v.w * scale * ww.w);
+            }
+        }
+        const float4* x4 = reinterpret_cast<const float4*>(x);
+        for (int idx = tid + PER * nt; idx < n4; idx += nt) {
+            const float4 ww = w4[idx], v = x4[idx];
+            y4[idx] = make_float4(v.x * scale * ww.x, v.y * scale * ww.y, v.z * scale * ww.z, v.w * scale * ww.w);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int idx = tid + i * nt;
+            if (idx < P.hidden) y[idx] = keep1[i] * scale * w[idx];
+        }
+        for (int idx = tid + PER * nt; idx < P.hidden; idx += nt) y[idx] = x[idx] * scale * w[idx];
+    }
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+hipError_t launch_norm(const NormParams& P, hipStream_t stream) {
+    const int64_t rows = P.rows_a + P.rows_b;
+    if (rows == 0) return hipSuccess;
+    if (rows > 0x7fffffff) return hipErrorInvalidValue;
+    const bool vec = P.hidden % 4 == 0 && aligned16(P.a) && aligned16(P.out_a) && aligned16(P.weight_a) &&
+                     (P.rows_b == 0 || (aligned16(P.b) && aligned16(P.out_b) && aligned16(P.weight_b)));
+    // one 16-byte piece (or value) per thread up to four per thread; at most 1024 threads
+    const int items = vec ? P.hidden / 4 : P.hidden;
+    int threads = 64;
+    while (threads < 1024 && threads < items) threads *= 2;
+    if (vec) rms_norm_kernel<true><<<(unsigned)rows, threads, 0, stream>>>(P);
+    else rms_norm_kernel<false><<<(unsigned)rows, threads, 0, stream>>>(P);
+    return hipGetLastError();
+}
+
+// ---- rotary embedding ----------------------------------------------------------------------
+__global__ void rope_pair_kernel(const float* __restrict__ cos_sin, const float* q, const float* k, float* q_out,
+                                 float* k_out, int64_t q_rows, int64_t k_rows, int seq, int q_heads, int k_heads,
+                                 int head_dim) {
+    const int half = head_dim >> 1;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (q_rows + k_rows) * half) return;
+    const int64_t row = idx / half;
+    const int d = (int)(idx - row * half);
+    const bool is_q = row < q_rows;
+    const int64_t local = is_q ? row : row - q_rows;
+    const int pos = (int)((local / (is_q ? q_heads : k_heads)) % seq);
+    const float* x = (is_q ? q : k) + local * head_dim;
+    float* y = (is_q ? q_out : k_out) + local * head_dim;
+    const float c = cos_sin[(int64_t)pos * head_dim + d], s = cos_sin[(int64_t)pos * head_dim + half + d];
+    const float x1 = x[d], x2 = x[half + d];
+    y[d] = x1 * c - x2 * s;
+    y[half + d] = x1 * s + x2 * c;
+}
+
+// ---- single-token GQA attention ------------------------------------------------------------
+struct AttnParams {
+    const float* q;
+    const float* k;
+    const float* v;
+    float* out;
+    float* part; // [heads][splits][head_dim + 2]: weighted value sums, running max, sum of weights
+    int heads, kv_heads, group;
+    int kv_len, chunk, splits; // split s covers positions [s * chunk, min(kv_len, (s + 1) * chunk))
+    int64_t kv_capacity;
+    float scale;
+};
+
+// weight of a partial result with running maximum m when merged under the maximum mn
+__device__ __forceinline__ float merge_weight(float m, float mn) { return m == -INFINITY ? 0.0f : expf(m - mn); }
+
+// NI = head_dim / 32; G query heads of one kv head per workgroup.  Lane j of an 8-lane row group
+// holds the elements 32 i + 4 j + c (i < NI, c < 4) of a cache row and of the query heads.
+template <int NI, int G>
+__global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
+    constexpr int HD = 32 * NI, E = 4 * NI;
+    __shared__ float red[4][G][HD + 2];
+    const int kvh = blockIdx.x, sp = blockIdx.y, h0 = kvh * P.group + blockIdx.z * G;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane & 7, slot = wave * 8 + (lane >> 3);
+
+    float qr[G][E];
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            const float4 t = *reinterpret_cast<const float4*>(P.q + (int64_t)(h0 + g) * HD + 32 * i + 4 * j);
+            qr[g][4 * i] = t.x, qr[g][4 * i + 1] = t.y, qr[g][4 * i + 2] = t.z, qr[g][4 * i + 3] = t.w;
+        }
+    float m[G], l[G], acc[G][E];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        m[g] = -INFINITY;
+        l[g] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < E; e++) acc[g][e] = 0.0f;
+    }
+    const int p0 = sp * P.chunk, p1 = min(P.kv_len, p0 + P.chunk);
+    const float* kb = P.k + (int64_t)kvh * P.kv_capacity * HD + 4 * j;
+    const float* vb = P.v + (int64_t)kvh * P.kv_capacity * HD + 4 * j;
+    for (int p = p0 + slot; p < p1; p += 32) {
+        float4 kr[NI], vr[NI];
+#pragma unroll
+        for (int i = 0; i < NI; i++) kr[i] = *reinterpret_cast<const float4*>(kb + (int64_t)p * HD + 32 * i);
+#pragma unroll
+        for (int i = 0; i < NI; i++) vr[i] = *reinterpret_cast<const float4*>(vb + (int64_t)p * HD + 32 * i);
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float dot = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NI; i++)
+                dot += qr[g][4 * i] * kr[i].x + qr[g][4 * i + 1] * kr[i].y + qr[g][4 * i + 2] * kr[i].z +
+                       qr[g][4 * i + 3] * kr[i].w;
+            dot += __shfl_xor(dot, 1);
+            dot += __shfl_xor(dot, 2);
+            dot += __shfl_xor(dot, 4);
+            const float s = dot * P.scale;
+            const float mn = fmaxf(m[g], s);
+            const float alpha = merge_weight(m[g], mn), pe = expf(s - mn);
+            l[g] = l[g] * alpha + pe;
+#pragma unroll
+            for (int i = 0; i < NI; i++) {
+                acc[g][4 * i] = acc[g][4 * i] * alpha + pe * vr[i].x;
+                acc[g][4 * i + 1] = acc[g][4 * i + 1] * alpha + pe * vr[i].y;
+                acc[g][4 * i + 2] = acc[g][4 * i + 2] * alpha + pe * vr[i].z;
+                acc[g][4 * i + 3] = acc[g][4 * i + 3] * alpha + pe * vr[i].w;
+            }
+            m[g] = mn;
+        }
+    }
+    // merge the 8 row groups of the wave (lane bits 3..5), then the 4 waves through LDS
+#pragma unroll
+    for (int o = 8; o < 64; o <<= 1) {
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const float mo = __shfl_xor(m[g], o), lo = __shfl_xor(l[g], o);
+            const float mn = fmaxf(m[g], mo);
+            const float wa = merge_weight(m[g], mn), wb = merge_weight(mo, mn);
+            l[g] = l[g] * wa + lo * wb;
+#pragma unroll
+            for (int e = 0; e < E; e++) acc[g][e] = acc[g][e] * wa + __shfl_xor(acc[g][e], o) * wb;
+            m[g] = mn;
+        }
+    }
+    if (lane < 8) {
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+#pragma unroll
+            for (int i = 0; i < NI; i++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) red[wave][g][32 * i + 4 * j + c] = acc[g][4 * i + c];
+            if (j == 0) red[wave][g][HD] = m[g], red[wave][g][HD + 1] = l[g];
+        }
+    }
+    __syncthreads();
+    for (int t = threadIdx.x; t < G * HD; t += 256) {
+        const int g = t / HD, d = t - g * HD;
+        float mn = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; w++) mn = fmaxf(mn, red[w][g][HD]);
+        float a = 0.0f, lsum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float ww = merge_weight(red[w][g][HD], mn);
+            a += red[w][g][d] * ww;
+            lsum += red[w][g][HD + 1] * ww;
+        }
+        const int h = h0 + g;
+        if (P.splits == 1) {
+            P.out[(int64_t)h * HD + d] = a * (1.0f / lsum);
+        } else {
+            float* dst = P.part + ((int64_t)h * P.splits + sp) * (HD + 2);
+            dst[d] = a;
+            if (d == 0) dst[HD] = mn, dst[HD + 1] = lsum;
+        }
+    }
+}
+
+// out[h] = merge of the splits' partial results
+__global__ void attn_merge_kernel(const float* __restrict__ part, float* __restrict__ out, int splits, int head_dim) {
+    const int h = blockIdx.x;
+    const float* base = part + (int64_t)h * splits * (head_dim + 2);
+    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+        float mn = -INFINITY;
+        for (int s = 0; s < splits; s++) mn = fmaxf(mn, base[(int64_t)s * (head_dim + 2) + head_dim]);
+        float a = 0.0f, lsum = 0.0f;
+        for (int s = 0; s < splits; s++) {
+            const float* ps = base + (int64_t)s * (head_dim + 2);
+            const float w = merge_weight(ps[head_dim], mn);
+            a += ps[d] * w;
+            lsum += ps[head_dim + 1] * w;
+        }
+        out[(int64_t)h * head_dim + d] = a * (1.0f / lsum);
+    }
+}
+
+template <int NI>
+hipError_t launch_attn_partial(const AttnParams& P, int g, dim3 grid, hipStream_t stream) {
+    if (g == 4) {
+        if constexpr (NI <= 4) attn_partial_kernel<NI, 4><<<grid, 256, 0, stream>>>(P);
+        else return hipErrorInvalidValue;
+    } else if (g == 2) {
+        attn_partial_kernel<NI, 2><<<grid, 256, 0, stream>>>(P);
+    } else {
+        attn_partial_kernel<NI, 1><<<grid, 256, 0, stream>>>(P);
+    }
+    return hipGetLastError();
+}
+
+} // namespace
+
+extern "C" {
+
+int izwi_rms_norm_f32(const float* x, const float* weight, int64_t rows, int64_t hidden, float eps, float* y,
+                      int mem_space, void* stream_) {
+    if (int rc = check_space(mem_space)) return rc;
+    if (rows < 0 || hidden <= 0 || hidden > 0x3fffffff)
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "rms_norm: bad shape [%lld, %lld]", (long long)rows, (long long)hidden);
+    if (rows == 0) return IZWI_QMM_OK;
+    if (!x || !weight || !y) return qmm_fail(IZWI_QMM_ERR_INVALID, "rms_norm: NULL buffer");
+    int device = 0, n_cus = 0;
+    if (int rc = qmm_current_device(&device, &n_cus)) return rc;
+    hipStream_t stream = (hipStream_t)stream_;
+    Buf xi, wi, yo;
+    OPS_TRY(xi.in(x, (size_t)rows * hidden * sizeof(float), mem_space));
+    OPS_TRY(wi.in(weight, (size_t)hidden * sizeof(float), mem_space));
+    OPS_TRY(yo.out(y, (size_t)rows * hidden * sizeof(float), mem_space));
+    NormParams P{(const float*)xi.dev, nullptr, (const float*)wi.dev, nullptr, (float*)yo.dev, nullptr, rows, 0,
+                 (int)hidden, eps};
+    OPS_TRY(launch_norm(P, stream));
+    OPS_TRY(yo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qk_rms_norm_f32(const float* q, const float* k, const float* qk_weight, int64_t q_rows, int64_t k_rows,
+                         int64_t head_dim, float eps, float* q_out, float* k_out, int mem_space, void* stream_) {
+    if (int rc = check_space(mem_space)) return rc;
+    if (q_rows < 0 || k_rows < 0 || head_dim <= 0 || head_dim > 8192)
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "qk_rms_norm: bad shape q [%lld, %lld], k [%lld, %lld]", (long long)q_rows,
+                        (long long)head_dim, (long long)k_rows, (long long)head_dim);
+    if (q_rows + k_rows == 0) return IZWI_QMM_OK;
+    if (!qk_weight || (q_rows && (!q || !q_out)) || (k_rows && (!k || !k_out)))
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "qk_rms_norm: NULL buffer");
+    int device = 0, n_cus = 0;
+    if (int rc = qmm_current_device(&device, &n_cus)) return rc;
+    hipStream_t stream = (hipStream_t)stream_;
+    Buf qi, ki, wi, qo, ko;
+    OPS_TRY(qi.in(q, (size_t)q_rows * head_dim * sizeof(float), mem_space));
+    OPS_TRY(ki.in(k, (size_t)k_rows * head_dim * sizeof(float), mem_space));
+    OPS_TRY(wi.in(qk_weight, (size_t)2 * head_dim * sizeof(float), mem_space));
+    OPS_TRY(qo.out(q_out, (size_t)q_rows * head_dim * sizeof(float), mem_space));
+    OPS_TRY(ko.out(k_out, (size_t)k_rows * head_dim * sizeof(float), mem_space));
+    // (with no q rows the first operand of the kernel is the k tensor)
+    NormParams P;
+    if (q_rows)
+        P = NormParams{(const float*)qi.dev, (const float*)ki.dev, (const float*)wi.dev, (const float*)wi.dev + head_dim,
+                       (float*)qo.dev, (float*)ko.dev, q_rows, k_rows, (int)head_dim, eps};
+    else
+        P = NormParams{(const float*)ki.dev, nullptr, (const float*)wi.dev + head_dim, nullptr, (float*)ko.dev, nullptr,
+                       k_rows, 0, (int)head_dim, eps};
+    if (P.rows_b == 0) P.b = nullptr, P.weight_b = nullptr, P.out_b = nullptr;
+    OPS_TRY(launch_norm(P, stream));
+    OPS_TRY(qo.finish(stream));
+    OPS_TRY(ko.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_rope_pair_bshd_f32(const float* q, const float* k, const float* cos_sin, int64_t batch, int64_t seq,
+                            int64_t q_heads, int64_t k_heads, int64_t head_dim, float* q_out, float* k_out,
+                            int mem_space, void* stream_) {
+    if (int rc = check_space(mem_space)) return rc;
+    if (batch < 0 || seq < 0 || q_heads < 0 || k_heads < 0 || head_dim <= 0 || head_dim % 2 || head_dim > 0x3fffffff ||
+        seq > 0x3fffffff || q_heads > 0x3fffffff || k_heads > 0x3fffffff)
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "rope_pair_bshd: bad shape [%lld, %lld, %lld | %lld, %lld] (head_dim must be even)",
+                        (long long)batch, (long long)seq, (long long)q_heads, (long long)k_heads, (long long)head_dim);
+    const int64_t q_rows = batch * seq * q_heads, k_rows = batch * seq * k_heads;
+    if (q_rows + k_rows == 0) return IZWI_QMM_OK;
+    if (!cos_sin || (q_rows && (!q || !q_out)) || (k_rows && (!k || !k_out)))
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "rope_pair_bshd: NULL buffer");
+    int device = 0, n_cus = 0;
+    if (int rc = qmm_current_device(&device, &n_cus)) return rc;
+    hipStream_t stream = (hipStream_t)stream_;
+    Buf qi, ki, ci, qo, ko;
+    OPS_TRY(qi.in(q, (size_t)q_rows * head_dim * sizeof(float), mem_space));
+    OPS_TRY(ki.in(k, (size_t)k_rows * head_dim * sizeof(float), mem_space));
+    OPS_TRY(ci.in(cos_sin, (size_t)seq * head_dim * sizeof(float), mem_space));
+    OPS_TRY(qo.out(q_out, (size_t)q_rows * head_dim * sizeof(float), mem_space));
+    OPS_TRY(ko.out(k_out, (size_t)k_rows * head_dim * sizeof(float), mem_space));
+    const int64_t pairs = (q_rows + k_rows) * (head_dim / 2);
+    const int64_t grid = (pairs + 255) / 256;
+    if (grid > 0x7fffffff) return qmm_fail(IZWI_QMM_ERR_UNSUPPORTED, "rope_pair_bshd: too many elements");
+    rope_pair_kernel<<<(unsigned)grid, 256, 0, stream>>>((const float*)ci.dev, (const float*)qi.dev, (const float*)ki.dev,
+                                                         (float*)qo.dev, (float*)ko.dev, q_rows, k_rows, (int)seq,
+                                                         (int)(q_heads ? q_heads : 1), (int)(k_heads ? k_heads : 1),
+                                                         (int)head_dim);
+    OPS_TRY(hipGetLastError());
+    OPS_TRY(qo.finish(stream));
+    OPS_TRY(ko.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_decode_gqa_attention_f32(const float* q, const float* k, const float* v, int64_t num_heads,
+                                  int64_t num_kv_heads, int64_t head_dim, int64_t kv_len, int64_t kv_capacity,
+                                  float scale, float* out, int mem_space, void* stream_) {
+    if (int rc = check_space(mem_space)) return rc;
+    if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || num_heads > 65535 || kv_len <= 0 ||
+        kv_len > kv_capacity || kv_capacity > 0x3fffffff || head_dim <= 0)
+        return qmm_fail(IZWI_QMM_ERR_INVALID,
+                        "decode_gqa_attention: bad shape (heads %lld, kv heads %lld, head_dim %lld, kv_len %lld of %lld)",
+                        (long long)num_heads, (long long)num_kv_heads, (long long)head_dim, (long long)kv_len,
+                        (long long)kv_capacity);
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+        return qmm_fail(IZWI_QMM_ERR_UNSUPPORTED, "decode_gqa_attention: head_dim %lld (64, 128 and 256 are built)",
+                        (long long)head_dim);
+    if (!q || !k || !v || !out) return qmm_fail(IZWI_QMM_ERR_INVALID, "decode_gqa_attention: NULL buffer");
+    int device = 0, n_cus = 0;
+    if (int rc = qmm_current_device(&device, &n_cus)) return rc;
+    hipStream_t stream = (hipStream_t)stream_;
+    const size_t qbytes = (size_t)num_heads * head_dim * sizeof(float);
+    const size_t cbytes = (size_t)num_kv_heads * kv_capacity * head_dim * sizeof(float);
+    Buf qi, ki, vi, oo;
+    OPS_TRY(qi.in(q, qbytes, mem_space));
+    OPS_TRY(ki.in(k, cbytes, mem_space));
+    OPS_TRY(vi.in(v, cbytes, mem_space));
+    OPS_TRY(oo.out(out, qbytes, mem_space));
+    const int group = (int)(num_heads / num_kv_heads);
+    // query heads per workgroup: as many of the group as the register file takes
+    int g = group % 4 == 0 && head_dim <= 128 ? 4 : (group % 2 == 0 ? 2 : 1);
+    const int z = group / g;
+    // enough workgroups for two per CU, at least 64 positions each (two per row group)
+    const int64_t base_wgs = num_kv_heads * z;
+    int64_t splits = (2 * (int64_t)n_cus + base_wgs - 1) / base_wgs;
+    const int64_t max_splits = (kv_len + 63) / 64;
+    if (splits > max_splits) splits = max_splits;
+    if (splits > 1024) splits = 1024;
+    if (splits < 1) splits = 1;
+    const int chunk = (int)((kv_len + splits - 1) / splits);
+    splits = (kv_len + chunk - 1) / chunk; // every split holds at least one position
+    AttnParams P;
+    P.q = (const float*)qi.dev;
+    P.k = (const float*)ki.dev;
+    P.v = (const float*)vi.dev;
+    P.out = (float*)oo.dev;
+    P.part = nullptr;
+    P.heads = (int)num_heads;
+    P.kv_heads = (int)num_kv_heads;
+    P.group = group;
+    P.kv_len = (int)kv_len;
+    P.chunk = chunk;
+    P.splits = (int)splits;
+    P.kv_capacity = kv_capacity;
+    P.scale = scale;
+    if (splits > 1) {
+        void* scratch = nullptr;
+        OPS_TRY(qmm_get_scratch(device, stream, (size_t)num_heads * splits * (head_dim + 2) * sizeof(float), &scratch));
+        P.part = (float*)scratch;
+    }
+    const dim3 grid((unsigned)num_kv_heads, (unsigned)splits, (unsigned)z);
+    hipError_t e = head_dim == 64    ? launch_attn_partial<2>(P, g, grid, stream)
+                   : head_dim == 128 ? launch_attn_partial<4>(P, g, grid, stream)
+                                     : launch_attn_partial<8>(P, g, grid, stream);
+    OPS_TRY(e);
+    if (splits > 1) {
+        attn_merge_kernel<<<(unsigned)num_heads, head_dim >= 128 ? 128 : 64, 0, stream>>>(P.part, P.out, (int)splits,
+                                                                                          (int)head_dim);
+        OPS_TRY(hipGetLastError());
+    }
+    OPS_TRY(oo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+} // extern "C"

@@ -337,6 +337,16 @@ struct ProfileScope {
 
 } // namespace
 
+// The current device, checked (a gfx950 device is present) and with its CU count; the library's
+// per-(device, stream) scratch buffer.  For the other source files of the library.
+int qmm_current_device(int* device, int* n_cus) {
+    if (int rc = current_device(device)) return rc;
+    return ensure_device(*device, n_cus);
+}
+hipError_t qmm_get_scratch(int device, hipStream_t stream, size_t bytes, void** out) {
+    return get_scratch(device, stream, bytes, out);
+}
+
 extern "C" {
 
 int izwi_qmm_abi_version(void) { return IZWI_QMM_ABI_VERSION; }

@@ -83,6 +83,12 @@ __device__ __forceinline__ void qmm_store(void* y, const QmmEpilogue& ep, int64_
 // Records the calling thread's error message (read with izwi_qmm_last_error) and returns `code`.
 int qmm_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 
+// The current HIP device, validated (IZWI_QMM_ERR_NO_DEVICE without one), and its CU count.
+int qmm_current_device(int* device, int* n_cus);
+// The library's scratch buffer of (device, stream): at least `bytes`, reused by the next call on
+// the same stream (work on a stream is ordered); grows with hipMalloc, never shrinks.
+hipError_t qmm_get_scratch(int device, hipStream_t stream, size_t bytes, void** out);
+
 // ---- launchers -------------------------------------------------------------
 hipError_t qmm_launch_repack(const QmmLayout& L, const void* native, void* tiled,
                              hipStream_t stream);

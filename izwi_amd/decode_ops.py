@@ -1,0 +1,84 @@
+"""Host-side mirror of the reference's fused-kernel hooks for the decode step
+(crates/izwi-core/src/kernels/mod.rs:109-225): the same names, argument meaning and "return None
+when the fused path does not apply" behaviour, over the C ABI of include/izwi_decode_ops.h.
+
+A hook returns None (the caller then runs its own eager operators, as the reference does) when
+its preconditions do not hold: f32, contiguous, on one GPU, the shapes the reference's wrapper
+checks (metal.rs:1921-1945, 1991-2003, 2043-2062, 2141-2172).  When they hold the HIP kernel runs;
+a failure inside it raises (there is no silent CPU path)."""
+from __future__ import annotations
+
+import torch
+
+from .capi import DEVICE, check, lib
+from .qmatmul import _stream_ptr
+
+
+def _ok(*tensors: torch.Tensor) -> bool:
+    dev = tensors[0].device
+    return all(t.is_cuda and t.device == dev and t.dtype == torch.float32 and t.is_contiguous() for t in tensors)
+
+
+def try_fused_rms_norm(input: torch.Tensor, weight: torch.Tensor, eps: float):  # noqa: A002
+    """kernels/mod.rs:141-155: input [..., hidden], weight [hidden] -> x * rsqrt(mean(x^2) + eps) * weight."""
+    if input.dim() < 1 or not _ok(input, weight):
+        return None
+    hidden = input.shape[-1]
+    if hidden == 0 or tuple(weight.shape) != (hidden,) or input.numel() == 0:
+        return None
+    out = torch.empty_like(input)
+    check(lib().izwi_rms_norm_f32(input.data_ptr(), weight.data_ptr(), input.numel() // hidden, hidden, eps,
+                                  out.data_ptr(), DEVICE, _stream_ptr(input)))
+    return out
+
+
+def try_fused_qk_rms_norm(q: torch.Tensor, k: torch.Tensor, qk_weight: torch.Tensor, eps: float):
+    """kernels/mod.rs:109-123: q [b, 1, heads, d], k [b, 1, kv_heads, d], qk_weight [2 d] -> (q_norm, k_norm)."""
+    if q.dim() != 4 or k.dim() != 4 or not _ok(q, k, qk_weight):
+        return None
+    if q.shape[1] != 1 or k.shape[1] != 1 or q.shape[0] != k.shape[0] or q.shape[3] != k.shape[3]:
+        return None
+    d = q.shape[3]
+    if d == 0 or tuple(qk_weight.shape) != (2 * d,):
+        return None
+    q_out, k_out = torch.empty_like(q), torch.empty_like(k)
+    check(lib().izwi_qk_rms_norm_f32(q.data_ptr(), k.data_ptr(), qk_weight.data_ptr(), q.numel() // d, k.numel() // d,
+                                     d, eps, q_out.data_ptr(), k_out.data_ptr(), DEVICE, _stream_ptr(q)))
+    return q_out, k_out
+
+
+def try_fused_rope_pair_bshd(q: torch.Tensor, k: torch.Tensor, cos_sin: torch.Tensor):
+    """kernels/mod.rs:157-171: q [b, s, hq, d], k [b, s, hk, d], cos_sin [s, d] (cos | sin) -> (q_rot, k_rot)."""
+    if q.dim() != 4 or k.dim() != 4 or not _ok(q, k, cos_sin):
+        return None
+    b, s, hq, d = q.shape
+    if k.shape[0] != b or k.shape[1] != s or k.shape[3] != d or d == 0 or d % 2 or tuple(cos_sin.shape) != (s, d):
+        return None
+    q_out, k_out = torch.empty_like(q), torch.empty_like(k)
+    check(lib().izwi_rope_pair_bshd_f32(q.data_ptr(), k.data_ptr(), cos_sin.data_ptr(), b, s, hq, k.shape[2], d,
+                                        q_out.data_ptr(), k_out.data_ptr(), DEVICE, _stream_ptr(q)))
+    return q_out, k_out
+
+
+def try_fused_decode_gqa_attention_with_kv_len(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: int,
+                                               num_kv_heads: int, head_dim: int, kv_len: int, scale: float):
+    """kernels/mod.rs:199-225: q [1, heads, 1, d], k / v [1, kv_heads, capacity, d], the first kv_len positions
+    count -> [1, heads, 1, d].  No limit on kv_len (the reference's shader stops at 2048)."""
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4 or not _ok(q, k, v):
+        return None
+    if (tuple(q.shape) != (1, num_heads, 1, head_dim) or k.shape[0] != 1 or k.shape[1] != num_kv_heads
+            or k.shape[3] != head_dim or tuple(v.shape) != tuple(k.shape) or kv_len == 0 or kv_len > k.shape[2]
+            or num_heads == 0 or num_kv_heads == 0 or num_heads % num_kv_heads or head_dim not in (64, 128, 256)):
+        return None
+    out = torch.empty_like(q)
+    check(lib().izwi_decode_gqa_attention_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), num_heads, num_kv_heads,
+                                              head_dim, kv_len, k.shape[2], scale, out.data_ptr(), DEVICE,
+                                              _stream_ptr(q)))
+    return out
+
+
+def try_fused_decode_gqa_attention(q, k, v, num_heads: int, num_kv_heads: int, head_dim: int, scale: float):
+    """kernels/mod.rs:173-197: all cached positions count."""
+    if k.dim() != 4:
+        return None
+    return try_fused_decode_gqa_attention_with_kv_len(q, k, v, num_heads, num_kv_heads, head_dim, k.shape[2], scale)

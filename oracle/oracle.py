@@ -65,6 +65,15 @@ def lib() -> C.CDLL:
                                          vp, vp, vp, vp, vp, vp, vp]
         L.oracle_fill_normal.restype = None
         L.oracle_fill_normal.argtypes = [C.c_uint64, i64, i64, C.c_float, C.c_float, vp]
+        f32 = C.c_float
+        L.oracle_rms_norm.restype = None
+        L.oracle_rms_norm.argtypes = [vp, vp, i64, i64, f32, vp]
+        L.oracle_qk_rms_norm.restype = None
+        L.oracle_qk_rms_norm.argtypes = [vp, vp, vp, i64, i64, i64, f32, vp, vp]
+        L.oracle_rope_pair_bshd.restype = None
+        L.oracle_rope_pair_bshd.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, vp, vp]
+        L.oracle_decode_gqa_attention.restype = C.c_int
+        L.oracle_decode_gqa_attention.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, f32, vp]
         L.oracle_get_scale_min_k4.restype = None
         L.oracle_get_scale_min_k4.argtypes = [C.c_int, vp, vp, vp]
         _lib = L
@@ -176,4 +185,49 @@ def moe_forward(dtype: int, x: np.ndarray, ids: np.ndarray, wts: np.ndarray, gat
                                   _ptr(wts), _ptr(gate), _ptr(up), _ptr(down), _ptr(out))
     if rc:
         raise ValueError("oracle_moe_forward rejected the shape")
+    return out
+
+
+# ---- decode-step neighbours (decode_ops_oracle.c) ---------------------------------------
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def rms_norm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:
+    """`try_fused_rms_norm`: x [..., hidden], weight [hidden]."""
+    x, weight = _f32(x), _f32(weight)
+    out = np.empty_like(x)
+    hidden = x.shape[-1]
+    lib().oracle_rms_norm(_ptr(x), _ptr(weight), x.size // hidden, hidden, eps, _ptr(out))
+    return out
+
+
+def qk_rms_norm(q: np.ndarray, k: np.ndarray, qk_weight: np.ndarray, eps: float):
+    """`try_fused_qk_rms_norm`: q, k [..., head_dim], qk_weight [2 * head_dim]."""
+    q, k, qk_weight = _f32(q), _f32(k), _f32(qk_weight)
+    d = q.shape[-1]
+    qo, ko = np.empty_like(q), np.empty_like(k)
+    lib().oracle_qk_rms_norm(_ptr(q), _ptr(k), _ptr(qk_weight), q.size // d, k.size // d, d, eps, _ptr(qo), _ptr(ko))
+    return qo, ko
+
+
+def rope_pair_bshd(q: np.ndarray, k: np.ndarray, cos_sin: np.ndarray):
+    """`try_fused_rope_pair_bshd`: q [b, s, hq, d], k [b, s, hk, d], cos_sin [s, d]."""
+    q, k, cos_sin = _f32(q), _f32(k), _f32(cos_sin)
+    b, s, hq, d = q.shape
+    qo, ko = np.empty_like(q), np.empty_like(k)
+    lib().oracle_rope_pair_bshd(_ptr(q), _ptr(k), _ptr(cos_sin), b, s, hq, k.shape[2], d, _ptr(qo), _ptr(ko))
+    return qo, ko
+
+
+def decode_gqa_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, kv_len: int, scale: float) -> np.ndarray:
+    """`try_fused_decode_gqa_attention_with_kv_len`: q [1, heads, 1, d], k / v [1, kv_heads, capacity, d]."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    _, heads, _, d = q.shape
+    _, kv_heads, cap, _ = k.shape
+    out = np.empty_like(q)
+    rc = lib().oracle_decode_gqa_attention(_ptr(q), _ptr(k), _ptr(v), heads, kv_heads, d, kv_len, cap, scale, _ptr(out))
+    if rc:
+        raise ValueError("oracle_decode_gqa_attention rejected the shape")
     return out

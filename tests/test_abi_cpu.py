@@ -11,10 +11,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def header_symbols():
     names = set()
-    for header in ("izwi_qmm.h", "izwi_gguf.h"):
+    for header in ("izwi_qmm.h", "izwi_gguf.h", "izwi_decode_ops.h"):
         text = open(os.path.join(ROOT, "include", header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-        names |= set(re.findall(r"\b(izwi_(?:qmm|moe|gguf)_[a-z0-9_]+)\s*\(", text))
+        names |= set(re.findall(r"\b(izwi_(?:qmm|moe|gguf|rms|qk|rope|decode)_[a-z0-9_]+)\s*\(", text))
     return sorted(names)
 
 

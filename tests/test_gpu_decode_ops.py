@@ -1,0 +1,188 @@
+"""GPU parity of the decode-step neighbours (pytest -m gpu): the HIP kernels behind the
+reference's fused-kernel hooks against the CPU oracle, through the C ABI.  Tolerance: the
+reference's own 1e-5 for f32 (kernels/metal.rs:2956), absolute on its O(1) test vectors and
+relative to max|y| on the model-sized inputs."""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+
+
+def _say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def qa():
+    if not torch.cuda.is_available():
+        pytest.fail("no GPU visible: the HIP path cannot run (there is no fallback)")
+    import izwi_amd
+    izwi_amd.lib()
+    torch.cuda.set_device(0)
+    return izwi_amd
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+def close(got, want, tol=TOL):
+    want = np.asarray(want, dtype=np.float64)
+    return float(np.abs(got.cpu().numpy() - want).max()) <= tol * max(1.0, float(np.abs(want).max()))
+
+
+REF_X3 = np.array([0.2, -0.4, 0.6, 0.8, -1.0, 1.2, -1.4, 1.6, 1.8, -2.0, 2.2, -2.4], np.float32)
+REF_W = np.array([1.0, 1.1, 0.9, 0.8], np.float32)
+
+
+def test_reference_test_vectors(qa, oracle):
+    """The four cases of the reference's own tests (metal.rs:2917-3290)."""
+    x = REF_X3.reshape(1, 3, 4)
+    assert close(qa.try_fused_rms_norm(dev(x), dev(REF_W), 1e-6), oracle.rms_norm(x, REF_W, 1e-6))
+    q = REF_X3[:8].reshape(1, 1, 2, 4)
+    k = np.array([0.3, -0.5, 0.7, -0.9], np.float32).reshape(1, 1, 1, 4)
+    qkw = np.concatenate([REF_W, np.array([0.7, 1.2, 0.6, 1.3], np.float32)])
+    qo, ko = qa.try_fused_qk_rms_norm(dev(q), dev(k), dev(qkw), 1e-6)
+    wq, wk = oracle.qk_rms_norm(q, k, qkw, 1e-6)
+    assert close(qo, wq) and close(ko, wk) and qo.shape == (1, 1, 2, 4) and ko.shape == (1, 1, 1, 4)
+    q = np.array([0.2, -0.4, 0.6, 0.8, -1.0, 1.2, -1.4, 1.6, 1.8, -2.0, 2.2, -2.4, -2.6, 2.8, -3.0, 3.2],
+                 np.float32).reshape(1, 2, 2, 4)
+    k = np.array([0.3, -0.5, 0.7, -0.9, 1.1, -1.3, 1.5, -1.7], np.float32).reshape(1, 2, 1, 4)
+    cs = np.array([[0.9, 0.8, 0.1, 0.2], [0.7, 0.6, 0.3, 0.4]], np.float32)
+    qo, ko = qa.try_fused_rope_pair_bshd(dev(q), dev(k), dev(cs))
+    wq, wk = oracle.rope_pair_bshd(q, k, cs)
+    assert close(qo, wq) and close(ko, wk)
+    # attention: head_dim 4 is below what the kernel is built for -> the hook declines (None), as the
+    # reference's does off Metal; the same case at head_dim 64 (zero-padded) is computed
+    q4 = REF_X3[:8].reshape(1, 2, 1, 4)
+    k4 = np.array([0.3, -0.5, 0.7, -0.9, 1.1, -1.3, 1.5, -1.7, 1.9, -2.1, 2.3, -2.5], np.float32).reshape(1, 1, 3, 4)
+    v4 = np.array([-0.2, 0.4, -0.6, 0.8, 1.0, -1.2, 1.4, -1.6, -1.8, 2.0, -2.2, 2.4], np.float32).reshape(1, 1, 3, 4)
+    assert qa.try_fused_decode_gqa_attention(dev(q4), dev(k4), dev(v4), 2, 1, 4, 0.5) is None
+    pad = lambda a: np.concatenate([a, np.zeros(a.shape[:-1] + (60,), np.float32)], axis=-1)  # noqa: E731
+    want = oracle.decode_gqa_attention(q4, k4, v4, 3, 0.5)
+    got = qa.try_fused_decode_gqa_attention(dev(pad(q4)), dev(pad(k4)), dev(pad(v4)), 2, 1, 64, 0.5)
+    assert close(got[..., :4], want) and not got[..., 4:].any()
+    # cache with capacity 5 whose tail must be ignored (metal.rs:3153-3181)
+    k5 = np.concatenate([k4, np.array([90, 91, 92, 93, -90, -91, -92, -93], np.float32).reshape(1, 1, 2, 4)], axis=2)
+    v5 = np.concatenate([v4, np.array([80, 81, 82, 83, -80, -81, -82, -83], np.float32).reshape(1, 1, 2, 4)], axis=2)
+    got = qa.try_fused_decode_gqa_attention_with_kv_len(dev(pad(q4)), dev(pad(k5)), dev(pad(v5)), 2, 1, 64, 3, 0.5)
+    assert close(got[..., :4], want)
+
+
+@pytest.mark.parametrize("rows,hidden", [(1, 4096), (16, 4096), (64, 4096), (3, 1024), (5, 100), (2, 6), (1, 12288),
+                                         (2, 20000), (7, 5120)])
+def test_rms_norm_shapes(qa, oracle, rows, hidden):
+    _say(f"rms_norm rows={rows} hidden={hidden}")
+    x = oracle.randn(rows + hidden, (rows, hidden))
+    w = oracle.randn(3, (hidden,), mean=1.0, std=0.1)
+    xd = dev(x)
+    got = qa.try_fused_rms_norm(xd, dev(w), 1e-6)
+    assert close(got, oracle.rms_norm(x, w, 1e-6))
+    # a view that is not 16-byte aligned takes the scalar path: same values within rounding
+    if hidden > 8:
+        flat = torch.zeros(rows * hidden + 1, device="cuda")
+        flat[1:] = xd.reshape(-1)
+        assert close(qa.try_fused_rms_norm(flat[1:].view(rows, hidden), dev(w), 1e-6), oracle.rms_norm(x, w, 1e-6))
+
+
+def test_rms_norm_in_place_through_the_c_abi(qa, oracle):
+    from izwi_amd import capi
+    x = oracle.randn(1, (4, 4096))
+    w = oracle.randn(2, (4096,), mean=1.0, std=0.1)
+    buf, wd = dev(x), dev(w)
+    assert capi.lib().izwi_rms_norm_f32(buf.data_ptr(), wd.data_ptr(), 4, 4096, 1e-6, buf.data_ptr(), capi.DEVICE, None) == 0
+    assert close(buf, oracle.rms_norm(x, w, 1e-6))
+    # host pointers
+    out = np.empty_like(x)
+    assert capi.lib().izwi_rms_norm_f32(x.ctypes.data, w.ctypes.data, 4, 4096, 1e-6, out.ctypes.data, capi.HOST, None) == 0
+    assert np.abs(out - oracle.rms_norm(x, w, 1e-6)).max() <= 1e-5 * np.abs(out).max()
+    assert capi.lib().izwi_rms_norm_f32(buf.data_ptr(), wd.data_ptr(), 4, 0, 1e-6, buf.data_ptr(), capi.DEVICE, None) == -1
+    assert capi.lib().izwi_rms_norm_f32(buf.data_ptr(), wd.data_ptr(), 0, 4096, 1e-6, buf.data_ptr(), capi.DEVICE, None) == 0
+
+
+@pytest.mark.parametrize("b,hq,hk,d", [(1, 32, 8, 128), (4, 32, 8, 128), (1, 16, 8, 64), (2, 5, 1, 256), (1, 3, 2, 20)])
+def test_qk_rms_norm_shapes(qa, oracle, b, hq, hk, d):
+    q, k = oracle.randn(1, (b, 1, hq, d)), oracle.randn(2, (b, 1, hk, d))
+    w = oracle.randn(3, (2 * d,), mean=1.0, std=0.2)
+    qo, ko = qa.try_fused_qk_rms_norm(dev(q), dev(k), dev(w), 1e-6)
+    wq, wk = oracle.qk_rms_norm(q, k, w, 1e-6)
+    assert close(qo, wq) and close(ko, wk)
+    # the pair equals two plain norms with the two halves of the weight
+    assert torch.equal(qo, qa.try_fused_rms_norm(dev(q), dev(w[:d]), 1e-6))
+    assert torch.equal(ko, qa.try_fused_rms_norm(dev(k), dev(w[d:]), 1e-6))
+
+
+@pytest.mark.parametrize("b,s,hq,hk,d", [(1, 1, 32, 8, 128), (2, 7, 32, 8, 128), (1, 300, 16, 2, 64), (3, 2, 1, 1, 2)])
+def test_rope_pair_shapes(qa, oracle, b, s, hq, hk, d):
+    q, k = oracle.randn(1, (b, s, hq, d)), oracle.randn(2, (b, s, hk, d))
+    ang = oracle.randn(3, (s, d // 2)) * 3.0
+    cs = np.concatenate([np.cos(ang), np.sin(ang)], axis=1).astype(np.float32)
+    qo, ko = qa.try_fused_rope_pair_bshd(dev(q), dev(k), dev(cs))
+    wq, wk = oracle.rope_pair_bshd(q, k, cs)
+    assert close(qo, wq) and close(ko, wk)
+    # a rotation keeps the length of every head vector
+    assert torch.allclose((qo ** 2).sum(-1), (dev(q) ** 2).sum(-1), rtol=1e-5)
+
+
+@pytest.mark.parametrize("heads,kv_heads,d,kv_len,cap", [
+    (32, 8, 128, 1, 1), (32, 8, 128, 17, 64), (32, 8, 128, 300, 512), (32, 8, 128, 2048, 2048),
+    (32, 8, 128, 5000, 8192), (16, 8, 128, 777, 1000), (8, 8, 128, 100, 100), (24, 4, 128, 129, 200),
+    (14, 2, 64, 333, 400), (16, 16, 64, 64, 64), (8, 2, 256, 500, 512), (3, 3, 256, 65, 65)])
+def test_decode_gqa_attention_shapes(qa, oracle, heads, kv_heads, d, kv_len, cap):
+    _say(f"attention heads={heads} kv_heads={kv_heads} d={d} kv_len={kv_len} cap={cap}")
+    q = oracle.randn(1, (1, heads, 1, d))
+    k, v = oracle.randn(2, (1, kv_heads, cap, d)), oracle.randn(3, (1, kv_heads, cap, d))
+    k[:, :, kv_len:] = 1e4  # whatever sits past kv_len must not count
+    v[:, :, kv_len:] = -1e4
+    scale = d ** -0.5
+    got = qa.try_fused_decode_gqa_attention_with_kv_len(dev(q), dev(k), dev(v), heads, kv_heads, d, kv_len, scale)
+    want = oracle.decode_gqa_attention(q, k, v, kv_len, scale)
+    assert got.shape == (1, heads, 1, d)
+    assert close(got, want)
+    if kv_len == cap:
+        assert torch.equal(got, qa.try_fused_decode_gqa_attention(dev(q), dev(k), dev(v), heads, kv_heads, d, scale))
+
+
+def test_decode_gqa_attention_long_cache_and_peaked_scores(qa, oracle):
+    """40960 positions (the longest context of the 8B model) split over many workgroups; and scores
+    spread over +-60 so that the running-maximum rescaling does all the work."""
+    heads, kv_heads, d, kv_len = 32, 8, 128, 40960
+    q = oracle.randn(1, (1, heads, 1, d))
+    k, v = oracle.randn(2, (1, kv_heads, kv_len, d)), oracle.randn(3, (1, kv_heads, kv_len, d))
+    got = qa.try_fused_decode_gqa_attention(dev(q), dev(k), dev(v), heads, kv_heads, d, d ** -0.5)
+    assert close(got, oracle.decode_gqa_attention(q, k, v, kv_len, d ** -0.5))
+    kv_len = 3000
+    k2 = k[:, :, :kv_len].copy() * 4.0
+    got = qa.try_fused_decode_gqa_attention(dev(q), dev(k2), dev(v[:, :, :kv_len]), heads, kv_heads, d, 0.5)
+    want = oracle.decode_gqa_attention(q, k2, v[:, :, :kv_len], kv_len, 0.5)
+    assert close(got, want, 2e-5)
+
+
+def test_hooks_decline_what_the_reference_declines(qa, oracle):
+    x = dev(oracle.randn(1, (2, 8)))
+    w = dev(oracle.randn(2, (8,)))
+    assert qa.try_fused_rms_norm(x.cpu(), w.cpu(), 1e-6) is None                 # not on the GPU
+    assert qa.try_fused_rms_norm(x.half(), w.half(), 1e-6) is None               # f16: not built here
+    assert qa.try_fused_rms_norm(x.t(), w[:2], 1e-6) is None                     # not contiguous
+    assert qa.try_fused_rms_norm(x, w[:4], 1e-6) is None                         # weight shape
+    q = dev(oracle.randn(3, (1, 2, 4, 8)))
+    assert qa.try_fused_qk_rms_norm(q, q, dev(oracle.randn(4, (16,))), 1e-6) is None   # seq != 1
+    assert qa.try_fused_rope_pair_bshd(q, q, dev(oracle.randn(5, (2, 6)))) is None      # cos_sin shape
+    q1 = dev(oracle.randn(6, (1, 4, 1, 64)))
+    kv = dev(oracle.randn(7, (1, 2, 10, 64)))
+    assert qa.try_fused_decode_gqa_attention_with_kv_len(q1, kv, kv, 4, 2, 64, 11, 1.0) is None  # kv_len > capacity
+    assert qa.try_fused_decode_gqa_attention(q1, kv, kv, 4, 3, 64, 1.0) is None                   # heads % kv_heads
+    from izwi_amd import capi
+    L = capi.lib()
+    out = torch.empty_like(q1)
+    assert L.izwi_decode_gqa_attention_f32(q1.data_ptr(), kv.data_ptr(), kv.data_ptr(), 4, 2, 48, 10, 10, C.c_float(1.0),
+                                           out.data_ptr(), capi.DEVICE, None) == -2
+    assert L.izwi_decode_gqa_attention_f32(q1.data_ptr(), kv.data_ptr(), kv.data_ptr(), 4, 2, 64, 0, 10, C.c_float(1.0),
+                                           out.data_ptr(), capi.DEVICE, None) == -1
