@@ -242,6 +242,110 @@ def prefill_extra(torch, qa, oracle, dtype, m, steps=20, warmup=5, only=None):
     return out
 
 
+def neighbours_extra(torch, qa, steps=10, warmup=3):
+    """Extra report (not `value`): the decode-step neighbours at Qwen3-8B shapes (32 query heads on
+    8 kv heads, head_dim 128, hidden 4096, f32): microseconds per call in a HIP-graph replay and, for
+    attention, KV-cache bytes (K and V read once) over time."""
+    heads, kvh, d, hidden = 32, 8, 128, 4096
+    out = {}
+    q = torch.randn(1, heads, 1, d, device="cuda")
+    for kv_len in (512, 4096, 32768):
+        n_caches = max(2, min(16, (1 << 29) // (kv_len * kvh * d * 8)))  # rotate caches: none stays in L2
+        ks = [torch.randn(1, kvh, kv_len, d, device="cuda") for _ in range(n_caches)]
+        vs = [torch.randn_like(k) for k in ks]
+        reps = max(1, 32 // n_caches)
+
+        def run():
+            for _ in range(reps):
+                for k, v in zip(ks, vs):
+                    qa.try_fused_decode_gqa_attention(q, k, v, heads, kvh, d, d ** -0.5)
+        ms, g = time_graph(torch, run, steps, warmup)
+        us = ms * 1e3 / (reps * n_caches)
+        out[f"attention_kv{kv_len}"] = {"us": round(us, 2), "gbs": round(2 * kvh * kv_len * d * 4 / us / 1e3, 1)}
+        del ks, vs, g
+    x, w = torch.randn(1, hidden, device="cuda"), torch.randn(hidden, device="cuda")
+    qq, kk = torch.randn(1, 1, heads, d, device="cuda"), torch.randn(1, 1, kvh, d, device="cuda")
+    qkw, cs = torch.randn(2 * d, device="cuda"), torch.randn(1, d, device="cuda")
+    for name, fn in (("rms_norm_1x4096", lambda: qa.try_fused_rms_norm(x, w, 1e-6)),
+                     ("qk_rms_norm_40x128", lambda: qa.try_fused_qk_rms_norm(qq, kk, qkw, 1e-6)),
+                     ("rope_40x128", lambda: qa.try_fused_rope_pair_bshd(qq, kk, cs))):
+        def run():
+            for _ in range(64):
+                fn()
+        ms, g = time_graph(torch, run, steps, warmup)
+        out[name] = {"us": round(ms * 1e3 / 64, 2)}
+        del g
+    torch.cuda.empty_cache()
+    return out
+
+
+def fused_and_q6k_extra(torch, qa, oracle, steps=10, warmup=3):
+    """Extra report (not `value`): (a) the o / down projections of the 8B stack with bf16 activations in,
+    residual added, bf16 out in one call each (izwi_qmm_forward_fused) against the same projections
+    as f32 calls with torch's cast / add / cast kernels around them; (b) Q6_K projections of a
+    Q4_K_M file (ffn_down, attn_v, output) at M = 1: microseconds and Q6_K bytes over time."""
+    import numpy as np
+    out = {}
+    rng = np.random.default_rng(5)
+
+    def q6k(n, k):
+        rows = min(n, 2048)
+        b = rng.integers(0, 256, size=(rows * k // 256, 210), dtype=np.uint8)
+        b[:, 208:210] = (1e-3 * rng.uniform(0.5, 2.0, size=b.shape[0])).astype(np.float16).view(np.uint8).reshape(-1, 2)
+        b = np.tile(b.reshape(rows, -1), ((n + rows - 1) // rows, 1))[:n]
+        return qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q6K, b.reshape(-1), (n, k)))
+
+    for name, n, k, copies in (("ffn_down", 4096, 12288, 8), ("attn_v", 1024, 4096, 16), ("output", 151936, 4096, 2)):
+        ws = [q6k(n, k) for _ in range(copies)]
+        x = torch.randn(1, k, device="cuda")
+        reps = max(1, 32 // copies)
+
+        def run():
+            for _ in range(reps):
+                for w in ws:
+                    w.forward(x)
+        ms, g = time_graph(torch, run, steps, warmup)
+        us = ms * 1e3 / (reps * copies)
+        out[f"q6k_m1_{name}"] = {"us": round(us, 2), "gbs": round(n * k // 256 * 210 / us / 1e3, 1)}
+        del ws, g
+        torch.cuda.empty_cache()
+    mats = []
+    for i in range(8):
+        mats.append(tuple(qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(
+            qa.GgmlDType.Q4K, make_blocks(oracle, Q4_K, 4096, k, 1003 if k == 4096 else 1006), (4096, k))) for k in (4096, 12288)))
+    xa, xh = torch.randn(1, 4096, device="cuda").bfloat16(), torch.randn(1, 12288, device="cuda").bfloat16()
+    res = torch.randn(1, 4096, device="cuda").bfloat16()
+
+    passes = 8  # 64 layers' worth of calls per graph replay, so that the replay's own start-up does not show
+
+    def fused():
+        for _ in range(passes):
+            for o, dn in mats:
+                o.forward_fused(xa, residual=res, out=res)
+                dn.forward_fused(xh, residual=res, out=res)
+
+    def unfused():
+        r = res
+        for _ in range(passes):
+            for o, dn in mats:
+                r = r + o.forward(xa.float()).bfloat16()
+                r = r + dn.forward(xh.float()).bfloat16()
+
+    def plain_f32():  # the same projections as plain f32 calls, nothing around them
+        xa32, xh32 = xa.float(), xh.float()
+        for _ in range(passes):
+            for o, dn in mats:
+                o.forward(xa32)
+                dn.forward(xh32)
+    for name, fn in (("fused", fused), ("unfused", unfused), ("plain_f32_calls_only", plain_f32)):
+        ms, g = time_graph(torch, fn, steps, warmup)
+        out[f"o_down_bf16_residual_{name}_us_per_layer"] = round(ms * 1e3 / (passes * len(mats)), 2)
+        del g
+    del mats
+    torch.cuda.empty_cache()
+    return out
+
+
 def moe_extra(torch, qa, oracle, steps=50, warmup=5):
     """One MoE layer (route + sort + grouped expert MLP + combine, HIP-graph replay) at the
     Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, expert intermediate 768, Q4_K; as one
@@ -458,6 +562,14 @@ def main():
             extras["moe_30b_a3b_q4k"] = moe_extra(torch, qa, oracle)
         except Exception as exc:
             extras["moe_error"] = repr(exc)
+        try:
+            extras["decode_step_neighbours_f32"] = neighbours_extra(torch, qa)
+        except Exception as exc:
+            extras["neighbours_error"] = repr(exc)
+        try:
+            extras["fused_call_and_q6k"] = fused_and_q6k_extra(torch, qa, oracle)
+        except Exception as exc:
+            extras["fused_q6k_error"] = repr(exc)
         try:
             extras["prefill_tflops_m2048_q4k"] = prefill_extra(torch, qa, oracle, Q4_K, 2048)
             extras["prefill_tflops_m2048_q8_0"] = prefill_extra(torch, qa, oracle, Q8_0, 2048)

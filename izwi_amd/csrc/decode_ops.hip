@@ -13,6 +13,7 @@
 #include <hip/hip_runtime.h>
 
 #include <math.h>
+#include <stdlib.h>
 
 #include "../../include/izwi_decode_ops.h"
 #include "qmm_internal.h"
@@ -210,8 +211,24 @@ struct AttnParams {
     float scale;
 };
 
+// e^x for x <= 0 on the hardware's exp2 (relative error about 2^-22; e^-inf = 0)
+__device__ __forceinline__ float exp_neg(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+
 // weight of a partial result with running maximum m when merged under the maximum mn
-__device__ __forceinline__ float merge_weight(float m, float mn) { return m == -INFINITY ? 0.0f : expf(m - mn); }
+__device__ __forceinline__ float merge_weight(float m, float mn) { return m == -INFINITY ? 0.0f : exp_neg(m - mn); }
+
+// sum over the 8 lanes of a row group, in every lane of the group (two quad permutes and a
+// mirror of the half row: no LDS traffic)
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float sum8(float v) {
+    v += dpp_f<0xB1>(v);  // quad_perm [1,0,3,2]
+    v += dpp_f<0x4E>(v);  // quad_perm [2,3,0,1]
+    v += dpp_f<0x141>(v); // row_half_mirror
+    return v;
+}
 
 // NI = head_dim / 32; G query heads of one kv head per workgroup.  Lane j of an 8-lane row group
 // holds the elements 32 i + 4 j + c (i < NI, c < 4) of a cache row and of the query heads.
@@ -255,21 +272,23 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
             for (int i = 0; i < NI; i++)
                 dot += qr[g][4 * i] * kr[i].x + qr[g][4 * i + 1] * kr[i].y + qr[g][4 * i + 2] * kr[i].z +
                        qr[g][4 * i + 3] * kr[i].w;
-            dot += __shfl_xor(dot, 1);
-            dot += __shfl_xor(dot, 2);
-            dot += __shfl_xor(dot, 4);
-            const float s = dot * P.scale;
-            const float mn = fmaxf(m[g], s);
-            const float alpha = merge_weight(m[g], mn), pe = expf(s - mn);
-            l[g] = l[g] * alpha + pe;
+            const float s = sum8(dot) * P.scale;
+            if (s > m[g]) { // a new maximum (rare after the first positions): rescale what was summed
+                const float alpha = merge_weight(m[g], s);
+                l[g] *= alpha;
+#pragma unroll
+                for (int e = 0; e < E; e++) acc[g][e] *= alpha;
+                m[g] = s;
+            }
+            const float pe = exp_neg(s - m[g]);
+            l[g] += pe;
 #pragma unroll
             for (int i = 0; i < NI; i++) {
-                acc[g][4 * i] = acc[g][4 * i] * alpha + pe * vr[i].x;
-                acc[g][4 * i + 1] = acc[g][4 * i + 1] * alpha + pe * vr[i].y;
-                acc[g][4 * i + 2] = acc[g][4 * i + 2] * alpha + pe * vr[i].z;
-                acc[g][4 * i + 3] = acc[g][4 * i + 3] * alpha + pe * vr[i].w;
+                acc[g][4 * i] += pe * vr[i].x;
+                acc[g][4 * i + 1] += pe * vr[i].y;
+                acc[g][4 * i + 2] += pe * vr[i].z;
+                acc[g][4 * i + 3] += pe * vr[i].w;
             }
-            m[g] = mn;
         }
     }
     // merge the 8 row groups of the wave (lane bits 3..5), then the 4 waves through LDS
@@ -320,21 +339,42 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
     }
 }
 
-// out[h] = merge of the splits' partial results
-__global__ void attn_merge_kernel(const float* __restrict__ part, float* __restrict__ out, int splits, int head_dim) {
-    const int h = blockIdx.x;
+// out[h] = merge of the splits' partial results.  One workgroup per head: the splits' maxima and
+// weights are worked out once, in parallel over the splits, and kept in LDS; the weighted sums
+// then run over the splits with their loads independent of each other (unrolled), not one memory
+// round trip per split.
+constexpr int kMaxSplits = 1024;
+__global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                         int splits, int head_dim) {
+    __shared__ float weight[kMaxSplits];
+    __shared__ float red[8];
+    const int h = blockIdx.x, tid = threadIdx.x;
     const float* base = part + (int64_t)h * splits * (head_dim + 2);
-    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-        float mn = -INFINITY;
-        for (int s = 0; s < splits; s++) mn = fmaxf(mn, base[(int64_t)s * (head_dim + 2) + head_dim]);
-        float a = 0.0f, lsum = 0.0f;
-        for (int s = 0; s < splits; s++) {
-            const float* ps = base + (int64_t)s * (head_dim + 2);
-            const float w = merge_weight(ps[head_dim], mn);
-            a += ps[d] * w;
-            lsum += ps[head_dim + 1] * w;
-        }
-        out[(int64_t)h * head_dim + d] = a * (1.0f / lsum);
+    float mloc = -INFINITY;
+    for (int s = tid; s < splits; s += 256) {
+        weight[s] = base[(int64_t)s * (head_dim + 2) + head_dim];
+        mloc = fmaxf(mloc, weight[s]);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mloc = fmaxf(mloc, __shfl_xor(mloc, o));
+    if ((tid & 63) == 0) red[tid >> 6] = mloc;
+    __syncthreads();
+    const float mn = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float lloc = 0.0f;
+    for (int s = tid; s < splits; s += 256) {
+        const float w = merge_weight(weight[s], mn);
+        weight[s] = w;
+        lloc += base[(int64_t)s * (head_dim + 2) + head_dim + 1] * w;
+    }
+    lloc = wave_sum(lloc);
+    if ((tid & 63) == 0) red[4 + (tid >> 6)] = lloc;
+    __syncthreads();
+    const float inv = 1.0f / (red[4] + red[5] + red[6] + red[7]);
+    for (int d = tid; d < head_dim; d += 256) {
+        float a = 0.0f;
+#pragma unroll 8
+        for (int s = 0; s < splits; s++) a += base[(int64_t)s * (head_dim + 2) + d] * weight[s];
+        out[(int64_t)h * head_dim + d] = a * inv;
     }
 }
 
@@ -471,12 +511,16 @@ int izwi_decode_gqa_attention_f32(const float* q, const float* k, const float* v
     // query heads per workgroup: as many of the group as the register file takes
     int g = group % 4 == 0 && head_dim <= 128 ? 4 : (group % 2 == 0 ? 2 : 1);
     const int z = group / g;
-    // enough workgroups for two per CU, at least 64 positions each (two per row group)
+    // Enough workgroups for one per CU (IZWI_ATTN_WGS_PER_CU, tuning knob), at least 64 positions
+    // each (IZWI_ATTN_MIN_CHUNK): more splits only add merge work (measured: 2 per CU is 5-10 %
+    // slower between 4k and 16k positions, 4 per CU 30 %).
+    static const int wgs_per_cu = [] { const char* e = getenv("IZWI_ATTN_WGS_PER_CU"); int v = e ? atoi(e) : 1; return v > 0 ? v : 1; }();
+    static const int min_chunk = [] { const char* e = getenv("IZWI_ATTN_MIN_CHUNK"); int v = e ? atoi(e) : 64; return v > 0 ? v : 64; }();
     const int64_t base_wgs = num_kv_heads * z;
-    int64_t splits = (2 * (int64_t)n_cus + base_wgs - 1) / base_wgs;
-    const int64_t max_splits = (kv_len + 63) / 64;
+    int64_t splits = (wgs_per_cu * (int64_t)n_cus + base_wgs - 1) / base_wgs;
+    const int64_t max_splits = (kv_len + min_chunk - 1) / min_chunk;
     if (splits > max_splits) splits = max_splits;
-    if (splits > 1024) splits = 1024;
+    if (splits > kMaxSplits) splits = kMaxSplits;
     if (splits < 1) splits = 1;
     const int chunk = (int)((kv_len + splits - 1) / splits);
     splits = (kv_len + chunk - 1) / chunk; // every split holds at least one position
@@ -505,8 +549,7 @@ int izwi_decode_gqa_attention_f32(const float* q, const float* k, const float* v
                                      : launch_attn_partial<8>(P, g, grid, stream);
     OPS_TRY(e);
     if (splits > 1) {
-        attn_merge_kernel<<<(unsigned)num_heads, head_dim >= 128 ? 128 : 64, 0, stream>>>(P.part, P.out, (int)splits,
-                                                                                          (int)head_dim);
+        attn_merge_kernel<<<(unsigned)num_heads, 256, 0, stream>>>(P.part, P.out, (int)splits, (int)head_dim);
         OPS_TRY(hipGetLastError());
     }
     OPS_TRY(oo.finish(stream));

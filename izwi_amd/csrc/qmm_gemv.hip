@@ -478,6 +478,12 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
             float acc[MT];
 #pragma unroll
             for (int mi = 0; mi < MT; mi++) acc[mi] = 0.0f;
+            // Epilogue with a residual, k split over waves: the lane that will store requests its
+            // residual value behind the first panel's loads, so that the value is there when the
+            // sums are (at the end it would be one more memory round trip on the kernel's critical
+            // path).  Like the other loads it is unconditional and branch-free: the aligned dword
+            // that holds the value (f32, or a bf16 pair), or the start of x for lanes without one.
+            uint32_t res_raw = 0;
             for (int ks = 0; ONESHOT ? ks < 1 : ks < P.kpw; ks++) {
                 const int kg = ks * P.nwk + wk;
                 const bool ok = rt < row_tiles && kg < P.k_groups;
@@ -493,7 +499,18 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                     float4 f[4];
                     float v[16];
                     const bool in0 = x_item_issue<MT, XB>(xs, group, group < items, f);
+                    if (IO != 0) __builtin_amdgcn_sched_barrier(0); // the activation loads stay in front
                     load_panel<QT>(p, wbase + off, P.slots, lane0, active);
+                    if (EP && ks == 0) {
+                        // (the lanes and conditions of the store at the end)
+                        const int mi = lane0 >> 4, row = rt * 16 + (lane0 & 15);
+                        const bool have = P.ep.residual != nullptr && P.nwk != 1 && wk == 0 && lane0 < 16 * MT &&
+                                          rt < row_tiles && row < n_rows && m0 + mi < m_end;
+                        const int64_t byte = ((int64_t)(m0 + mi) * n_rows + row) * (P.ep.y_bf16 ? 2 : 4);
+                        const uint8_t* rp = have ? static_cast<const uint8_t*>(P.ep.residual) + (byte & ~(int64_t)3)
+                                                 : reinterpret_cast<const uint8_t*>(P.x);
+                        res_raw = *reinterpret_cast<const uint32_t*>(rp);
+                    }
                     if (m0 != m_begin) lds_barrier(); // the previous rows' readers are done
                     x16_finish<XB>(f, in0, v);
                     if (group < items) x_item_quantize<QT, MT>(l, k_units, group, v);
@@ -554,8 +571,15 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                     const int row = rt * 16 + r;
                     if (rt < row_tiles && row < n_rows && m0 + mi < m_end) {
                         int64_t yr = GROUPED ? P.perm[m0 + mi] : m0 + mi;
-                        if (EP) qmm_store(y_out, P.ep, yr * n_rows + row, sum);
-                        else y_out[yr * n_rows + row] = GATED ? silu(sum) * sum2 : sum;
+                        if (EP) {
+                            const int64_t idx = yr * n_rows + row;
+                            const float res = P.ep.residual == nullptr ? 0.0f
+                                              : P.ep.y_bf16 ? qmm_bf16_bits_to_f32((uint16_t)(res_raw >> (16 * (int)(idx & 1))))
+                                                            : __uint_as_float(res_raw);
+                            qmm_store(y_out, QmmEpilogue{nullptr, P.ep.y_bf16}, idx, sum + res);
+                        } else {
+                            y_out[yr * n_rows + row] = GATED ? silu(sum) * sum2 : sum;
+                        }
                     }
                 }
                 red_buf ^= 1;
