@@ -424,6 +424,8 @@ def main():
                     help="grouped: qkv_proj.forward(x) and gate_up_proj.forward(x) are one call each, as "
                          "the reference's attention and MLP blocks make them (4 calls per layer); "
                          "per-projection: seven izwi_qmm_forward_f32 calls per layer")
+    ap.add_argument("--neighbours-only", action="store_true",
+                    help="time only the decode-step neighbours (norms, rotary, attention) and print them: for profiling")
     ap.add_argument("--prefill-only", default=None, choices=["q", "k", "gate", "down"],
                     help="profiling aid: run only the prefill call of one 8B projection (--m rows, default "
                          "2048 here; --steps calls) and print its TFLOP/s, nothing else")
@@ -441,6 +443,10 @@ def main():
     torch.cuda.set_device(0)
     qa.lib()
     dtype = Q4_K if args.workload == "decode_q4k_8b_stack" else Q8_0
+
+    if args.neighbours_only:
+        print(json.dumps({"decode_step_neighbours_f32": neighbours_extra(torch, qa, args.steps, args.warmup)}))
+        return
 
     if args.prefill_only:
         m = args.m if args.m > 1 else 2048

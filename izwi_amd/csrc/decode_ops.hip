@@ -235,7 +235,7 @@ __device__ __forceinline__ float sum8(float v) {
 template <int NI, int G>
 __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
     constexpr int HD = 32 * NI, E = 4 * NI;
-    __shared__ float red[4][G][HD + 2];
+    __shared__ __attribute__((aligned(16))) float red[16][G][HD + 4]; // [.. HD): sums, [HD]: maximum, [HD + 1]: weight sum
     const int kvh = blockIdx.x, sp = blockIdx.y, h0 = kvh * P.group + blockIdx.z * G;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane & 7, slot = wave * 8 + (lane >> 3);
@@ -291,28 +291,29 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
             }
         }
     }
-    // merge the 8 row groups of the wave (lane bits 3..5), then the 4 waves through LDS
+    // Merge the 32 row groups of the workgroup: neighbours 8 lanes apart inside a 16-lane row by a
+    // row rotation (no LDS), the remaining 16 partial results through LDS, where every output
+    // element then sums its 16 terms.  (Shuffling all partial sums across the wave three times was
+    // an LDS-latency chain of ~200 dependent permutes: 6 us of a 9 us kernel.)
 #pragma unroll
-    for (int o = 8; o < 64; o <<= 1) {
+    for (int g = 0; g < G; g++) {
+        const float mo = dpp_f<0x128>(m[g]), lo = dpp_f<0x128>(l[g]); // row_ror:8 = lane ^ 8
+        const float mn = fmaxf(m[g], mo);
+        const float wa = merge_weight(m[g], mn), wb = merge_weight(mo, mn);
+        l[g] = l[g] * wa + lo * wb;
 #pragma unroll
-        for (int g = 0; g < G; g++) {
-            const float mo = __shfl_xor(m[g], o), lo = __shfl_xor(l[g], o);
-            const float mn = fmaxf(m[g], mo);
-            const float wa = merge_weight(m[g], mn), wb = merge_weight(mo, mn);
-            l[g] = l[g] * wa + lo * wb;
-#pragma unroll
-            for (int e = 0; e < E; e++) acc[g][e] = acc[g][e] * wa + __shfl_xor(acc[g][e], o) * wb;
-            m[g] = mn;
-        }
+        for (int e = 0; e < E; e++) acc[g][e] = acc[g][e] * wa + dpp_f<0x128>(acc[g][e]) * wb;
+        m[g] = mn;
     }
-    if (lane < 8) {
+    if ((lane & 8) == 0) {
+        const int entry = wave * 4 + (lane >> 4);
 #pragma unroll
         for (int g = 0; g < G; g++) {
 #pragma unroll
             for (int i = 0; i < NI; i++)
-#pragma unroll
-                for (int c = 0; c < 4; c++) red[wave][g][32 * i + 4 * j + c] = acc[g][4 * i + c];
-            if (j == 0) red[wave][g][HD] = m[g], red[wave][g][HD + 1] = l[g];
+                *reinterpret_cast<float4*>(&red[entry][g][32 * i + 4 * j]) =
+                    make_float4(acc[g][4 * i], acc[g][4 * i + 1], acc[g][4 * i + 2], acc[g][4 * i + 3]);
+            if (j == 0) red[entry][g][HD] = m[g], red[entry][g][HD + 1] = l[g];
         }
     }
     __syncthreads();
@@ -320,10 +321,10 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
         const int g = t / HD, d = t - g * HD;
         float mn = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < 4; w++) mn = fmaxf(mn, red[w][g][HD]);
+        for (int w = 0; w < 16; w++) mn = fmaxf(mn, red[w][g][HD]);
         float a = 0.0f, lsum = 0.0f;
 #pragma unroll
-        for (int w = 0; w < 4; w++) {
+        for (int w = 0; w < 16; w++) {
             const float ww = merge_weight(red[w][g][HD], mn);
             a += red[w][g][d] * ww;
             lsum += red[w][g][HD + 1] * ww;
