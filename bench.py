@@ -346,6 +346,43 @@ def fused_and_q6k_extra(torch, qa, oracle, steps=10, warmup=3):
     return out
 
 
+def layer_stack_extra(torch, qa, oracle, dtype, steps=10, warmup=3):
+    """Extra report (not `value`): one whole decode step of the Qwen3-8B stack composed from the library's
+    calls (izwi_amd.qwen3_layer.Qwen3DecodeLayer: norms, q|k|v group, q/k norm, rotary, cache append,
+    attention, o and down with the residual folded in, gate/up with the activation) plus the final norm
+    and the LM head, f32 activations, HIP-graph replay, at several context lengths."""
+    from izwi_amd.qwen3_layer import Qwen3DecodeLayer
+    heads, kvh, d, hidden = 32, 8, 128, 4096
+    weights = build_decode_weights(torch, qa, oracle, dtype, N_LAYERS_8B, True)
+    per = len(LAYER_8B)
+    ones = lambda n: torch.ones(n, device="cuda")  # noqa: E731
+    layers = []
+    for i in range(N_LAYERS_8B):
+        q, k, v, o, gate, up, down = [w[0] for w in weights[i * per:(i + 1) * per]]
+        layers.append(Qwen3DecodeLayer(ones(hidden), ones(hidden), q, k, v, ones(2 * d), o, gate, up, down, heads, kvh, d))
+    lm_head, final_norm = weights[-1][0], ones(hidden)
+    x0 = torch.randn(1, hidden, device="cuda")
+    cos_sin = torch.randn(1, d, device="cuda")
+    out = {}
+    for kv_len in (256, 4096):
+        caches = [(torch.randn(1, kvh, kv_len, d, device="cuda") * 0.1, torch.randn(1, kvh, kv_len, d, device="cuda") * 0.1)
+                  for _ in range(N_LAYERS_8B)]
+
+        def step():
+            x = x0
+            for layer, (kc, vc) in zip(layers, caches):
+                x = layer.forward(x, cos_sin, kc, vc, kv_len - 1)
+            return lm_head.forward(qa.try_fused_rms_norm(x, final_norm, 1e-6))
+        ms, g = time_graph(torch, step, steps, warmup)
+        out[f"kv{kv_len}"] = {"ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1)}
+        del caches, g
+        torch.cuda.empty_cache()
+    out["launches_per_token"] = N_LAYERS_8B * 9 + 2
+    del layers, weights
+    torch.cuda.empty_cache()
+    return out
+
+
 def moe_extra(torch, qa, oracle, steps=50, warmup=5):
     """One MoE layer (route + sort + grouped expert MLP + combine, HIP-graph replay) at the
     Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, expert intermediate 768, Q4_K; as one
@@ -572,6 +609,10 @@ def main():
             extras["decode_step_neighbours_f32"] = neighbours_extra(torch, qa)
         except Exception as exc:
             extras["neighbours_error"] = repr(exc)
+        try:
+            extras["qwen3_8b_decode_step_all_calls"] = layer_stack_extra(torch, qa, oracle, dtype)
+        except Exception as exc:
+            extras["layer_stack_error"] = repr(exc)
         try:
             extras["fused_call_and_q6k"] = fused_and_q6k_extra(torch, qa, oracle)
         except Exception as exc:

@@ -51,6 +51,21 @@ int izwi_rope_pair_bshd_f32(const float* q, const float* k, const float* cos_sin
                             int64_t seq, int64_t q_heads, int64_t k_heads, int64_t head_dim,
                             float* q_out, float* k_out, int mem_space, void* stream);
 
+/* The single-token sequence of `Qwen3Attention::forward` between the q/k/v projections and the
+ * attention itself as ONE launch: `apply_qk_norm_pair` (qwen3/core.rs:1464-1478), `apply_rope_pair`
+ * (core.rs:1480-1575) and the append of the new key / value rows to the cache.  q is `[num_heads,
+ * head_dim]`, k and v are `[num_kv_heads, head_dim]` (the projections' outputs), qk_weight is
+ * `[2 * head_dim]` (q's norm weights, then k's), cos_sin is `[head_dim]` for this position
+ * (cos | sin).  Writes the normed, rotated q to q_out (may be q), the normed, rotated k and the
+ * unchanged v to position `pos` of the head-major caches `[num_kv_heads, kv_capacity, head_dim]`.
+ * Values are those of izwi_qk_rms_norm_f32 followed by izwi_rope_pair_bshd_f32 up to the order
+ * of the norm's sum.  Device pointers only (the caches live on the device).  It has no single counterpart among the
+ * reference's hooks: it is their composition for one token. */
+int izwi_qk_norm_rope_append_f32(const float* q, const float* k, const float* v, const float* qk_weight,
+                                 const float* cos_sin, int64_t num_heads, int64_t num_kv_heads,
+                                 int64_t head_dim, float eps, float* q_out, float* k_cache, float* v_cache,
+                                 int64_t kv_capacity, int64_t pos, void* stream);
+
 /* `try_fused_decode_gqa_attention_with_kv_len(q, k, v, num_heads, num_kv_heads, head_dim, kv_len,
  * scale)` (kernels/mod.rs:199-225, metal.rs:2121-2193, shader metal.rs:307-381): attention of one
  * query token.  q is `[1, num_heads, 1, head_dim]`, k and v are `[1, num_kv_heads, kv_capacity,

@@ -198,6 +198,69 @@ __global__ void rope_pair_kernel(const float* __restrict__ cos_sin, const float*
     y[half + d] = x1 * s + x2 * c;
 }
 
+// ---- q/k norm + rotary + cache append, one token ---------------------------------------------
+// One wave per head: rows 0 .. heads-1 are q, then kv_heads rows of k, then kv_heads rows of v.
+// Lane l holds the pairs (p, p + half) for p = l, l + 64, ..: the norm's sum runs over the wave,
+// the rotation stays inside the lane.  q goes to q_out, k and v to position `pos` of the caches.
+struct QkvPrepParams {
+    const float* q;
+    const float* k;
+    const float* v;
+    const float* qk_weight; // [2 * head_dim]
+    const float* cos_sin;   // [head_dim]: cos | sin of this position
+    float* q_out;
+    float* k_cache;
+    float* v_cache; // [kv_heads, capacity, head_dim]
+    int heads, kv_heads, head_dim;
+    int64_t capacity, pos;
+    float eps;
+};
+
+__global__ __launch_bounds__(256) void qkv_prep_kernel(QkvPrepParams P) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int total = P.heads + 2 * P.kv_heads;
+    if (row >= total) return;
+    const int hd = P.head_dim, half = hd >> 1;
+    if (row >= P.heads + P.kv_heads) { // v: a plain copy into the cache
+        const int h = row - P.heads - P.kv_heads;
+        const float* src = P.v + (int64_t)h * hd;
+        float* dst = P.v_cache + ((int64_t)h * P.capacity + P.pos) * hd;
+        for (int i = lane; i < hd; i += 64) dst[i] = src[i];
+        return;
+    }
+    const bool is_q = row < P.heads;
+    const int h = is_q ? row : row - P.heads;
+    const float* src = (is_q ? P.q : P.k) + (int64_t)h * hd;
+    const float* w = P.qk_weight + (is_q ? 0 : hd);
+    float* dst = is_q ? P.q_out + (int64_t)h * hd : P.k_cache + ((int64_t)h * P.capacity + P.pos) * hd;
+    constexpr int MAXP = 2; // pairs kept per lane: head_dim <= 256; longer heads are re-read
+    float x1[MAXP], x2[MAXP];
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MAXP; i++) {
+        const int p = lane + 64 * i;
+        x1[i] = p < half ? src[p] : 0.0f;
+        x2[i] = p < half ? src[half + p] : 0.0f;
+        sum += x1[i] * x1[i] + x2[i] * x2[i];
+    }
+    for (int p = lane + 64 * MAXP; p < half; p += 64) sum += src[p] * src[p] + src[half + p] * src[half + p];
+    sum = wave_sum(sum);
+    const float scale = 1.0f / sqrtf(sum / (float)hd + P.eps);
+    auto rotate = [&](int p, float a, float b) {
+        // the norm as the norm kernel writes it (x * scale * weight), then the rotation of the pair
+        const float n1 = a * scale * w[p], n2 = b * scale * w[half + p];
+        const float c = P.cos_sin[p], s = P.cos_sin[half + p];
+        dst[p] = n1 * c - n2 * s;
+        dst[half + p] = n1 * s + n2 * c;
+    };
+#pragma unroll
+    for (int i = 0; i < MAXP; i++) {
+        const int p = lane + 64 * i;
+        if (p < half) rotate(p, x1[i], x2[i]);
+    }
+    for (int p = lane + 64 * MAXP; p < half; p += 64) rotate(p, src[p], src[half + p]);
+}
+
 // ---- single-token GQA attention ------------------------------------------------------------
 struct AttnParams {
     const float* q;
@@ -481,6 +544,28 @@ int izwi_rope_pair_bshd_f32(const float* q, const float* k, const float* cos_sin
     OPS_TRY(hipGetLastError());
     OPS_TRY(qo.finish(stream));
     OPS_TRY(ko.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qk_norm_rope_append_f32(const float* q, const float* k, const float* v, const float* qk_weight,
+                                 const float* cos_sin, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                                 float eps, float* q_out, float* k_cache, float* v_cache, int64_t kv_capacity,
+                                 int64_t pos, void* stream_) {
+    if (num_heads <= 0 || num_kv_heads <= 0 || num_heads + 2 * num_kv_heads > 0x3fffffff || head_dim <= 0 ||
+        head_dim % 2 || head_dim > 8192 || pos < 0 || pos >= kv_capacity)
+        return qmm_fail(IZWI_QMM_ERR_INVALID,
+                        "qk_norm_rope_append: bad shape (heads %lld, kv heads %lld, head_dim %lld, position %lld of %lld)",
+                        (long long)num_heads, (long long)num_kv_heads, (long long)head_dim, (long long)pos,
+                        (long long)kv_capacity);
+    if (!q || !k || !v || !qk_weight || !cos_sin || !q_out || !k_cache || !v_cache)
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "qk_norm_rope_append: NULL buffer");
+    int device = 0, n_cus = 0;
+    if (int rc = qmm_current_device(&device, &n_cus)) return rc;
+    QkvPrepParams P{q, k, v, qk_weight, cos_sin, q_out, k_cache, v_cache, (int)num_heads, (int)num_kv_heads,
+                    (int)head_dim, kv_capacity, pos, eps};
+    const int64_t rows = num_heads + 2 * num_kv_heads;
+    qkv_prep_kernel<<<(unsigned)((rows + 3) / 4), 256, 0, (hipStream_t)stream_>>>(P);
+    OPS_TRY(hipGetLastError());
     return IZWI_QMM_OK;
 }
 

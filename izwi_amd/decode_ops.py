@@ -82,3 +82,24 @@ def try_fused_decode_gqa_attention(q, k, v, num_heads: int, num_kv_heads: int, h
     if k.dim() != 4:
         return None
     return try_fused_decode_gqa_attention_with_kv_len(q, k, v, num_heads, num_kv_heads, head_dim, k.shape[2], scale)
+
+
+def qk_norm_rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qk_weight: torch.Tensor,
+                        cos_sin: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pos: int, eps: float):
+    """apply_qk_norm_pair + apply_rope_pair + cache append of Qwen3Attention::forward for one token
+    (qwen3/core.rs:1464-1575) in one launch.  q [heads * d], k / v [kv_heads * d] (any shape with that many
+    elements), caches [1, kv_heads, capacity, d].  Returns the normed, rotated q as [1, heads, 1, d]; the caches
+    gain position `pos`."""
+    from .capi import QmmError
+    if not _ok(q, k, v, qk_weight, cos_sin, k_cache, v_cache) or k_cache.dim() != 4 or tuple(v_cache.shape) != tuple(k_cache.shape):
+        raise QmmError(-1, "qk_norm_rope_append: contiguous f32 CUDA tensors on one device expected")
+    _, kv_heads, cap, d = k_cache.shape
+    heads = q.numel() // d
+    if (q.numel() != heads * d or k.numel() != kv_heads * d or v.numel() != kv_heads * d or qk_weight.numel() != 2 * d
+            or cos_sin.numel() != d):
+        raise QmmError(-1, "qk_norm_rope_append: shapes do not match the caches")
+    q_out = torch.empty((1, heads, 1, d), dtype=torch.float32, device=q.device)
+    check(lib().izwi_qk_norm_rope_append_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), qk_weight.data_ptr(),
+                                             cos_sin.data_ptr(), heads, kv_heads, d, eps, q_out.data_ptr(),
+                                             k_cache.data_ptr(), v_cache.data_ptr(), cap, pos, _stream_ptr(q)))
+    return q_out

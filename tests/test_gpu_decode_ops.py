@@ -186,3 +186,33 @@ def test_hooks_decline_what_the_reference_declines(qa, oracle):
                                            out.data_ptr(), capi.DEVICE, None) == -2
     assert L.izwi_decode_gqa_attention_f32(q1.data_ptr(), kv.data_ptr(), kv.data_ptr(), 4, 2, 64, 0, 10, C.c_float(1.0),
                                            out.data_ptr(), capi.DEVICE, None) == -1
+
+
+@pytest.mark.parametrize("heads,kv_heads,d", [(32, 8, 128), (16, 8, 64), (4, 2, 256), (3, 1, 20), (2, 2, 512)])
+def test_qk_norm_rope_append_equals_the_separate_hooks(qa, oracle, heads, kv_heads, d):
+    """The one-launch form of q/k norm + rotary + cache append against the oracle's composition and the
+    library's own separate calls; positions other than `pos` of the caches stay untouched."""
+    cap, pos = 9, 5
+    q, k, v = oracle.randn(1, (heads * d,)), oracle.randn(2, (kv_heads * d,)), oracle.randn(3, (kv_heads * d,))
+    w = oracle.randn(4, (2 * d,), mean=1.0, std=0.2)
+    ang = oracle.randn(5, (d // 2,)) * 3.0
+    cs = np.concatenate([np.cos(ang), np.sin(ang)]).astype(np.float32).reshape(1, d)
+    kc0, vc0 = oracle.randn(6, (1, kv_heads, cap, d)), oracle.randn(7, (1, kv_heads, cap, d))
+    kc, vc = dev(kc0), dev(vc0)
+    q_rot = qa.qk_norm_rope_append(dev(q), dev(k), dev(v), dev(w), dev(cs), kc, vc, pos, 1e-6)
+    qn, kn = oracle.qk_rms_norm(q.reshape(1, 1, heads, d), k.reshape(1, 1, kv_heads, d), w, 1e-6)
+    qr, kr = oracle.rope_pair_bshd(qn, kn, cs)
+    assert q_rot.shape == (1, heads, 1, d) and close(q_rot.view(1, 1, heads, d), qr)
+    want_k, want_v = kc0.copy(), vc0.copy()
+    want_k[0, :, pos], want_v[0, :, pos] = kr.reshape(kv_heads, d), v.reshape(kv_heads, d)
+    assert close(kc, want_k) and torch.equal(vc, dev(want_v))
+    assert torch.equal(kc[0, :, :pos], dev(kc0)[0, :, :pos]) and torch.equal(kc[0, :, pos + 1:], dev(kc0)[0, :, pos + 1:])
+    if True:
+        q2, k2 = qa.try_fused_qk_rms_norm(dev(q).view(1, 1, heads, d), dev(k).view(1, 1, kv_heads, d), dev(w), 1e-6)
+        q2, k2 = qa.try_fused_rope_pair_bshd(q2, k2, dev(cs))
+        assert torch.allclose(q_rot.view(1, 1, heads, d), q2, rtol=2e-6, atol=1e-6)
+        assert torch.allclose(kc[0, :, pos], k2.view(kv_heads, d), rtol=2e-6, atol=1e-6)
+    from izwi_amd import capi
+    L = capi.lib()
+    assert L.izwi_qk_norm_rope_append_f32(kc.data_ptr(), kc.data_ptr(), kc.data_ptr(), kc.data_ptr(), kc.data_ptr(), heads,
+                                          kv_heads, d, 1e-6, kc.data_ptr(), kc.data_ptr(), vc.data_ptr(), cap, cap, None) == -1
