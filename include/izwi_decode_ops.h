@@ -80,6 +80,13 @@ int izwi_decode_gqa_attention_f32(const float* q, const float* k, const float* v
                                   int64_t kv_capacity, float scale, float* out, int mem_space,
                                   void* stream);
 
+/* Greedy next token: `argmax(&logits)` after the LM head (qwen3/chat.rs:574-597,
+ * qwen3/asr/mod.rs:2762-2789, i.e. `logits.argmax(D::Minus1)` as u32), on the device, so that four
+ * bytes per row come back instead of the logits.  logits is `[rows, n]`, out `[rows]`: the first
+ * index of the row's maximum (ties go to the smaller index, as a left-to-right scan keeps the
+ * first; a NaN is never the maximum; a row of NaNs gives 0). */
+int izwi_argmax_f32(const float* logits, int64_t rows, int64_t n, uint32_t* out, int mem_space, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

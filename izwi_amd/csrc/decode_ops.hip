@@ -198,6 +198,34 @@ __global__ void rope_pair_kernel(const float* __restrict__ cos_sin, const float*
     y[half + d] = x1 * s + x2 * c;
 }
 
+// ---- greedy sampling: first index of the row maximum ------------------------------------------
+// One workgroup per row; a thread keeps (value, index) of its strided share, ties to the smaller
+// index, NaN never wins; wave reduction by shuffles, then the waves' results through LDS.
+__device__ __forceinline__ void argmax_merge(float& v, unsigned& i, float ov, unsigned oi) {
+    if (ov > v || (ov == v && oi < i)) v = ov, i = oi;
+}
+__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ x, int64_t n, uint32_t* __restrict__ out) {
+    __shared__ float vals[16];
+    __shared__ unsigned idxs[16];
+    const float* row = x + (int64_t)blockIdx.x * n;
+    float v = -INFINITY;
+    unsigned idx = 0xffffffffu;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const float t = row[i];
+        if (t > v || idx == 0xffffffffu) { // strided visit in rising order: a later equal value never replaces
+            if (t > v || (idx == 0xffffffffu && !(t != t))) v = t, idx = (unsigned)i;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) argmax_merge(v, idx, __shfl_xor(v, o), (unsigned)__shfl_xor((int)idx, o));
+    if ((threadIdx.x & 63) == 0) vals[threadIdx.x >> 6] = v, idxs[threadIdx.x >> 6] = idx;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x >> 6); w++) argmax_merge(v, idx, vals[w], idxs[w]);
+        out[blockIdx.x] = idx == 0xffffffffu ? 0u : idx; // a row of NaNs: index 0
+    }
+}
+
 // ---- q/k norm + rotary + cache append, one token ---------------------------------------------
 // One wave per head: rows 0 .. heads-1 are q, then kv_heads rows of k, then kv_heads rows of v.
 // Lane l holds the pairs (p, p + half) for p = l, l + 64, ..: the norm's sum runs over the wave,
@@ -544,6 +572,26 @@ int izwi_rope_pair_bshd_f32(const float* q, const float* k, const float* cos_sin
     OPS_TRY(hipGetLastError());
     OPS_TRY(qo.finish(stream));
     OPS_TRY(ko.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_argmax_f32(const float* logits, int64_t rows, int64_t n, uint32_t* out, int mem_space, void* stream_) {
+    if (int rc = check_space(mem_space)) return rc;
+    if (rows < 0 || n <= 0 || n > 0xfffffffeLL || rows > 0x7fffffff)
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "argmax: bad shape [%lld, %lld]", (long long)rows, (long long)n);
+    if (rows == 0) return IZWI_QMM_OK;
+    if (!logits || !out) return qmm_fail(IZWI_QMM_ERR_INVALID, "argmax: NULL buffer");
+    int device = 0, n_cus = 0;
+    if (int rc = qmm_current_device(&device, &n_cus)) return rc;
+    hipStream_t stream = (hipStream_t)stream_;
+    Buf li, oo;
+    OPS_TRY(li.in(logits, (size_t)rows * n * sizeof(float), mem_space));
+    OPS_TRY(oo.out(out, (size_t)rows * sizeof(uint32_t), mem_space));
+    int threads = 64;
+    while (threads < 1024 && threads * 4 < n) threads *= 2;
+    argmax_kernel<<<(unsigned)rows, threads, 0, stream>>>((const float*)li.dev, n, (uint32_t*)oo.dev);
+    OPS_TRY(hipGetLastError());
+    OPS_TRY(oo.finish(stream));
     return IZWI_QMM_OK;
 }
 

@@ -103,3 +103,15 @@ def qk_norm_rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qk_we
                                              cos_sin.data_ptr(), heads, kv_heads, d, eps, q_out.data_ptr(),
                                              k_cache.data_ptr(), v_cache.data_ptr(), cap, pos, _stream_ptr(q)))
     return q_out
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """`logits.argmax(D::Minus1)` of the greedy samplers (qwen3/chat.rs:574-597): logits [..., n] f32 on the
+    GPU -> int32 indices [...] (first index of the maximum), computed on the device."""
+    from .capi import QmmError
+    if not _ok(logits) or logits.dim() < 1 or logits.shape[-1] == 0:
+        raise QmmError(-1, "argmax: a contiguous f32 CUDA tensor with a non-empty last dimension expected")
+    n = logits.shape[-1]
+    out = torch.empty(logits.shape[:-1], dtype=torch.int32, device=logits.device)
+    check(lib().izwi_argmax_f32(logits.data_ptr(), logits.numel() // n, n, out.data_ptr(), DEVICE, _stream_ptr(logits)))
+    return out

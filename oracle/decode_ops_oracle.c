@@ -105,3 +105,20 @@ int oracle_decode_gqa_attention(const float* q, const float* k, const float* v, 
     free(scores);
     return 0;
 }
+
+/* `logits.argmax(D::Minus1)` of the reference's greedy samplers (qwen3/chat.rs:592,
+ * qwen3/asr/mod.rs:2780; the reduction itself is candle-core's, not shipped): a left-to-right scan
+ * that replaces the running maximum only by a strictly larger value, i.e. the first index of the
+ * maximum.  Pinned by numpy.argmax (same definition); "parity unpinned" against the crate's own
+ * tie and NaN behaviour, which no test of the reference exercises. */
+void oracle_argmax(const float* x, int64_t rows, int64_t n, uint32_t* out) {
+    for (int64_t r = 0; r < rows; r++) {
+        const float* row = x + r * n;
+        int64_t best = -1;
+        for (int64_t i = 0; i < n; i++) {
+            if (row[i] != row[i]) continue;
+            if (best < 0 || row[i] > row[best]) best = i;
+        }
+        out[r] = best < 0 ? 0u : (uint32_t)best;
+    }
+}

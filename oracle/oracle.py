@@ -72,6 +72,8 @@ def lib() -> C.CDLL:
         L.oracle_qk_rms_norm.argtypes = [vp, vp, vp, i64, i64, i64, f32, vp, vp]
         L.oracle_rope_pair_bshd.restype = None
         L.oracle_rope_pair_bshd.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, vp, vp]
+        L.oracle_argmax.restype = None
+        L.oracle_argmax.argtypes = [vp, i64, i64, vp]
         L.oracle_decode_gqa_attention.restype = C.c_int
         L.oracle_decode_gqa_attention.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, f32, vp]
         L.oracle_get_scale_min_k4.restype = None
@@ -231,3 +233,12 @@ def decode_gqa_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, kv_len: in
     if rc:
         raise ValueError("oracle_decode_gqa_attention rejected the shape")
     return out
+
+
+def argmax(x: np.ndarray) -> np.ndarray:
+    """First index of each row's maximum, uint32 [rows]."""
+    x = _f32(x)
+    n = x.shape[-1]
+    out = np.empty(x.size // n, dtype=np.uint32)
+    lib().oracle_argmax(_ptr(x), x.size // n, n, _ptr(out))
+    return out.reshape(x.shape[:-1])

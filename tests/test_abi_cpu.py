@@ -14,7 +14,7 @@ def header_symbols():
     for header in ("izwi_qmm.h", "izwi_gguf.h", "izwi_decode_ops.h"):
         text = open(os.path.join(ROOT, "include", header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-        names |= set(re.findall(r"\b(izwi_(?:qmm|moe|gguf|rms|qk|rope|decode)_[a-z0-9_]+)\s*\(", text))
+        names |= set(re.findall(r"\b(izwi_(?:qmm|moe|gguf|rms|qk|rope|decode|argmax)_[a-z0-9_]+)\s*\(", text))
     return sorted(names)
 
 

@@ -216,3 +216,21 @@ def test_qk_norm_rope_append_equals_the_separate_hooks(qa, oracle, heads, kv_hea
     L = capi.lib()
     assert L.izwi_qk_norm_rope_append_f32(kc.data_ptr(), kc.data_ptr(), kc.data_ptr(), kc.data_ptr(), kc.data_ptr(), heads,
                                           kv_heads, d, 1e-6, kc.data_ptr(), kc.data_ptr(), vc.data_ptr(), cap, cap, None) == -1
+
+
+@pytest.mark.parametrize("rows,n", [(1, 151936), (4, 151936), (3, 1000), (2, 7), (1, 1), (5, 4097)])
+def test_argmax_on_device(qa, oracle, rows, n):
+    x = oracle.randn(rows + n, (rows, n))
+    if n > 20:
+        x[0, 17] = x[0, n - 3] = 9.0     # tie: first index
+        x[-1, :] = -np.inf
+        x[-1, 5] = np.nan
+    got = qa.argmax(dev(x))
+    assert got.dtype == torch.int32 and tuple(got.shape) == (rows,)
+    assert np.array_equal(got.cpu().numpy().astype(np.uint32), oracle.argmax(x))
+    # after the LM head: greedy token = argmax of the projection's output, no logits to the host
+    from izwi_amd import capi
+    out = np.empty(rows, np.uint32)
+    assert capi.lib().izwi_argmax_f32(x.ctypes.data, rows, n, out.ctypes.data, capi.HOST, None) == 0
+    assert np.array_equal(out, oracle.argmax(x))
+    assert capi.lib().izwi_argmax_f32(x.ctypes.data, rows, 0, out.ctypes.data, capi.HOST, None) == -1

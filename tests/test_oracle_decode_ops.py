@@ -116,3 +116,15 @@ def test_rope_and_attention_random_qwen3_shapes(oracle):
     # one position: the output is that position's value row, whatever the scores
     one = oracle.decode_gqa_attention(q1, kc, vc, 1, 1.0)
     assert np.allclose(one[0, :, 0], np.repeat(vc[0, :, 0], hq // hk, axis=0), atol=1e-6)
+
+
+def test_argmax_first_index_of_the_maximum(oracle):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((5, 1000)).astype(np.float32)
+    x[1, 17] = x[1, 900] = 9.0          # a tie: the first wins
+    x[2, :] = -np.inf                   # every value equal
+    x[3, 5] = np.nan                    # NaN is never the maximum
+    x[3, 6] = 50.0
+    got = oracle.argmax(x)
+    want = np.argmax(np.where(np.isnan(x), -np.inf, x), axis=1)
+    assert np.array_equal(got, want) and got[1] == 17 and got[2] == 0 and got[3] == 6
