@@ -514,8 +514,7 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
     Staged xi, yo;
     HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
     HIP_TRY(yo.out(y, (size_t)m * L.n * sizeof(float), mem_space));
-    if (m < mfma_min_m() || (L.dtype == IZWI_QMM_Q6_K && m <= 64)) {
-        // (Q6_K has no matrix-core decode form: the dot4 kernel takes its rows four at a time)
+    if (m < mfma_min_m()) {
         HIP_TRY(qmm_launch_gemv(L, w->tiled, (const float*)xi.dev, m, (float*)yo.dev, w->n_cus, stream));
     } else if (m <= 64) {
         void* scratch = nullptr;
@@ -715,7 +714,7 @@ int izwi_qmm_forward_fused(const izwi_qmm_weight* w, const void* x, int x_dtype,
     if (residual) HIP_TRY(ri.in(residual, ybytes, mem_space));
     HIP_TRY(yo.out(y, ybytes, mem_space));
     QmmIo io{x_bf16 ? 1 : 0, residual ? ri.dev : nullptr, y_bf16 ? 1 : 0};
-    if (m < mfma_min_m() || (L.dtype == IZWI_QMM_Q6_K && m <= 64)) {
+    if (m < mfma_min_m()) {
         const float* xf = (const float*)xi.dev;
         if (x_bf16 && m > 2) { // this kernel reads bf16 rows only in its one- and two-row forms
             void* wide = nullptr;

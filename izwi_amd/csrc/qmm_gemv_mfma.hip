@@ -69,12 +69,13 @@ struct Unit {
     // Q4_K: 16 row scales (f32), then per row the eight sub-block sums of the quants split
     // into two int8 planes (sum = 128 * hi + lo): 64 + 16 * 16 bytes.
     // Q8_0: one f32 scale per (block, row): 8 * 16 * 4 bytes.
-    static constexpr int kSide = QT == QMM_Q4_K ? 320 : 512;
+    // Q6_K: the record of Q4_K (the same Q8_K quantization; the sub-block sums go unused).
+    static constexpr int kSide = QT == QMM_Q8_0 ? 512 : 320;
     static constexpr int kBytes = kQuant + kSide;
 };
 constexpr int kWindowUnits = 32; // activation units resident in LDS at a time
 
-__host__ __device__ inline int unit_bytes(int qt) { return qt == QMM_Q4_K ? Unit<QMM_Q4_K>::kBytes : Unit<QMM_Q8_0>::kBytes; }
+__host__ __device__ inline int unit_bytes(int qt) { return qt == QMM_Q8_0 ? Unit<QMM_Q8_0>::kBytes : Unit<QMM_Q4_K>::kBytes; }
 
 // Workgroup barrier that orders LDS traffic only (the compiler's own barrier also
 // waits for every outstanding global load of the wave).
@@ -291,9 +292,12 @@ __device__ __forceinline__ void transpose_pair(u32x4& q0, u32x4& q1) {
 
 template <int QT>
 struct WPanel {
-    static constexpr int QC = QT == QMM_Q4_K ? 8 : 16;
+    // quant chunks held per lane: Q6_K's are the 8 of low nibbles and the 4 of high bit pairs
+    static constexpr int QC = QT == QMM_Q4_K ? 8 : (QT == QMM_Q6_K ? 12 : 16);
+    static constexpr int kLoads = QC + 4 + (QT == QMM_Q6_K ? 4 : 0); // vector loads of one panel
     u32x4 hdr[4]; // headers of the four units of row j
     u32x4 q[QC];
+    u32x4 dch[QT == QMM_Q6_K ? 4 : 1]; // Q6_K: the chunks that hold d of the four units of row j
 };
 
 // Unconditional loads (one basic block, so the waits can be counted): a lane
@@ -306,6 +310,20 @@ __device__ __forceinline__ void load_wpanel(WPanel<QT>& p, const uint8_t* __rest
     const int ln = lane < slots ? lane : 0;
 #pragma unroll
     for (int u = 0; u < 4; u++) p.hdr[u] = b[(u * 16 < slots ? u * 16 : 0) + j];
+    if (QT == QMM_Q6_K) {
+        // in the order panel_dot consumes them (loads return in order): per half of the units' 256
+        // elements first its two chunks of bit pairs, then its four of nibbles; d last
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+#pragma unroll
+            for (int c = 0; c < 2; c++) p.q[8 + 2 * h + c] = __builtin_nontemporal_load(b + (size_t)(9 + 2 * h + c) * slots + ln);
+#pragma unroll
+            for (int c = 0; c < 4; c++) p.q[4 * h + c] = __builtin_nontemporal_load(b + (size_t)(1 + 4 * h + c) * slots + ln);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) p.dch[u] = b[(size_t)13 * slots + (u * 16 < slots ? u * 16 : 0) + j];
+        return;
+    }
 #pragma unroll
     for (int c = 0; c < WPanel<QT>::QC; c++)
         p.q[c] = __builtin_nontemporal_load(b + (size_t)(1 + c) * slots + ln);
@@ -404,6 +422,71 @@ __device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int
                 acc[r] += (d * dxs[r]) * (float)isum[u][r] - (dmin * dxs[r]) * (float)msum;
             }
         }
+    } else if (QT == QMM_Q6_K) {
+        // Sub-block t = 4 h + g of a unit (32 elements) is nibble g / 2 of the nibble chunk pair
+        // 2 h + g % 2 with bit pair g of the bit-pair chunk pair h; each of its two 16-element
+        // groups has its own signed scale, and the matrix instruction sums 32: it runs twice, once
+        // with the upper two octets of the B operand zeroed and once with the lower two.
+        int isum[4][4];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) isum[u][r] = 0;
+#pragma unroll
+        for (int cp = 0; cp < 4; cp++) {
+            const int h = cp >> 1, gb = cp & 1;
+            if (FIRST) {
+                if (gb == 0) transpose_pair(p.q[8 + 2 * h], p.q[9 + 2 * h]);
+                transpose_pair(p.q[2 * cp], p.q[2 * cp + 1]);
+            }
+#pragma unroll
+            for (int hi = 0; hi < 2; hi++) {
+                const int g = gb + 2 * hi, t = 4 * h + g;
+#pragma unroll
+                for (int up = 0; up < 2; up++) {
+                    const u32x4 ql = p.q[2 * cp + up], qh = p.q[8 + 2 * h + up];
+                    i32x4 dlo[2], dhi[2];
+#pragma unroll
+                    for (int e = 0; e < 2; e++) {
+                        const int u = 2 * up + e;
+                        if (u >= n_units) continue; // uniform
+                        const uint32_t w0 = e ? ql.z : ql.x, w1 = e ? ql.w : ql.y;
+                        const uint32_t h0 = e ? qh.z : qh.x, h1 = e ? qh.w : qh.y;
+                        // six-bit quants, then q - 32 as int8 in every byte without a borrow
+                        const uint32_t v0 = ((w0 >> (4 * hi)) & kNib) | (((h0 >> (2 * g)) & 0x03030303u) << 4);
+                        const uint32_t v1 = ((w1 >> (4 * hi)) & kNib) | (((h1 >> (2 * g)) & 0x03030303u) << 4);
+                        const uint32_t s0 = ((v0 | 0x80808080u) - 0x20202020u) ^ 0x80808080u;
+                        const uint32_t s1 = ((v1 | 0x80808080u) - 0x20202020u) ^ 0x80808080u;
+                        const long bq = pack64(s0, s1);
+                        const long b_lo = grp < 2 ? bq : 0L, b_hi = grp < 2 ? 0L : bq;
+                        const long a = *reinterpret_cast<const long*>(xu0 + xo[u] + lane8 + t * 512);
+                        dlo[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b_lo, i32x4{0, 0, 0, 0}, 0, 0, 0);
+                        dhi[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b_hi, i32x4{0, 0, 0, 0}, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 2; e++) {
+                        const int u = 2 * up + e;
+                        if (u >= n_units) continue;
+                        const uint32_t hw = t < 2 ? p.hdr[u].x : t < 4 ? p.hdr[u].y : t < 6 ? p.hdr[u].z : p.hdr[u].w;
+                        const int sc_lo = (int)(int8_t)((hw >> (16 * (t & 1))) & 0xffu);
+                        const int sc_hi = (int)(int8_t)((hw >> (16 * (t & 1) + 8)) & 0xffu);
+#pragma unroll
+                        for (int r = 0; r < 4; r++) // |dot| <= 16 * 32 * 128, |scale| <= 128
+                            isum[u][r] += __mul24(sc_lo, dlo[e][r]) + __mul24(sc_hi, dhi[e][r]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            if (u >= n_units) continue;
+            const float d = qmm_f16_bits_to_f32((uint16_t)(p.dch[u].x & 0xffffu)) * ef[u];
+            const float4 dx = *reinterpret_cast<const float4*>(xu0 + xo[u] + Unit<QT>::kQuant + grp * 16);
+            acc[0] += (d * dx.x) * (float)isum[u][0];
+            acc[1] += (d * dx.y) * (float)isum[u][1];
+            acc[2] += (d * dx.z) * (float)isum[u][2];
+            acc[3] += (d * dx.w) * (float)isum[u][3];
+        }
     } else {
 #pragma unroll
         for (int b = 0; b < 8; b++) {
@@ -462,7 +545,7 @@ __device__ __forceinline__ void issue_window_copy(const uint8_t* __restrict__ sr
 template <int QT, bool SINGLE, bool GROUPED = false, bool EP = false>
 __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaParams P) {
     constexpr int UB = Unit<QT>::kBytes;
-    constexpr int NL = WPanel<QT>::QC + 4; // loads of one panel
+    constexpr int NL = WPanel<QT>::kLoads; // loads of one panel
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* lds_x = smem;                                                       // window_units * UB
     // the sums of the k-split (waves * 256 floats): behind the window(s); in the single-stage form
@@ -841,7 +924,7 @@ hipError_t qmm_launch_quantize_ws(int dtype, const float* x, int64_t m, int64_t 
     const int64_t k_units = (k + 255) / 256;
     const int64_t threads = (int64_t)n_tiles * 16 * k_units * 16;
     const unsigned grid = (unsigned)((threads + 255) / 256);
-    if (dtype == QMM_Q4_K) {
+    if (dtype == QMM_Q4_K || dtype == QMM_Q6_K) { // both dot types are Q8_K: one record format
         if (x_bf16) quantize_ws_kernel<QMM_Q4_K, true><<<grid, 256, 0, stream>>>(x, (int)m, (int)k, (int)k_units, n_tiles, (uint8_t*)workspace);
         else quantize_ws_kernel<QMM_Q4_K><<<grid, 256, 0, stream>>>(x, (int)m, (int)k, (int)k_units, n_tiles, (uint8_t*)workspace);
     } else {
@@ -940,6 +1023,9 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     if (L.dtype == QMM_Q4_K)
         return epilogue ? launch_dense_form<QMM_Q4_K, true>(form, P, grid, waves, lds, stream)
                         : launch_dense_form<QMM_Q4_K, false>(form, P, grid, waves, lds, stream);
+    if (L.dtype == QMM_Q6_K)
+        return epilogue ? launch_dense_form<QMM_Q6_K, true>(form, P, grid, waves, lds, stream)
+                        : launch_dense_form<QMM_Q6_K, false>(form, P, grid, waves, lds, stream);
     return epilogue ? launch_dense_form<QMM_Q8_0, true>(form, P, grid, waves, lds, stream)
                     : launch_dense_form<QMM_Q8_0, false>(form, P, grid, waves, lds, stream);
 }
