@@ -383,6 +383,59 @@ def layer_stack_extra(torch, qa, oracle, dtype, steps=10, warmup=3):
     return out
 
 
+def q4_k_m_mix_extra(torch, qa, oracle, m=1, steps=20, warmup=3):
+    """Extra report (not `value`): the decode stack with the tensor types of a Q4_K_M file of Qwen3-8B (the
+    reference's default chat model): attn_v and ffn_down are Q6_K in half of the layers (the first and last
+    eighth and every third layer between, as llama.cpp's Q4_K_M recipe picks them) and so is the output
+    matrix; everything else is Q4_K.  Q6_K weights are random block bytes with a finite scale (the oracle
+    has no Q6_K quantizer).  Same call structure as the headline; a q|k|v group with a Q6_K member runs as a
+    q|k group call plus one call for v."""
+    import numpy as np
+    rng = np.random.default_rng(11)
+
+    def q6k_blocks(n, k):
+        rows = min(n, 2048)
+        b = rng.integers(0, 256, size=(rows * k // 256, 210), dtype=np.uint8)
+        b[:, 208:210] = (1e-3 * rng.uniform(0.5, 2.0, size=b.shape[0])).astype(np.float16).view(np.uint8).reshape(-1, 2)
+        return np.tile(b.reshape(rows, -1), ((n + rows - 1) // rows, 1))[:n].reshape(-1)
+
+    def more_bits(i, n):
+        return i < n // 8 or i >= 7 * n // 8 or (i - n // 8) % 3 == 2
+    q4 = {name: make_blocks(oracle, Q4_K, n, k, 1000 + i) for i, (name, n, k) in enumerate(LAYER_8B)}
+    q6 = {name: q6k_blocks(n, k) for name, n, k in LAYER_8B if name in ("v", "down")}
+    shape = {name: (n, k) for name, n, k in LAYER_8B}
+    bytes_per = {Q4_K: 144, 14: 210}
+    xs = {k: torch.randn(m, k, device="cuda") for k in (4096, 12288)}
+    out = lambda n: torch.empty((m, n), dtype=torch.float32, device="cuda")  # noqa: E731
+    calls, total, n_q6 = [], 0.0, 0
+    for layer in range(N_LAYERS_8B):
+        w = {}
+        for name, (n, k) in shape.items():
+            six = name in q6 and more_bits(layer, N_LAYERS_8B)
+            n_q6 += six
+            dt = 14 if six else Q4_K
+            w[name] = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType(dt), q6[name] if six else q4[name], (n, k)))
+            total += n * k // 256 * bytes_per[dt] + 4 * m * k + 4 * m * n
+        if w["v"].qtensor.dtype() == qa.GgmlDType.Q4K:
+            calls.append(([w["q"], w["k"], w["v"]], xs[4096], [out(4096), out(1024), out(1024)]))
+        else:
+            calls.append(([w["q"], w["k"]], xs[4096], [out(4096), out(1024)]))
+            calls.append((w["v"], xs[4096], out(1024)))
+        calls.append((w["o"], xs[4096], out(4096)))
+        calls.append(([w["gate"], w["up"]], xs[4096], [out(12288), out(12288)]))
+        calls.append((w["down"], xs[12288], out(4096)))
+    name, n, k = LM_HEAD_8B
+    head = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q6K, q6k_blocks(n, k), (n, k)))
+    calls.append((head, xs[k], out(n)))
+    total += n * k // 256 * 210 + 4 * m * k + 4 * m * n
+    ms, g = time_graph(torch, lambda: run_calls(qa, calls), steps, warmup)
+    res = {"gbs": round(total / (ms * 1e-3) / 1e9, 1), "ms_per_step": round(ms, 4), "m": m, "calls_per_step": len(calls),
+           "q6k_tensors": n_q6 + 1, "gb_per_step": round(total / 1e9, 3)}
+    del calls, g
+    torch.cuda.empty_cache()
+    return res
+
+
 def moe_extra(torch, qa, oracle, steps=50, warmup=5):
     """One MoE layer (route + sort + grouped expert MLP + combine, HIP-graph replay) at the
     Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, expert intermediate 768, Q4_K; as one
@@ -609,6 +662,11 @@ def main():
             extras["decode_step_neighbours_f32"] = neighbours_extra(torch, qa)
         except Exception as exc:
             extras["neighbours_error"] = repr(exc)
+        try:
+            extras["decode_q4_k_m_mix_8b_stack"] = q4_k_m_mix_extra(torch, qa, oracle, 1)
+            extras["decode_q4_k_m_mix_8b_stack_m16"] = q4_k_m_mix_extra(torch, qa, oracle, 16)
+        except Exception as exc:
+            extras["q4_k_m_mix_error"] = repr(exc)
         try:
             extras["qwen3_8b_decode_step_all_calls"] = layer_stack_extra(torch, qa, oracle, dtype)
         except Exception as exc:
