@@ -719,7 +719,7 @@ hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
     if (grid > 0x7fffffff) return hipErrorInvalidValue;
     const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
     const bool x_tail = (P.k & 63) != 0;
-    constexpr bool kPipe = BM == 256 || BN == 256;
+    constexpr bool kPipe = (BM == 256 || BN == 256) && QT != QMM_Q6_K; // Q6_K: the plain tile kernel only
     const void* fn;
     if constexpr (kPipe)
         fn = x_tail ? reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, BN, true, NW>)
@@ -869,7 +869,13 @@ hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uin
     P.nibble_mask = 0x0f0f0f0fu;
     P.partial = (float*)workspace;
     P.residual = residual;
-    if (L.dtype == QMM_Q6_K) return launch_tile<QMM_Q6_K, 128, 128>(P, 1, stream); // the plain tile kernel only
+    if (L.dtype == QMM_Q6_K) {
+        // the plain tile kernel only (a 256 x 128 tile was no faster: 308 against 316 us on
+        // [4096, 12288] at m = 2048); half-height tiles when full ones would leave CUs idle
+        const int64_t t128 = ((m + 127) / 128) * ((L.n + 127) / 128);
+        if (t128 < (int64_t)n_cus && m > 64) return launch_tile<QMM_Q6_K, 64, 128>(P, 1, stream);
+        return launch_tile<QMM_Q6_K, 128, 128>(P, 1, stream);
+    }
     return L.dtype == QMM_Q4_K ? launch_qt<QMM_Q4_K>(P, n_cus, stream)
                                : launch_qt<QMM_Q8_0>(P, n_cus, stream);
 }
