@@ -1,6 +1,6 @@
 /*
  * izwi_decode_ops — the decode-step neighbours of the quantized projections: RMSNorm, the
- * q/k head norm, rotary embedding and single-token grouped-query attention, f32.
+ * q/k head norm, rotary embedding and single-token grouped-query attention, f32 and f16.
  *
  * Each entry point is the device side of one of the reference's fused-kernel hooks
  * (crates/izwi-core/src/kernels/mod.rs:109-225), which today dispatch to Metal only
@@ -12,7 +12,7 @@
  * Conventions are those of izwi_qmm.h: return IZWI_QMM_OK or a negative izwi_qmm_status, message
  * through izwi_qmm_last_error(); `mem_space` says whether the pointers are device or host
  * memory (host buffers are staged, synchronous); `stream` is a hipStream_t or NULL.  All tensors
- * are contiguous row-major f32.  Outputs may alias the corresponding inputs (in-place).
+ * are contiguous row-major, f32 unless the entry point's name says f16.  Outputs may alias the corresponding inputs (in-place).
  */
 #ifndef IZWI_DECODE_OPS_H
 #define IZWI_DECODE_OPS_H
@@ -50,6 +50,24 @@ int izwi_qk_rms_norm_f32(const float* q, const float* k, const float* qk_weight,
 int izwi_rope_pair_bshd_f32(const float* q, const float* k, const float* cos_sin, int64_t batch,
                             int64_t seq, int64_t q_heads, int64_t k_heads, int64_t head_dim,
                             float* q_out, float* k_out, int mem_space, void* stream);
+
+/* The hooks' `DType::F16` arm (the reference's `*_f16` shaders, metal.rs:103-144, 187-225, 267-305,
+ * 383-457): the same four operations on IEEE half tensors (raw bits as uint16_t), every tensor of a
+ * call f16 as the reference's wrappers require; values are widened on load, all arithmetic is f32
+ * and each result is rounded to f16 once.  The reference's tests allow 5e-3 for this arm
+ * (metal.rs:2956).  Shapes, limits and error behaviour are those of the f32 entry points. */
+int izwi_rms_norm_f16(const uint16_t* x, const uint16_t* weight, int64_t rows, int64_t hidden, float eps,
+                      uint16_t* y, int mem_space, void* stream);
+int izwi_qk_rms_norm_f16(const uint16_t* q, const uint16_t* k, const uint16_t* qk_weight, int64_t q_rows,
+                         int64_t k_rows, int64_t head_dim, float eps, uint16_t* q_out, uint16_t* k_out,
+                         int mem_space, void* stream);
+int izwi_rope_pair_bshd_f16(const uint16_t* q, const uint16_t* k, const uint16_t* cos_sin, int64_t batch,
+                            int64_t seq, int64_t q_heads, int64_t k_heads, int64_t head_dim,
+                            uint16_t* q_out, uint16_t* k_out, int mem_space, void* stream);
+int izwi_decode_gqa_attention_f16(const uint16_t* q, const uint16_t* k, const uint16_t* v, int64_t num_heads,
+                                  int64_t num_kv_heads, int64_t head_dim, int64_t kv_len,
+                                  int64_t kv_capacity, float scale, uint16_t* out, int mem_space,
+                                  void* stream);
 
 /* The single-token sequence of `Qwen3Attention::forward` between the q/k/v projections and the
  * attention itself as ONE launch: `apply_qk_norm_pair` (qwen3/core.rs:1464-1478), `apply_rope_pair`

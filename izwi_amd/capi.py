@@ -66,6 +66,11 @@ PROTOTYPES = {
     "izwi_rms_norm_f32": (C.c_int, [_vp, _vp, _i64, _i64, C.c_float, _vp, C.c_int, _vp]),
     "izwi_qk_rms_norm_f32": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, C.c_float, _vp, _vp, C.c_int, _vp]),
     "izwi_rope_pair_bshd_f32": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, C.c_int, _vp]),
+    "izwi_rms_norm_f16": (C.c_int, [_vp, _vp, _i64, _i64, C.c_float, _vp, C.c_int, _vp]),
+    "izwi_qk_rms_norm_f16": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, C.c_float, _vp, _vp, C.c_int, _vp]),
+    "izwi_rope_pair_bshd_f16": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, C.c_int, _vp]),
+    "izwi_decode_gqa_attention_f16": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, C.c_float, _vp,
+                                                C.c_int, _vp]),
     "izwi_argmax_f32": (C.c_int, [_vp, _i64, _i64, _vp, C.c_int, _vp]),
     "izwi_qk_norm_rope_append_f32": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, C.c_float, _vp, _vp, _vp,
                                                _i64, _i64, _vp]),

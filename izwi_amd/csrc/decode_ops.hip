@@ -71,6 +71,41 @@ int check_space(int mem_space) {
     return IZWI_QMM_OK;
 }
 
+// The hooks' two element types: f32, and f16 widened on load and rounded once on store (all
+// arithmetic is f32, as in the reference's *_f16 shaders, metal.rs:103-144, 187-225, 267-305,
+// 383-457).  A 16-byte piece holds kEC<T> consecutive elements.
+typedef _Float16 f16_t;
+template <typename T>
+constexpr int kEC = 16 / (int)sizeof(T);
+template <typename T>
+__device__ __forceinline__ float ld1(const T* p) { return (float)*p; }
+template <typename T>
+__device__ __forceinline__ void st1(T* p, float v) { *p = (T)v; }
+template <typename T>
+__device__ __forceinline__ void ld16(const T* p, float (&v)[kEC<T>]) {
+    if constexpr (sizeof(T) == 4) {
+        const float4 t = *reinterpret_cast<const float4*>(p);
+        v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+    } else {
+        typedef f16_t h8 __attribute__((ext_vector_type(8)));
+        const h8 t = *reinterpret_cast<const h8*>(p);
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = (float)t[i];
+    }
+}
+template <typename T>
+__device__ __forceinline__ void st16(T* p, const float (&v)[kEC<T>]) {
+    if constexpr (sizeof(T) == 4) {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+        typedef f16_t h8 __attribute__((ext_vector_type(8)));
+        h8 t;
+#pragma unroll
+        for (int i = 0; i < 8; i++) t[i] = (f16_t)v[i];
+        *reinterpret_cast<h8*>(p) = t;
+    }
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
@@ -81,52 +116,58 @@ __device__ __forceinline__ float wave_sum(float v) {
 // Row r < rows_a comes from a / goes to out_a with weight_a, the others from b (the q/k pair);
 // a plain RMSNorm has rows_b == 0.  VEC: hidden is a multiple of 4 and all rows are 16-byte
 // aligned.  A thread keeps up to PER values of its row in registers; longer rows are re-read.
+template <typename T>
 struct NormParams {
-    const float* a;
-    const float* b;
-    const float* weight_a;
-    const float* weight_b;
-    float* out_a;
-    float* out_b;
+    const T* a;
+    const T* b;
+    const T* weight_a;
+    const T* weight_b;
+    T* out_a;
+    T* out_b;
     int64_t rows_a, rows_b;
     int hidden;
     float eps;
 };
 
-template <bool VEC>
-__global__ void rms_norm_kernel(NormParams P) {
-    constexpr int PER = 4; // float4s (VEC) or floats kept per thread
+template <bool VEC, typename T>
+__global__ void rms_norm_kernel(NormParams<T> P) {
+    constexpr int PER = 4, EC = kEC<T>; // 16-byte pieces (VEC) or single values kept per thread
     __shared__ float partial[16];
     const int64_t row = blockIdx.x;
     const bool first = row < P.rows_a;
-    const float* x = first ? P.a + row * P.hidden : P.b + (row - P.rows_a) * P.hidden;
-    const float* w = first ? P.weight_a : P.weight_b;
-    float* y = first ? P.out_a + row * P.hidden : P.out_b + (row - P.rows_a) * P.hidden;
+    const T* x = first ? P.a + row * P.hidden : P.b + (row - P.rows_a) * P.hidden;
+    const T* w = first ? P.weight_a : P.weight_b;
+    T* y = first ? P.out_a + row * P.hidden : P.out_b + (row - P.rows_a) * P.hidden;
     const int tid = threadIdx.x, nt = blockDim.x;
     float sum = 0.0f;
-    float4 keep4[PER];
+    float keepv[PER][EC];
     float keep1[PER];
+    const int nv = P.hidden / EC;
     if (VEC) {
-        const int n4 = P.hidden >> 2;
-        const float4* x4 = reinterpret_cast<const float4*>(x);
 #pragma unroll
         for (int i = 0; i < PER; i++) {
             const int idx = tid + i * nt;
-            keep4[i] = idx < n4 ? x4[idx] : make_float4(0, 0, 0, 0);
-            sum += keep4[i].x * keep4[i].x + keep4[i].y * keep4[i].y + keep4[i].z * keep4[i].z + keep4[i].w * keep4[i].w;
+            if (idx < nv) ld16<T>(x + (int64_t)idx * EC, keepv[i]);
+#pragma unroll
+            for (int c = 0; c < EC; c++) {
+                if (idx >= nv) keepv[i][c] = 0.0f;
+                sum += keepv[i][c] * keepv[i][c];
+            }
         }
-        for (int idx = tid + PER * nt; idx < n4; idx += nt) {
-            const float4 v = x4[idx];
-            sum += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        for (int idx = tid + PER * nt; idx < nv; idx += nt) {
+            float v[EC];
+            ld16<T>(x + (int64_t)idx * EC, v);
+#pragma unroll
+            for (int c = 0; c < EC; c++) sum += v[c] * v[c];
         }
     } else {
 #pragma unroll
         for (int i = 0; i < PER; i++) {
             const int idx = tid + i * nt;
-            keep1[i] = idx < P.hidden ? x[idx] : 0.0f;
+            keep1[i] = idx < P.hidden ? ld1(x + idx) : 0.0f;
             sum += keep1[i] * keep1[i];
         }
-        for (int idx = tid + PER * nt; idx < P.hidden; idx += nt) sum += x[idx] * x[idx];
+        for (int idx = tid + PER * nt; idx < P.hidden; idx += nt) sum += ld1(x + idx) * ld1(x + idx);
     }
     sum = wave_sum(sum);
     if ((tid & 63) == 0) partial[tid >> 6] = sum;
@@ -135,53 +176,55 @@ __global__ void rms_norm_kernel(NormParams P) {
     for (int i = 0; i < (nt + 63) / 64; i++) total += partial[i];
     const float scale = 1.0f / sqrtf(total / (float)P.hidden + P.eps);
     if (VEC) {
-        const int n4 = P.hidden >> 2;
-        const float4* w4 = reinterpret_cast<const float4*>(w);
-        float4* y4 = reinterpret_cast<float4*>(y);
+        auto finish = [&](int idx, const float (&v)[EC]) {
+            float ww[EC], o[EC];
+            ld16<T>(w + (int64_t)idx * EC, ww);
+#pragma unroll
+            for (int c = 0; c < EC; c++) o[c] = v[c] * scale * ww[c];
+            st16<T>(y + (int64_t)idx * EC, o);
+        };
 #pragma unroll
         for (int i = 0; i < PER; i++) {
             const int idx = tid + i * nt;
-            if (idx < n4) {
-                const float4 ww = w4[idx], v = keep4[i];
-                y4[idx] = make_float4(v.x * scale * ww.x, v.y * scale * ww.y, v.z * scale * ww.z, v.w * scale * ww.w);
-            }
+            if (idx < nv) finish(idx, keepv[i]);
         }
-        const float4* x4 = reinterpret_cast<const float4*>(x);
-        for (int idx = tid + PER * nt; idx < n4; idx += nt) {
-            const float4 ww = w4[idx], v = x4[idx];
-            y4[idx] = make_float4(v.x * scale * ww.x, v.y * scale * ww.y, v.z * scale * ww.z, v.w * scale * ww.w);
+        for (int idx = tid + PER * nt; idx < nv; idx += nt) {
+            float v[EC];
+            ld16<T>(x + (int64_t)idx * EC, v);
+            finish(idx, v);
         }
     } else {
 #pragma unroll
         for (int i = 0; i < PER; i++) {
             const int idx = tid + i * nt;
-            if (idx < P.hidden) y[idx] = keep1[i] * scale * w[idx];
+            if (idx < P.hidden) st1(y + idx, keep1[i] * scale * ld1(w + idx));
         }
-        for (int idx = tid + PER * nt; idx < P.hidden; idx += nt) y[idx] = x[idx] * scale * w[idx];
+        for (int idx = tid + PER * nt; idx < P.hidden; idx += nt) st1(y + idx, ld1(x + idx) * scale * ld1(w + idx));
     }
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-hipError_t launch_norm(const NormParams& P, hipStream_t stream) {
+template <typename T>
+hipError_t launch_norm(const NormParams<T>& P, hipStream_t stream) {
     const int64_t rows = P.rows_a + P.rows_b;
     if (rows == 0) return hipSuccess;
     if (rows > 0x7fffffff) return hipErrorInvalidValue;
-    const bool vec = P.hidden % 4 == 0 && aligned16(P.a) && aligned16(P.out_a) && aligned16(P.weight_a) &&
+    const bool vec = P.hidden % kEC<T> == 0 && aligned16(P.a) && aligned16(P.out_a) && aligned16(P.weight_a) &&
                      (P.rows_b == 0 || (aligned16(P.b) && aligned16(P.out_b) && aligned16(P.weight_b)));
     // one 16-byte piece (or value) per thread up to four per thread; at most 1024 threads
-    const int items = vec ? P.hidden / 4 : P.hidden;
+    const int items = vec ? P.hidden / kEC<T> : P.hidden;
     int threads = 64;
     while (threads < 1024 && threads < items) threads *= 2;
-    if (vec) rms_norm_kernel<true><<<(unsigned)rows, threads, 0, stream>>>(P);
-    else rms_norm_kernel<false><<<(unsigned)rows, threads, 0, stream>>>(P);
+    if (vec) rms_norm_kernel<true, T><<<(unsigned)rows, threads, 0, stream>>>(P);
+    else rms_norm_kernel<false, T><<<(unsigned)rows, threads, 0, stream>>>(P);
     return hipGetLastError();
 }
 
 // ---- rotary embedding ----------------------------------------------------------------------
-__global__ void rope_pair_kernel(const float* __restrict__ cos_sin, const float* q, const float* k, float* q_out,
-                                 float* k_out, int64_t q_rows, int64_t k_rows, int seq, int q_heads, int k_heads,
-                                 int head_dim) {
+template <typename T>
+__global__ void rope_pair_kernel(const T* __restrict__ cos_sin, const T* q, const T* k, T* q_out, T* k_out,
+                                 int64_t q_rows, int64_t k_rows, int seq, int q_heads, int k_heads, int head_dim) {
     const int half = head_dim >> 1;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (q_rows + k_rows) * half) return;
@@ -190,12 +233,12 @@ __global__ void rope_pair_kernel(const float* __restrict__ cos_sin, const float*
     const bool is_q = row < q_rows;
     const int64_t local = is_q ? row : row - q_rows;
     const int pos = (int)((local / (is_q ? q_heads : k_heads)) % seq);
-    const float* x = (is_q ? q : k) + local * head_dim;
-    float* y = (is_q ? q_out : k_out) + local * head_dim;
-    const float c = cos_sin[(int64_t)pos * head_dim + d], s = cos_sin[(int64_t)pos * head_dim + half + d];
-    const float x1 = x[d], x2 = x[half + d];
-    y[d] = x1 * c - x2 * s;
-    y[half + d] = x1 * s + x2 * c;
+    const T* x = (is_q ? q : k) + local * head_dim;
+    T* y = (is_q ? q_out : k_out) + local * head_dim;
+    const float c = ld1(cos_sin + (int64_t)pos * head_dim + d), s = ld1(cos_sin + (int64_t)pos * head_dim + half + d);
+    const float x1 = ld1(x + d), x2 = ld1(x + half + d);
+    st1(y + d, x1 * c - x2 * s);
+    st1(y + half + d, x1 * s + x2 * c);
 }
 
 // ---- greedy sampling: first index of the row maximum ------------------------------------------
@@ -290,11 +333,12 @@ __global__ __launch_bounds__(256) void qkv_prep_kernel(QkvPrepParams P) {
 }
 
 // ---- single-token GQA attention ------------------------------------------------------------
+template <typename T>
 struct AttnParams {
-    const float* q;
-    const float* k;
-    const float* v;
-    float* out;
+    const T* q;
+    const T* k;
+    const T* v;
+    T* out;
     float* part; // [heads][splits][head_dim + 2]: weighted value sums, running max, sum of weights
     int heads, kv_heads, group;
     int kv_len, chunk, splits; // split s covers positions [s * chunk, min(kv_len, (s + 1) * chunk))
@@ -321,11 +365,12 @@ __device__ __forceinline__ float sum8(float v) {
     return v;
 }
 
-// NI = head_dim / 32; G query heads of one kv head per workgroup.  Lane j of an 8-lane row group
-// holds the elements 32 i + 4 j + c (i < NI, c < 4) of a cache row and of the query heads.
-template <int NI, int G>
-__global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
-    constexpr int HD = 32 * NI, E = 4 * NI;
+// HD = head_dim; G query heads of one kv head per workgroup.  Lane j of an 8-lane row group
+// holds, of a cache row and of the query heads, the 16-byte pieces j, j + 8, ..: elements
+// 8 EC i + EC j + c (i < NI, c < EC; EC = 4 for f32, 8 for f16).
+template <typename T, int HD, int G>
+__global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams<T> P) {
+    constexpr int EC = kEC<T>, NI = HD / (8 * EC), E = EC * NI;
     __shared__ __attribute__((aligned(16))) float red[16][G][HD + 4]; // [.. HD): sums, [HD]: maximum, [HD + 1]: weight sum
     const int kvh = blockIdx.x, sp = blockIdx.y, h0 = kvh * P.group + blockIdx.z * G;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -336,8 +381,10 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
     for (int g = 0; g < G; g++)
 #pragma unroll
         for (int i = 0; i < NI; i++) {
-            const float4 t = *reinterpret_cast<const float4*>(P.q + (int64_t)(h0 + g) * HD + 32 * i + 4 * j);
-            qr[g][4 * i] = t.x, qr[g][4 * i + 1] = t.y, qr[g][4 * i + 2] = t.z, qr[g][4 * i + 3] = t.w;
+            float t[EC];
+            ld16<T>(P.q + (int64_t)(h0 + g) * HD + 8 * EC * i + EC * j, t);
+#pragma unroll
+            for (int c = 0; c < EC; c++) qr[g][EC * i + c] = t[c];
         }
     float m[G], l[G], acc[G][E];
 #pragma unroll
@@ -348,21 +395,29 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
         for (int e = 0; e < E; e++) acc[g][e] = 0.0f;
     }
     const int p0 = sp * P.chunk, p1 = min(P.kv_len, p0 + P.chunk);
-    const float* kb = P.k + (int64_t)kvh * P.kv_capacity * HD + 4 * j;
-    const float* vb = P.v + (int64_t)kvh * P.kv_capacity * HD + 4 * j;
+    const T* kb = P.k + (int64_t)kvh * P.kv_capacity * HD + EC * j;
+    const T* vb = P.v + (int64_t)kvh * P.kv_capacity * HD + EC * j;
     for (int p = p0 + slot; p < p1; p += 32) {
-        float4 kr[NI], vr[NI];
+        float kr[E], vr[E];
 #pragma unroll
-        for (int i = 0; i < NI; i++) kr[i] = *reinterpret_cast<const float4*>(kb + (int64_t)p * HD + 32 * i);
+        for (int i = 0; i < NI; i++) {
+            float t[EC];
+            ld16<T>(kb + (int64_t)p * HD + 8 * EC * i, t);
 #pragma unroll
-        for (int i = 0; i < NI; i++) vr[i] = *reinterpret_cast<const float4*>(vb + (int64_t)p * HD + 32 * i);
+            for (int c = 0; c < EC; c++) kr[EC * i + c] = t[c];
+        }
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            float t[EC];
+            ld16<T>(vb + (int64_t)p * HD + 8 * EC * i, t);
+#pragma unroll
+            for (int c = 0; c < EC; c++) vr[EC * i + c] = t[c];
+        }
 #pragma unroll
         for (int g = 0; g < G; g++) {
             float dot = 0.0f;
 #pragma unroll
-            for (int i = 0; i < NI; i++)
-                dot += qr[g][4 * i] * kr[i].x + qr[g][4 * i + 1] * kr[i].y + qr[g][4 * i + 2] * kr[i].z +
-                       qr[g][4 * i + 3] * kr[i].w;
+            for (int e = 0; e < E; e++) dot += qr[g][e] * kr[e];
             const float s = sum8(dot) * P.scale;
             if (s > m[g]) { // a new maximum (rare after the first positions): rescale what was summed
                 const float alpha = merge_weight(m[g], s);
@@ -374,12 +429,7 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
             const float pe = exp_neg(s - m[g]);
             l[g] += pe;
 #pragma unroll
-            for (int i = 0; i < NI; i++) {
-                acc[g][4 * i] += pe * vr[i].x;
-                acc[g][4 * i + 1] += pe * vr[i].y;
-                acc[g][4 * i + 2] += pe * vr[i].z;
-                acc[g][4 * i + 3] += pe * vr[i].w;
-            }
+            for (int e = 0; e < E; e++) acc[g][e] += pe * vr[e];
         }
     }
     // Merge the 32 row groups of the workgroup: neighbours 8 lanes apart inside a 16-lane row by a
@@ -402,8 +452,10 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
         for (int g = 0; g < G; g++) {
 #pragma unroll
             for (int i = 0; i < NI; i++)
-                *reinterpret_cast<float4*>(&red[entry][g][32 * i + 4 * j]) =
-                    make_float4(acc[g][4 * i], acc[g][4 * i + 1], acc[g][4 * i + 2], acc[g][4 * i + 3]);
+#pragma unroll
+                for (int c = 0; c < EC; c += 4)
+                    *reinterpret_cast<float4*>(&red[entry][g][8 * EC * i + EC * j + c]) =
+                        make_float4(acc[g][EC * i + c], acc[g][EC * i + c + 1], acc[g][EC * i + c + 2], acc[g][EC * i + c + 3]);
             if (j == 0) red[entry][g][HD] = m[g], red[entry][g][HD + 1] = l[g];
         }
     }
@@ -422,7 +474,7 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
         }
         const int h = h0 + g;
         if (P.splits == 1) {
-            P.out[(int64_t)h * HD + d] = a * (1.0f / lsum);
+            st1(P.out + (int64_t)h * HD + d, a * (1.0f / lsum));
         } else {
             float* dst = P.part + ((int64_t)h * P.splits + sp) * (HD + 2);
             dst[d] = a;
@@ -436,7 +488,8 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams P) {
 // then run over the splits with their loads independent of each other (unrolled), not one memory
 // round trip per split.
 constexpr int kMaxSplits = 1024;
-__global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict__ part, float* __restrict__ out,
+template <typename T>
+__global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict__ part, T* __restrict__ out,
                                                          int splits, int head_dim) {
     __shared__ float weight[kMaxSplits];
     __shared__ float red[8];
@@ -466,28 +519,26 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict
         float a = 0.0f;
 #pragma unroll 8
         for (int s = 0; s < splits; s++) a += base[(int64_t)s * (head_dim + 2) + d] * weight[s];
-        out[(int64_t)h * head_dim + d] = a * inv;
+        st1(out + (int64_t)h * head_dim + d, a * inv);
     }
 }
 
-template <int NI>
-hipError_t launch_attn_partial(const AttnParams& P, int g, dim3 grid, hipStream_t stream) {
+template <typename T, int HD>
+hipError_t launch_attn_partial(const AttnParams<T>& P, int g, dim3 grid, hipStream_t stream) {
     if (g == 4) {
-        if constexpr (NI <= 4) attn_partial_kernel<NI, 4><<<grid, 256, 0, stream>>>(P);
+        if constexpr (HD <= 128) attn_partial_kernel<T, HD, 4><<<grid, 256, 0, stream>>>(P);
         else return hipErrorInvalidValue;
     } else if (g == 2) {
-        attn_partial_kernel<NI, 2><<<grid, 256, 0, stream>>>(P);
+        attn_partial_kernel<T, HD, 2><<<grid, 256, 0, stream>>>(P);
     } else {
-        attn_partial_kernel<NI, 1><<<grid, 256, 0, stream>>>(P);
+        attn_partial_kernel<T, HD, 1><<<grid, 256, 0, stream>>>(P);
     }
     return hipGetLastError();
 }
 
-} // namespace
 
-extern "C" {
-
-int izwi_rms_norm_f32(const float* x, const float* weight, int64_t rows, int64_t hidden, float eps, float* y,
+template <typename T>
+int rms_norm_impl(const T* x, const T* weight, int64_t rows, int64_t hidden, float eps, T* y,
                       int mem_space, void* stream_) {
     if (int rc = check_space(mem_space)) return rc;
     if (rows < 0 || hidden <= 0 || hidden > 0x3fffffff)
@@ -498,18 +549,19 @@ int izwi_rms_norm_f32(const float* x, const float* weight, int64_t rows, int64_t
     if (int rc = qmm_current_device(&device, &n_cus)) return rc;
     hipStream_t stream = (hipStream_t)stream_;
     Buf xi, wi, yo;
-    OPS_TRY(xi.in(x, (size_t)rows * hidden * sizeof(float), mem_space));
-    OPS_TRY(wi.in(weight, (size_t)hidden * sizeof(float), mem_space));
-    OPS_TRY(yo.out(y, (size_t)rows * hidden * sizeof(float), mem_space));
-    NormParams P{(const float*)xi.dev, nullptr, (const float*)wi.dev, nullptr, (float*)yo.dev, nullptr, rows, 0,
+    OPS_TRY(xi.in(x, (size_t)rows * hidden * sizeof(T), mem_space));
+    OPS_TRY(wi.in(weight, (size_t)hidden * sizeof(T), mem_space));
+    OPS_TRY(yo.out(y, (size_t)rows * hidden * sizeof(T), mem_space));
+    NormParams<T> P{(const T*)xi.dev, nullptr, (const T*)wi.dev, nullptr, (T*)yo.dev, nullptr, rows, 0,
                  (int)hidden, eps};
     OPS_TRY(launch_norm(P, stream));
     OPS_TRY(yo.finish(stream));
     return IZWI_QMM_OK;
 }
 
-int izwi_qk_rms_norm_f32(const float* q, const float* k, const float* qk_weight, int64_t q_rows, int64_t k_rows,
-                         int64_t head_dim, float eps, float* q_out, float* k_out, int mem_space, void* stream_) {
+template <typename T>
+int qk_rms_norm_impl(const T* q, const T* k, const T* qk_weight, int64_t q_rows, int64_t k_rows,
+                         int64_t head_dim, float eps, T* q_out, T* k_out, int mem_space, void* stream_) {
     if (int rc = check_space(mem_space)) return rc;
     if (q_rows < 0 || k_rows < 0 || head_dim <= 0 || head_dim > 8192)
         return qmm_fail(IZWI_QMM_ERR_INVALID, "qk_rms_norm: bad shape q [%lld, %lld], k [%lld, %lld]", (long long)q_rows,
@@ -521,18 +573,18 @@ int izwi_qk_rms_norm_f32(const float* q, const float* k, const float* qk_weight,
     if (int rc = qmm_current_device(&device, &n_cus)) return rc;
     hipStream_t stream = (hipStream_t)stream_;
     Buf qi, ki, wi, qo, ko;
-    OPS_TRY(qi.in(q, (size_t)q_rows * head_dim * sizeof(float), mem_space));
-    OPS_TRY(ki.in(k, (size_t)k_rows * head_dim * sizeof(float), mem_space));
-    OPS_TRY(wi.in(qk_weight, (size_t)2 * head_dim * sizeof(float), mem_space));
-    OPS_TRY(qo.out(q_out, (size_t)q_rows * head_dim * sizeof(float), mem_space));
-    OPS_TRY(ko.out(k_out, (size_t)k_rows * head_dim * sizeof(float), mem_space));
+    OPS_TRY(qi.in(q, (size_t)q_rows * head_dim * sizeof(T), mem_space));
+    OPS_TRY(ki.in(k, (size_t)k_rows * head_dim * sizeof(T), mem_space));
+    OPS_TRY(wi.in(qk_weight, (size_t)2 * head_dim * sizeof(T), mem_space));
+    OPS_TRY(qo.out(q_out, (size_t)q_rows * head_dim * sizeof(T), mem_space));
+    OPS_TRY(ko.out(k_out, (size_t)k_rows * head_dim * sizeof(T), mem_space));
     // (with no q rows the first operand of the kernel is the k tensor)
-    NormParams P;
+    NormParams<T> P;
     if (q_rows)
-        P = NormParams{(const float*)qi.dev, (const float*)ki.dev, (const float*)wi.dev, (const float*)wi.dev + head_dim,
-                       (float*)qo.dev, (float*)ko.dev, q_rows, k_rows, (int)head_dim, eps};
+        P = NormParams<T>{(const T*)qi.dev, (const T*)ki.dev, (const T*)wi.dev, (const T*)wi.dev + head_dim,
+                       (T*)qo.dev, (T*)ko.dev, q_rows, k_rows, (int)head_dim, eps};
     else
-        P = NormParams{(const float*)ki.dev, nullptr, (const float*)wi.dev + head_dim, nullptr, (float*)ko.dev, nullptr,
+        P = NormParams<T>{(const T*)ki.dev, nullptr, (const T*)wi.dev + head_dim, nullptr, (T*)ko.dev, nullptr,
                        k_rows, 0, (int)head_dim, eps};
     if (P.rows_b == 0) P.b = nullptr, P.weight_b = nullptr, P.out_b = nullptr;
     OPS_TRY(launch_norm(P, stream));
@@ -541,8 +593,9 @@ int izwi_qk_rms_norm_f32(const float* q, const float* k, const float* qk_weight,
     return IZWI_QMM_OK;
 }
 
-int izwi_rope_pair_bshd_f32(const float* q, const float* k, const float* cos_sin, int64_t batch, int64_t seq,
-                            int64_t q_heads, int64_t k_heads, int64_t head_dim, float* q_out, float* k_out,
+template <typename T>
+int rope_pair_impl(const T* q, const T* k, const T* cos_sin, int64_t batch, int64_t seq,
+                            int64_t q_heads, int64_t k_heads, int64_t head_dim, T* q_out, T* k_out,
                             int mem_space, void* stream_) {
     if (int rc = check_space(mem_space)) return rc;
     if (batch < 0 || seq < 0 || q_heads < 0 || k_heads < 0 || head_dim <= 0 || head_dim % 2 || head_dim > 0x3fffffff ||
@@ -557,22 +610,132 @@ int izwi_rope_pair_bshd_f32(const float* q, const float* k, const float* cos_sin
     if (int rc = qmm_current_device(&device, &n_cus)) return rc;
     hipStream_t stream = (hipStream_t)stream_;
     Buf qi, ki, ci, qo, ko;
-    OPS_TRY(qi.in(q, (size_t)q_rows * head_dim * sizeof(float), mem_space));
-    OPS_TRY(ki.in(k, (size_t)k_rows * head_dim * sizeof(float), mem_space));
-    OPS_TRY(ci.in(cos_sin, (size_t)seq * head_dim * sizeof(float), mem_space));
-    OPS_TRY(qo.out(q_out, (size_t)q_rows * head_dim * sizeof(float), mem_space));
-    OPS_TRY(ko.out(k_out, (size_t)k_rows * head_dim * sizeof(float), mem_space));
+    OPS_TRY(qi.in(q, (size_t)q_rows * head_dim * sizeof(T), mem_space));
+    OPS_TRY(ki.in(k, (size_t)k_rows * head_dim * sizeof(T), mem_space));
+    OPS_TRY(ci.in(cos_sin, (size_t)seq * head_dim * sizeof(T), mem_space));
+    OPS_TRY(qo.out(q_out, (size_t)q_rows * head_dim * sizeof(T), mem_space));
+    OPS_TRY(ko.out(k_out, (size_t)k_rows * head_dim * sizeof(T), mem_space));
     const int64_t pairs = (q_rows + k_rows) * (head_dim / 2);
     const int64_t grid = (pairs + 255) / 256;
     if (grid > 0x7fffffff) return qmm_fail(IZWI_QMM_ERR_UNSUPPORTED, "rope_pair_bshd: too many elements");
-    rope_pair_kernel<<<(unsigned)grid, 256, 0, stream>>>((const float*)ci.dev, (const float*)qi.dev, (const float*)ki.dev,
-                                                         (float*)qo.dev, (float*)ko.dev, q_rows, k_rows, (int)seq,
+    rope_pair_kernel<T><<<(unsigned)grid, 256, 0, stream>>>((const T*)ci.dev, (const T*)qi.dev, (const T*)ki.dev,
+                                                         (T*)qo.dev, (T*)ko.dev, q_rows, k_rows, (int)seq,
                                                          (int)(q_heads ? q_heads : 1), (int)(k_heads ? k_heads : 1),
                                                          (int)head_dim);
     OPS_TRY(hipGetLastError());
     OPS_TRY(qo.finish(stream));
     OPS_TRY(ko.finish(stream));
     return IZWI_QMM_OK;
+}
+
+template <typename T>
+int decode_attention_impl(const T* q, const T* k, const T* v, int64_t num_heads,
+                                  int64_t num_kv_heads, int64_t head_dim, int64_t kv_len, int64_t kv_capacity,
+                                  float scale, T* out, int mem_space, void* stream_) {
+    if (int rc = check_space(mem_space)) return rc;
+    if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || num_heads > 65535 || kv_len <= 0 ||
+        kv_len > kv_capacity || kv_capacity > 0x3fffffff || head_dim <= 0)
+        return qmm_fail(IZWI_QMM_ERR_INVALID,
+                        "decode_gqa_attention: bad shape (heads %lld, kv heads %lld, head_dim %lld, kv_len %lld of %lld)",
+                        (long long)num_heads, (long long)num_kv_heads, (long long)head_dim, (long long)kv_len,
+                        (long long)kv_capacity);
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256)
+        return qmm_fail(IZWI_QMM_ERR_UNSUPPORTED, "decode_gqa_attention: head_dim %lld (64, 128 and 256 are built)",
+                        (long long)head_dim);
+    if (!q || !k || !v || !out) return qmm_fail(IZWI_QMM_ERR_INVALID, "decode_gqa_attention: NULL buffer");
+    int device = 0, n_cus = 0;
+    if (int rc = qmm_current_device(&device, &n_cus)) return rc;
+    hipStream_t stream = (hipStream_t)stream_;
+    const size_t qbytes = (size_t)num_heads * head_dim * sizeof(T);
+    const size_t cbytes = (size_t)num_kv_heads * kv_capacity * head_dim * sizeof(T);
+    Buf qi, ki, vi, oo;
+    OPS_TRY(qi.in(q, qbytes, mem_space));
+    OPS_TRY(ki.in(k, cbytes, mem_space));
+    OPS_TRY(vi.in(v, cbytes, mem_space));
+    OPS_TRY(oo.out(out, qbytes, mem_space));
+    const int group = (int)(num_heads / num_kv_heads);
+    // query heads per workgroup: as many of the group as the register file takes
+    int g = group % 4 == 0 && head_dim <= 128 ? 4 : (group % 2 == 0 ? 2 : 1);
+    const int z = group / g;
+    // Enough workgroups for one per CU (IZWI_ATTN_WGS_PER_CU, tuning knob), at least 64 positions
+    // each (IZWI_ATTN_MIN_CHUNK): more splits only add merge work (measured: 2 per CU is 5-10 %
+    // slower between 4k and 16k positions, 4 per CU 30 %).
+    static const int wgs_per_cu = [] { const char* e = getenv("IZWI_ATTN_WGS_PER_CU"); int v = e ? atoi(e) : 1; return v > 0 ? v : 1; }();
+    static const int min_chunk = [] { const char* e = getenv("IZWI_ATTN_MIN_CHUNK"); int v = e ? atoi(e) : 64; return v > 0 ? v : 64; }();
+    const int64_t base_wgs = num_kv_heads * z;
+    int64_t splits = (wgs_per_cu * (int64_t)n_cus + base_wgs - 1) / base_wgs;
+    const int64_t max_splits = (kv_len + min_chunk - 1) / min_chunk;
+    if (splits > max_splits) splits = max_splits;
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    if (splits < 1) splits = 1;
+    const int chunk = (int)((kv_len + splits - 1) / splits);
+    splits = (kv_len + chunk - 1) / chunk; // every split holds at least one position
+    AttnParams<T> P;
+    P.q = (const T*)qi.dev;
+    P.k = (const T*)ki.dev;
+    P.v = (const T*)vi.dev;
+    P.out = (T*)oo.dev;
+    P.part = nullptr;
+    P.heads = (int)num_heads;
+    P.kv_heads = (int)num_kv_heads;
+    P.group = group;
+    P.kv_len = (int)kv_len;
+    P.chunk = chunk;
+    P.splits = (int)splits;
+    P.kv_capacity = kv_capacity;
+    P.scale = scale;
+    if (splits > 1) {
+        void* scratch = nullptr;
+        OPS_TRY(qmm_get_scratch(device, stream, (size_t)num_heads * splits * (head_dim + 2) * sizeof(float), &scratch));
+        P.part = (float*)scratch;
+    }
+    const dim3 grid((unsigned)num_kv_heads, (unsigned)splits, (unsigned)z);
+    hipError_t e = head_dim == 64    ? launch_attn_partial<T, 64>(P, g, grid, stream)
+                   : head_dim == 128 ? launch_attn_partial<T, 128>(P, g, grid, stream)
+                                     : launch_attn_partial<T, 256>(P, g, grid, stream);
+    OPS_TRY(e);
+    if (splits > 1) {
+        attn_merge_kernel<T><<<(unsigned)num_heads, 256, 0, stream>>>(P.part, P.out, (int)splits, (int)head_dim);
+        OPS_TRY(hipGetLastError());
+    }
+    OPS_TRY(oo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+
+} // namespace
+
+extern "C" {
+
+int izwi_rms_norm_f32(const float* x, const float* weight, int64_t rows, int64_t hidden, float eps, float* y,
+                      int mem_space, void* stream) {
+    return rms_norm_impl<float>(x, weight, rows, hidden, eps, y, mem_space, stream);
+}
+int izwi_rms_norm_f16(const uint16_t* x, const uint16_t* weight, int64_t rows, int64_t hidden, float eps, uint16_t* y,
+                      int mem_space, void* stream) {
+    return rms_norm_impl<f16_t>((const f16_t*)x, (const f16_t*)weight, rows, hidden, eps, (f16_t*)y, mem_space, stream);
+}
+
+int izwi_qk_rms_norm_f32(const float* q, const float* k, const float* qk_weight, int64_t q_rows, int64_t k_rows,
+                         int64_t head_dim, float eps, float* q_out, float* k_out, int mem_space, void* stream) {
+    return qk_rms_norm_impl<float>(q, k, qk_weight, q_rows, k_rows, head_dim, eps, q_out, k_out, mem_space, stream);
+}
+int izwi_qk_rms_norm_f16(const uint16_t* q, const uint16_t* k, const uint16_t* qk_weight, int64_t q_rows, int64_t k_rows,
+                         int64_t head_dim, float eps, uint16_t* q_out, uint16_t* k_out, int mem_space, void* stream) {
+    return qk_rms_norm_impl<f16_t>((const f16_t*)q, (const f16_t*)k, (const f16_t*)qk_weight, q_rows, k_rows, head_dim, eps,
+                                   (f16_t*)q_out, (f16_t*)k_out, mem_space, stream);
+}
+
+int izwi_rope_pair_bshd_f32(const float* q, const float* k, const float* cos_sin, int64_t batch, int64_t seq,
+                            int64_t q_heads, int64_t k_heads, int64_t head_dim, float* q_out, float* k_out,
+                            int mem_space, void* stream) {
+    return rope_pair_impl<float>(q, k, cos_sin, batch, seq, q_heads, k_heads, head_dim, q_out, k_out, mem_space, stream);
+}
+int izwi_rope_pair_bshd_f16(const uint16_t* q, const uint16_t* k, const uint16_t* cos_sin, int64_t batch, int64_t seq,
+                            int64_t q_heads, int64_t k_heads, int64_t head_dim, uint16_t* q_out, uint16_t* k_out,
+                            int mem_space, void* stream) {
+    return rope_pair_impl<f16_t>((const f16_t*)q, (const f16_t*)k, (const f16_t*)cos_sin, batch, seq, q_heads, k_heads,
+                                 head_dim, (f16_t*)q_out, (f16_t*)k_out, mem_space, stream);
 }
 
 int izwi_argmax_f32(const float* logits, int64_t rows, int64_t n, uint32_t* out, int mem_space, void* stream_) {
@@ -619,75 +782,15 @@ int izwi_qk_norm_rope_append_f32(const float* q, const float* k, const float* v,
 
 int izwi_decode_gqa_attention_f32(const float* q, const float* k, const float* v, int64_t num_heads,
                                   int64_t num_kv_heads, int64_t head_dim, int64_t kv_len, int64_t kv_capacity,
-                                  float scale, float* out, int mem_space, void* stream_) {
-    if (int rc = check_space(mem_space)) return rc;
-    if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || num_heads > 65535 || kv_len <= 0 ||
-        kv_len > kv_capacity || kv_capacity > 0x3fffffff || head_dim <= 0)
-        return qmm_fail(IZWI_QMM_ERR_INVALID,
-                        "decode_gqa_attention: bad shape (heads %lld, kv heads %lld, head_dim %lld, kv_len %lld of %lld)",
-                        (long long)num_heads, (long long)num_kv_heads, (long long)head_dim, (long long)kv_len,
-                        (long long)kv_capacity);
-    if (head_dim != 64 && head_dim != 128 && head_dim != 256)
-        return qmm_fail(IZWI_QMM_ERR_UNSUPPORTED, "decode_gqa_attention: head_dim %lld (64, 128 and 256 are built)",
-                        (long long)head_dim);
-    if (!q || !k || !v || !out) return qmm_fail(IZWI_QMM_ERR_INVALID, "decode_gqa_attention: NULL buffer");
-    int device = 0, n_cus = 0;
-    if (int rc = qmm_current_device(&device, &n_cus)) return rc;
-    hipStream_t stream = (hipStream_t)stream_;
-    const size_t qbytes = (size_t)num_heads * head_dim * sizeof(float);
-    const size_t cbytes = (size_t)num_kv_heads * kv_capacity * head_dim * sizeof(float);
-    Buf qi, ki, vi, oo;
-    OPS_TRY(qi.in(q, qbytes, mem_space));
-    OPS_TRY(ki.in(k, cbytes, mem_space));
-    OPS_TRY(vi.in(v, cbytes, mem_space));
-    OPS_TRY(oo.out(out, qbytes, mem_space));
-    const int group = (int)(num_heads / num_kv_heads);
-    // query heads per workgroup: as many of the group as the register file takes
-    int g = group % 4 == 0 && head_dim <= 128 ? 4 : (group % 2 == 0 ? 2 : 1);
-    const int z = group / g;
-    // Enough workgroups for one per CU (IZWI_ATTN_WGS_PER_CU, tuning knob), at least 64 positions
-    // each (IZWI_ATTN_MIN_CHUNK): more splits only add merge work (measured: 2 per CU is 5-10 %
-    // slower between 4k and 16k positions, 4 per CU 30 %).
-    static const int wgs_per_cu = [] { const char* e = getenv("IZWI_ATTN_WGS_PER_CU"); int v = e ? atoi(e) : 1; return v > 0 ? v : 1; }();
-    static const int min_chunk = [] { const char* e = getenv("IZWI_ATTN_MIN_CHUNK"); int v = e ? atoi(e) : 64; return v > 0 ? v : 64; }();
-    const int64_t base_wgs = num_kv_heads * z;
-    int64_t splits = (wgs_per_cu * (int64_t)n_cus + base_wgs - 1) / base_wgs;
-    const int64_t max_splits = (kv_len + min_chunk - 1) / min_chunk;
-    if (splits > max_splits) splits = max_splits;
-    if (splits > kMaxSplits) splits = kMaxSplits;
-    if (splits < 1) splits = 1;
-    const int chunk = (int)((kv_len + splits - 1) / splits);
-    splits = (kv_len + chunk - 1) / chunk; // every split holds at least one position
-    AttnParams P;
-    P.q = (const float*)qi.dev;
-    P.k = (const float*)ki.dev;
-    P.v = (const float*)vi.dev;
-    P.out = (float*)oo.dev;
-    P.part = nullptr;
-    P.heads = (int)num_heads;
-    P.kv_heads = (int)num_kv_heads;
-    P.group = group;
-    P.kv_len = (int)kv_len;
-    P.chunk = chunk;
-    P.splits = (int)splits;
-    P.kv_capacity = kv_capacity;
-    P.scale = scale;
-    if (splits > 1) {
-        void* scratch = nullptr;
-        OPS_TRY(qmm_get_scratch(device, stream, (size_t)num_heads * splits * (head_dim + 2) * sizeof(float), &scratch));
-        P.part = (float*)scratch;
-    }
-    const dim3 grid((unsigned)num_kv_heads, (unsigned)splits, (unsigned)z);
-    hipError_t e = head_dim == 64    ? launch_attn_partial<2>(P, g, grid, stream)
-                   : head_dim == 128 ? launch_attn_partial<4>(P, g, grid, stream)
-                                     : launch_attn_partial<8>(P, g, grid, stream);
-    OPS_TRY(e);
-    if (splits > 1) {
-        attn_merge_kernel<<<(unsigned)num_heads, 256, 0, stream>>>(P.part, P.out, (int)splits, (int)head_dim);
-        OPS_TRY(hipGetLastError());
-    }
-    OPS_TRY(oo.finish(stream));
-    return IZWI_QMM_OK;
+                                  float scale, float* out, int mem_space, void* stream) {
+    return decode_attention_impl<float>(q, k, v, num_heads, num_kv_heads, head_dim, kv_len, kv_capacity, scale, out,
+                                        mem_space, stream);
+}
+int izwi_decode_gqa_attention_f16(const uint16_t* q, const uint16_t* k, const uint16_t* v, int64_t num_heads,
+                                  int64_t num_kv_heads, int64_t head_dim, int64_t kv_len, int64_t kv_capacity,
+                                  float scale, uint16_t* out, int mem_space, void* stream) {
+    return decode_attention_impl<f16_t>((const f16_t*)q, (const f16_t*)k, (const f16_t*)v, num_heads, num_kv_heads,
+                                        head_dim, kv_len, kv_capacity, scale, (f16_t*)out, mem_space, stream);
 }
 
 } // extern "C"

@@ -3,7 +3,7 @@
 when the fused path does not apply" behaviour, over the C ABI of include/izwi_decode_ops.h.
 
 A hook returns None (the caller then runs its own eager operators, as the reference does) when
-its preconditions do not hold: f32, contiguous, on one GPU, the shapes the reference's wrapper
+its preconditions do not hold: f32 or f16 throughout, contiguous, on one GPU, the shapes the reference's wrapper
 checks (metal.rs:1921-1945, 1991-2003, 2043-2062, 2141-2172).  When they hold the HIP kernel runs;
 a failure inside it raises (there is no silent CPU path)."""
 from __future__ import annotations
@@ -15,8 +15,14 @@ from .qmatmul import _stream_ptr
 
 
 def _ok(*tensors: torch.Tensor) -> bool:
-    dev = tensors[0].device
-    return all(t.is_cuda and t.device == dev and t.dtype == torch.float32 and t.is_contiguous() for t in tensors)
+    """All on one GPU, contiguous, one dtype, f32 or f16 (the hooks' `matches!(dtype, F32 | F16)`)."""
+    dev, dt = tensors[0].device, tensors[0].dtype
+    return dt in (torch.float32, torch.float16) and all(
+        t.is_cuda and t.device == dev and t.dtype == dt and t.is_contiguous() for t in tensors)
+
+
+def _fn(name: str, t: torch.Tensor):
+    return getattr(lib(), f"izwi_{name}_{'f16' if t.dtype == torch.float16 else 'f32'}")
 
 
 def try_fused_rms_norm(input: torch.Tensor, weight: torch.Tensor, eps: float):  # noqa: A002
@@ -27,7 +33,7 @@ def try_fused_rms_norm(input: torch.Tensor, weight: torch.Tensor, eps: float):  
     if hidden == 0 or tuple(weight.shape) != (hidden,) or input.numel() == 0:
         return None
     out = torch.empty_like(input)
-    check(lib().izwi_rms_norm_f32(input.data_ptr(), weight.data_ptr(), input.numel() // hidden, hidden, eps,
+    check(_fn('rms_norm', input)(input.data_ptr(), weight.data_ptr(), input.numel() // hidden, hidden, eps,
                                   out.data_ptr(), DEVICE, _stream_ptr(input)))
     return out
 
@@ -42,7 +48,7 @@ def try_fused_qk_rms_norm(q: torch.Tensor, k: torch.Tensor, qk_weight: torch.Ten
     if d == 0 or tuple(qk_weight.shape) != (2 * d,):
         return None
     q_out, k_out = torch.empty_like(q), torch.empty_like(k)
-    check(lib().izwi_qk_rms_norm_f32(q.data_ptr(), k.data_ptr(), qk_weight.data_ptr(), q.numel() // d, k.numel() // d,
+    check(_fn('qk_rms_norm', q)(q.data_ptr(), k.data_ptr(), qk_weight.data_ptr(), q.numel() // d, k.numel() // d,
                                      d, eps, q_out.data_ptr(), k_out.data_ptr(), DEVICE, _stream_ptr(q)))
     return q_out, k_out
 
@@ -55,7 +61,7 @@ def try_fused_rope_pair_bshd(q: torch.Tensor, k: torch.Tensor, cos_sin: torch.Te
     if k.shape[0] != b or k.shape[1] != s or k.shape[3] != d or d == 0 or d % 2 or tuple(cos_sin.shape) != (s, d):
         return None
     q_out, k_out = torch.empty_like(q), torch.empty_like(k)
-    check(lib().izwi_rope_pair_bshd_f32(q.data_ptr(), k.data_ptr(), cos_sin.data_ptr(), b, s, hq, k.shape[2], d,
+    check(_fn('rope_pair_bshd', q)(q.data_ptr(), k.data_ptr(), cos_sin.data_ptr(), b, s, hq, k.shape[2], d,
                                         q_out.data_ptr(), k_out.data_ptr(), DEVICE, _stream_ptr(q)))
     return q_out, k_out
 
@@ -71,7 +77,7 @@ def try_fused_decode_gqa_attention_with_kv_len(q: torch.Tensor, k: torch.Tensor,
             or num_heads == 0 or num_kv_heads == 0 or num_heads % num_kv_heads or head_dim not in (64, 128, 256)):
         return None
     out = torch.empty_like(q)
-    check(lib().izwi_decode_gqa_attention_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), num_heads, num_kv_heads,
+    check(_fn('decode_gqa_attention', q)(q.data_ptr(), k.data_ptr(), v.data_ptr(), num_heads, num_kv_heads,
                                               head_dim, kv_len, k.shape[2], scale, out.data_ptr(), DEVICE,
                                               _stream_ptr(q)))
     return out
@@ -91,7 +97,8 @@ def qk_norm_rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qk_we
     elements), caches [1, kv_heads, capacity, d].  Returns the normed, rotated q as [1, heads, 1, d]; the caches
     gain position `pos`."""
     from .capi import QmmError
-    if not _ok(q, k, v, qk_weight, cos_sin, k_cache, v_cache) or k_cache.dim() != 4 or tuple(v_cache.shape) != tuple(k_cache.shape):
+    if (not _ok(q, k, v, qk_weight, cos_sin, k_cache, v_cache) or q.dtype != torch.float32 or k_cache.dim() != 4
+            or tuple(v_cache.shape) != tuple(k_cache.shape)):
         raise QmmError(-1, "qk_norm_rope_append: contiguous f32 CUDA tensors on one device expected")
     _, kv_heads, cap, d = k_cache.shape
     heads = q.numel() // d
@@ -109,7 +116,7 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     """`logits.argmax(D::Minus1)` of the greedy samplers (qwen3/chat.rs:574-597): logits [..., n] f32 on the
     GPU -> int32 indices [...] (first index of the maximum), computed on the device."""
     from .capi import QmmError
-    if not _ok(logits) or logits.dim() < 1 or logits.shape[-1] == 0:
+    if not _ok(logits) or logits.dtype != torch.float32 or logits.dim() < 1 or logits.shape[-1] == 0:
         raise QmmError(-1, "argmax: a contiguous f32 CUDA tensor with a non-empty last dimension expected")
     n = logits.shape[-1]
     out = torch.empty(logits.shape[:-1], dtype=torch.int32, device=logits.device)

@@ -169,7 +169,8 @@ def test_hooks_decline_what_the_reference_declines(qa, oracle):
     x = dev(oracle.randn(1, (2, 8)))
     w = dev(oracle.randn(2, (8,)))
     assert qa.try_fused_rms_norm(x.cpu(), w.cpu(), 1e-6) is None                 # not on the GPU
-    assert qa.try_fused_rms_norm(x.half(), w.half(), 1e-6) is None               # f16: not built here
+    assert qa.try_fused_rms_norm(x.bfloat16(), w.bfloat16(), 1e-6) is None       # the hooks take f32 and f16 only
+    assert qa.try_fused_rms_norm(x.half(), w, 1e-6) is None                      # mixed types
     assert qa.try_fused_rms_norm(x.t(), w[:2], 1e-6) is None                     # not contiguous
     assert qa.try_fused_rms_norm(x, w[:4], 1e-6) is None                         # weight shape
     q = dev(oracle.randn(3, (1, 2, 4, 8)))
@@ -234,3 +235,51 @@ def test_argmax_on_device(qa, oracle, rows, n):
     assert capi.lib().izwi_argmax_f32(x.ctypes.data, rows, n, out.ctypes.data, capi.HOST, None) == 0
     assert np.array_equal(out, oracle.argmax(x))
     assert capi.lib().izwi_argmax_f32(x.ctypes.data, rows, 0, out.ctypes.data, capi.HOST, None) == -1
+
+
+F16_TOL = 2.0 ** -10  # one rounding to f16 of an f32 result; the reference allows 5e-3 (metal.rs:2956)
+
+
+def half(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float16)).cuda()
+
+
+def close16(got, want_f32):
+    """got (f16 tensor) against the f32 oracle result rounded to f16: equal up to the last f16 bit of the sums."""
+    want = np.asarray(want_f32, dtype=np.float32).astype(np.float16).astype(np.float64)
+    g = got.float().cpu().numpy().astype(np.float64)
+    return got.dtype == torch.float16 and float(np.abs(g - want).max()) <= F16_TOL * max(1.0, float(np.abs(want).max()))
+
+
+def test_f16_arm_reference_vectors_and_model_shapes(qa, oracle):
+    """The hooks' F16 arm: the reference's test vectors (its tests run both dtypes, metal.rs:2920, 2969, 3076,
+    3202) and Qwen3 shapes; the oracle is the f32 oracle on the widened inputs, rounded once."""
+    w16 = lambda a: np.asarray(a, np.float16).astype(np.float32)  # noqa: E731  (the values the kernel sees)
+    x = w16(REF_X3.reshape(1, 3, 4))
+    assert close16(qa.try_fused_rms_norm(half(x), half(REF_W), 1e-6), oracle.rms_norm(x, w16(REF_W), 1e-6))
+    for rows, hidden in ((1, 4096), (5, 1000), (3, 36)):
+        xx, ww = w16(oracle.randn(1, (rows, hidden))), w16(oracle.randn(2, (hidden,), mean=1.0, std=0.1))
+        assert close16(qa.try_fused_rms_norm(half(xx), half(ww), 1e-6), oracle.rms_norm(xx, ww, 1e-6))
+    q, k = w16(oracle.randn(3, (2, 1, 32, 128))), w16(oracle.randn(4, (2, 1, 8, 128)))
+    qkw = w16(oracle.randn(5, (256,), mean=1.0, std=0.2))
+    qo, ko = qa.try_fused_qk_rms_norm(half(q), half(k), half(qkw), 1e-6)
+    wq, wk = oracle.qk_rms_norm(q, k, qkw, 1e-6)
+    assert close16(qo, wq) and close16(ko, wk)
+    q, k = w16(oracle.randn(6, (2, 5, 32, 128))), w16(oracle.randn(7, (2, 5, 8, 128)))
+    ang = oracle.randn(8, (5, 64)) * 3.0
+    cs = w16(np.concatenate([np.cos(ang), np.sin(ang)], axis=1))
+    qo, ko = qa.try_fused_rope_pair_bshd(half(q), half(k), half(cs))
+    wq, wk = oracle.rope_pair_bshd(q, k, cs)
+    assert close16(qo, wq) and close16(ko, wk)
+
+
+@pytest.mark.parametrize("heads,kv_heads,d,kv_len,cap", [(32, 8, 128, 1, 4), (32, 8, 128, 300, 512), (32, 8, 128, 5000, 5000),
+                                                         (14, 2, 64, 333, 400), (8, 2, 256, 500, 512), (16, 8, 128, 40960, 40960)])
+def test_f16_attention(qa, oracle, heads, kv_heads, d, kv_len, cap):
+    q = oracle.randn(1, (1, heads, 1, d)).astype(np.float16).astype(np.float32)
+    k = oracle.randn(2, (1, kv_heads, cap, d)).astype(np.float16).astype(np.float32)
+    v = oracle.randn(3, (1, kv_heads, cap, d)).astype(np.float16).astype(np.float32)
+    k[:, :, kv_len:], v[:, :, kv_len:] = 1e4, -1e4
+    got = qa.try_fused_decode_gqa_attention_with_kv_len(half(q), half(k), half(v), heads, kv_heads, d, kv_len, d ** -0.5)
+    assert got.shape == (1, heads, 1, d)
+    assert close16(got, oracle.decode_gqa_attention(q, k, v, kv_len, d ** -0.5))
