@@ -199,6 +199,29 @@ int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int6
 int izwi_qmm_forward_fused(const izwi_qmm_weight* w, const void* x, int x_dtype, int64_t m,
                            const void* residual, void* y, int y_dtype, int mem_space, void* stream);
 
+/* The RMSNorm that precedes a projection folded into the projection's call:
+ * `Qwen3Layer::forward`'s `input_layernorm.forward(x)` before the q/k/v projections and
+ * `post_attention_layernorm.forward(&x)` before gate/up (qwen3/core.rs:1872, 1877), and the final
+ * norm before the LM head.  y_i = QMatMul_i.forward(rms_norm(x, norm_weight, eps)) with
+ * rms_norm(x) = x * rsqrt(mean(x^2) + eps) * norm_weight (the reference's `try_fused_rms_norm`),
+ * norm_weight `[k]` f32.  For m <= 2 on device buffers this is ONE launch: the decode kernel, whose
+ * workgroups read all of x anyway, quantizes x * norm_weight, sums the squares on the side and
+ * multiplies the finished sums by the row's rsqrt (the activation quantizers are invariant under
+ * a positive scale of their input: the quants stay, the block scale moves).  Against the two
+ * separate calls the results differ by f32 rounding for Q4_K / Q6_K weights (a quant on a rounding
+ * tie may move by one); for Q8_0 weights, whose activation blocks carry an f16 scale, that scale is
+ * rounded before the row's factor is applied instead of after: up to 2^-11 per block, the size of
+ * the rounding the format has anyway.  Other sizes and memory spaces run the norm into scratch and
+ * the plain call after it. */
+int izwi_qmm_forward_normed_f32(const izwi_qmm_weight* w, const float* x, int64_t m, const float* norm_weight,
+                                float eps, float* y, int mem_space, void* stream);
+int izwi_qmm_forward_group_normed_f32(const izwi_qmm_weight* const* weights, int32_t n_weights, const float* x,
+                                      int64_t m, const float* norm_weight, float eps, float* const* ys,
+                                      int mem_space, void* stream);
+int izwi_qmm_forward_gate_up_silu_normed_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
+                                             const float* x, int64_t m, const float* norm_weight, float eps,
+                                             float* h, int mem_space, void* stream);
+
 /* `T::VecDotType::from_float` per row (candle-core k_quants.rs `matmul`):
  * the activation blocks the decode kernel builds on chip, written out in the
  * reference's block layout (BlockQ8_0, 34 B per 32 values, for Q8_0 weights;

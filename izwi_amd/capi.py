@@ -60,6 +60,9 @@ PROTOTYPES = {
     "izwi_qmm_forward_f32": (C.c_int, [_vp, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_group_f32": (C.c_int, [_vp, _i32, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_gate_up_silu_f32": (C.c_int, [_vp, _vp, _vp, _i64, _vp, C.c_int, _vp]),
+    "izwi_qmm_forward_normed_f32": (C.c_int, [_vp, _vp, _i64, _vp, C.c_float, _vp, C.c_int, _vp]),
+    "izwi_qmm_forward_group_normed_f32": (C.c_int, [_vp, _i32, _vp, _i64, _vp, C.c_float, _vp, C.c_int, _vp]),
+    "izwi_qmm_forward_gate_up_silu_normed_f32": (C.c_int, [_vp, _vp, _vp, _i64, _vp, C.c_float, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_bf16": (C.c_int, [_vp, _vp, _i64, _vp, C.c_int, C.c_int, _vp]),
     "izwi_qmm_forward_fused": (C.c_int, [_vp, _vp, C.c_int, _i64, _vp, _vp, C.c_int, C.c_int, _vp]),
     "izwi_qmm_quantize_activations": (C.c_int, [C.c_int, _vp, _i64, _i64, _vp, C.c_int, _vp]),

@@ -13,6 +13,9 @@
 #include <unordered_map>
 #include <vector>
 
+#include <algorithm>
+
+#include "izwi_decode_ops.h"
 #include "izwi_qmm.h"
 #include "qmm_internal.h"
 
@@ -538,9 +541,57 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
     return IZWI_QMM_OK;
 }
 
+} // extern "C"
+
+namespace {
+
+// Scratch a forward call on layout L with m rows may take from the start of the per-stream buffer
+// (quantized activations, or the bf16 copy and the split-k partial tiles): callers that keep data
+// of their own in the same buffer place it behind this many bytes.
+size_t forward_scratch_need(const QmmLayout& L, int64_t m, int n_cus) {
+    const size_t a = qmm_gemv_mfma_workspace_bytes(L, m);
+    const size_t b = ((((size_t)m * L.k * sizeof(uint16_t)) + 255) & ~(size_t)255) + qmm_gemm_workspace_bytes(L, m, n_cus);
+    return ((a > b ? a : b) + 255) & ~(size_t)255;
+}
+
+// rms_norm(x) * norm_weight into the per-stream scratch, behind `keep_free` bytes
+int normed_copy(const izwi_qmm_weight* w, const float* x_dev, int64_t m, const float* norm_weight, float eps,
+                size_t keep_free, size_t extra_behind, hipStream_t stream, float** out) {
+    void* scratch = nullptr;
+    const size_t bytes = (size_t)m * w->layout.k * sizeof(float);
+    HIP_TRY(get_scratch(w->device, stream, keep_free + ((bytes + 255) & ~(size_t)255) + extra_behind, &scratch));
+    float* normed = reinterpret_cast<float*>(static_cast<uint8_t*>(scratch) + keep_free);
+    if (int rc = izwi_rms_norm_f32(x_dev, norm_weight, m, w->layout.k, eps, normed, IZWI_QMM_DEVICE, stream)) return rc;
+    *out = normed;
+    return IZWI_QMM_OK;
+}
+
+int forward_group_impl(const izwi_qmm_weight* const* weights, int32_t n_weights, const float* x, int64_t m,
+                       float* const* ys, int mem_space, void* stream_, const float* norm_weight, float norm_eps);
+
+} // namespace
+
+extern "C" {
+
 int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_weights,
                                const float* x, int64_t m, float* const* ys, int mem_space,
                                void* stream_) {
+    return forward_group_impl(weights, n_weights, x, m, ys, mem_space, stream_, nullptr, 0.0f);
+}
+
+int izwi_qmm_forward_group_normed_f32(const izwi_qmm_weight* const* weights, int32_t n_weights, const float* x,
+                                      int64_t m, const float* norm_weight, float eps, float* const* ys,
+                                      int mem_space, void* stream_) {
+    if (!norm_weight) return fail(IZWI_QMM_ERR_INVALID, "norm_weight is NULL");
+    return forward_group_impl(weights, n_weights, x, m, ys, mem_space, stream_, norm_weight, eps);
+}
+
+} // extern "C"
+
+namespace {
+
+int forward_group_impl(const izwi_qmm_weight* const* weights, int32_t n_weights, const float* x, int64_t m,
+                       float* const* ys, int mem_space, void* stream_, const float* norm_weight, float norm_eps) {
     if (!weights || !ys) return fail(IZWI_QMM_ERR_INVALID, "NULL argument");
     if (n_weights < 1 || n_weights > QMM_MAX_GROUP)
         return fail(IZWI_QMM_ERR_INVALID, "projection group of %d weights (1..%d supported)", n_weights, QMM_MAX_GROUP);
@@ -561,6 +612,39 @@ int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_
     if (m < 0) return fail(IZWI_QMM_ERR_INVALID, "negative m");
     if (m == 0) return IZWI_QMM_OK;
     if (!x) return fail(IZWI_QMM_ERR_INVALID, "x is NULL");
+    if (norm_weight) {
+        hipStream_t stream = (hipStream_t)stream_;
+        const izwi_qmm_weight* w0 = weights[0];
+        // one launch: the decode kernel normalizes while it quantizes (device buffers, one block type, m <= 2)
+        if (mem_space == IZWI_QMM_DEVICE && uniform && m <= 2 && m < mfma_min_m()) {
+            const QmmLayout* layouts[QMM_MAX_GROUP];
+            const void* tiled[QMM_MAX_GROUP];
+            for (int i = 0; i < n_weights; i++) layouts[i] = &weights[i]->layout, tiled[i] = weights[i]->tiled;
+            const QmmNorm norm{norm_weight, norm_eps};
+            ProfileScope prof(w0, stream);
+            hipError_t e = qmm_launch_gemv_multi(layouts, tiled, n_weights, x, m, ys, w0->n_cus, stream, &norm);
+            if (e == hipSuccess) return IZWI_QMM_OK;
+            if (e != hipErrorNotSupported) return fail_hip(e, "grouped decode kernel");
+            (void)hipGetLastError();
+        }
+        // otherwise: the normalized activations into scratch (behind what the projections use of it),
+        // then the plain group call
+        Staged xi, wi, yo[QMM_MAX_GROUP];
+        HIP_TRY(xi.in(x, (size_t)m * w0->layout.k * sizeof(float), mem_space));
+        HIP_TRY(wi.in(norm_weight, (size_t)w0->layout.k * sizeof(float), mem_space));
+        float* ydev[QMM_MAX_GROUP];
+        size_t keep = 0;
+        for (int i = 0; i < n_weights; i++) {
+            HIP_TRY(yo[i].out(ys[i], (size_t)m * weights[i]->layout.n * sizeof(float), mem_space));
+            ydev[i] = (float*)yo[i].dev;
+            keep = std::max(keep, forward_scratch_need(weights[i]->layout, m, weights[i]->n_cus));
+        }
+        float* normed = nullptr;
+        if (int rc = normed_copy(w0, (const float*)xi.dev, m, (const float*)wi.dev, norm_eps, keep, 0, stream, &normed)) return rc;
+        if (int rc = forward_group_impl(weights, n_weights, normed, m, ydev, IZWI_QMM_DEVICE, stream_, nullptr, 0.0f)) return rc;
+        for (int i = 0; i < n_weights; i++) HIP_TRY(yo[i].finish(stream));
+        return IZWI_QMM_OK;
+    }
     // host buffers, mixed types, prefill sizes: one call per projection (same results)
     if (mem_space != IZWI_QMM_DEVICE || !uniform || n_weights == 1 || m > 64) {
         for (int i = 0; i < n_weights; i++)
@@ -609,9 +693,64 @@ int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_
     return IZWI_QMM_OK;
 }
 
+int gate_up_silu_impl(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const float* x, int64_t m, float* h,
+                      int mem_space, void* stream_, const float* norm_weight, float norm_eps);
+
+} // namespace
+
+extern "C" {
+
 int izwi_qmm_forward_gate_up_silu_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
                                       const float* x, int64_t m, float* h, int mem_space,
                                       void* stream_) {
+    return gate_up_silu_impl(gate, up, x, m, h, mem_space, stream_, nullptr, 0.0f);
+}
+
+int izwi_qmm_forward_gate_up_silu_normed_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const float* x,
+                                             int64_t m, const float* norm_weight, float eps, float* h,
+                                             int mem_space, void* stream_) {
+    if (!norm_weight) return fail(IZWI_QMM_ERR_INVALID, "norm_weight is NULL");
+    return gate_up_silu_impl(gate, up, x, m, h, mem_space, stream_, norm_weight, eps);
+}
+
+int izwi_qmm_forward_normed_f32(const izwi_qmm_weight* w, const float* x, int64_t m, const float* norm_weight,
+                                float eps, float* y, int mem_space, void* stream_) {
+    if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    if (!norm_weight) return fail(IZWI_QMM_ERR_INVALID, "norm_weight is NULL");
+    if (int rc = check_space(mem_space)) return rc;
+    const QmmLayout& L = w->layout;
+    if (L.n_stacked != 1) return fail(IZWI_QMM_ERR_INVALID, "forward on an expert stack");
+    if (m < 0) return fail(IZWI_QMM_ERR_INVALID, "negative m");
+    if (m == 0 || L.n == 0) return IZWI_QMM_OK;
+    if (!x || !y) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    hipStream_t stream = (hipStream_t)stream_;
+    if (mem_space == IZWI_QMM_DEVICE && m <= 2 && m < mfma_min_m()) {
+        const QmmNorm norm{norm_weight, eps};
+        ProfileScope prof(w, stream);
+        hipError_t e = qmm_launch_gemv(L, w->tiled, x, m, y, w->n_cus, stream, nullptr, &norm);
+        if (e == hipSuccess) return IZWI_QMM_OK;
+        if (e != hipErrorNotSupported) return fail_hip(e, "decode kernel");
+        (void)hipGetLastError();
+    }
+    Staged xi, wi, yo;
+    HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
+    HIP_TRY(wi.in(norm_weight, (size_t)L.k * sizeof(float), mem_space));
+    HIP_TRY(yo.out(y, (size_t)m * L.n * sizeof(float), mem_space));
+    float* normed = nullptr;
+    if (int rc = normed_copy(w, (const float*)xi.dev, m, (const float*)wi.dev, eps, forward_scratch_need(L, m, w->n_cus), 0,
+                             stream, &normed))
+        return rc;
+    if (int rc = izwi_qmm_forward_f32(w, normed, m, (float*)yo.dev, IZWI_QMM_DEVICE, stream_)) return rc;
+    HIP_TRY(yo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+} // extern "C"
+
+namespace {
+
+int gate_up_silu_impl(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const float* x, int64_t m, float* h,
+                      int mem_space, void* stream_, const float* norm_weight, float norm_eps) {
     if (!gate || !up) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(mem_space)) return rc;
     const QmmLayout& L = gate->layout;
@@ -631,11 +770,26 @@ int izwi_qmm_forward_gate_up_silu_f32(const izwi_qmm_weight* gate, const izwi_qm
     HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
     HIP_TRY(ho.out(h, (size_t)m * L.n * sizeof(float), mem_space));
     if (profiling()) g_silu_fused.fetch_add(1, std::memory_order_relaxed);
+    Staged wi;
+    if (norm_weight) HIP_TRY(wi.in(norm_weight, (size_t)L.k * sizeof(float), mem_space));
+    const float* xin = (const float*)xi.dev;
     if (m < mfma_min_m() && m <= 2 && L.dtype != IZWI_QMM_Q6_K) {
+        const QmmNorm norm{(const float*)wi.dev, norm_eps};
         ProfileScope prof(gate, stream);
-        HIP_TRY(qmm_launch_gemv_gated(L, gate->tiled, up->tiled, (const float*)xi.dev, m, (float*)ho.dev,
-                                      gate->n_cus, stream));
+        HIP_TRY(qmm_launch_gemv_gated(L, gate->tiled, up->tiled, xin, m, (float*)ho.dev, gate->n_cus, stream,
+                                      norm_weight ? &norm : nullptr));
     } else {
+        size_t behind = 0; // bytes of the scratch buffer's start that hold the normalized activations
+        if (norm_weight) {
+            // the normalized activations first (behind what the projections use), the two outputs behind them
+            const size_t keep = forward_scratch_need(L, m, gate->n_cus);
+            float* normed = nullptr;
+            if (int rc = normed_copy(gate, xin, m, (const float*)wi.dev, norm_eps, keep, 2 * (size_t)m * L.n * sizeof(float) + 512,
+                                     stream, &normed))
+                return rc;
+            xin = normed;
+            behind = keep + (((size_t)m * L.k * sizeof(float) + 255) & ~(size_t)255);
+        }
         // both projections into scratch (one projection-group call), then the elementwise product
         const size_t part = (size_t)m * L.n * sizeof(float);
         void* gu = nullptr;
@@ -645,19 +799,23 @@ int izwi_qmm_forward_gate_up_silu_f32(const izwi_qmm_weight* gate, const izwi_qm
             const size_t group_need =
                 m <= 64 ? qmm_gemv_mfma_workspace_bytes(L, m)
                         : ((((size_t)m * L.k * sizeof(uint16_t)) + 255) & ~(size_t)255) + qmm_gemm_workspace_bytes(L, m, gate->n_cus);
-            const size_t base = (group_need + 255) & ~(size_t)255;
+            const size_t base = std::max((group_need + 255) & ~(size_t)255, behind);
             void* scratch = nullptr;
             HIP_TRY(get_scratch(gate->device, stream, base + 2 * part, &scratch));
             gu = static_cast<uint8_t*>(scratch) + base;
         }
         const izwi_qmm_weight* ws[2] = {gate, up};
         float* ys[2] = {static_cast<float*>(gu), reinterpret_cast<float*>(static_cast<uint8_t*>(gu) + part)};
-        if (int rc = izwi_qmm_forward_group_f32(ws, 2, (const float*)xi.dev, m, ys, IZWI_QMM_DEVICE, stream_)) return rc;
+        if (int rc = izwi_qmm_forward_group_f32(ws, 2, xin, m, ys, IZWI_QMM_DEVICE, stream_)) return rc;
         HIP_TRY(qmm_launch_silu_mul(ys[0], ys[1], (float*)ho.dev, (int64_t)m * L.n, stream));
     }
     HIP_TRY(ho.finish(stream));
     return IZWI_QMM_OK;
 }
+
+} // namespace
+
+extern "C" {
 
 int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int64_t m, void* y,
                           int out_dtype, int mem_space, void* stream_) {

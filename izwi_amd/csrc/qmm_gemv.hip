@@ -56,6 +56,13 @@ __device__ __forceinline__ float row16_max(float v) {
     v = fmaxf(v, __int_as_float(dpp<kDppRor8>(__float_as_int(v))));
     return v;
 }
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __int_as_float(dpp<kDppXor1>(__float_as_int(v)));
+    v += __int_as_float(dpp<kDppXor2>(__float_as_int(v)));
+    v += __int_as_float(dpp<kDppRor4>(__float_as_int(v)));
+    v += __int_as_float(dpp<kDppRor8>(__float_as_int(v)));
+    return v;
+}
 __device__ __forceinline__ int row16_min(int v) {
     v = min(v, dpp<kDppXor1>(v));
     v = min(v, dpp<kDppXor2>(v));
@@ -435,6 +442,9 @@ struct GemvParams {
     float* yv[QMM_MAX_GROUP];
     // plain form only: y = sums (+ residual), stored as f32 or bf16 (P.y then points to bf16)
     QmmEpilogue ep;
+    // NORM variants: the activations are RMS-normalized on the way in (weight norm_w[k], eps)
+    const float* norm_w;
+    float norm_eps;
 };
 static_assert(offsetof(GemvParams, k_units) == 64, "first-load fields must fill one 64-byte line");
 
@@ -450,7 +460,11 @@ __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 // entry to the first load.
 // IO: 0 = f32 activations and a plain f32 store; 1 = f32 activations, 2 = bf16 activations, both
 // with the epilogue of P.ep (residual add, f32 or bf16 store).
-template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT, int IO = 0>
+// NORM: x is replaced by rms_norm(x) * norm_w.  The workgroup reads all of x anyway: every 16-lane
+// group adds the squares of its 256 raw values while it quantizes x * norm_w, and because the
+// quantizers are invariant under a positive scale of their input (the quants stay, the block scale
+// moves), the row's factor rsqrt(mean(x^2) + eps) multiplies the finished sums instead.
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT, int IO = 0, bool NORM = false>
 __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int m_end, const uint8_t* w_first,
                                           float* y_out, int n_rows, int row_tiles, int rtg0, uint8_t* smem) {
     constexpr bool XB = IO == 2, EP = IO != 0;
@@ -468,6 +482,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
     const int k_units = (P.k + 255) >> 8, s_units = P.slots >> 4;
     const uint8_t* wbase = stack ? P.w2 + (w_first - P.w) : w_first; // the second stack at the same offset
     const XLds<QT> l = carve<QT, MT>(smem, k_units);
+    float* xss = l.red + 2 * waves * MT * 16; // NORM: [MT][k_units] sums of squares, behind everything else
 
     for (int m0 = m_begin; ONESHOT ? m0 == m_begin : m0 < m_end; m0 += MT) {
         bool x_ready = false;
@@ -499,7 +514,9 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                     float4 f[4];
                     float v[16];
                     const bool in0 = x_item_issue<MT, XB>(xs, group, group < items, f);
-                    if (IO != 0) __builtin_amdgcn_sched_barrier(0); // the activation loads stay in front
+                    float4 fnw[4];
+                    if (NORM) x16_issue<false>(P.norm_w + (group / MT) * 256 + 16 * (threadIdx.x & 15), P.norm_w, in0, fnw);
+                    if (IO != 0 || NORM) __builtin_amdgcn_sched_barrier(0); // the activation loads stay in front
                     load_panel<QT>(p, wbase + off, P.slots, lane0, active);
                     if (EP && ks == 0) {
                         // (the lanes and conditions of the store at the end)
@@ -513,10 +530,22 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                     }
                     if (m0 != m_begin) lds_barrier(); // the previous rows' readers are done
                     x16_finish<XB>(f, in0, v);
+                    // NORM: sum of the raw squares of the item (all 16 lanes of the group), then x * norm_w
+                    auto norm_item = [&](int item, bool in_range, const float4 (&fw)[4]) {
+                        float wv[16], ss = 0.0f;
+                        x16_finish<false>(fw, in_range, wv);
+#pragma unroll
+                        for (int i = 0; i < 16; i++) ss += v[i] * v[i], v[i] *= wv[i];
+                        ss = row16_sum(ss);
+                        if ((threadIdx.x & 15) == 0) xss[(item % MT) * k_units + item / MT] = ss;
+                    };
+                    if (NORM && group < items) norm_item(group, in0, fnw);
                     if (group < items) x_item_quantize<QT, MT>(l, k_units, group, v);
                     for (int item = group + n_groups; item < items; item += n_groups) {
                         const bool in1 = x_item_issue<MT, XB>(xs, item, true, f);
+                        if (NORM) x16_issue<false>(P.norm_w + (item / MT) * 256 + 16 * (threadIdx.x & 15), P.norm_w, in1, fnw);
                         x16_finish<XB>(f, in1, v);
+                        if (NORM) norm_item(item, in1, fnw);
                         x_item_quantize<QT, MT>(l, k_units, item, v);
                     }
                     // One row, one row-tile per workgroup, four units per panel: wave wk has just
@@ -549,6 +578,11 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                     for (int mi = 0; mi < MT; mi++) {
                         if (m0 + mi < m_end) {
                             int64_t yr = GROUPED ? P.perm[m0 + mi] : m0 + mi;
+                            if (NORM) {
+                                float ssq = 0.0f;
+                                for (int u = 0; u < k_units; u++) ssq += xss[mi * k_units + u];
+                                acc[mi] *= 1.0f / sqrtf(ssq / (float)P.k + P.norm_eps);
+                            }
                             if (EP) qmm_store(y_out, P.ep, yr * n_rows + row, acc[mi]);
                             else y_out[yr * n_rows + row] = acc[mi];
                         }
@@ -569,6 +603,13 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                         if (GATED) sum2 += red[((stack_waves + wr * P.nwk + w2) * MT + mi) * 16 + r];
                     }
                     const int row = rt * 16 + r;
+                    if (NORM) {
+                        float ssq = 0.0f;
+                        for (int u = 0; u < k_units; u++) ssq += xss[mi * k_units + u];
+                        const float ns = 1.0f / sqrtf(ssq / (float)P.k + P.norm_eps);
+                        sum *= ns;
+                        sum2 *= ns;
+                    }
                     if (rt < row_tiles && row < n_rows && m0 + mi < m_end) {
                         int64_t yr = GROUPED ? P.perm[m0 + mi] : m0 + mi;
                         if (EP) {
@@ -594,9 +635,9 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
 // whether it exists or not.
 // The dense straight-line single-row Q4_K form is held to 80 registers: six waves per SIMD,
 // i.e. two 12-wave workgroups per CU.
-template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false, int IO = 0>
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false, int IO = 0, bool NORM = false>
 __global__ __launch_bounds__(64 * kMaxWaves)
-__attribute__((amdgpu_waves_per_eu((ONESHOT && !GROUPED && MT == 1 && QT == QMM_Q4_K) ? 6 : 3))) void gemv_kernel(GemvParams P) {
+__attribute__((amdgpu_waves_per_eu(NORM ? 4 : (ONESHOT && !GROUPED && MT == 1 && QT == QMM_Q4_K) ? 6 : 3))) void gemv_kernel(GemvParams P) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int m_begin = 0, m_end = P.m;
     int64_t w_offset = 0;
@@ -629,7 +670,7 @@ __attribute__((amdgpu_waves_per_eu((ONESHOT && !GROUPED && MT == 1 && QT == QMM_
         else
             gemv_body<QT, 4, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     } else {
-        gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
+        gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO, NORM>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     }
 }
 
@@ -665,10 +706,10 @@ void choose_split(const QmmLayout& L, int n_cus, int grid_y, bool gated, GemvPar
     P.wave_magic = (65536 + nwk - 1) / nwk;
 }
 
-template <int QT, int MT, bool GATED, bool GROUPED, int IO = 0>
+template <int QT, int MT, bool GATED, bool GROUPED, int IO = 0, bool NORM = false>
 hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipStream_t stream) {
     const int all_waves = GATED ? 2 * waves : waves;
-    size_t lds = lds_bytes<QT, MT>(P.k_units, all_waves);
+    size_t lds = lds_bytes<QT, MT>(P.k_units, all_waves) + (NORM ? (size_t)MT * P.k_units * sizeof(float) : 0);
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     int64_t cap = (int64_t)n_cus * 32;
     if (grid_y > 1) cap = cap / grid_y > 64 ? cap / grid_y : 64;
@@ -678,22 +719,29 @@ hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipS
     // grouped form), one row-tile group per workgroup, one k step
     constexpr bool kCanOneshot = GROUPED ? MT == QMM_MOE_SEG_ROWS : true;
     const bool oneshot = kCanOneshot && (GROUPED || P.m <= MT) && P.kpw == 1 && grid == P.rt_groups;
-    const void* fn = oneshot ? reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot, IO>)
-                             : reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, false, IO>);
+    const void* fn = oneshot ? reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot, IO, NORM>)
+                             : reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, false, IO, NORM>);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
     const dim3 g((unsigned)grid, (unsigned)grid_y), b(64 * all_waves);
     if (oneshot)
-        gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot, IO><<<g, b, lds, stream>>>(P);
+        gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot, IO, NORM><<<g, b, lds, stream>>>(P);
     else
-        gemv_kernel<QT, MT, GATED, GROUPED, false, IO><<<g, b, lds, stream>>>(P);
+        gemv_kernel<QT, MT, GATED, GROUPED, false, IO, NORM><<<g, b, lds, stream>>>(P);
     return hipGetLastError();
 }
 
 template <int QT>
 hipError_t launch_plain(const GemvParams& P, int waves, int n_cus, int io, hipStream_t stream) {
+    if (P.norm_w != nullptr) { // folded RMSNorm: f32 activations, plain store, one or two rows
+        if (io != 0 || P.m > 2) return hipErrorNotSupported;
+        if (P.m == 2 && lds_bytes<QT, 2>(P.k_units, waves) <= 64 * 1024)
+            return launch_mt<QT, 2, false, false, 0, true>(P, waves, n_cus, 1, stream);
+        if (P.m == 2) return hipErrorNotSupported;
+        return launch_mt<QT, 1, false, false, 0, true>(P, waves, n_cus, 1, stream);
+    }
     // the widest row tile whose quantized activations fit comfortably in LDS
     int mt = P.m >= 3 ? 4 : (P.m == 2 ? 2 : 1);
     if (mt == 4 && lds_bytes<QT, 4>(P.k_units, waves) > 64 * 1024) mt = 2;
@@ -742,6 +790,8 @@ bool make_params(const QmmLayout& L, const void* tiled, const float* x, int64_t 
     P.n_weights = 0;
     P.ep.residual = nullptr;
     P.ep.y_bf16 = 0;
+    P.norm_w = nullptr;
+    P.norm_eps = 0.0f;
     return true;
 }
 
@@ -795,10 +845,11 @@ __global__ void quantize_export_kernel(const float* __restrict__ x, int64_t m, i
 } // namespace
 
 hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
-                           float* y, int n_cus, hipStream_t stream, const QmmIo* io) {
+                           float* y, int n_cus, hipStream_t stream, const QmmIo* io, const QmmNorm* norm) {
     if (m <= 0 || L.n == 0) return hipSuccess;
     GemvParams P;
     if (!make_params(L, tiled, x, m, y, P)) return hipErrorInvalidValue;
+    if (norm) P.norm_w = norm->weight, P.norm_eps = norm->eps;
     // kernel variant: plain, or with the epilogue (and f32 / bf16 activations)
     const int iom = !io ? 0 : (io->x_bf16 ? 2 : (io->residual || io->y_bf16 ? 1 : 0));
     if (io) P.ep = QmmEpilogue{io->residual, io->y_bf16};
@@ -829,7 +880,8 @@ hipError_t qmm_launch_silu_mul(const float* gate, const float* up, float* out, i
 }
 
 hipError_t qmm_launch_gemv_gated(const QmmLayout& L, const void* tiled_gate, const void* tiled_up,
-                                 const float* x, int64_t m, float* y, int n_cus, hipStream_t stream) {
+                                 const float* x, int64_t m, float* y, int n_cus, hipStream_t stream,
+                                 const QmmNorm* norm) {
     if (m <= 0 || L.n == 0) return hipSuccess;
     if (m > 2 || L.dtype == QMM_Q6_K) return hipErrorNotSupported;
     GemvParams P;
@@ -837,6 +889,14 @@ hipError_t qmm_launch_gemv_gated(const QmmLayout& L, const void* tiled_gate, con
     P.w2 = (const uint8_t*)tiled_up;
     int waves;
     choose_split(L, n_cus, 1, true, P, waves);
+    if (norm) {
+        P.norm_w = norm->weight, P.norm_eps = norm->eps;
+        if (L.dtype == QMM_Q4_K)
+            return m == 2 ? launch_mt<QMM_Q4_K, 2, true, false, 0, true>(P, waves, n_cus, 1, stream)
+                          : launch_mt<QMM_Q4_K, 1, true, false, 0, true>(P, waves, n_cus, 1, stream);
+        return m == 2 ? launch_mt<QMM_Q8_0, 2, true, false, 0, true>(P, waves, n_cus, 1, stream)
+                      : launch_mt<QMM_Q8_0, 1, true, false, 0, true>(P, waves, n_cus, 1, stream);
+    }
     if (L.dtype == QMM_Q4_K)
         return m == 2 ? launch_mt<QMM_Q4_K, 2, true, false>(P, waves, n_cus, 1, stream)
                       : launch_mt<QMM_Q4_K, 1, true, false>(P, waves, n_cus, 1, stream);
@@ -846,7 +906,7 @@ hipError_t qmm_launch_gemv_gated(const QmmLayout& L, const void* tiled_gate, con
 
 hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
                                  const float* x, int64_t m, float* const* ys, int n_cus,
-                                 hipStream_t stream) {
+                                 hipStream_t stream, const QmmNorm* norm) {
     if (n_weights < 1 || n_weights > QMM_MAX_GROUP || m < 1 || m > 2) return hipErrorInvalidValue;
     const QmmLayout& L0 = *layouts[0];
     int64_t total_row_tiles = 0;
@@ -881,9 +941,23 @@ hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* co
     const int mt = m == 2 ? 2 : 1;
     const size_t lds = mt == 2 ? lds_bytes<QMM_Q4_K, 2>(P.k_units, waves) : lds_bytes<QMM_Q4_K, 1>(P.k_units, waves);
     const size_t lds8 = mt == 2 ? lds_bytes<QMM_Q8_0, 2>(P.k_units, waves) : lds_bytes<QMM_Q8_0, 1>(P.k_units, waves);
-    const size_t need = L0.dtype == QMM_Q4_K ? lds : lds8;
+    size_t need = L0.dtype == QMM_Q4_K ? lds : lds8;
+    if (norm) {
+        P.norm_w = norm->weight, P.norm_eps = norm->eps;
+        need += (size_t)mt * P.k_units * sizeof(float);
+    }
     if (need > 48 * 1024) return hipErrorNotSupported;
     const dim3 g((unsigned)groups), b(64 * waves);
+    if (norm) {
+        if (L0.dtype == QMM_Q4_K) {
+            if (mt == 2) gemv_kernel<QMM_Q4_K, 2, false, false, true, 0, true><<<g, b, need, stream>>>(P);
+            else gemv_kernel<QMM_Q4_K, 1, false, false, true, 0, true><<<g, b, need, stream>>>(P);
+        } else {
+            if (mt == 2) gemv_kernel<QMM_Q8_0, 2, false, false, true, 0, true><<<g, b, need, stream>>>(P);
+            else gemv_kernel<QMM_Q8_0, 1, false, false, true, 0, true><<<g, b, need, stream>>>(P);
+        }
+        return hipGetLastError();
+    }
     if (L0.dtype == QMM_Q4_K) {
         if (mt == 2) gemv_kernel<QMM_Q4_K, 2, false, false, true><<<g, b, need, stream>>>(P);
         else gemv_kernel<QMM_Q4_K, 1, false, false, true><<<g, b, need, stream>>>(P);

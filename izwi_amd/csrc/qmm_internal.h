@@ -67,6 +67,13 @@ struct QmmEpilogue {
     const void* residual;
     int y_bf16;
 };
+// RMSNorm folded into a decode kernel (m <= 2): the kernel reads x, multiplies by weight[k] and
+// applies rsqrt(mean(x^2) + eps) to the finished sums (the activation quantizers are invariant
+// under a positive scale of their input).
+struct QmmNorm {
+    const float* weight;
+    float eps;
+};
 
 #if defined(__HIPCC__)
 __device__ __forceinline__ void qmm_store(void* y, const QmmEpilogue& ep, int64_t idx, float v) {
@@ -102,13 +109,15 @@ hipError_t qmm_launch_dequant(const QmmLayout& L, const void* tiled, float* out,
 // With `io`: x and y are of the types it names (bf16 activations: m <= 2 only,
 // hipErrorNotSupported beyond).
 hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
-                           float* y, int n_cus, hipStream_t stream, const QmmIo* io = nullptr);
+                           float* y, int n_cus, hipStream_t stream, const QmmIo* io = nullptr,
+                           const QmmNorm* norm = nullptr);
 
 // Decode kernel for the gate / up pair of an MLP: y[m, n] = silu(W_gate x) * (W_up x), both
 // matrices of layout L, m <= 2 (hipErrorNotSupported beyond).  The sums are those of
 // qmm_launch_gemv; the product is applied where the waves that split k are combined.
 hipError_t qmm_launch_gemv_gated(const QmmLayout& L, const void* tiled_gate, const void* tiled_up,
-                                 const float* x, int64_t m, float* y, int n_cus, hipStream_t stream);
+                                 const float* x, int64_t m, float* y, int n_cus, hipStream_t stream,
+                                 const QmmNorm* norm = nullptr);
 // out[i] = silu(gate[i]) * up[i]
 hipError_t qmm_launch_silu_mul(const float* gate, const float* up, float* out, int64_t count,
                                hipStream_t stream);
@@ -152,7 +161,7 @@ hipError_t qmm_launch_f32_to_bf16(const float* x, uint16_t* out, int64_t count,
 #define QMM_MAX_GROUP 4
 hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
                                  const float* x, int64_t m, float* const* ys, int n_cus,
-                                 hipStream_t stream);
+                                 hipStream_t stream, const QmmNorm* norm = nullptr);
 
 // The same for 3 <= m <= 16 on the matrix cores: `workspace` holds the activations already
 // quantized (qmm_launch_quantize_ws), all weights read the same records in one launch.

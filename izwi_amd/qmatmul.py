@@ -163,6 +163,17 @@ class QMatMul:
             return y
         raise capi.QmmError(-1, f"unsupported dtype {x.dtype} for qmatmul, expected f32 or bf16")
 
+    def forward_normed(self, x: torch.Tensor, norm_weight: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+        """forward(rms_norm(x, norm_weight, eps)) in one call (the final norm in front of the LM head)."""
+        n, k = self.qtensor.dims2()
+        if x.dtype != torch.float32 or x.dim() < 1 or x.shape[-1] != k or not x.is_contiguous():
+            raise capi.QmmError(-1, f"expected a contiguous f32 input with last dim {k}")
+        assert norm_weight.dtype == torch.float32 and norm_weight.is_contiguous() and norm_weight.numel() == k
+        y = torch.empty(tuple(x.shape[:-1]) + (n,), dtype=torch.float32, device=x.device)
+        check(lib().izwi_qmm_forward_normed_f32(self.qtensor._h, x.data_ptr(), x.numel() // k if k else 0,
+                                                norm_weight.data_ptr(), eps, y.data_ptr(), _space(x), _stream_ptr(x)))
+        return y
+
     def forward_fused(self, x: torch.Tensor, residual: torch.Tensor | None = None,
                       out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
         """Qwen3Projection::forward (qwen3/core.rs:795-829) plus the layer's residual add
@@ -256,10 +267,13 @@ class Qwen3Projection:
         return self.qmatmul.forward(x.to(torch.float32)).to(x.dtype)
 
 
-def forward_group(projections: Sequence["QMatMul"], x: torch.Tensor):
+def forward_group(projections: Sequence["QMatMul"], x: torch.Tensor, norm_weight: torch.Tensor | None = None,
+                  eps: float = 1e-6):
     """Several projections on the same activations in one call (the `Separate` arms of
     Qwen3QkvProjection::forward / Qwen3GateUpProjection::forward, qwen3/core.rs:1119-1127,
-    1274-1282).  Returns one output per projection, identical to separate forwards."""
+    1274-1282).  Returns one output per projection, identical to separate forwards.
+    With ``norm_weight`` the projections see rms_norm(x, norm_weight, eps) (the layer norm in front of
+    them, core.rs:1872), folded into the same launch for one or two rows."""
     assert x.dtype == torch.float32 and x.is_contiguous()
     k = x.shape[-1]
     m = x.numel() // k if k else 0
@@ -268,7 +282,12 @@ def forward_group(projections: Sequence["QMatMul"], x: torch.Tensor):
           for p in projections]
     handles = (C.c_void_p * n)(*[p.qtensor._h for p in projections])
     outs = (C.c_void_p * n)(*[y.data_ptr() for y in ys])
-    check(lib().izwi_qmm_forward_group_f32(handles, n, x.data_ptr(), m, outs, _space(x), _stream_ptr(x)))
+    if norm_weight is not None:
+        assert norm_weight.dtype == torch.float32 and norm_weight.is_contiguous() and norm_weight.numel() == k
+        check(lib().izwi_qmm_forward_group_normed_f32(handles, n, x.data_ptr(), m, norm_weight.data_ptr(), eps, outs,
+                                                      _space(x), _stream_ptr(x)))
+    else:
+        check(lib().izwi_qmm_forward_group_f32(handles, n, x.data_ptr(), m, outs, _space(x), _stream_ptr(x)))
     return tuple(ys)
 
 
@@ -306,10 +325,12 @@ class Qwen3GateUpProjection(Qwen3QkvProjection):
     def new_separate(cls, gate_proj: "QMatMul", up_proj: "QMatMul"):  # noqa: D102
         return cls(parts=(gate_proj, up_proj))
 
-    def forward_silu_mul(self, x: torch.Tensor) -> torch.Tensor:
+    def forward_silu_mul(self, x: torch.Tensor, norm_weight: torch.Tensor | None = None, eps: float = 1e-6) -> torch.Tensor:
         """`forward(x)` followed by `try_fused_silu_mul(gate, up)` (qwen3/core.rs:1786-1796,
-        kernels/mod.rs:94-108) in one call: silu(gate x) * (up x)."""
+        kernels/mod.rs:94-108) in one call: silu(gate x) * (up x).  With ``norm_weight`` x is replaced by
+        rms_norm(x, norm_weight, eps) (post_attention_layernorm, core.rs:1877) in the same call."""
         if self._fused is not None:
+            assert norm_weight is None
             gate, up = self.forward(x)
             return torch.nn.functional.silu(gate) * up
         gate_proj, up_proj = self._parts
@@ -319,8 +340,14 @@ class Qwen3GateUpProjection(Qwen3QkvProjection):
             raise capi.QmmError(-1, f"shape mismatch in qmatmul, lhs: {tuple(x.shape)}, rhs: ({n}, {k})")
         m = x.numel() // k if k else 0
         h = torch.empty(tuple(x.shape[:-1]) + (n,), dtype=torch.float32, device=x.device)
-        check(lib().izwi_qmm_forward_gate_up_silu_f32(gate_proj.qtensor._h, up_proj.qtensor._h, x.data_ptr(), m,
-                                                      h.data_ptr(), _space(x), _stream_ptr(x)))
+        if norm_weight is not None:
+            assert norm_weight.dtype == torch.float32 and norm_weight.is_contiguous() and norm_weight.numel() == k
+            check(lib().izwi_qmm_forward_gate_up_silu_normed_f32(gate_proj.qtensor._h, up_proj.qtensor._h, x.data_ptr(), m,
+                                                                 norm_weight.data_ptr(), eps, h.data_ptr(), _space(x),
+                                                                 _stream_ptr(x)))
+        else:
+            check(lib().izwi_qmm_forward_gate_up_silu_f32(gate_proj.qtensor._h, up_proj.qtensor._h, x.data_ptr(), m,
+                                                          h.data_ptr(), _space(x), _stream_ptr(x)))
         return h
 
 

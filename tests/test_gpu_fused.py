@@ -136,3 +136,58 @@ def test_fused_host_memory_profile_counters_and_errors(qa, oracle):
         mm.forward_fused(xd, residual=torch.zeros(m, n + 1, device="cuda"))
     with pytest.raises(capi.QmmError):
         mm.forward_fused(xd, residual=torch.zeros(m, n, device="cuda", dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize("dtype", [Q4_K, Q8_0, Q6_K])
+@pytest.mark.parametrize("m", [1, 2, 3, 16, 80])
+def test_rms_norm_folded_into_the_projection_calls(qa, oracle, dtype, m):
+    """forward_normed / forward_group(norm_weight=) / forward_silu_mul(norm_weight=) against the norm
+    call followed by the plain call.  For m <= 2 the decode kernel does the norm itself (scale-invariance
+    of the quantizers): results agree to f32 rounding; beyond, the library runs the two steps itself."""
+    k, n1, n2 = 1024, 528, 272
+    a, b = make_qmatmul(qa, oracle, dtype, n1, k, 21), make_qmatmul(qa, oracle, dtype, n2, k, 22)
+    g, u = make_qmatmul(qa, oracle, dtype, n1, k, 23), make_qmatmul(qa, oracle, dtype, n1, k, 24)
+    x = torch.from_numpy(oracle.randn(50 + m, (m, k)) * 3.0).cuda()
+    w = torch.from_numpy(oracle.randn(7, (k,), mean=1.0, std=0.2)).cuda()
+    normed = qa.try_fused_rms_norm(x, w, 1e-6)
+
+    # Q8_0 rounds the activation blocks' scales to f16: folded, that rounding happens before the row's
+    # factor is applied instead of after it, a difference of up to 2^-11 per block
+    tol = 1.5e-3 if dtype == Q8_0 else 2e-4
+
+    def near(got, want):
+        return float((got - want).abs().max()) <= tol * float(want.abs().max())
+    assert near(a.forward_normed(x, w, 1e-6), a.forward(normed))
+    ya, yb = qa.forward_group([a, b], x, norm_weight=w, eps=1e-6)
+    assert near(ya, a.forward(normed)) and near(yb, b.forward(normed))
+    gu = qa.Qwen3GateUpProjection.new_separate(g, u)
+    assert near(gu.forward_silu_mul(x, norm_weight=w, eps=1e-6), gu.forward_silu_mul(normed))
+    # against the oracle's composition, where the library multiplies in integers as the oracle does
+    # (80 rows take the prefill kernel, which has its own, wider, bound)
+    xn = oracle.rms_norm(x.cpu().numpy(), w.cpu().numpy(), 1e-6)
+    if dtype != Q6_K and m <= 16:
+        want = oracle.qmatmul(dtype, xn, a.qtensor.data(), n1)
+        got = a.forward_normed(x, w, 1e-6).cpu().numpy()
+        assert np.abs(got - want).max() <= (tol + 1e-4) * np.abs(want).max()
+
+
+def test_rms_norm_folded_8b_shapes_host_space_and_errors(qa, oracle):
+    from izwi_amd import capi
+    q = make_qmatmul(qa, oracle, Q4_K, 4096, 4096, 31)
+    kk = make_qmatmul(qa, oracle, Q4_K, 1024, 4096, 32)
+    v = make_qmatmul(qa, oracle, Q4_K, 1024, 4096, 33)
+    x = torch.from_numpy(oracle.randn(60, (1, 4096))).cuda()
+    w = torch.from_numpy(oracle.randn(8, (4096,), mean=1.0, std=0.1)).cuda()
+    normed = qa.try_fused_rms_norm(x, w, 1e-6)
+    for got, mm in zip(qa.forward_group([q, kk, v], x, norm_weight=w), (q, kk, v)):
+        want = mm.forward(normed)
+        assert float((got - want).abs().max()) <= 2e-4 * float(want.abs().max())
+    head = make_qmatmul(qa, oracle, Q4_K, 40000, 4096, 34)  # tall: the looped form of the kernel
+    want = head.forward(normed)
+    assert float((head.forward_normed(x, w) - want).abs().max()) <= 2e-4 * float(want.abs().max())
+    # host pointers: staged, same values
+    got = q.forward_normed(x.cpu(), w.cpu())
+    assert float((got.cuda() - q.forward(normed)).abs().max()) <= 2e-4 * float(want.abs().max())
+    L = capi.lib()
+    y = torch.empty(1, 4096, device="cuda")
+    assert L.izwi_qmm_forward_normed_f32(q.qtensor._h, x.data_ptr(), 1, None, 1e-6, y.data_ptr(), capi.DEVICE, None) == -1
