@@ -23,6 +23,7 @@
 #include <utility>
 #include <vector>
 
+#include "izwi_decode_ops.h"
 #include "izwi_gguf.h"
 #include "izwi_qmm.h"
 
@@ -156,6 +157,20 @@ public:
         check(izwi_qmm_forward_bf16(q_->handle(), x, m, y, out_bf16 ? IZWI_QMM_OUT_BF16 : IZWI_QMM_OUT_F32,
                                     (int)space, stream));
     }
+    // The whole `Quantized` arm of `Qwen3Projection::forward` (core.rs:795-829) plus the residual add
+    // that follows o_proj / down_proj (core.rs:1875, 1879) in one call: x is f32 or bf16 (`x_bf16`),
+    // y = x W^T + residual stored as f32 or bf16 (`y_bf16`); residual has y's type, may be y, may be null.
+    void forward_fused(const void* x, bool x_bf16, int64_t m, const void* residual, void* y, bool y_bf16,
+                       MemSpace space, void* stream = nullptr) const {
+        check(izwi_qmm_forward_fused(q_->handle(), x, x_bf16 ? IZWI_QMM_OUT_BF16 : IZWI_QMM_OUT_F32, m, residual, y,
+                                     y_bf16 ? IZWI_QMM_OUT_BF16 : IZWI_QMM_OUT_F32, (int)space, stream));
+    }
+    // RMSNorm (weight `norm_weight` [k], `eps`) of x and the projection of the result, as one call
+    // (the final norm + lm_head, core.rs:1690-1702).
+    void forward_normed(const float* x, int64_t m, const float* norm_weight, float eps, float* y, MemSpace space,
+                        void* stream = nullptr) const {
+        check(izwi_qmm_forward_normed_f32(q_->handle(), x, m, norm_weight, eps, y, (int)space, stream));
+    }
     const std::shared_ptr<QTensor>& qtensor() const { return q_; }
     int64_t out_features() const { return q_->rows(); }
     int64_t in_features() const { return q_->cols(); }
@@ -198,6 +213,60 @@ inline void forward_group(const std::vector<const QMatMul*>& projections, const 
     for (const QMatMul* p : projections) handles.push_back(p->qtensor()->handle());
     check(izwi_qmm_forward_group_f32(handles.data(), (int32_t)handles.size(), x, m, ys.data(), (int)space, stream));
 }
+
+// The same with the RMSNorm that precedes the group folded in (input_layernorm + q / k / v,
+// core.rs:1866, 1455-1462): x is the un-normed hidden state.
+inline void forward_group_normed(const std::vector<const QMatMul*>& projections, const float* x, int64_t m,
+                                 const float* norm_weight, float eps, const std::vector<float*>& ys, MemSpace space,
+                                 void* stream = nullptr) {
+    std::vector<const izwi_qmm_weight*> handles;
+    for (const QMatMul* p : projections) handles.push_back(p->qtensor()->handle());
+    check(izwi_qmm_forward_group_normed_f32(handles.data(), (int32_t)handles.size(), x, m, norm_weight, eps, ys.data(),
+                                            (int)space, stream));
+}
+
+// `Qwen3GateUpProjection::forward_silu_mul` (core.rs:1250-1300), `Separate` arm: h = silu(x Wg^T) * (x Wu^T),
+// [m, intermediate]; with `norm_weight` the post-attention RMSNorm of x is folded in (core.rs:1877).
+inline void forward_gate_up_silu(const QMatMul& gate, const QMatMul& up, const float* x, int64_t m, float* h,
+                                 MemSpace space, void* stream = nullptr, const float* norm_weight = nullptr,
+                                 float eps = 1e-6f) {
+    if (norm_weight)
+        check(izwi_qmm_forward_gate_up_silu_normed_f32(gate.qtensor()->handle(), up.qtensor()->handle(), x, m,
+                                                       norm_weight, eps, h, (int)space, stream));
+    else
+        check(izwi_qmm_forward_gate_up_silu_f32(gate.qtensor()->handle(), up.qtensor()->handle(), x, m, h, (int)space,
+                                                stream));
+}
+
+// The fused-kernel hooks of crates/izwi-core/src/kernels/mod.rs:109-225, f32 arm.  The reference's
+// hooks return None where no kernel applies; these throw izwi::Error where the library refuses.
+namespace kernels {
+inline void rms_norm(const float* x, const float* weight, int64_t rows, int64_t hidden, float eps, float* y,
+                     MemSpace space, void* stream = nullptr) {
+    check(izwi_rms_norm_f32(x, weight, rows, hidden, eps, y, (int)space, stream));
+}
+inline void qk_rms_norm(const float* q, const float* k, const float* qk_weight, int64_t q_rows, int64_t k_rows,
+                        int64_t head_dim, float eps, float* q_out, float* k_out, MemSpace space,
+                        void* stream = nullptr) {
+    check(izwi_qk_rms_norm_f32(q, k, qk_weight, q_rows, k_rows, head_dim, eps, q_out, k_out, (int)space, stream));
+}
+inline void rope_pair_bshd(const float* q, const float* k, const float* cos_sin, int64_t batch, int64_t seq,
+                           int64_t q_heads, int64_t k_heads, int64_t head_dim, float* q_out, float* k_out,
+                           MemSpace space, void* stream = nullptr) {
+    check(izwi_rope_pair_bshd_f32(q, k, cos_sin, batch, seq, q_heads, k_heads, head_dim, q_out, k_out, (int)space,
+                                  stream));
+}
+inline void decode_gqa_attention(const float* q, const float* k, const float* v, int64_t num_heads,
+                                 int64_t num_kv_heads, int64_t head_dim, int64_t kv_len, int64_t kv_capacity,
+                                 float scale, float* out, MemSpace space, void* stream = nullptr) {
+    check(izwi_decode_gqa_attention_f32(q, k, v, num_heads, num_kv_heads, head_dim, kv_len, kv_capacity, scale, out,
+                                        (int)space, stream));
+}
+inline void argmax(const float* logits, int64_t rows, int64_t n, uint32_t* out, MemSpace space,
+                   void* stream = nullptr) {
+    check(izwi_argmax_f32(logits, rows, n, out, (int)space, stream));
+}
+} // namespace kernels
 
 // `Qwen3Projection` (quantized arm): the op always receives f32 activations and
 // returns f32 (core.rs:772-831); callers with other activation dtypes cast around it.

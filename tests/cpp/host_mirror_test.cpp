@@ -4,7 +4,8 @@
 //                          container parse of tests/golden/tiny.gguf
 //   host_mirror_test gpu   the reference's packed-projection test
 //                          (crates/izwi-core/src/models/architectures/qwen3/core.rs:3099-3142)
-//                          and a Q4_K projection, checked against the CPU oracle
+//                          and a Q4_K projection, the folded calls (norm, activation,
+//                          residual) and the hooks' namespace, checked against the CPU oracle
 // Test infrastructure: links the oracle (liboracle_qmm.so) as the checker.
 #include <cmath>
 #include <cstdio>
@@ -19,6 +20,8 @@ int oracle_qmatmul(int dtype, int64_t m, int64_t k, int64_t n, const float* lhs,
 int oracle_quantize(int dtype, int64_t rows, int64_t cols, const float* src, void* dst);
 int64_t oracle_storage_bytes(int dtype, int64_t rows, int64_t cols);
 void oracle_fill_normal(uint64_t seed, int64_t offset, int64_t count, float mean, float std, float* out);
+void oracle_rms_norm(const float* x, const float* weight, int64_t rows, int64_t hidden, float eps, float* y);
+void oracle_argmax(const float* x, int64_t rows, int64_t n, uint32_t* out);
 }
 
 static int failures = 0;
@@ -123,6 +126,54 @@ static void q4k_projection_matches_oracle() {
     EXPECT(max_rel(y, want) < 1e-4f);
 }
 
+// The folded calls of a decode step through the mirror, host pointers: the norm inside the
+// projection, the activation inside gate/up, the residual inside down, the greedy argmax.
+static void folded_calls_match_oracle() {
+    using izwi::GgmlDType;
+    using izwi::MemSpace;
+    const int64_t hidden = 512, inter = 768, m = 1;
+    std::vector<float> wg((size_t)inter * hidden), wu(wg.size()), wd((size_t)hidden * inter), x((size_t)m * hidden),
+        nw((size_t)hidden);
+    oracle_fill_normal(21, 0, (int64_t)wg.size(), 0.0f, 0.05f, wg.data());
+    oracle_fill_normal(22, 0, (int64_t)wu.size(), 0.0f, 0.05f, wu.data());
+    oracle_fill_normal(23, 0, (int64_t)wd.size(), 0.0f, 0.05f, wd.data());
+    oracle_fill_normal(24, 0, (int64_t)x.size(), 0.0f, 2.0f, x.data());
+    oracle_fill_normal(25, 0, (int64_t)nw.size(), 1.0f, 0.1f, nw.data());
+    auto bg = quantize(GgmlDType::Q4K, wg, inter, hidden), bu = quantize(GgmlDType::Q4K, wu, inter, hidden),
+         bd = quantize(GgmlDType::Q4K, wd, hidden, inter);
+    auto gate = izwi::QMatMul::from_arc(izwi::QTensor::from_blocks(GgmlDType::Q4K, bg.data(), bg.size(), inter, hidden));
+    auto up = izwi::QMatMul::from_arc(izwi::QTensor::from_blocks(GgmlDType::Q4K, bu.data(), bu.size(), inter, hidden));
+    auto down = izwi::QMatMul::from_arc(izwi::QTensor::from_blocks(GgmlDType::Q4K, bd.data(), bd.size(), hidden, inter));
+
+    // the oracle's composition: norm, two products, silu(g) * u, product, + x
+    std::vector<float> xn(x.size()), g((size_t)m * inter), u(g.size()), h(g.size()), want((size_t)m * hidden);
+    oracle_rms_norm(x.data(), nw.data(), m, hidden, 1e-6f, xn.data());
+    EXPECT(oracle_qmatmul((int)GgmlDType::Q4K, m, hidden, inter, xn.data(), bg.data(), g.data()) == 0);
+    EXPECT(oracle_qmatmul((int)GgmlDType::Q4K, m, hidden, inter, xn.data(), bu.data(), u.data()) == 0);
+    for (size_t i = 0; i < h.size(); i++) h[i] = g[i] / (1.0f + std::exp(-g[i])) * u[i];
+    EXPECT(oracle_qmatmul((int)GgmlDType::Q4K, m, inter, hidden, h.data(), bd.data(), want.data()) == 0);
+    for (size_t i = 0; i < want.size(); i++) want[i] += x[i];
+
+    std::vector<float> got_n(xn.size()), got_g(g.size()), got_h(h.size()), got((size_t)m * hidden);
+    izwi::kernels::rms_norm(x.data(), nw.data(), m, hidden, 1e-6f, got_n.data(), MemSpace::Host);
+    EXPECT(max_rel(got_n, xn) < 1e-5f);
+    gate.forward_normed(x.data(), m, nw.data(), 1e-6f, got_g.data(), MemSpace::Host);
+    EXPECT(max_rel(got_g, g) < 3e-4f);
+    izwi::forward_gate_up_silu(gate, up, x.data(), m, got_h.data(), MemSpace::Host, nullptr, nw.data(), 1e-6f);
+    EXPECT(max_rel(got_h, h) < 3e-4f);
+    down.forward_fused(got_h.data(), false, m, x.data(), got.data(), false, MemSpace::Host);
+    EXPECT(max_rel(got, want) < 1e-3f);
+    std::vector<float*> ys = {got_g.data(), got_h.data()};
+    izwi::forward_group_normed({&gate, &up}, x.data(), m, nw.data(), 1e-6f, ys, MemSpace::Host);
+    EXPECT(max_rel(got_g, g) < 3e-4f && max_rel(got_h, u) < 3e-4f);
+    uint32_t best = 0, best_want = 1;
+    izwi::kernels::argmax(got.data(), m, hidden, &best, MemSpace::Host);
+    oracle_argmax(got.data(), m, hidden, &best_want);
+    EXPECT(best == best_want);
+    EXPECT(throws(izwi::Error::Kind::InvalidInput, nullptr,
+                  [&] { izwi::kernels::rms_norm(x.data(), nw.data(), 1, 0, 1e-6f, got_n.data(), MemSpace::Host); }));
+}
+
 // The committed GGUF fixture (tests/golden/tiny.gguf, laid out by hand from the container
 // format): three tensors, alignment 64.  Parsing needs no GPU.
 static void gguf_parse(const std::string& fixture) {
@@ -175,6 +226,7 @@ int main(int argc, char** argv) {
     if (mode == "gpu") {
         packed_matches_separate_q8_0();
         q4k_projection_matches_oracle();
+        folded_calls_match_oracle();
         gguf_load(fixture);
     } else if (mode == "nodevice") {
         no_device_is_loud();
