@@ -283,7 +283,8 @@ def fused_and_q6k_extra(torch, qa, oracle, steps=10, warmup=3):
     """Extra report (not `value`): (a) the o / down projections of the 8B stack with bf16 activations in,
     residual added, bf16 out in one call each (izwi_qmm_forward_fused) against the same projections
     as f32 calls with torch's cast / add / cast kernels around them; (b) Q6_K projections of a
-    Q4_K_M file (ffn_down, attn_v, output) at M = 1: microseconds and Q6_K bytes over time."""
+    Q4_K_M file (ffn_down, attn_v, output) at M = 1: microseconds and Q6_K bytes over time, and their
+    prefill rate at M = 2048 and 512."""
     import numpy as np
     out = {}
     rng = np.random.default_rng(5)
@@ -307,6 +308,12 @@ def fused_and_q6k_extra(torch, qa, oracle, steps=10, warmup=3):
         ms, g = time_graph(torch, run, steps, warmup)
         us = ms * 1e3 / (reps * copies)
         out[f"q6k_m1_{name}"] = {"us": round(us, 2), "gbs": round(n * k // 256 * 210 / us / 1e3, 1)}
+        if name != "output":  # prefill of the same tensor: bf16 in, bf16 out, TFLOP/s
+            for m in (2048, 512):
+                xb = torch.randn(m, k, device="cuda").bfloat16()
+                ms = time_eager(torch, lambda: ws[0].forward(xb), 20, 5)
+                out[f"q6k_prefill_tflops_m{m}_{name}"] = round(2.0 * m * n * k / (ms * 1e-3) / 1e12, 1)
+                del xb
         del ws, g
         torch.cuda.empty_cache()
     mats = []

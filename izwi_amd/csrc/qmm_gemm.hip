@@ -369,9 +369,16 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
     constexpr int MT = BM / WM / 32, NT = BN / 64;       // 32 x 32 accumulator tiles per wave
     constexpr int XC = BM * 8 / THREADS;                 // 16-byte activation chunks per thread and k step
     constexpr int TPR = THREADS / BN;                    // threads that share a weight row: 1, 2 or 4
+    constexpr bool Q6 = QT == QMM_Q6_K;
+    static_assert(!Q6 || TPR == 2 || TPR == 4, "Q6_K is staged by two or four threads per weight row");
     constexpr int NCR = QT == QMM_Q4_K ? 2 : 4;          // 16-byte quant chunks per row and k step
-    constexpr int ND = 4 * NCR / TPR;                    // the thread's run of quant dwords: 2 .. 16
-    constexpr int NC = ND >= 4 ? ND / 4 : 1;             // loads per thread and k step (16 bytes; 8 if ND = 2)
+    // Q6_K: a half unit (two k steps) shares its 64 bytes of low nibbles and 32 bytes of bit pairs.
+    // A thread takes 16 of the 32 byte positions (the half `lh` = part & 1) in both 32-element groups
+    // of a step (two parts per row) or in one of them (four parts): NQL dwords of nibbles, NQH of
+    // bit pairs, held for both steps
+    constexpr int NGG = 4 / TPR, NQL = 4 * NGG, NQH = 4;
+    constexpr int ND = Q6 ? NQL + NQH : 4 * NCR / TPR;   // the thread's run of quant dwords: 2 .. 16
+    constexpr int NC = Q6 ? NGG : ND >= 4 ? ND / 4 : 1; // loads per thread and k step (16 bytes; 8 if ND = 2)
     constexpr int NP = 16 / TPR;                         // pieces of four weights per thread and k step
     constexpr int GPK = MT * NT / 4; // groups of four MFMAs per k16 step
     constexpr int NG = 4 * GPK;      // groups per k step: 16 (BM = 256) or 8 (BM = 128)
@@ -401,8 +408,11 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
     // before it is needed
     constexpr int XD = BN == 128 ? 2 : 1;
     u32x4 xr[XD][XC];
-    u32x4 w_hdr;      // header of the unit fetched last
-    uint32_t wq[2][ND]; // quant dwords of tile kt+1 (being dequantized) and tile kt+2 (in flight), by parity
+    u32x4 w_hdr;      // header of the unit fetched last (Q6_K: its 16 signed scales)
+    uint32_t w_d = 0; // Q6_K: the dword with d of that unit
+    // quant dwords of tile kt+1 (being dequantized) and tile kt+2 (in flight), by parity of the k step
+    // (Q6_K: of the half unit; low nibbles first, bit pairs behind them)
+    uint32_t wq[2][ND];
     // activations: uniform tile base + uniform column + per-lane (row, chunk) offset
     const uint8_t* x_tile = reinterpret_cast<const uint8_t*>(P.x) + m0 * P.k * 2;
     uint32_t x_off[XC];
@@ -427,9 +437,18 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
     // part p holds dwords p ND .. p ND + ND - 1 of the row's quant dwords of a step (Q4_K: 8
     // dwords of nibbles, dword D = elements 4 D .. (low) and 32 + 4 D .. (high); Q8_0: 16 dwords of
     // int8): its first chunk (and, for half a chunk, the offset inside it) and its LDS position
-    const int w_d0 = w_part * ND;
+    const int w_d0 = Q6 ? 0 : w_part * ND;
     const uint32_t w_off_q = w_off + (uint32_t)(w_d0 / 4) * slot_bytes + (uint32_t)(w_d0 % 4) * 4u;
-    const int w_lds = (BM + w_row) * kRowStride + w_d0 * 8;
+    // Q6_K: element 32 gg + l of the k step with nibble `nib` of half unit h is nibble `nib` of
+    // ql[64 h + 32 gg + l] with bit pair 2 nib + gg of qh[32 h + l]; its 16-element group is
+    // 4 (2 h + nib) + 2 gg + l / 16.  Part p: l = 16 lh .., lh = p & 1; gg = 0 and 1 (two parts)
+    // or p / 2 (four parts)
+    const int q6_lh = w_part & 1, q6_gg = TPR == 4 ? w_part >> 1 : 0;
+    const uint32_t w_off_ql = w_off + (uint32_t)(2 * q6_gg + q6_lh) * slot_bytes;
+    const uint32_t w_off_qh = w_off + (uint32_t)q6_lh * slot_bytes;
+    const int q6_pair_shift = 2 * q6_gg;
+    const int q6_scale_shift = 8 * (2 * q6_gg + q6_lh); // of the step's four scale bytes
+    const int w_lds = (BM + w_row) * kRowStride + (Q6 ? 32 * w_part : w_d0 * 8);
     // load cursor: the unit whose chunks are fetched next (clamped to the last unit)
     int cur_us = u0 < P.k_units ? u0 % P.s : 0;
     uint32_t cur_kg_off = (uint32_t)((u0 < P.k_units ? u0 / P.s : 0) * P.panel_bytes);
@@ -461,6 +480,19 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
     };
     auto w_load_hdr = [&]() {
         w_hdr = *reinterpret_cast<const u32x4*>(w_tile + (cur_kg_off + (uint32_t)cur_us * 256u) + w_off);
+        if constexpr (Q6)
+            w_d = *reinterpret_cast<const uint32_t*>(w_tile + (cur_kg_off + (uint32_t)cur_us * 256u + 13u * slot_bytes) + w_off);
+    };
+    // Q6_K: the low nibbles of the thread's group c (HI = 0) or its bit pairs (HI = 1, c = 0) of half
+    // unit HALF of the cursor's unit
+    auto w_load_q6 = [&](auto HALF, auto HI, int c) {
+        constexpr int half = decltype(HALF)::value, hi = decltype(HI)::value;
+        const uint8_t* src = w_tile +
+                             (cur_kg_off + (uint32_t)cur_us * 256u + (uint32_t)(hi ? 9 + 2 * half : 1 + 4 * half + 2 * c) * slot_bytes) +
+                             (hi ? w_off_qh : w_off_ql);
+        const u32x4 v = *reinterpret_cast<const u32x4*>(src);
+        constexpr int o = hi ? NQL : 0;
+        wq[half][o + 4 * c] = v.x, wq[half][o + 4 * c + 1] = v.y, wq[half][o + 4 * c + 2] = v.z, wq[half][o + 4 * c + 3] = v.w;
     };
     auto w_load_q = [&](int sub, int c) {
         const uint8_t* src =
@@ -481,6 +513,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
             hd = qmm_f16_bits_to_f32((uint16_t)(w_hdr.x & 0xffffu));
             hdmin = -qmm_f16_bits_to_f32((uint16_t)(w_hdr.x >> 16));
             qmm_unpack_q4k_scales(w_hdr.y, w_hdr.z, w_hdr.w, sc_lo, sc_hi, mn_lo, mn_hi);
+        } else if (Q6) {
+            hd = qmm_f16_bits_to_f32((uint16_t)(w_d & 0xffffu));
+            sc_lo = w_hdr.x, sc_hi = w_hdr.y, mn_lo = w_hdr.z, mn_hi = w_hdr.w; // scales 4 sub .. 4 sub + 3 in dword sub
         } else {
             sc_lo = w_hdr.x, sc_hi = w_hdr.y, mn_lo = w_hdr.z, mn_hi = w_hdr.w;
         }
@@ -496,6 +531,15 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
             ba = hdmin * ubyte_f32<(2 * g) & 3>(mn);
             sb = hd * ubyte_f32<(2 * g + 1) & 3>(sc);
             bb = hdmin * ubyte_f32<(2 * g + 1) & 3>(mn);
+        } else if (Q6) {
+            // the thread's 16-element group(s) of the step: w = d scale (q - 32)
+            const uint32_t four = g == 0 ? sc_lo : g == 1 ? sc_hi : g == 2 ? mn_lo : mn_hi;
+            sa = hd * (float)(int8_t)(four >> q6_scale_shift);
+            ba = -32.0f * sa;
+            if (TPR == 2) { // the same byte positions of the step's second 32-element group
+                sb = hd * (float)(int8_t)(four >> (q6_scale_shift + 16));
+                bb = -32.0f * sb;
+            }
         } else {
             const uint32_t pair = g == 0 ? sc_lo : g == 1 ? sc_hi : g == 2 ? mn_lo : mn_hi; // blocks 2g, 2g + 1
             sa = qmm_f16_bits_to_f32((uint16_t)(pair & 0xffffu));
@@ -511,10 +555,22 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
     // piece H of NP of the tile with sub-block parity PAR: four of the thread's weights (Q4_K: the
     // low or the high nibbles of one dword; Q8_0: one dword), converted and, every other piece,
     // written as 16 bytes
-    auto w_piece = [&](auto PAR, auto HH, uint8_t* stage) {
-        constexpr int par = decltype(PAR)::value, h = decltype(HH)::value;
+    auto w_piece = [&](auto NSUB, auto HH, uint8_t* stage) {
+        constexpr int par = decltype(NSUB)::value & 1, h = decltype(HH)::value;
         uint8_t* row = stage + w_lds;
-        if constexpr (QT == QMM_Q4_K) {
+        if constexpr (Q6) {
+            // dword h % 4 of the thread's 16 byte positions in its group h / 4: four elements
+            constexpr int half = decltype(NSUB)::value >> 1, nib = par, gi = h / 4, dw = h % 4;
+            const uint32_t v = wq[half][h], vh = wq[half][NQL + dw];
+            const uint32_t q4 = (nib ? v >> 4 : v) & nibble_mask;
+            const uint32_t two = (vh >> (4 * nib + 2 * gi + q6_pair_shift)) & 0x03030303u;
+            const uint32_t q6 = q4 | (two << 4);
+            const float sc = gi ? sb : sa, bi = gi ? bb : ba;
+            constexpr int o = (h % 2) * 2;
+            stash[o] = pack_bf16(__builtin_fmaf(sc, ubyte_f32<0>(q6), bi), __builtin_fmaf(sc, ubyte_f32<1>(q6), bi));
+            stash[o + 1] = pack_bf16(__builtin_fmaf(sc, ubyte_f32<2>(q6), bi), __builtin_fmaf(sc, ubyte_f32<3>(q6), bi));
+            if (h % 2) *reinterpret_cast<uint4*>(row + 64 * gi + 16 * (dw / 2)) = make_uint4(stash[0], stash[1], stash[2], stash[3]);
+        } else if constexpr (QT == QMM_Q4_K) {
             // the thread's dword pair pp: low nibbles of both dwords, then high nibbles of both
             constexpr int pp = h / 4, hi = (h % 4) / 2;
             const uint32_t v = wq[par][2 * pp + (h % 2)];
@@ -594,7 +650,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
                     w_scales(std::integral_constant<int, nsub>{});
                 }
                 static_for<p1 - p0>([&](auto PI) {
-                    w_piece(std::integral_constant<int, nsub & 1>{},
+                    w_piece(std::integral_constant<int, nsub>{},
                             std::integral_constant<int, (p0 + decltype(PI)::value) % NP>{}, next);
                 });
                 constexpr int xbuf = (sub + 1) % XD; // registers of tile kt+1, refilled with tile kt+1+XD
@@ -602,14 +658,21 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
                 for (int i = c0; i < c1; i++) x_write(kt + 1, xbuf, i, next);
 #pragma unroll
                 for (int i = l0; i < (g <= NGS ? l1 : l0); i++) x_load(kt + 1 + XD, xbuf, i);
-                if (g == 1 && sub == 2) {
-                    advance_cursor();
-                    w_load_hdr();
+                // Q6_K fetches by half units, a step earlier: step 1 requests the low nibbles of the
+                // next unit's first half, step 2 its bit pairs, step 3 the low nibbles of the second
+                // half and step 0 (of that unit) its bit pairs; each half is complete one step before
+                // its first tile is dequantized
+                if (g == 1 && sub == (Q6 ? 1 : 2)) advance_cursor();
+                if (g == 1 && sub == 2) w_load_hdr();
+                if (g >= 2 && g < 2 + NC) {
+                    if constexpr (!Q6) w_load_q(lsub, g - 2);
+                    else if constexpr (sub % 2 == 1 || g == 2)
+                        w_load_q6(std::integral_constant<int, (sub == 0 || sub == 3) ? 1 : 0>{},
+                                  std::integral_constant<int, (sub % 2 == 0) ? 1 : 0>{}, g - 2);
                 }
-                if (g >= 2 && g < 2 + NC) w_load_q(lsub, g - 2);
                 // inside the group: one MFMA, then its share of the other instructions, so
                 // the matrix pipe is fed while they issue
-                constexpr int valu = 3 * (p1 - p0) + (g == 0 ? 4 : 1);
+                constexpr int valu = (Q6 ? 4 : 3) * (p1 - p0) + (g == 0 ? 4 : 1);
                 constexpr int reads = GPK == 1 ? NT + MT : NT == 4 ? (gi < GPK / 2 ? 2 * NT / GPK : 2 * MT / GPK) : (gi == 0 ? NT + MT / 2 : MT / 2);
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
@@ -636,7 +699,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
         for (int i = 0; i < XC; i++) x_load(u0 * 4, 0, i);
         w_load_hdr();
 #pragma unroll
-        for (int c = 0; c < NC; c++) w_load_q(0, c);
+        for (int c = 0; c < NC; c++) {
+            if constexpr (Q6) {
+                w_load_q6(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, c);
+                if (c == 0) w_load_q6(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, 0);
+            } else {
+                w_load_q(0, c);
+            }
+        }
 #pragma unroll
         for (int i = 0; i < XC; i++) x_write(u0 * 4, 0, i, smem);
         w_unpack();
@@ -647,7 +717,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
 #pragma unroll
             for (int i = 0; i < XC; i++) x_load(u0 * 4 + d, d % XD, i);
 #pragma unroll
-        for (int c = 0; c < NC; c++) w_load_q(1, c);
+        for (int c = 0; c < NC; c++) {
+            if constexpr (Q6) w_load_q6(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, c);
+            else w_load_q(1, c);
+        }
         __syncthreads();
         static_for<GPK>([&](auto PART) { read_frags(smem, 0, 0, PART); });
 
@@ -718,11 +791,12 @@ hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
     const int64_t grid = (int64_t)P.tiles_m * P.tiles_n;
     if (grid > 0x7fffffff) return hipErrorInvalidValue;
     const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
-    const bool x_tail = (P.k & 63) != 0;
-    constexpr bool kPipe = (BM == 256 || BN == 256) && QT != QMM_Q6_K; // Q6_K: the plain tile kernel only
+    const bool x_tail = QT == QMM_Q8_0 && (P.k & 63) != 0; // the K-quant types have k a multiple of 256
+    // Q6_K is pipelined with eight waves only (two or four threads per weight row)
+    constexpr bool kPipe = (BM == 256 || BN == 256) && (QT != QMM_Q6_K || NW == 8);
     const void* fn;
     if constexpr (kPipe)
-        fn = x_tail ? reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, BN, true, NW>)
+        fn = x_tail ? reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, BN, QT == QMM_Q8_0, NW>)
                     : reinterpret_cast<const void*>(&gemm_pipe_kernel<QT, BM, BN, false, NW>);
     else fn = reinterpret_cast<const void*>(&gemm_kernel<QT, BM, BN>);
     if (lds > 48 * 1024) {
@@ -734,7 +808,7 @@ hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
         if (slices > 1) P.slice_units = (P.k_units + slices - 1) / slices;
         else P.partial = nullptr;
         const dim3 grid2((unsigned)grid, (unsigned)slices);
-        if (x_tail) gemm_pipe_kernel<QT, BM, BN, true, NW><<<grid2, dim3(64 * NW), lds, stream>>>(P);
+        if (x_tail) gemm_pipe_kernel<QT, BM, BN, QT == QMM_Q8_0, NW><<<grid2, dim3(64 * NW), lds, stream>>>(P);
         else gemm_pipe_kernel<QT, BM, BN, false, NW><<<grid2, dim3(64 * NW), lds, stream>>>(P);
         if (slices > 1) {
             const int64_t count = P.m * (P.n_end - P.n_begin);
@@ -831,14 +905,16 @@ hipError_t launch_qt(const GemmParams& P0, int n_cus, hipStream_t stream) {
     }
     if (plan.bm == 256 && plan.bn == 256) return launch_tile<QT, 256, 256, 8>(P, plan.slices, stream);
     if (plan.bm == 256) return launch_tile<QT, 256, 128, 8>(P, plan.slices, stream);
-    if (plan.bn == 256) return launch_tile<QT, 128, 256>(P, plan.slices, stream);
+    if constexpr (QT != QMM_Q6_K) { // the plan picks this tile for m <= 128 only, where Q6_K does not come here
+        if (plan.bn == 256) return launch_tile<QT, 128, 256>(P, plan.slices, stream);
+    }
     return launch_tile<QT, 128, 128>(P, 1, stream);
 }
 
 } // namespace
 
 size_t qmm_gemm_workspace_bytes(const QmmLayout& L, int64_t m, int n_cus) {
-    if (m <= 0 || L.n == 0 || L.dtype == QMM_Q6_K) return 0;
+    if (m <= 0 || L.n == 0 || (L.dtype == QMM_Q6_K && m <= 128)) return 0;
     const GemmPlan plan = plan_gemm(m, L.n, (int)L.k_units * 4, n_cus > 0 ? n_cus : 1);
     return plan.slices > 1 ? (size_t)plan.slices * (size_t)m * (size_t)L.n * sizeof(float) : 0;
 }
@@ -870,8 +946,9 @@ hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uin
     P.partial = (float*)workspace;
     P.residual = residual;
     if (L.dtype == QMM_Q6_K) {
-        // the plain tile kernel only (a 256 x 128 tile was no faster: 308 against 316 us on
-        // [4096, 12288] at m = 2048); half-height tiles when full ones would leave CUs idle
+        // more than 128 rows: the pipelined tiles; up to 128 the plain tile kernel, half-height
+        // tiles when full ones would leave CUs idle
+        if (m > 128 && !getenv("IZWI_QMM_Q6K_PLAIN_TILES")) return launch_qt<QMM_Q6_K>(P, n_cus, stream);
         const int64_t t128 = ((m + 127) / 128) * ((L.n + 127) / 128);
         if (t128 < (int64_t)n_cus && m > 64) return launch_tile<QMM_Q6_K, 64, 128>(P, 1, stream);
         return launch_tile<QMM_Q6_K, 128, 128>(P, 1, stream);
