@@ -395,8 +395,8 @@ def q4_k_m_mix_extra(torch, qa, oracle, m=1, steps=20, warmup=3):
     reference's default chat model): attn_v and ffn_down are Q6_K in half of the layers (the first and last
     eighth and every third layer between, as llama.cpp's Q4_K_M recipe picks them) and so is the output
     matrix; everything else is Q4_K.  Q6_K weights are random block bytes with a finite scale (the oracle
-    has no Q6_K quantizer).  Same call structure as the headline; a q|k|v group with a Q6_K member runs as a
-    q|k group call plus one call for v."""
+    has no Q6_K quantizer).  Same call structure as the headline; a q|k|v group with a Q6_K member is split by
+    type inside the library (q|k as one launch, v as another)."""
     import numpy as np
     rng = np.random.default_rng(11)
 
@@ -423,11 +423,7 @@ def q4_k_m_mix_extra(torch, qa, oracle, m=1, steps=20, warmup=3):
             dt = 14 if six else Q4_K
             w[name] = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType(dt), q6[name] if six else q4[name], (n, k)))
             total += n * k // 256 * bytes_per[dt] + 4 * m * k + 4 * m * n
-        if w["v"].qtensor.dtype() == qa.GgmlDType.Q4K:
-            calls.append(([w["q"], w["k"], w["v"]], xs[4096], [out(4096), out(1024), out(1024)]))
-        else:
-            calls.append(([w["q"], w["k"]], xs[4096], [out(4096), out(1024)]))
-            calls.append((w["v"], xs[4096], out(1024)))
+        calls.append(([w["q"], w["k"], w["v"]], xs[4096], [out(4096), out(1024), out(1024)]))
         calls.append((w["o"], xs[4096], out(4096)))
         calls.append(([w["gate"], w["up"]], xs[4096], [out(12288), out(12288)]))
         calls.append((w["down"], xs[12288], out(4096)))

@@ -50,7 +50,7 @@ typedef enum izwi_qmm_status {
 /* ggml / GGUF tensor type ids (candle-core GgmlDType) */
 #define IZWI_QMM_Q8_0 8
 #define IZWI_QMM_Q4_K 12
-#define IZWI_QMM_Q6_K 14 /* single projections only: no projection-group launch, no expert stacks */
+#define IZWI_QMM_Q6_K 14
 
 typedef enum izwi_qmm_mem_space { IZWI_QMM_DEVICE = 0, IZWI_QMM_HOST = 1 } izwi_qmm_mem_space;
 

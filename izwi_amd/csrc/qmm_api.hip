@@ -590,13 +590,16 @@ int izwi_qmm_forward_group_normed_f32(const izwi_qmm_weight* const* weights, int
 
 namespace {
 
+int batched_group_on_records(const izwi_qmm_weight* const* weights, int32_t n_weights, const float* x, int64_t m,
+                             float* const* ys, void* records, hipStream_t stream);
+
 int forward_group_impl(const izwi_qmm_weight* const* weights, int32_t n_weights, const float* x, int64_t m,
                        float* const* ys, int mem_space, void* stream_, const float* norm_weight, float norm_eps) {
     if (!weights || !ys) return fail(IZWI_QMM_ERR_INVALID, "NULL argument");
     if (n_weights < 1 || n_weights > QMM_MAX_GROUP)
         return fail(IZWI_QMM_ERR_INVALID, "projection group of %d weights (1..%d supported)", n_weights, QMM_MAX_GROUP);
     if (int rc = check_space(mem_space)) return rc;
-    bool uniform = true;
+    bool uniform = true, splittable = true;
     for (int i = 0; i < n_weights; i++) {
         if (!weights[i]) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
         const QmmLayout& L = weights[i]->layout;
@@ -604,17 +607,50 @@ int forward_group_impl(const izwi_qmm_weight* const* weights, int32_t n_weights,
         if (L.k != weights[0]->layout.k)
             return fail(IZWI_QMM_ERR_INVALID, "projection group input mismatch: expected %lld, got %lld",
                         (long long)weights[0]->layout.k, (long long)L.k);
-        if (L.dtype != weights[0]->layout.dtype || L.n == 0 || weights[i]->device != weights[0]->device ||
-            L.dtype == IZWI_QMM_Q6_K) // Q6_K has no multi-weight launch
+        if (L.dtype != weights[0]->layout.dtype || L.n == 0 || weights[i]->device != weights[0]->device)
             uniform = false;
+        if (L.n == 0 || weights[i]->device != weights[0]->device) splittable = false;
         if (m > 0 && L.n > 0 && !ys[i]) return fail(IZWI_QMM_ERR_INVALID, "y is NULL");
     }
     if (m < 0) return fail(IZWI_QMM_ERR_INVALID, "negative m");
     if (m == 0) return IZWI_QMM_OK;
     if (!x) return fail(IZWI_QMM_ERR_INVALID, "x is NULL");
+    // Several block types in one group (a Q4_K_M file keeps attn_v of some layers in Q6_K beside Q4_K
+    // attn_q / attn_k): one group call per type, in the order of each type's first member
+    const bool by_type = mem_space == IZWI_QMM_DEVICE && !uniform && splittable && n_weights >= 2 && m <= 64;
+    auto call_by_type = [&](const float* xin, const float* nw) -> int {
+        bool done[QMM_MAX_GROUP] = {};
+        // batched sizes: Q4_K and Q6_K weights dot against the same Q8_K records, quantized once
+        bool q8k_records = !nw && m >= mfma_min_m();
+        for (int i = 0; i < n_weights; i++)
+            if (weights[i]->layout.dtype != IZWI_QMM_Q4_K && weights[i]->layout.dtype != IZWI_QMM_Q6_K) q8k_records = false;
+        void* records = nullptr;
+        if (q8k_records) {
+            hipStream_t stream = (hipStream_t)stream_;
+            HIP_TRY(get_scratch(weights[0]->device, stream, qmm_gemv_mfma_workspace_bytes(weights[0]->layout, m), &records));
+            HIP_TRY(qmm_launch_quantize_ws(IZWI_QMM_Q4_K, xin, m, weights[0]->layout.k, records, stream));
+        }
+        for (int i = 0; i < n_weights; i++) {
+            if (done[i]) continue;
+            const izwi_qmm_weight* sub_w[QMM_MAX_GROUP];
+            float* sub_y[QMM_MAX_GROUP];
+            int n_sub = 0;
+            for (int j = i; j < n_weights; j++)
+                if (!done[j] && weights[j]->layout.dtype == weights[i]->layout.dtype)
+                    sub_w[n_sub] = weights[j], sub_y[n_sub] = ys[j], n_sub++, done[j] = true;
+            if (records) {
+                if (int rc = batched_group_on_records(sub_w, n_sub, xin, m, sub_y, records, (hipStream_t)stream_)) return rc;
+            } else if (int rc = forward_group_impl(sub_w, n_sub, xin, m, sub_y, mem_space, stream_, nw, norm_eps)) {
+                return rc;
+            }
+        }
+        return IZWI_QMM_OK;
+    };
     if (norm_weight) {
         hipStream_t stream = (hipStream_t)stream_;
         const izwi_qmm_weight* w0 = weights[0];
+        // each type's launch normalizes for itself: x is read by every workgroup anyway
+        if (by_type && m <= 2 && m < mfma_min_m()) return call_by_type(x, norm_weight);
         // one launch: the decode kernel normalizes while it quantizes (device buffers, one block type, m <= 2)
         if (mem_space == IZWI_QMM_DEVICE && uniform && m <= 2 && m < mfma_min_m()) {
             const QmmLayout* layouts[QMM_MAX_GROUP];
@@ -645,6 +681,7 @@ int forward_group_impl(const izwi_qmm_weight* const* weights, int32_t n_weights,
         for (int i = 0; i < n_weights; i++) HIP_TRY(yo[i].finish(stream));
         return IZWI_QMM_OK;
     }
+    if (by_type) return call_by_type(x, nullptr);
     // host buffers, mixed types, prefill sizes: one call per projection (same results)
     if (mem_space != IZWI_QMM_DEVICE || !uniform || n_weights == 1 || m > 64) {
         for (int i = 0; i < n_weights; i++)
@@ -675,19 +712,26 @@ int forward_group_impl(const izwi_qmm_weight* const* weights, int32_t n_weights,
     void* scratch = nullptr;
     HIP_TRY(get_scratch(w0->device, stream, qmm_gemv_mfma_workspace_bytes(w0->layout, m), &scratch));
     HIP_TRY(qmm_launch_quantize_ws(w0->layout.dtype, x, m, w0->layout.k, scratch, stream));
-    {
+    return batched_group_on_records(weights, n_weights, x, m, ys, scratch, stream);
+}
+
+// The batched decode kernel for a group of one block type whose quantized activations are in `records`.
+int batched_group_on_records(const izwi_qmm_weight* const* weights, int32_t n_weights, const float* x, int64_t m,
+                             float* const* ys, void* records, hipStream_t stream) {
+    const izwi_qmm_weight* w0 = weights[0];
+    if (n_weights > 1) {
         const QmmLayout* layouts[QMM_MAX_GROUP];
         const void* tiled[QMM_MAX_GROUP];
         for (int i = 0; i < n_weights; i++) layouts[i] = &weights[i]->layout, tiled[i] = weights[i]->tiled;
         ProfileScope prof(w0, stream);
-        hipError_t e = qmm_launch_gemv_mfma_multi(layouts, tiled, n_weights, m, ys, scratch, w0->n_cus, stream);
+        hipError_t e = qmm_launch_gemv_mfma_multi(layouts, tiled, n_weights, m, ys, records, w0->n_cus, stream);
         if (e == hipSuccess) return IZWI_QMM_OK;
         if (e != hipErrorNotSupported) return fail_hip(e, "grouped batched decode kernel");
         (void)hipGetLastError();
     }
     for (int i = 0; i < n_weights; i++) {
         ProfileScope prof(weights[i], stream);
-        HIP_TRY(qmm_launch_gemv_mfma(weights[i]->layout, weights[i]->tiled, x, m, ys[i], scratch,
+        HIP_TRY(qmm_launch_gemv_mfma(weights[i]->layout, weights[i]->tiled, x, m, ys[i], records,
                                      weights[i]->n_cus, stream, false));
     }
     return IZWI_QMM_OK;
@@ -773,7 +817,7 @@ int gate_up_silu_impl(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, co
     Staged wi;
     if (norm_weight) HIP_TRY(wi.in(norm_weight, (size_t)L.k * sizeof(float), mem_space));
     const float* xin = (const float*)xi.dev;
-    if (m < mfma_min_m() && m <= 2 && L.dtype != IZWI_QMM_Q6_K) {
+    if (m < mfma_min_m() && m <= 2) {
         const QmmNorm norm{(const float*)wi.dev, norm_eps};
         ProfileScope prof(gate, stream);
         HIP_TRY(qmm_launch_gemv_gated(L, gate->tiled, up->tiled, xin, m, (float*)ho.dev, gate->n_cus, stream,
@@ -975,8 +1019,6 @@ int moe_check_stacks(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, con
     const QmmLayout& D = down->layout;
     if (G.dtype != U.dtype || G.n != U.n || G.k != U.k || G.n_stacked != U.n_stacked)
         return fail(IZWI_QMM_ERR_INVALID, "gate and up stacks differ in shape or dtype");
-    if (G.dtype == IZWI_QMM_Q6_K || D.dtype == IZWI_QMM_Q6_K)
-        return fail(IZWI_QMM_ERR_UNSUPPORTED, "expert stacks of Q6_K weights are not supported (Q8_0, Q4_K)");
     if (D.n_stacked != G.n_stacked || D.k != G.n || D.n != G.k)
         return fail(IZWI_QMM_ERR_INVALID, "down stack [%lld, %lld] does not match gate/up [%lld, %lld]",
                     (long long)D.n, (long long)D.k, (long long)G.n, (long long)G.k);

@@ -25,6 +25,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstddef>
+#include <type_traits>
 
 #include "qmm_internal.h"
 
@@ -733,6 +734,14 @@ hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipS
     return hipGetLastError();
 }
 
+// f(std::integral_constant<int, block type>) for the layout's block type
+template <class F>
+hipError_t with_block_type(int dtype, F&& f) {
+    if (dtype == QMM_Q4_K) return f(std::integral_constant<int, QMM_Q4_K>{});
+    if (dtype == QMM_Q6_K) return f(std::integral_constant<int, QMM_Q6_K>{});
+    return f(std::integral_constant<int, QMM_Q8_0>{});
+}
+
 template <int QT>
 hipError_t launch_plain(const GemvParams& P, int waves, int n_cus, int io, hipStream_t stream) {
     if (P.norm_w != nullptr) { // folded RMSNorm: f32 activations, plain store, one or two rows
@@ -883,25 +892,21 @@ hipError_t qmm_launch_gemv_gated(const QmmLayout& L, const void* tiled_gate, con
                                  const float* x, int64_t m, float* y, int n_cus, hipStream_t stream,
                                  const QmmNorm* norm) {
     if (m <= 0 || L.n == 0) return hipSuccess;
-    if (m > 2 || L.dtype == QMM_Q6_K) return hipErrorNotSupported;
+    if (m > 2) return hipErrorNotSupported;
     GemvParams P;
     if (!make_params(L, tiled_gate, x, m, y, P)) return hipErrorInvalidValue;
     P.w2 = (const uint8_t*)tiled_up;
     int waves;
     choose_split(L, n_cus, 1, true, P, waves);
-    if (norm) {
-        P.norm_w = norm->weight, P.norm_eps = norm->eps;
-        if (L.dtype == QMM_Q4_K)
-            return m == 2 ? launch_mt<QMM_Q4_K, 2, true, false, 0, true>(P, waves, n_cus, 1, stream)
-                          : launch_mt<QMM_Q4_K, 1, true, false, 0, true>(P, waves, n_cus, 1, stream);
-        return m == 2 ? launch_mt<QMM_Q8_0, 2, true, false, 0, true>(P, waves, n_cus, 1, stream)
-                      : launch_mt<QMM_Q8_0, 1, true, false, 0, true>(P, waves, n_cus, 1, stream);
-    }
-    if (L.dtype == QMM_Q4_K)
-        return m == 2 ? launch_mt<QMM_Q4_K, 2, true, false>(P, waves, n_cus, 1, stream)
-                      : launch_mt<QMM_Q4_K, 1, true, false>(P, waves, n_cus, 1, stream);
-    return m == 2 ? launch_mt<QMM_Q8_0, 2, true, false>(P, waves, n_cus, 1, stream)
-                  : launch_mt<QMM_Q8_0, 1, true, false>(P, waves, n_cus, 1, stream);
+    if (norm) P.norm_w = norm->weight, P.norm_eps = norm->eps;
+    return with_block_type(L.dtype, [&](auto QT) {
+        constexpr int qt = decltype(QT)::value;
+        if (norm)
+            return m == 2 ? launch_mt<qt, 2, true, false, 0, true>(P, waves, n_cus, 1, stream)
+                          : launch_mt<qt, 1, true, false, 0, true>(P, waves, n_cus, 1, stream);
+        return m == 2 ? launch_mt<qt, 2, true, false>(P, waves, n_cus, 1, stream)
+                      : launch_mt<qt, 1, true, false>(P, waves, n_cus, 1, stream);
+    });
 }
 
 hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
@@ -915,7 +920,7 @@ hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* co
         if (L.dtype != L0.dtype || L.k != L0.k || L.n_stacked != 1 || L.n == 0) return hipErrorInvalidValue;
         total_row_tiles += L.row_tiles;
     }
-    if (L0.k_groups > kMaxWaves || L0.dtype == QMM_Q6_K) return hipErrorNotSupported; // no single-launch form: the caller launches one by one
+    if (L0.k_groups > kMaxWaves) return hipErrorNotSupported; // no single-launch form: the caller launches one by one
     GemvParams P;
     if (!make_params(L0, tiled[0], x, m, ys[0], P)) return hipErrorInvalidValue;
     // the split of a single matrix with all the row-tiles
@@ -939,33 +944,22 @@ hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* co
     if (groups > (int64_t)n_cus * 32) return hipErrorNotSupported;
     P.rt_groups = (int)groups;
     const int mt = m == 2 ? 2 : 1;
-    const size_t lds = mt == 2 ? lds_bytes<QMM_Q4_K, 2>(P.k_units, waves) : lds_bytes<QMM_Q4_K, 1>(P.k_units, waves);
-    const size_t lds8 = mt == 2 ? lds_bytes<QMM_Q8_0, 2>(P.k_units, waves) : lds_bytes<QMM_Q8_0, 1>(P.k_units, waves);
-    size_t need = L0.dtype == QMM_Q4_K ? lds : lds8;
-    if (norm) {
-        P.norm_w = norm->weight, P.norm_eps = norm->eps;
-        need += (size_t)mt * P.k_units * sizeof(float);
-    }
-    if (need > 48 * 1024) return hipErrorNotSupported;
+    if (norm) P.norm_w = norm->weight, P.norm_eps = norm->eps;
     const dim3 g((unsigned)groups), b(64 * waves);
-    if (norm) {
-        if (L0.dtype == QMM_Q4_K) {
-            if (mt == 2) gemv_kernel<QMM_Q4_K, 2, false, false, true, 0, true><<<g, b, need, stream>>>(P);
-            else gemv_kernel<QMM_Q4_K, 1, false, false, true, 0, true><<<g, b, need, stream>>>(P);
+    return with_block_type(L0.dtype, [&](auto QT) {
+        constexpr int qt = decltype(QT)::value;
+        size_t need = mt == 2 ? lds_bytes<qt, 2>(P.k_units, waves) : lds_bytes<qt, 1>(P.k_units, waves);
+        if (norm) need += (size_t)mt * P.k_units * sizeof(float);
+        if (need > 48 * 1024) return hipErrorNotSupported;
+        if (norm) {
+            if (mt == 2) gemv_kernel<qt, 2, false, false, true, 0, true><<<g, b, need, stream>>>(P);
+            else gemv_kernel<qt, 1, false, false, true, 0, true><<<g, b, need, stream>>>(P);
         } else {
-            if (mt == 2) gemv_kernel<QMM_Q8_0, 2, false, false, true, 0, true><<<g, b, need, stream>>>(P);
-            else gemv_kernel<QMM_Q8_0, 1, false, false, true, 0, true><<<g, b, need, stream>>>(P);
+            if (mt == 2) gemv_kernel<qt, 2, false, false, true><<<g, b, need, stream>>>(P);
+            else gemv_kernel<qt, 1, false, false, true><<<g, b, need, stream>>>(P);
         }
         return hipGetLastError();
-    }
-    if (L0.dtype == QMM_Q4_K) {
-        if (mt == 2) gemv_kernel<QMM_Q4_K, 2, false, false, true><<<g, b, need, stream>>>(P);
-        else gemv_kernel<QMM_Q4_K, 1, false, false, true><<<g, b, need, stream>>>(P);
-    } else {
-        if (mt == 2) gemv_kernel<QMM_Q8_0, 2, false, false, true><<<g, b, need, stream>>>(P);
-        else gemv_kernel<QMM_Q8_0, 1, false, false, true><<<g, b, need, stream>>>(P);
-    }
-    return hipGetLastError();
+    });
 }
 
 hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
@@ -975,7 +969,6 @@ hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const 
                                    int n_cus, hipStream_t stream) {
     if (max_segments <= 0 || L.n == 0) return hipSuccess;
     if (max_segments > 65535) return hipErrorInvalidValue;
-    if (L.dtype == QMM_Q6_K) return hipErrorNotSupported;
     GemvParams P;
     if (!make_params(L, tiled, x, 0, y, P)) return hipErrorInvalidValue;
     P.w2 = (const uint8_t*)tiled2;
@@ -991,6 +984,9 @@ hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const 
     if (L.dtype == QMM_Q4_K)
         return gated ? launch_mt<QMM_Q4_K, 4, true, true>(P, waves, n_cus, (int)max_segments, stream)
                      : launch_mt<QMM_Q4_K, 4, false, true>(P, waves, n_cus, (int)max_segments, stream);
+    if (L.dtype == QMM_Q6_K)
+        return gated ? launch_mt<QMM_Q6_K, 4, true, true>(P, waves, n_cus, (int)max_segments, stream)
+                     : launch_mt<QMM_Q6_K, 4, false, true>(P, waves, n_cus, (int)max_segments, stream);
     return gated ? launch_mt<QMM_Q8_0, 4, true, true>(P, waves, n_cus, (int)max_segments, stream)
                  : launch_mt<QMM_Q8_0, 4, false, true>(P, waves, n_cus, (int)max_segments, stream);
 }

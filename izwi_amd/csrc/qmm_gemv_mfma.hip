@@ -1043,7 +1043,7 @@ hipError_t qmm_launch_quantize_grouped(int dtype, const float* x, const float* x
     if (threads <= 0) return hipSuccess;
     if (threads > 0x7fffffff00ll || k > 0x3fffffff) return hipErrorInvalidValue;
     const unsigned grid = (unsigned)((threads + 255) / 256);
-    if (dtype == QMM_Q4_K)
+    if (dtype == QMM_Q4_K || dtype == QMM_Q6_K) // both dot against Q8_K activations: one record format
         quantize_grouped_kernel<QMM_Q4_K><<<grid, 256, 0, stream>>>(x, x2, x_div, (int)k, (int)k_units, perm,
                                                                     offsets, tile_offsets, n_experts,
                                                                     (uint8_t*)records);
@@ -1099,7 +1099,9 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     const void* fn = L.dtype == QMM_Q4_K
                          ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true>)
-                         : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, false, true>);
+                         : L.dtype == QMM_Q6_K
+                               ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q6_K, false, true>)
+                               : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, false, true>);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
@@ -1107,6 +1109,8 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     const dim3 grid((unsigned)P.rt_groups, (unsigned)n_experts, tiled2 ? 2u : 1u);
     if (L.dtype == QMM_Q4_K)
         gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true><<<grid, 64 * waves, lds, stream>>>(P);
+    else if (L.dtype == QMM_Q6_K)
+        gemv_mfma_oneshot_kernel<QMM_Q6_K, false, true><<<grid, 64 * waves, lds, stream>>>(P);
     else
         gemv_mfma_oneshot_kernel<QMM_Q8_0, false, true><<<grid, 64 * waves, lds, stream>>>(P);
     return hipGetLastError();
@@ -1175,14 +1179,17 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
     }
     const size_t lds = std::max((size_t)P.window_units * unit_bytes(L0.dtype), (size_t)waves * 256 * 4);
     if (lds > 160 * 1024) return hipErrorNotSupported;
-    const void* fn = L0.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true>)
-                                          : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, true>);
+    const void* fn = L0.dtype == QMM_Q4_K   ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true>)
+                     : L0.dtype == QMM_Q6_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q6_K, true>)
+                                            : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, true>);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
     if (L0.dtype == QMM_Q4_K)
         gemv_mfma_oneshot_kernel<QMM_Q4_K, true><<<(unsigned)groups, 64 * waves, lds, stream>>>(P);
+    else if (L0.dtype == QMM_Q6_K)
+        gemv_mfma_oneshot_kernel<QMM_Q6_K, true><<<(unsigned)groups, 64 * waves, lds, stream>>>(P);
     else
         gemv_mfma_oneshot_kernel<QMM_Q8_0, true><<<(unsigned)groups, 64 * waves, lds, stream>>>(P);
     return hipGetLastError();

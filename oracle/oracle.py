@@ -63,6 +63,9 @@ def lib() -> C.CDLL:
         L.oracle_moe_forward.restype = C.c_int
         L.oracle_moe_forward.argtypes = [C.c_int, i64, C.c_int, C.c_int, i64, i64,
                                          vp, vp, vp, vp, vp, vp, vp]
+        L.oracle_moe_forward_mixed.restype = C.c_int
+        L.oracle_moe_forward_mixed.argtypes = [C.c_int, C.c_int, i64, C.c_int, C.c_int, i64, i64,
+                                               vp, vp, vp, vp, vp, vp, vp]
         L.oracle_fill_normal.restype = None
         L.oracle_fill_normal.argtypes = [C.c_uint64, i64, i64, C.c_float, C.c_float, vp]
         f32 = C.c_float
@@ -176,15 +179,16 @@ def moe_sort(ids: np.ndarray, n_experts: int):
 
 
 def moe_forward(dtype: int, x: np.ndarray, ids: np.ndarray, wts: np.ndarray, gate: np.ndarray,
-                up: np.ndarray, down: np.ndarray, n_experts: int, inter: int) -> np.ndarray:
+                up: np.ndarray, down: np.ndarray, n_experts: int, inter: int, down_dtype: int | None = None) -> np.ndarray:
     x = np.ascontiguousarray(x, dtype=np.float32)
     T, hidden = x.shape
     ids = np.ascontiguousarray(ids, dtype=np.int32)
     wts = np.ascontiguousarray(wts, dtype=np.float32)
     top_k = ids.shape[1]
     out = np.empty((T, hidden), dtype=np.float32)
-    rc = lib().oracle_moe_forward(dtype, T, n_experts, top_k, hidden, inter, _ptr(x), _ptr(ids),
-                                  _ptr(wts), _ptr(gate), _ptr(up), _ptr(down), _ptr(out))
+    rc = lib().oracle_moe_forward_mixed(dtype, dtype if down_dtype is None else down_dtype, T, n_experts, top_k,
+                                        hidden, inter, _ptr(x), _ptr(ids), _ptr(wts), _ptr(gate), _ptr(up),
+                                        _ptr(down), _ptr(out))
     if rc:
         raise ValueError("oracle_moe_forward rejected the shape")
     return out

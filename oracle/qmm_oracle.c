@@ -673,11 +673,11 @@ void oracle_moe_sort(const int32_t* ids, int64_t T, int top_k, int E, int32_t* p
 static inline float silu_f32(float v) { return v / (1.0f + expf(-v)); }
 
 /* gate/up: [E][inter][hidden] blocks, down: [E][hidden][inter] blocks. */
-int oracle_moe_forward(int dtype, int64_t T, int E, int top_k, int64_t hidden, int64_t inter,
-                       const float* x, const int32_t* ids, const float* wts, const void* gate,
-                       const void* up, const void* down, float* out) {
+static int moe_forward_impl(int dtype, int down_dtype, int64_t T, int E, int top_k, int64_t hidden, int64_t inter,
+                            const float* x, const int32_t* ids, const float* wts, const void* gate,
+                            const void* up, const void* down, float* out) {
     int64_t gu_bytes = oracle_storage_bytes(dtype, inter, hidden);
-    int64_t dn_bytes = oracle_storage_bytes(dtype, hidden, inter);
+    int64_t dn_bytes = oracle_storage_bytes(down_dtype, hidden, inter);
     if (gu_bytes < 0 || dn_bytes < 0) return -1;
     float* g = (float*)malloc((size_t)inter * sizeof(float));
     float* u = (float*)malloc((size_t)inter * sizeof(float));
@@ -693,7 +693,7 @@ int oracle_moe_forward(int dtype, int64_t T, int E, int top_k, int64_t hidden, i
             oracle_qmatmul(dtype, 1, hidden, inter, x + t * hidden,
                            (const uint8_t*)up + (size_t)e * gu_bytes, u);
             for (int64_t c = 0; c < inter; c++) g[c] = silu_f32(g[c]) * u[c];
-            oracle_qmatmul(dtype, 1, inter, hidden, g, (const uint8_t*)down + (size_t)e * dn_bytes,
+            oracle_qmatmul(down_dtype, 1, inter, hidden, g, (const uint8_t*)down + (size_t)e * dn_bytes,
                            y);
             for (int64_t c = 0; c < hidden; c++) o[c] += w * y[c];
         }
@@ -702,6 +702,21 @@ int oracle_moe_forward(int dtype, int64_t T, int E, int top_k, int64_t hidden, i
     free(u);
     free(y);
     return 0;
+}
+
+int oracle_moe_forward(int dtype, int64_t T, int E, int top_k, int64_t hidden, int64_t inter,
+                       const float* x, const int32_t* ids, const float* wts, const void* gate,
+                       const void* up, const void* down, float* out) {
+    return moe_forward_impl(dtype, dtype, T, E, top_k, hidden, inter, x, ids, wts, gate, up, down, out);
+}
+
+/* The same with the down stack in a type of its own (a Q4_K_M file keeps ffn_down_exps of some
+ * layers in Q6_K beside Q4_K gate / up stacks): each product is the reference's QMatMul::forward
+ * for its tensor's type. */
+int oracle_moe_forward_mixed(int gate_up_dtype, int down_dtype, int64_t T, int E, int top_k, int64_t hidden,
+                             int64_t inter, const float* x, const int32_t* ids, const float* wts,
+                             const void* gate, const void* up, const void* down, float* out) {
+    return moe_forward_impl(gate_up_dtype, down_dtype, T, E, top_k, hidden, inter, x, ids, wts, gate, up, down, out);
 }
 
 /* ------------------------------------------------------- seeded inputs --- */

@@ -136,26 +136,69 @@ def test_q6_k_prefill_against_oracle(qa, oracle, m, n, k):
 
 
 def test_q6_k_in_groups_and_mlp(qa, oracle):
-    """A projection group or a gate/up pair with a Q6_K member runs projection by projection and
-    gives the results of separate calls; expert stacks of Q6_K are refused."""
-    from izwi_amd.capi import QmmError
+    """Projection groups and gate/up pairs with Q6_K members give the results of separate calls: a
+    group of one type is one launch (up to two rows) or one shared quantization (up to 64), a group of
+    several types runs type by type; with the RMSNorm folded in as well."""
     k, n = 1024, 512
     b6 = np_ref.random_q6_k_blocks(1, n, k)
+    b6b = np_ref.random_q6_k_blocks(3, 272, k)
     b4 = oracle.quantize(Q4_K, oracle.randn(2, (n, k), std=0.02))
+    b4b = oracle.quantize(Q4_K, oracle.randn(4, (272, k), std=0.02))
     w6 = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q6K, b6, (n, k)))
+    w6b = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q6K, b6b, (272, k)))
     w4 = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q4K, b4, (n, k)))
+    w4b = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q4K, b4b, (272, k)))
     gu = qa.Qwen3GateUpProjection.new_separate(w6, w6)
-    for m in (1, 5, 80):
+    nw = torch.from_numpy(oracle.randn(9, (k,), mean=1.0, std=0.2)).cuda()
+    for m in (1, 2, 5, 16, 80):
         x = torch.from_numpy(oracle.randn(10 + m, (m, k))).cuda()
-        ys = qa.forward_group([w4, w6, w6], x)
-        assert torch.equal(ys[0], w4.forward(x)) and torch.equal(ys[1], w6.forward(x)) and torch.equal(ys[2], ys[1])
+        for group in ([w4, w6, w6], [w6, w6b, w6], [w4, w4b, w6b], [w6b, w4]):
+            ys = qa.forward_group(group, x)
+            for y, w in zip(ys, group):
+                assert torch.equal(y, w.forward(x))
+            # the norm folded in: the single-weight normed call is the yardstick (same kernel variant)
+            ys = qa.forward_group(group, x, norm_weight=nw, eps=1e-6)
+            for y, w in zip(ys, group):
+                want = w.forward_normed(x, nw, 1e-6)
+                assert float((y - want).abs().max()) <= 2e-6 * float(want.abs().max())
         g = w6.forward(x)
         assert torch.allclose(gu.forward_silu_mul(x), torch.nn.functional.silu(g) * g, rtol=1e-5, atol=1e-6)
-    stack = lambda seed, rows, cols: qa.QTensor.from_blocks(  # noqa: E731
-        qa.GgmlDType.Q6K, np_ref.random_q6_k_blocks(seed, 2 * rows, cols), (2, rows, cols))
-    experts = qa.MoeExperts(stack(5, n, k), stack(6, n, k), stack(7, k, n))
-    ids = torch.zeros(1, 1, dtype=torch.int32, device="cuda")
-    perm, offsets = qa.moe_sort(ids, 2)
-    with pytest.raises(QmmError) as e:
-        experts.forward(torch.zeros(1, k, device="cuda"), ids, torch.ones(1, 1, device="cuda"), perm, offsets)
-    assert e.value.code == -2
+        gn = w6.forward_normed(x, nw, 1e-6)
+        assert torch.allclose(gu.forward_silu_mul(x, norm_weight=nw, eps=1e-6), torch.nn.functional.silu(gn) * gn,
+                              rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("gate_up_dtype,E,hidden,inter,t,top_k", [
+    (Q4_K, 8, 512, 768, 64, 4),    # the Q4_K_M case: Q4_K gate / up, Q6_K down; 32 pairs per expert: matrix-core tiles
+    (Q4_K, 16, 512, 512, 6, 8),    # 3 pairs per expert: 4-row segments
+    (Q4_K, 8, 1024, 256, 1, 2),    # one token
+    (Q6_K, 4, 768, 512, 40, 2),    # every stack Q6_K, ragged panels
+    (Q6_K, 8, 256, 512, 3, 2),
+])
+def test_moe_with_q6_k_expert_stacks(qa, oracle, gate_up_dtype, E, hidden, inter, t, top_k):
+    """Expert stacks in Q6_K (a Q4_K_M file keeps ffn_down_exps of some layers in it): the expert MLP
+    against the oracle's composition of per-type products, and the one-call layer against the three
+    calls."""
+    _say(f"q6k moe gate_up={gate_up_dtype} E={E} hidden={hidden} inter={inter} t={t}")
+    if gate_up_dtype == Q6_K:
+        gate = np_ref.random_q6_k_blocks(311, E * inter, hidden, d_scale=2e-3)
+        up = np_ref.random_q6_k_blocks(312, E * inter, hidden, d_scale=2e-3)
+    else:
+        gate = oracle.quantize(gate_up_dtype, oracle.randn(311, (E * inter, hidden), std=0.05))
+        up = oracle.quantize(gate_up_dtype, oracle.randn(312, (E * inter, hidden), std=0.05))
+    down = np_ref.random_q6_k_blocks(313, E * hidden, inter, d_scale=2e-3)
+    gdt = qa.GgmlDType(gate_up_dtype)
+    experts = qa.MoeExperts(qa.QTensor.from_blocks(gdt, gate, (E, inter, hidden)),
+                            qa.QTensor.from_blocks(gdt, up, (E, inter, hidden)),
+                            qa.QTensor.from_blocks(qa.GgmlDType.Q6K, down, (E, hidden, inter)))
+    x = oracle.randn(314, (t, hidden))
+    logits = oracle.randn(315, (t, E))
+    xd, ld = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
+    ids, wts = qa.moe_route(ld, top_k)
+    perm, offsets = qa.moe_sort(ids, E)
+    out = experts.forward(xd, ids, wts, perm, offsets)
+    want_ids, want_wts = oracle.moe_route(logits, top_k)
+    assert np.array_equal(ids.cpu().numpy(), want_ids)
+    want = oracle.moe_forward(gate_up_dtype, x, want_ids, want_wts, gate, up, down, E, inter, down_dtype=Q6_K)
+    assert rel_err(out.cpu().numpy(), want) < 1e-3
+    assert torch.equal(experts.layer(ld, xd, top_k), out)
