@@ -242,6 +242,57 @@ def prefill_extra(torch, qa, oracle, dtype, m, steps=20, warmup=5, only=None):
     return out
 
 
+def host_pointer_extra(qa, weights, m, passes=2):
+    """Extra report (not `value`): the same projections called one by one with HOST pointers, the literal
+    form of the reference's CPU call (activations in host memory in, results in host memory out): every
+    call stages x to the device, runs the kernel, copies y back and waits.  Wall clock, PCIe included."""
+    import time
+    import numpy as np
+    from izwi_amd import capi
+    L = capi.lib()
+    bufs = [(mm, np.random.default_rng(1).standard_normal((m, k)).astype(np.float32), np.empty((m, n), np.float32))
+            for mm, n, k in weights]
+    total = sum(mm.qtensor.storage_size_in_bytes() + 4 * m * k + 4 * m * n for mm, n, k in weights)
+
+    def one_pass():
+        for mm, x, y in bufs:
+            rc = L.izwi_qmm_forward_f32(mm.qtensor._h, x.ctypes.data, m, y.ctypes.data, capi.HOST, None)
+            if rc:
+                capi.check(rc)
+    one_pass()
+    t0 = time.perf_counter()
+    for _ in range(passes):
+        one_pass()
+    dt = (time.perf_counter() - t0) / passes
+    return {"gbs": round(total / dt / 1e9, 1), "ms_per_step": round(dt * 1e3, 3), "calls_per_step": len(bufs),
+            "us_per_call": round(dt * 1e6 / len(bufs), 1)}
+
+
+def hbm_ceiling_extra(torch, gib=2, reps=10):
+    """Extra report: what plain streaming kernels reach on this GPU, beside the nominal 8 TB/s the roofline
+    is priced against: a device-to-device copy (bytes read + written) and a read-only reduction (torch's
+    kernels), `gib` GiB per pass, far beyond the caches."""
+    n = gib * (1 << 30) // 4
+    x = torch.ones(n, dtype=torch.float32, device="cuda")
+    y = torch.empty_like(x)
+    copy_ms = time_eager(torch, lambda: y.copy_(x), reps, 2)
+    read_ms = time_eager(torch, lambda: x.sum(), reps, 2)
+    out = {"copy_gbs": round(2 * n * 4 / (copy_ms * 1e-3) / 1e9, 1), "read_gbs": round(n * 4 / (read_ms * 1e-3) / 1e9, 1),
+           "gib": gib}
+    try:  # the runtime's own device-to-device copy
+        import ctypes as C
+        hip = C.CDLL("libamdhip64.so")
+        hip.hipMemcpyAsync.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
+        sp = torch.cuda.current_stream().cuda_stream
+        ms = time_eager(torch, lambda: hip.hipMemcpyAsync(y.data_ptr(), x.data_ptr(), n * 4, 3, sp), reps, 2)
+        out["hip_memcpy_d2d_gbs"] = round(2 * n * 4 / (ms * 1e-3) / 1e9, 1)
+    except OSError:
+        pass
+    del x, y
+    torch.cuda.empty_cache()
+    return out
+
+
 def neighbours_extra(torch, qa, steps=10, warmup=3):
     """Extra report (not `value`): the decode-step neighbours at Qwen3-8B shapes (32 query heads on
     8 kv heads, head_dim 128, hidden 4096, f32): microseconds per call in a HIP-graph replay and, for
@@ -625,6 +676,8 @@ def main():
             extras["decode_per_projection_calls" if args.calls == "grouped" else "decode_grouped_calls"] = {
                 "gbs": round(tb / (t * 1e-3) / 1e9, 1), "ms_per_step": round(t, 4), "calls_per_step": len(c)}
             del c, g
+            extras["decode_host_pointer_calls"] = host_pointer_extra(qa, weights, args.m)
+            extras["hbm_ceiling_measured"] = hbm_ceiling_extra(torch)
         except Exception as exc:  # extras never invalidate the headline number
             extras["decode_error"] = repr(exc)
     del weights
