@@ -435,7 +435,7 @@ def layer_stack_extra(torch, qa, oracle, dtype, steps=10, warmup=3):
         out[f"kv{kv_len}"] = {"ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1)}
         del caches, g
         torch.cuda.empty_cache()
-    out["launches_per_token"] = N_LAYERS_8B * 7 + 2
+    out["launches_per_token"] = N_LAYERS_8B * 7 + 3  # LM head with the norm, two for the argmax
     del layers, weights
     torch.cuda.empty_cache()
     return out

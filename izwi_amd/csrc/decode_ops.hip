@@ -269,6 +269,41 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ 
     }
 }
 
+// Long rows of few: blockIdx.y scans a chunk of the row into a (value, index) candidate, a second
+// launch merges the candidates (same rule, so the result is the one-launch kernel's).
+__global__ __launch_bounds__(256) void argmax_part_kernel(const float* __restrict__ x, int64_t n, int64_t chunk,
+                                                          float* __restrict__ pv, uint32_t* __restrict__ pi) {
+    __shared__ float vals[4];
+    __shared__ unsigned idxs[4];
+    const float* row = x + (int64_t)blockIdx.x * n;
+    const int64_t begin = (int64_t)blockIdx.y * chunk, end = begin + chunk < n ? begin + chunk : n;
+    float v = -INFINITY;
+    unsigned idx = 0xffffffffu;
+    for (int64_t i = begin + threadIdx.x; i < end; i += blockDim.x) {
+        const float t = row[i];
+        if (t > v || (idx == 0xffffffffu && !(t != t))) v = t, idx = (unsigned)i;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) argmax_merge(v, idx, __shfl_xor(v, o), (unsigned)__shfl_xor((int)idx, o));
+    if ((threadIdx.x & 63) == 0) vals[threadIdx.x >> 6] = v, idxs[threadIdx.x >> 6] = idx;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x >> 6); w++) argmax_merge(v, idx, vals[w], idxs[w]);
+        pv[(int64_t)blockIdx.x * gridDim.y + blockIdx.y] = v;
+        pi[(int64_t)blockIdx.x * gridDim.y + blockIdx.y] = idx;
+    }
+}
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ pv, const uint32_t* __restrict__ pi,
+                                                          int parts, uint32_t* __restrict__ out) {
+    float v = -INFINITY;
+    unsigned idx = 0xffffffffu;
+    for (int p = threadIdx.x; p < parts; p += 64)
+        argmax_merge(v, idx, pv[(int64_t)blockIdx.x * parts + p], pi[(int64_t)blockIdx.x * parts + p]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) argmax_merge(v, idx, __shfl_xor(v, o), (unsigned)__shfl_xor((int)idx, o));
+    if (threadIdx.x == 0) out[blockIdx.x] = idx == 0xffffffffu ? 0u : idx;
+}
+
 // ---- q/k norm + rotary + cache append, one token ---------------------------------------------
 // One wave per head: rows 0 .. heads-1 are q, then kv_heads rows of k, then kv_heads rows of v.
 // Lane l holds the pairs (p, p + half) for p = l, l + 64, ..: the norm's sum runs over the wave,
@@ -750,10 +785,24 @@ int izwi_argmax_f32(const float* logits, int64_t rows, int64_t n, uint32_t* out,
     Buf li, oo;
     OPS_TRY(li.in(logits, (size_t)rows * n * sizeof(float), mem_space));
     OPS_TRY(oo.out(out, (size_t)rows * sizeof(uint32_t), mem_space));
-    int threads = 64;
-    while (threads < 1024 && threads * 4 < n) threads *= 2;
-    argmax_kernel<<<(unsigned)rows, threads, 0, stream>>>((const float*)li.dev, n, (uint32_t*)oo.dev);
-    OPS_TRY(hipGetLastError());
+    if (n > 16384 && rows < 2 * (int64_t)n_cus) {
+        // too few rows to fill the GPU with one workgroup each: chunks of the row, then a merge
+        const int64_t chunk = 2048;
+        const int64_t parts = (n + chunk - 1) / chunk;
+        void* scratch = nullptr;
+        OPS_TRY(qmm_get_scratch(device, stream, (size_t)rows * parts * 8, &scratch));
+        float* pv = (float*)scratch;
+        uint32_t* pi = (uint32_t*)scratch + rows * parts;
+        argmax_part_kernel<<<dim3((unsigned)rows, (unsigned)parts), 256, 0, stream>>>((const float*)li.dev, n, chunk, pv, pi);
+        OPS_TRY(hipGetLastError());
+        argmax_final_kernel<<<(unsigned)rows, 64, 0, stream>>>(pv, pi, (int)parts, (uint32_t*)oo.dev);
+        OPS_TRY(hipGetLastError());
+    } else {
+        int threads = 64;
+        while (threads < 1024 && threads * 4 < n) threads *= 2;
+        argmax_kernel<<<(unsigned)rows, threads, 0, stream>>>((const float*)li.dev, n, (uint32_t*)oo.dev);
+        OPS_TRY(hipGetLastError());
+    }
     OPS_TRY(oo.finish(stream));
     return IZWI_QMM_OK;
 }

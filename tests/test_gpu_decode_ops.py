@@ -219,7 +219,7 @@ def test_qk_norm_rope_append_equals_the_separate_hooks(qa, oracle, heads, kv_hea
                                           kv_heads, d, 1e-6, kc.data_ptr(), kc.data_ptr(), vc.data_ptr(), cap, cap, None) == -1
 
 
-@pytest.mark.parametrize("rows,n", [(1, 151936), (4, 151936), (3, 1000), (2, 7), (1, 1), (5, 4097)])
+@pytest.mark.parametrize("rows,n", [(1, 151936), (4, 151936), (3, 1000), (2, 7), (1, 1), (5, 4097), (3, 20000), (2, 16385)])
 def test_argmax_on_device(qa, oracle, rows, n):
     x = oracle.randn(rows + n, (rows, n))
     if n > 20:
