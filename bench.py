@@ -407,8 +407,8 @@ def fused_and_q6k_extra(torch, qa, oracle, steps=10, warmup=3):
 def layer_stack_extra(torch, qa, oracle, dtype, steps=10, warmup=3):
     """Extra report (not `value`): one whole decode step of the Qwen3-8B stack composed from the library's
     calls (izwi_amd.qwen3_layer.Qwen3DecodeLayer: q|k|v group and gate/up with their RMSNorm and the
-    activation folded in, q/k norm + rotary + cache append, attention, o and down with the residual folded
-    in) plus the final norm folded into the LM head and the greedy argmax, f32 activations, HIP-graph replay, at several context lengths."""
+    activation folded in, attention with q/k norm + rotary + cache append inside its launch and the merge
+    of its splits, o and down with the residual folded in) plus the final norm folded into the LM head and the greedy argmax, f32 activations, HIP-graph replay, at several context lengths."""
     from izwi_amd.qwen3_layer import Qwen3DecodeLayer
     heads, kvh, d, hidden = 32, 8, 128, 4096
     weights = build_decode_weights(torch, qa, oracle, dtype, N_LAYERS_8B, True)
@@ -435,7 +435,7 @@ def layer_stack_extra(torch, qa, oracle, dtype, steps=10, warmup=3):
         out[f"kv{kv_len}"] = {"ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1)}
         del caches, g
         torch.cuda.empty_cache()
-    out["launches_per_token"] = N_LAYERS_8B * 7 + 3  # LM head with the norm, two for the argmax
+    out["launches_per_token"] = N_LAYERS_8B * 6 + 3  # LM head with the norm, two for the argmax
     del layers, weights
     torch.cuda.empty_cache()
     return out

@@ -84,6 +84,17 @@ int izwi_qk_norm_rope_append_f32(const float* q, const float* k, const float* v,
                                  int64_t head_dim, float eps, float* q_out, float* k_cache, float* v_cache,
                                  int64_t kv_capacity, int64_t pos, void* stream);
 
+/* The same sequence AND the attention behind it as one launch (two when the positions are split):
+ * the attention kernel norms and rotates its query heads and the new key itself, takes the new
+ * (key, value) as position `pos` and appends them to the caches on its way.  Arguments as
+ * izwi_qk_norm_rope_append_f32 (without q_out) and izwi_decode_gqa_attention_f32 with
+ * kv_len = pos + 1; out is `[num_heads, head_dim]`.  Results are those of the two calls bit for bit
+ * (the same arithmetic in the same order).  Device pointers only; head_dim 64, 128 or 256. */
+int izwi_decode_attention_step_f32(const float* q, const float* k, const float* v, const float* qk_weight,
+                                   const float* cos_sin, int64_t num_heads, int64_t num_kv_heads,
+                                   int64_t head_dim, float eps, float* k_cache, float* v_cache,
+                                   int64_t kv_capacity, int64_t pos, float scale, float* out, void* stream);
+
 /* `try_fused_decode_gqa_attention_with_kv_len(q, k, v, num_heads, num_kv_heads, head_dim, kv_len,
  * scale)` (kernels/mod.rs:199-225, metal.rs:2121-2193, shader metal.rs:307-381): attention of one
  * query token.  q is `[1, num_heads, 1, head_dim]`, k and v are `[1, num_kv_heads, kv_capacity,

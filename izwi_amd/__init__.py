@@ -9,6 +9,7 @@ missing or no GPU is present, calls raise.
 from .capi import QmmError, lib, library_path  # noqa: F401
 from .decode_ops import (  # noqa: F401
     argmax,
+    decode_attention_step,
     qk_norm_rope_append,
     try_fused_decode_gqa_attention,
     try_fused_decode_gqa_attention_with_kv_len,

@@ -77,6 +77,8 @@ PROTOTYPES = {
     "izwi_argmax_f32": (C.c_int, [_vp, _i64, _i64, _vp, C.c_int, _vp]),
     "izwi_qk_norm_rope_append_f32": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, C.c_float, _vp, _vp, _vp,
                                                _i64, _i64, _vp]),
+    "izwi_decode_attention_step_f32": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, C.c_float, _vp, _vp, _i64,
+                                                 _i64, C.c_float, _vp, _vp]),
     "izwi_decode_gqa_attention_f32": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, C.c_float, _vp,
                                                 C.c_int, _vp]),
     "izwi_moe_route": (C.c_int, [_vp, _i64, _i32, _i32, _vp, _vp, C.c_int, _vp]),

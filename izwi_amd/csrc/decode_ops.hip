@@ -12,6 +12,8 @@
 //    every 128-byte segment (coalesced), 32 rows are in flight per workgroup.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include <math.h>
 #include <stdlib.h>
 
@@ -379,6 +381,16 @@ struct AttnParams {
     int kv_len, chunk, splits; // split s covers positions [s * chunk, min(kv_len, (s + 1) * chunk))
     int64_t kv_capacity;
     float scale;
+    // PREP form (f32, the step of one new token): q, k_new and v_new are the projections' outputs;
+    // the kernel norms and rotates q and k_new itself (the arithmetic of qkv_prep_kernel), takes
+    // (k_new, v_new) as position kv_len - 1 and appends them to the caches
+    const float* k_new;
+    const float* v_new;
+    const float* qk_weight; // [2 * head_dim]
+    const float* cos_sin;   // [head_dim]: cos | sin of position kv_len - 1
+    float* k_append;
+    float* v_append;
+    float eps;
 };
 
 // e^x for x <= 0 on the hardware's exp2 (relative error about 2^-22; e^-inf = 0)
@@ -403,37 +415,21 @@ __device__ __forceinline__ float sum8(float v) {
 // HD = head_dim; G query heads of one kv head per workgroup.  Lane j of an 8-lane row group
 // holds, of a cache row and of the query heads, the 16-byte pieces j, j + 8, ..: elements
 // 8 EC i + EC j + c (i < NI, c < EC; EC = 4 for f32, 8 for f16).
-template <typename T, int HD, int G>
+template <typename T, int HD, int G, bool PREP = false>
 __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams<T> P) {
+    static_assert(!PREP || std::is_same<T, float>::value, "the one-token step is built for f32");
     constexpr int EC = kEC<T>, NI = HD / (8 * EC), E = EC * NI;
     __shared__ __attribute__((aligned(16))) float red[16][G][HD + 4]; // [.. HD): sums, [HD]: maximum, [HD + 1]: weight sum
+    __shared__ __attribute__((aligned(16))) float prep[PREP ? G + 1 : 1][PREP ? HD : 4]; // normed, rotated q heads, then k_new
     const int kvh = blockIdx.x, sp = blockIdx.y, h0 = kvh * P.group + blockIdx.z * G;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane & 7, slot = wave * 8 + (lane >> 3);
-
-    float qr[G][E];
-#pragma unroll
-    for (int g = 0; g < G; g++)
-#pragma unroll
-        for (int i = 0; i < NI; i++) {
-            float t[EC];
-            ld16<T>(P.q + (int64_t)(h0 + g) * HD + 8 * EC * i + EC * j, t);
-#pragma unroll
-            for (int c = 0; c < EC; c++) qr[g][EC * i + c] = t[c];
-        }
-    float m[G], l[G], acc[G][E];
-#pragma unroll
-    for (int g = 0; g < G; g++) {
-        m[g] = -INFINITY;
-        l[g] = 0.0f;
-#pragma unroll
-        for (int e = 0; e < E; e++) acc[g][e] = 0.0f;
-    }
     const int p0 = sp * P.chunk, p1 = min(P.kv_len, p0 + P.chunk);
+    const int pos = P.kv_len - 1;
+    const int p1c = PREP ? min(p1, pos) : p1; // PREP: the new position is not in the cache yet
     const T* kb = P.k + (int64_t)kvh * P.kv_capacity * HD + EC * j;
     const T* vb = P.v + (int64_t)kvh * P.kv_capacity * HD + EC * j;
-    for (int p = p0 + slot; p < p1; p += 32) {
-        float kr[E], vr[E];
+    auto load_row = [&](int p, float (&kr)[E], float (&vr)[E]) {
 #pragma unroll
         for (int i = 0; i < NI; i++) {
             float t[EC];
@@ -448,6 +444,79 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams<T> P) {
 #pragma unroll
             for (int c = 0; c < EC; c++) vr[EC * i + c] = t[c];
         }
+    };
+    // PREP: the first cache row is requested before the query is prepared, so that its latency
+    // runs beside the norm's
+    float kr0[PREP ? E : 1], vr0[PREP ? E : 1];
+    const bool first = PREP && p0 + slot < p1c;
+    if constexpr (PREP) {
+        if (first) load_row(p0 + slot, kr0, vr0);
+    }
+
+    if constexpr (PREP) {
+        // a wave per row (the group's q heads, then the kv head's new k), as qkv_prep_kernel does it
+        constexpr int half = HD / 2, NP = (half + 63) / 64;
+        for (int r = wave; r <= G; r += 4) {
+            const float* src = r < G ? reinterpret_cast<const float*>(P.q) + (int64_t)(h0 + r) * HD : P.k_new + (int64_t)kvh * HD;
+            const float* w = P.qk_weight + (r < G ? 0 : HD);
+            float x1[NP], x2[NP];
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NP; i++) {
+                const int p = lane + 64 * i;
+                x1[i] = p < half ? src[p] : 0.0f;
+                x2[i] = p < half ? src[half + p] : 0.0f;
+                sum += x1[i] * x1[i] + x2[i] * x2[i];
+            }
+            sum = wave_sum(sum);
+            const float scale = 1.0f / sqrtf(sum / (float)HD + P.eps);
+#pragma unroll
+            for (int i = 0; i < NP; i++) {
+                const int p = lane + 64 * i;
+                if (p < half) {
+                    const float n1 = x1[i] * scale * w[p], n2 = x2[i] * scale * w[half + p];
+                    const float c = P.cos_sin[p], sn = P.cos_sin[half + p];
+                    prep[r][p] = n1 * c - n2 * sn;
+                    prep[r][half + p] = n1 * sn + n2 * c;
+                }
+            }
+        }
+        __syncthreads();
+        // the workgroup whose positions end with the new one appends it to the caches; nobody reads
+        // that cache row in this launch
+        if (pos >= p0 && pos < p1 && blockIdx.z == 0) {
+            for (int t = threadIdx.x; t < HD; t += 256) {
+                P.k_append[((int64_t)kvh * P.kv_capacity + pos) * HD + t] = prep[G][t];
+                P.v_append[((int64_t)kvh * P.kv_capacity + pos) * HD + t] = P.v_new[(int64_t)kvh * HD + t];
+            }
+        }
+    }
+
+    float qr[G][E];
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            float t[EC];
+            if constexpr (PREP) {
+#pragma unroll
+                for (int c = 0; c < EC; c++) t[c] = prep[g][8 * EC * i + EC * j + c];
+            } else {
+                ld16<T>(P.q + (int64_t)(h0 + g) * HD + 8 * EC * i + EC * j, t);
+            }
+#pragma unroll
+            for (int c = 0; c < EC; c++) qr[g][EC * i + c] = t[c];
+        }
+    float m[G], l[G], acc[G][E];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        m[g] = -INFINITY;
+        l[g] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < E; e++) acc[g][e] = 0.0f;
+    }
+    // one position into the running softmax of every query head of the group
+    auto accumulate = [&](const float (&kr)[E], const float (&vr)[E]) {
 #pragma unroll
         for (int g = 0; g < G; g++) {
             float dot = 0.0f;
@@ -465,6 +534,28 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams<T> P) {
             l[g] += pe;
 #pragma unroll
             for (int e = 0; e < E; e++) acc[g][e] += pe * vr[e];
+        }
+    };
+    if constexpr (PREP) {
+        if (first) accumulate(kr0, vr0);
+    }
+    for (int p = p0 + slot + (PREP ? 32 : 0); p < p1c; p += 32) {
+        float kr[E], vr[E];
+        load_row(p, kr, vr);
+        accumulate(kr, vr);
+    }
+    if constexpr (PREP) {
+        // the new position, last of its row group as it would be from the cache
+        if (pos >= p0 && pos < p1 && ((pos - p0) & 31) == slot) {
+            float kr[E], vr[E];
+#pragma unroll
+            for (int i = 0; i < NI; i++)
+#pragma unroll
+                for (int c = 0; c < EC; c++) {
+                    kr[EC * i + c] = prep[G][8 * EC * i + EC * j + c];
+                    vr[EC * i + c] = P.v_new[(int64_t)kvh * HD + 8 * EC * i + EC * j + c];
+                }
+            accumulate(kr, vr);
         }
     }
     // Merge the 32 row groups of the workgroup: neighbours 8 lanes apart inside a 16-lane row by a
@@ -558,18 +649,34 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict
     }
 }
 
-template <typename T, int HD>
-hipError_t launch_attn_partial(const AttnParams<T>& P, int g, dim3 grid, hipStream_t stream) {
+template <typename T, int HD, bool PREP>
+hipError_t launch_attn_partial_form(const AttnParams<T>& P, int g, dim3 grid, hipStream_t stream) {
     if (g == 4) {
-        if constexpr (HD <= 128) attn_partial_kernel<T, HD, 4><<<grid, 256, 0, stream>>>(P);
+        if constexpr (HD <= 128) attn_partial_kernel<T, HD, 4, PREP><<<grid, 256, 0, stream>>>(P);
         else return hipErrorInvalidValue;
     } else if (g == 2) {
-        attn_partial_kernel<T, HD, 2><<<grid, 256, 0, stream>>>(P);
+        attn_partial_kernel<T, HD, 2, PREP><<<grid, 256, 0, stream>>>(P);
     } else {
-        attn_partial_kernel<T, HD, 1><<<grid, 256, 0, stream>>>(P);
+        attn_partial_kernel<T, HD, 1, PREP><<<grid, 256, 0, stream>>>(P);
     }
     return hipGetLastError();
 }
+template <typename T, int HD>
+hipError_t launch_attn_partial(const AttnParams<T>& P, int g, dim3 grid, hipStream_t stream) {
+    if constexpr (std::is_same<T, float>::value) {
+        if (P.k_new) return launch_attn_partial_form<T, HD, true>(P, g, grid, stream);
+    }
+    return launch_attn_partial_form<T, HD, false>(P, g, grid, stream);
+}
+
+// The extra inputs of the one-token step (see AttnParams)
+struct AttnPrep {
+    const float* k_new;
+    const float* v_new;
+    const float* qk_weight;
+    const float* cos_sin;
+    float eps;
+};
 
 
 template <typename T>
@@ -666,7 +773,7 @@ int rope_pair_impl(const T* q, const T* k, const T* cos_sin, int64_t batch, int6
 template <typename T>
 int decode_attention_impl(const T* q, const T* k, const T* v, int64_t num_heads,
                                   int64_t num_kv_heads, int64_t head_dim, int64_t kv_len, int64_t kv_capacity,
-                                  float scale, T* out, int mem_space, void* stream_) {
+                                  float scale, T* out, int mem_space, void* stream_, const AttnPrep* prep = nullptr) {
     if (int rc = check_space(mem_space)) return rc;
     if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || num_heads > 65535 || kv_len <= 0 ||
         kv_len > kv_capacity || kv_capacity > 0x3fffffff || head_dim <= 0)
@@ -719,6 +826,14 @@ int decode_attention_impl(const T* q, const T* k, const T* v, int64_t num_heads,
     P.splits = (int)splits;
     P.kv_capacity = kv_capacity;
     P.scale = scale;
+    P.k_new = P.v_new = P.qk_weight = P.cos_sin = nullptr;
+    P.k_append = P.v_append = nullptr;
+    P.eps = 0.0f;
+    if (prep) { // device pointers only (checked by the caller): the caches are written in place
+        P.k_new = prep->k_new, P.v_new = prep->v_new, P.qk_weight = prep->qk_weight, P.cos_sin = prep->cos_sin;
+        P.k_append = (float*)ki.dev, P.v_append = (float*)vi.dev;
+        P.eps = prep->eps;
+    }
     if (splits > 1) {
         void* scratch = nullptr;
         OPS_TRY(qmm_get_scratch(device, stream, (size_t)num_heads * splits * (head_dim + 2) * sizeof(float), &scratch));
@@ -827,6 +942,19 @@ int izwi_qk_norm_rope_append_f32(const float* q, const float* k, const float* v,
     qkv_prep_kernel<<<(unsigned)((rows + 3) / 4), 256, 0, (hipStream_t)stream_>>>(P);
     OPS_TRY(hipGetLastError());
     return IZWI_QMM_OK;
+}
+
+int izwi_decode_attention_step_f32(const float* q, const float* k, const float* v, const float* qk_weight,
+                                   const float* cos_sin, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                                   float eps, float* k_cache, float* v_cache, int64_t kv_capacity, int64_t pos,
+                                   float scale, float* out, void* stream) {
+    if (pos < 0 || pos >= kv_capacity)
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "decode_attention_step: position %lld of %lld", (long long)pos,
+                        (long long)kv_capacity);
+    if (!k || !v || !qk_weight || !cos_sin) return qmm_fail(IZWI_QMM_ERR_INVALID, "decode_attention_step: NULL buffer");
+    const AttnPrep prep{k, v, qk_weight, cos_sin, eps};
+    return decode_attention_impl<float>(q, k_cache, v_cache, num_heads, num_kv_heads, head_dim, pos + 1, kv_capacity,
+                                        scale, out, IZWI_QMM_DEVICE, stream, &prep);
 }
 
 int izwi_decode_gqa_attention_f32(const float* q, const float* k, const float* v, int64_t num_heads,

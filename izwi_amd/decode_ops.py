@@ -112,6 +112,28 @@ def qk_norm_rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qk_we
     return q_out
 
 
+def decode_attention_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, qk_weight: torch.Tensor,
+                          cos_sin: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pos: int, eps: float,
+                          scale: float) -> torch.Tensor:
+    """`qk_norm_rope_append` and the attention over positions 0 .. pos behind it as one call: the attention
+    kernel prepares its query heads and the new key itself and appends the new key / value to the caches.
+    Arguments as `qk_norm_rope_append`; returns the attention output [1, heads, 1, d]."""
+    from .capi import QmmError
+    if (not _ok(q, k, v, qk_weight, cos_sin, k_cache, v_cache) or q.dtype != torch.float32 or k_cache.dim() != 4
+            or tuple(v_cache.shape) != tuple(k_cache.shape)):
+        raise QmmError(-1, "decode_attention_step: contiguous f32 CUDA tensors on one device expected")
+    _, kv_heads, cap, d = k_cache.shape
+    heads = q.numel() // d
+    if (q.numel() != heads * d or k.numel() != kv_heads * d or v.numel() != kv_heads * d or qk_weight.numel() != 2 * d
+            or cos_sin.numel() != d):
+        raise QmmError(-1, "decode_attention_step: shapes do not match the caches")
+    out = torch.empty((1, heads, 1, d), dtype=torch.float32, device=q.device)
+    check(lib().izwi_decode_attention_step_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), qk_weight.data_ptr(),
+                                               cos_sin.data_ptr(), heads, kv_heads, d, eps, k_cache.data_ptr(),
+                                               v_cache.data_ptr(), cap, pos, scale, out.data_ptr(), _stream_ptr(q)))
+    return out
+
+
 def argmax(logits: torch.Tensor) -> torch.Tensor:
     """`logits.argmax(D::Minus1)` of the greedy samplers (qwen3/chat.rs:574-597): logits [..., n] f32 on the
     GPU -> int32 indices [...] (first index of the maximum), computed on the device."""

@@ -219,6 +219,36 @@ def test_qk_norm_rope_append_equals_the_separate_hooks(qa, oracle, heads, kv_hea
                                           kv_heads, d, 1e-6, kc.data_ptr(), kc.data_ptr(), vc.data_ptr(), cap, cap, None) == -1
 
 
+@pytest.mark.parametrize("heads,kv_heads,d,pos,cap", [
+    (32, 8, 128, 0, 4), (32, 8, 128, 5, 9), (32, 8, 128, 300, 512), (32, 8, 128, 4095, 4096), (32, 8, 128, 1000, 1001),
+    (8, 8, 64, 77, 100), (6, 3, 256, 130, 200), (4, 4, 128, 64, 65),
+])
+def test_decode_attention_step_equals_prep_then_attention(qa, oracle, heads, kv_heads, d, pos, cap):
+    """The one-call form (q/k norm, rotary and cache append inside the attention launch) against the two
+    calls it replaces, bit for bit (output and caches), and against the oracle's composition."""
+    print(f"attention step heads={heads} kv={kv_heads} d={d} pos={pos} cap={cap}", flush=True)
+    q, k, v = oracle.randn(1, (heads * d,)), oracle.randn(2, (kv_heads * d,)), oracle.randn(3, (kv_heads * d,))
+    w = oracle.randn(4, (2 * d,), mean=1.0, std=0.2)
+    ang = oracle.randn(5, (d // 2,)) * 3.0
+    cs = np.concatenate([np.cos(ang), np.sin(ang)]).astype(np.float32).reshape(1, d)
+    kc0, vc0 = oracle.randn(6, (1, kv_heads, cap, d)), oracle.randn(7, (1, kv_heads, cap, d))
+    kc_a, vc_a, kc_b, vc_b = dev(kc0), dev(vc0), dev(kc0), dev(vc0)
+    scale = d ** -0.5
+    q_rot = qa.qk_norm_rope_append(dev(q), dev(k), dev(v), dev(w), dev(cs), kc_a, vc_a, pos, 1e-6)
+    want = qa.try_fused_decode_gqa_attention_with_kv_len(q_rot, kc_a, vc_a, heads, kv_heads, d, pos + 1, scale)
+    got = qa.decode_attention_step(dev(q), dev(k), dev(v), dev(w), dev(cs), kc_b, vc_b, pos, 1e-6, scale)
+    assert got.shape == (1, heads, 1, d)
+    assert torch.equal(got, want) and torch.equal(kc_b, kc_a) and torch.equal(vc_b, vc_a)
+    if pos <= 300:
+        qn, kn = oracle.qk_rms_norm(q.reshape(1, 1, heads, d), k.reshape(1, 1, kv_heads, d), w, 1e-6)
+        qr, kr = oracle.rope_pair_bshd(qn, kn, cs)
+        kc0[0, :, pos], vc0[0, :, pos] = kr.reshape(kv_heads, d), v.reshape(kv_heads, d)
+        assert close(got, oracle.decode_gqa_attention(qr.reshape(1, heads, 1, d), kc0, vc0, pos + 1, scale))
+    from izwi_amd import capi
+    p = kc_b.data_ptr()
+    assert capi.lib().izwi_decode_attention_step_f32(p, p, p, p, p, heads, kv_heads, d, 1e-6, p, p, cap, cap, scale, p, None) == -1
+
+
 @pytest.mark.parametrize("rows,n", [(1, 151936), (4, 151936), (3, 1000), (2, 7), (1, 1), (5, 4097), (3, 20000), (2, 16385)])
 def test_argmax_on_device(qa, oracle, rows, n):
     x = oracle.randn(rows + n, (rows, n))

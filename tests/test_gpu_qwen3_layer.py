@@ -23,9 +23,11 @@ def silu(v):
     return v / (1.0 + np.exp(-v))
 
 
-@pytest.mark.parametrize("fuse_prep,fuse_norm", [(True, True), (False, False), (True, False)])
+@pytest.mark.parametrize("fuse_prep,fuse_norm,fuse_step", [(True, True, True), (False, False, False), (True, False, False),
+                                                           (True, True, False)])
 @pytest.mark.parametrize("hidden,heads,kv_heads,d,inter,steps", [(1024, 8, 2, 128, 3072, 5), (512, 8, 8, 64, 1024, 3)])
-def test_decode_layer_matches_the_oracle_composition(qa, oracle, hidden, heads, kv_heads, d, inter, steps, fuse_prep, fuse_norm):
+def test_decode_layer_matches_the_oracle_composition(qa, oracle, hidden, heads, kv_heads, d, inter, steps, fuse_prep, fuse_norm,
+                                                     fuse_step):
     from izwi_amd.qwen3_layer import Qwen3DecodeLayer
     shapes = {"q": (heads * d, hidden), "k": (kv_heads * d, hidden), "v": (kv_heads * d, hidden),
               "o": (hidden, heads * d), "gate": (inter, hidden), "up": (inter, hidden), "down": (hidden, inter)}
@@ -36,7 +38,8 @@ def test_decode_layer_matches_the_oracle_composition(qa, oracle, hidden, heads, 
     qk_w = oracle.randn(32, (2 * d,), mean=1.0, std=0.1)
     dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
     layer = Qwen3DecodeLayer(dev(w_in), dev(w_post), mm["q"], mm["k"], mm["v"], dev(qk_w), mm["o"], mm["gate"],
-                             mm["up"], mm["down"], heads, kv_heads, d, 1e-6, fuse_prep=fuse_prep, fuse_norm=fuse_norm)
+                             mm["up"], mm["down"], heads, kv_heads, d, 1e-6, fuse_prep=fuse_prep, fuse_norm=fuse_norm,
+                             fuse_step=fuse_step)
     cap = 16
     kc_d, vc_d = torch.zeros(1, kv_heads, cap, d, device="cuda"), torch.zeros(1, kv_heads, cap, d, device="cuda")
     kc, vc = np.zeros((1, kv_heads, cap, d), np.float32), np.zeros((1, kv_heads, cap, d), np.float32)
