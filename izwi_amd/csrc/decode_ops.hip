@@ -799,11 +799,12 @@ int decode_attention_impl(const T* q, const T* k, const T* v, int64_t num_heads,
     // query heads per workgroup: as many of the group as the register file takes
     int g = group % 4 == 0 && head_dim <= 128 ? 4 : (group % 2 == 0 ? 2 : 1);
     const int z = group / g;
-    // Enough workgroups for one per CU (IZWI_ATTN_WGS_PER_CU, tuning knob), at least 64 positions
-    // each (IZWI_ATTN_MIN_CHUNK): more splits only add merge work (measured: 2 per CU is 5-10 %
-    // slower between 4k and 16k positions, 4 per CU 30 %).
+    // Enough workgroups for one per CU (IZWI_ATTN_WGS_PER_CU, tuning knob), at least 32 positions
+    // each (IZWI_ATTN_MIN_CHUNK: one per row group of a workgroup, a single round of loads; 64 was
+    // 4 % slower on a whole decode step at 256 positions, 16 no faster): more splits only add
+    // merge work (measured: 2 per CU is 5-10 % slower between 4k and 16k positions, 4 per CU 30 %).
     static const int wgs_per_cu = [] { const char* e = getenv("IZWI_ATTN_WGS_PER_CU"); int v = e ? atoi(e) : 1; return v > 0 ? v : 1; }();
-    static const int min_chunk = [] { const char* e = getenv("IZWI_ATTN_MIN_CHUNK"); int v = e ? atoi(e) : 64; return v > 0 ? v : 64; }();
+    static const int min_chunk = [] { const char* e = getenv("IZWI_ATTN_MIN_CHUNK"); int v = e ? atoi(e) : 32; return v > 0 ? v : 32; }();
     const int64_t base_wgs = num_kv_heads * z;
     int64_t splits = (wgs_per_cu * (int64_t)n_cus + base_wgs - 1) / base_wgs;
     const int64_t max_splits = (kv_len + min_chunk - 1) / min_chunk;
