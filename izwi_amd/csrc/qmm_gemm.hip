@@ -948,7 +948,8 @@ hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uin
     if (L.dtype == QMM_Q6_K) {
         // more than 128 rows: the pipelined tiles; up to 128 the plain tile kernel, half-height
         // tiles when full ones would leave CUs idle
-        if (m > 128 && !getenv("IZWI_QMM_Q6K_PLAIN_TILES")) return launch_qt<QMM_Q6_K>(P, n_cus, stream);
+        static const bool plain_only = getenv("IZWI_QMM_Q6K_PLAIN_TILES") != nullptr; // comparison aid
+        if (m > 128 && !plain_only) return launch_qt<QMM_Q6_K>(P, n_cus, stream);
         const int64_t t128 = ((m + 127) / 128) * ((L.n + 127) / 128);
         if (t128 < (int64_t)n_cus && m > 64) return launch_tile<QMM_Q6_K, 64, 128>(P, 1, stream);
         return launch_tile<QMM_Q6_K, 128, 128>(P, 1, stream);

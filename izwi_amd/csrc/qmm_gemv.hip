@@ -638,7 +638,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
 // i.e. two 12-wave workgroups per CU.
 template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false, int IO = 0, bool NORM = false>
 __global__ __launch_bounds__(64 * kMaxWaves)
-__attribute__((amdgpu_waves_per_eu(NORM ? 4 : (ONESHOT && !GROUPED && MT == 1 && QT == QMM_Q4_K) ? 6 : 3))) void gemv_kernel(GemvParams P) {
+__attribute__((amdgpu_waves_per_eu(NORM ? 3 : (ONESHOT && !GROUPED && MT == 1 && QT == QMM_Q4_K) ? 6 : 3))) void gemv_kernel(GemvParams P) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int m_begin = 0, m_end = P.m;
     int64_t w_offset = 0;
