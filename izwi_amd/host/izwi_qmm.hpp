@@ -262,6 +262,23 @@ inline void decode_gqa_attention(const float* q, const float* k, const float* v,
     check(izwi_decode_gqa_attention_f32(q, k, v, num_heads, num_kv_heads, head_dim, kv_len, kv_capacity, scale, out,
                                         (int)space, stream));
 }
+// One token of `Qwen3Attention::forward` between the projections and o_proj (core.rs:1464-1575): q/k
+// norm, rotary embedding, cache append and the attention over positions 0 .. pos, device pointers.
+inline void decode_attention_step(const float* q, const float* k, const float* v, const float* qk_weight,
+                                  const float* cos_sin, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                                  float eps, float* k_cache, float* v_cache, int64_t kv_capacity, int64_t pos,
+                                  float scale, float* out, void* stream = nullptr) {
+    check(izwi_decode_attention_step_f32(q, k, v, qk_weight, cos_sin, num_heads, num_kv_heads, head_dim, eps, k_cache,
+                                         v_cache, kv_capacity, pos, scale, out, stream));
+}
+// The same without the attention: q to q_out, the new key / value into position `pos` of the caches.
+inline void qk_norm_rope_append(const float* q, const float* k, const float* v, const float* qk_weight,
+                                const float* cos_sin, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                                float eps, float* q_out, float* k_cache, float* v_cache, int64_t kv_capacity,
+                                int64_t pos, void* stream = nullptr) {
+    check(izwi_qk_norm_rope_append_f32(q, k, v, qk_weight, cos_sin, num_heads, num_kv_heads, head_dim, eps, q_out,
+                                       k_cache, v_cache, kv_capacity, pos, stream));
+}
 inline void argmax(const float* logits, int64_t rows, int64_t n, uint32_t* out, MemSpace space,
                    void* stream = nullptr) {
     check(izwi_argmax_f32(logits, rows, n, out, (int)space, stream));
