@@ -1103,14 +1103,14 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
                                             max_tiles, records, stream);
         if (e == hipSuccess)
             e = qmm_launch_gemv_mfma_grouped(G, gate->tiled, up->tiled, records, h, u, perm, offsets, seg, n_experts,
-                                             stream);
+                                             stream, gate->n_cus);
         // silu(gate) * up is applied while the down projection's input is quantized
         if (e == hipSuccess)
             e = qmm_launch_quantize_grouped(D.dtype, h, u, 1, inter, perm, offsets, seg, n_experts, max_tiles,
                                             records, stream);
         if (e == hipSuccess)
             e = qmm_launch_gemv_mfma_grouped(D, down->tiled, nullptr, records, y, nullptr, perm, offsets, seg,
-                                             n_experts, stream);
+                                             n_experts, stream, down->n_cus);
     } else {
         if (!segments_ready)
             e = qmm_launch_moe_segments(offsets, n_experts, QMM_MOE_SEG_ROWS, seg, seg_expert, max_segments, stream);

@@ -897,6 +897,83 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_stream_kernel(MfmaPa
     }
 }
 
+// Expert form: a workgroup belongs to one expert (blockIdx.y) and one of the two weight stacks
+// (blockIdx.z); up to TC of the expert's 16-row activation tiles, over all of k, sit in LDS, and
+// every wave walks row-tiles of the expert's matrix on its own: load a panel, multiply it with
+// every tile, next panel; no wave waits for another after the tiles have landed.  The weights are
+// read once per TC tiles (an expert with more tiles takes another pass), and the waves of a CU
+// keep several panels in flight where the one-shot form is one chain of round trips per workgroup.
+// Eight waves: two per SIMD, 256 registers each; the compiler requests the next panel while the
+// current one is multiplied, which the 170 registers of twelve waves do not hold.
+constexpr int kExpertWaves = 8;
+template <int QT, int TC>
+__global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(MfmaParams P) {
+    constexpr int UB = Unit<QT>::kBytes;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = P.nwr;
+    const int j = lane & 15, grp = lane >> 4;
+    const int s_units = P.slots >> 4;
+    const int e = blockIdx.y;
+    const int tile_begin = P.tile_offsets[e];
+    const int n_tiles = P.tile_offsets[e + 1] - tile_begin;
+    if (n_tiles == 0) return; // uniform for the workgroup: nobody reaches a barrier
+    const int pos_begin = P.offsets[e], pos_end = P.offsets[e + 1];
+    const uint8_t* wbase = (blockIdx.z ? P.w2 : P.w) + (int64_t)e * P.matrix_bytes;
+    float* yout = blockIdx.z ? P.y2 : P.y;
+    const uint8_t* records = P.ws + (size_t)tile_begin * P.k_units * UB;
+
+    for (int t0 = 0; t0 < n_tiles; t0 += TC) {
+        const int nt = min(TC, n_tiles - t0);
+        if (t0 != 0) lds_barrier(); // every wave is done with the previous tiles
+        issue_window_copy<QT>(records + (size_t)t0 * P.k_units * UB, smem, nt * P.k_units, wave, waves, lane);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        lds_barrier();
+        for (int rt = blockIdx.x * waves + wave; rt < P.row_tiles; rt += gridDim.x * waves) {
+            float acc[TC][4];
+#pragma unroll
+            for (int t = 0; t < TC; t++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
+            for (int kg = 0; kg < P.k_groups; kg++) {
+                WPanel<QT> p;
+                load_wpanel<QT>(p, wbase + (int64_t)(rt * P.k_groups + kg) * P.panel_bytes, P.slots, lane, j);
+#pragma unroll
+                for (int b = 0; b < WPanel<QT>::QC / 2; b++) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
+                const int unit0 = kg * s_units;
+                const int n_units = min(s_units, P.k_units - unit0);
+#pragma unroll
+                for (int t = 0; t < TC; t++) {
+                    if (t < nt) // uniform
+                        panel_dot<QT, false>(p, smem + ((size_t)t * P.k_units + unit0) * UB, n_units, j, grp, acc[t]);
+                }
+            }
+            const int row = rt * 16 + j;
+            if (row < P.n) {
+#pragma unroll
+                for (int t = 0; t < TC; t++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int mm = (t0 + t) * 16 + grp * 4 + r;
+                        if (t < nt && pos_begin + mm < pos_end) yout[(int64_t)P.perm[pos_begin + mm] * P.n + row] = acc[t][r];
+                    }
+            }
+        }
+    }
+}
+
+template <int QT, int TC>
+hipError_t launch_expert_form(const MfmaParams& P, dim3 grid, int waves, size_t lds, hipStream_t stream) {
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_expert_kernel<QT, TC>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+    }
+    gemv_mfma_expert_kernel<QT, TC><<<grid, 64 * waves, lds, stream>>>(P);
+    return hipGetLastError();
+}
+
 } // namespace
 
 namespace {
@@ -1059,7 +1136,7 @@ bool qmm_gemv_mfma_grouped_supported(const QmmLayout& L) { return L.k_groups <= 
 hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
                                         const void* records, float* y, float* y2, const int32_t* perm,
                                         const int32_t* offsets, const int32_t* tile_offsets,
-                                        int n_experts, hipStream_t stream) {
+                                        int n_experts, hipStream_t stream, int n_cus) {
     if (L.n == 0 || n_experts <= 0) return hipSuccess;
     if (!qmm_gemv_mfma_grouped_supported(L) || n_experts > 65535 || L.n > 0x3fffffff)
         return hipErrorInvalidValue;
@@ -1092,10 +1169,42 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     P.w2 = (const uint8_t*)tiled2;
     P.y2 = y2;
     P.n_weights = 0;
+    {
+        // the expert form where at least two activation tiles over all of k fit in LDS
+        static const bool expert_form = [] { const char* e = getenv("IZWI_QMM_MOE_EXPERT_FORM"); return !(e && e[0] == '0'); }();
+        const size_t tile_bytes = (size_t)L.k_units * unit_bytes(L.dtype);
+        // (Q6_K: two tiles at a time, four do not fit the registers)
+        const int tc = L.dtype != QMM_Q6_K && 4 * tile_bytes <= 150 * 1024 ? 4 : (2 * tile_bytes <= 150 * 1024 ? 2 : 0);
+        if (expert_form && tc && n_cus > 0) {
+            MfmaParams E = P;
+            const int stacks = tiled2 ? 2 : 1;
+            int waves = kExpertWaves;
+            if (waves > L.row_tiles) waves = (int)L.row_tiles;
+            int parts = (n_cus + n_experts * stacks - 1) / (n_experts * stacks);
+            const int max_parts = (int)((L.row_tiles + waves - 1) / waves);
+            if (parts > max_parts) parts = max_parts;
+            if (parts < 1) parts = 1;
+            E.nwr = waves; // the workgroup's waves (every wave walks all of k)
+            const dim3 grid((unsigned)parts, (unsigned)n_experts, (unsigned)stacks);
+            const size_t lds = (size_t)tc * tile_bytes;
+            if (L.dtype == QMM_Q4_K)
+                return tc == 4 ? launch_expert_form<QMM_Q4_K, 4>(E, grid, waves, lds, stream)
+                               : launch_expert_form<QMM_Q4_K, 2>(E, grid, waves, lds, stream);
+            if (L.dtype == QMM_Q6_K) return launch_expert_form<QMM_Q6_K, 2>(E, grid, waves, lds, stream);
+            return tc == 4 ? launch_expert_form<QMM_Q8_0, 4>(E, grid, waves, lds, stream)
+                           : launch_expert_form<QMM_Q8_0, 2>(E, grid, waves, lds, stream);
+        }
+    }
     const int waves = P.nwk * P.nwr;
     const size_t window_bytes = (size_t)P.window_units * unit_bytes(L.dtype);
-    P.double_buf = 2 * window_bytes + (size_t)waves * 256 * 4 <= 160 * 1024;
-    const size_t lds = (P.double_buf ? 2 : 1) * window_bytes + (size_t)waves * 256 * 4;
+    // A second window buffer hides the next tile's copy, but a workgroup of an expert is a short
+    // chain of dependent round trips and only a second workgroup on the CU fills its gaps: two
+    // buffers only where two workgroups still fit (IZWI_QMM_MOE_DOUBLE_BUF=1 / 0 forces the choice)
+    static const int force_double = [] { const char* e = getenv("IZWI_QMM_MOE_DOUBLE_BUF"); return e ? atoi(e) : -1; }();
+    const size_t red_bytes = (size_t)waves * 256 * 4;
+    P.double_buf = force_double >= 0 ? (force_double && 2 * window_bytes + red_bytes <= 160 * 1024)
+                                     : 2 * (2 * window_bytes + red_bytes) <= 160 * 1024;
+    const size_t lds = (P.double_buf ? 2 : 1) * window_bytes + red_bytes;
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     const void* fn = L.dtype == QMM_Q4_K
                          ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true>)

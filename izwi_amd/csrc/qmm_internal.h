@@ -222,7 +222,7 @@ bool qmm_gemv_mfma_grouped_supported(const QmmLayout& L);
 hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
                                         const void* records, float* y, float* y2, const int32_t* perm,
                                         const int32_t* offsets, const int32_t* tile_offsets,
-                                        int n_experts, hipStream_t stream);
+                                        int n_experts, hipStream_t stream, int n_cus);
 
 // Small batches: routing, sort and the segment tables (seg_rows rows per segment) of the grouped
 // decode kernel in one launch; same results as route + sort + segments.
