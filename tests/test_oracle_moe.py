@@ -54,3 +54,35 @@ def test_moe_forward_against_per_pair_composition(oracle):
             y = oracle.qmatmul(Q4_K, h.astype(np.float32), down[e * dn:(e + 1) * dn], hidden)
             want[t] += wts[t, s] * y[0]
     assert np.abs(out - want).max() <= 1e-3 * np.abs(want).max()
+
+
+def test_moe_forward_with_a_down_stack_of_its_own_type(oracle):
+    """Q4_K gate / up with a Q6_K down stack (the mix of a Q4_K_M file): the per-pair composition of
+    per-type products; with one type on both sides the mixed entry is the plain one."""
+    import sys
+    import os
+    sys.path.insert(0, os.path.dirname(__file__))
+    import np_ref
+    Q6_K = 14
+    E, top_k, hidden, inter, T = 4, 2, 512, 256, 3
+    gate = np.concatenate([oracle.quantize(Q4_K, oracle.randn(140 + e, (inter, hidden), std=0.02)) for e in range(E)])
+    up = np.concatenate([oracle.quantize(Q4_K, oracle.randn(160 + e, (inter, hidden), std=0.02)) for e in range(E)])
+    down6 = np_ref.random_q6_k_blocks(7, E * hidden, inter, d_scale=2e-3)
+    down4 = np.concatenate([oracle.quantize(Q4_K, oracle.randn(180 + e, (hidden, inter), std=0.02)) for e in range(E)])
+    x = oracle.randn(199, (T, hidden))
+    ids, wts = oracle.moe_route(oracle.randn(198, (T, E)), top_k)
+    assert np.array_equal(oracle.moe_forward(Q4_K, x, ids, wts, gate, up, down4, E, inter, down_dtype=Q4_K),
+                          oracle.moe_forward(Q4_K, x, ids, wts, gate, up, down4, E, inter))
+    out = oracle.moe_forward(Q4_K, x, ids, wts, gate, up, down6, E, inter, down_dtype=Q6_K)
+    gu = oracle.storage_bytes(Q4_K, inter, hidden)
+    dn = oracle.storage_bytes(Q6_K, hidden, inter)
+    want = np.zeros((T, hidden), np.float32)
+    for t in range(T):
+        for s in range(top_k):
+            e = int(ids[t, s])
+            g = oracle.qmatmul(Q4_K, x[t:t + 1], gate[e * gu:(e + 1) * gu], inter)
+            u = oracle.qmatmul(Q4_K, x[t:t + 1], up[e * gu:(e + 1) * gu], inter)
+            h = (g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64)))) * u
+            y = oracle.qmatmul(Q6_K, h.astype(np.float32), down6[e * dn:(e + 1) * dn], hidden)
+            want[t] += wts[t, s] * y[0]
+    assert np.abs(out - want).max() <= 1e-3 * np.abs(want).max()
