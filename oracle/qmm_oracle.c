@@ -34,7 +34,9 @@
  *                                    unpinned" against the crate's own bytes
  *   moe_* .......................... no counterpart in the reference (it has no
  *                                    MoE code); defined by the build's config and
- *                                    pinned by brute force (numpy stable argsort).
+ *                                    pinned by brute force (numpy stable argsort; the
+ *                                    forward, also with a down stack of its own block
+ *                                    type, by the per-pair composition of qmatmul).
  *
  * Compile with -ffp-contract=off: every f32 expression below is meant to round
  * after each operation, as the Rust original does.
