@@ -42,12 +42,57 @@ def gemv_bytes(dtype, n, k, m):
     return n * k * BPE[dtype] + 4 * m * k + 4 * m * n
 
 
-def make_blocks(oracle, dtype, n, k, seed, pool_rows=None):
-    """Seeded N(0, 0.02) weights quantized with the oracle's quantizer.  For very tall
-    matrices only `pool_rows` distinct rows are generated and repeated."""
+def synth_normal(seed, shape, std=1.0, mean=0.0):
+    """Seeded N(mean, std) f32 values: the benchmark's own input generator."""
+    import numpy as np
+    v = np.random.default_rng(seed).standard_normal(shape, dtype=np.float32)
+    return (v * np.float32(std) + np.float32(mean)).astype(np.float32)
+
+
+def quantize_synthetic(dtype, w):
+    """GGUF block bytes of a [rows, k] f32 matrix by a plain per-block min / max quantizer (valid Q8_0 /
+    Q4_K blocks of the right statistics for a benchmark; not candle's search for the best scales, which no
+    timed region depends on)."""
+    import numpy as np
+    rows, k = w.shape
+    if dtype == Q8_0:
+        x = w.reshape(-1, 32)
+        d = (np.abs(x).max(axis=1) / 127.0).astype(np.float16)
+        df = d.astype(np.float32)
+        q = np.where(df[:, None] > 0, np.rint(x / np.where(df > 0, df, 1)[:, None]), 0).clip(-127, 127).astype(np.int8)
+        out = np.empty((x.shape[0], 34), np.uint8)
+        out[:, :2] = d.view(np.uint8).reshape(-1, 2)
+        out[:, 2:] = q.view(np.uint8)
+        return out.reshape(-1)
+    assert dtype == Q4_K and k % 256 == 0
+    x = w.reshape(-1, 8, 32)                                  # super-block, sub-block, element
+    mn = np.minimum(x.min(axis=2), 0.0)
+    scale = (x.max(axis=2) - mn) / 15.0                       # per sub-block
+    d = (scale.max(axis=1) / 63.0).astype(np.float16)
+    dmin = ((-mn).max(axis=1) / 63.0).astype(np.float16)
+    df, dmf = d.astype(np.float32), dmin.astype(np.float32)
+    sc = np.where(df[:, None] > 0, np.rint(scale / np.where(df > 0, df, 1)[:, None]), 0).clip(0, 63).astype(np.uint8)
+    m = np.where(dmf[:, None] > 0, np.rint(-mn / np.where(dmf > 0, dmf, 1)[:, None]), 0).clip(0, 63).astype(np.uint8)
+    step = df[:, None] * sc.astype(np.float32)
+    q = np.where(step[:, :, None] > 0, np.rint((x + (dmf[:, None] * m)[:, :, None]) / np.where(step > 0, step, 1)[:, :, None]), 0)
+    q = q.clip(0, 15).astype(np.uint8)
+    out = np.empty((x.shape[0], 144), np.uint8)
+    out[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
+    out[:, 2:4] = dmin.view(np.uint8).reshape(-1, 2)
+    out[:, 4:8] = (sc[:, 0:4] & 63) | ((sc[:, 4:8] >> 4) << 6)       # the 6-bit scales and mins in 12 bytes
+    out[:, 8:12] = (m[:, 0:4] & 63) | ((m[:, 4:8] >> 4) << 6)
+    out[:, 12:16] = (sc[:, 4:8] & 15) | ((m[:, 4:8] & 15) << 4)
+    qq = q.reshape(-1, 4, 2, 32)                              # 64-element pair, low / high nibble, byte
+    out[:, 16:] = (qq[:, :, 0, :] | (qq[:, :, 1, :] << 4)).reshape(-1, 128)
+    return out.reshape(-1)
+
+
+def make_blocks(dtype, n, k, seed, pool_rows=None):
+    """Seeded N(0, 0.02) weights quantized to GGUF blocks.  For very tall matrices only `pool_rows`
+    distinct rows are generated and repeated."""
     import numpy as np
     rows = n if pool_rows is None else min(n, pool_rows)
-    blocks = oracle.quantize(dtype, oracle.randn(seed, (rows, k), std=0.02))
+    blocks = quantize_synthetic(dtype, synth_normal(seed, (rows, k), std=0.02))
     if rows < n:
         per_row = blocks.size // rows
         reps = -(-n // rows)
@@ -95,29 +140,29 @@ def time_eager(torch, fn, steps, warmup):
     return start.elapsed_time(end) / steps
 
 
-def build_decode_weights(torch, qa, oracle, dtype, n_layers, with_lm_head):
+def build_decode_weights(torch, qa, dtype, n_layers, with_lm_head):
     """Distinct device buffers for every projection of every layer (same seeded
     byte content per projection kind).  Returns [(QMatMul, n, k)]."""
     gg = qa.GgmlDType(dtype)
-    host = {name: make_blocks(oracle, dtype, n, k, 1000 + i) for i, (name, n, k) in enumerate(LAYER_8B)}
+    host = {name: make_blocks(dtype, n, k, 1000 + i) for i, (name, n, k) in enumerate(LAYER_8B)}
     weights = []
     for _layer in range(n_layers):
         for name, n, k in LAYER_8B:
             weights.append((qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, host[name], (n, k))), n, k))
     if with_lm_head:
         name, n, k = LM_HEAD_8B
-        blocks = make_blocks(oracle, dtype, n, k, 2000, pool_rows=16384)
+        blocks = make_blocks(dtype, n, k, 2000, pool_rows=16384)
         weights.append((qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, blocks, (n, k))), n, k))
     del host
     return weights
 
 
-def build_packed_weights(torch, qa, oracle, dtype, n_layers):
+def build_packed_weights(torch, qa, dtype, n_layers):
     """The same stack with q|k|v and gate|up row-concatenated into one weight each, as the
     reference's packed_qmatmul_from_qtensors does where it enables projection grouping:
     4 launches per layer instead of 7, identical weight bytes and outputs."""
     gg = qa.GgmlDType(dtype)
-    host = {name: (make_blocks(oracle, dtype, n, k, 1000 + i), n, k) for i, (name, n, k) in enumerate(LAYER_8B)}
+    host = {name: (make_blocks(dtype, n, k, 1000 + i), n, k) for i, (name, n, k) in enumerate(LAYER_8B)}
 
     def packed(names):
         return qa.packed_qmatmul_from_qtensors([(gg, host[nm][0], (host[nm][1], host[nm][2])) for nm in names])
@@ -129,14 +174,14 @@ def build_packed_weights(torch, qa, oracle, dtype, n_layers):
         weights.append((packed(("gate", "up")), 2 * 12288, 4096))
         weights.append((qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, host["down"][0], (4096, 12288))), 4096, 12288))
     name, n, k = LM_HEAD_8B
-    blocks = make_blocks(oracle, dtype, n, k, 2000, pool_rows=16384)
+    blocks = make_blocks(dtype, n, k, 2000, pool_rows=16384)
     weights.append((qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, blocks, (n, k))), n, k))
     return weights
 
 
-def decode_calls(torch, oracle, dtype, weights, m):
+def decode_calls(torch, dtype, weights, m):
     """(calls, algorithmic bytes) of one decode step with m activation rows."""
-    xs = {k: torch.from_numpy(oracle.randn(7 + k, (m, k))).cuda() for k in (4096, 12288)}
+    xs = {k: torch.from_numpy(synth_normal(7 + k, (m, k))).cuda() for k in (4096, 12288)}
     calls, total = [], 0.0
     for mm, n, k in weights:
         calls.append((mm, xs[k], torch.empty((m, n), dtype=torch.float32, device="cuda")))
@@ -163,11 +208,11 @@ def run_calls(qa, calls):
             capi.check(rc)
 
 
-def grouped_decode_calls(torch, oracle, dtype, weights, m):
+def grouped_decode_calls(torch, dtype, weights, m):
     """The same projections called the way Qwen3Attention::forward / Qwen3Mlp::forward call
     them (qwen3/core.rs:1599, 1787): qkv_proj.forward(x) and gate_up_proj.forward(x) are one
     call each (three / two separate weights), o and down single calls: 4 calls per layer."""
-    xs = {k: torch.from_numpy(oracle.randn(7 + k, (m, k))).cuda() for k in (4096, 12288)}
+    xs = {k: torch.from_numpy(synth_normal(7 + k, (m, k))).cuda() for k in (4096, 12288)}
     out = lambda n: torch.empty((m, n), dtype=torch.float32, device="cuda")
     calls, total = [], 0.0
     per_layer = len(LAYER_8B)
@@ -191,7 +236,7 @@ def cpu_baseline(oracle, dtype, m, budget_s=12.0):
     import numpy as np
     mats = []
     for i, (name, n, k) in enumerate(LAYER_8B):
-        mats.append((n, k, make_blocks(oracle, dtype, n, k, 1000 + i), oracle.randn(7 + k, (m, k))))
+        mats.append((n, k, make_blocks(dtype, n, k, 1000 + i), synth_normal(7 + k, (m, k))))
     layer_bytes = sum(gemv_bytes(dtype, n, k, m) for n, k, _, _ in mats)
     for n, k, b, x in mats[:2]:
         oracle.qmatmul(dtype, x, b, n)  # warm
@@ -215,7 +260,7 @@ def cpu_baseline(oracle, dtype, m, budget_s=12.0):
     }
 
 
-def prefill_extra(torch, qa, oracle, dtype, m, steps=20, warmup=5, only=None):
+def prefill_extra(torch, qa, dtype, m, steps=20, warmup=5, only=None):
     """TFLOP/s of the prefill kernel per projection (extra report, not `value`):
     bf16 activations in HBM, bf16 output, called through the C ABI on preallocated buffers."""
     from izwi_amd import capi
@@ -226,8 +271,8 @@ def prefill_extra(torch, qa, oracle, dtype, m, steps=20, warmup=5, only=None):
     for i, (name, n, k) in enumerate([LAYER_8B[0], LAYER_8B[1], LAYER_8B[4], LAYER_8B[6]]):
         if only is not None and name != only:
             continue
-        mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, make_blocks(oracle, dtype, n, k, 1000 + i, 4096), (n, k)))
-        x = torch.from_numpy(oracle.randn(3, (m, k))).cuda().to(torch.bfloat16)
+        mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, make_blocks(dtype, n, k, 1000 + i, 4096), (n, k)))
+        x = torch.from_numpy(synth_normal(3, (m, k))).cuda().to(torch.bfloat16)
         y = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
         sp = _stream_ptr()
 
@@ -357,7 +402,7 @@ def neighbours_extra(torch, qa, steps=10, warmup=3):
     return out
 
 
-def fused_and_q6k_extra(torch, qa, oracle, steps=10, warmup=3):
+def fused_and_q6k_extra(torch, qa, steps=10, warmup=3):
     """Extra report (not `value`): (a) the o / down projections of the 8B stack with bf16 activations in,
     residual added, bf16 out in one call each (izwi_qmm_forward_fused) against the same projections
     as f32 calls with torch's cast / add / cast kernels around them; (b) Q6_K projections of a
@@ -397,7 +442,7 @@ def fused_and_q6k_extra(torch, qa, oracle, steps=10, warmup=3):
     mats = []
     for i in range(8):
         mats.append(tuple(qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(
-            qa.GgmlDType.Q4K, make_blocks(oracle, Q4_K, 4096, k, 1003 if k == 4096 else 1006), (4096, k))) for k in (4096, 12288)))
+            qa.GgmlDType.Q4K, make_blocks(Q4_K, 4096, k, 1003 if k == 4096 else 1006), (4096, k))) for k in (4096, 12288)))
     xa, xh = torch.randn(1, 4096, device="cuda").bfloat16(), torch.randn(1, 12288, device="cuda").bfloat16()
     res = torch.randn(1, 4096, device="cuda").bfloat16()
 
@@ -431,14 +476,14 @@ def fused_and_q6k_extra(torch, qa, oracle, steps=10, warmup=3):
     return out
 
 
-def layer_stack_extra(torch, qa, oracle, dtype, steps=10, warmup=3):
+def layer_stack_extra(torch, qa, dtype, steps=10, warmup=3):
     """Extra report (not `value`): one whole decode step of the Qwen3-8B stack composed from the library's
     calls (izwi_amd.qwen3_layer.Qwen3DecodeLayer: q|k|v group and gate/up with their RMSNorm and the
     activation folded in, attention with q/k norm + rotary + cache append inside its launch and the merge
     of its splits, o and down with the residual folded in) plus the final norm folded into the LM head and the greedy argmax, f32 activations, HIP-graph replay, at several context lengths."""
     from izwi_amd.qwen3_layer import Qwen3DecodeLayer
     heads, kvh, d, hidden = 32, 8, 128, 4096
-    weights = build_decode_weights(torch, qa, oracle, dtype, N_LAYERS_8B, True)
+    weights = build_decode_weights(torch, qa, dtype, N_LAYERS_8B, True)
     per = len(LAYER_8B)
     ones = lambda n: torch.ones(n, device="cuda")  # noqa: E731
     layers = []
@@ -468,13 +513,13 @@ def layer_stack_extra(torch, qa, oracle, dtype, steps=10, warmup=3):
     return out
 
 
-def q4_k_m_mix_extra(torch, qa, oracle, m=1, steps=20, warmup=3):
+def q4_k_m_mix_extra(torch, qa, m=1, steps=20, warmup=3):
     """Extra report (not `value`): the decode stack with the tensor types of a Q4_K_M file of Qwen3-8B (the
     reference's default chat model): attn_v and ffn_down are Q6_K in half of the layers (the first and last
     eighth and every third layer between, as llama.cpp's Q4_K_M recipe picks them) and so is the output
-    matrix; everything else is Q4_K.  Q6_K weights are random block bytes with a finite scale (the oracle
-    has no Q6_K quantizer).  Same call structure as the headline; a q|k|v group with a Q6_K member is split by
-    type inside the library (q|k as one launch, v as another)."""
+    matrix; everything else is Q4_K.  Q6_K weights are random block bytes with a finite scale.  Same call
+    structure as the headline; a q|k|v group with a Q6_K member is split by type inside the library (q|k
+    as one launch, v as another)."""
     import numpy as np
     rng = np.random.default_rng(11)
 
@@ -486,7 +531,7 @@ def q4_k_m_mix_extra(torch, qa, oracle, m=1, steps=20, warmup=3):
 
     def more_bits(i, n):
         return i < n // 8 or i >= 7 * n // 8 or (i - n // 8) % 3 == 2
-    q4 = {name: make_blocks(oracle, Q4_K, n, k, 1000 + i) for i, (name, n, k) in enumerate(LAYER_8B)}
+    q4 = {name: make_blocks(Q4_K, n, k, 1000 + i) for i, (name, n, k) in enumerate(LAYER_8B)}
     q6 = {name: q6k_blocks(n, k) for name, n, k in LAYER_8B if name in ("v", "down")}
     shape = {name: (n, k) for name, n, k in LAYER_8B}
     bytes_per = {Q4_K: 144, 14: 210}
@@ -517,7 +562,7 @@ def q4_k_m_mix_extra(torch, qa, oracle, m=1, steps=20, warmup=3):
     return res
 
 
-def moe_extra(torch, qa, oracle, steps=50, warmup=5):
+def moe_extra(torch, qa, steps=50, warmup=5):
     """One MoE layer (route + sort + grouped expert MLP + combine, HIP-graph replay) at the
     Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, expert intermediate 768, Q4_K; as one
     call and as the three calls it is composed of."""
@@ -525,7 +570,7 @@ def moe_extra(torch, qa, oracle, steps=50, warmup=5):
     gg = qa.GgmlDType(Q4_K)
 
     def stack(n, k, seed):
-        one = make_blocks(oracle, Q4_K, 8 * n, k, seed)  # 8 distinct experts, repeated
+        one = make_blocks(Q4_K, 8 * n, k, seed)  # 8 distinct experts, repeated
         import numpy as np
         return qa.QTensor.from_blocks(gg, np.tile(one, e // 8), (e, n, k))
 
@@ -533,8 +578,8 @@ def moe_extra(torch, qa, oracle, steps=50, warmup=5):
     out = {}
     expert_bytes = 3 * inter * hidden * BPE[Q4_K]
     for t in (1, 16, 512):
-        x = torch.from_numpy(oracle.randn(40 + t, (t, hidden))).cuda()
-        logits_h = oracle.randn(50 + t, (t, e))
+        x = torch.from_numpy(synth_normal(40 + t, (t, hidden))).cuda()
+        logits_h = synth_normal(50 + t, (t, e))
         logits = torch.from_numpy(logits_h).cuda()
 
         def three_calls():
@@ -547,8 +592,8 @@ def moe_extra(torch, qa, oracle, steps=50, warmup=5):
         # the same layer as one call (izwi_moe_layer_f32): identical results
         us, g = time_graph(torch, lambda: experts.layer(logits, x, top_k), steps, warmup)
         us *= 1e3
-        ids_h, _ = oracle.moe_route(logits_h, top_k)
-        distinct = len(set(ids_h.reshape(-1).tolist()))
+        ids_d, _ = qa.moe_route(logits, top_k)  # the library's own routing: which experts the tokens touch
+        distinct = len(set(ids_d.cpu().numpy().reshape(-1).tolist()))
         rec = {"us": round(us, 1), "us_route_sort_forward_as_three_calls": round(us3 * 1e3, 1),
                "distinct_experts": distinct}
         # algorithmic bytes: the distinct experts' weights + x in + out; flops: 3 matmuls per pair
@@ -608,7 +653,6 @@ def main():
 
     import torch
     import izwi_amd as qa
-    from oracle import oracle  # cpu_baseline leg and seeded input generation only
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
@@ -621,7 +665,7 @@ def main():
 
     if args.prefill_only:
         m = args.m if args.m > 1 else 2048
-        tf = prefill_extra(torch, qa, oracle, dtype, m, args.steps, args.warmup, only=args.prefill_only)
+        tf = prefill_extra(torch, qa, dtype, m, args.steps, args.warmup, only=args.prefill_only)
         print(json.dumps({"prefill_only": args.prefill_only, "m": m, "dtype": "Q4_K" if dtype == Q4_K else "Q8_0",
                           "tflops": tf[args.prefill_only]}))
         return
@@ -633,9 +677,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    weights = build_decode_weights(torch, qa, oracle, dtype, args.layers, True)
+    weights = build_decode_weights(torch, qa, dtype, args.layers, True)
     make_calls = grouped_decode_calls if args.calls == "grouped" else decode_calls
-    calls, total_bytes = make_calls(torch, oracle, dtype, weights, args.m)
+    calls, total_bytes = make_calls(torch, dtype, weights, args.m)
     launches = len(calls)
     ms, _graph = time_graph(torch, lambda: run_calls(qa, calls), args.steps, args.warmup)
     gbs = total_bytes / (ms * 1e-3) / 1e9
@@ -691,19 +735,19 @@ def main():
             for m in (8, 16):
                 if m == args.m:
                     continue
-                c, tb = make_calls(torch, oracle, dtype, weights, m)
+                c, tb = make_calls(torch, dtype, weights, m)
                 t, g = time_graph(torch, lambda: run_calls(qa, c), max(5, args.steps // 5), 3)
                 extras[f"decode_gbs_m{m}"] = round(tb / (t * 1e-3) / 1e9, 1)
                 extras[f"decode_ms_per_step_m{m}"] = round(t, 4)
                 del c, g
             # the other call structure at the headline's m
             other = decode_calls if args.calls == "grouped" else grouped_decode_calls
-            c, tb = other(torch, oracle, dtype, weights, args.m)
+            c, tb = other(torch, dtype, weights, args.m)
             t, g = time_graph(torch, lambda: run_calls(qa, c), max(5, args.steps // 2), 3)
             extras["decode_per_projection_calls" if args.calls == "grouped" else "decode_grouped_calls"] = {
                 "gbs": round(tb / (t * 1e-3) / 1e9, 1), "ms_per_step": round(t, 4), "calls_per_step": len(c)}
             del c, g
-            c, tb = make_calls(torch, oracle, dtype, weights, args.m)
+            c, tb = make_calls(torch, dtype, weights, args.m)
             extras["decode_overlap_what_if"] = overlap_what_if_extra(torch, qa, c, tb)
             del c
             extras["decode_host_pointer_calls"] = host_pointer_extra(qa, weights, args.m)
@@ -715,8 +759,8 @@ def main():
 
     if not args.no_extras:
         try:
-            pw = build_packed_weights(torch, qa, oracle, dtype, args.layers)
-            c, tb = decode_calls(torch, oracle, dtype, pw, args.m)
+            pw = build_packed_weights(torch, qa, dtype, args.layers)
+            c, tb = decode_calls(torch, dtype, pw, args.m)
             t, g = time_graph(torch, lambda: run_calls(qa, c), max(5, args.steps // 2), 3)
             extras["decode_packed_qkv_gateup"] = {
                 "gbs": round(tb / (t * 1e-3) / 1e9, 1), "ms_per_step": round(t, 4), "launches_per_step": len(c),
@@ -729,8 +773,8 @@ def main():
         try:
             # the other block format of the configuration on the same stack and call structure
             other_dtype = Q8_0 if dtype == Q4_K else Q4_K
-            ow = build_decode_weights(torch, qa, oracle, other_dtype, args.layers, True)
-            c, tb = make_calls(torch, oracle, other_dtype, ow, args.m)
+            ow = build_decode_weights(torch, qa, other_dtype, args.layers, True)
+            c, tb = make_calls(torch, other_dtype, ow, args.m)
             t, g = time_graph(torch, lambda: run_calls(qa, c), max(5, args.steps // 2), 3)
             extras["decode_q8_0_8b_stack" if other_dtype == Q8_0 else "decode_q4k_8b_stack"] = {
                 "gbs": round(tb / (t * 1e-3) / 1e9, 1), "ms_per_step": round(t, 4),
@@ -741,7 +785,7 @@ def main():
         except Exception as exc:
             extras["decode_other_dtype_error"] = repr(exc)
         try:
-            extras["moe_30b_a3b_q4k"] = moe_extra(torch, qa, oracle)
+            extras["moe_30b_a3b_q4k"] = moe_extra(torch, qa)
         except Exception as exc:
             extras["moe_error"] = repr(exc)
         try:
@@ -749,22 +793,22 @@ def main():
         except Exception as exc:
             extras["neighbours_error"] = repr(exc)
         try:
-            extras["decode_q4_k_m_mix_8b_stack"] = q4_k_m_mix_extra(torch, qa, oracle, 1)
-            extras["decode_q4_k_m_mix_8b_stack_m16"] = q4_k_m_mix_extra(torch, qa, oracle, 16)
+            extras["decode_q4_k_m_mix_8b_stack"] = q4_k_m_mix_extra(torch, qa, 1)
+            extras["decode_q4_k_m_mix_8b_stack_m16"] = q4_k_m_mix_extra(torch, qa, 16)
         except Exception as exc:
             extras["q4_k_m_mix_error"] = repr(exc)
         try:
-            extras["qwen3_8b_decode_step_all_calls"] = layer_stack_extra(torch, qa, oracle, dtype)
+            extras["qwen3_8b_decode_step_all_calls"] = layer_stack_extra(torch, qa, dtype)
         except Exception as exc:
             extras["layer_stack_error"] = repr(exc)
         try:
-            extras["fused_call_and_q6k"] = fused_and_q6k_extra(torch, qa, oracle)
+            extras["fused_call_and_q6k"] = fused_and_q6k_extra(torch, qa)
         except Exception as exc:
             extras["fused_q6k_error"] = repr(exc)
         try:
-            extras["prefill_tflops_m2048_q4k"] = prefill_extra(torch, qa, oracle, Q4_K, 2048)
-            extras["prefill_tflops_m2048_q8_0"] = prefill_extra(torch, qa, oracle, Q8_0, 2048)
-            extras["prefill_tflops_m512_q4k"] = prefill_extra(torch, qa, oracle, Q4_K, 512)
+            extras["prefill_tflops_m2048_q4k"] = prefill_extra(torch, qa, Q4_K, 2048)
+            extras["prefill_tflops_m2048_q8_0"] = prefill_extra(torch, qa, Q8_0, 2048)
+            extras["prefill_tflops_m512_q4k"] = prefill_extra(torch, qa, Q4_K, 512)
             best = max(extras["prefill_tflops_m2048_q4k"].values())
             extras["prefill_best_frac_of_bf16_peak"] = round(best / BF16_PEAK_TFLOPS, 4)
         except Exception as exc:  # extras never invalidate the headline number
@@ -773,6 +817,7 @@ def main():
         result["extras"] = extras
 
     if not args.no_cpu_baseline:
+        from oracle import oracle  # the checker, timed here as the CPU baseline; no other leg touches it
         result["cpu_baseline"] = cpu_baseline(oracle, dtype, args.m)
 
     print(json.dumps(result))

@@ -1170,8 +1170,10 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     P.y2 = y2;
     P.n_weights = 0;
     {
-        // the expert form where at least two activation tiles over all of k fit in LDS
-        static const bool expert_form = [] { const char* e = getenv("IZWI_QMM_MOE_EXPERT_FORM"); return !(e && e[0] == '0'); }();
+        // the expert form (IZWI_QMM_MOE_EXPERT_FORM=1; off by default: measured no faster than the one-shot
+        // form once the experts' tile counts are uneven) where at least two activation tiles over all of
+        // k fit in LDS
+        static const bool expert_form = [] { const char* e = getenv("IZWI_QMM_MOE_EXPERT_FORM"); return e && e[0] == '1'; }();
         const size_t tile_bytes = (size_t)L.k_units * unit_bytes(L.dtype);
         // (Q6_K: two tiles at a time, four do not fit the registers)
         const int tc = L.dtype != QMM_Q6_K && 4 * tile_bytes <= 150 * 1024 ? 4 : (2 * tile_bytes <= 150 * 1024 ? 2 : 0);
@@ -1180,7 +1182,8 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
             const int stacks = tiled2 ? 2 : 1;
             int waves = kExpertWaves;
             if (waves > L.row_tiles) waves = (int)L.row_tiles;
-            int parts = (n_cus + n_experts * stacks - 1) / (n_experts * stacks);
+            static const int wgs_per_cu = [] { const char* e = getenv("IZWI_QMM_MOE_EXPERT_WGS_PER_CU"); int v = e ? atoi(e) : 3; return v > 0 ? v : 3; }();
+            int parts = (wgs_per_cu * n_cus + n_experts * stacks - 1) / (n_experts * stacks);
             const int max_parts = (int)((L.row_tiles + waves - 1) / waves);
             if (parts > max_parts) parts = max_parts;
             if (parts < 1) parts = 1;
