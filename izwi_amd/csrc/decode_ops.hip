@@ -539,10 +539,24 @@ __global__ __launch_bounds__(256) void attn_partial_kernel(AttnParams<T> P) {
     if constexpr (PREP) {
         if (first) accumulate(kr0, vr0);
     }
-    for (int p = p0 + slot + (PREP ? 32 : 0); p < p1c; p += 32) {
-        float kr[E], vr[E];
-        load_row(p, kr, vr);
-        accumulate(kr, vr);
+    {
+        // the next row of the group is requested before the current one is used (two register sets,
+        // taken in turns), rows in rising order as before
+        float ka[E], va[E], kb2[E], vb2[E];
+        int pa = p0 + slot + (PREP ? 32 : 0);
+        bool have_a = pa < p1c;
+        if (have_a) load_row(pa, ka, va);
+        while (have_a) {
+            const int pb = pa + 32;
+            const bool have_b = pb < p1c;
+            if (have_b) load_row(pb, kb2, vb2);
+            accumulate(ka, va);
+            if (!have_b) break;
+            pa = pb + 32;
+            have_a = pa < p1c;
+            if (have_a) load_row(pa, ka, va);
+            accumulate(kb2, vb2);
+        }
     }
     if constexpr (PREP) {
         // the new position, last of its row group as it would be from the cache
