@@ -159,7 +159,9 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
  * activations, y_i = QMatMul_i.forward(x), bit-identical to n_weights calls of
  * izwi_qmm_forward_f32.  The weights must share k; with equal block types the decode
  * sizes run as one kernel launch (m <= 2) or share one activation quantization
- * (m <= 64).  n_weights <= 4. */
+ * (m <= 64); members of several block types (attn_q / attn_k in Q4_K beside attn_v in
+ * Q6_K, as Q4_K_M files have them) are grouped by type, one such launch per type.
+ * n_weights <= 4. */
 int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_weights,
                                const float* x, int64_t m, float* const* ys, int mem_space,
                                void* stream);
