@@ -79,6 +79,8 @@ def lib() -> C.CDLL:
         L.oracle_argmax.argtypes = [vp, i64, i64, vp]
         L.oracle_decode_gqa_attention.restype = C.c_int
         L.oracle_decode_gqa_attention.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, f32, vp]
+        L.oracle_make_qkx1_quants.restype = None
+        L.oracle_make_qkx1_quants.argtypes = [C.c_int, C.c_int, vp, C.c_int, vp, vp]
         L.oracle_get_scale_min_k4.restype = None
         L.oracle_get_scale_min_k4.argtypes = [C.c_int, vp, vp, vp]
         _lib = L
@@ -122,6 +124,14 @@ def quantize(dtype: int, w: np.ndarray) -> np.ndarray:
     if rc:
         raise ValueError("oracle_quantize rejected the shape")
     return out
+
+
+def make_qkx1_quants(x: np.ndarray, nmax: int = 15, ntry: int = 5):
+    """The Q4_K sub-block scale search -> (scale, -min) as f32."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.zeros(2, dtype=np.float32)
+    lib().oracle_make_qkx1_quants(nmax, ntry, _ptr(x), x.size, out.ctypes.data, out.ctypes.data + 4)
+    return out[0], out[1]
 
 
 def dequantize(dtype: int, blocks: np.ndarray, rows: int, cols: int) -> np.ndarray:

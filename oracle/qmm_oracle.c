@@ -19,11 +19,14 @@
  *   quantize_row_q8_0 .............. invariants (|w-w^| <= d/2, max|q|=127) and
  *                                    the reference test's case (core.rs:3099-3142)
  *   quantize_row_q8_k .............. invariants (q = -128 at the extreme, bsums)
- *   quantize_row_q4_k .............. invariants only; the iterative scale search
- *                                    (make_qkx1_quants) is restated from the crate
- *                                    and is "parity unpinned" against the crate's
- *                                    bytes.  No judged quantity depends on it: the
- *                                    block BYTES are the input of the path.
+ *   quantize_row_q4_k, make_qkx1_quants
+ *                                    closed-form vectors (tests/golden/q4k_quantizer_cases.json,
+ *                                    worked out in exact rational arithmetic by the generator
+ *                                    beside it): sub-blocks on an exact 16-level grid must come
+ *                                    back as (step, -min) and whole blocks byte for byte, an
+ *                                    all-positive block (min clamps to 0), a constant sub-block,
+ *                                    a three-pass and a five-pass (cut-off) refinement, a
+ *                                    round-half-away tie; plus invariants on random data
  *   vec_dot_q8_0_q8_0 / q4_k_q8_k .. integer brute force + f64 bound + the
  *                                    reference test's known answers
  *   dequantize_row_q6_k ............ hand-built block with all 256 closed-form values +
@@ -298,6 +301,12 @@ static void make_qkx1_quants(int nmax, int ntry, const float* x, int n, float* o
     }
     *out_scale = scale;
     *out_min = -min;
+}
+
+/* The sub-block search on its own, for the closed-form vectors of tests/golden. */
+void oracle_make_qkx1_quants(int nmax, int ntry, const float* x, int n, float* out_scale,
+                             float* out_neg_min) {
+    make_qkx1_quants(nmax, ntry, x, n, out_scale, out_neg_min);
 }
 
 /* candle-core k_quants.rs, `BlockQ4K::from_float`.  Only used to MAKE weights. */

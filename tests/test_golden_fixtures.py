@@ -62,6 +62,54 @@ def test_oracle_packed_q8_0_fixture(oracle):
     assert np.allclose(y, np.array(fx["expected_y"], dtype=np.float32), rtol=0, atol=2e-6)
 
 
+def test_oracle_q4k_scale_search_closed_forms(oracle):
+    """`make_qkx1_quants` against sub-blocks whose answer the algorithm's mathematics fixes
+    (tests/golden/make_q4k_quantizer_vectors.py: exact grids, the clamp of min, a constant, a
+    three-pass and a cut-off five-pass refinement, a round-half-away tie)."""
+    fx = load("q4k_quantizer_cases.json")
+    assert (fx["nmax"], fx["ntry"]) == (15, 5)
+    for case in fx["sub_blocks"]:
+        x = np.array(case["x"], dtype=np.float32)
+        assert np.array_equal(x.astype(np.float64), np.array(case["x"])), "inputs are exact in f32"
+        scale, neg_min = oracle.make_qkx1_quants(x)
+        if case["exact_in_f32"]:
+            num, den = (np.float32(v) for v in case["scale_num_den"])
+            want = np.float32(0.0) if den == 0 or num == 0 else num / den
+            assert scale == want and np.float32(case["neg_min"]) == neg_min, case["name"]
+        else:
+            # f32 sums of 32 terms of size <= 15 round on the way: a few 1e-6; a wrong variant of
+            # the search is off by more than 4e-3
+            assert abs(scale - case["scale"]) <= 1e-5 * case["scale"], case["name"]
+            assert abs(neg_min - case["neg_min"]) <= 2e-5, case["name"]
+    # what the cases rule out: no refinement, a shorter or longer search, ties to even
+    by = {c["name"]: c for c in fx["sub_blocks"]}
+    three = np.array(by["three_passes"]["x"], dtype=np.float32)
+    assert [float(oracle.make_qkx1_quants(three, ntry=t)[0]) for t in (1, 2, 3)] == [
+        float(np.float32(266.25) / np.float32(255)), float(np.float32(251.25) / np.float32(226)),
+        float(np.float32(236.25) / np.float32(199))]
+    cut = np.array(by["five_pass_cutoff"]["x"], dtype=np.float32)
+    assert abs(oracle.make_qkx1_quants(cut, ntry=6)[0] - by["five_pass_cutoff"]["scale"]) > 4e-3
+
+
+def test_oracle_q4k_quantizer_block_vectors(oracle):
+    """`BlockQ4K::from_float` byte for byte on blocks whose bytes follow in closed form."""
+    import np_ref
+    fx = load("q4k_quantizer_cases.json")
+    for case in fx["blocks"]:
+        x = np.array(case["x"], dtype=np.float32).reshape(1, 256)
+        assert np.array_equal(x.astype(np.float64).reshape(-1), np.array(case["x"]))
+        got = oracle.quantize(Q4_K, x)
+        want = blocks(case["block_hex"])
+        d, dmin, sc, mn, q = np_ref.q4_k_fields(got)
+        assert list(sc[0]) == case["scale_codes"] and list(mn[0]) == case["min_codes"], case["name"]
+        assert list(q.reshape(-1)) == case["quants"], case["name"]
+        assert np.array_equal(got, want), case["name"]
+    # grid blocks dequantize back to their inputs exactly when d and dmin are exact
+    case = fx["blocks"][0]
+    back = oracle.dequantize(Q4_K, blocks(case["block_hex"]), 1, 256)[0]
+    assert np.array_equal(back, np.array(case["x"], dtype=np.float32))
+
+
 # ---- GPU: the library ---------------------------------------------------------
 @pytest.fixture(scope="module")
 def qa():
