@@ -21,9 +21,20 @@
  *     IZWI_QMM_HOST (ordinary host memory; the library stages it and the call
  *     is synchronous).
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
- *   - all entry points are re-entrant; a weight handle is immutable after
- *     creation and may be shared by concurrent callers (the reference calls
- *     forward from several threads, engine/executor/dispatch.rs:150-204).
+ *   - all entry points may be called from several host threads at once; a
+ *     weight handle is immutable after creation and may be shared by
+ *     concurrent callers (the reference calls forward from several threads,
+ *     engine/executor/dispatch.rs:150-204, backends/policy.rs:28-30).  Calls
+ *     that need device scratch (m >= 3, split-k prefill, MoE, split attention)
+ *     take their stream's scratch buffer for the duration of the call: two
+ *     threads calling on the SAME stream (NULL included) are serialised while
+ *     one of them queues its launches, and the stream then runs the two calls
+ *     one after the other; calls on different streams neither wait nor share.
+ *     The scratch of a stream only grows; an outgrown buffer stays allocated
+ *     until the process ends (queued work and captured graphs may still
+ *     address it).  It cannot grow while its stream is being captured into a
+ *     HIP graph: such a call fails with IZWI_QMM_ERR_HIP; reserve beforehand
+ *     (izwi_qmm_scratch_reserve, or one eager call of the same size).
  *   - there is no CPU fallback: without a usable HIP device every call fails
  *     with IZWI_QMM_ERR_NO_DEVICE.
  */
@@ -133,6 +144,17 @@ void izwi_qmm_weight_destroy(izwi_qmm_weight* w);
 /* `QTensor::{dtype, shape}`. */
 int izwi_qmm_weight_get_info(const izwi_qmm_weight* w, izwi_qmm_weight_info* out);
 
+/* Arithmetic of the f32 / fused forward calls beyond 64 activation rows, process-wide (see
+ * izwi_qmm_forward_f32).  No counterpart in the reference, whose CPU path has one arithmetic. */
+typedef enum izwi_qmm_large_m { IZWI_QMM_LARGE_M_BF16 = 0, IZWI_QMM_LARGE_M_INT8 = 1 } izwi_qmm_large_m;
+int izwi_qmm_set_large_m_arithmetic(int mode);
+int izwi_qmm_get_large_m_arithmetic(void);
+
+/* Grows the scratch buffer of (current device, stream) to at least `bytes` now, so that later
+ * calls on that stream allocate nothing (needed before the stream is captured into a HIP graph).
+ * No counterpart in the reference. */
+int izwi_qmm_scratch_reserve(uint64_t bytes, void* stream);
+
 /* `QTensor::data()` (qwen3/core.rs:855,870): the original GGUF block bytes,
  * byte-identical to what weight_create was given. */
 int izwi_qmm_weight_data(const izwi_qmm_weight* w, void* out_blocks, uint64_t nbytes,
@@ -146,11 +168,22 @@ int izwi_qmm_dequantize_f32(const izwi_qmm_weight* w, float* out, int mem_space,
 
 /* `QMatMul::forward(x)` for f32 activations (qwen3/core.rs:812; the reference
  * always hands f32 to the op on accelerators, qwen3/core.rs:772-789).
- * x is `[m, k]` row-major contiguous, y is `[m, n]`.  Any m >= 0; m <= 64 runs
- * the fused decode kernel, larger m the tiled MFMA kernel.  Activations are
- * quantized on chip to the weight type's dot type exactly as candle-core does
- * (Q8_0 -> Q8_0 blocks, Q4_K and Q6_K -> Q8_K blocks), so results agree with the
- * reference's CPU path up to f32 summation order. */
+ * x is `[m, k]` row-major contiguous, y is `[m, n]`.  Any m >= 0.
+ * m <= 64: activations are quantized on chip to the weight type's dot type
+ * exactly as candle-core does (Q8_0 -> Q8_0 blocks, Q4_K and Q6_K -> Q8_K
+ * blocks) and multiplied as integers, so results agree with the reference's
+ * CPU path up to f32 summation order (about 1e-6 of max|y|).
+ * m > 64 (prefill sizes) is ANOTHER arithmetic by default: x is rounded to
+ * bf16, the weights are dequantized to bf16, products run on the bf16 matrix
+ * cores with f32 accumulation; the result differs from the reference's by up
+ * to about 5e-3 of max|y| (the reference's own int8 activation rounding is
+ * of that size; the stated bound is 1e-2).  A caller that wants the
+ * reference's arithmetic at every m selects it with
+ * izwi_qmm_set_large_m_arithmetic(IZWI_QMM_LARGE_M_INT8) or the environment
+ * variable IZWI_QMM_LARGE_M=int8: rows then run 64 at a time through the
+ * integer kernel (slower at prefill sizes: the weights are streamed once per
+ * 64 rows).  izwi_qmm_forward_group_f32, izwi_qmm_forward_gate_up_silu_f32,
+ * izwi_qmm_forward_fused and the *_normed_* calls follow the same rule. */
 int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, float* y,
                          int mem_space, void* stream);
 

@@ -86,6 +86,9 @@ PROTOTYPES = {
     "izwi_moe_layer_f32": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _vp, _vp, _vp, C.c_int, _vp]),
     "izwi_moe_forward_f32": (C.c_int, [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _vp, _vp,
                                        C.c_int, _vp]),
+    "izwi_qmm_set_large_m_arithmetic": (C.c_int, [C.c_int]),
+    "izwi_qmm_get_large_m_arithmetic": (C.c_int, []),
+    "izwi_qmm_scratch_reserve": (C.c_int, [_u64, _vp]),
     "izwi_qmm_profile_enable": (C.c_int, [C.c_int]),
     "izwi_qmm_profile_snapshot_get": (C.c_int, [C.POINTER(ProfileSnapshot)]),
     "izwi_qmm_profile_reset": (C.c_int, []),

@@ -849,6 +849,7 @@ int decode_attention_impl(const T* q, const T* k, const T* v, int64_t num_heads,
         P.k_append = (float*)ki.dev, P.v_append = (float*)vi.dev;
         P.eps = prep->eps;
     }
+    QmmCallScope call; // the split partials stay this call's until the merge is queued
     if (splits > 1) {
         void* scratch = nullptr;
         OPS_TRY(qmm_get_scratch(device, stream, (size_t)num_heads * splits * (head_dim + 2) * sizeof(float), &scratch));
@@ -904,6 +905,7 @@ int izwi_rope_pair_bshd_f16(const uint16_t* q, const uint16_t* k, const uint16_t
 }
 
 int izwi_argmax_f32(const float* logits, int64_t rows, int64_t n, uint32_t* out, int mem_space, void* stream_) {
+    QmmCallScope call;
     if (int rc = check_space(mem_space)) return rc;
     if (rows < 0 || n <= 0 || n > 0xfffffffeLL || rows > 0x7fffffff)
         return qmm_fail(IZWI_QMM_ERR_INVALID, "argmax: bad shape [%lld, %lld]", (long long)rows, (long long)n);

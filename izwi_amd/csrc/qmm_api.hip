@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -248,33 +249,95 @@ struct Staged {
 
 // Scratch for kernels that need device memory beyond inputs and outputs (the
 // quantized activations of the batched decode kernels, the intermediates of the
-// expert MLP, the counting sort's histograms).  One buffer per
-// (device, stream): work on a stream is ordered, so consecutive calls may reuse
-// it; different streams never share.  It only grows; growing frees the old
-// buffer with hipFree, which waits for the device first.  Growth is not
-// possible while the stream is being captured into a graph: run one call of
-// the same size before capturing.
+// expert MLP, the counting sort's histograms, split-k partial tiles).  One buffer
+// per (device, stream).
+//
+// Exclusive use: a library call that asks for scratch holds its stream's buffer
+// from that request until the call returns (QmmCallScope, below), i.e. until
+// every launch that reads or writes the buffer has been queued.  A second host
+// thread calling on the same stream waits there, so its launches are queued
+// behind the first call's and, work on a stream being ordered, run behind them:
+// two calls never interleave on one buffer.  Calls on different streams use
+// different buffers and do not wait for each other.
+//
+// Growth: a larger request allocates a new buffer; the old one is RETIRED, never
+// freed before the process ends: launches already queued, and HIP graphs captured
+// earlier, keep addresses into it.  Sizes grow geometrically, so the retired
+// buffers of a stream add up to less than four times its largest.  A request
+// that would have to grow while its stream is being captured fails
+// (hipErrorStreamCaptureUnsupported): allocate beforehand with
+// izwi_qmm_scratch_reserve or with one eager call of the same size.
 struct Scratch {
+    std::mutex in_use; // held by the call that uses the buffer, from its first request to its return
     void* ptr = nullptr;
     size_t bytes = 0;
+    std::vector<void*> retired;
 };
-std::mutex g_scratch_mutex;
-std::unordered_map<uint64_t, Scratch> g_scratch;
+std::mutex g_scratch_mutex;                              // guards the map, not the buffers
+std::unordered_map<uint64_t, std::unique_ptr<Scratch>> g_scratch;
+std::atomic<uint64_t> g_scratch_retired_bytes{0};
+
+thread_local int t_call_depth = 0;            // nested library calls of this thread
+thread_local std::vector<Scratch*> t_leased;  // buffers this thread's outermost call holds
+thread_local uint64_t t_thread_tag = 0;
+
+uint64_t scratch_key(int device, hipStream_t stream) {
+    uint64_t key = ((uint64_t)(uintptr_t)stream) ^ ((uint64_t)device << 56);
+    if (stream == hipStreamPerThread) {
+        // one handle value, a different stream in every host thread
+        static std::atomic<uint64_t> next{1};
+        if (!t_thread_tag) t_thread_tag = next.fetch_add(1);
+        key ^= t_thread_tag << 24;
+    }
+    return key;
+}
+
+bool stream_is_capturing(hipStream_t stream) {
+    if (!stream) return false; // the legacy default stream cannot be captured
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return st != hipStreamCaptureStatusNone;
+}
 
 hipError_t get_scratch(int device, hipStream_t stream, size_t bytes, void** out) {
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    Scratch& s = g_scratch[((uint64_t)(uintptr_t)stream) ^ ((uint64_t)device << 56)];
-    if (s.bytes < bytes) {
-        size_t want = bytes < (1u << 20) ? (1u << 20) : bytes + bytes / 4;
-        void* p = nullptr;
-        hipError_t e = hipMalloc(&p, want);
-        if (e != hipSuccess) return e;
-        if (s.ptr) (void)hipFree(s.ptr);
-        s.ptr = p;
-        s.bytes = want;
+    Scratch* s = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        auto& slot = g_scratch[scratch_key(device, stream)];
+        if (!slot) slot.reset(new Scratch());
+        s = slot.get();
     }
-    *out = s.ptr;
-    return hipSuccess;
+    const bool held = std::find(t_leased.begin(), t_leased.end(), s) != t_leased.end();
+    if (!held) s->in_use.lock();
+    hipError_t e = hipSuccess;
+    if (s->bytes < bytes) {
+        if (stream_is_capturing(stream)) {
+            e = hipErrorStreamCaptureUnsupported;
+        } else {
+            size_t want = bytes < (1u << 20) ? (1u << 20) : bytes + bytes / 2;
+            void* p = nullptr;
+            e = hipMalloc(&p, want);
+            if (e == hipSuccess) {
+                if (s->ptr) {
+                    s->retired.push_back(s->ptr);
+                    g_scratch_retired_bytes.fetch_add(s->bytes, std::memory_order_relaxed);
+                }
+                s->ptr = p;
+                s->bytes = want;
+            }
+        }
+    }
+    *out = s->ptr;
+    if (!held) {
+        // inside a library call: keep the buffer until the call returns; outside (a reservation):
+        // nothing is launched on it, release at once
+        if (t_call_depth > 0 && e == hipSuccess) t_leased.push_back(s);
+        else s->in_use.unlock();
+    }
+    return e;
 }
 
 // Smallest m that takes the batched (MFMA) decode kernel; below it the fused
@@ -285,6 +348,21 @@ int mfma_min_m() {
         int n = e ? atoi(e) : 0;
         return n > 0 ? n : 3;
     }();
+    return v;
+}
+
+// Arithmetic of f32 / fused calls with more than 64 activation rows: 0 = activations rounded to
+// bf16, weights dequantized to bf16, bf16 matrix cores (the prefill kernel); 1 = the reference's
+// integer block dots on quantized activations, 64 rows at a time through the batched decode kernel.
+// IZWI_QMM_LARGE_M=int8 selects 1 at start-up; izwi_qmm_set_large_m_arithmetic changes it later.
+std::atomic<int> g_large_m_mode{-1};
+int large_m_mode() {
+    int v = g_large_m_mode.load(std::memory_order_relaxed);
+    if (v < 0) {
+        const char* e = getenv("IZWI_QMM_LARGE_M");
+        v = (e && (!strcmp(e, "int8") || !strcmp(e, "1"))) ? IZWI_QMM_LARGE_M_INT8 : IZWI_QMM_LARGE_M_BF16;
+        g_large_m_mode.store(v, std::memory_order_relaxed);
+    }
     return v;
 }
 
@@ -325,6 +403,7 @@ struct ProfileScope {
     }
     ~ProfileScope() {
         if (!on) return;
+        if (stream_is_capturing(stream)) return; // nothing runs during a capture, and a wait would end it
         (void)hipStreamSynchronize(stream); // time the execution, not the launch
         uint64_t ns = (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(
                           std::chrono::steady_clock::now() - t0)
@@ -348,6 +427,12 @@ int qmm_current_device(int* device, int* n_cus) {
 }
 hipError_t qmm_get_scratch(int device, hipStream_t stream, size_t bytes, void** out) {
     return get_scratch(device, stream, bytes, out);
+}
+QmmCallScope::QmmCallScope() { t_call_depth++; }
+QmmCallScope::~QmmCallScope() {
+    if (--t_call_depth > 0) return;
+    for (Scratch* s : t_leased) s->in_use.unlock();
+    t_leased.clear();
 }
 
 extern "C" {
@@ -503,6 +588,7 @@ int izwi_qmm_quantize_activations(int ggml_weight_dtype, const float* x, int64_t
 
 int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, float* y,
                          int mem_space, void* stream_) {
+    QmmCallScope call;
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(mem_space)) return rc;
     const QmmLayout& L = w->layout;
@@ -519,11 +605,20 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
     HIP_TRY(yo.out(y, (size_t)m * L.n * sizeof(float), mem_space));
     if (m < mfma_min_m()) {
         HIP_TRY(qmm_launch_gemv(L, w->tiled, (const float*)xi.dev, m, (float*)yo.dev, w->n_cus, stream));
-    } else if (m <= 64) {
+    } else if (m <= 64 || large_m_mode() == IZWI_QMM_LARGE_M_INT8) {
+        // more than 64 rows in the integer arithmetic: 64 at a time, the records of one chunk
+        // are overwritten by the next chunk's quantizer, which the stream runs behind its reader
         void* scratch = nullptr;
-        HIP_TRY(get_scratch(w->device, stream, qmm_gemv_mfma_workspace_bytes(L, m), &scratch));
-        HIP_TRY(qmm_launch_gemv_mfma(L, w->tiled, (const float*)xi.dev, m, (float*)yo.dev, scratch,
-                                     w->n_cus, stream));
+        HIP_TRY(get_scratch(w->device, stream, qmm_gemv_mfma_workspace_bytes(L, m < 64 ? m : 64), &scratch));
+        for (int64_t r0 = 0; r0 < m; r0 += 64) {
+            const int64_t rows = m - r0 < 64 ? m - r0 : 64;
+            const float* xr = (const float*)xi.dev + r0 * L.k;
+            float* yr = (float*)yo.dev + r0 * L.n;
+            if (rows < mfma_min_m())
+                HIP_TRY(qmm_launch_gemv(L, w->tiled, xr, rows, yr, w->n_cus, stream));
+            else
+                HIP_TRY(qmm_launch_gemv_mfma(L, w->tiled, xr, rows, yr, scratch, w->n_cus, stream));
+        }
     } else {
         // prefill-sized m with f32 activations: convert once, then the MFMA kernel
         // scratch: [bf16 copy of x | split-k partial tiles]
@@ -595,6 +690,7 @@ int batched_group_on_records(const izwi_qmm_weight* const* weights, int32_t n_we
 
 int forward_group_impl(const izwi_qmm_weight* const* weights, int32_t n_weights, const float* x, int64_t m,
                        float* const* ys, int mem_space, void* stream_, const float* norm_weight, float norm_eps) {
+    QmmCallScope call;
     if (!weights || !ys) return fail(IZWI_QMM_ERR_INVALID, "NULL argument");
     if (n_weights < 1 || n_weights > QMM_MAX_GROUP)
         return fail(IZWI_QMM_ERR_INVALID, "projection group of %d weights (1..%d supported)", n_weights, QMM_MAX_GROUP);
@@ -759,6 +855,7 @@ int izwi_qmm_forward_gate_up_silu_normed_f32(const izwi_qmm_weight* gate, const 
 
 int izwi_qmm_forward_normed_f32(const izwi_qmm_weight* w, const float* x, int64_t m, const float* norm_weight,
                                 float eps, float* y, int mem_space, void* stream_) {
+    QmmCallScope call;
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (!norm_weight) return fail(IZWI_QMM_ERR_INVALID, "norm_weight is NULL");
     if (int rc = check_space(mem_space)) return rc;
@@ -795,6 +892,7 @@ namespace {
 
 int gate_up_silu_impl(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const float* x, int64_t m, float* h,
                       int mem_space, void* stream_, const float* norm_weight, float norm_eps) {
+    QmmCallScope call;
     if (!gate || !up) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(mem_space)) return rc;
     const QmmLayout& L = gate->layout;
@@ -863,6 +961,7 @@ extern "C" {
 
 int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int64_t m, void* y,
                           int out_dtype, int mem_space, void* stream_) {
+    QmmCallScope call;
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(mem_space)) return rc;
     if (out_dtype != IZWI_QMM_OUT_F32 && out_dtype != IZWI_QMM_OUT_BF16)
@@ -890,6 +989,7 @@ int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int6
 
 int izwi_qmm_forward_fused(const izwi_qmm_weight* w, const void* x, int x_dtype, int64_t m,
                            const void* residual, void* y, int y_dtype, int mem_space, void* stream_) {
+    QmmCallScope call;
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(mem_space)) return rc;
     if ((x_dtype != IZWI_QMM_OUT_F32 && x_dtype != IZWI_QMM_OUT_BF16) ||
@@ -926,21 +1026,34 @@ int izwi_qmm_forward_fused(const izwi_qmm_weight* w, const void* x, int x_dtype,
             io.x_bf16 = 0;
         }
         HIP_TRY(qmm_launch_gemv(L, w->tiled, xf, m, (float*)yo.dev, w->n_cus, stream, &io));
-    } else if (m <= 64) {
-        const size_t ws_bytes = (qmm_gemv_mfma_workspace_bytes(L, m) + 255) & ~(size_t)255;
+    } else if (m <= 64 || large_m_mode() == IZWI_QMM_LARGE_M_INT8) {
+        const int64_t chunk = m < 64 ? m : 64;
+        const size_t ws_bytes = (qmm_gemv_mfma_workspace_bytes(L, chunk) + 255) & ~(size_t)255;
+        const size_t xe = x_bf16 ? 2 : 4, ye = y_bf16 ? 2 : 4;
         void* scratch = nullptr;
-        HIP_TRY(get_scratch(w->device, stream, ws_bytes + (size_t)m * L.n * sizeof(float), &scratch));
-        hipError_t e = qmm_launch_gemv_mfma(L, w->tiled, (const float*)xi.dev, m, (float*)yo.dev, scratch, w->n_cus,
-                                            stream, true, &io);
-        if (e == hipErrorNotSupported) {
-            // (very tall matrix with k beyond one activation window) sums into scratch, then the epilogue
-            (void)hipGetLastError();
-            float* sums = reinterpret_cast<float*>(static_cast<uint8_t*>(scratch) + ws_bytes);
-            const QmmIo plain{io.x_bf16, nullptr, 0};
-            e = qmm_launch_gemv_mfma(L, w->tiled, (const float*)xi.dev, m, sums, scratch, w->n_cus, stream, true, &plain);
-            if (e == hipSuccess) e = qmm_launch_epilogue(sums, io.residual, yo.dev, io.y_bf16, m * L.n, stream);
+        HIP_TRY(get_scratch(w->device, stream, ws_bytes + (size_t)chunk * (L.n > L.k ? L.n : L.k) * sizeof(float), &scratch));
+        float* spare = reinterpret_cast<float*>(static_cast<uint8_t*>(scratch) + ws_bytes);
+        for (int64_t r0 = 0; r0 < m; r0 += 64) {
+            const int64_t rows = m - r0 < 64 ? m - r0 : 64;
+            const void* xr = static_cast<const uint8_t*>(xi.dev) + (size_t)r0 * L.k * xe;
+            void* yr = static_cast<uint8_t*>(yo.dev) + (size_t)r0 * L.n * ye;
+            QmmIo cio = io;
+            if (io.residual) cio.residual = static_cast<const uint8_t*>(io.residual) + (size_t)r0 * L.n * ye;
+            hipError_t e;
+            if (rows < mfma_min_m()) { // a tail of one or two rows: the single-launch kernel
+                e = qmm_launch_gemv(L, w->tiled, (const float*)xr, rows, (float*)yr, w->n_cus, stream, &cio);
+            } else {
+                e = qmm_launch_gemv_mfma(L, w->tiled, (const float*)xr, rows, (float*)yr, scratch, w->n_cus, stream, true, &cio);
+                if (e == hipErrorNotSupported) {
+                    // (very tall matrix with k beyond one activation window) sums into scratch, then the epilogue
+                    (void)hipGetLastError();
+                    const QmmIo plain{cio.x_bf16, nullptr, 0};
+                    e = qmm_launch_gemv_mfma(L, w->tiled, (const float*)xr, rows, spare, scratch, w->n_cus, stream, true, &plain);
+                    if (e == hipSuccess) e = qmm_launch_epilogue(spare, cio.residual, yr, cio.y_bf16, rows * L.n, stream);
+                }
+            }
+            if (e != hipSuccess) return fail_hip(e, "batched decode kernel");
         }
-        if (e != hipSuccess) return fail_hip(e, "batched decode kernel");
     } else {
         const size_t xb_bytes = x_bf16 ? 0 : ((((size_t)m * L.k * sizeof(uint16_t)) + 255) & ~(size_t)255);
         const size_t ws_bytes = qmm_gemm_workspace_bytes(L, m, w->n_cus);
@@ -986,6 +1099,7 @@ int izwi_moe_route(const float* logits, int64_t t, int32_t n_experts, int32_t to
 
 int izwi_moe_sort(const int32_t* ids, int64_t t, int32_t top_k, int32_t n_experts, int32_t* perm,
                   int32_t* offsets, int mem_space, void* stream_) {
+    QmmCallScope call;
     if (int rc = check_space(mem_space)) return rc;
     if (t < 0 || top_k < 1 || n_experts < 1 || n_experts > 8192)
         return fail(IZWI_QMM_ERR_INVALID, "bad sort shape t=%lld top_k=%d n_experts=%d", (long long)t, top_k, n_experts);
@@ -1134,6 +1248,7 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
                          const int32_t* ids, const float* weights, int32_t top_k,
                          const int32_t* perm, const int32_t* offsets, float* out, int mem_space,
                          void* stream_) {
+    QmmCallScope call;
     if (int rc = moe_check_stacks(gate, up, down)) return rc;
     if (int rc = check_space(mem_space)) return rc;
     if (t < 0 || top_k < 1) return fail(IZWI_QMM_ERR_INVALID, "bad t / top_k");
@@ -1162,6 +1277,7 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
 int izwi_moe_layer_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_qmm_weight* down,
                        const float* logits, const float* x, int64_t t, int32_t top_k, float* out,
                        int32_t* ids_out, float* weights_out, int mem_space, void* stream_) {
+    QmmCallScope call;
     if (int rc = moe_check_stacks(gate, up, down)) return rc;
     if (int rc = check_space(mem_space)) return rc;
     const int n_experts = (int)gate->layout.n_stacked;
@@ -1186,6 +1302,24 @@ int izwi_moe_layer_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, c
     HIP_TRY(oo.finish(stream));
     if (ids_out) HIP_TRY(io.finish(stream));
     if (weights_out) HIP_TRY(wo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_set_large_m_arithmetic(int mode) {
+    if (mode != IZWI_QMM_LARGE_M_BF16 && mode != IZWI_QMM_LARGE_M_INT8)
+        return fail(IZWI_QMM_ERR_INVALID, "bad large-m arithmetic %d (bf16 = 0, int8 = 1)", mode);
+    g_large_m_mode.store(mode, std::memory_order_relaxed);
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_get_large_m_arithmetic(void) { return large_m_mode(); }
+
+int izwi_qmm_scratch_reserve(uint64_t bytes, void* stream_) {
+    int device = 0;
+    if (int rc = current_device(&device)) return rc;
+    if (int rc = ensure_device(device, nullptr)) return rc;
+    void* p = nullptr;
+    HIP_TRY(get_scratch(device, (hipStream_t)stream_, (size_t)bytes, &p));
     return IZWI_QMM_OK;
 }
 

@@ -93,8 +93,20 @@ int qmm_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)
 // The current HIP device, validated (IZWI_QMM_ERR_NO_DEVICE without one), and its CU count.
 int qmm_current_device(int* device, int* n_cus);
 // The library's scratch buffer of (device, stream): at least `bytes`, reused by the next call on
-// the same stream (work on a stream is ordered); grows with hipMalloc, never shrinks.
+// the same stream (work on a stream is ordered).  The calling thread holds the buffer exclusively
+// from this request until its outermost QmmCallScope ends; other host threads that call on the
+// same stream wait for that.  Grows with hipMalloc (an outgrown buffer is kept until the process
+// ends, never freed); hipErrorStreamCaptureUnsupported if it would have to grow during a capture.
 hipError_t qmm_get_scratch(int device, hipStream_t stream, size_t bytes, void** out);
+// One library call on this thread: every exported entry point that may reach qmm_get_scratch
+// opens one first.  Scopes nest (entry points call each other); the outermost one releases the
+// scratch buffers its call took.
+struct QmmCallScope {
+    QmmCallScope();
+    ~QmmCallScope();
+    QmmCallScope(const QmmCallScope&) = delete;
+    QmmCallScope& operator=(const QmmCallScope&) = delete;
+};
 
 // ---- launchers -------------------------------------------------------------
 hipError_t qmm_launch_repack(const QmmLayout& L, const void* native, void* tiled,

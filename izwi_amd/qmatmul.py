@@ -255,15 +255,16 @@ class Qwen3Projection:
         return cls(packed_qmatmul_from_qtensors(parts))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        """qwen3/core.rs:791-831.  f32 goes straight to the op.  bf16 prefill-sized
-        inputs use the bf16 kernel (input and output casts fused away); other
-        dtypes are cast to f32 and back as the reference does on accelerators."""
+        """qwen3/core.rs:791-831.  f32 goes straight to the op.  bf16 inputs go through the
+        fused call, which reads them as they are and rounds the f32 sums back to bf16 (the
+        reference's cast to f32, QMatMul, cast back, with both casts inside the kernels); beyond 64
+        rows that call runs the bf16 matrix-core kernel unless the integer arithmetic was selected
+        (izwi_qmm_set_large_m_arithmetic).  Other dtypes are cast to f32 and back as the reference
+        does on accelerators."""
         if x.dtype == torch.float32:
             return self.qmatmul.forward(x)
-        k = x.shape[-1]
-        m = x.numel() // k if k else 0
-        if x.dtype == torch.bfloat16 and m > 64:
-            return self.qmatmul.forward(x)
+        if x.dtype == torch.bfloat16 and x.is_cuda:
+            return self.qmatmul.forward_fused(x)
         return self.qmatmul.forward(x.to(torch.float32)).to(x.dtype)
 
 

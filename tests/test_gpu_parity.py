@@ -152,6 +152,32 @@ def test_config3_lm_head_full_size(qa, oracle):
     assert rel_err(y, oracle.qmatmul(Q4_K, x, blocks, n)) < DECODE_TOL
 
 
+def sample_rows(blocks, dtype, n, k, count, seed):
+    """Block bytes of `count` weight rows spread over the matrix (first and last included), and
+    their indices: rows are independent, so the oracle's product over the subset is the
+    corresponding columns of the full product."""
+    rng = np.random.default_rng(seed)
+    rows = np.unique(np.concatenate([[0, n - 1], rng.choice(n, size=count - 2, replace=False)]))
+    row_bytes = k // {Q8_0: 32, Q4_K: 256}[dtype] * {Q8_0: 34, Q4_K: 144}[dtype]
+    return rows, np.ascontiguousarray(blocks.reshape(n, row_bytes)[rows]).reshape(-1)
+
+
+@pytest.mark.parametrize("m", [8, 16])
+def test_config3_lm_head_full_size_batched(qa, oracle, m):
+    # the full 151936 x 4096 matrix on the device; the oracle on ~2k of its rows
+    n, k = 151936, 4096
+    blocks = make_weight(oracle, Q4_K, n, k, 50)
+    x = oracle.randn(52 + m, (m, k))
+    _say(f"config3 lm_head m={m}")
+    y = run_forward(qa, Q4_K, blocks, n, k, x)
+    rows, sub = sample_rows(blocks, Q4_K, n, k, 2048, 53)
+    want = oracle.qmatmul(Q4_K, x, sub, rows.size)
+    assert rel_err(y[:, rows], want) < DECODE_TOL
+    # the rest of the output against the single-row call of every activation row (another kernel)
+    y1 = run_forward(qa, Q4_K, blocks, n, k, x[3:4])
+    assert rel_err(y[3:4], y1.astype(np.float64)) < DECODE_TOL
+
+
 @pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
 @pytest.mark.parametrize("n,k,m", [(1, 256, 1), (15, 256, 2), (17, 512, 3), (100, 768, 5), (250, 1280, 7),
                                    (33, 2048, 64), (7, 16384, 2), (4100, 256, 1),
@@ -287,7 +313,7 @@ def test_prefill_bf16_against_oracle(qa, oracle, dtype, m, n, k):
 
 @pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
 @pytest.mark.parametrize("m", [512, 2048])
-def test_config4_prefill_full_shapes_against_fp32(qa, oracle, dtype, m):
+def test_config4_prefill_full_shapes(qa, oracle, dtype, m):
     # full 8B shapes: checked against a plain fp32 matmul of the (bit-exact) dequantized weight
     for i, (name, n, k) in enumerate(SHAPES_8B):
         _say(f"config4 dtype={dtype} {name} m={m}")
@@ -298,6 +324,10 @@ def test_config4_prefill_full_shapes_against_fp32(qa, oracle, dtype, m):
         ref = xb.float() @ qt.dequantize().t()
         err = float((y - ref).abs().max() / ref.abs().max())
         assert err < 5e-3, (name, err)
+        # and against the reference's CPU arithmetic on a spread of 256 weight rows
+        rows, sub = sample_rows(blocks, dtype, n, k, 256, 170 + i)
+        want = oracle.qmatmul(dtype, xb.float().cpu().numpy(), sub, rows.size)
+        assert rel_err(y[:, torch.from_numpy(rows).cuda()].cpu().numpy(), want) < PREFILL_TOL, name
         del qt, y, ref
 
 
@@ -306,6 +336,45 @@ def test_forward_f32_large_m_uses_prefill_kernel(qa, oracle):
     x = oracle.randn(161, (200, 1024))
     y = run_forward(qa, Q4_K, blocks, 256, 1024, x)
     assert rel_err(y, oracle.qmatmul(Q4_K, x, blocks, 256)) < PREFILL_TOL
+
+
+def test_large_m_arithmetic_switch(qa, oracle):
+    """Beyond 64 rows `forward_f32` changes arithmetic (bf16 matrix cores on dequantized weights)
+    unless the caller selects the integer dots: the error against the reference's CPU result at
+    m = 64 and m = 65 on one shape, in both modes."""
+    from izwi_amd import capi
+    L = capi.lib()
+    n, k = 1024, 4096
+    blocks = make_weight(oracle, Q4_K, n, k, 165)
+    x = oracle.randn(166, (200, k))
+    want = oracle.qmatmul(Q4_K, x, blocks, n)
+    assert L.izwi_qmm_get_large_m_arithmetic() == 0
+    y64 = run_forward(qa, Q4_K, blocks, n, k, x[:64])
+    y65 = run_forward(qa, Q4_K, blocks, n, k, x[:65])
+    assert rel_err(y64, want[:64]) < DECODE_TOL
+    e65 = rel_err(y65, want[:65])
+    _say(f"m=64 err {rel_err(y64, want[:64]):.2e}, m=65 (bf16 matrix cores) err {e65:.2e}")
+    assert DECODE_TOL < e65 < PREFILL_TOL
+    capi.check(L.izwi_qmm_set_large_m_arithmetic(1))
+    try:
+        for m in (65, 130, 200):   # tails of 1, 2 and 8 rows behind the 64-row chunks
+            y = run_forward(qa, Q4_K, blocks, n, k, x[:m])
+            assert rel_err(y, want[:m]) < DECODE_TOL, m
+            assert np.array_equal(y[:64], y64), m
+        # the fused call (bf16 in, residual, bf16 out) follows the same switch
+        q = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType(Q4_K), blocks, (n, k)))
+        xb = torch.from_numpy(x[:130]).cuda().to(torch.bfloat16)
+        res = torch.from_numpy(oracle.randn(167, (130, n))).cuda().to(torch.bfloat16)
+        got = q.forward_fused(xb, residual=res)
+        plain = q.forward(xb.float())
+        assert rel_err(plain.cpu().numpy(), oracle.qmatmul(Q4_K, xb.float().cpu().numpy(), blocks, n)) < DECODE_TOL
+        assert torch.equal(got, (plain + res.float()).to(torch.bfloat16))
+        # Qwen3Projection.forward on bf16 activations: cast to f32, QMatMul, cast back
+        proj = qa.Qwen3Projection(q)
+        assert torch.equal(proj.forward(xb), plain.to(torch.bfloat16))
+    finally:
+        capi.check(L.izwi_qmm_set_large_m_arithmetic(0))
+    assert L.izwi_qmm_set_large_m_arithmetic(7) == -1 and L.izwi_qmm_get_large_m_arithmetic() == 0
 
 
 # --------------------------------------------------------------------- MoE --
