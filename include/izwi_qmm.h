@@ -187,6 +187,22 @@ int izwi_qmm_dequantize_f32(const izwi_qmm_weight* w, float* out, int mem_space,
 int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, float* y,
                          int mem_space, void* stream);
 
+/* izwi_qmm_forward_f32 for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same kernels and the same results, bit for bit, as izwi_qmm_forward_f32 with
+ * IZWI_QMM_DEVICE pointers; the quantized activation records of the batched kernels (3 <= m <= 64)
+ * live in a static device array of IZWI_QMM_NOALLOC_SCRATCH_BYTES inside the library's image
+ * (each GPU the library runs on holds its own copy until the process ends) instead of the
+ * per-stream scratch buffer, and the call performs no hipMalloc / hipFree whatever its size.
+ * Limits: x and y are device pointers; the weight's device must be the current device; m <= 64;
+ * ceil(m / 16) * (k / 256) records of 4416 (Q4_K, Q6_K) or 4608 (Q8_0) bytes must fit the array
+ * (k = 12288 at m = 64 does: 884,736 bytes), otherwise IZWI_QMM_ERR_UNSUPPORTED.
+ * Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (other
+ * streams, other threads) race on it; calls on one stream are ordered and safe.  The array keeps
+ * the previous call's contents; each call rewrites every record it reads. */
+#define IZWI_QMM_NOALLOC_SCRATCH_BYTES 1048576
+int izwi_qmm_forward_f32_noalloc(const izwi_qmm_weight* w, const float* x, int64_t m, float* y, void* stream);
+
 /* `Qwen3QkvProjection::forward` and `Qwen3GateUpProjection::forward`, `Separate` arms
  * (qwen3/core.rs:1119-1127, 1274-1282): several projections applied to the same
  * activations, y_i = QMatMul_i.forward(x), bit-identical to n_weights calls of

@@ -435,6 +435,32 @@ QmmCallScope::~QmmCallScope() {
     t_leased.clear();
 }
 
+// ---- the entry point that allocates nothing ---------------------------------
+// Scratch of izwi_qmm_forward_f32_noalloc: the quantized activation records of the batched decode
+// kernels (up to 64 rows), held in the library's image on every GPU it runs on instead of being
+// allocated.  `noalloc_scratch` is the host-side name of the array, not a device address: the
+// device address of each GPU's own copy is looked up once per device and only that pointer is
+// handed to kernels.
+static __device__ __align__(256) unsigned char noalloc_scratch[IZWI_QMM_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+std::mutex g_noalloc_mutex;
+void* g_noalloc_ptr[64] = {};
+
+// Device address of `device`'s copy of the array; `device` must be the current device.
+hipError_t noalloc_scratch_ptr(int device, void** out) {
+    std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+    if (!g_noalloc_ptr[device]) {
+        void* p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(noalloc_scratch));
+        if (e != hipSuccess) return e;
+        g_noalloc_ptr[device] = p;
+    }
+    *out = g_noalloc_ptr[device];
+    return hipSuccess;
+}
+} // namespace
+
 extern "C" {
 
 int izwi_qmm_abi_version(void) { return IZWI_QMM_ABI_VERSION; }
@@ -445,6 +471,8 @@ int izwi_qmm_init(int device) {
     int rc = ensure_device(device, nullptr);
     if (rc) return rc;
     HIP_TRY(hipSetDevice(device));
+    void* p = nullptr;
+    HIP_TRY(noalloc_scratch_ptr(device, &p)); // the static scratch of this device, looked up once
     return IZWI_QMM_OK;
 }
 
@@ -633,6 +661,39 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
         if (e != hipSuccess) return fail_hip(e, "prefill kernel");
     }
     HIP_TRY(yo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_forward_f32_noalloc(const izwi_qmm_weight* w, const float* x, int64_t m, float* y, void* stream_) {
+    if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    const QmmLayout& L = w->layout;
+    if (L.n_stacked != 1) return fail(IZWI_QMM_ERR_INVALID, "forward on an expert stack");
+    if (m < 0) return fail(IZWI_QMM_ERR_INVALID, "negative m");
+    if (m > 64)
+        return fail(IZWI_QMM_ERR_UNSUPPORTED, "izwi_qmm_forward_f32_noalloc takes at most 64 rows, got %lld",
+                    (long long)m);
+    if (m == 0 || L.n == 0) return IZWI_QMM_OK;
+    if (!x || !y) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    hipStream_t stream = (hipStream_t)stream_;
+    if (m < mfma_min_m()) { // one or two rows: the single-launch kernel has no scratch at all
+        HIP_TRY(qmm_launch_gemv(L, w->tiled, x, m, y, w->n_cus, stream));
+        return IZWI_QMM_OK;
+    }
+    const size_t need = qmm_gemv_mfma_workspace_bytes(L, m);
+    if (need > (size_t)IZWI_QMM_NOALLOC_SCRATCH_BYTES)
+        return fail(IZWI_QMM_ERR_UNSUPPORTED,
+                    "m = %lld rows of k = %lld need %zu bytes of activation records; the static scratch of "
+                    "izwi_qmm_forward_f32_noalloc holds %d",
+                    (long long)m, (long long)L.k, need, IZWI_QMM_NOALLOC_SCRATCH_BYTES);
+    int device = 0;
+    if (int rc = current_device(&device)) return rc;
+    if (device != w->device)
+        return fail(IZWI_QMM_ERR_INVALID, "the weight lives on device %d, the current device is %d", w->device, device);
+    void* scratch = nullptr;
+    HIP_TRY(noalloc_scratch_ptr(device, &scratch));
+    // the quantizer writes every record the matmul reads (whole 16-row tiles, rows beyond m as
+    // zeros), so nothing of an earlier call's contents is ever read
+    HIP_TRY(qmm_launch_gemv_mfma(L, w->tiled, x, m, y, scratch, w->n_cus, stream));
     return IZWI_QMM_OK;
 }
 
