@@ -18,9 +18,13 @@
  * negative izwi_qmm_status, the message is read with izwi_qmm_last_error().
  * Parsing, lookup and metadata need no GPU; only the load functions touch the
  * device.  The file is mapped read-only for the lifetime of the handle (the
- * reference's default for accelerator backends, model_io.rs:144-157); pointers
- * returned by this API stay valid until izwi_gguf_close.  A handle is immutable
- * and may be shared between threads.
+ * reference's default on every backend, model_io.rs:70-83, 144-157); if the
+ * mapping fails, or the mode is "off" (izwi_gguf_open_with_mode, IZWI_GGUF_MMAP),
+ * the file is read with buffered I/O into memory instead, as the reference falls
+ * back (model_io.rs:146-160).  Pointers returned by this API stay valid until
+ * izwi_gguf_close.  A handle is immutable and may be shared between threads.
+ * No C++ exception leaves these functions: running out of memory on a crafted
+ * file is IZWI_QMM_ERR_INVALID.
  */
 #ifndef IZWI_GGUF_H
 #define IZWI_GGUF_H
@@ -75,6 +79,20 @@ int izwi_gguf_is_gguf_file(const char* path);
  * IZWI_QMM_ERR_INVALID; the reference maps them to Error::ModelLoadError. */
 int izwi_gguf_open(const char* path, izwi_gguf** out);
 void izwi_gguf_close(izwi_gguf* g);
+
+/* `GgufMmapMode` and `open_gguf_reader_with_mode` (model_io.rs:13-45, 127-160).  The mode in force
+ * is the configured one, else the environment variable IZWI_GGUF_MMAP ("auto", "on" | "true" | "1" |
+ * "yes", "off" | "false" | "0" | "no", case and surrounding blanks ignored; anything else is
+ * ignored), else auto (`resolve_gguf_mmap_mode`, model_io.rs:63-67); auto maps.  A mapping that
+ * fails falls back to buffered I/O.  `mmap_mode` = -1 means "not configured"; izwi_gguf_open is
+ * izwi_gguf_open_with_mode(path, -1, out).  `parse_mmap_mode` returns the mode or -1 for a word it
+ * does not know (`GgufMmapMode::parse`); `reader_kind` is `GgufReader::kind`. */
+typedef enum izwi_gguf_mmap_mode { IZWI_GGUF_MMAP_AUTO = 0, IZWI_GGUF_MMAP_ON = 1, IZWI_GGUF_MMAP_OFF = 2 } izwi_gguf_mmap_mode;
+typedef enum izwi_gguf_reader_kind { IZWI_GGUF_READER_BUFFERED = 0, IZWI_GGUF_READER_MAPPED = 1 } izwi_gguf_reader_kind_t;
+int izwi_gguf_open_with_mode(const char* path, int mmap_mode, izwi_gguf** out);
+int izwi_gguf_parse_mmap_mode(const char* raw);
+int izwi_gguf_resolve_mmap_mode(int configured);
+int izwi_gguf_reader_kind(const izwi_gguf* g);
 
 /* Header fields: format version (1-3), `general.alignment` in force, offset of the tensor data
  * section in the file. */

@@ -187,6 +187,20 @@ int izwi_qmm_dequantize_f32(const izwi_qmm_weight* w, float* out, int mem_space,
 int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, float* y,
                          int mem_space, void* stream);
 
+/* `Qwen3Projection::logits_for_tokens` / `Qwen3Model::logits_from_hidden_for_tokens`, quantized
+ * arm (qwen3/core.rs:745-758, 2125-2131, 2155-2171): the reference computes the full LM head and
+ * then `index_select`s the wanted token ids.  Weight rows are independent, so this call reads only
+ * the 16-row tiles that hold a selected row (36 KB per token id at k = 4096 Q4_K instead of the
+ * 350 MB of a 151936-row head):
+ *     y[i, j] = forward_f32(x)[i, row_ids[j]]        y is [m, n_rows], row-major
+ * bit for bit (the same kernel with the same split along k, over a list of row-tiles).  The
+ * reference accepts one hidden state ([1, vocab] or [1, 1, vocab] logits); m = 1 or 2 here,
+ * IZWI_QMM_ERR_UNSUPPORTED beyond.  row_ids may repeat and need not be sorted; with host pointers
+ * an id >= n is IZWI_QMM_ERR_INVALID (as `index_select` refuses it), with device pointers (no host
+ * round trip) its outputs are NaN. */
+int izwi_qmm_forward_rows_f32(const izwi_qmm_weight* w, const uint32_t* row_ids, int64_t n_rows, const float* x,
+                              int64_t m, float* y, int mem_space, void* stream);
+
 /* izwi_qmm_forward_f32 for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
  * reference.  Same kernels and the same results, bit for bit, as izwi_qmm_forward_f32 with

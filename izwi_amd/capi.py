@@ -58,6 +58,7 @@ PROTOTYPES = {
     "izwi_qmm_weight_data": (C.c_int, [_vp, _vp, _u64, C.c_int, _vp]),
     "izwi_qmm_dequantize_f32": (C.c_int, [_vp, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_f32": (C.c_int, [_vp, _vp, _i64, _vp, C.c_int, _vp]),
+    "izwi_qmm_forward_rows_f32": (C.c_int, [_vp, _vp, _i64, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_f32_noalloc": (C.c_int, [_vp, _vp, _i64, _vp, _vp]),
     "izwi_qmm_forward_group_f32": (C.c_int, [_vp, _i32, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_gate_up_silu_f32": (C.c_int, [_vp, _vp, _vp, _i64, _vp, C.c_int, _vp]),
@@ -98,6 +99,10 @@ PROTOTYPES = {
     "izwi_gguf_is_gguf_file": (C.c_int, [C.c_char_p]),
     "izwi_gguf_open": (C.c_int, [C.c_char_p, _pp]),
     "izwi_gguf_close": (None, [_vp]),
+    "izwi_gguf_open_with_mode": (C.c_int, [C.c_char_p, C.c_int, _pp]),
+    "izwi_gguf_parse_mmap_mode": (C.c_int, [C.c_char_p]),
+    "izwi_gguf_resolve_mmap_mode": (C.c_int, [C.c_int]),
+    "izwi_gguf_reader_kind": (C.c_int, [_vp]),
     "izwi_gguf_header": (C.c_int, [_vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(_u64)]),
     "izwi_gguf_tensor_count": (_i64, [_vp]),
     "izwi_gguf_tensor_name": (C.c_int, [_vp, _i64, _cpp]),

@@ -11,8 +11,13 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <cerrno>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <exception>
+#include <new>
 #include <string>
 #include <unordered_map>
 #include <utility>
@@ -87,8 +92,9 @@ struct Tensor {
 
 struct izwi_gguf {
     std::string path;
-    const uint8_t* map = nullptr;
+    const uint8_t* map = nullptr; // the file's bytes: a read-only mapping, or a heap copy read with read(2)
     size_t size = 0;
+    bool mapped = false;
     uint32_t version = 0, alignment = 32;
     uint64_t data_offset = 0;
     std::vector<std::string> keys;
@@ -97,7 +103,8 @@ struct izwi_gguf {
     std::vector<Tensor> tensors;
     std::unordered_map<std::string, size_t> tensor_index;
     ~izwi_gguf() {
-        if (map) munmap(const_cast<uint8_t*>(map), size);
+        if (map && mapped) munmap(const_cast<uint8_t*>(map), size);
+        else if (map) free(const_cast<uint8_t*>(map));
     }
 };
 
@@ -161,8 +168,9 @@ bool read_value(Cursor& c, int type, Value& v, int depth) {
             return true;
         }
         if (v.elem_type == IZWI_GGUF_STRING) {
-            if (v.count > c.size - c.pos) return c.ok = false; // every string takes at least a length field
-            v.strs.reserve(v.count);
+            // every string takes at least its length field (8 bytes, 4 in version 1)
+            if (v.count > (c.size - c.pos) / (c.v1 ? 4 : 8)) return c.ok = false;
+            v.strs.reserve((size_t)std::min<uint64_t>(v.count, 1u << 16)); // grows as strings are really read
             for (uint64_t i = 0; i < v.count; i++) {
                 const char* p;
                 uint64_t n;
@@ -260,10 +268,62 @@ int izwi_gguf_is_gguf_file(const char* path) {
     return n == 4 && memcmp(magic, "GGUF", 4) == 0;
 }
 
-int izwi_gguf_open(const char* path, izwi_gguf** out) {
+// `GgufMmapMode::parse` (model_io.rs:26-35): -1 for the empty string and unknown words.
+int izwi_gguf_parse_mmap_mode(const char* raw) {
+    if (!raw) return -1;
+    std::string s(raw);
+    const size_t b = s.find_first_not_of(" \t\r\n"), e = s.find_last_not_of(" \t\r\n");
+    s = b == std::string::npos ? std::string() : s.substr(b, e - b + 1);
+    for (auto& ch : s) ch = (char)tolower((unsigned char)ch);
+    if (s == "auto") return IZWI_GGUF_MMAP_AUTO;
+    if (s == "on" || s == "true" || s == "1" || s == "yes") return IZWI_GGUF_MMAP_ON;
+    if (s == "off" || s == "false" || s == "0" || s == "no") return IZWI_GGUF_MMAP_OFF;
+    return -1;
+}
+
+// `resolve_gguf_mmap_mode` (model_io.rs:63-67): the configured mode, else IZWI_GGUF_MMAP, else auto.
+int izwi_gguf_resolve_mmap_mode(int configured) {
+    if (configured == IZWI_GGUF_MMAP_AUTO || configured == IZWI_GGUF_MMAP_ON || configured == IZWI_GGUF_MMAP_OFF)
+        return configured;
+    const int env = izwi_gguf_parse_mmap_mode(getenv("IZWI_GGUF_MMAP"));
+    return env >= 0 ? env : IZWI_GGUF_MMAP_AUTO;
+}
+
+int izwi_gguf_reader_kind(const izwi_gguf* g) {
+    if (!g) return -1;
+    return g->mapped ? IZWI_GGUF_READER_MAPPED : IZWI_GGUF_READER_BUFFERED;
+}
+
+} // extern "C"
+
+namespace {
+
+// The whole file through read(2) into one heap block (the buffered reader of model_io.rs:160; the
+// handle's tensor pointers must stay valid until close, so the bytes are kept rather than streamed).
+uint8_t* read_whole_file(int fd, size_t size) {
+    uint8_t* buf = static_cast<uint8_t*>(malloc(size));
+    if (!buf) return nullptr;
+    size_t done = 0;
+    while (done < size) {
+        const ssize_t n = read(fd, buf + done, std::min<size_t>(size - done, (size_t)1 << 30));
+        if (n < 0 && errno == EINTR) continue;
+        if (n <= 0) {
+            free(buf);
+            return nullptr;
+        }
+        done += (size_t)n;
+    }
+    return buf;
+}
+
+int open_impl(const char* path, int configured_mode, izwi_gguf** out) {
     if (!out) return qmm_fail(IZWI_QMM_ERR_INVALID, "out is NULL");
     *out = nullptr;
     if (!path) return qmm_fail(IZWI_QMM_ERR_INVALID, "path is NULL");
+    if (configured_mode < -1 || configured_mode > IZWI_GGUF_MMAP_OFF)
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "bad mmap mode %d", configured_mode);
+    // `gguf_mmap_enabled` (model_io.rs:77-83): auto maps on every backend
+    const bool mmap_enabled = izwi_gguf_resolve_mmap_mode(configured_mode) != IZWI_GGUF_MMAP_OFF;
     const int fd = open(path, O_RDONLY | O_CLOEXEC);
     if (fd < 0) return qmm_fail(IZWI_QMM_ERR_INVALID, "Failed to open GGUF file: %s: %s", path, strerror(errno));
     struct stat st;
@@ -271,13 +331,42 @@ int izwi_gguf_open(const char* path, izwi_gguf** out) {
         close(fd);
         return qmm_fail(IZWI_QMM_ERR_INVALID, "Failed to parse GGUF file: %s is empty or not a regular file", path);
     }
-    void* map = mmap(nullptr, (size_t)st.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
+    const uint8_t* bytes = nullptr;
+    bool mapped = false;
+    if (mmap_enabled) {
+        // IZWI_GGUF_TEST_FAIL_MMAP=1 makes the mapping attempt fail (fault injection for the test of
+        // the fallback below; a mapping of a readable regular file does not fail otherwise)
+        const char* inject = getenv("IZWI_GGUF_TEST_FAIL_MMAP");
+        void* map = (inject && inject[0] == '1') ? MAP_FAILED
+                                                 : mmap(nullptr, (size_t)st.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
+        if (map != MAP_FAILED) {
+            bytes = static_cast<const uint8_t*>(map);
+            mapped = true;
+        } else if (getenv("IZWI_GGUF_VERBOSE")) {
+            // the reference warns and falls back to buffered I/O (model_io.rs:146-157)
+            fprintf(stderr, "Failed to memory-map GGUF file %s; falling back to buffered I/O\n", path);
+        }
+    }
+    if (!bytes) {
+        bytes = read_whole_file(fd, (size_t)st.st_size);
+        if (!bytes) {
+            const int err = errno;
+            close(fd);
+            return qmm_fail(IZWI_QMM_ERR_INVALID, "Failed to open GGUF file: reading %s: %s", path,
+                            err ? strerror(err) : "short read or out of memory");
+        }
+    }
     close(fd);
-    if (map == MAP_FAILED) return qmm_fail(IZWI_QMM_ERR_INVALID, "Failed to open GGUF file: mmap of %s: %s", path, strerror(errno));
-    izwi_gguf* g = new izwi_gguf;
-    g->path = path;
-    g->map = static_cast<const uint8_t*>(map);
+    izwi_gguf* g = new (std::nothrow) izwi_gguf;
+    if (!g) {
+        if (mapped) munmap(const_cast<uint8_t*>(bytes), (size_t)st.st_size);
+        else free(const_cast<uint8_t*>(bytes));
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "Failed to open GGUF file: out of memory");
+    }
+    g->map = bytes;
     g->size = (size_t)st.st_size;
+    g->mapped = mapped;
+    g->path = path;
     auto bad = [&](const char* what) {
         const int rc = qmm_fail(IZWI_QMM_ERR_INVALID, "Failed to parse GGUF file: %s (%s)", what, path);
         delete g;
@@ -361,6 +450,33 @@ int izwi_gguf_open(const char* path, izwi_gguf** out) {
     }
     *out = g;
     return IZWI_QMM_OK;
+}
+
+// No C++ exception may cross the C boundary: a crafted file can make the parser ask for more
+// memory than there is.
+template <class F>
+int guarded(const char* what, F&& f) {
+    try {
+        return f();
+    } catch (const std::bad_alloc&) {
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "%s: out of memory", what);
+    } catch (const std::exception& e) {
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "%s: %s", what, e.what());
+    } catch (...) {
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "%s: unknown failure", what);
+    }
+}
+
+} // namespace
+
+extern "C" {
+
+int izwi_gguf_open(const char* path, izwi_gguf** out) {
+    return guarded("Failed to parse GGUF file", [&] { return open_impl(path, -1, out); });
+}
+
+int izwi_gguf_open_with_mode(const char* path, int mmap_mode, izwi_gguf** out) {
+    return guarded("Failed to parse GGUF file", [&] { return open_impl(path, mmap_mode, out); });
 }
 
 void izwi_gguf_close(izwi_gguf* g) { delete g; }
@@ -470,7 +586,7 @@ int izwi_gguf_metadata_array_string(const izwi_gguf* g, const char* key, uint64_
     return IZWI_QMM_OK;
 }
 
-int izwi_gguf_load_weight(const izwi_gguf* g, const char* name, izwi_qmm_weight** out) {
+static int gguf_load_weight_impl(const izwi_gguf* g, const char* name, izwi_qmm_weight** out) {
     if (!g || !name || !out) return qmm_fail(IZWI_QMM_ERR_INVALID, "NULL argument");
     const Tensor* t = find_tensor(g, name);
     if (!t) return qmm_fail(IZWI_QMM_ERR_INVALID, "Failed to load tensor '%s' from GGUF: tensor not found", name);
@@ -485,7 +601,7 @@ int izwi_gguf_load_weight(const izwi_gguf* g, const char* name, izwi_qmm_weight*
     return izwi_qmm_weight_create(ti.ggml_dtype, ti.dims[0], ti.dims[1], ti.data, ti.nbytes, IZWI_QMM_HOST, out);
 }
 
-int izwi_gguf_load_packed(const izwi_gguf* g, const char* const* names, int32_t n_names,
+static int gguf_load_packed_impl(const izwi_gguf* g, const char* const* names, int32_t n_names,
                           izwi_qmm_weight** out) {
     if (!g || !names || !out) return qmm_fail(IZWI_QMM_ERR_INVALID, "NULL argument");
     if (n_names < 1) return qmm_fail(IZWI_QMM_ERR_INVALID, "Cannot pack empty Qwen3 quantized projection group");
@@ -518,7 +634,7 @@ int izwi_gguf_load_packed(const izwi_gguf* g, const char* const* names, int32_t 
     return izwi_qmm_weight_create_packed(dtype, n_names, rows.data(), k, blocks.data(), nbytes.data(), IZWI_QMM_HOST, out);
 }
 
-int izwi_gguf_load_tensor_f32(const izwi_gguf* g, const char* name, float* out, uint64_t count,
+static int gguf_load_tensor_f32_impl(const izwi_gguf* g, const char* name, float* out, uint64_t count,
                               int mem_space, void* stream_) {
     if (!g || !name) return qmm_fail(IZWI_QMM_ERR_INVALID, "NULL argument");
     if (mem_space != IZWI_QMM_DEVICE && mem_space != IZWI_QMM_HOST)
@@ -597,6 +713,20 @@ int izwi_gguf_load_tensor_f32(const izwi_gguf* g, const char* name, float* out, 
                         "Failed to dequantize tensor '%s': ggml dtype %d is not supported (F32, F16, BF16, Q8_0, Q4_K, Q6_K)",
                         name, ti.ggml_dtype);
     }
+}
+
+int izwi_gguf_load_weight(const izwi_gguf* g, const char* name, izwi_qmm_weight** out) {
+    return guarded("Failed to load tensor from GGUF", [&] { return gguf_load_weight_impl(g, name, out); });
+}
+
+int izwi_gguf_load_packed(const izwi_gguf* g, const char* const* names, int32_t n_names, izwi_qmm_weight** out) {
+    return guarded("Failed to load tensors from GGUF", [&] { return gguf_load_packed_impl(g, names, n_names, out); });
+}
+
+int izwi_gguf_load_tensor_f32(const izwi_gguf* g, const char* name, float* out, uint64_t count, int mem_space,
+                              void* stream_) {
+    return guarded("Failed to load tensor from GGUF",
+                   [&] { return gguf_load_tensor_f32_impl(g, name, out, count, mem_space, stream_); });
 }
 
 } // extern "C"

@@ -664,6 +664,41 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
     return IZWI_QMM_OK;
 }
 
+int izwi_qmm_forward_rows_f32(const izwi_qmm_weight* w, const uint32_t* row_ids, int64_t n_rows, const float* x,
+                              int64_t m, float* y, int mem_space, void* stream_) {
+    QmmCallScope call;
+    if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    if (int rc = check_space(mem_space)) return rc;
+    const QmmLayout& L = w->layout;
+    if (L.n_stacked != 1) return fail(IZWI_QMM_ERR_INVALID, "forward on an expert stack");
+    if (m < 0 || n_rows < 0) return fail(IZWI_QMM_ERR_INVALID, "negative m or row count");
+    if (m > 2)
+        return fail(IZWI_QMM_ERR_UNSUPPORTED,
+                    "Qwen3 selected-token logits expected one hidden state ([1,vocab] or [1,1,vocab] logits), "
+                    "got %lld rows (at most 2 are supported)", (long long)m);
+    if (m == 0 || n_rows == 0) return IZWI_QMM_OK; // `logits_for_tokens` of an empty id list is empty
+    if (n_rows > (1 << 24)) return fail(IZWI_QMM_ERR_UNSUPPORTED, "too many selected rows (%lld)", (long long)n_rows);
+    if (!row_ids || !x || !y) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    if (L.n == 0) return fail(IZWI_QMM_ERR_INVALID, "row index out of range: the weight has no rows");
+    if (mem_space == IZWI_QMM_HOST) // `index_select` refuses an index beyond the dimension
+        for (int64_t i = 0; i < n_rows; i++)
+            if ((int64_t)row_ids[i] >= L.n)
+                return fail(IZWI_QMM_ERR_INVALID, "row index %u out of range for a weight of %lld rows", row_ids[i],
+                            (long long)L.n);
+    hipStream_t stream = (hipStream_t)stream_;
+    ProfileScope prof(w, stream);
+    Staged xi, ii, yo;
+    HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
+    HIP_TRY(ii.in(row_ids, (size_t)n_rows * sizeof(uint32_t), mem_space));
+    HIP_TRY(yo.out(y, (size_t)m * n_rows * sizeof(float), mem_space));
+    void* scratch = nullptr;
+    HIP_TRY(get_scratch(w->device, stream, qmm_gemv_rows_workspace_bytes(m, n_rows), &scratch));
+    HIP_TRY(qmm_launch_gemv_rows(L, w->tiled, (const float*)xi.dev, m, (const uint32_t*)ii.dev, n_rows, (float*)yo.dev,
+                                 scratch, w->n_cus, stream));
+    HIP_TRY(yo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
 int izwi_qmm_forward_f32_noalloc(const izwi_qmm_weight* w, const float* x, int64_t m, float* y, void* stream_) {
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     const QmmLayout& L = w->layout;
@@ -1312,8 +1347,11 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
     QmmCallScope call;
     if (int rc = moe_check_stacks(gate, up, down)) return rc;
     if (int rc = check_space(mem_space)) return rc;
-    if (t < 0 || top_k < 1) return fail(IZWI_QMM_ERR_INVALID, "bad t / top_k");
+    if (t < 0) return fail(IZWI_QMM_ERR_INVALID, "negative t");
+    if (top_k < 1 || top_k > 64 || top_k > (int)gate->layout.n_stacked)
+        return fail(IZWI_QMM_ERR_INVALID, "top_k = %d outside 1..min(n_experts, 64)", top_k);
     if (t == 0) return IZWI_QMM_OK;
+    if (t * (int64_t)top_k > 0x7fffffff) return fail(IZWI_QMM_ERR_UNSUPPORTED, "too many pairs");
     if (!x || !ids || !weights || !perm || !offsets || !out)
         return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
     const int64_t pairs = t * top_k;

@@ -446,6 +446,9 @@ struct GemvParams {
     // NORM variants: the activations are RMS-normalized on the way in (weight norm_w[k], eps)
     const float* norm_w;
     float norm_eps;
+    // TILEMAP variant (selected rows): row-tile i of the launch reads the weight's row-tile
+    // tile_ids[i]; row_tiles, rt_groups and n count the selected tiles, y is [m, 16 * tiles]
+    const int32_t* tile_ids;
 };
 static_assert(offsetof(GemvParams, k_units) == 64, "first-load fields must fill one 64-byte line");
 
@@ -465,7 +468,7 @@ __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 // group adds the squares of its 256 raw values while it quantizes x * norm_w, and because the
 // quantizers are invariant under a positive scale of their input (the quants stay, the block scale
 // moves), the row's factor rsqrt(mean(x^2) + eps) multiplies the finished sums instead.
-template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT, int IO = 0, bool NORM = false>
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT, int IO = 0, bool NORM = false, bool TILEMAP = false>
 __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int m_end, const uint8_t* w_first,
                                           float* y_out, int n_rows, int row_tiles, int rtg0, uint8_t* smem) {
     constexpr bool XB = IO == 2, EP = IO != 0;
@@ -491,6 +494,8 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
         for (int rtg = rtg0; ONESHOT ? rtg == rtg0 : rtg < P.rt_groups;
              rtg += ONESHOT ? 1 : (int)gridDim.x) {
             const int rt = rtg * P.nwr + wr;
+            // the weight's row-tile behind this one (uniform: a scalar load)
+            const int rt_w = TILEMAP ? P.tile_ids[rt < row_tiles ? rt : 0] : rt;
             float acc[MT];
 #pragma unroll
             for (int mi = 0; mi < MT; mi++) acc[mi] = 0.0f;
@@ -503,7 +508,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
             for (int ks = 0; ONESHOT ? ks < 1 : ks < P.kpw; ks++) {
                 const int kg = ks * P.nwk + wk;
                 const bool ok = rt < row_tiles && kg < P.k_groups;
-                const int64_t off = ok ? (int64_t)(rt * P.k_groups + kg) * P.panel_bytes : 0;
+                const int64_t off = ok ? ((int64_t)rt_w * P.k_groups + kg) * P.panel_bytes : 0;
                 Panel<QT> p;
                 const bool active = ok && lane_active;
                 if (!x_ready) {
@@ -636,7 +641,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
 // whether it exists or not.
 // The dense straight-line single-row Q4_K form is held to 80 registers: six waves per SIMD,
 // i.e. two 12-wave workgroups per CU.
-template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false, int IO = 0, bool NORM = false>
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false, int IO = 0, bool NORM = false, bool TILEMAP = false>
 __global__ __launch_bounds__(64 * kMaxWaves)
 __attribute__((amdgpu_waves_per_eu(NORM ? 3 : (ONESHOT && !GROUPED && MT == 1 && QT == QMM_Q4_K) ? 6 : 3))) void gemv_kernel(GemvParams P) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -671,7 +676,7 @@ __attribute__((amdgpu_waves_per_eu(NORM ? 3 : (ONESHOT && !GROUPED && MT == 1 &&
         else
             gemv_body<QT, 4, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     } else {
-        gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO, NORM>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
+        gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO, NORM, TILEMAP>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     }
 }
 
@@ -801,6 +806,7 @@ bool make_params(const QmmLayout& L, const void* tiled, const float* x, int64_t 
     P.ep.y_bf16 = 0;
     P.norm_w = nullptr;
     P.norm_eps = 0.0f;
+    P.tile_ids = nullptr;
     return true;
 }
 
@@ -867,6 +873,83 @@ hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x
     if (L.dtype == QMM_Q6_K) return launch_plain<QMM_Q6_K>(P, waves, n_cus, iom, stream);
     return L.dtype == QMM_Q4_K ? launch_plain<QMM_Q4_K>(P, waves, n_cus, iom, stream)
                                : launch_plain<QMM_Q8_0>(P, waves, n_cus, iom, stream);
+}
+
+namespace {
+
+// Selected rows: the looped form of the decode kernel over a list of row-tiles.
+template <int QT, int MT>
+hipError_t launch_rows_mt(const GemvParams& P, int waves, int n_cus, hipStream_t stream) {
+    const size_t lds = lds_bytes<QT, MT>(P.k_units, waves);
+    if (lds > 160 * 1024) return hipErrorInvalidValue;
+    const int64_t cap = (int64_t)n_cus * 32;
+    const int64_t grid = P.rt_groups < cap ? P.rt_groups : cap;
+    const void* fn = reinterpret_cast<const void*>(&gemv_kernel<QT, MT, false, false, false, 0, false, true>);
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+    }
+    gemv_kernel<QT, MT, false, false, false, 0, false, true><<<dim3((unsigned)grid), dim3(64 * waves), lds, stream>>>(P);
+    return hipGetLastError();
+}
+
+template <int QT>
+hipError_t launch_rows(const GemvParams& P, int waves, int n_cus, hipStream_t stream) {
+    // the row count per pass that the full product takes for this m (launch_plain)
+    if (P.m == 2 && lds_bytes<QT, 2>(P.k_units, waves) <= 64 * 1024) return launch_rows_mt<QT, 2>(P, waves, n_cus, stream);
+    return launch_rows_mt<QT, 1>(P, waves, n_cus, stream);
+}
+
+// tile_ids[i] = row-tile of token i (clamped into the matrix)
+__global__ void rows_prepare_kernel(const uint32_t* __restrict__ token_ids, int64_t count, int64_t n,
+                                    int32_t* __restrict__ tile_ids) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    const uint32_t t = token_ids[i];
+    tile_ids[i] = (int32_t)(((int64_t)t < n ? (int64_t)t : n - 1) >> 4);
+}
+
+// out[mi, i] = tiles[mi, 16 i + token_i % 16]; NaN for a token outside the matrix
+__global__ void rows_gather_kernel(const float* __restrict__ tiles, const uint32_t* __restrict__ token_ids,
+                                   int64_t count, int64_t n, int m, float* __restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    const uint32_t t = token_ids[i];
+    for (int mi = 0; mi < m; mi++)
+        out[mi * count + i] = (int64_t)t < n ? tiles[(mi * count + i) * 16 + (t & 15)] : __uint_as_float(0x7fc00000u);
+}
+
+} // namespace
+
+size_t qmm_gemv_rows_workspace_bytes(int64_t m, int64_t count) {
+    return (size_t)(((count * 4 + 255) & ~(int64_t)255) + m * count * 16 * 4);
+}
+
+hipError_t qmm_launch_gemv_rows(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
+                                const uint32_t* token_ids, int64_t count, float* out, void* workspace, int n_cus,
+                                hipStream_t stream) {
+    if (m <= 0 || count <= 0 || L.n == 0) return hipSuccess;
+    if (m > 2) return hipErrorNotSupported;
+    if (count > 0x7fffffff / 64) return hipErrorInvalidValue;
+    GemvParams P;
+    if (!make_params(L, tiled, x, m, nullptr, P)) return hipErrorInvalidValue;
+    int waves;
+    choose_split(L, n_cus, 1, false, P, waves); // the split along k of the full product: same sums
+    int32_t* tile_ids = static_cast<int32_t*>(workspace);
+    float* tiles = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + ((count * 4 + 255) & ~(int64_t)255));
+    P.tile_ids = tile_ids;
+    P.y = tiles;
+    P.row_tiles = (int)count;
+    P.n = (int)count * 16;
+    P.rt_groups = (int)((count + P.nwr - 1) / P.nwr);
+    const unsigned blocks = (unsigned)((count + 255) / 256);
+    rows_prepare_kernel<<<blocks, 256, 0, stream>>>(token_ids, count, L.n, tile_ids);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    e = with_block_type(L.dtype, [&](auto qt) { return launch_rows<decltype(qt)::value>(P, waves, n_cus, stream); });
+    if (e != hipSuccess) return e;
+    rows_gather_kernel<<<blocks, 256, 0, stream>>>(tiles, token_ids, count, L.n, (int)m, out);
+    return hipGetLastError();
 }
 
 namespace {

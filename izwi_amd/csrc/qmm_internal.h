@@ -124,6 +124,14 @@ hipError_t qmm_launch_gemv(const QmmLayout& L, const void* tiled, const float* x
                            float* y, int n_cus, hipStream_t stream, const QmmIo* io = nullptr,
                            const QmmNorm* norm = nullptr);
 
+// Selected output rows (m <= 2, hipErrorNotSupported beyond): out[mi, i] = row token_ids[i] of
+// the product, bit-identical to qmm_launch_gemv followed by a gather; only the 16-row tiles that
+// hold a selected row are read.  `workspace`: qmm_gemv_rows_workspace_bytes(m, count) bytes.
+size_t qmm_gemv_rows_workspace_bytes(int64_t m, int64_t count);
+hipError_t qmm_launch_gemv_rows(const QmmLayout& L, const void* tiled, const float* x, int64_t m,
+                                const uint32_t* token_ids, int64_t count, float* out, void* workspace, int n_cus,
+                                hipStream_t stream);
+
 // Decode kernel for the gate / up pair of an MLP: y[m, n] = silu(W_gate x) * (W_up x), both
 // matrices of layout L, m <= 2 (hipErrorNotSupported beyond).  The sums are those of
 // qmm_launch_gemv; the product is applied where the waves that split k are combined.

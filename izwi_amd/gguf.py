@@ -29,6 +29,32 @@ _SCALAR_FORMATS = {0: "<B", 1: "<b", 2: "<H", 3: "<h", 4: "<I", 5: "<i", 6: "<f"
 _STRING, _ARRAY = 8, 9
 
 
+class GgufMmapMode:
+    """backends/model_io.rs:13-45."""
+    AUTO, ON, OFF = 0, 1, 2
+    _NAMES = {0: "auto", 1: "on", 2: "off"}
+
+    @staticmethod
+    def parse(raw: str):
+        """GgufMmapMode::parse: the mode, or None for the empty string and unknown words."""
+        mode = lib().izwi_gguf_parse_mmap_mode(raw.encode("utf-8"))
+        return None if mode < 0 else mode
+
+    @classmethod
+    def as_str(cls, mode: int) -> str:
+        return cls._NAMES[mode]
+
+
+class GgufReaderKind:
+    """backends/model_io.rs:85-89."""
+    BUFFERED, MAPPED = 0, 1
+
+
+def resolve_gguf_mmap_mode(configured=None) -> int:
+    """model_io.rs:63-67: the configured mode, else IZWI_GGUF_MMAP, else auto."""
+    return lib().izwi_gguf_resolve_mmap_mode(-1 if configured is None else configured)
+
+
 def is_gguf_file(path) -> bool:
     """gguf.rs:366-377: true if the file starts with the magic bytes "GGUF"."""
     return bool(lib().izwi_gguf_is_gguf_file(os.fsencode(path)))
@@ -52,11 +78,16 @@ class GgufLoader:
         self.path = path
 
     @classmethod
-    def from_path(cls, path) -> "GgufLoader":
-        """GgufLoader::from_path (gguf.rs:44-70); parse errors raise (ModelLoadError upstream)."""
+    def from_path(cls, path, mmap_mode=None) -> "GgufLoader":
+        """GgufLoader::from_path (gguf.rs:44-70) over `open_gguf_reader_with_mode`
+        (model_io.rs:127-160); parse errors raise (ModelLoadError upstream)."""
         h = C.c_void_p()
-        check(lib().izwi_gguf_open(os.fsencode(path), C.byref(h)))
+        check(lib().izwi_gguf_open_with_mode(os.fsencode(path), -1 if mmap_mode is None else mmap_mode, C.byref(h)))
         return cls(h.value, os.fspath(path))
+
+    def reader_kind(self) -> int:
+        """GgufReader::kind (model_io.rs:96-103)."""
+        return lib().izwi_gguf_reader_kind(self._h)
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None

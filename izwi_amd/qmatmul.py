@@ -254,6 +254,26 @@ class Qwen3Projection:
     def packed_quantized(cls, parts) -> "Qwen3Projection":
         return cls(packed_qmatmul_from_qtensors(parts))
 
+    def logits_for_tokens(self, hidden: torch.Tensor, token_ids) -> list:
+        """qwen3/core.rs:745-758: [(token id, logit)] for the given ids of one hidden state
+        ([1, k] or [1, 1, k]); only the weight rows of those ids are read."""
+        ids = [int(t) for t in token_ids]
+        if not ids:
+            return []
+        k = hidden.shape[-1]
+        if hidden.numel() != k:
+            raise capi.QmmError(-1, f"Qwen3 selected-token logits expected [1,vocab] or [1,1,vocab], got {list(hidden.shape)[:-1] + ['vocab']}")
+        n = self.qmatmul.qtensor.dims2()[0]
+        if max(ids) >= n or min(ids) < 0:
+            raise capi.QmmError(-1, f"token id out of range for a vocabulary of {n}")
+        x = hidden.to(torch.float32).contiguous().view(1, k)
+        import numpy as np
+        idt = torch.from_numpy(np.asarray(ids, dtype=np.uint32).view(np.int32)).to(x.device)
+        y = torch.empty((1, len(ids)), dtype=torch.float32, device=x.device)
+        check(lib().izwi_qmm_forward_rows_f32(self.qmatmul.qtensor._h, idt.data_ptr(), len(ids), x.data_ptr(), 1,
+                                              y.data_ptr(), _space(x), _stream_ptr(x)))
+        return list(zip(ids, y.view(-1).tolist()))
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """qwen3/core.rs:791-831.  f32 goes straight to the op.  bf16 inputs go through the
         fused call, which reads them as they are and rounds the f32 sums back to bf16 (the

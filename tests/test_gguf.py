@@ -174,6 +174,74 @@ def test_malformed_files_are_errors(qa, tmp_path):
         qa.GgufLoader.from_path(p)
 
 
+def test_reader_policy_follows_the_reference(qa, tmp_path, monkeypatch):
+    """backends/model_io.rs:13-160 and its tests (`parse_mode_supports_aliases`,
+    `parse_mode_rejects_unknown_values`, `resolve_mode_prefers_explicit_value_then_env_then_auto_default`,
+    `open_reader_uses_buffered_mode_when_explicitly_disabled`), plus the fallback to buffered I/O
+    when the mapping fails (model_io.rs:146-160)."""
+    from izwi_amd.gguf import GgufMmapMode as M, GgufReaderKind as K, resolve_gguf_mmap_mode
+    assert M.parse("auto") == M.AUTO
+    for word in ("on", "true", "1", "yes", " ON ", "Yes"):
+        assert M.parse(word) == M.ON, word
+    for word in ("off", "false", "0", "no", "OFF\n"):
+        assert M.parse(word) == M.OFF, word
+    assert M.parse("") is None and M.parse("invalid") is None
+    assert [M.as_str(m) for m in (M.AUTO, M.ON, M.OFF)] == ["auto", "on", "off"]
+    monkeypatch.delenv("IZWI_GGUF_MMAP", raising=False)
+    assert resolve_gguf_mmap_mode(None) == M.AUTO
+    monkeypatch.setenv("IZWI_GGUF_MMAP", "off")
+    assert resolve_gguf_mmap_mode(None) == M.OFF
+    assert resolve_gguf_mmap_mode(M.ON) == M.ON
+    monkeypatch.setenv("IZWI_GGUF_MMAP", "nonsense")
+    assert resolve_gguf_mmap_mode(None) == M.AUTO
+
+    path, metadata, tensors, *_ = _sample(tmp_path)
+
+    def contents(g):
+        return (g.header(), g.tensor_names(), [g.tensor_bytes(n) for n in g.tensor_names()],
+                {k: g.metadata_value(k) for k in g.metadata_keys()} if hasattr(g, "metadata_keys") else None)
+
+    monkeypatch.delenv("IZWI_GGUF_MMAP", raising=False)
+    mapped = qa.GgufLoader.from_path(path)
+    assert mapped.reader_kind() == K.MAPPED                       # auto maps on every backend
+    assert qa.GgufLoader.from_path(path, M.ON).reader_kind() == K.MAPPED
+    buffered = qa.GgufLoader.from_path(path, M.OFF)
+    assert buffered.reader_kind() == K.BUFFERED
+    assert contents(buffered) == contents(mapped)
+    monkeypatch.setenv("IZWI_GGUF_MMAP", "0")                     # the environment when nothing is configured
+    assert qa.GgufLoader.from_path(path).reader_kind() == K.BUFFERED
+    assert qa.GgufLoader.from_path(path, M.ON).reader_kind() == K.MAPPED
+    monkeypatch.delenv("IZWI_GGUF_MMAP")
+    # a mapping that fails falls back to buffered I/O, with the same contents
+    monkeypatch.setenv("IZWI_GGUF_TEST_FAIL_MMAP", "1")
+    fell_back = qa.GgufLoader.from_path(path, M.ON)
+    assert fell_back.reader_kind() == K.BUFFERED and contents(fell_back) == contents(mapped)
+    monkeypatch.delenv("IZWI_GGUF_TEST_FAIL_MMAP")
+    # malformed input is an error in buffered mode too
+    from izwi_amd.capi import QmmError
+    bad = tmp_path / "bad.gguf"
+    bad.write_bytes(open(path, "rb").read()[:40])
+    with pytest.raises(QmmError):
+        qa.GgufLoader.from_path(bad, M.OFF)
+
+
+def test_crafted_counts_do_not_exhaust_memory(qa, tmp_path):
+    """An array-of-strings count far beyond what the file can hold is refused before anything is
+    reserved for it (8 bytes per entry at least, 4 in version 1)."""
+    from izwi_amd.capi import QmmError
+    for version, ln in ((3, "<Q"), (1, "<I")):
+        key = b"general.name"
+        head = b"GGUF" + struct.pack("<I", version) + struct.pack(ln, 0) + struct.pack(ln, 1)
+        kv = struct.pack(ln, len(key)) + key + struct.pack("<I", 9) + struct.pack("<I", 8)
+        body = bytes(64 * 1024)
+        # the count that would just pass a bytes-remaining bound but not the bytes / entry-size one
+        count = len(body) // (2 if version == 3 else 1)
+        p = tmp_path / f"crafted{version}.gguf"
+        p.write_bytes(head + kv + struct.pack(ln, count) + body)
+        with pytest.raises(QmmError, match="GGUF"):
+            qa.GgufLoader.from_path(p)
+
+
 def test_committed_fixture(qa):
     """tests/golden/tiny.gguf is data: the bytes of a small GGUF file and, beside it, what a
     reader must find in it (written once by tests/golden/make_fixtures.py)."""

@@ -338,6 +338,53 @@ def test_forward_f32_large_m_uses_prefill_kernel(qa, oracle):
     assert rel_err(y, oracle.qmatmul(Q4_K, x, blocks, 256)) < PREFILL_TOL
 
 
+def forward_rows(qa, q, ids, x):
+    """izwi_qmm_forward_rows_f32 through the C ABI on device or host tensors."""
+    from izwi_amd import capi
+    idt = torch.from_numpy(np.asarray(ids, dtype=np.uint32).view(np.int32)).to(x.device)
+    y = torch.empty((x.shape[0], len(ids)), dtype=torch.float32, device=x.device)
+    capi.check(capi.lib().izwi_qmm_forward_rows_f32(
+        q._h, idt.data_ptr(), len(ids), x.data_ptr(), x.shape[0], y.data_ptr(),
+        capi.DEVICE if x.is_cuda else capi.HOST, torch.cuda.current_stream().cuda_stream if x.is_cuda else None))
+    return y
+
+
+@pytest.mark.parametrize("dtype,n,k", [(Q4_K, 151936, 4096), (Q4_K, 4096, 4096), (Q4_K, 4096, 12288), (Q8_0, 3072, 1024),
+                                       (Q4_K, 1000, 768), (Q8_0, 50, 352)])
+def test_selected_rows_equal_full_forward_then_gather(qa, oracle, dtype, n, k):
+    """`logits_for_tokens` (qwen3/core.rs:745-758, 2155-2171): the reference runs the full LM head
+    and index_selects; the row-subset call must give those bits while reading only the selected tiles."""
+    _say(f"rows dtype={dtype} n={n} k={k}")
+    blocks = make_weight(oracle, dtype, n, k, 180)
+    q = qa.QTensor.from_blocks(qa.GgmlDType(dtype), blocks, (n, k))
+    mm = qa.QMatMul.from_qtensor(q)
+    rng = np.random.default_rng(181)
+    ids = [0, n - 1, n - 1, 17, 16, 15] + [int(v) for v in rng.integers(0, n, size=70)]   # repeats, unsorted, both ends
+    for m in (1, 2):
+        x = torch.from_numpy(oracle.randn(182 + m, (m, k))).cuda()
+        full = mm.forward(x)
+        got = forward_rows(qa, q, ids, x)
+        torch.cuda.synchronize()
+        assert torch.equal(got, full[:, torch.tensor(ids, device="cuda")]), m
+    # one id; host pointers (staged), where an id beyond the matrix is refused as index_select refuses it
+    assert torch.equal(forward_rows(qa, q, [n // 2], x), full[:, n // 2:n // 2 + 1])
+    assert torch.equal(forward_rows(qa, q, ids, x.cpu()), got.cpu())
+    from izwi_amd import capi
+    with pytest.raises(capi.QmmError, match="out of range"):
+        forward_rows(qa, q, [n], x.cpu())
+    assert torch.isnan(forward_rows(qa, q, [3, n, 5], x)[:, 1]).all()       # device ids: no host round trip
+    with pytest.raises(capi.QmmError, match="selected-token"):
+        forward_rows(qa, q, ids, torch.zeros((3, k), device="cuda"))
+    # the mirror of Qwen3Projection::logits_for_tokens: pairs (id, value) for one hidden state
+    proj = qa.Qwen3Projection(mm, is_lm_head=True)
+    pairs = proj.logits_for_tokens(x[:1].view(1, 1, k), ids[:9])
+    assert [p[0] for p in pairs] == ids[:9]
+    assert pairs == list(zip(ids[:9], mm.forward(x[:1])[0, torch.tensor(ids[:9], device="cuda")].tolist()))
+    assert proj.logits_for_tokens(x[:1], []) == []
+    with pytest.raises(capi.QmmError, match="selected-token"):
+        proj.logits_for_tokens(x, ids)
+
+
 def test_large_m_arithmetic_switch(qa, oracle):
     """Beyond 64 rows `forward_f32` changes arithmetic (bf16 matrix cores on dequantized weights)
     unless the caller selects the integer dots: the error against the reference's CPU result at
