@@ -150,6 +150,12 @@ typedef enum izwi_qmm_large_m { IZWI_QMM_LARGE_M_BF16 = 0, IZWI_QMM_LARGE_M_INT8
 int izwi_qmm_set_large_m_arithmetic(int mode);
 int izwi_qmm_get_large_m_arithmetic(void);
 
+/* Tuning switch of the MoE expert MLP at many pairs per expert: 1 = the expert form of the grouped
+ * matrix-core kernel (a workgroup per expert keeps up to four activation tiles in LDS), 0 = the
+ * one-shot form (default; also IZWI_QMM_MOE_EXPERT_FORM=1 at start-up).  Same results either way.
+ * No counterpart in the reference (it has no MoE code). */
+int izwi_qmm_set_moe_expert_form(int enabled);
+
 /* Grows the scratch buffer of (current device, stream) to at least `bytes` now, so that later
  * calls on that stream allocate nothing (needed before the stream is captured into a HIP graph).
  * No counterpart in the reference. */
@@ -338,8 +344,13 @@ int izwi_moe_layer_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
  * `is_lm_head` calls are additionally counted in lm_head_* when the caller
  * marks the handle with izwi_qmm_weight_set_lm_head. */
 int izwi_qmm_profile_enable(int enabled);
+int izwi_qmm_profile_enabled(void); /* `qwen3_runtime_profiling_enabled` (qwen3/core.rs:624-640): 1 or 0 */
 int izwi_qmm_profile_snapshot_get(izwi_qmm_profile_snapshot* out);
 int izwi_qmm_profile_reset(void);
+/* `argmax_calls` / `argmax_ms` of the ASR profile diagnostics `izwi bench` prints
+ * (qwen3/asr/mod.rs:116-131, crates/izwi-cli/src/commands/bench.rs:281-295): calls of
+ * izwi_argmax_f32 and their wall time in ns while profiling is enabled. */
+int izwi_qmm_profile_argmax_get(uint64_t* calls, uint64_t* ns);
 int izwi_qmm_weight_set_lm_head(izwi_qmm_weight* w, int is_lm_head);
 
 #ifdef __cplusplus

@@ -17,7 +17,7 @@ from .decode_ops import (  # noqa: F401
     try_fused_rms_norm,
     try_fused_rope_pair_bshd,
 )
-from .gguf import GgufLoader, GgufModelInfo, is_gguf_file  # noqa: F401
+from .gguf import GgufLoader, GgufMmapMode, GgufModelInfo, GgufReaderKind, is_gguf_file, resolve_gguf_mmap_mode  # noqa: F401
 from .qmatmul import (  # noqa: F401
     GgmlDType,
     MoeExperts,
@@ -27,6 +27,7 @@ from .qmatmul import (  # noqa: F401
     Qwen3Mlp,
     Qwen3Projection,
     Qwen3QkvProjection,
+    asr_profile_diagnostics,
     forward_group,
     moe_route,
     moe_sort,

@@ -90,10 +90,13 @@ PROTOTYPES = {
                                        C.c_int, _vp]),
     "izwi_qmm_set_large_m_arithmetic": (C.c_int, [C.c_int]),
     "izwi_qmm_get_large_m_arithmetic": (C.c_int, []),
+    "izwi_qmm_set_moe_expert_form": (C.c_int, [C.c_int]),
     "izwi_qmm_scratch_reserve": (C.c_int, [_u64, _vp]),
     "izwi_qmm_profile_enable": (C.c_int, [C.c_int]),
+    "izwi_qmm_profile_enabled": (C.c_int, []),
     "izwi_qmm_profile_snapshot_get": (C.c_int, [C.POINTER(ProfileSnapshot)]),
     "izwi_qmm_profile_reset": (C.c_int, []),
+    "izwi_qmm_profile_argmax_get": (C.c_int, [C.POINTER(_u64), C.POINTER(_u64)]),
     "izwi_qmm_weight_set_lm_head": (C.c_int, [_vp, C.c_int]),
     # include/izwi_gguf.h
     "izwi_gguf_is_gguf_file": (C.c_int, [C.c_char_p]),

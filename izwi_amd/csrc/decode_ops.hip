@@ -12,6 +12,8 @@
 //    every 128-byte segment (coalesced), 32 rows are in flight per workgroup.
 #include <hip/hip_runtime.h>
 
+#include <chrono>
+
 #include <type_traits>
 
 #include <math.h>
@@ -904,8 +906,28 @@ int izwi_rope_pair_bshd_f16(const uint16_t* q, const uint16_t* k, const uint16_t
                                  head_dim, (f16_t*)q_out, (f16_t*)k_out, mem_space, stream);
 }
 
+namespace {
+// `argmax_calls` / `argmax_ms` of the reference's ASR profile (asr/mod.rs:116-131): counted and,
+// outside a capture, timed to completion when profiling is on.
+struct ArgmaxProfile {
+    bool on;
+    hipStream_t stream;
+    std::chrono::steady_clock::time_point t0;
+    explicit ArgmaxProfile(hipStream_t s) : on(qmm_profiling()), stream(s) {
+        if (on) t0 = std::chrono::steady_clock::now();
+    }
+    ~ArgmaxProfile() {
+        if (!on) return;
+        if (!qmm_stream_is_capturing(stream)) (void)hipStreamSynchronize(stream);
+        qmm_profile_count_argmax((uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(
+                                     std::chrono::steady_clock::now() - t0).count());
+    }
+};
+} // namespace
+
 int izwi_argmax_f32(const float* logits, int64_t rows, int64_t n, uint32_t* out, int mem_space, void* stream_) {
     QmmCallScope call;
+    ArgmaxProfile prof((hipStream_t)stream_);
     if (int rc = check_space(mem_space)) return rc;
     if (rows < 0 || n <= 0 || n > 0xfffffffeLL || rows > 0x7fffffff)
         return qmm_fail(IZWI_QMM_ERR_INVALID, "argmax: bad shape [%lld, %lld]", (long long)rows, (long long)n);

@@ -375,7 +375,7 @@ int check_space(int mem_space) {
 // ---- profiling -----------------------------------------------------------
 std::atomic<int> g_profile{-1}; // -1: read the environment on first use
 std::atomic<uint64_t> g_calls{0}, g_ns{0}, g_in_casts{0}, g_in_cast_ns{0}, g_out_casts{0},
-    g_out_cast_ns{0}, g_lm_calls{0}, g_lm_ns{0}, g_silu_fused{0}, g_silu_fallback{0};
+    g_out_cast_ns{0}, g_lm_calls{0}, g_lm_ns{0}, g_silu_fused{0}, g_silu_fallback{0}, g_argmax_calls{0}, g_argmax_ns{0};
 
 bool parse_env_bool(const char* raw) {
     if (!raw) return false;
@@ -427,6 +427,22 @@ int qmm_current_device(int* device, int* n_cus) {
 }
 hipError_t qmm_get_scratch(int device, hipStream_t stream, size_t bytes, void** out) {
     return get_scratch(device, stream, bytes, out);
+}
+std::atomic<int> g_moe_expert_form{-1}; // -1: read IZWI_QMM_MOE_EXPERT_FORM on first use
+bool qmm_moe_expert_form() {
+    int v = g_moe_expert_form.load(std::memory_order_relaxed);
+    if (v < 0) {
+        const char* e = getenv("IZWI_QMM_MOE_EXPERT_FORM");
+        v = e && e[0] == '1';
+        g_moe_expert_form.store(v, std::memory_order_relaxed);
+    }
+    return v != 0;
+}
+bool qmm_profiling() { return profiling(); }
+bool qmm_stream_is_capturing(hipStream_t stream) { return stream_is_capturing(stream); }
+void qmm_profile_count_argmax(uint64_t ns) {
+    g_argmax_calls.fetch_add(1, std::memory_order_relaxed);
+    g_argmax_ns.fetch_add(ns, std::memory_order_relaxed);
 }
 QmmCallScope::QmmCallScope() { t_call_depth++; }
 QmmCallScope::~QmmCallScope() {
@@ -1413,6 +1429,11 @@ int izwi_qmm_set_large_m_arithmetic(int mode) {
 
 int izwi_qmm_get_large_m_arithmetic(void) { return large_m_mode(); }
 
+int izwi_qmm_set_moe_expert_form(int enabled) {
+    g_moe_expert_form.store(enabled ? 1 : 0, std::memory_order_relaxed);
+    return IZWI_QMM_OK;
+}
+
 int izwi_qmm_scratch_reserve(uint64_t bytes, void* stream_) {
     int device = 0;
     if (int rc = current_device(&device)) return rc;
@@ -1442,9 +1463,18 @@ int izwi_qmm_profile_snapshot_get(izwi_qmm_profile_snapshot* out) {
     return IZWI_QMM_OK;
 }
 
+int izwi_qmm_profile_enabled(void) { return profiling() ? 1 : 0; }
+
+int izwi_qmm_profile_argmax_get(uint64_t* calls, uint64_t* ns) {
+    if (!calls || !ns) return fail(IZWI_QMM_ERR_INVALID, "NULL argument");
+    *calls = g_argmax_calls.load(std::memory_order_relaxed);
+    *ns = g_argmax_ns.load(std::memory_order_relaxed);
+    return IZWI_QMM_OK;
+}
+
 int izwi_qmm_profile_reset(void) {
     for (auto* c : {&g_calls, &g_ns, &g_in_casts, &g_in_cast_ns, &g_out_casts, &g_out_cast_ns,
-                    &g_lm_calls, &g_lm_ns, &g_silu_fused, &g_silu_fallback})
+                    &g_lm_calls, &g_lm_ns, &g_silu_fused, &g_silu_fallback, &g_argmax_calls, &g_argmax_ns})
         c->store(0, std::memory_order_relaxed);
     return IZWI_QMM_OK;
 }

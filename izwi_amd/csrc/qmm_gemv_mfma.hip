@@ -1170,10 +1170,10 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     P.y2 = y2;
     P.n_weights = 0;
     {
-        // the expert form (IZWI_QMM_MOE_EXPERT_FORM=1; off by default: measured no faster than the one-shot
+        // the expert form (IZWI_QMM_MOE_EXPERT_FORM=1 or izwi_qmm_set_moe_expert_form; off by default: measured no faster than the one-shot
         // form once the experts' tile counts are uneven) where at least two activation tiles over all of
         // k fit in LDS
-        static const bool expert_form = [] { const char* e = getenv("IZWI_QMM_MOE_EXPERT_FORM"); return e && e[0] == '1'; }();
+        const bool expert_form = qmm_moe_expert_form();
         const size_t tile_bytes = (size_t)L.k_units * unit_bytes(L.dtype);
         // (Q6_K: two tiles at a time, four do not fit the registers)
         const int tc = L.dtype != QMM_Q6_K && 4 * tile_bytes <= 150 * 1024 ? 4 : (2 * tile_bytes <= 150 * 1024 ? 2 : 0);

@@ -98,6 +98,13 @@ int qmm_current_device(int* device, int* n_cus);
 // same stream wait for that.  Grows with hipMalloc (an outgrown buffer is kept until the process
 // ends, never freed); hipErrorStreamCaptureUnsupported if it would have to grow during a capture.
 hipError_t qmm_get_scratch(int device, hipStream_t stream, size_t bytes, void** out);
+// Profiling (IZWI_QWEN3_PROFILE / izwi_qmm_profile_enable) for the library's other source files:
+// whether it is on, whether a stream is being captured (no waits then), one device argmax call.
+bool qmm_profiling();
+bool qmm_stream_is_capturing(hipStream_t stream);
+void qmm_profile_count_argmax(uint64_t ns);
+// Whether the expert-grouped matrix-core kernel takes its expert form (a tuning switch, off by default).
+bool qmm_moe_expert_form();
 // One library call on this thread: every exported entry point that may reach qmm_get_scratch
 // opens one first.  Scopes nest (entry points call each other); the outermost one releases the
 // scratch buffers its call took.

@@ -254,6 +254,11 @@ class Qwen3Projection:
     def packed_quantized(cls, parts) -> "Qwen3Projection":
         return cls(packed_qmatmul_from_qtensors(parts))
 
+    def diagnostics(self) -> dict:
+        """Qwen3Projection::diagnostics (qwen3/core.rs:729-742) for the Quantized arm: the counts that
+        feed `qmatmul_projection_count` / `dense_projection_count` of the ASR execution diagnostics."""
+        return {"dense_projection_count": 0, "dense_bias_projection_count": 0, "quantized_projection_count": 1}
+
     def logits_for_tokens(self, hidden: torch.Tensor, token_ids) -> list:
         """qwen3/core.rs:745-758: [(token id, logit)] for the given ids of one hidden state
         ([1, k] or [1, 1, k]); only the weight rows of those ids are read."""
@@ -450,3 +455,26 @@ def profile_snapshot() -> dict:
     snap = capi.ProfileSnapshot()
     check(lib().izwi_qmm_profile_snapshot_get(C.byref(snap)))
     return {name: getattr(snap, name) for name, _ in snap._fields_}
+
+
+def asr_profile_diagnostics() -> dict:
+    """The fields of Qwen3AsrProfileDiagnostics (qwen3/asr/mod.rs:116-147) that `izwi bench` reads
+    (crates/izwi-cli/src/commands/bench.rs:281-295), filled from the library's counters the way
+    `update_from_runtime_delta` fills them: ns -> ms, plus the device argmax."""
+    snap = profile_snapshot()
+    calls, ns = C.c_uint64(), C.c_uint64()
+    check(lib().izwi_qmm_profile_argmax_get(C.byref(calls), C.byref(ns)))
+    ms = lambda v: v / 1e6  # noqa: E731
+    return {
+        "qwen3_profile_enabled": capi_profile_enabled(),
+        "qmatmul_calls": snap["qmatmul_calls"], "qmatmul_ms": ms(snap["qmatmul_ns"]),
+        "qmatmul_input_casts": snap["qmatmul_input_casts"], "qmatmul_input_cast_ms": ms(snap["qmatmul_input_cast_ns"]),
+        "qmatmul_output_casts": snap["qmatmul_output_casts"], "qmatmul_output_cast_ms": ms(snap["qmatmul_output_cast_ns"]),
+        "lm_head_calls": snap["lm_head_calls"], "lm_head_ms": ms(snap["lm_head_ns"]),
+        "silu_mul_fused_calls": snap["silu_mul_fused_calls"], "silu_mul_fallback_calls": snap["silu_mul_fallback_calls"],
+        "argmax_calls": calls.value, "argmax_ms": ms(ns.value),
+    }
+
+
+def capi_profile_enabled() -> bool:
+    return bool(lib().izwi_qmm_profile_enabled())

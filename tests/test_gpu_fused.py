@@ -122,7 +122,18 @@ def test_fused_host_memory_profile_counters_and_errors(qa, oracle):
     mm.forward_fused(xb)
     mm.forward_fused(xb, out_dtype=torch.float32)
     snap = qa.profile_snapshot()
+    # the ASR profile fields `izwi bench` prints (asr/mod.rs:116-147): the same counters in ms, plus the argmax
+    assert L.izwi_qmm_profile_enabled() == 1
+    logits = torch.from_numpy(oracle.randn(6, (2, 151936))).cuda()
+    assert qa.argmax(logits).cpu().tolist() == logits.argmax(dim=-1).cpu().tolist()
+    diag = qa.asr_profile_diagnostics()
+    assert diag["qwen3_profile_enabled"] and diag["argmax_calls"] == 1 and diag["argmax_ms"] > 0
+    assert diag["qmatmul_calls"] == 2 and diag["qmatmul_ms"] == snap["qmatmul_ns"] / 1e6
+    assert diag["silu_mul_fused_calls"] == 0 and diag["lm_head_calls"] == 0
     L.izwi_qmm_profile_enable(0)
+    assert L.izwi_qmm_profile_enabled() == 0
+    qa.argmax(logits)
+    assert qa.asr_profile_diagnostics()["argmax_calls"] == 1            # not counted while off
     assert snap["qmatmul_calls"] == 2 and snap["qmatmul_input_casts"] == 2 and snap["qmatmul_output_casts"] == 1
     assert snap["qmatmul_input_cast_ns"] == 0 and snap["qmatmul_output_cast_ns"] == 0
     y = torch.empty(m, n, device="cuda")

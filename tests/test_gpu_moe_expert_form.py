@@ -1,20 +1,24 @@
-"""The optional expert form of the grouped matrix-core kernel (IZWI_QMM_MOE_EXPERT_FORM=1, read once per
-process): the MoE parity tests once more in a child process with the switch on."""
-import os
-import subprocess
-import sys
-
+"""The optional expert form of the grouped matrix-core kernel (izwi_qmm_set_moe_expert_form /
+IZWI_QMM_MOE_EXPERT_FORM=1): the MoE parity tests once more, in this process, with the switch on, so
+that every case reports on its own."""
 import pytest
+
+# the tests themselves (collected here a second time, with their parameters) and the fixtures they use
+from test_gpu_parity import (  # noqa: F401
+    moe_weights,
+    qa,
+    test_config5_moe_forward,
+    test_config5_moe_layer_one_call_equals_the_three_calls,
+    test_moe_forward_small_shapes,
+)
+from test_gpu_q6k import test_moe_with_q6_k_expert_stacks  # noqa: F401
 
 pytestmark = pytest.mark.gpu
 
 
-def test_moe_parity_with_the_expert_form():
-    here = os.path.dirname(os.path.abspath(__file__))
-    env = dict(os.environ, IZWI_QMM_MOE_EXPERT_FORM="1")
-    cmd = [sys.executable, "-u", "-m", "pytest", "-x", "-q", "-m", "gpu", "--timeout", "120", "--timeout-method", "thread",
-           "-k", "moe_forward_small_shapes or moe_with_q6_k_expert_stacks or config5_moe_forward",
-           os.path.join(here, "test_gpu_parity.py"), os.path.join(here, "test_gpu_q6k.py")]
-    out = subprocess.run(cmd, env=env, cwd=os.path.dirname(here), capture_output=True, text=True, timeout=600)
-    assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-2000:]
-    assert " passed" in out.stdout and "failed" not in out.stdout
+@pytest.fixture(autouse=True)
+def expert_form():
+    from izwi_amd import capi
+    capi.check(capi.lib().izwi_qmm_set_moe_expert_form(1))
+    yield
+    capi.check(capi.lib().izwi_qmm_set_moe_expert_form(0))
