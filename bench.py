@@ -314,6 +314,36 @@ def overlap_what_if_extra(torch, qa, calls, total_bytes, n_streams=3, steps=20, 
             "note": "launches overlapped as if independent; not the model's dependent chain, not `value`"}
 
 
+def chained_extra(torch, qa, calls, total_bytes, steps=20, warmup=3):
+    """Extra report (not `value`): the headline's dependent calls as ONE launch (izwi_qmm_chain_*: a
+    resident grid walks through the steps, hand-over through write-through stores and counters, the
+    next step's weights requested before the wait); the LM head behind it as its own call.  Also a
+    144-step chain of the smallest projection alone, whose per-step time is the cost of one
+    grid-wide hand-over (its 9.4 MB stream in 1.2 us)."""
+    def as_step(c):
+        mm, x, y = c
+        return (list(mm), x, list(y)) if isinstance(mm, (list, tuple)) else ([mm], x, [y])
+    chain = qa.DecodeChain([as_step(c) for c in calls[:-1]])
+
+    def run():
+        chain.run()
+        run_calls(qa, calls[-1:])
+    ms, g = time_graph(torch, run, steps, warmup)
+    chain.status()
+    del g
+    small = [as_step(c) for c in calls[1:-1:4]]       # the o projections
+    chain_o = qa.DecodeChain(small)
+    ms_o, g = time_graph(torch, chain_o.run, steps, warmup)
+    chain_o.status()
+    del g
+    ms_o_calls, g = time_graph(torch, lambda: run_calls(qa, calls[1:-1:4]), steps, warmup)
+    del g
+    return {"gbs": round(total_bytes / (ms * 1e-3) / 1e9, 1), "ms_per_step": round(ms, 4), "launches_per_step": 2,
+            "us_per_dependent_step_4096x4096_chained": round(ms_o * 1e3 / len(small), 2),
+            "us_per_dependent_step_4096x4096_separate_calls": round(ms_o_calls * 1e3 / len(small), 2),
+            "note": "one resident kernel for the 144 dependent projection steps + the LM head call; not `value`"}
+
+
 def host_pointer_extra(qa, weights, m, passes=2):
     """Extra report (not `value`): the same projections called one by one with HOST pointers, the literal
     form of the reference's CPU call (activations in host memory in, results in host memory out): every
@@ -749,6 +779,8 @@ def main():
             del c, g
             c, tb = make_calls(torch, dtype, weights, args.m)
             extras["decode_overlap_what_if"] = overlap_what_if_extra(torch, qa, c, tb)
+            if args.m == 1 and args.calls == "grouped":
+                extras["decode_chained_one_launch"] = chained_extra(torch, qa, c, tb)
             del c
             extras["decode_host_pointer_calls"] = host_pointer_extra(qa, weights, args.m)
             extras["hbm_ceiling_measured"] = hbm_ceiling_extra(torch)

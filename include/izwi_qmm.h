@@ -207,6 +207,50 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
 int izwi_qmm_forward_rows_f32(const izwi_qmm_weight* w, const uint32_t* row_ids, int64_t n_rows, const float* x,
                               int64_t m, float* y, int mem_space, void* stream);
 
+/* --- chained decode: the projections of one token as one launch ----------- */
+
+/* One token's projections in the order `Qwen3Layer::forward` issues them (qwen3/core.rs:1863-1881:
+ * q|k|v, o, gate|up, down, layer after layer; `Qwen3Model::logits_from_hidden`, core.rs:2114-2125,
+ * at the end) depend on each other: each reads activations that an earlier one (or the attention /
+ * activation kernel between them) wrote.  As separate calls every one of them pays the gap
+ * between two dependent launches and its own ramp-up and drain.  A chain is that list of calls
+ * prepared once and run as ONE kernel launch per token; step i does not read its x before step
+ * i - 1 has completed (exactly the order a stream gives the separate calls), and the weights of
+ * the next step are requested while the current step finishes.
+ *
+ * A step is izwi_qmm_forward_group_f32 at m = 1: 1..4 weights of equal k, one x [k], one y [n_i]
+ * per weight; results are bit-identical to that call.  All buffers are device memory and must
+ * stay valid, at the same addresses, for the life of the chain; the weights of a chain share one
+ * block type and the current device; k <= 12288 (12 panels of 1024) and n < 256 * (compute units)
+ * (an LM head runs as a call of its own behind the chain).  The launch occupies every
+ * compute unit with one resident workgroup: run nothing else beside it.  Waits inside the kernel
+ * are bounded: if one gives up (another kernel held the GPU for about a second), the results of that
+ * run are invalid, every workgroup still exits, and izwi_qmm_chain_status returns IZWI_QMM_ERR_HIP
+ * (and makes the chain usable again).  izwi_qmm_chain_run is asynchronous on `stream`, allocates
+ * nothing and may be captured into a HIP graph; one chain must not run twice at the same time.
+ * Measured on MI355X (Qwen3-8B, Q4_K, 144 steps): 1.44 ms per token against 1.01 ms for the same
+ * steps as separate calls in a HIP graph: a grid-wide hand-over through memory (write-through
+ * stores, counters, device-scope loads) costs about 7 us per dependent step where a kernel
+ * boundary costs about 3.5, and the overlap of the next step's weight stream does not make up for
+ * it.  The separate calls stay the fast path; the chain is kept as the measured alternative.
+ * No counterpart in the reference, which issues one Candle op per projection. */
+typedef struct izwi_qmm_chain izwi_qmm_chain;
+typedef struct izwi_qmm_chain_step {
+    const izwi_qmm_weight* weights[4];
+    int32_t n_weights;
+    int32_t reserved;
+    const float* x; /* device, [k] */
+    float* ys[4];   /* device, [n_i] */
+} izwi_qmm_chain_step;
+int izwi_qmm_chain_create(const izwi_qmm_chain_step* steps, int32_t n_steps, izwi_qmm_chain** out);
+void izwi_qmm_chain_destroy(izwi_qmm_chain* chain);
+int izwi_qmm_chain_run(izwi_qmm_chain* chain, void* stream);
+/* Waits for `stream`, then reports whether a wait inside any run since the last status call gave up. */
+int izwi_qmm_chain_status(izwi_qmm_chain* chain, void* stream);
+/* Polls (about 0.5 us each) after which a wait gives up; default 2^21, also IZWI_QMM_CHAIN_SPIN_LIMIT.
+ * 0 makes every wait that is not already satisfied give up at once (for tests of the error path). */
+int izwi_qmm_chain_set_spin_limit(izwi_qmm_chain* chain, uint32_t polls);
+
 /* izwi_qmm_forward_f32 for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
  * reference.  Same kernels and the same results, bit for bit, as izwi_qmm_forward_f32 with

@@ -43,6 +43,12 @@ _i32, _i64, _u64, _vp = C.c_int32, C.c_int64, C.c_uint64, C.c_void_p
 _pp = C.POINTER(C.c_void_p)
 _cpp = C.POINTER(C.c_char_p)
 
+class ChainStep(C.Structure):
+    """izwi_qmm_chain_step"""
+    _fields_ = [("weights", C.c_void_p * 4), ("n_weights", C.c_int32), ("reserved", C.c_int32),
+                ("x", C.c_void_p), ("ys", C.c_void_p * 4)]
+
+
 # name -> (restype, argtypes); must list every symbol include/izwi_qmm.h and include/izwi_gguf.h declare
 PROTOTYPES = {
     "izwi_qmm_abi_version": (C.c_int, []),
@@ -58,6 +64,11 @@ PROTOTYPES = {
     "izwi_qmm_weight_data": (C.c_int, [_vp, _vp, _u64, C.c_int, _vp]),
     "izwi_qmm_dequantize_f32": (C.c_int, [_vp, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_f32": (C.c_int, [_vp, _vp, _i64, _vp, C.c_int, _vp]),
+    "izwi_qmm_chain_create": (C.c_int, [_vp, _i32, _pp]),
+    "izwi_qmm_chain_destroy": (None, [_vp]),
+    "izwi_qmm_chain_run": (C.c_int, [_vp, _vp]),
+    "izwi_qmm_chain_status": (C.c_int, [_vp, _vp]),
+    "izwi_qmm_chain_set_spin_limit": (C.c_int, [_vp, C.c_uint32]),
     "izwi_qmm_forward_rows_f32": (C.c_int, [_vp, _vp, _i64, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_f32_noalloc": (C.c_int, [_vp, _vp, _i64, _vp, _vp]),
     "izwi_qmm_forward_group_f32": (C.c_int, [_vp, _i32, _vp, _i64, _vp, C.c_int, _vp]),

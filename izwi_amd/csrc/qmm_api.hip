@@ -438,6 +438,9 @@ bool qmm_moe_expert_form() {
     }
     return v != 0;
 }
+const QmmLayout* qmm_weight_layout(const izwi_qmm_weight* w) { return &w->layout; }
+const void* qmm_weight_tiled(const izwi_qmm_weight* w) { return w->tiled; }
+int qmm_weight_device(const izwi_qmm_weight* w) { return w->device; }
 bool qmm_profiling() { return profiling(); }
 bool qmm_stream_is_capturing(hipStream_t stream) { return stream_is_capturing(stream); }
 void qmm_profile_count_argmax(uint64_t ns) {

@@ -105,6 +105,11 @@ bool qmm_stream_is_capturing(hipStream_t stream);
 void qmm_profile_count_argmax(uint64_t ns);
 // Whether the expert-grouped matrix-core kernel takes its expert form (a tuning switch, off by default).
 bool qmm_moe_expert_form();
+// A weight handle's layout, device matrix and device ordinal, for the library's other source files.
+struct izwi_qmm_weight;
+const QmmLayout* qmm_weight_layout(const izwi_qmm_weight* w);
+const void* qmm_weight_tiled(const izwi_qmm_weight* w);
+int qmm_weight_device(const izwi_qmm_weight* w);
 // One library call on this thread: every exported entry point that may reach qmm_get_scratch
 // opens one first.  Scopes nest (entry points call each other); the outermost one releases the
 // scratch buffers its call took.

@@ -317,6 +317,52 @@ def forward_group(projections: Sequence["QMatMul"], x: torch.Tensor, norm_weight
     return tuple(ys)
 
 
+class DecodeChain:
+    """One token's projections as one launch (izwi_qmm_chain_*): ``steps`` is a list of
+    ``(projections, x, ys)`` with 1..4 QMatMul of equal k, x a device f32 tensor of k values and one
+    device f32 output tensor per projection.  Step i reads x after step i - 1 has completed, as the
+    same calls issued one after the other on a stream would; results are those of `forward_group`
+    bit for bit.  The tensors must stay alive and in place while the chain exists."""
+
+    def __init__(self, steps):
+        n = len(steps)
+        arr = (capi.ChainStep * n)()
+        self._keep = []
+        for i, (projections, x, ys) in enumerate(steps):
+            assert 1 <= len(projections) <= 4 and len(ys) == len(projections)
+            assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous()
+            k = projections[0].qtensor.dims2()[1]
+            assert x.numel() == k, (x.shape, k)
+            arr[i].n_weights = len(projections)
+            arr[i].x = x.data_ptr()
+            for j, (p, y) in enumerate(zip(projections, ys)):
+                assert y.is_cuda and y.dtype == torch.float32 and y.is_contiguous() and y.numel() == p.qtensor.dims2()[0]
+                arr[i].weights[j] = p.qtensor._h
+                arr[i].ys[j] = y.data_ptr()
+            self._keep.append((projections, x, ys))
+        h = C.c_void_p()
+        check(lib().izwi_qmm_chain_create(arr, n, C.byref(h)))
+        self._h = h
+
+    def run(self) -> None:
+        check(lib().izwi_qmm_chain_run(self._h, torch.cuda.current_stream().cuda_stream))
+
+    def status(self) -> None:
+        """Waits for the current stream; raises if a wait inside a run gave up."""
+        check(lib().izwi_qmm_chain_status(self._h, torch.cuda.current_stream().cuda_stream))
+
+    def set_spin_limit(self, polls: int) -> None:
+        check(lib().izwi_qmm_chain_set_spin_limit(self._h, polls))
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            try:
+                lib().izwi_qmm_chain_destroy(h)
+            except Exception:
+                pass
+
+
 class Qwen3QkvProjection:
     """izwi-core's Qwen3QkvProjection with quantized weights: `new_separate` keeps q, k, v as
     three weights (the reference's default off Metal), `new_quantized_grouped` packs them."""
