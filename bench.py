@@ -261,29 +261,44 @@ def cpu_baseline(oracle, dtype, m, budget_s=12.0):
 
 
 def prefill_extra(torch, qa, dtype, m, steps=20, warmup=5, only=None):
-    """TFLOP/s of the prefill kernel per projection (extra report, not `value`):
-    bf16 activations in HBM, bf16 output, called through the C ABI on preallocated buffers."""
+    """TFLOP/s of the prefill kernel per projection and per projection group (extra report, not
+    `value`): bf16 activations in HBM, bf16 output, called through the C ABI on preallocated buffers.
+    `qkv` and `gate_up` are the calls Qwen3Attention::forward / Qwen3Mlp::forward make (q, k, v resp.
+    gate, up on the same activations) as one izwi_qmm_forward_group_bf16 call: one launch."""
+    import ctypes as C
     from izwi_amd import capi
     from izwi_amd.qmatmul import _stream_ptr
     L = capi.lib()
     out = {}
     gg = qa.GgmlDType(dtype)
-    for i, (name, n, k) in enumerate([LAYER_8B[0], LAYER_8B[1], LAYER_8B[4], LAYER_8B[6]]):
-        if only is not None and name != only:
+    shapes = {name: (i, n, k) for i, (name, n, k) in enumerate(LAYER_8B)}
+    cases = [("q", ("q",)), ("k", ("k",)), ("gate", ("gate",)), ("down", ("down",)),
+             ("qkv", ("q", "k", "v")), ("gate_up", ("gate", "up"))]
+    for label, names in cases:
+        if only is not None and label != only:
             continue
-        mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, make_blocks(dtype, n, k, 1000 + i, 4096), (n, k)))
+        k = shapes[names[0]][2]
+        mms = [qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(
+            gg, make_blocks(dtype, shapes[nm][1], k, 1000 + shapes[nm][0], 4096), (shapes[nm][1], k))) for nm in names]
         x = torch.from_numpy(synth_normal(3, (m, k))).cuda().to(torch.bfloat16)
-        y = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+        ys = [torch.empty((m, shapes[nm][1]), dtype=torch.bfloat16, device="cuda") for nm in names]
         sp = _stream_ptr()
+        n = len(names)
+        handles = (C.c_void_p * n)(*[mm.qtensor._h for mm in mms])
+        outs = (C.c_void_p * n)(*[y.data_ptr() for y in ys])
 
         def call():
-            rc = L.izwi_qmm_forward_bf16(mm.qtensor._h, x.data_ptr(), m, y.data_ptr(), capi.OUT_BF16, capi.DEVICE, sp)
+            if n == 1:
+                rc = L.izwi_qmm_forward_bf16(handles[0], x.data_ptr(), m, outs[0], capi.OUT_BF16, capi.DEVICE, sp)
+            else:
+                rc = L.izwi_qmm_forward_group_bf16(handles, n, x.data_ptr(), m, outs, capi.OUT_BF16, capi.DEVICE, sp)
             if rc:
                 capi.check(rc)
 
         ms = time_eager(torch, call, steps, warmup)
-        out[name] = round(2.0 * m * n * k / (ms * 1e-3) / 1e12, 2)
-        del mm, x, y
+        flops = sum(2.0 * m * shapes[nm][1] * k for nm in names)
+        out[label] = round(flops / (ms * 1e-3) / 1e12, 2)
+        del mms, x, ys
     return out
 
 
@@ -672,7 +687,7 @@ def main():
                          "per-projection: seven izwi_qmm_forward_f32 calls per layer")
     ap.add_argument("--neighbours-only", action="store_true",
                     help="time only the decode-step neighbours (norms, rotary, attention) and print them: for profiling")
-    ap.add_argument("--prefill-only", default=None, choices=["q", "k", "gate", "down"],
+    ap.add_argument("--prefill-only", default=None, choices=["q", "k", "gate", "down", "qkv", "gate_up"],
                     help="profiling aid: run only the prefill call of one 8B projection (--m rows, default "
                          "2048 here; --steps calls) and print its TFLOP/s, nothing else")
     args = ap.parse_args()

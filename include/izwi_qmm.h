@@ -270,14 +270,25 @@ int izwi_qmm_forward_f32_noalloc(const izwi_qmm_weight* w, const float* x, int64
 /* `Qwen3QkvProjection::forward` and `Qwen3GateUpProjection::forward`, `Separate` arms
  * (qwen3/core.rs:1119-1127, 1274-1282): several projections applied to the same
  * activations, y_i = QMatMul_i.forward(x), bit-identical to n_weights calls of
- * izwi_qmm_forward_f32.  The weights must share k; with equal block types the decode
+ * izwi_qmm_forward_f32 up to 128 rows (beyond, in the bf16 matrix-core arithmetic, equal up to the
+ * f32 summation order: the shared launch may split k differently).  The weights must share k; with equal block types the decode
  * sizes run as one kernel launch (m <= 2) or share one activation quantization
- * (m <= 64); members of several block types (attn_q / attn_k in Q4_K beside attn_v in
+ * (m <= 64), prefill sizes (m > 128, bf16 matrix-core arithmetic) share one conversion of x
+ * and one launch; members of several block types (attn_q / attn_k in Q4_K beside attn_v in
  * Q6_K, as Q4_K_M files have them) are grouped by type, one such launch per type.
  * n_weights <= 4. */
 int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_weights,
                                const float* x, int64_t m, float* const* ys, int mem_space,
                                void* stream);
+
+/* izwi_qmm_forward_group_f32 for bf16 activations (prefill): y_i = izwi_qmm_forward_bf16(weights[i], x)
+ * for 1..4 weights of equal k on the same x, `out_dtype` f32 or bf16 for every y_i.  With equal block
+ * types, device pointers and m > 128 the members run as ONE launch of the bf16 matrix-core kernel
+ * (its grid is the members' column tiles one after the other, planned as one matrix): k / v
+ * (n = 1024) no longer run alone on a quarter of the chip.  Results are those of the separate calls
+ * up to f32 summation order (the tile plan may split k differently). */
+int izwi_qmm_forward_group_bf16(const izwi_qmm_weight* const* weights, int32_t n_weights, const uint16_t* x_bf16,
+                                int64_t m, void* const* ys, int out_dtype, int mem_space, void* stream);
 
 /* The gate / up pair of `Qwen3Mlp::forward` (qwen3/core.rs:1786-1798) with its activation:
  *     h[m, n] = silu(gate.forward(x)) * up.forward(x)

@@ -893,6 +893,27 @@ int forward_group_impl(const izwi_qmm_weight* const* weights, int32_t n_weights,
         return IZWI_QMM_OK;
     }
     if (by_type) return call_by_type(x, nullptr);
+    // prefill sizes on the bf16 matrix cores: the activations are converted once and the members
+    // share one launch (its grid is the members' column tiles one after the other)
+    if (mem_space == IZWI_QMM_DEVICE && uniform && n_weights >= 2 && m > 128 && large_m_mode() == IZWI_QMM_LARGE_M_BF16) {
+        hipStream_t stream = (hipStream_t)stream_;
+        const izwi_qmm_weight* w0 = weights[0];
+        const QmmLayout* layouts[QMM_MAX_GROUP];
+        const void* tiled[QMM_MAX_GROUP];
+        void* outs[QMM_MAX_GROUP];
+        for (int i = 0; i < n_weights; i++) layouts[i] = &weights[i]->layout, tiled[i] = weights[i]->tiled, outs[i] = ys[i];
+        const size_t xb_bytes = (((size_t)m * w0->layout.k * sizeof(uint16_t)) + 255) & ~(size_t)255;
+        const size_t ws_bytes = qmm_gemm_group_workspace_bytes(layouts, n_weights, m, w0->n_cus);
+        void* xb = nullptr;
+        HIP_TRY(get_scratch(w0->device, stream, xb_bytes + ws_bytes, &xb));
+        ProfileScope prof(w0, stream);
+        HIP_TRY(qmm_launch_f32_to_bf16(x, (uint16_t*)xb, m * w0->layout.k, stream));
+        hipError_t e = qmm_launch_gemm_bf16_multi(layouts, tiled, n_weights, (const uint16_t*)xb, m, outs, 0,
+                                                  ws_bytes ? (uint8_t*)xb + xb_bytes : nullptr, w0->n_cus, stream);
+        if (e == hipSuccess) return IZWI_QMM_OK;
+        if (e != hipErrorNotSupported) return fail_hip(e, "grouped prefill kernel");
+        (void)hipGetLastError();
+    }
     // host buffers, mixed types, prefill sizes: one call per projection (same results)
     if (mem_space != IZWI_QMM_DEVICE || !uniform || n_weights == 1 || m > 64) {
         for (int i = 0; i < n_weights; i++)
@@ -1099,6 +1120,50 @@ int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int6
     HIP_TRY(qmm_launch_gemm_bf16(L, w->tiled, (const uint16_t*)xi.dev, m, yo.dev,
                                  out_dtype == IZWI_QMM_OUT_BF16, workspace, w->n_cus, stream));
     HIP_TRY(yo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_forward_group_bf16(const izwi_qmm_weight* const* weights, int32_t n_weights, const uint16_t* x_bf16,
+                                int64_t m, void* const* ys, int out_dtype, int mem_space, void* stream_) {
+    QmmCallScope call;
+    if (!weights || !ys) return fail(IZWI_QMM_ERR_INVALID, "NULL argument");
+    if (n_weights < 1 || n_weights > QMM_MAX_GROUP)
+        return fail(IZWI_QMM_ERR_INVALID, "projection group of %d weights (1..%d supported)", n_weights, QMM_MAX_GROUP);
+    if (int rc = check_space(mem_space)) return rc;
+    if (out_dtype != IZWI_QMM_OUT_F32 && out_dtype != IZWI_QMM_OUT_BF16)
+        return fail(IZWI_QMM_ERR_INVALID, "bad out_dtype %d", out_dtype);
+    bool uniform = true;
+    for (int i = 0; i < n_weights; i++) {
+        if (!weights[i]) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+        const QmmLayout& L = weights[i]->layout;
+        if (L.n_stacked != 1) return fail(IZWI_QMM_ERR_INVALID, "forward on an expert stack");
+        if (L.k != weights[0]->layout.k)
+            return fail(IZWI_QMM_ERR_INVALID, "projection group input mismatch: expected %lld, got %lld",
+                        (long long)weights[0]->layout.k, (long long)L.k);
+        if (L.dtype != weights[0]->layout.dtype || L.n == 0 || weights[i]->device != weights[0]->device) uniform = false;
+        if (m > 0 && L.n > 0 && !ys[i]) return fail(IZWI_QMM_ERR_INVALID, "y is NULL");
+    }
+    if (m < 0) return fail(IZWI_QMM_ERR_INVALID, "negative m");
+    if (m == 0) return IZWI_QMM_OK;
+    if (!x_bf16) return fail(IZWI_QMM_ERR_INVALID, "x is NULL");
+    if (mem_space == IZWI_QMM_DEVICE && uniform && n_weights >= 2 && m > 128) {
+        hipStream_t stream = (hipStream_t)stream_;
+        const izwi_qmm_weight* w0 = weights[0];
+        const QmmLayout* layouts[QMM_MAX_GROUP];
+        const void* tiled[QMM_MAX_GROUP];
+        for (int i = 0; i < n_weights; i++) layouts[i] = &weights[i]->layout, tiled[i] = weights[i]->tiled;
+        void* workspace = nullptr;
+        if (const size_t ws_bytes = qmm_gemm_group_workspace_bytes(layouts, n_weights, m, w0->n_cus))
+            HIP_TRY(get_scratch(w0->device, stream, ws_bytes, &workspace));
+        ProfileScope prof(w0, stream);
+        hipError_t e = qmm_launch_gemm_bf16_multi(layouts, tiled, n_weights, x_bf16, m, ys, out_dtype == IZWI_QMM_OUT_BF16,
+                                                  workspace, w0->n_cus, stream);
+        if (e == hipSuccess) return IZWI_QMM_OK;
+        if (e != hipErrorNotSupported) return fail_hip(e, "grouped prefill kernel");
+        (void)hipGetLastError();
+    }
+    for (int i = 0; i < n_weights; i++)
+        if (int rc = izwi_qmm_forward_bf16(weights[i], x_bf16, m, ys[i], out_dtype, mem_space, stream_)) return rc;
     return IZWI_QMM_OK;
 }
 

@@ -58,6 +58,15 @@ struct GemmParams {
     uint32_t nibble_mask;
     float* partial;
     const void* residual; // of y's type, added to the sums before they are stored (may alias y)
+    // several weights of equal k and type on the same activations in one launch (pipelined tiles
+    // only): column tile t of the grid belongs to weight i with tn_end[i - 1] <= t < tn_end[i];
+    // w / y / n / n_end / row_tiles / partial above are replaced by the member's at kernel entry
+    int n_weights; // 0 or 1: a single weight
+    int tn_end[QMM_MAX_GROUP];
+    const uint8_t* wv[QMM_MAX_GROUP];
+    void* yv[QMM_MAX_GROUP];
+    int64_t nv[QMM_MAX_GROUP], row_tiles_v[QMM_MAX_GROUP];
+    float* partial_v[QMM_MAX_GROUP];
 };
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
@@ -362,7 +371,19 @@ __device__ __forceinline__ void static_for(F&& f) {
 // computed once.  XTAIL: k is not a multiple of 64 (Q8_0 only), activation chunks at or
 // past k are zeroed on their way to LDS.
 template <int QT, int BM, int BN, bool XTAIL, int NW = 4>
-__global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
+__global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P_in) {
+    GemmParams P = P_in;
+    int tn_local = (int)(blockIdx.x / P_in.tiles_m);
+    if (P_in.n_weights > 1) { // a projection group: this workgroup's member (uniform)
+        int i = 0;
+        while (i + 1 < P_in.n_weights && tn_local >= P_in.tn_end[i]) i++;
+        tn_local -= i ? P_in.tn_end[i - 1] : 0;
+        P.w = P_in.wv[i];
+        P.y = P_in.yv[i];
+        P.n = P.n_end = P_in.nv[i];
+        P.row_tiles = P_in.row_tiles_v[i];
+        P.partial = P_in.partial ? P_in.partial_v[i] : nullptr;
+    }
     // NW waves as a (NW / 2) x 2 grid of wave tiles; with eight waves two share a SIMD, each with
     // half the accumulators, and one issues while the other waits
     constexpr int THREADS = 64 * NW, WM = NW / 2;
@@ -386,7 +407,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_pipe_kernel(GemmParams P) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const int tm = blockIdx.x % P.tiles_m;
-    const int tn = blockIdx.x / P.tiles_m;
+    const int tn = tn_local;
     const int64_t m0 = (int64_t)tm * BM, n0 = P.n_begin + (int64_t)tn * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -788,6 +809,11 @@ template <int QT, int BM, int BN, int NW = 4>
 hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
     P.tiles_m = (int)((P.m + BM - 1) / BM);
     P.tiles_n = (int)((P.n_end - P.n_begin + BN - 1) / BN);
+    if (P.n_weights > 1) { // a projection group: the members' column tiles one after the other
+        int64_t t = 0;
+        for (int i = 0; i < P.n_weights; i++) P.tn_end[i] = (int)(t += (P.nv[i] + BN - 1) / BN);
+        P.tiles_n = (int)t;
+    }
     const int64_t grid = (int64_t)P.tiles_m * P.tiles_n;
     if (grid > 0x7fffffff) return hipErrorInvalidValue;
     const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
@@ -810,7 +836,13 @@ hipError_t launch_tile(GemmParams P, int slices, hipStream_t stream) {
         const dim3 grid2((unsigned)grid, (unsigned)slices);
         if (x_tail) gemm_pipe_kernel<QT, BM, BN, QT == QMM_Q8_0, NW><<<grid2, dim3(64 * NW), lds, stream>>>(P);
         else gemm_pipe_kernel<QT, BM, BN, false, NW><<<grid2, dim3(64 * NW), lds, stream>>>(P);
-        if (slices > 1) {
+        if (slices > 1 && P.n_weights > 1) {
+            for (int i = 0; i < P.n_weights; i++) {
+                const int64_t count = P.m * P.nv[i];
+                splitk_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(
+                    P.partial_v[i], slices, P.m, P.nv[i], 0, P.nv[i], P.yv[i], P.out_bf16, nullptr);
+            }
+        } else if (slices > 1) {
             const int64_t count = P.m * (P.n_end - P.n_begin);
             splitk_reduce_kernel<<<(unsigned)((count + 255) / 256), 256, 0, stream>>>(
                 partial, slices, P.m, P.n, P.n_begin, P.n_end, P.y, P.out_bf16, P.residual);
@@ -849,7 +881,7 @@ bool forced_plan(GemmPlan& plan) {
     return true;
 }
 
-GemmPlan plan_gemm(int64_t m, int64_t n, int k_steps, int n_cus) {
+GemmPlan plan_gemm(int64_t m, int64_t n, int k_steps, int n_cus, bool group = false) {
     // relative rate of a half-size tile (256 x 128 dequantizes half as many weights per MFMA
     // as 128 x 256 and is used whenever there are more than 128 rows) and of a quarter-size one
     const double kQ128 = m > 128 ? 0.76 : 0.68, kQ64 = 0.4;
@@ -869,11 +901,12 @@ GemmPlan plan_gemm(int64_t m, int64_t n, int k_steps, int n_cus) {
         if (cost < 0.97 * best_cost) best = p, best_cost = cost;
     };
     consider({hm, hn, 1, 0}, rounds(tiles(hm, hn, n)) * k_steps * 0.5 / kQ128);
-    consider({128, 128, 1, 0}, rounds(tiles(128, 128, n)) * k_steps * 0.25 / kQ64);
+    // (a projection group runs on the pipelined tiles only, in one launch)
+    if (!group) consider({128, 128, 1, 0}, rounds(tiles(128, 128, n)) * k_steps * 0.25 / kQ64);
     // whole rounds of 256 x 256 tiles first, the remaining columns as half-size tiles
     const int64_t tiles_m256 = (m + 255) / 256, cols256 = (n + 255) / 256;
     const int64_t full_cols = (tiles_m256 * cols256 / n_cus) * n_cus / tiles_m256;
-    if (full_cols > 0 && full_cols < cols256)
+    if (!group && full_cols > 0 && full_cols < cols256)
         consider({hm, hn, 1, full_cols},
                  (double)(tiles_m256 * full_cols / n_cus) * k_steps +
                      rounds(tiles(hm, hn, n - full_cols * 256)) * k_steps * 0.5 / kQ128);
@@ -911,7 +944,85 @@ hipError_t launch_qt(const GemmParams& P0, int n_cus, hipStream_t stream) {
     return launch_tile<QT, 128, 128>(P, 1, stream);
 }
 
+// n of the single matrix a group is planned as: the members' columns, each rounded up to whole
+// 256-column strips
+int64_t group_columns(const QmmLayout* const* layouts, int n_weights) {
+    int64_t n = 0;
+    for (int i = 0; i < n_weights; i++) n += (layouts[i]->n + 255) / 256 * 256;
+    return n;
+}
+
+template <int QT>
+hipError_t launch_group_qt(GemmParams P, int64_t n_planned, int n_cus, hipStream_t stream) {
+    const GemmPlan plan = plan_gemm(P.m, n_planned, P.k_units * 4, n_cus, true);
+    if (plan.slices > 1) {
+        if (P.partial == nullptr) return hipErrorInvalidValue;
+        float* base = P.partial;
+        for (int i = 0; i < P.n_weights; i++) {
+            P.partial_v[i] = base;
+            base += (size_t)plan.slices * (size_t)P.m * (size_t)P.nv[i];
+        }
+    }
+    if (plan.bm == 256 && plan.bn == 256) return launch_tile<QT, 256, 256, 8>(P, plan.slices, stream);
+    if (plan.bm == 256 && plan.bn == 128) return launch_tile<QT, 256, 128, 8>(P, plan.slices, stream);
+    return hipErrorNotSupported;
+}
+
 } // namespace
+
+size_t qmm_gemm_group_workspace_bytes(const QmmLayout* const* layouts, int n_weights, int64_t m, int n_cus) {
+    if (m <= 128 || n_weights < 2) return 0;
+    const GemmPlan plan = plan_gemm(m, group_columns(layouts, n_weights), (int)layouts[0]->k_units * 4, n_cus > 0 ? n_cus : 1, true);
+    if (plan.slices <= 1) return 0;
+    size_t total = 0;
+    for (int i = 0; i < n_weights; i++) total += (size_t)plan.slices * (size_t)m * (size_t)layouts[i]->n * sizeof(float);
+    return total;
+}
+
+hipError_t qmm_launch_gemm_bf16_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
+                                      const uint16_t* x_bf16, int64_t m, void* const* ys, int out_bf16,
+                                      void* workspace, int n_cus, hipStream_t stream) {
+    if (n_weights < 2 || n_weights > QMM_MAX_GROUP) return hipErrorInvalidValue;
+    if (m <= 128) return hipErrorNotSupported; // the plain tile kernels: one call per weight
+    if (n_cus <= 0) n_cus = 1;
+    const QmmLayout& L0 = *layouts[0];
+    GemmParams P;
+    P.w = (const uint8_t*)tiled[0];
+    P.x = x_bf16;
+    P.y = ys[0];
+    P.m = m;
+    P.n = L0.n;
+    P.n_begin = 0;
+    P.n_end = L0.n;
+    P.k = L0.k;
+    P.k_units = (int)L0.k_units;
+    P.k_groups = (int)L0.k_groups;
+    P.s = L0.s;
+    P.slots = L0.slots;
+    P.row_tiles = L0.row_tiles;
+    P.panel_bytes = L0.panel_bytes;
+    P.out_bf16 = out_bf16;
+    P.tiles_m = P.tiles_n = 0;
+    P.slice_units = 0;
+    P.nibble_mask = 0x0f0f0f0fu;
+    P.partial = (float*)workspace;
+    P.residual = nullptr;
+    P.n_weights = n_weights;
+    for (int i = 0; i < n_weights; i++) {
+        const QmmLayout& L = *layouts[i];
+        if (L.dtype != L0.dtype || L.k != L0.k || L.n_stacked != 1 || L.n == 0) return hipErrorInvalidValue;
+        P.wv[i] = (const uint8_t*)tiled[i];
+        P.yv[i] = ys[i];
+        P.nv[i] = L.n;
+        P.row_tiles_v[i] = L.row_tiles;
+        P.partial_v[i] = nullptr;
+        P.tn_end[i] = 0;
+    }
+    const int64_t n_planned = group_columns(layouts, n_weights);
+    if (L0.dtype == QMM_Q6_K) return launch_group_qt<QMM_Q6_K>(P, n_planned, n_cus, stream);
+    return L0.dtype == QMM_Q4_K ? launch_group_qt<QMM_Q4_K>(P, n_planned, n_cus, stream)
+                                : launch_group_qt<QMM_Q8_0>(P, n_planned, n_cus, stream);
+}
 
 size_t qmm_gemm_workspace_bytes(const QmmLayout& L, int64_t m, int n_cus) {
     if (m <= 0 || L.n == 0 || (L.dtype == QMM_Q6_K && m <= 128)) return 0;
@@ -945,6 +1056,7 @@ hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uin
     P.nibble_mask = 0x0f0f0f0fu;
     P.partial = (float*)workspace;
     P.residual = residual;
+    P.n_weights = 0;
     if (L.dtype == QMM_Q6_K) {
         // more than 128 rows: the pipelined tiles; up to 128 the plain tile kernel, half-height
         // tiles when full ones would leave CUs idle

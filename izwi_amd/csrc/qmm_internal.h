@@ -177,6 +177,15 @@ size_t qmm_gemm_workspace_bytes(const QmmLayout& L, int64_t m, int n_cus);
 hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uint16_t* x_bf16,
                                 int64_t m, void* y, int out_bf16, void* workspace, int n_cus,
                                 hipStream_t stream, const void* residual = nullptr);
+// Several weights of equal k and type on the same bf16 activations in ONE launch of the pipelined
+// tiles (m > 128): the grid is the members' column tiles one after the other, planned as one
+// matrix with all the columns.  Per-member results are those of qmm_launch_gemm_bf16 up to the
+// tile plan (which may split k differently).  hipErrorNotSupported: no single-launch form
+// (m <= 128), call the members one by one.
+size_t qmm_gemm_group_workspace_bytes(const QmmLayout* const* layouts, int n_weights, int64_t m, int n_cus);
+hipError_t qmm_launch_gemm_bf16_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
+                                      const uint16_t* x_bf16, int64_t m, void* const* ys, int out_bf16,
+                                      void* workspace, int n_cus, hipStream_t stream);
 // y[i] = t[i] (+ residual[i]) as f32 or bf16: the epilogue as a kernel of its own, for the forms
 // that cannot fold it
 hipError_t qmm_launch_epilogue(const float* t, const void* residual, void* y, int y_bf16, int64_t count,

@@ -300,12 +300,18 @@ def forward_group(projections: Sequence["QMatMul"], x: torch.Tensor, norm_weight
     1274-1282).  Returns one output per projection, identical to separate forwards.
     With ``norm_weight`` the projections see rms_norm(x, norm_weight, eps) (the layer norm in front of
     them, core.rs:1872), folded into the same launch for one or two rows."""
-    assert x.dtype == torch.float32 and x.is_contiguous()
+    assert x.dtype in (torch.float32, torch.bfloat16) and x.is_contiguous()
     k = x.shape[-1]
     m = x.numel() // k if k else 0
     n = len(projections)
-    ys = [torch.empty(tuple(x.shape[:-1]) + (p.qtensor.dims2()[0],), dtype=torch.float32, device=x.device)
+    ys = [torch.empty(tuple(x.shape[:-1]) + (p.qtensor.dims2()[0],), dtype=x.dtype, device=x.device)
           for p in projections]
+    if x.dtype == torch.bfloat16:       # prefill: bf16 in, bf16 out (izwi_qmm_forward_group_bf16)
+        assert norm_weight is None
+        handles = (C.c_void_p * n)(*[p.qtensor._h for p in projections])
+        outs = (C.c_void_p * n)(*[y.data_ptr() for y in ys])
+        check(lib().izwi_qmm_forward_group_bf16(handles, n, x.data_ptr(), m, outs, capi.OUT_BF16, _space(x), _stream_ptr(x)))
+        return tuple(ys)
     handles = (C.c_void_p * n)(*[p.qtensor._h for p in projections])
     outs = (C.c_void_p * n)(*[y.data_ptr() for y in ys])
     if norm_weight is not None:

@@ -557,6 +557,42 @@ def test_projection_group_equals_separate_calls(qa, oracle, dtype, m):
     assert rel_err(v.cpu().numpy(), want) < tol
 
 
+@pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
+@pytest.mark.parametrize("m,k,ns", [(512, 4096, (4096, 1024, 1024)), (2048, 4096, (4096, 1024, 1024)),
+                                    (300, 768, (300, 200)), (200, 1024, (2048, 1000, 16, 512)), (129, 256, (256, 256))])
+def test_projection_group_at_prefill_sizes(qa, oracle, dtype, m, k, ns):
+    """Beyond 128 rows a projection group is ONE launch of the bf16 matrix-core kernel (the members'
+    column tiles side by side): every member equals its separate call up to the f32 summation order
+    (the plan may split k differently), for f32 activations (converted once) and bf16 activations."""
+    _say(f"group prefill dtype={dtype} m={m} k={k} ns={ns}")
+    dt = qa.GgmlDType(dtype)
+    blocks = [make_weight(oracle, dtype, n, k, 420 + n + i) for i, n in enumerate(ns)]
+    parts = [qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, b, (n, k))) for b, n in zip(blocks, ns)]
+    x = torch.from_numpy(oracle.randn(421 + m, (m, k))).cuda()
+    xb = x.to(torch.bfloat16)
+    got_f32 = qa.forward_group(parts, x)
+    got_bf16 = qa.forward_group(parts, xb)
+    for i, p in enumerate(parts):
+        sep = p.forward(x)
+        scale = float(sep.abs().max())
+        assert float((got_f32[i] - sep).abs().max()) <= 2e-5 * scale, i
+        sep_b = p.forward_bf16_to_f32(xb)
+        assert got_bf16[i].dtype == torch.bfloat16 and got_bf16[i].shape == (m, ns[i])
+        assert float((got_bf16[i].float() - sep_b).abs().max()) <= 2.0 ** -7 * float(sep_b.abs().max()), i
+    # the reference's CPU arithmetic on the narrowest member with at least 128 outputs, on the same
+    # (bf16-representable) activations
+    i = min((j for j, n in enumerate(ns) if n >= 128), key=lambda j: ns[j])
+    want = oracle.qmatmul(dtype, xb.float().cpu().numpy(), blocks[i], ns[i])
+    assert rel_err(got_bf16[i].float().cpu().numpy(), want) < PREFILL_TOL
+    # gate / up with its activation runs on the same group launch
+    if len(ns) >= 2 and ns[0] == ns[1] or len(ns) >= 3 and ns[1] == ns[2]:
+        a, b = (parts[1], parts[2]) if len(ns) >= 3 and ns[1] == ns[2] else (parts[0], parts[1])
+        h = qa.Qwen3GateUpProjection.new_separate(a, b).forward_silu_mul(x)
+        ga, ub = a.forward(x), b.forward(x)
+        ref = torch.nn.functional.silu(ga) * ub
+        assert float((h - ref).abs().max()) <= 1e-4 * float(ref.abs().max())
+
+
 def test_projection_group_8b_gate_up_and_errors(qa, oracle):
     dt = qa.GgmlDType.Q4K
     gate = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, make_weight(oracle, Q4_K, 12288, 4096, 410), (12288, 4096)))
