@@ -359,6 +359,79 @@ def chained_extra(torch, qa, calls, total_bytes, steps=20, warmup=3):
             "note": "one resident kernel for the 144 dependent projection steps + the LM head call; not `value`"}
 
 
+def records_path_extra(torch, qa, dtype, weights, m, steps=10, warmup=3):
+    """Extra report (not `value`): the headline stack at m rows where the projections whose activations
+    come out of an RMSNorm (q|k|v, gate|up, LM head) or out of silu(gate) * up (down) are handed
+    activation records by that producer (izwi_rms_norm_quantize_records_f32 /
+    izwi_qmm_silu_mul_quantize_records_f32) instead of launching a quantizer of their own; o (fed by
+    the attention) keeps its quantizer launch.  The producers are not projections and are timed beside
+    the stack: one launch each, in place of the norm / elementwise launch the layer has anyway."""
+    import ctypes as C
+    from izwi_amd import capi
+    L = capi.lib()
+    gd = qa.GgmlDType(dtype)
+    xs = {k: torch.from_numpy(synth_normal(7 + k, (m, k))).cuda() for k in (4096, 12288)}
+    recs = {k: qa.ActivationRecords.quantize(gd, xs[k]) for k in (4096, 12288)}
+    out = lambda n: torch.empty((m, n), dtype=torch.float32, device="cuda")  # noqa: E731
+    per_layer = len(LAYER_8B)
+    n_layers = (len(weights) - 1) // per_layer
+    plan, total = [], 0.0
+    for layer in range(n_layers):
+        w = weights[layer * per_layer:(layer + 1) * per_layer]  # q k v o gate up down
+        plan.append(("rec", [w[0][0], w[1][0], w[2][0]], recs[4096], [out(w[0][1]), out(w[1][1]), out(w[2][1])]))
+        plan.append(("x", w[3][0], xs[4096], out(w[3][1])))
+        plan.append(("rec", [w[4][0], w[5][0]], recs[4096], [out(w[4][1]), out(w[5][1])]))
+        plan.append(("rec", [w[6][0]], recs[12288], [out(w[6][1])]))
+        total += sum(gemv_bytes(dtype, n, k, m) for _, n, k in w)
+    mm, n, k = weights[-1]
+    plan.append(("rec", [mm], recs[k], [out(n)]))
+    total += gemv_bytes(dtype, n, k, m)
+    prepared = []
+    for kind, mms, src, ys in plan:
+        if kind == "rec":
+            nn = len(mms)
+            prepared.append((kind, (C.c_void_p * nn)(*[p.qtensor._h for p in mms]), nn, src.data.data_ptr(),
+                             (C.c_void_p * nn)(*[y.data_ptr() for y in ys])))
+        else:
+            prepared.append((kind, mms.qtensor._h, 1, src.data_ptr(), ys.data_ptr()))
+
+    def run():
+        sp = torch.cuda.current_stream().cuda_stream   # (the capturing stream)
+        for kind, h, nn, src, ys in prepared:
+            if kind == "rec":
+                rc = L.izwi_qmm_forward_group_records_f32(h, nn, src, m, ys, sp)
+            else:
+                rc = L.izwi_qmm_forward_f32(h, src, m, ys, capi.DEVICE, sp)
+            if rc:
+                capi.check(rc)
+    ms, g = time_graph(torch, run, steps, warmup)
+    del g
+    # the producers, per call, against the launches they replace
+    nw = torch.ones(4096, device="cuda")
+    gate = torch.from_numpy(synth_normal(5, (m, 12288))).cuda()
+    up = torch.from_numpy(synth_normal(6, (m, 12288))).cuda()
+    ynorm = torch.empty_like(xs[4096])
+    prod = {}
+    for name, fn in (("rms_norm_to_records_4096", lambda sp: L.izwi_rms_norm_quantize_records_f32(
+                         int(dtype), xs[4096].data_ptr(), nw.data_ptr(), m, 4096, 1e-6, recs[4096].data.data_ptr(), sp)),
+                     ("rms_norm_alone_4096", lambda sp: L.izwi_rms_norm_f32(xs[4096].data_ptr(), nw.data_ptr(), m, 4096, 1e-6,
+                                                                         ynorm.data_ptr(), capi.DEVICE, sp)),
+                     ("quantizer_alone_4096", lambda sp: L.izwi_qmm_quantize_records_f32(
+                         int(dtype), xs[4096].data_ptr(), m, 4096, recs[4096].data.data_ptr(), sp)),
+                     ("silu_mul_to_records_12288", lambda sp: L.izwi_qmm_silu_mul_quantize_records_f32(
+                         int(dtype), gate.data_ptr(), up.data_ptr(), m, 12288, recs[12288].data.data_ptr(), sp))):
+        def many(fn=fn):
+            sp = torch.cuda.current_stream().cuda_stream
+            for _ in range(32):
+                fn(sp)
+        t, g = time_graph(torch, many, steps, warmup)
+        prod[name + "_us"] = round(t * 1e3 / 32, 2)
+        del g
+    return {"gbs": round(total / (ms * 1e-3) / 1e9, 1), "ms_per_step": round(ms, 4), "m": m, "launches_per_step": 145 + n_layers,
+            "producers": prod,
+            "note": "q|k|v, gate|up, down, LM head read records written by their producers; o quantizes itself; not `value`"}
+
+
 def host_pointer_extra(qa, weights, m, passes=2):
     """Extra report (not `value`): the same projections called one by one with HOST pointers, the literal
     form of the reference's CPU call (activations in host memory in, results in host memory out): every
@@ -785,6 +858,9 @@ def main():
                 extras[f"decode_gbs_m{m}"] = round(tb / (t * 1e-3) / 1e9, 1)
                 extras[f"decode_ms_per_step_m{m}"] = round(t, 4)
                 del c, g
+            if args.calls == "grouped":
+                for m in (8, 16):
+                    extras[f"decode_records_path_m{m}"] = records_path_extra(torch, qa, dtype, weights, m)
             # the other call structure at the headline's m
             other = decode_calls if args.calls == "grouped" else grouped_decode_calls
             c, tb = other(torch, dtype, weights, args.m)

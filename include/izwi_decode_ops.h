@@ -58,6 +58,14 @@ int izwi_rope_pair_bshd_f32(const float* q, const float* k, const float* cos_sin
  * (metal.rs:2956).  Shapes, limits and error behaviour are those of the f32 entry points. */
 int izwi_rms_norm_f16(const uint16_t* x, const uint16_t* weight, int64_t rows, int64_t hidden, float eps,
                       uint16_t* y, int mem_space, void* stream);
+
+/* izwi_rms_norm_f32 whose result goes, quantized, straight into the activation records of the batched
+ * decode kernels (izwi_qmm.h, "activation records"): the layer norm in front of q|k|v and gate|up
+ * (qwen3/core.rs:1866, 1877) and the quantization inside the following `QMatMul::forward` as one
+ * launch.  The records equal izwi_qmm_quantize_records_f32(izwi_rms_norm_f32(x)) bit for bit.  f32,
+ * device pointers, hidden a multiple of 256 up to 16384, 16-byte aligned buffers. */
+int izwi_rms_norm_quantize_records_f32(int ggml_weight_dtype, const float* x, const float* weight, int64_t rows,
+                                       int64_t hidden, float eps, void* records, void* stream);
 int izwi_qk_rms_norm_f16(const uint16_t* q, const uint16_t* k, const uint16_t* qk_weight, int64_t q_rows,
                          int64_t k_rows, int64_t head_dim, float eps, uint16_t* q_out, uint16_t* k_out,
                          int mem_space, void* stream);

@@ -207,6 +207,29 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
 int izwi_qmm_forward_rows_f32(const izwi_qmm_weight* w, const uint32_t* row_ids, int64_t n_rows, const float* x,
                               int64_t m, float* y, int mem_space, void* stream);
 
+/* --- activation records: quantized activations handed over by their producer ---------- */
+
+/* For 3 <= m <= 64 rows izwi_qmm_forward_f32 is two launches: the activation quantizer (candle-core's
+ * `BlockQ8_0::from_float` / `BlockQ8K::from_float` per row, qwen3 call site core.rs:812) writes
+ * "records" into scratch, the matrix-core kernel multiplies them.  The kernel that PRODUCES the
+ * activations can write the records itself and save that launch on the token's critical path:
+ *   izwi_rms_norm_quantize_records_f32 (izwi_decode_ops.h)   input / post-attention RMSNorm -> q|k|v, gate|up
+ *   izwi_qmm_silu_mul_quantize_records_f32                    silu(gate) * up              -> down
+ *   izwi_qmm_quantize_records_f32                             any other f32 activations    (the plain quantizer)
+ * and izwi_qmm_forward_group_records_f32 is izwi_qmm_forward_group_f32 on such records: results
+ * are bit-identical to the calls on the f32 activations.  Records are opaque device memory of
+ * izwi_qmm_records_bytes(weight dtype, m, k) bytes, 16-byte aligned, valid for weights whose dot
+ * type matches (Q8_0 weights: Q8_0 records; Q4_K and Q6_K weights: the same Q8_K records).
+ * Device pointers only.  No counterpart in the reference, whose CPU matmul quantizes inside the op. */
+uint64_t izwi_qmm_records_bytes(int ggml_weight_dtype, int64_t m, int64_t k);
+int izwi_qmm_quantize_records_f32(int ggml_weight_dtype, const float* x, int64_t m, int64_t k, void* records,
+                                  void* stream);
+/* records of silu(gate[i]) * up[i] (`Qwen3Mlp::forward`, qwen3/core.rs:1786-1796), gate and up [m, k] */
+int izwi_qmm_silu_mul_quantize_records_f32(int ggml_weight_dtype, const float* gate, const float* up, int64_t m,
+                                           int64_t k, void* records, void* stream);
+int izwi_qmm_forward_group_records_f32(const izwi_qmm_weight* const* weights, int32_t n_weights, const void* records,
+                                       int64_t m, float* const* ys, void* stream);
+
 /* --- chained decode: the projections of one token as one launch ----------- */
 
 /* One token's projections in the order `Qwen3Layer::forward` issues them (qwen3/core.rs:1863-1881:

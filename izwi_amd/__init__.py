@@ -19,6 +19,7 @@ from .decode_ops import (  # noqa: F401
 )
 from .gguf import GgufLoader, GgufMmapMode, GgufModelInfo, GgufReaderKind, is_gguf_file, resolve_gguf_mmap_mode  # noqa: F401
 from .qmatmul import (  # noqa: F401
+    ActivationRecords,
     DecodeChain,
     GgmlDType,
     MoeExperts,

@@ -64,6 +64,11 @@ PROTOTYPES = {
     "izwi_qmm_weight_data": (C.c_int, [_vp, _vp, _u64, C.c_int, _vp]),
     "izwi_qmm_dequantize_f32": (C.c_int, [_vp, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_f32": (C.c_int, [_vp, _vp, _i64, _vp, C.c_int, _vp]),
+    "izwi_qmm_records_bytes": (_u64, [C.c_int, _i64, _i64]),
+    "izwi_qmm_quantize_records_f32": (C.c_int, [C.c_int, _vp, _i64, _i64, _vp, _vp]),
+    "izwi_qmm_silu_mul_quantize_records_f32": (C.c_int, [C.c_int, _vp, _vp, _i64, _i64, _vp, _vp]),
+    "izwi_qmm_forward_group_records_f32": (C.c_int, [_vp, _i32, _vp, _i64, _vp, _vp]),
+    "izwi_rms_norm_quantize_records_f32": (C.c_int, [C.c_int, _vp, _vp, _i64, _i64, C.c_float, _vp, _vp]),
     "izwi_qmm_chain_create": (C.c_int, [_vp, _i32, _pp]),
     "izwi_qmm_chain_destroy": (None, [_vp]),
     "izwi_qmm_chain_run": (C.c_int, [_vp, _vp]),

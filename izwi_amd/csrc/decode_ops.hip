@@ -21,6 +21,7 @@
 
 #include "../../include/izwi_decode_ops.h"
 #include "qmm_internal.h"
+#include "qmm_records.h"
 
 namespace {
 
@@ -131,13 +132,27 @@ struct NormParams {
     int64_t rows_a, rows_b;
     int hidden;
     float eps;
+    // REC variants: instead of out_a the normalized rows go, quantized, into the activation records
+    // of the batched decode kernels (row r of tile r / 16); rows rows_a .. rec_rows - 1 are zero rows
+    uint8_t* records;
+    int64_t rec_rows;
 };
 
-template <bool VEC, typename T>
+template <bool VEC, typename T, int REC = 0>
 __global__ void rms_norm_kernel(NormParams<T> P) {
     constexpr int PER = 4, EC = kEC<T>; // 16-byte pieces (VEC) or single values kept per thread
     __shared__ float partial[16];
+    extern __shared__ __attribute__((aligned(16))) float normed_row[]; // REC: the normalized row, [hidden]
     const int64_t row = blockIdx.x;
+    if constexpr (REC != 0) {
+        if (row >= P.rows_a) { // a padding row of the last 16-row tile: zeros
+            const float zero[16] = {};
+            for (int t = threadIdx.x; t < P.hidden / 16; t += blockDim.x)
+                quantize_into_record<REC>(zero, t & 15, (int)(row & 15),
+                                          P.records + ((row >> 4) * (P.hidden / 256) + (t >> 4)) * Unit<REC>::kBytes);
+            return;
+        }
+    }
     const bool first = row < P.rows_a;
     const T* x = first ? P.a + row * P.hidden : P.b + (row - P.rows_a) * P.hidden;
     const T* w = first ? P.weight_a : P.weight_b;
@@ -185,7 +200,12 @@ __global__ void rms_norm_kernel(NormParams<T> P) {
             ld16<T>(w + (int64_t)idx * EC, ww);
 #pragma unroll
             for (int c = 0; c < EC; c++) o[c] = v[c] * scale * ww[c];
-            st16<T>(y + (int64_t)idx * EC, o);
+            if constexpr (REC != 0) {
+#pragma unroll
+                for (int c = 0; c < EC; c++) normed_row[idx * EC + c] = o[c];
+            } else {
+                st16<T>(y + (int64_t)idx * EC, o);
+            }
         };
 #pragma unroll
         for (int i = 0; i < PER; i++) {
@@ -205,6 +225,20 @@ __global__ void rms_norm_kernel(NormParams<T> P) {
         }
         for (int idx = tid + PER * nt; idx < P.hidden; idx += nt) st1(y + idx, ld1(x + idx) * scale * ld1(w + idx));
     }
+    if constexpr (REC != 0) {
+        // the row as the record quantizer wants it: 16 consecutive values per lane, 16 lanes per unit
+        __syncthreads();
+        for (int t = tid; t < P.hidden / 16; t += nt) {
+            float v[16];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float4 f = *reinterpret_cast<const float4*>(normed_row + 16 * t + 4 * i);
+                v[4 * i] = f.x, v[4 * i + 1] = f.y, v[4 * i + 2] = f.z, v[4 * i + 3] = f.w;
+            }
+            quantize_into_record<REC>(v, t & 15, (int)(row & 15),
+                                      P.records + ((row >> 4) * (P.hidden / 256) + (t >> 4)) * Unit<REC>::kBytes);
+        }
+    }
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -222,6 +256,33 @@ hipError_t launch_norm(const NormParams<T>& P, hipStream_t stream) {
     while (threads < 1024 && threads < items) threads *= 2;
     if (vec) rms_norm_kernel<true, T><<<(unsigned)rows, threads, 0, stream>>>(P);
     else rms_norm_kernel<false, T><<<(unsigned)rows, threads, 0, stream>>>(P);
+    return hipGetLastError();
+}
+
+// RMSNorm straight into activation records (f32 rows, hidden a multiple of 256, 16-byte aligned):
+// the sums and products are those of rms_norm_kernel<true, float> with the same thread count, so
+// the records equal those of the norm followed by the record quantizer bit for bit.
+hipError_t launch_norm_records(NormParams<float> P, int weight_dtype, hipStream_t stream) {
+    if (P.rec_rows > 0x7fffffff) return hipErrorInvalidValue;
+    int threads = 64;
+    while (threads < 1024 && threads < P.hidden / 4) threads *= 2;
+    const size_t lds = (size_t)P.hidden * sizeof(float);
+    if (lds > 64 * 1024) return hipErrorNotSupported;
+    if (weight_dtype == IZWI_QMM_Q8_0) {
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&rms_norm_kernel<true, float, QMM_Q8_0>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+            if (e != hipSuccess) return e;
+        }
+        rms_norm_kernel<true, float, QMM_Q8_0><<<(unsigned)P.rec_rows, threads, lds, stream>>>(P);
+    } else { // Q4_K and Q6_K weights both dot against Q8_K activations: one record format
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&rms_norm_kernel<true, float, QMM_Q4_K>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+            if (e != hipSuccess) return e;
+        }
+        rms_norm_kernel<true, float, QMM_Q4_K><<<(unsigned)P.rec_rows, threads, lds, stream>>>(P);
+    }
     return hipGetLastError();
 }
 
@@ -711,7 +772,7 @@ int rms_norm_impl(const T* x, const T* weight, int64_t rows, int64_t hidden, flo
     OPS_TRY(wi.in(weight, (size_t)hidden * sizeof(T), mem_space));
     OPS_TRY(yo.out(y, (size_t)rows * hidden * sizeof(T), mem_space));
     NormParams<T> P{(const T*)xi.dev, nullptr, (const T*)wi.dev, nullptr, (T*)yo.dev, nullptr, rows, 0,
-                 (int)hidden, eps};
+                 (int)hidden, eps, nullptr, 0};
     OPS_TRY(launch_norm(P, stream));
     OPS_TRY(yo.finish(stream));
     return IZWI_QMM_OK;
@@ -740,10 +801,10 @@ int qk_rms_norm_impl(const T* q, const T* k, const T* qk_weight, int64_t q_rows,
     NormParams<T> P;
     if (q_rows)
         P = NormParams<T>{(const T*)qi.dev, (const T*)ki.dev, (const T*)wi.dev, (const T*)wi.dev + head_dim,
-                       (T*)qo.dev, (T*)ko.dev, q_rows, k_rows, (int)head_dim, eps};
+                       (T*)qo.dev, (T*)ko.dev, q_rows, k_rows, (int)head_dim, eps, nullptr, 0};
     else
         P = NormParams<T>{(const T*)ki.dev, nullptr, (const T*)wi.dev + head_dim, nullptr, (T*)ko.dev, nullptr,
-                       k_rows, 0, (int)head_dim, eps};
+                       k_rows, 0, (int)head_dim, eps, nullptr, 0};
     if (P.rows_b == 0) P.b = nullptr, P.weight_b = nullptr, P.out_b = nullptr;
     OPS_TRY(launch_norm(P, stream));
     OPS_TRY(qo.finish(stream));
@@ -878,6 +939,25 @@ extern "C" {
 int izwi_rms_norm_f32(const float* x, const float* weight, int64_t rows, int64_t hidden, float eps, float* y,
                       int mem_space, void* stream) {
     return rms_norm_impl<float>(x, weight, rows, hidden, eps, y, mem_space, stream);
+}
+int izwi_rms_norm_quantize_records_f32(int ggml_weight_dtype, const float* x, const float* weight, int64_t rows,
+                                       int64_t hidden, float eps, void* records, void* stream) {
+    if (ggml_weight_dtype != IZWI_QMM_Q8_0 && ggml_weight_dtype != IZWI_QMM_Q4_K && ggml_weight_dtype != IZWI_QMM_Q6_K)
+        return qmm_fail(IZWI_QMM_ERR_UNSUPPORTED, "ggml dtype %d is not supported", ggml_weight_dtype);
+    if (rows < 0 || hidden <= 0) return qmm_fail(IZWI_QMM_ERR_INVALID, "rms_norm: bad shape [%lld, %lld]", (long long)rows, (long long)hidden);
+    if (hidden % 256 || hidden > 16384)
+        return qmm_fail(IZWI_QMM_ERR_UNSUPPORTED, "rms_norm into records: hidden = %lld is not a multiple of 256 up to 16384",
+                        (long long)hidden);
+    if (rows == 0) return IZWI_QMM_OK;
+    if (!x || !weight || !records) return qmm_fail(IZWI_QMM_ERR_INVALID, "rms_norm: NULL buffer");
+    if (!aligned16(x) || !aligned16(weight) || !aligned16(records))
+        return qmm_fail(IZWI_QMM_ERR_INVALID, "rms_norm into records: buffers must be 16-byte aligned");
+    int device = 0, n_cus = 0;
+    if (int rc = qmm_current_device(&device, &n_cus)) return rc;
+    NormParams<float> P{x, nullptr, weight, nullptr, nullptr, nullptr, rows, 0, (int)hidden, eps,
+                        static_cast<uint8_t*>(records), (rows + 15) / 16 * 16};
+    OPS_TRY(launch_norm_records(P, ggml_weight_dtype, (hipStream_t)stream));
+    return IZWI_QMM_OK;
 }
 int izwi_rms_norm_f16(const uint16_t* x, const uint16_t* weight, int64_t rows, int64_t hidden, float eps, uint16_t* y,
                       int mem_space, void* stream) {

@@ -454,6 +454,11 @@ QmmCallScope::~QmmCallScope() {
     t_leased.clear();
 }
 
+namespace {
+int batched_group_on_records(const izwi_qmm_weight* const* weights, int32_t n_weights, const float* x, int64_t m,
+                             float* const* ys, void* records, hipStream_t stream);
+} // namespace
+
 // ---- the entry point that allocates nothing ---------------------------------
 // Scratch of izwi_qmm_forward_f32_noalloc: the quantized activation records of the batched decode
 // kernels (up to 64 rows), held in the library's image on every GPU it runs on instead of being
@@ -680,6 +685,77 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
         if (e != hipSuccess) return fail_hip(e, "prefill kernel");
     }
     HIP_TRY(yo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
+uint64_t izwi_qmm_records_bytes(int ggml_weight_dtype, int64_t m, int64_t k) {
+    if (!type_supported(ggml_weight_dtype) || m < 0 || k < 0) return 0;
+    return (uint64_t)qmm_records_bytes(ggml_weight_dtype, m, k);
+}
+
+namespace {
+int records_args(int dtype, int64_t m, int64_t k, const void* a, const void* b) {
+    if (!type_supported(dtype)) return fail(IZWI_QMM_ERR_UNSUPPORTED, "ggml dtype %d is not supported", dtype);
+    const int bs = dtype == IZWI_QMM_Q8_0 ? 32 : 256;
+    if (m < 0 || k <= 0 || k % bs) return fail(IZWI_QMM_ERR_INVALID, "bad shape [%lld, %lld] for block size %d", (long long)m, (long long)k, bs);
+    if (m > 0 && (!a || !b)) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    int device = 0;
+    if (int rc = current_device(&device)) return rc;
+    return ensure_device(device, nullptr);
+}
+} // namespace
+
+int izwi_qmm_quantize_records_f32(int ggml_weight_dtype, const float* x, int64_t m, int64_t k, void* records, void* stream) {
+    if (int rc = records_args(ggml_weight_dtype, m, k, x, records)) return rc;
+    if (m == 0) return IZWI_QMM_OK;
+    HIP_TRY(qmm_launch_quantize_ws(ggml_weight_dtype, x, m, k, records, (hipStream_t)stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_silu_mul_quantize_records_f32(int ggml_weight_dtype, const float* gate, const float* up, int64_t m, int64_t k,
+                                           void* records, void* stream) {
+    if (int rc = records_args(ggml_weight_dtype, m, k, gate, records)) return rc;
+    if (m == 0) return IZWI_QMM_OK;
+    if (!up) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    if (profiling()) g_silu_fused.fetch_add(1, std::memory_order_relaxed);
+    HIP_TRY(qmm_launch_quantize_silu_mul_ws(ggml_weight_dtype, gate, up, m, k, records, (hipStream_t)stream));
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_forward_group_records_f32(const izwi_qmm_weight* const* weights, int32_t n_weights, const void* records,
+                                       int64_t m, float* const* ys, void* stream_) {
+    if (!weights || !ys) return fail(IZWI_QMM_ERR_INVALID, "NULL argument");
+    if (n_weights < 1 || n_weights > QMM_MAX_GROUP)
+        return fail(IZWI_QMM_ERR_INVALID, "projection group of %d weights (1..%d supported)", n_weights, QMM_MAX_GROUP);
+    if (m < 3 || m > 64)
+        return fail(IZWI_QMM_ERR_UNSUPPORTED, "records are the input of the batched decode kernels (3 <= m <= 64), got m = %lld",
+                    (long long)m);
+    if (!records) return fail(IZWI_QMM_ERR_INVALID, "records is NULL");
+    const bool q8k = weights[0] && weights[0]->layout.dtype != IZWI_QMM_Q8_0;
+    for (int i = 0; i < n_weights; i++) {
+        if (!weights[i] || !ys[i]) return fail(IZWI_QMM_ERR_INVALID, "NULL weight or output");
+        const QmmLayout& L = weights[i]->layout;
+        if (L.n_stacked != 1 || L.n == 0) return fail(IZWI_QMM_ERR_INVALID, "forward on an expert stack or an empty weight");
+        if (L.k != weights[0]->layout.k)
+            return fail(IZWI_QMM_ERR_INVALID, "projection group input mismatch: expected %lld, got %lld",
+                        (long long)weights[0]->layout.k, (long long)L.k);
+        if ((L.dtype != IZWI_QMM_Q8_0) != q8k)
+            return fail(IZWI_QMM_ERR_INVALID, "the group mixes weights that dot against Q8_0 and against Q8_K records");
+        if (weights[i]->device != weights[0]->device) return fail(IZWI_QMM_ERR_INVALID, "weights on different devices");
+    }
+    hipStream_t stream = (hipStream_t)stream_;
+    // one launch per block type (Q4_K and Q6_K members read the same Q8_K records)
+    bool done[QMM_MAX_GROUP] = {};
+    for (int i = 0; i < n_weights; i++) {
+        if (done[i]) continue;
+        const izwi_qmm_weight* sub_w[QMM_MAX_GROUP];
+        float* sub_y[QMM_MAX_GROUP];
+        int n_sub = 0;
+        for (int j = i; j < n_weights; j++)
+            if (!done[j] && weights[j]->layout.dtype == weights[i]->layout.dtype)
+                sub_w[n_sub] = weights[j], sub_y[n_sub] = ys[j], n_sub++, done[j] = true;
+        if (int rc = batched_group_on_records(sub_w, n_sub, nullptr, m, sub_y, const_cast<void*>(records), stream)) return rc;
+    }
     return IZWI_QMM_OK;
 }
 

@@ -208,6 +208,10 @@ hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* co
 // quantized (qmm_launch_quantize_ws), all weights read the same records in one launch.
 hipError_t qmm_launch_quantize_ws(int dtype, const float* x, int64_t m, int64_t k, void* workspace,
                                   hipStream_t stream, bool x_bf16 = false);
+// silu(gate) * up quantized straight into the records; bytes of the records of m rows of k values
+hipError_t qmm_launch_quantize_silu_mul_ws(int dtype, const float* gate, const float* up, int64_t m, int64_t k,
+                                           void* workspace, hipStream_t stream);
+size_t qmm_records_bytes(int dtype, int64_t m, int64_t k);
 hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
                                       int64_t m, float* const* ys, const void* workspace, int n_cus,
                                       hipStream_t stream);

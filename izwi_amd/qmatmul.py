@@ -323,6 +323,57 @@ def forward_group(projections: Sequence["QMatMul"], x: torch.Tensor, norm_weight
     return tuple(ys)
 
 
+class ActivationRecords:
+    """Quantized activations in the layout the batched decode kernels read (3..64 rows), written by the
+    kernel that produces the activations instead of a quantizer launch of their own:
+    ``from_rms_norm`` (the layer norm in front of q|k|v and gate|up), ``from_silu_mul`` (silu(gate) * up in
+    front of down), ``quantize`` (anything else).  ``forward_group(projections)`` is `forward_group` on
+    them, bit-identical to the calls on the f32 activations."""
+
+    def __init__(self, weight_dtype: GgmlDType, m: int, k: int, device):
+        self.weight_dtype, self.m, self.k = GgmlDType(weight_dtype), m, k
+        nbytes = lib().izwi_qmm_records_bytes(int(weight_dtype), m, k)
+        self.data = torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+    @staticmethod
+    def _sp():
+        return torch.cuda.current_stream().cuda_stream
+
+    @classmethod
+    def quantize(cls, weight_dtype, x: torch.Tensor) -> "ActivationRecords":
+        assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2
+        r = cls(weight_dtype, x.shape[0], x.shape[1], x.device)
+        check(lib().izwi_qmm_quantize_records_f32(int(weight_dtype), x.data_ptr(), r.m, r.k, r.data.data_ptr(), cls._sp()))
+        return r
+
+    @classmethod
+    def from_rms_norm(cls, weight_dtype, x: torch.Tensor, norm_weight: torch.Tensor, eps: float = 1e-6) -> "ActivationRecords":
+        assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2
+        assert norm_weight.dtype == torch.float32 and norm_weight.is_contiguous() and norm_weight.numel() == x.shape[1]
+        r = cls(weight_dtype, x.shape[0], x.shape[1], x.device)
+        check(lib().izwi_rms_norm_quantize_records_f32(int(weight_dtype), x.data_ptr(), norm_weight.data_ptr(), r.m, r.k, eps,
+                                                       r.data.data_ptr(), cls._sp()))
+        return r
+
+    @classmethod
+    def from_silu_mul(cls, weight_dtype, gate: torch.Tensor, up: torch.Tensor) -> "ActivationRecords":
+        assert gate.is_cuda and gate.dtype == torch.float32 and gate.is_contiguous() and gate.dim() == 2
+        assert up.shape == gate.shape and up.dtype == torch.float32 and up.is_contiguous()
+        r = cls(weight_dtype, gate.shape[0], gate.shape[1], gate.device)
+        check(lib().izwi_qmm_silu_mul_quantize_records_f32(int(weight_dtype), gate.data_ptr(), up.data_ptr(), r.m, r.k,
+                                                           r.data.data_ptr(), cls._sp()))
+        return r
+
+    def forward_group(self, projections: Sequence["QMatMul"], outs=None):
+        n = len(projections)
+        ys = outs if outs is not None else [torch.empty((self.m, p.qtensor.dims2()[0]), dtype=torch.float32,
+                                                        device=self.data.device) for p in projections]
+        handles = (C.c_void_p * n)(*[p.qtensor._h for p in projections])
+        ptrs = (C.c_void_p * n)(*[y.data_ptr() for y in ys])
+        check(lib().izwi_qmm_forward_group_records_f32(handles, n, self.data.data_ptr(), self.m, ptrs, self._sp()))
+        return tuple(ys)
+
+
 class DecodeChain:
     """One token's projections as one launch (izwi_qmm_chain_*): ``steps`` is a list of
     ``(projections, x, ys)`` with 1..4 QMatMul of equal k, x a device f32 tensor of k values and one
