@@ -680,45 +680,57 @@ def q4_k_m_mix_extra(torch, qa, m=1, steps=20, warmup=3):
     return res
 
 
-def moe_extra(torch, qa, steps=50, warmup=5):
-    """One MoE layer (route + sort + grouped expert MLP + combine, HIP-graph replay) at the
-    Qwen3-30B-A3B shape: 128 experts, top-8, hidden 2048, expert intermediate 768, Q4_K; as one
-    call and as the three calls it is composed of."""
+def moe_extra(torch, qa, steps=20, warmup=3, layers=8, stacks=4):
+    """One MoE layer (route + sort + grouped expert MLP + combine) at the Qwen3-30B-A3B shape: 128
+    experts, top-8, hidden 2048, expert intermediate 768, Q4_K; as one call (izwi_moe_layer_f32) and as
+    the three calls it is composed of.  Timed as a HIP graph of `layers` consecutive layer calls that
+    cycle over `stacks` different sets of expert weights (as the layers of a model follow each other),
+    per layer; `us_single_call_graph` is the old figure, a graph that holds one call (it carries the
+    replay's own start-up)."""
+    import numpy as np
     e, top_k, hidden, inter = 128, 8, 2048, 768
     gg = qa.GgmlDType(Q4_K)
 
     def stack(n, k, seed):
         one = make_blocks(Q4_K, 8 * n, k, seed)  # 8 distinct experts, repeated
-        import numpy as np
         return qa.QTensor.from_blocks(gg, np.tile(one, e // 8), (e, n, k))
 
-    experts = qa.MoeExperts(stack(inter, hidden, 31), stack(inter, hidden, 32), stack(hidden, inter, 33))
+    experts = [qa.MoeExperts(stack(inter, hidden, 31 + 10 * i), stack(inter, hidden, 32 + 10 * i),
+                             stack(hidden, inter, 33 + 10 * i)) for i in range(stacks)]
     out = {}
     expert_bytes = 3 * inter * hidden * BPE[Q4_K]
     for t in (1, 16, 512):
         x = torch.from_numpy(synth_normal(40 + t, (t, hidden))).cuda()
-        logits_h = synth_normal(50 + t, (t, e))
-        logits = torch.from_numpy(logits_h).cuda()
+        logits = [torch.from_numpy(synth_normal(50 + t + 7 * i, (t, e))).cuda() for i in range(layers)]
 
         def three_calls():
-            ids, wts = qa.moe_route(logits, top_k)
-            perm, offsets = qa.moe_sort(ids, e)
-            return experts.forward(x, ids, wts, perm, offsets)
+            for i in range(layers):
+                ids, wts = qa.moe_route(logits[i], top_k)
+                perm, offsets = qa.moe_sort(ids, e)
+                experts[i % stacks].forward(x, ids, wts, perm, offsets)
 
-        us3, g3 = time_graph(torch, three_calls, steps, warmup)
+        def one_call():
+            for i in range(layers):
+                experts[i % stacks].layer(logits[i], x, top_k)
+
+        ms3, g3 = time_graph(torch, three_calls, steps, warmup)
         del g3
-        # the same layer as one call (izwi_moe_layer_f32): identical results
-        us, g = time_graph(torch, lambda: experts.layer(logits, x, top_k), steps, warmup)
-        us *= 1e3
-        ids_d, _ = qa.moe_route(logits, top_k)  # the library's own routing: which experts the tokens touch
-        distinct = len(set(ids_d.cpu().numpy().reshape(-1).tolist()))
-        rec = {"us": round(us, 1), "us_route_sort_forward_as_three_calls": round(us3 * 1e3, 1),
-               "distinct_experts": distinct}
+        ms, g = time_graph(torch, one_call, steps, warmup)
+        del g
+        ms1, g = time_graph(torch, lambda: experts[0].layer(logits[0], x, top_k), steps, warmup)
+        del g
+        us = ms * 1e3 / layers
+        distinct = 0
+        for i in range(layers):  # the library's own routing: which experts the tokens touch
+            ids_d, _ = qa.moe_route(logits[i], top_k)
+            distinct += len(set(ids_d.cpu().numpy().reshape(-1).tolist()))
+        distinct /= layers
+        rec = {"us": round(us, 1), "us_route_sort_forward_as_three_calls": round(ms3 * 1e3 / layers, 1),
+               "us_single_call_graph": round(ms1 * 1e3, 1), "distinct_experts": round(distinct, 1)}
         # algorithmic bytes: the distinct experts' weights + x in + out; flops: 3 matmuls per pair
         rec["gbs"] = round((distinct * expert_bytes + 2 * t * hidden * 4) / us / 1e3, 1)
         rec["tflops"] = round(2.0 * t * top_k * 3 * hidden * inter / us / 1e6, 2)
         out[f"t{t}"] = rec
-        del g
     return out
 
 

@@ -410,7 +410,9 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
  * (same results bit for bit).  logits `[t, n_experts]`, x and out `[t, hidden]`; ids_out /
  * weights_out `[t, top_k]` receive the routing if not NULL.  Up to 1024 (token, slot) pairs and
  * 256 experts, routing, sort and the kernel's segment tables are one launch (the layer is then 4
- * launches instead of 8). */
+ * launches instead of 8); up to 64 pairs (8 tokens at top-8) with an expert intermediate size up to
+ * 1024 the layer is TWO launches: every workgroup of the gate / up launch routes its own token, the
+ * down launch adds the slots in order (IZWI_QMM_MOE_SMALL_MAX_PAIRS changes the bound, 0 = never). */
 int izwi_moe_layer_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
                        const izwi_qmm_weight* down, const float* logits, const float* x, int64_t t,
                        int32_t top_k, float* out, int32_t* ids_out, float* weights_out,

@@ -112,6 +112,18 @@ int moe_mfma_min_rows() {
     return v;
 }
 
+// Most (token, slot) pairs for which izwi_moe_layer_f32 runs as two launches (every pair streams its
+// expert's weights on its own; measured at 128 experts, top-8: 13.7 / 15.7 / 24.8 / 40.2 us per layer at
+// 1 / 2 / 4 / 8 tokens against 23.3 / 26.5 / 33.4 / 46.6 on the grouped path, which reads an expert
+// once per segment and wins beyond).  IZWI_QMM_MOE_SMALL_MAX_PAIRS overrides; 0 turns it off.
+int moe_small_max_pairs() {
+    static const int v = [] {
+        const char* s = getenv("IZWI_QMM_MOE_SMALL_MAX_PAIRS");
+        return s ? atoi(s) : 64;
+    }();
+    return v;
+}
+
 // hipGetDevice with the missing-GPU case reported as such (not as a generic HIP error)
 int current_device(int* device) {
     hipError_t e = hipGetDevice(device);
@@ -1451,6 +1463,19 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
         int32_t* r_perm = (int32_t*)(r + 2 * p_bytes);
         int32_t* r_off = (int32_t*)(r + 3 * p_bytes);
         int32_t* r_sort = (int32_t*)(r + 3 * p_bytes + s_bytes);
+        // a handful of pairs: the whole layer in two launches (routing inside gate / up, combine
+        // inside down), same results
+        if (!tiles && pairs <= moe_small_max_pairs() && qmm_moe_small_supported(G, D, t, n_experts, top_k)) {
+            e = qmm_launch_moe_small(G, gate->tiled, up->tiled, D, down->tiled, logits, x, t, n_experts, top_k, h, r_ids,
+                                     r_w, ids_out, weights_out, out, max_segments, gate->n_cus, stream);
+            if (e == hipSuccess) {
+                if (profiling()) g_silu_fused.fetch_add(1, std::memory_order_relaxed);
+                return IZWI_QMM_OK;
+            }
+            if (e != hipErrorNotSupported) return fail_hip(e, "small-batch expert kernels");
+            (void)hipGetLastError();
+            e = hipSuccess;
+        }
         if (!tiles && qmm_moe_plan_small_supported(t, n_experts, top_k)) {
             e = qmm_launch_moe_plan_small(logits, t, n_experts, top_k, QMM_MOE_SEG_ROWS, max_segments, r_ids, r_w,
                                           r_perm, r_off, seg, seg_expert, stream);

@@ -30,6 +30,7 @@
 #include "qmm_internal.h"
 
 #include "qmm_gemv_blocks.h"
+#include "qmm_moe_route.h"
 
 namespace {
 
@@ -666,6 +667,157 @@ hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* co
             if (mt == 2) gemv_kernel<qt, 2, false, false, true><<<g, b, need, stream>>>(P);
             else gemv_kernel<qt, 1, false, false, true><<<g, b, need, stream>>>(P);
         }
+        return hipGetLastError();
+    });
+}
+
+// ---- expert MLP of a small batch in two launches --------------------------------------------
+// Launch 1: every workgroup routes its own token (a wave, 128 logits: cheaper than a launch of
+// its own), then runs the gated single-row decode body on the expert of its (token, slot) pair:
+// h[pair] = silu(W_gate[e] x_t) * (W_up[e] x_t).  blockIdx.y = pair.
+namespace {
+
+template <int QT, int PER_LANE>
+__global__ __launch_bounds__(64 * kMaxWaves) __attribute__((amdgpu_waves_per_eu(3)))
+void moe_small_gate_up_kernel(GemvParams P, const float* __restrict__ logits, int n_experts, int top_k,
+                              int32_t* __restrict__ ids, float* __restrict__ weights, int32_t* __restrict__ ids_out,
+                              float* __restrict__ weights_out) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ int expert_sh;
+    const int pair = blockIdx.y;
+    const int tok = pair / top_k, slot = pair - tok * top_k;
+    if (threadIdx.x < 64) {
+        int id;
+        float w;
+        moe_route::route_token<PER_LANE>(logits + (int64_t)tok * n_experts, n_experts, top_k, (int)threadIdx.x, id, w);
+        if ((int)threadIdx.x == slot) expert_sh = id;
+        if (blockIdx.x == 0 && slot == 0 && (int)threadIdx.x < top_k) { // once per token: the routing for launch 2
+            ids[tok * top_k + threadIdx.x] = id;
+            weights[tok * top_k + threadIdx.x] = w;
+            if (ids_out) ids_out[tok * top_k + threadIdx.x] = id;
+            if (weights_out) weights_out[tok * top_k + threadIdx.x] = w;
+        }
+    }
+    __syncthreads();
+    const int e = expert_sh;
+    GemvParams Q = P;
+    Q.x = P.x + (int64_t)tok * P.k;
+    gemv_body<QT, 1, true, false, true>(Q, 0, 1, P.w + (int64_t)e * P.matrix_bytes, P.y + (int64_t)pair * P.n, P.n,
+                                        P.row_tiles, blockIdx.x, smem);
+}
+
+// Launch 2: out[t] = sum over slots s (in order) of weights[t, s] * (W_down[e_s] h[t, s]).  A
+// workgroup is one 16-row tile of one token, a wave is one slot: it quantizes its h row, multiplies
+// its expert's panel (k fits one panel), and the slots are added in order through LDS, the sums and
+// products of the grouped decode kernel followed by the combine kernel.
+struct MoeSmallDown {
+    const uint8_t* w;
+    const float* h;        // [pairs, k]
+    const int32_t* ids;    // [pairs]
+    const float* weights;  // [pairs]
+    float* out;            // [t, n]
+    int n, k, k_units, slots, row_tiles, top_k;
+    int panel_bytes;
+    int64_t matrix_bytes;
+};
+
+template <int QT>
+__global__ __launch_bounds__(64 * kMaxWaves) void moe_small_down_kernel(MoeSmallDown P) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int rt = blockIdx.x, tok = blockIdx.y;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int pair = tok * P.top_k + wave;
+    const int e = P.ids[pair];
+    const size_t per_wave = (lds_bytes<QT, 1>(P.k_units, 0) + 15) & ~(size_t)15;
+    float* ysum = reinterpret_cast<float*>(smem + per_wave * P.top_k); // [top_k][16]
+    const XLds<QT> l = carve<QT, 1>(smem + per_wave * wave, P.k_units);
+    // activations first, the panel behind them
+    const int item = lane >> 4, j = lane & 15;
+    const bool item_ok = item < P.k_units;
+    const int k0 = item * 256 + 16 * j;
+    const bool in_range = item_ok && k0 + 16 <= P.k;
+    float4 f[4];
+    x16_issue<false>(P.h + (int64_t)pair * P.k + k0, P.h, in_range, f);
+    Panel<QT> p;
+    const bool active = lane < P.slots;
+    load_panel<QT>(p, P.w + (int64_t)e * P.matrix_bytes + (int64_t)rt * P.panel_bytes, P.slots, lane, active);
+    float v[16];
+    x16_finish<false>(f, in_range, v);
+    if (item_ok) x_item_quantize<QT, 1>(l, P.k_units, item, v);
+    for (int it = item + 4; it < P.k_units; it += 4) { // more than four units (k > 1024): not reached, k fits a panel
+        const int k1 = it * 256 + 16 * j;
+        const bool ok1 = k1 + 16 <= P.k;
+        x16_issue<false>(P.h + (int64_t)pair * P.k + k1, P.h, ok1, f);
+        x16_finish<false>(f, ok1, v);
+        x_item_quantize<QT, 1>(l, P.k_units, it, v);
+    }
+    // the wave reads back what its own lanes wrote: LDS serves a wave's accesses in order
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    mask_panel<QT>(p, active);
+    float acc[1] = {0.0f};
+    multiply_panel<QT, 1>(p, l, min(lane >> 4, P.k_units - 1), P.k_units, acc);
+    acc[0] += __shfl_xor(acc[0], 16);
+    acc[0] += __shfl_xor(acc[0], 32);
+    if (lane < 16) ysum[wave * 16 + lane] = acc[0];
+    __syncthreads();
+    if (wave == 0 && lane < 16) {
+        const int row = rt * 16 + lane;
+        float o = 0.0f;
+        for (int s = 0; s < P.top_k; s++) o += P.weights[tok * P.top_k + s] * ysum[s * 16 + lane];
+        if (row < P.n) P.out[(int64_t)tok * P.n + row] = o;
+    }
+}
+
+} // namespace
+
+bool qmm_moe_small_supported(const QmmLayout& G, const QmmLayout& D, int64_t t, int n_experts, int top_k) {
+    // one panel per row tile of the down projection (k = inter <= 1024), a wave per slot
+    return t >= 1 && t * top_k <= 64 && top_k <= kMaxWaves && n_experts <= 256 && D.k_groups == 1 && D.k_units <= 4 &&
+           G.k_groups <= kMaxWaves / 2;
+}
+
+hipError_t qmm_launch_moe_small(const QmmLayout& G, const void* gate, const void* up, const QmmLayout& D, const void* down,
+                                const float* logits, const float* x, int64_t t, int n_experts, int top_k, float* h,
+                                int32_t* ids, float* weights, int32_t* ids_out, float* weights_out, float* out,
+                                int64_t max_segments, int n_cus, hipStream_t stream) {
+    if (!qmm_moe_small_supported(G, D, t, n_experts, top_k)) return hipErrorNotSupported;
+    const int pairs = (int)(t * top_k);
+    GemvParams P;
+    if (!make_params(G, gate, x, 1, h, P)) return hipErrorInvalidValue;
+    P.w2 = (const uint8_t*)up;
+    int waves;
+    // the split of the grouped launch this replaces: same sums
+    choose_split(G, n_cus, (int)max_segments, true, P, waves);
+    if (P.kpw != 1 || P.rt_groups > n_cus * 32) return hipErrorNotSupported;
+    hipError_t e = with_block_type(G.dtype, [&](auto QT) {
+        constexpr int qt = decltype(QT)::value;
+        const size_t lds = lds_bytes<qt, 1>(P.k_units, 2 * waves);
+        if (lds > 48 * 1024) return hipErrorNotSupported;
+        const dim3 grid((unsigned)P.rt_groups, (unsigned)pairs), block(64 * 2 * waves);
+        if (n_experts <= 128)
+            moe_small_gate_up_kernel<qt, 2><<<grid, block, lds, stream>>>(P, logits, n_experts, top_k, ids, weights, ids_out, weights_out);
+        else
+            moe_small_gate_up_kernel<qt, 4><<<grid, block, lds, stream>>>(P, logits, n_experts, top_k, ids, weights, ids_out, weights_out);
+        return hipGetLastError();
+    });
+    if (e != hipSuccess) return e;
+    MoeSmallDown Q;
+    Q.w = (const uint8_t*)down;
+    Q.h = h;
+    Q.ids = ids;
+    Q.weights = weights;
+    Q.out = out;
+    Q.n = (int)D.n, Q.k = (int)D.k, Q.k_units = (int)D.k_units, Q.slots = D.slots, Q.row_tiles = (int)D.row_tiles;
+    Q.top_k = top_k;
+    Q.panel_bytes = (int)D.panel_bytes;
+    Q.matrix_bytes = D.matrix_bytes;
+    return with_block_type(D.dtype, [&](auto QT) {
+        constexpr int qt = decltype(QT)::value;
+        const size_t per_wave = (lds_bytes<qt, 1>(Q.k_units, 0) + 15) & ~(size_t)15;
+        const size_t lds = per_wave * top_k + (size_t)top_k * 16 * sizeof(float);
+        if (lds > 48 * 1024) return hipErrorNotSupported;
+        moe_small_down_kernel<qt><<<dim3((unsigned)D.row_tiles, (unsigned)t), dim3(64 * top_k), lds, stream>>>(Q);
         return hipGetLastError();
     });
 }

@@ -277,6 +277,17 @@ hipError_t qmm_launch_moe_plan_small(const float* logits, int64_t t, int n_exper
                                      int32_t* offsets, int32_t* seg_offsets, int32_t* seg_expert,
                                      hipStream_t stream);
 
+// The whole expert MLP of a small batch (t * top_k <= 64 pairs, inter <= 1024) in TWO launches:
+// routing inside the gate / up launch (every workgroup routes its own token), the weighted
+// combine inside the down launch (a wave per slot, slots added in order).  Same results as
+// route + sort + grouped kernels + combine.  `h` [pairs, inter], `ids` / `weights` [pairs] are
+// scratch; ids_out / weights_out may be NULL.  hipErrorNotSupported: use the general path.
+bool qmm_moe_small_supported(const QmmLayout& G, const QmmLayout& D, int64_t t, int n_experts, int top_k);
+hipError_t qmm_launch_moe_small(const QmmLayout& G, const void* gate, const void* up, const QmmLayout& D, const void* down,
+                                const float* logits, const float* x, int64_t t, int n_experts, int top_k, float* h,
+                                int32_t* ids, float* weights, int32_t* ids_out, float* weights_out, float* out,
+                                int64_t max_segments, int n_cus, hipStream_t stream);
+
 // out[t, :] = sum over slots s (in order) of weights[t, s] * y[t * top_k + s, :]
 hipError_t qmm_launch_moe_combine(const float* y, const float* weights, int64_t t, int top_k,
                                   int64_t hidden, float* out, hipStream_t stream);

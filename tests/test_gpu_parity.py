@@ -480,7 +480,7 @@ def test_config5_moe_forward(qa, oracle, moe_weights, t):
     assert np.isfinite(out).all()
 
 
-@pytest.mark.parametrize("t", [1, 3, 16, 100, 128, 129, 512])
+@pytest.mark.parametrize("t", [1, 2, 3, 16, 100, 128, 129, 512])
 def test_config5_moe_layer_one_call_equals_the_three_calls(qa, oracle, moe_weights, t):
     """izwi_moe_layer_f32 = route + sort + forward, bit for bit (ids, weights, outputs): up to
     1024 pairs routing, sort and segment tables come from one launch, beyond from the
@@ -518,6 +518,8 @@ def test_config5_moe_layer_one_call_equals_the_three_calls(qa, oracle, moe_weigh
     (Q8_0, 8, 512, 256, 64, 4),     # 32 pairs per expert: matrix-core tiles, Q8_0, one unit per panel
     (Q4_K, 4, 1280, 768, 40, 2),    # ragged k (5 units), three-unit panels on the way down
     (Q4_K, 16, 512, 512, 6, 8),     # 3 pairs per expert: 4-row segments
+    (Q8_0, 8, 512, 256, 2, 4),      # 8 pairs: the two-launch form (routing in gate / up, combine in down)
+    (Q4_K, 8, 1280, 1024, 3, 2),    # the same with four units per panel on the way down, ragged k on the way up
 ])
 def test_moe_forward_small_shapes(qa, oracle, dtype, E, hidden, inter, t, top_k):
     gate = oracle.quantize(dtype, oracle.randn(301, (E * inter, hidden), std=0.05))
