@@ -772,6 +772,9 @@ def main():
                          "per-projection: seven izwi_qmm_forward_f32 calls per layer")
     ap.add_argument("--neighbours-only", action="store_true",
                     help="time only the decode-step neighbours (norms, rotary, attention) and print them: for profiling")
+    ap.add_argument("--moe-only", action="store_true",
+                    help="profiling aid: run only izwi_moe_layer_f32 at the Qwen3-30B-A3B shape with --m tokens "
+                         "(--steps calls, eager) and print the time per call, nothing else")
     ap.add_argument("--prefill-only", default=None, choices=["q", "k", "gate", "down", "qkv", "gate_up"],
                     help="profiling aid: run only the prefill call of one 8B projection (--m rows, default "
                          "2048 here; --steps calls) and print its TFLOP/s, nothing else")
@@ -791,6 +794,20 @@ def main():
 
     if args.neighbours_only:
         print(json.dumps({"decode_step_neighbours_f32": neighbours_extra(torch, qa, args.steps, args.warmup)}))
+        return
+
+    if args.moe_only:
+        import numpy as np
+        e, top_k, hidden, inter, t = 128, 8, 2048, 768, args.m
+        gg = qa.GgmlDType(Q4_K)
+
+        def stack(n, k, seed):
+            return qa.QTensor.from_blocks(gg, np.tile(make_blocks(Q4_K, 8 * n, k, seed), e // 8), (e, n, k))
+        experts = qa.MoeExperts(stack(inter, hidden, 31), stack(inter, hidden, 32), stack(hidden, inter, 33))
+        x = torch.from_numpy(synth_normal(40 + t, (t, hidden))).cuda()
+        logits = torch.from_numpy(synth_normal(50 + t, (t, e))).cuda()
+        ms = time_eager(torch, lambda: experts.layer(logits, x, top_k), args.steps, args.warmup)
+        print(json.dumps({"moe_layer_us": round(ms * 1e3, 1), "tokens": t, "experts": e, "top_k": top_k}))
         return
 
     if args.prefill_only:

@@ -116,6 +116,114 @@ __global__ void sort_scatter_kernel(const int32_t* __restrict__ ids, int64_t pai
     }
 }
 
+// Rank of every lane's id among the equal ids of earlier lanes of its wave, and the number of lanes
+// that hold it: the lanes OR their bit into a 64-bit mask per expert in LDS (an OR is order-free), then
+// count the bits below their own.  `masks` = the wave's own [n_experts] pairs of 32-bit words, zeroed here.
+__device__ __forceinline__ void wave_ranks(int e, int n_experts, int lane, uint32_t* masks, int& rank, int& total) {
+    for (int i = lane; i < 2 * n_experts; i += 64) masks[i] = 0u;
+    __builtin_amdgcn_wave_barrier();
+    const bool ok = e >= 0 && e < n_experts;
+    if (ok) atomicOr(&masks[2 * e + (lane >> 5)], 1u << (lane & 31));
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const uint32_t lo = ok ? masks[2 * e] : 0u, hi = ok ? masks[2 * e + 1] : 0u;
+    const uint32_t below_lo = lane < 32 ? lo & ((1u << lane) - 1u) : lo;
+    const uint32_t below_hi = lane < 32 ? 0u : hi & ((1u << (lane & 31)) - 1u);
+    rank = __popc(below_lo) + __popc(below_hi);
+    total = __popc(lo) + __popc(hi);
+    __builtin_amdgcn_wave_barrier(); // the masks are reused by the wave's next run
+}
+
+// inclusive sum over the 64 lanes of a wave
+__device__ __forceinline__ int wave_inclusive_sum(int v, int lane) {
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int o = __shfl_up(v, d);
+        if (lane >= d) v += o;
+    }
+    return v;
+}
+
+// The whole stable counting sort in ONE workgroup (pairs up to 16384, n_experts up to 1024 as far as
+// LDS holds runs x experts counters): pairs are cut into runs of 64 (one wave each); a lane finds its
+// rank among the equal ids of its run through per-expert bit masks; the runs' per-expert counts are
+// scanned run by run (a wave per expert, a lane per run) and over the experts (wave scans); every
+// pair goes to offsets[e] + (pairs of e in earlier runs) + rank.  Integer arithmetic whose result does
+// not depend on the order of execution: the same perm / offsets as the three-kernel sort.
+constexpr int kBlockSortThreads = 1024, kBlockSortMaxRuns = 16; // runs per wave
+__global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int32_t* __restrict__ ids, int pairs,
+                                                                       int n_experts, int32_t* __restrict__ perm,
+                                                                       int32_t* __restrict__ offsets,
+                                                                       int32_t* __restrict__ seg_offsets) {
+    extern __shared__ int32_t sh[]; // hist[runs][n_experts] | start[n_experts + 1] | masks[waves][2 * n_experts]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = kBlockSortThreads / 64;
+    const int runs = (pairs + 63) / 64;
+    int32_t* start = sh + runs * n_experts;
+    uint32_t* masks = reinterpret_cast<uint32_t*>(start + n_experts + 1) + wave * 2 * n_experts;
+    __shared__ int32_t wave_tot[16], wave_seg[16];
+    for (int i = threadIdx.x; i < runs * n_experts; i += kBlockSortThreads) sh[i] = 0;
+    __syncthreads();
+    int my_e[kBlockSortMaxRuns], my_rank[kBlockSortMaxRuns];
+#pragma unroll
+    for (int j = 0; j < kBlockSortMaxRuns; j++) {
+        const int run = wave + j * waves;
+        my_e[j] = -1, my_rank[j] = 0;
+        if (run >= runs) continue; // uniform per wave
+        const int p = run * 64 + lane;
+        const int e = p < pairs ? ids[p] : -1;
+        int rank, total;
+        wave_ranks(e, n_experts, lane, masks, rank, total);
+        my_e[j] = e, my_rank[j] = rank;
+        if (e >= 0 && e < n_experts && rank == 0) sh[run * n_experts + e] = total; // the first of its expert in the run
+    }
+    __syncthreads();
+    // per expert (a wave each, in turn): the runs' counts become the number of earlier pairs of the
+    // expert; lane = run, 64 runs per step
+    for (int e = wave; e < n_experts; e += waves) {
+        int carry = 0;
+        for (int r0 = 0; r0 < runs; r0 += 64) {
+            const int r = r0 + lane;
+            const int h = r < runs ? sh[r * n_experts + e] : 0;
+            const int inc = wave_inclusive_sum(h, lane);
+            if (r < runs) sh[r * n_experts + e] = carry + inc - h;
+            carry += __shfl(inc, 63);
+        }
+        if (lane == 0) start[e] = carry; // the expert's total, for now
+    }
+    __syncthreads();
+    // exclusive scan over the experts: thread e holds expert e (n_experts <= 1024), wave scans, then the
+    // waves' totals
+    const int e0 = threadIdx.x;
+    const int c = e0 < n_experts ? start[e0] : 0;
+    const int sg = (c + QMM_MOE_SEG_ROWS - 1) / QMM_MOE_SEG_ROWS;
+    const int inc_c = wave_inclusive_sum(c, lane), inc_s = wave_inclusive_sum(sg, lane);
+    if (lane == 63) wave_tot[wave] = inc_c, wave_seg[wave] = inc_s;
+    __syncthreads();
+    int base_c = 0, base_s = 0;
+    for (int w = 0; w < wave; w++) base_c += wave_tot[w], base_s += wave_seg[w];
+    if (e0 <= n_experts) {
+        // (thread n_experts holds the grand totals: its own c is 0)
+        offsets[e0] = base_c + inc_c - c;
+        if (seg_offsets) seg_offsets[e0] = base_s + inc_s - sg;
+        start[e0] = base_c + inc_c - c;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kBlockSortMaxRuns; j++) {
+        const int run = wave + j * waves;
+        if (run >= runs) continue;
+        const int e = my_e[j];
+        if (e >= 0 && e < n_experts) perm[start[e] + sh[run * n_experts + e] + my_rank[j]] = run * 64 + lane;
+    }
+}
+
+bool block_sort_fits(int64_t pairs, int n_experts) {
+    if (pairs < 1 || n_experts >= kBlockSortThreads) return false;
+    const int64_t runs = (pairs + 63) / 64;
+    return runs <= (int64_t)kBlockSortMaxRuns * (kBlockSortThreads / 64) &&
+           ((runs + 1) * n_experts + 1 + 2 * n_experts * (kBlockSortThreads / 64)) * 4 <= 64 * 1024;
+}
+
 // seg_offsets[e] = sum over e' < e of ceil(count(e') / seg_rows).  One block:
 // every thread sums a contiguous run of experts, the runs are scanned in LDS.
 // With seg_expert: seg_expert[s] = expert of segment s, -1 for s past the last
@@ -250,6 +358,16 @@ hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts,
                                int32_t* offsets, int32_t* seg_offsets, int32_t* scratch,
                                hipStream_t stream) {
     if (n_experts < 1 || n_experts > 8192) return hipErrorInvalidValue;
+    if (block_sort_fits(pairs, n_experts)) {
+        const size_t lds = ((size_t)((pairs + 63) / 64 + 1) * n_experts + 1 + (size_t)2 * n_experts * (kBlockSortThreads / 64)) * sizeof(int32_t);
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sort_block_kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+            if (e != hipSuccess) return e;
+        }
+        sort_block_kernel<<<1, kBlockSortThreads, lds, stream>>>(ids, (int)pairs, n_experts, perm, offsets, seg_offsets);
+        return hipGetLastError();
+    }
     int64_t chunks = (pairs + kSortChunk - 1) / kSortChunk;
     if (chunks < 1) chunks = 1;
     size_t sh = (size_t)n_experts * sizeof(int32_t);
