@@ -299,6 +299,22 @@ public:
     std::vector<float> forward(const std::vector<float>& x) const { return mm_.forward(x); }
     const QMatMul& qmatmul() const { return mm_; }
 
+    // `Qwen3Projection::logits_for_tokens` (core.rs:745-758): (token id, logit) pairs of one hidden
+    // state for the given ids; only the weight rows of those ids are read.
+    std::vector<std::pair<uint32_t, float>> logits_for_tokens(const std::vector<float>& hidden,
+                                                              const std::vector<uint32_t>& token_ids) const {
+        std::vector<std::pair<uint32_t, float>> out;
+        if (token_ids.empty()) return out;
+        if ((int64_t)hidden.size() != mm_.qtensor()->cols())
+            throw Error(Error::Kind::InferenceError, IZWI_QMM_ERR_INVALID,
+                        "Qwen3 selected-token logits expected [1,vocab] or [1,1,vocab]");
+        std::vector<float> values(token_ids.size());
+        check(izwi_qmm_forward_rows_f32(mm_.qtensor()->handle(), token_ids.data(), (int64_t)token_ids.size(), hidden.data(),
+                                        1, values.data(), IZWI_QMM_HOST, nullptr));
+        for (size_t i = 0; i < token_ids.size(); i++) out.emplace_back(token_ids[i], values[i]);
+        return out;
+    }
+
 private:
     explicit Qwen3Projection(QMatMul mm) : mm_(std::move(mm)) {}
     QMatMul mm_;
@@ -307,13 +323,25 @@ private:
 // `is_gguf_file` (gguf.rs:366-377).
 inline bool is_gguf_file(const std::string& path) { return izwi_gguf_is_gguf_file(path.c_str()) != 0; }
 
-// `GgufLoader` (gguf.rs:36-203): one mapped GGUF file; tensors go from the mapping straight
-// into weight handles on the current HIP device.  Parsing and lookups need no GPU.
+// `GgufMmapMode` / `GgufReaderKind` (backends/model_io.rs:13-45, 85-89).
+enum class GgufMmapMode : int { Auto = IZWI_GGUF_MMAP_AUTO, On = IZWI_GGUF_MMAP_ON, Off = IZWI_GGUF_MMAP_OFF };
+enum class GgufReaderKind : int { Buffered = IZWI_GGUF_READER_BUFFERED, Mapped = IZWI_GGUF_READER_MAPPED };
+// `GgufMmapMode::parse`: false for the empty string and unknown words.
+inline bool parse_gguf_mmap_mode(const std::string& raw, GgufMmapMode* out) {
+    const int m = izwi_gguf_parse_mmap_mode(raw.c_str());
+    if (m < 0) return false;
+    *out = (GgufMmapMode)m;
+    return true;
+}
+
+// `GgufLoader` (gguf.rs:36-203): one GGUF file, mapped or (mode off, or a mapping that fails) read
+// with buffered I/O as `open_gguf_reader_with_mode` does (model_io.rs:127-160); tensors go from there
+// straight into weight handles on the current HIP device.  Parsing and lookups need no GPU.
 class GgufLoader {
 public:
-    static std::shared_ptr<GgufLoader> from_path(const std::string& path) {
+    static std::shared_ptr<GgufLoader> from_path(const std::string& path, const GgufMmapMode* configured = nullptr) {
         izwi_gguf* g = nullptr;
-        const int rc = izwi_gguf_open(path.c_str(), &g);
+        const int rc = izwi_gguf_open_with_mode(path.c_str(), configured ? (int)*configured : -1, &g);
         if (rc != IZWI_QMM_OK) // `Error::ModelLoadError("Failed to open / parse GGUF file: ...")`
             throw Error(Error::Kind::ModelLoadError, rc, izwi_qmm_last_error());
         return std::shared_ptr<GgufLoader>(new GgufLoader(g));
@@ -322,6 +350,7 @@ public:
     GgufLoader(const GgufLoader&) = delete;
     GgufLoader& operator=(const GgufLoader&) = delete;
 
+    GgufReaderKind reader_kind() const { return (GgufReaderKind)izwi_gguf_reader_kind(g_); }
     size_t tensor_count() const { return (size_t)izwi_gguf_tensor_count(g_); }
     std::vector<std::string> tensor_names() const {
         std::vector<std::string> out;

@@ -196,10 +196,38 @@ static void gguf_parse(const std::string& fixture) {
                   [&] { izwi::GgufLoader::from_path(fixture + ".absent"); }));
     EXPECT(throws(izwi::Error::Kind::ModelLoadError, "not supported", [&] { g->load_qtensor("a"); }));
     EXPECT(throws(izwi::Error::Kind::ModelLoadError, "tensor not found", [&] { g->load_qtensor("nope"); }));
+    // the reader policy of backends/model_io.rs: auto maps, "off" reads with buffered I/O, same contents
+    EXPECT(g->reader_kind() == izwi::GgufReaderKind::Mapped);
+    izwi::GgufMmapMode mode = izwi::GgufMmapMode::Auto;
+    EXPECT(izwi::parse_gguf_mmap_mode("no", &mode) && mode == izwi::GgufMmapMode::Off);
+    EXPECT(izwi::parse_gguf_mmap_mode(" TRUE ", &mode) && mode == izwi::GgufMmapMode::On);
+    EXPECT(!izwi::parse_gguf_mmap_mode("", &mode) && !izwi::parse_gguf_mmap_mode("invalid", &mode));
+    const izwi::GgufMmapMode off = izwi::GgufMmapMode::Off;
+    auto b = izwi::GgufLoader::from_path(fixture, &off);
+    EXPECT(b->reader_kind() == izwi::GgufReaderKind::Buffered && b->tensor_names() == names);
 }
 
 // ... and its tensors on the GPU: the Q4_K tensor is the hand-built block whose closed form
 // sums to 32224; the Q8_0 block is d = 1, q = -16 .. 15.
+// `logits_for_tokens` (core.rs:745-758): the selected ids of the full product, bit for bit.
+static void selected_token_logits() {
+    using izwi::GgmlDType;
+    const int64_t n = 4000, k = 1024;
+    std::vector<float> w((size_t)n * k), x((size_t)k);
+    oracle_fill_normal(71, 0, (int64_t)w.size(), 0.0f, 0.02f, w.data());
+    oracle_fill_normal(72, 0, k, 0.0f, 1.0f, x.data());
+    std::vector<uint8_t> blocks((size_t)oracle_storage_bytes((int)GgmlDType::Q4K, n, k));
+    EXPECT(oracle_quantize((int)GgmlDType::Q4K, n, k, w.data(), blocks.data()) == 0);
+    auto proj = izwi::Qwen3Projection::quantized(izwi::QTensor::from_blocks(GgmlDType::Q4K, blocks.data(), blocks.size(), n, k));
+    const std::vector<float> full = proj.forward(x);
+    const std::vector<uint32_t> ids = {3999, 0, 17, 17, 2048, 1};
+    const auto pairs = proj.logits_for_tokens(x, ids);
+    EXPECT(pairs.size() == ids.size());
+    for (size_t i = 0; i < pairs.size(); i++) EXPECT(pairs[i].first == ids[i] && pairs[i].second == full[ids[i]]);
+    EXPECT(proj.logits_for_tokens(x, {}).empty());
+    EXPECT(throws(izwi::Error::Kind::InvalidInput, "out of range", [&] { proj.logits_for_tokens(x, {4000}); }));
+}
+
 static void gguf_load(const std::string& fixture) {
     auto g = izwi::GgufLoader::from_path(fixture);
     auto q4 = g->load_qtensor("hand.q4k");
@@ -227,6 +255,7 @@ int main(int argc, char** argv) {
         packed_matches_separate_q8_0();
         q4k_projection_matches_oracle();
         folded_calls_match_oracle();
+        selected_token_logits();
         gguf_load(fixture);
     } else if (mode == "nodevice") {
         no_device_is_loud();
