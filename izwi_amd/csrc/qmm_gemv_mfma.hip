@@ -6,7 +6,7 @@
 // Two launches:
 //  1. the activations are quantized ONCE into a workspace of self-contained
 //     unit records (256 k-values of 16 rows): 4096 B of int8 laid out exactly as
-//     the MFMA A operand wants them ([sub-block][octet][row][8 B]) followed by
+//     the MFMA A operand wants them ([sub-block pair][octet][row][16 B]) followed by
 //     the unit's side information (row scales; for Q4_K also the sub-block sums
 //     as two int8 planes), so the matmul workgroups move a run of units to LDS
 //     verbatim with LDS-direct loads;
@@ -41,6 +41,7 @@ constexpr int kMaxWaves = 12;
 constexpr uint32_t kNib = 0x0f0f0f0fu;
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef long i64x2 __attribute__((ext_vector_type(2)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWindowUnits = 32; // activation units resident in LDS at a time
@@ -263,7 +264,7 @@ template <int QT, bool FIRST>
 __device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int n_units, int j, int grp,
                                           float (&acc)[4]) {
     constexpr int UB = Unit<QT>::kBytes;
-    const int lane8 = (grp * 16 + j) * 8;
+    const int lane16 = (grp * 16 + j) * 16; // this lane's 16 bytes of a sub-block pair
     // Units of the panel that do not exist (ragged k, S < 4) are not skipped, which
     // would split the arithmetic into many small blocks: they read unit 0's
     // activations and their weight scale is multiplied by zero.  (Their header is
@@ -304,9 +305,8 @@ __device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int
                     const int u = 2 * h + e;
                     if (u >= n_units) continue; // uniform
                     const uint32_t w0 = e ? qq.z : qq.x, w1 = e ? qq.w : qq.y;
-                    const uint8_t* xu = xu0 + xo[u] + lane8;
-                    const long a_lo = *reinterpret_cast<const long*>(xu + (2 * b) * 512);
-                    const long a_hi = *reinterpret_cast<const long*>(xu + (2 * b + 1) * 512);
+                    const i64x2 aa = *reinterpret_cast<const i64x2*>(xu0 + xo[u] + lane16 + b * 1024);
+                    const long a_lo = aa.x, a_hi = aa.y;
                     dlo[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, pack64(w0 & kNib, w1 & kNib),
                                                                    i32x4{0, 0, 0, 0}, 0, 0, 0);
                     dhi[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(
@@ -385,7 +385,7 @@ __device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int
                         const uint32_t s1 = ((v1 | 0x80808080u) - 0x20202020u) ^ 0x80808080u;
                         const long bq = pack64(s0, s1);
                         const long b_lo = grp < 2 ? bq : 0L, b_hi = grp < 2 ? 0L : bq;
-                        const long a = *reinterpret_cast<const long*>(xu0 + xo[u] + lane8 + t * 512);
+                        const long a = *reinterpret_cast<const long*>(xu0 + xo[u] + lane16 + (t >> 1) * 1024 + (t & 1) * 8);
                         dlo[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b_lo, i32x4{0, 0, 0, 0}, 0, 0, 0);
                         dhi[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b_hi, i32x4{0, 0, 0, 0}, 0, 0, 0);
                     }
@@ -423,7 +423,7 @@ __device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int
                 if (u >= n_units) continue; // uniform
                 const u32x4 qq = p.q[2 * b + (u >> 1)];
                 const uint32_t w0 = (u & 1) ? qq.z : qq.x, w1 = (u & 1) ? qq.w : qq.y;
-                const long a = *reinterpret_cast<const long*>(xu0 + xo[u] + lane8 + b * 512);
+                const long a = *reinterpret_cast<const long*>(xu0 + xo[u] + lane16 + (b >> 1) * 1024 + (b & 1) * 8);
                 dd[u] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, pack64(w0, w1), i32x4{0, 0, 0, 0}, 0, 0, 0);
             }
 #pragma unroll
@@ -521,7 +521,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
     // the first activation window goes first (loads return in order), then the panel
     const int w0_units = min(P.window_units, P.k_units);
     issue_window_copy<QT>(records, lds_x, w0_units, wave, waves, lane);
-    asm volatile("" ::: "memory");
+    // A CU's loads return in the order they were issued, for all its waves together: without this
+    // barrier the last wave's window pieces queue behind the other waves' panels, and the barrier
+    // below - the start of all arithmetic - waits for nearly the whole workgroup's weights.
+    asm volatile("s_barrier" ::: "memory");
     WPanel<QT> p;
     load_wpanel<QT>(p, wbase + (int64_t)((rt_ok ? rt : 0) * P.k_groups + wk) * P.panel_bytes, P.slots, lane, j);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory"); // the window has landed, the panel may still fly
@@ -714,13 +717,15 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(Mf
     for (int u = 0; u < 4; u++) {
         const uint8_t* rec = P.ws + (size_t)(unit0 + (u < n_units ? u : 0)) * UB; // missing units re-read unit 0
 #pragma unroll
-        for (int sb = 0; sb < 8; sb++) a[u][sb] = *reinterpret_cast<const long*>(rec + sb * 512 + lane * 8);
+        for (int b = 0; b < 4; b++) {
+            const i64x2 aa = *reinterpret_cast<const i64x2*>(rec + b * 1024 + lane * 16);
+            a[u][2 * b] = aa.x, a[u][2 * b + 1] = aa.y;
+        }
         const uint8_t* side = rec + Unit<QT>::kQuant;
         // the sub-block sums occupy k slots 0..7 of the min-term MFMA: the first 16-lane row only
-        const long lo = *reinterpret_cast<const long*>(side + 64 + j * 16);
-        const long hi = *reinterpret_cast<const long*>(side + 64 + j * 16 + 8);
-        bs_lo[u] = grp == 0 ? lo : 0L;
-        bs_hi[u] = grp == 0 ? hi : 0L;
+        const i64x2 planes = *reinterpret_cast<const i64x2*>(side + 64 + j * 16);
+        bs_lo[u] = grp == 0 ? planes.x : 0L;
+        bs_hi[u] = grp == 0 ? planes.y : 0L;
         dx[u] = *reinterpret_cast<const float4*>(side + grp * 16);
     }
     WPanel<QT> p;

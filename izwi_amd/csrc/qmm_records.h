@@ -35,7 +35,10 @@ __device__ __forceinline__ int row16_min(int v) {
 
 template <int QT>
 struct Unit {
-    static constexpr int kQuant = 4096; // [8 sub-blocks][4 octets][16 rows][8 B]
+    // [4 sub-block pairs][4 octets][16 rows][16 B]: the 8 quants of (sub-block 2b, octet, row), then
+    // those of sub-block 2b + 1 - one 16-byte load per lane (lane = 16 * octet + row) brings both
+    // matrix-core operands of a pair
+    static constexpr int kQuant = 4096;
     // Q4_K: 16 row scales (f32), then per row the eight sub-block sums of the quants split
     // into two int8 planes (sum = 128 * hi + lo): 64 + 16 * 16 bytes.
     // Q8_0: one f32 scale per (block, row): 8 * 16 * 4 bytes.
@@ -103,9 +106,9 @@ __device__ __forceinline__ void quantize_into_record(const float (&v)[16], int j
             planes[8 + s] = (uint8_t)(bsum >> 7);
         }
     }
-    uint8_t* dst = rec + (s * 4 + oct) * 128 + mr * 8;
+    uint8_t* dst = rec + (s >> 1) * 1024 + (oct * 16 + mr) * 16 + (s & 1) * 8;
     *reinterpret_cast<uint2*>(dst) = make_uint2(q[0], q[1]);
-    *reinterpret_cast<uint2*>(dst + 128) = make_uint2(q[2], q[3]);
+    *reinterpret_cast<uint2*>(dst + 256) = make_uint2(q[2], q[3]);
 }
 
 } // namespace
