@@ -256,19 +256,103 @@ __device__ __forceinline__ void load_wpanel(WPanel<QT>& p, const uint8_t* __rest
         p.q[c] = __builtin_nontemporal_load(b + (size_t)(1 + c) * slots + ln);
 }
 
+// The Q4_K arithmetic of one panel against one 16-row tile of activations, shared by the LDS forms
+// and the register-direct form.  `a_of(u, b)` returns the tile's two matrix-core operands of unit u,
+// sub-block pair b (16 bytes per lane), `side_of(u, bs_lo, bs_hi, dx)` the unit's sub-block sum planes
+// (k slots of the first 16-lane row only) and this lane group's four row scales.
+// NU: the number of the panel's units that exist as a compile-time constant - straight-line code, in
+// which the LDS reads, the matrix instructions and the integer scale multiply-adds of different units
+// interleave (a wave that is alone on its SIMD has nothing else to hide their latencies) - or 0:
+// `n_units` (uniform) at run time, with a branch around every unit.
+// FIRST: the quants are still in load layout and are transposed pair by pair, in load order.
+template <bool FIRST, int NU, class AFetch, class SFetch>
+__device__ __forceinline__ void q4k_panel_dot(WPanel<QMM_Q4_K>& p, int n_units, AFetch&& a_of, SFetch&& side_of,
+                                              float (&acc)[4]) {
+    const int nu = NU ? NU : n_units;
+    // 6-bit scales of the four units (byte i of sc_lo / sc_hi = scale i / i + 4); the mins are only
+    // needed at the end and are unpacked there
+    uint32_t sc_lo[4], sc_hi[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        sc_lo[u] = p.hdr[u].y & 0x3f3f3f3fu;
+        sc_hi[u] = (p.hdr[u].w & 0x0f0f0f0fu) | (((p.hdr[u].y >> 6) & 0x03030303u) << 4);
+    }
+    int isum[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) isum[u][r] = 0;
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        if (FIRST) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            // two units at a time: their four matrix instructions are issued back to back and the
+            // results consumed afterwards (the matrix pipe's latency is paid once)
+            const u32x4 qq = p.q[2 * b + h];
+            i32x4 dlo[2], dhi[2];
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int u = 2 * h + e;
+                if (u >= nu) continue; // compile-time, or uniform
+                const uint32_t w0 = e ? qq.z : qq.x, w1 = e ? qq.w : qq.y;
+                const i64x2 aa = a_of(u, b);
+                dlo[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(aa.x, pack64(w0 & kNib, w1 & kNib), i32x4{0, 0, 0, 0}, 0, 0, 0);
+                dhi[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(aa.y, pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib),
+                                                               i32x4{0, 0, 0, 0}, 0, 0, 0);
+            }
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int u = 2 * h + e;
+                if (u >= nu) continue;
+                const int sc0 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b);
+                const int sc1 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b + 1);
+#pragma unroll
+                for (int r = 0; r < 4; r++) // |dot| < 2^17, scale < 64
+                    isum[u][r] = __mul24(sc1, dhi[e][r]) + (__mul24(sc0, dlo[e][r]) + isum[u][r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        if (u >= nu) continue;
+        const float d = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x & 0xffffu));
+        const float dmin = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x >> 16));
+        const uint32_t mn_lo = p.hdr[u].z & 0x3f3f3f3fu;
+        const uint32_t mn_hi = ((p.hdr[u].w >> 4) & 0x0f0f0f0fu) | (((p.hdr[u].z >> 6) & 0x03030303u) << 4);
+        // min term: sum_s min_s * bsum_s as two matrix instructions over k = sub-block index; only
+        // the first 16-lane row carries data (k slots 0..7), the rest multiply zeros
+        long bs_lo, bs_hi;
+        float4 dx;
+        side_of(u, bs_lo, bs_hi, dx);
+        const long bmn = pack64(mn_lo, mn_hi);
+        const i32x4 m_lo = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_lo, bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
+        const i32x4 m_hi = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_hi, bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
+        const float dxs[4] = {dx.x, dx.y, dx.z, dx.w};
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            // (d isum - dmin msum) dx: both integers are exact in f32 (|isum| < 2^26 only in theory:
+            // 2^24 needs every product of a block at its extreme), two roundings per unit
+            const int msum = m_lo[r] + (m_hi[r] << 7);
+            acc[r] = fmaf(fmaf(-dmin, (float)msum, d * (float)isum[u][r]), dxs[r], acc[r]);
+        }
+    }
+}
+
+
 // acc[r] += block dots of the panel's units against activation rows 4 grp + r of
 // the tile whose unit records start at `xu0` (LDS, record of the panel's unit 0).
 // FIRST: the quants are still in load layout and are transposed pair by pair, in
 // load order.  `n_units` (uniform) is the number of the panel's units that exist.
-template <int QT, bool FIRST>
+template <int QT, bool FIRST, int NU = 0>
 __device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int n_units, int j, int grp,
                                           float (&acc)[4]) {
     constexpr int UB = Unit<QT>::kBytes;
     const int lane16 = (grp * 16 + j) * 16; // this lane's 16 bytes of a sub-block pair
-    // Units of the panel that do not exist (ragged k, S < 4) are not skipped, which
-    // would split the arithmetic into many small blocks: they read unit 0's
-    // activations and their weight scale is multiplied by zero.  (Their header is
-    // zero padding or a copy of unit 0's, so every factor is finite.)
+    // Q8_0 / Q6_K: units of the panel that do not exist (ragged k, S < 4) get unit 0's
+    // activations as their address and a weight scale multiplied by zero wherever the
+    // compiler keeps their arithmetic.  (Their header is zero padding or a copy of unit
+    // 0's, so every factor is finite.)
     int xo[4];
     float ef[4];
 #pragma unroll
@@ -277,78 +361,19 @@ __device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int
         xo[u] = exists ? u * UB : 0;
         ef[u] = exists ? 1.0f : 0.0f;
     }
-    if (QT == QMM_Q4_K) {
-        // 6-bit scales of the four units (byte i of sc_lo / sc_hi = scale i / i + 4); the
-        // mins are only needed at the end and are unpacked there
-        uint32_t sc_lo[4], sc_hi[4];
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            sc_lo[u] = p.hdr[u].y & 0x3f3f3f3fu;
-            sc_hi[u] = (p.hdr[u].w & 0x0f0f0f0fu) | (((p.hdr[u].y >> 6) & 0x03030303u) << 4);
-        }
-        int isum[4][4];
-#pragma unroll
-        for (int u = 0; u < 4; u++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) isum[u][r] = 0;
-#pragma unroll
-        for (int b = 0; b < 4; b++) {
-            if (FIRST) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
-#pragma unroll
-            for (int h = 0; h < 2; h++) {
-                // two units at a time: their four MFMAs are issued back to back and the
-                // results consumed afterwards (the matrix pipe's latency is paid once)
-                const u32x4 qq = p.q[2 * b + h];
-                i32x4 dlo[2], dhi[2];
-#pragma unroll
-                for (int e = 0; e < 2; e++) {
-                    const int u = 2 * h + e;
-                    if (u >= n_units) continue; // uniform
-                    const uint32_t w0 = e ? qq.z : qq.x, w1 = e ? qq.w : qq.y;
-                    const i64x2 aa = *reinterpret_cast<const i64x2*>(xu0 + xo[u] + lane16 + b * 1024);
-                    const long a_lo = aa.x, a_hi = aa.y;
-                    dlo[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, pack64(w0 & kNib, w1 & kNib),
-                                                                   i32x4{0, 0, 0, 0}, 0, 0, 0);
-                    dhi[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(
-                        a_hi, pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib), i32x4{0, 0, 0, 0}, 0, 0, 0);
-                }
-#pragma unroll
-                for (int e = 0; e < 2; e++) {
-                    const int u = 2 * h + e;
-                    if (u >= n_units) continue;
-                    const int sc0 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b);
-                    const int sc1 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b + 1);
-#pragma unroll
-                    for (int r = 0; r < 4; r++) // |dot| < 2^17, scale < 64
-                        isum[u][r] += __mul24(sc0, dlo[e][r]) + __mul24(sc1, dhi[e][r]);
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            if (u >= n_units) continue;
-            const float d = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x & 0xffffu)) * ef[u];
-            const float dmin = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x >> 16)) * ef[u];
-            const uint32_t mn_lo = p.hdr[u].z & 0x3f3f3f3fu;
-            const uint32_t mn_hi = ((p.hdr[u].w >> 4) & 0x0f0f0f0fu) | (((p.hdr[u].z >> 6) & 0x03030303u) << 4);
-            // min term: sum_s min_s * bsum_s as two MFMAs over k = sub-block index; only
-            // the first 16-lane row carries data (k slots 0..7), the rest multiply zeros
-            const uint8_t* side = xu0 + xo[u] + Unit<QT>::kQuant;
-            const uint8_t* planes = side + 64 + j * 16;
-            const long bs_lo = grp == 0 ? *reinterpret_cast<const long*>(planes) : 0L;
-            const long bs_hi = grp == 0 ? *reinterpret_cast<const long*>(planes + 8) : 0L;
-            const long bmn = pack64(mn_lo, mn_hi);
-            const i32x4 m_lo = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_lo, bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
-            const i32x4 m_hi = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_hi, bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
-            const float4 dx = *reinterpret_cast<const float4*>(side + grp * 16);
-            const float dxs[4] = {dx.x, dx.y, dx.z, dx.w};
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int msum = m_lo[r] + (m_hi[r] << 7);
-                acc[r] += (d * dxs[r]) * (float)isum[u][r] - (dmin * dxs[r]) * (float)msum;
-            }
-        }
-    } else if (QT == QMM_Q6_K) {
+    if constexpr (QT == QMM_Q4_K) {
+        q4k_panel_dot<FIRST, NU>(
+            p, n_units,
+            [&](int u, int b) { return *reinterpret_cast<const i64x2*>(xu0 + u * UB + lane16 + b * 1024); },
+            [&](int u, long& bs_lo, long& bs_hi, float4& dx) {
+                const uint8_t* side = xu0 + u * UB + Unit<QT>::kQuant;
+                const i64x2 planes = *reinterpret_cast<const i64x2*>(side + 64 + j * 16);
+                bs_lo = grp == 0 ? planes.x : 0L;
+                bs_hi = grp == 0 ? planes.y : 0L;
+                dx = *reinterpret_cast<const float4*>(side + grp * 16);
+            },
+            acc);
+    } else if constexpr (QT == QMM_Q6_K) {
         // Sub-block t = 4 h + g of a unit (32 elements) is nibble g / 2 of the nibble chunk pair
         // 2 h + g % 2 with bit pair g of the bit-pair chunk pair h; each of its two 16-element
         // groups has its own signed scale, and the matrix instruction sums 32: it runs twice, once
@@ -468,8 +493,10 @@ __device__ __forceinline__ void issue_window_copy(const uint8_t* __restrict__ sr
 // GROUPED: blockIdx.y is an expert; its weights are matrix blockIdx.y of the
 // stack, its rows the expert's tiles of sorted pairs, output row = pair index.
 // EP: the sums go through the epilogue of P.ep (residual add, f32 or bf16 store).
-template <int QT, bool SINGLE, bool GROUPED = false, bool EP = false>
-__global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaParams P) {
+// (the compact single-stage Q4_K form is held to the 80 registers of six waves per SIMD: two 12-wave
+// workgroups per CU keep every panel of gate | up in flight at once)
+template <int QT, bool SINGLE, bool GROUPED = false, bool EP = false, int NU = 0>
+__global__ __launch_bounds__(64 * kMaxWaves, (QT == QMM_Q4_K && SINGLE && NU == 0) ? 6 : 3) void gemv_mfma_oneshot_kernel(MfmaParams P) {
     constexpr int UB = Unit<QT>::kBytes;
     constexpr int NL = WPanel<QT>::kLoads; // loads of one panel
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -552,7 +579,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
         if (SINGLE || (unit0 >= wu0 && unit0 < wu0 + wn)) {
             const uint8_t* xu0 = cur + (size_t)(unit0 - wu0) * UB;
             if (SINGLE) {
-                panel_dot<QT, true>(p, xu0, n_units, j, grp, acc);
+                panel_dot<QT, true, NU>(p, xu0, n_units, j, grp, acc);
             } else {
                 // several stages reuse the panel: transpose it once, up front (one copy of
                 // the arithmetic in the code keeps the register count down)
@@ -618,68 +645,16 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_oneshot_kernel(MfmaP
 // units' side information) straight into registers, ahead of the panel: no LDS, no barrier
 // before the arithmetic, and k of any length (the LDS forms need several windows from 32
 // units on).  Returns acc[r] for activation rows 4 grp + r.
-__device__ __forceinline__ void panel_dot_direct_q4k(WPanel<QMM_Q4_K>& p, const long (&a)[4][8],
+template <int NU>
+__device__ __forceinline__ void panel_dot_direct_q4k(WPanel<QMM_Q4_K>& p, const i64x2 (&a)[4][4],
                                                      const long (&bs_lo)[4], const long (&bs_hi)[4],
                                                      const float4 (&dx)[4], int n_units, float (&acc)[4]) {
-    uint32_t sc_lo[4], sc_hi[4];
-#pragma unroll
-    for (int u = 0; u < 4; u++) {
-        sc_lo[u] = p.hdr[u].y & 0x3f3f3f3fu;
-        sc_hi[u] = (p.hdr[u].w & 0x0f0f0f0fu) | (((p.hdr[u].y >> 6) & 0x03030303u) << 4);
-    }
-    int isum[4][4];
-#pragma unroll
-    for (int u = 0; u < 4; u++)
-#pragma unroll
-        for (int r = 0; r < 4; r++) isum[u][r] = 0;
-#pragma unroll
-    for (int b = 0; b < 4; b++) {
-        transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const u32x4 qq = p.q[2 * b + h];
-            i32x4 dlo[2], dhi[2];
-#pragma unroll
-            for (int e = 0; e < 2; e++) {
-                const int u = 2 * h + e;
-                if (u >= n_units) continue; // uniform
-                const uint32_t w0 = e ? qq.z : qq.x, w1 = e ? qq.w : qq.y;
-                dlo[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[u][2 * b], pack64(w0 & kNib, w1 & kNib),
-                                                               i32x4{0, 0, 0, 0}, 0, 0, 0);
-                dhi[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[u][2 * b + 1], pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib),
-                                                               i32x4{0, 0, 0, 0}, 0, 0, 0);
-            }
-#pragma unroll
-            for (int e = 0; e < 2; e++) {
-                const int u = 2 * h + e;
-                if (u >= n_units) continue;
-                const int sc0 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b);
-                const int sc1 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b + 1);
-#pragma unroll
-                for (int r = 0; r < 4; r++) isum[u][r] += __mul24(sc0, dlo[e][r]) + __mul24(sc1, dhi[e][r]);
-            }
-        }
-    }
-#pragma unroll
-    for (int u = 0; u < 4; u++) {
-        if (u >= n_units) continue;
-        const float d = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x & 0xffffu));
-        const float dmin = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x >> 16));
-        const uint32_t mn_lo = p.hdr[u].z & 0x3f3f3f3fu;
-        const uint32_t mn_hi = ((p.hdr[u].w >> 4) & 0x0f0f0f0fu) | (((p.hdr[u].z >> 6) & 0x03030303u) << 4);
-        const long bmn = pack64(mn_lo, mn_hi);
-        const i32x4 m_lo = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_lo[u], bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
-        const i32x4 m_hi = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_hi[u], bmn, i32x4{0, 0, 0, 0}, 0, 0, 0);
-        const float dxs[4] = {dx[u].x, dx[u].y, dx[u].z, dx[u].w};
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int msum = m_lo[r] + (m_hi[r] << 7);
-            acc[r] += (d * dxs[r]) * (float)isum[u][r] - (dmin * dxs[r]) * (float)msum;
-        }
-    }
+    q4k_panel_dot<true, NU>(
+        p, n_units, [&](int u, int b) { return a[u][b]; },
+        [&](int u, long& lo, long& hi, float4& d4) { lo = bs_lo[u], hi = bs_hi[u], d4 = dx[u]; }, acc);
 }
 
-template <bool EP = false>
+template <bool EP = false, int NU = 0>
 __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(MfmaParams P) {
     constexpr int QT = QMM_Q4_K;
     constexpr int UB = Unit<QT>::kBytes;
@@ -711,16 +686,14 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(Mf
     const int row = rt * 16 + j;
 
     // the activations first (they come from the L2 and return first), then the panel
-    long a[4][8], bs_lo[4], bs_hi[4];
+    i64x2 a[4][4];
+    long bs_lo[4], bs_hi[4];
     float4 dx[4];
 #pragma unroll
     for (int u = 0; u < 4; u++) {
         const uint8_t* rec = P.ws + (size_t)(unit0 + (u < n_units ? u : 0)) * UB; // missing units re-read unit 0
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
-            const i64x2 aa = *reinterpret_cast<const i64x2*>(rec + b * 1024 + lane * 16);
-            a[u][2 * b] = aa.x, a[u][2 * b + 1] = aa.y;
-        }
+        for (int b = 0; b < 4; b++) a[u][b] = *reinterpret_cast<const i64x2*>(rec + b * 1024 + lane * 16);
         const uint8_t* side = rec + Unit<QT>::kQuant;
         // the sub-block sums occupy k slots 0..7 of the min-term MFMA: the first 16-lane row only
         const i64x2 planes = *reinterpret_cast<const i64x2*>(side + 64 + j * 16);
@@ -732,7 +705,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(Mf
     load_wpanel<QT>(p, wbase + (int64_t)((rt_ok ? rt : 0) * P.k_groups + wk) * P.panel_bytes, P.slots, lane, j);
 
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    panel_dot_direct_q4k(p, a, bs_lo, bs_hi, dx, n_units, acc);
+    panel_dot_direct_q4k<NU>(p, a, bs_lo, bs_hi, dx, n_units, acc);
 
     // combine the waves that split k, write y[4 grp + r][rt * 16 + j]
     if (P.nwk == 1) {
@@ -768,11 +741,13 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(Mf
 // and 11.9 against 12.7 us for the q|k|v group).  IZWI_QMM_MFMA_DIRECT=0 keeps the LDS forms
 // (tuning aid).
 bool direct_form_applies(int dtype, int n_tiles, int nwr, bool one_window) {
-    static const bool enabled = [] {
+    static const int mode = [] {
         const char* e = getenv("IZWI_QMM_MFMA_DIRECT");
-        return !(e && e[0] == '0');
+        return e && e[0] >= '0' && e[0] <= '2' ? e[0] - '0' : 1;
     }();
-    return enabled && dtype == QMM_Q4_K && n_tiles == 1 && nwr == 1 && !one_window;
+    if (mode == 0 || dtype != QMM_Q4_K || n_tiles != 1) return false;
+    if (mode == 2) return true; // every single-tile Q4_K call (tuning aid: measured slower where one window covers k)
+    return nwr == 1 && !one_window;
 }
 
 // Streaming form: wave `wave` of workgroup b owns row-tiles (b * waves + wave),
@@ -925,6 +900,18 @@ hipError_t launch_dense_form(int form, const MfmaParams& P, unsigned grid, int w
 }
 } // namespace
 
+namespace {
+// every panel of the matrix holds four units: the kernels' straight-line Q4_K arithmetic applies
+bool full_panels(const QmmLayout& L) { return L.s == 4 && L.k_units % 4 == 0; }
+
+// The straight-line arithmetic needs the registers of three waves per SIMD; a launch whose waves do
+// not all fit the chip at once at that occupancy (gate | up at the 8B shapes: six per SIMD) keeps
+// the compact form with a branch per unit, whose 80 registers let all of them be resident.
+bool straight_line_fits(int64_t groups, int waves, int n_cus) {
+    return groups * waves <= (int64_t)n_cus * kMaxWaves;
+}
+} // namespace
+
 hipError_t qmm_launch_quantize_ws(int dtype, const float* x, int64_t m, int64_t k, void* workspace,
                                   hipStream_t stream, bool x_bf16) {
     if (m <= 0 || k <= 0 || m > 0x3fffffff || k > 0x3fffffff) return hipErrorInvalidValue;
@@ -1039,13 +1026,30 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     }
     P.wave_magic = (65536 + P.nwk - 1) / P.nwk;
     if (oneshot && direct_form_applies(L.dtype, n_tiles, P.nwr, L.k_units <= P.window_units)) {
-        if (epilogue) gemv_mfma_direct_q4k_kernel<true><<<grid, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
-        else gemv_mfma_direct_q4k_kernel<false><<<grid, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
+        const size_t red = (size_t)waves * 256 * 4;
+        if (full_panels(L)) {
+            if (epilogue) gemv_mfma_direct_q4k_kernel<true, 4><<<grid, 64 * waves, red, stream>>>(P);
+            else gemv_mfma_direct_q4k_kernel<false, 4><<<grid, 64 * waves, red, stream>>>(P);
+        } else {
+            if (epilogue) gemv_mfma_direct_q4k_kernel<true><<<grid, 64 * waves, red, stream>>>(P);
+            else gemv_mfma_direct_q4k_kernel<false><<<grid, 64 * waves, red, stream>>>(P);
+        }
         return hipGetLastError();
     }
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     const bool single = n_tiles == 1 && L.k_units <= P.window_units;
     const int form = oneshot ? (single ? 0 : 1) : 2;
+    if (L.dtype == QMM_Q4_K && form == 0 && full_panels(L) && straight_line_fits(P.rt_groups, waves, n_cus)) {
+        const void* fn = epilogue ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, true, 4>)
+                                  : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4>);
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return e;
+        }
+        if (epilogue) gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, true, 4><<<grid, 64 * waves, lds, stream>>>(P);
+        else gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4><<<grid, 64 * waves, lds, stream>>>(P);
+        return hipGetLastError();
+    }
     if (L.dtype == QMM_Q4_K)
         return epilogue ? launch_dense_form<QMM_Q4_K, true>(form, P, grid, waves, lds, stream)
                         : launch_dense_form<QMM_Q4_K, false>(form, P, grid, waves, lds, stream);
@@ -1235,19 +1239,24 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
     P.rt_groups = (int)groups;
     const int waves = P.nwk * P.nwr;
     if (direct_form_applies(L0.dtype, 1, P.nwr, true)) {
-        gemv_mfma_direct_q4k_kernel<false><<<(unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
+        if (full_panels(L0)) gemv_mfma_direct_q4k_kernel<false, 4><<<(unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
+        else gemv_mfma_direct_q4k_kernel<false><<<(unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
         return hipGetLastError();
     }
     const size_t lds = std::max((size_t)P.window_units * unit_bytes(L0.dtype), (size_t)waves * 256 * 4);
     if (lds > 160 * 1024) return hipErrorNotSupported;
-    const void* fn = L0.dtype == QMM_Q4_K   ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true>)
+    const bool full = L0.dtype == QMM_Q4_K && full_panels(L0) && straight_line_fits(groups, waves, n_cus);
+    const void* fn = full                   ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4>)
+                     : L0.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true>)
                      : L0.dtype == QMM_Q6_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q6_K, true>)
                                             : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, true>);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
-    if (L0.dtype == QMM_Q4_K)
+    if (full)
+        gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4><<<(unsigned)groups, 64 * waves, lds, stream>>>(P);
+    else if (L0.dtype == QMM_Q4_K)
         gemv_mfma_oneshot_kernel<QMM_Q4_K, true><<<(unsigned)groups, 64 * waves, lds, stream>>>(P);
     else if (L0.dtype == QMM_Q6_K)
         gemv_mfma_oneshot_kernel<QMM_Q6_K, true><<<(unsigned)groups, 64 * waves, lds, stream>>>(P);
