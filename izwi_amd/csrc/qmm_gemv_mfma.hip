@@ -182,7 +182,9 @@ struct MfmaParams {
     int n_tiles;
     int window_units; // multiple of s, <= kWindowUnits
     int rt_groups;
-    // expert-grouped form: blockIdx.y is the expert
+    // expert-grouped form: a one-dimensional grid; a workgroup's (expert, stack, row-tile group)
+    // is decoded so that all workgroups of an expert run on one XCD (see the kernel)
+    int n_experts, stacks;
     const int32_t* perm;
     const int32_t* offsets;      // sorted pairs of expert e: [offsets[e], offsets[e + 1])
     const int32_t* tile_offsets; // its 16-row tiles (records): [tile_offsets[e], tile_offsets[e + 1])
@@ -340,6 +342,81 @@ __device__ __forceinline__ void q4k_panel_dot(WPanel<QMM_Q4_K>& p, int n_units, 
 }
 
 
+// A Q4_K panel prepared for several tiles of activations (the multi-stage forms: a batch of more
+// than 16 rows, an expert's tiles): what does not depend on the activations is done once per panel
+// instead of once per (panel, tile) - the nibbles split into the two matrix-core operands of every
+// (unit, sub-block pair), the 6-bit scales and mins unpacked, d and dmin converted.  Twice the
+// registers of the packed quants, so the units are walked one after the other (four running sums
+// instead of sixteen).  Same integers and the same f32 operations as q4k_panel_dot: same bits.
+template <int NU>
+struct Q4Prepared {
+    long lo[NU][4], hi[NU][4]; // [unit][pair]: quants of sub-block 2b / 2b + 1, this lane's octet
+    uint32_t sc_lo[NU], sc_hi[NU];
+    long bmn[NU];
+    float d[NU], dmin[NU];
+};
+
+// `p` transposed already (transpose_pair on every chunk pair).
+template <int NU>
+__device__ __forceinline__ void q4k_prepare(const WPanel<QMM_Q4_K>& p, Q4Prepared<NU>& t) {
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const u32x4 qq = p.q[2 * b + (u >> 1)];
+            const uint32_t w0 = (u & 1) ? qq.z : qq.x, w1 = (u & 1) ? qq.w : qq.y;
+            t.lo[u][b] = pack64(w0 & kNib, w1 & kNib);
+            t.hi[u][b] = pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib);
+        }
+        t.sc_lo[u] = p.hdr[u].y & 0x3f3f3f3fu;
+        t.sc_hi[u] = (p.hdr[u].w & 0x0f0f0f0fu) | (((p.hdr[u].y >> 6) & 0x03030303u) << 4);
+        const uint32_t mn_lo = p.hdr[u].z & 0x3f3f3f3fu;
+        const uint32_t mn_hi = ((p.hdr[u].w >> 4) & 0x0f0f0f0fu) | (((p.hdr[u].z >> 6) & 0x03030303u) << 4);
+        t.bmn[u] = pack64(mn_lo, mn_hi);
+        t.d[u] = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x & 0xffffu));
+        t.dmin[u] = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x >> 16));
+    }
+}
+
+template <int NU, class AFetch, class SFetch>
+__device__ __forceinline__ void q4k_tile_dot(const Q4Prepared<NU>& t, AFetch&& a_of, SFetch&& side_of, float (&acc)[4]) {
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+        int isum[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int b2 = 0; b2 < 2; b2++) {
+            i32x4 dlo[2], dhi[2];
+#pragma unroll
+            for (int bb = 0; bb < 2; bb++) {
+                const int b = 2 * b2 + bb;
+                const i64x2 aa = a_of(u, b);
+                dlo[bb] = __builtin_amdgcn_mfma_i32_16x16x32_i8(aa.x, t.lo[u][b], i32x4{0, 0, 0, 0}, 0, 0, 0);
+                dhi[bb] = __builtin_amdgcn_mfma_i32_16x16x32_i8(aa.y, t.hi[u][b], i32x4{0, 0, 0, 0}, 0, 0, 0);
+            }
+#pragma unroll
+            for (int bb = 0; bb < 2; bb++) {
+                const int b = 2 * b2 + bb;
+                const int sc0 = (int)qmm_byte_of(t.sc_lo[u], t.sc_hi[u], 2 * b);
+                const int sc1 = (int)qmm_byte_of(t.sc_lo[u], t.sc_hi[u], 2 * b + 1);
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    isum[r] = __mul24(sc1, dhi[bb][r]) + (__mul24(sc0, dlo[bb][r]) + isum[r]);
+            }
+        }
+        long bs_lo, bs_hi;
+        float4 dx;
+        side_of(u, bs_lo, bs_hi, dx);
+        const i32x4 m_lo = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_lo, t.bmn[u], i32x4{0, 0, 0, 0}, 0, 0, 0);
+        const i32x4 m_hi = __builtin_amdgcn_mfma_i32_16x16x32_i8(bs_hi, t.bmn[u], i32x4{0, 0, 0, 0}, 0, 0, 0);
+        const float dxs[4] = {dx.x, dx.y, dx.z, dx.w};
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int msum = m_lo[r] + (m_hi[r] << 7);
+            acc[r] = fmaf(fmaf(-t.dmin[u], (float)msum, t.d[u] * (float)isum[r]), dxs[r], acc[r]);
+        }
+    }
+}
+
 // acc[r] += block dots of the panel's units against activation rows 4 grp + r of
 // the tile whose unit records start at `xu0` (LDS, record of the panel's unit 0).
 // FIRST: the quants are still in load layout and are transposed pair by pair, in
@@ -490,7 +567,7 @@ __device__ __forceinline__ void issue_window_copy(const uint8_t* __restrict__ sr
 
 // One-shot form: wave (wr, wk) owns panel wk of row-tile blockIdx.x * nwr + wr.
 // SINGLE: one tile of rows and one activation window, i.e. straight-line code.
-// GROUPED: blockIdx.y is an expert; its weights are matrix blockIdx.y of the
+// GROUPED: the workgroup belongs to an expert; its weights are that matrix of the
 // stack, its rows the expert's tiles of sorted pairs, output row = pair index.
 // EP: the sums go through the epilogue of P.ep (residual add, f32 or bf16 store).
 // (the compact single-stage Q4_K form is held to the 80 registers of six waves per SIMD: two 12-wave
@@ -516,6 +593,20 @@ __global__ __launch_bounds__(64 * kMaxWaves, (QT == QMM_Q4_K && SINGLE && NU == 
     const uint8_t* wbase = P.w;
     float* yout = P.y;
     int n_rows = P.n, row_tiles = P.row_tiles, rtg = blockIdx.x;
+    // GROUPED: workgroups go to the eight XCDs round-robin by their linear index, and every XCD has
+    // its own L2: index = 8 * slot + (expert % 8), so the 2 * rt_groups workgroups of an expert share
+    // one L2 and all but the first find the expert's activation records there (measured neutral at
+    // T = 512: the records' first touch is not what a workgroup waits for longest).
+    int g_expert = 0, g_stack = 0;
+    if (GROUPED) {
+        const int per_expert = P.rt_groups * P.stacks;
+        const int slot = blockIdx.x >> 3;
+        const int e_hi = slot / per_expert, within = slot - e_hi * per_expert;
+        g_expert = e_hi * 8 + (int)(blockIdx.x & 7);
+        if (g_expert >= P.n_experts) return; // uniform for the workgroup
+        g_stack = within / P.rt_groups;
+        rtg = within - g_stack * P.rt_groups;
+    }
     if (SINGLE && !GROUPED && P.n_weights > 1) {
         int i = 0;
         while (i + 1 < P.n_weights && (int)blockIdx.x >= P.rtg_end[i]) i++;
@@ -534,8 +625,8 @@ __global__ __launch_bounds__(64 * kMaxWaves, (QT == QMM_Q4_K && SINGLE && NU == 
     const uint8_t* records = P.ws;
     int n_tiles = P.n_tiles, pos_begin = 0, pos_end = 0;
     if (GROUPED) {
-        const int e = blockIdx.y;
-        if (blockIdx.z != 0) wbase = P.w2, yout = P.y2; // second weight stack on the same activations
+        const int e = g_expert;
+        if (g_stack != 0) wbase = P.w2, yout = P.y2; // second weight stack on the same activations
         const int tile_begin = P.tile_offsets[e];
         n_tiles = P.tile_offsets[e + 1] - tile_begin;
         if (n_tiles == 0) return; // uniform for the workgroup: nobody reaches a barrier
@@ -556,6 +647,15 @@ __global__ __launch_bounds__(64 * kMaxWaves, (QT == QMM_Q4_K && SINGLE && NU == 
     load_wpanel<QT>(p, wbase + (int64_t)((rt_ok ? rt : 0) * P.k_groups + wk) * P.panel_bytes, P.slots, lane, j);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory"); // the window has landed, the panel may still fly
     lds_barrier();
+
+    // several stages reuse the panel: its activation-independent part once, up front
+    constexpr bool PREP = QT == QMM_Q4_K && !SINGLE && NU > 0;
+    Q4Prepared<PREP ? NU : 1> prep;
+    if constexpr (PREP) {
+#pragma unroll
+        for (int b = 0; b < WPanel<QT>::QC / 2; b++) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
+        q4k_prepare<NU>(p, prep);
+    }
 
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     // (row tile, window) stages in order; with two LDS buffers the next stage's window is
@@ -578,8 +678,20 @@ __global__ __launch_bounds__(64 * kMaxWaves, (QT == QMM_Q4_K && SINGLE && NU == 
             issue_window_copy<QT>(next_src, lds_x + ((s + 1) & 1) * buf_bytes, next_n, wave, waves, lane);
         if (SINGLE || (unit0 >= wu0 && unit0 < wu0 + wn)) {
             const uint8_t* xu0 = cur + (size_t)(unit0 - wu0) * UB;
-            if (SINGLE) {
+            if constexpr (SINGLE) {
                 panel_dot<QT, true, NU>(p, xu0, n_units, j, grp, acc);
+            } else if constexpr (PREP) {
+                const int lane16 = lane * 16;
+                q4k_tile_dot<NU>(
+                    prep, [&](int u, int b) { return *reinterpret_cast<const i64x2*>(xu0 + u * UB + lane16 + b * 1024); },
+                    [&](int u, long& bs_lo, long& bs_hi, float4& dx) {
+                        const uint8_t* side = xu0 + u * UB + Unit<QT>::kQuant;
+                        const i64x2 planes = *reinterpret_cast<const i64x2*>(side + 64 + j * 16);
+                        bs_lo = grp == 0 ? planes.x : 0L;
+                        bs_hi = grp == 0 ? planes.y : 0L;
+                        dx = *reinterpret_cast<const float4*>(side + grp * 16);
+                    },
+                    acc);
             } else {
                 // several stages reuse the panel: transpose it once, up front (one copy of
                 // the arithmetic in the code keeps the register count down)
@@ -903,6 +1015,8 @@ hipError_t launch_dense_form(int form, const MfmaParams& P, unsigned grid, int w
 namespace {
 // every panel of the matrix holds four units: the kernels' straight-line Q4_K arithmetic applies
 bool full_panels(const QmmLayout& L) { return L.s == 4 && L.k_units % 4 == 0; }
+// the units of every panel when all panels hold the same number (3: k = 768), else 0
+int uniform_panel_units(const QmmLayout& L) { return L.k_units % L.s == 0 ? L.s : 0; }
 
 // The straight-line arithmetic needs the registers of three waves per SIMD; a launch whose waves do
 // not all fit the chip at once at that occupancy (gate | up at the 8B shapes: six per SIMD) keeps
@@ -987,6 +1101,8 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     P.perm = nullptr;
     P.offsets = nullptr;
     P.tile_offsets = nullptr;
+    P.n_experts = 0;
+    P.stacks = 1;
     P.matrix_bytes = 0;
     P.w2 = nullptr;
     P.y2 = nullptr;
@@ -1153,13 +1269,14 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     }
     const int waves = P.nwk * P.nwr;
     const size_t window_bytes = (size_t)P.window_units * unit_bytes(L.dtype);
-    // A second window buffer hides the next tile's copy, but a workgroup of an expert is a short
-    // chain of dependent round trips and only a second workgroup on the CU fills its gaps: two
-    // buffers only where two workgroups still fit (IZWI_QMM_MOE_DOUBLE_BUF=1 / 0 forces the choice)
+    // A second window buffer hides the next tile's copy under this tile's arithmetic.  The kernel's
+    // registers (135 - 167) admit one 12-wave workgroup per CU whatever its LDS, so the buffer is free
+    // where it fits (T = 512, 128 experts: 248 -> 241 us per layer; smaller workgroups, two or three per
+    // CU, were measured slower: 275 - 290 us - a workgroup's time is mostly the latency of its chain of
+    // round trips, which halving its work does not shorten).  IZWI_QMM_MOE_DOUBLE_BUF=1 / 0 forces the choice.
     static const int force_double = [] { const char* e = getenv("IZWI_QMM_MOE_DOUBLE_BUF"); return e ? atoi(e) : -1; }();
     const size_t red_bytes = (size_t)waves * 256 * 4;
-    P.double_buf = force_double >= 0 ? (force_double && 2 * window_bytes + red_bytes <= 160 * 1024)
-                                     : 2 * (2 * window_bytes + red_bytes) <= 160 * 1024;
+    P.double_buf = (force_double != 0) && 2 * window_bytes + red_bytes <= 160 * 1024;
     const size_t lds = (P.double_buf ? 2 : 1) * window_bytes + red_bytes;
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     const void* fn = L.dtype == QMM_Q4_K
@@ -1171,7 +1288,21 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
-    const dim3 grid((unsigned)P.rt_groups, (unsigned)n_experts, tiled2 ? 2u : 1u);
+    P.n_experts = n_experts;
+    P.stacks = tiled2 ? 2 : 1;
+    const unsigned grid = (unsigned)(((n_experts + 7) / 8) * 8 * P.rt_groups * P.stacks);
+    const int nu = L.dtype == QMM_Q4_K ? uniform_panel_units(L) : 0;
+    if (nu == 4 || nu == 3) {
+        const void* fp = nu == 4 ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true, false, 4>)
+                                 : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true, false, 3>);
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(fp, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return e;
+        }
+        if (nu == 4) gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true, false, 4><<<grid, 64 * waves, lds, stream>>>(P);
+        else gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true, false, 3><<<grid, 64 * waves, lds, stream>>>(P);
+        return hipGetLastError();
+    }
     if (L.dtype == QMM_Q4_K)
         gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true><<<grid, 64 * waves, lds, stream>>>(P);
     else if (L.dtype == QMM_Q6_K)
@@ -1210,6 +1341,8 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
     P.perm = nullptr;
     P.offsets = nullptr;
     P.tile_offsets = nullptr;
+    P.n_experts = 0;
+    P.stacks = 1;
     P.matrix_bytes = 0;
     P.w2 = nullptr;
     P.y2 = nullptr;
