@@ -1166,6 +1166,18 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
         else gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4><<<grid, 64 * waves, lds, stream>>>(P);
         return hipGetLastError();
     }
+    if (L.dtype == QMM_Q4_K && form == 1 && full_panels(L)) {
+        // several tiles of rows against a resident panel: its activation-independent part once
+        const void* fn = epilogue ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false, false, true, 4>)
+                                  : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false, false, false, 4>);
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return e;
+        }
+        if (epilogue) gemv_mfma_oneshot_kernel<QMM_Q4_K, false, false, true, 4><<<grid, 64 * waves, lds, stream>>>(P);
+        else gemv_mfma_oneshot_kernel<QMM_Q4_K, false, false, false, 4><<<grid, 64 * waves, lds, stream>>>(P);
+        return hipGetLastError();
+    }
     if (L.dtype == QMM_Q4_K)
         return epilogue ? launch_dense_form<QMM_Q4_K, true>(form, P, grid, waves, lds, stream)
                         : launch_dense_form<QMM_Q4_K, false>(form, P, grid, waves, lds, stream);
