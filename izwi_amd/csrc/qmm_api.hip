@@ -440,15 +440,15 @@ int qmm_current_device(int* device, int* n_cus) {
 hipError_t qmm_get_scratch(int device, hipStream_t stream, size_t bytes, void** out) {
     return get_scratch(device, stream, bytes, out);
 }
-std::atomic<int> g_moe_expert_form{-1}; // -1: read IZWI_QMM_MOE_EXPERT_FORM on first use
-bool qmm_moe_expert_form() {
+std::atomic<int> g_moe_expert_form{-2}; // -2: read IZWI_QMM_MOE_EXPERT_FORM on first use; then -1 (by size), 0, 1
+int qmm_moe_expert_form() {
     int v = g_moe_expert_form.load(std::memory_order_relaxed);
-    if (v < 0) {
+    if (v < -1) {
         const char* e = getenv("IZWI_QMM_MOE_EXPERT_FORM");
-        v = e && e[0] == '1';
+        v = e && e[0] == '1' ? 1 : e && e[0] == '0' ? 0 : -1;
         g_moe_expert_form.store(v, std::memory_order_relaxed);
     }
-    return v != 0;
+    return v;
 }
 const QmmLayout* qmm_weight_layout(const izwi_qmm_weight* w) { return &w->layout; }
 const void* qmm_weight_tiled(const izwi_qmm_weight* w) { return w->tiled; }
@@ -1498,14 +1498,14 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
                                             max_tiles, records, stream);
         if (e == hipSuccess)
             e = qmm_launch_gemv_mfma_grouped(G, gate->tiled, up->tiled, records, h, u, perm, offsets, seg, n_experts,
-                                             stream, gate->n_cus);
+                                             pairs, stream, gate->n_cus);
         // silu(gate) * up is applied while the down projection's input is quantized
         if (e == hipSuccess)
             e = qmm_launch_quantize_grouped(D.dtype, h, u, 1, inter, perm, offsets, seg, n_experts, max_tiles,
                                             records, stream);
         if (e == hipSuccess)
             e = qmm_launch_gemv_mfma_grouped(D, down->tiled, nullptr, records, y, nullptr, perm, offsets, seg,
-                                             n_experts, stream, down->n_cus);
+                                             n_experts, pairs, stream, down->n_cus);
     } else {
         if (!segments_ready)
             e = qmm_launch_moe_segments(offsets, n_experts, QMM_MOE_SEG_ROWS, seg, seg_expert, max_segments, stream);
@@ -1599,7 +1599,7 @@ int izwi_qmm_set_large_m_arithmetic(int mode) {
 int izwi_qmm_get_large_m_arithmetic(void) { return large_m_mode(); }
 
 int izwi_qmm_set_moe_expert_form(int enabled) {
-    g_moe_expert_form.store(enabled ? 1 : 0, std::memory_order_relaxed);
+    g_moe_expert_form.store(enabled < 0 ? -1 : enabled ? 1 : 0, std::memory_order_relaxed);
     return IZWI_QMM_OK;
 }
 

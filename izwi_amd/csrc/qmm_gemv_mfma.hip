@@ -645,7 +645,12 @@ __global__ __launch_bounds__(64 * kMaxWaves, (QT == QMM_Q4_K && SINGLE && NU == 
     asm volatile("s_barrier" ::: "memory");
     WPanel<QT> p;
     load_wpanel<QT>(p, wbase + (int64_t)((rt_ok ? rt : 0) * P.k_groups + wk) * P.panel_bytes, P.slots, lane, j);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory"); // the window has landed, the panel may still fly
+    // The window has landed.  The single-stage form lets the panel fly on: its arithmetic starts on the
+    // first chunk pair, and all NL loads of the panel are behind the window (every one of them is used:
+    // a load the compiler drops would make the count too lenient).  The other forms transpose the whole
+    // panel before their first stage anyway and wait for everything.
+    if (SINGLE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     lds_barrier();
 
     // several stages reuse the panel: its activation-independent part once, up front
@@ -981,6 +986,98 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
     }
 }
 
+// The expert form for Q4_K matrices whose panels all hold NU units: the panel's activation-
+// independent part is prepared once and serves the TC tiles, and the next panel of the wave's walk
+// (row-tile after row-tile, panel after panel) is requested before the arithmetic of the current
+// one starts - its registers are free as soon as the panel is prepared - so a wave always has a
+// panel in flight under its own arithmetic.
+template <int TC, int NU>
+__global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel(MfmaParams P) {
+    constexpr int QT = QMM_Q4_K;
+    constexpr int UB = Unit<QT>::kBytes;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = P.nwr;
+    const int j = lane & 15, grp = lane >> 4;
+    const int e = blockIdx.y;
+    const int tile_begin = P.tile_offsets[e];
+    const int n_tiles = P.tile_offsets[e + 1] - tile_begin;
+    if (n_tiles == 0) return; // uniform for the workgroup: nobody reaches a barrier
+    const int pos_begin = P.offsets[e], pos_end = P.offsets[e + 1];
+    const uint8_t* wbase = (blockIdx.z ? P.w2 : P.w) + (int64_t)e * P.matrix_bytes;
+    float* yout = blockIdx.z ? P.y2 : P.y;
+    const uint8_t* records = P.ws + (size_t)tile_begin * P.k_units * UB;
+    const int rt_first = blockIdx.x * waves + wave, rt_step = gridDim.x * waves;
+    const int lane16 = lane * 16;
+
+    for (int t0 = 0; t0 < n_tiles; t0 += TC) {
+        const int nt = min(TC, n_tiles - t0);
+        if (t0 != 0) lds_barrier(); // every wave is done with the previous tiles
+        issue_window_copy<QT>(records + (size_t)t0 * P.k_units * UB, smem, nt * P.k_units, wave, waves, lane);
+        WPanel<QT> p;
+        if (rt_first < P.row_tiles) // (uniform) the wave's first panel, needed whole before its first tile
+            load_wpanel<QT>(p, wbase + (int64_t)rt_first * P.k_groups * P.panel_bytes, P.slots, lane, j);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        lds_barrier();
+        for (int rt = rt_first; rt < P.row_tiles; rt += rt_step) {
+            float acc[TC][4];
+#pragma unroll
+            for (int t = 0; t < TC; t++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
+            for (int kg = 0; kg < P.k_groups; kg++) {
+#pragma unroll
+                for (int b = 0; b < WPanel<QT>::QC / 2; b++) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
+                Q4Prepared<NU> prep;
+                q4k_prepare<NU>(p, prep);
+                // the next panel of the walk, if any, into the registers just freed
+                int nrt = rt, nkg = kg + 1;
+                if (nkg == P.k_groups) nkg = 0, nrt = rt + rt_step;
+                if (nrt < P.row_tiles)
+                    load_wpanel<QT>(p, wbase + (int64_t)(nrt * P.k_groups + nkg) * P.panel_bytes, P.slots, lane, j);
+                const int unit0 = kg * NU;
+#pragma unroll
+                for (int t = 0; t < TC; t++) {
+                    if (t >= nt) continue; // uniform
+                    const uint8_t* xu0 = smem + ((size_t)t * P.k_units + unit0) * UB;
+                    q4k_tile_dot<NU>(
+                        prep, [&](int u, int b) { return *reinterpret_cast<const i64x2*>(xu0 + u * UB + lane16 + b * 1024); },
+                        [&](int u, long& bs_lo, long& bs_hi, float4& dx) {
+                            const uint8_t* side = xu0 + u * UB + Unit<QT>::kQuant;
+                            const i64x2 planes = *reinterpret_cast<const i64x2*>(side + 64 + j * 16);
+                            bs_lo = grp == 0 ? planes.x : 0L;
+                            bs_hi = grp == 0 ? planes.y : 0L;
+                            dx = *reinterpret_cast<const float4*>(side + grp * 16);
+                        },
+                        acc[t]);
+                }
+            }
+            const int row = rt * 16 + j;
+            if (row < P.n) {
+#pragma unroll
+                for (int t = 0; t < TC; t++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int mm = (t0 + t) * 16 + grp * 4 + r;
+                        if (t < nt && pos_begin + mm < pos_end) yout[(int64_t)P.perm[pos_begin + mm] * P.n + row] = acc[t][r];
+                    }
+            }
+        }
+    }
+}
+
+template <int TC, int NU>
+hipError_t launch_expert_q4k(const MfmaParams& P, dim3 grid, int waves, size_t lds, hipStream_t stream) {
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_expert_q4k_kernel<TC, NU>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+    }
+    gemv_mfma_expert_q4k_kernel<TC, NU><<<grid, 64 * waves, lds, stream>>>(P);
+    return hipGetLastError();
+}
+
 template <int QT, int TC>
 hipError_t launch_expert_form(const MfmaParams& P, dim3 grid, int waves, size_t lds, hipStream_t stream) {
     if (lds > 48 * 1024) {
@@ -1217,7 +1314,7 @@ bool qmm_gemv_mfma_grouped_supported(const QmmLayout& L) { return L.k_groups <= 
 hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
                                         const void* records, float* y, float* y2, const int32_t* perm,
                                         const int32_t* offsets, const int32_t* tile_offsets,
-                                        int n_experts, hipStream_t stream, int n_cus) {
+                                        int n_experts, int64_t pairs, hipStream_t stream, int n_cus) {
     if (L.n == 0 || n_experts <= 0) return hipSuccess;
     if (!qmm_gemv_mfma_grouped_supported(L) || n_experts > 65535 || L.n > 0x3fffffff)
         return hipErrorInvalidValue;
@@ -1251,10 +1348,13 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     P.y2 = y2;
     P.n_weights = 0;
     {
-        // the expert form (IZWI_QMM_MOE_EXPERT_FORM=1 or izwi_qmm_set_moe_expert_form; off by default: measured no faster than the one-shot
-        // form once the experts' tile counts are uneven) where at least two activation tiles over all of
-        // k fit in LDS
-        const bool expert_form = qmm_moe_expert_form();
+        // The expert form where up to four activation tiles of an expert over all of k fit in LDS and
+        // the experts have at most about three tiles each (an expert with more than four takes another
+        // pass over its weights): measured at 128 experts, top-8, per layer, expert / one-shot form:
+        // 127 / 161 us at 128 tokens, 165 / 185 at 256, 231 / 252 at 512, 388 / 380 at 1024, 663 / 621
+        // at 2048.  IZWI_QMM_MOE_EXPERT_FORM=1 / 0 or izwi_qmm_set_moe_expert_form force the choice.
+        const int mode = qmm_moe_expert_form();
+        const bool expert_form = mode >= 0 ? mode != 0 : pairs <= (int64_t)48 * n_experts;
         const size_t tile_bytes = (size_t)L.k_units * unit_bytes(L.dtype);
         // (Q6_K: two tiles at a time, four do not fit the registers)
         const int tc = L.dtype != QMM_Q6_K && 4 * tile_bytes <= 150 * 1024 ? 4 : (2 * tile_bytes <= 150 * 1024 ? 2 : 0);
@@ -1263,7 +1363,7 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
             const int stacks = tiled2 ? 2 : 1;
             int waves = kExpertWaves;
             if (waves > L.row_tiles) waves = (int)L.row_tiles;
-            static const int wgs_per_cu = [] { const char* e = getenv("IZWI_QMM_MOE_EXPERT_WGS_PER_CU"); int v = e ? atoi(e) : 3; return v > 0 ? v : 3; }();
+            static const int wgs_per_cu = [] { const char* e = getenv("IZWI_QMM_MOE_EXPERT_WGS_PER_CU"); int v = e ? atoi(e) : 2; return v > 0 ? v : 2; }();
             int parts = (wgs_per_cu * n_cus + n_experts * stacks - 1) / (n_experts * stacks);
             const int max_parts = (int)((L.row_tiles + waves - 1) / waves);
             if (parts > max_parts) parts = max_parts;
@@ -1271,6 +1371,10 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
             E.nwr = waves; // the workgroup's waves (every wave walks all of k)
             const dim3 grid((unsigned)parts, (unsigned)n_experts, (unsigned)stacks);
             const size_t lds = (size_t)tc * tile_bytes;
+            if (L.dtype == QMM_Q4_K && uniform_panel_units(L) == 4)
+                return tc == 4 ? launch_expert_q4k<4, 4>(E, grid, waves, lds, stream) : launch_expert_q4k<2, 4>(E, grid, waves, lds, stream);
+            if (L.dtype == QMM_Q4_K && uniform_panel_units(L) == 3)
+                return tc == 4 ? launch_expert_q4k<4, 3>(E, grid, waves, lds, stream) : launch_expert_q4k<2, 3>(E, grid, waves, lds, stream);
             if (L.dtype == QMM_Q4_K)
                 return tc == 4 ? launch_expert_form<QMM_Q4_K, 4>(E, grid, waves, lds, stream)
                                : launch_expert_form<QMM_Q4_K, 2>(E, grid, waves, lds, stream);

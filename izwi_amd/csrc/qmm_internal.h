@@ -104,7 +104,7 @@ bool qmm_profiling();
 bool qmm_stream_is_capturing(hipStream_t stream);
 void qmm_profile_count_argmax(uint64_t ns);
 // Whether the expert-grouped matrix-core kernel takes its expert form (a tuning switch, off by default).
-bool qmm_moe_expert_form();
+int qmm_moe_expert_form(); // 1 / 0: forced on / off, -1: chosen by the number of pairs per expert
 // A weight handle's layout, device matrix and device ordinal, for the library's other source files.
 struct izwi_qmm_weight;
 const QmmLayout* qmm_weight_layout(const izwi_qmm_weight* w);
@@ -267,7 +267,7 @@ bool qmm_gemv_mfma_grouped_supported(const QmmLayout& L);
 hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
                                         const void* records, float* y, float* y2, const int32_t* perm,
                                         const int32_t* offsets, const int32_t* tile_offsets,
-                                        int n_experts, hipStream_t stream, int n_cus);
+                                        int n_experts, int64_t pairs, hipStream_t stream, int n_cus);
 
 // Small batches: routing, sort and the segment tables (seg_rows rows per segment) of the grouped
 // decode kernel in one launch; same results as route + sort + segments.

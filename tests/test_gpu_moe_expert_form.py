@@ -1,6 +1,7 @@
-"""The optional expert form of the grouped matrix-core kernel (izwi_qmm_set_moe_expert_form /
-IZWI_QMM_MOE_EXPERT_FORM=1): the MoE parity tests once more, in this process, with the switch on, so
-that every case reports on its own."""
+"""The two forms of the grouped matrix-core kernel (izwi_qmm_set_moe_expert_form /
+IZWI_QMM_MOE_EXPERT_FORM): by default the library picks one per call from the number of pairs per
+expert; here the MoE parity tests run once more, in this process, with each form forced, so that every
+case reports on its own."""
 import pytest
 
 # the tests themselves (collected here a second time, with their parameters) and the fixtures they use
@@ -16,9 +17,9 @@ from test_gpu_q6k import test_moe_with_q6_k_expert_stacks  # noqa: F401
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True)
-def expert_form():
+@pytest.fixture(autouse=True, params=[1, 0], ids=["expert_form", "one_shot_form"])
+def forced_form(request):
     from izwi_amd import capi
-    capi.check(capi.lib().izwi_qmm_set_moe_expert_form(1))
+    capi.check(capi.lib().izwi_qmm_set_moe_expert_form(request.param))
     yield
-    capi.check(capi.lib().izwi_qmm_set_moe_expert_form(0))
+    capi.check(capi.lib().izwi_qmm_set_moe_expert_form(-1))  # back to the choice by size
