@@ -1443,7 +1443,8 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
         const size_t r2 = qmm_moe_records_bytes(D.dtype, max_tiles, inter);
         r_bytes = align256(r1 > r2 ? r1 : r2);
     }
-    const size_t mid_bytes = tiles ? h_bytes + r_bytes : align256((size_t)max_segments * 4);
+    const size_t te_bytes = tiles ? align256((size_t)max_tiles * 4) : 0; // tile -> expert
+    const size_t mid_bytes = tiles ? h_bytes + r_bytes + te_bytes : align256((size_t)max_segments * 4);
     const size_t p_bytes = align256((size_t)pairs * 4);
     const size_t sort_bytes = align256((size_t)qmm_moe_sort_scratch_ints(pairs, n_experts) * sizeof(int32_t));
     const size_t route_bytes = logits ? 3 * p_bytes + s_bytes + sort_bytes : 0;
@@ -1454,6 +1455,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
     int32_t* seg = (int32_t*)(ws + h_bytes + y_bytes);
     uint8_t* mid = ws + h_bytes + y_bytes + s_bytes;
     int32_t* seg_expert = (int32_t*)mid; // 4-row segment path only
+    int32_t* tile_expert = (int32_t*)(mid + h_bytes + r_bytes); // tile path only
     bool segments_ready = false;
     hipError_t e = hipSuccess;
     if (logits) {
@@ -1482,7 +1484,11 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
             segments_ready = true;
         } else {
             e = qmm_launch_moe_route(logits, t, n_experts, top_k, r_ids, r_w, stream);
-            if (e == hipSuccess) e = qmm_launch_moe_sort(r_ids, pairs, n_experts, r_perm, r_off, nullptr, r_sort, stream);
+            // the sort also leaves the table of 16-row tiles the matrix-core path walks
+            if (e == hipSuccess)
+                e = qmm_launch_moe_sort(r_ids, pairs, n_experts, r_perm, r_off, tiles ? seg : nullptr, r_sort, stream,
+                                        tiles ? QMM_MOE_TILE_ROWS : QMM_MOE_SEG_ROWS, tiles ? tile_expert : nullptr, max_tiles);
+            segments_ready = tiles;
         }
         if (e != hipSuccess) return fail_hip(e, "routing kernels");
         if (ids_out) HIP_TRY(hipMemcpyAsync(ids_out, r_ids, (size_t)pairs * 4, hipMemcpyDeviceToDevice, stream));
@@ -1492,17 +1498,17 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
     if (tiles) {
         float* u = (float*)mid;
         void* records = mid + h_bytes;
-        e = qmm_launch_moe_segments(offsets, n_experts, QMM_MOE_TILE_ROWS, seg, nullptr, 0, stream);
+        if (!segments_ready) e = qmm_launch_moe_segments(offsets, n_experts, QMM_MOE_TILE_ROWS, seg, tile_expert, max_tiles, stream);
         if (e == hipSuccess)
             e = qmm_launch_quantize_grouped(G.dtype, x, nullptr, top_k, hidden, perm, offsets, seg, n_experts,
-                                            max_tiles, records, stream);
+                                            max_tiles, records, stream, tile_expert);
         if (e == hipSuccess)
             e = qmm_launch_gemv_mfma_grouped(G, gate->tiled, up->tiled, records, h, u, perm, offsets, seg, n_experts,
                                              pairs, stream, gate->n_cus);
         // silu(gate) * up is applied while the down projection's input is quantized
         if (e == hipSuccess)
             e = qmm_launch_quantize_grouped(D.dtype, h, u, 1, inter, perm, offsets, seg, n_experts, max_tiles,
-                                            records, stream);
+                                            records, stream, tile_expert);
         if (e == hipSuccess)
             e = qmm_launch_gemv_mfma_grouped(D, down->tiled, nullptr, records, y, nullptr, perm, offsets, seg,
                                              n_experts, pairs, stream, down->n_cus);

@@ -131,18 +131,22 @@ __global__ void quantize_grouped_kernel(const float* __restrict__ x, const float
                                         int k, int k_units, const int32_t* __restrict__ perm,
                                         const int32_t* __restrict__ offsets,
                                         const int32_t* __restrict__ tile_offsets, int n_experts,
-                                        uint8_t* __restrict__ ws) {
+                                        const int32_t* __restrict__ tile_expert, uint8_t* __restrict__ ws) {
     const int64_t group = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
     const int j = threadIdx.x & 15;
     const int64_t row = group / k_units;
     const int unit = (int)(group - row * k_units);
     const int tile = (int)(row >> 4), mr = (int)(row & 15);
     if (tile >= tile_offsets[n_experts]) return; // whole 16-lane groups leave together
-    int lo = 0, hi = n_experts; // last e with tile_offsets[e] <= tile
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (tile_offsets[mid] <= tile) lo = mid;
-        else hi = mid;
+    int lo = 0, hi = n_experts; // last e with tile_offsets[e] <= tile: from the table, or searched for
+    if (tile_expert) {
+        lo = tile_expert[tile];
+    } else {
+        while (hi - lo > 1) { // seven dependent loads at 128 experts
+            const int mid = (lo + hi) >> 1;
+            if (tile_offsets[mid] <= tile) lo = mid;
+            else hi = mid;
+        }
     }
     const int pos = offsets[lo] + (tile - tile_offsets[lo]) * 16 + mr;
     const bool row_ok = pos < offsets[lo + 1];
@@ -1292,7 +1296,8 @@ size_t qmm_moe_records_bytes(int dtype, int64_t max_tiles, int64_t k) {
 hipError_t qmm_launch_quantize_grouped(int dtype, const float* x, const float* x2, int x_div,
                                        int64_t k, const int32_t* perm, const int32_t* offsets,
                                        const int32_t* tile_offsets, int n_experts,
-                                       int64_t max_tiles, void* records, hipStream_t stream) {
+                                       int64_t max_tiles, void* records, hipStream_t stream,
+                                       const int32_t* tile_expert) {
     const int64_t k_units = (k + 255) / 256;
     const int64_t threads = max_tiles * 16 * k_units * 16;
     if (threads <= 0) return hipSuccess;
@@ -1300,11 +1305,11 @@ hipError_t qmm_launch_quantize_grouped(int dtype, const float* x, const float* x
     const unsigned grid = (unsigned)((threads + 255) / 256);
     if (dtype == QMM_Q4_K || dtype == QMM_Q6_K) // both dot against Q8_K activations: one record format
         quantize_grouped_kernel<QMM_Q4_K><<<grid, 256, 0, stream>>>(x, x2, x_div, (int)k, (int)k_units, perm,
-                                                                    offsets, tile_offsets, n_experts,
+                                                                    offsets, tile_offsets, n_experts, tile_expert,
                                                                     (uint8_t*)records);
     else
         quantize_grouped_kernel<QMM_Q8_0><<<grid, 256, 0, stream>>>(x, x2, x_div, (int)k, (int)k_units, perm,
-                                                                    offsets, tile_offsets, n_experts,
+                                                                    offsets, tile_offsets, n_experts, tile_expert,
                                                                     (uint8_t*)records);
     return hipGetLastError();
 }

@@ -224,11 +224,14 @@ hipError_t qmm_launch_moe_route(const float* logits, int64_t t, int n_experts, i
                                 int32_t* ids, float* weights, hipStream_t stream);
 
 // Stable counting sort of `pairs` expert ids.  `seg_offsets` (n_experts + 1 ints,
-// may be NULL) receives the exclusive prefix sum of ceil(count / QMM_MOE_SEG_ROWS).
+// may be NULL) receives the exclusive prefix sum of ceil(count / seg_rows): the table of the
+// 4-row segments or of the 16-row tiles, whichever the expert MLP behind the sort runs on, and
+// `seg_expert` (may be NULL; up to max_segments entries) the expert of every such segment.
 // `scratch` must hold qmm_moe_sort_scratch_ints(pairs, n_experts) ints.
 hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts, int32_t* perm,
                                int32_t* offsets, int32_t* seg_offsets, int32_t* scratch,
-                               hipStream_t stream);
+                               hipStream_t stream, int seg_rows = QMM_MOE_SEG_ROWS, int32_t* seg_expert = nullptr,
+                               int64_t max_segments = 0);
 int64_t qmm_moe_sort_scratch_ints(int64_t pairs, int n_experts);
 
 // Expert-grouped decode kernel over sorted pairs.  Row i of the sorted list is
@@ -259,7 +262,8 @@ size_t qmm_moe_records_bytes(int dtype, int64_t max_tiles, int64_t k);
 hipError_t qmm_launch_quantize_grouped(int dtype, const float* x, const float* x2, int x_div,
                                        int64_t k, const int32_t* perm, const int32_t* offsets,
                                        const int32_t* tile_offsets, int n_experts,
-                                       int64_t max_tiles, void* records, hipStream_t stream);
+                                       int64_t max_tiles, void* records, hipStream_t stream,
+                                       const int32_t* tile_expert = nullptr);
 // false if the matrix shape has no grouped matrix-core form (too many panels per row-tile)
 bool qmm_gemv_mfma_grouped_supported(const QmmLayout& L);
 // With tiled2 / y2 a second stack of the same shape is multiplied by the same records

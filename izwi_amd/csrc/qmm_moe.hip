@@ -48,7 +48,8 @@ __global__ void sort_hist_kernel(const int32_t* __restrict__ ids, int64_t pairs,
 // One block: offsets = exclusive scan of the per-expert totals; hist[c][e] is
 // replaced by the position where chunk c starts writing expert e.
 __global__ void sort_scan_kernel(int32_t* __restrict__ hist, int64_t chunks, int n_experts,
-                                 int32_t* __restrict__ offsets, int32_t* __restrict__ seg_offsets) {
+                                 int32_t* __restrict__ offsets, int32_t* __restrict__ seg_offsets, int seg_rows,
+                                 int32_t* __restrict__ seg_expert, int max_segments) {
     extern __shared__ int32_t sh[]; // totals[n_experts]
     for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
         int32_t tot = 0;
@@ -63,16 +64,18 @@ __global__ void sort_scan_kernel(int32_t* __restrict__ hist, int64_t chunks, int
         for (int i = 0; i < e && i < n_experts; i++) {
             const int32_t c = sh[i];
             run += c;
-            seg += (c + QMM_MOE_SEG_ROWS - 1) / QMM_MOE_SEG_ROWS;
+            seg += (c + seg_rows - 1) / seg_rows;
         }
         __syncthreads();
         if (e < n_experts) {
             offsets[e] = run;
             if (seg_offsets) seg_offsets[e] = seg;
             const int32_t c = sh[e];
+            if (seg_expert)
+                for (int i = 0, n = (c + seg_rows - 1) / seg_rows; i < n && seg + i < max_segments; i++) seg_expert[seg + i] = e;
             if (e == n_experts - 1) {
                 offsets[n_experts] = run + c;
-                if (seg_offsets) seg_offsets[n_experts] = seg + (c + QMM_MOE_SEG_ROWS - 1) / QMM_MOE_SEG_ROWS;
+                if (seg_offsets) seg_offsets[n_experts] = seg + (c + seg_rows - 1) / seg_rows;
             }
             sh[e] = run;
         }
@@ -84,7 +87,9 @@ __global__ void sort_scan_kernel(int32_t* __restrict__ hist, int64_t chunks, int
             if (seg_offsets) seg_offsets[e] = seg;
             sh[e] = run;
             run += c;
-            seg += (c + QMM_MOE_SEG_ROWS - 1) / QMM_MOE_SEG_ROWS;
+            if (seg_expert)
+                for (int i = 0, n = (c + seg_rows - 1) / seg_rows; i < n && seg + i < max_segments; i++) seg_expert[seg + i] = e;
+            seg += (c + seg_rows - 1) / seg_rows;
         }
         offsets[n_experts] = run;
         if (seg_offsets) seg_offsets[n_experts] = seg;
@@ -154,7 +159,8 @@ constexpr int kBlockSortThreads = 1024, kBlockSortMaxRuns = 16; // runs per wave
 __global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int32_t* __restrict__ ids, int pairs,
                                                                        int n_experts, int32_t* __restrict__ perm,
                                                                        int32_t* __restrict__ offsets,
-                                                                       int32_t* __restrict__ seg_offsets) {
+                                                                       int32_t* __restrict__ seg_offsets, int seg_rows,
+                                                                       int32_t* __restrict__ seg_expert, int max_segments) {
     extern __shared__ int32_t sh[]; // hist[runs][n_experts] | start[n_experts + 1] | masks[waves][2 * n_experts]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = kBlockSortThreads / 64;
     const int runs = (pairs + 63) / 64;
@@ -195,7 +201,7 @@ __global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int
     // waves' totals
     const int e0 = threadIdx.x;
     const int c = e0 < n_experts ? start[e0] : 0;
-    const int sg = (c + QMM_MOE_SEG_ROWS - 1) / QMM_MOE_SEG_ROWS;
+    const int sg = (c + seg_rows - 1) / seg_rows;
     const int inc_c = wave_inclusive_sum(c, lane), inc_s = wave_inclusive_sum(sg, lane);
     if (lane == 63) wave_tot[wave] = inc_c, wave_seg[wave] = inc_s;
     __syncthreads();
@@ -206,6 +212,9 @@ __global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int
         offsets[e0] = base_c + inc_c - c;
         if (seg_offsets) seg_offsets[e0] = base_s + inc_s - sg;
         start[e0] = base_c + inc_c - c;
+        // segment -> expert (the segments of expert e0 are consecutive)
+        if (seg_expert)
+            for (int i = 0, first = base_s + inc_s - sg; i < sg && first + i < max_segments; i++) seg_expert[first + i] = e0;
     }
     __syncthreads();
 #pragma unroll
@@ -356,7 +365,8 @@ int64_t qmm_moe_sort_scratch_ints(int64_t pairs, int n_experts) {
 
 hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts, int32_t* perm,
                                int32_t* offsets, int32_t* seg_offsets, int32_t* scratch,
-                               hipStream_t stream) {
+                               hipStream_t stream, int seg_rows, int32_t* seg_expert, int64_t max_segments) {
+    if (seg_rows < 1 || max_segments > 0x7fffffff) return hipErrorInvalidValue;
     if (n_experts < 1 || n_experts > 8192) return hipErrorInvalidValue;
     if (block_sort_fits(pairs, n_experts)) {
         const size_t lds = ((size_t)((pairs + 63) / 64 + 1) * n_experts + 1 + (size_t)2 * n_experts * (kBlockSortThreads / 64)) * sizeof(int32_t);
@@ -365,14 +375,15 @@ hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
             if (e != hipSuccess) return e;
         }
-        sort_block_kernel<<<1, kBlockSortThreads, lds, stream>>>(ids, (int)pairs, n_experts, perm, offsets, seg_offsets);
+        sort_block_kernel<<<1, kBlockSortThreads, lds, stream>>>(ids, (int)pairs, n_experts, perm, offsets, seg_offsets, seg_rows, seg_expert, (int)max_segments);
         return hipGetLastError();
     }
     int64_t chunks = (pairs + kSortChunk - 1) / kSortChunk;
     if (chunks < 1) chunks = 1;
     size_t sh = (size_t)n_experts * sizeof(int32_t);
     sort_hist_kernel<<<(unsigned)chunks, kSortChunk, sh, stream>>>(ids, pairs, n_experts, scratch);
-    sort_scan_kernel<<<1, 256, sh, stream>>>(scratch, chunks, n_experts, offsets, seg_offsets);
+    sort_scan_kernel<<<1, 256, sh, stream>>>(scratch, chunks, n_experts, offsets, seg_offsets, seg_rows, seg_expert,
+                                             (int)max_segments);
     if (pairs > 0)
         sort_scatter_kernel<<<(unsigned)chunks, 128, 0, stream>>>(ids, pairs, n_experts, scratch,
                                                                   perm);
