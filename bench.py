@@ -598,7 +598,9 @@ def layer_stack_extra(torch, qa, dtype, steps=10, warmup=3):
     """Extra report (not `value`): one whole decode step of the Qwen3-8B stack composed from the library's
     calls (izwi_amd.qwen3_layer.Qwen3DecodeLayer: q|k|v group and gate/up with their RMSNorm and the
     activation folded in, attention with q/k norm + rotary + cache append inside its launch and the merge
-    of its splits, o and down with the residual folded in) plus the final norm folded into the LM head and the greedy argmax, f32 activations, HIP-graph replay, at several context lengths."""
+    of its splits, o and down with the residual folded in), from the embedding row of the previous token (read from the
+    quantized table) to the final norm folded into the LM head and the greedy argmax: every replay consumes the token
+    the one before produced.  f32 activations, HIP-graph replay, at several context lengths."""
     from izwi_amd.qwen3_layer import Qwen3DecodeLayer
     heads, kvh, d, hidden = 32, 8, 128, 4096
     weights = build_decode_weights(torch, qa, dtype, N_LAYERS_8B, True)
@@ -609,7 +611,10 @@ def layer_stack_extra(torch, qa, dtype, steps=10, warmup=3):
         q, k, v, o, gate, up, down = [w[0] for w in weights[i * per:(i + 1) * per]]
         layers.append(Qwen3DecodeLayer(ones(hidden), ones(hidden), q, k, v, ones(2 * d), o, gate, up, down, heads, kvh, d))
     lm_head, final_norm = weights[-1][0], ones(hidden)
-    x0 = torch.randn(1, hidden, device="cuda")
+    # token in, token out, all on the device: the step starts with the embedding row of the token the
+    # previous step's argmax left (the table is the LM head's quantized matrix, as in a tied checkpoint)
+    embed = qa.QuantizedEmbedding(lm_head.qtensor)
+    token = torch.zeros(1, dtype=torch.int32, device="cuda")
     cos_sin = torch.randn(1, d, device="cuda")
     out = {}
     for kv_len in (256, 4096):
@@ -617,15 +622,15 @@ def layer_stack_extra(torch, qa, dtype, steps=10, warmup=3):
                   for _ in range(N_LAYERS_8B)]
 
         def step():
-            x = x0
+            x = embed.forward(token)
             for layer, (kc, vc) in zip(layers, caches):
                 x = layer.forward(x, cos_sin, kc, vc, kv_len - 1)
-            return qa.argmax(lm_head.forward_normed(x, final_norm, 1e-6))  # final norm + LM head, greedy next token
+            token.copy_(qa.argmax(lm_head.forward_normed(x, final_norm, 1e-6)))  # final norm + LM head, greedy next token
         ms, g = time_graph(torch, step, steps, warmup)
         out[f"kv{kv_len}"] = {"ms_per_token": round(ms, 4), "tokens_per_s": round(1e3 / ms, 1)}
         del caches, g
         torch.cuda.empty_cache()
-    out["launches_per_token"] = N_LAYERS_8B * 6 + 3  # LM head with the norm, two for the argmax
+    out["launches_per_token"] = N_LAYERS_8B * 6 + 5  # embedding row, LM head with the norm, two for the argmax, the token copy
     del layers, weights
     torch.cuda.empty_cache()
     return out

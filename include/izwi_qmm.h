@@ -174,6 +174,17 @@ int izwi_qmm_weight_data(const izwi_qmm_weight* w, void* out_blocks, uint64_t nb
  * bit-identical to candle-core's `to_float`. */
 int izwi_qmm_dequantize_f32(const izwi_qmm_weight* w, float* out, int mem_space, void* stream);
 
+/* The embedding lookup: `Qwen3Model::embeddings` = `Embedding::forward(input_ids)` (qwen3/core.rs:2083-2085)
+ * on the table that `GgufLoader::load_tensor` dequantizes and casts to the model dtype
+ * (qwen3/core.rs:2000-2007, shared/weights/gguf.rs:127-143): out[i, :] = row row_ids[i] of
+ * izwi_qmm_dequantize_f32's matrix (first matrix of the handle), value for value, as f32 or rounded to
+ * bf16 (izwi_qmm_out_dtype) - without the dense [vocab, hidden] table in memory.  `row_ids` may be host
+ * or device memory (the id the device argmax left); host ids outside [0, n) are refused as the
+ * reference's index_select refuses them, device ids are not read by the host: such a row comes back
+ * as zeros.  out is `[n_rows, k]`. */
+int izwi_qmm_dequantize_rows(const izwi_qmm_weight* w, const int32_t* row_ids, int64_t n_rows, int ids_mem_space,
+                             void* out, int out_dtype, int out_mem_space, void* stream);
+
 /* --- forward: QMatMul::forward ------------------------------------------ */
 
 /* `QMatMul::forward(x)` for f32 activations (qwen3/core.rs:812; the reference

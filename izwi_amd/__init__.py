@@ -25,6 +25,7 @@ from .qmatmul import (  # noqa: F401
     MoeExperts,
     QMatMul,
     QTensor,
+    QuantizedEmbedding,
     Qwen3GateUpProjection,
     Qwen3Mlp,
     Qwen3Projection,

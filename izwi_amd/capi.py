@@ -63,6 +63,7 @@ PROTOTYPES = {
     "izwi_qmm_weight_get_info": (C.c_int, [_vp, C.POINTER(WeightInfo)]),
     "izwi_qmm_weight_data": (C.c_int, [_vp, _vp, _u64, C.c_int, _vp]),
     "izwi_qmm_dequantize_f32": (C.c_int, [_vp, _vp, C.c_int, _vp]),
+    "izwi_qmm_dequantize_rows": (C.c_int, [_vp, _vp, _i64, C.c_int, _vp, C.c_int, C.c_int, _vp]),
     "izwi_qmm_forward_f32": (C.c_int, [_vp, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_records_bytes": (_u64, [C.c_int, _i64, _i64]),
     "izwi_qmm_quantize_records_f32": (C.c_int, [C.c_int, _vp, _i64, _i64, _vp, _vp]),

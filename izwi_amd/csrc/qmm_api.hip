@@ -627,6 +627,35 @@ int izwi_qmm_dequantize_f32(const izwi_qmm_weight* w, float* out, int mem_space,
     return IZWI_QMM_OK;
 }
 
+int izwi_qmm_dequantize_rows(const izwi_qmm_weight* w, const int32_t* row_ids, int64_t n_rows, int ids_mem_space,
+                             void* out, int out_dtype, int out_mem_space, void* stream_) {
+    if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    if (int rc = check_space(ids_mem_space)) return rc;
+    if (int rc = check_space(out_mem_space)) return rc;
+    if (out_dtype != IZWI_QMM_OUT_F32 && out_dtype != IZWI_QMM_OUT_BF16)
+        return fail(IZWI_QMM_ERR_INVALID, "out_dtype %d is neither f32 nor bf16", out_dtype);
+    if (n_rows < 0 || n_rows > 0x7fffffff) return fail(IZWI_QMM_ERR_INVALID, "n_rows = %lld is out of range", (long long)n_rows);
+    const QmmLayout& L = w->layout;
+    if (n_rows == 0 || L.k == 0) return IZWI_QMM_OK;
+    if (!row_ids || !out) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    if (ids_mem_space == IZWI_QMM_HOST) // the reference's index_select refuses such an id; ids in device memory are not read here
+        for (int64_t i = 0; i < n_rows; i++)
+            if (row_ids[i] < 0 || row_ids[i] >= L.n)
+                return fail(IZWI_QMM_ERR_INVALID, "row id %d at position %lld is out of range for %lld rows", row_ids[i],
+                            (long long)i, (long long)L.n);
+    int device = 0;
+    if (int rc = current_device(&device)) return rc;
+    if (device != w->device) return fail(IZWI_QMM_ERR_INVALID, "weight lives on device %d, current device is %d", w->device, device);
+    hipStream_t stream = (hipStream_t)stream_;
+    Staged ids, o;
+    HIP_TRY(ids.in(row_ids, (size_t)n_rows * sizeof(int32_t), ids_mem_space));
+    HIP_TRY(o.out(out, (size_t)n_rows * L.k * (out_dtype == IZWI_QMM_OUT_BF16 ? 2 : 4), out_mem_space));
+    HIP_TRY(qmm_launch_dequant_rows(L, w->tiled, (const int32_t*)ids.dev, n_rows, o.dev, out_dtype == IZWI_QMM_OUT_BF16, stream));
+    HIP_TRY(o.finish(stream));
+    if (ids.owned) HIP_TRY(hipStreamSynchronize(stream)); // the staged ids are freed on return
+    return IZWI_QMM_OK;
+}
+
 int izwi_qmm_quantize_activations(int ggml_weight_dtype, const float* x, int64_t m, int64_t k,
                                   void* out_blocks, int mem_space, void* stream_) {
     if (!type_supported(ggml_weight_dtype))

@@ -127,6 +127,10 @@ hipError_t qmm_launch_unpack(const QmmLayout& L, const void* tiled, void* native
                              hipStream_t stream);
 hipError_t qmm_launch_dequant(const QmmLayout& L, const void* tiled, float* out,
                               hipStream_t stream);
+// out[i, :] = row rows[i] (device ints) of the first matrix, dequantized as above, f32 or rounded to bf16;
+// a row id outside [0, n) gives zeros.
+hipError_t qmm_launch_dequant_rows(const QmmLayout& L, const void* tiled, const int32_t* rows, int64_t n_rows,
+                                   void* out, int out_bf16, hipStream_t stream);
 
 // Decode kernel: y[m, n] = QMatMul(x[m, k]) for one matrix of the handle.
 // `n_cus` sizes the grid.  Returns hipErrorInvalidValue for shapes it cannot run.

@@ -247,6 +247,104 @@ __global__ void dequant_q6k_tiled_kernel(QmmLayout L, const uint8_t* __restrict_
     y[l + 96] = __fmul_rn(__fmul_rn(d, (float)sc[is + 6]), (float)q4);
 }
 
+// ---- selected rows of the dequantized matrix (the embedding lookup) -----------------------------
+// out[i, :] = row rows[i] of the first matrix, the arithmetic of the kernels above value for value,
+// stored as f32 or rounded to bf16 (nearest even, what a cast of the f32 table gives).  A row id
+// outside [0, n) gives a row of zeros.
+__device__ __forceinline__ void store_row_value(void* out, int out_bf16, int64_t i, float v) {
+    if (out_bf16) reinterpret_cast<uint16_t*>(out)[i] = qmm_f32_to_bf16_bits(v);
+    else reinterpret_cast<float*>(out)[i] = v;
+}
+
+__global__ void dequant_rows_q4k_kernel(QmmLayout L, const uint8_t* __restrict__ tiled,
+                                        const int32_t* __restrict__ rows, void* __restrict__ out, int out_bf16,
+                                        int64_t n_chunks) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_chunks) return;
+    int c = (int)(idx & 7);
+    int64_t blk = idx >> 3;
+    int64_t unit = blk % L.k_units, ri = blk / L.k_units;
+    const int64_t row = rows[ri];
+    const bool ok = row >= 0 && row < L.n;
+    const int64_t r = ok ? row : 0;
+    uint4 hdr = *reinterpret_cast<const uint4*>(tiled + piece_offset(L, 0, r, unit, 0));
+    uint4 qv = *reinterpret_cast<const uint4*>(tiled + piece_offset(L, 0, r, unit, 1 + c));
+    float d = qmm_f16_bits_to_f32((uint16_t)(hdr.x & 0xffffu));
+    float dmin = qmm_f16_bits_to_f32((uint16_t)(hdr.x >> 16));
+    uint32_t sc_lo, sc_hi, mn_lo, mn_hi;
+    qmm_unpack_q4k_scales(hdr.y, hdr.z, hdr.w, sc_lo, sc_hi, mn_lo, mn_hi);
+    int g = c >> 1, h = c & 1;
+    int s0 = 2 * g, s1 = 2 * g + 1;
+    float d1 = __fmul_rn(d, (float)qmm_byte_of(sc_lo, sc_hi, s0));
+    float m1 = __fmul_rn(dmin, (float)qmm_byte_of(mn_lo, mn_hi, s0));
+    float d2 = __fmul_rn(d, (float)qmm_byte_of(sc_lo, sc_hi, s1));
+    float m2 = __fmul_rn(dmin, (float)qmm_byte_of(mn_lo, mn_hi, s1));
+    const int64_t o = ri * L.k + unit * 256 + 64 * g + 16 * h;
+    uint32_t w[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            uint32_t byte = (w[j] >> (8 * b)) & 0xffu;
+            store_row_value(out, out_bf16, o + 4 * j + b, ok ? __fsub_rn(__fmul_rn(d1, (float)(byte & 0xF)), m1) : 0.0f);
+            store_row_value(out, out_bf16, o + 32 + 4 * j + b, ok ? __fsub_rn(__fmul_rn(d2, (float)(byte >> 4)), m2) : 0.0f);
+        }
+    }
+}
+
+__global__ void dequant_rows_q80_kernel(QmmLayout L, const uint8_t* __restrict__ tiled,
+                                        const int32_t* __restrict__ rows, void* __restrict__ out, int out_bf16,
+                                        int64_t n_chunks) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; // 16-byte half block
+    if (idx >= n_chunks) return;
+    const int64_t blocks_per_row = L.k / 32;
+    int h = (int)(idx & 1);
+    int64_t blk = idx >> 1;
+    int64_t kb = blk % blocks_per_row, ri = blk / blocks_per_row;
+    const int64_t row = rows[ri];
+    const bool ok = row >= 0 && row < L.n;
+    const int64_t r = ok ? row : 0;
+    int64_t unit = kb / 8;
+    int b = (int)(kb % 8);
+    uint16_t dbits = reinterpret_cast<const uint16_t*>(tiled + piece_offset(L, 0, r, unit, 0))[b];
+    float d = qmm_f16_bits_to_f32(dbits);
+    uint4 qv = *reinterpret_cast<const uint4*>(tiled + piece_offset(L, 0, r, unit, 1 + 2 * b + h));
+    const int64_t o = ri * L.k + kb * 32 + 16 * h;
+    uint32_t w[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            store_row_value(out, out_bf16, o + 4 * j + i, ok ? __fmul_rn((float)(int8_t)((w[j] >> (8 * i)) & 0xffu), d) : 0.0f);
+}
+
+__global__ void dequant_rows_q6k_kernel(QmmLayout L, const uint8_t* __restrict__ tiled,
+                                        const int32_t* __restrict__ rows, void* __restrict__ out, int out_bf16,
+                                        int64_t n_items) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_items) return;
+    const int l = (int)(idx & 31), half = (int)(idx >> 5) & 1, is = l >> 4;
+    int64_t blk = idx >> 6;
+    int64_t unit = blk % L.k_units, ri = blk / L.k_units;
+    const int64_t row = rows[ri];
+    const bool ok = row >= 0 && row < L.n;
+    const int64_t r = ok ? row : 0;
+    const int8_t* sc = reinterpret_cast<const int8_t*>(tiled + piece_offset(L, 0, r, unit, 0)) + 8 * half;
+    const uint8_t qa = tiled[piece_offset(L, 0, r, unit, 1 + 4 * half + (l >> 4)) + (l & 15)];
+    const uint8_t qb = tiled[piece_offset(L, 0, r, unit, 1 + 4 * half + 2 + (l >> 4)) + (l & 15)];
+    const uint8_t qh = tiled[piece_offset(L, 0, r, unit, 9 + 2 * half + (l >> 4)) + (l & 15)];
+    const float d = qmm_f16_bits_to_f32(*reinterpret_cast<const uint16_t*>(tiled + piece_offset(L, 0, r, unit, 13)));
+    const int q1 = (int)((qa & 0xF) | ((qh & 3) << 4)) - 32;
+    const int q2 = (int)((qb & 0xF) | (((qh >> 2) & 3) << 4)) - 32;
+    const int q3 = (int)((qa >> 4) | (((qh >> 4) & 3) << 4)) - 32;
+    const int q4 = (int)((qb >> 4) | (((qh >> 6) & 3) << 4)) - 32;
+    const int64_t y = ri * L.k + unit * 256 + 128 * half;
+    store_row_value(out, out_bf16, y + l, ok ? __fmul_rn(__fmul_rn(d, (float)sc[is]), (float)q1) : 0.0f);
+    store_row_value(out, out_bf16, y + l + 32, ok ? __fmul_rn(__fmul_rn(d, (float)sc[is + 2]), (float)q2) : 0.0f);
+    store_row_value(out, out_bf16, y + l + 64, ok ? __fmul_rn(__fmul_rn(d, (float)sc[is + 4]), (float)q3) : 0.0f);
+    store_row_value(out, out_bf16, y + l + 96, ok ? __fmul_rn(__fmul_rn(d, (float)sc[is + 6]), (float)q4) : 0.0f);
+}
+
 inline unsigned grid_for(int64_t n, int block) { return (unsigned)((n + block - 1) / block); }
 
 } // namespace
@@ -305,6 +403,25 @@ hipError_t qmm_launch_dequant(const QmmLayout& L, const void* tiled, float* out,
         if (n_chunks == 0) return hipSuccess;
         dequant_q80_kernel<<<grid_for(n_chunks, 256), 256, 0, stream>>>(L, (const uint8_t*)tiled,
                                                                         out, n_chunks);
+    }
+    return hipGetLastError();
+}
+
+hipError_t qmm_launch_dequant_rows(const QmmLayout& L, const void* tiled, const int32_t* rows, int64_t n_rows,
+                                   void* out, int out_bf16, hipStream_t stream) {
+    if (n_rows <= 0 || L.k == 0) return hipSuccess;
+    if (L.dtype == QMM_Q4_K) {
+        const int64_t n_chunks = n_rows * L.k_units * 8;
+        dequant_rows_q4k_kernel<<<grid_for(n_chunks, 256), 256, 0, stream>>>(L, (const uint8_t*)tiled, rows, out,
+                                                                             out_bf16, n_chunks);
+    } else if (L.dtype == QMM_Q6_K) {
+        const int64_t n_items = n_rows * L.k_units * 64;
+        dequant_rows_q6k_kernel<<<grid_for(n_items, 256), 256, 0, stream>>>(L, (const uint8_t*)tiled, rows, out,
+                                                                            out_bf16, n_items);
+    } else {
+        const int64_t n_chunks = n_rows * (L.k / 32) * 2;
+        dequant_rows_q80_kernel<<<grid_for(n_chunks, 256), 256, 0, stream>>>(L, (const uint8_t*)tiled, rows, out,
+                                                                             out_bf16, n_chunks);
     }
     return hipGetLastError();
 }

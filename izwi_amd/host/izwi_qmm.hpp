@@ -112,6 +112,14 @@ public:
         check(izwi_qmm_dequantize_f32(h_, out.data(), IZWI_QMM_HOST, nullptr));
         return out;
     }
+    // `Embedding::forward(input_ids)` on the dequantized table (qwen3/core.rs:2000-2007, 2083-2085):
+    // f32 [ids.size(), k], the rows of `dequantize()` with those ids; an id outside [0, n) is an error.
+    std::vector<float> dequantize_rows(const std::vector<int32_t>& ids) const {
+        std::vector<float> out(ids.size() * (size_t)info_.k);
+        check(izwi_qmm_dequantize_rows(h_, ids.data(), (int64_t)ids.size(), IZWI_QMM_HOST, out.data(), IZWI_QMM_OUT_F32,
+                                       IZWI_QMM_HOST, nullptr));
+        return out;
+    }
     izwi_qmm_weight* handle() const { return h_; }
 
 private:

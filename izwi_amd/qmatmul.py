@@ -130,6 +130,40 @@ class QTensor:
         return out if self._e == 1 else out.view(self._e, self._n, self._k)
 
 
+    def dequantize_rows(self, row_ids: torch.Tensor, dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        """Rows ``row_ids`` (int32 / int64 tensor, host or device) of ``dequantize()``, value for value,
+        as f32 or bf16, without building the dense matrix."""
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise capi.QmmError(-1, f"dequantize_rows gives f32 or bf16, not {dtype}")
+        self.dims2()
+        ids = row_ids.to(torch.int32).contiguous().view(-1)
+        device = ids.device if ids.is_cuda else torch.device("cuda")
+        out = torch.empty((ids.numel(), self._k), dtype=dtype, device=device)
+        check(lib().izwi_qmm_dequantize_rows(self._h, ids.data_ptr(), ids.numel(), _space(ids), out.data_ptr(),
+                                             1 if dtype == torch.bfloat16 else 0, _space(out), _stream_ptr(out)))
+        return out
+
+
+class QuantizedEmbedding:
+    """The embedding lookup of the reference's decoders: ``Embedding::new(loader.load_tensor(name, dtype,
+    device), hidden)`` followed by ``forward(input_ids)`` (qwen3/core.rs:2000-2007, 2083-2085) - the rows
+    of the dequantized table, cast to the model dtype - read from the quantized tensor itself."""
+
+    def __init__(self, qtensor: QTensor, dtype: torch.dtype = torch.float32):
+        self.qtensor = qtensor
+        self.dtype = dtype
+        self.vocab_size, self.hidden_size = qtensor.dims2()
+
+    def forward(self, input_ids: torch.Tensor) -> torch.Tensor:
+        """[..., hidden] for ids of any shape (index_select + reshape, as candle_nn's Embedding)."""
+        rows = self.qtensor.dequantize_rows(input_ids.reshape(-1), self.dtype)
+        return rows.view(*input_ids.shape, self.hidden_size)
+
+    def embeddings(self) -> torch.Tensor:
+        """The dense table (what a tied LM head multiplies by when a checkpoint has no lm_head)."""
+        return self.qtensor.dequantize().to(self.dtype)
+
+
 class QMatMul:
     """candle_core::quantized::QMatMul (the QTensor arm): ``forward(x) = x @ W^T``."""
 

@@ -237,6 +237,9 @@ static void gguf_load(const std::string& fixture) {
     for (float f : deq) sum += f;
     EXPECT(sum == 32224.0 && deq[224] == 346.5f && deq[32] == -2.5f);
     EXPECT(g->load_tensor("hand.q4k") == deq);
+    EXPECT(q4->dequantize_rows({0, 0}) == [&] { std::vector<float> two = deq; two.insert(two.end(), deq.begin(), deq.end()); return two; }());
+    EXPECT(q4->dequantize_rows({}).empty());
+    EXPECT(throws(izwi::Error::Kind::InvalidInput, "out of range", [&] { q4->dequantize_rows({1}); }));
     const std::vector<float> q8 = g->load_tensor("blk.q");
     EXPECT(q8.size() == 32 && q8[0] == -16.0f && q8[31] == 15.0f);
     EXPECT((g->load_tensor("a") == std::vector<float>{1.0f, 2.0f, 3.0f, 4.0f}));

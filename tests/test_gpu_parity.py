@@ -663,3 +663,47 @@ def test_gate_up_silu_mlp_mirror_host_pointers_and_errors(qa, oracle):
         qa.Qwen3GateUpProjection.new_separate(gate, q8).forward_silu_mul(xc)
     with pytest.raises(qa.QmmError, match="shape mismatch"):
         proj.forward_silu_mul(torch.zeros((1, 256), device="cuda"))
+
+
+@pytest.mark.parametrize("dtype,n,k", [(Q4_K, 1000, 1024), (Q8_0, 300, 96), (Q4_K, 151936, 256)])
+def test_embedding_rows_equal_rows_of_the_dequantized_table(qa, oracle, dtype, n, k):
+    """`Embedding::forward(input_ids)` on the dequantized table (qwen3/core.rs:2000-2007, 2083-2085):
+    the selected rows bit for bit, f32 and cast to bf16; ids from host and from device memory."""
+    w = oracle.randn(4100 + n, (min(n, 4096), k), std=0.05)
+    if n > 4096:
+        w = np.tile(w, ((n + 4095) // 4096, 1))[:n]
+    blocks = oracle.quantize(dtype, w)
+    q = qa.QTensor.from_blocks(qa.GgmlDType(dtype), blocks, (n, k))
+    table = q.dequantize()
+    assert np.array_equal(table.cpu().numpy().view(np.uint32), oracle.dequantize(dtype, blocks, n, k).view(np.uint32))
+    ids = np.array([0, n - 1, 17, 17, n // 2, 3, n - 2, 1], dtype=np.int64)
+    for where in ("cpu", "cuda"):
+        idt = torch.from_numpy(ids).to(where)
+        got = q.dequantize_rows(idt)
+        assert torch.equal(got.view(torch.int32), table[torch.from_numpy(ids).cuda()].view(torch.int32)), where
+        got16 = q.dequantize_rows(idt, torch.bfloat16)
+        assert torch.equal(got16.view(torch.int16), table[torch.from_numpy(ids).cuda()].to(torch.bfloat16).view(torch.int16))
+    emb = qa.QuantizedEmbedding(q, torch.bfloat16)
+    batch = torch.from_numpy(ids.reshape(2, 4)).cuda()
+    out = emb.forward(batch)
+    assert out.shape == (2, 4, k) and out.dtype == torch.bfloat16
+    assert torch.equal(out.view(-1, k).view(torch.int16), got16.view(torch.int16))
+    assert q.dequantize_rows(torch.zeros(0, dtype=torch.int64)).shape == (0, k)
+    from izwi_amd import capi
+    with pytest.raises(capi.QmmError, match="out of range"):
+        q.dequantize_rows(torch.tensor([0, n]))
+    with pytest.raises(capi.QmmError, match="out of range"):
+        q.dequantize_rows(torch.tensor([-1]))
+    # ids in device memory are not read by the host: a row of zeros
+    z = q.dequantize_rows(torch.tensor([n, 1], device="cuda"))
+    assert torch.count_nonzero(z[0]) == 0 and torch.equal(z[1].view(torch.int32), table[1].view(torch.int32))
+
+
+def test_embedding_rows_q6k(qa, oracle):
+    n, k = 200, 512
+    blocks = np_ref.random_q6_k_blocks(77, n, k)
+    q = qa.QTensor.from_blocks(qa.GgmlDType.Q6K, blocks, (n, k))
+    table = q.dequantize()
+    ids = torch.tensor([199, 0, 5, 5, 100], device="cuda")
+    assert torch.equal(q.dequantize_rows(ids).view(torch.int32), table[ids].view(torch.int32))
+    assert torch.equal(q.dequantize_rows(ids, torch.bfloat16).view(torch.int16), table[ids].to(torch.bfloat16).view(torch.int16))
