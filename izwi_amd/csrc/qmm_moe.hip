@@ -139,13 +139,17 @@ __device__ __forceinline__ void wave_ranks(int e, int n_experts, int lane, uint3
     __builtin_amdgcn_wave_barrier(); // the masks are reused by the wave's next run
 }
 
-// inclusive sum over the 64 lanes of a wave
+// inclusive sum over the 64 lanes of a wave: shifts inside the 16-lane rows, then the last lane of a
+// row broadcast to the rows behind it (data-parallel primitives on the vector ALU: six adds; the
+// shuffle form goes through the LDS crossbar six times).  All lanes must be active.
 __device__ __forceinline__ int wave_inclusive_sum(int v, int lane) {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int o = __shfl_up(v, d);
-        if (lane >= d) v += o;
-    }
+    (void)lane;
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false); // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false); // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false); // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false); // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false); // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false); // row_bcast:31 into rows 2 and 3
     return v;
 }
 
@@ -161,26 +165,34 @@ __global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int
                                                                        int32_t* __restrict__ offsets,
                                                                        int32_t* __restrict__ seg_offsets, int seg_rows,
                                                                        int32_t* __restrict__ seg_expert, int max_segments) {
-    extern __shared__ int32_t sh[]; // hist[runs][n_experts] | start[n_experts + 1] | masks[waves][2 * n_experts]
+    // hist[runs][stride] | start[n_experts + 1] | masks[waves][2 * n_experts]; the rows of hist have an odd
+    // stride: a wave that reads one expert's count of 64 runs would otherwise hit one LDS bank 64 times
+    extern __shared__ int32_t sh[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = kBlockSortThreads / 64;
     const int runs = (pairs + 63) / 64;
-    int32_t* start = sh + runs * n_experts;
+    const int stride = n_experts | 1;
+    int32_t* start = sh + runs * stride;
     uint32_t* masks = reinterpret_cast<uint32_t*>(start + n_experts + 1) + wave * 2 * n_experts;
     __shared__ int32_t wave_tot[16], wave_seg[16];
-    for (int i = threadIdx.x; i < runs * n_experts; i += kBlockSortThreads) sh[i] = 0;
-    __syncthreads();
     int my_e[kBlockSortMaxRuns], my_rank[kBlockSortMaxRuns];
+    // all ids of the wave's runs are requested before anything waits for one
+#pragma unroll
+    for (int j = 0; j < kBlockSortMaxRuns; j++) {
+        const int p = (wave + j * waves) * 64 + lane;
+        my_e[j] = p < pairs ? ids[p] : -1;
+    }
+    for (int i = threadIdx.x; i < runs * stride; i += kBlockSortThreads) sh[i] = 0;
+    __syncthreads();
 #pragma unroll
     for (int j = 0; j < kBlockSortMaxRuns; j++) {
         const int run = wave + j * waves;
-        my_e[j] = -1, my_rank[j] = 0;
+        my_rank[j] = 0;
         if (run >= runs) continue; // uniform per wave
-        const int p = run * 64 + lane;
-        const int e = p < pairs ? ids[p] : -1;
+        const int e = my_e[j];
         int rank, total;
         wave_ranks(e, n_experts, lane, masks, rank, total);
-        my_e[j] = e, my_rank[j] = rank;
-        if (e >= 0 && e < n_experts && rank == 0) sh[run * n_experts + e] = total; // the first of its expert in the run
+        my_rank[j] = rank;
+        if (e >= 0 && e < n_experts && rank == 0) sh[run * stride + e] = total; // the first of its expert in the run
     }
     __syncthreads();
     // per expert (a wave each, in turn): the runs' counts become the number of earlier pairs of the
@@ -189,9 +201,9 @@ __global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int
         int carry = 0;
         for (int r0 = 0; r0 < runs; r0 += 64) {
             const int r = r0 + lane;
-            const int h = r < runs ? sh[r * n_experts + e] : 0;
+            const int h = r < runs ? sh[r * stride + e] : 0;
             const int inc = wave_inclusive_sum(h, lane);
-            if (r < runs) sh[r * n_experts + e] = carry + inc - h;
+            if (r < runs) sh[r * stride + e] = carry + inc - h;
             carry += __shfl(inc, 63);
         }
         if (lane == 0) start[e] = carry; // the expert's total, for now
@@ -222,7 +234,7 @@ __global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int
         const int run = wave + j * waves;
         if (run >= runs) continue;
         const int e = my_e[j];
-        if (e >= 0 && e < n_experts) perm[start[e] + sh[run * n_experts + e] + my_rank[j]] = run * 64 + lane;
+        if (e >= 0 && e < n_experts) perm[start[e] + sh[run * stride + e] + my_rank[j]] = run * 64 + lane;
     }
 }
 
@@ -230,7 +242,7 @@ bool block_sort_fits(int64_t pairs, int n_experts) {
     if (pairs < 1 || n_experts >= kBlockSortThreads) return false;
     const int64_t runs = (pairs + 63) / 64;
     return runs <= (int64_t)kBlockSortMaxRuns * (kBlockSortThreads / 64) &&
-           ((runs + 1) * n_experts + 1 + 2 * n_experts * (kBlockSortThreads / 64)) * 4 <= 64 * 1024;
+           (runs * (n_experts | 1) + n_experts + 1 + 2 * n_experts * (kBlockSortThreads / 64)) * 4 <= 64 * 1024;
 }
 
 // seg_offsets[e] = sum over e' < e of ceil(count(e') / seg_rows).  One block:
@@ -369,7 +381,7 @@ hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts,
     if (seg_rows < 1 || max_segments > 0x7fffffff) return hipErrorInvalidValue;
     if (n_experts < 1 || n_experts > 8192) return hipErrorInvalidValue;
     if (block_sort_fits(pairs, n_experts)) {
-        const size_t lds = ((size_t)((pairs + 63) / 64 + 1) * n_experts + 1 + (size_t)2 * n_experts * (kBlockSortThreads / 64)) * sizeof(int32_t);
+        const size_t lds = ((size_t)((pairs + 63) / 64) * (n_experts | 1) + n_experts + 1 + (size_t)2 * n_experts * (kBlockSortThreads / 64)) * sizeof(int32_t);
         if (lds > 48 * 1024) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sort_block_kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
