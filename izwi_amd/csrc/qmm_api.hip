@@ -102,11 +102,14 @@ int ensure_device(int device, int* n_cus) {
 }
 
 // Average sorted pairs per expert from which the expert MLP runs on 16-row matrix-core
-// tiles instead of 4-row dot4 segments (IZWI_QMM_MOE_MFMA_MIN_ROWS, default 8).
+// tiles instead of 4-row dot4 segments (IZWI_QMM_MOE_MFMA_MIN_ROWS, default 4).  Measured at 128
+// experts, top-8, per layer, segments / tiles: 61 / 104 us at 16 tokens, 87 / 109 at 32, 110 / 114 at 48
+// (3 pairs per expert), 131 / 116 at 64 (4 pairs), 183 / 119 at 96: the tile path reads every expert
+// once and costs about the same from 16 to 128 tokens, the segment path grows with the pairs.
 int moe_mfma_min_rows() {
     static const int v = [] {
         const char* s = getenv("IZWI_QMM_MOE_MFMA_MIN_ROWS");
-        int n = s ? atoi(s) : 8;
+        int n = s ? atoi(s) : 4;
         return n < 1 ? 1 : n;
     }();
     return v;
@@ -1513,11 +1516,13 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
             segments_ready = true;
         } else {
             e = qmm_launch_moe_route(logits, t, n_experts, top_k, r_ids, r_w, stream);
-            // the sort also leaves the table of 16-row tiles the matrix-core path walks
+            // the sort also leaves the table of the 16-row tiles the matrix-core path walks, or of the
+            // 4-row segments of the decode kernel, with the expert of every tile / segment
             if (e == hipSuccess)
-                e = qmm_launch_moe_sort(r_ids, pairs, n_experts, r_perm, r_off, tiles ? seg : nullptr, r_sort, stream,
-                                        tiles ? QMM_MOE_TILE_ROWS : QMM_MOE_SEG_ROWS, tiles ? tile_expert : nullptr, max_tiles);
-            segments_ready = tiles;
+                e = qmm_launch_moe_sort(r_ids, pairs, n_experts, r_perm, r_off, seg, r_sort, stream,
+                                        tiles ? QMM_MOE_TILE_ROWS : QMM_MOE_SEG_ROWS, tiles ? tile_expert : seg_expert,
+                                        tiles ? max_tiles : max_segments);
+            segments_ready = true;
         }
         if (e != hipSuccess) return fail_hip(e, "routing kernels");
         if (ids_out) HIP_TRY(hipMemcpyAsync(ids_out, r_ids, (size_t)pairs * 4, hipMemcpyDeviceToDevice, stream));

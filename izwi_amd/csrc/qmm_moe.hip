@@ -51,6 +51,7 @@ __global__ void sort_scan_kernel(int32_t* __restrict__ hist, int64_t chunks, int
                                  int32_t* __restrict__ offsets, int32_t* __restrict__ seg_offsets, int seg_rows,
                                  int32_t* __restrict__ seg_expert, int max_segments) {
     extern __shared__ int32_t sh[]; // totals[n_experts]
+    __shared__ int32_t total_segments;
     for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
         int32_t tot = 0;
         for (int64_t c = 0; c < chunks; c++) tot += hist[c * n_experts + e];
@@ -76,6 +77,7 @@ __global__ void sort_scan_kernel(int32_t* __restrict__ hist, int64_t chunks, int
             if (e == n_experts - 1) {
                 offsets[n_experts] = run + c;
                 if (seg_offsets) seg_offsets[n_experts] = seg + (c + seg_rows - 1) / seg_rows;
+                total_segments = seg + (c + seg_rows - 1) / seg_rows;
             }
             sh[e] = run;
         }
@@ -93,8 +95,11 @@ __global__ void sort_scan_kernel(int32_t* __restrict__ hist, int64_t chunks, int
         }
         offsets[n_experts] = run;
         if (seg_offsets) seg_offsets[n_experts] = seg;
+        total_segments = seg;
     }
     __syncthreads();
+    if (seg_expert) // entries past the last segment say so
+        for (int i = total_segments + (int)threadIdx.x; i < max_segments; i += blockDim.x) seg_expert[i] = -1;
     for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
         int32_t run = sh[e];
         for (int64_t c = 0; c < chunks; c++) {
@@ -159,21 +164,25 @@ __device__ __forceinline__ int wave_inclusive_sum(int v, int lane) {
 // scanned run by run (a wave per expert, a lane per run) and over the experts (wave scans); every
 // pair goes to offsets[e] + (pairs of e in earlier runs) + rank.  Integer arithmetic whose result does
 // not depend on the order of execution: the same perm / offsets as the three-kernel sort.
+// `ids`: the pairs' experts, in global memory or in LDS (the one-launch plan of small batches routes
+// them there first).  `sh`: block_sort_lds_ints(pairs, n_experts) ints of LDS.  Called by all
+// kBlockSortThreads threads of the workgroup.
 constexpr int kBlockSortThreads = 1024, kBlockSortMaxRuns = 16; // runs per wave
-__global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int32_t* __restrict__ ids, int pairs,
-                                                                       int n_experts, int32_t* __restrict__ perm,
-                                                                       int32_t* __restrict__ offsets,
-                                                                       int32_t* __restrict__ seg_offsets, int seg_rows,
-                                                                       int32_t* __restrict__ seg_expert, int max_segments) {
+__host__ __device__ inline int64_t block_sort_lds_ints(int64_t pairs, int n_experts) {
+    return ((pairs + 63) / 64) * (n_experts | 1) + n_experts + 1 + (int64_t)2 * n_experts * (kBlockSortThreads / 64);
+}
+__device__ __forceinline__ void block_sort_body(const int32_t* ids, int pairs, int n_experts, int32_t* __restrict__ perm,
+                                                int32_t* __restrict__ offsets, int32_t* __restrict__ seg_offsets,
+                                                int seg_rows, int32_t* __restrict__ seg_expert, int max_segments,
+                                                int32_t* sh) {
     // hist[runs][stride] | start[n_experts + 1] | masks[waves][2 * n_experts]; the rows of hist have an odd
     // stride: a wave that reads one expert's count of 64 runs would otherwise hit one LDS bank 64 times
-    extern __shared__ int32_t sh[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = kBlockSortThreads / 64;
     const int runs = (pairs + 63) / 64;
     const int stride = n_experts | 1;
     int32_t* start = sh + runs * stride;
     uint32_t* masks = reinterpret_cast<uint32_t*>(start + n_experts + 1) + wave * 2 * n_experts;
-    __shared__ int32_t wave_tot[16], wave_seg[16];
+    __shared__ int32_t wave_tot[16], wave_seg[16], total_segments;
     int my_e[kBlockSortMaxRuns], my_rank[kBlockSortMaxRuns];
     // all ids of the wave's runs are requested before anything waits for one
 #pragma unroll
@@ -227,8 +236,12 @@ __global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int
         // segment -> expert (the segments of expert e0 are consecutive)
         if (seg_expert)
             for (int i = 0, first = base_s + inc_s - sg; i < sg && first + i < max_segments; i++) seg_expert[first + i] = e0;
+        if (e0 == n_experts) total_segments = base_s + inc_s;
     }
     __syncthreads();
+    // entries past the last segment say so (the grouped decode launch has one workgroup per entry)
+    if (seg_expert)
+        for (int i = total_segments + (int)threadIdx.x; i < max_segments; i += kBlockSortThreads) seg_expert[i] = -1;
 #pragma unroll
     for (int j = 0; j < kBlockSortMaxRuns; j++) {
         const int run = wave + j * waves;
@@ -238,11 +251,19 @@ __global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int
     }
 }
 
+__global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int32_t* __restrict__ ids, int pairs,
+                                                                       int n_experts, int32_t* __restrict__ perm,
+                                                                       int32_t* __restrict__ offsets,
+                                                                       int32_t* __restrict__ seg_offsets, int seg_rows,
+                                                                       int32_t* __restrict__ seg_expert, int max_segments) {
+    extern __shared__ int32_t sh[];
+    block_sort_body(ids, pairs, n_experts, perm, offsets, seg_offsets, seg_rows, seg_expert, max_segments, sh);
+}
+
 bool block_sort_fits(int64_t pairs, int n_experts) {
     if (pairs < 1 || n_experts >= kBlockSortThreads) return false;
     const int64_t runs = (pairs + 63) / 64;
-    return runs <= (int64_t)kBlockSortMaxRuns * (kBlockSortThreads / 64) &&
-           (runs * (n_experts | 1) + n_experts + 1 + 2 * n_experts * (kBlockSortThreads / 64)) * 4 <= 64 * 1024;
+    return runs <= (int64_t)kBlockSortMaxRuns * (kBlockSortThreads / 64) && block_sort_lds_ints(pairs, n_experts) * 4 <= 64 * 1024;
 }
 
 // seg_offsets[e] = sum over e' < e of ceil(count(e') / seg_rows).  One block:
@@ -280,63 +301,34 @@ __global__ void segments_kernel(const int32_t* __restrict__ offsets, int n_exper
         for (int s = total + threadIdx.x; s < max_segments; s += 256) seg_expert[s] = -1;
 }
 
-// Small batches (t * top_k <= kPlanMaxPairs): routing, stable counting sort and the segment tables
-// of the grouped decode kernel in ONE workgroup and launch.  Results equal route_kernel +
-// sort_* + segments_kernel bit for bit (same routing function, integer-only sort).
-constexpr int kPlanMaxPairs = 1024, kPlanMaxExperts = 256, kPlanThreads = 256;
+// Small batches (up to kPlanMaxTokens tokens): routing, stable counting sort and the segment tables of
+// the grouped decode kernel in ONE workgroup and launch: a wave routes a token (all tokens at once), the
+// ids stay in LDS and go through the one-workgroup sort above.  Results equal route_kernel + sort_* +
+// segments_kernel bit for bit (same routing function, integer-only sort).  (A first version ran four
+// waves, routed the tokens four at a time and ranked every pair against all earlier ones: 17.6 us at 16
+// tokens, 54 us at 64, where routing and sort as two launches take 10.)
+constexpr int kPlanMaxTokens = kBlockSortThreads / 64, kPlanMaxExperts = 256;
 template <int PER_LANE>
-__global__ __launch_bounds__(kPlanThreads) void moe_plan_small_kernel(
+__global__ __launch_bounds__(kBlockSortThreads) void moe_plan_small_kernel(
     const float* __restrict__ logits, int t, int n_experts, int top_k, int max_segments,
     int32_t* __restrict__ ids, float* __restrict__ weights, int32_t* __restrict__ perm,
     int32_t* __restrict__ offsets, int32_t* __restrict__ seg_offsets, int32_t* __restrict__ seg_expert) {
-    __shared__ int32_t s_ids[kPlanMaxPairs];
-    __shared__ int32_t s_count[kPlanMaxExperts], s_start[kPlanMaxExperts];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = kPlanThreads / 64;
+    extern __shared__ int32_t sh[]; // the sort's counters | the ids
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int pairs = t * top_k;
-    constexpr int seg_rows = QMM_MOE_SEG_ROWS; // a constant: the divisions below are shifts
-    for (int e = threadIdx.x; e < n_experts; e += kPlanThreads) s_count[e] = 0;
-    // 1. routing: one wave per token
-    for (int tok = wave; tok < t; tok += waves) {
+    int32_t* s_ids = sh + block_sort_lds_ints(pairs, n_experts);
+    if (wave < t) { // uniform per wave
         int id;
         float w;
-        route_token<PER_LANE>(logits + (int64_t)tok * n_experts, n_experts, top_k, lane, id, w);
+        route_token<PER_LANE>(logits + (int64_t)wave * n_experts, n_experts, top_k, lane, id, w);
         if (lane < top_k) {
-            ids[tok * top_k + lane] = id;
-            weights[tok * top_k + lane] = w;
-            s_ids[tok * top_k + lane] = id;
+            ids[wave * top_k + lane] = id;
+            weights[wave * top_k + lane] = w;
+            s_ids[wave * top_k + lane] = id;
         }
     }
     __syncthreads();
-    // 2. per-expert counts (integer adds: order-free)
-    for (int p = threadIdx.x; p < pairs; p += kPlanThreads) atomicAdd(&s_count[s_ids[p]], 1);
-    __syncthreads();
-    // 3. exclusive prefix sums of the counts and of the segment counts: thread e sums what lies
-    //    before expert e (LDS broadcast reads)
-    for (int e = threadIdx.x; e <= n_experts; e += kPlanThreads) {
-        int32_t run = 0, seg = 0;
-        for (int i = 0; i < e; i++) {
-            const int32_t c = s_count[i];
-            run += c;
-            seg += (c + seg_rows - 1) / seg_rows;
-        }
-        offsets[e] = run;
-        seg_offsets[e] = seg;
-        if (e < n_experts) {
-            s_start[e] = run;
-            const int32_t n = (s_count[e] + seg_rows - 1) / seg_rows;
-            for (int32_t i = 0; i < n && seg + i < max_segments; i++) seg_expert[seg + i] = e;
-        } else {
-            for (int sidx = seg; sidx < max_segments; sidx++) seg_expert[sidx] = -1; // past the last segment
-        }
-    }
-    __syncthreads();
-    // 4. stable scatter: pair p goes behind the earlier pairs of its expert
-    for (int p = threadIdx.x; p < pairs; p += kPlanThreads) {
-        const int32_t e = s_ids[p];
-        int32_t rank = 0;
-        for (int q = 0; q < p; q++) rank += s_ids[q] == e;
-        perm[s_start[e] + rank] = p;
-    }
+    block_sort_body(s_ids, pairs, n_experts, perm, offsets, seg_offsets, QMM_MOE_SEG_ROWS, seg_expert, max_segments, sh);
 }
 
 __global__ void combine_kernel(const float* __restrict__ y, const float* __restrict__ weights,
@@ -381,7 +373,7 @@ hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts,
     if (seg_rows < 1 || max_segments > 0x7fffffff) return hipErrorInvalidValue;
     if (n_experts < 1 || n_experts > 8192) return hipErrorInvalidValue;
     if (block_sort_fits(pairs, n_experts)) {
-        const size_t lds = ((size_t)((pairs + 63) / 64) * (n_experts | 1) + n_experts + 1 + (size_t)2 * n_experts * (kBlockSortThreads / 64)) * sizeof(int32_t);
+        const size_t lds = (size_t)block_sort_lds_ints(pairs, n_experts) * sizeof(int32_t);
         if (lds > 48 * 1024) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sort_block_kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
@@ -411,7 +403,8 @@ hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int se
 }
 
 bool qmm_moe_plan_small_supported(int64_t t, int n_experts, int top_k) {
-    return t > 0 && t * top_k <= kPlanMaxPairs && n_experts <= kPlanMaxExperts && top_k <= 64 && top_k <= n_experts;
+    return t > 0 && t <= kPlanMaxTokens && n_experts <= kPlanMaxExperts && top_k <= 64 && top_k <= n_experts &&
+           block_sort_fits(t * top_k, n_experts) && (block_sort_lds_ints(t * top_k, n_experts) + t * top_k) * 4 <= 64 * 1024;
 }
 
 hipError_t qmm_launch_moe_plan_small(const float* logits, int64_t t, int n_experts, int top_k, int seg_rows,
@@ -420,12 +413,19 @@ hipError_t qmm_launch_moe_plan_small(const float* logits, int64_t t, int n_exper
                                      hipStream_t stream) {
     if (!qmm_moe_plan_small_supported(t, n_experts, top_k) || max_segments > 0x7fffffff || seg_rows != QMM_MOE_SEG_ROWS)
         return hipErrorInvalidValue;
+    const size_t lds = (size_t)(block_sort_lds_ints(t * top_k, n_experts) + t * top_k) * sizeof(int32_t);
+    const void* fn = n_experts <= 128 ? reinterpret_cast<const void*>(&moe_plan_small_kernel<2>)
+                                      : reinterpret_cast<const void*>(&moe_plan_small_kernel<4>);
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+        if (e != hipSuccess) return e;
+    }
     if (n_experts <= 128)
-        moe_plan_small_kernel<2><<<1, kPlanThreads, 0, stream>>>(logits, (int)t, n_experts, top_k, (int)max_segments,
-                                                                 ids, weights, perm, offsets, seg_offsets, seg_expert);
+        moe_plan_small_kernel<2><<<1, kBlockSortThreads, lds, stream>>>(logits, (int)t, n_experts, top_k, (int)max_segments,
+                                                                       ids, weights, perm, offsets, seg_offsets, seg_expert);
     else
-        moe_plan_small_kernel<4><<<1, kPlanThreads, 0, stream>>>(logits, (int)t, n_experts, top_k, (int)max_segments,
-                                                                 ids, weights, perm, offsets, seg_offsets, seg_expert);
+        moe_plan_small_kernel<4><<<1, kBlockSortThreads, lds, stream>>>(logits, (int)t, n_experts, top_k, (int)max_segments,
+                                                                       ids, weights, perm, offsets, seg_offsets, seg_expert);
     return hipGetLastError();
 }
 
