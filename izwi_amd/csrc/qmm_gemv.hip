@@ -267,9 +267,8 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
 // whether it exists or not.
 // The dense straight-line single-row Q4_K form is held to 80 registers: six waves per SIMD,
 // i.e. two 12-wave workgroups per CU.
-template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false, int IO = 0, bool NORM = false, bool TILEMAP = false>
-__global__ __launch_bounds__(64 * kMaxWaves)
-__attribute__((amdgpu_waves_per_eu(NORM ? 3 : (ONESHOT && !GROUPED && MT == 1 && QT == QMM_Q4_K) ? 6 : 3))) void gemv_kernel(GemvParams P) {
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT, int IO, bool NORM, bool TILEMAP>
+__device__ __forceinline__ void gemv_entry(const GemvParams& P, const GemvParams& P0, int n_weights) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int m_begin = 0, m_end = P.m;
     int64_t w_offset = 0;
@@ -284,14 +283,25 @@ __attribute__((amdgpu_waves_per_eu(NORM ? 3 : (ONESHOT && !GROUPED && MT == 1 &&
     const uint8_t* w_first = P.w + w_offset;
     float* y_out = P.y;
     int n_rows = P.n, row_tiles = P.row_tiles, rtg0 = blockIdx.x;
-    if (!GROUPED && ONESHOT && P.n_weights > 1) {
-        int i = 0;
-        while (i + 1 < P.n_weights && (int)blockIdx.x >= P.rtg_end[i]) i++;
-        rtg0 = blockIdx.x - (i ? P.rtg_end[i - 1] : 0);
-        w_first = P.wv[i];
-        y_out = P.yv[i];
-        n_rows = P.nv[i];
-        row_tiles = P.row_tiles_v[i];
+    if (!GROUPED && ONESHOT && n_weights > 1) {
+        // The tables are read whole (independent scalar loads, one round trip) and the
+        // workgroup's entry is picked with selects; rtg_end ascends, so the entry is the
+        // number of ends at or below the workgroup index.  Entries past n_weights hold
+        // whatever the host left there and are never picked.
+        static_assert(QMM_MAX_GROUP == 4, "the selects below name four entries");
+        const int b = blockIdx.x;
+        const int e0 = P0.rtg_end[0], e1 = P0.rtg_end[1], e2 = P0.rtg_end[2];
+        const bool c1 = b >= e0, c2 = n_weights > 2 && b >= e1, c3 = n_weights > 3 && b >= e2;
+        auto pick = [c1, c2, c3](auto v0, auto v1, auto v2, auto v3) {
+            auto v = c1 ? v1 : v0;
+            v = c2 ? v2 : v;
+            return c3 ? v3 : v;
+        };
+        rtg0 = b - pick(0, e0, e1, e2);
+        w_first = pick(P0.wv[0], P0.wv[1], P0.wv[2], P0.wv[3]);
+        y_out = pick(P0.yv[0], P0.yv[1], P0.yv[2], P0.yv[3]);
+        n_rows = pick(P0.nv[0], P0.nv[1], P0.nv[2], P0.nv[3]);
+        row_tiles = pick(P0.row_tiles_v[0], P0.row_tiles_v[1], P0.row_tiles_v[2], P0.row_tiles_v[3]);
     }
     if (GROUPED && ONESHOT && MT == 4) {
         const int rows = m_end - m_begin;
@@ -304,6 +314,39 @@ __attribute__((amdgpu_waves_per_eu(NORM ? 3 : (ONESHOT && !GROUPED && MT == 1 &&
     } else {
         gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO, NORM, TILEMAP>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     }
+}
+
+// The dense launches.  What the first loads' addresses need comes in the 14 leading argument
+// dwords, which the command processor writes into scalar registers when it starts a wave
+// (kernel-argument preload): the first load does not wait for a read of the argument block.
+// The rest of the parameter block is read from memory when its first use comes (the tables
+// of a group of weights are indexed in the block itself, P0).
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT = false, int IO = 0, bool NORM = false, bool TILEMAP = false>
+__global__ __launch_bounds__(64 * kMaxWaves)
+__attribute__((amdgpu_waves_per_eu(NORM ? 3 : (ONESHOT && MT == 1 && QT == QMM_Q4_K) ? 6 : 3)))
+void gemv_kernel(const uint8_t* w_arg, const float* x_arg, float* y_arg, int m_arg, int n_arg, int k_arg, int k_groups_arg,
+                 int panel_bytes_arg, int row_tiles_arg, int split_arg, int wave_magic_arg, GemvParams P0) {
+    static_assert(!GROUPED, "the expert-grouped launches go through gemv_grouped_kernel");
+    GemvParams P = P0;
+    P.w = w_arg, P.x = x_arg, P.y = y_arg, P.m = m_arg, P.n = n_arg, P.k = k_arg, P.k_groups = k_groups_arg;
+    P.panel_bytes = panel_bytes_arg, P.row_tiles = row_tiles_arg, P.wave_magic = wave_magic_arg;
+    P.nwk = split_arg & 255, P.nwr = (split_arg >> 8) & 255, P.slots = (split_arg >> 16) & 255;
+    gemv_entry<QT, MT, GATED, false, ONESHOT, IO, NORM, TILEMAP>(P, P0, split_arg >> 24);
+}
+
+// The expert-grouped launches: thousands of short workgroups, whose waves start faster with
+// fewer scalar registers to fill (measured: 1 us of 19 - 30 lost with preloaded arguments), so
+// the parameter block stays one block in memory.
+template <int QT, int MT, bool GATED, bool ONESHOT>
+__global__ __launch_bounds__(64 * kMaxWaves) __attribute__((amdgpu_waves_per_eu(3))) void gemv_grouped_kernel(GemvParams P) {
+    gemv_entry<QT, MT, GATED, true, ONESHOT, 0, false, false>(P, P, 0);
+}
+
+// The launch of a gemv_kernel: its leading arguments are the fields of P that the first loads need.
+template <class Kernel>
+void launch_gemv(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const GemvParams& P) {
+    kernel<<<grid, block, lds, stream>>>(P.w, P.x, P.y, P.m, P.n, P.k, P.k_groups, P.panel_bytes, P.row_tiles,
+                                         P.nwk | (P.nwr << 8) | (P.slots << 16) | (P.n_weights << 24), P.wave_magic, P);
 }
 
 // Waves per workgroup and their split: as many waves along k as there are
@@ -351,17 +394,27 @@ hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipS
     // grouped form), one row-tile group per workgroup, one k step
     constexpr bool kCanOneshot = GROUPED ? MT == QMM_MOE_SEG_ROWS : true;
     const bool oneshot = kCanOneshot && (GROUPED || P.m <= MT) && P.kpw == 1 && grid == P.rt_groups;
-    const void* fn = oneshot ? reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot, IO, NORM>)
-                             : reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, GROUPED, false, IO, NORM>);
-    if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-    }
     const dim3 g((unsigned)grid, (unsigned)grid_y), b(64 * all_waves);
-    if (oneshot)
-        gemv_kernel<QT, MT, GATED, GROUPED, kCanOneshot, IO, NORM><<<g, b, lds, stream>>>(P);
-    else
-        gemv_kernel<QT, MT, GATED, GROUPED, false, IO, NORM><<<g, b, lds, stream>>>(P);
+    if constexpr (GROUPED) {
+        static_assert(IO == 0 && !NORM, "the grouped form has no epilogue and no folded norm");
+        const void* fn = oneshot ? reinterpret_cast<const void*>(&gemv_grouped_kernel<QT, MT, GATED, kCanOneshot>)
+                                 : reinterpret_cast<const void*>(&gemv_grouped_kernel<QT, MT, GATED, false>);
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return e;
+        }
+        if (oneshot) gemv_grouped_kernel<QT, MT, GATED, kCanOneshot><<<g, b, lds, stream>>>(P);
+        else gemv_grouped_kernel<QT, MT, GATED, false><<<g, b, lds, stream>>>(P);
+    } else {
+        const void* fn = oneshot ? reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, false, kCanOneshot, IO, NORM>)
+                                 : reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, false, false, IO, NORM>);
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return e;
+        }
+        if (oneshot) launch_gemv(gemv_kernel<QT, MT, GATED, false, kCanOneshot, IO, NORM>, g, b, lds, stream, P);
+        else launch_gemv(gemv_kernel<QT, MT, GATED, false, false, IO, NORM>, g, b, lds, stream, P);
+    }
     return hipGetLastError();
 }
 
@@ -515,7 +568,7 @@ hipError_t launch_rows_mt(const GemvParams& P, int waves, int n_cus, hipStream_t
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
-    gemv_kernel<QT, MT, false, false, false, 0, false, true><<<dim3((unsigned)grid), dim3(64 * waves), lds, stream>>>(P);
+    launch_gemv(gemv_kernel<QT, MT, false, false, false, 0, false, true>, dim3((unsigned)grid), dim3(64 * waves), lds, stream, P);
     return hipGetLastError();
 }
 
@@ -661,11 +714,11 @@ hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* co
         if (norm) need += (size_t)mt * P.k_units * sizeof(float);
         if (need > 48 * 1024) return hipErrorNotSupported;
         if (norm) {
-            if (mt == 2) gemv_kernel<qt, 2, false, false, true, 0, true><<<g, b, need, stream>>>(P);
-            else gemv_kernel<qt, 1, false, false, true, 0, true><<<g, b, need, stream>>>(P);
+            if (mt == 2) launch_gemv(gemv_kernel<qt, 2, false, false, true, 0, true>, g, b, need, stream, P);
+            else launch_gemv(gemv_kernel<qt, 1, false, false, true, 0, true>, g, b, need, stream, P);
         } else {
-            if (mt == 2) gemv_kernel<qt, 2, false, false, true><<<g, b, need, stream>>>(P);
-            else gemv_kernel<qt, 1, false, false, true><<<g, b, need, stream>>>(P);
+            if (mt == 2) launch_gemv(gemv_kernel<qt, 2, false, false, true>, g, b, need, stream, P);
+            else launch_gemv(gemv_kernel<qt, 1, false, false, true>, g, b, need, stream, P);
         }
         return hipGetLastError();
     });

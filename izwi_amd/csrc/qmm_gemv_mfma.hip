@@ -197,6 +197,49 @@ struct MfmaParams {
     QmmEpilogue ep;
 };
 
+// The matrix-core kernels take the fields that their first loads need as leading scalar arguments
+// (14 dwords): those arrive in scalar registers with the wave (kernel-argument preload), the
+// rest of the parameter block is read from memory.  with_leading_args puts them back into a
+// copy of the block; the tables of a group of weights are indexed in the block itself (P0).
+__device__ __forceinline__ MfmaParams with_leading_args(const MfmaParams& P0, const uint8_t* w, const uint8_t* ws, float* y,
+                                                        int k_units, int k_groups, int row_tiles, int panel_bytes,
+                                                        int split, int wave_magic, int n_tiles, int window) {
+    MfmaParams P = P0;
+    P.w = w, P.ws = ws, P.y = y, P.k_units = k_units, P.k_groups = k_groups, P.row_tiles = row_tiles;
+    P.panel_bytes = panel_bytes, P.wave_magic = wave_magic, P.n_tiles = n_tiles;
+    P.nwk = split & 255, P.nwr = (split >> 8) & 255, P.slots = (split >> 16) & 255, P.n_weights = split >> 24;
+    P.window_units = window & 0xffff, P.double_buf = window >> 16;
+    return P;
+}
+
+template <class Kernel>
+void launch_mfma(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const MfmaParams& P) {
+    kernel<<<grid, block, lds, stream>>>(P.w, P.ws, P.y, P.k_units, P.k_groups, P.row_tiles, P.panel_bytes,
+                                         P.nwk | (P.nwr << 8) | (P.slots << 16) | (P.n_weights << 24), P.wave_magic, P.n_tiles,
+                                         P.window_units | (P.double_buf << 16), P);
+}
+
+// The entry of a group of weights for workgroup b: the tables are read whole (independent scalar
+// loads, one round trip) and the entry is picked with selects; rtg_end ascends, so the entry is
+// the number of ends at or below b.  Entries past n_weights hold whatever the host left there
+// and are never picked.
+__device__ __forceinline__ void pick_group_entry(const MfmaParams& P0, int n_weights, int b, int& rtg, const uint8_t*& wbase,
+                                                 float*& yout, int& n_rows, int& row_tiles) {
+    static_assert(QMM_MAX_GROUP == 4, "the selects below name four entries");
+    const int e0 = P0.rtg_end[0], e1 = P0.rtg_end[1], e2 = P0.rtg_end[2];
+    const bool c1 = b >= e0, c2 = n_weights > 2 && b >= e1, c3 = n_weights > 3 && b >= e2;
+    auto pick = [c1, c2, c3](auto v0, auto v1, auto v2, auto v3) {
+        auto v = c1 ? v1 : v0;
+        v = c2 ? v2 : v;
+        return c3 ? v3 : v;
+    };
+    rtg = b - pick(0, e0, e1, e2);
+    wbase = pick(P0.wv[0], P0.wv[1], P0.wv[2], P0.wv[3]);
+    yout = pick(P0.yv[0], P0.yv[1], P0.yv[2], P0.yv[3]);
+    n_rows = pick(P0.nv[0], P0.nv[1], P0.nv[2], P0.nv[3]);
+    row_tiles = pick(P0.row_tiles_v[0], P0.row_tiles_v[1], P0.row_tiles_v[2], P0.row_tiles_v[3]);
+}
+
 // 4x4 transpose of one dword between the four 16-lane rows: on entry row u
 // holds X_u[t] in r[t]; on exit row t holds X_u[t] in r[u].
 __device__ __forceinline__ void transpose_rows(uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3) {
@@ -576,8 +619,8 @@ __device__ __forceinline__ void issue_window_copy(const uint8_t* __restrict__ sr
 // EP: the sums go through the epilogue of P.ep (residual add, f32 or bf16 store).
 // (the compact single-stage Q4_K form is held to the 80 registers of six waves per SIMD: two 12-wave
 // workgroups per CU keep every panel of gate | up in flight at once)
-template <int QT, bool SINGLE, bool GROUPED = false, bool EP = false, int NU = 0>
-__global__ __launch_bounds__(64 * kMaxWaves, (QT == QMM_Q4_K && SINGLE && NU == 0) ? 6 : 3) void gemv_mfma_oneshot_kernel(MfmaParams P) {
+template <int QT, bool SINGLE, bool GROUPED, bool EP, int NU>
+__device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaParams& P0) {
     constexpr int UB = Unit<QT>::kBytes;
     constexpr int NL = WPanel<QT>::kLoads; // loads of one panel
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -611,15 +654,7 @@ __global__ __launch_bounds__(64 * kMaxWaves, (QT == QMM_Q4_K && SINGLE && NU == 
         g_stack = within / P.rt_groups;
         rtg = within - g_stack * P.rt_groups;
     }
-    if (SINGLE && !GROUPED && P.n_weights > 1) {
-        int i = 0;
-        while (i + 1 < P.n_weights && (int)blockIdx.x >= P.rtg_end[i]) i++;
-        rtg = blockIdx.x - (i ? P.rtg_end[i - 1] : 0);
-        wbase = P.wv[i];
-        yout = P.yv[i];
-        n_rows = P.nv[i];
-        row_tiles = P.row_tiles_v[i];
-    }
+    if (SINGLE && !GROUPED && P.n_weights > 1) pick_group_entry(P0, P.n_weights, blockIdx.x, rtg, wbase, yout, n_rows, row_tiles);
     const int rt = rtg * P.nwr + wr;
     const bool rt_ok = rt < row_tiles;
     const int unit0 = wk * s_units;                       // first unit of this wave's panel
@@ -758,6 +793,24 @@ __global__ __launch_bounds__(64 * kMaxWaves, (QT == QMM_Q4_K && SINGLE && NU == 
         tile = ntile, win = nwin;
     }
 }
+// The dense launches of the one-shot form: leading scalar arguments (see with_leading_args).
+template <int QT, bool SINGLE, bool GROUPED = false, bool EP = false, int NU = 0>
+__global__ __launch_bounds__(64 * kMaxWaves, (QT == QMM_Q4_K && SINGLE && NU == 0) ? 6 : 3) void gemv_mfma_oneshot_kernel(
+        const uint8_t* w_arg, const uint8_t* ws_arg, float* y_arg, int k_units_arg, int k_groups_arg, int row_tiles_arg, int panel_bytes_arg,
+        int split_arg, int wave_magic_arg, int n_tiles_arg, int window_arg, MfmaParams P0) {
+    static_assert(!GROUPED, "the expert-grouped launches go through gemv_mfma_grouped_kernel");
+    const MfmaParams P = with_leading_args(P0, w_arg, ws_arg, y_arg, k_units_arg, k_groups_arg, row_tiles_arg, panel_bytes_arg, split_arg,
+                                             wave_magic_arg, n_tiles_arg, window_arg);
+    oneshot_body<QT, SINGLE, false, EP, NU>(P, P0);
+}
+
+// The expert-grouped launches: thousands of short workgroups, whose waves start faster with
+// fewer scalar registers to fill (measured: the grouped one-row kernels lost 1 us of 19 - 30
+// with preloaded arguments), so the parameter block stays one block in memory.
+template <int QT, int NU = 0>
+__global__ __launch_bounds__(64 * kMaxWaves, 3) void gemv_mfma_grouped_kernel(MfmaParams P) {
+    oneshot_body<QT, false, true, false, NU>(P, P);
+}
 
 // Register-direct form (Q4_K, one row tile of activations, one row-tile of weights per
 // workgroup): wave wk multiplies panel wk, which needs only units 4 wk .. 4 wk + 3 of the
@@ -776,7 +829,11 @@ __device__ __forceinline__ void panel_dot_direct_q4k(WPanel<QMM_Q4_K>& p, const 
 }
 
 template <bool EP = false, int NU = 0>
-__global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(MfmaParams P) {
+__global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(
+        const uint8_t* w_arg, const uint8_t* ws_arg, float* y_arg, int k_units_arg, int k_groups_arg, int row_tiles_arg, int panel_bytes_arg,
+        int split_arg, int wave_magic_arg, int n_tiles_arg, int window_arg, MfmaParams P0) {
+    const MfmaParams P = with_leading_args(P0, w_arg, ws_arg, y_arg, k_units_arg, k_groups_arg, row_tiles_arg, panel_bytes_arg, split_arg,
+                                             wave_magic_arg, n_tiles_arg, window_arg);
     constexpr int QT = QMM_Q4_K;
     constexpr int UB = Unit<QT>::kBytes;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -791,15 +848,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(Mf
     const uint8_t* wbase = P.w;
     float* yout = P.y;
     int n_rows = P.n, row_tiles = P.row_tiles, rtg = blockIdx.x;
-    if (P.n_weights > 1) {
-        int i = 0;
-        while (i + 1 < P.n_weights && (int)blockIdx.x >= P.rtg_end[i]) i++;
-        rtg = blockIdx.x - (i ? P.rtg_end[i - 1] : 0);
-        wbase = P.wv[i];
-        yout = P.yv[i];
-        n_rows = P.nv[i];
-        row_tiles = P.row_tiles_v[i];
-    }
+    if (P.n_weights > 1) pick_group_entry(P0, P.n_weights, blockIdx.x, rtg, wbase, yout, n_rows, row_tiles);
     const int rt = rtg * P.nwr + wr;
     const bool rt_ok = rt < row_tiles;
     const int unit0 = wk * s_units;
@@ -1106,8 +1155,8 @@ hipError_t launch_dense_form(int form, const MfmaParams& P, unsigned grid, int w
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
     }
-    if (form == 0) gemv_mfma_oneshot_kernel<QT, true, false, EP><<<grid, 64 * waves, lds, stream>>>(P);
-    else if (form == 1) gemv_mfma_oneshot_kernel<QT, false, false, EP><<<grid, 64 * waves, lds, stream>>>(P);
+    if (form == 0) launch_mfma(gemv_mfma_oneshot_kernel<QT, true, false, EP>, grid, 64 * waves, lds, stream, P);
+    else if (form == 1) launch_mfma(gemv_mfma_oneshot_kernel<QT, false, false, EP>, grid, 64 * waves, lds, stream, P);
     else gemv_mfma_stream_kernel<QT, EP><<<grid, 64 * waves, lds, stream>>>(P);
     return hipGetLastError();
 }
@@ -1177,7 +1226,7 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     const int n_tiles = (int)((m + 15) / 16);
     uint8_t* ws = (uint8_t*)workspace;
     const bool epilogue = io && (io->residual || io->y_bf16);
-    MfmaParams P;
+    MfmaParams P{};
     P.ep = QmmEpilogue{nullptr, 0};
     if (io) P.ep = QmmEpilogue{io->residual, io->y_bf16};
     P.window_units = (kWindowUnits / L.s) * L.s;
@@ -1245,11 +1294,11 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     if (oneshot && direct_form_applies(L.dtype, n_tiles, P.nwr, L.k_units <= P.window_units)) {
         const size_t red = (size_t)waves * 256 * 4;
         if (full_panels(L)) {
-            if (epilogue) gemv_mfma_direct_q4k_kernel<true, 4><<<grid, 64 * waves, red, stream>>>(P);
-            else gemv_mfma_direct_q4k_kernel<false, 4><<<grid, 64 * waves, red, stream>>>(P);
+            if (epilogue) launch_mfma(gemv_mfma_direct_q4k_kernel<true, 4>, grid, 64 * waves, red, stream, P);
+            else launch_mfma(gemv_mfma_direct_q4k_kernel<false, 4>, grid, 64 * waves, red, stream, P);
         } else {
-            if (epilogue) gemv_mfma_direct_q4k_kernel<true><<<grid, 64 * waves, red, stream>>>(P);
-            else gemv_mfma_direct_q4k_kernel<false><<<grid, 64 * waves, red, stream>>>(P);
+            if (epilogue) launch_mfma(gemv_mfma_direct_q4k_kernel<true>, grid, 64 * waves, red, stream, P);
+            else launch_mfma(gemv_mfma_direct_q4k_kernel<false>, grid, 64 * waves, red, stream, P);
         }
         return hipGetLastError();
     }
@@ -1263,8 +1312,8 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
             hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return e;
         }
-        if (epilogue) gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, true, 4><<<grid, 64 * waves, lds, stream>>>(P);
-        else gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4><<<grid, 64 * waves, lds, stream>>>(P);
+        if (epilogue) launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, true, 4>, grid, 64 * waves, lds, stream, P);
+        else launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4>, grid, 64 * waves, lds, stream, P);
         return hipGetLastError();
     }
     if (L.dtype == QMM_Q4_K && form == 1 && full_panels(L)) {
@@ -1275,8 +1324,8 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
             hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return e;
         }
-        if (epilogue) gemv_mfma_oneshot_kernel<QMM_Q4_K, false, false, true, 4><<<grid, 64 * waves, lds, stream>>>(P);
-        else gemv_mfma_oneshot_kernel<QMM_Q4_K, false, false, false, 4><<<grid, 64 * waves, lds, stream>>>(P);
+        if (epilogue) launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q4_K, false, false, true, 4>, grid, 64 * waves, lds, stream, P);
+        else launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q4_K, false, false, false, 4>, grid, 64 * waves, lds, stream, P);
         return hipGetLastError();
     }
     if (L.dtype == QMM_Q4_K)
@@ -1323,7 +1372,7 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     if (L.n == 0 || n_experts <= 0) return hipSuccess;
     if (!qmm_gemv_mfma_grouped_supported(L) || n_experts > 65535 || L.n > 0x3fffffff)
         return hipErrorInvalidValue;
-    MfmaParams P;
+    MfmaParams P{};
     P.ep = QmmEpilogue{nullptr, 0};
     P.w = (const uint8_t*)tiled;
     P.ws = (const uint8_t*)records;
@@ -1401,10 +1450,10 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     const size_t lds = (P.double_buf ? 2 : 1) * window_bytes + red_bytes;
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     const void* fn = L.dtype == QMM_Q4_K
-                         ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true>)
+                         ? reinterpret_cast<const void*>(&gemv_mfma_grouped_kernel<QMM_Q4_K>)
                          : L.dtype == QMM_Q6_K
-                               ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q6_K, false, true>)
-                               : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, false, true>);
+                               ? reinterpret_cast<const void*>(&gemv_mfma_grouped_kernel<QMM_Q6_K>)
+                               : reinterpret_cast<const void*>(&gemv_mfma_grouped_kernel<QMM_Q8_0>);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
@@ -1414,22 +1463,22 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     const unsigned grid = (unsigned)(((n_experts + 7) / 8) * 8 * P.rt_groups * P.stacks);
     const int nu = L.dtype == QMM_Q4_K ? uniform_panel_units(L) : 0;
     if (nu == 4 || nu == 3) {
-        const void* fp = nu == 4 ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true, false, 4>)
-                                 : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true, false, 3>);
+        const void* fp = nu == 4 ? reinterpret_cast<const void*>(&gemv_mfma_grouped_kernel<QMM_Q4_K, 4>)
+                                 : reinterpret_cast<const void*>(&gemv_mfma_grouped_kernel<QMM_Q4_K, 3>);
         if (lds > 48 * 1024) {
             hipError_t e = hipFuncSetAttribute(fp, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return e;
         }
-        if (nu == 4) gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true, false, 4><<<grid, 64 * waves, lds, stream>>>(P);
-        else gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true, false, 3><<<grid, 64 * waves, lds, stream>>>(P);
+        if (nu == 4) gemv_mfma_grouped_kernel<QMM_Q4_K, 4><<<grid, 64 * waves, lds, stream>>>(P);
+        else gemv_mfma_grouped_kernel<QMM_Q4_K, 3><<<grid, 64 * waves, lds, stream>>>(P);
         return hipGetLastError();
     }
     if (L.dtype == QMM_Q4_K)
-        gemv_mfma_oneshot_kernel<QMM_Q4_K, false, true><<<grid, 64 * waves, lds, stream>>>(P);
+        gemv_mfma_grouped_kernel<QMM_Q4_K><<<grid, 64 * waves, lds, stream>>>(P);
     else if (L.dtype == QMM_Q6_K)
-        gemv_mfma_oneshot_kernel<QMM_Q6_K, false, true><<<grid, 64 * waves, lds, stream>>>(P);
+        gemv_mfma_grouped_kernel<QMM_Q6_K><<<grid, 64 * waves, lds, stream>>>(P);
     else
-        gemv_mfma_oneshot_kernel<QMM_Q8_0, false, true><<<grid, 64 * waves, lds, stream>>>(P);
+        gemv_mfma_grouped_kernel<QMM_Q8_0><<<grid, 64 * waves, lds, stream>>>(P);
     return hipGetLastError();
 }
 
@@ -1446,7 +1495,7 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
             return hipErrorInvalidValue;
         total_row_tiles += L.row_tiles;
     }
-    MfmaParams P;
+    MfmaParams P{};
     P.ep = QmmEpilogue{nullptr, 0};
     P.w = (const uint8_t*)tiled[0];
     P.ws = (const uint8_t*)workspace;
@@ -1493,8 +1542,8 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
     P.rt_groups = (int)groups;
     const int waves = P.nwk * P.nwr;
     if (direct_form_applies(L0.dtype, 1, P.nwr, true)) {
-        if (full_panels(L0)) gemv_mfma_direct_q4k_kernel<false, 4><<<(unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
-        else gemv_mfma_direct_q4k_kernel<false><<<(unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream>>>(P);
+        if (full_panels(L0)) launch_mfma(gemv_mfma_direct_q4k_kernel<false, 4>, (unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream, P);
+        else launch_mfma(gemv_mfma_direct_q4k_kernel<false>, (unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream, P);
         return hipGetLastError();
     }
     const size_t lds = std::max((size_t)P.window_units * unit_bytes(L0.dtype), (size_t)waves * 256 * 4);
@@ -1509,12 +1558,12 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
         if (e != hipSuccess) return e;
     }
     if (full)
-        gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4><<<(unsigned)groups, 64 * waves, lds, stream>>>(P);
+        launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4>, (unsigned)groups, 64 * waves, lds, stream, P);
     else if (L0.dtype == QMM_Q4_K)
-        gemv_mfma_oneshot_kernel<QMM_Q4_K, true><<<(unsigned)groups, 64 * waves, lds, stream>>>(P);
+        launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q4_K, true>, (unsigned)groups, 64 * waves, lds, stream, P);
     else if (L0.dtype == QMM_Q6_K)
-        gemv_mfma_oneshot_kernel<QMM_Q6_K, true><<<(unsigned)groups, 64 * waves, lds, stream>>>(P);
+        launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q6_K, true>, (unsigned)groups, 64 * waves, lds, stream, P);
     else
-        gemv_mfma_oneshot_kernel<QMM_Q8_0, true><<<(unsigned)groups, 64 * waves, lds, stream>>>(P);
+        launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q8_0, true>, (unsigned)groups, 64 * waves, lds, stream, P);
     return hipGetLastError();
 }
