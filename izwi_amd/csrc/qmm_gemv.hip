@@ -47,7 +47,7 @@ struct GemvParams {
     int nwk, nwr;
     int wave_magic; // ceil(65536 / nwk): wave / nwk == (wave * wave_magic) >> 16
     // ---- 64 bytes ----
-    int k_units, s;
+    int k_units;
     const uint8_t* w2; // gated form only: the second stack ("up"), same layout as w
     int64_t matrix_bytes;
     int kpw;        // ceil(k_groups / nwk): panels per row-tile for every wave
@@ -96,7 +96,8 @@ __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 // moves), the row's factor rsqrt(mean(x^2) + eps) multiplies the finished sums instead.
 template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT, int IO = 0, bool NORM = false, bool TILEMAP = false>
 __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int m_end, const uint8_t* w_first,
-                                          float* y_out, int n_rows, int row_tiles, int rtg0, uint8_t* smem) {
+                                          float* y_out, int n_rows, int row_tiles, int rtg0, uint8_t* smem,
+                                          int item_bias = 0) {
     constexpr bool XB = IO == 2, EP = IO != 0;
     const int lane0 = threadIdx.x & 63;
     // wave-uniform by construction; said so, the row-tile, panel offset and output row that
@@ -119,7 +120,9 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
         int red_buf = 0;
         for (int rtg = rtg0; ONESHOT ? rtg == rtg0 : rtg < P.rt_groups;
              rtg += ONESHOT ? 1 : (int)gridDim.x) {
-            const int rt = rtg * P.nwr + wr;
+            // the wave's row-tile (item_bias: a group launch counts its row-tiles over all weights and
+            // this is minus the first one of the wave's weight; uniform)
+            const int rt = rtg * P.nwr + wr + item_bias;
             // the weight's row-tile behind this one (uniform: a scalar load)
             const int rt_w = TILEMAP ? P.tile_ids[rt < row_tiles ? rt : 0] : rt;
             float acc[MT];
@@ -283,13 +286,18 @@ __device__ __forceinline__ void gemv_entry(const GemvParams& P, const GemvParams
     const uint8_t* w_first = P.w + w_offset;
     float* y_out = P.y;
     int n_rows = P.n, row_tiles = P.row_tiles, rtg0 = blockIdx.x;
-    if (!GROUPED && ONESHOT && n_weights > 1) {
-        // The tables are read whole (independent scalar loads, one round trip) and the
-        // workgroup's entry is picked with selects; rtg_end ascends, so the entry is the
-        // number of ends at or below the workgroup index.  Entries past n_weights hold
-        // whatever the host left there and are never picked.
+    int item_bias = 0;
+    if (!GROUPED && !GATED && ONESHOT && n_weights > 1) {
+        // A group of weights: the launch's row-tiles are counted over all weights, rtg_end[i] = the
+        // end of weight i's row-tiles, and every WAVE finds the weight of its own row-tile (a
+        // workgroup may straddle two weights; its waves only share the quantized
+        // activations and the LDS of the k-split).  The tables are read whole (independent scalar
+        // loads, one round trip) and the entry is picked with selects; rtg_end ascends, so the entry
+        // is the number of ends at or below the row-tile's index.  Entries past n_weights hold whatever
+        // the host left there and are never picked.
         static_assert(QMM_MAX_GROUP == 4, "the selects below name four entries");
-        const int b = blockIdx.x;
+        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const int b = blockIdx.x * P.nwr + ((wave * P.wave_magic) >> 16);
         const int e0 = P0.rtg_end[0], e1 = P0.rtg_end[1], e2 = P0.rtg_end[2];
         const bool c1 = b >= e0, c2 = n_weights > 2 && b >= e1, c3 = n_weights > 3 && b >= e2;
         auto pick = [c1, c2, c3](auto v0, auto v1, auto v2, auto v3) {
@@ -297,7 +305,7 @@ __device__ __forceinline__ void gemv_entry(const GemvParams& P, const GemvParams
             v = c2 ? v2 : v;
             return c3 ? v3 : v;
         };
-        rtg0 = b - pick(0, e0, e1, e2);
+        item_bias = -pick(0, e0, e1, e2);
         w_first = pick(P0.wv[0], P0.wv[1], P0.wv[2], P0.wv[3]);
         y_out = pick(P0.yv[0], P0.yv[1], P0.yv[2], P0.yv[3]);
         n_rows = pick(P0.nv[0], P0.nv[1], P0.nv[2], P0.nv[3]);
@@ -312,7 +320,7 @@ __device__ __forceinline__ void gemv_entry(const GemvParams& P, const GemvParams
         else
             gemv_body<QT, 4, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     } else {
-        gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO, NORM, TILEMAP>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
+        gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO, NORM, TILEMAP>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem, item_bias);
     }
 }
 
@@ -362,7 +370,12 @@ void choose_split(const QmmLayout& L, int n_cus, int grid_y, bool gated, GemvPar
     const int budget = gated ? total / 2 : total;
     int nwk = (int)(L.k_groups < budget ? L.k_groups : budget);
     int nwr_max = budget / nwk;
-    int64_t want = L.row_tiles * grid_y / (n_cus > 0 ? n_cus : 1);
+    // Dense launches: as few workgroups as CUs where the waves allow it, i.e. ceil(row-tiles / CUs)
+    // row-tiles side by side (measured, k = 4096, one row: 384 row-tiles as 192 workgroups of two
+    // 5.05 us, as 384 of one 5.78 - the second workgroup of a CU starts late and quantizes the
+    // activations again; 576..704 row-tiles as workgroups of three 6.3 - 7.0 us, of two 6.9 - 7.5).
+    const int64_t cus = n_cus > 0 ? n_cus : 1;
+    int64_t want = grid_y == 1 ? (L.row_tiles + cus - 1) / cus : L.row_tiles * grid_y / cus;
     int nwr = (int)(want < 1 ? 1 : (want > nwr_max ? nwr_max : want));
     // More than one full workgroup per CU (gate|up group): the register count lets 20 waves
     // share a CU, so two 8-wave workgroups run side by side (one loads while the other
@@ -469,7 +482,6 @@ bool make_params(const QmmLayout& L, const void* tiled, const float* x, int64_t 
     P.k = (int)L.k;
     P.k_units = (int)L.k_units;
     P.k_groups = (int)L.k_groups;
-    P.s = L.s;
     P.slots = L.slots;
     P.row_tiles = (int)L.row_tiles;
     P.panel_bytes = (int)L.panel_bytes;
@@ -692,17 +704,18 @@ hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* co
     choose_split(all, n_cus, 1, false, P, waves);
     if (P.kpw != 1) return hipErrorNotSupported;
     P.n_weights = n_weights;
-    int64_t groups = 0;
+    int64_t tiles_all = 0;
     for (int i = 0; i < n_weights; i++) {
         const QmmLayout& L = *layouts[i];
         if (L.n > 0x3fffffff) return hipErrorInvalidValue;
-        groups += (L.row_tiles + P.nwr - 1) / P.nwr;
-        P.rtg_end[i] = (int)groups;
+        tiles_all += L.row_tiles;
+        P.rtg_end[i] = (int)tiles_all; // in row-tiles, not workgroups: see the kernel
         P.nv[i] = (int)L.n;
         P.row_tiles_v[i] = (int)L.row_tiles;
         P.wv[i] = (const uint8_t*)tiled[i];
         P.yv[i] = ys[i];
     }
+    const int64_t groups = (tiles_all + P.nwr - 1) / P.nwr;
     if (groups > (int64_t)n_cus * 32) return hipErrorNotSupported;
     P.rt_groups = (int)groups;
     const int mt = m == 2 ? 2 : 1;
