@@ -654,7 +654,7 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
         g_stack = within / P.rt_groups;
         rtg = within - g_stack * P.rt_groups;
     }
-    if (SINGLE && !GROUPED && P.n_weights > 1) pick_group_entry(P0, P.n_weights, blockIdx.x, rtg, wbase, yout, n_rows, row_tiles);
+    if (!GROUPED && P.n_weights > 1) pick_group_entry(P0, P.n_weights, blockIdx.x, rtg, wbase, yout, n_rows, row_tiles);
     const int rt = rtg * P.nwr + wr;
     const bool rt_ok = rt < row_tiles;
     const int unit0 = wk * s_units;                       // first unit of this wave's panel
@@ -1273,7 +1273,7 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     if (oneshot) {
         P.nwk = (int)L.k_groups;
         int nwr_max = kMaxWaves / P.nwk;
-        int64_t want = L.row_tiles / n_cus;
+        int64_t want = (L.row_tiles + n_cus - 1) / n_cus; // as few workgroups as CUs where the waves allow it
         P.nwr = (int)(want < 1 ? 1 : (want > nwr_max ? nwr_max : want));
         waves = P.nwk * P.nwr;
         P.rt_groups = (int)((L.row_tiles + P.nwr - 1) / P.nwr);
@@ -1507,7 +1507,6 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
     P.slots = L0.slots;
     P.row_tiles = (int)L0.row_tiles;
     P.panel_bytes = (int)L0.panel_bytes;
-    P.n_tiles = 1;
     P.perm = nullptr;
     P.offsets = nullptr;
     P.tile_offsets = nullptr;
@@ -1520,12 +1519,16 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
     P.window_units = (kWindowUnits / L0.s) * L0.s;
     const int padded_units = (int)(L0.k_groups * L0.s);
     if (P.window_units > padded_units) P.window_units = padded_units;
-    // the straight-line form only: one row tile, one window, one wave per panel of a row-tile
-    if (m > 16 || L0.k_units > P.window_units || L0.k_groups > kMaxWaves || total_row_tiles >= 8 * (int64_t)n_cus)
+    // the one-shot forms with one window: one wave per panel of a row-tile, up to four tiles of rows
+    if (m > 64 || L0.k_units > P.window_units || L0.k_groups > kMaxWaves || total_row_tiles >= 8 * (int64_t)n_cus)
         return hipErrorNotSupported;
+    const int n_tiles = (int)((m + 15) / 16);
+    P.n_tiles = n_tiles;
     P.nwk = (int)L0.k_groups;
     const int nwr_max = kMaxWaves / P.nwk;
-    const int64_t want = total_row_tiles / n_cus;
+    // as few workgroups as CUs where the waves allow it (q|k|v of the 8B shapes, 384 row-tiles: 7.3 us as
+    // 192 workgroups of two row-tiles, 7.5 - 7.7 as 384 of one)
+    const int64_t want = (total_row_tiles + n_cus - 1) / n_cus;
     P.nwr = (int)(want < 1 ? 1 : (want > nwr_max ? nwr_max : want));
     P.wave_magic = (65536 + P.nwk - 1) / P.nwk;
     P.n_weights = n_weights;
@@ -1541,6 +1544,27 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
     }
     P.rt_groups = (int)groups;
     const int waves = P.nwk * P.nwr;
+    if (n_tiles > 1) {
+        // several tiles of rows against a resident panel (the form of the single-weight call at these m)
+        const size_t window_bytes = (size_t)P.window_units * unit_bytes(L0.dtype), red_bytes = (size_t)waves * 256 * 4;
+        P.double_buf = 2 * window_bytes + red_bytes <= 160 * 1024;
+        const size_t lds = (P.double_buf ? 2 : 1) * window_bytes + red_bytes;
+        if (lds > 160 * 1024) return hipErrorNotSupported;
+        const bool prepared = L0.dtype == QMM_Q4_K && full_panels(L0);
+        const void* fn = prepared               ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false, false, false, 4>)
+                         : L0.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, false>)
+                         : L0.dtype == QMM_Q6_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q6_K, false>)
+                                                : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q8_0, false>);
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return e;
+        }
+        if (prepared) launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q4_K, false, false, false, 4>, (unsigned)groups, 64 * waves, lds, stream, P);
+        else if (L0.dtype == QMM_Q4_K) launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q4_K, false>, (unsigned)groups, 64 * waves, lds, stream, P);
+        else if (L0.dtype == QMM_Q6_K) launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q6_K, false>, (unsigned)groups, 64 * waves, lds, stream, P);
+        else launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q8_0, false>, (unsigned)groups, 64 * waves, lds, stream, P);
+        return hipGetLastError();
+    }
     if (direct_form_applies(L0.dtype, 1, P.nwr, true)) {
         if (full_panels(L0)) launch_mfma(gemv_mfma_direct_q4k_kernel<false, 4>, (unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream, P);
         else launch_mfma(gemv_mfma_direct_q4k_kernel<false>, (unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream, P);

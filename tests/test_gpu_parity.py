@@ -560,6 +560,24 @@ def test_projection_group_equals_separate_calls(qa, oracle, dtype, m):
 
 
 @pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
+@pytest.mark.parametrize("m", [17, 32, 33, 64])
+@pytest.mark.parametrize("k,ns", [(4096, (4096, 1024, 1024)), (2048, (1536, 1536)), (768, (2000, 48, 16, 512))])
+def test_projection_group_on_several_row_tiles(qa, oracle, dtype, m, k, ns):
+    """17 <= m <= 64 (two to four 16-row tiles of activations): the group is one launch of the
+    batched decode kernel's several-tiles form and equals the separate forwards bit for bit."""
+    _say(f"group tiles dtype={dtype} m={m} k={k} ns={ns}")
+    dt = qa.GgmlDType(dtype)
+    blocks = [make_weight(oracle, dtype, n, k, 700 + n + i) for i, n in enumerate(ns)]
+    parts = [qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, b, (n, k))) for b, n in zip(blocks, ns)]
+    x = torch.from_numpy(oracle.randn(701 + m, (m, k))).cuda()
+    outs = qa.forward_group(parts, x)
+    for got, p in zip(outs, parts):
+        assert torch.equal(got, p.forward(x))
+    want = oracle.qmatmul(dtype, x.cpu().numpy(), blocks[-1], ns[-1])
+    assert rel_err(outs[-1].cpu().numpy(), want) < DECODE_TOL
+
+
+@pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
 @pytest.mark.parametrize("m,k,ns", [(512, 4096, (4096, 1024, 1024)), (2048, 4096, (4096, 1024, 1024)),
                                     (300, 768, (300, 200)), (200, 1024, (2048, 1000, 16, 512)), (129, 256, (256, 256))])
 def test_projection_group_at_prefill_sizes(qa, oracle, dtype, m, k, ns):
