@@ -310,8 +310,8 @@ int izwi_qmm_forward_f32_noalloc(const izwi_qmm_weight* w, const float* x, int64
  * activations, y_i = QMatMul_i.forward(x), bit-identical to n_weights calls of
  * izwi_qmm_forward_f32 up to 128 rows (beyond, in the bf16 matrix-core arithmetic, equal up to the
  * f32 summation order: the shared launch may split k differently).  The weights must share k; with equal block types the decode
- * sizes run as one kernel launch (m <= 2) or share one activation quantization
- * (m <= 64), prefill sizes (m > 128, bf16 matrix-core arithmetic) share one conversion of x
+ * sizes run as one kernel launch (m <= 2) or as one activation quantization and one
+ * matmul launch (m <= 64), prefill sizes (m > 128, bf16 matrix-core arithmetic) share one conversion of x
  * and one launch; members of several block types (attn_q / attn_k in Q4_K beside attn_v in
  * Q6_K, as Q4_K_M files have them) are grouped by type, one such launch per type.
  * n_weights <= 4. */
