@@ -1417,7 +1417,13 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
             const int stacks = tiled2 ? 2 : 1;
             int waves = kExpertWaves;
             if (waves > L.row_tiles) waves = (int)L.row_tiles;
-            static const int wgs_per_cu = [] { const char* e = getenv("IZWI_QMM_MOE_EXPERT_WGS_PER_CU"); int v = e ? atoi(e) : 2; return v > 0 ? v : 2; }();
+            // Workgroups per CU: one while the experts hold about one or two tiles (all of an expert's rows
+            // in one workgroup: its tiles are copied once), two from there on (the tile counts differ more
+            // from expert to expert and a second workgroup evens the CUs out).  Measured per layer at 128
+            // experts, top-8, one / two per CU: 109 / 115 us at 64 tokens, 113 / 119 at 128, 150 / 154
+            // at 256, 190 / 189 at 384, 223 / 216 at 512.  IZWI_QMM_MOE_EXPERT_WGS_PER_CU forces it.
+            static const int forced_wgs_per_cu = [] { const char* e = getenv("IZWI_QMM_MOE_EXPERT_WGS_PER_CU"); int v = e ? atoi(e) : 0; return v > 0 ? v : 0; }();
+            const int wgs_per_cu = forced_wgs_per_cu ? forced_wgs_per_cu : (pairs <= (int64_t)20 * n_experts ? 1 : 2);
             int parts = (wgs_per_cu * n_cus + n_experts * stacks - 1) / (n_experts * stacks);
             const int max_parts = (int)((L.row_tiles + waves - 1) / waves);
             if (parts > max_parts) parts = max_parts;
