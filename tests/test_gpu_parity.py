@@ -560,6 +560,26 @@ def test_projection_group_equals_separate_calls(qa, oracle, dtype, m):
 
 
 @pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
+@pytest.mark.parametrize("m", [1, 2, 3, 16])
+@pytest.mark.parametrize("k,ns", [(1024, (4000, 1000, 600)), (4096, (4096, 1000, 1048)), (2048, (3000, 3000, 3000, 200)),
+                                  (1024, (16, 8200))])
+def test_projection_group_workgroups_straddle_weights(qa, oracle, dtype, m, k, ns):
+    """More row-tiles than CUs: a workgroup takes several row-tiles, the launch's row-tiles are
+    counted over all weights and a workgroup may hold the last row-tile of one weight beside the
+    first of the next (m <= 2); every output equals the separate forward bit for bit."""
+    _say(f"group straddle dtype={dtype} m={m} k={k} ns={ns}")
+    dt = qa.GgmlDType(dtype)
+    blocks = [make_weight(oracle, dtype, n, k, 900 + n + i) for i, n in enumerate(ns)]
+    parts = [qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, b, (n, k))) for b, n in zip(blocks, ns)]
+    x = torch.from_numpy(oracle.randn(901 + m, (m, k))).cuda()
+    outs = qa.forward_group(parts, x)
+    for got, p in zip(outs, parts):
+        assert torch.equal(got, p.forward(x))
+    want = oracle.qmatmul(dtype, x.cpu().numpy(), blocks[1], ns[1])
+    assert rel_err(outs[1].cpu().numpy(), want) < DECODE_TOL
+
+
+@pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
 @pytest.mark.parametrize("m", [17, 32, 33, 64])
 @pytest.mark.parametrize("k,ns", [(4096, (4096, 1024, 1024)), (2048, (1536, 1536)), (768, (2000, 48, 16, 512))])
 def test_projection_group_on_several_row_tiles(qa, oracle, dtype, m, k, ns):
