@@ -483,6 +483,43 @@ def hbm_ceiling_extra(torch, gib=2, reps=10):
     return out
 
 
+def read_only_floor_extra(torch, qa, dtype, weights, m, steps=10, warmup=3):
+    """Extra report (not `value`): the same step with every launch replaced by a launch that only
+    READS as many bytes (izwi_qmm_probe_stream_read over its own buffers, one per call of the
+    headline structure: q|k|v, o, gate|up, down per layer + LM head; distinct buffers, one graph,
+    the same dependent chain of 145 launches).  What plain reads of the same bytes in the same
+    launches reach on this GPU: the headline is to be read against it as well as against the nominal
+    peak."""
+    import ctypes as C
+    from izwi_amd import capi
+    L = capi.lib()
+    per_layer = len(LAYER_8B)
+    n_layers = (len(weights) - 1) // per_layer
+    kinds = ([0, 1, 2], [3], [4, 5], [6])
+    sizes = []
+    for layer in range(n_layers):
+        w = weights[layer * per_layer:(layer + 1) * per_layer]
+        for idx in kinds:
+            sizes.append(int(sum(gemv_bytes(dtype, w[i][1], w[i][2], m) for i in idx)))
+    sizes.append(int(gemv_bytes(dtype, weights[-1][1], weights[-1][2], m)))
+    bufs = [torch.randint(0, 255, ((sz + 15) // 16 * 16,), dtype=torch.uint8, device="cuda") for sz in sizes]
+
+    def run():
+        sp = torch.cuda.current_stream().cuda_stream
+        for b in bufs:
+            rc = L.izwi_qmm_probe_stream_read(b.data_ptr(), b.numel(), sp)
+            if rc:
+                capi.check(rc)
+
+    t, g = time_graph(torch, run, steps, warmup)
+    total = float(sum(sizes))
+    out = {"gbs": round(total / (t * 1e-3) / 1e9, 1), "ms_per_step": round(t, 4), "launches_per_step": len(bufs),
+           "note": "read-only launches of the same sizes in the same dependent chain; not `value`"}
+    del g, bufs
+    torch.cuda.empty_cache()
+    return out
+
+
 def neighbours_extra(torch, qa, steps=10, warmup=3):
     """Extra report (not `value`): the decode-step neighbours at Qwen3-8B shapes (32 query heads on
     8 kv heads, head_dim 128, hidden 4096, f32): microseconds per call in a HIP-graph replay and, for
@@ -909,6 +946,8 @@ def main():
             del c
             extras["decode_host_pointer_calls"] = host_pointer_extra(qa, weights, args.m)
             extras["hbm_ceiling_measured"] = hbm_ceiling_extra(torch)
+            if args.calls == "grouped":
+                extras["decode_read_only_floor"] = read_only_floor_extra(torch, qa, dtype, weights, args.m)
         except Exception as exc:  # extras never invalidate the headline number
             extras["decode_error"] = repr(exc)
     del weights
@@ -937,7 +976,12 @@ def main():
                 "gbs": round(tb / (t * 1e-3) / 1e9, 1), "ms_per_step": round(t, 4),
                 "pct_of_hbm_peak": round(100.0 * tb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2), "m": args.m,
                 "calls_per_step": len(c)}
-            del ow, c, g
+            del c, g
+            if args.calls == "grouped":
+                floor = read_only_floor_extra(torch, qa, other_dtype, ow, args.m)
+                extras["decode_q8_0_8b_stack" if other_dtype == Q8_0 else "decode_q4k_8b_stack"]["read_only_floor"] = {
+                    "gbs": floor["gbs"], "ms_per_step": floor["ms_per_step"]}
+            del ow
             torch.cuda.empty_cache()
         except Exception as exc:
             extras["decode_other_dtype_error"] = repr(exc)

@@ -1672,6 +1672,16 @@ int izwi_qmm_profile_snapshot_get(izwi_qmm_profile_snapshot* out) {
     return IZWI_QMM_OK;
 }
 
+int izwi_qmm_probe_stream_read(const void* device_buffer, uint64_t bytes, void* stream) {
+    QmmCallScope call;
+    if (!device_buffer) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    if (((uintptr_t)device_buffer & 15) != 0) return fail(IZWI_QMM_ERR_INVALID, "buffer is not 16-byte aligned");
+    int device = 0, n_cus = 0;
+    if (int rc = qmm_current_device(&device, &n_cus)) return rc;
+    HIP_TRY(qmm_launch_stream_read(device_buffer, (size_t)bytes, n_cus, (hipStream_t)stream));
+    return IZWI_QMM_OK;
+}
+
 int izwi_qmm_profile_enabled(void) { return profiling() ? 1 : 0; }
 
 int izwi_qmm_profile_argmax_get(uint64_t* calls, uint64_t* ns) {
