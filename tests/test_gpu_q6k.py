@@ -150,7 +150,7 @@ def test_q6_k_in_groups_and_mlp(qa, oracle):
     w4b = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType.Q4K, b4b, (272, k)))
     gu = qa.Qwen3GateUpProjection.new_separate(w6, w6)
     nw = torch.from_numpy(oracle.randn(9, (k,), mean=1.0, std=0.2)).cuda()
-    for m in (1, 2, 5, 16, 80):
+    for m in (1, 2, 5, 16, 33, 64, 80):
         x = torch.from_numpy(oracle.randn(10 + m, (m, k))).cuda()
         for group in ([w4, w6, w6], [w6, w6b, w6], [w4, w4b, w6b], [w6b, w4]):
             ys = qa.forward_group(group, x)
