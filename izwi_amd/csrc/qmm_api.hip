@@ -102,14 +102,15 @@ int ensure_device(int device, int* n_cus) {
 }
 
 // Average sorted pairs per expert from which the expert MLP runs on 16-row matrix-core
-// tiles instead of 4-row dot4 segments (IZWI_QMM_MOE_MFMA_MIN_ROWS, default 4).  Measured at 128
-// experts, top-8, per layer, segments / tiles: 61 / 104 us at 16 tokens, 87 / 109 at 32, 110 / 114 at 48
-// (3 pairs per expert), 131 / 116 at 64 (4 pairs), 183 / 119 at 96: the tile path reads every expert
-// once and costs about the same from 16 to 128 tokens, the segment path grows with the pairs.
+// tiles instead of 4-row dot4 segments (IZWI_QMM_MOE_MFMA_MIN_ROWS, default 3).  Measured at 128
+// experts, top-8, per layer, segments / tiles: 60 / 101 us at 16 tokens, 73 / 101 at 24, 88 / 102 at 32,
+// 101 / 107 at 40, 114 / 107 at 48 (3 pairs per expert), 128 / 109 at 56, 131 / 109 at 64 (4 pairs),
+// 183 / 113 at 96: the tile path reads every expert once and costs about the same from 16 to 128
+// tokens, the segment path grows with the pairs.
 int moe_mfma_min_rows() {
     static const int v = [] {
         const char* s = getenv("IZWI_QMM_MOE_MFMA_MIN_ROWS");
-        int n = s ? atoi(s) : 4;
+        int n = s ? atoi(s) : 3;
         return n < 1 ? 1 : n;
     }();
     return v;
