@@ -138,6 +138,17 @@ int izwi_qmm_weight_create_stacked(int ggml_dtype, int32_t n_experts, int64_t n,
                                    const void* blocks, uint64_t nbytes, int mem_space,
                                    izwi_qmm_weight** out);
 
+/* `QTensor::quantize(&tensor, dtype)` (candle-core quantized/mod.rs; the reference's own use:
+ * qwen3/core.rs:3112, where its packed-projection test builds Q8_0 tensors from f32 ones): the
+ * GGUF block bytes of an f32 `[n, k]` matrix, rows contiguous, blocks along k — BlockQ8_0::from_float
+ * (34 bytes per 32 values) or BlockQ4K::from_float (144 bytes per 256 values: the
+ * `make_qkx1_quants(15, 5, ..)` search per sub-block, 6-bit scales and mins, nibble pairs), value
+ * for value what the reference's CPU quantizer writes.  `out_blocks` receives
+ * izwi_qmm_storage_bytes(dtype, n, k) bytes and is what izwi_qmm_weight_create takes.  Other
+ * target types: IZWI_QMM_ERR_UNSUPPORTED. */
+int izwi_qmm_quantize_weights_f32(int ggml_dtype, const float* w, int64_t n, int64_t k, void* out_blocks,
+                                  int mem_space, void* stream);
+
 /* Drop of the Arc<QTensor>. NULL is ignored. */
 void izwi_qmm_weight_destroy(izwi_qmm_weight* w);
 

@@ -78,6 +78,7 @@ PROTOTYPES = {
     "izwi_qmm_forward_rows_f32": (C.c_int, [_vp, _vp, _i64, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_f32_noalloc": (C.c_int, [_vp, _vp, _i64, _vp, _vp]),
     "izwi_qmm_probe_stream_read": (C.c_int, [_vp, C.c_uint64, _vp]),
+    "izwi_qmm_quantize_weights_f32": (C.c_int, [C.c_int, _vp, _i64, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_group_f32": (C.c_int, [_vp, _i32, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_group_bf16": (C.c_int, [_vp, _i32, _vp, _i64, _vp, C.c_int, C.c_int, _vp]),
     "izwi_qmm_forward_gate_up_silu_f32": (C.c_int, [_vp, _vp, _vp, _i64, _vp, C.c_int, _vp]),

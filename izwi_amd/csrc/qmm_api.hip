@@ -683,6 +683,33 @@ int izwi_qmm_quantize_activations(int ggml_weight_dtype, const float* x, int64_t
     return IZWI_QMM_OK;
 }
 
+int izwi_qmm_quantize_weights_f32(int ggml_dtype, const float* w, int64_t n, int64_t k, void* out_blocks,
+                                  int mem_space, void* stream_) {
+    if (ggml_dtype != IZWI_QMM_Q8_0 && ggml_dtype != IZWI_QMM_Q4_K)
+        return fail(IZWI_QMM_ERR_UNSUPPORTED, "quantize to ggml dtype %d (Q8_0 and Q4_K are built)", ggml_dtype);
+    if (int rc = check_space(mem_space)) return rc;
+    if (n < 0 || k < 0) return fail(IZWI_QMM_ERR_INVALID, "negative shape");
+    const int bs = ggml_dtype == IZWI_QMM_Q8_0 ? 32 : 256;
+    const int ts = ggml_dtype == IZWI_QMM_Q8_0 ? 34 : 144;
+    if (k % bs) return fail(IZWI_QMM_ERR_INVALID, "k = %lld is not a multiple of the block size %d", (long long)k, bs);
+    if (n == 0 || k == 0) return IZWI_QMM_OK;
+    if (!w || !out_blocks) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
+    if (n > 0x7fffffffffffLL / k) return fail(IZWI_QMM_ERR_UNSUPPORTED, "tensor too large");
+    int device = 0;
+    if (int rc = current_device(&device)) return rc;
+    if (int rc = ensure_device(device, nullptr)) return rc;
+    hipStream_t stream = (hipStream_t)stream_;
+    Staged wi, o;
+    HIP_TRY(wi.in(w, (size_t)n * k * sizeof(float), mem_space));
+    HIP_TRY(o.out(out_blocks, (size_t)n * (k / bs) * ts, mem_space));
+    if (ggml_dtype == IZWI_QMM_Q8_0) // BlockQ8_0::from_float row by row: the activation quantizer's blocks
+        HIP_TRY(qmm_launch_quantize_activations(IZWI_QMM_Q8_0, (const float*)wi.dev, n, k, o.dev, stream));
+    else
+        HIP_TRY(qmm_launch_quantize_q4k_weights((const float*)wi.dev, n * (k / 256), o.dev, stream));
+    HIP_TRY(o.finish(stream));
+    return IZWI_QMM_OK;
+}
+
 int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, float* y,
                          int mem_space, void* stream_) {
     QmmCallScope call;

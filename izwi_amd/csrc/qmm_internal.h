@@ -129,6 +129,8 @@ hipError_t qmm_launch_dequant(const QmmLayout& L, const void* tiled, float* out,
                               hipStream_t stream);
 // out[i, :] = row rows[i] (device ints) of the first matrix, dequantized as above, f32 or rounded to bf16;
 // a row id outside [0, n) gives zeros.
+// BlockQ4K::from_float over `n_blocks` blocks of 256 consecutive f32 values: 144 bytes each into `out`
+hipError_t qmm_launch_quantize_q4k_weights(const float* x, int64_t n_blocks, void* out, hipStream_t stream);
 // read-only stream of `bytes` of device memory (diagnostic)
 hipError_t qmm_launch_stream_read(const void* src, size_t bytes, int n_cus, hipStream_t stream);
 hipError_t qmm_launch_dequant_rows(const QmmLayout& L, const void* tiled, const int32_t* rows, int64_t n_rows,

@@ -469,3 +469,130 @@ hipError_t qmm_launch_stream_read(const void* src, size_t bytes, int n_cus, hipS
     }
     return hipGetLastError();
 }
+
+// ---- QTensor::quantize for Q4_K: f32 rows -> GGUF block bytes -----------------------------------
+// candle-core k_quants.rs `BlockQ4K::from_float` with utils.rs `make_qkx1_quants(15, 5, ..)`: a
+// thread owns one sub-block of 32 values and runs the search exactly as the scalar code does (the
+// same f32 operations in the same order: the sums over the 32 values are sequential), the eight
+// threads of a block share their scale and min through wave shuffles, and the quants of the block
+// pass through LDS on their way into the nibble-pair layout.  Load-time work, not a hot path.
+namespace {
+__device__ __forceinline__ int nearest_int_f(float v) { return (int)roundf(v); } // half away from zero
+
+__global__ __launch_bounds__(256) void quantize_q4k_weights_kernel(const float* __restrict__ x, int64_t n_blocks,
+                                                                   uint8_t* __restrict__ out) {
+    __shared__ uint8_t l_sh[32][256];
+    const int64_t sub = (int64_t)blockIdx.x * 256 + threadIdx.x; // sub-block of 32 values
+    const int64_t blk = sub >> 3;
+    const int j = (int)(threadIdx.x & 7), bl = (int)(threadIdx.x >> 3);
+    const bool live = blk < n_blocks;
+    float v[32];
+#pragma unroll
+    for (int i = 0; i < 32; i++) v[i] = live ? x[sub * 32 + i] : 0.0f;
+    // make_qkx1_quants(nmax = 15, ntry = 5)
+    float scale = 0.0f, neg_min = 0.0f;
+    {
+        uint8_t l[32];
+#pragma unroll
+        for (int i = 0; i < 32; i++) l[i] = 0;
+        float mn = v[0], mx = v[0];
+#pragma unroll
+        for (int i = 1; i < 32; i++) {
+            if (v[i] < mn) mn = v[i];
+            if (v[i] > mx) mx = v[i];
+        }
+        if (mx != mn) {
+            if (mn > 0.0f) mn = 0.0f;
+            float iscale = 15.0f / (mx - mn);
+            scale = 1.0f / iscale;
+            for (int t = 0; t < 5; t++) {
+                float sumlx = 0.0f;
+                int suml2 = 0;
+                bool did_change = false;
+#pragma unroll
+                for (int i = 0; i < 32; i++) {
+                    int li = nearest_int_f(iscale * (v[i] - mn));
+                    li = li < 0 ? 0 : (li > 15 ? 15 : li);
+                    if ((uint8_t)li != l[i]) l[i] = (uint8_t)li, did_change = true;
+                    sumlx += (v[i] - mn) * (float)li;
+                    suml2 += li * li;
+                }
+                scale = sumlx / (float)suml2;
+                float sum = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 32; i++) sum += v[i] - scale * (float)l[i];
+                mn = sum / 32.0f;
+                if (mn > 0.0f) mn = 0.0f;
+                iscale = 1.0f / scale;
+                if (!did_change) break;
+            }
+            neg_min = -mn;
+        }
+    }
+    // the block's largest scale and min (the eight threads of a block are neighbours in a wave)
+    // (the scalar code starts both maxima at +0.0 and replaces them on `>`: a min of -0.0 stays +0.0)
+    float max_scale = scale > 0.0f ? scale : 0.0f, max_min = neg_min > 0.0f ? neg_min : 0.0f;
+#pragma unroll
+    for (int d = 1; d < 8; d <<= 1) {
+        const float os = __shfl_xor(max_scale, d), om = __shfl_xor(max_min, d);
+        max_scale = os > max_scale ? os : max_scale;
+        max_min = om > max_min ? om : max_min;
+    }
+    const float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+    const float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+    int ls = nearest_int_f(inv_scale * scale), lm = nearest_int_f(inv_min * neg_min);
+    ls = ls > 63 ? 63 : ls;
+    lm = lm > 63 ? 63 : lm;
+    const uint16_t d_bits = qmm_f32_to_f16_bits(max_scale / 63.0f), dmin_bits = qmm_f32_to_f16_bits(max_min / 63.0f);
+    // quants against the block's rounded scales (what get_scale_min_k4 returns is ls, lm again)
+    const float d = qmm_f16_bits_to_f32(d_bits) * (float)ls;
+    if (d != 0.0f) {
+        const float dm = qmm_f16_bits_to_f32(dmin_bits) * (float)lm;
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            int lv = nearest_int_f((v[i] + dm) / d);
+            l_sh[bl][32 * j + i] = (uint8_t)(lv < 0 ? 0 : (lv > 15 ? 15 : lv));
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 32; i++) l_sh[bl][32 * j + i] = 0;
+    }
+    // the 12 scale bytes: sub-blocks 0..3 hold their six bits whole, 4..7 split them
+    int ls_all[8], lm_all[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        ls_all[q] = __shfl(ls, (int)((threadIdx.x & 63) & ~7) + q);
+        lm_all[q] = __shfl(lm, (int)((threadIdx.x & 63) & ~7) + q);
+    }
+    __syncthreads();
+    if (!live) return;
+    uint8_t* b = out + blk * 144;
+    if (j == 0) {
+        uint8_t sc[12];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            sc[q] = (uint8_t)(ls_all[q] | ((ls_all[q + 4] >> 4) << 6));
+            sc[q + 4] = (uint8_t)(lm_all[q] | ((lm_all[q + 4] >> 4) << 6));
+            sc[q + 8] = (uint8_t)((ls_all[q + 4] & 0xF) | ((lm_all[q + 4] & 0xF) << 4));
+        }
+        b[0] = (uint8_t)(d_bits & 0xff), b[1] = (uint8_t)(d_bits >> 8);
+        b[2] = (uint8_t)(dmin_bits & 0xff), b[3] = (uint8_t)(dmin_bits >> 8);
+#pragma unroll
+        for (int q = 0; q < 12; q++) b[4 + q] = sc[q];
+    }
+    // qs: byte (c * 32 + i) = l[64 c + i] | l[64 c + 32 + i] << 4; thread j packs bytes 16 j .. 16 j + 15
+#pragma unroll
+    for (int q = 0; q < 16; q++) {
+        const int byte = 16 * j + q, c = byte >> 5, i = byte & 31;
+        b[16 + byte] = (uint8_t)(l_sh[bl][64 * c + i] | (l_sh[bl][64 * c + 32 + i] << 4));
+    }
+}
+} // namespace
+
+hipError_t qmm_launch_quantize_q4k_weights(const float* x, int64_t n_blocks, void* out, hipStream_t stream) {
+    if (n_blocks <= 0) return hipSuccess;
+    const int64_t wgs = (n_blocks * 8 + 255) / 256;
+    if (wgs > 0x7fffffff) return hipErrorInvalidValue;
+    quantize_q4k_weights_kernel<<<(unsigned)wgs, 256, 0, stream>>>(x, n_blocks, (uint8_t*)out);
+    return hipGetLastError();
+}

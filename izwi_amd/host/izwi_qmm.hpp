@@ -83,6 +83,15 @@ public:
         check(izwi_qmm_weight_create_stacked((int)dtype, n_experts, n, k, blocks, nbytes, (int)space, &h));
         return std::shared_ptr<QTensor>(new QTensor(h));
     }
+    // `QTensor::quantize(&tensor, dtype)` (candle-core quantized/mod.rs; the reference's use: qwen3/core.rs:3112):
+    // an f32 [n, k] matrix in host memory -> Q8_0 / Q4_K tensor, blocks as the reference's CPU quantizer writes them.
+    static std::shared_ptr<QTensor> quantize(const std::vector<float>& w, int64_t n, int64_t k, GgmlDType dtype) {
+        if ((int64_t)w.size() != n * k)
+            throw Error(Error::Kind::InvalidInput, IZWI_QMM_ERR_INVALID, "quantize: the tensor does not hold n * k values");
+        std::vector<uint8_t> blocks(quantized_storage_bytes(n, k, dtype));
+        check(izwi_qmm_quantize_weights_f32((int)dtype, w.data(), n, k, blocks.data(), IZWI_QMM_HOST, nullptr));
+        return from_blocks(dtype, blocks.data(), blocks.size(), n, k);
+    }
     // takes ownership of a handle made by the C ABI
     static std::shared_ptr<QTensor> adopt(izwi_qmm_weight* h) { return std::shared_ptr<QTensor>(new QTensor(h)); }
     ~QTensor() { izwi_qmm_weight_destroy(h_); }

@@ -94,6 +94,24 @@ class QTensor:
         del keep
         return cls(h.value)
 
+    @classmethod
+    def quantize(cls, tensor: torch.Tensor, dtype: GgmlDType) -> "QTensor":
+        """QTensor::quantize(&tensor, dtype) (candle-core quantized/mod.rs; the reference's use:
+        qwen3/core.rs:3112): an f32 [n, k] matrix (host or device) -> Q8_0 / Q4_K tensor on the GPU,
+        the blocks value for value those of the reference's CPU quantizer.  The last dimension
+        must divide by the block size (the reference's own requirement)."""
+        if tensor.dim() != 2:
+            raise capi.QmmError(-1, f"unexpected rank, expected: 2, got: {tensor.dim()} ({tuple(tensor.shape)})")
+        w = tensor.to(torch.float32).contiguous()
+        n, k = w.shape
+        nbytes = quantized_storage_bytes(n, k, dtype)
+        blocks = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+        check(lib().izwi_qmm_quantize_weights_f32(int(dtype), w.data_ptr(), n, k, blocks.data_ptr(), _space(w),
+                                                  _stream_ptr(w)))
+        if w.is_cuda:
+            torch.cuda.current_stream().synchronize()
+        return cls.from_blocks(dtype, blocks, (n, k))
+
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
         if h:

@@ -90,6 +90,9 @@ static void packed_matches_separate_q8_0() {
     auto q1 = izwi::QTensor::from_blocks(GgmlDType::Q8_0, b1.data(), b1.size(), 2, 32);
     auto q2 = izwi::QTensor::from_blocks(GgmlDType::Q8_0, b2.data(), b2.size(), 1, 32);
     EXPECT(q1->data() == b1 && q2->data() == b2);
+    // the reference's test builds its tensors with QTensor::quantize: the same blocks
+    EXPECT(izwi::QTensor::quantize(w1, 2, 32, GgmlDType::Q8_0)->data() == b1);
+    EXPECT(izwi::QTensor::quantize(w2, 1, 32, GgmlDType::Q8_0)->data() == b2);
     auto y1 = izwi::QMatMul::from_arc(q1).forward(x);
     auto y2 = izwi::QMatMul::from_qtensor(q2).forward(x);
     auto packed = izwi::Qwen3Projection::packed_quantized({q1, q2});
@@ -120,6 +123,7 @@ static void q4k_projection_matches_oracle() {
     auto q = izwi::QTensor::from_blocks(GgmlDType::Q4K, blocks.data(), blocks.size(), n, k);
     EXPECT(q->dtype() == GgmlDType::Q4K && q->dims2().first == n && q->dims2().second == k);
     EXPECT(q->data() == blocks);
+    EXPECT(izwi::QTensor::quantize(w, n, k, GgmlDType::Q4K)->data() == blocks);
     auto y = izwi::Qwen3Projection::quantized(q).forward(x);
     std::vector<float> want((size_t)m * n);
     EXPECT(oracle_qmatmul((int)GgmlDType::Q4K, m, k, n, x.data(), blocks.data(), want.data()) == 0);
