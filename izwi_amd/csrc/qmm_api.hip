@@ -102,15 +102,15 @@ int ensure_device(int device, int* n_cus) {
 }
 
 // Average sorted pairs per expert from which the expert MLP runs on 16-row matrix-core
-// tiles instead of 4-row dot4 segments (IZWI_QMM_MOE_MFMA_MIN_ROWS, default 3).  Measured at 128
-// experts, top-8, per layer, segments / tiles: 60 / 101 us at 16 tokens, 73 / 101 at 24, 88 / 102 at 32,
-// 101 / 107 at 40, 114 / 107 at 48 (3 pairs per expert), 128 / 109 at 56, 131 / 109 at 64 (4 pairs),
-// 183 / 113 at 96: the tile path reads every expert once and costs about the same from 16 to 128
-// tokens, the segment path grows with the pairs.
+// tiles instead of 4-row dot4 segments (IZWI_QMM_MOE_MFMA_MIN_ROWS, default 4).  Measured at 128
+// experts, top-8, per layer, segments / tiles: 60 / 101 us at 16 tokens, 69 / 101 at 24, 80 / 102 at 32,
+// 88 / 107 at 40, 101 / 110 at 48 (3 pairs per expert), 104 / 111 at 56, 115 / 110 at 64 (4 pairs),
+// 123 / 112 at 72, 132 / 111 at 80: the tile path reads every expert once and costs about the same from
+// 16 to 128 tokens, the segment path grows with the pairs.
 int moe_mfma_min_rows() {
     static const int v = [] {
         const char* s = getenv("IZWI_QMM_MOE_MFMA_MIN_ROWS");
-        int n = s ? atoi(s) : 3;
+        int n = s ? atoi(s) : 4;
         return n < 1 ? 1 : n;
     }();
     return v;
@@ -1507,7 +1507,14 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
     const size_t mid_bytes = tiles ? h_bytes + r_bytes + te_bytes : align256((size_t)max_segments * 4);
     const size_t p_bytes = align256((size_t)pairs * 4);
     const size_t sort_bytes = align256((size_t)qmm_moe_sort_scratch_ints(pairs, n_experts) * sizeof(int32_t));
-    const size_t route_bytes = logits ? 3 * p_bytes + s_bytes + sort_bytes : 0;
+    // Segment path with the routing computed here, beyond the one-launch plan's sizes: the routing kernel
+    // also quantizes the token rows (x blocks), which the gate / up launch then copies instead of
+    // quantizing them in every workgroup of a segment.  Measured per layer at 128 experts, top-8,
+    // without / with: 74 / 70 us at 24 tokens, 90 / 80 at 32, 103 / 90 at 40; up to 16 tokens, where most
+    // segments hold one row and routing, sort and tables are one workgroup, it does not pay (60.4 / 62.6).
+    const size_t xb_bytes = logits && !tiles && !qmm_moe_plan_small_supported(t, n_experts, top_k)
+                                ? align256(qmm_x_blocks_bytes(t, hidden)) : 0;
+    const size_t route_bytes = logits ? 3 * p_bytes + s_bytes + sort_bytes + xb_bytes : 0;
     uint8_t* ws = nullptr;
     HIP_TRY(get_scratch(gate->device, stream, h_bytes + y_bytes + s_bytes + mid_bytes + route_bytes, (void**)&ws));
     float* h = (float*)ws;
@@ -1517,6 +1524,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
     int32_t* seg_expert = (int32_t*)mid; // 4-row segment path only
     int32_t* tile_expert = (int32_t*)(mid + h_bytes + r_bytes); // tile path only
     bool segments_ready = false;
+    void* x_blocks = nullptr; // written by the routing kernels below when set
     hipError_t e = hipSuccess;
     if (logits) {
         uint8_t* r = mid + mid_bytes;
@@ -1525,6 +1533,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
         int32_t* r_perm = (int32_t*)(r + 2 * p_bytes);
         int32_t* r_off = (int32_t*)(r + 3 * p_bytes);
         int32_t* r_sort = (int32_t*)(r + 3 * p_bytes + s_bytes);
+        if (xb_bytes) x_blocks = r + 3 * p_bytes + s_bytes + sort_bytes;
         // a handful of pairs: the whole layer in two launches (routing inside gate / up, combine
         // inside down), same results
         if (!tiles && pairs <= moe_small_max_pairs() && qmm_moe_small_supported(G, D, t, n_experts, top_k)) {
@@ -1543,7 +1552,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
                                           r_perm, r_off, seg, seg_expert, stream);
             segments_ready = true;
         } else {
-            e = qmm_launch_moe_route(logits, t, n_experts, top_k, r_ids, r_w, stream);
+            e = qmm_launch_moe_route(logits, t, n_experts, top_k, r_ids, r_w, stream, x, hidden, G.dtype, x_blocks);
             // the sort also leaves the table of the 16-row tiles the matrix-core path walks, or of the
             // 4-row segments of the decode kernel, with the expert of every tile / segment
             if (e == hipSuccess)
@@ -1579,7 +1588,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
             e = qmm_launch_moe_segments(offsets, n_experts, QMM_MOE_SEG_ROWS, seg, seg_expert, max_segments, stream);
         if (e == hipSuccess)
             e = qmm_launch_gemv_grouped(G, gate->tiled, up->tiled, x, top_k, h, perm, offsets, seg, seg_expert,
-                                        n_experts, max_segments, gate->n_cus, stream);
+                                        n_experts, max_segments, gate->n_cus, stream, x_blocks, t);
         if (e == hipSuccess)
             e = qmm_launch_gemv_grouped(D, down->tiled, nullptr, h, 1, y, perm, offsets, seg, seg_expert, n_experts,
                                         max_segments, gate->n_cus, stream);

@@ -72,6 +72,9 @@ struct GemvParams {
     // NORM variants: the activations are RMS-normalized on the way in (weight norm_w[k], eps)
     const float* norm_w;
     float norm_eps;
+    // expert-grouped form: the token rows quantized ahead of the launch (x blocks of row p / x_div for
+    // pair p); xb.xq == nullptr: the workgroups quantize their rows themselves
+    XBlocks xb;
     // TILEMAP variant (selected rows): row-tile i of the launch reads the weight's row-tile
     // tile_ids[i]; row_tiles, rt_groups and n count the selected tiles, y is [m, 16 * tiles]
     const int32_t* tile_ids;
@@ -94,7 +97,9 @@ __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 // group adds the squares of its 256 raw values while it quantizes x * norm_w, and because the
 // quantizers are invariant under a positive scale of their input (the quants stay, the block scale
 // moves), the row's factor rsqrt(mean(x^2) + eps) multiplies the finished sums instead.
-template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT, int IO = 0, bool NORM = false, bool TILEMAP = false>
+// XBLK (expert-grouped form): the rows' x blocks were made ahead of the launch and are copied.
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT, int IO = 0, bool NORM = false, bool TILEMAP = false,
+          bool XBLK = false>
 __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int m_end, const uint8_t* w_first,
                                           float* y_out, int n_rows, int row_tiles, int rtg0, uint8_t* smem,
                                           int item_bias = 0) {
@@ -140,7 +145,23 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                 const int64_t off = ok ? ((int64_t)rt_w * P.k_groups + kg) * P.panel_bytes : 0;
                 Panel<QT> p;
                 const bool active = ok && lane_active;
-                if (!x_ready) {
+                if (XBLK && GROUPED && !x_ready) {
+                    // the rows' x blocks were made ahead of the launch: copy them (a quarter of the f32
+                    // bytes, no arithmetic); first item ahead of the panel as below
+                    const int group = threadIdx.x >> 4, n_groups = 4 * waves;
+                    const int items = MT * k_units;
+                    auto copy_item = [&](int item) {
+                        const int mi = item % MT, unit = item / MT;
+                        const bool row_ok = m0 + mi < m_end;
+                        const int64_t token = row_ok ? P.perm[m0 + mi] / P.x_div : 0;
+                        x_blocks_to_lds<QT>(l, mi * k_units + unit, P.xb, token * k_units + unit, row_ok);
+                    };
+                    if (group < items) copy_item(group);
+                    load_panel<QT>(p, wbase + off, P.slots, lane0, active);
+                    for (int item = group + n_groups; item < items; item += n_groups) copy_item(item);
+                    lds_barrier();
+                    x_ready = true;
+                } else if (!x_ready) {
                     // Loads return in issue order: the small activation load goes first so
                     // that it can be consumed (quantized) while the panel loads still fly.
                     const int group = threadIdx.x >> 4, n_groups = 4 * waves; // = blockDim.x / 16
@@ -270,7 +291,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
 // whether it exists or not.
 // The dense straight-line single-row Q4_K form is held to 80 registers: six waves per SIMD,
 // i.e. two 12-wave workgroups per CU.
-template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT, int IO, bool NORM, bool TILEMAP>
+template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT, int IO, bool NORM, bool TILEMAP, bool XBLK = false>
 __device__ __forceinline__ void gemv_entry(const GemvParams& P, const GemvParams& P0, int n_weights) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int m_begin = 0, m_end = P.m;
@@ -314,13 +335,13 @@ __device__ __forceinline__ void gemv_entry(const GemvParams& P, const GemvParams
     if (GROUPED && ONESHOT && MT == 4) {
         const int rows = m_end - m_begin;
         if (rows == 1)
-            gemv_body<QT, 1, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
+            gemv_body<QT, 1, GATED, GROUPED, ONESHOT, 0, false, false, XBLK>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
         else if (rows == 2)
-            gemv_body<QT, 2, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
+            gemv_body<QT, 2, GATED, GROUPED, ONESHOT, 0, false, false, XBLK>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
         else
-            gemv_body<QT, 4, GATED, GROUPED, ONESHOT>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
+            gemv_body<QT, 4, GATED, GROUPED, ONESHOT, 0, false, false, XBLK>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     } else {
-        gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO, NORM, TILEMAP>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem, item_bias);
+        gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO, NORM, TILEMAP, XBLK>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem, item_bias);
     }
 }
 
@@ -345,9 +366,9 @@ void gemv_kernel(const uint8_t* w_arg, const float* x_arg, float* y_arg, int m_a
 // The expert-grouped launches: thousands of short workgroups, whose waves start faster with
 // fewer scalar registers to fill (measured: 1 us of 19 - 30 lost with preloaded arguments), so
 // the parameter block stays one block in memory.
-template <int QT, int MT, bool GATED, bool ONESHOT>
+template <int QT, int MT, bool GATED, bool ONESHOT, bool XBLK = false>
 __global__ __launch_bounds__(64 * kMaxWaves) __attribute__((amdgpu_waves_per_eu(3))) void gemv_grouped_kernel(GemvParams P) {
-    gemv_entry<QT, MT, GATED, true, ONESHOT, 0, false, false>(P, P, 0);
+    gemv_entry<QT, MT, GATED, true, ONESHOT, 0, false, false, XBLK>(P, P, 0);
 }
 
 // The launch of a gemv_kernel: its leading arguments are the fields of P that the first loads need.
@@ -416,7 +437,15 @@ hipError_t launch_mt(const GemvParams& P, int waves, int n_cus, int grid_y, hipS
             hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return e;
         }
-        if (oneshot) gemv_grouped_kernel<QT, MT, GATED, kCanOneshot><<<g, b, lds, stream>>>(P);
+        // (x blocks: gate / up of the straight-line form copies them; every other form quantizes P.x itself)
+        if (GATED && oneshot && P.xb.xq != nullptr) {
+            if (lds > 48 * 1024) {
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_grouped_kernel<QT, MT, GATED, kCanOneshot, GATED>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return e;
+            }
+            gemv_grouped_kernel<QT, MT, GATED, kCanOneshot, GATED><<<g, b, lds, stream>>>(P);
+        } else if (oneshot) gemv_grouped_kernel<QT, MT, GATED, kCanOneshot><<<g, b, lds, stream>>>(P);
         else gemv_grouped_kernel<QT, MT, GATED, false><<<g, b, lds, stream>>>(P);
     } else {
         const void* fn = oneshot ? reinterpret_cast<const void*>(&gemv_kernel<QT, MT, GATED, false, kCanOneshot, IO, NORM>)
@@ -497,6 +526,7 @@ bool make_params(const QmmLayout& L, const void* tiled, const float* x, int64_t 
     P.ep.y_bf16 = 0;
     P.norm_w = nullptr;
     P.norm_eps = 0.0f;
+    P.xb = XBlocks{nullptr, nullptr, nullptr};
     P.tile_ids = nullptr;
     return true;
 }
@@ -892,7 +922,7 @@ hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const 
                                    const float* x, int x_div, float* y, const int32_t* perm,
                                    const int32_t* offsets, const int32_t* seg_offsets,
                                    const int32_t* seg_expert, int n_experts, int64_t max_segments,
-                                   int n_cus, hipStream_t stream) {
+                                   int n_cus, hipStream_t stream, const void* x_blocks, int64_t x_rows) {
     if (max_segments <= 0 || L.n == 0) return hipSuccess;
     if (max_segments > 65535) return hipErrorInvalidValue;
     GemvParams P;
@@ -904,6 +934,7 @@ hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const 
     P.seg_expert = seg_expert;
     P.n_experts = n_experts;
     P.x_div = x_div;
+    if (x_blocks) P.xb = x_blocks_carve(const_cast<void*>(x_blocks), x_rows, L.k_units);
     const bool gated = tiled2 != nullptr;
     int waves;
     choose_split(L, n_cus, (int)max_segments, gated, P, waves);

@@ -257,6 +257,96 @@ __device__ __forceinline__ void x_item_quantize(const XLds<QT>& l, int k_units, 
         make_uint4(q[0], q[1], q[2], q[3]);
 }
 
+// ---- activations quantized ahead of the kernel ("x blocks") ---------------------------------
+// What the quantizer above leaves in LDS per (row, unit), kept in device memory for rows that many
+// workgroups need (the tokens of an expert-grouped launch: every workgroup of a segment would
+// quantize the same rows again): three arrays over slot = row * k_units + unit, strides as in LDS.
+struct XBlocks {
+    uint8_t* xq; // [rows * k_units][kXUnitStride]
+    float* xd;   // [rows * k_units][kXdPerItem]
+    int* xbs;    // [rows * k_units][kXbsPerItem]
+};
+__host__ __device__ inline size_t x_blocks_part_bytes(size_t n) { return (n + 255) & ~(size_t)255; }
+// (the largest per-slot sizes of the three block types: one buffer layout for all of them)
+__host__ __device__ inline size_t x_blocks_bytes(int64_t rows, int64_t k_units) {
+    const size_t slots = (size_t)rows * (size_t)k_units;
+    return x_blocks_part_bytes(slots * kXUnitStride) + x_blocks_part_bytes(slots * 8 * sizeof(float)) +
+           x_blocks_part_bytes(slots * 16 * sizeof(int));
+}
+__host__ __device__ inline XBlocks x_blocks_carve(void* base, int64_t rows, int64_t k_units) {
+    const size_t slots = (size_t)rows * (size_t)k_units;
+    uint8_t* b = static_cast<uint8_t*>(base);
+    XBlocks xb;
+    xb.xq = b;
+    xb.xd = reinterpret_cast<float*>(b + x_blocks_part_bytes(slots * kXUnitStride));
+    xb.xbs = reinterpret_cast<int*>(b + x_blocks_part_bytes(slots * kXUnitStride) + x_blocks_part_bytes(slots * 8 * sizeof(float)));
+    return xb;
+}
+
+// One wave quantizes row `row` of x [rows, k] (f32) into its x blocks: its four 16-lane groups take
+// the units in turn, with the quantizer of the kernels (the same values as quantizing in the kernel).
+// Two steps, so that the caller can put other work between the loads of the first two units of
+// every group (k <= 2048: all of the row) and their use.
+struct XRowLoads {
+    float4 f[2][4];
+    bool in_range[2];
+};
+__device__ __forceinline__ void x_row_issue(const float* __restrict__ x, int64_t row, int k, int k_units, XRowLoads& ld) {
+    const int lane = threadIdx.x & 63, j = lane & 15;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int unit = (lane >> 4) + 4 * i;
+        const int k0 = unit * 256 + 16 * j;
+        ld.in_range[i] = unit < k_units && k0 + 16 <= k;
+        x16_issue<false>(x + row * k + k0, x, ld.in_range[i], ld.f[i]);
+    }
+}
+template <int QT>
+__device__ __forceinline__ void x_row_to_blocks(const float* __restrict__ x, int64_t row, int k, int k_units,
+                                                const XBlocks& xb, const XRowLoads& ld) {
+    const int lane = threadIdx.x & 63, j = lane & 15;
+    XLds<QT> g;
+    g.xq = xb.xq + (size_t)row * k_units * kXUnitStride;
+    g.xd = xb.xd + (size_t)row * k_units * kXdPerItem<QT>;
+    g.xbs = xb.xbs + (size_t)row * k_units * kXbsPerItem<QT>;
+    g.red = nullptr;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int unit = (lane >> 4) + 4 * i;
+        if (unit < k_units) { // uniform for the 16-lane group
+            float v[16];
+            x16_finish<false>(ld.f[i], ld.in_range[i], v);
+            x_item_quantize<QT, 1>(g, k_units, unit, v);
+        }
+    }
+    for (int unit = (lane >> 4) + 8; unit < k_units; unit += 4) {
+        const int k0 = unit * 256 + 16 * j;
+        const bool in_range = k0 + 16 <= k;
+        float4 f[4];
+        float v[16];
+        x16_issue<false>(x + row * k + k0, x, in_range, f);
+        x16_finish<false>(f, in_range, v);
+        x_item_quantize<QT, 1>(g, k_units, unit, v);
+    }
+}
+
+// A 16-lane group copies the x blocks of (source row, unit) into LDS slot `dst_slot`; zeros for a
+// row that does not exist (what the quantizer makes of a zero row).
+template <int QT>
+__device__ __forceinline__ void x_blocks_to_lds(const XLds<QT>& l, int dst_slot, const XBlocks& xb, int64_t src_slot,
+                                                bool row_ok) {
+    const int j = threadIdx.x & 15;
+    const int64_t s = row_ok ? src_slot : 0;
+    uint4 q = *reinterpret_cast<const uint4*>(xb.xq + (size_t)s * kXUnitStride + 16 * j);
+    float d = j < kXdPerItem<QT> ? xb.xd[s * kXdPerItem<QT> + j] : 0.0f;
+    int bs = 0;
+    if (kXbsPerItem<QT> > 0) bs = j < kXbsPerItem<QT> ? xb.xbs[s * (kXbsPerItem<QT> > 0 ? kXbsPerItem<QT> : 1) + j] : 0;
+    if (!row_ok) q = make_uint4(0, 0, 0, 0), d = 0.0f, bs = 0;
+    *reinterpret_cast<uint4*>(l.xq + (size_t)dst_slot * kXUnitStride + 16 * j) = q;
+    if (j < kXdPerItem<QT>) l.xd[dst_slot * kXdPerItem<QT> + j] = d;
+    if (kXbsPerItem<QT> > 0 && j < kXbsPerItem<QT>) l.xbs[dst_slot * (kXbsPerItem<QT> > 0 ? kXbsPerItem<QT> : 1) + j] = bs;
+}
+
 // ---- panel registers ----------------------------------------------------------
 template <int QT>
 struct Panel {

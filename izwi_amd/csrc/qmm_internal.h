@@ -229,7 +229,10 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
 #define QMM_MOE_SEG_ROWS 4
 
 hipError_t qmm_launch_moe_route(const float* logits, int64_t t, int n_experts, int top_k,
-                                int32_t* ids, float* weights, hipStream_t stream);
+                                int32_t* ids, float* weights, hipStream_t stream,
+                                const float* x = nullptr, int64_t k = 0, int dot_dtype = 0, void* x_blocks = nullptr);
+// (x, k, dot_dtype, x_blocks: the wave that routes a token also quantizes the token's row of x [t, k]
+// for weights of block type `dot_dtype` into its x blocks)
 
 // Stable counting sort of `pairs` expert ids.  `seg_offsets` (n_experts + 1 ints,
 // may be NULL) receives the exclusive prefix sum of ceil(count / seg_rows): the table of the
@@ -249,7 +252,10 @@ hipError_t qmm_launch_gemv_grouped(const QmmLayout& L, const void* tiled, const 
                                    const float* x, int x_div, float* y, const int32_t* perm,
                                    const int32_t* offsets, const int32_t* seg_offsets,
                                    const int32_t* seg_expert, int n_experts, int64_t max_segments,
-                                   int n_cus, hipStream_t stream);
+                                   int n_cus, hipStream_t stream, const void* x_blocks = nullptr, int64_t x_rows = 0);
+// `x_blocks`: the x_rows activation rows quantized ahead of the launch (qmm_x_blocks_bytes bytes, written
+// by the routing kernels below when they are given x); then the workgroups copy instead of quantizing.
+size_t qmm_x_blocks_bytes(int64_t rows, int64_t k);
 
 // seg_offsets[e] = exclusive prefix sum of ceil(count(e) / seg_rows) from caller-provided
 // offsets; seg_expert (may be NULL; max_segments ints) = the expert of every segment, -1

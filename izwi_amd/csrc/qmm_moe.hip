@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include "qmm_internal.h"
+#include "qmm_gemv_blocks.h"
 #include "qmm_moe_route.h"
 
 namespace {
@@ -12,13 +13,33 @@ constexpr int kSortChunk = 256; // pairs per chunk of the sort
 
 using moe_route::route_token;
 
-// One wavefront per token.
+// The x blocks of one token row, for weights of block type `dot_dtype` (a wave; xb.xq == nullptr:
+// nothing).  The loads are issued before the routing and used after it.
+__device__ __forceinline__ void token_x_issue(const float* __restrict__ x, int64_t tok, int k, const XBlocks& xb,
+                                              XRowLoads& ld) {
+    if (xb.xq == nullptr) return; // uniform
+    x_row_issue(x, tok, k, (k + 255) >> 8, ld);
+}
+__device__ __forceinline__ void token_to_x_blocks(const float* __restrict__ x, int64_t tok, int k, int dot_dtype,
+                                                  const XBlocks& xb, const XRowLoads& ld) {
+    if (xb.xq == nullptr) return; // uniform
+    const int k_units = (k + 255) >> 8;
+    if (dot_dtype == QMM_Q8_0) x_row_to_blocks<QMM_Q8_0>(x, tok, k, k_units, xb, ld);
+    else if (dot_dtype == QMM_Q6_K) x_row_to_blocks<QMM_Q6_K>(x, tok, k, k_units, xb, ld);
+    else x_row_to_blocks<QMM_Q4_K>(x, tok, k, k_units, xb, ld);
+}
+
+// One wavefront per token.  With x blocks to fill, the wave also quantizes its token's activation row
+// (the rows the expert-grouped decode kernel would otherwise quantize in every workgroup of a segment).
 template <int PER_LANE>
 __global__ void route_kernel(const float* __restrict__ logits, int64_t t, int n_experts, int top_k,
-                             int32_t* __restrict__ ids, float* __restrict__ weights) {
+                             int32_t* __restrict__ ids, float* __restrict__ weights,
+                             const float* __restrict__ x, int k, int dot_dtype, XBlocks xb) {
     const int lane = threadIdx.x & 63;
     const int64_t tok = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (tok >= t) return; // whole waves leave together
+    XRowLoads ld;
+    token_x_issue(x, tok, k, xb, ld);
     int id;
     float w;
     route_token<PER_LANE>(logits + tok * n_experts, n_experts, top_k, lane, id, w);
@@ -26,6 +47,7 @@ __global__ void route_kernel(const float* __restrict__ logits, int64_t t, int n_
         ids[tok * top_k + lane] = id;
         weights[tok * top_k + lane] = w;
     }
+    token_to_x_blocks(x, tok, k, dot_dtype, xb, ld);
 }
 
 // ---- sort ----------------------------------------------------------------
@@ -344,20 +366,25 @@ __global__ void combine_kernel(const float* __restrict__ y, const float* __restr
 
 } // namespace
 
+size_t qmm_x_blocks_bytes(int64_t rows, int64_t k) { return x_blocks_bytes(rows, (k + 255) / 256); }
+
 hipError_t qmm_launch_moe_route(const float* logits, int64_t t, int n_experts, int top_k,
-                                int32_t* ids, float* weights, hipStream_t stream) {
+                                int32_t* ids, float* weights, hipStream_t stream,
+                                const float* x, int64_t k, int dot_dtype, void* x_blocks) {
     if (t <= 0) return hipSuccess;
+    if (x_blocks && (!x || k <= 0 || k > 0x3fffffff || k % 32)) return hipErrorInvalidValue;
+    const XBlocks xb = x_blocks ? x_blocks_carve(x_blocks, t, (k + 255) / 256) : XBlocks{nullptr, nullptr, nullptr};
     if (n_experts < 1 || n_experts > 1024 || top_k < 1 || top_k > 64 || top_k > n_experts)
         return hipErrorInvalidValue;
     const int waves_per_block = 4;
     unsigned grid = (unsigned)((t + waves_per_block - 1) / waves_per_block);
     int per_lane = (n_experts + 63) / 64;
     if (per_lane <= 2)
-        route_kernel<2><<<grid, 256, 0, stream>>>(logits, t, n_experts, top_k, ids, weights);
+        route_kernel<2><<<grid, 256, 0, stream>>>(logits, t, n_experts, top_k, ids, weights, x, (int)k, dot_dtype, xb);
     else if (per_lane <= 4)
-        route_kernel<4><<<grid, 256, 0, stream>>>(logits, t, n_experts, top_k, ids, weights);
+        route_kernel<4><<<grid, 256, 0, stream>>>(logits, t, n_experts, top_k, ids, weights, x, (int)k, dot_dtype, xb);
     else
-        route_kernel<16><<<grid, 256, 0, stream>>>(logits, t, n_experts, top_k, ids, weights);
+        route_kernel<16><<<grid, 256, 0, stream>>>(logits, t, n_experts, top_k, ids, weights, x, (int)k, dot_dtype, xb);
     return hipGetLastError();
 }
 
