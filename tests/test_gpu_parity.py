@@ -480,7 +480,7 @@ def test_config5_moe_forward(qa, oracle, moe_weights, t):
     assert np.isfinite(out).all()
 
 
-@pytest.mark.parametrize("t", [1, 2, 3, 16, 100, 128, 129, 512])
+@pytest.mark.parametrize("t", [1, 2, 3, 16, 17, 24, 40, 63, 100, 128, 129, 512])
 def test_config5_moe_layer_one_call_equals_the_three_calls(qa, oracle, moe_weights, t):
     """izwi_moe_layer_f32 = route + sort + forward, bit for bit (ids, weights, outputs): up to
     1024 pairs routing, sort and segment tables come from one launch, beyond from the
@@ -512,6 +512,39 @@ def test_config5_moe_layer_one_call_equals_the_three_calls(qa, oracle, moe_weigh
     if t <= 16:  # host pointers
         out_h = experts.layer(logits.cpu(), x.cpu(), 8)
         assert torch.equal(out_h.view(torch.int32), want.cpu().view(torch.int32))
+
+
+@pytest.mark.parametrize("dtype,E,hidden,inter,t,top_k", [
+    (Q8_0, 64, 512, 256, 20, 4),    # 17..: the routing kernel quantizes the token rows, gate / up copies the blocks
+    (Q4_K, 64, 1280, 768, 33, 2),   # the same with five units per row (two rounds of a wave's four groups)
+    (Q4_K, 32, 2560, 256, 17, 2),   # ten units per row: units beyond the eight that are loaded ahead of the routing
+    (Q8_0, 48, 1056, 256, 40, 3),   # a row that ends inside a unit
+])
+def test_moe_layer_with_token_rows_quantized_by_the_routing_kernel(qa, oracle, dtype, E, hidden, inter, t, top_k):
+    """More than 16 tokens and fewer than four pairs per expert: izwi_moe_layer_f32 quantizes every
+    token row once, in the routing kernel; route + sort + forward (rows quantized in the grouped
+    kernel's workgroups) must give the same bits."""
+    _say(f"moe x blocks dtype={dtype} E={E} hidden={hidden} inter={inter} t={t} top_k={top_k}")
+    assert t > 16 and t * top_k < 4 * E
+    gate = oracle.quantize(dtype, oracle.randn(311, (E * inter, hidden), std=0.05))
+    up = oracle.quantize(dtype, oracle.randn(312, (E * inter, hidden), std=0.05))
+    down = oracle.quantize(dtype, oracle.randn(313, (E * hidden, inter), std=0.05))
+    dt = qa.GgmlDType(dtype)
+    experts = qa.MoeExperts(qa.QTensor.from_blocks(dt, gate, (E, inter, hidden)),
+                            qa.QTensor.from_blocks(dt, up, (E, inter, hidden)),
+                            qa.QTensor.from_blocks(dt, down, (E, hidden, inter)))
+    x_h = oracle.randn(314, (t, hidden))
+    x_h[3, :] = 0.0  # a zero row: scale 0
+    logits_h = oracle.randn(315, (t, E))
+    x, logits = torch.from_numpy(x_h).cuda(), torch.from_numpy(logits_h).cuda()
+    ids, wts = qa.moe_route(logits, top_k)
+    perm, offsets = qa.moe_sort(ids, E)
+    want = experts.forward(x, ids, wts, perm, offsets)
+    out = experts.layer(logits, x, top_k)
+    assert torch.equal(out.view(torch.int32), want.view(torch.int32))
+    want_ids, want_wts = oracle.moe_route(logits_h, top_k)
+    ref = oracle.moe_forward(dtype, x_h, want_ids, want_wts, gate, up, down, E, inter)
+    assert rel_err(out.cpu().numpy(), ref) < 1e-3
 
 
 @pytest.mark.parametrize("dtype,E,hidden,inter,t,top_k", [

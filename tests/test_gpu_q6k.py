@@ -174,6 +174,8 @@ def test_q6_k_in_groups_and_mlp(qa, oracle):
     (Q4_K, 8, 1024, 256, 1, 2),    # one token
     (Q6_K, 4, 768, 512, 40, 2),    # every stack Q6_K, ragged panels
     (Q6_K, 8, 256, 512, 3, 2),
+    (Q6_K, 64, 768, 256, 24, 2),   # more than 16 tokens on the segment path: token rows quantized by the routing kernel
+    (Q4_K, 64, 512, 512, 30, 3),   # the same, Q4_K gate / up with a Q6_K down stack
 ])
 def test_moe_with_q6_k_expert_stacks(qa, oracle, gate_up_dtype, E, hidden, inter, t, top_k):
     """Expert stacks in Q6_K (a Q4_K_M file keeps ffn_down_exps of some layers in it): the expert MLP
