@@ -97,12 +97,49 @@ __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 // group adds the squares of its 256 raw values while it quantizes x * norm_w, and because the
 // quantizers are invariant under a positive scale of their input (the quants stay, the block scale
 // moves), the row's factor rsqrt(mean(x^2) + eps) multiplies the finished sums instead.
+// The weight of a wave's row-tile in a group launch (straight-line form), looked up BEHIND the
+// activation loads: those need nothing from the tables, so the tables' round trip hides behind them.
+// The launch's row-tiles are counted over all weights, rtg_end[i] = the end of weight i's row-tiles,
+// and every WAVE finds the weight of its own row-tile (a workgroup may straddle two weights; its
+// waves only share the quantized activations and the LDS of the k-split).  The tables are read
+// whole (independent scalar loads, one round trip) and the entry is picked with selects; rtg_end
+// ascends, so the entry is the number of ends at or below the row-tile's index.  Entries past
+// n_weights hold whatever the host left there and are never picked.
+struct NoGroupPick {
+    static constexpr bool kActive = false;
+    __device__ __forceinline__ void operator()(int, const uint8_t*&, float*&, int&, int&, int&) const {}
+};
+struct GroupPick {
+    static constexpr bool kActive = true;
+    const GemvParams& P0;
+    int n_weights;
+    // b: the wave's row-tile counted over the launch
+    __device__ __forceinline__ void operator()(int b, const uint8_t*& w_first, float*& y_out, int& n_rows, int& row_tiles,
+                                               int& item_bias) const {
+        if (n_weights <= 1) return; // uniform
+        static_assert(QMM_MAX_GROUP == 4, "the selects below name four entries");
+        const int e0 = P0.rtg_end[0], e1 = P0.rtg_end[1], e2 = P0.rtg_end[2];
+        const bool c1 = b >= e0, c2 = n_weights > 2 && b >= e1, c3 = n_weights > 3 && b >= e2;
+        auto pick = [c1, c2, c3](auto v0, auto v1, auto v2, auto v3) {
+            auto v = c1 ? v1 : v0;
+            v = c2 ? v2 : v;
+            return c3 ? v3 : v;
+        };
+        item_bias = -pick(0, e0, e1, e2);
+        w_first = pick(P0.wv[0], P0.wv[1], P0.wv[2], P0.wv[3]);
+        y_out = pick(P0.yv[0], P0.yv[1], P0.yv[2], P0.yv[3]);
+        n_rows = pick(P0.nv[0], P0.nv[1], P0.nv[2], P0.nv[3]);
+        row_tiles = pick(P0.row_tiles_v[0], P0.row_tiles_v[1], P0.row_tiles_v[2], P0.row_tiles_v[3]);
+    }
+};
+
 // XBLK (expert-grouped form): the rows' x blocks were made ahead of the launch and are copied.
 template <int QT, int MT, bool GATED, bool GROUPED, bool ONESHOT, int IO = 0, bool NORM = false, bool TILEMAP = false,
-          bool XBLK = false>
+          bool XBLK = false, class Pick = NoGroupPick>
 __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int m_end, const uint8_t* w_first,
                                           float* y_out, int n_rows, int row_tiles, int rtg0, uint8_t* smem,
-                                          int item_bias = 0) {
+                                          int item_bias = 0, Pick group_pick = Pick{}) {
+    static_assert(!Pick::kActive || (ONESHOT && !GATED && !GROUPED && !TILEMAP), "group launches are dense straight-line launches");
     constexpr bool XB = IO == 2, EP = IO != 0;
     const int lane0 = threadIdx.x & 63;
     // wave-uniform by construction; said so, the row-tile, panel offset and output row that
@@ -116,7 +153,8 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
     const int wk = sw - wr * P.nwk;
     const bool lane_active = lane0 < P.slots;
     const int k_units = (P.k + 255) >> 8, s_units = P.slots >> 4;
-    const uint8_t* wbase = stack ? P.w2 + (w_first - P.w) : w_first; // the second stack at the same offset
+    const uint8_t* wbase_init = stack ? P.w2 + (w_first - P.w) : w_first; // the second stack at the same offset
+    const uint8_t* wbase = wbase_init; // (set again by a group pick)
     const XLds<QT> l = carve<QT, MT>(smem, k_units);
     float* xss = l.red + 2 * waves * MT * 16; // NORM: [MT][k_units] sums of squares, behind everything else
 
@@ -127,9 +165,9 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
              rtg += ONESHOT ? 1 : (int)gridDim.x) {
             // the wave's row-tile (item_bias: a group launch counts its row-tiles over all weights and
             // this is minus the first one of the wave's weight; uniform)
-            const int rt = rtg * P.nwr + wr + item_bias;
+            int rt = rtg * P.nwr + wr + item_bias;
             // the weight's row-tile behind this one (uniform: a scalar load)
-            const int rt_w = TILEMAP ? P.tile_ids[rt < row_tiles ? rt : 0] : rt;
+            int rt_w = TILEMAP ? P.tile_ids[rt < row_tiles ? rt : 0] : rt;
             float acc[MT];
 #pragma unroll
             for (int mi = 0; mi < MT; mi++) acc[mi] = 0.0f;
@@ -141,10 +179,10 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
             uint32_t res_raw = 0;
             for (int ks = 0; ONESHOT ? ks < 1 : ks < P.kpw; ks++) {
                 const int kg = ks * P.nwk + wk;
-                const bool ok = rt < row_tiles && kg < P.k_groups;
-                const int64_t off = ok ? ((int64_t)rt_w * P.k_groups + kg) * P.panel_bytes : 0;
+                bool ok = rt < row_tiles && kg < P.k_groups;
+                int64_t off = ok ? ((int64_t)rt_w * P.k_groups + kg) * P.panel_bytes : 0;
                 Panel<QT> p;
-                const bool active = ok && lane_active;
+                bool active = ok && lane_active;
                 if (XBLK && GROUPED && !x_ready) {
                     // the rows' x blocks were made ahead of the launch: copy them (a quarter of the f32
                     // bytes, no arithmetic); first item ahead of the panel as below
@@ -173,6 +211,15 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                     float4 fnw[4];
                     if (NORM) x16_issue<false>(P.norm_w + (group / MT) * 256 + 16 * (threadIdx.x & 15), P.norm_w, in0, fnw);
                     if (IO != 0 || NORM) __builtin_amdgcn_sched_barrier(0); // the activation loads stay in front
+                    if constexpr (Pick::kActive) {
+                        group_pick(rt, w_first, y_out, n_rows, row_tiles, item_bias);
+                        wbase = w_first;
+                        rt = rtg * P.nwr + wr + item_bias;
+                        rt_w = rt;
+                        ok = rt < row_tiles && kg < P.k_groups;
+                        off = ok ? ((int64_t)rt_w * P.k_groups + kg) * P.panel_bytes : 0;
+                        active = ok && lane_active;
+                    }
                     load_panel<QT>(p, wbase + off, P.slots, lane0, active);
                     if (EP && ks == 0) {
                         // (the lanes and conditions of the store at the end)
@@ -307,31 +354,6 @@ __device__ __forceinline__ void gemv_entry(const GemvParams& P, const GemvParams
     const uint8_t* w_first = P.w + w_offset;
     float* y_out = P.y;
     int n_rows = P.n, row_tiles = P.row_tiles, rtg0 = blockIdx.x;
-    int item_bias = 0;
-    if (!GROUPED && !GATED && ONESHOT && n_weights > 1) {
-        // A group of weights: the launch's row-tiles are counted over all weights, rtg_end[i] = the
-        // end of weight i's row-tiles, and every WAVE finds the weight of its own row-tile (a
-        // workgroup may straddle two weights; its waves only share the quantized
-        // activations and the LDS of the k-split).  The tables are read whole (independent scalar
-        // loads, one round trip) and the entry is picked with selects; rtg_end ascends, so the entry
-        // is the number of ends at or below the row-tile's index.  Entries past n_weights hold whatever
-        // the host left there and are never picked.
-        static_assert(QMM_MAX_GROUP == 4, "the selects below name four entries");
-        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-        const int b = blockIdx.x * P.nwr + ((wave * P.wave_magic) >> 16);
-        const int e0 = P0.rtg_end[0], e1 = P0.rtg_end[1], e2 = P0.rtg_end[2];
-        const bool c1 = b >= e0, c2 = n_weights > 2 && b >= e1, c3 = n_weights > 3 && b >= e2;
-        auto pick = [c1, c2, c3](auto v0, auto v1, auto v2, auto v3) {
-            auto v = c1 ? v1 : v0;
-            v = c2 ? v2 : v;
-            return c3 ? v3 : v;
-        };
-        item_bias = -pick(0, e0, e1, e2);
-        w_first = pick(P0.wv[0], P0.wv[1], P0.wv[2], P0.wv[3]);
-        y_out = pick(P0.yv[0], P0.yv[1], P0.yv[2], P0.yv[3]);
-        n_rows = pick(P0.nv[0], P0.nv[1], P0.nv[2], P0.nv[3]);
-        row_tiles = pick(P0.row_tiles_v[0], P0.row_tiles_v[1], P0.row_tiles_v[2], P0.row_tiles_v[3]);
-    }
     if (GROUPED && ONESHOT && MT == 4) {
         const int rows = m_end - m_begin;
         if (rows == 1)
@@ -341,7 +363,11 @@ __device__ __forceinline__ void gemv_entry(const GemvParams& P, const GemvParams
         else
             gemv_body<QT, 4, GATED, GROUPED, ONESHOT, 0, false, false, XBLK>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     } else {
-        gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO, NORM, TILEMAP, XBLK>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem, item_bias);
+        if constexpr (!GROUPED && !GATED && ONESHOT && !TILEMAP)
+            gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO, NORM, TILEMAP, XBLK, GroupPick>(
+                P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem, 0, GroupPick{P0, n_weights});
+        else
+            gemv_body<QT, MT, GATED, GROUPED, ONESHOT, IO, NORM, TILEMAP, XBLK>(P, m_begin, m_end, w_first, y_out, n_rows, row_tiles, rtg0, smem);
     }
 }
 

@@ -654,12 +654,8 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
         g_stack = within / P.rt_groups;
         rtg = within - g_stack * P.rt_groups;
     }
-    if (!GROUPED && P.n_weights > 1) pick_group_entry(P0, P.n_weights, blockIdx.x, rtg, wbase, yout, n_rows, row_tiles);
-    const int rt = rtg * P.nwr + wr;
-    const bool rt_ok = rt < row_tiles;
     const int unit0 = wk * s_units;                       // first unit of this wave's panel
     const int n_units = min(s_units, P.k_units - unit0);  // its units that exist (>= 1)
-    const int row = rt * 16 + j;
 
     const uint8_t* records = P.ws;
     int n_tiles = P.n_tiles, pos_begin = 0, pos_end = 0;
@@ -682,6 +678,11 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
     // barrier the last wave's window pieces queue behind the other waves' panels, and the barrier
     // below - the start of all arithmetic - waits for nearly the whole workgroup's weights.
     asm volatile("s_barrier" ::: "memory");
+    // (a group's tables are read here, behind the window copies: those need nothing from them)
+    if (!GROUPED && P.n_weights > 1) pick_group_entry(P0, P.n_weights, blockIdx.x, rtg, wbase, yout, n_rows, row_tiles);
+    const int rt = rtg * P.nwr + wr;
+    const bool rt_ok = rt < row_tiles;
+    const int row = rt * 16 + j;
     WPanel<QT> p;
     load_wpanel<QT>(p, wbase + (int64_t)((rt_ok ? rt : 0) * P.k_groups + wk) * P.panel_bytes, P.slots, lane, j);
     // The window has landed.  The single-stage form lets the panel fly on: its arithmetic starts on the
