@@ -18,8 +18,9 @@
  *     ggml dtype ids as in GGUF: Q8_0 = 8, Q4_K = 12, Q6_K = 14.
  *   - `mem_space` says where the caller's buffers live: IZWI_QMM_DEVICE (HIP
  *     device pointers, the fast path, asynchronous on `stream`) or
- *     IZWI_QMM_HOST (ordinary host memory; the library stages it and the call
- *     is synchronous).
+ *     IZWI_QMM_HOST (ordinary host memory; the library stages it through
+ *     pooled pinned buffers that it keeps for the life of the process, and
+ *     the call is synchronous).
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
  *   - all entry points may be called from several host threads at once; a
  *     weight handle is immutable after creation and may be shared by

@@ -224,41 +224,170 @@ int create_from_parts(int dtype, int64_t n_stacked, int64_t n, int64_t k, const 
 }
 
 // Device view of a caller buffer: the pointer itself, or a staged copy.
+// Host-pointer calls: inputs are copied to the device before the launches and outputs back behind
+// them.  Up to kStageMaxBytes a copy goes through a pooled pair of buffers (pinned host memory +
+// device memory, kept until the process ends and reused by the next call): no allocation, no free
+// and no pageable transfer per call.  Inputs: memcpy into the pinned buffer, then a copy kernel
+// into the device buffer (the launches read an input many times: once over the host link, then
+// from device memory).  Outputs: the kernels store straight into the pinned buffer (posted writes
+// over the host link, no transfer behind the last launch), memcpy to the caller after the wait.
+// The pool hands a pair to one Staged object at a time; the object gives it back when it is
+// destroyed, after the stream has been waited for (finish() of the call's outputs, or the
+// destructor itself on a path that returns early).  Larger copies allocate for the call and use
+// pageable transfers.
+constexpr size_t kStageMaxBytes = (size_t)8 << 20;
+struct StagePair {
+    int device = -1;
+    void* pinned = nullptr;
+    void* dev = nullptr;
+    size_t cap = 0;
+};
+std::mutex g_stage_mutex;
+std::vector<StagePair*> g_stage_free;
+thread_local uint64_t t_stage_syncs = 0; // stream waits done by finish() on this thread
+
+hipError_t stage_acquire(size_t bytes, StagePair** out) {
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return e;
+    StagePair* best = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_stage_mutex);
+        size_t at = 0;
+        for (size_t i = 0; i < g_stage_free.size(); i++) {
+            StagePair* c = g_stage_free[i];
+            if (c->device != device) continue;
+            // the smallest pair that is large enough, else the largest one (it grows below)
+            const bool better = !best || (best->cap >= bytes ? (c->cap >= bytes && c->cap < best->cap) : c->cap > best->cap);
+            if (better) best = c, at = i;
+        }
+        if (best) g_stage_free.erase(g_stage_free.begin() + (ptrdiff_t)at);
+    }
+    if (!best) {
+        best = new (std::nothrow) StagePair;
+        if (!best) return hipErrorOutOfMemory;
+        best->device = device;
+    }
+    if (best->cap < bytes) {
+        // nobody uses this pair: its last user waited for its stream before giving it back
+        if (best->pinned) (void)hipHostFree(best->pinned);
+        if (best->dev) (void)hipFree(best->dev);
+        best->pinned = best->dev = nullptr;
+        size_t cap = best->cap * 2 > bytes ? best->cap * 2 : bytes;
+        cap = (cap + 65535) & ~(size_t)65535;
+        best->cap = 0;
+        e = hipHostMalloc(&best->pinned, cap, hipHostMallocDefault);
+        if (e == hipSuccess) e = hipMalloc(&best->dev, cap);
+        if (e != hipSuccess) {
+            if (best->pinned) (void)hipHostFree(best->pinned);
+            delete best;
+            return e;
+        }
+        best->cap = cap;
+    }
+    *out = best;
+    return hipSuccess;
+}
+void stage_release(StagePair* p) {
+    std::lock_guard<std::mutex> lock(g_stage_mutex);
+    g_stage_free.push_back(p);
+}
+
+// pinned host memory -> device memory by a kernel (16 bytes per thread and step; n16 = bytes / 16
+// rounded up, both buffers are sized in multiples of 64 KiB): a launch starts sooner than a copy
+// engine transfer of a few KB
+__global__ void stage_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+
 struct Staged {
     void* dev = nullptr;
     void* host = nullptr;
     size_t bytes = 0;
-    bool owned = false;
+    bool owned = false; // dev was allocated for this call (copies beyond kStageMaxBytes)
     bool copy_back = false;
+    StagePair* pair = nullptr;
+    bool direct = false;
+    hipStream_t pair_stream = nullptr;
+    uint64_t syncs_at_start = 0;
+    Staged() = default;
+    Staged(const Staged&) = delete;
+    Staged& operator=(const Staged&) = delete;
     ~Staged() {
         if (owned && dev) (void)hipFree(dev);
+        if (pair) {
+            // (a path that returned before any finish(): queued work may still touch the pair)
+            if (t_stage_syncs == syncs_at_start) (void)hipStreamSynchronize(pair_stream);
+            stage_release(pair);
+        }
     }
-    hipError_t in(const void* p, size_t n, int mem_space) {
+    hipError_t in(const void* p, size_t n, int mem_space, hipStream_t stream) {
         bytes = n;
         if (mem_space == IZWI_QMM_DEVICE || n == 0) {
             dev = const_cast<void*>(p);
             return hipSuccess;
+        }
+        if (n <= kStageMaxBytes) {
+            hipError_t e = stage_acquire(n, &pair);
+            if (e != hipSuccess) return e;
+            pair_stream = stream;
+            syncs_at_start = t_stage_syncs;
+            dev = pair->dev;
+            memcpy(pair->pinned, p, n);
+            {
+                void* src = nullptr;
+                hipError_t e2 = hipHostGetDevicePointer(&src, pair->pinned, 0);
+                if (e2 != hipSuccess) return e2;
+                const size_t n16 = (n + 15) / 16;
+                const unsigned grid = (unsigned)((n16 + 255) / 256 < 1024 ? (n16 + 255) / 256 : 1024);
+                stage_copy_kernel<<<grid, 256, 0, stream>>>((const uint4*)src, (uint4*)dev, n16);
+                return hipGetLastError();
+            }
         }
         owned = true;
         hipError_t e = hipMalloc(&dev, n);
         if (e != hipSuccess) return e;
         return hipMemcpy(dev, p, n, hipMemcpyHostToDevice);
     }
-    hipError_t out(void* p, size_t n, int mem_space) {
+    // direct_ok: every byte of the output is written by kernel stores and read by no launch (false
+    // for the target of a copy call, which wants device memory)
+    hipError_t out(void* p, size_t n, int mem_space, hipStream_t stream, bool direct_ok = true) {
         bytes = n;
         if (mem_space == IZWI_QMM_DEVICE || n == 0) {
             dev = p;
             return hipSuccess;
         }
-        owned = true;
         copy_back = true;
         host = p;
+        if (n <= kStageMaxBytes) {
+            hipError_t e = stage_acquire(n, &pair);
+            if (e != hipSuccess) return e;
+            pair_stream = stream;
+            syncs_at_start = t_stage_syncs;
+            // the kernels store straight into the pinned buffer (posted writes over the host link):
+            // no copy engine transfer behind the last launch
+            direct = direct_ok;
+            if (direct) return hipHostGetDevicePointer(&dev, pair->pinned, 0);
+            dev = pair->dev;
+            return hipSuccess;
+        }
+        owned = true;
         return hipMalloc(&dev, n);
     }
     hipError_t finish(hipStream_t stream) {
         if (!copy_back) return hipSuccess;
+        if (pair) {
+            hipError_t e = direct ? hipSuccess : hipMemcpyAsync(pair->pinned, dev, bytes, hipMemcpyDeviceToHost, stream);
+            if (e == hipSuccess) e = hipStreamSynchronize(stream);
+            if (e != hipSuccess) return e;
+            t_stage_syncs++;
+            memcpy(host, pair->pinned, bytes);
+            return hipSuccess;
+        }
         hipError_t e = hipStreamSynchronize(stream);
         if (e != hipSuccess) return e;
+        t_stage_syncs++;
         return hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost);
     }
 };
@@ -610,7 +739,7 @@ int izwi_qmm_weight_data(const izwi_qmm_weight* w, void* out_blocks, uint64_t nb
     if (!out_blocks) return fail(IZWI_QMM_ERR_INVALID, "out_blocks is NULL");
     hipStream_t stream = (hipStream_t)stream_;
     Staged o;
-    HIP_TRY(o.out(out_blocks, nbytes, mem_space));
+    HIP_TRY(o.out(out_blocks, nbytes, mem_space, stream));
     HIP_TRY(qmm_launch_unpack(w->layout, w->tiled, o.dev, stream));
     HIP_TRY(o.finish(stream));
     return IZWI_QMM_OK;
@@ -625,7 +754,7 @@ int izwi_qmm_dequantize_f32(const izwi_qmm_weight* w, float* out, int mem_space,
     if (!out) return fail(IZWI_QMM_ERR_INVALID, "out is NULL");
     hipStream_t stream = (hipStream_t)stream_;
     Staged o;
-    HIP_TRY(o.out(out, bytes, mem_space));
+    HIP_TRY(o.out(out, bytes, mem_space, stream));
     HIP_TRY(qmm_launch_dequant(L, w->tiled, (float*)o.dev, stream));
     HIP_TRY(o.finish(stream));
     return IZWI_QMM_OK;
@@ -652,8 +781,8 @@ int izwi_qmm_dequantize_rows(const izwi_qmm_weight* w, const int32_t* row_ids, i
     if (device != w->device) return fail(IZWI_QMM_ERR_INVALID, "weight lives on device %d, current device is %d", w->device, device);
     hipStream_t stream = (hipStream_t)stream_;
     Staged ids, o;
-    HIP_TRY(ids.in(row_ids, (size_t)n_rows * sizeof(int32_t), ids_mem_space));
-    HIP_TRY(o.out(out, (size_t)n_rows * L.k * (out_dtype == IZWI_QMM_OUT_BF16 ? 2 : 4), out_mem_space));
+    HIP_TRY(ids.in(row_ids, (size_t)n_rows * sizeof(int32_t), ids_mem_space, stream));
+    HIP_TRY(o.out(out, (size_t)n_rows * L.k * (out_dtype == IZWI_QMM_OUT_BF16 ? 2 : 4), out_mem_space, stream));
     HIP_TRY(qmm_launch_dequant_rows(L, w->tiled, (const int32_t*)ids.dev, n_rows, o.dev, out_dtype == IZWI_QMM_OUT_BF16, stream));
     HIP_TRY(o.finish(stream));
     if (ids.owned) HIP_TRY(hipStreamSynchronize(stream)); // the staged ids are freed on return
@@ -676,8 +805,8 @@ int izwi_qmm_quantize_activations(int ggml_weight_dtype, const float* x, int64_t
     if (int rc = ensure_device(device, nullptr)) return rc;
     hipStream_t stream = (hipStream_t)stream_;
     Staged xi, o;
-    HIP_TRY(xi.in(x, (size_t)m * k * sizeof(float), mem_space));
-    HIP_TRY(o.out(out_blocks, (size_t)m * (k / bs) * ts, mem_space));
+    HIP_TRY(xi.in(x, (size_t)m * k * sizeof(float), mem_space, stream));
+    HIP_TRY(o.out(out_blocks, (size_t)m * (k / bs) * ts, mem_space, stream));
     HIP_TRY(qmm_launch_quantize_activations(ggml_weight_dtype, (const float*)xi.dev, m, k, o.dev, stream));
     HIP_TRY(o.finish(stream));
     return IZWI_QMM_OK;
@@ -700,8 +829,8 @@ int izwi_qmm_quantize_weights_f32(int ggml_dtype, const float* w, int64_t n, int
     if (int rc = ensure_device(device, nullptr)) return rc;
     hipStream_t stream = (hipStream_t)stream_;
     Staged wi, o;
-    HIP_TRY(wi.in(w, (size_t)n * k * sizeof(float), mem_space));
-    HIP_TRY(o.out(out_blocks, (size_t)n * (k / bs) * ts, mem_space));
+    HIP_TRY(wi.in(w, (size_t)n * k * sizeof(float), mem_space, stream));
+    HIP_TRY(o.out(out_blocks, (size_t)n * (k / bs) * ts, mem_space, stream));
     if (ggml_dtype == IZWI_QMM_Q8_0) // BlockQ8_0::from_float row by row: the activation quantizer's blocks
         HIP_TRY(qmm_launch_quantize_activations(IZWI_QMM_Q8_0, (const float*)wi.dev, n, k, o.dev, stream));
     else
@@ -725,8 +854,8 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
     hipStream_t stream = (hipStream_t)stream_;
     ProfileScope prof(w, stream);
     Staged xi, yo;
-    HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
-    HIP_TRY(yo.out(y, (size_t)m * L.n * sizeof(float), mem_space));
+    HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space, stream));
+    HIP_TRY(yo.out(y, (size_t)m * L.n * sizeof(float), mem_space, stream));
     if (m < mfma_min_m()) {
         HIP_TRY(qmm_launch_gemv(L, w->tiled, (const float*)xi.dev, m, (float*)yo.dev, w->n_cus, stream));
     } else if (m <= 64 || large_m_mode() == IZWI_QMM_LARGE_M_INT8) {
@@ -855,9 +984,9 @@ int izwi_qmm_forward_rows_f32(const izwi_qmm_weight* w, const uint32_t* row_ids,
     hipStream_t stream = (hipStream_t)stream_;
     ProfileScope prof(w, stream);
     Staged xi, ii, yo;
-    HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
-    HIP_TRY(ii.in(row_ids, (size_t)n_rows * sizeof(uint32_t), mem_space));
-    HIP_TRY(yo.out(y, (size_t)m * n_rows * sizeof(float), mem_space));
+    HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space, stream));
+    HIP_TRY(ii.in(row_ids, (size_t)n_rows * sizeof(uint32_t), mem_space, stream));
+    HIP_TRY(yo.out(y, (size_t)m * n_rows * sizeof(float), mem_space, stream));
     void* scratch = nullptr;
     HIP_TRY(get_scratch(w->device, stream, qmm_gemv_rows_workspace_bytes(m, n_rows), &scratch));
     HIP_TRY(qmm_launch_gemv_rows(L, w->tiled, (const float*)xi.dev, m, (const uint32_t*)ii.dev, n_rows, (float*)yo.dev,
@@ -1025,12 +1154,12 @@ int forward_group_impl(const izwi_qmm_weight* const* weights, int32_t n_weights,
         // otherwise: the normalized activations into scratch (behind what the projections use of it),
         // then the plain group call
         Staged xi, wi, yo[QMM_MAX_GROUP];
-        HIP_TRY(xi.in(x, (size_t)m * w0->layout.k * sizeof(float), mem_space));
-        HIP_TRY(wi.in(norm_weight, (size_t)w0->layout.k * sizeof(float), mem_space));
+        HIP_TRY(xi.in(x, (size_t)m * w0->layout.k * sizeof(float), mem_space, stream));
+        HIP_TRY(wi.in(norm_weight, (size_t)w0->layout.k * sizeof(float), mem_space, stream));
         float* ydev[QMM_MAX_GROUP];
         size_t keep = 0;
         for (int i = 0; i < n_weights; i++) {
-            HIP_TRY(yo[i].out(ys[i], (size_t)m * weights[i]->layout.n * sizeof(float), mem_space));
+            HIP_TRY(yo[i].out(ys[i], (size_t)m * weights[i]->layout.n * sizeof(float), mem_space, stream));
             ydev[i] = (float*)yo[i].dev;
             keep = std::max(keep, forward_scratch_need(weights[i]->layout, m, weights[i]->n_cus));
         }
@@ -1158,9 +1287,9 @@ int izwi_qmm_forward_normed_f32(const izwi_qmm_weight* w, const float* x, int64_
         (void)hipGetLastError();
     }
     Staged xi, wi, yo;
-    HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
-    HIP_TRY(wi.in(norm_weight, (size_t)L.k * sizeof(float), mem_space));
-    HIP_TRY(yo.out(y, (size_t)m * L.n * sizeof(float), mem_space));
+    HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space, stream));
+    HIP_TRY(wi.in(norm_weight, (size_t)L.k * sizeof(float), mem_space, stream));
+    HIP_TRY(yo.out(y, (size_t)m * L.n * sizeof(float), mem_space, stream));
     float* normed = nullptr;
     if (int rc = normed_copy(w, (const float*)xi.dev, m, (const float*)wi.dev, eps, forward_scratch_need(L, m, w->n_cus), 0,
                              stream, &normed))
@@ -1193,11 +1322,11 @@ int gate_up_silu_impl(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, co
     if (!h) return fail(IZWI_QMM_ERR_INVALID, "h is NULL");
     hipStream_t stream = (hipStream_t)stream_;
     Staged xi, ho;
-    HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space));
-    HIP_TRY(ho.out(h, (size_t)m * L.n * sizeof(float), mem_space));
+    HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space, stream));
+    HIP_TRY(ho.out(h, (size_t)m * L.n * sizeof(float), mem_space, stream));
     if (profiling()) g_silu_fused.fetch_add(1, std::memory_order_relaxed);
     Staged wi;
-    if (norm_weight) HIP_TRY(wi.in(norm_weight, (size_t)L.k * sizeof(float), mem_space));
+    if (norm_weight) HIP_TRY(wi.in(norm_weight, (size_t)L.k * sizeof(float), mem_space, stream));
     const float* xin = (const float*)xi.dev;
     if (m < mfma_min_m() && m <= 2) {
         const QmmNorm norm{(const float*)wi.dev, norm_eps};
@@ -1260,8 +1389,8 @@ int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int6
     ProfileScope prof(w, stream);
     const size_t ybytes = (size_t)m * L.n * (out_dtype == IZWI_QMM_OUT_BF16 ? 2 : 4);
     Staged xi, yo;
-    HIP_TRY(xi.in(x_bf16, (size_t)m * L.k * sizeof(uint16_t), mem_space));
-    HIP_TRY(yo.out(y, ybytes, mem_space));
+    HIP_TRY(xi.in(x_bf16, (size_t)m * L.k * sizeof(uint16_t), mem_space, stream));
+    HIP_TRY(yo.out(y, ybytes, mem_space, stream));
     void* workspace = nullptr; // split-k partial tiles, for products with few output tiles only
     if (const size_t ws_bytes = qmm_gemm_workspace_bytes(L, m, w->n_cus))
         HIP_TRY(get_scratch(w->device, stream, ws_bytes, &workspace));
@@ -1340,9 +1469,9 @@ int izwi_qmm_forward_fused(const izwi_qmm_weight* w, const void* x, int x_dtype,
     ProfileScope prof(w, stream);
     const size_t xbytes = (size_t)m * L.k * (x_bf16 ? 2 : 4), ybytes = (size_t)m * L.n * (y_bf16 ? 2 : 4);
     Staged xi, ri, yo;
-    HIP_TRY(xi.in(x, xbytes, mem_space));
-    if (residual) HIP_TRY(ri.in(residual, ybytes, mem_space));
-    HIP_TRY(yo.out(y, ybytes, mem_space));
+    HIP_TRY(xi.in(x, xbytes, mem_space, stream));
+    if (residual) HIP_TRY(ri.in(residual, ybytes, mem_space, stream));
+    HIP_TRY(yo.out(y, ybytes, mem_space, stream));
     QmmIo io{x_bf16 ? 1 : 0, residual ? ri.dev : nullptr, y_bf16 ? 1 : 0};
     if (m < mfma_min_m()) {
         const float* xf = (const float*)xi.dev;
@@ -1415,9 +1544,9 @@ int izwi_moe_route(const float* logits, int64_t t, int32_t n_experts, int32_t to
     if (int rc = ensure_device(device, nullptr)) return rc;
     hipStream_t stream = (hipStream_t)stream_;
     Staged li, io, wo;
-    HIP_TRY(li.in(logits, (size_t)t * n_experts * sizeof(float), mem_space));
-    HIP_TRY(io.out(ids, (size_t)t * top_k * sizeof(int32_t), mem_space));
-    HIP_TRY(wo.out(weights, (size_t)t * top_k * sizeof(float), mem_space));
+    HIP_TRY(li.in(logits, (size_t)t * n_experts * sizeof(float), mem_space, stream));
+    HIP_TRY(io.out(ids, (size_t)t * top_k * sizeof(int32_t), mem_space, stream));
+    HIP_TRY(wo.out(weights, (size_t)t * top_k * sizeof(float), mem_space, stream));
     HIP_TRY(qmm_launch_moe_route((const float*)li.dev, t, n_experts, top_k, (int32_t*)io.dev,
                                  (float*)wo.dev, stream));
     HIP_TRY(io.finish(stream));
@@ -1439,9 +1568,10 @@ int izwi_moe_sort(const int32_t* ids, int64_t t, int32_t top_k, int32_t n_expert
     if (int rc = ensure_device(device, nullptr)) return rc;
     hipStream_t stream = (hipStream_t)stream_;
     Staged ii, po, oo;
-    HIP_TRY(ii.in(ids, (size_t)pairs * sizeof(int32_t), mem_space));
-    HIP_TRY(po.out(perm, (size_t)pairs * sizeof(int32_t), mem_space));
-    HIP_TRY(oo.out(offsets, (size_t)(n_experts + 1) * sizeof(int32_t), mem_space));
+    HIP_TRY(ii.in(ids, (size_t)pairs * sizeof(int32_t), mem_space, stream));
+    // (the sort's later passes read what its earlier ones wrote: device memory)
+    HIP_TRY(po.out(perm, (size_t)pairs * sizeof(int32_t), mem_space, stream, false));
+    HIP_TRY(oo.out(offsets, (size_t)(n_experts + 1) * sizeof(int32_t), mem_space, stream, false));
     void* scratch = nullptr;
     HIP_TRY(get_scratch(device, stream, (size_t)qmm_moe_sort_scratch_ints(pairs, n_experts) * sizeof(int32_t), &scratch));
     hipError_t e = qmm_launch_moe_sort((const int32_t*)ii.dev, pairs, n_experts, (int32_t*)po.dev,
@@ -1621,12 +1751,12 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
     const int64_t hidden = gate->layout.k;
     hipStream_t stream = (hipStream_t)stream_;
     Staged xi, ii, wi, pi, oi, oo;
-    HIP_TRY(xi.in(x, (size_t)t * hidden * sizeof(float), mem_space));
-    HIP_TRY(ii.in(ids, (size_t)pairs * sizeof(int32_t), mem_space));
-    HIP_TRY(wi.in(weights, (size_t)pairs * sizeof(float), mem_space));
-    HIP_TRY(pi.in(perm, (size_t)pairs * sizeof(int32_t), mem_space));
-    HIP_TRY(oi.in(offsets, (size_t)(n_experts + 1) * sizeof(int32_t), mem_space));
-    HIP_TRY(oo.out(out, (size_t)t * hidden * sizeof(float), mem_space));
+    HIP_TRY(xi.in(x, (size_t)t * hidden * sizeof(float), mem_space, stream));
+    HIP_TRY(ii.in(ids, (size_t)pairs * sizeof(int32_t), mem_space, stream));
+    HIP_TRY(wi.in(weights, (size_t)pairs * sizeof(float), mem_space, stream));
+    HIP_TRY(pi.in(perm, (size_t)pairs * sizeof(int32_t), mem_space, stream));
+    HIP_TRY(oi.in(offsets, (size_t)(n_experts + 1) * sizeof(int32_t), mem_space, stream));
+    HIP_TRY(oo.out(out, (size_t)t * hidden * sizeof(float), mem_space, stream));
     if (int rc = moe_core(gate, up, down, (const float*)xi.dev, t, top_k, nullptr, (const int32_t*)ii.dev,
                           (const float*)wi.dev, (const int32_t*)pi.dev, (const int32_t*)oi.dev, nullptr, nullptr,
                           (float*)oo.dev, stream))
@@ -1652,11 +1782,12 @@ int izwi_moe_layer_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, c
     const int64_t pairs = t * top_k, hidden = gate->layout.k;
     hipStream_t stream = (hipStream_t)stream_;
     Staged li, xi, oo, io, wo;
-    HIP_TRY(li.in(logits, (size_t)t * n_experts * sizeof(float), mem_space));
-    HIP_TRY(xi.in(x, (size_t)t * hidden * sizeof(float), mem_space));
-    HIP_TRY(oo.out(out, (size_t)t * hidden * sizeof(float), mem_space));
-    if (ids_out) HIP_TRY(io.out(ids_out, (size_t)pairs * sizeof(int32_t), mem_space));
-    if (weights_out) HIP_TRY(wo.out(weights_out, (size_t)pairs * sizeof(float), mem_space));
+    HIP_TRY(li.in(logits, (size_t)t * n_experts * sizeof(float), mem_space, stream));
+    HIP_TRY(xi.in(x, (size_t)t * hidden * sizeof(float), mem_space, stream));
+    HIP_TRY(oo.out(out, (size_t)t * hidden * sizeof(float), mem_space, stream));
+    // (ids and weights reach their outputs through device-to-device copy calls)
+    if (ids_out) HIP_TRY(io.out(ids_out, (size_t)pairs * sizeof(int32_t), mem_space, stream, false));
+    if (weights_out) HIP_TRY(wo.out(weights_out, (size_t)pairs * sizeof(float), mem_space, stream, false));
     if (int rc = moe_core(gate, up, down, (const float*)xi.dev, t, top_k, (const float*)li.dev, nullptr, nullptr,
                           nullptr, nullptr, (int32_t*)io.dev, (float*)wo.dev, (float*)oo.dev, stream))
         return rc;
