@@ -353,6 +353,19 @@ int izwi_qmm_forward_gate_up_silu_f32(const izwi_qmm_weight* gate, const izwi_qm
                                       const float* x, int64_t m, float* h, int mem_space,
                                       void* stream);
 
+/* `Qwen3Mlp::forward` (qwen3/core.rs:1786-1798) as one call:
+ *     y[m, hidden] = down.forward( silu(gate.forward(x)) * up.forward(x) )
+ * `gate` and `up` are [intermediate, hidden] weights of the same shape, `down` is
+ * [hidden, intermediate]; any of the built block types.  The results are those of
+ * izwi_qmm_forward_gate_up_silu_f32 followed by izwi_qmm_forward_f32, bit for bit.  What the call
+ * adds is the route between the three projections: for 3 <= m <= 64 (gate and up of one block
+ * type) x is quantized once, gate | up run as one launch on its records, silu(g) * u is quantized
+ * straight into the records that `down` multiplies (four launches; the separate calls take five
+ * and write and read the intermediate as an f32 matrix); other sizes run the two calls with the
+ * intermediate in the stream's scratch. */
+int izwi_qmm_mlp_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_qmm_weight* down,
+                             const float* x, int64_t m, float* y, int mem_space, void* stream);
+
 /* Prefill form: bf16 activations `[m, k]`, weights dequantized to bf16 in LDS,
  * MFMA with f32 accumulation; y is f32 or bf16 per `out_dtype`.  Replaces the
  * to_dtype(F32) -> QMatMul -> to_dtype(activation dtype) sequence of

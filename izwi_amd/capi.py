@@ -82,6 +82,7 @@ PROTOTYPES = {
     "izwi_qmm_forward_group_f32": (C.c_int, [_vp, _i32, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_group_bf16": (C.c_int, [_vp, _i32, _vp, _i64, _vp, C.c_int, C.c_int, _vp]),
     "izwi_qmm_forward_gate_up_silu_f32": (C.c_int, [_vp, _vp, _vp, _i64, _vp, C.c_int, _vp]),
+    "izwi_qmm_mlp_forward_f32": (C.c_int, [_vp, _vp, _vp, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_normed_f32": (C.c_int, [_vp, _vp, _i64, _vp, C.c_float, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_group_normed_f32": (C.c_int, [_vp, _i32, _vp, _i64, _vp, C.c_float, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_gate_up_silu_normed_f32": (C.c_int, [_vp, _vp, _vp, _i64, _vp, C.c_float, _vp, C.c_int, _vp]),

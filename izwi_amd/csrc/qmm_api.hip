@@ -1266,6 +1266,71 @@ int izwi_qmm_forward_gate_up_silu_normed_f32(const izwi_qmm_weight* gate, const 
     return gate_up_silu_impl(gate, up, x, m, h, mem_space, stream_, norm_weight, eps);
 }
 
+int izwi_qmm_mlp_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_qmm_weight* down,
+                             const float* x, int64_t m, float* y, int mem_space, void* stream_) {
+    QmmCallScope call;
+    if (!gate || !up || !down) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
+    if (int rc = check_space(mem_space)) return rc;
+    const QmmLayout& G = gate->layout;
+    const QmmLayout& U = up->layout;
+    const QmmLayout& D = down->layout;
+    if (G.n_stacked != 1 || U.n_stacked != 1 || D.n_stacked != 1) return fail(IZWI_QMM_ERR_INVALID, "forward on an expert stack");
+    if (G.n != U.n || G.k != U.k)
+        return fail(IZWI_QMM_ERR_INVALID, "gate is [%lld, %lld], up is [%lld, %lld]", (long long)G.n, (long long)G.k,
+                    (long long)U.n, (long long)U.k);
+    if (D.k != G.n)
+        return fail(IZWI_QMM_ERR_INVALID, "shape mismatch in qmatmul, lhs: [%lld, %lld], rhs: (%lld, %lld)", (long long)m,
+                    (long long)G.n, (long long)D.n, (long long)D.k);
+    if (gate->device != up->device || gate->device != down->device)
+        return fail(IZWI_QMM_ERR_INVALID, "the weights live on different devices");
+    if (m < 0) return fail(IZWI_QMM_ERR_INVALID, "negative m");
+    if (m == 0 || D.n == 0) return IZWI_QMM_OK;
+    if (!x) return fail(IZWI_QMM_ERR_INVALID, "x is NULL");
+    if (!y) return fail(IZWI_QMM_ERR_INVALID, "y is NULL");
+    hipStream_t stream = (hipStream_t)stream_;
+    Staged xi, yo;
+    HIP_TRY(xi.in(x, (size_t)m * G.k * sizeof(float), mem_space, stream));
+    HIP_TRY(yo.out(y, (size_t)m * D.n * sizeof(float), mem_space, stream));
+    auto align256 = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t part = align256((size_t)m * G.n * sizeof(float)); // one [m, intermediate] f32 matrix
+    const bool records = m >= mfma_min_m() && m <= 64 && G.dtype == U.dtype;
+    if (records) {
+        // Rows for the matrix-core kernels: activation records all the way.  x is quantized once for
+        // gate | up (one launch for both), silu(g) * u is quantized straight into the records that
+        // down reads: four launches, the intermediate never exists as an f32 matrix of its own
+        // beside g and u.  The arithmetic is that of the separate calls (same quantizers, same
+        // kernels), so are the bits.
+        const size_t rx = align256(qmm_records_bytes(G.dtype, m, G.k)), rh = align256(qmm_records_bytes(D.dtype, m, D.k));
+        uint8_t* ws = nullptr;
+        HIP_TRY(get_scratch(gate->device, stream, rx + 2 * part + rh, (void**)&ws));
+        float* g = reinterpret_cast<float*>(ws + rx);
+        float* u = reinterpret_cast<float*>(ws + rx + part);
+        uint8_t* rec_h = ws + rx + 2 * part;
+        if (profiling()) g_silu_fused.fetch_add(1, std::memory_order_relaxed);
+        HIP_TRY(qmm_launch_quantize_ws(G.dtype, (const float*)xi.dev, m, G.k, ws, stream));
+        const izwi_qmm_weight* gu[2] = {gate, up};
+        float* gu_y[2] = {g, u};
+        if (int rc = batched_group_on_records(gu, 2, nullptr, m, gu_y, ws, stream)) return rc;
+        HIP_TRY(qmm_launch_quantize_silu_mul_ws(D.dtype, g, u, m, D.k, rec_h, stream));
+        float* dy[1] = {(float*)yo.dev};
+        if (int rc = batched_group_on_records(&down, 1, nullptr, m, dy, rec_h, stream)) return rc;
+    } else {
+        // One or two rows (the activation is applied inside the gate | up launch), prefill sizes and
+        // a gate / up pair of two block types: the two calls, with the intermediate in the stream's
+        // scratch behind everything those calls use of it themselves.
+        const size_t gu_need = forward_scratch_need(G, m, gate->n_cus) + align256((size_t)m * G.k * sizeof(float)) + 2 * part + 1024;
+        const size_t d_need = forward_scratch_need(D, m, down->n_cus);
+        const size_t inner = align256(gu_need > d_need ? gu_need : d_need);
+        uint8_t* ws = nullptr;
+        HIP_TRY(get_scratch(gate->device, stream, inner + part, (void**)&ws));
+        float* h = reinterpret_cast<float*>(ws + inner);
+        if (int rc = gate_up_silu_impl(gate, up, (const float*)xi.dev, m, h, IZWI_QMM_DEVICE, stream_, nullptr, 0.0f)) return rc;
+        if (int rc = izwi_qmm_forward_f32(down, h, m, (float*)yo.dev, IZWI_QMM_DEVICE, stream_)) return rc;
+    }
+    HIP_TRY(yo.finish(stream));
+    return IZWI_QMM_OK;
+}
+
 int izwi_qmm_forward_normed_f32(const izwi_qmm_weight* w, const float* x, int64_t m, const float* norm_weight,
                                 float eps, float* y, int mem_space, void* stream_) {
     QmmCallScope call;

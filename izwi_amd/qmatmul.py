@@ -540,7 +540,21 @@ class Qwen3Mlp:
         self.gate_up_proj, self.down_proj = gate_up_proj, down_proj
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.down_proj.forward(self.gate_up_proj.forward_silu_mul(x))
+        parts = self.gate_up_proj._parts
+        if parts is None or x.dtype != torch.float32:
+            return self.down_proj.forward(self.gate_up_proj.forward_silu_mul(x))
+        # separate gate / up weights, f32 activations: the three projections as one library call
+        gate_proj, up_proj = parts
+        n, k = gate_proj.qtensor.dims2()
+        if x.dim() < 1 or x.shape[-1] != k:
+            raise capi.QmmError(-1, f"shape mismatch in qmatmul, lhs: {tuple(x.shape)}, rhs: ({n}, {k})")
+        if not x.is_contiguous():
+            raise capi.QmmError(-1, "qmatmul requires a contiguous input")
+        m = x.numel() // k if k else 0
+        y = torch.empty(tuple(x.shape[:-1]) + (self.down_proj.qtensor.dims2()[0],), dtype=torch.float32, device=x.device)
+        check(lib().izwi_qmm_mlp_forward_f32(gate_proj.qtensor._h, up_proj.qtensor._h, self.down_proj.qtensor._h,
+                                             x.data_ptr(), m, y.data_ptr(), _space(x), _stream_ptr(x)))
+        return y
 
 
 def quantize_activations(weight_dtype: GgmlDType, x: torch.Tensor) -> torch.Tensor:
