@@ -255,6 +255,14 @@ inline void forward_gate_up_silu(const QMatMul& gate, const QMatMul& up, const f
                                                 stream));
 }
 
+// `Qwen3Mlp::forward` (core.rs:1786-1798), `Separate` gate / up pair: y = down(silu(x Wg^T) * (x Wu^T)),
+// [m, hidden], the results of forward_gate_up_silu followed by down.forward bit for bit.
+inline void mlp_forward(const QMatMul& gate, const QMatMul& up, const QMatMul& down, const float* x, int64_t m,
+                        float* y, MemSpace space, void* stream = nullptr) {
+    check(izwi_qmm_mlp_forward_f32(gate.qtensor()->handle(), up.qtensor()->handle(), down.qtensor()->handle(), x, m, y,
+                                   (int)space, stream));
+}
+
 // The fused-kernel hooks of crates/izwi-core/src/kernels/mod.rs:109-225, f32 arm.  The reference's
 // hooks return None where no kernel applies; these throw izwi::Error where the library refuses.
 namespace kernels {

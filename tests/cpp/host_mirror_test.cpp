@@ -170,6 +170,14 @@ static void folded_calls_match_oracle() {
     std::vector<float*> ys = {got_g.data(), got_h.data()};
     izwi::forward_group_normed({&gate, &up}, x.data(), m, nw.data(), 1e-6f, ys, MemSpace::Host);
     EXPECT(max_rel(got_g, g) < 3e-4f && max_rel(got_h, u) < 3e-4f);
+    {
+        // Qwen3Mlp::forward as one call: the two calls' bits (no norm, no residual here)
+        std::vector<float> h2(h.size()), y2((size_t)m * hidden), y1((size_t)m * hidden);
+        izwi::forward_gate_up_silu(gate, up, x.data(), m, h2.data(), MemSpace::Host);
+        down.forward(h2.data(), m, y2.data(), MemSpace::Host);
+        izwi::mlp_forward(gate, up, down, x.data(), m, y1.data(), MemSpace::Host);
+        EXPECT(y1 == y2);
+    }
     uint32_t best = 0, best_want = 1;
     izwi::kernels::argmax(got.data(), m, hidden, &best, MemSpace::Host);
     oracle_argmax(got.data(), m, hidden, &best_want);
