@@ -364,6 +364,37 @@ __global__ void combine_kernel(const float* __restrict__ y, const float* __restr
     out[idx] = acc;
 }
 
+// The same sums, four columns per thread, the loads of eight slots requested before the first is
+// used (the loop above waits for one slot's load per step: eight round trips in a row).  The slots
+// are still added in order s = 0, 1, ..: the same bits.
+__global__ void combine4_kernel(const float* __restrict__ y, const float* __restrict__ weights,
+                                int64_t t, int top_k, int64_t hidden4, float* __restrict__ out) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= t * hidden4) return;
+    const int64_t tok = idx / hidden4, c4 = idx - tok * hidden4;
+    const float4* yr = reinterpret_cast<const float4*>(y) + tok * top_k * hidden4 + c4;
+    const float* w = weights + tok * top_k;
+    float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (int s0 = 0; s0 < top_k; s0 += 8) {
+        float4 v[8];
+        float ww[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int s = s0 + i < top_k ? s0 + i : top_k - 1; // (a slot past the end: a valid address, unused)
+            v[i] = yr[s * hidden4];
+            ww[i] = w[s];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (s0 + i < top_k) { // uniform
+                acc.x += ww[i] * v[i].x, acc.y += ww[i] * v[i].y;
+                acc.z += ww[i] * v[i].z, acc.w += ww[i] * v[i].w;
+            }
+        }
+    }
+    reinterpret_cast<float4*>(out)[idx] = acc;
+}
+
 } // namespace
 
 size_t qmm_x_blocks_bytes(int64_t rows, int64_t k) { return x_blocks_bytes(rows, (k + 255) / 256); }
@@ -460,6 +491,12 @@ hipError_t qmm_launch_moe_combine(const float* y, const float* weights, int64_t 
                                   int64_t hidden, float* out, hipStream_t stream) {
     int64_t total = t * hidden;
     if (total <= 0) return hipSuccess;
+    if (hidden % 4 == 0 && ((uintptr_t)y | (uintptr_t)out) % 16 == 0) {
+        // (64 threads per workgroup: a few tokens still spread over many CUs)
+        const int64_t total4 = total / 4;
+        combine4_kernel<<<(unsigned)((total4 + 63) / 64), 64, 0, stream>>>(y, weights, t, top_k, hidden / 4, out);
+        return hipGetLastError();
+    }
     combine_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(y, weights, t, top_k,
                                                                         hidden, out);
     return hipGetLastError();
