@@ -228,16 +228,30 @@ __device__ __forceinline__ void block_sort_body(const int32_t* ids, int pairs, i
     __syncthreads();
     // per expert (a wave each, in turn): the runs' counts become the number of earlier pairs of the
     // expert; lane = run, 64 runs per step
-    for (int e = wave; e < n_experts; e += waves) {
-        int carry = 0;
-        for (int r0 = 0; r0 < runs; r0 += 64) {
-            const int r = r0 + lane;
-            const int h = r < runs ? sh[r * stride + e] : 0;
-            const int inc = wave_inclusive_sum(h, lane);
-            if (r < runs) sh[r * stride + e] = carry + inc - h;
-            carry += __shfl(inc, 63);
+    // (few runs: a thread per expert walks them - consecutive experts, consecutive LDS words - instead
+    // of eight wave scans in a row per wave with two lanes in use)
+    if (runs <= 16) {
+        for (int e = threadIdx.x; e < n_experts; e += kBlockSortThreads) {
+            int carry = 0;
+            for (int r = 0; r < runs; r++) {
+                const int h = sh[r * stride + e];
+                sh[r * stride + e] = carry;
+                carry += h;
+            }
+            start[e] = carry;
         }
-        if (lane == 0) start[e] = carry; // the expert's total, for now
+    } else {
+        for (int e = wave; e < n_experts; e += waves) {
+            int carry = 0;
+            for (int r0 = 0; r0 < runs; r0 += 64) {
+                const int r = r0 + lane;
+                const int h = r < runs ? sh[r * stride + e] : 0;
+                const int inc = wave_inclusive_sum(h, lane);
+                if (r < runs) sh[r * stride + e] = carry + inc - h;
+                carry += __shfl(inc, 63);
+            }
+            if (lane == 0) start[e] = carry; // the expert's total, for now
+        }
     }
     __syncthreads();
     // exclusive scan over the experts: thread e holds expert e (n_experts <= 1024), wave scans, then the
