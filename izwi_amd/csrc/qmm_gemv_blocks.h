@@ -61,16 +61,15 @@ __device__ __forceinline__ int row16_min(int v) {
 // four dwords, the block scale and the sum of this lane's 16 quants (bsums[j]).
 __device__ __forceinline__ void quantize_q8k_lane(const float (&v)[16], int j, uint32_t (&q)[4],
                                                   float& d, int& sum16) {
-    float amax = 0.0f;
+    // the lane's first value of largest magnitude (strictly greater: an equal later one does not
+    // replace it; a NaN never wins, as with fmaxf), with its sign
+    float best = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 16; i++) amax = fmaxf(amax, fabsf(v[i]));
-    amax = row16_max(amax);
-    // the reference keeps the FIRST value whose magnitude equals the maximum:
-    // key = position << 1 | sign, smallest key over the block wins
-    int key = 0x7fffffff;
-#pragma unroll
-    for (int i = 15; i >= 0; i--)
-        if (fabsf(v[i]) == amax) key = ((16 * j + i) << 1) | (v[i] < 0.0f ? 1 : 0);
+    for (int i = 0; i < 16; i++) best = fabsf(v[i]) > fabsf(best) ? v[i] : best;
+    const float amax = row16_max(fabsf(best));
+    // the reference keeps the FIRST value of the block whose magnitude equals the maximum: the
+    // lowest lane that holds it (key = lane << 1 | sign, smallest key over the block wins)
+    int key = fabsf(best) == amax ? (j << 1) | (int)(__float_as_uint(best) >> 31) : 0x7fffffff;
     key = row16_min(key);
     sum16 = 0;
     if (amax == 0.0f) {
@@ -83,15 +82,11 @@ __device__ __forceinline__ void quantize_q8k_lane(const float (&v)[16], int j, u
     d = __fdiv_rn(1.0f, iscale);
 #pragma unroll
     for (int w = 0; w < 4; w++) {
-        uint32_t packed = 0;
+        int qi[4];
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
-            float r = roundf(__fmul_rn(iscale, v[4 * w + b]));
-            int qi = (int)fminf(fmaxf(r, -128.0f), 127.0f);
-            sum16 += qi;
-            packed |= ((uint32_t)qi & 0xffu) << (8 * b);
-        }
-        q[w] = packed;
+        for (int b = 0; b < 4; b++) qi[b] = qmm_round_clamp_i8(__fmul_rn(iscale, v[4 * w + b]));
+        q[w] = qmm_pack_i8x4(qi[0], qi[1], qi[2], qi[3]);
+        sum16 = __builtin_amdgcn_sdot4((int)q[w], 0x01010101, sum16, false);
     }
 }
 
@@ -109,14 +104,10 @@ __device__ __forceinline__ void quantize_q80_lane(const float (&v)[16], uint32_t
     d_f16 = qmm_f16_bits_to_f32(d_bits);
 #pragma unroll
     for (int w = 0; w < 4; w++) {
-        uint32_t packed = 0;
+        int qi[4];
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
-            float r = roundf(__fmul_rn(v[4 * w + b], id));
-            int qi = (int)fminf(fmaxf(r, -128.0f), 127.0f);
-            packed |= ((uint32_t)qi & 0xffu) << (8 * b);
-        }
-        q[w] = packed;
+        for (int b = 0; b < 4; b++) qi[b] = qmm_round_clamp_i8(__fmul_rn(v[4 * w + b], id));
+        q[w] = qmm_pack_i8x4(qi[0], qi[1], qi[2], qi[3]);
     }
 }
 

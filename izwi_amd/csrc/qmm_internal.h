@@ -41,6 +41,24 @@ __device__ __forceinline__ uint32_t qmm_byte_of(uint32_t lo, uint32_t hi, int j)
     return ((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xffu;
 }
 
+// The activation quantizers' `round` (Rust f32::round / C roundf: halves away from zero) and clamp
+// as three instructions: the truncation of v + copysign(0.5 - 2^-25, v), the float just below a
+// half.  For every float of magnitude below 2^22 that is roundf(v) exactly (checked over all of
+// them up to 512: where v + 0.5 would round a value just below a half up to the next integer, this
+// sum stays below it, and an exact half still reaches the integer because the sum's tie rounds to
+// even); beyond the clamp nothing changes.  NaN gives 0.
+__device__ __forceinline__ int qmm_round_clamp_i8(float v) {
+    const float half_below = __uint_as_float(0x3effffffu | (__float_as_uint(v) & 0x80000000u));
+    const int q = (int)__fadd_rn(v, half_below);
+    return min(max(q, -128), 127);
+}
+// The low bytes of four ints as one dword (a, b, c, d from the lowest byte up).
+__device__ __forceinline__ uint32_t qmm_pack_i8x4(int a, int b, int c, int d) {
+    const uint32_t ab = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
+    const uint32_t cd = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
+}
+
 __device__ __forceinline__ float qmm_bf16_bits_to_f32(uint16_t b) {
     return __uint_as_float((uint32_t)b << 16);
 }

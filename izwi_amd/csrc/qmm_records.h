@@ -53,18 +53,19 @@ struct Unit {
 // the row inside the 16-row tile whose record starts at `rec`.
 template <int QT>
 __device__ __forceinline__ void quantize_into_record(const float (&v)[16], int j, int mr, uint8_t* rec) {
-    float amax = 0.0f;
+    // the lane's first value of largest magnitude (strictly greater: an equal later one does not
+    // replace it; a NaN never wins, as with fmaxf), with its sign
+    float best = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 16; i++) amax = fmaxf(amax, fabsf(v[i]));
+    for (int i = 0; i < 16; i++) best = fabsf(v[i]) > fabsf(best) ? v[i] : best;
+    float amax = fabsf(best);
     float scale_mul; // quant = round(v * scale_mul)
     float* side = reinterpret_cast<float*>(rec + Unit<QT>::kQuant);
     if (QT == QMM_Q4_K) {
-        // BlockQ8K::from_float: iscale = -128 / (first value of largest magnitude)
+        // BlockQ8K::from_float: iscale = -128 / (first value of largest magnitude): the lowest lane
+        // that holds the block's maximum decides the sign
         amax = row16_max(amax);
-        int key = 0x7fffffff;
-#pragma unroll
-        for (int i = 15; i >= 0; i--)
-            if (fabsf(v[i]) == amax) key = ((16 * j + i) << 1) | (v[i] < 0.0f ? 1 : 0);
+        int key = fabsf(best) == amax ? (j << 1) | (int)(__float_as_uint(best) >> 31) : 0x7fffffff;
         key = row16_min(key);
         float d = 0.0f;
         scale_mul = 0.0f;
@@ -83,15 +84,11 @@ __device__ __forceinline__ void quantize_into_record(const float (&v)[16], int j
     uint32_t q[4];
 #pragma unroll
     for (int w = 0; w < 4; w++) {
-        uint32_t packed = 0;
+        int qi[4];
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
-            // both reference quantizers compute scale * value in f32 and round half away
-            float r = roundf(QT == QMM_Q4_K ? __fmul_rn(scale_mul, v[4 * w + b]) : __fmul_rn(v[4 * w + b], scale_mul));
-            int qi = (int)fminf(fmaxf(r, -128.0f), 127.0f);
-            packed |= ((uint32_t)qi & 0xffu) << (8 * b);
-        }
-        q[w] = packed;
+        for (int b = 0; b < 4; b++) // both reference quantizers compute scale * value in f32 and round half away
+            qi[b] = qmm_round_clamp_i8(QT == QMM_Q4_K ? __fmul_rn(scale_mul, v[4 * w + b]) : __fmul_rn(v[4 * w + b], scale_mul));
+        q[w] = qmm_pack_i8x4(qi[0], qi[1], qi[2], qi[3]);
     }
     const int s = j >> 1, oct = 2 * (j & 1);
     if (QT == QMM_Q4_K) {

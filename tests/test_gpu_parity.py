@@ -97,6 +97,43 @@ def test_activation_quantizer_bit_exact(qa, oracle, dtype):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("dtype", [Q8_0, Q4_K])
+def test_activation_quantizer_rounds_halves_away_from_zero_like_the_reference(qa, oracle, dtype):
+    """Blocks whose scale is exactly 1 (Q8_K: first maximum -128, Q8_0: maximum 127), so that the
+    values ARE the products the quantizers round: exact halves, the floats next to a half on both
+    sides, values at and beyond the clamp; once with the block maximum in front (it decides Q8_K's
+    sign) and once with an equal maximum of the other sign behind it.  Bit-equal blocks from the
+    single-row kernel's quantizer (the exported one), the record quantizer (through a 5-row forward
+    against the oracle product) and the oracle."""
+    k = 512
+    top = -128.0 if dtype == Q4_K else 127.0
+    below = np.nextafter(np.float32(0.5), np.float32(0.0))
+    above = np.nextafter(np.float32(0.5), np.float32(1.0))
+    specials = []
+    for base in (0, 1, 2, 7, 63, 100, 126):
+        for frac in (np.float32(0.5), below, above):
+            specials += [np.float32(base) + frac, -(np.float32(base) + frac)]
+    specials += [126.5, 127.49, -127.5, -127.49, 0.0, -0.0, 1e-30, -1e-30, 0.25, -0.75]
+    x = np.zeros((5, k), dtype=np.float32)
+    rng = np.random.default_rng(5)
+    for r in range(5):
+        for blk in range(k // 32):
+            vals = rng.permutation(np.array(specials, dtype=np.float32))[:31]
+            x[r, 32 * blk] = top
+            x[r, 32 * blk + 1:32 * blk + 32] = vals
+    x[1, 300] = -top  # an equal maximum of the other sign behind the first: the first still decides
+    x[2, 0], x[2, 5] = 3.5, top  # the maximum not in the first lane's values
+    got = qa.quantize_activations(qa.GgmlDType(dtype), torch.from_numpy(x).cuda()).cpu().numpy()
+    want = oracle.quantize_activations(dtype, x)
+    assert np.array_equal(got, want)
+    blocks = make_weight(oracle, dtype, 64, k, 3)
+    y = run_forward(qa, dtype, blocks, 64, k, x)
+    ref = oracle.qmatmul(dtype, x, blocks, 64)
+    assert rel_err(y, ref) < DECODE_TOL
+    y1 = run_forward(qa, dtype, blocks, 64, k, x[:1])
+    assert rel_err(y1, ref[:1]) < DECODE_TOL
+
+
 # ------------------------------------------------------------------ decode --
 def run_forward(qa, dtype, blocks, n, k, x):
     q = qa.QTensor.from_blocks(qa.GgmlDType(dtype), blocks, (n, k))
