@@ -43,10 +43,10 @@ __device__ __forceinline__ uint32_t qmm_byte_of(uint32_t lo, uint32_t hi, int j)
 
 // The activation quantizers' `round` (Rust f32::round / C roundf: halves away from zero) and clamp
 // as three instructions: the truncation of v + copysign(0.5 - 2^-25, v), the float just below a
-// half.  For every float of magnitude below 2^22 that is roundf(v) exactly (checked over all of
-// them up to 512: where v + 0.5 would round a value just below a half up to the next integer, this
-// sum stays below it, and an exact half still reaches the integer because the sum's tie rounds to
-// even); beyond the clamp nothing changes.  NaN gives 0.
+// half.  For every float of magnitude below 2^22 that is roundf(v) exactly (tests/test_round_identity.py
+// checks every float up to 512: where v + 0.5 would round a value just below a half up to the next
+// integer, this sum stays below it, and an exact half still reaches the integer because the sum's
+// tie rounds to even); beyond the clamp nothing changes.  NaN gives 0.
 __device__ __forceinline__ int qmm_round_clamp_i8(float v) {
     const float half_below = __uint_as_float(0x3effffffu | (__float_as_uint(v) & 0x80000000u));
     const int q = (int)__fadd_rn(v, half_below);
