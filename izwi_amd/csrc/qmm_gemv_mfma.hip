@@ -132,11 +132,15 @@ __global__ void quantize_grouped_kernel(const float* __restrict__ x, const float
                                         const int32_t* __restrict__ offsets,
                                         const int32_t* __restrict__ tile_offsets, int n_experts,
                                         const int32_t* __restrict__ tile_expert, uint8_t* __restrict__ ws) {
+    // a workgroup of 256 threads = the 16 rows of one (tile, unit): it writes that unit record whole
+    // (with a row's units side by side in a workgroup, every record was put together from the 8-byte
+    // pieces of 16 workgroups)
     const int64_t group = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
     const int j = threadIdx.x & 15;
-    const int64_t row = group / k_units;
-    const int unit = (int)(group - row * k_units);
-    const int tile = (int)(row >> 4), mr = (int)(row & 15);
+    const int mr = (int)(group & 15);
+    const int64_t tu = group >> 4;
+    const int tile = (int)(tu / k_units);
+    const int unit = (int)(tu - (int64_t)tile * k_units);
     if (tile >= tile_offsets[n_experts]) return; // whole 16-lane groups leave together
     int lo = 0, hi = n_experts; // last e with tile_offsets[e] <= tile: from the table, or searched for
     if (tile_expert) {
