@@ -86,12 +86,14 @@ __device__ __forceinline__ void load_run16(const void* __restrict__ src, const v
 template <int QT, bool XB = false>
 __global__ void quantize_ws_kernel(const void* __restrict__ x, int m, int k, int k_units, int n_tiles,
                                    uint8_t* __restrict__ ws) {
+    // (a workgroup of 256 threads = the 16 rows of one (tile, unit): it writes that unit record whole)
     const int group = (blockIdx.x * blockDim.x + threadIdx.x) >> 4;
     const int j = threadIdx.x & 15;
     const int rows = n_tiles * 16;
     if (group >= rows * k_units) return; // whole 16-lane groups leave together
-    const int row = group / k_units, unit = group - row * k_units;
-    const int tile = row >> 4, mr = row & 15;
+    const int mr = group & 15, tu = group >> 4;
+    const int tile = tu / k_units, unit = tu - tile * k_units;
+    const int row = tile * 16 + mr;
     float v[16];
     const int k0 = unit * 256 + 16 * j;
     if (XB) load_run16<true>(static_cast<const uint16_t*>(x) + (int64_t)row * k + k0, x, row < m && k0 + 16 <= k, v);
@@ -109,8 +111,9 @@ __global__ void quantize_silu_mul_ws_kernel(const float* __restrict__ gate, cons
     const int j = threadIdx.x & 15;
     const int rows = n_tiles * 16;
     if (group >= rows * k_units) return; // whole 16-lane groups leave together
-    const int row = group / k_units, unit = group - row * k_units;
-    const int tile = row >> 4, mr = row & 15;
+    const int mr = group & 15, tu = group >> 4; // (a workgroup = the 16 rows of one (tile, unit), as above)
+    const int tile = tu / k_units, unit = tu - tile * k_units;
+    const int row = tile * 16 + mr;
     float g[16], u[16];
     const int k0 = unit * 256 + 16 * j;
     const bool ok = row < m && k0 + 16 <= k;
