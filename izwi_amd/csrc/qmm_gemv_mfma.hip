@@ -312,6 +312,18 @@ __device__ __forceinline__ void load_wpanel(WPanel<QT>& p, const uint8_t* __rest
         p.q[c] = __builtin_nontemporal_load(b + (size_t)(1 + c) * slots + ln);
 }
 
+// sum + s0 * d0 + s1 * d1 (24-bit factors) as two multiply-adds.  The empty statement behind each
+// keeps the compiler from regrouping the sums into two multiplies and a three-operand add: three
+// instructions where two do (the scale multiplies are the largest share of these kernels' vector
+// instructions).  It names only `sum`, the result of a vector instruction.
+__device__ __forceinline__ int scaled_pair_sum(int s0, int d0, int s1, int d1, int sum) {
+    sum = __mul24(s0, d0) + sum;
+    asm volatile("" : "+v"(sum));
+    sum = __mul24(s1, d1) + sum;
+    asm volatile("" : "+v"(sum));
+    return sum;
+}
+
 // The Q4_K arithmetic of one panel against one 16-row tile of activations, shared by the LDS forms
 // and the register-direct form.  `a_of(u, b)` returns the tile's two matrix-core operands of unit u,
 // sub-block pair b (16 bytes per lane), `side_of(u, bs_lo, bs_hi, dx)` the unit's sub-block sum planes
@@ -365,7 +377,7 @@ __device__ __forceinline__ void q4k_panel_dot(WPanel<QMM_Q4_K>& p, int n_units, 
                 const int sc1 = (int)qmm_byte_of(sc_lo[u], sc_hi[u], 2 * b + 1);
 #pragma unroll
                 for (int r = 0; r < 4; r++) // |dot| < 2^17, scale < 64
-                    isum[u][r] = __mul24(sc1, dhi[e][r]) + (__mul24(sc0, dlo[e][r]) + isum[u][r]);
+                    isum[u][r] = scaled_pair_sum(sc0, dlo[e][r], sc1, dhi[e][r], isum[u][r]);
             }
         }
     }
@@ -453,8 +465,7 @@ __device__ __forceinline__ void q4k_tile_dot(const Q4Prepared<NU>& t, AFetch&& a
                 const int sc0 = (int)qmm_byte_of(t.sc_lo[u], t.sc_hi[u], 2 * b);
                 const int sc1 = (int)qmm_byte_of(t.sc_lo[u], t.sc_hi[u], 2 * b + 1);
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    isum[r] = __mul24(sc1, dhi[bb][r]) + (__mul24(sc0, dlo[bb][r]) + isum[r]);
+                for (int r = 0; r < 4; r++) isum[r] = scaled_pair_sum(sc0, dlo[bb][r], sc1, dhi[bb][r], isum[r]);
             }
         }
         long bs_lo, bs_hi;
