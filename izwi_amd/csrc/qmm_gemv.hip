@@ -232,7 +232,9 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                         res_raw = *reinterpret_cast<const uint32_t*>(rp);
                     }
                     if (m0 != m_begin) lds_barrier(); // the previous rows' readers are done
-                    x16_finish<XB>(f, in0, v);
+                    // one row of whole 256-value units: an item that exists is in range, and only those are quantized
+                    constexpr bool kWhole = MT == 1 && QT != QMM_Q8_0 && !GATED; // (the gated form measured no faster with it)
+                    x16_finish<XB, kWhole>(f, in0, v);
                     // NORM: sum of the raw squares of the item (all 16 lanes of the group), then x * norm_w
                     auto norm_item = [&](int item, bool in_range, const float4 (&fw)[4]) {
                         float wv[16], ss = 0.0f;
@@ -247,7 +249,7 @@ __device__ __forceinline__ void gemv_body(const GemvParams& P, int m_begin, int 
                     for (int item = group + n_groups; item < items; item += n_groups) {
                         const bool in1 = x_item_issue<MT, XB>(xs, item, true, f);
                         if (NORM) x16_issue<false>(P.norm_w + (item / MT) * 256 + 16 * (threadIdx.x & 15), P.norm_w, in1, fnw);
-                        x16_finish<XB>(f, in1, v);
+                        x16_finish<XB, kWhole>(f, in1, v);
                         if (NORM) norm_item(item, in1, fnw);
                         x_item_quantize<QT, MT>(l, k_units, item, v);
                     }

@@ -125,8 +125,10 @@ __device__ __forceinline__ void x16_issue(const void* __restrict__ src, const vo
 #pragma unroll
     for (int i = 0; i < (XB ? 2 : 4); i++) f[i] = p[i];
 }
-template <bool XB = false>
+// WHOLE: the caller knows the run is in range (it uses the values only then): no selects.
+template <bool XB = false, bool WHOLE = false>
 __device__ __forceinline__ void x16_finish(const float4 (&f)[4], bool in_range, float (&v)[16]) {
+    if (WHOLE) in_range = true;
     if (XB) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
