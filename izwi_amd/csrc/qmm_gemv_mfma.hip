@@ -565,7 +565,7 @@ __device__ __forceinline__ void panel_dot(WPanel<QT>& p, const uint8_t* xu0, int
                         const int sc_hi = (int)(int8_t)((hw >> (16 * (t & 1) + 8)) & 0xffu);
 #pragma unroll
                         for (int r = 0; r < 4; r++) // |dot| <= 16 * 32 * 128, |scale| <= 128
-                            isum[u][r] += __mul24(sc_lo, dlo[e][r]) + __mul24(sc_hi, dhi[e][r]);
+                            isum[u][r] = scaled_pair_sum(sc_lo, dlo[e][r], sc_hi, dhi[e][r], isum[u][r]);
                     }
                 }
             }
