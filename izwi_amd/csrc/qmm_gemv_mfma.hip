@@ -424,7 +424,7 @@ struct Q4Prepared {
 
 // `p` transposed already (transpose_pair on every chunk pair).
 template <int NU>
-__device__ __forceinline__ void q4k_prepare(const WPanel<QMM_Q4_K>& p, Q4Prepared<NU>& t) {
+__device__ __forceinline__ void q4k_prepare(const WPanel<QMM_Q4_K>& p, Q4Prepared<NU>& t, int grp) {
 #pragma unroll
     for (int u = 0; u < NU; u++) {
 #pragma unroll
@@ -438,7 +438,9 @@ __device__ __forceinline__ void q4k_prepare(const WPanel<QMM_Q4_K>& p, Q4Prepare
         t.sc_hi[u] = (p.hdr[u].w & 0x0f0f0f0fu) | (((p.hdr[u].y >> 6) & 0x03030303u) << 4);
         const uint32_t mn_lo = p.hdr[u].z & 0x3f3f3f3fu;
         const uint32_t mn_hi = ((p.hdr[u].w >> 4) & 0x0f0f0f0fu) | (((p.hdr[u].z >> 6) & 0x03030303u) << 4);
-        t.bmn[u] = pack64(mn_lo, mn_hi);
+        // the min term's matrix instructions use k slots 0..7 (the first 16-lane row); the other rows'
+        // slots are made zero HERE, once per panel, so that the activation side needs no select per tile
+        t.bmn[u] = grp == 0 ? pack64(mn_lo, mn_hi) : 0L;
         t.d[u] = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x & 0xffffu));
         t.dmin[u] = qmm_f16_bits_to_f32((uint16_t)(p.hdr[u].x >> 16));
     }
@@ -717,7 +719,7 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
     if constexpr (PREP) {
 #pragma unroll
         for (int b = 0; b < WPanel<QT>::QC / 2; b++) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
-        q4k_prepare<NU>(p, prep);
+        q4k_prepare<NU>(p, prep, grp);
     }
 
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -750,8 +752,7 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
                     [&](int u, long& bs_lo, long& bs_hi, float4& dx) {
                         const uint8_t* side = xu0 + u * UB + Unit<QT>::kQuant;
                         const i64x2 planes = *reinterpret_cast<const i64x2*>(side + 64 + j * 16);
-                        bs_lo = grp == 0 ? planes.x : 0L;
-                        bs_hi = grp == 0 ? planes.y : 0L;
+                        bs_lo = planes.x, bs_hi = planes.y; // (every lane row: the prepared mins are zero past the first)
                         dx = *reinterpret_cast<const float4*>(side + grp * 16);
                     },
                     acc);
@@ -1102,7 +1103,7 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
 #pragma unroll
                 for (int b = 0; b < WPanel<QT>::QC / 2; b++) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
                 Q4Prepared<NU> prep;
-                q4k_prepare<NU>(p, prep);
+                q4k_prepare<NU>(p, prep, grp);
                 // the next panel of the walk, if any, into the registers just freed
                 int nrt = rt, nkg = kg + 1;
                 if (nkg == P.k_groups) nkg = 0, nrt = rt + rt_step;
@@ -1118,8 +1119,7 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
                         [&](int u, long& bs_lo, long& bs_hi, float4& dx) {
                             const uint8_t* side = xu0 + u * UB + Unit<QT>::kQuant;
                             const i64x2 planes = *reinterpret_cast<const i64x2*>(side + 64 + j * 16);
-                            bs_lo = grp == 0 ? planes.x : 0L;
-                            bs_hi = grp == 0 ? planes.y : 0L;
+                            bs_lo = planes.x, bs_hi = planes.y; // (every lane row: the prepared mins are zero past the first)
                             dx = *reinterpret_cast<const float4*>(side + grp * 16);
                         },
                         acc[t]);
