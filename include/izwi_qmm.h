@@ -162,6 +162,20 @@ typedef enum izwi_qmm_large_m { IZWI_QMM_LARGE_M_BF16 = 0, IZWI_QMM_LARGE_M_INT8
 int izwi_qmm_set_large_m_arithmetic(int mode);
 int izwi_qmm_get_large_m_arithmetic(void);
 
+/* Form of the bf16 prefill product (more than 128 activation rows, Q4_K / Q8_0 weights, k a multiple
+ * of 64), process-wide.  IZWI_QMM_PREFILL_LDS: the weights are dequantized to bf16 inside the matmul
+ * kernel, tile by tile, on their way into LDS.  IZWI_QMM_PREFILL_PLANE: one pass per call dequantizes
+ * the weight into a bf16 plane in the stream's scratch memory (2 bytes per weight element, see
+ * izwi_qmm_scratch_reserve), and the matmul kernel streams both operands into LDS without touching
+ * them.  IZWI_QMM_PREFILL_AUTO (the default): chosen by size - today the in-LDS form everywhere, which
+ * is the faster one up to 4096 rows on the Qwen3-8B shapes.  IZWI_QMM_PREFILL_FORM=lds / plane at
+ * start-up forces one.  Same bf16 operands and f32 accumulation in both; the sums may
+ * differ in their last bits (order of the k steps inside a matrix instruction is the same, the split
+ * of k over workgroups is not).  No counterpart in the reference. */
+typedef enum izwi_qmm_prefill_form { IZWI_QMM_PREFILL_AUTO = -1, IZWI_QMM_PREFILL_LDS = 0, IZWI_QMM_PREFILL_PLANE = 1 } izwi_qmm_prefill_form;
+int izwi_qmm_set_prefill_form(int form);
+int izwi_qmm_get_prefill_form(void);
+
 /* Form of the MoE expert MLP at many pairs per expert (16-row tiles on the matrix cores): 1 = the
  * expert form (a workgroup per expert and part of its rows keeps up to four activation tiles in LDS,
  * every wave walks weight panels on its own), 0 = the one-shot form (a workgroup per group of row

@@ -32,10 +32,12 @@ from .qmatmul import (  # noqa: F401
     Qwen3QkvProjection,
     asr_profile_diagnostics,
     forward_group,
+    get_prefill_form,
     moe_route,
     moe_sort,
     packed_qmatmul_from_qtensors,
     profile_snapshot,
     quantize_activations,
     quantized_storage_bytes,
+    set_prefill_form,
 )

@@ -111,6 +111,8 @@ PROTOTYPES = {
                                        C.c_int, _vp]),
     "izwi_qmm_set_large_m_arithmetic": (C.c_int, [C.c_int]),
     "izwi_qmm_get_large_m_arithmetic": (C.c_int, []),
+    "izwi_qmm_set_prefill_form": (C.c_int, [C.c_int]),
+    "izwi_qmm_get_prefill_form": (C.c_int, []),
     "izwi_qmm_set_moe_expert_form": (C.c_int, [C.c_int]),
     "izwi_qmm_scratch_reserve": (C.c_int, [_u64, _vp]),
     "izwi_qmm_profile_enable": (C.c_int, [C.c_int]),

@@ -1871,6 +1871,15 @@ int izwi_qmm_set_large_m_arithmetic(int mode) {
 
 int izwi_qmm_get_large_m_arithmetic(void) { return large_m_mode(); }
 
+int izwi_qmm_set_prefill_form(int form) {
+    if (form < IZWI_QMM_PREFILL_AUTO || form > IZWI_QMM_PREFILL_PLANE)
+        return fail(IZWI_QMM_ERR_INVALID, "bad prefill form %d (auto = -1, lds = 0, plane = 1)", form);
+    qmm_set_prefill_form(form);
+    return IZWI_QMM_OK;
+}
+
+int izwi_qmm_get_prefill_form(void) { return qmm_get_prefill_form(); }
+
 int izwi_qmm_set_moe_expert_form(int enabled) {
     g_moe_expert_form.store(enabled < 0 ? -1 : enabled ? 1 : 0, std::memory_order_relaxed);
     return IZWI_QMM_OK;

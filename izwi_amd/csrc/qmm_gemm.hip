@@ -970,8 +970,20 @@ hipError_t launch_group_qt(GemmParams P, int64_t n_planned, int n_cus, hipStream
 
 } // namespace
 
+// a group takes the plane form when every member can
+static bool group_plane_applies(const QmmLayout* const* layouts, int n_weights, int64_t m) {
+    for (int i = 0; i < n_weights; i++)
+        if (!qmm_gemm_plane_applies(*layouts[i], m) || layouts[i]->k != layouts[0]->k) return false;
+    return n_weights >= 1;
+}
+
 size_t qmm_gemm_group_workspace_bytes(const QmmLayout* const* layouts, int n_weights, int64_t m, int n_cus) {
     if (m <= 128 || n_weights < 2) return 0;
+    if (group_plane_applies(layouts, n_weights, m)) {
+        size_t total = 0;
+        for (int i = 0; i < n_weights; i++) total += qmm_gemm_plane_bytes(*layouts[i]);
+        return total;
+    }
     const GemmPlan plan = plan_gemm(m, group_columns(layouts, n_weights), (int)layouts[0]->k_units * 4, n_cus > 0 ? n_cus : 1, true);
     if (plan.slices <= 1) return 0;
     size_t total = 0;
@@ -985,6 +997,10 @@ hipError_t qmm_launch_gemm_bf16_multi(const QmmLayout* const* layouts, const voi
     if (n_weights < 2 || n_weights > QMM_MAX_GROUP) return hipErrorInvalidValue;
     if (m <= 128) return hipErrorNotSupported; // the plain tile kernels: one call per weight
     if (n_cus <= 0) n_cus = 1;
+    if (group_plane_applies(layouts, n_weights, m)) {
+        if (workspace == nullptr) return hipErrorInvalidValue;
+        return qmm_launch_gemm_plane(layouts, tiled, n_weights, x_bf16, m, ys, out_bf16, workspace, n_cus, stream);
+    }
     const QmmLayout& L0 = *layouts[0];
     GemmParams P;
     P.w = (const uint8_t*)tiled[0];
@@ -1026,6 +1042,7 @@ hipError_t qmm_launch_gemm_bf16_multi(const QmmLayout* const* layouts, const voi
 
 size_t qmm_gemm_workspace_bytes(const QmmLayout& L, int64_t m, int n_cus) {
     if (m <= 0 || L.n == 0 || (L.dtype == QMM_Q6_K && m <= 128)) return 0;
+    if (qmm_gemm_plane_applies(L, m)) return qmm_gemm_plane_bytes(L);
     const GemmPlan plan = plan_gemm(m, L.n, (int)L.k_units * 4, n_cus > 0 ? n_cus : 1);
     return plan.slices > 1 ? (size_t)plan.slices * (size_t)m * (size_t)L.n * sizeof(float) : 0;
 }
@@ -1035,6 +1052,11 @@ hipError_t qmm_launch_gemm_bf16(const QmmLayout& L, const void* tiled, const uin
                                 hipStream_t stream, const void* residual) {
     if (m <= 0 || L.n == 0) return hipSuccess;
     if (n_cus <= 0) n_cus = 1;
+    if (qmm_gemm_plane_applies(L, m)) {
+        if (workspace == nullptr) return hipErrorInvalidValue;
+        const QmmLayout* lp = &L;
+        return qmm_launch_gemm_plane(&lp, &tiled, 1, x_bf16, m, &y, out_bf16, workspace, n_cus, stream, residual);
+    }
     GemmParams P;
     P.w = (const uint8_t*)tiled;
     P.x = x_bf16;

@@ -212,6 +212,18 @@ size_t qmm_gemm_group_workspace_bytes(const QmmLayout* const* layouts, int n_wei
 hipError_t qmm_launch_gemm_bf16_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
                                       const uint16_t* x_bf16, int64_t m, void* const* ys, int out_bf16,
                                       void* workspace, int n_cus, hipStream_t stream);
+// Plane form of the prefill product (Q4_K / Q8_0, k a multiple of 64, more than 128 rows): the
+// weights are dequantized once per call into a bf16 plane in `planes` (qmm_gemm_plane_bytes per
+// member, members one after the other) and multiplied by a plain bf16 matrix-core loop fed with
+// LDS-direct loads.  qmm_gemm_plane_applies: whether a call of m rows takes this form
+// (qmm_set_prefill_form: 0 in-LDS form always, 1 plane form wherever it can run, -1 by size).
+bool qmm_gemm_plane_applies(const QmmLayout& L, int64_t m);
+size_t qmm_gemm_plane_bytes(const QmmLayout& L);
+void qmm_set_prefill_form(int form);
+int qmm_get_prefill_form();
+hipError_t qmm_launch_gemm_plane(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
+                                 const uint16_t* x_bf16, int64_t m, void* const* ys, int out_bf16, void* planes,
+                                 int n_cus, hipStream_t stream, const void* residual = nullptr);
 // y[i] = t[i] (+ residual[i]) as f32 or bf16: the epilogue as a kernel of its own, for the forms
 // that cannot fold it
 hipError_t qmm_launch_epilogue(const float* t, const void* residual, void* y, int y_bf16, int64_t count,

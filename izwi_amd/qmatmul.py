@@ -645,5 +645,19 @@ def asr_profile_diagnostics() -> dict:
     }
 
 
+PREFILL_AUTO, PREFILL_LDS, PREFILL_PLANE = -1, 0, 1
+
+
+def set_prefill_form(form: int) -> None:
+    """Form of the bf16 prefill product, process-wide (izwi_qmm_set_prefill_form): PREFILL_LDS
+    dequantizes the weights inside the matmul kernel on their way into LDS, PREFILL_PLANE once per
+    call into a bf16 plane in scratch memory that a plain bf16 matrix-core loop then reads."""
+    capi.check(capi.lib().izwi_qmm_set_prefill_form(int(form)))
+
+
+def get_prefill_form() -> int:
+    return int(capi.lib().izwi_qmm_get_prefill_form())
+
+
 def capi_profile_enabled() -> bool:
     return bool(lib().izwi_qmm_profile_enabled())
