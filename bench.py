@@ -38,6 +38,27 @@ LM_HEAD_8B = ("lm_head", 151936, 4096)
 N_LAYERS_8B = 36
 
 
+_PROBE = None
+
+
+def probe():
+    """bench_probe/libbench_probe.so: the read-only and copy kernels this benchmark times beside the
+    library (built by `make -C bench_probe` / __graft_entry__.build(); not part of libizwi_qmm.so)."""
+    global _PROBE
+    if _PROBE is None:
+        import ctypes as C
+        path = os.path.join(ROOT, "bench_probe", "libbench_probe.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: run `make -C bench_probe`")
+        lib = C.CDLL(path)
+        lib.bench_probe_stream_read.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p]
+        lib.bench_probe_stream_read.restype = C.c_int
+        lib.bench_probe_stream_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int, C.c_void_p]
+        lib.bench_probe_stream_copy.restype = C.c_int
+        _PROBE = lib
+    return _PROBE
+
+
 def gemv_bytes(dtype, n, k, m):
     return n * k * BPE[dtype] + 4 * m * k + 4 * m * n
 
@@ -260,15 +281,138 @@ def cpu_baseline(oracle, dtype, m, budget_s=12.0):
     }
 
 
-def prefill_extra(torch, qa, dtype, m, steps=20, warmup=5, only=None):
+def cpu_baseline_table(oracle, torch, qa):
+    """Part of the cpu_baseline leg (the only one that touches the oracle): for every BASELINE
+    configuration a bounded sample on which the CPU restatement is timed (all host threads) and the HIP
+    path's result is compared with it (max |y - y_ref| / max |y_ref|; dequantization bit for bit).
+    The GPU times of the same configurations are the bench's other figures."""
+    import numpy as np
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+
+    def timed(fn, min_s=0.2):
+        fn()
+        n, t0 = 0, time.perf_counter()
+        while True:
+            r = fn()
+            n += 1
+            dt = time.perf_counter() - t0
+            if dt > min_s:
+                return dt / n, r
+
+    def rel(y, want):
+        return float(np.abs(y.astype(np.float64) - want).max() / max(float(np.abs(want).max()), 1e-30))
+
+    def projection_rows(dtype, shapes, m, seed):
+        cpu_s, worst, exact = 0.0, 0.0, True
+        gg = qa.GgmlDType(dtype)
+        for i, (name, n, k) in enumerate(shapes):
+            blocks = make_blocks(dtype, n, k, seed + i)
+            x = synth_normal(seed + 50 + k, (m, k))
+            dt, want = timed(lambda: oracle.qmatmul(dtype, x, blocks, n), 0.05)
+            cpu_s += dt
+            qt = qa.QTensor.from_blocks(gg, blocks, (n, k))
+            y = qa.QMatMul.from_qtensor(qt).forward(torch.from_numpy(x).cuda()).cpu().numpy()
+            worst = max(worst, rel(y, want))
+            if i == 0:
+                exact = exact and np.array_equal(qt.dequantize().cpu().numpy().view(np.uint32),
+                                                 oracle.dequantize(dtype, blocks, n, k).view(np.uint32))
+            del qt
+        return {"cpu_ms": round(cpu_s * 1e3, 3), "max_rel_err": float(f"{worst:.2e}"), "dequant_bit_exact": bool(exact)}
+
+    table = {"threads": threads}
+    table["C1_q8_0_3072x1024_m1"] = projection_rows(Q8_0, [("up", 3072, 1024)], 1, 3100)
+    table["C2_q8_0_0p6b_layer"] = {f"m{m}": projection_rows(Q8_0, LAYER_06B, m, 3200) for m in (1, 4, 16, 64)}
+    table["C3_q4k_8b_layer"] = {f"m{m}": projection_rows(Q4_K, LAYER_8B, m, 3300) for m in (1, 8, 16)}
+    # C4: bf16 activations, prefill kernel; the CPU restatement on one 1024 x 4096 projection at M = 512
+    c4 = {}
+    for dtype, label in ((Q4_K, "q4k"), (Q8_0, "q8_0")):
+        n, k, m = 1024, 4096, 512
+        blocks = make_blocks(dtype, n, k, 3400)
+        xb = torch.from_numpy(synth_normal(3401, (m, k))).cuda().to(torch.bfloat16)
+        xf = xb.float().cpu().numpy()
+        dt, want = timed(lambda: oracle.qmatmul(dtype, xf, blocks, n), 0.05)
+        y = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType(dtype), blocks, (n, k))).forward_bf16_to_f32(xb)
+        c4[f"{label}_k_proj_m512"] = {"cpu_ms": round(dt * 1e3, 2), "max_rel_err": float(f"{rel(y.cpu().numpy(), want):.2e}")}
+    table["C4_prefill_sample"] = c4
+    # C5: the MoE layer; the oracle is scalar per pair, so T = 512 is checked and timed on 16 of its tokens
+    e, top_k, hidden, inter = 128, 8, 2048, 768
+    gate = np.tile(make_blocks(Q4_K, 8 * inter, hidden, 31), e // 8)
+    up = np.tile(make_blocks(Q4_K, 8 * inter, hidden, 32), e // 8)
+    down = np.tile(make_blocks(Q4_K, 8 * hidden, inter, 33), e // 8)
+    gg = qa.GgmlDType(Q4_K)
+    experts = qa.MoeExperts(qa.QTensor.from_blocks(gg, gate, (e, inter, hidden)), qa.QTensor.from_blocks(gg, up, (e, inter, hidden)),
+                            qa.QTensor.from_blocks(gg, down, (e, hidden, inter)))
+    c5 = {}
+    for t in (1, 16, 512):
+        x = synth_normal(40 + t, (t, hidden))
+        logits = synth_normal(50 + t, (t, e))
+        ids, wts = qa.moe_route(torch.from_numpy(logits).cuda(), top_k)
+        perm, offsets = qa.moe_sort(ids, e)
+        out = experts.forward(torch.from_numpy(x).cuda(), ids, wts, perm, offsets).cpu().numpy()
+        want_ids, want_wts = oracle.moe_route(logits, top_k)
+        want_perm, want_offsets = oracle.moe_sort(want_ids, e)
+        rows = np.arange(t) if t <= 16 else np.linspace(0, t - 1, 16).astype(np.int64)
+        t0 = time.perf_counter()
+        want = oracle.moe_forward(Q4_K, x[rows], want_ids[rows], want_wts[rows], gate, up, down, e, inter)
+        dt = time.perf_counter() - t0
+        c5[f"t{t}"] = {"cpu_ms_per_token": round(dt * 1e3 / rows.size, 3), "tokens_timed": int(rows.size),
+                       "max_rel_err": float(f"{rel(out[rows], want):.2e}"),
+                       "indices_bit_exact": bool(np.array_equal(ids.cpu().numpy(), want_ids)
+                                                 and np.array_equal(perm.cpu().numpy(), want_perm)
+                                                 and np.array_equal(offsets.cpu().numpy(), want_offsets))}
+    table["C5_moe_q4k_30b_a3b"] = c5
+    del experts
+    torch.cuda.empty_cache()
+    return table
+
+
+def prefill_extra(torch, qa, dtype, m, steps=20, warmup=5, only=None, form=None):
     """TFLOP/s of the prefill kernel per projection and per projection group (extra report, not
     `value`): bf16 activations in HBM, bf16 output, called through the C ABI on preallocated buffers.
     `qkv` and `gate_up` are the calls Qwen3Attention::forward / Qwen3Mlp::forward make (q, k, v resp.
-    gate, up on the same activations) as one izwi_qmm_forward_group_bf16 call: one launch."""
+    gate, up on the same activations) as one izwi_qmm_forward_group_bf16 call: one launch.
+    `form`: None = the library's default (weights dequantized to bf16 in LDS inside the matmul kernel),
+    "plane" = the alternative (one dequantization pass per call into a bf16 plane, then a plain bf16
+    matrix-core loop; the pass is inside the timed call)."""
     import ctypes as C
     from izwi_amd import capi
     from izwi_amd.qmatmul import _stream_ptr
     L = capi.lib()
+    before = qa.get_prefill_form()
+    if form is not None:
+        qa.set_prefill_form({"lds": 0, "plane": 1}[form])
+    try:
+        return _prefill_extra(torch, qa, dtype, m, steps, warmup, only, C, capi, _stream_ptr, L)
+    finally:
+        qa.set_prefill_form(before)
+
+
+def library_gemm_extra(torch, m=2048, steps=20, warmup=5):
+    """Extra report, NOT a rate of the path: the vendor library's plain bf16 GEMM (torch.matmul, i.e.
+    hipBLASLt: no quantized weights, no dequantization anywhere) at the shapes of the prefill figures, on
+    the same kind of data (N(0,1) activations, N(0,0.02) weights) and on zeros.  It prices the target:
+    with real data the chip is power-limited under bf16 matrix instructions, and what a tuned pure-bf16
+    kernel reaches at these shapes on this box is the practical ceiling of any kernel that also has to
+    dequantize."""
+    out = {}
+    for label, n, k in (("gate_up", 24576, 4096), ("down", 4096, 12288), ("qkv", 6144, 4096)):
+        x = torch.from_numpy(synth_normal(3, (m, k))).cuda().to(torch.bfloat16)
+        w = torch.from_numpy(synth_normal(4, (n, k), std=0.02)).cuda().to(torch.bfloat16)
+        y = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+        ms = time_eager(torch, lambda: torch.matmul(x, w.t(), out=y), steps, warmup)
+        out[label] = round(2.0 * m * n * k / (ms * 1e-3) / 1e12, 1)
+        if label == "gate_up":
+            x.zero_(), w.zero_()
+            ms = time_eager(torch, lambda: torch.matmul(x, w.t(), out=y), steps, warmup)
+            out["gate_up_all_zero_operands"] = round(2.0 * m * n * k / (ms * 1e-3) / 1e12, 1)
+        del x, w, y
+    torch.cuda.empty_cache()
+    out["note"] = ("torch.matmul bf16 (the vendor GEMM library) on plain bf16 matrices of the same shapes; zeros draw "
+                   "less power and run at a higher clock; not the path, not `value`")
+    return out
+
+
+def _prefill_extra(torch, qa, dtype, m, steps, warmup, only, C, capi, _stream_ptr, L):
     out = {}
     gg = qa.GgmlDType(dtype)
     shapes = {name: (i, n, k) for i, (name, n, k) in enumerate(LAYER_8B)}
@@ -299,6 +443,59 @@ def prefill_extra(torch, qa, dtype, m, steps=20, warmup=5, only=None):
         flops = sum(2.0 * m * shapes[nm][1] * k for nm in names)
         out[label] = round(flops / (ms * 1e-3) / 1e12, 2)
         del mms, x, ys
+    return out
+
+
+LAYER_06B = [("q", 2048, 1024), ("k", 1024, 1024), ("v", 1024, 1024), ("o", 1024, 2048),
+             ("gate", 3072, 1024), ("up", 3072, 1024), ("down", 1024, 3072)]
+
+
+def small_configs_extra(torch, qa, steps=20, warmup=3, n_layers=28):
+    """Extra report (not `value`): BASELINE configurations 1 and 2, which are parity cases first.
+    Config 1: one Q8_0 [3072, 1024] matvec (M = 1), the same weight called back to back in a graph: it is
+    3.3 MB and stays in the caches, so this is launch + critical-path time, not an HBM rate.
+    Config 2: the seven Q8_0 projections of a Qwen3-0.6B-shaped layer at M = 1 / 4 / 16 / 64, called as the
+    reference's blocks call them (q|k|v group, o, gate|up group, down): `hbm` = 28 layers with their own
+    buffers in one graph (470 MB of weights per step: they stream from HBM), `hot` = one layer's buffers
+    replayed 28 times (17 MB: cache-resident)."""
+    gg = qa.GgmlDType(Q8_0)
+    out = {}
+    mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, make_blocks(Q8_0, 3072, 1024, 11), (3072, 1024)))
+    x = torch.from_numpy(synth_normal(12, (1, 1024))).cuda()
+    y = torch.empty((1, 3072), dtype=torch.float32, device="cuda")
+    calls = [(mm, x, y)] * 64
+    t, g = time_graph(torch, lambda: run_calls(qa, calls), steps, warmup)
+    b = gemv_bytes(Q8_0, 3072, 1024, 1)
+    out["config1_q8_0_3072x1024_m1"] = {"us_per_call": round(t * 1e3 / 64, 2), "gbs": round(b / (t * 1e-3 / 64) / 1e9, 1),
+                                        "note": "same 3.3 MB weight every call: cache-resident, launch-bound"}
+    del g, calls, mm
+    host = {name: make_blocks(Q8_0, n, k, 1100 + i) for i, (name, n, k) in enumerate(LAYER_06B)}
+
+    def layer():
+        return [(qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(gg, host[name], (n, k))), n, k) for name, n, k in LAYER_06B]
+    layers = [layer() for _ in range(n_layers)]
+    c2 = {}
+    for m in (1, 4, 16, 64):
+        xs = {k: torch.from_numpy(synth_normal(7 + k, (m, k))).cuda() for k in (1024, 2048, 3072)}
+        outb = lambda n: torch.empty((m, n), dtype=torch.float32, device="cuda")
+
+        def layer_calls(w):
+            return [([w[0][0], w[1][0], w[2][0]], xs[1024], [outb(2048), outb(1024), outb(1024)]),
+                    (w[3][0], xs[2048], outb(1024)),
+                    ([w[4][0], w[5][0]], xs[1024], [outb(3072), outb(3072)]),
+                    (w[6][0], xs[3072], outb(1024))]
+        layer_bytes = sum(gemv_bytes(Q8_0, n, k, m) for _, n, k in LAYER_06B)
+        cold = [c for w in layers for c in layer_calls(w)]
+        t, g = time_graph(torch, lambda: run_calls(qa, cold), max(5, steps // 2), warmup)
+        del g
+        hot = layer_calls(layers[0]) * n_layers
+        th, g = time_graph(torch, lambda: run_calls(qa, hot), max(5, steps // 2), warmup)
+        del g
+        c2[f"m{m}"] = {"hbm_us_per_layer": round(t * 1e3 / n_layers, 2),
+                       "hbm_gbs": round(layer_bytes * n_layers / (t * 1e-3) / 1e9, 1),
+                       "hot_us_per_layer": round(th * 1e3 / n_layers, 2),
+                       "pct_of_hbm_peak": round(100.0 * layer_bytes * n_layers / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 1)}
+    out["config2_q8_0_0p6b_layer"] = c2
     return out
 
 
@@ -460,20 +657,32 @@ def host_pointer_extra(qa, weights, m, passes=2):
 
 def hbm_ceiling_extra(torch, gib=2, reps=10):
     """Extra report: what plain streaming kernels reach on this GPU, beside the nominal 8 TB/s the roofline
-    is priced against: a device-to-device copy (bytes read + written) and a read-only reduction (torch's
-    kernels), `gib` GiB per pass, far beyond the caches."""
+    is priced against, `gib` GiB per pass (far beyond the caches): this benchmark's own read-only kernel
+    (the decode kernel's load shape: one 768-thread workgroup per CU, nine 16-byte non-temporal loads per
+    lane in flight) and its copy kernel (bytes read + written, best of a few grid sizes), and for
+    comparison the runtime's device-to-device copy and torch's copy / reduction kernels."""
     n = gib * (1 << 30) // 4
     x = torch.ones(n, dtype=torch.float32, device="cuda")
     y = torch.empty_like(x)
-    copy_ms = time_eager(torch, lambda: y.copy_(x), reps, 2)
-    read_ms = time_eager(torch, lambda: x.sum(), reps, 2)
-    out = {"copy_gbs": round(2 * n * 4 / (copy_ms * 1e-3) / 1e9, 1), "read_gbs": round(n * 4 / (read_ms * 1e-3) / 1e9, 1),
-           "gib": gib}
+    P = probe()
+    sp = torch.cuda.current_stream().cuda_stream
+
+    def checked(rc):
+        if rc:
+            raise RuntimeError(f"bench_probe call failed: hipError {rc}")
+    read_ms = time_eager(torch, lambda: checked(P.bench_probe_stream_read(x.data_ptr(), n * 4, sp)), reps, 2)
+    copy_ms = min(time_eager(torch, lambda: checked(P.bench_probe_stream_copy(x.data_ptr(), y.data_ptr(), n * 4, w, sp)), reps, 2)
+                  for w in (2, 4, 8))
+    out = {"read_gbs": round(n * 4 / (read_ms * 1e-3) / 1e9, 1), "copy_gbs": round(2 * n * 4 / (copy_ms * 1e-3) / 1e9, 1),
+           "gib": gib, "kernels": "bench_probe_stream_read / bench_probe_stream_copy (this benchmark's own)"}
+    t_copy = time_eager(torch, lambda: y.copy_(x), reps, 2)
+    t_read = time_eager(torch, lambda: x.sum(), reps, 2)
+    out["torch_copy_gbs"] = round(2 * n * 4 / (t_copy * 1e-3) / 1e9, 1)
+    out["torch_sum_read_gbs"] = round(n * 4 / (t_read * 1e-3) / 1e9, 1)
     try:  # the runtime's own device-to-device copy
         import ctypes as C
         hip = C.CDLL("libamdhip64.so")
         hip.hipMemcpyAsync.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
-        sp = torch.cuda.current_stream().cuda_stream
         ms = time_eager(torch, lambda: hip.hipMemcpyAsync(y.data_ptr(), x.data_ptr(), n * 4, 3, sp), reps, 2)
         out["hip_memcpy_d2d_gbs"] = round(2 * n * 4 / (ms * 1e-3) / 1e9, 1)
     except OSError:
@@ -485,14 +694,12 @@ def hbm_ceiling_extra(torch, gib=2, reps=10):
 
 def read_only_floor_extra(torch, qa, dtype, weights, m, steps=10, warmup=3):
     """Extra report (not `value`): the same step with every launch replaced by a launch that only
-    READS as many bytes (izwi_qmm_probe_stream_read over its own buffers, one per call of the
+    READS as many bytes (bench_probe_stream_read over its own buffers, one per call of the
     headline structure: q|k|v, o, gate|up, down per layer + LM head; distinct buffers, one graph,
     the same dependent chain of 145 launches).  What plain reads of the same bytes in the same
     launches reach on this GPU: the headline is to be read against it as well as against the nominal
     peak."""
-    import ctypes as C
-    from izwi_amd import capi
-    L = capi.lib()
+    P = probe()
     per_layer = len(LAYER_8B)
     n_layers = (len(weights) - 1) // per_layer
     kinds = ([0, 1, 2], [3], [4, 5], [6])
@@ -507,9 +714,9 @@ def read_only_floor_extra(torch, qa, dtype, weights, m, steps=10, warmup=3):
     def run():
         sp = torch.cuda.current_stream().cuda_stream
         for b in bufs:
-            rc = L.izwi_qmm_probe_stream_read(b.data_ptr(), b.numel(), sp)
+            rc = P.bench_probe_stream_read(b.data_ptr(), b.numel(), sp)
             if rc:
-                capi.check(rc)
+                raise RuntimeError(f"bench_probe_stream_read failed: hipError {rc}")
 
     t, g = time_graph(torch, run, steps, warmup)
     total = float(sum(sizes))
@@ -817,6 +1024,8 @@ def main():
     ap.add_argument("--moe-only", action="store_true",
                     help="profiling aid: run only izwi_moe_layer_f32 at the Qwen3-30B-A3B shape with --m tokens "
                          "(--steps calls, eager) and print the time per call, nothing else")
+    ap.add_argument("--prefill-form", default=None, choices=["lds", "plane"],
+                    help="with --prefill-only: the form of the prefill product (default: the library's own choice)")
     ap.add_argument("--prefill-only", default=None, choices=["q", "k", "gate", "down", "qkv", "gate_up"],
                     help="profiling aid: run only the prefill call of one 8B projection (--m rows, default "
                          "2048 here; --steps calls) and print its TFLOP/s, nothing else")
@@ -854,9 +1063,9 @@ def main():
 
     if args.prefill_only:
         m = args.m if args.m > 1 else 2048
-        tf = prefill_extra(torch, qa, dtype, m, args.steps, args.warmup, only=args.prefill_only)
+        tf = prefill_extra(torch, qa, dtype, m, args.steps, args.warmup, only=args.prefill_only, form=args.prefill_form)
         print(json.dumps({"prefill_only": args.prefill_only, "m": m, "dtype": "Q4_K" if dtype == Q4_K else "Q8_0",
-                          "tflops": tf[args.prefill_only]}))
+                          "form": args.prefill_form or "default", "tflops": tf[args.prefill_only]}))
         return
 
     if args.calibrate_copy:
@@ -913,6 +1122,7 @@ def main():
             "traffic": measured_traffic(f"{args.workload}:{args.calls}", args.m, total_bytes / launches),
             "avg_launch_us": round(ms * 1e3 / launches, 3),
             "avg_algorithmic_bytes_per_launch": int(total_bytes / launches),
+            "floor": None,  # filled below from the read-only launches of the same structure (extras)
         },
     }
     del calls, _graph
@@ -947,7 +1157,15 @@ def main():
             extras["decode_host_pointer_calls"] = host_pointer_extra(qa, weights, args.m)
             extras["hbm_ceiling_measured"] = hbm_ceiling_extra(torch)
             if args.calls == "grouped":
-                extras["decode_read_only_floor"] = read_only_floor_extra(torch, qa, dtype, weights, args.m)
+                floor = read_only_floor_extra(torch, qa, dtype, weights, args.m)
+                extras["decode_read_only_floor"] = floor
+                # what this launch structure allows: plain reads of the same bytes in the same dependent launches
+                result["roofline"]["floor"] = {
+                    "gbs": floor["gbs"], "frac_of_peak": round(floor["gbs"] / HBM_PEAK_GBS, 4),
+                    "achieved_over_floor": round(gbs / floor["gbs"], 4),
+                    "what": f"read-only launches of the same sizes in the same dependent chain of {launches} launches "
+                            "(bench_probe_stream_read, 16-byte non-temporal loads, best launch shape per size): the "
+                            "rate that one launch per projection call can reach on this GPU at these sizes"}
         except Exception as exc:  # extras never invalidate the headline number
             extras["decode_error"] = repr(exc)
     del weights
@@ -977,6 +1195,12 @@ def main():
                 "pct_of_hbm_peak": round(100.0 * tb / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 2), "m": args.m,
                 "calls_per_step": len(c)}
             del c, g
+            other_key = "decode_q8_0_8b_stack" if other_dtype == Q8_0 else "decode_q4k_8b_stack"
+            for m in (8, 16):  # the same stack at the other batch sizes of the configuration
+                c, tb = make_calls(torch, other_dtype, ow, m)
+                t, g = time_graph(torch, lambda: run_calls(qa, c), max(5, args.steps // 5), 3)
+                extras[other_key][f"m{m}"] = {"gbs": round(tb / (t * 1e-3) / 1e9, 1), "ms_per_step": round(t, 4)}
+                del c, g
             if args.calls == "grouped":
                 floor = read_only_floor_extra(torch, qa, other_dtype, ow, args.m)
                 extras["decode_q8_0_8b_stack" if other_dtype == Q8_0 else "decode_q4k_8b_stack"]["read_only_floor"] = {
@@ -985,6 +1209,10 @@ def main():
             torch.cuda.empty_cache()
         except Exception as exc:
             extras["decode_other_dtype_error"] = repr(exc)
+        try:
+            extras["small_configs_q8_0"] = small_configs_extra(torch, qa)
+        except Exception as exc:
+            extras["small_configs_error"] = repr(exc)
         try:
             extras["moe_30b_a3b_q4k"] = moe_extra(torch, qa)
         except Exception as exc:
@@ -1012,6 +1240,8 @@ def main():
             extras["prefill_tflops_m512_q4k"] = prefill_extra(torch, qa, Q4_K, 512)
             best = max(extras["prefill_tflops_m2048_q4k"].values())
             extras["prefill_best_frac_of_bf16_peak"] = round(best / BF16_PEAK_TFLOPS, 4)
+            extras["prefill_tflops_m2048_q4k_plane_form"] = prefill_extra(torch, qa, Q4_K, 2048, form="plane")
+            extras["prefill_library_bf16_gemm_m2048"] = library_gemm_extra(torch, 2048)
         except Exception as exc:  # extras never invalidate the headline number
             extras["error"] = repr(exc)
     if extras:
@@ -1020,6 +1250,11 @@ def main():
     if not args.no_cpu_baseline:
         from oracle import oracle  # the checker, timed here as the CPU baseline; no other leg touches it
         result["cpu_baseline"] = cpu_baseline(oracle, dtype, args.m)
+        if not args.no_extras:
+            try:
+                result["cpu_baseline"]["per_config"] = cpu_baseline_table(oracle, torch, qa)
+            except Exception as exc:
+                result["cpu_baseline"]["per_config_error"] = repr(exc)
 
     print(json.dumps(result))
 

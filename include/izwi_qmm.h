@@ -472,14 +472,6 @@ int izwi_moe_layer_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
                        int32_t top_k, float* out, int32_t* ids_out, float* weights_out,
                        int mem_space, void* stream);
 
-/* Diagnostic, no counterpart in the reference: one launch that only READS `bytes` of device memory
- * (16-byte non-temporal loads, several in flight per lane, nothing stored; the launch shape is the
- * best of a sweep for the size).  Timed over buffers of the sizes of a model's weights, in the order
- * and with the dependencies of its decode calls, it shows what a plain read of the same bytes in
- * the same launches reaches on this GPU; bench.py reports it beside the decode figures.
- * `device_buffer` must be 16-byte aligned; bytes beyond a multiple of 16 are not read. */
-int izwi_qmm_probe_stream_read(const void* device_buffer, uint64_t bytes, void* stream);
-
 /* --- profiling counters (IZWI_QWEN3_PROFILE, qwen3/core.rs:624-657) ------ */
 
 /* Enabled by izwi_qmm_profile_enable(1) or the IZWI_QWEN3_PROFILE env toggle.

@@ -9,6 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 OK = 0
 DEVICE, HOST = 0, 1
 OUT_F32, OUT_BF16 = 0, 1
+LARGE_M_BF16, LARGE_M_INT8 = 0, 1  # izwi_qmm_large_m
 
 
 class QmmError(RuntimeError):
@@ -77,7 +78,6 @@ PROTOTYPES = {
     "izwi_qmm_chain_set_spin_limit": (C.c_int, [_vp, C.c_uint32]),
     "izwi_qmm_forward_rows_f32": (C.c_int, [_vp, _vp, _i64, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_f32_noalloc": (C.c_int, [_vp, _vp, _i64, _vp, _vp]),
-    "izwi_qmm_probe_stream_read": (C.c_int, [_vp, C.c_uint64, _vp]),
     "izwi_qmm_quantize_weights_f32": (C.c_int, [C.c_int, _vp, _i64, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_group_f32": (C.c_int, [_vp, _i32, _vp, _i64, _vp, C.c_int, _vp]),
     "izwi_qmm_forward_group_bf16": (C.c_int, [_vp, _i32, _vp, _i64, _vp, C.c_int, C.c_int, _vp]),

@@ -938,10 +938,13 @@ extern "C" {
 
 int izwi_rms_norm_f32(const float* x, const float* weight, int64_t rows, int64_t hidden, float eps, float* y,
                       int mem_space, void* stream) {
+    return qmm_guarded("izwi_rms_norm_f32", [&]() -> int {
     return rms_norm_impl<float>(x, weight, rows, hidden, eps, y, mem_space, stream);
+    });
 }
 int izwi_rms_norm_quantize_records_f32(int ggml_weight_dtype, const float* x, const float* weight, int64_t rows,
                                        int64_t hidden, float eps, void* records, void* stream) {
+    return qmm_guarded("izwi_rms_norm_quantize_records_f32", [&]() -> int {
     if (ggml_weight_dtype != IZWI_QMM_Q8_0 && ggml_weight_dtype != IZWI_QMM_Q4_K && ggml_weight_dtype != IZWI_QMM_Q6_K)
         return qmm_fail(IZWI_QMM_ERR_UNSUPPORTED, "ggml dtype %d is not supported", ggml_weight_dtype);
     if (rows < 0 || hidden <= 0) return qmm_fail(IZWI_QMM_ERR_INVALID, "rms_norm: bad shape [%lld, %lld]", (long long)rows, (long long)hidden);
@@ -958,32 +961,43 @@ int izwi_rms_norm_quantize_records_f32(int ggml_weight_dtype, const float* x, co
                         static_cast<uint8_t*>(records), (rows + 15) / 16 * 16};
     OPS_TRY(launch_norm_records(P, ggml_weight_dtype, (hipStream_t)stream));
     return IZWI_QMM_OK;
+    });
 }
 int izwi_rms_norm_f16(const uint16_t* x, const uint16_t* weight, int64_t rows, int64_t hidden, float eps, uint16_t* y,
                       int mem_space, void* stream) {
+    return qmm_guarded("izwi_rms_norm_f16", [&]() -> int {
     return rms_norm_impl<f16_t>((const f16_t*)x, (const f16_t*)weight, rows, hidden, eps, (f16_t*)y, mem_space, stream);
+    });
 }
 
 int izwi_qk_rms_norm_f32(const float* q, const float* k, const float* qk_weight, int64_t q_rows, int64_t k_rows,
                          int64_t head_dim, float eps, float* q_out, float* k_out, int mem_space, void* stream) {
+    return qmm_guarded("izwi_qk_rms_norm_f32", [&]() -> int {
     return qk_rms_norm_impl<float>(q, k, qk_weight, q_rows, k_rows, head_dim, eps, q_out, k_out, mem_space, stream);
+    });
 }
 int izwi_qk_rms_norm_f16(const uint16_t* q, const uint16_t* k, const uint16_t* qk_weight, int64_t q_rows, int64_t k_rows,
                          int64_t head_dim, float eps, uint16_t* q_out, uint16_t* k_out, int mem_space, void* stream) {
+    return qmm_guarded("izwi_qk_rms_norm_f16", [&]() -> int {
     return qk_rms_norm_impl<f16_t>((const f16_t*)q, (const f16_t*)k, (const f16_t*)qk_weight, q_rows, k_rows, head_dim, eps,
                                    (f16_t*)q_out, (f16_t*)k_out, mem_space, stream);
+    });
 }
 
 int izwi_rope_pair_bshd_f32(const float* q, const float* k, const float* cos_sin, int64_t batch, int64_t seq,
                             int64_t q_heads, int64_t k_heads, int64_t head_dim, float* q_out, float* k_out,
                             int mem_space, void* stream) {
+    return qmm_guarded("izwi_rope_pair_bshd_f32", [&]() -> int {
     return rope_pair_impl<float>(q, k, cos_sin, batch, seq, q_heads, k_heads, head_dim, q_out, k_out, mem_space, stream);
+    });
 }
 int izwi_rope_pair_bshd_f16(const uint16_t* q, const uint16_t* k, const uint16_t* cos_sin, int64_t batch, int64_t seq,
                             int64_t q_heads, int64_t k_heads, int64_t head_dim, uint16_t* q_out, uint16_t* k_out,
                             int mem_space, void* stream) {
+    return qmm_guarded("izwi_rope_pair_bshd_f16", [&]() -> int {
     return rope_pair_impl<f16_t>((const f16_t*)q, (const f16_t*)k, (const f16_t*)cos_sin, batch, seq, q_heads, k_heads,
                                  head_dim, (f16_t*)q_out, (f16_t*)k_out, mem_space, stream);
+    });
 }
 
 namespace {
@@ -1006,6 +1020,7 @@ struct ArgmaxProfile {
 } // namespace
 
 int izwi_argmax_f32(const float* logits, int64_t rows, int64_t n, uint32_t* out, int mem_space, void* stream_) {
+    return qmm_guarded("izwi_argmax_f32", [&]() -> int {
     QmmCallScope call;
     ArgmaxProfile prof((hipStream_t)stream_);
     if (int rc = check_space(mem_space)) return rc;
@@ -1039,12 +1054,14 @@ int izwi_argmax_f32(const float* logits, int64_t rows, int64_t n, uint32_t* out,
     }
     OPS_TRY(oo.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qk_norm_rope_append_f32(const float* q, const float* k, const float* v, const float* qk_weight,
                                  const float* cos_sin, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
                                  float eps, float* q_out, float* k_cache, float* v_cache, int64_t kv_capacity,
                                  int64_t pos, void* stream_) {
+    return qmm_guarded("izwi_qk_norm_rope_append_f32", [&]() -> int {
     if (num_heads <= 0 || num_kv_heads <= 0 || num_heads + 2 * num_kv_heads > 0x3fffffff || head_dim <= 0 ||
         head_dim % 2 || head_dim > 8192 || pos < 0 || pos >= kv_capacity)
         return qmm_fail(IZWI_QMM_ERR_INVALID,
@@ -1061,12 +1078,14 @@ int izwi_qk_norm_rope_append_f32(const float* q, const float* k, const float* v,
     qkv_prep_kernel<<<(unsigned)((rows + 3) / 4), 256, 0, (hipStream_t)stream_>>>(P);
     OPS_TRY(hipGetLastError());
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_decode_attention_step_f32(const float* q, const float* k, const float* v, const float* qk_weight,
                                    const float* cos_sin, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
                                    float eps, float* k_cache, float* v_cache, int64_t kv_capacity, int64_t pos,
                                    float scale, float* out, void* stream) {
+    return qmm_guarded("izwi_decode_attention_step_f32", [&]() -> int {
     if (pos < 0 || pos >= kv_capacity)
         return qmm_fail(IZWI_QMM_ERR_INVALID, "decode_attention_step: position %lld of %lld", (long long)pos,
                         (long long)kv_capacity);
@@ -1074,19 +1093,24 @@ int izwi_decode_attention_step_f32(const float* q, const float* k, const float* 
     const AttnPrep prep{k, v, qk_weight, cos_sin, eps};
     return decode_attention_impl<float>(q, k_cache, v_cache, num_heads, num_kv_heads, head_dim, pos + 1, kv_capacity,
                                         scale, out, IZWI_QMM_DEVICE, stream, &prep);
+    });
 }
 
 int izwi_decode_gqa_attention_f32(const float* q, const float* k, const float* v, int64_t num_heads,
                                   int64_t num_kv_heads, int64_t head_dim, int64_t kv_len, int64_t kv_capacity,
                                   float scale, float* out, int mem_space, void* stream) {
+    return qmm_guarded("izwi_decode_gqa_attention_f32", [&]() -> int {
     return decode_attention_impl<float>(q, k, v, num_heads, num_kv_heads, head_dim, kv_len, kv_capacity, scale, out,
                                         mem_space, stream);
+    });
 }
 int izwi_decode_gqa_attention_f16(const uint16_t* q, const uint16_t* k, const uint16_t* v, int64_t num_heads,
                                   int64_t num_kv_heads, int64_t head_dim, int64_t kv_len, int64_t kv_capacity,
                                   float scale, uint16_t* out, int mem_space, void* stream) {
+    return qmm_guarded("izwi_decode_gqa_attention_f16", [&]() -> int {
     return decode_attention_impl<f16_t>((const f16_t*)q, (const f16_t*)k, (const f16_t*)v, num_heads, num_kv_heads,
                                         head_dim, kv_len, kv_capacity, scale, (f16_t*)out, mem_space, stream);
+    });
 }
 
 } // extern "C"

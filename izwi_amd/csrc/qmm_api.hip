@@ -29,6 +29,8 @@ struct izwi_qmm_weight {
     std::atomic<int> is_lm_head;
 };
 
+static_assert(QMM_ERR_HIP_CODE == IZWI_QMM_ERR_HIP, "qmm_guarded reports IZWI_QMM_ERR_HIP");
+
 namespace {
 
 thread_local std::string g_error;
@@ -637,27 +639,34 @@ int izwi_qmm_abi_version(void) { return IZWI_QMM_ABI_VERSION; }
 const char* izwi_qmm_last_error(void) { return g_error.c_str(); }
 
 int izwi_qmm_init(int device) {
+    return qmm_guarded("izwi_qmm_abi_version", [&]() -> int {
     int rc = ensure_device(device, nullptr);
     if (rc) return rc;
     HIP_TRY(hipSetDevice(device));
     void* p = nullptr;
     HIP_TRY(noalloc_scratch_ptr(device, &p)); // the static scratch of this device, looked up once
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_storage_bytes(int ggml_dtype, int64_t rows, int64_t cols, uint64_t* out_bytes) {
+    return qmm_guarded("izwi_qmm_storage_bytes", [&]() -> int {
     if (!out_bytes) return fail(IZWI_QMM_ERR_INVALID, "out_bytes is NULL");
     return storage_bytes(ggml_dtype, rows, cols, out_bytes);
+    });
 }
 
 int izwi_qmm_weight_create(int ggml_dtype, int64_t n, int64_t k, const void* blocks,
                            uint64_t nbytes, int mem_space, izwi_qmm_weight** out) {
+    return qmm_guarded("izwi_qmm_weight_create", [&]() -> int {
     return izwi_qmm_weight_create_stacked(ggml_dtype, 1, n, k, blocks, nbytes, mem_space, out);
+    });
 }
 
 int izwi_qmm_weight_create_stacked(int ggml_dtype, int32_t n_experts, int64_t n, int64_t k,
                                    const void* blocks, uint64_t nbytes, int mem_space,
                                    izwi_qmm_weight** out) {
+    return qmm_guarded("izwi_qmm_weight_create_stacked", [&]() -> int {
     if (n_experts < 1) return fail(IZWI_QMM_ERR_INVALID, "n_experts must be >= 1");
     uint64_t expected = 0;
     int rc = storage_bytes(ggml_dtype, (int64_t)n_experts * n, k, &expected);
@@ -668,12 +677,14 @@ int izwi_qmm_weight_create_stacked(int ggml_dtype, int32_t n_experts, int64_t n,
     if (expected && !blocks) return fail(IZWI_QMM_ERR_INVALID, "blocks is NULL");
     Part part{blocks, nbytes};
     return create_from_parts(ggml_dtype, n_experts, n, k, &part, 1, mem_space, out);
+    });
 }
 
 int izwi_qmm_weight_create_packed(int ggml_dtype, int32_t n_parts, const int64_t* part_rows,
                                   int64_t k, const void* const* part_blocks,
                                   const uint64_t* part_nbytes, int mem_space,
                                   izwi_qmm_weight** out) {
+    return qmm_guarded("izwi_qmm_weight_create_packed", [&]() -> int {
     if (n_parts <= 0 || !part_rows || !part_blocks || !part_nbytes)
         return fail(IZWI_QMM_ERR_INVALID, "Cannot pack empty Qwen3 quantized projection group");
     int64_t total_rows = 0;
@@ -702,6 +713,7 @@ int izwi_qmm_weight_create_packed(int ggml_dtype, int32_t n_parts, const int64_t
                     "Qwen3 packed quantized projection has %llu bytes, expected %llu",
                     (unsigned long long)total_bytes, (unsigned long long)expected_total);
     return create_from_parts(ggml_dtype, 1, total_rows, k, parts.data(), n_parts, mem_space, out);
+    });
 }
 
 void izwi_qmm_weight_destroy(izwi_qmm_weight* w) {
@@ -711,6 +723,7 @@ void izwi_qmm_weight_destroy(izwi_qmm_weight* w) {
 }
 
 int izwi_qmm_weight_get_info(const izwi_qmm_weight* w, izwi_qmm_weight_info* out) {
+    return qmm_guarded("izwi_qmm_weight_get_info", [&]() -> int {
     if (!w || !out) return fail(IZWI_QMM_ERR_INVALID, "NULL argument");
     out->ggml_dtype = w->layout.dtype;
     out->n_stacked = (int32_t)w->layout.n_stacked;
@@ -720,16 +733,20 @@ int izwi_qmm_weight_get_info(const izwi_qmm_weight* w, izwi_qmm_weight_info* out
     out->device = w->device;
     out->reserved = 0;
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_weight_set_lm_head(izwi_qmm_weight* w, int is_lm_head) {
+    return qmm_guarded("izwi_qmm_weight_set_lm_head", [&]() -> int {
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     w->is_lm_head.store(is_lm_head ? 1 : 0, std::memory_order_relaxed);
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_weight_data(const izwi_qmm_weight* w, void* out_blocks, uint64_t nbytes,
                          int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_weight_data", [&]() -> int {
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(mem_space)) return rc;
     if (nbytes != w->nbytes)
@@ -743,9 +760,11 @@ int izwi_qmm_weight_data(const izwi_qmm_weight* w, void* out_blocks, uint64_t nb
     HIP_TRY(qmm_launch_unpack(w->layout, w->tiled, o.dev, stream));
     HIP_TRY(o.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_dequantize_f32(const izwi_qmm_weight* w, float* out, int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_dequantize_f32", [&]() -> int {
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(mem_space)) return rc;
     const QmmLayout& L = w->layout;
@@ -758,10 +777,12 @@ int izwi_qmm_dequantize_f32(const izwi_qmm_weight* w, float* out, int mem_space,
     HIP_TRY(qmm_launch_dequant(L, w->tiled, (float*)o.dev, stream));
     HIP_TRY(o.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_dequantize_rows(const izwi_qmm_weight* w, const int32_t* row_ids, int64_t n_rows, int ids_mem_space,
                              void* out, int out_dtype, int out_mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_dequantize_rows", [&]() -> int {
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(ids_mem_space)) return rc;
     if (int rc = check_space(out_mem_space)) return rc;
@@ -787,10 +808,12 @@ int izwi_qmm_dequantize_rows(const izwi_qmm_weight* w, const int32_t* row_ids, i
     HIP_TRY(o.finish(stream));
     if (ids.owned) HIP_TRY(hipStreamSynchronize(stream)); // the staged ids are freed on return
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_quantize_activations(int ggml_weight_dtype, const float* x, int64_t m, int64_t k,
                                   void* out_blocks, int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_quantize_activations", [&]() -> int {
     if (!type_supported(ggml_weight_dtype))
         return fail(IZWI_QMM_ERR_UNSUPPORTED, "ggml dtype %d is not supported", ggml_weight_dtype);
     if (int rc = check_space(mem_space)) return rc;
@@ -810,10 +833,12 @@ int izwi_qmm_quantize_activations(int ggml_weight_dtype, const float* x, int64_t
     HIP_TRY(qmm_launch_quantize_activations(ggml_weight_dtype, (const float*)xi.dev, m, k, o.dev, stream));
     HIP_TRY(o.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_quantize_weights_f32(int ggml_dtype, const float* w, int64_t n, int64_t k, void* out_blocks,
                                   int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_quantize_weights_f32", [&]() -> int {
     if (ggml_dtype != IZWI_QMM_Q8_0 && ggml_dtype != IZWI_QMM_Q4_K)
         return fail(IZWI_QMM_ERR_UNSUPPORTED, "quantize to ggml dtype %d (Q8_0 and Q4_K are built)", ggml_dtype);
     if (int rc = check_space(mem_space)) return rc;
@@ -837,10 +862,12 @@ int izwi_qmm_quantize_weights_f32(int ggml_dtype, const float* w, int64_t n, int
         HIP_TRY(qmm_launch_quantize_q4k_weights((const float*)wi.dev, n * (k / 256), o.dev, stream));
     HIP_TRY(o.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, float* y,
                          int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_forward_f32", [&]() -> int {
     QmmCallScope call;
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(mem_space)) return rc;
@@ -887,6 +914,7 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
     }
     HIP_TRY(yo.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 uint64_t izwi_qmm_records_bytes(int ggml_weight_dtype, int64_t m, int64_t k) {
@@ -907,24 +935,29 @@ int records_args(int dtype, int64_t m, int64_t k, const void* a, const void* b) 
 } // namespace
 
 int izwi_qmm_quantize_records_f32(int ggml_weight_dtype, const float* x, int64_t m, int64_t k, void* records, void* stream) {
+    return qmm_guarded("izwi_qmm_quantize_records_f32", [&]() -> int {
     if (int rc = records_args(ggml_weight_dtype, m, k, x, records)) return rc;
     if (m == 0) return IZWI_QMM_OK;
     HIP_TRY(qmm_launch_quantize_ws(ggml_weight_dtype, x, m, k, records, (hipStream_t)stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_silu_mul_quantize_records_f32(int ggml_weight_dtype, const float* gate, const float* up, int64_t m, int64_t k,
                                            void* records, void* stream) {
+    return qmm_guarded("izwi_qmm_silu_mul_quantize_records_f32", [&]() -> int {
     if (int rc = records_args(ggml_weight_dtype, m, k, gate, records)) return rc;
     if (m == 0) return IZWI_QMM_OK;
     if (!up) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
     if (profiling()) g_silu_fused.fetch_add(1, std::memory_order_relaxed);
     HIP_TRY(qmm_launch_quantize_silu_mul_ws(ggml_weight_dtype, gate, up, m, k, records, (hipStream_t)stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_forward_group_records_f32(const izwi_qmm_weight* const* weights, int32_t n_weights, const void* records,
                                        int64_t m, float* const* ys, void* stream_) {
+    return qmm_guarded("izwi_qmm_forward_group_records_f32", [&]() -> int {
     if (!weights || !ys) return fail(IZWI_QMM_ERR_INVALID, "NULL argument");
     if (n_weights < 1 || n_weights > QMM_MAX_GROUP)
         return fail(IZWI_QMM_ERR_INVALID, "projection group of %d weights (1..%d supported)", n_weights, QMM_MAX_GROUP);
@@ -944,6 +977,10 @@ int izwi_qmm_forward_group_records_f32(const izwi_qmm_weight* const* weights, in
             return fail(IZWI_QMM_ERR_INVALID, "the group mixes weights that dot against Q8_0 and against Q8_K records");
         if (weights[i]->device != weights[0]->device) return fail(IZWI_QMM_ERR_INVALID, "weights on different devices");
     }
+    int device = 0;
+    if (int rc = current_device(&device)) return rc;
+    if (device != weights[0]->device)
+        return fail(IZWI_QMM_ERR_INVALID, "the weights live on device %d, the current device is %d", weights[0]->device, device);
     hipStream_t stream = (hipStream_t)stream_;
     // one launch per block type (Q4_K and Q6_K members read the same Q8_K records)
     bool done[QMM_MAX_GROUP] = {};
@@ -958,10 +995,12 @@ int izwi_qmm_forward_group_records_f32(const izwi_qmm_weight* const* weights, in
         if (int rc = batched_group_on_records(sub_w, n_sub, nullptr, m, sub_y, const_cast<void*>(records), stream)) return rc;
     }
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_forward_rows_f32(const izwi_qmm_weight* w, const uint32_t* row_ids, int64_t n_rows, const float* x,
                               int64_t m, float* y, int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_forward_rows_f32", [&]() -> int {
     QmmCallScope call;
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(mem_space)) return rc;
@@ -993,9 +1032,11 @@ int izwi_qmm_forward_rows_f32(const izwi_qmm_weight* w, const uint32_t* row_ids,
                                  scratch, w->n_cus, stream));
     HIP_TRY(yo.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_forward_f32_noalloc(const izwi_qmm_weight* w, const float* x, int64_t m, float* y, void* stream_) {
+    return qmm_guarded("izwi_qmm_forward_f32_noalloc", [&]() -> int {
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     const QmmLayout& L = w->layout;
     if (L.n_stacked != 1) return fail(IZWI_QMM_ERR_INVALID, "forward on an expert stack");
@@ -1006,6 +1047,10 @@ int izwi_qmm_forward_f32_noalloc(const izwi_qmm_weight* w, const float* x, int64
     if (m == 0 || L.n == 0) return IZWI_QMM_OK;
     if (!x || !y) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
     hipStream_t stream = (hipStream_t)stream_;
+    int device = 0;
+    if (int rc = current_device(&device)) return rc;
+    if (device != w->device) // (before any launch: the one- and two-row kernel too runs on the weight's pointers)
+        return fail(IZWI_QMM_ERR_INVALID, "the weight lives on device %d, the current device is %d", w->device, device);
     if (m < mfma_min_m()) { // one or two rows: the single-launch kernel has no scratch at all
         HIP_TRY(qmm_launch_gemv(L, w->tiled, x, m, y, w->n_cus, stream));
         return IZWI_QMM_OK;
@@ -1016,16 +1061,13 @@ int izwi_qmm_forward_f32_noalloc(const izwi_qmm_weight* w, const float* x, int64
                     "m = %lld rows of k = %lld need %zu bytes of activation records; the static scratch of "
                     "izwi_qmm_forward_f32_noalloc holds %d",
                     (long long)m, (long long)L.k, need, IZWI_QMM_NOALLOC_SCRATCH_BYTES);
-    int device = 0;
-    if (int rc = current_device(&device)) return rc;
-    if (device != w->device)
-        return fail(IZWI_QMM_ERR_INVALID, "the weight lives on device %d, the current device is %d", w->device, device);
     void* scratch = nullptr;
     HIP_TRY(noalloc_scratch_ptr(device, &scratch));
     // the quantizer writes every record the matmul reads (whole 16-row tiles, rows beyond m as
     // zeros), so nothing of an earlier call's contents is ever read
     HIP_TRY(qmm_launch_gemv_mfma(L, w->tiled, x, m, y, scratch, w->n_cus, stream));
     return IZWI_QMM_OK;
+    });
 }
 
 } // extern "C"
@@ -1063,14 +1105,18 @@ extern "C" {
 int izwi_qmm_forward_group_f32(const izwi_qmm_weight* const* weights, int32_t n_weights,
                                const float* x, int64_t m, float* const* ys, int mem_space,
                                void* stream_) {
+    return qmm_guarded("izwi_qmm_forward_group_f32", [&]() -> int {
     return forward_group_impl(weights, n_weights, x, m, ys, mem_space, stream_, nullptr, 0.0f);
+    });
 }
 
 int izwi_qmm_forward_group_normed_f32(const izwi_qmm_weight* const* weights, int32_t n_weights, const float* x,
                                       int64_t m, const float* norm_weight, float eps, float* const* ys,
                                       int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_forward_group_normed_f32", [&]() -> int {
     if (!norm_weight) return fail(IZWI_QMM_ERR_INVALID, "norm_weight is NULL");
     return forward_group_impl(weights, n_weights, x, m, ys, mem_space, stream_, norm_weight, eps);
+    });
 }
 
 } // extern "C"
@@ -1256,18 +1302,23 @@ extern "C" {
 int izwi_qmm_forward_gate_up_silu_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
                                       const float* x, int64_t m, float* h, int mem_space,
                                       void* stream_) {
+    return qmm_guarded("izwi_qmm_forward_gate_up_silu_f32", [&]() -> int {
     return gate_up_silu_impl(gate, up, x, m, h, mem_space, stream_, nullptr, 0.0f);
+    });
 }
 
 int izwi_qmm_forward_gate_up_silu_normed_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const float* x,
                                              int64_t m, const float* norm_weight, float eps, float* h,
                                              int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_forward_gate_up_silu_normed_f32", [&]() -> int {
     if (!norm_weight) return fail(IZWI_QMM_ERR_INVALID, "norm_weight is NULL");
     return gate_up_silu_impl(gate, up, x, m, h, mem_space, stream_, norm_weight, eps);
+    });
 }
 
 int izwi_qmm_mlp_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_qmm_weight* down,
                              const float* x, int64_t m, float* y, int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_mlp_forward_f32", [&]() -> int {
     QmmCallScope call;
     if (!gate || !up || !down) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(mem_space)) return rc;
@@ -1329,10 +1380,12 @@ int izwi_qmm_mlp_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight*
     }
     HIP_TRY(yo.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_forward_normed_f32(const izwi_qmm_weight* w, const float* x, int64_t m, const float* norm_weight,
                                 float eps, float* y, int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_forward_normed_f32", [&]() -> int {
     QmmCallScope call;
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (!norm_weight) return fail(IZWI_QMM_ERR_INVALID, "norm_weight is NULL");
@@ -1362,6 +1415,7 @@ int izwi_qmm_forward_normed_f32(const izwi_qmm_weight* w, const float* x, int64_
     if (int rc = izwi_qmm_forward_f32(w, normed, m, (float*)yo.dev, IZWI_QMM_DEVICE, stream_)) return rc;
     HIP_TRY(yo.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 } // extern "C"
@@ -1439,6 +1493,7 @@ extern "C" {
 
 int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int64_t m, void* y,
                           int out_dtype, int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_forward_bf16", [&]() -> int {
     QmmCallScope call;
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(mem_space)) return rc;
@@ -1463,10 +1518,12 @@ int izwi_qmm_forward_bf16(const izwi_qmm_weight* w, const uint16_t* x_bf16, int6
                                  out_dtype == IZWI_QMM_OUT_BF16, workspace, w->n_cus, stream));
     HIP_TRY(yo.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_forward_group_bf16(const izwi_qmm_weight* const* weights, int32_t n_weights, const uint16_t* x_bf16,
                                 int64_t m, void* const* ys, int out_dtype, int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_forward_group_bf16", [&]() -> int {
     QmmCallScope call;
     if (!weights || !ys) return fail(IZWI_QMM_ERR_INVALID, "NULL argument");
     if (n_weights < 1 || n_weights > QMM_MAX_GROUP)
@@ -1507,10 +1564,12 @@ int izwi_qmm_forward_group_bf16(const izwi_qmm_weight* const* weights, int32_t n
     for (int i = 0; i < n_weights; i++)
         if (int rc = izwi_qmm_forward_bf16(weights[i], x_bf16, m, ys[i], out_dtype, mem_space, stream_)) return rc;
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_forward_fused(const izwi_qmm_weight* w, const void* x, int x_dtype, int64_t m,
                            const void* residual, void* y, int y_dtype, int mem_space, void* stream_) {
+    return qmm_guarded("izwi_qmm_forward_fused", [&]() -> int {
     QmmCallScope call;
     if (!w) return fail(IZWI_QMM_ERR_INVALID, "NULL weight");
     if (int rc = check_space(mem_space)) return rc;
@@ -1592,10 +1651,12 @@ int izwi_qmm_forward_fused(const izwi_qmm_weight* w, const void* x, int x_dtype,
     }
     HIP_TRY(yo.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_moe_route(const float* logits, int64_t t, int32_t n_experts, int32_t top_k, int32_t* ids,
                    float* weights, int mem_space, void* stream_) {
+    return qmm_guarded("izwi_moe_route", [&]() -> int {
     if (int rc = check_space(mem_space)) return rc;
     if (t < 0) return fail(IZWI_QMM_ERR_INVALID, "negative t");
     if (n_experts < 1 || n_experts > 1024)
@@ -1617,10 +1678,12 @@ int izwi_moe_route(const float* logits, int64_t t, int32_t n_experts, int32_t to
     HIP_TRY(io.finish(stream));
     HIP_TRY(wo.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_moe_sort(const int32_t* ids, int64_t t, int32_t top_k, int32_t n_experts, int32_t* perm,
                   int32_t* offsets, int mem_space, void* stream_) {
+    return qmm_guarded("izwi_moe_sort", [&]() -> int {
     QmmCallScope call;
     if (int rc = check_space(mem_space)) return rc;
     if (t < 0 || top_k < 1 || n_experts < 1 || n_experts > 8192)
@@ -1645,6 +1708,7 @@ int izwi_moe_sort(const int32_t* ids, int64_t t, int32_t top_k, int32_t n_expert
     HIP_TRY(po.finish(stream));
     HIP_TRY(oo.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 namespace {
@@ -1801,6 +1865,7 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
                          const int32_t* ids, const float* weights, int32_t top_k,
                          const int32_t* perm, const int32_t* offsets, float* out, int mem_space,
                          void* stream_) {
+    return qmm_guarded("izwi_moe_forward_f32", [&]() -> int {
     QmmCallScope call;
     if (int rc = moe_check_stacks(gate, up, down)) return rc;
     if (int rc = check_space(mem_space)) return rc;
@@ -1828,11 +1893,13 @@ int izwi_moe_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up,
         return rc;
     HIP_TRY(oo.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_moe_layer_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_qmm_weight* down,
                        const float* logits, const float* x, int64_t t, int32_t top_k, float* out,
                        int32_t* ids_out, float* weights_out, int mem_space, void* stream_) {
+    return qmm_guarded("izwi_moe_layer_f32", [&]() -> int {
     QmmCallScope call;
     if (int rc = moe_check_stacks(gate, up, down)) return rc;
     if (int rc = check_space(mem_space)) return rc;
@@ -1860,46 +1927,58 @@ int izwi_moe_layer_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, c
     if (ids_out) HIP_TRY(io.finish(stream));
     if (weights_out) HIP_TRY(wo.finish(stream));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_set_large_m_arithmetic(int mode) {
+    return qmm_guarded("izwi_qmm_set_large_m_arithmetic", [&]() -> int {
     if (mode != IZWI_QMM_LARGE_M_BF16 && mode != IZWI_QMM_LARGE_M_INT8)
         return fail(IZWI_QMM_ERR_INVALID, "bad large-m arithmetic %d (bf16 = 0, int8 = 1)", mode);
     g_large_m_mode.store(mode, std::memory_order_relaxed);
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_get_large_m_arithmetic(void) { return large_m_mode(); }
 
 int izwi_qmm_set_prefill_form(int form) {
+    return qmm_guarded("izwi_qmm_get_large_m_arithmetic", [&]() -> int {
     if (form < IZWI_QMM_PREFILL_AUTO || form > IZWI_QMM_PREFILL_PLANE)
         return fail(IZWI_QMM_ERR_INVALID, "bad prefill form %d (auto = -1, lds = 0, plane = 1)", form);
     qmm_set_prefill_form(form);
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_get_prefill_form(void) { return qmm_get_prefill_form(); }
 
 int izwi_qmm_set_moe_expert_form(int enabled) {
+    return qmm_guarded("izwi_qmm_get_prefill_form", [&]() -> int {
     g_moe_expert_form.store(enabled < 0 ? -1 : enabled ? 1 : 0, std::memory_order_relaxed);
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_scratch_reserve(uint64_t bytes, void* stream_) {
+    return qmm_guarded("izwi_qmm_scratch_reserve", [&]() -> int {
     int device = 0;
     if (int rc = current_device(&device)) return rc;
     if (int rc = ensure_device(device, nullptr)) return rc;
     void* p = nullptr;
     HIP_TRY(get_scratch(device, (hipStream_t)stream_, (size_t)bytes, &p));
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_profile_enable(int enabled) {
+    return qmm_guarded("izwi_qmm_profile_enable", [&]() -> int {
     g_profile.store(enabled ? 1 : 0, std::memory_order_relaxed);
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_profile_snapshot_get(izwi_qmm_profile_snapshot* out) {
+    return qmm_guarded("izwi_qmm_profile_snapshot_get", [&]() -> int {
     if (!out) return fail(IZWI_QMM_ERR_INVALID, "out is NULL");
     out->qmatmul_calls = g_calls.load(std::memory_order_relaxed);
     out->qmatmul_ns = g_ns.load(std::memory_order_relaxed);
@@ -1912,32 +1991,27 @@ int izwi_qmm_profile_snapshot_get(izwi_qmm_profile_snapshot* out) {
     out->silu_mul_fused_calls = g_silu_fused.load(std::memory_order_relaxed);
     out->silu_mul_fallback_calls = g_silu_fallback.load(std::memory_order_relaxed);
     return IZWI_QMM_OK;
-}
-
-int izwi_qmm_probe_stream_read(const void* device_buffer, uint64_t bytes, void* stream) {
-    QmmCallScope call;
-    if (!device_buffer) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
-    if (((uintptr_t)device_buffer & 15) != 0) return fail(IZWI_QMM_ERR_INVALID, "buffer is not 16-byte aligned");
-    int device = 0, n_cus = 0;
-    if (int rc = qmm_current_device(&device, &n_cus)) return rc;
-    HIP_TRY(qmm_launch_stream_read(device_buffer, (size_t)bytes, n_cus, (hipStream_t)stream));
-    return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_profile_enabled(void) { return profiling() ? 1 : 0; }
 
 int izwi_qmm_profile_argmax_get(uint64_t* calls, uint64_t* ns) {
+    return qmm_guarded("izwi_qmm_profile_enabled", [&]() -> int {
     if (!calls || !ns) return fail(IZWI_QMM_ERR_INVALID, "NULL argument");
     *calls = g_argmax_calls.load(std::memory_order_relaxed);
     *ns = g_argmax_ns.load(std::memory_order_relaxed);
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_profile_reset(void) {
+    return qmm_guarded("izwi_qmm_profile_reset", [&]() -> int {
     for (auto* c : {&g_calls, &g_ns, &g_in_casts, &g_in_cast_ns, &g_out_casts, &g_out_cast_ns,
                     &g_lm_calls, &g_lm_ns, &g_silu_fused, &g_silu_fallback, &g_argmax_calls, &g_argmax_ns})
         c->store(0, std::memory_order_relaxed);
     return IZWI_QMM_OK;
+    });
 }
 
 } // extern "C"

@@ -279,6 +279,7 @@ int fail_hip(hipError_t e, const char* what) {
 extern "C" {
 
 int izwi_qmm_chain_create(const izwi_qmm_chain_step* steps, int32_t n_steps, izwi_qmm_chain** out) {
+    return qmm_guarded("izwi_qmm_chain_create", [&]() -> int {
     if (!out) return qmm_fail(IZWI_QMM_ERR_INVALID, "out is NULL");
     *out = nullptr;
     if (!steps || n_steps < 1 || n_steps > 65536)
@@ -367,26 +368,32 @@ int izwi_qmm_chain_create(const izwi_qmm_chain_step* steps, int32_t n_steps, izw
     }
     *out = c;
     return IZWI_QMM_OK;
+    });
 }
 
 void izwi_qmm_chain_destroy(izwi_qmm_chain* c) { delete c; }
 
 int izwi_qmm_chain_set_spin_limit(izwi_qmm_chain* c, uint32_t polls) {
+    return qmm_guarded("izwi_qmm_chain_set_spin_limit", [&]() -> int {
     if (!c) return qmm_fail(IZWI_QMM_ERR_INVALID, "NULL chain");
     c->spin_limit = polls;
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_chain_run(izwi_qmm_chain* c, void* stream) {
+    return qmm_guarded("izwi_qmm_chain_run", [&]() -> int {
     if (!c) return qmm_fail(IZWI_QMM_ERR_INVALID, "NULL chain");
     hipError_t e = c->dtype == IZWI_QMM_Q4_K   ? launch_chain<QMM_Q4_K>(c, (hipStream_t)stream)
                    : c->dtype == IZWI_QMM_Q6_K ? launch_chain<QMM_Q6_K>(c, (hipStream_t)stream)
                                                : launch_chain<QMM_Q8_0>(c, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip(e, "chained decode kernel");
     return IZWI_QMM_OK;
+    });
 }
 
 int izwi_qmm_chain_status(izwi_qmm_chain* c, void* stream) {
+    return qmm_guarded("izwi_qmm_chain_status", [&]() -> int {
     if (!c) return qmm_fail(IZWI_QMM_ERR_INVALID, "NULL chain");
     hipError_t e = hipStreamSynchronize((hipStream_t)stream);
     if (e != hipSuccess) return fail_hip(e, "hipStreamSynchronize");
@@ -402,6 +409,7 @@ int izwi_qmm_chain_status(izwi_qmm_chain* c, void* stream) {
     return qmm_fail(IZWI_QMM_ERR_HIP,
                     "chained decode: a wait for an earlier step gave up after %u polls (results of that run are invalid)",
                     c->spin_limit);
+    });
 }
 
 } // extern "C"

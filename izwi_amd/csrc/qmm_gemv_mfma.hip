@@ -706,10 +706,15 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
     WPanel<QT> p;
     load_wpanel<QT>(p, wbase + (int64_t)((rt_ok ? rt : 0) * P.k_groups + wk) * P.panel_bytes, P.slots, lane, j);
     // The window has landed.  The single-stage form lets the panel fly on: its arithmetic starts on the
-    // first chunk pair, and all NL loads of the panel are behind the window (every one of them is used:
-    // a load the compiler drops would make the count too lenient).  The other forms transpose the whole
-    // panel before their first stage anyway and wait for everything.
-    if (SINGLE) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
+    // first chunk pair, and all NL loads of the panel are behind the window.  That count is right only
+    // while the compiler keeps every load of the panel: it drops a load whose value no path uses (the
+    // fourth header of a panel instantiated for three units), and the wait is then one short.  So the
+    // counted wait is taken only where every loaded register is used on some path - the unit count a
+    // run-time value (NU = 0: Q8_0, Q6_K, compact Q4_K) or all four units present (NU = 4) - and every
+    // other instantiation waits for everything, as the multi-stage forms do anyway (they transpose the
+    // whole panel before their first stage).
+    constexpr bool kEveryPanelLoadUsed = NU == 0 || NU == 4;
+    if (SINGLE && kEveryPanelLoadUsed) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     lds_barrier();
 

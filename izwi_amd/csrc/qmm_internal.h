@@ -3,6 +3,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <exception>
+#include <new>
+
 #include "qmm_layout.h"
 
 // ---- device helpers --------------------------------------------------------
@@ -105,8 +108,25 @@ __device__ __forceinline__ void qmm_store(void* y, const QmmEpilogue& ep, int64_
 }
 #endif
 
+#define QMM_ERR_HIP_CODE (-3) /* IZWI_QMM_ERR_HIP (checked by a static_assert in qmm_api.hip) */
 // Records the calling thread's error message (read with izwi_qmm_last_error) and returns `code`.
 int qmm_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// No C++ exception may cross the C boundary (the entry points use std::vector, std::unordered_map,
+// std::string and new): every exported function with a status result runs its body through this.
+// The status is IZWI_QMM_ERR_HIP ("the call could not be carried out"), the message names the call.
+template <class F>
+int qmm_guarded(const char* what, F&& f) {
+    try {
+        return f();
+    } catch (const std::bad_alloc&) {
+        return qmm_fail(QMM_ERR_HIP_CODE, "%s: out of host memory", what);
+    } catch (const std::exception& e) {
+        return qmm_fail(QMM_ERR_HIP_CODE, "%s: %s", what, e.what());
+    } catch (...) {
+        return qmm_fail(QMM_ERR_HIP_CODE, "%s: unknown failure", what);
+    }
+}
 
 // The current HIP device, validated (IZWI_QMM_ERR_NO_DEVICE without one), and its CU count.
 int qmm_current_device(int* device, int* n_cus);
@@ -149,8 +169,6 @@ hipError_t qmm_launch_dequant(const QmmLayout& L, const void* tiled, float* out,
 // a row id outside [0, n) gives zeros.
 // BlockQ4K::from_float over `n_blocks` blocks of 256 consecutive f32 values: 144 bytes each into `out`
 hipError_t qmm_launch_quantize_q4k_weights(const float* x, int64_t n_blocks, void* out, hipStream_t stream);
-// read-only stream of `bytes` of device memory (diagnostic)
-hipError_t qmm_launch_stream_read(const void* src, size_t bytes, int n_cus, hipStream_t stream);
 hipError_t qmm_launch_dequant_rows(const QmmLayout& L, const void* tiled, const int32_t* rows, int64_t n_rows,
                                    void* out, int out_bf16, hipStream_t stream);
 

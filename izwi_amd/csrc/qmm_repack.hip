@@ -426,50 +426,6 @@ hipError_t qmm_launch_dequant_rows(const QmmLayout& L, const void* tiled, const 
     return hipGetLastError();
 }
 
-// ---- diagnostic: what a read-only stream of a buffer reaches ------------------------------------
-// Every lane keeps U 16-byte non-temporal loads in flight and folds what it read into a register
-// that an empty volatile asm statement consumes: nothing is stored, and the loads cannot be
-// dropped.  Two launch shapes, each the best of a sweep (unroll 4 / 8 / 9 / 16, 256 / 512 /
-// 768 threads, 1 - 16 workgroups per CU) for its sizes on an MI355X: from 40 MB one 768-thread
-// workgroup per CU with nine loads per lane in flight (the decode kernel's own shape: 350 MB in
-// 54.9 us, 56.7 MB in 9.7 us), below it 256-thread workgroups, up to sixteen per CU, four loads per
-// lane (28.4 MB in 5.65 us, 14.2 MB in 3.8, 9.4 MB in 3.1; per launch in a graph of 36).
-namespace {
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-template <int U, int T>
-__global__ __launch_bounds__(T) void stream_read_kernel(const u32x4* __restrict__ src, int64_t n16) {
-    const int64_t stride = (int64_t)gridDim.x * T;
-    uint32_t fold = 0;
-    int64_t i = (int64_t)blockIdx.x * T + threadIdx.x;
-    for (; i + (U - 1) * stride < n16; i += U * stride) {
-        u32x4 v[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) v[u] = __builtin_nontemporal_load(src + i + u * stride);
-#pragma unroll
-        for (int u = 0; u < U; u++) fold |= v[u].x & v[u].y & v[u].z & v[u].w;
-    }
-    for (; i < n16; i += stride) {
-        const u32x4 a = __builtin_nontemporal_load(src + i);
-        fold |= a.x & a.y & a.z & a.w;
-    }
-    asm volatile("" ::"v"(fold));
-}
-} // namespace
-
-hipError_t qmm_launch_stream_read(const void* src, size_t bytes, int n_cus, hipStream_t stream) {
-    const int64_t n16 = (int64_t)(bytes / 16);
-    if (n16 == 0) return hipSuccess;
-    if (n_cus <= 0) n_cus = 1;
-    if (bytes >= ((size_t)40 << 20)) {
-        stream_read_kernel<9, 768><<<(unsigned)n_cus, 768, 0, stream>>>((const u32x4*)src, n16);
-    } else {
-        int64_t wgs = (n16 + 4 * 256 - 1) / (4 * 256);
-        if (wgs > (int64_t)n_cus * 16) wgs = (int64_t)n_cus * 16;
-        stream_read_kernel<4, 256><<<(unsigned)wgs, 256, 0, stream>>>((const u32x4*)src, n16);
-    }
-    return hipGetLastError();
-}
-
 // ---- QTensor::quantize for Q4_K: f32 rows -> GGUF block bytes -----------------------------------
 // candle-core k_quants.rs `BlockQ4K::from_float` with utils.rs `make_qkx1_quants(15, 5, ..)`: a
 // thread owns one sub-block of 32 values and runs the search exactly as the scalar code does (the

@@ -358,8 +358,16 @@ def forward_group(projections: Sequence["QMatMul"], x: torch.Tensor, norm_weight
     n = len(projections)
     ys = [torch.empty(tuple(x.shape[:-1]) + (p.qtensor.dims2()[0],), dtype=x.dtype, device=x.device)
           for p in projections]
-    if x.dtype == torch.bfloat16:       # prefill: bf16 in, bf16 out (izwi_qmm_forward_group_bf16)
+    if x.dtype == torch.bfloat16:
         assert norm_weight is None
+        # Up to 64 rows (or with the integer arithmetic selected for larger batches) a projection on bf16
+        # activations runs the reference's integer block dots (Qwen3Projection.forward -> forward_fused);
+        # the group must give the same bits as its members' separate forwards, so it takes that path
+        # member by member.  Beyond: one launch of the bf16 matrix-core kernel for the whole group.
+        if m <= 64 or lib().izwi_qmm_get_large_m_arithmetic() == capi.LARGE_M_INT8:
+            for p, y in zip(projections, ys):
+                p.forward_fused(x, out=y)
+            return tuple(ys)
         handles = (C.c_void_p * n)(*[p.qtensor._h for p in projections])
         outs = (C.c_void_p * n)(*[y.data_ptr() for y in ys])
         check(lib().izwi_qmm_forward_group_bf16(handles, n, x.data_ptr(), m, outs, capi.OUT_BF16, _space(x), _stream_ptr(x)))
@@ -418,6 +426,13 @@ class ActivationRecords:
 
     def forward_group(self, projections: Sequence["QMatMul"], outs=None):
         n = len(projections)
+        for p in projections:
+            # the C entry takes the records as a bare pointer: records made for another k or for the other
+            # record type (Q8_0 blocks against Q8_K blocks) would be read out of bounds or as garbage
+            if p.qtensor.dims2()[1] != self.k:
+                raise capi.QmmError(-1, f"records of k = {self.k} given to a projection of k = {p.qtensor.dims2()[1]}")
+            if (p.qtensor.dtype() == GgmlDType.Q8_0) != (self.weight_dtype == GgmlDType.Q8_0):
+                raise capi.QmmError(-1, f"records for {self.weight_dtype.name} weights given to a {p.qtensor.dtype().name} projection")
         ys = outs if outs is not None else [torch.empty((self.m, p.qtensor.dims2()[0]), dtype=torch.float32,
                                                         device=self.data.device) for p in projections]
         handles = (C.c_void_p * n)(*[p.qtensor._h for p in projections])

@@ -703,6 +703,34 @@ def test_projection_group_at_prefill_sizes(qa, oracle, dtype, m, k, ns):
         assert float((h - ref).abs().max()) <= 1e-4 * float(ref.abs().max())
 
 
+@pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
+@pytest.mark.parametrize("m", [1, 2, 16, 64, 100])
+def test_projection_group_on_bf16_activations_equals_the_members_forwards(qa, oracle, dtype, m):
+    """forward_group on bf16 activations gives, bit for bit, what Qwen3Projection.forward gives for
+    every member (the reference's Separate arms just call each projection, qwen3/core.rs:1119-1127):
+    up to 64 rows that is the integer block-dot arithmetic, not the bf16 matrix-core kernel; with
+    the integer arithmetic selected for larger batches too, also beyond."""
+    _say(f"group bf16 policy dtype={dtype} m={m}")
+    dt = qa.GgmlDType(dtype)
+    k, ns = 1024, (512, 256, 48)
+    blocks = [make_weight(oracle, dtype, n, k, 470 + n) for n in ns]
+    parts = [qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, b, (n, k))) for b, n in zip(blocks, ns)]
+    xb = torch.from_numpy(oracle.randn(471 + m, (m, k))).cuda().to(torch.bfloat16)
+    lib = qa.lib()
+    try:
+        if m > 64:
+            assert lib.izwi_qmm_set_large_m_arithmetic(1) == 0
+        got = qa.forward_group(parts, xb)
+        for i, p in enumerate(parts):
+            sep = qa.Qwen3Projection(p).forward(xb)
+            assert got[i].dtype == torch.bfloat16 and torch.equal(got[i], sep), i
+        # and it is the integer arithmetic: the reference's CPU result on the same activations
+        want = oracle.qmatmul(dtype, xb.float().cpu().numpy(), blocks[0], ns[0])
+        assert rel_err(got[0].float().cpu().numpy(), want) < 5e-3  # bf16 rounding of the output
+    finally:
+        lib.izwi_qmm_set_large_m_arithmetic(0)
+
+
 def test_projection_group_8b_gate_up_and_errors(qa, oracle):
     dt = qa.GgmlDType.Q4K
     gate = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, make_weight(oracle, Q4_K, 12288, 4096, 410), (12288, 4096)))

@@ -89,3 +89,32 @@ def test_prefill_scaling_row_independence_repeatability(qa, oracle, weights, dty
         # f32 output of the same kernel rounds to the bf16 output
         yf = mm.forward_bf16_to_f32(x)
         assert torch.equal(yf.to(torch.bfloat16).view(torch.int16), y.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [12, 8, 14])
+@pytest.mark.parametrize("k", [4096, 768, 1280, 512, 2048])
+@pytest.mark.parametrize("m", [3, 16])
+def test_single_stage_batched_decode_is_repeatable(qa, oracle, dtype, k, m):
+    """Every single-stage instantiation of the batched decode kernel (one tile of rows, one activation
+    window; Q4_K with four-unit panels in straight-line and compact form, three- and two-unit panels,
+    a ragged last panel, Q8_0, Q6_K) starts its arithmetic on a counted wait for the activation window
+    while the weight panel is still in flight.  A count that is one short shows as results that change
+    from run to run while the chip is busy: the same call six times on a matrix of many row-tiles gives
+    identical bits, and they are the oracle's sums."""
+    import np_ref
+    n = 8192 if k <= 2048 else 6144
+    if dtype == 14:
+        blocks = np_ref.random_q6_k_blocks(700 + k, n, k)
+    else:
+        blocks = oracle.quantize(dtype, oracle.randn(701 + k, (n, k), std=0.02))
+    q = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(qa.GgmlDType(dtype), blocks, (n, k)))
+    x = torch.from_numpy(oracle.randn(702 + m, (m, k))).cuda()
+    outs = [q.forward(x) for _ in range(6)]
+    torch.cuda.synchronize()
+    for o in outs[1:]:
+        assert torch.equal(o.view(torch.int32), outs[0].view(torch.int32))
+    rows = np.unique(np.random.default_rng(k + m).integers(0, n, 64))
+    bpr = blocks.size // n
+    want = oracle.qmatmul(dtype, x.cpu().numpy(), blocks.reshape(n, bpr)[rows].reshape(-1), rows.size)
+    got = outs[0][:, torch.from_numpy(rows).cuda()].cpu().numpy()
+    assert float(np.abs(got - want).max()) <= 1e-4 * float(np.abs(want).max())
