@@ -273,7 +273,18 @@ int izwi_qmm_forward_group_records_f32(const izwi_qmm_weight* const* weights, in
 
 /* --- chained decode: the projections of one token as one launch ----------- */
 
-/* One token's projections in the order `Qwen3Layer::forward` issues them (qwen3/core.rs:1863-1881:
+/* EXPERIMENTAL, and SLOWER than the separate calls it replaces (1.44 against 1.01 ms per Qwen3-8B token,
+ * see the end of this comment): kept as the measured alternative for callers whose constraint is the
+ * number of launches, not time.  The interface may change or go.  Restrictions that follow from its
+ * design (one resident workgroup per compute unit, steps handed over through counters in memory):
+ *  - single stream, not re-entrant: a chain owns one set of counters and one error word; running the
+ *    same chain on two streams, or twice at the same time, corrupts both runs and nothing detects it;
+ *  - nothing else may run on the GPU beside it (it needs every compute unit for the whole launch);
+ *  - once a wait inside a run has given up, the error word stays set: every later run or graph replay
+ *    leaves all its waits at once and writes invalid results until izwi_qmm_chain_status has been
+ *    called (it reports the failure and clears the word).  Call it after every token you care about.
+ *
+ * One token's projections in the order `Qwen3Layer::forward` issues them (qwen3/core.rs:1863-1881:
  * q|k|v, o, gate|up, down, layer after layer; `Qwen3Model::logits_from_hidden`, core.rs:2114-2125,
  * at the end) depend on each other: each reads activations that an earlier one (or the attention /
  * activation kernel between them) wrote.  As separate calls every one of them pays the gap
