@@ -499,6 +499,33 @@ def small_configs_extra(torch, qa, steps=20, warmup=3, n_layers=28):
     return out
 
 
+def batched_percall(torch, qa, dtype, m, steps=30, warmup=5):
+    """Profiling aid (--batched-percall): microseconds per call of the four projection calls of a
+    Qwen3-8B layer at `m` rows on activation records (the matmul launch alone), each kind as a graph of
+    36 layers' distinct weights."""
+    weights = build_decode_weights(torch, qa, dtype, N_LAYERS_8B, False)
+    per = len(LAYER_8B)
+    xs = {k: torch.from_numpy(synth_normal(7 + k, (m, k))).cuda() for k in (4096, 12288)}
+    recs = {k: qa.ActivationRecords.quantize(qa.GgmlDType(dtype), xs[k]) for k in xs}
+    kinds = {"qkv": ([0, 1, 2], 4096), "o": ([3], 4096), "gate_up": ([4, 5], 4096), "down": ([6], 12288)}
+    res = {}
+    for name, (idx, k) in kinds.items():
+        groups = []
+        for layer in range(N_LAYERS_8B):
+            w = weights[layer * per:(layer + 1) * per]
+            groups.append(([w[i][0] for i in idx],
+                           [torch.empty((m, w[i][1]), dtype=torch.float32, device="cuda") for i in idx]))
+
+        def fn():
+            for ps, outs in groups:
+                recs[k].forward_group(ps, outs)
+        ms, g = time_graph(torch, fn, steps, warmup)
+        res[name] = round(ms * 1e3 / N_LAYERS_8B, 2)
+        del g
+    res["layer"] = round(sum(res.values()), 2)
+    return res
+
+
 def overlap_what_if_extra(torch, qa, calls, total_bytes, n_streams=3, steps=20, warmup=3):
     """Extra report, NOT a rate of the path: the headline's launches spread round-robin over several
     streams inside the graph, so that a launch starts while its predecessor still runs.  That is only
@@ -1024,6 +1051,9 @@ def main():
     ap.add_argument("--moe-only", action="store_true",
                     help="profiling aid: run only izwi_moe_layer_f32 at the Qwen3-30B-A3B shape with --m tokens "
                          "(--steps calls, eager) and print the time per call, nothing else")
+    ap.add_argument("--batched-percall", action="store_true",
+                    help="profiling aid: time only the four projection calls of an 8B layer at --m rows (3..64) on "
+                         "activation records, per call, and print them")
     ap.add_argument("--prefill-form", default=None, choices=["lds", "plane"],
                     help="with --prefill-only: the form of the prefill product (default: the library's own choice)")
     ap.add_argument("--prefill-only", default=None, choices=["q", "k", "gate", "down", "qkv", "gate_up"],
@@ -1042,6 +1072,11 @@ def main():
     torch.cuda.set_device(0)
     qa.lib()
     dtype = Q4_K if args.workload == "decode_q4k_8b_stack" else Q8_0
+
+    if args.batched_percall:
+        print(json.dumps({"batched_percall_us": batched_percall(torch, qa, dtype, args.m if args.m >= 3 else 16),
+                          "m": args.m if args.m >= 3 else 16, "dtype": "Q4_K" if dtype == Q4_K else "Q8_0"}))
+        return
 
     if args.neighbours_only:
         print(json.dumps({"decode_step_neighbours_f32": neighbours_extra(torch, qa, args.steps, args.warmup)}))

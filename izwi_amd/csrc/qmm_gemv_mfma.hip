@@ -35,6 +35,14 @@
 #include "qmm_internal.h"
 #include "qmm_records.h"
 
+// Timing-only ablations of the Q4_K single-tile arithmetic (results are WRONG when set; never defined
+// in the library's build): bit 0 drops the integer scale multiply-adds (the matrix instruction
+// accumulates instead), bit 1 the in-register transposition, bit 2 the nibble split, bit 3 the f32
+// finish and the min term, bit 4 the copy of the activation window into LDS, bit 5 the stores.
+#ifndef QMM_MFMA_ABL
+#define QMM_MFMA_ABL 0
+#endif
+
 namespace {
 
 constexpr int kMaxWaves = 12;
@@ -352,7 +360,7 @@ __device__ __forceinline__ void q4k_panel_dot(WPanel<QMM_Q4_K>& p, int n_units, 
         for (int r = 0; r < 4; r++) isum[u][r] = 0;
 #pragma unroll
     for (int b = 0; b < 4; b++) {
-        if (FIRST) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
+        if (FIRST && !(QMM_MFMA_ABL & 2)) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             // two units at a time: their four matrix instructions are issued back to back and the
@@ -365,10 +373,24 @@ __device__ __forceinline__ void q4k_panel_dot(WPanel<QMM_Q4_K>& p, int n_units, 
                 if (u >= nu) continue; // compile-time, or uniform
                 const uint32_t w0 = e ? qq.z : qq.x, w1 = e ? qq.w : qq.y;
                 const i64x2 aa = a_of(u, b);
+                if (QMM_MFMA_ABL & 5) { // timing only: no scale products (the sums chain through the matrix
+                                        // instructions) and / or no nibble split
+                    const long blo = (QMM_MFMA_ABL & 4) ? pack64(w0, w1) : pack64(w0 & kNib, w1 & kNib);
+                    const long bhi = (QMM_MFMA_ABL & 4) ? pack64(w1, w0) : pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib);
+                    const i32x4 c0 = (QMM_MFMA_ABL & 1) ? i32x4{isum[u][0], isum[u][1], isum[u][2], isum[u][3]} : i32x4{0, 0, 0, 0};
+                    dlo[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(aa.x, blo, c0, 0, 0, 0);
+                    dhi[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(aa.y, bhi, (QMM_MFMA_ABL & 1) ? dlo[e] : i32x4{0, 0, 0, 0}, 0, 0, 0);
+                    if (QMM_MFMA_ABL & 1) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) isum[u][r] = dhi[e][r];
+                    }
+                    continue;
+                }
                 dlo[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(aa.x, pack64(w0 & kNib, w1 & kNib), i32x4{0, 0, 0, 0}, 0, 0, 0);
                 dhi[e] = __builtin_amdgcn_mfma_i32_16x16x32_i8(aa.y, pack64((w0 >> 4) & kNib, (w1 >> 4) & kNib),
                                                                i32x4{0, 0, 0, 0}, 0, 0, 0);
             }
+            if (QMM_MFMA_ABL & 1) continue;
 #pragma unroll
             for (int e = 0; e < 2; e++) {
                 const int u = 2 * h + e;
@@ -380,6 +402,13 @@ __device__ __forceinline__ void q4k_panel_dot(WPanel<QMM_Q4_K>& p, int n_units, 
                     isum[u][r] = scaled_pair_sum(sc0, dlo[e][r], sc1, dhi[e][r], isum[u][r]);
             }
         }
+    }
+    if (QMM_MFMA_ABL & 8) { // timing only: no min term, no f32 finish
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] += __int_as_float(isum[u][r] + (int)p.hdr[u].x);
+        return;
     }
 #pragma unroll
     for (int u = 0; u < 4; u++) {
@@ -693,7 +722,7 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
 
     // the first activation window goes first (loads return in order), then the panel
     const int w0_units = min(P.window_units, P.k_units);
-    issue_window_copy<QT>(records, lds_x, w0_units, wave, waves, lane);
+    if (!(QMM_MFMA_ABL & 16)) issue_window_copy<QT>(records, lds_x, w0_units, wave, waves, lane);
     // A CU's loads return in the order they were issued, for all its waves together: without this
     // barrier the last wave's window pieces queue behind the other waves' panels, and the barrier
     // below - the start of all arithmetic - waits for nearly the whole workgroup's weights.
@@ -777,6 +806,7 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
             // y[tile*16 + 4*grp + r][rt*16 + j] (grouped: the row is a sorted position of the
             // expert, the y row its pair index)
             auto store = [&](int r, float v) {
+                if ((QMM_MFMA_ABL & 32) && v != 12345.0f) return; // timing only: (almost) nothing is stored
                 const int mm = tile * 16 + grp * 4 + r;
                 if (GROUPED) {
                     if (pos_begin + mm < pos_end) yout[(int64_t)P.perm[pos_begin + mm] * n_rows + row] = v;
@@ -789,6 +819,29 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
                 if (rt_ok && row < n_rows) {
 #pragma unroll
                     for (int r = 0; r < 4; r++) store(r, acc[r]);
+                }
+            } else if (!GROUPED && !(QMM_MFMA_ABL & 64)) {
+                // Dense forms: every thread of the workgroup finishes outputs - one (activation row, weight
+                // row) pair at a time, the nwk partial sums added in the order wave wk = 0 adds them - and
+                // consecutive threads store consecutive weight rows of one activation row: nwr * 64 bytes
+                // in one piece (a wave of the k-split storing its own tile writes 64-byte pieces, and the
+                // other nwk - 1 waves of the tile stand by meanwhile).
+                if (SINGLE || tile != 0) lds_barrier(); // the window / the previous tile's sums have been read
+#pragma unroll
+                for (int r = 0; r < 4; r++) lds_red[(wave * 4 + r) * 64 + lane] = acc[r];
+                lds_barrier();
+                const int cols = P.nwr * 16;
+                for (int o = (int)threadIdx.x; o < cols * 16; o += waves * 64) {
+                    const int mrow = o / cols, c = o - mrow * cols;
+                    const int wr2 = c >> 4, j2 = c & 15;
+                    const float* part = lds_red + ((wr2 * P.nwk) * 4 + (mrow & 3)) * 64 + (mrow >> 2) * 16 + j2;
+                    float sum = 0.0f;
+                    for (int w2 = 0; w2 < P.nwk; w2++) sum += part[w2 * 256];
+                    const int rt2 = rtg * P.nwr + wr2, col = rt2 * 16 + j2, mm = tile * 16 + mrow;
+                    if (rt2 < row_tiles && col < n_rows && mm < P.m) {
+                        if (EP) qmm_store(yout, P.ep, (int64_t)mm * n_rows + col, sum);
+                        else yout[(int64_t)mm * n_rows + col] = sum;
+                    }
                 }
             } else {
                 if (SINGLE || tile != 0) lds_barrier(); // the window / the previous tile's sums have been read
@@ -917,15 +970,19 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(
 #pragma unroll
     for (int r = 0; r < 4; r++) lds_red[(wave * 4 + r) * 64 + lane] = acc[r];
     lds_barrier();
-    if (wk == 0 && rt_ok && row < n_rows) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            float sum = 0.0f;
-            for (int w2 = 0; w2 < P.nwk; w2++) sum += lds_red[((wr * P.nwk + w2) * 4 + r) * 64 + lane];
-            if (grp * 4 + r < P.m) {
-                if (EP) qmm_store(yout, P.ep, (int64_t)(grp * 4 + r) * n_rows + row, sum);
-                else yout[(int64_t)(grp * 4 + r) * n_rows + row] = sum;
-            }
+    // every thread finishes outputs (see the one-shot form): the partial sums of a pair added in wave
+    // order, consecutive threads storing consecutive weight rows of one activation row
+    const int cols = P.nwr * 16, threads = P.nwk * P.nwr * 64;
+    for (int o = (int)threadIdx.x; o < cols * 16; o += threads) {
+        const int mrow = o / cols, c = o - mrow * cols;
+        const int wr2 = c >> 4, j2 = c & 15;
+        const float* part = lds_red + ((wr2 * P.nwk) * 4 + (mrow & 3)) * 64 + (mrow >> 2) * 16 + j2;
+        float sum = 0.0f;
+        for (int w2 = 0; w2 < P.nwk; w2++) sum += part[w2 * 256];
+        const int rt2 = rtg * P.nwr + wr2, col = rt2 * 16 + j2;
+        if (rt2 < row_tiles && col < n_rows && mrow < P.m) {
+            if (EP) qmm_store(yout, P.ep, (int64_t)mrow * n_rows + col, sum);
+            else yout[(int64_t)mrow * n_rows + col] = sum;
         }
     }
 }
