@@ -21,8 +21,11 @@
  * reference's default on every backend, model_io.rs:70-83, 144-157); if the
  * mapping fails, or the mode is "off" (izwi_gguf_open_with_mode, IZWI_GGUF_MMAP),
  * the file is read with buffered I/O into memory instead, as the reference falls
- * back (model_io.rs:146-160).  Pointers returned by this API stay valid until
- * izwi_gguf_close.  A handle is immutable and may be shared between threads.
+ * back (model_io.rs:146-160).  In that buffered mode the WHOLE file stays on the host heap for the
+ * life of the handle (the returned tensor pointers point into it): as many bytes of host memory as the
+ * file has, beside the device copies of the tensors that are loaded - close the handle once the
+ * weights are on the device.  The reference's BufReader streams instead; it has no such pointers to keep
+ * valid.  Pointers returned by this API stay valid until izwi_gguf_close.  A handle is immutable and may be shared between threads.
  * No C++ exception leaves these functions: running out of memory on a crafted
  * file is IZWI_QMM_ERR_INVALID.
  */

@@ -300,15 +300,23 @@ namespace {
 
 // The whole file through read(2) into one heap block (the buffered reader of model_io.rs:160; the
 // handle's tensor pointers must stay valid until close, so the bytes are kept rather than streamed).
+// On failure returns NULL and leaves errno describing it: ENOMEM, the error of read(2), or 0 for a
+// file that ended before `size` bytes (read returned 0: errno would otherwise be stale).
 uint8_t* read_whole_file(int fd, size_t size) {
     uint8_t* buf = static_cast<uint8_t*>(malloc(size));
-    if (!buf) return nullptr;
+    if (!buf) {
+        errno = ENOMEM;
+        return nullptr;
+    }
     size_t done = 0;
     while (done < size) {
+        errno = 0;
         const ssize_t n = read(fd, buf + done, std::min<size_t>(size - done, (size_t)1 << 30));
         if (n < 0 && errno == EINTR) continue;
         if (n <= 0) {
+            const int err = n == 0 ? 0 : errno;
             free(buf);
+            errno = err;
             return nullptr;
         }
         done += (size_t)n;
@@ -334,9 +342,10 @@ int open_impl(const char* path, int configured_mode, izwi_gguf** out) {
     const uint8_t* bytes = nullptr;
     bool mapped = false;
     if (mmap_enabled) {
-        // IZWI_GGUF_TEST_FAIL_MMAP=1 makes the mapping attempt fail (fault injection for the test of
-        // the fallback below; a mapping of a readable regular file does not fail otherwise)
-        const char* inject = getenv("IZWI_GGUF_TEST_FAIL_MMAP");
+        // _IZWI_GGUF_PRIVATE_TEST_FAIL_MMAP=1 makes the mapping attempt fail: a private hook of this
+        // library's own test of the fallback below (a mapping of a readable regular file does not fail
+        // otherwise); not a setting, not part of the interface
+        const char* inject = getenv("_IZWI_GGUF_PRIVATE_TEST_FAIL_MMAP");
         void* map = (inject && inject[0] == '1') ? MAP_FAILED
                                                  : mmap(nullptr, (size_t)st.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
         if (map != MAP_FAILED) {
@@ -353,7 +362,7 @@ int open_impl(const char* path, int configured_mode, izwi_gguf** out) {
             const int err = errno;
             close(fd);
             return qmm_fail(IZWI_QMM_ERR_INVALID, "Failed to open GGUF file: reading %s: %s", path,
-                            err ? strerror(err) : "short read or out of memory");
+                            err ? strerror(err) : "unexpected end of file");
         }
     }
     close(fd);

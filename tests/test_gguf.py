@@ -213,10 +213,10 @@ def test_reader_policy_follows_the_reference(qa, tmp_path, monkeypatch):
     assert qa.GgufLoader.from_path(path, M.ON).reader_kind() == K.MAPPED
     monkeypatch.delenv("IZWI_GGUF_MMAP")
     # a mapping that fails falls back to buffered I/O, with the same contents
-    monkeypatch.setenv("IZWI_GGUF_TEST_FAIL_MMAP", "1")
+    monkeypatch.setenv("_IZWI_GGUF_PRIVATE_TEST_FAIL_MMAP", "1")
     fell_back = qa.GgufLoader.from_path(path, M.ON)
     assert fell_back.reader_kind() == K.BUFFERED and contents(fell_back) == contents(mapped)
-    monkeypatch.delenv("IZWI_GGUF_TEST_FAIL_MMAP")
+    monkeypatch.delenv("_IZWI_GGUF_PRIVATE_TEST_FAIL_MMAP")
     # malformed input is an error in buffered mode too
     from izwi_amd.capi import QmmError
     bad = tmp_path / "bad.gguf"
