@@ -38,7 +38,9 @@
 // Timing-only ablations of the Q4_K single-tile arithmetic (results are WRONG when set; never defined
 // in the library's build): bit 0 drops the integer scale multiply-adds (the matrix instruction
 // accumulates instead), bit 1 the in-register transposition, bit 2 the nibble split, bit 3 the f32
-// finish and the min term, bit 4 the copy of the activation window into LDS, bit 5 the stores.
+// finish and the min term, bit 4 the copy of the activation window into LDS, bit 5 the stores; bit 6
+// restores the one-wave k-split finish; bit 7 (Q4_K expert form) keeps a panel's load and preparation
+// and drops its arithmetic against the tiles.
 #ifndef QMM_MFMA_ABL
 #define QMM_MFMA_ABL 0
 #endif
@@ -184,7 +186,7 @@ struct MfmaParams {
     const uint8_t* w;
     const uint8_t* ws; // unit records [n_tiles][k_units]
     float* y;
-    const uint8_t* w2; // grouped form, blockIdx.z == 1: second stack and its output
+    const uint8_t* w2; // grouped and expert forms: second stack and its output
     float* y2;
     int double_buf;    // two LDS windows
     // several weights of equal k and type on the same records in one launch (SINGLE form):
@@ -204,6 +206,7 @@ struct MfmaParams {
     // expert-grouped form: a one-dimensional grid; a workgroup's (expert, stack, row-tile group)
     // is decoded so that all workgroups of an expert run on one XCD (see the kernel)
     int n_experts, stacks;
+    int parts; // expert forms: the row tiles of a stack are shared out to this many items
     const int32_t* perm;
     const int32_t* offsets;      // sorted pairs of expert e: [offsets[e], offsets[e + 1])
     const int32_t* tile_offsets; // its 16-row tiles (records): [tile_offsets[e], tile_offsets[e + 1])
@@ -299,8 +302,15 @@ __device__ __forceinline__ void load_wpanel(WPanel<QT>& p, const uint8_t* __rest
                                             int lane, int j) {
     const u32x4* b = reinterpret_cast<const u32x4*>(base);
     const int ln = lane < slots ? lane : 0;
+    // Addresses as the uniform `base` plus a 32-bit lane offset (the scalar-base form of the load).  The
+    // empty statements keep the offsets' widening to 64 bits in this block: moved out of a caller's
+    // loop, the widened offsets are a register pair and a 64-bit add per load.
+    uint32_t j16 = (uint32_t)j * 16u, ln16 = (uint32_t)ln * 16u;
+    asm volatile("" : "+v"(j16));
+    asm volatile("" : "+v"(ln16));
 #pragma unroll
-    for (int u = 0; u < 4; u++) p.hdr[u] = b[(u * 16 < slots ? u * 16 : 0) + j];
+    for (int u = 0; u < 4; u++)
+        p.hdr[u] = *reinterpret_cast<const u32x4*>(base + ((uint32_t)(u * 16 < slots ? u * 256 : 0) + j16));
     if (QT == QMM_Q6_K) {
         // in the order panel_dot consumes them (loads return in order): per half of the units' 256
         // elements first its two chunks of bit pairs, then its four of nibbles; d last
@@ -315,9 +325,13 @@ __device__ __forceinline__ void load_wpanel(WPanel<QT>& p, const uint8_t* __rest
         for (int u = 0; u < 4; u++) p.dch[u] = b[(size_t)13 * slots + (u * 16 < slots ? u * 16 : 0) + j];
         return;
     }
+    // (a uniform chunk address plus one 32-bit lane offset for all chunks: the scalar-base form of the
+    // load, where a 64-bit address per lane and chunk costs two registers and an add each)
 #pragma unroll
-    for (int c = 0; c < WPanel<QT>::QC; c++)
-        p.q[c] = __builtin_nontemporal_load(b + (size_t)(1 + c) * slots + ln);
+    for (int c = 0; c < WPanel<QT>::QC; c++) {
+        const uint32_t off = (uint32_t)((1 + c) * slots * 16) + ln16; // (a panel is under 32 KiB)
+        p.q[c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + off));
+    }
 }
 
 // sum + s0 * d0 + s1 * d1 (24-bit factors) as two multiply-adds.  The empty statement behind each
@@ -1055,6 +1069,49 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_stream_kernel(MfmaPa
     }
 }
 
+// ---- the expert forms' work items ------------------------------------------------------------
+// An item is (expert, weight stack, part of the stack's row tiles).  Where the items are two per CU, a
+// launch is one workgroup per CU that takes two items in turn; two things decide how evenly the CUs
+// finish:
+//   * an item lives in proportion to its expert's tile count (measured at 128 experts, top-8, 512
+//     tokens, gate | up: 36 us with two tiles, 47 with three), and
+//   * a grid of one workgroup per ITEM leaves the pairing of items on a CU to the order in which
+//     workgroups happen to end, and the hardware places the workgroups of the second round slowly
+//     (measured: CUs idle for 2 - 15 us between their two workgroups, finishing 60 - 101 us after the
+//     launch's start).
+// So the experts are ranked by falling tile count (ties by index) and the items numbered in that
+// order; workgroup c of G takes items c and 2G - 1 - c: a heavy and a light item on every CU.  Every
+// workgroup ranks the experts itself (counts in LDS, one thread per expert against all: under a
+// microsecond up to kRankedExperts experts; past that the experts keep their own order).
+constexpr int kRankedExperts = 512;
+constexpr int kExpertRounds = 2; // items a workgroup takes at most (the kernels' round loops are unrolled)
+
+// order[r] = the expert of rank r.  Returns whether the experts were ranked.  Contains barriers.
+__device__ __forceinline__ bool rank_experts(const int32_t* __restrict__ tile_offsets, int n_experts, int* order, int* scratch) {
+    if (n_experts > kRankedExperts) return false;
+    for (int i = threadIdx.x; i < n_experts; i += blockDim.x) scratch[i] = tile_offsets[i + 1] - tile_offsets[i];
+    __syncthreads();
+    for (int i = threadIdx.x; i < n_experts; i += blockDim.x) {
+        const int c = scratch[i];
+        int rank = 0;
+        for (int o = 0; o < n_experts; o++) {
+            const int co = scratch[o];
+            rank += (co > c || (co == c && o < i)) ? 1 : 0;
+        }
+        order[rank] = i; // a permutation: every slot is written once
+    }
+    __syncthreads(); // (also: `scratch` may be overwritten from here on)
+    return true;
+}
+
+// The item of this workgroup in round `round`: -1 when the rounds are over, -2 when this round has none.
+__device__ __forceinline__ int expert_item(int round, int n_items) {
+    const int g = gridDim.x, base = round * g;
+    if (base >= n_items) return -1;
+    const int item = base + ((round & 1) ? g - 1 - (int)blockIdx.x : (int)blockIdx.x);
+    return item < n_items ? item : -2;
+}
+
 // Expert form: a workgroup belongs to one expert (blockIdx.y) and one of the two weight stacks
 // (blockIdx.z); up to TC of the expert's 16-row activation tiles, over all of k, sit in LDS, and
 // every wave walks row-tiles of the expert's matrix on its own: load a panel, multiply it with
@@ -1064,6 +1121,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_stream_kernel(MfmaPa
 // Eight waves: two per SIMD, 256 registers each; the compiler requests the next panel while the
 // current one is multiplied, which the 170 registers of twelve waves do not hold.
 constexpr int kExpertWaves = 8;
+constexpr int kExpertMaxWindowBytes = 160 * 1024 - kRankedExperts * 4 - 1024; // beside the rank table
 template <int QT, int TC>
 __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(MfmaParams P) {
     constexpr int UB = Unit<QT>::kBytes;
@@ -1073,22 +1131,35 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
     const int waves = P.nwr;
     const int j = lane & 15, grp = lane >> 4;
     const int s_units = P.slots >> 4;
-    const int e = blockIdx.y;
+    __shared__ int order[kRankedExperts];
+    const bool ranked = rank_experts(P.tile_offsets, P.n_experts, order, reinterpret_cast<int*>(smem));
+    const int per_expert = P.parts * P.stacks;
+    bool window_used = false;
+    for (int round = 0; round < kExpertRounds; round++) {
+    const int item = expert_item(round, P.n_experts * per_expert);
+    if (item == -1) break;
+    if (item == -2) continue;
+    const int pos = item / per_expert, stack = (item - pos * per_expert) / P.parts, part = item - pos * per_expert - stack * P.parts;
+    const int e = __builtin_amdgcn_readfirstlane(ranked ? order[pos] : pos); // (uniform: scalar registers)
     const int tile_begin = P.tile_offsets[e];
     const int n_tiles = P.tile_offsets[e + 1] - tile_begin;
-    if (n_tiles == 0) return; // uniform for the workgroup: nobody reaches a barrier
+    if (n_tiles == 0) { // uniform for the workgroup: nobody waits at a barrier
+        if (ranked) break; // (every later item's expert has no tile either)
+        continue;
+    }
     const int pos_begin = P.offsets[e], pos_end = P.offsets[e + 1];
-    const uint8_t* wbase = (blockIdx.z ? P.w2 : P.w) + (int64_t)e * P.matrix_bytes;
-    float* yout = blockIdx.z ? P.y2 : P.y;
+    const uint8_t* wbase = (stack ? P.w2 : P.w) + (int64_t)e * P.matrix_bytes;
+    float* yout = stack ? P.y2 : P.y;
     const uint8_t* records = P.ws + (size_t)tile_begin * P.k_units * UB;
 
     for (int t0 = 0; t0 < n_tiles; t0 += TC) {
         const int nt = min(TC, n_tiles - t0);
-        if (t0 != 0) lds_barrier(); // every wave is done with the previous tiles
+        if (window_used) lds_barrier(); // every wave is done with the previous tiles
+        window_used = true;
         issue_window_copy<QT>(records + (size_t)t0 * P.k_units * UB, smem, nt * P.k_units, wave, waves, lane);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         lds_barrier();
-        for (int rt = blockIdx.x * waves + wave; rt < P.row_tiles; rt += gridDim.x * waves) {
+        for (int rt = part * waves + wave; rt < P.row_tiles; rt += P.parts * waves) {
             float acc[TC][4];
 #pragma unroll
             for (int t = 0; t < TC; t++)
@@ -1119,6 +1190,7 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
             }
         }
     }
+    } // rounds
 }
 
 // The expert form for Q4_K matrices whose panels all hold NU units: the panel's activation-
@@ -1131,24 +1203,42 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
     constexpr int QT = QMM_Q4_K;
     constexpr int UB = Unit<QT>::kBytes;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    const int lane = threadIdx.x & 63;
+    const int lane_id = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int waves = P.nwr;
+    __shared__ int order[kRankedExperts];
+    const bool ranked = rank_experts(P.tile_offsets, P.n_experts, order, reinterpret_cast<int*>(smem));
+    const int per_expert = P.parts * P.stacks;
+    bool window_used = false;
+#pragma unroll
+    for (int round = 0; round < kExpertRounds; round++) {
+    // (the lane's offsets are derived anew for every item: hoisted out of this loop they would stay in
+    // registers beside a panel walk that needs all 256)
+    int lane = lane_id;
+    asm volatile("" : "+v"(lane));
     const int j = lane & 15, grp = lane >> 4;
-    const int e = blockIdx.y;
+    const int lane16 = lane * 16;
+    const int item = expert_item(round, P.n_experts * per_expert);
+    if (item == -1) break;
+    if (item == -2) continue;
+    const int pos = item / per_expert, stack = (item - pos * per_expert) / P.parts, part = item - pos * per_expert - stack * P.parts;
+    const int e = __builtin_amdgcn_readfirstlane(ranked ? order[pos] : pos); // (uniform: scalar registers)
     const int tile_begin = P.tile_offsets[e];
     const int n_tiles = P.tile_offsets[e + 1] - tile_begin;
-    if (n_tiles == 0) return; // uniform for the workgroup: nobody reaches a barrier
+    if (n_tiles == 0) { // uniform for the workgroup: nobody waits at a barrier
+        if (ranked) break; // (every later item's expert has no tile either)
+        continue;
+    }
     const int pos_begin = P.offsets[e], pos_end = P.offsets[e + 1];
-    const uint8_t* wbase = (blockIdx.z ? P.w2 : P.w) + (int64_t)e * P.matrix_bytes;
-    float* yout = blockIdx.z ? P.y2 : P.y;
+    const uint8_t* wbase = (stack ? P.w2 : P.w) + (int64_t)e * P.matrix_bytes;
+    float* yout = stack ? P.y2 : P.y;
     const uint8_t* records = P.ws + (size_t)tile_begin * P.k_units * UB;
-    const int rt_first = blockIdx.x * waves + wave, rt_step = gridDim.x * waves;
-    const int lane16 = lane * 16;
+    const int rt_first = part * waves + wave, rt_step = P.parts * waves;
 
     for (int t0 = 0; t0 < n_tiles; t0 += TC) {
         const int nt = min(TC, n_tiles - t0);
-        if (t0 != 0) lds_barrier(); // every wave is done with the previous tiles
+        if (window_used) lds_barrier(); // every wave is done with the previous tiles
+        window_used = true;
         issue_window_copy<QT>(records + (size_t)t0 * P.k_units * UB, smem, nt * P.k_units, wave, waves, lane);
         WPanel<QT> p;
         if (rt_first < P.row_tiles) // (uniform) the wave's first panel, needed whole before its first tile
@@ -1175,6 +1265,17 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
 #pragma unroll
                 for (int t = 0; t < TC; t++) {
                     if (t >= nt) continue; // uniform
+                    if (QMM_MFMA_ABL & 128) { // timing only: the panel stream without the tiles' arithmetic
+                        if (t == 0) {
+                            long x = 0;
+#pragma unroll
+                            for (int u = 0; u < NU; u++)
+#pragma unroll
+                                for (int b = 0; b < 4; b++) x ^= prep.lo[u][b] ^ prep.hi[u][b];
+                            acc[0][0] += __int_as_float((int)x ^ (int)(x >> 32)) + prep.d[0] + prep.dmin[NU - 1];
+                        }
+                        continue;
+                    }
                     const uint8_t* xu0 = smem + ((size_t)t * P.k_units + unit0) * UB;
                     q4k_tile_dot<NU>(
                         prep, [&](int u, int b) { return *reinterpret_cast<const i64x2*>(xu0 + u * UB + lane16 + b * 1024); },
@@ -1199,13 +1300,14 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
             }
         }
     }
+    } // rounds
 }
 
 template <int TC, int NU>
 hipError_t launch_expert_q4k(const MfmaParams& P, dim3 grid, int waves, size_t lds, hipStream_t stream) {
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_expert_q4k_kernel<TC, NU>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kExpertMaxWindowBytes);
         if (e != hipSuccess) return e;
     }
     gemv_mfma_expert_q4k_kernel<TC, NU><<<grid, 64 * waves, lds, stream>>>(P);
@@ -1216,7 +1318,7 @@ template <int QT, int TC>
 hipError_t launch_expert_form(const MfmaParams& P, dim3 grid, int waves, size_t lds, hipStream_t stream) {
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_mfma_expert_kernel<QT, TC>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kExpertMaxWindowBytes);
         if (e != hipSuccess) return e;
     }
     gemv_mfma_expert_kernel<QT, TC><<<grid, 64 * waves, lds, stream>>>(P);
@@ -1498,19 +1600,26 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
             const int stacks = tiled2 ? 2 : 1;
             int waves = kExpertWaves;
             if (waves > L.row_tiles) waves = (int)L.row_tiles;
-            // Workgroups per CU: one while the experts hold about one or two tiles (all of an expert's rows
-            // in one workgroup: its tiles are copied once), two from there on (the tile counts differ more
-            // from expert to expert and a second workgroup evens the CUs out).  Measured per layer at 128
-            // experts, top-8, one / two per CU: 109 / 115 us at 64 tokens, 113 / 119 at 128, 150 / 154
-            // at 256, 190 / 189 at 384, 223 / 216 at 512.  IZWI_QMM_MOE_EXPERT_WGS_PER_CU forces it.
+            // Items per CU: one while the experts hold about one or two tiles (all of an expert's rows in
+            // one item: its tiles are copied once), two from there on (the tile counts differ more from
+            // expert to expert and a heavy and a light item on each CU even the CUs out).  Measured per
+            // layer at 128 experts, top-8, one / two per CU (as one workgroup per item): 109 / 115 us at
+            // 64 tokens, 113 / 119 at 128, 150 / 154 at 256, 190 / 189 at 384, 223 / 216 at 512.
+            // IZWI_QMM_MOE_EXPERT_WGS_PER_CU forces it.  The stacks' row tiles are shared out to `parts`
+            // items so that the items are at most that many per CU; a workgroup takes up to
+            // kExpertRounds items, so the launch is (items / kExpertRounds) workgroups, all resident at
+            // once unless experts x stacks alone exceed two per CU.
             static const int forced_wgs_per_cu = [] { const char* e = getenv("IZWI_QMM_MOE_EXPERT_WGS_PER_CU"); int v = e ? atoi(e) : 0; return v > 0 ? v : 0; }();
-            const int wgs_per_cu = forced_wgs_per_cu ? forced_wgs_per_cu : (pairs <= (int64_t)20 * n_experts ? 1 : 2);
-            int parts = (wgs_per_cu * n_cus + n_experts * stacks - 1) / (n_experts * stacks);
+            int per_cu = forced_wgs_per_cu ? forced_wgs_per_cu : (pairs <= (int64_t)20 * n_experts ? 1 : 2);
+            if (per_cu > kExpertRounds) per_cu = kExpertRounds;
+            int parts = (int)((int64_t)per_cu * n_cus / ((int64_t)n_experts * stacks));
             const int max_parts = (int)((L.row_tiles + waves - 1) / waves);
             if (parts > max_parts) parts = max_parts;
             if (parts < 1) parts = 1;
             E.nwr = waves; // the workgroup's waves (every wave walks all of k)
-            const dim3 grid((unsigned)parts, (unsigned)n_experts, (unsigned)stacks);
+            E.n_experts = n_experts, E.stacks = stacks, E.parts = parts;
+            const int64_t n_items = (int64_t)parts * stacks * n_experts;
+            const dim3 grid((unsigned)(per_cu == 1 ? n_items : (n_items + kExpertRounds - 1) / kExpertRounds));
             const size_t lds = (size_t)tc * tile_bytes;
             if (L.dtype == QMM_Q4_K && uniform_panel_units(L) == 4)
                 return tc == 4 ? launch_expert_q4k<4, 4>(E, grid, waves, lds, stream) : launch_expert_q4k<2, 4>(E, grid, waves, lds, stream);
