@@ -45,6 +45,19 @@
 #define QMM_MFMA_ABL 0
 #endif
 
+// Measurement build only (-DQMM_EXPERT_TRACE, never defined in the library's build): the Q4_K expert
+// kernel records, per work item and wave, the 100 MHz clock at the item's start, when its tiles had
+// landed and at its end, with the CU it ran on; izwi_qmm_expert_trace_read copies the records out
+// (izwi_amd/csrc/expert_trace.py prints a summary).  Record (w, i) of 8 words sits at ((launch kind *
+// 512 + round * 256 + workgroup) * 8 + wave) * 8; launch kind 0: four-unit panels, 1: three-unit panels.
+#ifdef QMM_EXPERT_TRACE
+__device__ unsigned long long g_expert_trace[8 * 8192];
+extern "C" int izwi_qmm_expert_trace_read(void* dst, size_t bytes) {
+    if (bytes > sizeof(unsigned long long) * 8 * 8192) return -1;
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_expert_trace), bytes, 0, hipMemcpyDeviceToHost);
+}
+#endif
+
 namespace {
 
 constexpr int kMaxWaves = 12;
@@ -1218,6 +1231,10 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
     asm volatile("" : "+v"(lane));
     const int j = lane & 15, grp = lane >> 4;
     const int lane16 = lane * 16;
+#ifdef QMM_EXPERT_TRACE
+    const unsigned long long t_start = wall_clock64();
+    unsigned long long t_window = 0;
+#endif
     const int item = expert_item(round, P.n_experts * per_expert);
     if (item == -1) break;
     if (item == -2) continue;
@@ -1245,6 +1262,9 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
             load_wpanel<QT>(p, wbase + (int64_t)rt_first * P.k_groups * P.panel_bytes, P.slots, lane, j);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         lds_barrier();
+#ifdef QMM_EXPERT_TRACE
+        if (t0 == 0) t_window = wall_clock64();
+#endif
         for (int rt = rt_first; rt < P.row_tiles; rt += rt_step) {
             float acc[TC][4];
 #pragma unroll
@@ -1300,6 +1320,14 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
             }
         }
     }
+#ifdef QMM_EXPERT_TRACE
+    if (lane == 0 && blockIdx.x < 256) {
+        const unsigned hw = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (31 << 11));   // HW_ID: CU, SE
+        const unsigned xcc = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (31 << 11)); // XCC_ID
+        unsigned long long* o = g_expert_trace + ((size_t)((NU == 3 ? 512 : 0) + round * 256 + blockIdx.x) * 8 + wave) * 8;
+        o[0] = t_start, o[1] = t_window, o[2] = wall_clock64(), o[3] = hw, o[4] = xcc, o[5] = (unsigned)n_tiles, o[6] = (unsigned)e, o[7] = NU;
+    }
+#endif
     } // rounds
 }
 
