@@ -688,6 +688,19 @@ __device__ __forceinline__ void issue_window_copy(const uint8_t* __restrict__ sr
     }
 }
 
+// Several 16-row tiles of activations on the single-stage forms: one workgroup per (row-tile group,
+// tile), each exactly the workgroup of a call of up to 16 rows.  The launch is one-dimensional and
+// index = ((group / 8) * n_tiles + tile) * 8 + group % 8: workgroups go to the eight XCDs round-robin
+// by their index, so the n_tiles workgroups that read the same weight panels sit on one XCD, eight
+// positions apart in the order of placement, and all but the first find the panels in that XCD's L2.
+// Returns false for the padding past the last group (uniform).
+__device__ __forceinline__ bool tile_parallel_decode(int n_tiles, int rt_groups, int& rtg, int& tile) {
+    const int slot = blockIdx.x >> 3, hi = slot / n_tiles;
+    tile = slot - hi * n_tiles;
+    rtg = hi * 8 + (int)(blockIdx.x & 7);
+    return rtg < rt_groups;
+}
+
 // One-shot form: wave (wr, wk) owns panel wk of row-tile blockIdx.x * nwr + wr.
 // SINGLE: one tile of rows and one activation window, i.e. straight-line code.
 // GROUPED: the workgroup belongs to an expert; its weights are that matrix of the
@@ -715,7 +728,9 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
     const int s_units = P.slots >> 4;
     const uint8_t* wbase = P.w;
     float* yout = P.y;
-    int n_rows = P.n, row_tiles = P.row_tiles, rtg = blockIdx.x;
+    int n_rows = P.n, row_tiles = P.row_tiles, rtg = blockIdx.x, tile0 = 0;
+    if (SINGLE && P.n_tiles > 1 && !tile_parallel_decode(P.n_tiles, P.rt_groups, rtg, tile0)) return;
+    const int group_index = rtg; // (over all weights of a group)
     // GROUPED: workgroups go to the eight XCDs round-robin by their linear index, and every XCD has
     // its own L2: index = 8 * slot + (expert % 8), so the 2 * rt_groups workgroups of an expert share
     // one L2 and all but the first find the expert's activation records there (measured neutral at
@@ -733,7 +748,7 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
     const int unit0 = wk * s_units;                       // first unit of this wave's panel
     const int n_units = min(s_units, P.k_units - unit0);  // its units that exist (>= 1)
 
-    const uint8_t* records = P.ws;
+    const uint8_t* records = P.ws + (size_t)tile0 * P.k_units * UB;
     int n_tiles = P.n_tiles, pos_begin = 0, pos_end = 0;
     if (GROUPED) {
         const int e = g_expert;
@@ -755,7 +770,7 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
     // below - the start of all arithmetic - waits for nearly the whole workgroup's weights.
     asm volatile("s_barrier" ::: "memory");
     // (a group's tables are read here, behind the window copies: those need nothing from them)
-    if (!GROUPED && P.n_weights > 1) pick_group_entry(P0, P.n_weights, blockIdx.x, rtg, wbase, yout, n_rows, row_tiles);
+    if (!GROUPED && P.n_weights > 1) pick_group_entry(P0, P.n_weights, group_index, rtg, wbase, yout, n_rows, row_tiles);
     const int rt = rtg * P.nwr + wr;
     const bool rt_ok = rt < row_tiles;
     const int row = rt * 16 + j;
@@ -790,7 +805,7 @@ __device__ __forceinline__ void oneshot_body(const MfmaParams& P, const MfmaPara
     const int n_stages = SINGLE ? 1 : n_tiles * n_win;
     const size_t buf_bytes = (size_t)P.window_units * UB;
     bool transposed = false;
-    int tile = 0, win = 0;
+    int tile = tile0, win = 0;
     for (int s = 0; s < n_stages; s++) {
         const int wu0 = win * P.window_units;
         const int wn = min(P.window_units, P.k_units - wu0);
@@ -952,8 +967,11 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(
     const int s_units = P.slots >> 4;
     const uint8_t* wbase = P.w;
     float* yout = P.y;
-    int n_rows = P.n, row_tiles = P.row_tiles, rtg = blockIdx.x;
-    if (P.n_weights > 1) pick_group_entry(P0, P.n_weights, blockIdx.x, rtg, wbase, yout, n_rows, row_tiles);
+    int n_rows = P.n, row_tiles = P.row_tiles, rtg = blockIdx.x, tile0 = 0;
+    if (P.n_tiles > 1 && !tile_parallel_decode(P.n_tiles, P.rt_groups, rtg, tile0)) return;
+    if (P.n_weights > 1) pick_group_entry(P0, P.n_weights, rtg, rtg, wbase, yout, n_rows, row_tiles);
+    const uint8_t* records = P.ws + (size_t)tile0 * P.k_units * UB;
+    const int m_base = tile0 * 16; // the tile's first activation row
     const int rt = rtg * P.nwr + wr;
     const bool rt_ok = rt < row_tiles;
     const int unit0 = wk * s_units;
@@ -966,7 +984,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(
     float4 dx[4];
 #pragma unroll
     for (int u = 0; u < 4; u++) {
-        const uint8_t* rec = P.ws + (size_t)(unit0 + (u < n_units ? u : 0)) * UB; // missing units re-read unit 0
+        const uint8_t* rec = records + (size_t)(unit0 + (u < n_units ? u : 0)) * UB; // missing units re-read unit 0
 #pragma unroll
         for (int b = 0; b < 4; b++) a[u][b] = *reinterpret_cast<const i64x2*>(rec + b * 1024 + lane * 16);
         const uint8_t* side = rec + Unit<QT>::kQuant;
@@ -987,9 +1005,9 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(
         if (rt_ok && row < n_rows) {
 #pragma unroll
             for (int r = 0; r < 4; r++)
-                if (grp * 4 + r < P.m) {
-                    if (EP) qmm_store(yout, P.ep, (int64_t)(grp * 4 + r) * n_rows + row, acc[r]);
-                    else yout[(int64_t)(grp * 4 + r) * n_rows + row] = acc[r];
+                if (m_base + grp * 4 + r < P.m) {
+                    if (EP) qmm_store(yout, P.ep, (int64_t)(m_base + grp * 4 + r) * n_rows + row, acc[r]);
+                    else yout[(int64_t)(m_base + grp * 4 + r) * n_rows + row] = acc[r];
                 }
         }
         return;
@@ -1006,10 +1024,10 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(
         const float* part = lds_red + ((wr2 * P.nwk) * 4 + (mrow & 3)) * 64 + (mrow >> 2) * 16 + j2;
         float sum = 0.0f;
         for (int w2 = 0; w2 < P.nwk; w2++) sum += part[w2 * 256];
-        const int rt2 = rtg * P.nwr + wr2, col = rt2 * 16 + j2;
-        if (rt2 < row_tiles && col < n_rows && mrow < P.m) {
-            if (EP) qmm_store(yout, P.ep, (int64_t)mrow * n_rows + col, sum);
-            else yout[(int64_t)mrow * n_rows + col] = sum;
+        const int rt2 = rtg * P.nwr + wr2, col = rt2 * 16 + j2, mm = m_base + mrow;
+        if (rt2 < row_tiles && col < n_rows && mm < P.m) {
+            if (EP) qmm_store(yout, P.ep, (int64_t)mm * n_rows + col, sum);
+            else yout[(int64_t)mm * n_rows + col] = sum;
         }
     }
 }
@@ -1019,6 +1037,18 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(
 // per call; with k = 4096 the single-window LDS form is the faster one, 10.2 against 10.4 us
 // and 11.9 against 12.7 us for the q|k|v group).  IZWI_QMM_MFMA_DIRECT=0 keeps the LDS forms
 // (tuning aid).
+// Two to four tiles of rows: one single-stage workgroup per tile (tile_parallel_decode) instead of one
+// workgroup that walks the tiles stage by stage.  IZWI_QMM_MFMA_TILE_PARALLEL=0 / 1 forces the choice
+// (tuning aid).
+bool tile_parallel_applies(int n_tiles) {
+    static const int mode = [] {
+        const char* e = getenv("IZWI_QMM_MFMA_TILE_PARALLEL");
+        return e && (e[0] == '0' || e[0] == '1') ? e[0] - '0' : -1;
+    }();
+    if (n_tiles < 2 || n_tiles > 4) return false;
+    return mode != 0;
+}
+
 bool direct_form_applies(int dtype, int n_tiles, int nwr, bool one_window) {
     static const int mode = [] {
         const char* e = getenv("IZWI_QMM_MFMA_DIRECT");
@@ -1478,18 +1508,27 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
     // matrices (many row-tiles per CU) amortize the activation window better when it
     // stays resident while a wave walks whole row-tiles.
     const bool oneshot = L.k_groups <= kMaxWaves && L.row_tiles < 8 * (int64_t)n_cus;
+    // (tiles a workgroup walks: one when every tile has workgroups of its own)
+    int oneshot_nwr = 1; // row tiles per workgroup of the one-shot forms
+    if (oneshot) {
+        const int nwr_max = kMaxWaves / (int)L.k_groups;
+        const int64_t want = (L.row_tiles + n_cus - 1) / n_cus; // as few workgroups as CUs where the waves allow it
+        oneshot_nwr = (int)(want < 1 ? 1 : (want > nwr_max ? nwr_max : want));
+    }
+    const bool tile_parallel = oneshot && tile_parallel_applies(n_tiles) &&
+                               (L.k_units <= P.window_units || direct_form_applies(L.dtype, 1, oneshot_nwr, false));
+    const int stage_tiles = tile_parallel ? 1 : n_tiles;
     size_t lds;
     unsigned grid;
     int waves;
     if (oneshot) {
         P.nwk = (int)L.k_groups;
-        int nwr_max = kMaxWaves / P.nwk;
-        int64_t want = (L.row_tiles + n_cus - 1) / n_cus; // as few workgroups as CUs where the waves allow it
-        P.nwr = (int)(want < 1 ? 1 : (want > nwr_max ? nwr_max : want));
+        P.nwr = oneshot_nwr;
         waves = P.nwk * P.nwr;
         P.rt_groups = (int)((L.row_tiles + P.nwr - 1) / P.nwr);
         grid = (unsigned)P.rt_groups;
-        const bool single_stage = n_tiles == 1 && L.k_units <= P.window_units;
+        if (tile_parallel) grid = (unsigned)(((P.rt_groups + 7) / 8) * 8 * n_tiles);
+        const bool single_stage = stage_tiles == 1 && L.k_units <= P.window_units;
         P.double_buf = !single_stage && 2 * window_bytes + (size_t)waves * 256 * 4 <= 160 * 1024;
         lds = single_stage ? std::max(window_bytes, (size_t)waves * 256 * 4)
                            : (P.double_buf ? 2 : 1) * window_bytes + (size_t)waves * 256 * 4;
@@ -1502,7 +1541,7 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
         lds = window_bytes;
     }
     P.wave_magic = (65536 + P.nwk - 1) / P.nwk;
-    if (oneshot && direct_form_applies(L.dtype, n_tiles, P.nwr, L.k_units <= P.window_units)) {
+    if (oneshot && direct_form_applies(L.dtype, stage_tiles, P.nwr, L.k_units <= P.window_units)) {
         const size_t red = (size_t)waves * 256 * 4;
         if (full_panels(L)) {
             if (epilogue) launch_mfma(gemv_mfma_direct_q4k_kernel<true, 4>, grid, 64 * waves, red, stream, P);
@@ -1514,9 +1553,10 @@ hipError_t qmm_launch_gemv_mfma(const QmmLayout& L, const void* tiled, const flo
         return hipGetLastError();
     }
     if (lds > 160 * 1024) return hipErrorInvalidValue;
-    const bool single = n_tiles == 1 && L.k_units <= P.window_units;
+    const bool single = stage_tiles == 1 && L.k_units <= P.window_units;
     const int form = oneshot ? (single ? 0 : 1) : 2;
-    if (L.dtype == QMM_Q4_K && form == 0 && full_panels(L) && straight_line_fits(P.rt_groups, waves, n_cus)) {
+    if (form == 1 && tile_parallel) return hipErrorInvalidValue; // (not reached: tile_parallel implies a single-stage form)
+    if (L.dtype == QMM_Q4_K && form == 0 && full_panels(L) && straight_line_fits((int64_t)P.rt_groups * (tile_parallel ? n_tiles : 1), waves, n_cus)) {
         const void* fn = epilogue ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, true, 4>)
                                   : reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4>);
         if (lds > 48 * 1024) {
@@ -1768,7 +1808,10 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
     }
     P.rt_groups = (int)groups;
     const int waves = P.nwk * P.nwr;
-    if (n_tiles > 1) {
+    // (every tile of rows with workgroups of its own: the single-stage forms below, a longer launch)
+    const bool tile_parallel = tile_parallel_applies(n_tiles);
+    const unsigned grid = tile_parallel ? (unsigned)(((groups + 7) / 8) * 8 * n_tiles) : (unsigned)groups;
+    if (n_tiles > 1 && !tile_parallel) {
         // several tiles of rows against a resident panel (the form of the single-weight call at these m)
         const size_t window_bytes = (size_t)P.window_units * unit_bytes(L0.dtype), red_bytes = (size_t)waves * 256 * 4;
         P.double_buf = 2 * window_bytes + red_bytes <= 160 * 1024;
@@ -1790,13 +1833,13 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
         return hipGetLastError();
     }
     if (direct_form_applies(L0.dtype, 1, P.nwr, true)) {
-        if (full_panels(L0)) launch_mfma(gemv_mfma_direct_q4k_kernel<false, 4>, (unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream, P);
-        else launch_mfma(gemv_mfma_direct_q4k_kernel<false>, (unsigned)groups, 64 * waves, (size_t)waves * 256 * 4, stream, P);
+        if (full_panels(L0)) launch_mfma(gemv_mfma_direct_q4k_kernel<false, 4>, grid, 64 * waves, (size_t)waves * 256 * 4, stream, P);
+        else launch_mfma(gemv_mfma_direct_q4k_kernel<false>, grid, 64 * waves, (size_t)waves * 256 * 4, stream, P);
         return hipGetLastError();
     }
     const size_t lds = std::max((size_t)P.window_units * unit_bytes(L0.dtype), (size_t)waves * 256 * 4);
     if (lds > 160 * 1024) return hipErrorNotSupported;
-    const bool full = L0.dtype == QMM_Q4_K && full_panels(L0) && straight_line_fits(groups, waves, n_cus);
+    const bool full = L0.dtype == QMM_Q4_K && full_panels(L0) && straight_line_fits(groups * (tile_parallel ? n_tiles : 1), waves, n_cus);
     const void* fn = full                   ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4>)
                      : L0.dtype == QMM_Q4_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q4_K, true>)
                      : L0.dtype == QMM_Q6_K ? reinterpret_cast<const void*>(&gemv_mfma_oneshot_kernel<QMM_Q6_K, true>)
@@ -1806,12 +1849,12 @@ hipError_t qmm_launch_gemv_mfma_multi(const QmmLayout* const* layouts, const voi
         if (e != hipSuccess) return e;
     }
     if (full)
-        launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4>, (unsigned)groups, 64 * waves, lds, stream, P);
+        launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q4_K, true, false, false, 4>, grid, 64 * waves, lds, stream, P);
     else if (L0.dtype == QMM_Q4_K)
-        launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q4_K, true>, (unsigned)groups, 64 * waves, lds, stream, P);
+        launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q4_K, true>, grid, 64 * waves, lds, stream, P);
     else if (L0.dtype == QMM_Q6_K)
-        launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q6_K, true>, (unsigned)groups, 64 * waves, lds, stream, P);
+        launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q6_K, true>, grid, 64 * waves, lds, stream, P);
     else
-        launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q8_0, true>, (unsigned)groups, 64 * waves, lds, stream, P);
+        launch_mfma(gemv_mfma_oneshot_kernel<QMM_Q8_0, true>, grid, 64 * waves, lds, stream, P);
     return hipGetLastError();
 }

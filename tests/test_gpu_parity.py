@@ -181,6 +181,30 @@ def test_config3_8b_shapes(qa, oracle, dtype, m):
         assert rel_err(y, oracle.qmatmul(dtype, x, blocks, n)) < DECODE_TOL, name
 
 
+@pytest.mark.parametrize("dtype,n,k,m", [
+    (Q4_K, 1000, 12288, 40),   # k past one LDS window: the register-direct form, three tiles, ragged rows
+    (Q4_K, 4096, 4096, 64),    # four tiles, four-unit panels
+    (Q4_K, 72, 1280, 33),      # ragged k (five units), a handful of row tiles, the last tile one row
+    (Q8_0, 1024, 3072, 64),    # the down projection of config 2
+    (Q8_0, 3000, 1056, 50),    # ragged k and rows
+])
+def test_several_tiles_of_rows_one_workgroup_each(qa, oracle, dtype, n, k, m):
+    """17 .. 64 activation rows: every 16-row tile gets workgroups of its own on the single-stage kernels
+    (the launch's index decodes to row-tile group and tile); each tile's rows land in their own rows of
+    y and rows past m are not written."""
+    _say(f"several tiles dtype={dtype} n={n} k={k} m={m}")
+    blocks = make_weight(oracle, dtype, n, k, 60 + m)
+    x = oracle.randn(61 + m, (m, k))
+    dt = qa.GgmlDType(dtype)
+    mm = qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, blocks, (n, k)))
+    rows = ((m + 15) // 16) * 16
+    y = torch.full((rows + 1, n), 7.0, dtype=torch.float32, device="cuda")
+    mm.forward_fused(torch.from_numpy(x).cuda(), out=y[:m])
+    torch.cuda.synchronize()
+    assert rel_err(y[:m].cpu().numpy(), oracle.qmatmul(dtype, x, blocks, n)) < DECODE_TOL
+    assert bool((y[m:] == 7.0).all())
+
+
 def test_config3_lm_head_full_size(qa, oracle):
     n, k = 151936, 4096
     blocks = make_weight(oracle, Q4_K, n, k, 50)
