@@ -464,8 +464,8 @@ __device__ __forceinline__ void q4k_panel_dot(WPanel<QMM_Q4_K>& p, int n_units, 
 }
 
 
-// A Q4_K panel prepared for several tiles of activations (the multi-stage forms: a batch of more
-// than 16 rows, an expert's tiles): what does not depend on the activations is done once per panel
+// A Q4_K panel prepared for several tiles of activations (the multi-stage forms: an expert's tiles, a
+// batch of more than 16 rows walked inside one workgroup): what does not depend on the activations is done once per panel
 // instead of once per (panel, tile) - the nibbles split into the two matrix-core operands of every
 // (unit, sub-block pair), the 6-bit scales and mins unpacked, d and dmin converted.  Twice the
 // registers of the packed quants, so the units are walked one after the other (four running sums
