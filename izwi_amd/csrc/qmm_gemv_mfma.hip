@@ -1032,11 +1032,6 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gemv_mfma_direct_q4k_kernel(
     }
 }
 
-// One row tile of activations (m <= 16), one row-tile of weights per workgroup, Q4_K, and k
-// longer than one LDS window (measured on the 8B shapes at m = 16: 4096 x 12288 17.0 -> 15.4 us
-// per call; with k = 4096 the single-window LDS form is the faster one, 10.2 against 10.4 us
-// and 11.9 against 12.7 us for the q|k|v group).  IZWI_QMM_MFMA_DIRECT=0 keeps the LDS forms
-// (tuning aid).
 // Two to four tiles of rows: one single-stage workgroup per tile (tile_parallel_decode) instead of one
 // workgroup that walks the tiles stage by stage.  IZWI_QMM_MFMA_TILE_PARALLEL=0 / 1 forces the choice
 // (tuning aid).
@@ -1049,6 +1044,11 @@ bool tile_parallel_applies(int n_tiles) {
     return mode != 0;
 }
 
+// One row tile of activations (m <= 16), one row-tile of weights per workgroup, Q4_K, and k
+// longer than one LDS window (measured on the 8B shapes at m = 16: 4096 x 12288 17.0 -> 15.4 us
+// per call; with k = 4096 the single-window LDS form is the faster one, 10.2 against 10.4 us
+// and 11.9 against 12.7 us for the q|k|v group).  IZWI_QMM_MFMA_DIRECT=0 keeps the LDS forms
+// (tuning aid).
 bool direct_form_applies(int dtype, int n_tiles, int nwr, bool one_window) {
     static const int mode = [] {
         const char* e = getenv("IZWI_QMM_MFMA_DIRECT");
@@ -1155,9 +1155,9 @@ __device__ __forceinline__ int expert_item(int round, int n_items) {
     return item < n_items ? item : -2;
 }
 
-// Expert form: a workgroup belongs to one expert (blockIdx.y) and one of the two weight stacks
-// (blockIdx.z); up to TC of the expert's 16-row activation tiles, over all of k, sit in LDS, and
-// every wave walks row-tiles of the expert's matrix on its own: load a panel, multiply it with
+// Expert form: a work item belongs to one expert and one of the two weight stacks; up to TC of the
+// expert's 16-row activation tiles, over all of k, sit in LDS, and every wave walks row-tiles of the
+// expert's matrix on its own: load a panel, multiply it with
 // every tile, next panel; no wave waits for another after the tiles have landed.  The weights are
 // read once per TC tiles (an expert with more tiles takes another pass), and the waves of a CU
 // keep several panels in flight where the one-shot form is one chain of round trips per workgroup.
