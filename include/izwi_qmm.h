@@ -250,7 +250,8 @@ int izwi_qmm_forward_rows_f32(const izwi_qmm_weight* w, const uint32_t* row_ids,
 
 /* --- activation records: quantized activations handed over by their producer ---------- */
 
-/* For 3 <= m <= 64 rows izwi_qmm_forward_f32 is two launches: the activation quantizer (candle-core's
+/* For 3 <= m <= 64 rows (5 <= m <= 64 where k <= 3072: three and four rows of a short k stay on the
+ * single-launch kernel, four rows per pass) izwi_qmm_forward_f32 is two launches: the activation quantizer (candle-core's
  * `BlockQ8_0::from_float` / `BlockQ8K::from_float` per row, qwen3 call site core.rs:812) writes
  * "records" into scratch, the matrix-core kernel multiplies them.  The kernel that PRODUCES the
  * activations can write the records itself and save that launch on the token's critical path:
@@ -258,7 +259,9 @@ int izwi_qmm_forward_rows_f32(const izwi_qmm_weight* w, const uint32_t* row_ids,
  *   izwi_qmm_silu_mul_quantize_records_f32                    silu(gate) * up              -> down
  *   izwi_qmm_quantize_records_f32                             any other f32 activations    (the plain quantizer)
  * and izwi_qmm_forward_group_records_f32 is izwi_qmm_forward_group_f32 on such records: results
- * are bit-identical to the calls on the f32 activations.  Records are opaque device memory of
+ * are bit-identical to the calls on the f32 activations at the row counts named above (for fewer rows
+ * the call on f32 activations runs the single-launch kernel: the same integer block dots, the f32
+ * sums in another order).  Records are opaque device memory of
  * izwi_qmm_records_bytes(weight dtype, m, k) bytes, 16-byte aligned, valid for weights whose dot
  * type matches (Q8_0 weights: Q8_0 records; Q4_K and Q6_K weights: the same Q8_K records).
  * Device pointers only.  No counterpart in the reference, whose CPU matmul quantizes inside the op. */
@@ -329,7 +332,8 @@ int izwi_qmm_chain_set_spin_limit(izwi_qmm_chain* chain, uint32_t polls);
 /* izwi_qmm_forward_f32 for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
  * reference.  Same kernels and the same results, bit for bit, as izwi_qmm_forward_f32 with
- * IZWI_QMM_DEVICE pointers; the quantized activation records of the batched kernels (3 <= m <= 64)
+ * IZWI_QMM_DEVICE pointers; the quantized activation records of the batched kernels (from three rows on,
+ * from five where k <= 3072)
  * live in a static device array of IZWI_QMM_NOALLOC_SCRATCH_BYTES inside the library's image
  * (each GPU the library runs on holds its own copy until the process ends) instead of the
  * per-stream scratch buffer, and the call performs no hipMalloc / hipFree whatever its size.
@@ -347,7 +351,7 @@ int izwi_qmm_forward_f32_noalloc(const izwi_qmm_weight* w, const float* x, int64
  * activations, y_i = QMatMul_i.forward(x), bit-identical to n_weights calls of
  * izwi_qmm_forward_f32 up to 128 rows (beyond, in the bf16 matrix-core arithmetic, equal up to the
  * f32 summation order: the shared launch may split k differently).  The weights must share k; with equal block types the decode
- * sizes run as one kernel launch (m <= 2) or as one activation quantization and one
+ * sizes run as one kernel launch (m <= 2; m <= 4 where k <= 3072) or as one activation quantization and one
  * matmul launch (m <= 64), prefill sizes (m > 128, bf16 matrix-core arithmetic) share one conversion of x
  * and one launch; members of several block types (attn_q / attn_k in Q4_K beside attn_v in
  * Q6_K, as Q4_K_M files have them) are grouped by type, one such launch per type.
@@ -383,8 +387,8 @@ int izwi_qmm_forward_gate_up_silu_f32(const izwi_qmm_weight* gate, const izwi_qm
  * `gate` and `up` are [intermediate, hidden] weights of the same shape, `down` is
  * [hidden, intermediate]; any of the built block types.  The results are those of
  * izwi_qmm_forward_gate_up_silu_f32 followed by izwi_qmm_forward_f32, bit for bit.  What the call
- * adds is the route between the three projections: for 3 <= m <= 64 (gate and up of one block
- * type) x is quantized once, gate | up run as one launch on its records, silu(g) * u is quantized
+ * adds is the route between the three projections: for 3 <= m <= 64 (5 <= m where hidden or
+ * intermediate is at most 3072; gate and up of one block type) x is quantized once, gate | up run as one launch on its records, silu(g) * u is quantized
  * straight into the records that `down` multiplies (four launches; the separate calls take five
  * and write and read the intermediate as an f32 matrix); other sizes run the two calls with the
  * intermediate in the stream's scratch. */

@@ -487,15 +487,24 @@ hipError_t get_scratch(int device, hipStream_t stream, size_t bytes, void** out)
     return e;
 }
 
-// Smallest m that takes the batched (MFMA) decode kernel; below it the fused
-// single-launch kernel runs.  IZWI_QMM_MFMA_MIN_M overrides (tuning knob).
-int mfma_min_m() {
-    static int v = [] {
+// Smallest m that takes the batched (MFMA) decode kernel for a weight of this k; below it the fused
+// single-launch kernel runs.  Three, and five where k is short (up to 3072): a call of three or four
+// rows on the batched kernels is two launches whose chains - quantizer, window copy, panel, k-split -
+// take 9 us however small the matrix, the single-launch kernel with four rows per pass takes 6 (Q8_0 at
+// the 0.6B shapes, per call: 5.9 against 9.2 us for o, 6.3 against 9.4 for down), while at k = 4096 and
+// beyond it re-reads enough activations per workgroup to lose (8B shapes: o 8.2 against 8.3, down 15.0
+// against 12.6).  The rule looks at k only, which the members of a projection group share: a group and
+// its members' separate calls take the same kernel, so their results stay the same bits.
+// IZWI_QMM_MFMA_MIN_M overrides it for every k (tuning knob).
+constexpr int64_t kShortK = 3072;
+int mfma_min_m(int64_t k) {
+    static int forced = [] {
         const char* e = getenv("IZWI_QMM_MFMA_MIN_M");
         int n = e ? atoi(e) : 0;
-        return n > 0 ? n : 3;
+        return n > 0 ? n : 0;
     }();
-    return v;
+    if (forced) return forced;
+    return k <= kShortK ? 5 : 3;
 }
 
 // Arithmetic of f32 / fused calls with more than 64 activation rows: 0 = activations rounded to
@@ -883,7 +892,7 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
     Staged xi, yo;
     HIP_TRY(xi.in(x, (size_t)m * L.k * sizeof(float), mem_space, stream));
     HIP_TRY(yo.out(y, (size_t)m * L.n * sizeof(float), mem_space, stream));
-    if (m < mfma_min_m()) {
+    if (m < mfma_min_m(L.k)) {
         HIP_TRY(qmm_launch_gemv(L, w->tiled, (const float*)xi.dev, m, (float*)yo.dev, w->n_cus, stream));
     } else if (m <= 64 || large_m_mode() == IZWI_QMM_LARGE_M_INT8) {
         // more than 64 rows in the integer arithmetic: 64 at a time, the records of one chunk
@@ -894,7 +903,7 @@ int izwi_qmm_forward_f32(const izwi_qmm_weight* w, const float* x, int64_t m, fl
             const int64_t rows = m - r0 < 64 ? m - r0 : 64;
             const float* xr = (const float*)xi.dev + r0 * L.k;
             float* yr = (float*)yo.dev + r0 * L.n;
-            if (rows < mfma_min_m())
+            if (rows < mfma_min_m(L.k))
                 HIP_TRY(qmm_launch_gemv(L, w->tiled, xr, rows, yr, w->n_cus, stream));
             else
                 HIP_TRY(qmm_launch_gemv_mfma(L, w->tiled, xr, rows, yr, scratch, w->n_cus, stream));
@@ -1051,7 +1060,7 @@ int izwi_qmm_forward_f32_noalloc(const izwi_qmm_weight* w, const float* x, int64
     if (int rc = current_device(&device)) return rc;
     if (device != w->device) // (before any launch: the one- and two-row kernel too runs on the weight's pointers)
         return fail(IZWI_QMM_ERR_INVALID, "the weight lives on device %d, the current device is %d", w->device, device);
-    if (m < mfma_min_m()) { // one or two rows: the single-launch kernel has no scratch at all
+    if (m < mfma_min_m(L.k)) { // a few rows: the single-launch kernel has no scratch at all
         HIP_TRY(qmm_launch_gemv(L, w->tiled, x, m, y, w->n_cus, stream));
         return IZWI_QMM_OK;
     }
@@ -1155,7 +1164,7 @@ int forward_group_impl(const izwi_qmm_weight* const* weights, int32_t n_weights,
     auto call_by_type = [&](const float* xin, const float* nw) -> int {
         bool done[QMM_MAX_GROUP] = {};
         // batched sizes: Q4_K and Q6_K weights dot against the same Q8_K records, quantized once
-        bool q8k_records = !nw && m >= mfma_min_m();
+        bool q8k_records = !nw && m >= mfma_min_m(weights[0]->layout.k);
         for (int i = 0; i < n_weights; i++)
             if (weights[i]->layout.dtype != IZWI_QMM_Q4_K && weights[i]->layout.dtype != IZWI_QMM_Q6_K) q8k_records = false;
         void* records = nullptr;
@@ -1184,9 +1193,9 @@ int forward_group_impl(const izwi_qmm_weight* const* weights, int32_t n_weights,
         hipStream_t stream = (hipStream_t)stream_;
         const izwi_qmm_weight* w0 = weights[0];
         // each type's launch normalizes for itself: x is read by every workgroup anyway
-        if (by_type && m <= 2 && m < mfma_min_m()) return call_by_type(x, norm_weight);
+        if (by_type && m <= 2 && m < mfma_min_m(weights[0]->layout.k)) return call_by_type(x, norm_weight);
         // one launch: the decode kernel normalizes while it quantizes (device buffers, one block type, m <= 2)
-        if (mem_space == IZWI_QMM_DEVICE && uniform && m <= 2 && m < mfma_min_m()) {
+        if (mem_space == IZWI_QMM_DEVICE && uniform && m <= 2 && m < mfma_min_m(w0->layout.k)) {
             const QmmLayout* layouts[QMM_MAX_GROUP];
             const void* tiled[QMM_MAX_GROUP];
             for (int i = 0; i < n_weights; i++) layouts[i] = &weights[i]->layout, tiled[i] = weights[i]->tiled;
@@ -1245,13 +1254,13 @@ int forward_group_impl(const izwi_qmm_weight* const* weights, int32_t n_weights,
     }
     hipStream_t stream = (hipStream_t)stream_;
     const izwi_qmm_weight* w0 = weights[0];
-    if (m < mfma_min_m()) {
+    if (m < mfma_min_m(w0->layout.k)) {
         const QmmLayout* layouts[QMM_MAX_GROUP];
         const void* tiled[QMM_MAX_GROUP];
         for (int i = 0; i < n_weights; i++) layouts[i] = &weights[i]->layout, tiled[i] = weights[i]->tiled;
-        // one launch for up to two rows; more rows on this kernel (threshold raised through the
-        // environment) go projection by projection
-        if (m <= 2) {
+        // one launch for up to four rows (one pass of the kernel); more rows on this kernel (threshold
+        // raised through the environment) go projection by projection
+        if (m <= 4) {
             ProfileScope prof(w0, stream);
             hipError_t e = qmm_launch_gemv_multi(layouts, tiled, n_weights, x, m, ys, w0->n_cus, stream);
             if (e == hipSuccess) return IZWI_QMM_OK;
@@ -1344,7 +1353,7 @@ int izwi_qmm_mlp_forward_f32(const izwi_qmm_weight* gate, const izwi_qmm_weight*
     HIP_TRY(yo.out(y, (size_t)m * D.n * sizeof(float), mem_space, stream));
     auto align256 = [](size_t v) { return (v + 255) & ~(size_t)255; };
     const size_t part = align256((size_t)m * G.n * sizeof(float)); // one [m, intermediate] f32 matrix
-    const bool records = m >= mfma_min_m() && m <= 64 && G.dtype == U.dtype;
+    const bool records = m >= mfma_min_m(G.k) && m >= mfma_min_m(D.k) && m <= 64 && G.dtype == U.dtype;
     if (records) {
         // Rows for the matrix-core kernels: activation records all the way.  x is quantized once for
         // gate | up (one launch for both), silu(g) * u is quantized straight into the records that
@@ -1396,7 +1405,7 @@ int izwi_qmm_forward_normed_f32(const izwi_qmm_weight* w, const float* x, int64_
     if (m == 0 || L.n == 0) return IZWI_QMM_OK;
     if (!x || !y) return fail(IZWI_QMM_ERR_INVALID, "NULL buffer");
     hipStream_t stream = (hipStream_t)stream_;
-    if (mem_space == IZWI_QMM_DEVICE && m <= 2 && m < mfma_min_m()) {
+    if (mem_space == IZWI_QMM_DEVICE && m <= 2 && m < mfma_min_m(L.k)) {
         const QmmNorm norm{norm_weight, eps};
         ProfileScope prof(w, stream);
         hipError_t e = qmm_launch_gemv(L, w->tiled, x, m, y, w->n_cus, stream, nullptr, &norm);
@@ -1447,7 +1456,7 @@ int gate_up_silu_impl(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, co
     Staged wi;
     if (norm_weight) HIP_TRY(wi.in(norm_weight, (size_t)L.k * sizeof(float), mem_space, stream));
     const float* xin = (const float*)xi.dev;
-    if (m < mfma_min_m() && m <= 2) {
+    if (m < mfma_min_m(L.k) && m <= 2) {
         const QmmNorm norm{(const float*)wi.dev, norm_eps};
         ProfileScope prof(gate, stream);
         HIP_TRY(qmm_launch_gemv_gated(L, gate->tiled, up->tiled, xin, m, (float*)ho.dev, gate->n_cus, stream,
@@ -1597,7 +1606,7 @@ int izwi_qmm_forward_fused(const izwi_qmm_weight* w, const void* x, int x_dtype,
     if (residual) HIP_TRY(ri.in(residual, ybytes, mem_space, stream));
     HIP_TRY(yo.out(y, ybytes, mem_space, stream));
     QmmIo io{x_bf16 ? 1 : 0, residual ? ri.dev : nullptr, y_bf16 ? 1 : 0};
-    if (m < mfma_min_m()) {
+    if (m < mfma_min_m(L.k)) {
         const float* xf = (const float*)xi.dev;
         if (x_bf16 && m > 2) { // this kernel reads bf16 rows only in its one- and two-row forms
             void* wide = nullptr;
@@ -1621,7 +1630,7 @@ int izwi_qmm_forward_fused(const izwi_qmm_weight* w, const void* x, int x_dtype,
             QmmIo cio = io;
             if (io.residual) cio.residual = static_cast<const uint8_t*>(io.residual) + (size_t)r0 * L.n * ye;
             hipError_t e;
-            if (rows < mfma_min_m()) { // a tail of one or two rows: the single-launch kernel
+            if (rows < mfma_min_m(L.k)) { // a tail of a few rows: the single-launch kernel
                 e = qmm_launch_gemv(L, w->tiled, (const float*)xr, rows, (float*)yr, w->n_cus, stream, &cio);
             } else {
                 e = qmm_launch_gemv_mfma(L, w->tiled, (const float*)xr, rows, (float*)yr, scratch, w->n_cus, stream, true, &cio);

@@ -744,7 +744,8 @@ hipError_t qmm_launch_gemv_gated(const QmmLayout& L, const void* tiled_gate, con
 hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* const* tiled, int n_weights,
                                  const float* x, int64_t m, float* const* ys, int n_cus,
                                  hipStream_t stream, const QmmNorm* norm) {
-    if (n_weights < 1 || n_weights > QMM_MAX_GROUP || m < 1 || m > 2) return hipErrorInvalidValue;
+    if (n_weights < 1 || n_weights > QMM_MAX_GROUP || m < 1 || m > 4) return hipErrorInvalidValue;
+    if (norm && m > 2) return hipErrorNotSupported; // (the folded norm: one or two rows)
     const QmmLayout& L0 = *layouts[0];
     int64_t total_row_tiles = 0;
     for (int i = 0; i < n_weights; i++) {
@@ -776,14 +777,18 @@ hipError_t qmm_launch_gemv_multi(const QmmLayout* const* layouts, const void* co
     const int64_t groups = (tiles_all + P.nwr - 1) / P.nwr;
     if (groups > (int64_t)n_cus * 32) return hipErrorNotSupported;
     P.rt_groups = (int)groups;
-    const int mt = m == 2 ? 2 : 1;
+    const int mt = m > 2 ? 4 : (m == 2 ? 2 : 1); // rows per pass: one pass
     if (norm) P.norm_w = norm->weight, P.norm_eps = norm->eps;
     const dim3 g((unsigned)groups), b(64 * waves);
     return with_block_type(L0.dtype, [&](auto QT) {
         constexpr int qt = decltype(QT)::value;
-        size_t need = mt == 2 ? lds_bytes<qt, 2>(P.k_units, waves) : lds_bytes<qt, 1>(P.k_units, waves);
+        size_t need = mt == 4 ? lds_bytes<qt, 4>(P.k_units, waves) : mt == 2 ? lds_bytes<qt, 2>(P.k_units, waves) : lds_bytes<qt, 1>(P.k_units, waves);
         if (norm) need += (size_t)mt * P.k_units * sizeof(float);
         if (need > 48 * 1024) return hipErrorNotSupported;
+        if (mt == 4) {
+            launch_gemv(gemv_kernel<qt, 4, false, false, true>, g, b, need, stream, P);
+            return hipGetLastError();
+        }
         if (norm) {
             if (mt == 2) launch_gemv(gemv_kernel<qt, 2, false, false, true, 0, true>, g, b, need, stream, P);
             else launch_gemv(gemv_kernel<qt, 1, false, false, true, 0, true>, g, b, need, stream, P);

@@ -635,10 +635,11 @@ def test_moe_forward_small_shapes(qa, oracle, dtype, E, hidden, inter, t, top_k)
 
 
 @pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
-@pytest.mark.parametrize("m", [1, 2, 5, 16, 40, 80])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 16, 40, 80])
 def test_projection_group_equals_separate_calls(qa, oracle, dtype, m):
     """Qwen3QkvProjection / Qwen3GateUpProjection `Separate` arms as one call: bit-identical to
-    separate forwards (one launch for m <= 2, shared activation quantization up to 64)."""
+    separate forwards (one launch of the decode kernel for m <= 2 and, at this k, for m <= 4; shared
+    activation quantization up to 64)."""
     k = 1024
     dt = qa.GgmlDType(dtype)
     parts = [qa.QMatMul.from_qtensor(qa.QTensor.from_blocks(dt, make_weight(oracle, dtype, n, k, 400 + n), (n, k)))

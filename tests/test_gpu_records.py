@@ -32,25 +32,36 @@ def weight(qa, oracle, dtype, n, k, seed):
 
 @pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
 @pytest.mark.parametrize("m,k,ns", [(16, 4096, (4096, 1024, 1024)), (8, 4096, (12288, 12288)), (5, 1024, (2048, 1000)),
-                                    (40, 2048, (512,)), (64, 12288, (4096,)), (3, 256, (16, 48))])
+                                    (40, 2048, (512,)), (64, 12288, (4096,)), (3, 4096, (16, 48)), (5, 256, (16, 48)),
+                                    (3, 256, (16, 48))])
 def test_records_from_their_producers_equal_the_two_launch_path(qa, oracle, dtype, m, k, ns):
     print(f"records dtype={dtype} m={m} k={k} ns={ns}", flush=True)
     parts = [weight(qa, oracle, dtype, n, k, 5000 + n + i)[0] for i, n in enumerate(ns)]
     x = torch.from_numpy(oracle.randn(5001 + m, (m, k))).cuda()
     nw = torch.from_numpy(oracle.randn(5002, (k,), mean=1.0, std=0.1)).cuda()
     gd = qa.GgmlDType(dtype)
+    # The call on x takes the batched kernels - quantizer, then the kernel that reads records - from
+    # three rows on, from five where k is at most 3072 (three and four rows of a short k run on the
+    # single-launch kernel: same integers, another order of the f32 sums).
+    same_kernel = m >= (5 if k <= 3072 else 3)
+
+    def check(a, b):
+        if same_kernel:
+            assert torch.equal(a, b)
+        else:
+            assert float((a - b).abs().max()) <= 2e-6 * float(b.abs().max())
     # plain quantizer: forward_group on records == forward_group on x
     want = qa.forward_group(parts, x)
     got = qa.ActivationRecords.quantize(gd, x).forward_group(parts)
     for a, b in zip(got, want):
-        assert torch.equal(a, b)
+        check(a, b)
     # RMSNorm -> records == RMSNorm, then the projections
     normed = qa.try_fused_rms_norm(x, nw, 1e-6)
     want = qa.forward_group(parts, normed)
     rec = qa.ActivationRecords.from_rms_norm(gd, x, nw, 1e-6)
     assert torch.equal(rec.data, qa.ActivationRecords.quantize(gd, normed).data)      # the records themselves
     for a, b in zip(rec.forward_group(parts), want):
-        assert torch.equal(a, b)
+        check(a, b)
 
 
 def test_silu_mul_records_bit_equal_to_the_mlp_call(qa, oracle):
