@@ -655,7 +655,7 @@ def test_projection_group_equals_separate_calls(qa, oracle, dtype, m):
 
 
 @pytest.mark.parametrize("dtype", [Q4_K, Q8_0])
-@pytest.mark.parametrize("m", [1, 2, 3, 16])
+@pytest.mark.parametrize("m", [1, 2, 3, 16, 40])
 @pytest.mark.parametrize("k,ns", [(1024, (4000, 1000, 600)), (4096, (4096, 1000, 1048)), (2048, (3000, 3000, 3000, 200)),
                                   (1024, (16, 8200))])
 def test_projection_group_workgroups_straddle_weights(qa, oracle, dtype, m, k, ns):
@@ -679,7 +679,8 @@ def test_projection_group_workgroups_straddle_weights(qa, oracle, dtype, m, k, n
 @pytest.mark.parametrize("k,ns", [(4096, (4096, 1024, 1024)), (2048, (1536, 1536)), (768, (2000, 48, 16, 512))])
 def test_projection_group_on_several_row_tiles(qa, oracle, dtype, m, k, ns):
     """17 <= m <= 64 (two to four 16-row tiles of activations): the group is one launch of the
-    batched decode kernel's several-tiles form and equals the separate forwards bit for bit."""
+    batched decode kernel, workgroups of their own for every tile of rows, and equals the separate
+    forwards bit for bit."""
     _say(f"group tiles dtype={dtype} m={m} k={k} ns={ns}")
     dt = qa.GgmlDType(dtype)
     blocks = [make_weight(oracle, dtype, n, k, 700 + n + i) for i, n in enumerate(ns)]
