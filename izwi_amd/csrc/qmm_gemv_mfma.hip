@@ -1175,6 +1175,10 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
     const int j = lane & 15, grp = lane >> 4;
     const int s_units = P.slots >> 4;
     __shared__ int order[kRankedExperts];
+    // The output rows (pair indices) of the tiles in the window, -1 past the expert's last pair: read
+    // from LDS where the sums are stored.  (Read from `perm` there, every row tile of a wave ended in
+    // sixteen dependent loads in front of its stores.)
+    __shared__ __attribute__((aligned(16))) int tile_rows[TC * 16];
     const bool ranked = rank_experts(P.tile_offsets, P.n_experts, order, reinterpret_cast<int*>(smem));
     const int per_expert = P.parts * P.stacks;
     bool window_used = false;
@@ -1200,6 +1204,10 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
         if (window_used) lds_barrier(); // every wave is done with the previous tiles
         window_used = true;
         issue_window_copy<QT>(records + (size_t)t0 * P.k_units * UB, smem, nt * P.k_units, wave, waves, lane);
+        if (threadIdx.x < TC * 16) { // the tiles' output rows, once per window (see tile_rows)
+            const int mm = t0 * 16 + (int)threadIdx.x;
+            tile_rows[threadIdx.x] = pos_begin + mm < pos_end ? P.perm[pos_begin + mm] : -1;
+        }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         lds_barrier();
         for (int rt = part * waves + wave; rt < P.row_tiles; rt += P.parts * waves) {
@@ -1224,12 +1232,14 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
             const int row = rt * 16 + j;
             if (row < P.n) {
 #pragma unroll
-                for (int t = 0; t < TC; t++)
+                for (int t = 0; t < TC; t++) {
+                    if (t >= nt) continue; // uniform
+                    const int4 rows4 = *reinterpret_cast<const int4*>(&tile_rows[t * 16 + grp * 4]);
+                    const int out_row[4] = {rows4.x, rows4.y, rows4.z, rows4.w};
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        const int mm = (t0 + t) * 16 + grp * 4 + r;
-                        if (t < nt && pos_begin + mm < pos_end) yout[(int64_t)P.perm[pos_begin + mm] * P.n + row] = acc[t][r];
-                    }
+                    for (int r = 0; r < 4; r++)
+                        if (out_row[r] >= 0) yout[(int64_t)out_row[r] * P.n + row] = acc[t][r];
+                }
             }
         }
     }
@@ -1250,6 +1260,10 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int waves = P.nwr;
     __shared__ int order[kRankedExperts];
+    // The output rows (pair indices) of the tiles in the window, -1 past the expert's last pair: read
+    // from LDS where the sums are stored.  (Read from `perm` there, every row tile of a wave ended in
+    // sixteen dependent loads in front of its stores.)
+    __shared__ __attribute__((aligned(16))) int tile_rows[TC * 16];
     const bool ranked = rank_experts(P.tile_offsets, P.n_experts, order, reinterpret_cast<int*>(smem));
     const int per_expert = P.parts * P.stacks;
     bool window_used = false;
@@ -1287,6 +1301,10 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
         if (window_used) lds_barrier(); // every wave is done with the previous tiles
         window_used = true;
         issue_window_copy<QT>(records + (size_t)t0 * P.k_units * UB, smem, nt * P.k_units, wave, waves, lane);
+        if (threadIdx.x < TC * 16) { // the tiles' output rows, once per window (see tile_rows)
+            const int mm = t0 * 16 + (int)threadIdx.x;
+            tile_rows[threadIdx.x] = pos_begin + mm < pos_end ? P.perm[pos_begin + mm] : -1;
+        }
         WPanel<QT> p;
         if (rt_first < P.row_tiles) // (uniform) the wave's first panel, needed whole before its first tile
             load_wpanel<QT>(p, wbase + (int64_t)rt_first * P.k_groups * P.panel_bytes, P.slots, lane, j);
@@ -1341,12 +1359,14 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
             const int row = rt * 16 + j;
             if (row < P.n) {
 #pragma unroll
-                for (int t = 0; t < TC; t++)
+                for (int t = 0; t < TC; t++) {
+                    if (t >= nt) continue; // uniform
+                    const int4 rows4 = *reinterpret_cast<const int4*>(&tile_rows[t * 16 + grp * 4]);
+                    const int out_row[4] = {rows4.x, rows4.y, rows4.z, rows4.w};
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        const int mm = (t0 + t) * 16 + grp * 4 + r;
-                        if (t < nt && pos_begin + mm < pos_end) yout[(int64_t)P.perm[pos_begin + mm] * P.n + row] = acc[t][r];
-                    }
+                    for (int r = 0; r < 4; r++)
+                        if (out_row[r] >= 0) yout[(int64_t)out_row[r] * P.n + row] = acc[t][r];
+                }
             }
         }
     }
