@@ -179,8 +179,8 @@ int izwi_qmm_get_prefill_form(void);
 /* Form of the MoE expert MLP at many pairs per expert (16-row tiles on the matrix cores): 1 = the
  * expert form (a workgroup per expert and part of its rows keeps up to four activation tiles in LDS,
  * every wave walks weight panels on its own), 0 = the one-shot form (a workgroup per group of row
- * tiles, all panels requested at once), negative = chosen per call by the number of pairs per expert
- * (the default: the expert form up to 48 pairs per expert on average).  IZWI_QMM_MOE_EXPERT_FORM=1 / 0
+ * tiles, all panels requested at once), negative = chosen per call (the default: the expert form
+ * wherever two activation tiles of an expert over all of k fit in LDS).  IZWI_QMM_MOE_EXPERT_FORM=1 / 0
  * at start-up forces one.  The integer block dots are the same; the two forms add the k panels of
  * a row in a different order, so results can differ in the last bits of the f32 sums.
  * No counterpart in the reference (it has no MoE code). */

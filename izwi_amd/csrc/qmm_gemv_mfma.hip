@@ -1210,6 +1210,7 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         lds_barrier();
+        int walk = 0; // panels of this wave's walk so far
         for (int rt = part * waves + wave; rt < P.row_tiles; rt += P.parts * waves) {
             float acc[TC][4];
 #pragma unroll
@@ -1217,6 +1218,10 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
 #pragma unroll
                 for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
             for (int kg = 0; kg < P.k_groups; kg++) {
+                // (the two waves of a SIMD take turns at the higher priority: see the Q4_K kernel below)
+                if ((walk + (wave >> 2)) & 1) __builtin_amdgcn_s_setprio(1); // (uniform)
+                else __builtin_amdgcn_s_setprio(0);
+                walk++;
                 WPanel<QT> p;
                 load_wpanel<QT>(p, wbase + (int64_t)(rt * P.k_groups + kg) * P.panel_bytes, P.slots, lane, j);
 #pragma unroll
@@ -1313,6 +1318,7 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
 #ifdef QMM_EXPERT_TRACE
         if (t0 == 0) t_window = wall_clock64();
 #endif
+        int walk = 0; // panels of this wave's walk so far
         for (int rt = rt_first; rt < P.row_tiles; rt += rt_step) {
             float acc[TC][4];
 #pragma unroll
@@ -1320,6 +1326,14 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
 #pragma unroll
                 for (int r = 0; r < 4; r++) acc[t][r] = 0.0f;
             for (int kg = 0; kg < P.k_groups; kg++) {
+                // The two waves of a SIMD take turns at the higher priority, panel by panel: at equal
+                // priority the SIMD issues from the older wave whenever both are ready, and the younger
+                // one of each pair finishes a quarter later (measured: waves 0 - 3 of a workgroup end an
+                // item after 33.7 us, waves 4 - 7 after 42.3, alone on their SIMDs for the last 8.6 us; with
+                // the turns 37.9 and 40.2.  Turns tile by tile were measured slower than none).
+                if ((walk + (wave >> 2)) & 1) __builtin_amdgcn_s_setprio(1); // (uniform)
+                else __builtin_amdgcn_s_setprio(0);
+                walk++;
 #pragma unroll
                 for (int b = 0; b < WPanel<QT>::QC / 2; b++) transpose_pair(p.q[2 * b], p.q[2 * b + 1]);
                 Q4Prepared<NU> prep;
@@ -1673,13 +1687,13 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
     P.y2 = y2;
     P.n_weights = 0;
     {
-        // The expert form where up to four activation tiles of an expert over all of k fit in LDS and
-        // the experts have at most about three tiles each (an expert with more than four takes another
-        // pass over its weights): measured at 128 experts, top-8, per layer, expert / one-shot form:
-        // 127 / 161 us at 128 tokens, 165 / 185 at 256, 231 / 252 at 512, 388 / 380 at 1024, 663 / 621
-        // at 2048.  IZWI_QMM_MOE_EXPERT_FORM=1 / 0 or izwi_qmm_set_moe_expert_form force the choice.
+        // The expert form wherever up to four (at least two) activation tiles of an expert over all of k
+        // fit in LDS; an expert with more tiles takes another pass over its weights per four.  Measured at
+        // 128 experts, top-8, per layer, expert / one-shot form: 106 / 161 us at 128 tokens, 136 / 185
+        // at 256, 179 / 252 at 512, 295 / 351 at 1024, 487 / 557 at 2048, 956 / 1010 at 4096, 1756 / 1891
+        // at 8192.  IZWI_QMM_MOE_EXPERT_FORM=1 / 0 or izwi_qmm_set_moe_expert_form force the choice.
         const int mode = qmm_moe_expert_form();
-        const bool expert_form = mode >= 0 ? mode != 0 : pairs <= (int64_t)48 * n_experts;
+        const bool expert_form = mode >= 0 ? mode != 0 : true;
         const size_t tile_bytes = (size_t)L.k_units * unit_bytes(L.dtype);
         // (Q6_K: two tiles at a time, four do not fit the registers)
         const int tc = L.dtype != QMM_Q6_K && 4 * tile_bytes <= 150 * 1024 ? 4 : (2 * tile_bytes <= 150 * 1024 ? 2 : 0);
