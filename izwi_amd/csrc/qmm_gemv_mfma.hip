@@ -1148,10 +1148,21 @@ __device__ __forceinline__ bool rank_experts(const int32_t* __restrict__ tile_of
 }
 
 // The item of this workgroup in round `round`: -1 when the rounds are over, -2 when this round has none.
-__device__ __forceinline__ int expert_item(int round, int n_items) {
+// Workgroups go to the eight XCDs round-robin by their index, and every XCD has its own L2: the
+// per_expert items of an expert (its stacks and parts, which all copy the same activation tiles) are
+// given to workgroups of one XCD, so that all but the first find the tiles in that L2 - position
+// c = x + 8 (q + per_expert * j) takes item (8 j + x) * per_expert + q.  The second item of a workgroup,
+// 2G - 1 - (its first), then belongs to one expert for the same per_expert workgroups as well.
+__device__ __forceinline__ int expert_item(int round, int n_items, int per_expert) {
     const int g = gridDim.x, base = round * g;
     if (base >= n_items) return -1;
-    const int item = base + ((round & 1) ? g - 1 - (int)blockIdx.x : (int)blockIdx.x);
+    int c = blockIdx.x;
+    if (g % (8 * per_expert) == 0) {
+        const int x = c & 7, y = c >> 3;
+        const int j = y / per_expert, q = y - j * per_expert;
+        c = (8 * j + x) * per_expert + q;
+    }
+    const int item = base + ((round & 1) ? g - 1 - c : c);
     return item < n_items ? item : -2;
 }
 
@@ -1183,7 +1194,7 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
     const int per_expert = P.parts * P.stacks;
     bool window_used = false;
     for (int round = 0; round < kExpertRounds; round++) {
-    const int item = expert_item(round, P.n_experts * per_expert);
+    const int item = expert_item(round, P.n_experts * per_expert, per_expert);
     if (item == -1) break;
     if (item == -2) continue;
     const int pos = item / per_expert, stack = (item - pos * per_expert) / P.parts, part = item - pos * per_expert - stack * P.parts;
@@ -1284,7 +1295,7 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
     const unsigned long long t_start = wall_clock64();
     unsigned long long t_window = 0;
 #endif
-    const int item = expert_item(round, P.n_experts * per_expert);
+    const int item = expert_item(round, P.n_experts * per_expert, per_expert);
     if (item == -1) break;
     if (item == -2) continue;
     const int pos = item / per_expert, stack = (item - pos * per_expert) / P.parts, part = item - pos * per_expert - stack * P.parts;
