@@ -818,9 +818,13 @@ void moe_small_gate_up_kernel(GemvParams P, const float* __restrict__ logits, in
     if (threadIdx.x < 64) {
         int id;
         float w;
-        moe_route::route_token<PER_LANE>(logits + (int64_t)tok * n_experts, n_experts, top_k, (int)threadIdx.x, id, w);
+        // (only the workgroup that writes the token's routing needs all slots and their weights; the
+        // others stop behind their own slot: the arg-max rounds stand in front of every load of weights)
+        const bool writes_routing = blockIdx.x == 0 && slot == 0;
+        moe_route::route_token<PER_LANE>(logits + (int64_t)tok * n_experts, n_experts, top_k, (int)threadIdx.x, id, w,
+                                         writes_routing ? -1 : slot + 1);
         if ((int)threadIdx.x == slot) expert_sh = id;
-        if (blockIdx.x == 0 && slot == 0 && (int)threadIdx.x < top_k) { // once per token: the routing for launch 2
+        if (writes_routing && (int)threadIdx.x < top_k) { // once per token: the routing for launch 2
             ids[tok * top_k + threadIdx.x] = id;
             weights[tok * top_k + threadIdx.x] = w;
             if (ids_out) ids_out[tok * top_k + threadIdx.x] = id;

@@ -41,9 +41,13 @@ __device__ __forceinline__ uint32_t route_key(float v) {
 // wave-wide arg-max (larger logit first, lower expert index on ties): the maximum key by DPP,
 // then the first lane (lowest index) that holds it by ballot.  Lane s < top_k returns slot s
 // in (id, weight): weights = exp(l - lmax) over the selected slots, summed in slot order.
+// `rounds` < top_k (uniform): only the slots below `rounds` are selected and no weight is worked out -
+// for a caller that needs the expert of one slot (lane `rounds - 1` then holds its id).
 template <int PER_LANE>
 __device__ __forceinline__ void route_token(const float* __restrict__ row, int n_experts, int top_k, int lane,
-                                            int& id, float& weight) {
+                                            int& id, float& weight, int rounds = -1) {
+    const bool ids_only = rounds >= 0 && rounds < top_k;
+    const int n_rounds = ids_only ? rounds : top_k;
     float v[PER_LANE];
     uint32_t key[PER_LANE];
 #pragma unroll
@@ -55,7 +59,7 @@ __device__ __forceinline__ void route_token(const float* __restrict__ row, int n
     float my_logit = 0.0f; // lane s keeps the logit of slot s
     int my_id = 0;
     float lmax = 0.0f;
-    for (int s = 0; s < top_k; s++) {
+    for (int s = 0; s < n_rounds; s++) {
         uint32_t kbest = 0;
 #pragma unroll
         for (int i = 0; i < PER_LANE; i++) kbest = max(kbest, key[i]);
@@ -77,6 +81,11 @@ __device__ __forceinline__ void route_token(const float* __restrict__ row, int n
             my_logit = bv;
             my_id = win;
         }
+    }
+    if (ids_only) {
+        id = my_id;
+        weight = 0.0f;
+        return;
     }
     const float p = lane < top_k ? expf(my_logit - lmax) : 0.0f;
     float denom = 0.0f;
