@@ -183,6 +183,10 @@ int izwi_qmm_get_prefill_form(void);
  * wherever two activation tiles of an expert over all of k fit in LDS).  IZWI_QMM_MOE_EXPERT_FORM=1 / 0
  * at start-up forces one.  The integer block dots are the same; the two forms add the k panels of
  * a row in a different order, so results can differ in the last bits of the f32 sums.
+ * In the expert form every activation row is quantized once, on its own (the token rows inside the
+ * routing kernel), and a workgroup puts its tiles together from the rows' records; 2 = the expert
+ * form on records quantized tile by tile through the sort's tables, as the one-shot form reads them
+ * (kept for comparison: the same bits as 1, one more launch and an index chain per tile).
  * No counterpart in the reference (it has no MoE code). */
 int izwi_qmm_set_moe_expert_form(int enabled);
 

@@ -584,12 +584,12 @@ int qmm_current_device(int* device, int* n_cus) {
 hipError_t qmm_get_scratch(int device, hipStream_t stream, size_t bytes, void** out) {
     return get_scratch(device, stream, bytes, out);
 }
-std::atomic<int> g_moe_expert_form{-2}; // -2: read IZWI_QMM_MOE_EXPERT_FORM on first use; then -1 (by size), 0, 1
+std::atomic<int> g_moe_expert_form{-2}; // -2: read IZWI_QMM_MOE_EXPERT_FORM on first use; then -1 (by size), 0, 1, 2
 int qmm_moe_expert_form() {
     int v = g_moe_expert_form.load(std::memory_order_relaxed);
     if (v < -1) {
         const char* e = getenv("IZWI_QMM_MOE_EXPERT_FORM");
-        v = e && e[0] == '1' ? 1 : e && e[0] == '0' ? 0 : -1;
+        v = e && e[0] == '2' ? 2 : e && e[0] == '1' ? 1 : e && e[0] == '0' ? 0 : -1;
         g_moe_expert_form.store(v, std::memory_order_relaxed);
     }
     return v;
@@ -1765,10 +1765,15 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
     const size_t y_bytes = align256((size_t)pairs * hidden * sizeof(float));
     const size_t s_bytes = align256((size_t)(n_experts + 1) * sizeof(int32_t));
     const int64_t max_tiles = pairs / QMM_MOE_TILE_ROWS + (pairs < n_experts ? pairs : n_experts);
+    // Where a stack runs in the expert form, its activations are quantized row by row (the token rows
+    // inside the routing kernel, the rows of silu(gate) * up in pair order) and the kernel puts its tiles
+    // together from the rows' records; otherwise tile by tile through the sort's tables.
+    const bool g_rows = tiles && qmm_moe_row_records_apply(G, gate->n_cus, pairs, t, top_k);
+    const bool d_rows = tiles && qmm_moe_row_records_apply(D, down->n_cus, pairs, pairs, 1);
     size_t r_bytes = 0;
     if (tiles) {
-        const size_t r1 = qmm_moe_records_bytes(G.dtype, max_tiles, hidden);
-        const size_t r2 = qmm_moe_records_bytes(D.dtype, max_tiles, inter);
+        const size_t r1 = g_rows ? qmm_row_records_bytes(t, hidden) : qmm_moe_records_bytes(G.dtype, max_tiles, hidden);
+        const size_t r2 = d_rows ? qmm_row_records_bytes(pairs, inter) : qmm_moe_records_bytes(D.dtype, max_tiles, inter);
         r_bytes = align256(r1 > r2 ? r1 : r2);
     }
     const size_t te_bytes = tiles ? align256((size_t)max_tiles * 4) : 0; // tile -> expert
@@ -1793,6 +1798,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
     int32_t* tile_expert = (int32_t*)(mid + h_bytes + r_bytes); // tile path only
     bool segments_ready = false;
     void* x_blocks = nullptr; // written by the routing kernels below when set
+    bool x_rows_ready = false; // the routing kernel has written the token rows' records
     hipError_t e = hipSuccess;
     if (logits) {
         uint8_t* r = mid + mid_bytes;
@@ -1820,7 +1826,13 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
                                           r_perm, r_off, seg, seg_expert, stream);
             segments_ready = true;
         } else {
-            e = qmm_launch_moe_route(logits, t, n_experts, top_k, r_ids, r_w, stream, x, hidden, G.dtype, x_blocks);
+            if (g_rows) {
+                e = qmm_launch_moe_route_rows(logits, t, n_experts, top_k, r_ids, r_w, stream, x, hidden, G.dtype,
+                                              mid + h_bytes);
+                x_rows_ready = true;
+            } else {
+                e = qmm_launch_moe_route(logits, t, n_experts, top_k, r_ids, r_w, stream, x, hidden, G.dtype, x_blocks);
+            }
             // the sort also leaves the table of the 16-row tiles the matrix-core path walks, or of the
             // 4-row segments of the decode kernel, with the expert of every tile / segment
             if (e == hipSuccess)
@@ -1838,19 +1850,21 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
         float* u = (float*)mid;
         void* records = mid + h_bytes;
         if (!segments_ready) e = qmm_launch_moe_segments(offsets, n_experts, QMM_MOE_TILE_ROWS, seg, tile_expert, max_tiles, stream);
-        if (e == hipSuccess)
-            e = qmm_launch_quantize_grouped(G.dtype, x, nullptr, top_k, hidden, perm, offsets, seg, n_experts,
-                                            max_tiles, records, stream, tile_expert);
+        if (e == hipSuccess && !x_rows_ready)
+            e = g_rows ? qmm_launch_quantize_rows(G.dtype, x, nullptr, t, hidden, records, stream)
+                       : qmm_launch_quantize_grouped(G.dtype, x, nullptr, top_k, hidden, perm, offsets, seg, n_experts,
+                                                     max_tiles, records, stream, tile_expert);
         if (e == hipSuccess)
             e = qmm_launch_gemv_mfma_grouped(G, gate->tiled, up->tiled, records, h, u, perm, offsets, seg, n_experts,
-                                             pairs, stream, gate->n_cus);
+                                             pairs, stream, gate->n_cus, g_rows ? top_k : 0);
         // silu(gate) * up is applied while the down projection's input is quantized
         if (e == hipSuccess)
-            e = qmm_launch_quantize_grouped(D.dtype, h, u, 1, inter, perm, offsets, seg, n_experts, max_tiles,
-                                            records, stream, tile_expert);
+            e = d_rows ? qmm_launch_quantize_rows(D.dtype, h, u, pairs, inter, records, stream)
+                       : qmm_launch_quantize_grouped(D.dtype, h, u, 1, inter, perm, offsets, seg, n_experts, max_tiles,
+                                                     records, stream, tile_expert);
         if (e == hipSuccess)
             e = qmm_launch_gemv_mfma_grouped(D, down->tiled, nullptr, records, y, nullptr, perm, offsets, seg,
-                                             n_experts, pairs, stream, down->n_cus);
+                                             n_experts, pairs, stream, down->n_cus, d_rows ? 1 : 0);
     } else {
         if (!segments_ready)
             e = qmm_launch_moe_segments(offsets, n_experts, QMM_MOE_SEG_ROWS, seg, seg_expert, max_segments, stream);
@@ -1963,7 +1977,7 @@ int izwi_qmm_get_prefill_form(void) { return qmm_get_prefill_form(); }
 
 int izwi_qmm_set_moe_expert_form(int enabled) {
     return qmm_guarded("izwi_qmm_get_prefill_form", [&]() -> int {
-    g_moe_expert_form.store(enabled < 0 ? -1 : enabled ? 1 : 0, std::memory_order_relaxed);
+    g_moe_expert_form.store(enabled < 0 ? -1 : enabled == 2 ? 2 : enabled ? 1 : 0, std::memory_order_relaxed);
     return IZWI_QMM_OK;
     });
 }

@@ -33,6 +33,7 @@
 #include <cstdlib>
 
 #include "qmm_internal.h"
+#include "qmm_moe_route.h"
 #include "qmm_records.h"
 
 // Timing-only ablations of the Q4_K single-tile arithmetic (results are WRONG when set; never defined
@@ -194,6 +195,78 @@ __global__ void quantize_grouped_kernel(const float* __restrict__ x, const float
     quantize_into_record<QT>(v, j, mr, ws + ((int64_t)tile * k_units + unit) * Unit<QT>::kBytes);
 }
 
+// Row records (see kRowUnitBytes): rows [0, rows) of x, or of silu(x) * x2, one 16-lane group per
+// (row, unit), no index tables.
+template <int QT>
+__global__ void quantize_rows_kernel(const float* __restrict__ x, const float* __restrict__ x2, int64_t rows, int k,
+                                     int k_units, uint8_t* __restrict__ out) {
+    const int64_t group = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+    const int j = threadIdx.x & 15;
+    if (group >= rows * k_units) return; // whole 16-lane groups leave together
+    const int64_t row = group / k_units;
+    const int unit = (int)(group - row * k_units);
+    const int k0 = unit * 256 + 16 * j;
+    const bool in_range = k0 + 16 <= k;
+    float v[16];
+    load_run16(x + row * k + k0, x, in_range, v);
+    if (x2 != nullptr) {
+        float u[16];
+        load_run16(x2 + row * k + k0, x2, in_range, u);
+#pragma unroll
+        for (int i = 0; i < 16; i++) v[i] = silu_f(v[i]) * u[i];
+    }
+    quantize_into_record<QT, true>(v, j, 0, out + group * kRowUnitBytes);
+}
+
+// Routing of the tokens, one wavefront per token, which also writes the row records of its token's
+// activation row (requested before the routing, quantized behind it): the routing kernel of
+// qmm_moe.hip with the matrix-core kernels' quantizer.
+template <int PER_LANE, int QT>
+__global__ void route_rows_kernel(const float* __restrict__ logits, int64_t t, int n_experts, int top_k,
+                                  int32_t* __restrict__ ids, float* __restrict__ weights,
+                                  const float* __restrict__ x, int k, int k_units, uint8_t* __restrict__ out) {
+    const int lane = threadIdx.x & 63, j = lane & 15;
+    const int64_t tok = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (tok >= t) return; // whole waves leave together
+    float4 f[2][4]; // units lane / 16 and lane / 16 + 4: all of a row of up to 2048 values
+    bool in_range[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int k0 = ((lane >> 4) + 4 * i) * 256 + 16 * j;
+        in_range[i] = k0 + 16 <= k;
+        const float4* src = reinterpret_cast<const float4*>(in_range[i] ? x + tok * k + k0 : x);
+#pragma unroll
+        for (int c = 0; c < 4; c++) f[i][c] = src[c];
+    }
+    int id;
+    float w;
+    moe_route::route_token<PER_LANE>(logits + tok * n_experts, n_experts, top_k, lane, id, w);
+    if (lane < top_k) {
+        ids[tok * top_k + lane] = id;
+        weights[tok * top_k + lane] = w;
+    }
+    uint8_t* rec = out + tok * k_units * kRowUnitBytes;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int unit = (lane >> 4) + 4 * i;
+        if (unit < k_units) { // uniform for the 16-lane group
+            float v[16];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                v[4 * c] = in_range[i] ? f[i][c].x : 0.0f, v[4 * c + 1] = in_range[i] ? f[i][c].y : 0.0f;
+                v[4 * c + 2] = in_range[i] ? f[i][c].z : 0.0f, v[4 * c + 3] = in_range[i] ? f[i][c].w : 0.0f;
+            }
+            quantize_into_record<QT, true>(v, j, 0, rec + unit * kRowUnitBytes);
+        }
+    }
+    for (int unit = (lane >> 4) + 8; unit < k_units; unit += 4) {
+        const int k0 = unit * 256 + 16 * j;
+        float v[16];
+        load_run16(x + tok * k + k0, x, k0 + 16 <= k, v);
+        quantize_into_record<QT, true>(v, j, 0, rec + unit * kRowUnitBytes);
+    }
+}
+
 // ---- launch 2 ------------------------------------------------------------------
 struct MfmaParams {
     const uint8_t* w;
@@ -220,6 +293,10 @@ struct MfmaParams {
     // is decoded so that all workgroups of an expert run on one XCD (see the kernel)
     int n_experts, stacks;
     int parts; // expert forms: the row tiles of a stack are shared out to this many items
+    // expert forms on row records (row_div > 0): ws holds one record per (source row, unit) and sorted
+    // pair p reads source row perm[p] / row_div = (perm[p] * row_magic) >> 32
+    int row_div;
+    uint32_t row_magic;
     const int32_t* perm;
     const int32_t* offsets;      // sorted pairs of expert e: [offsets[e], offsets[e + 1])
     const int32_t* tile_offsets; // its 16-row tiles (records): [tile_offsets[e], tile_offsets[e + 1])
@@ -686,6 +763,65 @@ __device__ __forceinline__ void issue_window_copy(const uint8_t* __restrict__ sr
             asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(src + off)
                          : "memory", "m0");
     }
+}
+
+// The same window put together from row records: the unit records of up to TC tiles whose sixteen
+// rows each are rows of `rows` (row_off: the lane's byte offsets of the rows lane % 16 of the tiles).
+// A unit record is six pieces of one instruction each: the four KiB of quants (lane = (octet, row):
+// the row's chunk of that octet), and the side data - Q4_K records: the sixteen scales (a dword from
+// each row, lanes 0 - 15) and the sixteen rows of sum bytes (16 B from each row, lanes 0 - 15); Q8_0:
+// twice four blocks' scales of the sixteen rows (a dword per lane).
+template <int QT, int TC>
+__device__ __forceinline__ void issue_window_gather(const uint8_t* __restrict__ rows, const uint32_t (&row_off)[TC],
+                                                    uint8_t* lds, int nt, int k_units, int wave, int waves, int lane) {
+    const uint32_t lds_base = (uint32_t)(uintptr_t)lds; // LDS byte address (uniform)
+    const uint32_t grp16 = (uint32_t)(lane >> 4) * 16u;
+#pragma unroll
+    for (int t = 0; t < TC; t++) {
+        if (t >= nt) continue; // uniform
+        const uint8_t* src_row = rows + row_off[t];
+        for (int piece = wave; piece < k_units * 6; piece += waves) {
+            const int u = piece / 6, sub = piece - 6 * u; // (uniform)
+            const uint32_t unit_lds = lds_base + (uint32_t)(t * k_units + u) * Unit<QT>::kBytes;
+            const uint8_t* src = src_row + u * kRowUnitBytes;
+            if (sub < 4) {
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(unit_lds + sub * 1024);
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(src + sub * 64 + grp16)
+                             : "memory", "m0");
+            } else if (QT == QMM_Q8_0) {
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(unit_lds + Unit<QT>::kQuant + (sub - 4) * 256);
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(dst), "v"(src + 256 + (sub - 4) * 16 + (grp16 >> 2))
+                             : "memory", "m0");
+            } else if (sub == 4) {
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(unit_lds + Unit<QT>::kQuant);
+                if (lane < 16)
+                    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(dst), "v"(src + 272) : "memory", "m0");
+            } else {
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(unit_lds + Unit<QT>::kQuant + 64);
+                if (lane < 16)
+                    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(src + 256) : "memory", "m0");
+            }
+        }
+    }
+}
+
+// The lane's row offsets for issue_window_gather, in two steps (a kernel puts the loads it can
+// request without them in between): the pairs of row lane % 16 of the tiles t0 .. t0 + TC - 1 of the
+// expert whose sorted pairs are [pos_begin, pos_end) - a row past the end reads the expert's first
+// row, its sums are never stored - and from them the byte offsets of their source rows.
+template <int TC>
+__device__ __forceinline__ void gather_pairs(const int32_t* __restrict__ perm, int pos_begin, int pos_end, int t0, int nt,
+                                             int lane, uint32_t (&pair)[TC]) {
+#pragma unroll
+    for (int t = 0; t < TC; t++) {
+        const int pos = pos_begin + (t0 + t) * 16 + (lane & 15);
+        pair[t] = (uint32_t)perm[t < nt && pos < pos_end ? pos : pos_begin];
+    }
+}
+template <int TC>
+__device__ __forceinline__ void gather_row_offsets(uint32_t (&pair)[TC], int row_div, uint32_t row_magic, uint32_t row_bytes) {
+#pragma unroll
+    for (int t = 0; t < TC; t++) pair[t] = (row_div == 1 ? pair[t] : __umulhi(pair[t], row_magic)) * row_bytes;
 }
 
 // Several 16-row tiles of activations on the single-stage forms: one workgroup per (row-tile group,
@@ -1214,7 +1350,14 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
         const int nt = min(TC, n_tiles - t0);
         if (window_used) lds_barrier(); // every wave is done with the previous tiles
         window_used = true;
-        issue_window_copy<QT>(records + (size_t)t0 * P.k_units * UB, smem, nt * P.k_units, wave, waves, lane);
+        if (P.row_div) { // (uniform)
+            uint32_t row_off[TC];
+            gather_pairs<TC>(P.perm, pos_begin, pos_end, t0, nt, lane, row_off);
+            gather_row_offsets<TC>(row_off, P.row_div, P.row_magic, (uint32_t)P.k_units * kRowUnitBytes);
+            issue_window_gather<QT, TC>(P.ws, row_off, smem, nt, P.k_units, wave, waves, lane);
+        } else {
+            issue_window_copy<QT>(records + (size_t)t0 * P.k_units * UB, smem, nt * P.k_units, wave, waves, lane);
+        }
         if (threadIdx.x < TC * 16) { // the tiles' output rows, once per window (see tile_rows)
             const int mm = t0 * 16 + (int)threadIdx.x;
             tile_rows[threadIdx.x] = pos_begin + mm < pos_end ? P.perm[pos_begin + mm] : -1;
@@ -1316,7 +1459,9 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
         const int nt = min(TC, n_tiles - t0);
         if (window_used) lds_barrier(); // every wave is done with the previous tiles
         window_used = true;
-        issue_window_copy<QT>(records + (size_t)t0 * P.k_units * UB, smem, nt * P.k_units, wave, waves, lane);
+        uint32_t row_off[TC];
+        if (P.row_div) gather_pairs<TC>(P.perm, pos_begin, pos_end, t0, nt, lane, row_off); // (uniform)
+        else issue_window_copy<QT>(records + (size_t)t0 * P.k_units * UB, smem, nt * P.k_units, wave, waves, lane);
         if (threadIdx.x < TC * 16) { // the tiles' output rows, once per window (see tile_rows)
             const int mm = t0 * 16 + (int)threadIdx.x;
             tile_rows[threadIdx.x] = pos_begin + mm < pos_end ? P.perm[pos_begin + mm] : -1;
@@ -1324,6 +1469,10 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
         WPanel<QT> p;
         if (rt_first < P.row_tiles) // (uniform) the wave's first panel, needed whole before its first tile
             load_wpanel<QT>(p, wbase + (int64_t)rt_first * P.k_groups * P.panel_bytes, P.slots, lane, j);
+        if (P.row_div) { // (the rows' pairs have arrived while the panel was requested)
+            gather_row_offsets<TC>(row_off, P.row_div, P.row_magic, (uint32_t)P.k_units * kRowUnitBytes);
+            issue_window_gather<QT, TC>(P.ws, row_off, smem, nt, P.k_units, wave, waves, lane);
+        }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         lds_barrier();
 #ifdef QMM_EXPERT_TRACE
@@ -1661,13 +1810,67 @@ hipError_t qmm_launch_quantize_grouped(int dtype, const float* x, const float* x
 
 bool qmm_gemv_mfma_grouped_supported(const QmmLayout& L) { return L.k_groups <= kMaxWaves; }
 
+namespace {
+// Activation tiles of an expert that the expert form holds in LDS at a time (0: the form does not
+// apply): up to four, at least two, over all of k.
+int expert_form_tiles(const QmmLayout& L, int n_cus) {
+    const int mode = qmm_moe_expert_form();
+    const bool expert_form = mode >= 0 ? mode != 0 : true;
+    if (!expert_form || n_cus <= 0) return 0;
+    const size_t tile_bytes = (size_t)L.k_units * unit_bytes(L.dtype);
+    // (Q6_K: two tiles at a time, four do not fit the registers)
+    return L.dtype != QMM_Q6_K && 4 * tile_bytes <= 150 * 1024 ? 4 : (2 * tile_bytes <= 150 * 1024 ? 2 : 0);
+}
+} // namespace
+
+bool qmm_moe_row_records_apply(const QmmLayout& L, int n_cus, int64_t pairs, int64_t rows, int row_div) {
+    // (form 2: the expert form on tile records, kept for comparison)
+    if (qmm_moe_expert_form() == 2 || !qmm_gemv_mfma_grouped_supported(L) || expert_form_tiles(L, n_cus) == 0) return false;
+    // (the kernel's 32-bit row offsets and its division by multiplication)
+    return row_div >= 1 && pairs * row_div < ((int64_t)1 << 32) && rows * L.k_units * kRowUnitBytes < ((int64_t)1 << 32);
+}
+
+size_t qmm_row_records_bytes(int64_t rows, int64_t k) { return (size_t)rows * (size_t)((k + 255) / 256) * kRowUnitBytes; }
+
+hipError_t qmm_launch_quantize_rows(int dtype, const float* x, const float* x2, int64_t rows, int64_t k,
+                                    void* row_records, hipStream_t stream) {
+    const int64_t k_units = (k + 255) / 256;
+    const int64_t threads = rows * k_units * 16;
+    if (threads <= 0) return hipSuccess;
+    if (threads > 0x7fffffff00ll || k > 0x3fffffff || k % 32) return hipErrorInvalidValue;
+    const unsigned grid = (unsigned)((threads + 255) / 256);
+    if (dtype == QMM_Q4_K || dtype == QMM_Q6_K) // both dot against Q8_K activations: one record format
+        quantize_rows_kernel<QMM_Q4_K><<<grid, 256, 0, stream>>>(x, x2, rows, (int)k, (int)k_units, (uint8_t*)row_records);
+    else
+        quantize_rows_kernel<QMM_Q8_0><<<grid, 256, 0, stream>>>(x, x2, rows, (int)k, (int)k_units, (uint8_t*)row_records);
+    return hipGetLastError();
+}
+
+hipError_t qmm_launch_moe_route_rows(const float* logits, int64_t t, int n_experts, int top_k, int32_t* ids,
+                                     float* weights, hipStream_t stream, const float* x, int64_t k, int dtype,
+                                     void* row_records) {
+    if (t <= 0) return hipSuccess;
+    if (!x || !row_records || k <= 0 || k > 0x3fffffff || k % 32) return hipErrorInvalidValue;
+    if (n_experts < 1 || n_experts > 1024 || top_k < 1 || top_k > 64 || top_k > n_experts) return hipErrorInvalidValue;
+    const unsigned grid = (unsigned)((t + 3) / 4);
+    const int per_lane = (n_experts + 63) / 64, k_units = (int)((k + 255) / 256);
+    const bool q8k = dtype == QMM_Q4_K || dtype == QMM_Q6_K;
+    auto launch = [&](auto kernel) { kernel<<<grid, 256, 0, stream>>>(logits, t, n_experts, top_k, ids, weights, x, (int)k, k_units, (uint8_t*)row_records); };
+    if (per_lane <= 2) q8k ? launch(route_rows_kernel<2, QMM_Q4_K>) : launch(route_rows_kernel<2, QMM_Q8_0>);
+    else if (per_lane <= 4) q8k ? launch(route_rows_kernel<4, QMM_Q4_K>) : launch(route_rows_kernel<4, QMM_Q8_0>);
+    else q8k ? launch(route_rows_kernel<16, QMM_Q4_K>) : launch(route_rows_kernel<16, QMM_Q8_0>);
+    return hipGetLastError();
+}
+
 hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
                                         const void* records, float* y, float* y2, const int32_t* perm,
                                         const int32_t* offsets, const int32_t* tile_offsets,
-                                        int n_experts, int64_t pairs, hipStream_t stream, int n_cus) {
+                                        int n_experts, int64_t pairs, hipStream_t stream, int n_cus, int row_div) {
     if (L.n == 0 || n_experts <= 0) return hipSuccess;
     if (!qmm_gemv_mfma_grouped_supported(L) || n_experts > 65535 || L.n > 0x3fffffff)
         return hipErrorInvalidValue;
+    if (row_div && (expert_form_tiles(L, n_cus) == 0 || row_div < 0 || pairs * row_div >= ((int64_t)1 << 32)))
+        return hipErrorInvalidValue; // (row records are read by the expert form only)
     MfmaParams P{};
     P.ep = QmmEpilogue{nullptr, 0};
     P.w = (const uint8_t*)tiled;
@@ -1703,13 +1906,12 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
         // 128 experts, top-8, per layer, expert / one-shot form: 106 / 161 us at 128 tokens, 136 / 185
         // at 256, 179 / 252 at 512, 295 / 351 at 1024, 487 / 557 at 2048, 956 / 1010 at 4096, 1756 / 1891
         // at 8192.  IZWI_QMM_MOE_EXPERT_FORM=1 / 0 or izwi_qmm_set_moe_expert_form force the choice.
-        const int mode = qmm_moe_expert_form();
-        const bool expert_form = mode >= 0 ? mode != 0 : true;
         const size_t tile_bytes = (size_t)L.k_units * unit_bytes(L.dtype);
-        // (Q6_K: two tiles at a time, four do not fit the registers)
-        const int tc = L.dtype != QMM_Q6_K && 4 * tile_bytes <= 150 * 1024 ? 4 : (2 * tile_bytes <= 150 * 1024 ? 2 : 0);
-        if (expert_form && tc && n_cus > 0) {
+        const int tc = expert_form_tiles(L, n_cus);
+        if (tc) {
             MfmaParams E = P;
+            E.row_div = row_div;
+            E.row_magic = row_div > 1 ? (uint32_t)((((uint64_t)1 << 32) / (uint32_t)row_div) + 1) : 0;
             const int stacks = tiled2 ? 2 : 1;
             int waves = kExpertWaves;
             if (waves > L.row_tiles) waves = (int)L.row_tiles;

@@ -330,10 +330,24 @@ hipError_t qmm_launch_quantize_grouped(int dtype, const float* x, const float* x
 bool qmm_gemv_mfma_grouped_supported(const QmmLayout& L);
 // With tiled2 / y2 a second stack of the same shape is multiplied by the same records
 // in the same launch (the expert MLP's gate and up projections).
+// row_div > 0: `records` are row records (below) and sorted pair p reads source row perm[p] / row_div.
 hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
                                         const void* records, float* y, float* y2, const int32_t* perm,
                                         const int32_t* offsets, const int32_t* tile_offsets,
-                                        int n_experts, int64_t pairs, hipStream_t stream, int n_cus);
+                                        int n_experts, int64_t pairs, hipStream_t stream, int n_cus,
+                                        int row_div = 0);
+// Row records: every source row is quantized once, on its own (no tile tables), and the expert form
+// of the grouped kernel puts its tiles together from the rows' records while it copies them to LDS.
+// Whether a stack of layout L with `rows` source rows, read as perm[p] / row_div, runs that way:
+bool qmm_moe_row_records_apply(const QmmLayout& L, int n_cus, int64_t pairs, int64_t rows, int row_div);
+size_t qmm_row_records_bytes(int64_t rows, int64_t k);
+// rows of x, or of silu(x) * x2
+hipError_t qmm_launch_quantize_rows(int dtype, const float* x, const float* x2, int64_t rows, int64_t k,
+                                    void* row_records, hipStream_t stream);
+// qmm_launch_moe_route that also writes the row records of the tokens' activation rows x [t, k]
+hipError_t qmm_launch_moe_route_rows(const float* logits, int64_t t, int n_experts, int top_k, int32_t* ids,
+                                     float* weights, hipStream_t stream, const float* x, int64_t k, int dtype,
+                                     void* row_records);
 
 // Small batches: routing, sort and the segment tables (seg_rows rows per segment) of the grouped
 // decode kernel in one launch; same results as route + sort + segments.

@@ -47,11 +47,18 @@ struct Unit {
     static constexpr int kBytes = kQuant + kSide;
 };
 
+// A row record holds what ONE row contributes to a unit record, in 16-byte pieces that a copy can
+// place into the unit record of any tile the row belongs to: the sixteen chunks (sub-block pair b,
+// octet o) at 16 (4 b + o), then the side data of the row - Q4_K / Q6_K: the sixteen sum bytes at 256
+// and the scale at 272; Q8_0: the eight block scales at 256.
+constexpr int kRowUnitBytes = 288;
+
 // ---- launch 1: activation quantizer into the unit records -------------------
 // One 16-lane group per (row, unit); lane j holds elements 16j..16j+15 of the
 // unit in v, i.e. sub-block j / 2, octets 2 (j % 2) and 2 (j % 2) + 1.  `mr` is
-// the row inside the 16-row tile whose record starts at `rec`.
-template <int QT>
+// the row inside the 16-row tile whose record starts at `rec`; with ROW, `rec` is
+// the row's own record of the unit (see kRowUnitBytes) and `mr` is unused.
+template <int QT, bool ROW = false>
 __device__ __forceinline__ void quantize_into_record(const float (&v)[16], int j, int mr, uint8_t* rec) {
     // the lane's first value of largest magnitude (strictly greater: an equal later one does not
     // replace it; a NaN never wins, as with fmaxf), with its sign
@@ -60,7 +67,7 @@ __device__ __forceinline__ void quantize_into_record(const float (&v)[16], int j
     for (int i = 0; i < 16; i++) best = fabsf(v[i]) > fabsf(best) ? v[i] : best;
     float amax = fabsf(best);
     float scale_mul; // quant = round(v * scale_mul)
-    float* side = reinterpret_cast<float*>(rec + Unit<QT>::kQuant);
+    float* side = reinterpret_cast<float*>(rec + (ROW ? 256 : Unit<QT>::kQuant));
     if (QT == QMM_Q4_K) {
         // BlockQ8K::from_float: iscale = -128 / (first value of largest magnitude): the lowest lane
         // that holds the block's maximum decides the sign
@@ -73,13 +80,13 @@ __device__ __forceinline__ void quantize_into_record(const float (&v)[16], int j
             scale_mul = __fdiv_rn(-128.0f, (key & 1) ? -amax : amax);
             d = __fdiv_rn(1.0f, scale_mul);
         }
-        if (j == 0) side[mr] = d;
+        if (j == 0) side[ROW ? 4 : mr] = d;
     } else {
         // BlockQ8_0::from_float on the lane pair's 32 values
         amax = fmaxf(amax, __int_as_float(dpp<kDppXor1>(__float_as_int(amax))));
         const float d = __fdiv_rn(amax, 127.0f);
         scale_mul = d != 0.0f ? __fdiv_rn(1.0f, d) : 0.0f;
-        if ((j & 1) == 0) side[(j >> 1) * 16 + mr] = qmm_f16_bits_to_f32(qmm_f32_to_f16_bits(d));
+        if ((j & 1) == 0) side[ROW ? (j >> 1) : (j >> 1) * 16 + mr] = qmm_f16_bits_to_f32(qmm_f32_to_f16_bits(d));
     }
     uint32_t q[4];
 #pragma unroll
@@ -98,14 +105,15 @@ __device__ __forceinline__ void quantize_into_record(const float (&v)[16], int j
         s16 = __builtin_amdgcn_sdot4((int)q[3], 0x01010101, s16, false);
         const int bsum = s16 + dpp<kDppXor1>(s16); // the sub-block's 32 quants
         if ((j & 1) == 0) {
-            uint8_t* planes = reinterpret_cast<uint8_t*>(side + 16) + mr * 16;
+            uint8_t* planes = ROW ? reinterpret_cast<uint8_t*>(side) : reinterpret_cast<uint8_t*>(side + 16) + mr * 16;
             planes[s] = (uint8_t)(bsum & 127);
             planes[8 + s] = (uint8_t)(bsum >> 7);
         }
     }
-    uint8_t* dst = rec + (s >> 1) * 1024 + (oct * 16 + mr) * 16 + (s & 1) * 8;
+    uint8_t* dst = ROW ? rec + ((s >> 1) * 4 + oct) * 16 + (s & 1) * 8
+                       : rec + (s >> 1) * 1024 + (oct * 16 + mr) * 16 + (s & 1) * 8;
     *reinterpret_cast<uint2*>(dst) = make_uint2(q[0], q[1]);
-    *reinterpret_cast<uint2*>(dst + 256) = make_uint2(q[2], q[3]);
+    *reinterpret_cast<uint2*>(dst + (ROW ? 16 : 256)) = make_uint2(q[2], q[3]);
 }
 
 } // namespace

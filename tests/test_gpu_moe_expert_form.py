@@ -83,3 +83,38 @@ def test_expert_form_items(qa, oracle, dtype, E, hidden, inter, t, top_k, silent
     # bit; seen as isolated outputs off by 1e-3 .. 2e-3 of the largest one.  A wrong item - rows of
     # another expert, a stack or a part left out - is off by the size of the outputs themselves.)
     assert rel_err(out, want) < 5e-3
+
+
+@pytest.mark.parametrize("dtype,E,hidden,inter,t,top_k", [
+    (Q4_K, 128, 2048, 768, 512, 8),   # the benchmark's layer: panels of four units (gate | up) and of three (down)
+    (Q4_K, 128, 2048, 768, 70, 8),    # tiles with a few rows, experts without a pair
+    (Q4_K, 16, 1280, 256, 300, 4),    # k of five units: the general kernel; experts of five and more tiles (two windows)
+    (Q8_0, 5, 352, 256, 40, 2),       # Q8_0 records (block scales), a ragged last unit
+    (Q4_K, 3, 512, 256, 96, 1),       # top-1: a pair is its token
+])
+def test_row_records_equal_tile_records(qa, oracle, dtype, E, hidden, inter, t, top_k):
+    """The expert form puts its activation tiles together from records of single rows (form 1) or
+    copies records that were quantized tile by tile (form 2): the same quantizer on the same values,
+    so the same bits, through the layer call (routing kernel writes the token rows' records) and
+    through forward (rows quantized by a launch of their own)."""
+    import torch
+    from izwi_amd import capi
+    gate = oracle.quantize(dtype, oracle.randn(821, (E * inter, hidden), std=0.05))
+    up = oracle.quantize(dtype, oracle.randn(822, (E * inter, hidden), std=0.05))
+    down = oracle.quantize(dtype, oracle.randn(823, (E * hidden, inter), std=0.05))
+    dt = qa.GgmlDType(dtype)
+    experts = qa.MoeExperts(qa.QTensor.from_blocks(dt, gate, (E, inter, hidden)),
+                            qa.QTensor.from_blocks(dt, up, (E, inter, hidden)),
+                            qa.QTensor.from_blocks(dt, down, (E, hidden, inter)))
+    x = torch.from_numpy(oracle.randn(824, (t, hidden))).cuda()
+    logits = torch.from_numpy(oracle.randn(825, (t, E))).cuda()
+    ids, wts = qa.moe_route(logits, top_k)
+    perm, offsets = qa.moe_sort(ids, E)
+    got = {}
+    for form in (1, 2):
+        capi.check(capi.lib().izwi_qmm_set_moe_expert_form(form))
+        got[form] = (experts.layer(logits, x, top_k), experts.forward(x, ids, wts, perm, offsets))
+    torch.cuda.synchronize()
+    assert torch.equal(got[1][0].view(torch.int32), got[2][0].view(torch.int32))
+    assert torch.equal(got[1][1].view(torch.int32), got[2][1].view(torch.int32))
+    assert torch.equal(got[1][0].view(torch.int32), got[1][1].view(torch.int32))
