@@ -88,8 +88,8 @@ __device__ __forceinline__ void route_token(const float* __restrict__ row, int n
         return;
     }
     const float p = lane < top_k ? expf(my_logit - lmax) : 0.0f;
-    float denom = 0.0f;
-    for (int s = 0; s < top_k; s++) denom += __shfl(p, s);
+    float denom = 0.0f; // (slot s from lane s, a scalar read: a shuffle goes through the LDS crossbar)
+    for (int s = 0; s < top_k; s++) denom += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), s));
     id = my_id;
     weight = p / denom;
 }
