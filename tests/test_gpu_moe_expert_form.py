@@ -91,6 +91,7 @@ def test_expert_form_items(qa, oracle, dtype, E, hidden, inter, t, top_k, silent
     (Q4_K, 16, 1280, 256, 300, 4),    # k of five units: the general kernel; experts of five and more tiles (two windows)
     (Q8_0, 5, 352, 256, 40, 2),       # Q8_0 records (block scales), a ragged last unit
     (Q4_K, 3, 512, 256, 96, 1),       # top-1: a pair is its token
+    (Q4_K, 8, 2304, 256, 200, 2),     # nine units per row: two tiles at a time, the routing kernel's loop past eight units
 ])
 def test_row_records_equal_tile_records(qa, oracle, dtype, E, hidden, inter, t, top_k):
     """The expert form puts its activation tiles together from records of single rows (form 1) or
