@@ -1915,17 +1915,18 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
             const int stacks = tiled2 ? 2 : 1;
             int waves = kExpertWaves;
             if (waves > L.row_tiles) waves = (int)L.row_tiles;
-            // Items per CU: one while the experts hold a tile or two (all of an expert's rows in one item:
-            // its tiles are copied once), two from 16 pairs per expert on average (the tile counts differ
-            // more from expert to expert and a heavy and a light item on each CU even the CUs out).
-            // Measured per layer at 128 experts, top-8, one / two per CU: 102 / 106 us at 64 tokens, 105 /
-            // 111 at 128, 125 / 122 at 192, 134 / 134 at 256, 152 / 148 at 320, 162 / 156 at 384.
+            // Items per CU: one while every expert holds one tile (all of an expert's rows in one item: its
+            // tile is copied once), two beyond 8 pairs per expert on average, where the first experts get
+            // a second tile (the tile counts differ from expert to expert and a heavy and a light item
+            // on each CU even the CUs out).  Measured per layer at 128 experts, top-8, one / two per CU:
+            // 93.6 / 100.0 us at 64 tokens, 98.0 / 103.7 at 128, 116.8 / 112.7 at 136, 119.5 / 114.9 at 160,
+            // 120.9 / 116.6 at 192, 124.2 / 124.3 at 256, 152.6 / 134.5 at 320, 183.5 / 155.9 at 512.
             // IZWI_QMM_MOE_EXPERT_WGS_PER_CU forces it.  The stacks' row tiles are shared out to `parts`
             // items so that the items are at most that many per CU; a workgroup takes up to
             // kExpertRounds items, so the launch is (items / kExpertRounds) workgroups, all resident at
             // once unless experts x stacks alone exceed two per CU.
             static const int forced_wgs_per_cu = [] { const char* e = getenv("IZWI_QMM_MOE_EXPERT_WGS_PER_CU"); int v = e ? atoi(e) : 0; return v > 0 ? v : 0; }();
-            int per_cu = forced_wgs_per_cu ? forced_wgs_per_cu : (pairs <= (int64_t)16 * n_experts ? 1 : 2);
+            int per_cu = forced_wgs_per_cu ? forced_wgs_per_cu : (pairs <= (int64_t)8 * n_experts ? 1 : 2);
             if (per_cu > kExpertRounds) per_cu = kExpertRounds;
             int parts = (int)((int64_t)per_cu * n_cus / ((int64_t)n_experts * stacks));
             const int max_parts = (int)((L.row_tiles + waves - 1) / waves);
