@@ -1787,7 +1787,9 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
     // segments hold one row and routing, sort and tables are one workgroup, it does not pay (60.4 / 62.6).
     const size_t xb_bytes = logits && !tiles && !qmm_moe_plan_small_supported(t, n_experts, top_k)
                                 ? align256(qmm_x_blocks_bytes(t, hidden)) : 0;
-    const size_t route_bytes = logits ? 3 * p_bytes + s_bytes + sort_bytes + xb_bytes : 0;
+    // (the one-workgroup sort also ranks the experts by tile count for the expert kernels' work items)
+    const bool sort_ranks = logits && tiles && qmm_moe_sort_ranks_experts(pairs, n_experts);
+    const size_t route_bytes = logits ? 3 * p_bytes + s_bytes + sort_bytes + xb_bytes + (sort_ranks ? s_bytes : 0) : 0;
     uint8_t* ws = nullptr;
     HIP_TRY(get_scratch(gate->device, stream, h_bytes + y_bytes + s_bytes + mid_bytes + route_bytes, (void**)&ws));
     float* h = (float*)ws;
@@ -1799,6 +1801,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
     bool segments_ready = false;
     void* x_blocks = nullptr; // written by the routing kernels below when set
     bool x_rows_ready = false; // the routing kernel has written the token rows' records
+    int32_t* expert_order = nullptr; // written by the sort below when set
     hipError_t e = hipSuccess;
     if (logits) {
         uint8_t* r = mid + mid_bytes;
@@ -1808,6 +1811,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
         int32_t* r_off = (int32_t*)(r + 3 * p_bytes);
         int32_t* r_sort = (int32_t*)(r + 3 * p_bytes + s_bytes);
         if (xb_bytes) x_blocks = r + 3 * p_bytes + s_bytes + sort_bytes;
+        if (sort_ranks) expert_order = (int32_t*)(r + 3 * p_bytes + s_bytes + sort_bytes + xb_bytes);
         // a handful of pairs: the whole layer in two launches (routing inside gate / up, combine
         // inside down), same results
         if (!tiles && pairs <= moe_small_max_pairs() && qmm_moe_small_supported(G, D, t, n_experts, top_k)) {
@@ -1838,7 +1842,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
             if (e == hipSuccess)
                 e = qmm_launch_moe_sort(r_ids, pairs, n_experts, r_perm, r_off, seg, r_sort, stream,
                                         tiles ? QMM_MOE_TILE_ROWS : QMM_MOE_SEG_ROWS, tiles ? tile_expert : seg_expert,
-                                        tiles ? max_tiles : max_segments);
+                                        tiles ? max_tiles : max_segments, expert_order);
             segments_ready = true;
         }
         if (e != hipSuccess) return fail_hip(e, "routing kernels");
@@ -1856,7 +1860,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
                                                      max_tiles, records, stream, tile_expert);
         if (e == hipSuccess)
             e = qmm_launch_gemv_mfma_grouped(G, gate->tiled, up->tiled, records, h, u, perm, offsets, seg, n_experts,
-                                             pairs, stream, gate->n_cus, g_rows ? top_k : 0);
+                                             pairs, stream, gate->n_cus, g_rows ? top_k : 0, expert_order);
         // silu(gate) * up is applied while the down projection's input is quantized
         if (e == hipSuccess)
             e = d_rows ? qmm_launch_quantize_rows(D.dtype, h, u, pairs, inter, records, stream)
@@ -1864,7 +1868,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
                                                      records, stream, tile_expert);
         if (e == hipSuccess)
             e = qmm_launch_gemv_mfma_grouped(D, down->tiled, nullptr, records, y, nullptr, perm, offsets, seg,
-                                             n_experts, pairs, stream, down->n_cus, d_rows ? 1 : 0);
+                                             n_experts, pairs, stream, down->n_cus, d_rows ? 1 : 0, expert_order);
     } else {
         if (!segments_ready)
             e = qmm_launch_moe_segments(offsets, n_experts, QMM_MOE_SEG_ROWS, seg, seg_expert, max_segments, stream);

@@ -297,6 +297,7 @@ struct MfmaParams {
     // pair p reads source row perm[p] / row_div = (perm[p] * row_magic) >> 32
     int row_div;
     uint32_t row_magic;
+    const int32_t* expert_order; // expert forms: the experts by falling tile count, or NULL (ranked in the kernel)
     const int32_t* perm;
     const int32_t* offsets;      // sorted pairs of expert e: [offsets[e], offsets[e + 1])
     const int32_t* tile_offsets; // its 16-row tiles (records): [tile_offsets[e], tile_offsets[e + 1])
@@ -1326,7 +1327,7 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
     // from LDS where the sums are stored.  (Read from `perm` there, every row tile of a wave ended in
     // sixteen dependent loads in front of its stores.)
     __shared__ __attribute__((aligned(16))) int tile_rows[TC * 16];
-    const bool ranked = rank_experts(P.tile_offsets, P.n_experts, order, reinterpret_cast<int*>(smem));
+    const bool ranked = P.expert_order ? true : rank_experts(P.tile_offsets, P.n_experts, order, reinterpret_cast<int*>(smem));
     const int per_expert = P.parts * P.stacks;
     bool window_used = false;
     for (int round = 0; round < kExpertRounds; round++) {
@@ -1334,7 +1335,7 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
     if (item == -1) break;
     if (item == -2) continue;
     const int pos = item / per_expert, stack = (item - pos * per_expert) / P.parts, part = item - pos * per_expert - stack * P.parts;
-    const int e = __builtin_amdgcn_readfirstlane(ranked ? order[pos] : pos); // (uniform: scalar registers)
+    const int e = __builtin_amdgcn_readfirstlane(P.expert_order ? P.expert_order[pos] : ranked ? order[pos] : pos); // (uniform: scalar registers)
     const int tile_begin = P.tile_offsets[e];
     const int n_tiles = P.tile_offsets[e + 1] - tile_begin;
     if (n_tiles == 0) { // uniform for the workgroup: nobody waits at a barrier
@@ -1423,7 +1424,7 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
     // from LDS where the sums are stored.  (Read from `perm` there, every row tile of a wave ended in
     // sixteen dependent loads in front of its stores.)
     __shared__ __attribute__((aligned(16))) int tile_rows[TC * 16];
-    const bool ranked = rank_experts(P.tile_offsets, P.n_experts, order, reinterpret_cast<int*>(smem));
+    const bool ranked = P.expert_order ? true : rank_experts(P.tile_offsets, P.n_experts, order, reinterpret_cast<int*>(smem));
     const int per_expert = P.parts * P.stacks;
     bool window_used = false;
 #pragma unroll
@@ -1442,7 +1443,7 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
     if (item == -1) break;
     if (item == -2) continue;
     const int pos = item / per_expert, stack = (item - pos * per_expert) / P.parts, part = item - pos * per_expert - stack * P.parts;
-    const int e = __builtin_amdgcn_readfirstlane(ranked ? order[pos] : pos); // (uniform: scalar registers)
+    const int e = __builtin_amdgcn_readfirstlane(P.expert_order ? P.expert_order[pos] : ranked ? order[pos] : pos); // (uniform: scalar registers)
     const int tile_begin = P.tile_offsets[e];
     const int n_tiles = P.tile_offsets[e + 1] - tile_begin;
     if (n_tiles == 0) { // uniform for the workgroup: nobody waits at a barrier
@@ -1865,7 +1866,8 @@ hipError_t qmm_launch_moe_route_rows(const float* logits, int64_t t, int n_exper
 hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, const void* tiled2,
                                         const void* records, float* y, float* y2, const int32_t* perm,
                                         const int32_t* offsets, const int32_t* tile_offsets,
-                                        int n_experts, int64_t pairs, hipStream_t stream, int n_cus, int row_div) {
+                                        int n_experts, int64_t pairs, hipStream_t stream, int n_cus, int row_div,
+                                        const int32_t* expert_order) {
     if (L.n == 0 || n_experts <= 0) return hipSuccess;
     if (!qmm_gemv_mfma_grouped_supported(L) || n_experts > 65535 || L.n > 0x3fffffff)
         return hipErrorInvalidValue;
@@ -1911,6 +1913,7 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
         if (tc) {
             MfmaParams E = P;
             E.row_div = row_div;
+            E.expert_order = expert_order;
             E.row_magic = row_div > 1 ? (uint32_t)((((uint64_t)1 << 32) / (uint32_t)row_div) + 1) : 0;
             const int stacks = tiled2 ? 2 : 1;
             int waves = kExpertWaves;

@@ -287,10 +287,14 @@ hipError_t qmm_launch_moe_route(const float* logits, int64_t t, int n_experts, i
 // 4-row segments or of the 16-row tiles, whichever the expert MLP behind the sort runs on, and
 // `seg_expert` (may be NULL; up to max_segments entries) the expert of every such segment.
 // `scratch` must hold qmm_moe_sort_scratch_ints(pairs, n_experts) ints.
+// `expert_order` (n_experts ints, may be NULL; only where qmm_moe_sort_ranks_experts says so): the
+// experts by falling segment count, ties by index - the order in which the expert form of the
+// grouped matrix-core kernel numbers its work items (it ranks the experts itself without it).
 hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts, int32_t* perm,
                                int32_t* offsets, int32_t* seg_offsets, int32_t* scratch,
                                hipStream_t stream, int seg_rows = QMM_MOE_SEG_ROWS, int32_t* seg_expert = nullptr,
-                               int64_t max_segments = 0);
+                               int64_t max_segments = 0, int32_t* expert_order = nullptr);
+bool qmm_moe_sort_ranks_experts(int64_t pairs, int n_experts);
 int64_t qmm_moe_sort_scratch_ints(int64_t pairs, int n_experts);
 
 // Expert-grouped decode kernel over sorted pairs.  Row i of the sorted list is
@@ -335,7 +339,7 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
                                         const void* records, float* y, float* y2, const int32_t* perm,
                                         const int32_t* offsets, const int32_t* tile_offsets,
                                         int n_experts, int64_t pairs, hipStream_t stream, int n_cus,
-                                        int row_div = 0);
+                                        int row_div = 0, const int32_t* expert_order = nullptr);
 // Row records: every source row is quantized once, on its own (no tile tables), and the expert form
 // of the grouped kernel puts its tiles together from the rows' records while it copies them to LDS.
 // Whether a stack of layout L with `rows` source rows, read as perm[p] / row_div, runs that way:

@@ -196,7 +196,7 @@ __host__ __device__ inline int64_t block_sort_lds_ints(int64_t pairs, int n_expe
 __device__ __forceinline__ void block_sort_body(const int32_t* ids, int pairs, int n_experts, int32_t* __restrict__ perm,
                                                 int32_t* __restrict__ offsets, int32_t* __restrict__ seg_offsets,
                                                 int seg_rows, int32_t* __restrict__ seg_expert, int max_segments,
-                                                int32_t* sh) {
+                                                int32_t* sh, int32_t* __restrict__ expert_order = nullptr) {
     // hist[runs][stride] | start[n_experts + 1] | masks[waves][2 * n_experts]; the rows of hist have an odd
     // stride: a wave that reads one expert's count of 64 runs would otherwise hit one LDS bank 64 times
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = kBlockSortThreads / 64;
@@ -274,6 +274,19 @@ __device__ __forceinline__ void block_sort_body(const int32_t* ids, int pairs, i
             for (int i = 0, first = base_s + inc_s - sg; i < sg && first + i < max_segments; i++) seg_expert[first + i] = e0;
         if (e0 == n_experts) total_segments = base_s + inc_s;
     }
+    if (expert_order) { // (uniform) the experts by falling segment count, ties by index
+        int32_t* counts = start + n_experts + 1; // (the first wave's bit masks: done with)
+        if (e0 < n_experts) counts[e0] = sg;
+        __syncthreads();
+        if (e0 < n_experts) {
+            int rank = 0;
+            for (int o = 0; o < n_experts; o++) {
+                const int co = counts[o];
+                rank += (co > sg || (co == sg && o < e0)) ? 1 : 0;
+            }
+            expert_order[rank] = e0; // a permutation: every slot is written once
+        }
+    }
     __syncthreads();
     // entries past the last segment say so (the grouped decode launch has one workgroup per entry)
     if (seg_expert)
@@ -291,9 +304,10 @@ __global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int
                                                                        int n_experts, int32_t* __restrict__ perm,
                                                                        int32_t* __restrict__ offsets,
                                                                        int32_t* __restrict__ seg_offsets, int seg_rows,
-                                                                       int32_t* __restrict__ seg_expert, int max_segments) {
+                                                                       int32_t* __restrict__ seg_expert, int max_segments,
+                                                                       int32_t* __restrict__ expert_order) {
     extern __shared__ int32_t sh[];
-    block_sort_body(ids, pairs, n_experts, perm, offsets, seg_offsets, seg_rows, seg_expert, max_segments, sh);
+    block_sort_body(ids, pairs, n_experts, perm, offsets, seg_offsets, seg_rows, seg_expert, max_segments, sh, expert_order);
 }
 
 bool block_sort_fits(int64_t pairs, int n_experts) {
@@ -441,9 +455,11 @@ int64_t qmm_moe_sort_scratch_ints(int64_t pairs, int n_experts) {
 
 hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts, int32_t* perm,
                                int32_t* offsets, int32_t* seg_offsets, int32_t* scratch,
-                               hipStream_t stream, int seg_rows, int32_t* seg_expert, int64_t max_segments) {
+                               hipStream_t stream, int seg_rows, int32_t* seg_expert, int64_t max_segments,
+                               int32_t* expert_order) {
     if (seg_rows < 1 || max_segments > 0x7fffffff) return hipErrorInvalidValue;
     if (n_experts < 1 || n_experts > 8192) return hipErrorInvalidValue;
+    if (expert_order && !block_sort_fits(pairs, n_experts)) return hipErrorInvalidValue; // (qmm_moe_sort_ranks_experts)
     if (block_sort_fits(pairs, n_experts)) {
         const size_t lds = (size_t)block_sort_lds_ints(pairs, n_experts) * sizeof(int32_t);
         if (lds > 48 * 1024) {
@@ -451,7 +467,7 @@ hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
             if (e != hipSuccess) return e;
         }
-        sort_block_kernel<<<1, kBlockSortThreads, lds, stream>>>(ids, (int)pairs, n_experts, perm, offsets, seg_offsets, seg_rows, seg_expert, (int)max_segments);
+        sort_block_kernel<<<1, kBlockSortThreads, lds, stream>>>(ids, (int)pairs, n_experts, perm, offsets, seg_offsets, seg_rows, seg_expert, (int)max_segments, expert_order);
         return hipGetLastError();
     }
     int64_t chunks = (pairs + kSortChunk - 1) / kSortChunk;
@@ -465,6 +481,8 @@ hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts,
                                                                   perm);
     return hipGetLastError();
 }
+
+bool qmm_moe_sort_ranks_experts(int64_t pairs, int n_experts) { return block_sort_fits(pairs, n_experts); }
 
 hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int seg_rows,
                                    int32_t* seg_offsets, int32_t* seg_expert, int64_t max_segments,
