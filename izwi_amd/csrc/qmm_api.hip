@@ -1789,7 +1789,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
                                 ? align256(qmm_x_blocks_bytes(t, hidden)) : 0;
     // (the one-workgroup sort also ranks the experts by tile count for the expert kernels' work items)
     const bool sort_ranks = logits && tiles && qmm_moe_sort_ranks_experts(pairs, n_experts);
-    const size_t route_bytes = logits ? 3 * p_bytes + s_bytes + sort_bytes + xb_bytes + (sort_ranks ? s_bytes : 0) : 0;
+    const size_t route_bytes = logits ? 3 * p_bytes + s_bytes + sort_bytes + xb_bytes + (sort_ranks ? align256((size_t)n_experts * 32) : 0) : 0;
     uint8_t* ws = nullptr;
     HIP_TRY(get_scratch(gate->device, stream, h_bytes + y_bytes + s_bytes + mid_bytes + route_bytes, (void**)&ws));
     float* h = (float*)ws;

@@ -297,7 +297,9 @@ struct MfmaParams {
     // pair p reads source row perm[p] / row_div = (perm[p] * row_magic) >> 32
     int row_div;
     uint32_t row_magic;
-    const int32_t* expert_order; // expert forms: the experts by falling tile count, or NULL (ranked in the kernel)
+    // expert forms: the experts by falling tile count with their ranges (8 ints per rank: expert, first
+    // tile, tiles, first and last + 1 sorted pair), or NULL (ranked in the kernel, ranges from the tables)
+    const int32_t* expert_order;
     const int32_t* perm;
     const int32_t* offsets;      // sorted pairs of expert e: [offsets[e], offsets[e + 1])
     const int32_t* tile_offsets; // its 16-row tiles (records): [tile_offsets[e], tile_offsets[e + 1])
@@ -1335,14 +1337,23 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(Mfm
     if (item == -1) break;
     if (item == -2) continue;
     const int pos = item / per_expert, stack = (item - pos * per_expert) / P.parts, part = item - pos * per_expert - stack * P.parts;
-    const int e = __builtin_amdgcn_readfirstlane(P.expert_order ? P.expert_order[pos] : ranked ? order[pos] : pos); // (uniform: scalar registers)
-    const int tile_begin = P.tile_offsets[e];
-    const int n_tiles = P.tile_offsets[e + 1] - tile_begin;
+    // (uniform: scalar registers; with the sort's table one load brings the expert and its ranges)
+    int e, tile_begin, n_tiles, pos_begin, pos_end;
+    if (P.expert_order) {
+        const int32_t* d = P.expert_order + 8 * pos;
+        e = __builtin_amdgcn_readfirstlane(d[0]), tile_begin = __builtin_amdgcn_readfirstlane(d[1]);
+        n_tiles = __builtin_amdgcn_readfirstlane(d[2]);
+        pos_begin = __builtin_amdgcn_readfirstlane(d[3]), pos_end = __builtin_amdgcn_readfirstlane(d[4]);
+    } else {
+        e = __builtin_amdgcn_readfirstlane(ranked ? order[pos] : pos);
+        tile_begin = P.tile_offsets[e];
+        n_tiles = P.tile_offsets[e + 1] - tile_begin;
+    }
     if (n_tiles == 0) { // uniform for the workgroup: nobody waits at a barrier
         if (ranked) break; // (every later item's expert has no tile either)
         continue;
     }
-    const int pos_begin = P.offsets[e], pos_end = P.offsets[e + 1];
+    if (!P.expert_order) pos_begin = P.offsets[e], pos_end = P.offsets[e + 1];
     const uint8_t* wbase = (stack ? P.w2 : P.w) + (int64_t)e * P.matrix_bytes;
     float* yout = stack ? P.y2 : P.y;
     const uint8_t* records = P.ws + (size_t)tile_begin * P.k_units * UB;
@@ -1443,14 +1454,23 @@ __global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_q4k_kernel
     if (item == -1) break;
     if (item == -2) continue;
     const int pos = item / per_expert, stack = (item - pos * per_expert) / P.parts, part = item - pos * per_expert - stack * P.parts;
-    const int e = __builtin_amdgcn_readfirstlane(P.expert_order ? P.expert_order[pos] : ranked ? order[pos] : pos); // (uniform: scalar registers)
-    const int tile_begin = P.tile_offsets[e];
-    const int n_tiles = P.tile_offsets[e + 1] - tile_begin;
+    // (uniform: scalar registers; with the sort's table one load brings the expert and its ranges)
+    int e, tile_begin, n_tiles, pos_begin, pos_end;
+    if (P.expert_order) {
+        const int32_t* d = P.expert_order + 8 * pos;
+        e = __builtin_amdgcn_readfirstlane(d[0]), tile_begin = __builtin_amdgcn_readfirstlane(d[1]);
+        n_tiles = __builtin_amdgcn_readfirstlane(d[2]);
+        pos_begin = __builtin_amdgcn_readfirstlane(d[3]), pos_end = __builtin_amdgcn_readfirstlane(d[4]);
+    } else {
+        e = __builtin_amdgcn_readfirstlane(ranked ? order[pos] : pos);
+        tile_begin = P.tile_offsets[e];
+        n_tiles = P.tile_offsets[e + 1] - tile_begin;
+    }
     if (n_tiles == 0) { // uniform for the workgroup: nobody waits at a barrier
         if (ranked) break; // (every later item's expert has no tile either)
         continue;
     }
-    const int pos_begin = P.offsets[e], pos_end = P.offsets[e + 1];
+    if (!P.expert_order) pos_begin = P.offsets[e], pos_end = P.offsets[e + 1];
     const uint8_t* wbase = (stack ? P.w2 : P.w) + (int64_t)e * P.matrix_bytes;
     float* yout = stack ? P.y2 : P.y;
     const uint8_t* records = P.ws + (size_t)tile_begin * P.k_units * UB;

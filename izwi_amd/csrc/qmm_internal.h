@@ -287,9 +287,10 @@ hipError_t qmm_launch_moe_route(const float* logits, int64_t t, int n_experts, i
 // 4-row segments or of the 16-row tiles, whichever the expert MLP behind the sort runs on, and
 // `seg_expert` (may be NULL; up to max_segments entries) the expert of every such segment.
 // `scratch` must hold qmm_moe_sort_scratch_ints(pairs, n_experts) ints.
-// `expert_order` (n_experts ints, may be NULL; only where qmm_moe_sort_ranks_experts says so): the
+// `expert_order` (8 ints per expert, may be NULL; only where qmm_moe_sort_ranks_experts says so): the
 // experts by falling segment count, ties by index - the order in which the expert form of the
 // grouped matrix-core kernel numbers its work items (it ranks the experts itself without it).
+// Entry r: the expert of rank r, its first segment, its segment count, its first and last + 1 sorted pair.
 hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts, int32_t* perm,
                                int32_t* offsets, int32_t* seg_offsets, int32_t* scratch,
                                hipStream_t stream, int seg_rows = QMM_MOE_SEG_ROWS, int32_t* seg_expert = nullptr,

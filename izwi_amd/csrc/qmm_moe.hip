@@ -284,7 +284,9 @@ __device__ __forceinline__ void block_sort_body(const int32_t* ids, int pairs, i
                 const int co = counts[o];
                 rank += (co > sg || (co == sg && o < e0)) ? 1 : 0;
             }
-            expert_order[rank] = e0; // a permutation: every slot is written once
+            // (a permutation: every slot is written once) the expert and where its segments and pairs sit
+            int32_t* d = expert_order + 8 * rank;
+            d[0] = e0, d[1] = base_s + inc_s - sg, d[2] = sg, d[3] = base_c + inc_c - c, d[4] = base_c + inc_c;
         }
     }
     __syncthreads();
