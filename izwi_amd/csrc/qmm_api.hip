@@ -1787,11 +1787,13 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
     // segments hold one row and routing, sort and tables are one workgroup, it does not pay (60.4 / 62.6).
     const size_t xb_bytes = logits && !tiles && !qmm_moe_plan_small_supported(t, n_experts, top_k)
                                 ? align256(qmm_x_blocks_bytes(t, hidden)) : 0;
-    // (the one-workgroup sort also ranks the experts by tile count for the expert kernels' work items)
-    const bool sort_ranks = logits && tiles && qmm_moe_sort_ranks_experts(pairs, n_experts);
-    const size_t route_bytes = logits ? 3 * p_bytes + s_bytes + sort_bytes + xb_bytes + (sort_ranks ? align256((size_t)n_experts * 32) : 0) : 0;
+    // (the one-workgroup sort, or the tile-table launch behind a caller's sort, also ranks the experts by
+    // tile count for the expert kernels' work items)
+    const bool order_ready = tiles && (logits ? qmm_moe_sort_ranks_experts(pairs, n_experts) : qmm_moe_segments_rank_experts(n_experts));
+    const size_t order_bytes = order_ready ? align256((size_t)n_experts * 32) : 0;
+    const size_t route_bytes = logits ? 3 * p_bytes + s_bytes + sort_bytes + xb_bytes : 0;
     uint8_t* ws = nullptr;
-    HIP_TRY(get_scratch(gate->device, stream, h_bytes + y_bytes + s_bytes + mid_bytes + route_bytes, (void**)&ws));
+    HIP_TRY(get_scratch(gate->device, stream, h_bytes + y_bytes + s_bytes + mid_bytes + route_bytes + order_bytes, (void**)&ws));
     float* h = (float*)ws;
     float* y = (float*)(ws + h_bytes);
     int32_t* seg = (int32_t*)(ws + h_bytes + y_bytes);
@@ -1801,7 +1803,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
     bool segments_ready = false;
     void* x_blocks = nullptr; // written by the routing kernels below when set
     bool x_rows_ready = false; // the routing kernel has written the token rows' records
-    int32_t* expert_order = nullptr; // written by the sort below when set
+    int32_t* expert_order = order_ready ? (int32_t*)(mid + mid_bytes + route_bytes) : nullptr; // written by the sort / the tile-table launch
     hipError_t e = hipSuccess;
     if (logits) {
         uint8_t* r = mid + mid_bytes;
@@ -1811,7 +1813,6 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
         int32_t* r_off = (int32_t*)(r + 3 * p_bytes);
         int32_t* r_sort = (int32_t*)(r + 3 * p_bytes + s_bytes);
         if (xb_bytes) x_blocks = r + 3 * p_bytes + s_bytes + sort_bytes;
-        if (sort_ranks) expert_order = (int32_t*)(r + 3 * p_bytes + s_bytes + sort_bytes + xb_bytes);
         // a handful of pairs: the whole layer in two launches (routing inside gate / up, combine
         // inside down), same results
         if (!tiles && pairs <= moe_small_max_pairs() && qmm_moe_small_supported(G, D, t, n_experts, top_k)) {
@@ -1853,7 +1854,8 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
     if (tiles) {
         float* u = (float*)mid;
         void* records = mid + h_bytes;
-        if (!segments_ready) e = qmm_launch_moe_segments(offsets, n_experts, QMM_MOE_TILE_ROWS, seg, tile_expert, max_tiles, stream);
+        if (!segments_ready)
+            e = qmm_launch_moe_segments(offsets, n_experts, QMM_MOE_TILE_ROWS, seg, tile_expert, max_tiles, stream, expert_order);
         if (e == hipSuccess && !x_rows_ready)
             e = g_rows ? qmm_launch_quantize_rows(G.dtype, x, nullptr, t, hidden, records, stream)
                        : qmm_launch_quantize_grouped(G.dtype, x, nullptr, top_k, hidden, perm, offsets, seg, n_experts,

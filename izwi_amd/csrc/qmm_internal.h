@@ -312,10 +312,12 @@ size_t qmm_x_blocks_bytes(int64_t rows, int64_t k);
 
 // seg_offsets[e] = exclusive prefix sum of ceil(count(e) / seg_rows) from caller-provided
 // offsets; seg_expert (may be NULL; max_segments ints) = the expert of every segment, -1
-// past the last one.
+// past the last one.  `expert_order` (may be NULL; only where qmm_moe_segments_rank_experts says so): the
+// table of the ranked experts that qmm_launch_moe_sort describes.
 hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int seg_rows,
                                    int32_t* seg_offsets, int32_t* seg_expert, int64_t max_segments,
-                                   hipStream_t stream);
+                                   hipStream_t stream, int32_t* expert_order = nullptr);
+bool qmm_moe_segments_rank_experts(int n_experts);
 
 // Expert-grouped batched decode on the int8 matrix cores (many pairs per expert).
 // Sorted pairs are cut into tiles of QMM_MOE_TILE_ROWS rows that share one expert;

@@ -320,10 +320,14 @@ bool block_sort_fits(int64_t pairs, int n_experts) {
 // every thread sums a contiguous run of experts, the runs are scanned in LDS.
 // With seg_expert: seg_expert[s] = expert of segment s, -1 for s past the last
 // segment (up to max_segments entries).
+// With expert_order (n_experts <= kSegmentsRankedExperts): the table of the ranked experts that the
+// one-workgroup sort writes (see block_sort_body).
+constexpr int kSegmentsRankedExperts = 512;
 __global__ void segments_kernel(const int32_t* __restrict__ offsets, int n_experts, int seg_rows,
                                 int32_t* __restrict__ seg_offsets, int32_t* __restrict__ seg_expert,
-                                int max_segments) {
+                                int max_segments, int32_t* __restrict__ expert_order) {
     __shared__ int32_t part[256];
+    __shared__ int32_t counts[kSegmentsRankedExperts];
     const int per = (n_experts + 255) / 256;
     const int e0 = min(n_experts, (int)threadIdx.x * per), e1 = min(n_experts, e0 + per);
     int32_t sum = 0;
@@ -343,7 +347,23 @@ __global__ void segments_kernel(const int32_t* __restrict__ offsets, int n_exper
         const int32_t n = (offsets[e + 1] - offsets[e] + seg_rows - 1) / seg_rows;
         if (seg_expert)
             for (int32_t i = 0; i < n && run + i < max_segments; i++) seg_expert[run + i] = e;
+        if (expert_order) counts[e] = n;
         run += n;
+    }
+    if (expert_order) { // (uniform) the experts by falling segment count, ties by index
+        __syncthreads();
+        int32_t first = part[threadIdx.x] - sum;
+        for (int e = e0; e < e1; e++) {
+            const int32_t n = counts[e];
+            int rank = 0;
+            for (int o = 0; o < n_experts; o++) {
+                const int co = counts[o];
+                rank += (co > n || (co == n && o < e)) ? 1 : 0;
+            }
+            int32_t* d = expert_order + 8 * rank;
+            d[0] = e, d[1] = first, d[2] = n, d[3] = offsets[e], d[4] = offsets[e + 1];
+            first += n;
+        }
     }
     const int32_t total = part[255];
     if (threadIdx.x == 255) seg_offsets[n_experts] = total;
@@ -484,11 +504,14 @@ hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts,
 
 bool qmm_moe_sort_ranks_experts(int64_t pairs, int n_experts) { return block_sort_fits(pairs, n_experts); }
 
+bool qmm_moe_segments_rank_experts(int n_experts) { return n_experts <= kSegmentsRankedExperts; }
+
 hipError_t qmm_launch_moe_segments(const int32_t* offsets, int n_experts, int seg_rows,
                                    int32_t* seg_offsets, int32_t* seg_expert, int64_t max_segments,
-                                   hipStream_t stream) {
+                                   hipStream_t stream, int32_t* expert_order) {
+    if (expert_order && !qmm_moe_segments_rank_experts(n_experts)) return hipErrorInvalidValue;
     segments_kernel<<<1, 256, 0, stream>>>(offsets, n_experts, seg_rows, seg_offsets, seg_expert,
-                                           (int)max_segments);
+                                           (int)max_segments, expert_order);
     return hipGetLastError();
 }
 
