@@ -94,6 +94,7 @@ def test_expert_form_items(qa, oracle, dtype, E, hidden, inter, t, top_k, silent
     (Q4_K, 8, 2304, 256, 200, 2),     # nine units per row: two tiles at a time, the routing kernel's loop past eight units
     (Q4_K, 12, 512, 256, 150, 3),     # top-k that is no power of two: pair -> token by multiplication
     (Q8_0, 10, 256, 256, 120, 6),
+    (Q4_K, 8, 256, 256, 2200, 8),     # 17600 pairs: past the one-workgroup sort (three sort launches, experts ranked in the kernels)
 ])
 def test_row_records_equal_tile_records(qa, oracle, dtype, E, hidden, inter, t, top_k):
     """The expert form puts its activation tiles together from records of single rows (form 1) or
