@@ -1315,8 +1315,11 @@ __device__ __forceinline__ int expert_item(int round, int n_items, int per_exper
 // current one is multiplied, which the 170 registers of twelve waves do not hold.
 constexpr int kExpertWaves = 8;
 constexpr int kExpertMaxWindowBytes = 160 * 1024 - kRankedExperts * 4 - 1024; // beside the rank table
+// (this general kernel requests a panel where it multiplies it and needs about 150 registers: twelve
+// waves, three per SIMD, hide a panel's round trip better than eight)
+constexpr int kExpertWavesGeneral = 12;
 template <int QT, int TC>
-__global__ __launch_bounds__(64 * kExpertWaves) void gemv_mfma_expert_kernel(MfmaParams P) {
+__global__ __launch_bounds__(64 * kExpertWavesGeneral) void gemv_mfma_expert_kernel(MfmaParams P) {
     constexpr int UB = Unit<QT>::kBytes;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int lane = threadIdx.x & 63;
@@ -1839,8 +1842,7 @@ int expert_form_tiles(const QmmLayout& L, int n_cus) {
     const bool expert_form = mode >= 0 ? mode != 0 : true;
     if (!expert_form || n_cus <= 0) return 0;
     const size_t tile_bytes = (size_t)L.k_units * unit_bytes(L.dtype);
-    // (Q6_K: two tiles at a time, four do not fit the registers)
-    return L.dtype != QMM_Q6_K && 4 * tile_bytes <= 150 * 1024 ? 4 : (2 * tile_bytes <= 150 * 1024 ? 2 : 0);
+    return 4 * tile_bytes <= 150 * 1024 ? 4 : (2 * tile_bytes <= 150 * 1024 ? 2 : 0);
 }
 } // namespace
 
@@ -1929,14 +1931,20 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
         // at 256, 179 / 252 at 512, 295 / 351 at 1024, 487 / 557 at 2048, 956 / 1010 at 4096, 1756 / 1891
         // at 8192.  IZWI_QMM_MOE_EXPERT_FORM=1 / 0 or izwi_qmm_set_moe_expert_form force the choice.
         const size_t tile_bytes = (size_t)L.k_units * unit_bytes(L.dtype);
-        const int tc = expert_form_tiles(L, n_cus);
+        int tc = expert_form_tiles(L, n_cus);
+        // (Q6_K, a tile per expert: the kernel for two tiles at a time needs twelve registers less and is
+        // the faster one, 108 against 109.5 us per layer at 64 tokens; beyond, four tiles save passes over
+        // the weights: 185 against 195 us at 512 tokens)
+        if (L.dtype == QMM_Q6_K && tc == 4 && pairs <= (int64_t)8 * n_experts) tc = 2;
         if (tc) {
             MfmaParams E = P;
             E.row_div = row_div;
             E.expert_order = expert_order;
             E.row_magic = row_div > 1 ? (uint32_t)((((uint64_t)1 << 32) / (uint32_t)row_div) + 1) : 0;
             const int stacks = tiled2 ? 2 : 1;
-            int waves = kExpertWaves;
+            const bool prepared_q4k = L.dtype == QMM_Q4_K && (uniform_panel_units(L) == 4 || uniform_panel_units(L) == 3);
+            static const int general_waves = [] { const char* e = getenv("IZWI_QMM_EXP_GENERAL_WAVES"); int v = e ? atoi(e) : 0; return v >= 1 && v <= kExpertWavesGeneral ? v : kExpertWavesGeneral; }();
+            int waves = prepared_q4k ? kExpertWaves : general_waves;
             if (waves > L.row_tiles) waves = (int)L.row_tiles;
             // Items per CU: one while every expert holds one tile (all of an expert's rows in one item: its
             // tile is copied once), two beyond 8 pairs per expert on average, where the first experts get
@@ -1967,7 +1975,9 @@ hipError_t qmm_launch_gemv_mfma_grouped(const QmmLayout& L, const void* tiled, c
             if (L.dtype == QMM_Q4_K)
                 return tc == 4 ? launch_expert_form<QMM_Q4_K, 4>(E, grid, waves, lds, stream)
                                : launch_expert_form<QMM_Q4_K, 2>(E, grid, waves, lds, stream);
-            if (L.dtype == QMM_Q6_K) return launch_expert_form<QMM_Q6_K, 2>(E, grid, waves, lds, stream);
+            if (L.dtype == QMM_Q6_K)
+                return tc == 4 ? launch_expert_form<QMM_Q6_K, 4>(E, grid, waves, lds, stream)
+                               : launch_expert_form<QMM_Q6_K, 2>(E, grid, waves, lds, stream);
             return tc == 4 ? launch_expert_form<QMM_Q8_0, 4>(E, grid, waves, lds, stream)
                            : launch_expert_form<QMM_Q8_0, 2>(E, grid, waves, lds, stream);
         }
