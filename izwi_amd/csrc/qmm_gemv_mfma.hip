@@ -1311,8 +1311,9 @@ __device__ __forceinline__ int expert_item(int round, int n_items, int per_exper
 // every tile, next panel; no wave waits for another after the tiles have landed.  The weights are
 // read once per TC tiles (an expert with more tiles takes another pass), and the waves of a CU
 // keep several panels in flight where the one-shot form is one chain of round trips per workgroup.
-// Eight waves: two per SIMD, 256 registers each; the compiler requests the next panel while the
-// current one is multiplied, which the 170 registers of twelve waves do not hold.
+// The Q4_K kernel for whole panels (below) runs eight waves: two per SIMD, 256 registers each - it
+// requests the next panel while the current one is multiplied, which the 170 registers of twelve
+// waves do not hold.
 constexpr int kExpertWaves = 8;
 constexpr int kExpertMaxWindowBytes = 160 * 1024 - kRankedExperts * 4 - 1024; // beside the rank table
 // (this general kernel requests a panel where it multiplies it and needs about 150 registers: twelve
