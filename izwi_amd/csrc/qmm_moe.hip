@@ -274,8 +274,8 @@ __device__ __forceinline__ void block_sort_body(const int32_t* ids, int pairs, i
             for (int i = 0, first = base_s + inc_s - sg; i < sg && first + i < max_segments; i++) seg_expert[first + i] = e0;
         if (e0 == n_experts) total_segments = base_s + inc_s;
     }
-    int32_t* counts = start + n_experts + 1; // (the first wave's bit masks: done with)
-    if (expert_order && e0 < n_experts) counts[e0] = sg;
+    int32_t* counts = start + n_experts + 1; // (the first wave's bit masks: done with) counts | ranks
+    if (expert_order && e0 < n_experts) counts[e0] = sg, counts[n_experts + e0] = 0;
     __syncthreads();
     // entries past the last segment say so (the grouped decode launch has one workgroup per entry)
     if (seg_expert)
@@ -287,16 +287,27 @@ __device__ __forceinline__ void block_sort_body(const int32_t* ids, int pairs, i
         const int e = my_e[j];
         if (e >= 0 && e < n_experts) perm[start[e] + sh[run * stride + e] + my_rank[j]] = run * 64 + lane;
     }
-    // the experts by falling segment count, ties by index (behind the stores above, which drain meanwhile)
-    if (expert_order && e0 < n_experts) {
-        int rank = 0;
-        for (int o = 0; o < n_experts; o++) {
-            const int co = counts[o];
-            rank += (co > sg || (co == sg && o < e0)) ? 1 : 0;
+    // the experts by falling segment count, ties by index (behind the stores above, which drain
+    // meanwhile): all threads share the comparisons, thread (expert, slice of the experts) adds its
+    // part of the expert's rank (integer adds: order-free)
+    if (expert_order) { // (uniform)
+        const int slices = max(1, kBlockSortThreads / n_experts), per = (n_experts + slices - 1) / slices;
+        const int e = (int)threadIdx.x % n_experts, slice = (int)threadIdx.x / n_experts;
+        if (slice < slices) {
+            const int mine = counts[e];
+            int part = 0;
+            for (int o = slice * per, o_end = min(n_experts, o + per); o < o_end; o++) {
+                const int co = counts[o];
+                part += (co > mine || (co == mine && o < e)) ? 1 : 0;
+            }
+            if (part) atomicAdd(&counts[n_experts + e], part);
         }
-        // (a permutation: every slot is written once) the expert and where its segments and pairs sit
-        int32_t* d = expert_order + 8 * rank;
-        d[0] = e0, d[1] = base_s + inc_s - sg, d[2] = sg, d[3] = base_c + inc_c - c, d[4] = base_c + inc_c;
+        __syncthreads();
+        if (e0 < n_experts) {
+            // (a permutation: every slot is written once) the expert and where its segments and pairs sit
+            int32_t* d = expert_order + 8 * counts[n_experts + e0];
+            d[0] = e0, d[1] = base_s + inc_s - sg, d[2] = sg, d[3] = base_c + inc_c - c, d[4] = base_c + inc_c;
+        }
     }
 }
 
