@@ -218,48 +218,31 @@ __global__ void quantize_rows_kernel(const float* __restrict__ x, const float* _
     quantize_into_record<QT, true>(v, j, 0, out + group * kRowUnitBytes);
 }
 
-// Routing of the tokens, one wavefront per token, which also writes the row records of its token's
-// activation row (requested before the routing, quantized behind it): the routing kernel of
-// qmm_moe.hip with the matrix-core kernels' quantizer.
+// Routing of the tokens with the row records of their activation rows: the routing kernel of
+// qmm_moe.hip with the matrix-core kernels' quantizer.  Two wavefronts per token, in the two halves
+// of the workgroup: one routes, the other quantizes the token's row meanwhile (one wave doing both in
+// turn made the launch as long as their sum, and the sort waits for this launch to end).
 template <int PER_LANE, int QT>
 __global__ void route_rows_kernel(const float* __restrict__ logits, int64_t t, int n_experts, int top_k,
                                   int32_t* __restrict__ ids, float* __restrict__ weights,
                                   const float* __restrict__ x, int k, int k_units, uint8_t* __restrict__ out) {
     const int lane = threadIdx.x & 63, j = lane & 15;
-    const int64_t tok = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int wave = threadIdx.x >> 6, tokens_per_block = blockDim.x >> 7;
+    const bool quantizes = wave >= tokens_per_block; // (uniform per wave)
+    const int64_t tok = (int64_t)blockIdx.x * tokens_per_block + (quantizes ? wave - tokens_per_block : wave);
     if (tok >= t) return; // whole waves leave together
-    float4 f[2][4]; // units lane / 16 and lane / 16 + 4: all of a row of up to 2048 values
-    bool in_range[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int k0 = ((lane >> 4) + 4 * i) * 256 + 16 * j;
-        in_range[i] = k0 + 16 <= k;
-        const float4* src = reinterpret_cast<const float4*>(in_range[i] ? x + tok * k + k0 : x);
-#pragma unroll
-        for (int c = 0; c < 4; c++) f[i][c] = src[c];
-    }
-    int id;
-    float w;
-    moe_route::route_token<PER_LANE>(logits + tok * n_experts, n_experts, top_k, lane, id, w);
-    if (lane < top_k) {
-        ids[tok * top_k + lane] = id;
-        weights[tok * top_k + lane] = w;
+    if (!quantizes) {
+        int id;
+        float w;
+        moe_route::route_token<PER_LANE>(logits + tok * n_experts, n_experts, top_k, lane, id, w);
+        if (lane < top_k) {
+            ids[tok * top_k + lane] = id;
+            weights[tok * top_k + lane] = w;
+        }
+        return;
     }
     uint8_t* rec = out + tok * k_units * kRowUnitBytes;
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int unit = (lane >> 4) + 4 * i;
-        if (unit < k_units) { // uniform for the 16-lane group
-            float v[16];
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                v[4 * c] = in_range[i] ? f[i][c].x : 0.0f, v[4 * c + 1] = in_range[i] ? f[i][c].y : 0.0f;
-                v[4 * c + 2] = in_range[i] ? f[i][c].z : 0.0f, v[4 * c + 3] = in_range[i] ? f[i][c].w : 0.0f;
-            }
-            quantize_into_record<QT, true>(v, j, 0, rec + unit * kRowUnitBytes);
-        }
-    }
-    for (int unit = (lane >> 4) + 8; unit < k_units; unit += 4) {
+    for (int unit = lane >> 4; unit < k_units; unit += 4) {
         const int k0 = unit * 256 + 16 * j;
         float v[16];
         load_run16(x + tok * k + k0, x, k0 + 16 <= k, v);
@@ -1876,10 +1859,10 @@ hipError_t qmm_launch_moe_route_rows(const float* logits, int64_t t, int n_exper
     if (t <= 0) return hipSuccess;
     if (!x || !row_records || k <= 0 || k > 0x3fffffff || k % 32) return hipErrorInvalidValue;
     if (n_experts < 1 || n_experts > 1024 || top_k < 1 || top_k > 64 || top_k > n_experts) return hipErrorInvalidValue;
-    const unsigned grid = (unsigned)((t + 3) / 4);
+    const unsigned grid = (unsigned)((t + 3) / 4); // four tokens per workgroup: four routing waves, four quantizing
     const int per_lane = (n_experts + 63) / 64, k_units = (int)((k + 255) / 256);
     const bool q8k = dtype == QMM_Q4_K || dtype == QMM_Q6_K;
-    auto launch = [&](auto kernel) { kernel<<<grid, 256, 0, stream>>>(logits, t, n_experts, top_k, ids, weights, x, (int)k, k_units, (uint8_t*)row_records); };
+    auto launch = [&](auto kernel) { kernel<<<grid, 512, 0, stream>>>(logits, t, n_experts, top_k, ids, weights, x, (int)k, k_units, (uint8_t*)row_records); };
     if (per_lane <= 2) q8k ? launch(route_rows_kernel<2, QMM_Q4_K>) : launch(route_rows_kernel<2, QMM_Q8_0>);
     else if (per_lane <= 4) q8k ? launch(route_rows_kernel<4, QMM_Q4_K>) : launch(route_rows_kernel<4, QMM_Q8_0>);
     else q8k ? launch(route_rows_kernel<16, QMM_Q4_K>) : launch(route_rows_kernel<16, QMM_Q8_0>);
