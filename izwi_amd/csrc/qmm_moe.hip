@@ -29,17 +29,25 @@ __device__ __forceinline__ void token_to_x_blocks(const float* __restrict__ x, i
     else x_row_to_blocks<QMM_Q4_K>(x, tok, k, k_units, xb, ld);
 }
 
-// One wavefront per token.  With x blocks to fill, the wave also quantizes its token's activation row
-// (the rows the expert-grouped decode kernel would otherwise quantize in every workgroup of a segment).
+// One wavefront per token.  With x blocks to fill, a second wavefront per token (the second half of
+// the workgroup) quantizes the token's activation row meanwhile (the rows the expert-grouped decode
+// kernel would otherwise quantize in every workgroup of a segment; one wave doing both in turn made
+// the launch as long as their sum, and the sort waits for this launch to end).
 template <int PER_LANE>
 __global__ void route_kernel(const float* __restrict__ logits, int64_t t, int n_experts, int top_k,
                              int32_t* __restrict__ ids, float* __restrict__ weights,
                              const float* __restrict__ x, int k, int dot_dtype, XBlocks xb) {
-    const int lane = threadIdx.x & 63;
-    const int64_t tok = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tokens_per_block = xb.xq != nullptr ? blockDim.x >> 7 : blockDim.x >> 6;
+    const bool quantizes = wave >= tokens_per_block; // (uniform per wave)
+    const int64_t tok = (int64_t)blockIdx.x * tokens_per_block + (quantizes ? wave - tokens_per_block : wave);
     if (tok >= t) return; // whole waves leave together
-    XRowLoads ld;
-    token_x_issue(x, tok, k, xb, ld);
+    if (quantizes) {
+        XRowLoads ld;
+        token_x_issue(x, tok, k, xb, ld);
+        token_to_x_blocks(x, tok, k, dot_dtype, xb, ld);
+        return;
+    }
     int id;
     float w;
     route_token<PER_LANE>(logits + tok * n_experts, n_experts, top_k, lane, id, w);
@@ -47,7 +55,6 @@ __global__ void route_kernel(const float* __restrict__ logits, int64_t t, int n_
         ids[tok * top_k + lane] = id;
         weights[tok * top_k + lane] = w;
     }
-    token_to_x_blocks(x, tok, k, dot_dtype, xb, ld);
 }
 
 // ---- sort ----------------------------------------------------------------
@@ -466,15 +473,16 @@ hipError_t qmm_launch_moe_route(const float* logits, int64_t t, int n_experts, i
     const XBlocks xb = x_blocks ? x_blocks_carve(x_blocks, t, (k + 255) / 256) : XBlocks{nullptr, nullptr, nullptr};
     if (n_experts < 1 || n_experts > 1024 || top_k < 1 || top_k > 64 || top_k > n_experts)
         return hipErrorInvalidValue;
-    const int waves_per_block = 4;
-    unsigned grid = (unsigned)((t + waves_per_block - 1) / waves_per_block);
+    const int tokens_per_block = 4;
+    unsigned grid = (unsigned)((t + tokens_per_block - 1) / tokens_per_block);
+    const unsigned block = 64 * tokens_per_block * (x_blocks ? 2 : 1); // (a quantizing wave beside every routing wave)
     int per_lane = (n_experts + 63) / 64;
     if (per_lane <= 2)
-        route_kernel<2><<<grid, 256, 0, stream>>>(logits, t, n_experts, top_k, ids, weights, x, (int)k, dot_dtype, xb);
+        route_kernel<2><<<grid, block, 0, stream>>>(logits, t, n_experts, top_k, ids, weights, x, (int)k, dot_dtype, xb);
     else if (per_lane <= 4)
-        route_kernel<4><<<grid, 256, 0, stream>>>(logits, t, n_experts, top_k, ids, weights, x, (int)k, dot_dtype, xb);
+        route_kernel<4><<<grid, block, 0, stream>>>(logits, t, n_experts, top_k, ids, weights, x, (int)k, dot_dtype, xb);
     else
-        route_kernel<16><<<grid, 256, 0, stream>>>(logits, t, n_experts, top_k, ids, weights, x, (int)k, dot_dtype, xb);
+        route_kernel<16><<<grid, block, 0, stream>>>(logits, t, n_experts, top_k, ids, weights, x, (int)k, dot_dtype, xb);
     return hipGetLastError();
 }
 
