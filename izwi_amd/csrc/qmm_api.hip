@@ -103,19 +103,19 @@ int ensure_device(int device, int* n_cus) {
     return IZWI_QMM_OK;
 }
 
-// Average sorted pairs per expert from which the expert MLP runs on 16-row matrix-core
-// tiles instead of 4-row dot4 segments (IZWI_QMM_MOE_MFMA_MIN_ROWS, default 4).  Measured at 128
-// experts, top-8, per layer, segments / tiles: 60 / 101 us at 16 tokens, 69 / 101 at 24, 80 / 102 at 32,
-// 88 / 107 at 40, 101 / 110 at 48 (3 pairs per expert), 104 / 111 at 56, 115 / 110 at 64 (4 pairs),
-// 123 / 112 at 72, 132 / 111 at 80: the tile path reads every expert once and costs about the same from
-// 16 to 128 tokens, the segment path grows with the pairs.
-int moe_mfma_min_rows() {
-    static const int v = [] {
+// Whether the expert MLP runs on 16-row matrix-core tiles instead of 4-row dot4 segments: from 3.5
+// sorted pairs per expert on average (IZWI_QMM_MOE_MFMA_MIN_ROWS = a whole number of pairs instead).
+// Measured at 128 experts, top-8, per layer, segments / tiles: 68.6 / 80.4 us at 32 tokens, 78.1 / 83.9
+// at 40, 83.5 / 85.4 at 48 (3 pairs per expert), 91.0 / 86.1 at 56, 99 / 87.1 at 64 (4 pairs): the tile
+// path reads every expert once and costs about the same from 16 to 128 tokens, the segment path
+// grows with the pairs.
+bool moe_on_tiles(int64_t pairs, int n_experts) {
+    static const int forced = [] {
         const char* s = getenv("IZWI_QMM_MOE_MFMA_MIN_ROWS");
-        int n = s ? atoi(s) : 4;
-        return n < 1 ? 1 : n;
+        const int n = s ? atoi(s) : 0;
+        return n < 1 ? 0 : n;
     }();
-    return v;
+    return forced ? pairs >= (int64_t)forced * n_experts : 2 * pairs >= (int64_t)7 * n_experts;
 }
 
 // Most (token, slot) pairs for which izwi_moe_layer_f32 runs as two launches (every pair streams its
@@ -1753,7 +1753,7 @@ int moe_core(const izwi_qmm_weight* gate, const izwi_qmm_weight* up, const izwi_
 
     // Many pairs per expert: 16-row tiles on the int8 matrix cores (the weights of an
     // expert are read once for all its pairs).  Few: 4-row segments on the dot4 kernel.
-    const bool tiles = pairs >= (int64_t)moe_mfma_min_rows() * n_experts &&
+    const bool tiles = moe_on_tiles(pairs, n_experts) &&
                        qmm_gemv_mfma_grouped_supported(G) && qmm_gemv_mfma_grouped_supported(D);
     if (!tiles && max_segments > 65535)
         return fail(IZWI_QMM_ERR_UNSUPPORTED, "t * top_k = %lld is too large for one grouped launch", (long long)pairs);
