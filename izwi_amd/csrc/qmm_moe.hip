@@ -237,7 +237,7 @@ __device__ __forceinline__ void block_sort_body(const int32_t* ids, int pairs, i
     // expert; lane = run, 64 runs per step
     // (few runs: a thread per expert walks them - consecutive experts, consecutive LDS words - instead
     // of eight wave scans in a row per wave with two lanes in use)
-    if (runs <= 16) {
+    if (runs <= 64) {
         for (int e = threadIdx.x; e < n_experts; e += kBlockSortThreads) {
             int carry = 0;
             for (int r = 0; r < runs; r++) {
