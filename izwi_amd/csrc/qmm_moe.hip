@@ -197,6 +197,7 @@ __device__ __forceinline__ int wave_inclusive_sum(int v, int lane) {
 // them there first).  `sh`: block_sort_lds_ints(pairs, n_experts) ints of LDS.  Called by all
 // kBlockSortThreads threads of the workgroup.
 constexpr int kBlockSortThreads = 1024, kBlockSortMaxRuns = 16; // runs per wave
+constexpr int kBlockSortMaxLds = 152 * 1024; // (of the CU's 160 KB: 16384 pairs of 128 experts take 149 KB)
 __host__ __device__ inline int64_t block_sort_lds_ints(int64_t pairs, int n_experts) {
     return ((pairs + 63) / 64) * (n_experts | 1) + n_experts + 1 + (int64_t)2 * n_experts * (kBlockSortThreads / 64);
 }
@@ -331,7 +332,7 @@ __global__ __launch_bounds__(kBlockSortThreads) void sort_block_kernel(const int
 bool block_sort_fits(int64_t pairs, int n_experts) {
     if (pairs < 1 || n_experts >= kBlockSortThreads) return false;
     const int64_t runs = (pairs + 63) / 64;
-    return runs <= (int64_t)kBlockSortMaxRuns * (kBlockSortThreads / 64) && block_sort_lds_ints(pairs, n_experts) * 4 <= 64 * 1024;
+    return runs <= (int64_t)kBlockSortMaxRuns * (kBlockSortThreads / 64) && block_sort_lds_ints(pairs, n_experts) * 4 <= kBlockSortMaxLds;
 }
 
 // seg_offsets[e] = sum over e' < e of ceil(count(e') / seg_rows).  One block:
@@ -503,7 +504,7 @@ hipError_t qmm_launch_moe_sort(const int32_t* ids, int64_t pairs, int n_experts,
         const size_t lds = (size_t)block_sort_lds_ints(pairs, n_experts) * sizeof(int32_t);
         if (lds > 48 * 1024) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sort_block_kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kBlockSortMaxLds);
             if (e != hipSuccess) return e;
         }
         sort_block_kernel<<<1, kBlockSortThreads, lds, stream>>>(ids, (int)pairs, n_experts, perm, offsets, seg_offsets, seg_rows, seg_expert, (int)max_segments, expert_order);
