@@ -502,11 +502,20 @@ def test_moe_route_and_sort_bit_exact(qa, oracle, t):
     assert np.array_equal(offsets.cpu().numpy(), want_off)
 
 
-def test_moe_sort_many_pairs(qa, oracle):
-    rng = np.random.default_rng(3)
-    ids = rng.integers(0, 128, size=(5000, 8)).astype(np.int32)
-    perm, offsets = qa.moe_sort(torch.from_numpy(ids).cuda(), 128)
-    want_perm, want_off = oracle.moe_sort(ids, 128)
+@pytest.mark.parametrize("rows,experts", [
+    (5000, 128),   # 40000 pairs: the three-launch sort
+    (1024, 128),   # 8192 pairs: one workgroup, 83 KB of LDS
+    (2048, 128),   # 16384 pairs: the most one workgroup takes (149 KB)
+    (2049, 128),   # one row more: three launches
+    (1500, 200),   # 12000 pairs of 200 experts: 152 KB would not do, three launches
+    (700, 512),    # many experts, few runs
+])
+def test_moe_sort_many_pairs(qa, oracle, rows, experts):
+    rng = np.random.default_rng(3 + rows)
+    ids = rng.integers(0, experts, size=(rows, 8)).astype(np.int32)
+    ids[:, 3] = 5  # an expert with a pair of every row
+    perm, offsets = qa.moe_sort(torch.from_numpy(ids).cuda(), experts)
+    want_perm, want_off = oracle.moe_sort(ids, experts)
     assert np.array_equal(perm.cpu().numpy(), want_perm) and np.array_equal(offsets.cpu().numpy(), want_off)
 
 
