@@ -95,6 +95,7 @@ def test_expert_form_items(qa, oracle, dtype, E, hidden, inter, t, top_k, silent
     (Q4_K, 12, 512, 256, 150, 3),     # top-k that is no power of two: pair -> token by multiplication
     (Q8_0, 10, 256, 256, 120, 6),
     (Q4_K, 8, 256, 256, 2200, 8),     # 17600 pairs: past the one-workgroup sort (three sort launches, experts ranked in the kernels)
+    (Q4_K, 16, 256, 256, 1024, 8),    # 8192 pairs: the one-workgroup sort on more than 64 KB of LDS
 ])
 def test_row_records_equal_tile_records(qa, oracle, dtype, E, hidden, inter, t, top_k):
     """The expert form puts its activation tiles together from records of single rows (form 1) or
